@@ -1,0 +1,185 @@
+/*
+ * tnn_rocm.h — C ABI of the MI355X (gfx950) kernels behind the DEVICE_ROCM backend.
+ *
+ * This is the only interface between the g++-compiled host code (the layer accelerators that
+ * implement the engine's AbstractDevice / Context / AbstractLayerAcc contract) and the
+ * hipcc-compiled kernels.  Signatures use plain pointers and sizes only.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a positive hipError_t value when a HIP call failed,
+ *     or a negative TNN_ROCM_E* code for a rejected argument; tnn_rocm_last_error() returns a
+ *     message for the most recent failure on the calling thread.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Work is only
+ *     enqueued; nothing synchronises unless the name says so.
+ *   - all data pointers are device pointers unless the parameter name starts with `host_`.
+ *   - `dtype` uses the engine's DataType numbering (include/tnn/core/common.h:51-66 of the
+ *     reference): 0 float32, 1 float16, 2 int8, 3 int32, 4 bfloat16.
+ *   - matrices are row-major; "rows" are tokens (T = batch * sequence).
+ *
+ * Each entry point names the reference function whose result it reproduces (paths relative to
+ * the reference tree).
+ */
+#ifndef TNN_ROCM_H_
+#define TNN_ROCM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TNN_ROCM_API __attribute__((visibility("default")))
+
+enum {
+    TNN_ROCM_F32  = 0,
+    TNN_ROCM_F16  = 1,
+    TNN_ROCM_I8   = 2,
+    TNN_ROCM_I32  = 3,
+    TNN_ROCM_BF16 = 4
+};
+
+enum {
+    TNN_ROCM_EINVAL   = -1, /* bad argument (null pointer, negative size, unknown enum)            */
+    TNN_ROCM_ESHAPE   = -2, /* shape the kernel family does not implement                          */
+    TNN_ROCM_EDTYPE   = -3, /* dtype the entry point does not implement                            */
+    TNN_ROCM_EALIGN   = -4, /* pointer or leading dimension not aligned as documented              */
+    TNN_ROCM_ENODEV   = -5  /* no gfx950 device visible                                            */
+};
+
+/* ---- runtime: what AbstractDevice / Context need -------------------------------------------
+ * replaces source/tnn/device/cuda/cuda_device.cc:53-137 (Allocate/Free/CopyTo/FromDevice) and
+ * source/tnn/device/cuda/cuda_context.cc:47-154 (stream create / synchronize) in role. */
+TNN_ROCM_API const char *tnn_rocm_last_error(void);
+TNN_ROCM_API int tnn_rocm_device_count(int *count);
+TNN_ROCM_API int tnn_rocm_set_device(int device_id);
+TNN_ROCM_API int tnn_rocm_device_name(int device_id, char *buf, size_t buf_len);
+TNN_ROCM_API int tnn_rocm_malloc(void **ptr, size_t bytes);
+TNN_ROCM_API int tnn_rocm_free(void *ptr);
+TNN_ROCM_API int tnn_rocm_memset(void *ptr, int value, size_t bytes, void *stream);
+TNN_ROCM_API int tnn_rocm_memcpy_h2d(void *dst, const void *host_src, size_t bytes, void *stream);
+TNN_ROCM_API int tnn_rocm_memcpy_d2h(void *host_dst, const void *src, size_t bytes, void *stream);
+TNN_ROCM_API int tnn_rocm_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
+TNN_ROCM_API int tnn_rocm_stream_create(void **stream);
+TNN_ROCM_API int tnn_rocm_stream_destroy(void *stream);
+TNN_ROCM_API int tnn_rocm_stream_sync(void *stream);
+/* hipEvent timing on a stream, for the profiler hook of Context (source/tnn/core/context.cc:84-100) */
+TNN_ROCM_API int tnn_rocm_event_create(void **event);
+TNN_ROCM_API int tnn_rocm_event_destroy(void *event);
+TNN_ROCM_API int tnn_rocm_event_record(void *event, void *stream);
+TNN_ROCM_API int tnn_rocm_event_elapsed_ms(void *start, void *stop, float *ms); /* synchronises on `stop` */
+
+/* ---- dense contractions --------------------------------------------------------------------
+ * GEMM epilogue selectors (combinable): y = act(acc + bias) + residual                       */
+enum {
+    TNN_ROCM_EPI_NONE     = 0,
+    TNN_ROCM_EPI_BIAS     = 1, /* + bias[N] (fp32 vector)                                     */
+    TNN_ROCM_EPI_GELU     = 2, /* erf GELU: 0.5*x*(erf(x*0.70710679)+1)  (cpu_gelu_layer_acc.cc:42-45) */
+    TNN_ROCM_EPI_RESIDUAL = 4  /* + residual[M,N] (same dtype as C)                            */
+};
+
+/* C[batch][M,N] = A[batch][M,K] * op(B) with fp32 accumulation.
+ *   b_is_nk = 1: B is [N,K] row-major (InnerProduct weight layout; y = x * W^T):
+ *       NaiveFC                      source/tnn/utils/naive_compute.cc:271-288
+ *       X86InnerProductLayerAcc      source/tnn/device/x86/acc/x86_inner_product_layer_acc.cc:226-273
+ *   b_is_nk = 0: B is [K,N] row-major (MatMul layout):
+ *       CpuMatMulLayerAcc::Forward   source/tnn/device/cpu/acc/cpu_mat_mul_layer_acc.cc:64-117
+ *       X86MatMulLayerAcc::DoForward source/tnn/device/x86/acc/x86_mat_mul_layer_acc.cc:49-114
+ * Batches: `batch` output matrices; A uses matrix (i % batch_a), B uses (i % batch_b) — the
+ * reference's broadcast rule (cpu_mat_mul_layer_acc.cc:99-100).
+ * dtype: F32, F16 or BF16 for A, B, C and residual; bias is always fp32.
+ * lda/ldb/ldc are row strides in elements. */
+TNN_ROCM_API int tnn_rocm_gemm(void *stream, int dtype, int b_is_nk, const void *A, const void *B, void *C, int M,
+                               int N, int K, int lda, int ldb, int ldc, int batch, int batch_a, int batch_b,
+                               int epilogue, const float *bias, const void *residual, int ldr);
+
+/* int8 x int8 -> int32 GEMM with the reference requantisation fused:
+ *   acc[m][n] = sum_k A[m][k]*W[n][k] (+ bias_i32[n]);  out = float2int8((float)acc * scale[n])
+ *       NaiveFCBias   source/tnn/utils/naive_compute.cc:316-347   (zero zero-points)
+ *       X86GemvInt8   source/tnn/device/x86/acc/compute/x86_compute_int8.cc:833-914
+ *       float2int8    source/tnn/utils/naive_compute.cc:32-34
+ * scale[n] is the host-prepared w_scale[n]/o_scale (x86_inner_product_layer_acc.cc:212-220).
+ * out_i8 and/or acc_i32 may be NULL (acc_i32 exposes the exact accumulators for parity tests).
+ * Optional fused dequantisation for a float consumer: if out_f (dtype out_f_dtype F32/F16) is
+ * non-NULL it receives (float)q * dequant_scale, the value a following Reformat layer would
+ * produce (x86_compute_int8.cc:1193-1252). */
+TNN_ROCM_API int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W, const int32_t *bias,
+                                  const float *scale, int8_t *out_i8, int32_t *acc_i32, int M, int N, int K, int lda,
+                                  int ldw, int ldo, void *out_f, int out_f_dtype, float dequant_scale);
+
+/* ---- fused attention core -------------------------------------------------------------------
+ * out = softmax(Q K^T * scale + mask) V per (batch, head): the sub-graph
+ *   MatMul -> Mul/Div -> Add(mask) -> Softmax(axis=-1) -> MatMul
+ * of cpu_mat_mul_layer_acc.cc:64-117, compute_elewise.cc:37-65, cpu_softmax_layer_acc.cc:30-97,
+ * without materialising the [B*h,S,S] scores.  fp32 accumulation, online softmax.
+ * Element (b, head, s, e) of Q is at q[b*q_sb + head*q_sh + s*q_ss + e] (e contiguous); same for
+ * K, V (kv strides) and out.  head_dim must be 64.  dtype F16 or BF16.
+ *   mask   : optional additive fp32 [B, S] (broadcast over heads and query rows), e.g. 0 / -10000
+ *   kv_len : optional int32 [B]; keys j >= kv_len[b] are excluded exactly (−inf) and their tiles
+ *            skipped. */
+TNN_ROCM_API int tnn_rocm_attention(void *stream, int dtype, const void *q, const void *k, const void *v, void *out,
+                                    int B, int heads, int S, int head_dim, long q_sb, long q_sh, long q_ss, long kv_sb,
+                                    long kv_sh, long kv_ss, long o_sb, long o_sh, long o_ss, float scale,
+                                    const float *mask, const int32_t *kv_len);
+
+/* kv_len[b] = 1 + the last key index whose additive mask value is > threshold (0 if none). */
+TNN_ROCM_API int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_t *kv_len, int B, int S,
+                                         float threshold);
+
+/* ---- row-wise ops ---------------------------------------------------------------------------
+ * Softmax over `channel` of x viewed as [outer][channel][inner]
+ *       cpu_softmax_layer_acc.cc:30-97 ; x86_softmax_layer_acc.cc:28-151 */
+TNN_ROCM_API int tnn_rocm_softmax(void *stream, int dtype, const void *x, void *y, int outer, int channel, int inner);
+
+/* y = LayerNorm(x (+ residual)) * gamma + beta over the last `cols` elements of each row;
+ * one-pass E[x^2]-E[x]^2 variance as the reference (cpu_layer_norm_layer_acc.cc:63-140,
+ * x86_layer_norm_layer_acc.cc:26-86); gamma/beta fp32.  residual may be NULL.
+ * Optional fused quantisation: if out_q is non-NULL it also receives
+ * float2int8(y * q_inv_scale) (X86FloatToInt8, x86_compute_int8.cc:1254-1318). */
+TNN_ROCM_API int tnn_rocm_layernorm(void *stream, int dtype, const void *x, const void *residual, const float *gamma,
+                                    const float *beta, void *y, int rows, int cols, float eps, int8_t *out_q,
+                                    float q_inv_scale);
+
+/* ---- element-wise ops -----------------------------------------------------------------------
+ * erf GELU   cpu_gelu_layer_acc.cc:31-51 */
+TNN_ROCM_API int tnn_rocm_gelu(void *stream, int dtype, const void *x, void *y, size_t count);
+
+/* out = a op b with numpy-style broadcast (shapes right-aligned, rank <= 6)
+ *       CPU_ELEWISE  source/tnn/device/cpu/acc/compute/compute_elewise.cc:37-65
+ * op: 0 add, 1 sub, 2 mul, 3 div. */
+TNN_ROCM_API int tnn_rocm_binary(void *stream, int dtype, int op, const void *a, const int *host_shape_a, int rank_a,
+                                 const void *b, const int *host_shape_b, int rank_b, void *out,
+                                 const int *host_shape_out, int rank_out);
+
+/* out dims[j] = in dims[order[j]]   NaivePermute, source/tnn/utils/naive_compute.cc:943-956 */
+TNN_ROCM_API int tnn_rocm_permute(void *stream, int elem_bytes, const void *in, void *out, const int *host_in_dims,
+                                  const int *host_order, int rank);
+
+/* out[b][i][:] = data[b][indices[i]][:]; negative indices wrap; an out-of-range index leaves the
+ * row zero-filled and sets *error_flag (device int32) to 1.
+ *       CpuGatherLayerAcc::Forward  source/tnn/device/cpu/acc/cpu_gather_layer_acc.cc:27-86 */
+TNN_ROCM_API int tnn_rocm_gather(void *stream, const void *data, const int32_t *indices, void *out, int batch,
+                                 int slices, size_t slice_bytes, int n_indices, int32_t *error_flag);
+
+/* dtype conversion between F32, F16 and BF16 (round to nearest even) */
+TNN_ROCM_API int tnn_rocm_cast(void *stream, int src_dtype, const void *src, int dst_dtype, void *dst, size_t count);
+
+/* ---- int8 boundary ops ----------------------------------------------------------------------
+ * q = float2int8(x * inv_scale), inv_scale = (float)(1.0/scale) prepared by the host
+ *       X86FloatToInt8  x86_compute_int8.cc:1254-1318 ; x86_reformat_layer_acc.cc:66-75 */
+TNN_ROCM_API int tnn_rocm_quantize(void *stream, int src_dtype, const void *x, float inv_scale, int8_t *q,
+                                   size_t count);
+/* x = (float)q * scale     X86Int8ToFloat  x86_compute_int8.cc:1193-1252 */
+TNN_ROCM_API int tnn_rocm_dequantize(void *stream, const int8_t *q, float scale, int dst_dtype, void *x, size_t count);
+/* y = float2int8(((float)a*sa + (float)b*sb) * inv_so)   X86MatrixAddInt8 x86_compute_int8.cc:795-831 */
+TNN_ROCM_API int tnn_rocm_add_i8(void *stream, const int8_t *a, float sa, const int8_t *b, float sb, float inv_so,
+                                 int8_t *y, size_t count);
+/* q_out = float2int8(gelu((float)q_in * in_scale) * out_inv_scale): Reformat -> GELU -> Reformat
+ * collapsed into one pass (same three roundings as the separate layers). */
+TNN_ROCM_API int tnn_rocm_gelu_i8(void *stream, const int8_t *q_in, float in_scale, float out_inv_scale,
+                                  int8_t *q_out, size_t count);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TNN_ROCM_H_ */

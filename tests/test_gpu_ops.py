@@ -1,0 +1,492 @@
+"""GPU parity tests: every C-ABI entry point against the CPU checker on the same seeded inputs.
+
+Tolerances (stated per assertion):
+  fp32  : max|d| / max|ref| <= 2e-3   (most ops are asserted far tighter)
+  fp16  : max|d| / max|ref| <= 1e-2, reference computed in fp32 on the fp16-rounded inputs
+  int8 / int32 / index work: bit-exact
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import orc
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 2e-3
+FP16_TOL = 1e-2
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+def ops():
+    from tnn_amd import ops as o
+    return o
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return t if dtype is None else t.to(dtype)
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.float().cpu().numpy() if t.dtype in (torch.float16, torch.bfloat16) else t.cpu().numpy()
+
+
+def rel_err(got, ref):
+    ref = np.asarray(ref, np.float64)
+    got = np.asarray(got, np.float64)
+    return float(np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30))
+
+
+def r16(a):
+    """round to fp16 and back: the values an fp16 kernel actually sees"""
+    return np.asarray(a, np.float32).astype(np.float16).astype(np.float32)
+
+
+# ---------------------------------------------------------------------------------------------
+def test_library_loads_on_gpu():
+    from tnn_amd import capi
+    import ctypes as C
+    n = C.c_int(0)
+    capi.call("tnn_rocm_device_count", C.byref(n))
+    assert n.value >= 1
+    buf = C.create_string_buffer(256)
+    capi.call("tnn_rocm_device_name", 0, buf, 256)
+    say("device: " + buf.value.decode())
+    assert b"gfx950" in buf.value
+
+
+@pytest.mark.parametrize("n", [1, 7, 4096, 128 * 3072 + 3])
+def test_gelu_fp32(n):
+    say("gelu fp32 n=%d" % n)
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 3).astype(np.float32)
+    x[:1] = -2.281006575  # the point where the tanh form is visibly wrong
+    got = host(ops().gelu(dev(x)))
+    ref = orc.gelu(x)
+    assert rel_err(got, ref) <= 1e-6
+    # special values
+    sp = np.array([0.0, -0.0, np.inf, -40.0, 40.0], np.float32)
+    got = host(ops().gelu(dev(sp)))
+    assert got[0] == 0 and got[1] == 0 and got[2] == np.inf and got[3] == 0 and got[4] == 40.0
+
+
+def test_gelu_fp16():
+    say("gelu fp16")
+    rng = np.random.default_rng(1)
+    x = r16(rng.standard_normal(10001) * 3)
+    got = host(ops().gelu(dev(x, torch.float16)))
+    assert rel_err(got, orc.gelu(x)) <= 1e-3  # one fp16 rounding of the result
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 8), (5, 768), (33, 1024), (7, 100), (3, 5000), (4096, 768)])
+def test_layernorm_fp32(rows, cols):
+    say("layernorm fp32 %dx%d" % (rows, cols))
+    rng = np.random.default_rng(rows * 131 + cols)
+    x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(np.float32)
+    g = rng.standard_normal(cols).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    for eps in (1e-5, 1e-12):
+        got = host(ops().layernorm(dev(x), dev(g), dev(b), eps))
+        ref = orc.layernorm(x, g, b, eps)
+        assert rel_err(got, ref) <= 2e-6, (rows, cols, eps)
+
+
+def test_layernorm_large_mean_fp32():
+    # a large common offset makes E[x^2]-E[x]^2 cancel; the double-precision statistics must cope
+    say("layernorm fp32 large mean")
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((16, 768)) + 100.0).astype(np.float32)
+    g = np.ones(768, np.float32)
+    b = np.zeros(768, np.float32)
+    got = host(ops().layernorm(dev(x), dev(g), dev(b), 1e-5))
+    assert rel_err(got, orc.layernorm(x, g, b, 1e-5)) <= 1e-4
+
+
+def test_layernorm_residual_and_quant():
+    say("layernorm fp32 residual + fused quantise")
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((64, 768)).astype(np.float32)
+    r = rng.standard_normal((64, 768)).astype(np.float32)
+    g = rng.standard_normal(768).astype(np.float32)
+    b = rng.standard_normal(768).astype(np.float32)
+    scale = np.float32(0.031)
+    inv = np.float32(1.0 / np.float64(scale))
+    y, q = ops().layernorm(dev(x), dev(g), dev(b), 1e-5, residual=dev(r), q_inv_scale=float(inv))
+    ref = orc.layernorm(orc.binary("add", x, r), g, b, 1e-5)
+    y = host(y)
+    assert rel_err(y, ref) <= 2e-6
+    # the quantised copy must be exactly the quantisation of the y the kernel stored
+    assert np.array_equal(host(q), orc.quantize_x86(y, scale))
+
+
+def test_layernorm_fp16():
+    say("layernorm fp16")
+    rng = np.random.default_rng(7)
+    x = r16(rng.standard_normal((384, 768)))
+    r = r16(rng.standard_normal((384, 768)))
+    g = np.ones(768, np.float32)
+    b = np.zeros(768, np.float32)
+    got = host(ops().layernorm(dev(x, torch.float16), dev(g), dev(b), 1e-12, residual=dev(r, torch.float16)))
+    ref = orc.layernorm(x + r, g, b, 1e-12)
+    assert rel_err(got, ref) <= 2e-3
+    # gamma=1, beta=0: rows have mean 0 and variance 1
+    assert abs(got.mean(-1)).max() < 2e-3 and abs(got.var(-1) - 1).max() < 5e-3
+
+
+def test_layernorm_rejects_empty():
+    from tnn_amd import capi
+    o = ops()
+    x = torch.zeros(4, device="cuda")
+    with pytest.raises(capi.TnnRocmError):
+        capi.call("tnn_rocm_layernorm", None, 0, x.data_ptr(), None, x.data_ptr(), x.data_ptr(), x.data_ptr(), 0, 4,
+                  1e-5, None, 0.0)
+    assert o is not None
+
+
+@pytest.mark.parametrize("shape,axis", [((4, 16), -1), ((3, 5, 7), 1), ((2, 12, 33, 33), -1), ((2, 3, 4, 5, 6), 2),
+                                        ((8, 512), 1), ((3, 2000), 1), ((6, 1, 9), 0)])
+def test_softmax_fp32(shape, axis):
+    say("softmax fp32 %s axis=%d" % (shape, axis))
+    rng = np.random.default_rng(sum(shape) + axis)
+    x = (rng.standard_normal(shape) * 4).astype(np.float32)
+    got = host(ops().softmax(dev(x), axis))
+    ref = orc.softmax(x, axis)
+    # the reference adds the exponentials sequentially in fp32; a tree sum differs by a few ulp
+    assert rel_err(got, ref) <= 1e-5
+    assert np.abs(got.sum(axis) - 1).max() <= 1e-5
+
+
+def test_softmax_masked_columns_are_exact_zero():
+    say("softmax -inf columns")
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((8, 64)).astype(np.float32)
+    x[:, 40:] = -np.inf
+    got = host(ops().softmax(dev(x), -1))
+    assert np.all(got[:, 40:] == 0)
+    assert rel_err(got, orc.softmax(x, -1)) <= 1e-6
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+@pytest.mark.parametrize("sa,sb", [((4, 8, 16), (16,)), ((4, 8, 16), (4, 8, 16)), ((4, 8, 16), (1,)),
+                                   ((2, 12, 33, 33), (2, 1, 1, 33)), ((5, 1, 7), (1, 6, 7)), ((3, 4), (4, 3, 4)),
+                                   ((1024, 768), (768,))])
+def test_binary_fp32(op, sa, sb):
+    say("binary %s %s %s" % (op, sa, sb))
+    rng = np.random.default_rng(len(sa) * 7 + len(sb))
+    a = rng.standard_normal(sa).astype(np.float32)
+    b = (rng.standard_normal(sb) + 3).astype(np.float32)
+    got = host(ops().binary(op, dev(a), dev(b)))
+    ref = orc.binary(op, a, b)
+    assert got.shape == ref.shape
+    assert np.array_equal(got, ref)  # single IEEE operations: bit-exact
+
+
+def test_binary_fp16():
+    say("binary fp16 add bias")
+    rng = np.random.default_rng(9)
+    a = r16(rng.standard_normal((96, 768)))
+    b = r16(rng.standard_normal(768))
+    got = host(ops().binary("add", dev(a, torch.float16), dev(b, torch.float16)))
+    assert np.array_equal(got, r16(a + b))
+
+
+@pytest.mark.parametrize("shape,order", [((128, 12, 64), (1, 0, 2)), ((128, 12, 64), (1, 2, 0)),
+                                         ((2, 16, 12, 64), (0, 2, 1, 3)), ((3, 4, 5, 6, 7), (4, 0, 3, 1, 2)),
+                                         ((9,), (0,))])
+def test_permute(shape, order):
+    say("permute %s %s" % (shape, order))
+    rng = np.random.default_rng(len(shape))
+    x = rng.standard_normal(shape).astype(np.float32)
+    got = host(ops().permute(dev(x), order))
+    ref = orc.permute(x, order)
+    assert np.array_equal(got, ref) and np.array_equal(ref, np.transpose(x, order))
+    x8 = rng.integers(-128, 128, shape, dtype=np.int8)
+    assert np.array_equal(host(ops().permute(dev(x8), order)), np.transpose(x8, order))
+    x16 = x.astype(np.float16)
+    assert np.array_equal(ops().permute(dev(x16), order).cpu().numpy(), np.transpose(x16, order))
+
+
+def test_gather_embedding():
+    say("gather")
+    rng = np.random.default_rng(11)
+    table = rng.standard_normal((30522, 96)).astype(np.float32)
+    idx = rng.integers(0, 30522, (4, 37)).astype(np.int32)
+    idx[0, 0] = -1  # wraps to the last row
+    got, flag = ops().gather(dev(table), dev(idx), 0)
+    ref, rc = orc.gather(table, idx, 0)
+    assert rc == 0 and int(flag.item()) == 0
+    assert np.array_equal(host(got), ref)
+    # out-of-range index: reference reports an error; the kernel raises its flag
+    idx[1, 1] = 30522
+    got, flag = ops().gather(dev(table), dev(idx), 0)
+    assert orc.gather(table, idx, 0)[1] != 0 and int(flag.item()) == 1
+    # odd slice size (3 bytes) and a batch axis
+    t8 = rng.integers(-128, 128, (3, 50, 3), dtype=np.int8)
+    i2 = rng.integers(0, 50, (11,)).astype(np.int32)
+    got, flag = ops().gather(dev(t8), dev(i2), 1)
+    assert np.array_equal(host(got), orc.gather(t8, i2, 1)[0])
+
+
+def test_cast_roundtrip():
+    say("cast")
+    rng = np.random.default_rng(12)
+    x = (rng.standard_normal(100003) * 100).astype(np.float32)
+    h = ops().cast(dev(x), torch.float16)
+    assert np.array_equal(h.cpu().numpy(), x.astype(np.float16))
+    assert np.array_equal(host(ops().cast(h, torch.float32)), x.astype(np.float16).astype(np.float32))
+    bf = ops().cast(dev(x), torch.bfloat16)
+    assert torch.equal(bf.cpu(), torch.from_numpy(x).to(torch.bfloat16))
+
+
+# ---- int8 boundary ops: bit-exact ---------------------------------------------------------------
+def _half_integer_grid(scale):
+    """values whose scaled image sits on and next to every .5 boundary of the int8 range"""
+    k = np.arange(-130, 131, dtype=np.float64) + 0.5
+    base = (k * np.float64(scale)).astype(np.float32)
+    out = [base]
+    for _ in range(3):
+        out.append(np.nextafter(out[-1], np.float32(np.inf)))
+    lo = base
+    for _ in range(3):
+        lo = np.nextafter(lo, np.float32(-np.inf))
+        out.append(lo)
+    return np.concatenate(out).astype(np.float32)
+
+
+@pytest.mark.parametrize("scale", [0.05, 0.0123, 1.0, 3.7e-3])
+def test_quantize_bit_exact(scale):
+    say("quantize scale=%g" % scale)
+    rng = np.random.default_rng(13)
+    scale = np.float32(scale)
+    inv = np.float32(1.0 / np.float64(scale))
+    x = np.concatenate([_half_integer_grid(scale), (rng.standard_normal(200001) * 40 * scale).astype(np.float32),
+                        np.array([0.0, -0.0, 1e30, -1e30], np.float32)])
+    got = host(ops().quantize(dev(x), float(inv)))
+    assert np.array_equal(got, orc.quantize_x86(x, scale))
+
+
+def test_dequantize_and_add_i8_bit_exact():
+    say("dequantize / add_i8")
+    rng = np.random.default_rng(14)
+    q = rng.integers(-128, 128, 100001, dtype=np.int8)
+    assert np.array_equal(host(ops().dequantize(dev(q), 0.0371)), orc.dequantize(q, np.float32(0.0371)))
+    a = rng.integers(-128, 128, 100001, dtype=np.int8)
+    sa, sb, so = np.float32(0.021), np.float32(0.047), np.float32(0.052)
+    inv = np.float32(1.0 / np.float64(so))
+    got = host(ops().add_i8(dev(a), float(sa), dev(q), float(sb), float(inv)))
+    assert np.array_equal(got, orc.add_int8_x86(a, sa, q, sb, so))
+
+
+def test_gelu_i8_matches_three_layer_chain():
+    say("gelu_i8")
+    q = np.arange(-128, 128, dtype=np.int8)
+    q = np.tile(q, 64)
+    s_in, s_out = np.float32(0.043), np.float32(0.019)
+    inv = np.float32(1.0 / np.float64(s_out))
+    got = host(ops().gelu_i8(dev(q), float(s_in), float(inv)))
+    ref = orc.quantize_x86(orc.gelu(orc.dequantize(q, s_in)), s_out)
+    # erff on the device and in glibc may differ in the last ulp, which can flip a value that lands on
+    # a rounding boundary: allow +-1 LSB there but require near-total equality
+    diff = np.abs(got.astype(np.int32) - ref.astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+
+
+# ---- GEMM ------------------------------------------------------------------------------------------
+GEMM_SHAPES = [(1, 1, 1), (3, 4, 9), (8, 21, 10), (11, 50, 19), (33, 65, 130), (128, 768, 768), (130, 96, 264),
+               (256, 3072, 768), (64, 768, 3072), (200, 2304, 768)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+@pytest.mark.parametrize("b_is_nk", [True, False])
+def test_gemm_fp32(M, N, K, b_is_nk):
+    say("gemm fp32 M=%d N=%d K=%d nk=%s" % (M, N, K, b_is_nk))
+    rng = np.random.default_rng(M * 7 + N * 3 + K)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    if b_is_nk:
+        got = host(ops().gemm(dev(a), dev(w), True, bias=dev(bias)))
+        ref = orc.inner_product(a, w, bias)           # NaiveFC
+    else:
+        wt = np.ascontiguousarray(w.T)
+        got = host(ops().gemm(dev(a), dev(wt), False))
+        ref = orc.matmul(a, wt)                       # double-accumulated MatMul
+    assert rel_err(got, ref) <= 1e-5  # far inside the 2e-3 fp32 bar
+
+
+def test_gemm_identity_and_onehot():
+    # closed forms that catch a transposed operand or a wrong index
+    say("gemm identity / one-hot")
+    rng = np.random.default_rng(21)
+    a = rng.standard_normal((70, 96)).astype(np.float32)
+    eye = np.eye(96, dtype=np.float32)
+    assert np.array_equal(host(ops().gemm(dev(a), dev(eye), True)), a)
+    assert np.array_equal(host(ops().gemm(dev(a), dev(eye), False)), a)
+    w = np.zeros((5, 96), np.float32)
+    for n, k in enumerate([3, 95, 0, 17, 64]):
+        w[n, k] = 2.0
+    assert np.array_equal(host(ops().gemm(dev(a), dev(w), True)), 2 * a[:, [3, 95, 0, 17, 64]])
+    assert np.array_equal(host(ops().gemm(dev(a), dev(np.ascontiguousarray(w.T)), False)),
+                          2 * a[:, [3, 95, 0, 17, 64]])
+
+
+@pytest.mark.parametrize("ba,bb", [(12, 12), (12, 1), (1, 12), (6, 3)])
+def test_gemm_batched_broadcast_fp32(ba, bb):
+    say("gemm batched ba=%d bb=%d" % (ba, bb))
+    rng = np.random.default_rng(ba * 13 + bb)
+    a = rng.standard_normal((ba, 40, 64)).astype(np.float32)
+    b = rng.standard_normal((bb, 64, 48)).astype(np.float32)
+    got = host(ops().gemm(dev(a), dev(b), False))
+    assert rel_err(got, orc.matmul(a, b)) <= 1e-5
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 768, 768), (384, 2304, 768), (200, 3072, 768), (96, 768, 3072),
+                                   (17, 40, 24), (5, 7, 9)])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_half_epilogues(M, N, K, dtype):
+    say("gemm %s M=%d N=%d K=%d" % (dtype, M, N, K))
+    td = torch.float16 if dtype == "f16" else torch.bfloat16
+    rng = np.random.default_rng(M + N + K)
+    a = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(td)
+    w = torch.from_numpy((rng.standard_normal((N, K)) * 0.02).astype(np.float32)).to(td)
+    res = torch.from_numpy(rng.standard_normal((M, N)).astype(np.float32)).to(td)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    af, wf, rf = a.float().numpy(), w.float().numpy(), res.float().numpy()
+    tol = FP16_TOL if dtype == "f16" else 2e-2  # bf16 keeps 8 mantissa bits
+    got = host(ops().gemm(a.cuda(), w.cuda(), True, bias=dev(bias)))
+    assert rel_err(got, orc.inner_product(af, wf, bias)) <= tol
+    got = host(ops().gemm(a.cuda(), w.cuda(), True, bias=dev(bias), gelu=True))
+    assert rel_err(got, orc.gelu(orc.inner_product(af, wf, bias))) <= tol
+    got = host(ops().gemm(a.cuda(), w.cuda(), True, bias=dev(bias), residual=res.cuda()))
+    assert rel_err(got, orc.inner_product(af, wf, bias) + rf) <= tol
+
+
+# ---- int8 GEMM: bit-exact accumulators and outputs -----------------------------------------------
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (2, 4, 9), (2, 16, 19), (7, 32, 16), (128, 3072, 768), (128, 768, 3072),
+                                   (300, 768, 768), (65, 100, 200)])
+def test_gemm_i8_bit_exact(M, N, K):
+    say("gemm_i8 M=%d N=%d K=%d" % (M, N, K))
+    rng = np.random.default_rng(M * 5 + N + K)
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)   # full int8 range, not the unit tests' [-8,8)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    bias = rng.integers(-20000, 20000, N).astype(np.int32)
+    w_scale = (rng.uniform(0.5, 1.5, N) * 1e-3).astype(np.float32)
+    scale = orc.fc_int8_scale(w_scale, np.float32(0.37), N)
+    # make sure real rounding happens: typical |acc*scale| ~ tens
+    q, acc, outf = ops().gemm_i8(dev(a), dev(w), dev(bias), dev(scale), want_acc=True, dequant_scale=0.37)
+    ref_q, ref_acc = orc.fc_int8(a, w, bias, scale)
+    assert np.array_equal(host(acc), ref_acc)
+    assert np.array_equal(ref_acc, a.astype(np.int64) @ w.astype(np.int64).T + bias)  # pins the checker itself
+    assert np.array_equal(host(q), ref_q)
+    assert np.array_equal(host(outf), orc.dequantize(ref_q, np.float32(0.37)))
+
+
+def test_gemm_i8_large_accumulators():
+    # |acc| > 2^24: (float)acc rounds before the scale multiply on every path
+    say("gemm_i8 saturating inputs")
+    M, N, K = 64, 64, 3072
+    a = np.full((M, K), 127, np.int8)
+    w = np.full((N, K), 127, np.int8)
+    w[1::2] = -127
+    scale = np.full(N, 2.0e-6, np.float32)
+    q, acc, _ = ops().gemm_i8(dev(a), dev(w), None, dev(scale), want_acc=True)
+    ref_q, ref_acc = orc.fc_int8(a, w, None, scale)
+    assert np.array_equal(host(acc), ref_acc) and abs(int(ref_acc[0, 0])) > 2 ** 24
+    assert np.array_equal(host(q), ref_q)
+
+
+# ---- fused attention ------------------------------------------------------------------------------
+def _attn_case(B, h, S, lens, seed, dtype=torch.float16, with_mask=False):
+    rng = np.random.default_rng(seed)
+    q = torch.from_numpy(rng.standard_normal((B, h, S, 64)).astype(np.float32)).to(dtype)
+    k = torch.from_numpy(rng.standard_normal((B, h, S, 64)).astype(np.float32)).to(dtype)
+    v = torch.from_numpy(rng.standard_normal((B, h, S, 64)).astype(np.float32)).to(dtype)
+    mask = None
+    if lens is not None:
+        mask = np.zeros((B, S), np.float32)
+        for b, l in enumerate(lens):
+            mask[b, l:] = -np.inf
+    o = ops()
+    kv = None if lens is None else dev(np.asarray(lens, np.int32))
+    add_mask = None
+    if with_mask:  # TNN-style additive padding mask (0 / -10000) given as data
+        add_mask = np.where(np.isinf(mask), np.float32(-10000.0), np.float32(0)) if mask is not None else None
+    got = host(o.attention(q.cuda(), k.cuda(), v.cuda(), 0.125, mask=None if add_mask is None else dev(add_mask),
+                           kv_len=kv))
+    ref = orc.attention_core(q.float().numpy(), k.float().numpy(), v.float().numpy(), 0.125,
+                             add_mask if with_mask else mask)
+    return got, ref
+
+
+@pytest.mark.parametrize("B,h,S", [(1, 1, 32), (1, 12, 128), (2, 3, 200), (2, 2, 384), (1, 2, 65), (1, 1, 1)])
+def test_attention_fp16_full(B, h, S):
+    say("attention fp16 B=%d h=%d S=%d" % (B, h, S))
+    got, ref = _attn_case(B, h, S, None, seed=S)
+    assert rel_err(got, ref) <= FP16_TOL
+
+
+def test_attention_fp16_varlen():
+    say("attention fp16 variable lengths")
+    lens = [16, 512, 100, 257, 64, 1, 333, 480]
+    got, ref = _attn_case(8, 2, 512, lens, seed=99)
+    assert rel_err(got, ref) <= FP16_TOL
+    # the same padding expressed the TNN way: additive -10000 mask + kv_len hint
+    got2, ref2 = _attn_case(8, 2, 512, lens, seed=99, with_mask=True)
+    assert rel_err(got2, ref2) <= FP16_TOL
+    assert rel_err(got2, got) <= 1e-6
+
+
+def test_attention_fp16_128row_blocks():
+    # enough (batch, head, query-block) work that the launcher picks the 4-wave / 128-row variant
+    say("attention fp16 4-wave variant")
+    rng = np.random.default_rng(7)
+    lens = rng.integers(16, 513, 8).tolist()
+    got, ref = _attn_case(8, 16, 512, lens, seed=123)
+    assert rel_err(got, ref) <= FP16_TOL
+
+
+def test_attention_bf16():
+    say("attention bf16")
+    got, ref = _attn_case(2, 4, 192, [192, 77], seed=5, dtype=torch.bfloat16)
+    assert rel_err(got, ref) <= 3e-2
+
+
+def test_attention_packed_qkv_layout():
+    say("attention packed [T,3H]")
+    B, S, h = 2, 96, 12
+    H = h * 64
+    rng = np.random.default_rng(31)
+    qkv = torch.from_numpy(rng.standard_normal((B * S, 3 * H)).astype(np.float32)).half()
+    lens = np.array([96, 50], np.int32)
+    out = host(ops().attention_packed(qkv.cuda(), B, S, h, 0.125, kv_len=dev(lens)))
+    x = qkv.float().numpy().reshape(B, S, 3, h, 64)
+    q, k, v = (np.ascontiguousarray(x[:, :, i].transpose(0, 2, 1, 3)) for i in range(3))
+    mask = np.zeros((B, S), np.float32)
+    mask[1, 50:] = -np.inf
+    ref = orc.attention_core(q, k, v, 0.125, mask).transpose(0, 2, 1, 3).reshape(B * S, H)
+    assert rel_err(out, ref) <= FP16_TOL
+
+
+def test_mask_to_kv_len():
+    say("mask_to_kv_len")
+    m = np.zeros((5, 300), np.float32)
+    lens = [300, 1, 64, 65, 299]
+    for b, l in enumerate(lens):
+        m[b, l:] = -10000.0
+    got = host(ops().mask_to_kv_len(dev(m)))
+    assert got.tolist() == lens
+
+
+def test_attention_rejects_bad_args():
+    from tnn_amd import capi
+    q = torch.zeros(1, 1, 8, 32, dtype=torch.float16, device="cuda")
+    with pytest.raises(capi.TnnRocmError):
+        ops().attention(q, q, q, 1.0)  # head_dim 32 is not implemented

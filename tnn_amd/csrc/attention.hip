@@ -1,0 +1,345 @@
+// Fused attention core for gfx950: out = softmax(Q K^T * scale + mask) V, head_dim 64, fp16/bf16
+// inputs with fp32 accumulation and an online (running max / running sum) softmax, so the
+// [B*h, S, S] score tensor of the decomposed graph never exists in memory.
+//
+// Work split: one workgroup = one (batch, head, block of NW*32 query rows); each 64-lane wave owns
+// 32 query rows.  Keys/values are walked in tiles of 64 keys staged in LDS (double buffered, the
+// next tile's global loads are in flight during the current tile's MFMAs).
+//
+// The scores are computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16: in the 32x32
+// accumulator layout a lane then holds ONE query column (lane % 32) and 16 of the 32 keys of the
+// block, so the row max / row sum of the softmax are 16 in-register operations plus a single
+// exchange with lane^32, and the rescale factor of the running output is a per-lane scalar.
+// The probabilities are already in the register order the second MFMA wants for its B operand
+// (O^T = V^T P^T): slot e of lane-half g of a 16-key step maps to key
+//     16*step + 4*g + e        (e < 4)      and      16*step + 8 + 4*g + (e-4)   (e >= 4),
+// so V is stored transposed in LDS ([d][key]) and each lane fetches its two 4-key groups with two
+// 8-byte reads.  Padding keys (>= kv_len) are excluded exactly (−inf) in-register and whole tiles
+// past kv_len are never loaded.
+#include "common.h"
+
+using namespace tnn_rocm;
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kD        = 64;            // head dim
+constexpr int kTileKV   = 64;            // keys per LDS tile
+constexpr int kRowBytes = kD * 2 + 16;   // padded LDS row (K: one key's 64 halfs; V^T: one d's 64 keys)
+constexpr float kLog2e  = 1.4426950408889634f;
+
+template <int DT> struct AttnT;
+template <> struct AttnT<TNN_ROCM_F16> {
+    static __device__ __forceinline__ void mma(const uint4 &a, const uint4 &b, f32x16 &c) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
+                                                   0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        half_t l = (half_t)lo, h = (half_t)hi;
+        return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+    }
+};
+template <> struct AttnT<TNN_ROCM_BF16> {
+    static __device__ __forceinline__ void mma(const uint4 &a, const uint4 &b, f32x16 &c) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                    0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+    }
+};
+
+struct AttnParams {
+    const uint16_t *q, *k, *v;
+    uint16_t *o;
+    long q_sb, q_sh, q_ss, kv_sb, kv_sh, kv_ss, o_sb, o_sh, o_ss;
+    int S;
+    float scale_log2e;  // scale * log2(e)
+    const float *mask;  // [B,S] additive or null
+    const int32_t *kv_len;
+};
+
+template <int DT, int NW>
+__global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
+    constexpr int NT = NW * 64;
+    constexpr int BQ = NW * 32;
+    // per tile: 64 keys x 8 sixteen-byte chunks
+    constexpr int KV_VECS = kTileKV * 8 / NT;
+    static_assert(kTileKV * 8 % NT == 0, "tile must divide over the workgroup");
+
+    __shared__ __attribute__((aligned(16))) unsigned char lds_k[2][kTileKV * kRowBytes];
+    __shared__ __attribute__((aligned(16))) unsigned char lds_vt[2][kD * kRowBytes];
+    __shared__ __attribute__((aligned(16))) float lds_bias[2][kTileKV];
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int g    = lane >> 5;  // lane half
+    const int lq   = lane & 31;  // query column owned by this lane
+    const int b    = blockIdx.z;
+    const int head = blockIdx.y;
+    const int q0   = blockIdx.x * BQ + wave * 32;
+    const int S    = p.S;
+
+    int kv_end = S;
+    if (p.kv_len) {
+        int l  = p.kv_len[b];
+        kv_end = l < 0 ? 0 : (l < S ? l : S);
+    }
+    const int n_tiles = (kv_end + kTileKV - 1) / kTileKV;
+
+    const uint16_t *qb = p.q + (size_t)b * p.q_sb + (size_t)head * p.q_sh;
+    const uint16_t *kb = p.k + (size_t)b * p.kv_sb + (size_t)head * p.kv_sh;
+    const uint16_t *vb = p.v + (size_t)b * p.kv_sb + (size_t)head * p.kv_sh;
+    uint16_t *ob       = p.o + (size_t)b * p.o_sb + (size_t)head * p.o_sh;
+    const float *mb    = p.mask ? p.mask + (size_t)b * S : nullptr;
+
+    // Q fragments (B operand of S^T = K Q^T): lane (lq, g) holds Q[q0+lq][16*kk + 8*g .. +7]
+    uint4 qf[4];
+    {
+        int qrow = q0 + lq;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            qf[kk] = make_uint4(0, 0, 0, 0);
+            if (qrow < S)
+                qf[kk] = *reinterpret_cast<const uint4 *>(qb + (size_t)qrow * p.q_ss + kk * 16 + g * 8);
+        }
+    }
+
+    uint4 rk[KV_VECS], rv[KV_VECS];
+    float rbias = 0.f;
+
+    auto load_tile = [&](int t) {
+        int kv0 = t * kTileKV;
+#pragma unroll
+        for (int i = 0; i < KV_VECS; ++i) {
+            int v   = tid + i * NT;
+            int key = kv0 + (v >> 3), ch = v & 7;
+            rk[i] = make_uint4(0, 0, 0, 0);
+            rv[i] = make_uint4(0, 0, 0, 0);
+            if (key < kv_end) {
+                rk[i] = *reinterpret_cast<const uint4 *>(kb + (size_t)key * p.kv_ss + ch * 8);
+                rv[i] = *reinterpret_cast<const uint4 *>(vb + (size_t)key * p.kv_ss + ch * 8);
+            }
+        }
+        if (tid < kTileKV) {
+            int key = kv0 + tid;
+            rbias   = key < kv_end ? (mb ? mb[key] * kLog2e : 0.f) : -INFINITY;
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < KV_VECS; ++i) {
+            int v   = tid + i * NT;
+            int key = v >> 3, ch = v & 7;
+            *reinterpret_cast<uint4 *>(&lds_k[buf][key * kRowBytes + ch * 16]) = rk[i];
+            const uint16_t *e = reinterpret_cast<const uint16_t *>(&rv[i]);
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                *reinterpret_cast<uint16_t *>(&lds_vt[buf][(ch * 8 + t) * kRowBytes + key * 2]) = e[t];
+        }
+        if (tid < kTileKV)
+            lds_bias[buf][tid] = rbias;
+    };
+
+    f32x16 oacc[2];
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            oacc[dt][r] = 0.f;
+    float m_i = -INFINITY, l_i = 0.f;
+
+    if (n_tiles > 0) {
+        load_tile(0);
+        store_tile(0);
+    }
+    __syncthreads();
+
+    for (int t = 0; t < n_tiles; ++t) {
+        const int buf = t & 1;
+        if (t + 1 < n_tiles)
+            load_tile(t + 1);
+
+        // ---- S^T = K Q^T for the 64 keys of the tile: two 32-key blocks
+        f32x16 sacc[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                sacc[kt][r] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                uint4 kf =
+                    *reinterpret_cast<const uint4 *>(&lds_k[buf][(kt * 32 + lq) * kRowBytes + kk * 32 + g * 16]);
+                AttnT<DT>::mma(kf, qf[kk], sacc[kt]);
+            }
+        }
+
+        // ---- online softmax; register r of block kt is key kt*32 + 8*(r/4) + 4*g + (r%4)
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                float4 bias = *reinterpret_cast<const float4 *>(&lds_bias[buf][kt * 32 + r4 * 8 + g * 4]);
+                float bv[4] = {bias.x, bias.y, bias.z, bias.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float s2             = sacc[kt][r4 * 4 + e] * p.scale_log2e + bv[e];
+                    sacc[kt][r4 * 4 + e] = s2;
+                    mx                   = fmaxf(mx, s2);
+                }
+            }
+        }
+        mx          = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        float m_new = fmaxf(m_i, mx);
+        float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
+        float rs    = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float pv    = __builtin_amdgcn_exp2f(sacc[kt][r] - m_use);
+                sacc[kt][r] = pv;
+                rs += pv;
+            }
+        rs += __shfl_xor(rs, 32, 64);
+        l_i = l_i * alpha + rs;
+        m_i = m_new;
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                oacc[dt][r] *= alpha;
+
+        // ---- O^T += V^T P^T : four 16-key steps
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            const int kt = st >> 1, j = st & 1;
+            uint4 pf;
+            pf.x = AttnT<DT>::pack2(sacc[kt][8 * j + 0], sacc[kt][8 * j + 1]);
+            pf.y = AttnT<DT>::pack2(sacc[kt][8 * j + 2], sacc[kt][8 * j + 3]);
+            pf.z = AttnT<DT>::pack2(sacc[kt][8 * j + 4], sacc[kt][8 * j + 5]);
+            pf.w = AttnT<DT>::pack2(sacc[kt][8 * j + 6], sacc[kt][8 * j + 7]);
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt) {
+                const unsigned char *row = &lds_vt[buf][(dt * 32 + lq) * kRowBytes + (st * 16 + g * 4) * 2];
+                uint2 lo                 = *reinterpret_cast<const uint2 *>(row);
+                uint2 hi                 = *reinterpret_cast<const uint2 *>(row + 16);
+                uint4 vf                 = make_uint4(lo.x, lo.y, hi.x, hi.y);
+                AttnT<DT>::mma(vf, pf, oacc[dt]);
+            }
+        }
+
+        if (t + 1 < n_tiles)
+            store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- normalise and store: lane owns query row q0+lq; register r of block dt is
+    //      d = dt*32 + 8*(r/4) + 4*g + (r%4)  -> four consecutive d per register group
+    const int qrow = q0 + lq;
+    if (qrow < S) {
+        float inv = l_i > 0.f ? 1.0f / l_i : 0.f;
+        uint16_t *orow = ob + (size_t)qrow * p.o_ss;
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                uint2 w;
+                w.x = AttnT<DT>::pack2(oacc[dt][r4 * 4 + 0] * inv, oacc[dt][r4 * 4 + 1] * inv);
+                w.y = AttnT<DT>::pack2(oacc[dt][r4 * 4 + 2] * inv, oacc[dt][r4 * 4 + 3] * inv);
+                *reinterpret_cast<uint2 *>(orow + dt * 32 + r4 * 8 + g * 4) = w;
+            }
+    }
+}
+
+__global__ void mask_to_kv_len_kernel(const float *__restrict__ mask, int32_t *__restrict__ kv_len, int S,
+                                      float threshold) {
+    // one wave per batch row: the largest index whose mask value is above the threshold
+    const int b    = blockIdx.x;
+    const int lane = threadIdx.x;
+    int last       = -1;
+    for (int j = lane; j < S; j += 64)
+        if (mask[(size_t)b * S + j] > threshold)
+            last = j;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        int other = __shfl_xor(last, o, 64);
+        last      = other > last ? other : last;
+    }
+    if (lane == 0)
+        kv_len[b] = last + 1;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tnn_rocm_attention(void *stream, int dtype, const void *q, const void *k, const void *v, void *out, int B,
+                       int heads, int S, int head_dim, long q_sb, long q_sh, long q_ss, long kv_sb, long kv_sh,
+                       long kv_ss, long o_sb, long o_sh, long o_ss, float scale, const float *mask,
+                       const int32_t *kv_len) {
+    TR_REQUIRE(B >= 0 && heads >= 0 && S >= 0, TNN_ROCM_ESHAPE, "attention: negative size");
+    if (B == 0 || heads == 0 || S == 0)
+        return 0;
+    TR_REQUIRE(q && k && v && out, TNN_ROCM_EINVAL, "attention: null pointer");
+    TR_REQUIRE(head_dim == kD, TNN_ROCM_ESHAPE, "attention: head_dim %d unsupported (64 only)", head_dim);
+    TR_REQUIRE(dtype == TNN_ROCM_F16 || dtype == TNN_ROCM_BF16, TNN_ROCM_EDTYPE,
+               "attention: dtype %d unsupported (F16 or BF16)", dtype);
+    TR_REQUIRE(B <= 65535 && heads <= 65535, TNN_ROCM_ESHAPE, "attention: batch/heads exceed the grid limit");
+    auto ok = [](const void *ptr, long a, long b2, long c) {
+        return ((((uintptr_t)ptr) & 15u) == 0) && a % 8 == 0 && b2 % 8 == 0 && c % 8 == 0;
+    };
+    TR_REQUIRE(ok(q, q_sb, q_sh, q_ss) && ok(k, kv_sb, kv_sh, kv_ss) && ok(v, kv_sb, kv_sh, kv_ss) &&
+                   ok(out, o_sb, o_sh, o_ss),
+               TNN_ROCM_EALIGN, "attention: pointers must be 16-byte aligned and strides multiples of 8 elements");
+    TR_REQUIRE(q_ss >= kD && kv_ss >= kD && o_ss >= kD, TNN_ROCM_ESHAPE, "attention: row stride below head_dim");
+    AttnParams p;
+    p.q = (const uint16_t *)q;
+    p.k = (const uint16_t *)k;
+    p.v = (const uint16_t *)v;
+    p.o = (uint16_t *)out;
+    p.q_sb = q_sb, p.q_sh = q_sh, p.q_ss = q_ss;
+    p.kv_sb = kv_sb, p.kv_sh = kv_sh, p.kv_ss = kv_ss;
+    p.o_sb = o_sb, p.o_sh = o_sh, p.o_ss = o_ss;
+    p.S           = S;
+    p.scale_log2e = scale * kLog2e;
+    p.mask        = mask;
+    p.kv_len      = kv_len;
+    hipStream_t s = (hipStream_t)stream;
+    // 128-row query blocks when that already gives >= 2 workgroups per CU, else 64-row blocks
+    long blocks128 = (long)((S + 127) / 128) * heads * B;
+    if (blocks128 >= 512) {
+        dim3 grid((S + 127) / 128, heads, B);
+        if (dtype == TNN_ROCM_F16)
+            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_F16, 4>), grid, dim3(256), 0, s, p);
+        else
+            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_BF16, 4>), grid, dim3(256), 0, s, p);
+    } else {
+        dim3 grid((S + 63) / 64, heads, B);
+        if (dtype == TNN_ROCM_F16)
+            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_F16, 2>), grid, dim3(128), 0, s, p);
+        else
+            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_BF16, 2>), grid, dim3(128), 0, s, p);
+    }
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_t *kv_len, int B, int S, float threshold) {
+    TR_REQUIRE(B >= 0 && S >= 0, TNN_ROCM_ESHAPE, "mask_to_kv_len: negative size");
+    if (B == 0)
+        return 0;
+    TR_REQUIRE(mask && kv_len, TNN_ROCM_EINVAL, "mask_to_kv_len: null pointer");
+    hipLaunchKernelGGL(mask_to_kv_len_kernel, dim3(B), dim3(64), 0, (hipStream_t)stream, mask, kv_len, S, threshold);
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+}  // extern "C"

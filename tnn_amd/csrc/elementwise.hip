@@ -1,0 +1,549 @@
+// HBM-bound element-wise kernels: GELU, broadcast binary ops, permute, gather, casts and the
+// int8 boundary ops (quantize / dequantize / int8 add / int8 GELU).
+//
+// All kernels move 16 bytes per lane per access where the pointers allow it, with a grid-stride
+// loop over enough workgroups to cover the 256 CUs several times.
+#include "common.h"
+
+using namespace tnn_rocm;
+
+namespace {
+
+constexpr int kBlock     = 256;
+constexpr int kMaxBlocks = 256 * 16;
+
+inline int grid_for(size_t work_items) {
+    size_t b = (work_items + kBlock - 1) / kBlock;
+    if (b < 1)
+        b = 1;
+    if (b > (size_t)kMaxBlocks)
+        b = kMaxBlocks;
+    return (int)b;
+}
+
+inline bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+
+// ---- generic unary map over a float dtype, VEC elements (16 bytes) per lane -------------------
+template <int DT, typename F>
+__global__ void __launch_bounds__(kBlock) unary_vec_kernel(const typename Elem<DT>::type *__restrict__ x,
+                                                           typename Elem<DT>::type *__restrict__ y, size_t n, F f) {
+    typedef typename Elem<DT>::type T;
+    constexpr int VEC = 16 / sizeof(T);
+    size_t nvec       = n / VEC;
+    size_t stride     = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) {
+        uint4 raw = reinterpret_cast<const uint4 *>(x)[i];
+        T *e      = reinterpret_cast<T *>(&raw);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            Elem<DT>::st(&e[j], f(Elem<DT>::ld(&e[j])));
+        reinterpret_cast<uint4 *>(y)[i] = raw;
+    }
+    // tail
+    size_t t = nvec * VEC + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < n)
+        Elem<DT>::st(&y[t], f(Elem<DT>::ld(&x[t])));
+}
+
+template <int DT, typename F>
+__global__ void __launch_bounds__(kBlock) unary_scalar_kernel(const typename Elem<DT>::type *__restrict__ x,
+                                                              typename Elem<DT>::type *__restrict__ y, size_t n, F f) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        Elem<DT>::st(&y[i], f(Elem<DT>::ld(&x[i])));
+}
+
+struct GeluOp {
+    __device__ __forceinline__ float operator()(float v) const { return gelu_erf(v); }
+};
+
+template <int DT, typename F>
+int launch_unary(hipStream_t s, const void *x, void *y, size_t n, F f) {
+    typedef typename Elem<DT>::type T;
+    constexpr int VEC = 16 / sizeof(T);
+    if (aligned16(x) && aligned16(y)) {
+        // the tail is handled by the first (n % VEC) lanes of the grid, so the grid must hold them
+        hipLaunchKernelGGL((unary_vec_kernel<DT, F>), dim3(grid_for(n / VEC + VEC)), dim3(kBlock), 0, s, (const T *)x,
+                           (T *)y, n, f);
+    } else {
+        hipLaunchKernelGGL((unary_scalar_kernel<DT, F>), dim3(grid_for(n)), dim3(kBlock), 0, s, (const T *)x, (T *)y,
+                           n, f);
+    }
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+// ---- broadcast binary -----------------------------------------------------------------------
+struct BcastDesc {
+    int rank;
+    int out_dim[6];
+    long a_stride[6];  // 0 where the operand broadcasts along the axis
+    long b_stride[6];
+};
+
+template <int DT, int OP>
+__global__ void __launch_bounds__(kBlock) binary_bcast_kernel(const typename Elem<DT>::type *__restrict__ a,
+                                                              const typename Elem<DT>::type *__restrict__ b,
+                                                              typename Elem<DT>::type *__restrict__ out, size_t n,
+                                                              BcastDesc d) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        size_t rem = i;
+        long oa = 0, ob = 0;
+#pragma unroll
+        for (int ax = 5; ax >= 0; --ax) {
+            if (ax < d.rank) {
+                int idx = (int)(rem % (size_t)d.out_dim[ax]);
+                rem /= (size_t)d.out_dim[ax];
+                oa += idx * d.a_stride[ax];
+                ob += idx * d.b_stride[ax];
+            }
+        }
+        float va = Elem<DT>::ld(&a[oa]);
+        float vb = Elem<DT>::ld(&b[ob]);
+        float r;
+        if (OP == 0)
+            r = __fadd_rn(va, vb);
+        else if (OP == 1)
+            r = __fsub_rn(va, vb);
+        else if (OP == 2)
+            r = __fmul_rn(va, vb);
+        else
+            r = __fdiv_rn(va, vb);
+        Elem<DT>::st(&out[i], r);
+    }
+}
+
+// Fast path: b is a vector over the last axis (bias add, gamma scale) or a scalar, a and out
+// have the same shape.  16 bytes per lane.
+template <int DT, int OP>
+__global__ void __launch_bounds__(kBlock) binary_lastaxis_kernel(const typename Elem<DT>::type *__restrict__ a,
+                                                                 const typename Elem<DT>::type *__restrict__ b,
+                                                                 typename Elem<DT>::type *__restrict__ out,
+                                                                 size_t nvec, int cols_vec, int b_is_scalar,
+                                                                 int b_is_full) {
+    typedef typename Elem<DT>::type T;
+    constexpr int VEC = 16 / sizeof(T);
+    size_t stride     = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) {
+        uint4 ra = reinterpret_cast<const uint4 *>(a)[i];
+        T *ea    = reinterpret_cast<T *>(&ra);
+        uint4 rb;
+        T *eb = reinterpret_cast<T *>(&rb);
+        if (b_is_full) {
+            rb = reinterpret_cast<const uint4 *>(b)[i];
+        } else if (!b_is_scalar) {
+            rb = reinterpret_cast<const uint4 *>(b)[i % (size_t)cols_vec];
+        }
+        float sb = b_is_scalar ? Elem<DT>::ld(&b[0]) : 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            float va = Elem<DT>::ld(&ea[j]);
+            float vb = b_is_scalar ? sb : Elem<DT>::ld(&eb[j]);
+            float r;
+            if (OP == 0)
+                r = __fadd_rn(va, vb);
+            else if (OP == 1)
+                r = __fsub_rn(va, vb);
+            else if (OP == 2)
+                r = __fmul_rn(va, vb);
+            else
+                r = __fdiv_rn(va, vb);
+            Elem<DT>::st(&ea[j], r);
+        }
+        reinterpret_cast<uint4 *>(out)[i] = ra;
+    }
+}
+
+template <int DT>
+int launch_binary(hipStream_t s, int op, const void *a, const void *b, void *out, size_t n, const BcastDesc &d,
+                  int fast_kind, int cols) {
+    typedef typename Elem<DT>::type T;
+    constexpr int VEC = 16 / sizeof(T);
+    bool fast = fast_kind != 0 && aligned16(a) && aligned16(out) && (n % VEC) == 0 &&
+                (fast_kind == 2 || (aligned16(b) && (fast_kind == 3 || cols % VEC == 0)));
+#define TR_BIN_CASE(OPV)                                                                                              \
+    case OPV:                                                                                                         \
+        if (fast)                                                                                                     \
+            hipLaunchKernelGGL((binary_lastaxis_kernel<DT, OPV>), dim3(grid_for(n / VEC)), dim3(kBlock), 0, s,        \
+                               (const T *)a, (const T *)b, (T *)out, n / VEC, cols / VEC > 0 ? cols / VEC : 1,        \
+                               fast_kind == 2 ? 1 : 0, fast_kind == 3 ? 1 : 0);                                       \
+        else                                                                                                          \
+            hipLaunchKernelGGL((binary_bcast_kernel<DT, OPV>), dim3(grid_for(n)), dim3(kBlock), 0, s, (const T *)a,   \
+                               (const T *)b, (T *)out, n, d);                                                         \
+        break;
+    switch (op) {
+        TR_BIN_CASE(0)
+        TR_BIN_CASE(1)
+        TR_BIN_CASE(2)
+        TR_BIN_CASE(3)
+        default:
+            set_error("binary: unknown op %d", op);
+            return TNN_ROCM_EINVAL;
+    }
+#undef TR_BIN_CASE
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+// ---- permute -----------------------------------------------------------------------------------
+struct PermDesc {
+    int rank;
+    int out_dim[6];
+    long in_stride_of_out_axis[6];
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) permute_kernel(const T *__restrict__ in, T *__restrict__ out, size_t n,
+                                                         PermDesc d) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        size_t rem = i;
+        long src   = 0;
+#pragma unroll
+        for (int ax = 5; ax >= 0; --ax) {
+            if (ax < d.rank) {
+                int idx = (int)(rem % (size_t)d.out_dim[ax]);
+                rem /= (size_t)d.out_dim[ax];
+                src += idx * d.in_stride_of_out_axis[ax];
+            }
+        }
+        out[i] = in[src];
+    }
+}
+
+// ---- gather --------------------------------------------------------------------------------------
+// one workgroup per output row; rows are copied in 4-byte words when the slice size allows it.
+__global__ void __launch_bounds__(kBlock) gather_kernel(const char *__restrict__ data, const int32_t *__restrict__ idx,
+                                                        char *__restrict__ out, int slices, size_t slice_bytes,
+                                                        int n_indices, int32_t *error_flag) {
+    int row   = blockIdx.x;  // b * n_indices + i
+    int b     = row / n_indices;
+    int i     = row - b * n_indices;
+    int s     = idx[i];
+    if (s < 0)
+        s += slices;
+    bool bad        = (s < 0 || s >= slices);
+    const char *src = data + ((size_t)b * slices + (bad ? 0 : s)) * slice_bytes;
+    char *dst       = out + (size_t)row * slice_bytes;
+    if (bad && threadIdx.x == 0 && error_flag)
+        *error_flag = 1;
+    if ((slice_bytes & 3) == 0 && ((((uintptr_t)src) | ((uintptr_t)dst)) & 3) == 0) {
+        size_t words = slice_bytes >> 2;
+        for (size_t w = threadIdx.x; w < words; w += blockDim.x)
+            reinterpret_cast<uint32_t *>(dst)[w] = bad ? 0u : reinterpret_cast<const uint32_t *>(src)[w];
+    } else {
+        for (size_t w = threadIdx.x; w < slice_bytes; w += blockDim.x)
+            dst[w] = bad ? 0 : src[w];
+    }
+}
+
+// ---- casts ---------------------------------------------------------------------------------------
+template <int SDT, int DDT>
+__global__ void __launch_bounds__(kBlock) cast_kernel(const typename Elem<SDT>::type *__restrict__ x,
+                                                      typename Elem<DDT>::type *__restrict__ y, size_t n) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t n4     = n / 4;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            Elem<DDT>::st(&y[i * 4 + j], Elem<SDT>::ld(&x[i * 4 + j]));
+    }
+    size_t t = n4 * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < n)
+        Elem<DDT>::st(&y[t], Elem<SDT>::ld(&x[t]));
+}
+
+// ---- int8 boundary ops -----------------------------------------------------------------------------
+template <int DT>
+__global__ void __launch_bounds__(kBlock) quantize_kernel(const typename Elem<DT>::type *__restrict__ x, float inv,
+                                                          int8_t *__restrict__ q, size_t n) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t n4     = n / 4;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+        char4 o;
+        o.x = float2int8_ref(__fmul_rn(Elem<DT>::ld(&x[i * 4 + 0]), inv));
+        o.y = float2int8_ref(__fmul_rn(Elem<DT>::ld(&x[i * 4 + 1]), inv));
+        o.z = float2int8_ref(__fmul_rn(Elem<DT>::ld(&x[i * 4 + 2]), inv));
+        o.w = float2int8_ref(__fmul_rn(Elem<DT>::ld(&x[i * 4 + 3]), inv));
+        if ((((uintptr_t)q) & 3) == 0) {
+            reinterpret_cast<char4 *>(q)[i] = o;
+        } else {
+            q[i * 4 + 0] = o.x;
+            q[i * 4 + 1] = o.y;
+            q[i * 4 + 2] = o.z;
+            q[i * 4 + 3] = o.w;
+        }
+    }
+    size_t t = n4 * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < n)
+        q[t] = float2int8_ref(__fmul_rn(Elem<DT>::ld(&x[t]), inv));
+}
+
+template <int DT>
+__global__ void __launch_bounds__(kBlock) dequantize_kernel(const int8_t *__restrict__ q, float scale,
+                                                            typename Elem<DT>::type *__restrict__ x, size_t n) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        Elem<DT>::st(&x[i], __fmul_rn((float)q[i], scale));
+}
+
+__global__ void __launch_bounds__(kBlock) add_i8_kernel(const int8_t *__restrict__ a, float sa,
+                                                        const int8_t *__restrict__ b, float sb, float inv_so,
+                                                        int8_t *__restrict__ y, size_t n) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        float pa = __fmul_rn((float)a[i], sa);
+        float pb = __fmul_rn((float)b[i], sb);
+        float s  = __fadd_rn(pa, pb);
+        y[i]     = float2int8_ref(__fmul_rn(s, inv_so));
+    }
+}
+
+__global__ void __launch_bounds__(kBlock) gelu_i8_kernel(const int8_t *__restrict__ qi, float in_scale,
+                                                         float out_inv, int8_t *__restrict__ qo, size_t n) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        float x = __fmul_rn((float)qi[i], in_scale);
+        float g = gelu_erf(x);
+        qo[i]   = float2int8_ref(__fmul_rn(g, out_inv));
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int tnn_rocm_gelu(void *stream, int dtype, const void *x, void *y, size_t count) {
+    if (count == 0)
+        return 0;
+    TR_REQUIRE(x && y, TNN_ROCM_EINVAL, "gelu: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case TNN_ROCM_F32: return launch_unary<TNN_ROCM_F32>(s, x, y, count, GeluOp());
+        case TNN_ROCM_F16: return launch_unary<TNN_ROCM_F16>(s, x, y, count, GeluOp());
+        case TNN_ROCM_BF16: return launch_unary<TNN_ROCM_BF16>(s, x, y, count, GeluOp());
+        default: set_error("gelu: unsupported dtype %d", dtype); return TNN_ROCM_EDTYPE;
+    }
+}
+
+int tnn_rocm_binary(void *stream, int dtype, int op, const void *a, const int *sa, int ra, const void *b,
+                    const int *sb, int rb, void *out, const int *so, int ro) {
+    TR_REQUIRE(a && b && out && sa && sb && so, TNN_ROCM_EINVAL, "binary: null pointer");
+    TR_REQUIRE(ro >= 1 && ro <= 6 && ra >= 0 && ra <= ro && rb >= 0 && rb <= ro, TNN_ROCM_ESHAPE,
+               "binary: ranks a=%d b=%d out=%d unsupported (max 6, operands may not exceed the output rank)", ra, rb,
+               ro);
+    BcastDesc d;
+    d.rank   = ro;
+    size_t n = 1;
+    for (int i = 0; i < 6; ++i) {
+        d.out_dim[i]  = 1;
+        d.a_stride[i] = 0;
+        d.b_stride[i] = 0;
+    }
+    for (int i = 0; i < ro; ++i) {
+        TR_REQUIRE(so[i] >= 0, TNN_ROCM_ESHAPE, "binary: negative dim");
+        d.out_dim[i] = so[i];
+        n *= (size_t)so[i];
+    }
+    if (n == 0)
+        return 0;
+    // right-aligned strides; an operand dim of 1 (or smaller than the output) broadcasts.
+    auto fill = [&](const int *shape, int rank, long *stride) -> bool {
+        long acc = 1;
+        for (int i = rank - 1; i >= 0; --i) {
+            int oi = i + (ro - rank);
+            if (shape[i] == so[oi])
+                stride[oi] = acc;
+            else if (shape[i] == 1)
+                stride[oi] = 0;
+            else
+                return false;
+            acc *= shape[i];
+        }
+        return true;
+    };
+    TR_REQUIRE(fill(sa, ra, d.a_stride) && fill(sb, rb, d.b_stride), TNN_ROCM_ESHAPE,
+               "binary: operand shape does not broadcast to the output shape");
+    // classify the fast cases: a has the full output shape and b is scalar / last-axis vector / full.
+    size_t na = 1, nb = 1;
+    for (int i = 0; i < ra; ++i)
+        na *= (size_t)sa[i];
+    for (int i = 0; i < rb; ++i)
+        nb *= (size_t)sb[i];
+    int fast_kind = 0, cols = so[ro - 1];
+    if (na == n) {
+        if (nb == 1)
+            fast_kind = 2;
+        else if (nb == n)
+            fast_kind = 3;
+        else if (nb == (size_t)cols && rb >= 1 && sb[rb - 1] == cols)
+            fast_kind = 1;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case TNN_ROCM_F32: return launch_binary<TNN_ROCM_F32>(s, op, a, b, out, n, d, fast_kind, cols);
+        case TNN_ROCM_F16: return launch_binary<TNN_ROCM_F16>(s, op, a, b, out, n, d, fast_kind, cols);
+        case TNN_ROCM_BF16: return launch_binary<TNN_ROCM_BF16>(s, op, a, b, out, n, d, fast_kind, cols);
+        default: set_error("binary: unsupported dtype %d", dtype); return TNN_ROCM_EDTYPE;
+    }
+}
+
+int tnn_rocm_permute(void *stream, int elem_bytes, const void *in, void *out, const int *in_dims, const int *order,
+                     int rank) {
+    TR_REQUIRE(in && out && in_dims && order, TNN_ROCM_EINVAL, "permute: null pointer");
+    TR_REQUIRE(rank >= 1 && rank <= 6, TNN_ROCM_ESHAPE, "permute: rank %d unsupported (1..6)", rank);
+    long in_stride[6];
+    size_t n = 1;
+    bool seen[6] = {false, false, false, false, false, false};
+    for (int i = rank - 1; i >= 0; --i) {
+        TR_REQUIRE(in_dims[i] >= 0, TNN_ROCM_ESHAPE, "permute: negative dim");
+        in_stride[i] = (long)n;
+        n *= (size_t)in_dims[i];
+    }
+    PermDesc d;
+    d.rank = rank;
+    for (int j = 0; j < 6; ++j) {
+        d.out_dim[j]               = 1;
+        d.in_stride_of_out_axis[j] = 0;
+    }
+    for (int j = 0; j < rank; ++j) {
+        TR_REQUIRE(order[j] >= 0 && order[j] < rank && !seen[order[j]], TNN_ROCM_EINVAL,
+                   "permute: order is not a permutation");
+        seen[order[j]]             = true;
+        d.out_dim[j]               = in_dims[order[j]];
+        d.in_stride_of_out_axis[j] = in_stride[order[j]];
+    }
+    if (n == 0)
+        return 0;
+    hipStream_t s = (hipStream_t)stream;
+    switch (elem_bytes) {
+        case 1:
+            hipLaunchKernelGGL(permute_kernel<uint8_t>, dim3(grid_for(n)), dim3(kBlock), 0, s, (const uint8_t *)in,
+                               (uint8_t *)out, n, d);
+            break;
+        case 2:
+            hipLaunchKernelGGL(permute_kernel<uint16_t>, dim3(grid_for(n)), dim3(kBlock), 0, s, (const uint16_t *)in,
+                               (uint16_t *)out, n, d);
+            break;
+        case 4:
+            hipLaunchKernelGGL(permute_kernel<uint32_t>, dim3(grid_for(n)), dim3(kBlock), 0, s, (const uint32_t *)in,
+                               (uint32_t *)out, n, d);
+            break;
+        default: set_error("permute: element size %d unsupported", elem_bytes); return TNN_ROCM_EDTYPE;
+    }
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+int tnn_rocm_gather(void *stream, const void *data, const int32_t *indices, void *out, int batch, int slices,
+                    size_t slice_bytes, int n_indices, int32_t *error_flag) {
+    TR_REQUIRE(batch >= 0 && slices >= 0 && n_indices >= 0, TNN_ROCM_ESHAPE, "gather: negative size");
+    if (batch == 0 || n_indices == 0 || slice_bytes == 0)
+        return 0;
+    TR_REQUIRE(data && indices && out, TNN_ROCM_EINVAL, "gather: null pointer");
+    TR_REQUIRE(slices > 0, TNN_ROCM_ESHAPE, "gather: empty table");
+    TR_REQUIRE((long)batch * n_indices < (1l << 31), TNN_ROCM_ESHAPE, "gather: too many rows");
+    hipLaunchKernelGGL(gather_kernel, dim3(batch * n_indices), dim3(kBlock), 0, (hipStream_t)stream,
+                       (const char *)data, indices, (char *)out, slices, slice_bytes, n_indices, error_flag);
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+int tnn_rocm_cast(void *stream, int sdt, const void *src, int ddt, void *dst, size_t n) {
+    if (n == 0)
+        return 0;
+    TR_REQUIRE(src && dst, TNN_ROCM_EINVAL, "cast: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    int g         = grid_for(n / 4 + 4);
+#define TR_CAST(S, D)                                                                                                 \
+    if (sdt == S && ddt == D) {                                                                                       \
+        hipLaunchKernelGGL((cast_kernel<S, D>), dim3(g), dim3(kBlock), 0, s, (const Elem<S>::type *)src,              \
+                           (Elem<D>::type *)dst, n);                                                                  \
+        TR_CHECK_LAUNCH();                                                                                            \
+        return 0;                                                                                                     \
+    }
+    TR_CAST(TNN_ROCM_F32, TNN_ROCM_F16)
+    TR_CAST(TNN_ROCM_F16, TNN_ROCM_F32)
+    TR_CAST(TNN_ROCM_F32, TNN_ROCM_BF16)
+    TR_CAST(TNN_ROCM_BF16, TNN_ROCM_F32)
+    TR_CAST(TNN_ROCM_F16, TNN_ROCM_BF16)
+    TR_CAST(TNN_ROCM_BF16, TNN_ROCM_F16)
+    TR_CAST(TNN_ROCM_F32, TNN_ROCM_F32)
+    TR_CAST(TNN_ROCM_F16, TNN_ROCM_F16)
+    TR_CAST(TNN_ROCM_BF16, TNN_ROCM_BF16)
+#undef TR_CAST
+    set_error("cast: unsupported dtype pair %d -> %d", sdt, ddt);
+    return TNN_ROCM_EDTYPE;
+}
+
+int tnn_rocm_quantize(void *stream, int sdt, const void *x, float inv_scale, int8_t *q, size_t n) {
+    if (n == 0)
+        return 0;
+    TR_REQUIRE(x && q, TNN_ROCM_EINVAL, "quantize: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    int g         = grid_for(n / 4 + 4);
+    switch (sdt) {
+        case TNN_ROCM_F32:
+            hipLaunchKernelGGL(quantize_kernel<TNN_ROCM_F32>, dim3(g), dim3(kBlock), 0, s, (const float *)x, inv_scale,
+                               q, n);
+            break;
+        case TNN_ROCM_F16:
+            hipLaunchKernelGGL(quantize_kernel<TNN_ROCM_F16>, dim3(g), dim3(kBlock), 0, s, (const half_t *)x,
+                               inv_scale, q, n);
+            break;
+        case TNN_ROCM_BF16:
+            hipLaunchKernelGGL(quantize_kernel<TNN_ROCM_BF16>, dim3(g), dim3(kBlock), 0, s, (const bf16_bits *)x,
+                               inv_scale, q, n);
+            break;
+        default: set_error("quantize: unsupported source dtype %d", sdt); return TNN_ROCM_EDTYPE;
+    }
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+int tnn_rocm_dequantize(void *stream, const int8_t *q, float scale, int ddt, void *x, size_t n) {
+    if (n == 0)
+        return 0;
+    TR_REQUIRE(x && q, TNN_ROCM_EINVAL, "dequantize: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    int g         = grid_for(n);
+    switch (ddt) {
+        case TNN_ROCM_F32:
+            hipLaunchKernelGGL(dequantize_kernel<TNN_ROCM_F32>, dim3(g), dim3(kBlock), 0, s, q, scale, (float *)x, n);
+            break;
+        case TNN_ROCM_F16:
+            hipLaunchKernelGGL(dequantize_kernel<TNN_ROCM_F16>, dim3(g), dim3(kBlock), 0, s, q, scale, (half_t *)x, n);
+            break;
+        case TNN_ROCM_BF16:
+            hipLaunchKernelGGL(dequantize_kernel<TNN_ROCM_BF16>, dim3(g), dim3(kBlock), 0, s, q, scale, (bf16_bits *)x,
+                               n);
+            break;
+        default: set_error("dequantize: unsupported destination dtype %d", ddt); return TNN_ROCM_EDTYPE;
+    }
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+int tnn_rocm_add_i8(void *stream, const int8_t *a, float sa, const int8_t *b, float sb, float inv_so, int8_t *y,
+                    size_t n) {
+    if (n == 0)
+        return 0;
+    TR_REQUIRE(a && b && y, TNN_ROCM_EINVAL, "add_i8: null pointer");
+    hipLaunchKernelGGL(add_i8_kernel, dim3(grid_for(n)), dim3(kBlock), 0, (hipStream_t)stream, a, sa, b, sb, inv_so, y,
+                       n);
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+int tnn_rocm_gelu_i8(void *stream, const int8_t *qi, float in_scale, float out_inv_scale, int8_t *qo, size_t n) {
+    if (n == 0)
+        return 0;
+    TR_REQUIRE(qi && qo, TNN_ROCM_EINVAL, "gelu_i8: null pointer");
+    hipLaunchKernelGGL(gelu_i8_kernel, dim3(grid_for(n)), dim3(kBlock), 0, (hipStream_t)stream, qi, in_scale,
+                       out_inv_scale, qo, n);
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,194 @@
+"""Thin tensor-level wrappers over the C ABI.
+
+torch is used only as plumbing: it owns device memory and the stream.  Every function passes raw
+device pointers into libtnn_rocm.so; there is no torch implementation behind any of them.
+"""
+import torch
+
+from . import capi
+from .capi import F32, F16, I8, I32, BF16, EPI_BIAS, EPI_GELU, EPI_RESIDUAL, EPI_NONE  # noqa: F401
+
+_DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.int8: I8, torch.int32: I32}
+
+
+def dt(t):
+    return _DT[t.dtype]
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _chk(*ts):
+    for t in ts:
+        if t is not None:
+            assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensors only"
+
+
+def gemm(a, b, b_is_nk=True, bias=None, gelu=False, residual=None, out=None):
+    """a: [batch?, M, K]; b: [N, K] (b_is_nk) or [K, N]; optional leading batch dims broadcast by modulo."""
+    _chk(a, b, bias, residual, out)
+    M, K = a.shape[-2], a.shape[-1]
+    N = b.shape[-2] if b_is_nk else b.shape[-1]
+    assert (b.shape[-1] if b_is_nk else b.shape[-2]) == K
+    batch_a = a.numel() // (M * K) if M * K else 1
+    batch_b = b.numel() // (N * K) if N * K else 1
+    batch = max(batch_a, batch_b)
+    if out is None:
+        lead = a.shape[:-2] if batch_a >= batch_b else b.shape[:-2]
+        out = torch.empty(*lead, M, N, dtype=a.dtype, device=a.device)
+    epi = (EPI_BIAS if bias is not None else 0) | (EPI_GELU if gelu else 0) | (EPI_RESIDUAL if residual is not None else 0)
+    capi.call("tnn_rocm_gemm", _stream(), dt(a), 1 if b_is_nk else 0, _p(a), _p(b), _p(out), M, N, K,
+              K, K if b_is_nk else N, N, batch, batch_a, batch_b, epi, _p(bias), _p(residual), N)
+    return out
+
+
+def gemm_i8(a, w, bias, scale, want_acc=False, want_q=True, dequant_scale=None, dequant_dtype=torch.float32):
+    _chk(a, w, bias, scale)
+    M, K = a.shape
+    N = w.shape[0]
+    q = torch.empty(M, N, dtype=torch.int8, device=a.device) if want_q else None
+    acc = torch.empty(M, N, dtype=torch.int32, device=a.device) if want_acc else None
+    outf = torch.empty(M, N, dtype=dequant_dtype, device=a.device) if dequant_scale is not None else None
+    capi.call("tnn_rocm_gemm_i8", _stream(), _p(a), _p(w), _p(bias), _p(scale), _p(q), _p(acc), M, N, K, K, K, N,
+              _p(outf), _DT[dequant_dtype], float(dequant_scale or 0.0))
+    return q, acc, outf
+
+
+def attention(q, k, v, scale, mask=None, kv_len=None, out=None):
+    """q, k, v: [B, h, S, d] contiguous."""
+    _chk(q, k, v, mask, kv_len)
+    B, h, S, d = q.shape
+    if out is None:
+        out = torch.empty_like(q)
+    capi.call("tnn_rocm_attention", _stream(), dt(q), _p(q), _p(k), _p(v), _p(out), B, h, S, d,
+              h * S * d, S * d, d, h * S * d, S * d, d, h * S * d, S * d, d, float(scale), _p(mask), _p(kv_len))
+    return out
+
+
+def attention_packed(qkv, B, S, heads, scale, mask=None, kv_len=None, out=None):
+    """qkv: [B*S, 3*H] (Q | K | V column blocks, heads contiguous inside each); out: [B*S, H]."""
+    _chk(qkv, mask, kv_len, out)
+    H = qkv.shape[1] // 3
+    d = H // heads
+    if out is None:
+        out = torch.empty(B * S, H, dtype=qkv.dtype, device=qkv.device)
+    es = qkv.element_size()
+    base = qkv.data_ptr()
+    capi.call("tnn_rocm_attention", _stream(), dt(qkv), base, base + H * es, base + 2 * H * es, _p(out), B, heads, S, d,
+              S * 3 * H, d, 3 * H, S * 3 * H, d, 3 * H, S * H, d, H, float(scale), _p(mask), _p(kv_len))
+    return out
+
+
+def mask_to_kv_len(mask, threshold=-1000.0):
+    _chk(mask)
+    B, S = mask.shape
+    out = torch.empty(B, dtype=torch.int32, device=mask.device)
+    capi.call("tnn_rocm_mask_to_kv_len", _stream(), _p(mask), _p(out), B, S, float(threshold))
+    return out
+
+
+def softmax(x, axis=-1):
+    _chk(x)
+    axis = axis % x.dim()
+    outer = 1
+    for s in x.shape[:axis]:
+        outer *= s
+    inner = 1
+    for s in x.shape[axis + 1:]:
+        inner *= s
+    y = torch.empty_like(x)
+    capi.call("tnn_rocm_softmax", _stream(), dt(x), _p(x), _p(y), outer, x.shape[axis], inner)
+    return y
+
+
+def layernorm(x, gamma, beta, eps, residual=None, q_inv_scale=None):
+    _chk(x, gamma, beta, residual)
+    cols = gamma.numel()
+    rows = x.numel() // cols
+    y = torch.empty_like(x)
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device) if q_inv_scale is not None else None
+    capi.call("tnn_rocm_layernorm", _stream(), dt(x), _p(x), _p(residual), _p(gamma), _p(beta), _p(y), rows, cols,
+              float(eps), _p(q), float(q_inv_scale or 0.0))
+    return (y, q) if q is not None else y
+
+
+def gelu(x):
+    _chk(x)
+    y = torch.empty_like(x)
+    capi.call("tnn_rocm_gelu", _stream(), dt(x), _p(x), _p(y), x.numel())
+    return y
+
+
+def binary(op, a, b, out_shape=None):
+    _chk(a, b)
+    if out_shape is None:
+        out_shape = torch.broadcast_shapes(a.shape, b.shape)
+    out = torch.empty(*out_shape, dtype=a.dtype, device=a.device)
+    capi.call("tnn_rocm_binary", _stream(), dt(a), {"add": 0, "sub": 1, "mul": 2, "div": 3}[op], _p(a),
+              capi.int_array(a.shape), a.dim(), _p(b), capi.int_array(b.shape), b.dim(), _p(out),
+              capi.int_array(out_shape), len(out_shape))
+    return out
+
+
+def permute(x, order):
+    _chk(x)
+    out = torch.empty(*[x.shape[o] for o in order], dtype=x.dtype, device=x.device)
+    capi.call("tnn_rocm_permute", _stream(), x.element_size(), _p(x), _p(out), capi.int_array(x.shape),
+              capi.int_array(order), x.dim())
+    return out
+
+
+def gather(data, indices, axis=0):
+    _chk(data, indices)
+    batch = 1
+    for s in data.shape[:axis]:
+        batch *= s
+    slices = data.shape[axis]
+    slice_elems = 1
+    for s in data.shape[axis + 1:]:
+        slice_elems *= s
+    out = torch.empty(*data.shape[:axis], *indices.shape, *data.shape[axis + 1:], dtype=data.dtype, device=data.device)
+    flag = torch.zeros(1, dtype=torch.int32, device=data.device)
+    capi.call("tnn_rocm_gather", _stream(), _p(data), _p(indices), _p(out), batch, slices,
+              slice_elems * data.element_size(), indices.numel(), _p(flag))
+    return out, flag
+
+
+def cast(x, dtype):
+    _chk(x)
+    y = torch.empty(x.shape, dtype=dtype, device=x.device)
+    capi.call("tnn_rocm_cast", _stream(), dt(x), _p(x), _DT[dtype], _p(y), x.numel())
+    return y
+
+
+def quantize(x, inv_scale):
+    _chk(x)
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    capi.call("tnn_rocm_quantize", _stream(), dt(x), _p(x), float(inv_scale), _p(q), x.numel())
+    return q
+
+
+def dequantize(q, scale, dtype=torch.float32):
+    _chk(q)
+    x = torch.empty(q.shape, dtype=dtype, device=q.device)
+    capi.call("tnn_rocm_dequantize", _stream(), _p(q), float(scale), _DT[dtype], _p(x), q.numel())
+    return x
+
+
+def add_i8(a, sa, b, sb, inv_so):
+    _chk(a, b)
+    y = torch.empty_like(a)
+    capi.call("tnn_rocm_add_i8", _stream(), _p(a), float(sa), _p(b), float(sb), float(inv_so), _p(y), a.numel())
+    return y
+
+
+def gelu_i8(q, in_scale, out_inv_scale):
+    _chk(q)
+    y = torch.empty_like(q)
+    capi.call("tnn_rocm_gelu_i8", _stream(), _p(q), float(in_scale), float(out_inv_scale), _p(y), q.numel())
+    return y
