@@ -1,0 +1,131 @@
+// Drives the reference engine's own CPU paths (DEVICE_NAIVE / DEVICE_X86) through its public API
+// (include/tnn/core/tnn.h:34-66, instance.h:42-144, mat.h:53-87) from a .tnnproto text and a .tnnmodel
+// blob held in memory.  TEST INFRASTRUCTURE ONLY: it is built into oracle/_ref/ together with the
+// reference library, serves as the checker for the model-file writer and the DEVICE_ROCM host, and is
+// the timed CPU baseline ("reference") of the benchmark.  Nothing shipped links against it.
+#include <chrono>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "tnn/core/blob.h"
+#include "tnn/core/instance.h"
+#include "tnn/core/mat.h"
+#include "tnn/core/tnn.h"
+
+using namespace TNN_NS;
+
+namespace {
+struct Session {
+    TNN net;
+    std::shared_ptr<Instance> inst;
+    std::string err;
+};
+void put_err(char *buf, size_t n, const std::string &s) {
+    if (buf && n) {
+        snprintf(buf, n, "%s", s.c_str());
+    }
+}
+}  // namespace
+
+extern "C" {
+
+#define REF_API __attribute__((visibility("default")))
+
+// device: "NAIVE" or "X86".  Returns nullptr and fills err on failure.
+REF_API void *tnn_ref_create(const char *proto, size_t proto_len, const char *model, size_t model_len,
+                             const char *device, int threads, char *err, size_t err_len) {
+    std::unique_ptr<Session> s(new Session);
+    ModelConfig mc;
+    mc.model_type = MODEL_TYPE_TNN;
+    mc.params.push_back(std::string(proto, proto_len));
+    mc.params.push_back(std::string(model, model_len));
+    Status st = s->net.Init(mc);
+    if (st != TNN_OK) {
+        put_err(err, err_len, "TNN::Init: " + st.description());
+        return nullptr;
+    }
+    NetworkConfig nc;
+    nc.device_type  = (std::string(device) == "X86") ? DEVICE_X86 : DEVICE_NAIVE;
+    nc.network_type = NETWORK_TYPE_DEFAULT;
+    nc.precision    = PRECISION_HIGH;
+    s->inst         = s->net.CreateInst(nc, st);
+    if (st != TNN_OK || !s->inst) {
+        put_err(err, err_len, "TNN::CreateInst: " + st.description());
+        return nullptr;
+    }
+    if (threads > 0)
+        s->inst->SetCpuNumThreads(threads);
+    return s.release();
+}
+
+REF_API void tnn_ref_destroy(void *h) { delete static_cast<Session *>(h); }
+
+// mat_type: 0 = NCHW_FLOAT (fp32 data), 1 = NC_INT32 (int32 data)
+REF_API int tnn_ref_set_input(void *h, const char *name, const void *data, int mat_type, const int *dims, int ndims) {
+    Session *s = static_cast<Session *>(h);
+    DimsVector d(dims, dims + ndims);
+    auto mat = std::make_shared<Mat>(DEVICE_NAIVE, mat_type == 1 ? NC_INT32 : NCHW_FLOAT, d, const_cast<void *>(data));
+    Status st = s->inst->SetInputMat(mat, MatConvertParam(), name);
+    if (st != TNN_OK) {
+        s->err = st.description();
+        return (int)st;
+    }
+    return 0;
+}
+
+REF_API int tnn_ref_forward(void *h) {
+    Session *s = static_cast<Session *>(h);
+    Status st  = s->inst->Forward();
+    if (st != TNN_OK) {
+        s->err = st.description();
+        return (int)st;
+    }
+    return 0;
+}
+
+// Copies output blob `name` as fp32 into out (capacity in elements); dims/ndims receive its shape.
+REF_API int tnn_ref_get_output(void *h, const char *name, float *out, size_t capacity, int *dims, int *ndims) {
+    Session *s = static_cast<Session *>(h);
+    std::shared_ptr<Mat> mat;
+    Status st = s->inst->GetOutputMat(mat, MatConvertParam(), name, DEVICE_NAIVE, NCHW_FLOAT);
+    if (st != TNN_OK || !mat) {
+        s->err = st.description();
+        return st != TNN_OK ? (int)st : -1;
+    }
+    DimsVector d = mat->GetDims();
+    size_t count = 1;
+    for (int v : d)
+        count *= (size_t)v;
+    if (ndims)
+        *ndims = (int)d.size();
+    if (dims)
+        for (size_t i = 0; i < d.size() && i < 8; ++i)
+            dims[i] = d[i];
+    if (count > capacity) {
+        s->err = "output buffer too small";
+        return -2;
+    }
+    memcpy(out, mat->GetData(), count * sizeof(float));
+    return 0;
+}
+
+REF_API const char *tnn_ref_last_error(void *h) { return static_cast<Session *>(h)->err.c_str(); }
+
+// Mean wall time (seconds) of `iters` Forward() calls after `warmup` untimed ones.
+REF_API double tnn_ref_time_forward(void *h, int warmup, int iters) {
+    Session *s = static_cast<Session *>(h);
+    for (int i = 0; i < warmup; ++i)
+        if (s->inst->Forward() != TNN_OK)
+            return -1.0;
+    auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < iters; ++i)
+        if (s->inst->Forward() != TNN_OK)
+            return -1.0;
+    auto t1 = std::chrono::steady_clock::now();
+    return std::chrono::duration<double>(t1 - t0).count() / (iters > 0 ? iters : 1);
+}
+
+}  // extern "C"

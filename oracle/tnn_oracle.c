@@ -130,13 +130,18 @@ ORC_API void orc_layernorm_f32(const float *x, const float *gamma, const float *
 
 /* ---------------------------------------------------------------------------------------------
  * GELU   device/cpu/acc/cpu_gelu_layer_acc.cc:42-45 ;  erf-based, never the tanh form.
- * The reference calls the overloaded erf on a float argument, i.e. erff.
+ * The source reads 0.5f * x * (erf(x*0.707106793288165f) + 1.0f) with only <cmath> included, so the
+ * unqualified erf resolves to the C library's double erf(double): the argument product and 0.5f*x
+ * are fp32, erf and the final product are double, and the store rounds to fp32.  (Checked against
+ * the compiled reference: this form is bit-identical, the erff form differs in the last ulp.)
  * ------------------------------------------------------------------------------------------- */
 ORC_API void orc_gelu_f32(const float *x, float *y, size_t count) {
 #pragma omp parallel for schedule(static)
     for (size_t i = 0; i < count; ++i) {
-        float v = x[i];
-        y[i]    = 0.5f * v * (erff(v * 0.707106793288165f) + 1.0f);
+        float v  = x[i];
+        float hv = 0.5f * v;
+        double e = erf((double)(v * 0.707106793288165f)) + 1.0f;
+        y[i]     = (float)(hv * e);
     }
 }
 

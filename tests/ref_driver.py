@@ -1,0 +1,101 @@
+"""ctypes front-end of oracle/_ref (the reference engine's own CPU paths, built from its sources).
+Test infrastructure only; absent on machines where oracle/_ref was never built."""
+import ctypes as C
+import os
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "oracle", "_ref", "libtnn_ref_driver.so")
+_lib = None
+
+
+def available():
+    return os.path.exists(LIB)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = C.CDLL(LIB)
+        _lib.tnn_ref_create.restype = C.c_void_p
+        _lib.tnn_ref_create.argtypes = [C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t, C.c_char_p, C.c_int,
+                                        C.c_char_p, C.c_size_t]
+        _lib.tnn_ref_destroy.argtypes = [C.c_void_p]
+        _lib.tnn_ref_set_input.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]
+        _lib.tnn_ref_forward.argtypes = [C.c_void_p]
+        _lib.tnn_ref_get_output.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
+                                            C.POINTER(C.c_int)]
+        _lib.tnn_ref_last_error.restype = C.c_char_p
+        _lib.tnn_ref_last_error.argtypes = [C.c_void_p]
+        _lib.tnn_ref_time_forward.restype = C.c_double
+        _lib.tnn_ref_time_forward.argtypes = [C.c_void_p, C.c_int, C.c_int]
+    return _lib
+
+
+class RefSession:
+    def __init__(self, graph, device="NAIVE", threads=0):
+        proto = graph.proto().encode()
+        model = graph.model()
+        err = C.create_string_buffer(512)
+        self.h = lib().tnn_ref_create(proto, len(proto), model, len(model), device.encode(), threads, err, 512)
+        if not self.h:
+            raise RuntimeError("reference engine refused the model: " + err.value.decode())
+        self._keep = []
+
+    def _check(self, rc, what):
+        if rc != 0:
+            raise RuntimeError("%s failed (0x%x): %s" % (what, rc, lib().tnn_ref_last_error(self.h).decode()))
+
+    def set_input(self, name, arr):
+        a = np.ascontiguousarray(arr)
+        assert a.dtype in (np.float32, np.int32)
+        self._keep.append(a)
+        dims = (C.c_int * a.ndim)(*a.shape)
+        self._check(lib().tnn_ref_set_input(self.h, name.encode(), a.ctypes.data_as(C.c_void_p),
+                                            1 if a.dtype == np.int32 else 0, dims, a.ndim), "SetInputMat")
+
+    def forward(self):
+        self._check(lib().tnn_ref_forward(self.h), "Forward")
+
+    def output(self, name, max_elems=1 << 26):
+        buf = np.empty(max_elems, np.float32)
+        dims = (C.c_int * 8)()
+        nd = C.c_int(0)
+        self._check(lib().tnn_ref_get_output(self.h, name.encode(), buf.ctypes.data_as(C.c_void_p), max_elems, dims,
+                                             C.byref(nd)), "GetOutputMat")
+        shape = [dims[i] for i in range(nd.value)]
+        return buf[:int(np.prod(shape))].reshape(shape).copy()
+
+    def time_forward(self, warmup, iters):
+        t = lib().tnn_ref_time_forward(self.h, warmup, iters)
+        if t < 0:
+            raise RuntimeError("Forward failed while timing")
+        return t
+
+    def close(self):
+        if self.h:
+            lib().tnn_ref_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()
+
+
+def time_encoder(cfg, weights, ids, seg, mask):
+    """CPU baseline of the benchmark: the reference's DEVICE_X86 path on the same synthetic encoder, all host
+    cores (OpenMP), `ids.shape[0]` sequences through all layers."""
+    from tnn_amd import tnnmodel
+    B, S = ids.shape
+    g = tnnmodel.encoder_graph(cfg, weights, B, S)
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    s = RefSession(g, "X86", threads)
+    s.set_input("input_ids", ids.astype(np.int32))
+    s.set_input("token_type_ids", seg.astype(np.int32))
+    s.set_input("attention_bias", mask.reshape(B, 1, 1, S).astype(np.float32))
+    t = s.time_forward(1, 3)
+    s.close()
+    return {"value": B / t, "unit": "sequences/s", "cores": threads, "kind": "reference",
+            "sample": "%d sequences (S=%d) through all %d layers on the reference engine's DEVICE_X86 path "
+                      "(fp32, AVX2 + OpenMP; its MatMul/Softmax/LayerNorm kernels are single-threaded), "
+                      "mean of 3 Forward() calls after 1 warm-up" % (B, S, cfg.layers)}

@@ -1,0 +1,176 @@
+"""Pins the CPU checker (oracle/tnn_oracle.c) against the reference engine itself: the same synthetic graphs
+are written as .tnnproto/.tnnmodel, loaded by the reference's own parser and run on its DEVICE_NAIVE and
+DEVICE_X86 paths (oracle/_ref, built from the reference sources), then compared with the restatement.
+
+Skipped where oracle/_ref has not been built (it needs the reference tree at build time)."""
+import numpy as np
+import pytest
+
+import encoder_ref
+import orc
+import ref_driver
+from tnn_amd import tnnmodel
+from tnn_amd.encoder import EncoderConfig, make_weights, make_inputs
+
+pytestmark = pytest.mark.skipif(not ref_driver.available(), reason="oracle/_ref not built")
+
+
+def rel(a, b):
+    return float(np.abs(np.asarray(a, np.float64) - b).max() / np.abs(b).max())
+
+
+def test_config1_attention_layer_naive_and_x86():
+    # BASELINE config 1: B1 S128 H768 h12 fp32, N(0,1) input, N(0,0.02) weights, zero biases, mask all ones
+    cfg = EncoderConfig(1, 768, 12, 3072)
+    lw = make_weights(cfg, seed=1, with_embeddings=False)["layers"][0]
+    x = np.random.default_rng(2).standard_normal((128, 768)).astype(np.float32)
+    g = tnnmodel.attention_layer_graph(lw, 128, 768, 12)
+    outs = {}
+    for dev in ("NAIVE", "X86"):
+        s = ref_driver.RefSession(g, dev, 1)
+        s.set_input("x", x)
+        s.forward()
+        outs[dev] = s.output("y")
+        s.close()
+    # the restatement of the same graph (InnerProduct = NaiveFC with float accumulation)
+    def fc(t, w, b):
+        return orc.inner_product(t, w, b)
+    q = orc.permute(fc(x, lw["wq"], lw["bq"]).reshape(128, 12, 64), (1, 0, 2))
+    kt = orc.permute(fc(x, lw["wk"], lw["bk"]).reshape(128, 12, 64), (1, 2, 0))
+    v = orc.permute(fc(x, lw["wv"], lw["bv"]).reshape(128, 12, 64), (1, 0, 2))
+    s_ = orc.binary("mul", orc.matmul(q, kt), np.array([0.125], np.float32))
+    c = orc.permute(orc.matmul(orc.softmax(s_, 2), v), (1, 0, 2)).reshape(128, 768)
+    mine = fc(c, lw["wo"], lw["bo"])
+    assert outs["NAIVE"].shape == (128, 768)
+    assert np.array_equal(mine, outs["NAIVE"]), rel(mine, outs["NAIVE"])   # same arithmetic: bit-identical
+    assert rel(outs["X86"], outs["NAIVE"]) <= 2e-3                          # second witness within the fp32 bar
+    # and the composite used by the GPU tests equals the op-by-op graph
+    q4, k4, v4 = (orc.permute(fc(x, lw["w" + n], lw["b" + n]).reshape(1, 128, 12, 64), (0, 2, 1, 3)) for n in "qkv")
+    comp = orc.permute(orc.attention_core(q4, k4, v4, np.float32(0.125)), (0, 2, 1, 3)).reshape(128, 768)
+    assert np.array_equal(fc(comp, lw["wo"], lw["bo"]), mine)
+
+
+@pytest.mark.parametrize("dev", ["NAIVE", "X86"])
+def test_encoder_graph_with_embeddings_and_mask(dev):
+    cfg = EncoderConfig(2, 128, 2, 256, vocab=1000, max_pos=64)
+    w = make_weights(cfg, seed=3, bias_std=0.02)
+    for lw in w["layers"]:  # non-trivial gamma/beta so LayerNorm's affine part is exercised
+        lw["ln1_g"] = (1 + 0.1 * np.random.default_rng(1).standard_normal(128)).astype(np.float32)
+        lw["ln2_b"] = (0.1 * np.random.default_rng(2).standard_normal(128)).astype(np.float32)
+    B, S = 2, 48
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 10, 48, seed=4)
+    g = tnnmodel.encoder_graph(cfg, w, B, S, extra_outputs=["x0", "l0_probs", "l0_x1"])
+    s = ref_driver.RefSession(g, dev, 2)
+    s.set_input("input_ids", ids)
+    s.set_input("token_type_ids", seg)
+    s.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+    s.forward()
+    x0 = encoder_ref.embed(w, ids, seg, cfg.eps)
+    ref = encoder_ref.encoder(w, cfg, x0, B, S, mask)
+    got_x0 = s.output("x0").reshape(B * S, -1)
+    got = s.output("last_hidden").reshape(B * S, -1)
+    probs = s.output("l0_probs")
+    s.close()
+    assert probs.shape == (B, 2, S, S)
+    # padded keys get exactly zero probability on NAIVE (expf underflow of -10000)
+    for b in range(B):
+        assert np.all(probs[b, :, :, lens[b]:] < 1e-30)
+    if dev == "NAIVE":
+        assert np.array_equal(got_x0, x0)
+        assert np.array_equal(got, ref)
+    else:
+        assert rel(got_x0, x0) <= 1e-5
+        assert rel(got, ref) <= 2e-3
+
+
+def _run(g, inputs, out, dev):
+    s = ref_driver.RefSession(g, dev, 1)
+    for k, v in inputs.items():
+        s.set_input(k, v)
+    s.forward()
+    r = s.output(out)
+    s.close()
+    return r
+
+
+def test_single_ops_bit_identical_on_naive():
+    rng = np.random.default_rng(0)
+    # GELU (the compiled reference evaluates erf in double: see the checker's comment)
+    x = (rng.standard_normal((4, 3000)) * 3).astype(np.float32)
+    x[0, 0] = -2.281006575
+    g = tnnmodel.Graph()
+    g.add_input("x", [4, 3000])
+    g.add_layer("GELU", "g", ["x"], ["y"])
+    g.add_output("y")
+    assert np.array_equal(_run(g, {"x": x}, "y", "NAIVE"), orc.gelu(x))
+    assert rel(_run(g, {"x": x}, "y", "X86"), orc.gelu(x)) <= 2e-3
+    # LayerNorm with affine parameters from the constant map, BERT's eps
+    x = (rng.standard_normal((6, 128)) * 2 + 0.3).astype(np.float32)
+    ga, be = rng.standard_normal(128).astype(np.float32), rng.standard_normal(128).astype(np.float32)
+    g = tnnmodel.Graph()
+    g.add_input("x", [6, 128])
+    g.add_constant("ga", ga)
+    g.add_constant("be", be)
+    g.add_layer("LayerNorm", "ln", ["x", "ga", "be"], ["y"], [1, "1e-12"])
+    g.add_output("y")
+    assert np.array_equal(_run(g, {"x": x}, "y", "NAIVE"), orc.layernorm(x, ga, be, 1e-12))
+    assert rel(_run(g, {"x": x}, "y", "X86"), orc.layernorm(x, ga, be, 1e-12)) <= 1e-5
+    # Softmax over an inner axis and the last axis
+    x = (rng.standard_normal((2, 3, 16, 16)) * 4).astype(np.float32)
+    for axis in (1, 3):
+        g = tnnmodel.Graph()
+        g.add_input("x", [2, 3, 16, 16])
+        g.add_layer("Softmax", "s", ["x"], ["y"], [axis])
+        g.add_output("y")
+        assert np.array_equal(_run(g, {"x": x}, "y", "NAIVE"), orc.softmax(x, axis))
+    # batched MatMul with broadcast of the second operand, and Permute
+    a = rng.standard_normal((2, 3, 8, 16)).astype(np.float32)
+    b = rng.standard_normal((3, 16, 9)).astype(np.float32)
+    g = tnnmodel.Graph()
+    g.add_input("a", [2, 3, 8, 16])
+    g.add_input("b", [3, 16, 9])
+    g.add_layer("MatMul", "mm", ["a", "b"], ["c"], [-1])
+    g.add_layer("Permute", "pm", ["c"], ["y"], [4, 0, 2, 3, 1])
+    g.add_output("y")
+    ref = orc.permute(orc.matmul(a, b), (0, 2, 3, 1))
+    assert np.array_equal(_run(g, {"a": a, "b": b}, "y", "NAIVE"), ref)
+
+
+@pytest.mark.parametrize("dev", ["NAIVE", "X86"])
+def test_int8_ffn_bit_identical(dev):
+    """QuantizedInnerProduct -> GELU -> QuantizedInnerProduct with full-range int8 data: int8 outputs of the
+    reference (after its own dequantisation) equal the restatement exactly."""
+    rng = np.random.default_rng(0)
+    T, K, F = 32, 64, 128
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    w1 = rng.integers(-127, 128, (F, K), dtype=np.int8)
+    w2 = rng.integers(-127, 128, (K, F), dtype=np.int8)
+    b1 = rng.integers(-500, 500, F).astype(np.int32)
+    b2 = rng.integers(-500, 500, K).astype(np.int32)
+    ws1 = (rng.uniform(0.5, 1.5, F) * 2e-4).astype(np.float32)
+    ws2 = (rng.uniform(0.5, 1.5, K) * 2e-4).astype(np.float32)
+    s_a, s_h, s_g, s_y = (np.float32(v) for v in (0.031, 0.045, 0.027, 0.052))
+    g = tnnmodel.int8_ffn_graph(T, K, F, w1, b1, ws1, w2, b2, ws2, s_a, s_h, s_g, s_y)
+    got = _run(g, {"x": x}, "y", dev)
+    qa = orc.quantize_x86(x, s_a)
+    h, _ = orc.fc_int8(qa, w1, b1, orc.fc_int8_scale(ws1, s_h, F))
+    gq = orc.quantize_x86(orc.gelu(orc.dequantize(h, s_h)), s_g)
+    yq, _ = orc.fc_int8(gq, w2, b2, orc.fc_int8_scale(ws2, s_y, K))
+    assert np.array_equal(got, orc.dequantize(yq, s_y))
+
+
+def test_float2int8_exhaustive_band_against_definition():
+    # every fp32 within +-3 ulp of every half-integer in [-130.5, 130.5]: the add-then-truncate definition
+    k = (np.arange(-261, 262, dtype=np.float64) * 0.5).astype(np.float32)
+    vals = [k]
+    up, dn = k, k
+    for _ in range(3):
+        up = np.nextafter(up, np.float32(np.inf))
+        dn = np.nextafter(dn, np.float32(-np.inf))
+        vals += [up, dn]
+    v = np.concatenate(vals)
+    t = (v + np.where(v >= 0, np.float32(0.5), np.float32(-0.5))).astype(np.float32)
+    expect = np.trunc(np.clip(t, -128, 127)).astype(np.int8)
+    assert np.array_equal(orc.float2int8(v), expect)
+    # ties go away from zero; 0.49999997 + 0.5 rounds up to 1.0 in fp32 and therefore quantises to 1
+    assert orc.float2int8(np.array([0.5, -0.5, 2.5, -2.5, 0.49999997], np.float32)).tolist() == [1, -1, 3, -3, 1]

@@ -1,0 +1,264 @@
+"""Writer for the engine's on-disk model formats: the .tnnproto text graph and the .tnnmodel weight blob.
+
+Format facts (reference tree):
+  proto  : source/tnn/interpreter/tnn/model_interpreter.cc:174-398, model_packer.cc:70-184
+           line0 "1 <nblobs> 1 <magic> ," ; line1 inputs (v2: "name rank d0.. dtype" joined by ':') ;
+           line2 blob names ; line3 outputs ; line4 layer count ; then one line per layer
+           "Type name n_in n_out inputs.. outputs.. params.. ,"
+  model  : model_packer.cc:186-248 / model_interpreter.cc:400-476
+           u32 magic ; i32 resource count ; per resource {i32 type, str type_str, str name, payload} ;
+           then {u32 magic, i32 n, (str key, raw buffer)*n} for the constant map.
+  raw    : objseri.h:57-77   {u32 0x0FABC0004, i32 dtype, i32 nbytes, [i32 ndims, dims.., bytes]}
+  strings: i32 byte length + bytes.
+
+`Graph` collects layers, resources and constants; `encoder_graph()` emits the decomposed BERT encoder the
+way an ONNX export looks after conversion (MatMul+Add projections, Reshape/Permute head split, MatMul,
+Mul, Add(mask), Softmax, MatMul, LayerNorm, GELU), and `int8_ffn_graph()` the QuantizedInnerProduct variant.
+"""
+import struct
+
+import numpy as np
+
+MAGIC_V2 = 0x0FABC0004
+DT_FLOAT, DT_HALF, DT_INT8, DT_INT32 = 0, 1, 2, 3
+_NP2DT = {np.dtype(np.float32): DT_FLOAT, np.dtype(np.float16): DT_HALF, np.dtype(np.int8): DT_INT8,
+          np.dtype(np.int32): DT_INT32}
+
+# LayerType numbers (source/tnn/core/layer_type.h) for the resource headers; the reader re-derives the type
+# from the type string, the number only has to be in range.
+_LAYER_TYPE_NUM = {"InnerProduct": 19, "QuantizedInnerProduct": 19, "Add": 38, "Mul": 42, "Sub": 39, "Div": 43,
+                   "Gather": 104, "MatMul": 105, "BlobScale": 600}
+BLOB_SCALE_SUFFIX = "_scale_data_"
+
+
+def _i32(v):
+    return struct.pack("<i", int(v))
+
+
+def _u32(v):
+    return struct.pack("<I", int(v))
+
+
+def _str(s):
+    b = s.encode("utf-8")
+    return _i32(len(b)) + b
+
+
+def raw_buffer(arr, dims=None):
+    """Serialise one RawBuffer record.  `arr` None or empty gives the zero-length form."""
+    if arr is None or arr.size == 0:
+        return _u32(MAGIC_V2) + _i32(DT_FLOAT) + _i32(0)
+    a = np.ascontiguousarray(arr)
+    dt = _NP2DT[a.dtype]
+    dims = list(a.shape if dims is None else dims)
+    out = _u32(MAGIC_V2) + _i32(dt) + _i32(a.nbytes) + _i32(len(dims))
+    out += b"".join(_i32(d) for d in dims)
+    return out + a.tobytes()
+
+
+class Graph:
+    def __init__(self):
+        self.inputs = []      # (name, dims, dtype)
+        self.outputs = []
+        self.layers = []      # (type, name, inputs, outputs, params)
+        self.resources = []   # (name, type_str, payload bytes) in layer order
+        self.constants = {}   # blob name -> ndarray
+        self.blobs = []
+
+    def _blob(self, name):
+        if name not in self.blobs:
+            self.blobs.append(name)
+
+    def add_input(self, name, dims, dtype=DT_FLOAT):
+        self.inputs.append((name, list(dims), dtype))
+        self._blob(name)
+
+    def add_output(self, name):
+        self.outputs.append(name)
+
+    def add_constant(self, name, arr):
+        self.constants[name] = np.ascontiguousarray(arr)
+        self._blob(name)
+
+    def add_layer(self, type_str, name, inputs, outputs, params=()):
+        for b in list(inputs) + list(outputs):
+            self._blob(b)
+        self.layers.append((type_str, name, list(inputs), list(outputs), [str(p) for p in params]))
+
+    # ---- resources ------------------------------------------------------------------------------
+    def _res(self, name, type_str, payload):
+        self.resources.append((name, type_str, payload))
+
+    def res_matmul(self, name, weight_kn):
+        self._res(name, "MatMul", raw_buffer(weight_kn))
+
+    def res_eltwise(self, name, type_str, element):
+        self._res(name, type_str, raw_buffer(element))
+
+    def res_gather(self, name, data, indices=None):
+        p = _i32(1) + raw_buffer(data)
+        p += (_i32(1) + raw_buffer(indices)) if indices is not None else _i32(0)
+        self._res(name, "Gather", p)
+
+    def res_inner_product(self, name, weight_nk, bias=None, quant_scale=None):
+        """fp32: weight [N,K] + bias [N].  int8: int8 weight, int32 bias, zero points (int8 zeros), fp32 scale."""
+        p = _str(name) + raw_buffer(weight_nk) + raw_buffer(bias)
+        type_str = "InnerProduct"
+        if quant_scale is not None:
+            type_str = "QuantizedInnerProduct"
+            zp = np.zeros(quant_scale.shape, np.int8)
+            p += raw_buffer(zp) + raw_buffer(np.asarray(quant_scale, np.float32))
+        self._res(name, type_str, p)
+
+    def res_blob_scale(self, blob_name, scale):
+        scale = np.atleast_1d(np.asarray(scale, np.float32))
+        zp = np.zeros(scale.shape, np.int8)
+        bias = np.zeros(scale.shape, np.int32)
+        self._res(blob_name + BLOB_SCALE_SUFFIX, "BlobScale", raw_buffer(zp) + raw_buffer(scale) + raw_buffer(bias))
+
+    # ---- serialisation ------------------------------------------------------------------------------
+    def proto(self):
+        lines = ['"1 %d 1 %d ,"' % (len(self.blobs), MAGIC_V2)]
+        ins = []
+        for name, dims, dt in self.inputs:
+            ins.append("%s %d %s %d" % (name, len(dims), " ".join(str(d) for d in dims), dt))
+        lines.append('"%s ,"' % " : ".join(ins))
+        lines.append('" %s ,"' % " ".join(self.blobs))
+        lines.append('"%s ,"' % " ".join(self.outputs))
+        lines.append('" %d ,"' % len(self.layers))
+        for t, n, i, o, p in self.layers:
+            lines.append('"%s ,"' % " ".join([t, n, str(len(i)), str(len(o))] + i + o + p))
+        return "\n".join(lines) + "\n"
+
+    def model(self):
+        out = _u32(MAGIC_V2) + _i32(len(self.resources))
+        for name, type_str, payload in self.resources:
+            out += _i32(_LAYER_TYPE_NUM.get(type_str, 0)) + _str(type_str) + _str(name) + payload
+        if self.constants:
+            out += _u32(MAGIC_V2) + _i32(len(self.constants))
+            for key in sorted(self.constants):
+                out += _str(key) + raw_buffer(self.constants[key])
+        return out
+
+
+# ---------------------------------------------------------------------------------------------------
+def _linear(g, name, x, out, w_nk, bias):
+    """y = x W^T + b as the ONNX-exported pair MatMul(weight [K,N] in the resource) + Add(bias resource)."""
+    g.add_layer("MatMul", name + "_mm", [x], [name + "_mm_o"], [1])
+    g.res_matmul(name + "_mm", np.ascontiguousarray(w_nk.T))
+    g.add_layer("Add", name + "_add", [name + "_mm_o"], [out], [1])
+    g.res_eltwise(name + "_add", "Add", bias)
+
+
+def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=()):
+    """The decomposed encoder graph.  Inputs: input_ids, token_type_ids [B,S] int32 (or `hidden` [B,S,H] fp32
+    without embeddings) and `attention_bias` [B,1,1,S] fp32 additive mask.  Output: `last_hidden` [B,S,H]."""
+    g = Graph()
+    H, h, d = cfg.hidden, cfg.heads, cfg.head_dim
+    if with_embeddings:
+        g.add_input("input_ids", [B, S], DT_INT32)
+        g.add_input("token_type_ids", [B, S], DT_INT32)
+    else:
+        g.add_input("hidden", [B, S, H], DT_FLOAT)
+    g.add_input("attention_bias", [B, 1, 1, S], DT_FLOAT)
+    if with_embeddings:
+        g.add_layer("Gather", "emb_word", ["input_ids"], ["emb_word_o"], [0, 1, 0])
+        g.res_gather("emb_word", weights["word_emb"])
+        g.add_layer("Gather", "emb_type", ["token_type_ids"], ["emb_type_o"], [0, 1, 0])
+        g.res_gather("emb_type", weights["type_emb"])
+        g.add_layer("Add", "emb_pos", ["emb_word_o"], ["emb_pos_o"], [1])
+        g.res_eltwise("emb_pos", "Add", weights["pos_emb"][:S])
+        g.add_layer("Add", "emb_sum", ["emb_pos_o", "emb_type_o"], ["emb_sum_o"], [1])
+        g.add_constant("emb_ln_gamma", weights["emb_ln_g"])
+        g.add_constant("emb_ln_beta", weights["emb_ln_b"])
+        g.add_layer("LayerNorm", "emb_ln", ["emb_sum_o", "emb_ln_gamma", "emb_ln_beta"], ["x0"], [1, repr(cfg.eps)])
+        x = "x0"
+    else:
+        x = "hidden"
+    for li, lw in enumerate(weights["layers"]):
+        p = "l%d_" % li
+        for nm in ("q", "k", "v"):
+            _linear(g, p + nm, x, p + nm + "_o", lw["w" + nm], lw["b" + nm])
+            g.add_layer("Reshape", p + nm + "_rs", [p + nm + "_o"], [p + nm + "_4d"], [0, 4, 4, B, S, h, d, 0])
+        g.add_layer("Permute", p + "q_pm", [p + "q_4d"], [p + "qh"], [4, 0, 2, 1, 3])
+        g.add_layer("Permute", p + "k_pm", [p + "k_4d"], [p + "kt"], [4, 0, 2, 3, 1])
+        g.add_layer("Permute", p + "v_pm", [p + "v_4d"], [p + "vh"], [4, 0, 2, 1, 3])
+        g.add_layer("MatMul", p + "qk", [p + "qh", p + "kt"], [p + "scores"], [-1])
+        g.add_layer("Mul", p + "scale", [p + "scores"], [p + "scaled"], [1])
+        g.res_eltwise(p + "scale", "Mul", np.array([1.0 / np.sqrt(d)], np.float32))
+        g.add_layer("Add", p + "mask", [p + "scaled", "attention_bias"], [p + "masked"], [1])
+        g.add_layer("Softmax", p + "sm", [p + "masked"], [p + "probs"], [3])
+        g.add_layer("MatMul", p + "pv", [p + "probs", p + "vh"], [p + "ctx_h"], [-1])
+        g.add_layer("Permute", p + "ctx_pm", [p + "ctx_h"], [p + "ctx_4d"], [4, 0, 2, 1, 3])
+        g.add_layer("Reshape", p + "ctx_rs", [p + "ctx_4d"], [p + "ctx"], [0, 3, 3, B, S, H, 0])
+        _linear(g, p + "o", p + "ctx", p + "attn_o", lw["wo"], lw["bo"])
+        g.add_layer("Add", p + "res1", [x, p + "attn_o"], [p + "sum1"], [1])
+        g.add_constant(p + "ln1_gamma", lw["ln1_g"])
+        g.add_constant(p + "ln1_beta", lw["ln1_b"])
+        g.add_layer("LayerNorm", p + "ln1", [p + "sum1", p + "ln1_gamma", p + "ln1_beta"], [p + "x1"],
+                    [1, repr(cfg.eps)])
+        _linear(g, p + "ffn1", p + "x1", p + "ffn1_o", lw["w1"], lw["b1"])
+        g.add_layer("GELU", p + "gelu", [p + "ffn1_o"], [p + "act"], [])
+        _linear(g, p + "ffn2", p + "act", p + "ffn2_o", lw["w2"], lw["b2"])
+        g.add_layer("Add", p + "res2", [p + "x1", p + "ffn2_o"], [p + "sum2"], [1])
+        g.add_constant(p + "ln2_gamma", lw["ln2_g"])
+        g.add_constant(p + "ln2_beta", lw["ln2_b"])
+        out = "last_hidden" if li == len(weights["layers"]) - 1 else p + "x2"
+        g.add_layer("LayerNorm", p + "ln2", [p + "sum2", p + "ln2_gamma", p + "ln2_beta"], [out], [1, repr(cfg.eps)])
+        x = out
+    g.add_output("last_hidden")
+    for e in extra_outputs:
+        g.add_output(e)
+    return g
+
+
+def attention_layer_graph(lw, S, H, heads):
+    """Benchmark config 1: one self-attention layer on a [S,H] fp32 input with InnerProduct projections
+    (mask all ones, so no Add(mask); scale applied by a Mul)."""
+    g = Graph()
+    d = H // heads
+    g.add_input("x", [S, H], DT_FLOAT)
+    for nm in ("q", "k", "v"):
+        g.add_layer("InnerProduct", "fc_" + nm, ["x"], [nm], [H, 1, 0, 1])
+        g.res_inner_product("fc_" + nm, lw["w" + nm], lw["b" + nm])
+        g.add_layer("Reshape", "rs_" + nm, [nm], [nm + "3"], [0, 3, 3, S, heads, d, 0])
+    g.add_layer("Permute", "pm_q", ["q3"], ["qh"], [3, 1, 0, 2])
+    g.add_layer("Permute", "pm_k", ["k3"], ["kh"], [3, 1, 2, 0])
+    g.add_layer("Permute", "pm_v", ["v3"], ["vh"], [3, 1, 0, 2])
+    g.add_layer("MatMul", "mm_qk", ["qh", "kh"], ["s"], [-1])
+    g.add_layer("Mul", "scale", ["s"], ["ss"], [1])
+    g.res_eltwise("scale", "Mul", np.array([1.0 / np.sqrt(d)], np.float32))
+    g.add_layer("Softmax", "sm", ["ss"], ["p"], [2])
+    g.add_layer("MatMul", "mm_pv", ["p", "vh"], ["c"], [-1])
+    g.add_layer("Permute", "pm_c", ["c"], ["ch"], [3, 1, 0, 2])
+    g.add_layer("Reshape", "rs_c", ["ch"], ["c2"], [0, 2, 2, S, H, 0])
+    g.add_layer("InnerProduct", "fc_o", ["c2"], ["y"], [H, 1, 0, 1])
+    g.res_inner_product("fc_o", lw["wo"], lw["bo"])
+    g.add_output("y")
+    return g
+
+
+def int8_ffn_graph(T, K, F, w1_q, b1_q, w1_scale, w2_q, b2_q, w2_scale, s_in, s_h, s_act, s_out):
+    """fp32 [T,K] -> quantize -> QuantizedInnerProduct K->F -> dequantize -> GELU -> quantize ->
+    QuantizedInnerProduct F->K -> dequantize -> fp32 [T,K].  The float<->int8 Reformat layers are not written:
+    the engine's optimizer inserts them wherever a quantized layer meets a float one
+    (source/tnn/optimizer/net_optimizer_insert_int8_reformat.cc:66-181); the two Mul-by-one layers keep the
+    model input and output in fp32.  Blob scales are BlobScale resources named <blob>_scale_data_."""
+    g = Graph()
+    one = np.array([1.0], np.float32)
+    g.add_input("x", [T, K])
+    g.add_layer("Mul", "in_copy", ["x"], ["a"], [1])
+    g.res_eltwise("in_copy", "Mul", one)
+    g.add_layer("QuantizedInnerProduct", "fc1", ["a"], ["h"], [F, 1, 0, 1])
+    g.res_blob_scale("a", s_in)
+    g.res_inner_product("fc1", w1_q, b1_q, quant_scale=w1_scale)
+    g.res_blob_scale("h", s_h)
+    g.add_layer("GELU", "act", ["h"], ["g"])
+    g.add_layer("QuantizedInnerProduct", "fc2", ["g"], ["yq"], [K, 1, 0, 1])
+    g.res_blob_scale("g", s_act)
+    g.res_inner_product("fc2", w2_q, b2_q, quant_scale=w2_scale)
+    g.res_blob_scale("yq", s_out)
+    g.add_layer("Mul", "out_copy", ["yq"], ["y"], [1])
+    g.res_eltwise("out_copy", "Mul", one)
+    g.add_output("y")
+    return g
