@@ -56,6 +56,10 @@ TNN_ROCM_API int tnn_rocm_set_device(int device_id);
 TNN_ROCM_API int tnn_rocm_device_name(int device_id, char *buf, size_t buf_len);
 TNN_ROCM_API int tnn_rocm_malloc(void **ptr, size_t bytes);
 TNN_ROCM_API int tnn_rocm_free(void *ptr);
+/* page-locked host memory that kernels can also write (used for the context's error word, which the
+ * host reads after a stream synchronise instead of issuing a device-to-host copy per forward) */
+TNN_ROCM_API int tnn_rocm_malloc_host(void **host_ptr, size_t bytes);
+TNN_ROCM_API int tnn_rocm_free_host(void *host_ptr);
 TNN_ROCM_API int tnn_rocm_memset(void *ptr, int value, size_t bytes, void *stream);
 TNN_ROCM_API int tnn_rocm_memcpy_h2d(void *dst, const void *host_src, size_t bytes, void *stream);
 TNN_ROCM_API int tnn_rocm_memcpy_d2h(void *host_dst, const void *src, size_t bytes, void *stream);

@@ -22,6 +22,8 @@ SIGNATURES = {
     "tnn_rocm_device_name": [_i, C.c_char_p, _sz],
     "tnn_rocm_malloc": [C.POINTER(_vp), _sz],
     "tnn_rocm_free": [_vp],
+    "tnn_rocm_malloc_host": [C.POINTER(_vp), _sz],
+    "tnn_rocm_free_host": [_vp],
     "tnn_rocm_memset": [_vp, _i, _sz, _vp],
     "tnn_rocm_memcpy_h2d": [_vp, _vp, _sz, _vp],
     "tnn_rocm_memcpy_d2h": [_vp, _vp, _sz, _vp],

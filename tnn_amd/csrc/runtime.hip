@@ -63,6 +63,22 @@ int tnn_rocm_free(void *ptr) {
     return 0;
 }
 
+int tnn_rocm_malloc_host(void **host_ptr, size_t bytes) {
+    TR_REQUIRE(host_ptr, TNN_ROCM_EINVAL, "malloc_host: null output");
+    *host_ptr = nullptr;
+    if (bytes == 0)
+        return 0;
+    TR_CHECK_HIP(hipHostMalloc(host_ptr, bytes, hipHostMallocMapped));
+    memset(*host_ptr, 0, bytes);
+    return 0;
+}
+
+int tnn_rocm_free_host(void *host_ptr) {
+    if (host_ptr)
+        TR_CHECK_HIP(hipHostFree(host_ptr));
+    return 0;
+}
+
 int tnn_rocm_memset(void *ptr, int value, size_t bytes, void *stream) {
     if (bytes == 0)
         return 0;

@@ -1,0 +1,127 @@
+"""ctypes front-end of the C++ host (tnn_amd/lib/libtnn_rocm_host.so): an engine Instance on DEVICE_ROCM created
+from .tnnproto text + .tnnmodel bytes.  No fallback: a missing library or a failed call raises."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import capi
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libtnn_rocm_host.so")
+
+SIGNATURES = {
+    "tnn_host_create": (C.c_void_p, [C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t, C.c_int, C.c_int, C.c_char_p,
+                                     C.c_size_t]),
+    "tnn_host_destroy": (None, [C.c_void_p]),
+    "tnn_host_last_error": (C.c_char_p, [C.c_void_p]),
+    "tnn_host_set_input": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]),
+    "tnn_host_forward": (C.c_int, [C.c_void_p]),
+    "tnn_host_forward_async": (C.c_int, [C.c_void_p]),
+    "tnn_host_sync": (C.c_int, [C.c_void_p]),
+    "tnn_host_stream": (C.c_void_p, [C.c_void_p]),
+    "tnn_host_get_output": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
+                                      C.POINTER(C.c_int)]),
+    "tnn_host_layer_count": (C.c_int, [C.c_void_p]),
+    "tnn_host_layer_summary": (C.c_char_p, [C.c_void_p]),
+    "tnn_host_profile_start": (None, [C.c_void_p]),
+    "tnn_host_profile_finish": (C.c_int, [C.c_void_p, C.POINTER(C.c_double), C.c_int]),
+}
+_lib = None
+
+
+def load():
+    global _lib
+    if _lib is None:
+        capi.load()  # the kernel library first: the host links against it
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError("%s not found: run `make -C tnn_amd/host`" % LIB_PATH)
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+class HostError(RuntimeError):
+    pass
+
+
+class RocmInstance:
+    """precision: "fp32" (PRECISION_HIGH) or "fp16" (PRECISION_AUTO: fp16 activations + fused kernels)."""
+
+    def __init__(self, proto, model, precision="fp16", device_id=0):
+        lib = load()
+        if isinstance(proto, str):
+            proto = proto.encode()
+        err = C.create_string_buffer(1024)
+        self._h = lib.tnn_host_create(proto, len(proto), model, len(model), device_id,
+                                      0 if precision == "fp32" else 1, err, 1024)
+        if not self._h:
+            raise HostError("Instance::Init failed: " + err.value.decode())
+        self._keep = []
+
+    @classmethod
+    def from_graph(cls, graph, precision="fp16"):
+        return cls(graph.proto(), graph.model(), precision)
+
+    def _check(self, rc, what):
+        if rc != 0:
+            raise HostError("%s failed (0x%x): %s" % (what, rc & 0xFFFFFFFF, load().tnn_host_last_error(self._h).decode()))
+
+    def set_input(self, name, arr):
+        a = np.ascontiguousarray(arr)
+        if a.dtype not in (np.float32, np.int32):
+            raise TypeError("inputs are fp32 (NCHW_FLOAT) or int32 (NC_INT32) host arrays")
+        dims = (C.c_int * max(a.ndim, 1))(*a.shape)
+        self._check(load().tnn_host_set_input(self._h, name.encode(), a.ctypes.data_as(C.c_void_p),
+                                              1 if a.dtype == np.int32 else 0, dims, a.ndim), "SetInputMat")
+
+    def forward(self):
+        self._check(load().tnn_host_forward(self._h), "Forward")
+
+    def forward_async(self):
+        self._check(load().tnn_host_forward_async(self._h), "ForwardAsync")
+
+    def sync(self):
+        self._check(load().tnn_host_sync(self._h), "Synchronize")
+
+    @property
+    def stream(self):
+        return load().tnn_host_stream(self._h)
+
+    def output(self, name="", max_elems=1 << 25):
+        buf = np.empty(max_elems, np.float32)
+        dims = (C.c_int * 8)()
+        nd = C.c_int(0)
+        self._check(load().tnn_host_get_output(self._h, name.encode(), buf.ctypes.data_as(C.c_void_p), max_elems, dims,
+                                               C.byref(nd)), "GetOutputMat")
+        shape = [dims[i] for i in range(nd.value)]
+        return buf[:int(np.prod(shape, dtype=np.int64))].reshape(shape).copy()
+
+    def layers(self):
+        text = load().tnn_host_layer_summary(self._h).decode()
+        return [tuple(line.split(" ", 1)) for line in text.splitlines() if line]
+
+    def profile(self, iters=10):
+        """per-layer mean milliseconds over `iters` forwards (hipEvent timing on the instance's stream)"""
+        lib = load()
+        lib.tnn_host_profile_start(self._h)
+        for _ in range(iters):
+            self.forward()
+        n = lib.tnn_host_layer_count(self._h)
+        ms = (C.c_double * n)()
+        lib.tnn_host_profile_finish(self._h, ms, n)
+        return [(t, nm, ms[i]) for i, (t, nm) in enumerate(self.layers())]
+
+    def close(self):
+        if getattr(self, "_h", None):
+            load().tnn_host_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

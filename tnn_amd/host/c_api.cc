@@ -1,0 +1,133 @@
+// C entry points over the host (Instance on DEVICE_ROCM) for drivers written in other languages:
+// the Python bench and tests create an instance from proto text + model bytes, feed host arrays,
+// call Forward and read outputs back — the same sequence as the engine's TNNTest
+// (test/test.cc:101-152: ConvertFromMat -> Forward -> ConvertToMat).
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "tnn_host.h"
+#include "tnn_rocm.h"
+
+using namespace TNN_NS;
+
+namespace {
+struct Handle {
+    std::shared_ptr<Instance> inst;
+    std::string err;
+    std::string summary;
+};
+int fail(Handle *h, const Status &st) {
+    h->err = st.description();
+    return (int)st == 0 ? -1 : (int)st;
+}
+}  // namespace
+
+extern "C" {
+#define HOST_API __attribute__((visibility("default")))
+
+// precision: 0 = fp32 blobs (PRECISION_HIGH), 1 = fp16 activations (PRECISION_AUTO).  Returns NULL on failure and
+// writes the status text to err.
+HOST_API void *tnn_host_create(const char *proto, size_t proto_len, const char *model, size_t model_len, int device_id,
+                               int precision, char *err, size_t err_len) {
+    auto h = new Handle;
+    NetworkConfig nc;
+    nc.device_type = DEVICE_ROCM;
+    nc.device_id   = device_id;
+    nc.precision   = precision == 0 ? PRECISION_HIGH : PRECISION_AUTO;
+    ModelConfig mc;
+    mc.params.push_back(std::string(proto, proto_len));
+    mc.params.push_back(std::string(model, model_len));
+    h->inst   = std::make_shared<Instance>(nc, mc);
+    Status st = h->inst->Init();
+    if (st != TNN_OK) {
+        if (err && err_len)
+            snprintf(err, err_len, "%s", st.description().c_str());
+        delete h;
+        return nullptr;
+    }
+    return h;
+}
+
+HOST_API void tnn_host_destroy(void *hp) { delete static_cast<Handle *>(hp); }
+HOST_API const char *tnn_host_last_error(void *hp) { return static_cast<Handle *>(hp)->err.c_str(); }
+
+// mat_type: 0 NCHW_FLOAT (fp32 host data), 1 NC_INT32
+HOST_API int tnn_host_set_input(void *hp, const char *name, const void *data, int mat_type, const int *dims, int ndims) {
+    auto h = static_cast<Handle *>(hp);
+    DimsVector d(dims, dims + ndims);
+    auto mat  = std::make_shared<Mat>(DEVICE_NAIVE, mat_type == 1 ? NC_INT32 : NCHW_FLOAT, d, const_cast<void *>(data));
+    Status st = h->inst->SetInputMat(mat, MatConvertParam(), name ? name : "");
+    return st == TNN_OK ? 0 : fail(h, st);
+}
+
+HOST_API int tnn_host_forward(void *hp) {
+    auto h    = static_cast<Handle *>(hp);
+    Status st = h->inst->Forward();
+    return st == TNN_OK ? 0 : fail(h, st);
+}
+
+// enqueue only; pair with tnn_host_sync
+HOST_API int tnn_host_forward_async(void *hp) {
+    auto h    = static_cast<Handle *>(hp);
+    Status st = h->inst->ForwardAsync();
+    return st == TNN_OK ? 0 : fail(h, st);
+}
+
+HOST_API int tnn_host_sync(void *hp) {
+    auto h  = static_cast<Handle *>(hp);
+    void *q = nullptr;
+    h->inst->GetCommandQueue(&q);
+    int rc = tnn_rocm_stream_sync(q);
+    if (rc != 0)
+        h->err = tnn_rocm_last_error();
+    return rc;
+}
+
+HOST_API void *tnn_host_stream(void *hp) {
+    void *q = nullptr;
+    static_cast<Handle *>(hp)->inst->GetCommandQueue(&q);
+    return q;
+}
+
+HOST_API int tnn_host_get_output(void *hp, const char *name, float *out, size_t capacity, int *dims, int *ndims) {
+    auto h = static_cast<Handle *>(hp);
+    std::shared_ptr<Mat> mat;
+    Status st = h->inst->GetOutputMat(mat, MatConvertParam(), name ? name : "", DEVICE_NAIVE, NCHW_FLOAT);
+    if (st != TNN_OK)
+        return fail(h, st);
+    DimsVector d = mat->GetDims();
+    size_t count = (size_t)DimsVectorUtils::Count(d);
+    if (ndims)
+        *ndims = (int)d.size();
+    if (dims)
+        for (size_t i = 0; i < d.size() && i < 8; ++i)
+            dims[i] = d[i];
+    if (count > capacity) {
+        h->err = "output buffer too small";
+        return -2;
+    }
+    memcpy(out, mat->GetData(), count * sizeof(float));
+    return 0;
+}
+
+HOST_API int tnn_host_layer_count(void *hp) { return static_cast<Handle *>(hp)->inst->GetNetwork()->LayerCount(); }
+
+// "Type name\n" per layer of the optimised graph
+HOST_API const char *tnn_host_layer_summary(void *hp) {
+    auto h     = static_cast<Handle *>(hp);
+    h->summary = h->inst->GetNetwork()->LayerSummary();
+    return h->summary.c_str();
+}
+
+HOST_API void tnn_host_profile_start(void *hp) { static_cast<Handle *>(hp)->inst->GetNetwork()->StartProfile(); }
+
+// Fills up to `capacity` entries with the per-layer mean milliseconds since tnn_host_profile_start; returns the
+// number of layers.  Names come from tnn_host_layer_summary (same order).
+HOST_API int tnn_host_profile_finish(void *hp, double *ms, int capacity) {
+    auto prof = static_cast<Handle *>(hp)->inst->GetNetwork()->FinishProfile();
+    for (int i = 0; i < (int)prof.size() && i < capacity; ++i)
+        ms[i] = prof[i].calls > 0 ? prof[i].ms / prof[i].calls : 0.0;
+    return (int)prof.size();
+}
+}

@@ -1,0 +1,400 @@
+// RocmDevice / RocmContext / RocmLayerAcc / RocmBlobConverterAcc.
+#include "rocm_device.h"
+
+#include <cstdio>
+
+namespace TNN_NS {
+
+Status RocmStatus(int rc, int tnn_code, const char *what) {
+    char buf[768];
+    snprintf(buf, sizeof(buf), "%s failed (%d): %s", what, rc, tnn_rocm_last_error());
+    // hipErrorOutOfMemory == 2
+    return Status(rc == 2 ? (int)TNNERR_OUTOFMEMORY : tnn_code, buf);
+}
+
+// ---- context --------------------------------------------------------------------------------
+RocmContext::RocmContext(int device_id) : device_id_(device_id) {}
+
+Status RocmContext::Setup() {
+    int n = 0;
+    tnn_rocm_device_count(&n);
+    if (device_id_ < 0 || device_id_ >= n)
+        return Status(TNNERR_DEVICE_CONTEXT_CREATE, "no ROCm device with the requested id");
+    if (tnn_rocm_set_device(device_id_) != 0 || tnn_rocm_stream_create(&stream_) != 0)
+        return RocmStatus(-1, TNNERR_DEVICE_CONTEXT_CREATE, "stream creation");
+    void *flag = nullptr;
+    if (tnn_rocm_malloc_host(&flag, 64) != 0)
+        return RocmStatus(-1, TNNERR_DEVICE_CONTEXT_CREATE, "error flag allocation");
+    error_flag_ = (int32_t *)flag;
+    return TNN_OK;
+}
+
+RocmContext::~RocmContext() {
+    if (stream_)
+        tnn_rocm_stream_sync(stream_);
+    tnn_rocm_free(workspace_);
+    tnn_rocm_free_host(error_flag_);
+    tnn_rocm_stream_destroy(stream_);
+}
+
+Status RocmContext::GetCommandQueue(void **command_queue) {
+    if (!command_queue)
+        return Status(TNNERR_DEVICE_INVALID_COMMAND_QUEUE, "command_queue is nil");
+    *command_queue = stream_;
+    return TNN_OK;
+}
+
+Status RocmContext::OnInstanceForwardBegin() {
+    // one context per instance, used by one thread at a time; select its device for this thread
+    ROCM_CALL(tnn_rocm_set_device(device_id_));
+    return TNN_OK;
+}
+
+Status RocmContext::Synchronize() {
+    int rc = tnn_rocm_stream_sync(stream_);
+    if (rc != 0)
+        return RocmStatus(rc, TNNERR_CUDA_SYNC_ERROR, "stream synchronize");
+    if (error_flag_ && *error_flag_ != 0) {
+        *error_flag_ = 0;
+        // cpu_gather_layer_acc.cc:72-78 reports this as TNNERR_MODEL_ERR
+        return Status(TNNERR_MODEL_ERR, "RocmGatherLayerAcc::Forward invalid slice_index");
+    }
+    return TNN_OK;
+}
+
+Status RocmContext::Workspace(size_t bytes, void **ptr) {
+    if (bytes > workspace_sz_) {
+        ROCM_CALL(tnn_rocm_stream_sync(stream_));
+        tnn_rocm_free(workspace_);
+        workspace_    = nullptr;
+        workspace_sz_ = 0;
+        size_t want   = bytes + bytes / 4;
+        int rc        = tnn_rocm_malloc(&workspace_, want);
+        if (rc != 0)
+            return RocmStatus(rc, TNNERR_OUTOFMEMORY, "workspace allocation");
+        workspace_sz_ = want;
+    }
+    *ptr = workspace_;
+    return TNN_OK;
+}
+
+// ---- device ---------------------------------------------------------------------------------
+std::map<LayerType, std::shared_ptr<LayerAccCreator>> &RocmDevice::GetLayerCreatorMap() {
+    static std::map<LayerType, std::shared_ptr<LayerAccCreator>> m;
+    return m;
+}
+Status RocmDevice::RegisterLayerAccCreator(LayerType type, LayerAccCreator *creator) {
+    GetLayerCreatorMap()[type] = std::shared_ptr<LayerAccCreator>(creator);
+    return TNN_OK;
+}
+AbstractLayerAcc *RocmDevice::CreateLayerAcc(LayerType type) {
+    auto &m = GetLayerCreatorMap();
+    auto it = m.find(type);
+    return it == m.end() ? nullptr : it->second->CreateLayerAcc(type);
+}
+Context *RocmDevice::CreateContext(int device_id) {
+    auto ctx = new RocmContext(device_id);
+    if (ctx->Setup() != TNN_OK) {
+        delete ctx;
+        return nullptr;
+    }
+    return ctx;
+}
+std::shared_ptr<const ImplementedPrecision> RocmDevice::GetImplementedPrecision(LayerType) {
+    auto p               = std::make_shared<ImplementedPrecision>();
+    p->fp32_implemented  = true;
+    p->fp16_implemented  = true;
+    p->bfp16_implemented = false;
+    return p;
+}
+BlobMemorySizeInfo RocmDevice::Calculate(BlobDesc &desc) {
+    // plain row-major ("NCHW" of any rank) in the blob's own data type; int8 blobs are NOT padded to
+    // NHWC4 as on x86 (x86_device.cc:27-38): every channel count on this path is a multiple of 4
+    BlobMemorySizeInfo info;
+    info.data_type = desc.data_type;
+    info.dims      = desc.dims;
+    if (info.dims.empty())
+        info.dims = {1};
+    return info;
+}
+Status RocmDevice::Allocate(void **handle, MatType mat_type, DimsVector dims) {
+    BlobMemorySizeInfo info;
+    info.data_type = (mat_type == NCHW_FLOAT) ? DATA_TYPE_FLOAT : (mat_type == NC_INT32 ? DATA_TYPE_INT32 : DATA_TYPE_INT8);
+    info.dims      = dims;
+    return Allocate(handle, info);
+}
+Status RocmDevice::Allocate(void **handle, BlobMemorySizeInfo &size_info) {
+    if (!handle)
+        return Status(TNNERR_NULL_PARAM, "handle is nil");
+    int64_t bytes = GetBlobMemoryBytesSize(size_info);
+    if (bytes < 0)
+        return Status(TNNERR_PARAM_ERR, "negative blob size");
+    int rc = tnn_rocm_malloc(handle, (size_t)(bytes > 0 ? bytes : 16));
+    if (rc != 0)
+        return RocmStatus(rc, TNNERR_OUTOFMEMORY, "hipMalloc");
+    return TNN_OK;
+}
+Status RocmDevice::Free(void *handle) {
+    int rc = tnn_rocm_free(handle);
+    return rc == 0 ? Status(TNN_OK) : RocmStatus(rc, TNNERR_COMMON_ERROR, "hipFree");
+}
+Status RocmDevice::CopyToDevice(BlobHandle *dst, const BlobHandle *src, BlobDesc &desc, void *q) {
+    auto info  = Calculate(desc);
+    int rc     = tnn_rocm_memcpy_h2d((char *)dst->base + dst->bytes_offset, (const char *)src->base + src->bytes_offset,
+                                     (size_t)GetBlobMemoryBytesSize(info), q);
+    return rc == 0 ? Status(TNN_OK) : RocmStatus(rc, TNNERR_CUDA_MEMCPY_ERROR, "host to device copy");
+}
+Status RocmDevice::CopyFromDevice(BlobHandle *dst, const BlobHandle *src, BlobDesc &desc, void *q) {
+    auto info = Calculate(desc);
+    int rc    = tnn_rocm_memcpy_d2h((char *)dst->base + dst->bytes_offset, (const char *)src->base + src->bytes_offset,
+                                    (size_t)GetBlobMemoryBytesSize(info), q);
+    return rc == 0 ? Status(TNN_OK) : RocmStatus(rc, TNNERR_CUDA_MEMCPY_ERROR, "device to host copy");
+}
+
+static TypeDeviceRegister<RocmDevice> g_rocm_device_register(DEVICE_ROCM);
+
+// ---- layer acc base -----------------------------------------------------------------------------
+RocmLayerAcc::~RocmLayerAcc() {
+    for (void *p : owned_device_)
+        tnn_rocm_free(p);
+}
+Status RocmLayerAcc::Init(Context *context, LayerParam *param, LayerResource *resource,
+                          const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) {
+    context_ = dynamic_cast<RocmContext *>(context);
+    if (!context_)
+        return Status(TNNERR_NULL_PARAM, "RocmLayerAcc needs a RocmContext");
+    param_    = param;
+    resource_ = resource;
+    return ReloadConstantBlobs(inputs, false);
+}
+std::vector<DataFormat> RocmLayerAcc::SupportDataFormat(DataType, int, BlobType) {
+    // row-major for every rank, as the naive device does (cpu_layer_acc.cc:70-78)
+    return {DATA_FORMAT_NCHW};
+}
+DataType RocmLayerAcc::ConstantBlobDataType(const std::vector<Blob *> &inputs, int) {
+    for (auto b : inputs)
+        if (!b->IsConstant())
+            return b->GetBlobDesc().data_type;
+    return DATA_TYPE_FLOAT;
+}
+Status RocmLayerAcc::UploadConverted(const void *host, size_t count, DataType src, DataType dst, void **out) {
+    size_t sb = (size_t)DataTypeUtils::GetBytesSize(src), db = (size_t)DataTypeUtils::GetBytesSize(dst);
+    void *dev = nullptr;
+    int rc    = tnn_rocm_malloc(&dev, count * db > 0 ? count * db : 16);
+    if (rc != 0)
+        return RocmStatus(rc, TNNERR_OUTOFMEMORY, "constant upload");
+    owned_device_.push_back(dev);
+    *out = dev;
+    if (count == 0)
+        return TNN_OK;
+    if (src == dst) {
+        ROCM_CALL(tnn_rocm_memcpy_h2d(dev, host, count * sb, Stream()));
+        return TNN_OK;
+    }
+    bool s_float = src == DATA_TYPE_FLOAT || src == DATA_TYPE_HALF || src == DATA_TYPE_BFP16;
+    bool d_float = dst == DATA_TYPE_FLOAT || dst == DATA_TYPE_HALF || dst == DATA_TYPE_BFP16;
+    if (!s_float || !d_float)
+        return Status(TNNERR_PARAM_ERR, "constant conversion between non-float types");
+    void *tmp = nullptr;
+    rc        = tnn_rocm_malloc(&tmp, count * sb);
+    if (rc != 0)
+        return RocmStatus(rc, TNNERR_OUTOFMEMORY, "constant staging");
+    rc = tnn_rocm_memcpy_h2d(tmp, host, count * sb, Stream());
+    if (rc == 0)
+        rc = tnn_rocm_cast(Stream(), (int)src, tmp, (int)dst, dev, count);
+    if (rc == 0)
+        rc = tnn_rocm_stream_sync(Stream());
+    tnn_rocm_free(tmp);
+    return rc == 0 ? Status(TNN_OK) : RocmStatus(rc, TNNERR_CUDA_MEMCPY_ERROR, "constant conversion");
+}
+Status RocmLayerAcc::ReloadConstantBlobs(const std::vector<Blob *> &inputs, bool only_reload_shape_differ_blob) {
+    if (!const_resource_ || only_reload_shape_differ_blob)
+        return TNN_OK;
+    for (int i = 0; i < (int)inputs.size(); ++i) {
+        Blob *b   = inputs[i];
+        auto it   = const_resource_->find(b->GetBlobDesc().name);
+        if (it == const_resource_->end() || !b->IsConstant())
+            continue;
+        if (const_blob_map_.count(b->GetBlobDesc().name))
+            continue;
+        auto &buf    = *it->second;
+        DataType dst = ConstantBlobDataType(inputs, i);
+        if (buf.GetDataType() == DATA_TYPE_INT32 || buf.GetDataType() == DATA_TYPE_INT8)
+            dst = buf.GetDataType();
+        // a constant shared by several layers may need different storage types, so each acc keeps
+        // its own device copy and publishes it through a blob of its own
+        void *dev = nullptr;
+        RETURN_ON_NEQ(UploadConverted(buf.force_to<void *>(), (size_t)buf.GetDataCount(), buf.GetDataType(), dst, &dev),
+                      TNN_OK);
+        BlobDesc desc  = b->GetBlobDesc();
+        desc.data_type = dst;
+        BlobHandle h;
+        h.base = dev;
+        const_blob_map_[desc.name] = std::make_shared<Blob>(desc, h);
+    }
+    return TNN_OK;
+}
+
+// ---- blob converter (role of source/tnn/device/cuda/cuda_blob_converter.cc:36-234) -------------------
+class RocmBlobConverterAcc : public BlobConverterAcc {
+public:
+    explicit RocmBlobConverterAcc(Blob *blob) : BlobConverterAcc(blob) {}
+    ~RocmBlobConverterAcc() override { tnn_rocm_free(staging_); }
+
+    Status ConvertFromMat(Mat &mat, MatConvertParam param, void *q) override {
+        RETURN_ON_NEQ(ConvertFromMatAsync(mat, param, q), TNN_OK);
+        ROCM_CALL(tnn_rocm_stream_sync(q));
+        return TNN_OK;
+    }
+    Status ConvertToMat(Mat &mat, MatConvertParam param, void *q) override {
+        // the device-to-host copy below blocks until the data has arrived
+        return ConvertToMatAsync(mat, param, q);
+    }
+
+    Status ConvertFromMatAsync(Mat &mat, MatConvertParam param, void *q) override {
+        auto &desc   = blob_->GetBlobDesc();
+        size_t count = (size_t)DimsVectorUtils::Count(desc.dims);
+        if (mat.GetDeviceType() != DEVICE_NAIVE)
+            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: only host mats are supported");
+        if ((size_t)DimsVectorUtils::Count(mat.GetDims()) != count)
+            return Status(TNNERR_INVALID_INPUT, "mat and blob element counts differ");
+        void *dst = (char *)blob_->GetHandle().base + blob_->GetHandle().bytes_offset;
+        if (count == 0)
+            return TNN_OK;
+        if (mat.GetMatType() == NC_INT32) {
+            if (desc.data_type != DATA_TYPE_INT32)
+                return Status(TNNERR_PARAM_ERR, "NC_INT32 mat needs an int32 blob");
+            ROCM_CALL(tnn_rocm_memcpy_h2d(dst, mat.GetData(), count * 4, q));
+            return TNN_OK;
+        }
+        if (mat.GetMatType() == RESERVED_INT8_TEST) {
+            if (desc.data_type != DATA_TYPE_INT8)
+                return Status(TNNERR_PARAM_ERR, "int8 mat needs an int8 blob");
+            ROCM_CALL(tnn_rocm_memcpy_h2d(dst, mat.GetData(), count, q));
+            return TNN_OK;
+        }
+        if (mat.GetMatType() != NCHW_FLOAT)
+            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported mat type");
+        const float *src = (const float *)mat.GetData();
+        std::vector<float> scaled;
+        if (NeedsScaleBias(param, desc.dims)) {  // per-channel x*scale+bias over dims[1] (blob_converter_default.cc:281-291)
+            scaled.resize(count);
+            ApplyScaleBias(src, scaled.data(), desc.dims, param);
+            src = scaled.data();
+        }
+        if (desc.data_type == DATA_TYPE_FLOAT) {
+            ROCM_CALL(tnn_rocm_memcpy_h2d(dst, src, count * 4, q));
+            return TNN_OK;
+        }
+        RETURN_ON_NEQ(Staging(count * 4), TNN_OK);
+        ROCM_CALL(tnn_rocm_memcpy_h2d(staging_, src, count * 4, q));
+        if (desc.data_type == DATA_TYPE_HALF || desc.data_type == DATA_TYPE_BFP16) {
+            ROCM_CALL(tnn_rocm_cast(q, TNN_ROCM_F32, staging_, (int)desc.data_type, dst, count));
+        } else if (desc.data_type == DATA_TYPE_INT8) {
+            // float mat into an int8 blob goes through the blob's scale (blob_converter_default.cc:396-403),
+            // with the reciprocal-multiply quantiser of the x86 path
+            auto bi = dynamic_cast<BlobInt8 *>(blob_);
+            if (!bi || !bi->GetIntResource() || bi->GetIntResource()->scale_handle.GetDataCount() < 1)
+                return Status(TNNERR_NULL_PARAM, "int8 blob without scale resource");
+            float s   = bi->GetIntResource()->scale_handle.force_to<float *>()[0];
+            float inv = (float)(1.0 / s);
+            ROCM_CALL(tnn_rocm_quantize(q, TNN_ROCM_F32, staging_, inv, (int8_t *)dst, count));
+        } else {
+            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported blob data type");
+        }
+        return TNN_OK;
+    }
+
+    Status ConvertToMatAsync(Mat &mat, MatConvertParam param, void *q) override {
+        auto &desc   = blob_->GetBlobDesc();
+        size_t count = (size_t)DimsVectorUtils::Count(desc.dims);
+        if ((size_t)DimsVectorUtils::Count(mat.GetDims()) != count)
+            return Status(TNNERR_INVALID_INPUT, "mat and blob element counts differ");
+        void *src = (char *)blob_->GetHandle().base + blob_->GetHandle().bytes_offset;
+        if (count == 0)
+            return TNN_OK;
+        if (mat.GetMatType() == NC_INT32 && desc.data_type == DATA_TYPE_INT32) {
+            ROCM_CALL(tnn_rocm_memcpy_d2h(mat.GetData(), src, count * 4, q));
+            return TNN_OK;
+        }
+        if (mat.GetMatType() == RESERVED_INT8_TEST && desc.data_type == DATA_TYPE_INT8) {
+            ROCM_CALL(tnn_rocm_memcpy_d2h(mat.GetData(), src, count, q));
+            return TNN_OK;
+        }
+        if (mat.GetMatType() != NCHW_FLOAT)
+            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported mat type");
+        if (desc.data_type == DATA_TYPE_FLOAT) {
+            ROCM_CALL(tnn_rocm_memcpy_d2h(mat.GetData(), src, count * 4, q));
+        } else {
+            RETURN_ON_NEQ(Staging(count * 4), TNN_OK);
+            if (desc.data_type == DATA_TYPE_HALF || desc.data_type == DATA_TYPE_BFP16) {
+                ROCM_CALL(tnn_rocm_cast(q, (int)desc.data_type, src, TNN_ROCM_F32, staging_, count));
+            } else if (desc.data_type == DATA_TYPE_INT8) {
+                auto bi = dynamic_cast<BlobInt8 *>(blob_);
+                if (!bi || !bi->GetIntResource() || bi->GetIntResource()->scale_handle.GetDataCount() < 1)
+                    return Status(TNNERR_NULL_PARAM, "int8 blob without scale resource");
+                float s = bi->GetIntResource()->scale_handle.force_to<float *>()[0];
+                ROCM_CALL(tnn_rocm_dequantize(q, (const int8_t *)src, s, TNN_ROCM_F32, staging_, count));
+            } else {
+                return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported blob data type");
+            }
+            ROCM_CALL(tnn_rocm_memcpy_d2h(mat.GetData(), staging_, count * 4, q));
+        }
+        if (NeedsScaleBias(param, desc.dims)) {
+            std::vector<float> tmp(count);
+            ApplyScaleBias((const float *)mat.GetData(), tmp.data(), desc.dims, param);
+            memcpy(mat.GetData(), tmp.data(), count * 4);
+        }
+        return TNN_OK;
+    }
+
+private:
+    static bool NeedsScaleBias(const MatConvertParam &p, const DimsVector &dims) {
+        for (float s : p.scale)
+            if (s != 1.0f)
+                return true;
+        for (float b : p.bias)
+            if (b != 0.0f)
+                return true;
+        (void)dims;
+        return false;
+    }
+    static void ApplyScaleBias(const float *src, float *dst, const DimsVector &dims, const MatConvertParam &p) {
+        int n = dims.size() > 0 ? dims[0] : 1, c = dims.size() > 1 ? dims[1] : 1;
+        int hw = DimsVectorUtils::Count(dims, 2);
+        for (int i = 0; i < n; ++i)
+            for (int j = 0; j < c; ++j) {
+                float s = j < (int)p.scale.size() ? p.scale[j] : 1.0f;
+                float b = j < (int)p.bias.size() ? p.bias[j] : 0.0f;
+                for (int k = 0; k < hw; ++k) {
+                    size_t o = ((size_t)i * c + j) * hw + k;
+                    dst[o]   = src[o] * s + b;
+                }
+            }
+    }
+    Status Staging(size_t bytes) {
+        if (bytes > staging_sz_) {
+            tnn_rocm_free(staging_);
+            staging_    = nullptr;
+            staging_sz_ = 0;
+            int rc      = tnn_rocm_malloc(&staging_, bytes);
+            if (rc != 0)
+                return RocmStatus(rc, TNNERR_OUTOFMEMORY, "converter staging");
+            staging_sz_ = bytes;
+        }
+        return TNN_OK;
+    }
+    void *staging_     = nullptr;
+    size_t staging_sz_ = 0;
+};
+
+class RocmBlobConverterAccCreater : public BlobConverterAccCreater {
+    std::shared_ptr<BlobConverterAcc> CreateBlobConverterAcc(Blob *blob) override {
+        return std::make_shared<RocmBlobConverterAcc>(blob);
+    }
+};
+static struct RegisterRocmConverter {
+    RegisterRocmConverter() { GetBlobConverterCreaterMap()[DEVICE_ROCM] = std::make_shared<RocmBlobConverterAccCreater>(); }
+} g_register_rocm_converter;
+
+}  // namespace TNN_NS

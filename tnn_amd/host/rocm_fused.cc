@@ -1,0 +1,526 @@
+// The ROCm-only graph rewrite and the two fused layers it produces.
+//
+// The engine runs a transformer encoder layer as ~45 separate ops (MatMul, Add, Reshape, Permute, MatMul,
+// Mul, Add, Softmax, MatMul, ... one AbstractLayerAcc::Forward each: source/tnn/core/default_network.cc:571-631).
+// This pass, registered like the engine's own optimizers (source/tnn/optimizer/net_optimizer_manager.h:32-66,
+// gated on the device like net_optimizer_insert_int8_reformat.cc:41-45) and run on the instance's private
+// copy of the graph, collapses them into
+//   RocmFusedLinear    : y = act(x W^T + b) (+ residual)     <- MatMul(weight)+Add(bias) [+GELU] [+Add(residual)]
+//                                                               or InnerProduct
+//   RocmFusedAttention : ctx = softmax(QK^T*scale + mask)V    <- three projections, head split, MatMul, Mul/Div,
+//                        with Q,K,V = x Wqkv^T + bqkv            Add(mask), Softmax, MatMul, head merge
+// so that a BERT layer becomes 7 launches.  A sub-graph is only rewritten when every intermediate blob has a
+// single reader and is not a model output; anything that does not match is left as it is.
+#include <algorithm>
+#include <cmath>
+
+#include "rocm_device.h"
+
+namespace TNN_NS {
+
+namespace {
+
+struct GraphIndex {
+    std::map<std::string, int> producer;
+    std::map<std::string, std::vector<int>> consumers;
+    explicit GraphIndex(const std::vector<std::shared_ptr<LayerInfo>> &layers) {
+        for (int i = 0; i < (int)layers.size(); ++i) {
+            if (!layers[i])
+                continue;
+            for (auto &o : layers[i]->outputs)
+                producer[o] = i;
+            for (auto &in : layers[i]->inputs)
+                consumers[in].push_back(i);
+        }
+    }
+    int sole_consumer(const std::string &blob) const {
+        auto it = consumers.find(blob);
+        return (it == consumers.end() || it->second.size() != 1) ? -1 : it->second[0];
+    }
+    int producer_of(const std::string &blob) const {
+        auto it = producer.find(blob);
+        return it == producer.end() ? -1 : it->second;
+    }
+};
+
+class RocmFusionPass : public NetOptimizer {
+public:
+    std::string Strategy() override { return "net_optimizer_rocm_fuse_encoder"; }
+    bool IsSupported(const NetworkConfig &c) override {
+        half_ = c.precision != PRECISION_HIGH;
+        return c.device_type == DEVICE_ROCM;
+    }
+
+    Status Optimize(NetStructure *s, NetResource *r) override {
+        structure_ = s;
+        resource_  = r;
+        FuseLinear();
+        FoldGelu();
+        FoldResidual();
+        if (half_)
+            FuseAttention();  // the attention kernel computes in fp16; fp32 nets keep the decomposed core
+        return TNN_OK;
+    }
+
+private:
+    bool IsModelOutput(const std::string &b) const { return structure_->outputs.count(b) > 0; }
+    void Compact() {
+        auto &L = structure_->layers;
+        L.erase(std::remove(L.begin(), L.end(), nullptr), L.end());
+    }
+    template <typename T> T *ParamOf(const std::shared_ptr<LayerInfo> &l) { return dynamic_cast<T *>(l->param.get()); }
+    template <typename T> T *ResOf(const std::string &name) {
+        auto it = resource_->resource_map.find(name);
+        return it == resource_->resource_map.end() ? nullptr : dynamic_cast<T *>(it->second.get());
+    }
+
+    std::shared_ptr<LayerInfo> MakeLinear(const std::string &name, const std::string &in, const std::string &out, int N,
+                                          int K, const float *w_nk_or_null, const float *w_kn_or_null, const float *bias,
+                                          bool has_bias) {
+        auto l       = std::make_shared<LayerInfo>();
+        l->type      = LAYER_ROCM_FUSED_LINEAR;
+        l->type_str  = "RocmFusedLinear";
+        l->name      = name;
+        l->inputs    = {in};
+        l->outputs   = {out};
+        auto p       = std::make_shared<RocmFusedLinearParam>();
+        p->type      = l->type_str;
+        p->name      = name;
+        p->num_output = N;
+        p->has_bias  = has_bias ? 1 : 0;
+        l->param     = p;
+        auto res     = std::make_shared<RocmFusedLinearResource>();
+        res->name    = name;
+        res->weight_nk = RawBuffer(N * K * 4, {N, K});
+        float *w     = res->weight_nk.force_to<float *>();
+        if (w_nk_or_null) {
+            memcpy(w, w_nk_or_null, (size_t)N * K * 4);
+        } else {
+            for (int k = 0; k < K; ++k)
+                for (int n = 0; n < N; ++n)
+                    w[(size_t)n * K + k] = w_kn_or_null[(size_t)k * N + n];
+        }
+        if (has_bias) {
+            res->bias = RawBuffer(N * 4, {N});
+            memcpy(res->bias.force_to<float *>(), bias, (size_t)N * 4);
+        }
+        resource_->resource_map[name] = res;
+        return l;
+    }
+
+    // MatMul(weight_position=1, fp32 [K,N] resource) -> Add(bias resource of N values)   ==> RocmFusedLinear
+    // InnerProduct (float, axis = last)                                                 ==> RocmFusedLinear
+    void FuseLinear() {
+        auto &L = structure_->layers;
+        GraphIndex g(L);
+        for (int i = 0; i < (int)L.size(); ++i) {
+            auto l = L[i];
+            if (!l)
+                continue;
+            if (l->type == LAYER_MATMUL && l->inputs.size() == 1) {
+                auto mp = ParamOf<MatMulLayerParam>(l);
+                auto mr = ResOf<MatMulLayerResource>(l->name);
+                if (!mp || !mr || mp->weight_position != 1 || mr->weight.GetDataType() != DATA_TYPE_FLOAT)
+                    continue;
+                auto wd = mr->weight.GetBufferDims();
+                if (wd.size() != 2)
+                    continue;
+                int K = wd[0], N = wd[1];
+                const std::string &mid = l->outputs[0];
+                int j = g.sole_consumer(mid);
+                const float *bias = nullptr;
+                std::string out   = mid;
+                if (j > i && L[j] && L[j]->type == LAYER_ADD && L[j]->inputs.size() == 1 && !IsModelOutput(mid)) {
+                    auto ar = ResOf<EltwiseLayerResource>(L[j]->name);
+                    if (ar && ar->element_handle.GetDataType() == DATA_TYPE_FLOAT && ar->element_handle.GetDataCount() == N) {
+                        auto ad = ar->element_handle.GetBufferDims();
+                        if (ad.empty() || ad.back() == N) {  // a vector over the last axis
+                            bias = ar->element_handle.force_to<float *>();
+                            out  = L[j]->outputs[0];
+                        }
+                    }
+                }
+                auto fused = MakeLinear(l->name + "_fused", l->inputs[0], out, N, K, nullptr,
+                                        mr->weight.force_to<float *>(), bias, bias != nullptr);
+                L[i] = fused;
+                if (bias)
+                    L[j] = nullptr;
+            } else if (l->type == LAYER_INNER_PRODUCT && !l->param->quantized) {
+                auto ip = ParamOf<InnerProductLayerParam>(l);
+                auto ir = ResOf<InnerProductLayerResource>(l->name);
+                if (!ip || !ir || ir->weight_handle.GetDataType() != DATA_TYPE_FLOAT || ip->transpose != 0)
+                    continue;
+                int N = ip->num_output;
+                if (N <= 0 || ir->weight_handle.GetDataCount() % N != 0)
+                    continue;
+                int K = ir->weight_handle.GetDataCount() / N;
+                // only the "last axis" form is a row-wise linear map; shapes are not known here, so require the
+                // usual exported forms axis = 1 on [T,K] blobs (checked again by the layer's shape inference)
+                if (ip->axis != 1)
+                    continue;
+                bool hb = ip->has_bias && ir->bias_handle.GetDataCount() == N &&
+                          ir->bias_handle.GetDataType() == DATA_TYPE_FLOAT;
+                auto fused = MakeLinear(l->name + "_fused", l->inputs[0], l->outputs[0], N, K,
+                                        ir->weight_handle.force_to<float *>(), nullptr,
+                                        hb ? ir->bias_handle.force_to<float *>() : nullptr, hb);
+                ParamOf<RocmFusedLinearParam>(fused)->axis = ip->axis;
+                L[i] = fused;
+            }
+        }
+        Compact();
+    }
+
+    void FoldGelu() {
+        auto &L = structure_->layers;
+        GraphIndex g(L);
+        for (int i = 0; i < (int)L.size(); ++i) {
+            auto l = L[i];
+            if (!l || l->type != LAYER_ROCM_FUSED_LINEAR)
+                continue;
+            int j = g.sole_consumer(l->outputs[0]);
+            if (j > i && L[j] && L[j]->type == LAYER_GELU && !IsModelOutput(l->outputs[0])) {
+                ParamOf<RocmFusedLinearParam>(l)->gelu = 1;
+                l->outputs[0]                           = L[j]->outputs[0];
+                L[j]                                    = nullptr;
+            }
+        }
+        Compact();
+    }
+
+    void FoldResidual() {
+        auto &L = structure_->layers;
+        GraphIndex g(L);
+        for (int i = 0; i < (int)L.size(); ++i) {
+            auto l = L[i];
+            if (!l || l->type != LAYER_ROCM_FUSED_LINEAR)
+                continue;
+            auto p = ParamOf<RocmFusedLinearParam>(l);
+            if (p->gelu || p->has_residual || IsModelOutput(l->outputs[0]))
+                continue;
+            int j = g.sole_consumer(l->outputs[0]);
+            if (j <= i || !L[j] || L[j]->type != LAYER_ADD || L[j]->inputs.size() != 2 || L[j]->param->quantized ||
+                ResOf<EltwiseLayerResource>(L[j]->name))
+                continue;
+            const std::string &other = L[j]->inputs[0] == l->outputs[0] ? L[j]->inputs[1] : L[j]->inputs[0];
+            if (other == l->outputs[0])
+                continue;
+            int po = g.producer_of(other);
+            bool available = po >= 0 ? po < i : structure_->inputs_shape_map.count(other) > 0;
+            if (!available)
+                continue;
+            // the residual must have the linear's output shape; the layer's Init re-checks this
+            p->has_residual = 1;
+            l->inputs.push_back(other);
+            l->outputs[0] = L[j]->outputs[0];
+            L[j]          = nullptr;
+        }
+        Compact();
+    }
+
+    // follow `blob` back through Reshape(-> rank 3/4 head split) and Permute(order) to a fused linear on x
+    int HeadSplitSource(const GraphIndex &g, const std::string &blob, const std::vector<int> &order4,
+                        const std::vector<int> &order3, std::vector<int> *chain, DimsVector *split_shape) {
+        auto &L = structure_->layers;
+        int pi  = g.producer_of(blob);
+        if (pi < 0 || !L[pi] || L[pi]->type != LAYER_PERMUTE || g.sole_consumer(blob) < 0 || IsModelOutput(blob))
+            return -1;
+        auto pp = ParamOf<PermuteLayerParam>(L[pi]);
+        if (!pp || (pp->orders != order4 && pp->orders != order3))
+            return -1;
+        const std::string &rb = L[pi]->inputs[0];
+        int ri                = g.producer_of(rb);
+        if (ri < 0 || !L[ri] || L[ri]->type != LAYER_RESHAPE || g.sole_consumer(rb) != pi || IsModelOutput(rb))
+            return -1;
+        auto rp = ParamOf<ReshapeLayerParam>(L[ri]);
+        if (!rp || rp->axis != 0 || rp->shape.size() != pp->orders.size() || L[ri]->inputs.size() != 1)
+            return -1;
+        const std::string &lb = L[ri]->inputs[0];
+        int li                = g.producer_of(lb);
+        if (li < 0 || !L[li] || L[li]->type != LAYER_ROCM_FUSED_LINEAR || g.sole_consumer(lb) != ri || IsModelOutput(lb))
+            return -1;
+        auto lp = ParamOf<RocmFusedLinearParam>(L[li]);
+        if (lp->gelu || lp->has_residual)
+            return -1;
+        chain->push_back(pi);
+        chain->push_back(ri);
+        chain->push_back(li);
+        *split_shape = rp->shape;
+        return li;
+    }
+
+    void FuseAttention() {
+        auto &L = structure_->layers;
+        bool changed = true;
+        while (changed) {
+            changed = false;
+            GraphIndex g(L);
+            for (int si = 0; si < (int)L.size() && !changed; ++si) {
+                auto sm = L[si];
+                if (!sm || sm->type != LAYER_SOFTMAX)
+                    continue;
+                std::vector<int> chain = {si};
+                // ---- upstream of the softmax: [Add(mask)] <- Mul|Div(scale) <- MatMul(q, k^T)
+                std::string cur = sm->inputs[0];
+                std::string mask;
+                float scale = 1.0f;
+                bool have_scale = false;
+                int qk = -1;
+                for (int step = 0; step < 3 && qk < 0; ++step) {
+                    int pi = g.producer_of(cur);
+                    if (pi < 0 || !L[pi] || g.sole_consumer(cur) < 0 || IsModelOutput(cur))
+                        break;
+                    auto pl = L[pi];
+                    if (pl->type == LAYER_ADD && pl->inputs.size() == 2 && mask.empty() && !have_scale) {
+                        // scores + mask : the operand that is not produced by the score chain is the mask
+                        int p0 = g.producer_of(pl->inputs[0]);
+                        bool first_is_scores = p0 >= 0 && L[p0] &&
+                                               (L[p0]->type == LAYER_MUL || L[p0]->type == LAYER_DIV || L[p0]->type == LAYER_MATMUL);
+                        mask = first_is_scores ? pl->inputs[1] : pl->inputs[0];
+                        cur  = first_is_scores ? pl->inputs[0] : pl->inputs[1];
+                        chain.push_back(pi);
+                    } else if ((pl->type == LAYER_MUL || pl->type == LAYER_DIV) && pl->inputs.size() == 1 && !have_scale) {
+                        auto er = ResOf<EltwiseLayerResource>(pl->name);
+                        if (!er || er->element_handle.GetDataCount() != 1 || er->element_handle.GetDataType() != DATA_TYPE_FLOAT)
+                            break;
+                        float v    = er->element_handle.force_to<float *>()[0];
+                        scale      = pl->type == LAYER_MUL ? v : 1.0f / v;
+                        have_scale = true;
+                        cur        = pl->inputs[0];
+                        chain.push_back(pi);
+                    } else if (pl->type == LAYER_MATMUL && pl->inputs.size() == 2) {
+                        qk = pi;
+                        chain.push_back(pi);
+                    } else {
+                        break;
+                    }
+                }
+                if (qk < 0)
+                    continue;
+                // ---- q and k^T operands
+                DimsVector shape_q, shape_k, shape_v;
+                int lq = HeadSplitSource(g, L[qk]->inputs[0], {0, 2, 1, 3}, {1, 0, 2}, &chain, &shape_q);
+                int lk = HeadSplitSource(g, L[qk]->inputs[1], {0, 2, 3, 1}, {1, 2, 0}, &chain, &shape_k);
+                if (lq < 0 || lk < 0)
+                    continue;
+                // ---- downstream: MatMul(probs, v) -> Permute -> Reshape
+                int pv = g.sole_consumer(sm->outputs[0]);
+                if (pv < 0 || !L[pv] || L[pv]->type != LAYER_MATMUL || L[pv]->inputs.size() != 2 ||
+                    L[pv]->inputs[0] != sm->outputs[0] || IsModelOutput(sm->outputs[0]))
+                    continue;
+                chain.push_back(pv);
+                int lv = HeadSplitSource(g, L[pv]->inputs[1], {0, 2, 1, 3}, {1, 0, 2}, &chain, &shape_v);
+                if (lv < 0 || shape_q != shape_k || shape_q != shape_v)
+                    continue;
+                int pm = g.sole_consumer(L[pv]->outputs[0]);
+                if (pm < 0 || !L[pm] || L[pm]->type != LAYER_PERMUTE || IsModelOutput(L[pv]->outputs[0]))
+                    continue;
+                auto pmp = ParamOf<PermuteLayerParam>(L[pm]);
+                if (!pmp || (pmp->orders != std::vector<int>{0, 2, 1, 3} && pmp->orders != std::vector<int>{1, 0, 2}))
+                    continue;
+                int rs = g.sole_consumer(L[pm]->outputs[0]);
+                if (rs < 0 || !L[rs] || L[rs]->type != LAYER_RESHAPE || IsModelOutput(L[pm]->outputs[0]))
+                    continue;
+                chain.push_back(pm);
+                chain.push_back(rs);
+                // ---- the three projections read the same x and are plain linears of equal width
+                if (L[lq]->inputs[0] != L[lk]->inputs[0] || L[lq]->inputs[0] != L[lv]->inputs[0])
+                    continue;
+                auto rq = ResOf<RocmFusedLinearResource>(L[lq]->name), rk = ResOf<RocmFusedLinearResource>(L[lk]->name),
+                     rv = ResOf<RocmFusedLinearResource>(L[lv]->name);
+                if (!rq || !rk || !rv)
+                    continue;
+                auto dq = rq->weight_nk.GetBufferDims();
+                if (dq != rk->weight_nk.GetBufferDims() || dq != rv->weight_nk.GetBufferDims())
+                    continue;
+                int H = dq[0], K = dq[1];
+                int heads    = shape_q[shape_q.size() - 2];
+                int head_dim = shape_q.back();
+                int seq      = shape_q[shape_q.size() - 3];
+                if (heads * head_dim != H || head_dim != 64 || seq <= 0)
+                    continue;
+                int first = *std::min_element(chain.begin(), chain.end());
+                if (!mask.empty()) {
+                    int pmask = g.producer_of(mask);
+                    bool ok   = pmask >= 0 ? pmask < first : structure_->inputs_shape_map.count(mask) > 0 ||
+                                                                 resource_->constant_map.count(mask) > 0;
+                    if (!ok)
+                        continue;
+                }
+                // ---- build the fused layer
+                auto fl      = std::make_shared<LayerInfo>();
+                fl->type     = LAYER_ROCM_FUSED_ATTENTION;
+                fl->type_str = "RocmFusedAttention";
+                fl->name     = sm->name + "_fused_attention";
+                fl->inputs   = {L[lq]->inputs[0]};
+                if (!mask.empty())
+                    fl->inputs.push_back(mask);
+                fl->outputs  = {L[rs]->outputs[0]};
+                auto fp      = std::make_shared<RocmFusedAttentionParam>();
+                fp->type     = fl->type_str;
+                fp->name     = fl->name;
+                fp->heads    = heads;
+                fp->head_dim = head_dim;
+                fp->scale    = scale;
+                fp->has_mask = mask.empty() ? 0 : 1;
+                fl->param    = fp;
+                fp->seq_len  = seq;
+                auto fr       = std::make_shared<RocmFusedLinearResource>();
+                fr->name      = fl->name;
+                fr->weight_nk = RawBuffer(3 * H * K * 4, {3 * H, K});
+                fr->bias      = RawBuffer(3 * H * 4, {3 * H});
+                RocmFusedLinearResource *src[3] = {rq, rk, rv};
+                for (int t = 0; t < 3; ++t) {
+                    memcpy(fr->weight_nk.force_to<float *>() + (size_t)t * H * K, src[t]->weight_nk.force_to<float *>(),
+                           (size_t)H * K * 4);
+                    if (src[t]->bias.GetDataCount() == H)
+                        memcpy(fr->bias.force_to<float *>() + (size_t)t * H, src[t]->bias.force_to<float *>(), (size_t)H * 4);
+                }
+                resource_->resource_map[fl->name] = fr;
+                for (int idx : chain)
+                    L[idx] = nullptr;
+                L[first] = fl;
+                changed  = true;
+            }
+            Compact();
+        }
+    }
+
+    NetStructure *structure_ = nullptr;
+    NetResource *resource_   = nullptr;
+    bool half_               = true;
+};
+
+struct RegisterRocmFusion {
+    RegisterRocmFusion() { RegisterNetOptimizer(1, std::make_shared<RocmFusionPass>()); }
+} g_register_rocm_fusion;
+
+}  // namespace
+
+// ---- RocmFusedLinear ------------------------------------------------------------------------------------------
+// y[rows,N] = act(x[rows,K] W^T + b) (+ residual): the arithmetic of MatMul+Add (cpu_mat_mul_layer_acc.cc:64-117,
+// compute_elewise.cc:37-65) or InnerProduct (naive_compute.cc:271-288), GELU (cpu_gelu_layer_acc.cc:42-45) and the
+// residual Add, in one MFMA GEMM launch with the epilogue applied on the fp32 accumulators.
+class RocmFusedLinearLayerAcc : public RocmLayerAcc {
+public:
+    Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        if (weight_)
+            return TNN_OK;
+        auto res = dynamic_cast<RocmFusedLinearResource *>(resource_);
+        auto p   = dynamic_cast<RocmFusedLinearParam *>(param_);
+        CHECK_PARAM_NULL(res);
+        CHECK_PARAM_NULL(p);
+        auto wd = res->weight_nk.GetBufferDims();
+        auto in = inputs[0]->GetBlobDesc().dims;
+        int k_in = p->axis >= 0 ? DimsVectorUtils::Count(in, p->axis) : (in.empty() ? 0 : in.back());
+        if (wd.size() != 2 || in.empty() || k_in != wd[1] || wd[0] != p->num_output)
+            return Status(TNNERR_PARAM_ERR, "fused linear: weight [N,K] does not match the contracted input dimensions");
+        if (p->has_residual) {
+            if (inputs.size() != 2 || inputs[1]->GetBlobDesc().dims != outputs[0]->GetBlobDesc().dims ||
+                inputs[1]->GetBlobDesc().data_type != outputs[0]->GetBlobDesc().data_type)
+                return Status(TNNERR_PARAM_ERR, "fused linear: residual must have the output's shape and type");
+        }
+        DataType dt = inputs[0]->GetBlobDesc().data_type;
+        RETURN_ON_NEQ(UploadConverted(res->weight_nk.force_to<void *>(), (size_t)wd[0] * wd[1], DATA_TYPE_FLOAT, dt, &weight_),
+                      TNN_OK);
+        if (p->has_bias)
+            RETURN_ON_NEQ(UploadConverted(res->bias.force_to<void *>(), (size_t)wd[0], DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &bias_),
+                          TNN_OK);
+        return TNN_OK;
+    }
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto p  = dynamic_cast<RocmFusedLinearParam *>(param_);
+        auto in = inputs[0]->GetBlobDesc().dims;
+        int K = p->axis >= 0 ? DimsVectorUtils::Count(in, p->axis) : in.back();
+        int N = p->num_output, rows = DimsVectorUtils::Count(in) / (K > 0 ? K : 1);
+        int epi = (p->has_bias ? TNN_ROCM_EPI_BIAS : 0) | (p->gelu ? TNN_ROCM_EPI_GELU : 0) |
+                  (p->has_residual ? TNN_ROCM_EPI_RESIDUAL : 0);
+        ROCM_CALL(tnn_rocm_gemm(Stream(), (int)inputs[0]->GetBlobDesc().data_type, 1, Ptr(inputs[0]), weight_, Ptr(outputs[0]),
+                                rows, N, K, K, K, N, 1, 1, 1, epi, (const float *)bias_,
+                                p->has_residual ? Ptr(In(inputs[1])) : nullptr, N));
+        return TNN_OK;
+    }
+
+private:
+    void *weight_ = nullptr, *bias_ = nullptr;
+};
+REGISTER_ROCM_ACC(RocmFusedLinearLayerAcc, LAYER_ROCM_FUSED_LINEAR);
+
+// ---- RocmFusedAttention -----------------------------------------------------------------------------------------
+// x [B,S,H] (or [T,H]) -> packed QKV = x Wqkv^T + bqkv in the context workspace -> flash-style attention kernel
+// reading Q/K/V straight out of the packed buffer (no Reshape/Permute copies) -> ctx [B,S,H].
+// The additive mask blob (broadcastable to [B,1,1,S]) is brought to fp32 [B,S] once per forward; from it the
+// per-sequence valid length is derived on the device so whole key tiles of padding are skipped.
+class RocmFusedAttentionLayerAcc : public RocmLayerAcc {
+public:
+    Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto res = dynamic_cast<RocmFusedLinearResource *>(resource_);
+        auto p   = dynamic_cast<RocmFusedAttentionParam *>(param_);
+        CHECK_PARAM_NULL(res);
+        CHECK_PARAM_NULL(p);
+        auto in = inputs[0]->GetBlobDesc().dims;
+        H_      = p->heads * p->head_dim;
+        if (in.empty() || in.back() != H_ || res->weight_nk.GetBufferDims() != DimsVector({3 * H_, H_}))
+            return Status(TNNERR_PARAM_ERR, "fused attention: hidden size mismatch");
+        DataType dt = inputs[0]->GetBlobDesc().data_type;
+        if (dt != DATA_TYPE_HALF && dt != DATA_TYPE_BFP16)
+            return Status(TNNERR_LAYER_ERR, "fused attention runs in fp16/bf16 only");
+        T_   = DimsVectorUtils::Count(in) / H_;
+        seq_ = p->seq_len > 0 ? p->seq_len : (in.size() >= 3 ? in[in.size() - 2] : T_);
+        if (seq_ <= 0 || T_ % seq_ != 0)
+            return Status(TNNERR_PARAM_ERR, "fused attention: token count is not a multiple of the sequence length");
+        B_ = T_ / seq_;
+        if (p->has_mask) {
+            if (inputs.size() < 2 || DimsVectorUtils::Count(In(inputs[1])->GetBlobDesc().dims) != B_ * seq_)
+                return Status(TNNERR_PARAM_ERR, "fused attention: mask must hold B*S additive values");
+        }
+        if (!weight_) {
+            RETURN_ON_NEQ(UploadConverted(res->weight_nk.force_to<void *>(), (size_t)3 * H_ * H_, DATA_TYPE_FLOAT, dt, &weight_),
+                          TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(res->bias.force_to<void *>(), (size_t)3 * H_, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &bias_),
+                          TNN_OK);
+            std::vector<int32_t> zeros(B_ > 0 ? B_ : 1, 0);
+            RETURN_ON_NEQ(UploadConverted(zeros.data(), zeros.size(), DATA_TYPE_INT32, DATA_TYPE_INT32, &kv_len_), TNN_OK);
+            std::vector<float> mz((size_t)(B_ * seq_ > 0 ? B_ * seq_ : 1), 0.f);
+            RETURN_ON_NEQ(UploadConverted(mz.data(), mz.size(), DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &mask_f32_), TNN_OK);
+        }
+        return TNN_OK;
+    }
+
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto p      = dynamic_cast<RocmFusedAttentionParam *>(param_);
+        DataType dt = inputs[0]->GetBlobDesc().data_type;
+        size_t es   = (size_t)DataTypeUtils::GetBytesSize(dt);
+        void *qkv   = nullptr;
+        RETURN_ON_NEQ(context_->Workspace((size_t)T_ * 3 * H_ * es, &qkv), TNN_OK);
+        ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 1, Ptr(inputs[0]), weight_, qkv, T_, 3 * H_, H_, H_, H_, 3 * H_, 1, 1, 1,
+                                TNN_ROCM_EPI_BIAS, (const float *)bias_, nullptr, 0));
+        const float *mask = nullptr;
+        const int32_t *kv = nullptr;
+        if (p->has_mask) {
+            Blob *mb = In(inputs[1]);
+            if (mb->GetBlobDesc().data_type == DATA_TYPE_FLOAT) {
+                mask = (const float *)Ptr(mb);
+            } else {
+                ROCM_CALL(tnn_rocm_cast(Stream(), (int)mb->GetBlobDesc().data_type, Ptr(mb), TNN_ROCM_F32, mask_f32_,
+                                        (size_t)B_ * seq_));
+                mask = (const float *)mask_f32_;
+            }
+            // keys whose mask is <= -1000 after the last visible key contribute exp(-1000 - max) == 0 in fp32
+            ROCM_CALL(tnn_rocm_mask_to_kv_len(Stream(), mask, (int32_t *)kv_len_, B_, seq_, -1000.0f));
+            kv = (const int32_t *)kv_len_;
+        }
+        const char *base = (const char *)qkv;
+        long row = 3L * H_, d = p->head_dim;
+        ROCM_CALL(tnn_rocm_attention(Stream(), (int)dt, base, base + (size_t)H_ * es, base + (size_t)2 * H_ * es,
+                                     Ptr(outputs[0]), B_, p->heads, seq_, p->head_dim, (long)seq_ * row, d, row,
+                                     (long)seq_ * row, d, row, (long)seq_ * H_, d, (long)H_, p->scale, mask, kv));
+        return TNN_OK;
+    }
+
+private:
+    void *weight_ = nullptr, *bias_ = nullptr, *kv_len_ = nullptr, *mask_f32_ = nullptr;
+    int H_ = 0, T_ = 0, B_ = 0, seq_ = 0;
+};
+REGISTER_ROCM_ACC(RocmFusedAttentionLayerAcc, LAYER_ROCM_FUSED_ATTENTION);
+
+}  // namespace TNN_NS

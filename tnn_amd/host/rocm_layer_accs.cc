@@ -1,0 +1,437 @@
+// One AbstractLayerAcc per op of the decomposed encoder graph, so unchanged protos run on DEVICE_ROCM
+// before (or without) the fusion pass: MatMul, InnerProduct (fp and int8), Add/Sub/Mul/Div, Softmax,
+// LayerNorm, GELU, Permute, Reshape, Reformat, Gather, Cast.
+//
+// Each Forward only enqueues kernels on the context's stream (DefaultNetwork::Forward synchronises once
+// at the end, source/tnn/core/default_network.cc:632-633).  dtype-dependent preparation (weight upload in
+// the activation dtype) happens in Reshape(), when every blob's data type is final.
+#include <cfloat>
+#include <cmath>
+
+#include "rocm_device.h"
+
+namespace TNN_NS {
+
+namespace {
+bool IsFloatType(DataType t) { return t == DATA_TYPE_FLOAT || t == DATA_TYPE_HALF || t == DATA_TYPE_BFP16; }
+Status Unsupported(const std::string &who, DataType t) {
+    return Status(TNNERR_LAYER_ERR, who + " dont support data type: " + std::to_string((int)t));
+}
+}  // namespace
+
+// ---- MatMul (cpu_mat_mul_layer_acc.cc:64-117, x86_mat_mul_layer_acc.cc:49-114) ---------------------
+class RocmMatMulLayerAcc : public RocmLayerAcc {
+public:
+    Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        if (inputs.size() == 2 || weight_)
+            return TNN_OK;
+        auto res = dynamic_cast<MatMulLayerResource *>(resource_);
+        CHECK_PARAM_NULL(res);
+        DataType wt = res->weight.GetDataType();
+        if (wt != DATA_TYPE_FLOAT && wt != DATA_TYPE_HALF)  // cpu_mat_mul_layer_acc.cc:45-56
+            return Status(TNNERR_PARAM_ERR, "MatMul has invalid direction param");
+        return UploadConverted(res->weight.force_to<void *>(), (size_t)res->weight.GetDataCount(), wt,
+                               inputs[0]->GetBlobDesc().data_type, &weight_);
+    }
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto param = dynamic_cast<MatMulLayerParam *>(param_);
+        CHECK_PARAM_NULL(param);
+        DataType dt = inputs[0]->GetBlobDesc().data_type;
+        if (!IsFloatType(dt))
+            return Unsupported("RocmMatMulLayerAcc", dt);
+        DimsVector a_dims = param->matrix_a_dims, b_dims = param->matrix_b_dims;
+        if (a_dims.size() == 1)
+            a_dims.insert(a_dims.begin(), 1);
+        if (b_dims.size() == 1)
+            b_dims.push_back(1);
+        const void *a, *b;
+        if (inputs.size() == 2) {
+            a = Ptr(In(inputs[0]));
+            b = Ptr(In(inputs[1]));
+        } else {
+            a = param->weight_position == 0 ? weight_ : Ptr(inputs[0]);
+            b = param->weight_position == 1 ? weight_ : Ptr(inputs[0]);
+        }
+        auto c_dims = outputs[0]->GetBlobDesc().dims;
+        int M = a_dims[a_dims.size() - 2], K = a_dims.back(), N = b_dims.back();
+        if (M * K == 0 || K * N == 0 || M * N == 0)
+            return TNN_OK;
+        int batch_a = DimsVectorUtils::Count(a_dims) / (M * K);
+        int batch_b = DimsVectorUtils::Count(b_dims) / (K * N);
+        int batch_c = DimsVectorUtils::Count(c_dims) / (M * N);
+        if (batch_a == batch_c && batch_b == 1 && batch_c > 1) {
+            // weight / shared right operand: fold the batch into the rows, one large GEMM
+            ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 0, a, b, Ptr(outputs[0]), M * batch_c, N, K, K, N, N, 1, 1, 1, 0,
+                                    nullptr, nullptr, 0));
+            return TNN_OK;
+        }
+        if (batch_a > batch_c || batch_b > batch_c)
+            return Status(TNNERR_PARAM_ERR, "MatMul batch broadcast not representable");
+        ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 0, a, b, Ptr(outputs[0]), M, N, K, K, N, N, batch_c, batch_a, batch_b,
+                                0, nullptr, nullptr, 0));
+        return TNN_OK;
+    }
+
+private:
+    void *weight_ = nullptr;
+};
+REGISTER_ROCM_ACC(RocmMatMulLayerAcc, LAYER_MATMUL);
+
+// ---- InnerProduct (fp: naive_compute.cc:271-288 ; int8: naive_compute.cc:316-347, x86_compute_int8.cc:833-914) ----
+class RocmInnerProductLayerAcc : public RocmLayerAcc {
+public:
+    Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        if (weight_)
+            return TNN_OK;
+        auto param = dynamic_cast<InnerProductLayerParam *>(param_);
+        auto res   = dynamic_cast<InnerProductLayerResource *>(resource_);
+        if (!param)
+            return Status(TNNERR_MODEL_ERR, "Error: InnerProductLayerParam is nil");
+        if (!res)
+            return Status(TNNERR_MODEL_ERR, "Error: InnerProductLayerResource is nil");
+        DataType dt  = outputs[0]->GetBlobDesc().data_type;
+        const int N  = param->num_output;
+        auto in_dims = inputs[0]->GetBlobDesc().dims;
+        const int K  = DimsVectorUtils::Count(in_dims, param->axis);
+        if ((long)res->weight_handle.GetDataCount() != (long)N * K)
+            return Status(TNNERR_MODEL_ERR, "InnerProduct weight size does not match num_output x K");
+        if (dt == DATA_TYPE_INT8) {
+            if (res->weight_handle.GetDataType() != DATA_TYPE_INT8)
+                return Status(TNNERR_MODEL_ERR, "quantized InnerProduct needs int8 weights");
+            RETURN_ON_NEQ(UploadConverted(res->weight_handle.force_to<void *>(), (size_t)N * K, DATA_TYPE_INT8,
+                                          DATA_TYPE_INT8, &weight_), TNN_OK);
+            // requantisation factor = w_scale / o_scale as one fp32 division on the host, 0 when o_scale < FLT_MIN
+            // (cpu_inner_product_layer_acc.cc:50-76, x86_inner_product_layer_acc.cc:197-222)
+            auto out8 = dynamic_cast<BlobInt8 *>(outputs[0]);
+            if (!out8 || !out8->GetIntResource())
+                return Status(TNNERR_NULL_PARAM, "int8 output blob without scale resource");
+            const float *w_scale = res->scale_handle.force_to<float *>();
+            CHECK_PARAM_NULL(w_scale);
+            const float *o_scale = out8->GetIntResource()->scale_handle.force_to<float *>();
+            int n_w = res->scale_handle.GetDataCount(), n_o = out8->GetIntResource()->scale_handle.GetDataCount();
+            std::vector<float> scale(N);
+            for (int i = 0; i < N; ++i) {
+                float os = o_scale[n_o == 1 ? 0 : i];
+                scale[i] = os >= FLT_MIN ? w_scale[n_w == 1 ? 0 : i] / os : 0.0f;
+            }
+            RETURN_ON_NEQ(UploadConverted(scale.data(), (size_t)N, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &scale_), TNN_OK);
+            if (param->has_bias && res->bias_handle.GetDataCount() == N)
+                RETURN_ON_NEQ(UploadConverted(res->bias_handle.force_to<void *>(), (size_t)N, DATA_TYPE_INT32,
+                                              DATA_TYPE_INT32, &bias_), TNN_OK);
+            return TNN_OK;
+        }
+        if (!IsFloatType(dt))
+            return Unsupported("RocmInnerProductLayerAcc", dt);
+        DataType wt = res->weight_handle.GetDataType();
+        if (!IsFloatType(wt))
+            return Status(TNNERR_MODEL_ERR, "float InnerProduct needs float weights");
+        RETURN_ON_NEQ(UploadConverted(res->weight_handle.force_to<void *>(), (size_t)N * K, wt, dt, &weight_), TNN_OK);
+        if (param->has_bias && res->bias_handle.GetDataCount() == N)
+            RETURN_ON_NEQ(UploadConverted(res->bias_handle.force_to<void *>(), (size_t)N, res->bias_handle.GetDataType(),
+                                          DATA_TYPE_FLOAT, &bias_), TNN_OK);
+        return TNN_OK;
+    }
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto param   = dynamic_cast<InnerProductLayerParam *>(param_);
+        auto in_dims = inputs[0]->GetBlobDesc().dims;
+        const int N = param->num_output, K = DimsVectorUtils::Count(in_dims, param->axis);
+        const int rows = DimsVectorUtils::Count(in_dims, 0, param->axis);
+        DataType dt    = outputs[0]->GetBlobDesc().data_type;
+        if (dt == DATA_TYPE_INT8) {
+            ROCM_CALL(tnn_rocm_gemm_i8(Stream(), (const int8_t *)Ptr(inputs[0]), (const int8_t *)weight_,
+                                       (const int32_t *)bias_, (const float *)scale_, (int8_t *)Ptr(outputs[0]), nullptr,
+                                       rows, N, K, K, K, N, nullptr, 0, 0.f));
+            return TNN_OK;
+        }
+        ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 1, Ptr(inputs[0]), weight_, Ptr(outputs[0]), rows, N, K, K, K, N, 1, 1, 1,
+                                bias_ ? TNN_ROCM_EPI_BIAS : 0, (const float *)bias_, nullptr, 0));
+        return TNN_OK;
+    }
+
+private:
+    void *weight_ = nullptr, *bias_ = nullptr, *scale_ = nullptr;
+};
+REGISTER_ROCM_ACC(RocmInnerProductLayerAcc, LAYER_INNER_PRODUCT);
+
+// ---- Add / Sub / Mul / Div (compute_elewise.cc:37-65 ; int8 add x86_compute_int8.cc:795-831) ----------
+template <int OP> class RocmBinaryLayerAcc : public RocmLayerAcc {
+public:
+    Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto res = dynamic_cast<EltwiseLayerResource *>(resource_);
+        if (!res || weight_ || res->element_handle.GetBytesSize() == 0)
+            return TNN_OK;
+        DataType dt = inputs[0]->GetBlobDesc().data_type;
+        if (!IsFloatType(dt))
+            return Unsupported("RocmBinaryLayerAcc", dt);
+        return UploadConverted(res->element_handle.force_to<void *>(), (size_t)res->element_handle.GetDataCount(),
+                               res->element_handle.GetDataType(), dt, &weight_);
+    }
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto param = dynamic_cast<MultidirBroadcastLayerParam *>(param_);
+        auto res   = dynamic_cast<EltwiseLayerResource *>(resource_);
+        DataType dt = outputs[0]->GetBlobDesc().data_type;
+        auto out_dims = outputs[0]->GetBlobDesc().dims;
+        if (dt == DATA_TYPE_INT8) {
+            if (OP != 0 || inputs.size() != 2)
+                return Status(TNNERR_LAYER_ERR, "int8 element-wise op other than a 2-input Add");
+            float s[3];
+            Blob *bl[3] = {inputs[0], inputs[1], outputs[0]};
+            for (int i = 0; i < 3; ++i) {
+                auto b8 = dynamic_cast<BlobInt8 *>(bl[i]);
+                if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1)
+                    return Status(TNNERR_LAYER_ERR, "int8 Add needs per-tensor blob scales");
+                s[i] = b8->GetIntResource()->scale_handle.force_to<float *>()[0];
+            }
+            float inv_so = (float)(1.0 / s[2]);  // x86_add_layer_acc.cc:54-58
+            ROCM_CALL(tnn_rocm_add_i8(Stream(), (const int8_t *)Ptr(inputs[0]), s[0], (const int8_t *)Ptr(inputs[1]), s[1],
+                                      inv_so, (int8_t *)Ptr(outputs[0]), (size_t)DimsVectorUtils::Count(out_dims)));
+            return TNN_OK;
+        }
+        if (!IsFloatType(dt))
+            return Unsupported("RocmBinaryLayerAcc", dt);
+        // operand list in evaluation order: inputs, with the resource weight spliced in at weight_input_index
+        struct Operand {
+            const void *ptr;
+            DimsVector dims;
+        };
+        std::vector<Operand> ops;
+        for (auto b : inputs)
+            ops.push_back({Ptr(In(b)), In(b)->GetBlobDesc().dims});
+        if (weight_ && res) {
+            Operand w{weight_, res->element_shape};
+            if (param && param->weight_input_index == 0)
+                ops.insert(ops.begin(), w);
+            else
+                ops.push_back(w);
+        }
+        if (ops.size() < 2)
+            return Status(TNNERR_LAYER_ERR, "binary op needs two operands");
+        if (out_dims.size() > 6)
+            return Status(TNNERR_LAYER_ERR, "binary op rank above 6");
+        const void *acc_ptr = ops[0].ptr;
+        DimsVector acc_dims = ops[0].dims;
+        for (size_t i = 1; i < ops.size(); ++i) {
+            bool last = i + 1 == ops.size();
+            // intermediate results of >2-operand chains take the output buffer as well (same shape from i=1 on)
+            DimsVector cur_out = out_dims;
+            ROCM_CALL(tnn_rocm_binary(Stream(), (int)dt, OP, acc_ptr, acc_dims.data(), (int)acc_dims.size(), ops[i].ptr,
+                                      ops[i].dims.data(), (int)ops[i].dims.size(), Ptr(outputs[0]), cur_out.data(),
+                                      (int)cur_out.size()));
+            acc_ptr  = Ptr(outputs[0]);
+            acc_dims = cur_out;
+            (void)last;
+        }
+        return TNN_OK;
+    }
+
+private:
+    void *weight_ = nullptr;
+};
+typedef RocmBinaryLayerAcc<0> RocmAddLayerAcc;
+typedef RocmBinaryLayerAcc<1> RocmSubLayerAcc;
+typedef RocmBinaryLayerAcc<2> RocmMulLayerAcc;
+typedef RocmBinaryLayerAcc<3> RocmDivLayerAcc;
+REGISTER_ROCM_ACC(RocmAddLayerAcc, LAYER_ADD);
+REGISTER_ROCM_ACC(RocmSubLayerAcc, LAYER_SUB);
+REGISTER_ROCM_ACC(RocmMulLayerAcc, LAYER_MUL);
+REGISTER_ROCM_ACC(RocmDivLayerAcc, LAYER_DIV);
+
+// ---- Softmax (cpu_softmax_layer_acc.cc:30-97) -----------------------------------------------------------
+class RocmSoftmaxLayerAcc : public RocmLayerAcc {
+public:
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto param = dynamic_cast<SoftmaxLayerParam *>(param_);
+        if (!param)
+            return Status(TNNERR_MODEL_ERR, "Error: SoftmaxLayerParam is unsupported");
+        auto dims   = inputs[0]->GetBlobDesc().dims;
+        DataType dt = inputs[0]->GetBlobDesc().data_type;
+        if (!IsFloatType(dt))
+            return Unsupported("RocmSoftmaxLayerAcc", dt);
+        if (dims.empty())
+            return Status(TNNERR_PARAM_ERR, "softmax on a rank-0 blob");
+        int axis = (int)((param->axis + (int)dims.size()) % (int)dims.size());
+        ROCM_CALL(tnn_rocm_softmax(Stream(), (int)dt, Ptr(inputs[0]), Ptr(outputs[0]), DimsVectorUtils::Count(dims, 0, axis),
+                                   dims[axis], DimsVectorUtils::Count(dims, axis + 1)));
+        return TNN_OK;
+    }
+};
+REGISTER_ROCM_ACC(RocmSoftmaxLayerAcc, LAYER_SOFTMAX);
+
+// ---- LayerNorm (cpu_layer_norm_layer_acc.cc:30-140) ------------------------------------------------------
+class RocmLayerNormLayerAcc : public RocmLayerAcc {
+public:
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto param = dynamic_cast<LayerNormLayerParam *>(param_);
+        CHECK_PARAM_NULL(param);
+        if (inputs.size() < 3)
+            return Status(TNNERR_PARAM_ERR, "LayerNormLayer has no input blob of scale or bias");
+        Blob *scale = In(inputs[1]), *bias = In(inputs[2]);
+        auto dims_in = inputs[0]->GetBlobDesc().dims, dims_s = scale->GetBlobDesc().dims;
+        if (!DimsVectorUtils::Equal(dims_s, bias->GetBlobDesc().dims))
+            return Status(TNNERR_PARAM_ERR, "LayerNormLayer has invalid dims for input blob of scale or bias");
+        int offset = (int)dims_in.size() - (int)dims_s.size();
+        for (int i = 0; i < (int)dims_s.size(); ++i)
+            if (offset < 0 || dims_in[i + offset] != dims_s[i])
+                return Status(TNNERR_PARAM_ERR, "LayerNormLayer has invalid dims for input blob");
+        param->reduce_dims_size = (int)dims_s.size();  // InferRuntimeOutputShape, cpu_layer_norm_layer_acc.cc:30-61
+        if (scale->GetBlobDesc().data_type != DATA_TYPE_FLOAT || bias->GetBlobDesc().data_type != DATA_TYPE_FLOAT)
+            return Status(TNNERR_LAYER_ERR, "LayerNorm scale/bias must be fp32 on DEVICE_ROCM");
+        DataType dt = outputs[0]->GetBlobDesc().data_type;
+        if (!IsFloatType(dt))
+            return Unsupported("RocmLayerNormLayerAcc", dt);
+        int rows = DimsVectorUtils::Count(dims_in, 0, offset), cols = DimsVectorUtils::Count(dims_in, offset);
+        if (rows == 0 || cols == 0)
+            return Status(TNNERR_COMMON_ERROR, "Error: blob count is zero");
+        ROCM_CALL(tnn_rocm_layernorm(Stream(), (int)dt, Ptr(inputs[0]), nullptr, (const float *)Ptr(scale),
+                                     (const float *)Ptr(bias), Ptr(outputs[0]), rows, cols, param->eps, nullptr, 0.f));
+        return TNN_OK;
+    }
+
+protected:
+    DataType ConstantBlobDataType(const std::vector<Blob *> &, int) override { return DATA_TYPE_FLOAT; }
+};
+REGISTER_ROCM_ACC(RocmLayerNormLayerAcc, LAYER_LAYER_NORM);
+
+// ---- GELU (cpu_gelu_layer_acc.cc:31-51) --------------------------------------------------------------------
+class RocmGeluLayerAcc : public RocmLayerAcc {
+public:
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        DataType dt = outputs[0]->GetBlobDesc().data_type;
+        if (!IsFloatType(dt))
+            return Status(TNNERR_NO_RESULT, "RocmGeluLayerAcc dont support data type");
+        ROCM_CALL(tnn_rocm_gelu(Stream(), (int)dt, Ptr(inputs[0]), Ptr(outputs[0]),
+                                (size_t)DimsVectorUtils::Count(outputs[0]->GetBlobDesc().dims)));
+        return TNN_OK;
+    }
+};
+REGISTER_ROCM_ACC(RocmGeluLayerAcc, LAYER_GELU);
+
+// ---- Permute / Reshape (naive_compute.cc:943-956 ; reshape is a copy) ----------------------------------------
+class RocmPermuteLayerAcc : public RocmLayerAcc {
+public:
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto param = dynamic_cast<PermuteLayerParam *>(param_);
+        CHECK_PARAM_NULL(param);
+        auto dims = inputs[0]->GetBlobDesc().dims;
+        if (dims.size() > 6 || param->orders.size() != dims.size())
+            return Status(TNNERR_PARAM_ERR, "Permute rank unsupported or order size mismatch");
+        int es = DataTypeUtils::GetBytesSize(inputs[0]->GetBlobDesc().data_type);
+        ROCM_CALL(tnn_rocm_permute(Stream(), es, Ptr(inputs[0]), Ptr(outputs[0]), dims.data(), param->orders.data(),
+                                   (int)dims.size()));
+        return TNN_OK;
+    }
+};
+REGISTER_ROCM_ACC(RocmPermuteLayerAcc, LAYER_PERMUTE);
+
+class RocmReshapeLayerAcc : public RocmLayerAcc {
+public:
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto param = dynamic_cast<ReshapeLayerParam *>(param_);
+        if (param && param->reshape_type != 0)
+            return Status(TNNERR_LAYER_ERR, "Reshape type nhwc is not implemented on DEVICE_ROCM");
+        size_t bytes = (size_t)DimsVectorUtils::Count(outputs[0]->GetBlobDesc().dims) *
+                       DataTypeUtils::GetBytesSize(outputs[0]->GetBlobDesc().data_type);
+        ROCM_CALL(tnn_rocm_memcpy_d2d(Ptr(outputs[0]), Ptr(inputs[0]), bytes, Stream()));
+        return TNN_OK;
+    }
+};
+REGISTER_ROCM_ACC(RocmReshapeLayerAcc, LAYER_RESHAPE);
+
+// ---- Reformat: float <-> int8 (x86_reformat_layer_acc.cc:50-80, x86_compute_int8.cc:1193-1318) -------------------
+class RocmReformatLayerAcc : public RocmLayerAcc {
+public:
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto param = dynamic_cast<ReformatLayerParam *>(param_);
+        CHECK_PARAM_NULL(param);
+        for (size_t i = 0; i < inputs.size(); ++i) {
+            size_t count = (size_t)DimsVectorUtils::Count(outputs[i]->GetBlobDesc().dims);
+            DataType st = inputs[i]->GetBlobDesc().data_type, dt = outputs[i]->GetBlobDesc().data_type;
+            if (param->type == QUANT_ONLY) {
+                auto b8 = dynamic_cast<BlobInt8 *>(outputs[i]);
+                if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1)
+                    return Status(TNNERR_LAYER_ERR, "Reformat(quant) needs a per-tensor blob scale");
+                float s   = b8->GetIntResource()->scale_handle.force_to<float *>()[0];
+                float inv = (float)(1.0 / s);  // x86_reformat_layer_acc.cc:70 : double division, stored as float
+                ROCM_CALL(tnn_rocm_quantize(Stream(), (int)st, Ptr(inputs[i]), inv, (int8_t *)Ptr(outputs[i]), count));
+            } else if (param->type == DEQUANT_ONLY) {
+                auto b8 = dynamic_cast<BlobInt8 *>(inputs[i]);
+                if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1)
+                    return Status(TNNERR_LAYER_ERR, "Reformat(dequant) needs a per-tensor blob scale");
+                float s = b8->GetIntResource()->scale_handle.force_to<float *>()[0];
+                ROCM_CALL(tnn_rocm_dequantize(Stream(), (const int8_t *)Ptr(inputs[i]), s, (int)dt, Ptr(outputs[i]), count));
+            } else if (IsFloatType(st) && IsFloatType(dt)) {
+                ROCM_CALL(tnn_rocm_cast(Stream(), (int)st, Ptr(inputs[i]), (int)dt, Ptr(outputs[i]), count));
+            } else {
+                return Status(TNNERR_MODEL_ERR, "unsupport precision mode");
+            }
+        }
+        return TNN_OK;
+    }
+};
+REGISTER_ROCM_ACC(RocmReformatLayerAcc, LAYER_REFORMAT);
+
+// ---- Gather (cpu_gather_layer_acc.cc:27-86) -----------------------------------------------------------------------
+class RocmGatherLayerAcc : public RocmLayerAcc {
+public:
+    Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto param = dynamic_cast<GatherLayerParam *>(param_);
+        auto res   = dynamic_cast<GatherLayerResource *>(resource_);
+        CHECK_PARAM_NULL(param);
+        if ((param->data_in_resource || param->indices_in_resource) && !res)
+            return Status(TNNERR_MODEL_ERR, "Gather resource is invalid");
+        if (param->data_in_resource && !data_) {
+            DataType st = res->data.GetDataType(), dt = outputs[0]->GetBlobDesc().data_type;
+            RETURN_ON_NEQ(UploadConverted(res->data.force_to<void *>(), (size_t)res->data.GetDataCount(), st,
+                                          IsFloatType(st) ? dt : st, &data_), TNN_OK);
+        }
+        if (param->indices_in_resource && !indices_) {
+            if (res->indices.GetDataType() != DATA_TYPE_INT32)
+                return Status(TNNERR_MODEL_ERR, "Gather indices must be int32");
+            RETURN_ON_NEQ(UploadConverted(res->indices.force_to<void *>(), (size_t)res->indices.GetDataCount(),
+                                          DATA_TYPE_INT32, DATA_TYPE_INT32, &indices_), TNN_OK);
+        }
+        return TNN_OK;
+    }
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto param = dynamic_cast<GatherLayerParam *>(param_);
+        auto res   = dynamic_cast<GatherLayerResource *>(resource_);
+        DimsVector data_dims = param->data_in_resource ? res->data.GetBufferDims() : inputs.front()->GetBlobDesc().dims;
+        DimsVector idx_dims  = param->indices_in_resource ? res->indices.GetBufferDims() : inputs.back()->GetBlobDesc().dims;
+        const void *data = param->data_in_resource ? data_ : Ptr(In(inputs.front()));
+        const void *idx  = param->indices_in_resource ? indices_ : Ptr(In(inputs.back()));
+        if (!param->indices_in_resource && inputs.back()->GetBlobDesc().data_type != DATA_TYPE_INT32)
+            return Status(TNNERR_MODEL_ERR, "Gather indices blob must be int32");
+        int axis  = param->axis;
+        int es    = DataTypeUtils::GetBytesSize(outputs[0]->GetBlobDesc().data_type);
+        int batch = DimsVectorUtils::Count(data_dims, 0, axis), slices = data_dims[axis];
+        size_t slice_bytes = (size_t)DimsVectorUtils::Count(data_dims, axis + 1) * es;
+        ROCM_CALL(tnn_rocm_gather(Stream(), data, (const int32_t *)idx, Ptr(outputs[0]), batch, slices, slice_bytes,
+                                  DimsVectorUtils::Count(idx_dims), context_->ErrorFlag()));
+        return TNN_OK;
+    }
+
+private:
+    void *data_ = nullptr, *indices_ = nullptr;
+};
+REGISTER_ROCM_ACC(RocmGatherLayerAcc, LAYER_GATHER);
+
+// ---- Cast ----------------------------------------------------------------------------------------------------------
+class RocmCastLayerAcc : public RocmLayerAcc {
+public:
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        DataType st = inputs[0]->GetBlobDesc().data_type, dt = outputs[0]->GetBlobDesc().data_type;
+        size_t count = (size_t)DimsVectorUtils::Count(outputs[0]->GetBlobDesc().dims);
+        if (IsFloatType(st) && IsFloatType(dt)) {
+            ROCM_CALL(tnn_rocm_cast(Stream(), (int)st, Ptr(inputs[0]), (int)dt, Ptr(outputs[0]), count));
+            return TNN_OK;
+        }
+        if (st == dt) {
+            ROCM_CALL(tnn_rocm_memcpy_d2d(Ptr(outputs[0]), Ptr(inputs[0]), count * DataTypeUtils::GetBytesSize(st), Stream()));
+            return TNN_OK;
+        }
+        return Status(TNNERR_LAYER_ERR, "Cast between these data types is not implemented on DEVICE_ROCM");
+    }
+};
+REGISTER_ROCM_ACC(RocmCastLayerAcc, LAYER_CAST);
+
+}  // namespace TNN_NS
