@@ -1,12 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the transformer-encoder hot path on one MI355X.
 
-A "step" is one forward pass of the 12-layer BERT-base encoder (hidden 768, 12 heads, FFN 3072, post-LN,
-fp16 activations/weights with fp32 accumulation) over one synthetic batch of 8 sequences of 384 tokens with
-per-sequence valid lengths uniform in [200, 384] — token ids to last hidden state, inputs resident in HBM.
+A "step" is one Instance::Forward() of the DEVICE_ROCM backend on the 12-layer BERT-base encoder (hidden 768,
+12 heads, FFN 3072, post-LN; fp16 activations/weights, fp32 accumulation) over one synthetic batch of 8 sequences
+of 384 tokens with per-sequence valid lengths uniform in [200, 384]: token ids -> last hidden state.  The model is
+written as .tnnproto/.tnnmodel (the decomposed op graph), loaded by the C++ host, rewritten by the ROCm fusion pass
+and executed layer by layer; inputs are resident in their HBM blobs when the timed region starts.
 
-Prints ONE JSON line:  sequences/s (whole job), the roofline of the dominant kernel (measured live with
-events on the launch stream inside the timed region) and the CPU baseline timed on this box's host cores.
+Prints ONE JSON line: sequences/s, the roofline of the dominant kernel (events on the instance's stream inside the
+timed region) and the CPU baseline (the reference engine's own DEVICE_X86 path, when its prebuilt library is
+present) timed on this box's host cores.
 """
 import argparse
 import json
@@ -18,7 +21,6 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
-PEAK_HBM_GBS = 8000.0
 
 
 def parse():
@@ -35,25 +37,21 @@ def parse():
 
 
 def cpu_baseline(cfg, weights, ids, seg, mask, n_seqs):
-    """Times the CPU path on a bounded sample (n_seqs sequences through all layers).
-
-    Uses the reference engine's own DEVICE_X86 path when the prebuilt driver from oracle/_ref is present
-    ("reference"); otherwise the plain-C restatement under oracle/ ("port")."""
+    """Bounded CPU sample: n_seqs sequences through all layers.  "reference" = the reference engine's DEVICE_X86 path
+    (oracle/_ref, prebuilt); "port" = the plain-C restatement under oracle/ when that library is absent."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     B, S = ids.shape
     n = min(n_seqs, B)
     try:
-        import ref_driver  # tests/ref_driver.py: ctypes front-end of oracle/_ref
+        import ref_driver
         if ref_driver.available():
             return ref_driver.time_encoder(cfg, weights, ids[:n], seg[:n], mask[:n])
-    except ImportError:
-        pass
+    except (ImportError, OSError) as e:  # library missing or not loadable on this box
+        print("bench.py: reference CPU library unavailable (%s); timing the restatement" % e, file=sys.stderr)
     import encoder_ref
-    import numpy as np
-    w32 = weights
     t0 = time.perf_counter()
-    x0 = encoder_ref.embed(w32, ids[:n], seg[:n], cfg.eps)
-    encoder_ref.encoder(w32, cfg, x0, n, S, mask[:n])
+    x0 = encoder_ref.embed(weights, ids[:n], seg[:n], cfg.eps)
+    encoder_ref.encoder(weights, cfg, x0, n, S, mask[:n])
     dt = time.perf_counter() - t0
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     return {"value": n / dt, "unit": "sequences/s", "cores": cores, "kind": "port",
@@ -61,111 +59,113 @@ def cpu_baseline(cfg, weights, ids, seg, mask, n_seqs):
                       "DEVICE_NAIVE graph, OpenMP over rows" % (n, B, S, cfg.layers)}
 
 
+def classify(layer_name):
+    for key in ("_ffn1_", "_ffn2_", "_o_mm"):
+        if key in layer_name:
+            return {"_ffn1_": "gemm_ffn1", "_ffn2_": "gemm_ffn2", "_o_mm": "gemm_out"}[key]
+    return "other"
+
+
 def main():
     args = parse()
     if args.gpus != 1:
-        print("bench.py: this build runs the hot path on ONE GPU; --gpus %d is not supported (the path shards "
-              "by batch with no exchange: run one process per GPU on its own share of the batch)" % args.gpus,
+        print("bench.py: this build runs the hot path on ONE GPU; --gpus %d is not supported (the path shards by "
+              "batch with no exchange: one process per GPU, each on its own share of the batch)" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
     import numpy as np
     import torch
-    from tnn_amd import capi
-    from tnn_amd.encoder import EncoderConfig, make_weights, make_inputs, DeviceEncoder
+    from tnn_amd import host, ops, tnnmodel
+    from tnn_amd.encoder import EncoderConfig, make_weights, make_inputs
 
-    capi.load()  # fails loudly if the HIP library is not built
+    host.load()  # fails loudly if the HIP library or the host library is not built
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     cfg = EncoderConfig.bert_base(args.layers)
     B, S = args.batch, args.seq
     weights = make_weights(cfg, seed=20240601)
-    ids, seg, lens, mask = make_inputs(cfg, B, S, 200, min(384, S), seed=20240602)
-    enc = DeviceEncoder(cfg, weights, torch.float16)
-    d_ids = torch.from_numpy(ids).cuda()
-    d_seg = torch.from_numpy(seg).cuda()
-    d_mask = torch.from_numpy(mask).cuda()
-
-    def step():
-        return enc.forward(d_ids, d_seg, mask=d_mask)
+    ids, seg, lens, mask = make_inputs(cfg, B, S, min(200, S), min(384, S), seed=20240602)
+    graph = tnnmodel.encoder_graph(cfg, weights, B, S)
+    inst = host.RocmInstance.from_graph(graph, "fp16")
+    layer_types = [t for t, _ in inst.layers()]
+    inst.set_input("input_ids", ids)
+    inst.set_input("token_type_ids", seg)
+    inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
 
     for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+        inst.forward()
 
-    # ---- which launch class dominates?  one instrumented (untimed) pass with events around every launch
-    records = {}
-
-    def hook_all(name, fn):
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        r = fn()
-        e.record()
-        records.setdefault(name, []).append((s, e))
-        return r
-
-    enc.hook = hook_all
-    for _ in range(3):
-        step()
-    torch.cuda.synchronize()
-    enc.hook = None
-    breakdown = {k: sum(s.elapsed_time(e) for s, e in v) / 3.0 for k, v in records.items()}  # ms per step
-    gemm_names = [k for k in breakdown if k.startswith("gemm_")]
-    dominant = max(gemm_names, key=lambda k: breakdown[k])
-
-    # ---- timed region: exactly K steps, events only around the dominant kernel's launches
-    dom_events = []
-
-    def hook_dom(name, fn):
-        if name != dominant:
-            return fn()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        r = fn()
-        e.record()
-        dom_events.append((s, e))
-        return r
-
-    enc.hook = hook_dom
-    torch.cuda.synchronize()
+    # ---- timed region: exactly K Instance::Forward() calls; events only around the GEMM layers
+    inst.profile_start("RocmFusedLinear")
+    inst.sync()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
+        inst.forward()
+    inst.sync()
     dt = time.perf_counter() - t0
-    enc.hook = None
+    gemm_prof = inst.profile_finish()
 
     ms_per_step = dt / args.steps * 1e3
     seqs_per_s = B * args.steps / dt
     T, H, F = B * S, cfg.hidden, cfg.ffn
-    gemm_flops = {"gemm_qkv": 2.0 * T * 3 * H * H, "gemm_out": 2.0 * T * H * H, "gemm_ffn1": 2.0 * T * F * H,
-                  "gemm_ffn2": 2.0 * T * H * F}
-    dom_ms = sum(s.elapsed_time(e) for s, e in dom_events) / len(dom_events)
+    gemm_flops = {"gemm_out": 2.0 * T * H * H, "gemm_ffn1": 2.0 * T * F * H, "gemm_ffn2": 2.0 * T * H * F}
+    per_class = {}
+    for t, name, ms in gemm_prof:
+        if t == "RocmFusedLinear":
+            per_class.setdefault(classify(name), []).append(ms)
+    dominant = max((k for k in per_class if k in gemm_flops), key=lambda k: sum(per_class[k]))
+    dom_ms = sum(per_class[dominant]) / len(per_class[dominant])
     achieved = gemm_flops[dominant] / (dom_ms * 1e-3) / 1e12
-    attn_ms = breakdown["attention"] / cfg.layers
+
+    # ---- untimed: full per-layer profile and the attention kernel on its own
+    full = inst.profile(5)
+    breakdown = {}
+    for t, name, ms in full:
+        key = classify(name) if t == "RocmFusedLinear" else t
+        breakdown[key] = breakdown.get(key, 0.0) + ms
+    out_final = inst.output("last_hidden")
+    assert np.isfinite(out_final).all()
+
+    d_lens = torch.from_numpy(lens).cuda()
+    qkv = torch.randn(T, 3 * H, device="cuda").half()
+    ctx = torch.empty(T, H, device="cuda", dtype=torch.float16)
+    for _ in range(5):
+        ops.attention_packed(qkv, B, S, cfg.heads, 0.125, kv_len=d_lens, out=ctx)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(50):
+        ops.attention_packed(qkv, B, S, cfg.heads, 0.125, kv_len=d_lens, out=ctx)
+    e1.record()
+    torch.cuda.synchronize()
+    attn_ms = e0.elapsed_time(e1) / 50
     attn_eff_flops = 4.0 * H * S * float(lens.sum())
     attn_pad_flops = 4.0 * B * S * S * H
 
+    full_cfg = (B, S, args.layers) == (8, 384, 12)
     out = {
         "metric": "BERT-base seq384 fp16 sequences/sec on 1 MI355X; fused-attention TFLOP/s",
         "value": round(seqs_per_s, 2), "unit": "sequences/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "12-layer BERT-base encoder fp16, batch 8, seq 384, valid lengths U[200,384] "
-                               "(BASELINE.json configs[1])" if (B, S, args.layers) == (8, 384, 12) else
+        "config": {"workload": ("12-layer BERT-base encoder fp16, batch 8, seq 384, valid lengths U[200,384] "
+                                "(BASELINE.json configs[1])") if full_cfg else
                    "%d-layer BERT-base encoder fp16, batch %d, seq %d" % (args.layers, B, S),
+                   "path": "Instance::Forward on DEVICE_ROCM from .tnnproto/.tnnmodel, ROCm fusion pass on",
                    "layers": args.layers, "batch": B, "seq_len": S, "hidden": H, "heads": cfg.heads, "ffn": F,
-                   "sum_valid_len": int(lens.sum())},
+                   "sum_valid_len": int(lens.sum()), "host_layers": len(layer_types)},
         "model_tflops": round(cfg.flops_per_sequence(S) * seqs_per_s / 1e12, 2),
         "attention_tflops": {"effective": round(attn_eff_flops / (attn_ms * 1e-3) / 1e12, 2),
                              "padded": round(attn_pad_flops / (attn_ms * 1e-3) / 1e12, 2),
                              "us_per_launch": round(attn_ms * 1e3, 2),
                              "frac_of_fp16_peak_effective": round(attn_eff_flops / (attn_ms * 1e-3) / 1e12 /
                                                                   PEAK_FP16_TFLOPS, 4)},
-        "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(achieved, 2), "peak": PEAK_FP16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None,
-                     "us_per_launch": round(dom_ms * 1e3, 2), "launches_timed": len(dom_events),
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel (%s)" % dominant, "achieved": round(achieved, 2),
+                     "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
+                     "traffic": None, "us_per_launch": round(dom_ms * 1e3, 2),
+                     "launches_timed": len(per_class[dominant]) * args.steps,
                      "flops_per_launch": gemm_flops[dominant]},
-        "launch_breakdown_ms_per_step": {k: round(v, 4) for k, v in sorted(breakdown.items())},
+        "layer_breakdown_ms_per_step": {k: round(v, 4) for k, v in sorted(breakdown.items())},
     }
+    inst.close()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, weights, ids, seg, mask, args.cpu_seqs)
     print(json.dumps(out))

@@ -24,7 +24,7 @@ SIGNATURES = {
                                       C.POINTER(C.c_int)]),
     "tnn_host_layer_count": (C.c_int, [C.c_void_p]),
     "tnn_host_layer_summary": (C.c_char_p, [C.c_void_p]),
-    "tnn_host_profile_start": (None, [C.c_void_p]),
+    "tnn_host_profile_start": (None, [C.c_void_p, C.c_char_p]),
     "tnn_host_profile_finish": (C.c_int, [C.c_void_p, C.POINTER(C.c_double), C.c_int]),
 }
 _lib = None
@@ -104,10 +104,21 @@ class RocmInstance:
         text = load().tnn_host_layer_summary(self._h).decode()
         return [tuple(line.split(" ", 1)) for line in text.splitlines() if line]
 
+    def profile_start(self, only_type=""):
+        load().tnn_host_profile_start(self._h, only_type.encode())
+
+    def profile_finish(self):
+        """[(type, name, mean ms per forward)] since profile_start (hipEvents on the instance's stream)"""
+        lib = load()
+        n = lib.tnn_host_layer_count(self._h)
+        ms = (C.c_double * n)()
+        lib.tnn_host_profile_finish(self._h, ms, n)
+        return [(t, nm, ms[i]) for i, (t, nm) in enumerate(self.layers())]
+
     def profile(self, iters=10):
         """per-layer mean milliseconds over `iters` forwards (hipEvent timing on the instance's stream)"""
         lib = load()
-        lib.tnn_host_profile_start(self._h)
+        lib.tnn_host_profile_start(self._h, b"")
         for _ in range(iters):
             self.forward()
         n = lib.tnn_host_layer_count(self._h)

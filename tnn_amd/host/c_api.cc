@@ -120,7 +120,10 @@ HOST_API const char *tnn_host_layer_summary(void *hp) {
     return h->summary.c_str();
 }
 
-HOST_API void tnn_host_profile_start(void *hp) { static_cast<Handle *>(hp)->inst->GetNetwork()->StartProfile(); }
+// only_type: NULL or "" times every layer, otherwise only layers of that type string
+HOST_API void tnn_host_profile_start(void *hp, const char *only_type) {
+    static_cast<Handle *>(hp)->inst->GetNetwork()->StartProfile(only_type ? only_type : "");
+}
 
 // Fills up to `capacity` entries with the per-layer mean milliseconds since tnn_host_profile_start; returns the
 // number of layers.  Names come from tnn_host_layer_summary (same order).

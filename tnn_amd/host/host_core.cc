@@ -1186,10 +1186,11 @@ Status DefaultNetwork::ForwardAsync() {
     if (profiling_)
         context_->GetCommandQueue(&stream);
     for (size_t i = 0; i < layers_.size(); ++i) {
-        if (profiling_)
+        const bool timed = profiling_ && prof_on_[i];
+        if (timed)
             tnn_rocm_event_record(prof_events_[i].first, stream);
         Status st = layers_[i]->Forward();
-        if (profiling_)
+        if (timed)
             tnn_rocm_event_record(prof_events_[i].second, stream);
         if (st != TNN_OK)  // default_network.cc:599-605
             return Status((int)st, "Forward error of layer " + layers_[i]->GetLayerName() + ": " + st.description());
@@ -1197,6 +1198,8 @@ Status DefaultNetwork::ForwardAsync() {
     if (profiling_) {
         for (size_t i = 0; i < layers_.size(); ++i) {
             float ms = 0;
+            if (!prof_on_[i])
+                continue;
             if (tnn_rocm_event_elapsed_ms(prof_events_[i].first, prof_events_[i].second, &ms) == 0) {
                 prof_[i].ms += ms;
                 prof_[i].calls += 1;
@@ -1224,8 +1227,11 @@ std::string DefaultNetwork::LayerSummary() const {
         os << l->type_str << " " << l->name << "\n";
     return os.str();
 }
-void DefaultNetwork::StartProfile() {
+void DefaultNetwork::StartProfile(const std::string &only_type) {
     prof_.clear();
+    prof_on_.clear();
+    for (auto &l : structure_.layers)
+        prof_on_.push_back(only_type.empty() || l->type_str == only_type ? 1 : 0);
     for (size_t i = prof_events_.size(); i < layers_.size(); ++i) {
         void *a = nullptr, *b = nullptr;
         tnn_rocm_event_create(&a);

@@ -628,7 +628,8 @@ public:
     int LayerCount() const { return (int)layers_.size(); }
     std::string LayerSummary() const;
     // per-layer hipEvent timing (the engine's TNN_PROFILE hook, source/tnn/core/profile.cc:111-201)
-    void StartProfile();
+    // only layers whose type string equals `only_type` are timed when it is non-empty
+    void StartProfile(const std::string &only_type = "");
     std::vector<LayerProfile> FinishProfile();
 
 private:
@@ -644,6 +645,7 @@ private:
     std::vector<void *> allocations_;
     BlobMap inputs_, outputs_;
     bool profiling_ = false;
+    std::vector<char> prof_on_;
     std::vector<std::pair<void *, void *>> prof_events_;
     std::vector<LayerProfile> prof_;
 };
