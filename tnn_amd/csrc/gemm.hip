@@ -18,6 +18,8 @@
 //
 // Output layout of a 32x32 block: lane l holds column (l % 32); accumulator register r holds row
 // 8*(r/4) + 4*(l/32) + (r%4).
+#include <type_traits>
+
 #include "common.h"
 
 using namespace tnn_rocm;
@@ -69,6 +71,12 @@ template <> struct GemmTraits<TNN_ROCM_F32> {
     }
 };
 
+// 4-element vector of T as one memory transaction
+template <typename T> struct Vec4;
+template <> struct Vec4<float> { typedef float4 type; };
+template <> struct Vec4<half_t> { typedef uint2 type; };
+template <> struct Vec4<bf16_bits> { typedef uint2 type; };
+
 // ---- epilogues ----------------------------------------------------------------------------------
 template <int DT> struct FloatEpilogue {
     typedef typename Elem<DT>::type T;
@@ -95,6 +103,32 @@ template <int DT> struct FloatEpilogue {
         if (flags & TNN_ROCM_EPI_RESIDUAL)
             v = v + Elem<DT>::ld(&residual[(size_t)m * ldr + n]);
         Elem<DT>::st(&C[(size_t)m * ldc + n], v);
+    }
+    // four consecutive columns n..n+3 of row m (n % 4 == 0, n + 3 < N, rows 4-element aligned)
+    __device__ __forceinline__ void store4(int m, int n, const float (&acc)[4]) const {
+        float v[4] = {acc[0], acc[1], acc[2], acc[3]};
+        if (flags & TNN_ROCM_EPI_BIAS) {
+            float4 b = *reinterpret_cast<const float4 *>(bias + n);
+            v[0] += b.x, v[1] += b.y, v[2] += b.z, v[3] += b.w;
+        }
+        if (flags & TNN_ROCM_EPI_GELU) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                v[t] = (DT == TNN_ROCM_F32) ? gelu_erf(v[t]) : gelu_erf_fast(v[t]);
+        }
+        T packed[4];
+        if (flags & TNN_ROCM_EPI_RESIDUAL) {
+            *reinterpret_cast<typename Vec4<T>::type *>(packed) =
+                *reinterpret_cast<const typename Vec4<T>::type *>(residual + (size_t)m * ldr + n);
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                v[t] += Elem<DT>::ld(&packed[t]);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            Elem<DT>::st(&packed[t], v[t]);
+        *reinterpret_cast<typename Vec4<T>::type *>(C + (size_t)m * ldc + n) =
+            *reinterpret_cast<const typename Vec4<T>::type *>(packed);
     }
 };
 
@@ -137,6 +171,11 @@ struct Int8Epilogue {
                     ((half_t *)out_f)[(size_t)m * ldo + n] = (half_t)d;
             }
         }
+    }
+    __device__ __forceinline__ void store4(int m, int n, const int (&acc)[4]) const {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            store(m, n + t, acc[t], col_const(n + t));
     }
 };
 
@@ -344,6 +383,228 @@ __global__ void __launch_bounds__(WM *WN * 64)
     }
 }
 
+
+// ---- pipelined variant for the aligned x * W^T case ---------------------------------------------------
+// Same tiling idea as gemm_kernel, tuned for the encoder's projection shapes:
+//   * k-slabs of SLAB bytes per row (128 for the large-K launches), so a barrier is amortised over
+//     SLAB/32 MFMA steps per 32x32 block;
+//   * two slabs in flight in registers in addition to the one being consumed from LDS (global loads for
+//     slab k+2 are issued before the MFMAs of slab k), which covers the L2/HBM latency that a one-slab
+//     look-ahead leaves exposed;
+//   * the MFMA operands are swapped (the W panel is the "A" operand), so a lane ends up owning one output
+//     ROW and four consecutive columns per accumulator group: the epilogue reads bias/residual and writes
+//     C with 8-byte (fp16) / 16-byte (fp32) accesses instead of 2-byte ones.
+// LDS is dynamic: 2 buffers x (BM + BN) rows x (SLAB + 16) bytes.
+template <int DT, int BM, int BN, int SLAB, typename Epi>
+__global__ void __launch_bounds__(256)
+    gemm_nk_pipelined_kernel(const typename GemmTraits<DT>::elem *__restrict__ A,
+                             const typename GemmTraits<DT>::elem *__restrict__ B, int M, int N, int K, long lda,
+                             long ldb, int tiles_m, int tiles_n, Epi epi) {
+    typedef typename GemmTraits<DT>::elem T;
+    typedef typename GemmTraits<DT>::acc Acc;
+    constexpr int NT     = 256;
+    constexpr int VEC    = 16 / sizeof(T);
+    constexpr int KB     = SLAB / sizeof(T);
+    constexpr int VPR    = SLAB / 16;  // 16-byte vectors per slab row
+    constexpr int STRIDE = SLAB + 16;
+    constexpr int MT     = BM / 64;
+    constexpr int NTL    = BN / 64;
+    constexpr int A_VECS = BM * VPR / NT;
+    constexpr int B_VECS = BN * VPR / NT;
+    static_assert(BM % 64 == 0 && BN % 64 == 0 && (BM * VPR) % NT == 0 && (BN * VPR) % NT == 0, "tile shape");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_dyn[];
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm   = wave >> 1;
+    const int wn   = wave & 1;
+
+    int pid           = blockIdx.x;
+    const int n_tiles = tiles_m * tiles_n;
+    if ((n_tiles & 7) == 0)
+        pid = (pid & 7) * (n_tiles >> 3) + (pid >> 3);
+    const int m0 = (pid / tiles_n) * BM;
+    const int n0 = (pid % tiles_n) * BN;
+
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 ra0[A_VECS], rb0[B_VECS], ra1[A_VECS], rb1[B_VECS];
+
+    // Loads carry no bounds branches: rows past the matrix edge are clamped to the last row (their products
+    // land in accumulators that the epilogue never stores) and K is a whole number of slabs (checked by the
+    // launcher), so every global load of a slab can be in flight at once.
+    // vector v = tid + i*NT sits in slab row v / VPR at 16-byte column v % VPR; NT is a multiple of VPR, so
+    // the column is the same for every i and the row advances by NT / VPR
+    constexpr int ROW_STEP = NT / VPR;
+    const int vrow = tid / VPR, vcol = tid % VPR;
+    uint32_t a_off[A_VECS], b_off[B_VECS];  // element offsets (the launcher checks they fit 32 bits)
+#pragma unroll
+    for (int i = 0; i < A_VECS; ++i) {
+        int row  = m0 + vrow + i * ROW_STEP;
+        row      = row < M ? row : M - 1;
+        a_off[i] = (uint32_t)row * (uint32_t)lda + (uint32_t)(vcol * VEC);
+    }
+#pragma unroll
+    for (int i = 0; i < B_VECS; ++i) {
+        int row  = n0 + vrow + i * ROW_STEP;
+        row      = row < N ? row : N - 1;
+        b_off[i] = (uint32_t)row * (uint32_t)ldb + (uint32_t)(vcol * VEC);
+    }
+// The three pipeline stages are macros on purpose: passing the register arrays through lambdas kept them in
+// scratch memory (the compiler did not promote them), which costs more than the prefetch gains.
+#define TR_LOAD_GLOBAL(RA, RB, K0)                                                                                    \
+    {                                                                                                                 \
+        _Pragma("unroll") for (int i = 0; i < A_VECS; ++i) RA[i] =                                                    \
+            *reinterpret_cast<const u32x4 *>(A + a_off[i] + (K0));                                                    \
+        _Pragma("unroll") for (int i = 0; i < B_VECS; ++i) RB[i] =                                                    \
+            *reinterpret_cast<const u32x4 *>(B + b_off[i] + (K0));                                                    \
+    }
+#define TR_STORE_LDS(BUF, RA, RB)                                                                                     \
+    {                                                                                                                 \
+        _Pragma("unroll") for (int i = 0; i < A_VECS; ++i) *reinterpret_cast<u32x4 *>(                                \
+            lds_a##BUF + (vrow + i * ROW_STEP) * STRIDE + vcol * 16) = RA[i];                                         \
+        _Pragma("unroll") for (int i = 0; i < B_VECS; ++i) *reinterpret_cast<u32x4 *>(                                \
+            lds_b##BUF + (vrow + i * ROW_STEP) * STRIDE + vcol * 16) = RB[i];                                         \
+    }
+#define TR_COMPUTE(BUF)                                                                                               \
+    {                                                                                                                 \
+        _Pragma("unroll") for (int kk = 0; kk < SLAB / 32; ++kk) {                                                    \
+            uint4 fa[MT], fb[NTL];                                                                                    \
+            _Pragma("unroll") for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const uint4 *>(                  \
+                lds_a##BUF + (wm * (BM / 2) + i * 32 + frag_row) * STRIDE + kk * 32 + frag_off);                      \
+            _Pragma("unroll") for (int j = 0; j < NTL; ++j) fb[j] = *reinterpret_cast<const uint4 *>(                 \
+                lds_b##BUF + (wn * (BN / 2) + j * 32 + frag_row) * STRIDE + kk * 32 + frag_off);                      \
+            _Pragma("unroll") for (int i = 0; i < MT; ++i) _Pragma("unroll") for (int j = 0; j < NTL; ++j)            \
+                GemmTraits<DT>::mma(fb[j], fa[i], acc[i][j]); /* rows of D = n, lanes of D = m */                     \
+        }                                                                                                             \
+    }
+
+    unsigned char *const lds_a0 = lds_dyn, *const lds_b0 = lds_dyn + BM * STRIDE;
+    unsigned char *const lds_a1 = lds_dyn + (BM + BN) * STRIDE, *const lds_b1 = lds_a1 + BM * STRIDE;
+
+    Acc acc[MT][NTL];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NTL; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0;
+
+    const int frag_row = lane & 31;
+    const int frag_off = (lane >> 5) * 16;
+
+    // Slab schedule (two slabs in flight in registers, one in LDS being consumed).  The loop body is branch
+    // free: look-ahead loads past the last slab are clamped to it and their LDS copy is never consumed.
+    const int nk   = K / KB;
+    const int last = (nk - 1) * KB;
+#define TR_CLAMPK(SLABIDX) (((SLABIDX)*KB) < last ? ((SLABIDX)*KB) : last)
+    TR_LOAD_GLOBAL(ra0, rb0, 0);
+    TR_LOAD_GLOBAL(ra1, rb1, TR_CLAMPK(1));
+    TR_STORE_LDS(0, ra0, rb0);
+    __syncthreads();
+    for (int kt = 0; kt + 2 <= nk; kt += 2) {
+        TR_LOAD_GLOBAL(ra0, rb0, TR_CLAMPK(kt + 2));
+        TR_COMPUTE(0);
+        TR_STORE_LDS(1, ra1, rb1);
+        __syncthreads();
+        TR_LOAD_GLOBAL(ra1, rb1, TR_CLAMPK(kt + 3));
+        TR_COMPUTE(1);
+        TR_STORE_LDS(0, ra0, rb0);
+        __syncthreads();
+    }
+    if (nk & 1)
+        TR_COMPUTE(0);
+#undef TR_LOAD_GLOBAL
+#undef TR_STORE_LDS
+#undef TR_COMPUTE
+#undef TR_CLAMPK
+
+    // epilogue: lane owns row m; accumulator group r4 holds columns 8*r4 + 4*(lane/32) + 0..3
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int m = m0 + wm * (BM / 2) + i * 32 + (lane & 31);
+        if (m >= M)
+            continue;
+#pragma unroll
+        for (int j = 0; j < NTL; ++j) {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int n = n0 + wn * (BN / 2) + j * 32 + 8 * r4 + 4 * (lane >> 5);
+                if (n + 3 < N) {
+                    typename std::remove_reference<decltype(acc[i][j][0])>::type v[4] = {
+                        acc[i][j][r4 * 4 + 0], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2], acc[i][j][r4 * 4 + 3]};
+                    epi.store4(m, n, v);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        if (n + t < N)
+                            epi.store(m, n + t, acc[i][j][r4 * 4 + t], epi.col_const(n + t));
+                }
+            }
+        }
+    }
+}
+
+// tuning override for experiments: 0 = heuristic, otherwise (BM, BN, SLAB) of the pipelined kernel
+int g_gemm_force_cfg = 0;
+
+template <int DT, int BM, int BN, int SLAB, typename Epi>
+int launch_pipelined(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb,
+                     const Epi &epi) {
+    typedef typename GemmTraits<DT>::elem T;
+    int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    size_t lds  = (size_t)2 * (BM + BN) * (SLAB + 16);
+    auto kern   = gemm_nk_pipelined_kernel<DT, BM, BN, SLAB, Epi>;
+    if (lds > 64 * 1024) {
+        static bool attr_set = false;  // per instantiation
+        if (!attr_set) {
+            TR_CHECK_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            attr_set = true;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), lds, s, (const T *)A, (const T *)B, M, N, K,
+                       lda, ldb, tiles_m, tiles_n, epi);
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+// Shape heuristic for the pipelined kernel (measured on MI355X at the encoder's projection shapes).
+template <int DT, typename Epi>
+int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb,
+                     const Epi &epi) {
+    auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    int cfg = g_gemm_force_cfg > 0 ? g_gemm_force_cfg : 0;
+    if (cfg == 0) {
+        size_t kbytes = (size_t)K * sizeof(typename GemmTraits<DT>::elem);
+        bool slab128  = kbytes % 128 == 0;
+        // measured on MI355X (fp16): with fewer than ~2 full-size tiles per CU the launch is dominated by pipeline
+        // fill/drain and 64x64 tiles at 4-5 workgroups per CU win (QKV 25 us vs 26, out-proj 12.8 vs 18, FFN2 34.9
+        // vs 38.3 at M=3072); from ~500 tiles of 128x128 on the larger tile wins (M=8192: 34 us vs 37, 89 vs 125)
+        if (tiles(128, 128) >= 500)
+            cfg = slab128 ? 1281281 : 1281280;
+        else
+            cfg = slab128 ? 64641 : 64640;
+    }
+    if (((size_t)K * sizeof(typename GemmTraits<DT>::elem)) % ((cfg % 10) ? 128 : 64) != 0) {
+        set_error("gemm: K=%d is not a whole number of slabs for tuning configuration %d", K, cfg);
+        return TNN_ROCM_ESHAPE;
+    }
+#define TR_FAST(BMv, BNv, SLABv) return launch_pipelined<DT, BMv, BNv, SLABv, Epi>(s, A, B, M, N, K, lda, ldb, epi)
+    switch (cfg) {
+        case 1281281: TR_FAST(128, 128, 128);
+        case 1281280: TR_FAST(128, 128, 64);
+        case 128641: TR_FAST(128, 64, 128);
+        case 128640: TR_FAST(128, 64, 64);
+        case 641281: TR_FAST(64, 128, 128);
+        case 64641: TR_FAST(64, 64, 128);
+        case 64640: TR_FAST(64, 64, 64);
+        default: set_error("gemm: unknown tuning configuration %d", cfg); return TNN_ROCM_EINVAL;
+    }
+#undef TR_FAST
+}
+
 template <int DT, int BM, int BN, int WM, int WN, typename Epi>
 int launch_gemm_cfg(hipStream_t s, bool b_nk, bool aligned, const void *A, const void *B, int M, int N, int K, long lda,
                     long ldb, int batch, int batch_a, int batch_b, long stride_a, long stride_b, const Epi &epi) {
@@ -426,6 +687,11 @@ int tnn_rocm_gemm(void *stream, int dtype, int b_is_nk, const void *A, const voi
         epi.ldc            = ldc;                                                                                     \
         epi.batch_stride_c = sc;                                                                                      \
         epi.batch_stride_r = sr;                                                                                      \
+        bool vec_out = N % 4 == 0 && ldc % 4 == 0 && (((uintptr_t)C) & 15u) == 0 &&                                   \
+                       (!(epilogue & TNN_ROCM_EPI_RESIDUAL) || (ldr % 4 == 0 && (((uintptr_t)residual) & 15u) == 0)) &&\
+                       (!(epilogue & TNN_ROCM_EPI_BIAS) || (((uintptr_t)bias) & 15u) == 0);                            \
+        if (b_is_nk && aligned && batch == 1 && vec_out && g_gemm_force_cfg >= 0 && (K * sizeof(T)) % 64 == 0)        \
+            return launch_gemm_fast<DT, FloatEpilogue<DT>>(s, A, B, M, N, K, lda, ldb, epi);                          \
         return launch_gemm<DT, FloatEpilogue<DT>>(s, b_is_nk != 0, aligned, A, B, M, N, K, lda, ldb, batch, batch_a,  \
                                                   batch_b, sa, sb, epi);                                              \
     }
@@ -461,8 +727,17 @@ int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W, const int32
     epi.out_f       = out_f;
     epi.out_f_dtype = out_f_dtype;
     epi.dq          = dequant_scale;
+    if (aligned && g_gemm_force_cfg >= 0 && K % 64 == 0)
+        return launch_gemm_fast<TNN_ROCM_I8, Int8Epilogue>((hipStream_t)stream, A, W, M, N, K, lda, ldw, epi);
     return launch_gemm<TNN_ROCM_I8, Int8Epilogue>((hipStream_t)stream, true, aligned, A, W, M, N, K, lda, ldw, 1, 1, 1,
                                                   0, 0, epi);
+}
+
+// Experiment hook (not part of the documented ABI): 0 restores the shape heuristic, -1 forces the baseline
+// kernel, other values select a (BM, BN, SLAB) instantiation of the pipelined kernel.
+__attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_config(int cfg) {
+    g_gemm_force_cfg = cfg;
+    return 0;
 }
 
 }  // extern "C"
