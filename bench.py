@@ -125,15 +125,17 @@ def main():
     out_final = inst.output("last_hidden")
     assert np.isfinite(out_final).all()
 
+    # the attention kernel on its own, in the layout the fused layer uses (Q|K row-major, V transposed per head)
     d_lens = torch.from_numpy(lens).cuda()
-    qkv = torch.randn(T, 3 * H, device="cuda").half()
+    qk = torch.randn(T, 2 * H, device="cuda").half()
+    vt = torch.randn(B, cfg.heads, 64, S, device="cuda").half()
     ctx = torch.empty(T, H, device="cuda", dtype=torch.float16)
     for _ in range(5):
-        ops.attention_packed(qkv, B, S, cfg.heads, 0.125, kv_len=d_lens, out=ctx)
+        ops.attention_qk_vt(qk, vt, B, S, cfg.heads, 0.125, kv_len=d_lens, out=ctx)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(50):
-        ops.attention_packed(qkv, B, S, cfg.heads, 0.125, kv_len=d_lens, out=ctx)
+        ops.attention_qk_vt(qk, vt, B, S, cfg.heads, 0.125, kv_len=d_lens, out=ctx)
     e1.record()
     torch.cuda.synchronize()
     attn_ms = e0.elapsed_time(e1) / 50

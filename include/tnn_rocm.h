@@ -126,6 +126,22 @@ TNN_ROCM_API int tnn_rocm_attention(void *stream, int dtype, const void *q, cons
                                     long kv_sh, long kv_ss, long o_sb, long o_sh, long o_ss, float scale,
                                     const float *mask, const int32_t *kv_len);
 
+/* Same computation with V supplied transposed per head, V^T[b][head][d][s] (element at
+ * vt[b*vt_sb + head*vt_sh + d*vt_sd + s], s contiguous, S a multiple of 8): the layout tnn_rocm_gemm_qkv_split
+ * writes, which lets the kernel stage V tiles with 16-byte copies instead of transposing them. */
+TNN_ROCM_API int tnn_rocm_attention_vt(void *stream, int dtype, const void *q, const void *k, const void *vt, void *out,
+                                       int B, int heads, int S, int head_dim, long q_sb, long q_sh, long q_ss,
+                                       long k_sb, long k_sh, long k_ss, long vt_sb, long vt_sh, long vt_sd, long o_sb,
+                                       long o_sh, long o_ss, float scale, const float *mask, const int32_t *kv_len);
+
+/* Fused QKV projection for the attention layer: [T,K] x Wqkv[3H,K]^T + bqkv with the result split on the way out:
+ * Q and K go to qk[T, 2H] (row-major, Q | K column blocks), V goes transposed per head to
+ * vt[B][heads][64][S] (T = B*S tokens, H = heads*64).  Same arithmetic as three MatMul+Add pairs
+ * (cpu_mat_mul_layer_acc.cc:64-117, compute_elewise.cc:37-65) followed by the head-split Permutes
+ * (naive_compute.cc:943-956).  dtype F16 or BF16; K and H multiples of 64. */
+TNN_ROCM_API int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *wqkv, const float *bqkv,
+                                         void *qk, void *vt, int B, int S, int heads, int K);
+
 /* kv_len[b] = 1 + the last key index whose additive mask value is > threshold (0 if none). */
 TNN_ROCM_API int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_t *kv_len, int B, int S,
                                          float threshold);

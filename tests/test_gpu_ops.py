@@ -475,6 +475,38 @@ def test_attention_packed_qkv_layout():
     assert rel_err(out, ref) <= FP16_TOL
 
 
+def test_qkv_split_and_attention_vt():
+    say("qkv_split GEMM + attention with transposed V")
+    B, S, h = 3, 200, 12
+    H = h * 64
+    rng = np.random.default_rng(41)
+    x = torch.from_numpy(rng.standard_normal((B * S, H)).astype(np.float32)).half()
+    w = torch.from_numpy((rng.standard_normal((3 * H, H)) * 0.05).astype(np.float32)).half()
+    bias = (rng.standard_normal(3 * H) * 0.1).astype(np.float32)
+    qk, vt = ops().qkv_split(x.cuda(), w.cuda(), dev(bias), B, S, h)
+    ref = orc.inner_product(x.float().numpy(), w.float().numpy(), bias)
+    got_qk = host(qk)
+    got_v = host(vt).transpose(0, 3, 1, 2).reshape(B * S, H)   # [B,h,64,S] -> [B*S, H]
+    assert rel_err(got_qk, ref[:, :2 * H]) <= FP16_TOL
+    assert rel_err(got_v, ref[:, 2 * H:]) <= FP16_TOL
+    # the transposed copy is exactly the fp16 rounding the row-major epilogue would store
+    plain = host(ops().gemm(x.cuda(), w.cuda(), True, bias=dev(bias)))
+    assert np.array_equal(got_qk, plain[:, :2 * H]) and np.array_equal(got_v, plain[:, 2 * H:])
+    lens = np.array([200, 37, 128], np.int32)
+    out = host(ops().attention_qk_vt(qk, vt, B, S, h, 0.125, kv_len=dev(lens)))
+    # same inputs through the kernel that transposes V itself: results must agree bit for bit
+    qkv = torch.from_numpy(plain.astype(np.float16))
+    out2 = host(ops().attention_packed(qkv.cuda(), B, S, h, 0.125, kv_len=dev(lens)))
+    assert np.array_equal(out, out2)
+    xq = plain.reshape(B, S, 3, h, 64)
+    q, k, v = (np.ascontiguousarray(xq[:, :, i].transpose(0, 2, 1, 3)) for i in range(3))
+    mask = np.zeros((B, S), np.float32)
+    for b_, l in enumerate(lens):
+        mask[b_, l:] = -np.inf
+    ref_o = orc.attention_core(q, k, v, 0.125, mask).transpose(0, 2, 1, 3).reshape(B * S, H)
+    assert rel_err(out, ref_o) <= FP16_TOL
+
+
 def test_mask_to_kv_len():
     say("mask_to_kv_len")
     m = np.zeros((5, 300), np.float32)

@@ -56,13 +56,14 @@ struct AttnParams {
     const uint16_t *q, *k, *v;
     uint16_t *o;
     long q_sb, q_sh, q_ss, kv_sb, kv_sh, kv_ss, o_sb, o_sh, o_ss;
+    long vt_sb, vt_sh, vt_sd;  // V^T layout (VT kernels): element (b, head, d, s) at v[b*vt_sb + head*vt_sh + d*vt_sd + s]
     int S;
     float scale_log2e;  // scale * log2(e)
     const float *mask;  // [B,S] additive or null
     const int32_t *kv_len;
 };
 
-template <int DT, int NW>
+template <int DT, int NW, bool VT>
 __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
     constexpr int NT = NW * 64;
     constexpr int BQ = NW * 32;
@@ -93,7 +94,8 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
 
     const uint16_t *qb = p.q + (size_t)b * p.q_sb + (size_t)head * p.q_sh;
     const uint16_t *kb = p.k + (size_t)b * p.kv_sb + (size_t)head * p.kv_sh;
-    const uint16_t *vb = p.v + (size_t)b * p.kv_sb + (size_t)head * p.kv_sh;
+    const uint16_t *vb = VT ? p.v + (size_t)b * p.vt_sb + (size_t)head * p.vt_sh
+                            : p.v + (size_t)b * p.kv_sb + (size_t)head * p.kv_sh;
     uint16_t *ob       = p.o + (size_t)b * p.o_sb + (size_t)head * p.o_sh;
     const float *mb    = p.mask ? p.mask + (size_t)b * S : nullptr;
 
@@ -122,7 +124,15 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
             rv[i] = make_uint4(0, 0, 0, 0);
             if (key < kv_end) {
                 rk[i] = *reinterpret_cast<const uint4 *>(kb + (size_t)key * p.kv_ss + ch * 8);
-                rv[i] = *reinterpret_cast<const uint4 *>(vb + (size_t)key * p.kv_ss + ch * 8);
+                if (!VT)
+                    rv[i] = *reinterpret_cast<const uint4 *>(vb + (size_t)key * p.kv_ss + ch * 8);
+            }
+            if (VT) {
+                // V^T tile: row d = v >> 3, eight consecutive keys per vector; S is a multiple of 8 (checked by
+                // the launcher), so a vector is either fully inside [0, S) or skipped
+                int d = v >> 3, k8 = kv0 + ch * 8;
+                if (k8 < S)
+                    rv[i] = *reinterpret_cast<const uint4 *>(vb + (size_t)d * p.vt_sd + k8);
             }
         }
         if (tid < kTileKV) {
@@ -136,10 +146,14 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
             int v   = tid + i * NT;
             int key = v >> 3, ch = v & 7;
             *reinterpret_cast<uint4 *>(&lds_k[buf][key * kRowBytes + ch * 16]) = rk[i];
-            const uint16_t *e = reinterpret_cast<const uint16_t *>(&rv[i]);
+            if (VT) {
+                *reinterpret_cast<uint4 *>(&lds_vt[buf][key * kRowBytes + ch * 16]) = rv[i];  // row = d, 8 keys
+            } else {
+                const uint16_t *e = reinterpret_cast<const uint16_t *>(&rv[i]);
 #pragma unroll
-            for (int t = 0; t < 8; ++t)
-                *reinterpret_cast<uint16_t *>(&lds_vt[buf][(ch * 8 + t) * kRowBytes + key * 2]) = e[t];
+                for (int t = 0; t < 8; ++t)
+                    *reinterpret_cast<uint16_t *>(&lds_vt[buf][(ch * 8 + t) * kRowBytes + key * 2]) = e[t];
+            }
         }
         if (tid < kTileKV)
             lds_bias[buf][tid] = rbias;
@@ -189,7 +203,7 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
                 float bv[4] = {bias.x, bias.y, bias.z, bias.w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float s2             = sacc[kt][r4 * 4 + e] * p.scale_log2e + bv[e];
+                    float s2             = fmaf(sacc[kt][r4 * 4 + e], p.scale_log2e, bv[e]);
                     sacc[kt][r4 * 4 + e] = s2;
                     mx                   = fmaxf(mx, s2);
                 }
@@ -277,6 +291,26 @@ __global__ void mask_to_kv_len_kernel(const float *__restrict__ mask, int32_t *_
         kv_len[b] = last + 1;
 }
 
+// 128-row query blocks when that already gives >= 2 workgroups per CU, else 64-row blocks
+template <bool VT> int launch_attention(hipStream_t s, int dtype, const AttnParams &p, int B, int heads, int S) {
+    long blocks128 = (long)((S + 127) / 128) * heads * B;
+    if (blocks128 >= 512) {
+        dim3 grid((S + 127) / 128, heads, B);
+        if (dtype == TNN_ROCM_F16)
+            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_F16, 4, VT>), grid, dim3(256), 0, s, p);
+        else
+            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_BF16, 4, VT>), grid, dim3(256), 0, s, p);
+    } else {
+        dim3 grid((S + 63) / 64, heads, B);
+        if (dtype == TNN_ROCM_F16)
+            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_F16, 2, VT>), grid, dim3(128), 0, s, p);
+        else
+            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_BF16, 2, VT>), grid, dim3(128), 0, s, p);
+    }
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -312,24 +346,44 @@ int tnn_rocm_attention(void *stream, int dtype, const void *q, const void *k, co
     p.scale_log2e = scale * kLog2e;
     p.mask        = mask;
     p.kv_len      = kv_len;
-    hipStream_t s = (hipStream_t)stream;
-    // 128-row query blocks when that already gives >= 2 workgroups per CU, else 64-row blocks
-    long blocks128 = (long)((S + 127) / 128) * heads * B;
-    if (blocks128 >= 512) {
-        dim3 grid((S + 127) / 128, heads, B);
-        if (dtype == TNN_ROCM_F16)
-            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_F16, 4>), grid, dim3(256), 0, s, p);
-        else
-            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_BF16, 4>), grid, dim3(256), 0, s, p);
-    } else {
-        dim3 grid((S + 63) / 64, heads, B);
-        if (dtype == TNN_ROCM_F16)
-            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_F16, 2>), grid, dim3(128), 0, s, p);
-        else
-            hipLaunchKernelGGL((attention_kernel<TNN_ROCM_BF16, 2>), grid, dim3(128), 0, s, p);
-    }
-    TR_CHECK_LAUNCH();
-    return 0;
+    p.vt_sb = p.vt_sh = p.vt_sd = 0;
+    return launch_attention<false>((hipStream_t)stream, dtype, p, B, heads, S);
+}
+
+int tnn_rocm_attention_vt(void *stream, int dtype, const void *q, const void *k, const void *vt, void *out, int B,
+                          int heads, int S, int head_dim, long q_sb, long q_sh, long q_ss, long k_sb, long k_sh,
+                          long k_ss, long vt_sb, long vt_sh, long vt_sd, long o_sb, long o_sh, long o_ss, float scale,
+                          const float *mask, const int32_t *kv_len) {
+    TR_REQUIRE(B >= 0 && heads >= 0 && S >= 0, TNN_ROCM_ESHAPE, "attention_vt: negative size");
+    if (B == 0 || heads == 0 || S == 0)
+        return 0;
+    TR_REQUIRE(q && k && vt && out, TNN_ROCM_EINVAL, "attention_vt: null pointer");
+    TR_REQUIRE(head_dim == kD, TNN_ROCM_ESHAPE, "attention_vt: head_dim %d unsupported (64 only)", head_dim);
+    TR_REQUIRE(dtype == TNN_ROCM_F16 || dtype == TNN_ROCM_BF16, TNN_ROCM_EDTYPE,
+               "attention_vt: dtype %d unsupported (F16 or BF16)", dtype);
+    TR_REQUIRE(B <= 65535 && heads <= 65535, TNN_ROCM_ESHAPE, "attention_vt: batch/heads exceed the grid limit");
+    TR_REQUIRE(S % 8 == 0, TNN_ROCM_ESHAPE, "attention_vt: S=%d must be a multiple of 8 (16-byte V^T vectors)", S);
+    auto ok = [](const void *ptr, long a, long b2, long c) {
+        return ((((uintptr_t)ptr) & 15u) == 0) && a % 8 == 0 && b2 % 8 == 0 && c % 8 == 0;
+    };
+    TR_REQUIRE(ok(q, q_sb, q_sh, q_ss) && ok(k, k_sb, k_sh, k_ss) && ok(vt, vt_sb, vt_sh, vt_sd) &&
+                   ok(out, o_sb, o_sh, o_ss),
+               TNN_ROCM_EALIGN, "attention_vt: pointers must be 16-byte aligned and strides multiples of 8 elements");
+    TR_REQUIRE(q_ss >= kD && k_ss >= kD && o_ss >= kD && vt_sd >= S, TNN_ROCM_ESHAPE, "attention_vt: stride too small");
+    AttnParams p;
+    p.q = (const uint16_t *)q;
+    p.k = (const uint16_t *)k;
+    p.v = (const uint16_t *)vt;
+    p.o = (uint16_t *)out;
+    p.q_sb = q_sb, p.q_sh = q_sh, p.q_ss = q_ss;
+    p.kv_sb = k_sb, p.kv_sh = k_sh, p.kv_ss = k_ss;
+    p.vt_sb = vt_sb, p.vt_sh = vt_sh, p.vt_sd = vt_sd;
+    p.o_sb = o_sb, p.o_sh = o_sh, p.o_ss = o_ss;
+    p.S           = S;
+    p.scale_log2e = scale * kLog2e;
+    p.mask        = mask;
+    p.kv_len      = kv_len;
+    return launch_attention<true>((hipStream_t)stream, dtype, p, B, heads, S);
 }
 
 int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_t *kv_len, int B, int S, float threshold) {

@@ -132,6 +132,46 @@ template <int DT> struct FloatEpilogue {
     }
 };
 
+// QKV projection epilogue: columns [0,2H) -> qk[T,2H]; columns [2H,3H) -> V^T[b][head][d][s]
+template <int DT> struct QkvSplitEpilogue {
+    typedef typename Elem<DT>::type T;
+    const float *bias;
+    T *qk;
+    T *vt;
+    int H, S, heads;
+    __device__ __forceinline__ void set_batch(int) {}
+    __device__ __forceinline__ float col_const(int n) const { return bias ? bias[n] : 0.f; }
+    __device__ __forceinline__ void store(int m, int n, float acc, float bias_n) const {
+        float v = acc + bias_n;
+        if (n < 2 * H) {
+            Elem<DT>::st(&qk[(size_t)m * 2 * H + n], v);
+        } else {
+            int c = n - 2 * H, b = m / S, s = m - b * S;
+            Elem<DT>::st(&vt[(((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s], v);
+        }
+    }
+    __device__ __forceinline__ void store4(int m, int n, const float (&acc)[4]) const {
+        float v[4] = {acc[0], acc[1], acc[2], acc[3]};
+        if (bias) {
+            float4 b4 = *reinterpret_cast<const float4 *>(bias + n);
+            v[0] += b4.x, v[1] += b4.y, v[2] += b4.z, v[3] += b4.w;
+        }
+        if (n < 2 * H) {  // H is a multiple of 64, so a group of four never straddles the boundary
+            T packed[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                Elem<DT>::st(&packed[t], v[t]);
+            *reinterpret_cast<uint2 *>(qk + (size_t)m * 2 * H + n) = *reinterpret_cast<const uint2 *>(packed);
+        } else {
+            int c = n - 2 * H, b = m / S, s = m - b * S;
+            T *dst = vt + (((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s;  // lanes = consecutive s
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                Elem<DT>::st(dst + (size_t)t * S, v[t]);
+        }
+    }
+};
+
 struct Int8Epilogue {
     const int32_t *bias;
     const float *scale;
@@ -731,6 +771,37 @@ int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W, const int32
         return launch_gemm_fast<TNN_ROCM_I8, Int8Epilogue>((hipStream_t)stream, A, W, M, N, K, lda, ldw, epi);
     return launch_gemm<TNN_ROCM_I8, Int8Epilogue>((hipStream_t)stream, true, aligned, A, W, M, N, K, lda, ldw, 1, 1, 1,
                                                   0, 0, epi);
+}
+
+int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *wqkv, const float *bqkv, void *qk,
+                            void *vt, int B, int S, int heads, int K) {
+    TR_REQUIRE(B >= 0 && S >= 0 && heads >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_qkv_split: negative size");
+    if (B == 0 || S == 0 || heads == 0)
+        return 0;
+    TR_REQUIRE(x && wqkv && qk && vt, TNN_ROCM_EINVAL, "gemm_qkv_split: null pointer");
+    TR_REQUIRE(dtype == TNN_ROCM_F16 || dtype == TNN_ROCM_BF16, TNN_ROCM_EDTYPE, "gemm_qkv_split: F16 or BF16 only");
+    TR_REQUIRE(K > 0 && K % 64 == 0, TNN_ROCM_ESHAPE, "gemm_qkv_split: K=%d must be a positive multiple of 64", K);
+    TR_REQUIRE((long)B * S < (1l << 24) && (long)B * S * 3 * heads * 64 < (1l << 31), TNN_ROCM_ESHAPE,
+               "gemm_qkv_split: problem too large for 32-bit panel offsets");
+    TR_REQUIRE(al16(x) && al16(wqkv) && al16(qk) && al16(vt) && (!bqkv || al16(bqkv)), TNN_ROCM_EALIGN,
+               "gemm_qkv_split: pointers must be 16-byte aligned");
+    const int H = heads * 64, T = B * S;
+#define TR_QKV(DT)                                                                                                    \
+    {                                                                                                                 \
+        QkvSplitEpilogue<DT> epi;                                                                                     \
+        epi.bias  = bqkv;                                                                                             \
+        epi.qk    = (Elem<DT>::type *)qk;                                                                             \
+        epi.vt    = (Elem<DT>::type *)vt;                                                                             \
+        epi.H     = H;                                                                                                \
+        epi.S     = S;                                                                                                \
+        epi.heads = heads;                                                                                            \
+        return launch_gemm_fast<DT, QkvSplitEpilogue<DT>>((hipStream_t)stream, x, wqkv, T, 3 * H, K, K, K, epi);      \
+    }
+    if (dtype == TNN_ROCM_F16)
+        TR_QKV(TNN_ROCM_F16)
+    else
+        TR_QKV(TNN_ROCM_BF16)
+#undef TR_QKV
 }
 
 // Experiment hook (not part of the documented ABI): 0 restores the shape heuristic, -1 forces the baseline

@@ -33,6 +33,8 @@ RocmContext::~RocmContext() {
     if (stream_)
         tnn_rocm_stream_sync(stream_);
     tnn_rocm_free(workspace_);
+    tnn_rocm_free(mask_cache_.mask_f32);
+    tnn_rocm_free(mask_cache_.kv_len);
     tnn_rocm_free_host(error_flag_);
     tnn_rocm_stream_destroy(stream_);
 }
@@ -47,6 +49,33 @@ Status RocmContext::GetCommandQueue(void **command_queue) {
 Status RocmContext::OnInstanceForwardBegin() {
     // one context per instance, used by one thread at a time; select its device for this thread
     ROCM_CALL(tnn_rocm_set_device(device_id_));
+    ++forward_epoch_;
+    return TNN_OK;
+}
+
+Status RocmContext::AttentionMask(const void *mask_blob, int mask_dtype, int B, int S, const float **mask_f32,
+                                  const int32_t **kv_len) {
+    auto &c = mask_cache_;
+    if (c.B != B || c.S != S || !c.kv_len) {
+        ROCM_CALL(tnn_rocm_stream_sync(stream_));
+        tnn_rocm_free(c.mask_f32);
+        tnn_rocm_free(c.kv_len);
+        c.mask_f32 = c.kv_len = nullptr;
+        ROCM_CALL(tnn_rocm_malloc(&c.mask_f32, (size_t)B * S * sizeof(float)));
+        ROCM_CALL(tnn_rocm_malloc(&c.kv_len, (size_t)B * sizeof(int32_t)));
+        c.B = B, c.S = S, c.src = nullptr;
+    }
+    const float *m = mask_dtype == TNN_ROCM_F32 ? (const float *)mask_blob : (const float *)c.mask_f32;
+    if (c.src != mask_blob || c.epoch != forward_epoch_) {
+        if (mask_dtype != TNN_ROCM_F32)
+            ROCM_CALL(tnn_rocm_cast(stream_, mask_dtype, mask_blob, TNN_ROCM_F32, c.mask_f32, (size_t)B * S));
+        // keys whose additive mask is <= -1000 after the last visible key contribute exp(-1000 - max) == 0 in fp32
+        ROCM_CALL(tnn_rocm_mask_to_kv_len(stream_, m, (int32_t *)c.kv_len, B, S, -1000.0f));
+        c.src   = mask_blob;
+        c.epoch = forward_epoch_;
+    }
+    *mask_f32 = m;
+    *kv_len   = (const int32_t *)c.kv_len;
     return TNN_OK;
 }
 

@@ -39,6 +39,10 @@ public:
     Status Workspace(size_t bytes, void **ptr);
     // page-locked word kernels raise on a data error (e.g. Gather index out of range)
     int32_t *ErrorFlag() { return error_flag_; }
+    // The padding mask is one blob shared by every attention layer of a forward pass: the first layer that asks
+    // derives its fp32 copy and the per-sequence key counts, later layers of the same forward reuse them.
+    Status AttentionMask(const void *mask_blob, int mask_dtype, int B, int S, const float **mask_f32,
+                         const int32_t **kv_len);
 
 private:
     int device_id_       = 0;
@@ -46,6 +50,13 @@ private:
     void *workspace_     = nullptr;
     size_t workspace_sz_ = 0;
     int32_t *error_flag_ = nullptr;
+    uint64_t forward_epoch_ = 0;
+    struct MaskEntry {
+        const void *src = nullptr;
+        uint64_t epoch  = 0;
+        int B = 0, S = 0;
+        void *mask_f32 = nullptr, *kv_len = nullptr;
+    } mask_cache_;
 };
 
 class RocmDevice : public AbstractDevice {

@@ -478,10 +478,6 @@ public:
                           TNN_OK);
             RETURN_ON_NEQ(UploadConverted(res->bias.force_to<void *>(), (size_t)3 * H_, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &bias_),
                           TNN_OK);
-            std::vector<int32_t> zeros(B_ > 0 ? B_ : 1, 0);
-            RETURN_ON_NEQ(UploadConverted(zeros.data(), zeros.size(), DATA_TYPE_INT32, DATA_TYPE_INT32, &kv_len_), TNN_OK);
-            std::vector<float> mz((size_t)(B_ * seq_ > 0 ? B_ * seq_ : 1), 0.f);
-            RETURN_ON_NEQ(UploadConverted(mz.data(), mz.size(), DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &mask_f32_), TNN_OK);
         }
         return TNN_OK;
     }
@@ -492,25 +488,30 @@ public:
         size_t es   = (size_t)DataTypeUtils::GetBytesSize(dt);
         void *qkv   = nullptr;
         RETURN_ON_NEQ(context_->Workspace((size_t)T_ * 3 * H_ * es, &qkv), TNN_OK);
-        ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 1, Ptr(inputs[0]), weight_, qkv, T_, 3 * H_, H_, H_, H_, 3 * H_, 1, 1, 1,
-                                TNN_ROCM_EPI_BIAS, (const float *)bias_, nullptr, 0));
         const float *mask = nullptr;
         const int32_t *kv = nullptr;
         if (p->has_mask) {
             Blob *mb = In(inputs[1]);
-            if (mb->GetBlobDesc().data_type == DATA_TYPE_FLOAT) {
-                mask = (const float *)Ptr(mb);
-            } else {
-                ROCM_CALL(tnn_rocm_cast(Stream(), (int)mb->GetBlobDesc().data_type, Ptr(mb), TNN_ROCM_F32, mask_f32_,
-                                        (size_t)B_ * seq_));
-                mask = (const float *)mask_f32_;
-            }
-            // keys whose mask is <= -1000 after the last visible key contribute exp(-1000 - max) == 0 in fp32
-            ROCM_CALL(tnn_rocm_mask_to_kv_len(Stream(), mask, (int32_t *)kv_len_, B_, seq_, -1000.0f));
-            kv = (const int32_t *)kv_len_;
+            RETURN_ON_NEQ(context_->AttentionMask(Ptr(mb), (int)mb->GetBlobDesc().data_type, B_, seq_, &mask, &kv), TNN_OK);
         }
         const char *base = (const char *)qkv;
-        long row = 3L * H_, d = p->head_dim;
+        const long d     = p->head_dim;
+        if (seq_ % 8 == 0 && H_ % 64 == 0) {
+            // projection writes Q|K row-major and V already transposed per head: the attention kernel then stages
+            // V tiles with 16-byte copies
+            char *vt = (char *)qkv + (size_t)T_ * 2 * H_ * es;
+            ROCM_CALL(tnn_rocm_gemm_qkv_split(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_, qkv, vt, B_,
+                                              seq_, p->heads, H_));
+            const long row = 2L * H_;
+            ROCM_CALL(tnn_rocm_attention_vt(Stream(), (int)dt, base, base + (size_t)H_ * es, vt, Ptr(outputs[0]), B_, p->heads,
+                                            seq_, p->head_dim, (long)seq_ * row, d, row, (long)seq_ * row, d, row,
+                                            (long)p->heads * 64 * seq_, 64L * seq_, (long)seq_, (long)seq_ * H_, d, (long)H_,
+                                            p->scale, mask, kv));
+            return TNN_OK;
+        }
+        ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 1, Ptr(inputs[0]), weight_, qkv, T_, 3 * H_, H_, H_, H_, 3 * H_, 1, 1, 1,
+                                TNN_ROCM_EPI_BIAS, (const float *)bias_, nullptr, 0));
+        const long row = 3L * H_;
         ROCM_CALL(tnn_rocm_attention(Stream(), (int)dt, base, base + (size_t)H_ * es, base + (size_t)2 * H_ * es,
                                      Ptr(outputs[0]), B_, p->heads, seq_, p->head_dim, (long)seq_ * row, d, row,
                                      (long)seq_ * row, d, row, (long)seq_ * H_, d, (long)H_, p->scale, mask, kv));
@@ -518,7 +519,7 @@ public:
     }
 
 private:
-    void *weight_ = nullptr, *bias_ = nullptr, *kv_len_ = nullptr, *mask_f32_ = nullptr;
+    void *weight_ = nullptr, *bias_ = nullptr;
     int H_ = 0, T_ = 0, B_ = 0, seq_ = 0;
 };
 REGISTER_ROCM_ACC(RocmFusedAttentionLayerAcc, LAYER_ROCM_FUSED_ATTENTION);

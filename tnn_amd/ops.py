@@ -84,6 +84,31 @@ def attention_packed(qkv, B, S, heads, scale, mask=None, kv_len=None, out=None):
     return out
 
 
+def qkv_split(x, wqkv, bqkv, B, S, heads):
+    """x [B*S, K], wqkv [3H, K] -> (qk [B*S, 2H], vt [B, heads, 64, S])"""
+    _chk(x, wqkv, bqkv)
+    H = heads * 64
+    qk = torch.empty(B * S, 2 * H, dtype=x.dtype, device=x.device)
+    vt = torch.empty(B, heads, 64, S, dtype=x.dtype, device=x.device)
+    capi.call("tnn_rocm_gemm_qkv_split", _stream(), dt(x), _p(x), _p(wqkv), _p(bqkv), _p(qk), _p(vt), B, S, heads,
+              x.shape[1])
+    return qk, vt
+
+
+def attention_qk_vt(qk, vt, B, S, heads, scale, mask=None, kv_len=None, out=None):
+    """qk [B*S, 2H] (Q | K), vt [B, heads, 64, S]; out [B*S, H]"""
+    _chk(qk, vt, mask, kv_len, out)
+    H = heads * 64
+    if out is None:
+        out = torch.empty(B * S, H, dtype=qk.dtype, device=qk.device)
+    es = qk.element_size()
+    base = qk.data_ptr()
+    capi.call("tnn_rocm_attention_vt", _stream(), dt(qk), base, base + H * es, _p(vt), _p(out), B, heads, S, 64,
+              S * 2 * H, 64, 2 * H, S * 2 * H, 64, 2 * H, heads * 64 * S, 64 * S, S, S * H, 64, H, float(scale),
+              _p(mask), _p(kv_len))
+    return out
+
+
 def mask_to_kv_len(mask, threshold=-1000.0):
     _chk(mask)
     B, S = mask.shape
