@@ -33,7 +33,7 @@ constexpr float kLog2e  = 1.4426950408889634f;
 
 template <int DT> struct AttnT;
 template <> struct AttnT<TNN_ROCM_F16> {
-    static __device__ __forceinline__ void mma(const uint4 &a, const uint4 &b, f32x16 &c) {
+    template <typename V> static __device__ __forceinline__ void mma(const V &a, const V &b, f32x16 &c) {
         c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
                                                    0);
     }
@@ -43,7 +43,7 @@ template <> struct AttnT<TNN_ROCM_F16> {
     }
 };
 template <> struct AttnT<TNN_ROCM_BF16> {
-    static __device__ __forceinline__ void mma(const uint4 &a, const uint4 &b, f32x16 &c) {
+    template <typename V> static __device__ __forceinline__ void mma(const V &a, const V &b, f32x16 &c) {
         c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
                                                     0, 0);
     }
@@ -63,12 +63,16 @@ struct AttnParams {
     const int32_t *kv_len;
 };
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
 template <int DT, int NW, bool VT>
 __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
     constexpr int NT = NW * 64;
     constexpr int BQ = NW * 32;
-    // per tile: 64 keys x 8 sixteen-byte chunks
-    constexpr int KV_VECS = kTileKV * 8 / NT;
+    // per tile: 64 rows (keys, or d for V^T) x 8 sixteen-byte chunks
+    constexpr int KV_VECS  = kTileKV * 8 / NT;
+    constexpr int ROW_STEP = NT / 8;
     static_assert(kTileKV * 8 % NT == 0, "tile must divide over the workgroup");
 
     __shared__ __attribute__((aligned(16))) unsigned char lds_k[2][kTileKV * kRowBytes];
@@ -99,65 +103,65 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
     uint16_t *ob       = p.o + (size_t)b * p.o_sb + (size_t)head * p.o_sh;
     const float *mb    = p.mask ? p.mask + (size_t)b * S : nullptr;
 
+    // No load below is guarded by a branch: row indices past the end are clamped to the last valid row.  Keys at or
+    // beyond kv_end then carry finite (wrong) data, and their score bias of -inf makes their probability exactly 0,
+    // so neither the max, the sum nor P.V sees them; query rows past S are computed but never stored.
     // Q fragments (B operand of S^T = K Q^T): lane (lq, g) holds Q[q0+lq][16*kk + 8*g .. +7]
-    uint4 qf[4];
+    u32x4 qf[4];
     {
         int qrow = q0 + lq;
+        qrow     = qrow < S ? qrow : S - 1;
+        const uint16_t *qp = qb + (size_t)qrow * p.q_ss + g * 8;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            qf[kk] = make_uint4(0, 0, 0, 0);
-            if (qrow < S)
-                qf[kk] = *reinterpret_cast<const uint4 *>(qb + (size_t)qrow * p.q_ss + kk * 16 + g * 8);
-        }
+        for (int kk = 0; kk < 4; ++kk)
+            qf[kk] = *reinterpret_cast<const u32x4 *>(qp + kk * 16);
     }
 
-    uint4 rk[KV_VECS], rv[KV_VECS];
+    const int vrow = tid >> 3, vch = tid & 7;  // this thread's row / 16-byte chunk inside a tile (plus i*ROW_STEP)
+    u32x4 rk[KV_VECS], rv[KV_VECS];
     float rbias = 0.f;
 
-    auto load_tile = [&](int t) {
-        int kv0 = t * kTileKV;
-#pragma unroll
-        for (int i = 0; i < KV_VECS; ++i) {
-            int v   = tid + i * NT;
-            int key = kv0 + (v >> 3), ch = v & 7;
-            rk[i] = make_uint4(0, 0, 0, 0);
-            rv[i] = make_uint4(0, 0, 0, 0);
-            if (key < kv_end) {
-                rk[i] = *reinterpret_cast<const uint4 *>(kb + (size_t)key * p.kv_ss + ch * 8);
-                if (!VT)
-                    rv[i] = *reinterpret_cast<const uint4 *>(vb + (size_t)key * p.kv_ss + ch * 8);
-            }
-            if (VT) {
-                // V^T tile: row d = v >> 3, eight consecutive keys per vector; S is a multiple of 8 (checked by
-                // the launcher), so a vector is either fully inside [0, S) or skipped
-                int d = v >> 3, k8 = kv0 + ch * 8;
-                if (k8 < S)
-                    rv[i] = *reinterpret_cast<const uint4 *>(vb + (size_t)d * p.vt_sd + k8);
-            }
-        }
-        if (tid < kTileKV) {
-            int key = kv0 + tid;
-            rbias   = key < kv_end ? (mb ? mb[key] * kLog2e : 0.f) : -INFINITY;
-        }
-    };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < KV_VECS; ++i) {
-            int v   = tid + i * NT;
-            int key = v >> 3, ch = v & 7;
-            *reinterpret_cast<uint4 *>(&lds_k[buf][key * kRowBytes + ch * 16]) = rk[i];
-            if (VT) {
-                *reinterpret_cast<uint4 *>(&lds_vt[buf][key * kRowBytes + ch * 16]) = rv[i];  // row = d, 8 keys
-            } else {
-                const uint16_t *e = reinterpret_cast<const uint16_t *>(&rv[i]);
-#pragma unroll
-                for (int t = 0; t < 8; ++t)
-                    *reinterpret_cast<uint16_t *>(&lds_vt[buf][(ch * 8 + t) * kRowBytes + key * 2]) = e[t];
-            }
-        }
-        if (tid < kTileKV)
-            lds_bias[buf][tid] = rbias;
-    };
+#define TR_LOAD_TILE(T)                                                                                               \
+    {                                                                                                                 \
+        const int kv0 = (T) * kTileKV;                                                                                \
+        _Pragma("unroll") for (int i = 0; i < KV_VECS; ++i) {                                                         \
+            int key = kv0 + vrow + i * ROW_STEP;                                                                      \
+            key     = key < S ? key : S - 1;                                                                          \
+            rk[i]   = *reinterpret_cast<const u32x4 *>(kb + (size_t)key * p.kv_ss + vch * 8);                         \
+            if (VT) {                                                                                                 \
+                int k8 = kv0 + vch * 8;                                                                               \
+                k8     = k8 < S ? k8 : S - 8;                                                                         \
+                rv[i]  = *reinterpret_cast<const u32x4 *>(vb + (size_t)(vrow + i * ROW_STEP) * p.vt_sd + k8);         \
+            } else {                                                                                                  \
+                rv[i] = *reinterpret_cast<const u32x4 *>(vb + (size_t)key * p.kv_ss + vch * 8);                       \
+            }                                                                                                         \
+        }                                                                                                             \
+        if (tid < kTileKV) {                                                                                          \
+            int key  = kv0 + tid;                                                                                     \
+            int keyc = key < S ? key : S - 1;                                                                         \
+            float mv = mb ? mb[keyc] * kLog2e : 0.f;                                                                  \
+            rbias    = key < kv_end ? mv : -INFINITY;                                                                 \
+        }                                                                                                             \
+    }
+#define TR_STORE_TILE(BUF)                                                                                            \
+    {                                                                                                                 \
+        _Pragma("unroll") for (int i = 0; i < KV_VECS; ++i) {                                                         \
+            const int row = vrow + i * ROW_STEP;                                                                      \
+            *reinterpret_cast<u32x4 *>(&lds_k[BUF][row * kRowBytes + vch * 16]) = rk[i];                              \
+            if (VT) {                                                                                                 \
+                *reinterpret_cast<u32x4 *>(&lds_vt[BUF][row * kRowBytes + vch * 16]) = rv[i]; /* row = d, 8 keys */   \
+            } else {                                                                                                  \
+                _Pragma("unroll") for (int t = 0; t < 4; ++t) {                                                       \
+                    *reinterpret_cast<uint16_t *>(&lds_vt[BUF][(vch * 8 + 2 * t) * kRowBytes + row * 2]) =            \
+                        (uint16_t)(rv[i][t] & 0xffffu);                                                               \
+                    *reinterpret_cast<uint16_t *>(&lds_vt[BUF][(vch * 8 + 2 * t + 1) * kRowBytes + row * 2]) =        \
+                        (uint16_t)(rv[i][t] >> 16);                                                                   \
+                }                                                                                                     \
+            }                                                                                                         \
+        }                                                                                                             \
+        if (tid < kTileKV)                                                                                            \
+            lds_bias[BUF][tid] = rbias;                                                                               \
+    }
 
     f32x16 oacc[2];
 #pragma unroll
@@ -168,15 +172,16 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
     float m_i = -INFINITY, l_i = 0.f;
 
     if (n_tiles > 0) {
-        load_tile(0);
-        store_tile(0);
+        TR_LOAD_TILE(0);
+        TR_STORE_TILE(0);
     }
     __syncthreads();
 
     for (int t = 0; t < n_tiles; ++t) {
         const int buf = t & 1;
-        if (t + 1 < n_tiles)
-            load_tile(t + 1);
+        // look-ahead load of the next tile (clamped to the last one: the redundant copy is never consumed)
+        const int tn = t + 1 < n_tiles ? t + 1 : t;
+        TR_LOAD_TILE(tn);
 
         // ---- S^T = K Q^T for the 64 keys of the tile: two 32-key blocks
         f32x16 sacc[2];
@@ -187,8 +192,7 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
                 sacc[kt][r] = 0.f;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
-                uint4 kf =
-                    *reinterpret_cast<const uint4 *>(&lds_k[buf][(kt * 32 + lq) * kRowBytes + kk * 32 + g * 16]);
+                u32x4 kf = *reinterpret_cast<const u32x4 *>(&lds_k[buf][(kt * 32 + lq) * kRowBytes + kk * 32 + g * 16]);
                 AttnT<DT>::mma(kf, qf[kk], sacc[kt]);
             }
         }
@@ -223,37 +227,41 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
                 rs += pv;
             }
         rs += __shfl_xor(rs, 32, 64);
-        l_i = l_i * alpha + rs;
+        l_i = fmaf(l_i, alpha, rs);
+        // the running maximum rarely moves after the first tiles: skip the 32 rescale multiplies when no lane's did
+        if (!__all(m_new == m_i)) {
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    oacc[dt][r] *= alpha;
+        }
         m_i = m_new;
-#pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                oacc[dt][r] *= alpha;
 
         // ---- O^T += V^T P^T : four 16-key steps
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
             const int kt = st >> 1, j = st & 1;
-            uint4 pf;
-            pf.x = AttnT<DT>::pack2(sacc[kt][8 * j + 0], sacc[kt][8 * j + 1]);
-            pf.y = AttnT<DT>::pack2(sacc[kt][8 * j + 2], sacc[kt][8 * j + 3]);
-            pf.z = AttnT<DT>::pack2(sacc[kt][8 * j + 4], sacc[kt][8 * j + 5]);
-            pf.w = AttnT<DT>::pack2(sacc[kt][8 * j + 6], sacc[kt][8 * j + 7]);
+            u32x4 pf;
+            pf[0] = AttnT<DT>::pack2(sacc[kt][8 * j + 0], sacc[kt][8 * j + 1]);
+            pf[1] = AttnT<DT>::pack2(sacc[kt][8 * j + 2], sacc[kt][8 * j + 3]);
+            pf[2] = AttnT<DT>::pack2(sacc[kt][8 * j + 4], sacc[kt][8 * j + 5]);
+            pf[3] = AttnT<DT>::pack2(sacc[kt][8 * j + 6], sacc[kt][8 * j + 7]);
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt) {
                 const unsigned char *row = &lds_vt[buf][(dt * 32 + lq) * kRowBytes + (st * 16 + g * 4) * 2];
-                uint2 lo                 = *reinterpret_cast<const uint2 *>(row);
-                uint2 hi                 = *reinterpret_cast<const uint2 *>(row + 16);
-                uint4 vf                 = make_uint4(lo.x, lo.y, hi.x, hi.y);
+                u32x2 lo                 = *reinterpret_cast<const u32x2 *>(row);
+                u32x2 hi                 = *reinterpret_cast<const u32x2 *>(row + 16);
+                u32x4 vf                 = {lo[0], lo[1], hi[0], hi[1]};
                 AttnT<DT>::mma(vf, pf, oacc[dt]);
             }
         }
 
-        if (t + 1 < n_tiles)
-            store_tile(buf ^ 1);
+        TR_STORE_TILE(buf ^ 1);
         __syncthreads();
     }
+#undef TR_LOAD_TILE
+#undef TR_STORE_TILE
 
     // ---- normalise and store: lane owns query row q0+lq; register r of block dt is
     //      d = dt*32 + 8*(r/4) + 4*g + (r%4)  -> four consecutive d per register group
@@ -265,10 +273,10 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-                uint2 w;
-                w.x = AttnT<DT>::pack2(oacc[dt][r4 * 4 + 0] * inv, oacc[dt][r4 * 4 + 1] * inv);
-                w.y = AttnT<DT>::pack2(oacc[dt][r4 * 4 + 2] * inv, oacc[dt][r4 * 4 + 3] * inv);
-                *reinterpret_cast<uint2 *>(orow + dt * 32 + r4 * 8 + g * 4) = w;
+                u32x2 w;
+                w[0] = AttnT<DT>::pack2(oacc[dt][r4 * 4 + 0] * inv, oacc[dt][r4 * 4 + 1] * inv);
+                w[1] = AttnT<DT>::pack2(oacc[dt][r4 * 4 + 2] * inv, oacc[dt][r4 * 4 + 3] * inv);
+                *reinterpret_cast<u32x2 *>(orow + dt * 32 + r4 * 8 + g * 4) = w;
             }
     }
 }
