@@ -73,6 +73,14 @@ TNN_ROCM_API int tnn_rocm_event_destroy(void *event);
 TNN_ROCM_API int tnn_rocm_event_record(void *event, void *stream);
 TNN_ROCM_API int tnn_rocm_event_elapsed_ms(void *start, void *stop, float *ms); /* synchronises on `stop` */
 
+/* Stream capture into an executable graph, used by the network to replay a whole forward pass (about ninety
+ * launches for a 12-layer encoder) with one submission.  Only kernel launches may be issued on the stream between
+ * begin and end (no allocation, synchronisation or memset). */
+TNN_ROCM_API int tnn_rocm_graph_begin_capture(void *stream);
+TNN_ROCM_API int tnn_rocm_graph_end_capture(void *stream, void **graph_exec);
+TNN_ROCM_API int tnn_rocm_graph_launch(void *graph_exec, void *stream);
+TNN_ROCM_API int tnn_rocm_graph_destroy(void *graph_exec);
+
 /* ---- dense contractions --------------------------------------------------------------------
  * GEMM epilogue selectors (combinable): y = act(acc + bias) + residual                       */
 enum {

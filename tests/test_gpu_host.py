@@ -165,3 +165,35 @@ def test_host_error_paths():
     with pytest.raises(host.HostError, match="invalid slice_index"):
         inst.forward()
     inst.close()
+
+
+def test_graph_replay_matches_eager_on_every_replay(monkeypatch):
+    """The whole-forward graph (recorded on the third Forward) must reproduce the eager result on every replay, with
+    new inputs each time and unrelated eager GPU work and synchronisations between the replays."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: graph replay vs eager")
+    cfg = EncoderConfig.bert_base(2)
+    w = make_weights(cfg, seed=13, bias_std=0.02)
+    B, S = 2, 128
+    g = tnnmodel.encoder_graph(cfg, w, B, S)
+    monkeypatch.setenv("TNN_ROCM_GRAPH", "0")
+    eager = host.RocmInstance.from_graph(g, "fp16")
+    monkeypatch.setenv("TNN_ROCM_GRAPH", "1")
+    graph = host.RocmInstance.from_graph(g, "fp16")
+    scratch = torch.zeros(1 << 20, device="cuda")
+    for it in range(7):
+        ids, seg, lens, mask = make_inputs(cfg, B, S, 20, 128, seed=100 + it)
+        outs = []
+        for inst in (eager, graph):
+            inst.set_input("input_ids", ids)
+            inst.set_input("token_type_ids", seg)
+            inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+            inst.forward()
+            outs.append(inst.output("last_hidden"))
+        assert np.array_equal(outs[0], outs[1]), "replay %d differs from eager" % it
+        # unrelated eager work + a device synchronisation between replays
+        scratch.add_(1.0)
+        assert float(scratch.sum().item()) == (it + 1) * (1 << 20)
+        torch.cuda.synchronize()
+    eager.close()
+    graph.close()

@@ -31,6 +31,10 @@ SIGNATURES = {
     "tnn_rocm_stream_create": [C.POINTER(_vp)],
     "tnn_rocm_stream_destroy": [_vp],
     "tnn_rocm_stream_sync": [_vp],
+    "tnn_rocm_graph_begin_capture": [_vp],
+    "tnn_rocm_graph_end_capture": [_vp, C.POINTER(_vp)],
+    "tnn_rocm_graph_launch": [_vp, _vp],
+    "tnn_rocm_graph_destroy": [_vp],
     "tnn_rocm_event_create": [C.POINTER(_vp)],
     "tnn_rocm_event_destroy": [_vp],
     "tnn_rocm_event_record": [_vp, _vp],

@@ -619,10 +619,11 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
     if (cfg == 0) {
         size_t kbytes = (size_t)K * sizeof(typename GemmTraits<DT>::elem);
         bool slab128  = kbytes % 128 == 0;
-        // measured on MI355X (fp16): with fewer than ~2 full-size tiles per CU the launch is dominated by pipeline
-        // fill/drain and 64x64 tiles at 4-5 workgroups per CU win (QKV 25 us vs 26, out-proj 12.8 vs 18, FFN2 34.9
-        // vs 38.3 at M=3072); from ~500 tiles of 128x128 on the larger tile wins (M=8192: 34 us vs 37, 89 vs 125)
-        if (tiles(128, 128) >= 500)
+        // measured on MI355X (fp16): with only a few full-size tiles per CU the launch is dominated by pipeline
+        // fill/drain and 64x64 tiles at 4-5 workgroups per CU win (M=3072: QKV 25 us vs 26, out-proj 12.8 vs 18,
+        // FFN1 38 vs 50, FFN2 34.9 vs 38.3); with ~4 tiles of 128x128 per CU the larger tile wins
+        // (M=8192: N=3072 93 us vs 114, N=4096 138 vs 160, K=4096 89 vs 125)
+        if (tiles(128, 128) >= 1000)
             cfg = slab128 ? 1281281 : 1281280;
         else
             cfg = slab128 ? 64641 : 64640;

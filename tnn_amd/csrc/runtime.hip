@@ -134,6 +134,40 @@ int tnn_rocm_stream_sync(void *stream) {
     return 0;
 }
 
+int tnn_rocm_graph_begin_capture(void *stream) {
+    TR_REQUIRE(stream, TNN_ROCM_EINVAL, "graph capture needs a non-default stream");
+    TR_CHECK_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+    return 0;
+}
+
+int tnn_rocm_graph_end_capture(void *stream, void **graph_exec) {
+    TR_REQUIRE(stream && graph_exec, TNN_ROCM_EINVAL, "graph_end_capture: null argument");
+    *graph_exec     = nullptr;
+    hipGraph_t graph = nullptr;
+    TR_CHECK_HIP(hipStreamEndCapture((hipStream_t)stream, &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e        = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    hipGraphDestroy(graph);
+    if (e != hipSuccess) {
+        set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
+        return (int)e;
+    }
+    *graph_exec = (void *)exec;
+    return 0;
+}
+
+int tnn_rocm_graph_launch(void *graph_exec, void *stream) {
+    TR_REQUIRE(graph_exec, TNN_ROCM_EINVAL, "graph_launch: null graph");
+    TR_CHECK_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+    return 0;
+}
+
+int tnn_rocm_graph_destroy(void *graph_exec) {
+    if (graph_exec)
+        TR_CHECK_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+    return 0;
+}
+
 int tnn_rocm_event_create(void **event) {
     TR_REQUIRE(event, TNN_ROCM_EINVAL, "event_create: null output");
     hipEvent_t e;

@@ -967,6 +967,7 @@ DefaultNetwork::~DefaultNetwork() {
     if (device_)
         for (void *p : allocations_)
             device_->Free(p);
+    tnn_rocm_graph_destroy(graph_exec_);
     for (auto &e : prof_events_) {
         tnn_rocm_event_destroy(e.first);
         tnn_rocm_event_destroy(e.second);
@@ -976,6 +977,8 @@ DefaultNetwork::~DefaultNetwork() {
 
 Status DefaultNetwork::Init(NetworkConfig &net_config, ModelInterpreter *interpreter) {
     config_ = net_config;
+    if (const char *g = getenv("TNN_ROCM_GRAPH"))
+        graph_enabled_ = atoi(g) != 0;
     device_ = GetDevice(net_config.device_type);
     if (!device_)  // instance.cc:60-62
         return Status(TNNERR_DEVICE_NOT_SUPPORT, "device not support");
@@ -1180,21 +1183,57 @@ Status DefaultNetwork::AllocateBlobMemory() {
     return TNN_OK;
 }
 
-Status DefaultNetwork::ForwardAsync() {
-    RETURN_ON_NEQ(context_->OnInstanceForwardBegin(), TNN_OK);
-    void *stream = nullptr;
-    if (profiling_)
-        context_->GetCommandQueue(&stream);
+Status DefaultNetwork::RunLayers(void *prof_stream) {
     for (size_t i = 0; i < layers_.size(); ++i) {
         const bool timed = profiling_ && prof_on_[i];
         if (timed)
-            tnn_rocm_event_record(prof_events_[i].first, stream);
+            tnn_rocm_event_record(prof_events_[i].first, prof_stream);
         Status st = layers_[i]->Forward();
         if (timed)
-            tnn_rocm_event_record(prof_events_[i].second, stream);
+            tnn_rocm_event_record(prof_events_[i].second, prof_stream);
         if (st != TNN_OK)  // default_network.cc:599-605
             return Status((int)st, "Forward error of layer " + layers_[i]->GetLayerName() + ": " + st.description());
     }
+    return TNN_OK;
+}
+
+// The layer loop of default_network.cc:571-631.  On DEVICE_ROCM the sequence of launches of a forward pass is
+// fixed once the instance is initialised (static shapes, stable blob/workspace addresses), so after two eager
+// passes (which also perform every lazy allocation) the third is recorded into an executable graph and later calls
+// replay it with a single submission; per-layer profiling and TNN_ROCM_GRAPH=0 keep the eager loop.
+Status DefaultNetwork::ForwardAsync() {
+    RETURN_ON_NEQ(context_->OnInstanceForwardBegin(), TNN_OK);
+    void *stream = nullptr;
+    context_->GetCommandQueue(&stream);
+    const bool use_graph = graph_enabled_ && !profiling_ && config_.device_type == DEVICE_ROCM && stream != nullptr;
+    if (use_graph && graph_exec_) {
+        if (tnn_rocm_graph_launch(graph_exec_, stream) != 0)
+            return Status(TNNERR_CUDA_KERNEL_LAUNCH_ERROR, std::string("graph launch failed: ") + tnn_rocm_last_error());
+        return context_->OnInstanceForwardEnd();
+    }
+    if (use_graph && eager_forwards_ >= 2) {
+        if (tnn_rocm_graph_begin_capture(stream) == 0) {
+            Status st = RunLayers(nullptr);
+            void *exec = nullptr;
+            int rc     = tnn_rocm_graph_end_capture(stream, &exec);
+            if (st != TNN_OK) {
+                tnn_rocm_graph_destroy(exec);
+                return st;
+            }
+            if (rc == 0 && exec) {
+                graph_exec_ = exec;
+                if (tnn_rocm_graph_launch(graph_exec_, stream) != 0)
+                    return Status(TNNERR_CUDA_KERNEL_LAUNCH_ERROR,
+                                  std::string("graph launch failed: ") + tnn_rocm_last_error());
+                return context_->OnInstanceForwardEnd();
+            }
+            graph_enabled_ = false;  // capture not possible for this graph of layers: stay eager
+        } else {
+            graph_enabled_ = false;
+        }
+    }
+    RETURN_ON_NEQ(RunLayers(stream), TNN_OK);
+    ++eager_forwards_;
     if (profiling_) {
         for (size_t i = 0; i < layers_.size(); ++i) {
             float ms = 0;

@@ -646,6 +646,11 @@ private:
     BlobMap inputs_, outputs_;
     bool profiling_ = false;
     std::vector<char> prof_on_;
+    // whole-forward graph replay (see ForwardAsync)
+    Status RunLayers(void *prof_stream);
+    bool graph_enabled_  = true;
+    void *graph_exec_    = nullptr;
+    int eager_forwards_  = 0;
     std::vector<std::pair<void *, void *>> prof_events_;
     std::vector<LayerProfile> prof_;
 };
