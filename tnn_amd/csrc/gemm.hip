@@ -31,6 +31,7 @@ typedef int i32x16 __attribute__((ext_vector_type(16)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kSlabBytes  = 64;               // bytes of k per row per LDS slab
 constexpr int kLdsStride  = kSlabBytes + 16;  // padded row stride in bytes (bank spread for b128 reads)
@@ -130,6 +131,45 @@ template <int DT> struct FloatEpilogue {
         *reinterpret_cast<typename Vec4<T>::type *>(C + (size_t)m * ldc + n) =
             *reinterpret_cast<const typename Vec4<T>::type *>(packed);
     }
+    // true: this workgroup's columns are better written straight from the accumulator layout (store4)
+    __device__ __forceinline__ bool direct(int) const { return false; }
+    // eight consecutive columns n..n+7 of row m (n % 8 == 0, n + 7 < N, rows 16-byte aligned): whole 16-byte
+    // (half) / 32-byte (fp32) pieces, so that the lanes of one row together write full cache lines
+    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8]) const {
+        float v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            v[t] = acc[t];
+        if (flags & TNN_ROCM_EPI_BIAS) {
+            float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
+            v[0] += b0.x, v[1] += b0.y, v[2] += b0.z, v[3] += b0.w;
+            v[4] += b1.x, v[5] += b1.y, v[6] += b1.z, v[7] += b1.w;
+        }
+        if (flags & TNN_ROCM_EPI_GELU) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                v[t] = (DT == TNN_ROCM_F32) ? gelu_erf(v[t]) : gelu_erf_fast(v[t]);
+        }
+        constexpr int NV = 8 * sizeof(T) / 16;  // 16-byte vectors per eight elements
+        u32x4 packed[NV];
+        T *pe = reinterpret_cast<T *>(packed);
+        if (flags & TNN_ROCM_EPI_RESIDUAL) {
+            const u32x4 *rp = reinterpret_cast<const u32x4 *>(residual + (size_t)m * ldr + n);
+#pragma unroll
+            for (int q = 0; q < NV; ++q)
+                packed[q] = rp[q];
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                v[t] += Elem<DT>::ld(&pe[t]);
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            Elem<DT>::st(&pe[t], v[t]);
+        u32x4 *cp = reinterpret_cast<u32x4 *>(C + (size_t)m * ldc + n);
+#pragma unroll
+        for (int q = 0; q < NV; ++q)
+            cp[q] = packed[q];
+    }
 };
 
 // QKV projection epilogue: columns [0,2H) -> qk[T,2H]; columns [2H,3H) -> V^T[b][head][d][s]
@@ -167,6 +207,37 @@ template <int DT> struct QkvSplitEpilogue {
             T *dst = vt + (((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s;  // lanes = consecutive s
 #pragma unroll
             for (int t = 0; t < 4; ++t)
+                Elem<DT>::st(dst + (size_t)t * S, v[t]);
+        }
+    }
+    // the V^T columns are written with lanes along s (the accumulator layout); Q|K rows go through store8
+    __device__ __forceinline__ bool direct(int n0) const { return n0 >= 2 * H; }
+    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8]) const {
+        float v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            v[t] = acc[t];
+        if (bias) {
+            float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
+            v[0] += b0.x, v[1] += b0.y, v[2] += b0.z, v[3] += b0.w;
+            v[4] += b1.x, v[5] += b1.y, v[6] += b1.z, v[7] += b1.w;
+        }
+        if (n < 2 * H) {
+            constexpr int NV = 8 * sizeof(T) / 16;
+            u32x4 packed[NV];
+            T *pe = reinterpret_cast<T *>(packed);
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                Elem<DT>::st(&pe[t], v[t]);
+            u32x4 *cp = reinterpret_cast<u32x4 *>(qk + (size_t)m * 2 * H + n);
+#pragma unroll
+            for (int q = 0; q < NV; ++q)
+                cp[q] = packed[q];
+        } else {
+            int c = n - 2 * H, b = m / S, s_ = m - b * S;
+            T *dst = vt + (((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s_;
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
                 Elem<DT>::st(dst + (size_t)t * S, v[t]);
         }
     }
@@ -216,6 +287,54 @@ struct Int8Epilogue {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
             store(m, n + t, acc[t], col_const(n + t));
+    }
+    __device__ __forceinline__ bool direct(int) const { return false; }
+    // eight consecutive columns (n % 8 == 0, n + 7 < N, ldo % 8 == 0): same arithmetic as store(), vector accesses
+    __device__ __forceinline__ void store8(int m, int n, const int (&acc)[8]) const {
+        int a[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            a[t] = acc[t];
+        if (bias) {
+            i32x4 b0 = *reinterpret_cast<const i32x4 *>(bias + n), b1 = *reinterpret_cast<const i32x4 *>(bias + n + 4);
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                a[t] += b0[t], a[4 + t] += b1[t];
+        }
+        const size_t o = (size_t)m * ldo + n;
+        if (acc_out) {
+            i32x4 *ap = reinterpret_cast<i32x4 *>(acc_out + o);
+            ap[0] = i32x4{a[0], a[1], a[2], a[3]};
+            ap[1] = i32x4{a[4], a[5], a[6], a[7]};
+        }
+        if (out || out_f) {
+            float sc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            if (scale) {
+                float4 s0 = *reinterpret_cast<const float4 *>(scale + n), s1 = *reinterpret_cast<const float4 *>(scale + n + 4);
+                sc[0] = s0.x, sc[1] = s0.y, sc[2] = s0.z, sc[3] = s0.w, sc[4] = s1.x, sc[5] = s1.y, sc[6] = s1.z, sc[7] = s1.w;
+            }
+            int8_t q[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                q[t] = float2int8_ref(__fmul_rn((float)a[t], sc[t]));
+            if (out)
+                *reinterpret_cast<uint2 *>(out + o) = *reinterpret_cast<const uint2 *>(q);
+            if (out_f) {
+                if (out_f_dtype == TNN_ROCM_F32) {
+                    float4 *fp = reinterpret_cast<float4 *>((float *)out_f + o);
+                    fp[0] = make_float4(__fmul_rn((float)q[0], dq), __fmul_rn((float)q[1], dq), __fmul_rn((float)q[2], dq),
+                                        __fmul_rn((float)q[3], dq));
+                    fp[1] = make_float4(__fmul_rn((float)q[4], dq), __fmul_rn((float)q[5], dq), __fmul_rn((float)q[6], dq),
+                                        __fmul_rn((float)q[7], dq));
+                } else {
+                    half_t h[8];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)
+                        h[t] = (half_t)__fmul_rn((float)q[t], dq);
+                    *reinterpret_cast<u32x4 *>((half_t *)out_f + o) = *reinterpret_cast<const u32x4 *>(h);
+                }
+            }
+        }
     }
 };
 
@@ -468,7 +587,6 @@ __global__ void __launch_bounds__(256)
     const int m0 = (pid / tiles_n) * BM;
     const int n0 = (pid % tiles_n) * BN;
 
-    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
     u32x4 ra0[A_VECS], rb0[B_VECS], ra1[A_VECS], rb1[B_VECS];
 
     // Loads carry no bounds branches: rows past the matrix edge are clamped to the last row (their products
@@ -544,6 +662,8 @@ __global__ void __launch_bounds__(256)
     TR_LOAD_GLOBAL(ra1, rb1, TR_CLAMPK(1));
     TR_STORE_LDS(0, ra0, rb0);
     __syncthreads();
+    // (forcing the look-ahead loads to the top of each phase with sched_barrier was measured slower: the compiler's
+    // own interleaving of loads, LDS traffic and MFMAs is kept)
     for (int kt = 0; kt + 2 <= nk; kt += 2) {
         TR_LOAD_GLOBAL(ra0, rb0, TR_CLAMPK(kt + 2));
         TR_COMPUTE(0);
@@ -561,29 +681,84 @@ __global__ void __launch_bounds__(256)
 #undef TR_COMPUTE
 #undef TR_CLAMPK
 
-    // epilogue: lane owns row m; accumulator group r4 holds columns 8*r4 + 4*(lane/32) + 0..3
+    typedef typename std::remove_reference<decltype(acc[0][0][0])>::type AccT;
+    if (epi.direct(n0)) {
+        // straight from the accumulator layout: lane owns row m; group r4 holds columns 8*r4 + 4*(lane/32) + 0..3
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        const int m = m0 + wm * (BM / 2) + i * 32 + (lane & 31);
-        if (m >= M)
-            continue;
+        for (int i = 0; i < MT; ++i) {
+            const int m = m0 + wm * (BM / 2) + i * 32 + (lane & 31);
+            if (m >= M)
+                continue;
 #pragma unroll
-        for (int j = 0; j < NTL; ++j) {
+            for (int j = 0; j < NTL; ++j) {
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const int n = n0 + wn * (BN / 2) + j * 32 + 8 * r4 + 4 * (lane >> 5);
-                if (n + 3 < N) {
-                    typename std::remove_reference<decltype(acc[i][j][0])>::type v[4] = {
-                        acc[i][j][r4 * 4 + 0], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2], acc[i][j][r4 * 4 + 3]};
-                    epi.store4(m, n, v);
-                } else {
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    const int n = n0 + wn * (BN / 2) + j * 32 + 8 * r4 + 4 * (lane >> 5);
+                    if (n + 3 < N) {
+                        AccT v[4] = {acc[i][j][r4 * 4 + 0], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2],
+                                     acc[i][j][r4 * 4 + 3]};
+                        epi.store4(m, n, v);
+                    } else {
 #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        if (n + t < N)
-                            epi.store(m, n + t, acc[i][j][r4 * 4 + t], epi.col_const(n + t));
+                        for (int t = 0; t < 4; ++t)
+                            if (n + t < N)
+                                epi.store(m, n + t, acc[i][j][r4 * 4 + t], epi.col_const(n + t));
+                    }
                 }
             }
         }
+        return;
+    }
+
+    // Row-contiguous epilogue.  In the accumulator layout one store instruction touches 32 rows with 16 bytes
+    // each, i.e. 32 partial cache lines; the L2 then sees eight times as many write requests as there are lines.
+    // Each wave therefore turns its 32 x CW accumulator block through a private LDS region (the slab buffers are
+    // free after the main loop) and leaves with CW/8 lanes per row, eight columns per lane: a store instruction
+    // covers whole 128-byte (half) lines of C, and bias/residual are read in the same coalesced shape.
+    constexpr int CW   = NTL * 32;  // columns per wave
+    constexpr int SSTR = CW + 4;    // staged row stride in 32-bit words (16-byte pad: spreads the b128 banks)
+    constexpr int LPR  = CW / 8;    // lanes per row on the way out
+    constexpr int RPP  = 64 / LPR;  // rows per pass
+    static_assert(4 * 32 * SSTR * 4 <= 2 * (BM + BN) * STRIDE, "staging must fit the slab buffers");
+    __syncthreads();  // every wave is done reading the slabs
+    AccT *stage = reinterpret_cast<AccT *>(lds_dyn) + wave * (32 * SSTR);
+    typedef AccT acc4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int j = 0; j < NTL; ++j)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4)
+                *reinterpret_cast<acc4 *>(stage + (lane & 31) * SSTR + j * 32 + 8 * r4 + 4 * (lane >> 5)) =
+                    acc4{acc[i][j][r4 * 4 + 0], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2], acc[i][j][r4 * 4 + 3]};
+        // the region is private to this wave: LDS operations of one wave complete in order, the fence only keeps
+        // the compiler from moving the reads above the writes
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int p = 0; p < 32 / RPP; ++p) {
+            const int row = p * RPP + lane / LPR;
+            const int c8  = (lane % LPR) * 8;
+            const acc4 lo = *reinterpret_cast<const acc4 *>(stage + row * SSTR + c8);
+            const acc4 hi = *reinterpret_cast<const acc4 *>(stage + row * SSTR + c8 + 4);
+            const int m   = m0 + wm * (BM / 2) + i * 32 + row;
+            const int n   = n0 + wn * (BN / 2) + c8;
+            if (m < M) {
+                AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                if (n + 7 < N) {
+                    epi.store8(m, n, v);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)
+                        if (n + t < N)
+                            epi.store(m, n + t, v[t], epi.col_const(n + t));
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 }
 
@@ -728,8 +903,8 @@ int tnn_rocm_gemm(void *stream, int dtype, int b_is_nk, const void *A, const voi
         epi.ldc            = ldc;                                                                                     \
         epi.batch_stride_c = sc;                                                                                      \
         epi.batch_stride_r = sr;                                                                                      \
-        bool vec_out = N % 4 == 0 && ldc % 4 == 0 && (((uintptr_t)C) & 15u) == 0 &&                                   \
-                       (!(epilogue & TNN_ROCM_EPI_RESIDUAL) || (ldr % 4 == 0 && (((uintptr_t)residual) & 15u) == 0)) &&\
+        bool vec_out = N % 4 == 0 && ldc % VEC == 0 && (((uintptr_t)C) & 15u) == 0 &&                                 \
+                       (!(epilogue & TNN_ROCM_EPI_RESIDUAL) || (ldr % VEC == 0 && (((uintptr_t)residual) & 15u) == 0)) &&\
                        (!(epilogue & TNN_ROCM_EPI_BIAS) || (((uintptr_t)bias) & 15u) == 0);                            \
         if (b_is_nk && aligned && batch == 1 && vec_out && g_gemm_force_cfg >= 0 && (K * sizeof(T)) % 64 == 0)        \
             return launch_gemm_fast<DT, FloatEpilogue<DT>>(s, A, B, M, N, K, lda, ldb, epi);                          \
@@ -768,7 +943,9 @@ int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W, const int32
     epi.out_f       = out_f;
     epi.out_f_dtype = out_f_dtype;
     epi.dq          = dequant_scale;
-    if (aligned && g_gemm_force_cfg >= 0 && K % 64 == 0)
+    bool vec_out = ldo % 8 == 0 && (!bias || al16(bias)) && (!scale || al16(scale)) &&
+                   (!out_i8 || (((uintptr_t)out_i8) & 7u) == 0) && (!acc_i32 || al16(acc_i32)) && (!out_f || al16(out_f));
+    if (aligned && vec_out && g_gemm_force_cfg >= 0 && K % 64 == 0)
         return launch_gemm_fast<TNN_ROCM_I8, Int8Epilogue>((hipStream_t)stream, A, W, M, N, K, lda, ldw, epi);
     return launch_gemm<TNN_ROCM_I8, Int8Epilogue>((hipStream_t)stream, true, aligned, A, W, M, N, K, lda, ldw, 1, 1, 1,
                                                   0, 0, epi);
