@@ -1,0 +1,51 @@
+/* C entry points of libtnn_rocm_host.so: the engine-side host (Instance on DEVICE_ROCM) behind plain pointers, for
+ * drivers written in other languages.  Each call maps onto one method of the engine's public Instance
+ * (reference include/tnn/core/instance.h:42-135) in the order the engine's own test driver uses them
+ * (reference test/test.cc:101-152: SetInputMat -> Forward -> GetOutputMat).
+ *
+ * All int-returning functions return 0 on success and a non-zero engine status code otherwise; the text of the last
+ * failure of a handle is tnn_host_last_error(handle). */
+#ifndef TNN_ROCM_HOST_H_
+#define TNN_ROCM_HOST_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Instance(net_config{DEVICE_ROCM, device_id, precision}, model_config{proto text, model bytes}) + Init()
+ * (reference include/tnn/core/instance.h:44-49, include/tnn/core/common.h:142-183).
+ * precision: 0 = PRECISION_HIGH (fp32 blobs), 1 = PRECISION_AUTO (fp16 activations).
+ * Returns NULL on failure and writes the status text to err[err_len]. */
+void *tnn_host_create(const char *proto, size_t proto_len, const char *model, size_t model_len, int device_id,
+                      int precision, char *err, size_t err_len);
+/* ~Instance (instance.h:46) */
+void tnn_host_destroy(void *handle);
+const char *tnn_host_last_error(void *handle);
+
+/* Instance::SetInputMat (instance.h:123) from a host array.  mat_type: 0 = NCHW_FLOAT (fp32), 1 = NC_INT32.
+ * name NULL or "" selects the only input. */
+int tnn_host_set_input(void *handle, const char *name, const void *data, int mat_type, const int *dims, int ndims);
+/* Instance::Forward (instance.h:78): runs every layer and waits for the stream */
+int tnn_host_forward(void *handle);
+/* Instance::ForwardAsync (instance.h:92): enqueue only; pair with tnn_host_sync */
+int tnn_host_forward_async(void *handle);
+int tnn_host_sync(void *handle);
+/* Instance::GetCommandQueue (instance.h:71): the hipStream_t the instance launches on */
+void *tnn_host_stream(void *handle);
+/* Instance::GetOutputMat (instance.h:128) converted to fp32 NCHW on the host.  dims must hold 8 ints. */
+int tnn_host_get_output(void *handle, const char *name, float *out, size_t capacity, int *dims, int *ndims);
+
+/* The optimised layer list ("Type name\n" per layer) and per-layer timing with events on the instance's stream
+ * (the engine's TNN_PROFILE facility, reference source/tnn/core/profile.h:29-100).  only_type NULL or "" times every
+ * layer.  tnn_host_profile_finish fills up to `capacity` mean milliseconds (layer order) and returns the layer count. */
+int tnn_host_layer_count(void *handle);
+const char *tnn_host_layer_summary(void *handle);
+void tnn_host_profile_start(void *handle, const char *only_type);
+int tnn_host_profile_finish(void *handle, double *ms, int capacity);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TNN_ROCM_HOST_H_ */
