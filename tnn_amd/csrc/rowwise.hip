@@ -93,8 +93,15 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
             for (int t = 0; t < VEC; ++t) {
                 int c   = vi * VEC + t;
                 float k = gamma[c];
-                float b = beta[c] - mrs * k;
-                o[t]    = v[j][t] * rstd * k + b;
+                if (DT == TNN_ROCM_F32) {
+                    // the reference's operand order and widths (cpu_layer_norm_layer_acc.cc:126-131): the shifted
+                    // bias is formed in double and rounded to float, the affine combination is evaluated in double
+                    float b = (float)((double)beta[c] - mean * rstdd * (double)k);
+                    o[t]    = (float)((double)v[j][t] * rstdd * (double)k + (double)b);
+                } else {
+                    float b = beta[c] - mrs * k;
+                    o[t]    = v[j][t] * rstd * k + b;
+                }
             }
             if (VECTOR) {
                 uint4 raw;
@@ -157,7 +164,13 @@ __global__ void __launch_bounds__(kBlock) layernorm_long_kernel(const typename E
         if (pr)
             f = __fadd_rn(f, Elem<DT>::ld(&pr[c]));
         float k = gamma[c];
-        float o = f * rstd * k + (beta[c] - mrs * k);
+        float o;
+        if (DT == TNN_ROCM_F32) {
+            float b = (float)((double)beta[c] - mean * rstdd * (double)k);
+            o       = (float)((double)f * rstdd * (double)k + (double)b);
+        } else {
+            o = f * rstd * k + (beta[c] - mrs * k);
+        }
         T tmp;
         Elem<DT>::st(&tmp, o);
         py[c] = tmp;
