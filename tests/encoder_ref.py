@@ -50,3 +50,37 @@ def encoder(w, cfg, x, B, S, mask):
     for lw in w["layers"]:
         x = encoder_layer(x, lw, B, S, cfg.heads, mask, cfg.eps)
     return x
+
+
+def int8_encoder(w, cfg, scales, x0, B, S, mask, quantize=None):
+    """The graph of tnn_amd.quant.int8_encoder_graph evaluated with the checker: every projection is
+    quantise(input) -> int8 FC (int32 accumulate, requantise) -> dequantise; everything else in fp32.
+    `quantize` is orc.quantize_x86 (multiply by the reciprocal scale, the x86 Reformat) or orc.quantize_naive (divide).
+    Returns (last hidden [T,H] fp32, {blob name: int8 array} of every int8 blob)."""
+    from tnn_amd import quant
+    quantize = quantize or orc.quantize_x86
+    heads, d = cfg.heads, cfg.head_dim
+    q8 = {}
+
+    def qfc(src_name, src, dst_name, wt, bias):
+        w_q, b_q, w_s = quant.quantize_fc_params(wt, bias, scales[src_name])
+        if src_name not in q8:
+            q8[src_name] = quantize(src, scales[src_name])
+        y, _ = orc.fc_int8(q8[src_name], w_q, b_q, orc.fc_int8_scale(w_s, scales[dst_name], w_q.shape[0]))
+        q8[dst_name] = y
+        return orc.dequantize(y, scales[dst_name])
+
+    x, xn = x0, "x0"
+    for li, lw in enumerate(w["layers"]):
+        p = "l%d_" % li
+        q, k, v = (qfc(xn, x, p + nm + "_o", lw["w" + nm], lw["b" + nm]).reshape(B, S, heads, d) for nm in "qkv")
+        q, k, v = (orc.permute(t, (0, 2, 1, 3)) for t in (q, k, v))
+        ctx = orc.attention_core(q, k, v, np.float32(1.0 / np.sqrt(d)), mask)
+        ctx = orc.permute(ctx, (0, 2, 1, 3)).reshape(B * S, cfg.hidden)
+        a = qfc(p + "ctx", ctx, p + "attn_o", lw["wo"], lw["bo"])
+        x1 = orc.layernorm(orc.binary("add", x, a), lw["ln1_g"], lw["ln1_b"], cfg.eps)
+        h = orc.gelu(qfc(p + "x1", x1, p + "ffn1_o", lw["w1"], lw["b1"]))
+        y = qfc(p + "act", h, p + "ffn2_o", lw["w2"], lw["b2"])
+        x = orc.layernorm(orc.binary("add", x1, y), lw["ln2_g"], lw["ln2_b"], cfg.eps)
+        xn = p + "x2"
+    return x, q8

@@ -139,11 +139,36 @@ def int8_ffn():
                         scales=scales, y_x86=y_x86, y_naive=y_naive)
 
 
+def int8_encoder():
+    """One-layer int8 encoder (hidden 128, 2 heads, FFN 256, B2 S16): calibrated on the fp32 NAIVE forward, run on
+    DEVICE_X86; weights are regenerated from the seed (digest stored), scales and every int8 blob are stored."""
+    from tnn_amd import quant
+    cfg = EncoderConfig(1, 128, 2, 256, vocab=1000, max_pos=64)
+    w = make_weights(cfg, seed=21, bias_std=0.02)
+    B, S = 2, 16
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 5, 16, seed=22)
+    inputs = {"input_ids": ids, "token_type_ids": seg, "attention_bias": mask.reshape(B, 1, 1, S)}
+    names = quant.calibration_outputs(cfg)
+    acts = dict(zip(names, run(tnnmodel.encoder_graph(cfg, w, B, S, extra_outputs=names), inputs, names, "NAIVE")))
+    scales = quant.scales_from_activations(acts)
+    blobs = ["x0"] + ["l0_" + b for b in quant.CALIBRATION_BLOBS]
+    g = quant.int8_encoder_graph(cfg, w, scales, B, S, extra_outputs=blobs)
+    outs = run(g, inputs, ["last_hidden"] + blobs, "X86")
+    out = {"ids": ids, "seg": seg, "mask": mask, "x86_last_hidden": outs[0],
+           "w_digest": np.float64(sum(float(np.abs(v).astype(np.float64).sum()) for v in w["layers"][0].values()))}
+    for n, v in zip(blobs, outs[1:]):
+        out["x86_" + n] = v
+    for n in names:
+        out["scale_" + n] = scales[n]
+    np.savez_compressed(os.path.join(HERE, "int8_encoder_x86.npz"), **out)
+
+
 if __name__ == "__main__":
     assert ref_driver.available(), "oracle/_ref is not built: run `make -C oracle` where the reference tree is present"
     single_ops()
     tiny_encoder()
     config1_summary()
     int8_ffn()
+    int8_encoder()
     for f in sorted(os.listdir(HERE)):
         print("%8d  %s" % (os.path.getsize(os.path.join(HERE, f)), f))

@@ -35,3 +35,47 @@ def config1_inputs():
     assert float(lw["wq"].astype(np.float64).sum()) == float(f["wq_sum"])
     assert float(lw["wo"].astype(np.float64).sum()) == float(f["wo_sum"])
     return lw, x, f
+
+
+def int8_encoder():
+    """-> (cfg, weights, B, S, scales, fixture) of int8_encoder_x86.npz; weights are regenerated from the seed and
+    checked against the stored digest."""
+    from tnn_amd.encoder import EncoderConfig, make_weights
+    f = load("int8_encoder_x86.npz")
+    cfg = EncoderConfig(1, 128, 2, 256, vocab=1000, max_pos=64)
+    w = make_weights(cfg, seed=21, bias_std=0.02)
+    digest = sum(float(np.abs(v).astype(np.float64).sum()) for v in w["layers"][0].values())
+    assert digest == float(f["w_digest"])
+    B, S = f["ids"].shape
+    scales = {k[len("scale_"):]: np.float32(v) for k, v in f.items() if k.startswith("scale_")}
+    return cfg, w, B, S, scales, f
+
+
+def int8_projections(cfg, w, li=0):
+    """(input blob, output blob, weight [N,K], bias) of the six projections of layer li in the int8 encoder graph"""
+    lw, p = w["layers"][li], "l%d_" % li
+    xin = "x0" if li == 0 else "l%d_x2" % (li - 1)
+    return [(xin, p + "q_o", lw["wq"], lw["bq"]), (xin, p + "k_o", lw["wk"], lw["bk"]), (xin, p + "v_o", lw["wv"], lw["bv"]),
+            (p + "ctx", p + "attn_o", lw["wo"], lw["bo"]), (p + "x1", p + "ffn1_o", lw["w1"], lw["b1"]),
+            (p + "act", p + "ffn2_o", lw["w2"], lw["b2"])]
+
+
+def check_projections_bit_exact(cfg, w, scales, blobs, T, quantize, layers=None):
+    """Teacher forcing: every projection, fed with the float blob the run itself produced (quantised as its Reformat
+    layer does), must reproduce the run's own int8 output exactly.  `blobs` maps blob name -> dequantised array."""
+    import orc
+    from tnn_amd import quant
+    n = 0
+    for li in (range(cfg.layers) if layers is None else layers):
+        for src, dst, wt, bias in int8_projections(cfg, w, li):
+            if src not in blobs or dst not in blobs:
+                continue
+            w_q, b_q, w_s = quant.quantize_fc_params(wt, bias, scales[src])
+            src_q = quantize(np.ascontiguousarray(blobs[src], np.float32).reshape(T, -1), scales[src])
+            y, acc = orc.fc_int8(src_q, w_q, b_q, orc.fc_int8_scale(w_s, scales[dst], w_q.shape[0]))
+            got = blobs[dst].reshape(T, -1) / scales[dst]
+            assert np.abs(got - np.rint(got)).max() < 1e-3, dst
+            bad = int((np.rint(got).astype(np.int8) != y).sum())
+            assert bad == 0, "%s: %d of %d int8 outputs differ" % (dst, bad, y.size)
+            n += 1
+    return n

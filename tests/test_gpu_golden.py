@@ -83,3 +83,36 @@ def test_int8_ffn_bit_exact_against_reference_x86():
     # int8 GEMMs and quantisers are bit-exact; the fp32 GELU between them may move a value across a rounding
     # boundary of the second quantiser (device erff vs the CPU's double erf): at most 1 LSB on at most 0.1 %
     assert diff.max() <= 1 and (diff != 0).mean() <= 1e-3
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_int8_encoder_against_reference_x86(precision):
+    """Int8 encoder (QuantizedInnerProduct projections, float attention core / LayerNorm / GELU) on the host:
+    each projection is bit-exact given its own input blob; the network output stays within the float bar of the
+    reference's DEVICE_X86 run."""
+    import orc
+    from tnn_amd import host, quant
+    cfg, w, B, S, scales, f = golden_util.int8_encoder()
+    say("golden: int8 encoder on the host vs reference X86 fixture, " + precision)
+    blobs = ["x0"] + ["l0_" + b for b in quant.CALIBRATION_BLOBS]
+    g = quant.int8_encoder_graph(cfg, w, scales, B, S, extra_outputs=blobs)
+    inst = host.RocmInstance.from_graph(g, precision)
+    types = [t for t, _ in inst.layers()]
+    say("  layers: " + " ".join(sorted(set(types))))
+    assert types.count("QuantizedInnerProduct") == 6
+    inst.set_input("input_ids", f["ids"])
+    inst.set_input("token_type_ids", f["seg"])
+    inst.set_input("attention_bias", f["mask"].reshape(B, 1, 1, S))
+    inst.forward()
+    got = inst.output("last_hidden")
+    mine = {n: inst.output(n) for n in blobs}
+    inst.close()
+    # float blobs that feed a projection are quantised by the Reformat kernel with the reciprocal scale, as on x86;
+    # in fp16 mode those blobs are fp16 values, which the read-back reproduces exactly
+    assert golden_util.check_projections_bit_exact(cfg, w, scales, mine, B * S, orc.quantize_x86) == 6
+    ref = f["x86_last_hidden"].reshape(got.shape)
+    err = rel_err(got, ref)
+    say("  max rel err vs X86 %.3g" % err)
+    # one int8 step of a projection output is ~1/127 of its range, so a float difference upstream that flips a
+    # rounding moves the result by more than the float bar; the bound below is two such steps on the final LayerNorm
+    assert err <= (2e-2 if precision == "fp16" else 1e-2)

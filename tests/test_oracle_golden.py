@@ -61,3 +61,34 @@ def test_int8_ffn_bit_identical_to_reference_x86_and_naive():
     yq, _ = orc.fc_int8(gq, f["w2"], f["b2"], orc.fc_int8_scale(f["ws2"], s_y, K))
     assert np.array_equal(orc.dequantize(yq, s_y), f["y_x86"])
     assert np.array_equal(f["y_naive"], f["y_x86"])
+
+
+def test_fc_quantisation_convention():
+    """tnn_amd.quant against what the convention fixes: per-channel scale max|w*s_in|/127, weights reach +-127
+    exactly on the extreme element, std::round ties, truncated bias, zero rows."""
+    from tnn_amd import quant
+    w = np.array([[0.5, -1.0, 0.25, 0.0], [0.0, 0.0, 0.0, 0.0], [3.0, 1.5, -0.75, 0.0]], np.float32)
+    b = np.array([0.1, 5.0, -0.2], np.float32)
+    wq, bq, ws = quant.quantize_fc_params(w, b, np.float32(2.0))
+    assert np.allclose(ws, [2.0 / 127, 0.0, 6.0 / 127], rtol=1e-7)
+    assert wq[0].tolist() == [64, -127, 32, 0]       # 63.5 -> 64 (half away from zero), 31.75 -> 32
+    assert wq[1].tolist() == [0, 0, 0, 0] and bq[1] == 0
+    assert wq[2].tolist() == [127, 64, -32, 0]       # 63.5 -> 64, -31.75 -> -32
+    assert bq[0] == int(np.float32(0.1) / ws[0]) and bq[2] == int(np.float32(-0.2) / ws[2])  # truncation toward zero
+    rng = np.random.default_rng(5)
+    w = (rng.standard_normal((64, 96)) * 0.02).astype(np.float32)
+    wq, bq, ws = quant.quantize_fc_params(w, np.zeros(64, np.float32), np.float32(0.03))
+    assert np.abs(wq).max(axis=1).tolist() == [127] * 64
+    assert np.abs(wq.astype(np.float32) * ws[:, None] - w * np.float32(0.03)).max() <= ws.max() * 0.5 * (1 + 1e-6)
+
+
+def test_int8_encoder_fixture_projections_bit_exact_and_output_close():
+    """The committed DEVICE_X86 run of the int8 encoder: the checker reproduces each projection's int8 output exactly
+    from the run's own inputs, and the whole network within the fp32 bar."""
+    cfg, w, B, S, scales, f = golden_util.int8_encoder()
+    blobs = {k[4:]: v for k, v in f.items() if k.startswith("x86_") and k != "x86_last_hidden"}
+    assert golden_util.check_projections_bit_exact(cfg, w, scales, blobs, B * S, orc.quantize_x86) == 6
+    x0 = encoder_ref.embed(w, f["ids"], f["seg"], cfg.eps)
+    mine, _ = encoder_ref.int8_encoder(w, cfg, scales, x0, B, S, f["mask"], orc.quantize_x86)
+    ref = f["x86_last_hidden"].reshape(B * S, -1)
+    assert np.abs(mine - ref).max() / np.abs(ref).max() <= 2e-3

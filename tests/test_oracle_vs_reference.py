@@ -174,3 +174,66 @@ def test_float2int8_exhaustive_band_against_definition():
     assert np.array_equal(orc.float2int8(v), expect)
     # ties go away from zero; 0.49999997 + 0.5 rounds up to 1.0 in fp32 and therefore quantises to 1
     assert orc.float2int8(np.array([0.5, -0.5, 2.5, -2.5, 0.49999997], np.float32)).tolist() == [1, -1, 3, -3, 1]
+
+
+def _int8_encoder_case():
+    """Small encoder, calibrated on the reference's own fp32 NAIVE forward, quantised with the calibration tool's
+    convention (tnn_amd.quant)."""
+    from tnn_amd import quant
+    cfg = EncoderConfig(2, 128, 2, 256, vocab=1000, max_pos=64)
+    w = make_weights(cfg, seed=3, bias_std=0.02)
+    B, S = 2, 16
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 5, 16, seed=4)
+    inputs = {"input_ids": ids, "token_type_ids": seg, "attention_bias": mask.reshape(B, 1, 1, S)}
+    names = quant.calibration_outputs(cfg)
+    s = ref_driver.RefSession(tnnmodel.encoder_graph(cfg, w, B, S, extra_outputs=names), "NAIVE", 1)
+    for k, v in inputs.items():
+        s.set_input(k, v)
+    s.forward()
+    acts = {n: s.output(n) for n in names}
+    float_out = s.output("last_hidden")
+    s.close()
+    return cfg, w, B, S, ids, seg, mask, inputs, quant.scales_from_activations(acts), float_out
+
+
+@pytest.mark.parametrize("dev", ["NAIVE", "X86"])
+def test_int8_encoder_against_reference(dev):
+    from tnn_amd import quant
+    cfg, w, B, S, ids, seg, mask, inputs, scales, float_out = _int8_encoder_case()
+    blobs = ["x0"] + ["l%d_%s" % (li, b) for li in range(cfg.layers) for b in quant.CALIBRATION_BLOBS]
+    g = quant.int8_encoder_graph(cfg, w, scales, B, S, extra_outputs=blobs)
+    s = ref_driver.RefSession(g, dev, 1)
+    for k, v in inputs.items():
+        s.set_input(k, v)
+    s.forward()
+    got = s.output("last_hidden").reshape(B * S, -1)
+    ref_blobs = {n: s.output(n) for n in blobs}
+    s.close()
+    assert rel(got, float_out.reshape(B * S, -1)) <= 0.02  # the quantised network still computes the same function
+    x0 = encoder_ref.embed(w, ids, seg, cfg.eps)
+    mine, q8 = encoder_ref.int8_encoder(w, cfg, scales, x0, B, S, mask,
+                                        orc.quantize_naive if dev == "NAIVE" else orc.quantize_x86)
+    if dev == "NAIVE":
+        assert np.array_equal(mine, got)  # same arithmetic end to end: bit-identical
+    else:
+        assert rel(mine, got) <= 2e-3     # x86 float ops (softmax, LayerNorm, GELU) use their own approximations
+    # every projection, fed with the reference's own int8 input, reproduces the reference's int8 output exactly
+    def q_of(name):
+        v = ref_blobs[name] / scales[name]
+        assert np.abs(v - np.rint(v)).max() < 1e-3, name
+        return np.rint(v).astype(np.int8)
+    quantize = orc.quantize_naive if dev == "NAIVE" else orc.quantize_x86
+    checked = 0
+    for li, lw in enumerate(w["layers"]):
+        p = "l%d_" % li
+        xin = "x0" if li == 0 else "l%d_x2" % (li - 1)
+        for src, dst, wt, bias in ((p + "ctx", p + "attn_o", lw["wo"], lw["bo"]), (p + "x1", p + "ffn1_o", lw["w1"], lw["b1"]),
+                                   (p + "act", p + "ffn2_o", lw["w2"], lw["b2"])) + \
+                (((xin, p + "q_o", lw["wq"], lw["bq"]),) if li == 0 else ()):
+            w_q, b_q, w_s = quant.quantize_fc_params(wt, bias, scales[src])
+            src_q = quantize(ref_blobs[src].reshape(B * S, -1), scales[src])  # the float blob the Reformat layer read
+            y, acc = orc.fc_int8(src_q, w_q, b_q, orc.fc_int8_scale(w_s, scales[dst], w_q.shape[0]))
+            assert np.array_equal(acc, src_q.astype(np.int32) @ w_q.astype(np.int32).T + b_q)
+            assert np.array_equal(y, q_of(dst).reshape(y.shape)), (dev, dst)
+            checked += 1
+    assert checked == 3 * cfg.layers + 1

@@ -543,43 +543,59 @@ __global__ void __launch_bounds__(WM *WN * 64)
 }
 
 
-// ---- pipelined variant for the aligned x * W^T case ---------------------------------------------------
-// Same tiling idea as gemm_kernel, tuned for the encoder's projection shapes:
-//   * k-slabs of SLAB bytes per row (128 for the large-K launches), so a barrier is amortised over
-//     SLAB/32 MFMA steps per 32x32 block;
-//   * two slabs in flight in registers in addition to the one being consumed from LDS (global loads for
-//     slab k+2 are issued before the MFMAs of slab k), which covers the L2/HBM latency that a one-slab
-//     look-ahead leaves exposed;
-//   * the MFMA operands are swapped (the W panel is the "A" operand), so a lane ends up owning one output
-//     ROW and four consecutive columns per accumulator group: the epilogue reads bias/residual and writes
-//     C with 8-byte (fp16) / 16-byte (fp32) accesses instead of 2-byte ones.
-// LDS is dynamic: 2 buffers x (BM + BN) rows x (SLAB + 16) bytes.
-template <int DT, int BM, int BN, int SLAB, typename Epi>
+// ---- tiled, pipelined kernel for the aligned x * W^T case ----------------------------------------------
+// One workgroup of four waves (one per SIMD) per output tile.  The waves form a WGM x WGN x WGK grid: a wave
+// owns a (32*TM) x (32*TN) block of the tile and, when WGK > 1, every WGK-th 32-byte k-step of each slab
+// (the partial sums of the WGK waves are added in the epilogue).  Tile = (32*TM*WGM) x (32*TN*WGN).
+//   * the launcher picks the shape so that the tile count is at most (or a multiple of) the CU count with
+//     tiles as large as registers allow: fewer bytes per flop from L2 and LDS, no second partial round;
+//   * k-slabs of SLAB bytes per row; two slabs in flight in registers in addition to the one being consumed
+//     from LDS (global loads for slab k+2 are issued before the MFMAs of slab k);
+//   * the MFMA operands are swapped (the W panel is the "A" operand), so a lane owns one output ROW and
+//     four consecutive columns per accumulator group;
+//   * the epilogue turns the accumulators through LDS into a row-contiguous layout, so C, bias and residual
+//     move as whole cache lines.
+// LDS is dynamic: max(2 buffers x (BM + BN) rows x (SLAB + 16) bytes, 4 x 32 x (32*TN + 4) words of staging).
+template <int TM_, int TN_, int WGM_, int WGN_, int WGK_, int SLAB_> struct TileCfg {
+    static constexpr int TM = TM_, TN = TN_, WGM = WGM_, WGN = WGN_, WGK = WGK_, SLAB = SLAB_;
+    static constexpr int BM = 32 * TM * WGM, BN = 32 * TN * WGN;
+    static constexpr int STRIDE = SLAB + 16;
+    static constexpr int SSTR   = 32 * TN + 4;  // staged row stride in 32-bit words
+    static constexpr size_t slab_bytes  = (size_t)2 * (BM + BN) * STRIDE;
+    static constexpr size_t stage_bytes = (size_t)4 * 32 * SSTR * 4;
+    static constexpr size_t lds_bytes   = slab_bytes > stage_bytes ? slab_bytes : stage_bytes;
+    static_assert(WGM * WGN * WGK == 4, "four waves per workgroup");
+    static_assert((SLAB / 32) % WGK == 0, "k-steps of a slab must split evenly over the k-waves");
+    static_assert((BM * (SLAB / 16)) % 256 == 0 && (BN * (SLAB / 16)) % 256 == 0, "slab must divide over the workgroup");
+};
+
+template <int DT, typename CFG, typename Epi>
 __global__ void __launch_bounds__(256)
-    gemm_nk_pipelined_kernel(const typename GemmTraits<DT>::elem *__restrict__ A,
-                             const typename GemmTraits<DT>::elem *__restrict__ B, int M, int N, int K, long lda,
-                             long ldb, int tiles_m, int tiles_n, Epi epi) {
+    gemm_nk_tiled_kernel(const typename GemmTraits<DT>::elem *__restrict__ A,
+                         const typename GemmTraits<DT>::elem *__restrict__ B, int M, int N, int K, long lda, long ldb,
+                         int tiles_m, int tiles_n, Epi epi) {
     typedef typename GemmTraits<DT>::elem T;
     typedef typename GemmTraits<DT>::acc Acc;
+    constexpr int TM = CFG::TM, TN = CFG::TN, WGN = CFG::WGN, WGK = CFG::WGK, SLAB = CFG::SLAB;
+    constexpr int BM = CFG::BM, BN = CFG::BN, STRIDE = CFG::STRIDE;
     constexpr int NT     = 256;
     constexpr int VEC    = 16 / sizeof(T);
     constexpr int KB     = SLAB / sizeof(T);
     constexpr int VPR    = SLAB / 16;  // 16-byte vectors per slab row
-    constexpr int STRIDE = SLAB + 16;
-    constexpr int MT     = BM / 64;
-    constexpr int NTL    = BN / 64;
     constexpr int A_VECS = BM * VPR / NT;
     constexpr int B_VECS = BN * VPR / NT;
-    static_assert(BM % 64 == 0 && BN % 64 == 0 && (BM * VPR) % NT == 0 && (BN * VPR) % NT == 0, "tile shape");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_dyn[];
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm   = wave >> 1;
-    const int wn   = wave & 1;
+    const int wk   = wave % WGK;
+    const int wn   = (wave / WGK) % WGN;
+    const int wm   = wave / (WGK * WGN);
 
+    // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so give each XCD a contiguous run of
+    // tiles (shared A row panels stay in one L2)
     int pid           = blockIdx.x;
     const int n_tiles = tiles_m * tiles_n;
     if ((n_tiles & 7) == 0)
@@ -627,13 +643,13 @@ __global__ void __launch_bounds__(256)
     }
 #define TR_COMPUTE(BUF)                                                                                               \
     {                                                                                                                 \
-        _Pragma("unroll") for (int kk = 0; kk < SLAB / 32; ++kk) {                                                    \
-            uint4 fa[MT], fb[NTL];                                                                                    \
-            _Pragma("unroll") for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const uint4 *>(                  \
-                lds_a##BUF + (wm * (BM / 2) + i * 32 + frag_row) * STRIDE + kk * 32 + frag_off);                      \
-            _Pragma("unroll") for (int j = 0; j < NTL; ++j) fb[j] = *reinterpret_cast<const uint4 *>(                 \
-                lds_b##BUF + (wn * (BN / 2) + j * 32 + frag_row) * STRIDE + kk * 32 + frag_off);                      \
-            _Pragma("unroll") for (int i = 0; i < MT; ++i) _Pragma("unroll") for (int j = 0; j < NTL; ++j)            \
+        _Pragma("unroll") for (int kk = wk; kk < SLAB / 32; kk += WGK) {                                              \
+            uint4 fa[TM], fb[TN];                                                                                     \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const uint4 *>(                  \
+                lds_a##BUF + ((wm * TM + i) * 32 + frag_row) * STRIDE + kk * 32 + frag_off);                          \
+            _Pragma("unroll") for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const uint4 *>(                  \
+                lds_b##BUF + ((wn * TN + j) * 32 + frag_row) * STRIDE + kk * 32 + frag_off);                          \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i) _Pragma("unroll") for (int j = 0; j < TN; ++j)             \
                 GemmTraits<DT>::mma(fb[j], fa[i], acc[i][j]); /* rows of D = n, lanes of D = m */                     \
         }                                                                                                             \
     }
@@ -641,11 +657,11 @@ __global__ void __launch_bounds__(256)
     unsigned char *const lds_a0 = lds_dyn, *const lds_b0 = lds_dyn + BM * STRIDE;
     unsigned char *const lds_a1 = lds_dyn + (BM + BN) * STRIDE, *const lds_b1 = lds_a1 + BM * STRIDE;
 
-    Acc acc[MT][NTL];
+    Acc acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < NTL; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 acc[i][j][r] = 0;
@@ -655,6 +671,8 @@ __global__ void __launch_bounds__(256)
 
     // Slab schedule (two slabs in flight in registers, one in LDS being consumed).  The loop body is branch
     // free: look-ahead loads past the last slab are clamped to it and their LDS copy is never consumed.
+    // (Forcing the look-ahead loads to the top of each phase with sched_barrier was measured slower: the
+    // compiler's own interleaving of loads, LDS traffic and MFMAs is kept.)
     const int nk   = K / KB;
     const int last = (nk - 1) * KB;
 #define TR_CLAMPK(SLABIDX) (((SLABIDX)*KB) < last ? ((SLABIDX)*KB) : last)
@@ -662,8 +680,6 @@ __global__ void __launch_bounds__(256)
     TR_LOAD_GLOBAL(ra1, rb1, TR_CLAMPK(1));
     TR_STORE_LDS(0, ra0, rb0);
     __syncthreads();
-    // (forcing the look-ahead loads to the top of each phase with sched_barrier was measured slower: the compiler's
-    // own interleaving of loads, LDS traffic and MFMAs is kept)
     for (int kt = 0; kt + 2 <= nk; kt += 2) {
         TR_LOAD_GLOBAL(ra0, rb0, TR_CLAMPK(kt + 2));
         TR_COMPUTE(0);
@@ -682,18 +698,18 @@ __global__ void __launch_bounds__(256)
 #undef TR_CLAMPK
 
     typedef typename std::remove_reference<decltype(acc[0][0][0])>::type AccT;
-    if (epi.direct(n0)) {
+    if (WGK == 1 && epi.direct(n0)) {
         // straight from the accumulator layout: lane owns row m; group r4 holds columns 8*r4 + 4*(lane/32) + 0..3
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const int m = m0 + wm * (BM / 2) + i * 32 + (lane & 31);
+        for (int i = 0; i < TM; ++i) {
+            const int m = m0 + (wm * TM + i) * 32 + (lane & 31);
             if (m >= M)
                 continue;
 #pragma unroll
-            for (int j = 0; j < NTL; ++j) {
+            for (int j = 0; j < TN; ++j) {
 #pragma unroll
                 for (int r4 = 0; r4 < 4; ++r4) {
-                    const int n = n0 + wn * (BN / 2) + j * 32 + 8 * r4 + 4 * (lane >> 5);
+                    const int n = n0 + (wn * TN + j) * 32 + 8 * r4 + 4 * (lane >> 5);
                     if (n + 3 < N) {
                         AccT v[4] = {acc[i][j][r4 * 4 + 0], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2],
                                      acc[i][j][r4 * 4 + 3]};
@@ -712,38 +728,46 @@ __global__ void __launch_bounds__(256)
 
     // Row-contiguous epilogue.  In the accumulator layout one store instruction touches 32 rows with 16 bytes
     // each, i.e. 32 partial cache lines; the L2 then sees eight times as many write requests as there are lines.
-    // Each wave therefore turns its 32 x CW accumulator block through a private LDS region (the slab buffers are
-    // free after the main loop) and leaves with CW/8 lanes per row, eight columns per lane: a store instruction
-    // covers whole 128-byte (half) lines of C, and bias/residual are read in the same coalesced shape.
-    constexpr int CW   = NTL * 32;  // columns per wave
-    constexpr int SSTR = CW + 4;    // staged row stride in 32-bit words (16-byte pad: spreads the b128 banks)
-    constexpr int LPR  = CW / 8;    // lanes per row on the way out
-    constexpr int RPP  = 64 / LPR;  // rows per pass
-    static_assert(4 * 32 * SSTR * 4 <= 2 * (BM + BN) * STRIDE, "staging must fit the slab buffers");
-    __syncthreads();  // every wave is done reading the slabs
-    AccT *stage = reinterpret_cast<AccT *>(lds_dyn) + wave * (32 * SSTR);
+    // For each 32-row group every wave writes its 32 x CW accumulator block to its own LDS region (the slab
+    // buffers are free after the main loop); the workgroup then walks the staged rows with eight columns per
+    // thread, adds the WGK partial sums and applies the epilogue, so a store instruction covers whole lines of C
+    // and bias/residual are read in the same coalesced shape.
+    constexpr int CW   = TN * 32;       // columns per wave
+    constexpr int SSTR = CFG::SSTR;     // staged row stride in 32-bit words (16-byte pad spreads the b128 banks)
+    constexpr int CPR  = CW / 8;        // 8-column pieces per staged row
+    constexpr int POS  = 4 / WGK;       // wave positions (wm, wn) in the tile
+    constexpr int ITEMS = POS * 32 * CPR;
     typedef AccT acc4 __attribute__((ext_vector_type(4)));
+    AccT *const stage_all = reinterpret_cast<AccT *>(lds_dyn);
+    AccT *const stage_me  = stage_all + wave * (32 * SSTR);  // wave = (wm*WGN + wn)*WGK + wk
+    __syncthreads();  // every wave is done reading the slabs
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int j = 0; j < NTL; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4)
-                *reinterpret_cast<acc4 *>(stage + (lane & 31) * SSTR + j * 32 + 8 * r4 + 4 * (lane >> 5)) =
+                *reinterpret_cast<acc4 *>(stage_me + (lane & 31) * SSTR + j * 32 + 8 * r4 + 4 * (lane >> 5)) =
                     acc4{acc[i][j][r4 * 4 + 0], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2], acc[i][j][r4 * 4 + 3]};
-        // the region is private to this wave: LDS operations of one wave complete in order, the fence only keeps
-        // the compiler from moving the reads above the writes
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __syncthreads();
 #pragma unroll
-        for (int p = 0; p < 32 / RPP; ++p) {
-            const int row = p * RPP + lane / LPR;
-            const int c8  = (lane % LPR) * 8;
-            const acc4 lo = *reinterpret_cast<const acc4 *>(stage + row * SSTR + c8);
-            const acc4 hi = *reinterpret_cast<const acc4 *>(stage + row * SSTR + c8 + 4);
-            const int m   = m0 + wm * (BM / 2) + i * 32 + row;
-            const int n   = n0 + wn * (BN / 2) + c8;
+        for (int it = 0; it < (ITEMS + NT - 1) / NT; ++it) {
+            const int item = it * NT + tid;
+            if (ITEMS % NT != 0 && item >= ITEMS)
+                break;
+            const int c8  = (item % CPR) * 8;
+            const int row = (item / CPR) % 32;
+            const int pos = item / (CPR * 32);  // = pm * WGN + pn
+            const AccT *src = stage_all + (pos * WGK) * (32 * SSTR) + row * SSTR + c8;
+            acc4 lo = *reinterpret_cast<const acc4 *>(src);
+            acc4 hi = *reinterpret_cast<const acc4 *>(src + 4);
+#pragma unroll
+            for (int q = 1; q < WGK; ++q) {
+                lo += *reinterpret_cast<const acc4 *>(src + q * (32 * SSTR));
+                hi += *reinterpret_cast<const acc4 *>(src + q * (32 * SSTR) + 4);
+            }
+            const int m = m0 + ((pos / WGN) * TM + i) * 32 + row;
+            const int n = n0 + (pos % WGN) * CW + c8;
             if (m < M) {
                 AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 if (n + 7 < N) {
@@ -756,22 +780,20 @@ __global__ void __launch_bounds__(256)
                 }
             }
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (i + 1 < TM)
+            __syncthreads();
     }
 }
 
-// tuning override for experiments: 0 = heuristic, otherwise (BM, BN, SLAB) of the pipelined kernel
+// tuning override for experiments: 0 = heuristic, otherwise a configuration code of the tiled kernel
 int g_gemm_force_cfg = 0;
 
-template <int DT, int BM, int BN, int SLAB, typename Epi>
-int launch_pipelined(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb,
-                     const Epi &epi) {
+template <int DT, typename CFG, typename Epi>
+int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb, const Epi &epi) {
     typedef typename GemmTraits<DT>::elem T;
-    int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    size_t lds  = (size_t)2 * (BM + BN) * (SLAB + 16);
-    auto kern   = gemm_nk_pipelined_kernel<DT, BM, BN, SLAB, Epi>;
+    int tiles_m = (M + CFG::BM - 1) / CFG::BM, tiles_n = (N + CFG::BN - 1) / CFG::BN;
+    size_t lds  = CFG::lds_bytes;
+    auto kern   = gemm_nk_tiled_kernel<DT, CFG, Epi>;
     if (lds > 64 * 1024) {
         static bool attr_set = false;  // per instantiation
         if (!attr_set) {
@@ -785,40 +807,73 @@ int launch_pipelined(hipStream_t s, const void *A, const void *B, int M, int N, 
     return 0;
 }
 
-// Shape heuristic for the pipelined kernel (measured on MI355X at the encoder's projection shapes).
+// Configuration codes: TM TN WGM WGN WGK S (one decimal digit each; S = 1 for 128-byte slabs, 0 for 64-byte).
+//   112210 / 112211   64 x  64      222210 / 222211  128 x 128      331141   96 x 96, four k-waves
+// Larger tiles with one wave per SIMD (128x256, 256x128, 192x192) and two-k-wave shapes were measured and never
+// won with compiler-scheduled code: they need more latency hiding than a single wave per SIMD provides.
+constexpr int kNumCU = 256;
+
+// Shape heuristic, from measurements on MI355X (fp16; M in {1024, 3072, 4096, 16384}, N and K in
+// {768, 1024, 2304, 3072, 4096}):
+//   * more than one round of 128x128 tiles at two workgroups per CU: 128x128; with short K the 64-byte slab
+//     version wins (fewer registers and less LDS: three to four workgroups per CU hide latency better), e.g.
+//     M=4096 N=3072 K=1024: 43 us vs 52; M=16384 N=3072 K=768: 135 vs 140; long K prefers 128-byte slabs
+//     (M=16384 N=768 K=3072: 106 vs 115) -- unless the second round would be nearly empty (M=3072 N=3072:
+//     576 tiles for 512 slots, 64x64 tiles 32.5 us vs 34);
+//   * between one and two workgroups of 128x128 per CU: 128x128 (M=3072 N=2304: 22.3 us vs 23.3 for 64x64);
+//   * fewer: 64x64 tiles keep every CU busy (M=3072 N=768 K=768: 12.0 us vs 13.9), except for a long K with
+//     about one 96x96 tile per CU, where four k-waves on one 96x96 tile re-read the least
+//     (M=3072 N=768 K=3072: 29.5 us vs 33.9), or at least half a 128x128 tile per CU
+//     (M=4096 N=1024 K=4096: 54 us vs 66).
+inline int pick_tile_config(long M, long N, size_t kbytes, bool allow_ksplit) {
+    auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    const bool s128 = kbytes % 128 == 0;
+    const long t128 = tiles(128, 128), slots = 2 * kNumCU;
+    if (t128 > slots) {
+        if (t128 < 2 * slots && (t128 % slots) * 4 < slots)
+            return s128 ? 112211 : 112210;
+        return (s128 && kbytes >= 4096) ? 222211 : 222210;
+    }
+    if (t128 > kNumCU)
+        return 222210;
+    if (s128 && kbytes >= 4096) {
+        const long t96 = tiles(96, 96);
+        if (allow_ksplit && t96 <= kNumCU && t96 > kNumCU / 2)
+            return 331141;
+        if (t128 > kNumCU / 2)
+            return 222211;
+    }
+    return s128 ? 112211 : 112210;
+}
+
 template <int DT, typename Epi>
 int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb,
-                     const Epi &epi) {
-    auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    int cfg = g_gemm_force_cfg > 0 ? g_gemm_force_cfg : 0;
-    if (cfg == 0) {
-        size_t kbytes = (size_t)K * sizeof(typename GemmTraits<DT>::elem);
-        bool slab128  = kbytes % 128 == 0;
-        // measured on MI355X (fp16): with only a few full-size tiles per CU the launch is dominated by pipeline
-        // fill/drain and 64x64 tiles at 4-5 workgroups per CU win (M=3072: QKV 25 us vs 26, out-proj 12.8 vs 18,
-        // FFN1 38 vs 50, FFN2 34.9 vs 38.3); with ~4 tiles of 128x128 per CU the larger tile wins
-        // (M=8192: N=3072 93 us vs 114, N=4096 138 vs 160, K=4096 89 vs 125)
-        if (tiles(128, 128) >= 1000)
-            cfg = slab128 ? 1281281 : 1281280;
-        else
-            cfg = slab128 ? 64641 : 64640;
-    }
-    if (((size_t)K * sizeof(typename GemmTraits<DT>::elem)) % ((cfg % 10) ? 128 : 64) != 0) {
+                     const Epi &epi, bool allow_ksplit = true) {
+    typedef typename GemmTraits<DT>::elem T;
+    int cfg       = g_gemm_force_cfg > 0 ? g_gemm_force_cfg : 0;
+    size_t kbytes = (size_t)K * sizeof(T);
+    if (cfg == 0)
+        cfg = pick_tile_config(M, N, kbytes, allow_ksplit && DT != TNN_ROCM_F32);
+    if (kbytes % ((cfg % 10) ? 128 : 64) != 0) {
         set_error("gemm: K=%d is not a whole number of slabs for tuning configuration %d", K, cfg);
         return TNN_ROCM_ESHAPE;
     }
-#define TR_FAST(BMv, BNv, SLABv) return launch_pipelined<DT, BMv, BNv, SLABv, Epi>(s, A, B, M, N, K, lda, ldb, epi)
+#define TR_FAST(TMv, TNv, WGMv, WGNv, WGKv, SLABv)                                                                    \
+    return launch_tiled<DT, TileCfg<TMv, TNv, WGMv, WGNv, WGKv, SLABv>, Epi>(s, A, B, M, N, K, lda, ldb, epi)
     switch (cfg) {
-        case 1281281: TR_FAST(128, 128, 128);
-        case 1281280: TR_FAST(128, 128, 64);
-        case 128641: TR_FAST(128, 64, 128);
-        case 128640: TR_FAST(128, 64, 64);
-        case 641281: TR_FAST(64, 128, 128);
-        case 64641: TR_FAST(64, 64, 128);
-        case 64640: TR_FAST(64, 64, 64);
-        default: set_error("gemm: unknown tuning configuration %d", cfg); return TNN_ROCM_EINVAL;
+        case 112210: TR_FAST(1, 1, 2, 2, 1, 64);
+        case 112211: TR_FAST(1, 1, 2, 2, 1, 128);
+        case 222210: TR_FAST(2, 2, 2, 2, 1, 64);
+        case 222211: TR_FAST(2, 2, 2, 2, 1, 128);
+        default: break;
+    }
+    if constexpr (DT != TNN_ROCM_F32) {
+        if (cfg == 331141)
+            TR_FAST(3, 3, 1, 1, 4, 128);
     }
 #undef TR_FAST
+    set_error("gemm: unknown tuning configuration %d", cfg);
+    return TNN_ROCM_EINVAL;
 }
 
 template <int DT, int BM, int BN, int WM, int WN, typename Epi>
@@ -973,7 +1028,8 @@ int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *
         epi.H     = H;                                                                                                \
         epi.S     = S;                                                                                                \
         epi.heads = heads;                                                                                            \
-        return launch_gemm_fast<DT, QkvSplitEpilogue<DT>>((hipStream_t)stream, x, wqkv, T, 3 * H, K, K, K, epi);      \
+        return launch_gemm_fast<DT, QkvSplitEpilogue<DT>>((hipStream_t)stream, x, wqkv, T, 3 * H, K, K, K, epi,    \
+                                                               /*allow_ksplit=*/false);      \
     }
     if (dtype == TNN_ROCM_F16)
         TR_QKV(TNN_ROCM_F16)
@@ -983,7 +1039,7 @@ int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *
 }
 
 // Experiment hook (not part of the documented ABI): 0 restores the shape heuristic, -1 forces the baseline
-// kernel, other values select a (BM, BN, SLAB) instantiation of the pipelined kernel.
+// kernel, other values select a configuration code of the tiled kernel.
 __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_config(int cfg) {
     g_gemm_force_cfg = cfg;
     return 0;
