@@ -33,6 +33,9 @@ def parse():
     ap.add_argument("--layers", type=int, default=12)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seqs", type=int, default=2, help="sequences in the bounded CPU-baseline sample")
+    ap.add_argument("--counter-reference", action="store_true",
+                    help="also launch one element-wise kernel of known size (64 MiB read, 64 MiB written) so that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command carries its own scale factor")
     return ap.parse_args()
 
 
@@ -149,6 +152,12 @@ def main():
     attn_ms = e0.elapsed_time(e1) / 50
     attn_eff_flops = 4.0 * H * S * float(lens.sum())
     attn_pad_flops = 4.0 * B * S * S * H
+
+    if args.counter_reference:
+        big = torch.randn(16 * 1024 * 1024, device="cuda", dtype=torch.float32)
+        torch.cuda.synchronize()
+        ops.gelu(big)  # unary_kernel: reads 64 MiB, writes 64 MiB
+        torch.cuda.synchronize()
 
     full_cfg = (B, S, args.layers) == (8, 384, 12)
     out = {

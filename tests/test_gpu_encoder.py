@@ -87,4 +87,6 @@ def test_encoder_layer_linearity_of_scale_full_size():
     assert np.isfinite(full).all()
     assert np.abs(full.mean(-1)).max() < 5e-3 and np.abs(full.var(-1) - 1).max() < 2e-2
     part = host(enc.forward(dev(ids[3:5]), dev(seg[3:5]), mask=dev(mask[3:5]))).reshape(2, S, -1)
-    assert np.array_equal(part, full[3:5])  # batch rows are independent: bit-identical
+    # batch rows are independent.  The two launches differ in M, so the GEMM picks other tile shapes, some of which
+    # split K over waves and add the fp32 partial sums in another order: equal up to a few fp16 roundings
+    assert rel_err(part, full[3:5]) <= 4e-3

@@ -57,7 +57,7 @@ struct AttnParams {
     uint16_t *o;
     long q_sb, q_sh, q_ss, kv_sb, kv_sh, kv_ss, o_sb, o_sh, o_ss;
     long vt_sb, vt_sh, vt_sd;  // V^T layout (VT kernels): element (b, head, d, s) at v[b*vt_sb + head*vt_sh + d*vt_sd + s]
-    int S;
+    int S, B, heads;
     float scale_log2e;  // scale * log2(e)
     const float *mask;  // [B,S] additive or null
     const int32_t *kv_len;
@@ -84,10 +84,20 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
     const int wave = tid >> 6;
     const int g    = lane >> 5;  // lane half
     const int lq   = lane & 31;  // query column owned by this lane
-    const int b    = blockIdx.z;
-    const int head = blockIdx.y;
-    const int q0   = blockIdx.x * BQ + wave * 32;
     const int S    = p.S;
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Every XCD takes a contiguous run of
+    // (batch, head) pairs and all query tiles of a pair, so the K and V of a head are fetched into one L2 only
+    // (with the plain 3-D grid the query tiles of one head land on different XCDs and each re-reads K and V).
+    const int n_q   = (S + BQ - 1) / BQ;
+    const int total = n_q * p.heads * p.B;
+    const int per   = (total + 7) >> 3;
+    const int vid   = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
+    if (vid >= total)
+        return;  // the grid is padded to a multiple of 8; whole workgroups leave before any barrier
+    const int bh   = vid / n_q;
+    const int b    = bh / p.heads;
+    const int head = bh - b * p.heads;
+    const int q0   = (vid - bh * n_q) * BQ + wave * 32;
 
     int kv_end = S;
     if (p.kv_len) {
@@ -302,14 +312,15 @@ __global__ void mask_to_kv_len_kernel(const float *__restrict__ mask, int32_t *_
 // 128-row query blocks when that already gives >= 2 workgroups per CU, else 64-row blocks
 template <bool VT> int launch_attention(hipStream_t s, int dtype, const AttnParams &p, int B, int heads, int S) {
     long blocks128 = (long)((S + 127) / 128) * heads * B;
+    auto padded = [&](long n_q) { return dim3((unsigned)(((n_q * heads * B + 7) / 8) * 8)); };
     if (blocks128 >= 512) {
-        dim3 grid((S + 127) / 128, heads, B);
+        dim3 grid = padded((S + 127) / 128);
         if (dtype == TNN_ROCM_F16)
             hipLaunchKernelGGL((attention_kernel<TNN_ROCM_F16, 4, VT>), grid, dim3(256), 0, s, p);
         else
             hipLaunchKernelGGL((attention_kernel<TNN_ROCM_BF16, 4, VT>), grid, dim3(256), 0, s, p);
     } else {
-        dim3 grid((S + 63) / 64, heads, B);
+        dim3 grid = padded((S + 63) / 64);
         if (dtype == TNN_ROCM_F16)
             hipLaunchKernelGGL((attention_kernel<TNN_ROCM_F16, 2, VT>), grid, dim3(128), 0, s, p);
         else
@@ -351,6 +362,8 @@ int tnn_rocm_attention(void *stream, int dtype, const void *q, const void *k, co
     p.kv_sb = kv_sb, p.kv_sh = kv_sh, p.kv_ss = kv_ss;
     p.o_sb = o_sb, p.o_sh = o_sh, p.o_ss = o_ss;
     p.S           = S;
+    p.B           = B;
+    p.heads       = heads;
     p.scale_log2e = scale * kLog2e;
     p.mask        = mask;
     p.kv_len      = kv_len;
@@ -388,6 +401,8 @@ int tnn_rocm_attention_vt(void *stream, int dtype, const void *q, const void *k,
     p.vt_sb = vt_sb, p.vt_sh = vt_sh, p.vt_sd = vt_sd;
     p.o_sb = o_sb, p.o_sh = o_sh, p.o_ss = o_ss;
     p.S           = S;
+    p.B           = B;
+    p.heads       = heads;
     p.scale_log2e = scale * kLog2e;
     p.mask        = mask;
     p.kv_len      = kv_len;

@@ -72,11 +72,6 @@ template <> struct GemmTraits<TNN_ROCM_F32> {
     }
 };
 
-// 4-element vector of T as one memory transaction
-template <typename T> struct Vec4;
-template <> struct Vec4<float> { typedef float4 type; };
-template <> struct Vec4<half_t> { typedef uint2 type; };
-template <> struct Vec4<bf16_bits> { typedef uint2 type; };
 
 // ---- epilogues ----------------------------------------------------------------------------------
 template <int DT> struct FloatEpilogue {
@@ -105,33 +100,7 @@ template <int DT> struct FloatEpilogue {
             v = v + Elem<DT>::ld(&residual[(size_t)m * ldr + n]);
         Elem<DT>::st(&C[(size_t)m * ldc + n], v);
     }
-    // four consecutive columns n..n+3 of row m (n % 4 == 0, n + 3 < N, rows 4-element aligned)
-    __device__ __forceinline__ void store4(int m, int n, const float (&acc)[4]) const {
-        float v[4] = {acc[0], acc[1], acc[2], acc[3]};
-        if (flags & TNN_ROCM_EPI_BIAS) {
-            float4 b = *reinterpret_cast<const float4 *>(bias + n);
-            v[0] += b.x, v[1] += b.y, v[2] += b.z, v[3] += b.w;
-        }
-        if (flags & TNN_ROCM_EPI_GELU) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-                v[t] = (DT == TNN_ROCM_F32) ? gelu_erf(v[t]) : gelu_erf_fast(v[t]);
-        }
-        T packed[4];
-        if (flags & TNN_ROCM_EPI_RESIDUAL) {
-            *reinterpret_cast<typename Vec4<T>::type *>(packed) =
-                *reinterpret_cast<const typename Vec4<T>::type *>(residual + (size_t)m * ldr + n);
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-                v[t] += Elem<DT>::ld(&packed[t]);
-        }
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            Elem<DT>::st(&packed[t], v[t]);
-        *reinterpret_cast<typename Vec4<T>::type *>(C + (size_t)m * ldc + n) =
-            *reinterpret_cast<const typename Vec4<T>::type *>(packed);
-    }
-    // true: this workgroup's columns are better written straight from the accumulator layout (store4)
+    // true: this workgroup's columns go to a transposed layout, so the epilogue hands out rows to consecutive lanes
     __device__ __forceinline__ bool direct(int) const { return false; }
     // eight consecutive columns n..n+7 of row m (n % 8 == 0, n + 7 < N, rows 16-byte aligned): whole 16-byte
     // (half) / 32-byte (fp32) pieces, so that the lanes of one row together write full cache lines
@@ -190,27 +159,7 @@ template <int DT> struct QkvSplitEpilogue {
             Elem<DT>::st(&vt[(((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s], v);
         }
     }
-    __device__ __forceinline__ void store4(int m, int n, const float (&acc)[4]) const {
-        float v[4] = {acc[0], acc[1], acc[2], acc[3]};
-        if (bias) {
-            float4 b4 = *reinterpret_cast<const float4 *>(bias + n);
-            v[0] += b4.x, v[1] += b4.y, v[2] += b4.z, v[3] += b4.w;
-        }
-        if (n < 2 * H) {  // H is a multiple of 64, so a group of four never straddles the boundary
-            T packed[4];
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-                Elem<DT>::st(&packed[t], v[t]);
-            *reinterpret_cast<uint2 *>(qk + (size_t)m * 2 * H + n) = *reinterpret_cast<const uint2 *>(packed);
-        } else {
-            int c = n - 2 * H, b = m / S, s = m - b * S;
-            T *dst = vt + (((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s;  // lanes = consecutive s
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-                Elem<DT>::st(dst + (size_t)t * S, v[t]);
-        }
-    }
-    // the V^T columns are written with lanes along s (the accumulator layout); Q|K rows go through store8
+    // the V^T columns are written with consecutive lanes along s; Q|K rows with consecutive lanes along the row
     __device__ __forceinline__ bool direct(int n0) const { return n0 >= 2 * H; }
     __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8]) const {
         float v[8];
@@ -282,11 +231,6 @@ struct Int8Epilogue {
                     ((half_t *)out_f)[(size_t)m * ldo + n] = (half_t)d;
             }
         }
-    }
-    __device__ __forceinline__ void store4(int m, int n, const int (&acc)[4]) const {
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            store(m, n + t, acc[t], col_const(n + t));
     }
     __device__ __forceinline__ bool direct(int) const { return false; }
     // eight consecutive columns (n % 8 == 0, n + 7 < N, ldo % 8 == 0): same arithmetic as store(), vector accesses
@@ -544,7 +488,7 @@ __global__ void __launch_bounds__(WM *WN * 64)
 
 
 // ---- tiled, pipelined kernel for the aligned x * W^T case ----------------------------------------------
-// One workgroup of four waves (one per SIMD) per output tile.  The waves form a WGM x WGN x WGK grid: a wave
+// One workgroup of four or eight waves (one or two per SIMD) per output tile.  The waves form a WGM x WGN x WGK grid: a wave
 // owns a (32*TM) x (32*TN) block of the tile and, when WGK > 1, every WGK-th 32-byte k-step of each slab
 // (the partial sums of the WGK waves are added in the epilogue).  Tile = (32*TM*WGM) x (32*TN*WGN).
 //   * the launcher picks the shape so that the tile count is at most (or a multiple of) the CU count with
@@ -562,23 +506,24 @@ template <int TM_, int TN_, int WGM_, int WGN_, int WGK_, int SLAB_> struct Tile
     static constexpr int STRIDE = SLAB + 16;
     static constexpr int SSTR   = 32 * TN + 4;  // staged row stride in 32-bit words
     static constexpr size_t slab_bytes  = (size_t)2 * (BM + BN) * STRIDE;
-    static constexpr size_t stage_bytes = (size_t)4 * 32 * SSTR * 4;
+    static constexpr size_t stage_bytes = (size_t)WGM_ * WGN_ * WGK_ * 32 * SSTR * 4;
     static constexpr size_t lds_bytes   = slab_bytes > stage_bytes ? slab_bytes : stage_bytes;
-    static_assert(WGM * WGN * WGK == 4, "four waves per workgroup");
+    static constexpr int NW = WGM * WGN * WGK, NT = 64 * NW;  // waves and threads per workgroup
+    static_assert(NW == 4 || NW == 8, "four or eight waves per workgroup");
     static_assert((SLAB / 32) % WGK == 0, "k-steps of a slab must split evenly over the k-waves");
-    static_assert((BM * (SLAB / 16)) % 256 == 0 && (BN * (SLAB / 16)) % 256 == 0, "slab must divide over the workgroup");
+    static_assert((BM * (SLAB / 16)) % NT == 0 && (BN * (SLAB / 16)) % NT == 0, "slab must divide over the workgroup");
 };
 
 template <int DT, typename CFG, typename Epi>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(CFG::NT)
     gemm_nk_tiled_kernel(const typename GemmTraits<DT>::elem *__restrict__ A,
                          const typename GemmTraits<DT>::elem *__restrict__ B, int M, int N, int K, long lda, long ldb,
-                         int tiles_m, int tiles_n, Epi epi) {
+                         int tiles_m, int tiles_n, int group_m, Epi epi) {
     typedef typename GemmTraits<DT>::elem T;
     typedef typename GemmTraits<DT>::acc Acc;
     constexpr int TM = CFG::TM, TN = CFG::TN, WGN = CFG::WGN, WGK = CFG::WGK, SLAB = CFG::SLAB;
     constexpr int BM = CFG::BM, BN = CFG::BN, STRIDE = CFG::STRIDE;
-    constexpr int NT     = 256;
+    constexpr int NT     = CFG::NT;
     constexpr int VEC    = 16 / sizeof(T);
     constexpr int KB     = SLAB / sizeof(T);
     constexpr int VPR    = SLAB / 16;  // 16-byte vectors per slab row
@@ -594,14 +539,23 @@ __global__ void __launch_bounds__(256)
     const int wn   = (wave / WGK) % WGN;
     const int wm   = wave / (WGK * WGN);
 
-    // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so give each XCD a contiguous run of
-    // tiles (shared A row panels stay in one L2)
-    int pid           = blockIdx.x;
+    // Tile order.  Workgroups are dealt round-robin to the 8 XCDs, each with its own 4 MB L2, and run roughly in
+    // launch order.  Every XCD takes a contiguous run of a "grouped" tile order (group_m tile rows at a time, down
+    // the rows first, then the next tile column), so the tiles that are resident together on one XCD form a
+    // compact block of the tile grid: their A and W panels fit that L2 and are fetched from HBM once, instead of
+    // the whole W panel streaming through every L2 once per tile row.
     const int n_tiles = tiles_m * tiles_n;
-    if ((n_tiles & 7) == 0)
-        pid = (pid & 7) * (n_tiles >> 3) + (pid >> 3);
-    const int m0 = (pid / tiles_n) * BM;
-    const int n0 = (pid % tiles_n) * BN;
+    const int per_xcd = (n_tiles + 7) >> 3;
+    const int vid     = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (vid >= n_tiles)
+        return;  // the grid is padded to a multiple of 8; whole workgroups leave before any barrier
+    const int group_sz = group_m * tiles_n;
+    const int grp      = vid / group_sz;
+    const int first_m  = grp * group_m;
+    const int rows_g   = tiles_m - first_m < group_m ? tiles_m - first_m : group_m;
+    const int in_grp   = vid - grp * group_sz;
+    const int m0       = (first_m + in_grp % rows_g) * BM;
+    const int n0       = (in_grp / rows_g) * BN;
 
     u32x4 ra0[A_VECS], rb0[B_VECS], ra1[A_VECS], rb1[B_VECS];
 
@@ -698,34 +652,6 @@ __global__ void __launch_bounds__(256)
 #undef TR_CLAMPK
 
     typedef typename std::remove_reference<decltype(acc[0][0][0])>::type AccT;
-    if (WGK == 1 && epi.direct(n0)) {
-        // straight from the accumulator layout: lane owns row m; group r4 holds columns 8*r4 + 4*(lane/32) + 0..3
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int m = m0 + (wm * TM + i) * 32 + (lane & 31);
-            if (m >= M)
-                continue;
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    const int n = n0 + (wn * TN + j) * 32 + 8 * r4 + 4 * (lane >> 5);
-                    if (n + 3 < N) {
-                        AccT v[4] = {acc[i][j][r4 * 4 + 0], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2],
-                                     acc[i][j][r4 * 4 + 3]};
-                        epi.store4(m, n, v);
-                    } else {
-#pragma unroll
-                        for (int t = 0; t < 4; ++t)
-                            if (n + t < N)
-                                epi.store(m, n + t, acc[i][j][r4 * 4 + t], epi.col_const(n + t));
-                    }
-                }
-            }
-        }
-        return;
-    }
-
     // Row-contiguous epilogue.  In the accumulator layout one store instruction touches 32 rows with 16 bytes
     // each, i.e. 32 partial cache lines; the L2 then sees eight times as many write requests as there are lines.
     // For each 32-row group every wave writes its 32 x CW accumulator block to its own LDS region (the slab
@@ -735,11 +661,12 @@ __global__ void __launch_bounds__(256)
     constexpr int CW   = TN * 32;       // columns per wave
     constexpr int SSTR = CFG::SSTR;     // staged row stride in 32-bit words (16-byte pad spreads the b128 banks)
     constexpr int CPR  = CW / 8;        // 8-column pieces per staged row
-    constexpr int POS  = 4 / WGK;       // wave positions (wm, wn) in the tile
+    constexpr int POS  = CFG::NW / WGK;  // wave positions (wm, wn) in the tile
     constexpr int ITEMS = POS * 32 * CPR;
     typedef AccT acc4 __attribute__((ext_vector_type(4)));
     AccT *const stage_all = reinterpret_cast<AccT *>(lds_dyn);
     AccT *const stage_me  = stage_all + wave * (32 * SSTR);  // wave = (wm*WGN + wn)*WGK + wk
+    const bool by_rows = epi.direct(n0);
     __syncthreads();  // every wave is done reading the slabs
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -755,8 +682,10 @@ __global__ void __launch_bounds__(256)
             const int item = it * NT + tid;
             if (ITEMS % NT != 0 && item >= ITEMS)
                 break;
-            const int c8  = (item % CPR) * 8;
-            const int row = (item / CPR) % 32;
+            // consecutive threads walk along a row of C, or down the rows where the epilogue writes a transposed
+            // layout (consecutive rows are then consecutive in memory)
+            const int c8  = by_rows ? ((item >> 5) % CPR) * 8 : (item % CPR) * 8;
+            const int row = by_rows ? (item & 31) : (item / CPR) % 32;
             const int pos = item / (CPR * 32);  // = pm * WGN + pn
             const AccT *src = stage_all + (pos * WGK) * (32 * SSTR) + row * SSTR + c8;
             acc4 lo = *reinterpret_cast<const acc4 *>(src);
@@ -787,6 +716,7 @@ __global__ void __launch_bounds__(256)
 
 // tuning override for experiments: 0 = heuristic, otherwise a configuration code of the tiled kernel
 int g_gemm_force_cfg = 0;
+int g_gemm_group_m   = 0;  // 0 = derived from the tile count; otherwise forced
 
 template <int DT, typename CFG, typename Epi>
 int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb, const Epi &epi) {
@@ -801,60 +731,74 @@ int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int 
             attr_set = true;
         }
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), lds, s, (const T *)A, (const T *)B, M, N, K,
-                       lda, ldb, tiles_m, tiles_n, epi);
+    // tiles resident together on one XCD (32 CUs): a square-ish group keeps their panels in that L2
+    const long lds_per_cu = 160 * 1024;
+    long per_cu   = lds_per_cu / (long)(lds + 1024);
+    per_cu        = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
+    long resident = 32 * per_cu, per_xcd = ((long)tiles_m * tiles_n + 7) / 8;
+    resident      = resident < per_xcd ? resident : per_xcd;
+    int group_m   = g_gemm_group_m > 0 ? g_gemm_group_m : 1;
+    if (g_gemm_group_m <= 0)
+        while ((long)(group_m + 1) * (group_m + 1) <= resident)
+            ++group_m;
+    group_m = group_m > tiles_m ? tiles_m : group_m;
+    unsigned grid = (unsigned)(((tiles_m * tiles_n + 7) / 8) * 8);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(CFG::NT), lds, s, (const T *)A, (const T *)B, M, N, K, lda, ldb, tiles_m, tiles_n,
+                       group_m, epi);
     TR_CHECK_LAUNCH();
     return 0;
 }
 
-// Configuration codes: TM TN WGM WGN WGK S (one decimal digit each; S = 1 for 128-byte slabs, 0 for 64-byte).
-//   112210 / 112211   64 x  64      222210 / 222211  128 x 128      331141   96 x 96, four k-waves
-// Larger tiles with one wave per SIMD (128x256, 256x128, 192x192) and two-k-wave shapes were measured and never
-// won with compiler-scheduled code: they need more latency hiding than a single wave per SIMD provides.
+// Configuration codes: TM TN WGM WGN WGK S (one decimal digit each; slab bytes = 64 << S).
+//   112210 / 112211   64 x  64, 4 waves                 222210  128 x 128, 4 waves
+//   222221           128 x 128, 8 waves (two k-waves)   224211  256 x 128, 8 waves
+//   332221           192 x 192, 8 waves (two k-waves)   331182   96 x  96, 8 k-waves, 256-byte slabs
+// Eight-wave workgroups put two waves on every SIMD inside one tile: while one waits for its LDS fragments the
+// other issues MFMAs, and a larger tile per CU moves fewer bytes through LDS and L2 per flop.  Four-wave tiles
+// larger than 128 x 128 (one wave per SIMD) were measured and never won with compiler-scheduled code.
 constexpr int kNumCU = 256;
 
 // Shape heuristic, from measurements on MI355X (fp16; M in {1024, 3072, 4096, 16384}, N and K in
-// {768, 1024, 2304, 3072, 4096}):
-//   * more than one round of 128x128 tiles at two workgroups per CU: 128x128; with short K the 64-byte slab
-//     version wins (fewer registers and less LDS: three to four workgroups per CU hide latency better), e.g.
-//     M=4096 N=3072 K=1024: 43 us vs 52; M=16384 N=3072 K=768: 135 vs 140; long K prefers 128-byte slabs
-//     (M=16384 N=768 K=3072: 106 vs 115) -- unless the second round would be nearly empty (M=3072 N=3072:
-//     576 tiles for 512 slots, 64x64 tiles 32.5 us vs 34);
-//   * between one and two workgroups of 128x128 per CU: 128x128 (M=3072 N=2304: 22.3 us vs 23.3 for 64x64);
-//   * fewer: 64x64 tiles keep every CU busy (M=3072 N=768 K=768: 12.0 us vs 13.9), except for a long K with
-//     about one 96x96 tile per CU, where four k-waves on one 96x96 tile re-read the least
-//     (M=3072 N=768 K=3072: 29.5 us vs 33.9), or at least half a 128x128 tile per CU
-//     (M=4096 N=1024 K=4096: 54 us vs 66).
-inline int pick_tile_config(long M, long N, size_t kbytes, bool allow_ksplit) {
+// {768, 1024, 2304, 3072, 4096}; times in us, best alternative in parentheses):
+//   * default 128x128 with eight waves: M=4096 N=3072 K=1024 37 (4 waves 43), M=4096 N=1024 K=4096 45 (54),
+//     M=16384 N=3072 K=768 122 (135), M=16384 N=768 K=3072 95 (106);
+//   * small launches (at most ~0.6 tiles of 128x128 per CU): 64x64 tiles keep every CU busy
+//     (M=3072 N=768 K=768 12.4 vs 12.9; M=1024 shapes 9.5-19 vs 13-35);
+//   * a narrow N with a long K and about one 96x96 tile per CU: eight k-waves on one 96x96 tile
+//     (M=3072 N=768 K=3072 25.6 vs 30.7);
+//   * between one and two 128x128 tiles per CU: 256x128 when that is a single round (M=3072 N=2304 19.7 vs 20.6);
+//   * slightly more than one round of 128x128 at two workgroups per CU, but a single round of 192x192
+//     (M=3072 N=3072: 576 tiles for 512 slots): 192x192 (28.8 vs 31.9).
+inline int pick_tile_config(long M, long N, size_t kbytes) {
     auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    const bool s128 = kbytes % 128 == 0;
     const long t128 = tiles(128, 128), slots = 2 * kNumCU;
-    if (t128 > slots) {
-        if (t128 < 2 * slots && (t128 % slots) * 4 < slots)
-            return s128 ? 112211 : 112210;
-        return (s128 && kbytes >= 4096) ? 222211 : 222210;
-    }
-    if (t128 > kNumCU)
-        return 222210;
-    if (s128 && kbytes >= 4096) {
+    if (kbytes % 128 != 0)
+        return t128 > kNumCU ? 222210 : 112210;
+    if (kbytes >= 4096 && kbytes % 256 == 0) {
         const long t96 = tiles(96, 96);
-        if (allow_ksplit && t96 <= kNumCU && t96 > kNumCU / 2)
-            return 331141;
-        if (t128 > kNumCU / 2)
-            return 222211;
+        if (t96 <= kNumCU && t96 > kNumCU / 2 && t128 <= kNumCU)
+            return 331182;
     }
-    return s128 ? 112211 : 112210;
+    if (t128 * 10 <= kNumCU * 6)
+        return 112211;
+    if (t128 > kNumCU && t128 <= slots && tiles(256, 128) <= kNumCU)
+        return 224211;
+    if (t128 > slots && t128 < slots + slots / 4 && tiles(192, 192) <= kNumCU)
+        return 332221;
+    return 222221;
 }
 
 template <int DT, typename Epi>
 int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb,
-                     const Epi &epi, bool allow_ksplit = true) {
+                     const Epi &epi) {
     typedef typename GemmTraits<DT>::elem T;
     int cfg       = g_gemm_force_cfg > 0 ? g_gemm_force_cfg : 0;
     size_t kbytes = (size_t)K * sizeof(T);
     if (cfg == 0)
-        cfg = pick_tile_config(M, N, kbytes, allow_ksplit && DT != TNN_ROCM_F32);
-    if (kbytes % ((cfg % 10) ? 128 : 64) != 0) {
+        cfg = pick_tile_config(M, N, kbytes);
+    if (DT == TNN_ROCM_F32 && (cfg == 224211 || cfg == 332221 || cfg == 331182))
+        cfg = 222221;
+    if (kbytes % (64u << (cfg % 10)) != 0) {
         set_error("gemm: K=%d is not a whole number of slabs for tuning configuration %d", K, cfg);
         return TNN_ROCM_ESHAPE;
     }
@@ -864,12 +808,16 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
         case 112210: TR_FAST(1, 1, 2, 2, 1, 64);
         case 112211: TR_FAST(1, 1, 2, 2, 1, 128);
         case 222210: TR_FAST(2, 2, 2, 2, 1, 64);
-        case 222211: TR_FAST(2, 2, 2, 2, 1, 128);
+        case 222221: TR_FAST(2, 2, 2, 2, 2, 128);
         default: break;
     }
     if constexpr (DT != TNN_ROCM_F32) {
-        if (cfg == 331141)
-            TR_FAST(3, 3, 1, 1, 4, 128);
+        switch (cfg) {
+            case 224211: TR_FAST(2, 2, 4, 2, 1, 128);
+            case 332221: TR_FAST(3, 3, 2, 2, 2, 128);
+            case 331182: TR_FAST(3, 3, 1, 1, 8, 256);
+            default: break;
+        }
     }
 #undef TR_FAST
     set_error("gemm: unknown tuning configuration %d", cfg);
@@ -1028,8 +976,7 @@ int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *
         epi.H     = H;                                                                                                \
         epi.S     = S;                                                                                                \
         epi.heads = heads;                                                                                            \
-        return launch_gemm_fast<DT, QkvSplitEpilogue<DT>>((hipStream_t)stream, x, wqkv, T, 3 * H, K, K, K, epi,    \
-                                                               /*allow_ksplit=*/false);      \
+        return launch_gemm_fast<DT, QkvSplitEpilogue<DT>>((hipStream_t)stream, x, wqkv, T, 3 * H, K, K, K, epi);      \
     }
     if (dtype == TNN_ROCM_F16)
         TR_QKV(TNN_ROCM_F16)
@@ -1042,6 +989,10 @@ int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *
 // kernel, other values select a configuration code of the tiled kernel.
 __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_config(int cfg) {
     g_gemm_force_cfg = cfg;
+    return 0;
+}
+__attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_group_m(int group_m) {
+    g_gemm_group_m = group_m;
     return 0;
 }
 
