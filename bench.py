@@ -22,6 +22,16 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 
+# HBM bytes per launch (fetched + written) of the projection GEMMs at the batch-8 / seq-384 workload, from two
+# rocprofv3 --pmc runs of this command (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
+# --counter-reference kernel (64 MiB in, 64 MiB out): FETCH_SIZE reads half the bytes, WRITE_SIZE all of them.
+MEASURED_HBM_BYTES_PER_LAUNCH = {
+    "gemm_qkv": int((2 * 14354.1 + 13970.0) * 1024),   # algorithmic: 4.5 + 3.4 in, 13.5 out MiB
+    "gemm_out": int((2 * 10431.5 + 4608.0) * 1024),    # algorithmic: 4.5 + 1.1 + 4.5 in, 4.5 out MiB
+    "gemm_ffn1": int((2 * 16358.3 + 18432.0) * 1024),  # algorithmic: 4.5 + 4.5 in, 18 out MiB
+    "gemm_ffn2": int((2 * 37064.9 + 4608.3) * 1024),   # algorithmic: 18 + 4.5 + 4.5 in, 4.5 out MiB
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -106,28 +116,48 @@ def main():
     inst.sync()
     dt = time.perf_counter() - t0
 
-    # ---- per-launch durations of the GEMM layers: a captured graph cannot carry per-launch events, so the same K
-    # steps are run once more through the eager layer loop with events around every RocmFusedLinear launch on the
-    # instance's stream (rocprofv3's kernel trace of this command reports the same averages)
-    inst.profile_start("RocmFusedLinear")
-    for _ in range(args.steps):
-        inst.forward()
-    inst.sync()
-    gemm_prof = inst.profile_finish()
-
     ms_per_step = dt / args.steps * 1e3
     seqs_per_s = B * args.steps / dt
     T, H, F = B * S, cfg.hidden, cfg.ffn
-    gemm_flops = {"gemm_out": 2.0 * T * H * H, "gemm_ffn1": 2.0 * T * F * H, "gemm_ffn2": 2.0 * T * H * F}
-    per_class = {}
-    for t, name, ms in gemm_prof:
-        if t == "RocmFusedLinear":
-            per_class.setdefault(classify(name), []).append(ms)
-    dominant = max((k for k in per_class if k in gemm_flops), key=lambda k: sum(per_class[k]))
-    dom_ms = sum(per_class[dominant]) / len(per_class[dominant])
+
+    # ---- per-launch duration of the four projection GEMMs.  A captured graph cannot carry per-launch events and an
+    # event pair around one 10-30 us launch in the eager layer loop also times the launch gap, so each GEMM is
+    # launched back to back (same shapes, same fused epilogue, through the same C entry point the layers call)
+    # between two events on the launch stream; rocprofv3's kernel trace of this command reports the same averages.
+    def timed(fn, n):
+        for _ in range(5):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    n_gemm = max(args.steps, 20) * cfg.layers
+    x_h = torch.randn(T, H, device="cuda").half()
+    x_f = torch.randn(T, F, device="cuda").half()
+    res = torch.randn(T, H, device="cuda").half()
+    w_qkv, w_o = (torch.randn(3 * H, H, device="cuda") * 0.02).half(), (torch.randn(H, H, device="cuda") * 0.02).half()
+    w_1, w_2 = (torch.randn(F, H, device="cuda") * 0.02).half(), (torch.randn(H, F, device="cuda") * 0.02).half()
+    b_qkv, b_h, b_f = (torch.randn(n, device="cuda") * 0.02 for n in (3 * H, H, F))
+    o_h = torch.empty(T, H, device="cuda", dtype=torch.float16)
+    o_f = torch.empty(T, F, device="cuda", dtype=torch.float16)
+    gemm_ms = {
+        "gemm_qkv": timed(lambda: ops.qkv_split(x_h, w_qkv, b_qkv, B, S, cfg.heads), n_gemm),
+        "gemm_out": timed(lambda: ops.gemm(x_h, w_o, True, bias=b_h, residual=res, out=o_h), n_gemm),
+        "gemm_ffn1": timed(lambda: ops.gemm(x_h, w_1, True, bias=b_f, gelu=True, out=o_f), n_gemm),
+        "gemm_ffn2": timed(lambda: ops.gemm(x_f, w_2, True, bias=b_h, residual=res, out=o_h), n_gemm),
+    }
+    gemm_flops = {"gemm_qkv": 2.0 * T * 3 * H * H, "gemm_out": 2.0 * T * H * H, "gemm_ffn1": 2.0 * T * F * H,
+                  "gemm_ffn2": 2.0 * T * H * F}
+    gemm_shape = {"gemm_qkv": (T, 3 * H, H), "gemm_out": (T, H, H), "gemm_ffn1": (T, F, H), "gemm_ffn2": (T, H, F)}
+    dominant = max(gemm_ms, key=lambda k: gemm_ms[k])
+    dom_ms = gemm_ms[dominant]
     achieved = gemm_flops[dominant] / (dom_ms * 1e-3) / 1e12
 
-    # ---- untimed: full per-layer profile and the attention kernel on its own
+    # ---- untimed: per-layer profile of the eager layer loop (events around every layer; includes launch gaps)
     full = inst.profile(5)
     breakdown = {}
     for t, name, ms in full:
@@ -136,22 +166,23 @@ def main():
     out_final = inst.output("last_hidden")
     assert np.isfinite(out_final).all()
 
-    # the attention kernel on its own, in the layout the fused layer uses (Q|K row-major, V transposed per head)
-    d_lens = torch.from_numpy(lens).cuda()
-    qk = torch.randn(T, 2 * H, device="cuda").half()
-    vt = torch.randn(B, cfg.heads, 64, S, device="cuda").half()
-    ctx = torch.empty(T, H, device="cuda", dtype=torch.float16)
-    for _ in range(5):
-        ops.attention_qk_vt(qk, vt, B, S, cfg.heads, 0.125, kv_len=d_lens, out=ctx)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(50):
-        ops.attention_qk_vt(qk, vt, B, S, cfg.heads, 0.125, kv_len=d_lens, out=ctx)
-    e1.record()
-    torch.cuda.synchronize()
-    attn_ms = e0.elapsed_time(e1) / 50
-    attn_eff_flops = 4.0 * H * S * float(lens.sum())
-    attn_pad_flops = 4.0 * B * S * S * H
+    # the attention kernel on its own, in the layout the fused layer uses (Q|K row-major, V transposed per head):
+    # this workload's shape, and the variable-length stress shape (B32, 12 heads x 64, S 512, lengths U[16,512])
+    def attention_tflops(B_, S_, lens_):
+        d_lens = torch.from_numpy(lens_.astype(np.int32)).cuda()
+        qk = torch.randn(B_ * S_, 2 * H, device="cuda").half()
+        vt = torch.randn(B_, cfg.heads, 64, S_, device="cuda").half()
+        ctx = torch.empty(B_ * S_, H, device="cuda", dtype=torch.float16)
+        ms = timed(lambda: ops.attention_qk_vt(qk, vt, B_, S_, cfg.heads, 0.125, kv_len=d_lens, out=ctx), 100)
+        eff, pad = 4.0 * H * S_ * float(lens_.sum()), 4.0 * B_ * S_ * S_ * H
+        return {"effective": round(eff / (ms * 1e-3) / 1e12, 2), "padded": round(pad / (ms * 1e-3) / 1e12, 2),
+                "us_per_launch": round(ms * 1e3, 2),
+                "frac_of_fp16_peak_effective": round(eff / (ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 4)}
+
+    attn_here = attention_tflops(B, S, lens)
+    stress_lens = np.random.default_rng(20240603).integers(16, 513, 32)
+    attn_stress = attention_tflops(32, 512, stress_lens)
+    attn_stress["workload"] = "B32 h12 d64 S512, valid lengths U[16,512] (BASELINE.json configs[2])"
 
     if args.counter_reference:
         big = torch.randn(16 * 1024 * 1024, device="cuda", dtype=torch.float32)
@@ -173,18 +204,19 @@ def main():
                    "layers": args.layers, "batch": B, "seq_len": S, "hidden": H, "heads": cfg.heads, "ffn": F,
                    "sum_valid_len": int(lens.sum()), "host_layers": len(layer_types)},
         "model_tflops": round(cfg.flops_per_sequence(S) * seqs_per_s / 1e12, 2),
-        "attention_tflops": {"effective": round(attn_eff_flops / (attn_ms * 1e-3) / 1e12, 2),
-                             "padded": round(attn_pad_flops / (attn_ms * 1e-3) / 1e12, 2),
-                             "us_per_launch": round(attn_ms * 1e3, 2),
-                             "frac_of_fp16_peak_effective": round(attn_eff_flops / (attn_ms * 1e-3) / 1e12 /
-                                                                  PEAK_FP16_TFLOPS, 4)},
-        "roofline": {"bound": "mfma", "kernel": "gemm_kernel (%s)" % dominant, "achieved": round(achieved, 2),
-                     "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
-                     "traffic": None, "us_per_launch": round(dom_ms * 1e3, 2),
-                     "timed_over": "%d eager steps with events on the launch stream, right after the timed region "
-                                   "(which replays a captured graph)" % args.steps,
-                     "launches_timed": len(per_class[dominant]) * args.steps,
-                     "flops_per_launch": gemm_flops[dominant]},
+        "attention_tflops": attn_here,
+        "attention_tflops_varlen_stress": attn_stress,
+        "roofline": {"bound": "mfma",
+                     "kernel": "gemm_nk_tiled_kernel (%s: M=%d N=%d K=%d, fused epilogue)" % ((dominant,) + gemm_shape[dominant]),
+                     "achieved": round(achieved, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
+                     "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get(dominant) if full_cfg else None,
+                     "us_per_launch": round(dom_ms * 1e3, 2),
+                     "timed_over": "%d back-to-back launches between two events on the launch stream, right after "
+                                   "the timed region (which replays a captured graph)" % n_gemm,
+                     "flops_per_launch": gemm_flops[dominant],
+                     "all_gemms_us_per_launch": {k: round(v * 1e3, 2) for k, v in sorted(gemm_ms.items())},
+                     "all_gemms_tflops": {k: round(gemm_flops[k] / (v * 1e-3) / 1e12, 1) for k, v in sorted(gemm_ms.items())}},
         "layer_breakdown_ms_per_step": {k: round(v, 4) for k, v in sorted(breakdown.items())},
     }
     inst.close()
