@@ -441,7 +441,8 @@ def test_attention_fp16_varlen():
     # the same padding expressed the TNN way: additive -10000 mask + kv_len hint
     got2, ref2 = _attn_case(8, 2, 512, lens, seed=99, with_mask=True)
     assert rel_err(got2, ref2) <= FP16_TOL
-    assert rel_err(got2, got) <= 1e-6
+    # tiles without a mask take a shorter path (one fused multiply-add per score): equal up to an fp16 rounding
+    assert rel_err(got2, got) <= 1e-3
 
 
 def test_attention_fp16_128row_blocks():

@@ -41,6 +41,17 @@ template <> struct AttnT<TNN_ROCM_F16> {
         half_t l = (half_t)lo, h = (half_t)hi;
         return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
     }
+    // Probabilities (0..1) for the second MFMA: one v_cvt_pkrtz per pair.  The row sum is taken over the SAME
+    // rounded values (v_dot2 with (1,1), fp32 accumulate), so numerator and denominator of the softmax stay
+    // consistent and the truncation does not bias the normalised weights.
+    static __device__ __forceinline__ uint32_t pack_prob(float lo, float hi, float &sum) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        typedef __fp16 fp16x2 __attribute__((ext_vector_type(2)));
+        fp16x2 pk = __builtin_amdgcn_cvt_pkrtz(lo, hi);
+        h2 one    = {(_Float16)1.0f, (_Float16)1.0f};
+        sum       = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, pk), one, sum, false);
+        return __builtin_bit_cast(uint32_t, pk);
+    }
 };
 template <> struct AttnT<TNN_ROCM_BF16> {
     template <typename V> static __device__ __forceinline__ void mma(const V &a, const V &b, f32x16 &c) {
@@ -49,6 +60,11 @@ template <> struct AttnT<TNN_ROCM_BF16> {
     }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+    }
+    static __device__ __forceinline__ uint32_t pack_prob(float lo, float hi, float &sum) {
+        uint32_t l = float_to_bf16(lo), h = float_to_bf16(hi);
+        sum += __uint_as_float(l << 16) + __uint_as_float(h << 16);  // the rounded values, as in the fp16 path
+        return l | (h << 16);
     }
 };
 
@@ -66,8 +82,22 @@ struct AttnParams {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
+// Combine a value with the one held by lane ^ 32 (the other half of the same query column) with one
+// v_permlane32_swap: after swapping the upper half of one copy with the lower half of the other, every lane
+// holds its own value in one register and its partner's in the other.
+__device__ __forceinline__ float half_swap_max(float v) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_swap_sum(float v) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// The second launch bound (at least two waves per SIMD) caps the kernel at 256 registers, which keeps the MFMA accumulators in ordinary VGPRs: the softmax
+// reads and rescales them with VALU instructions, and accumulators parked in AGPRs cost a move per access.
 template <int DT, int NW, bool VT>
-__global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
+__global__ void __launch_bounds__(NW * 64, 2) attention_kernel(AttnParams p) {
     constexpr int NT = NW * 64;
     constexpr int BQ = NW * 32;
     // per tile: 64 rows (keys, or d for V^T) x 8 sixteen-byte chunks
@@ -75,9 +105,14 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
     constexpr int ROW_STEP = NT / 8;
     static_assert(kTileKV * 8 % NT == 0, "tile must divide over the workgroup");
 
-    __shared__ __attribute__((aligned(16))) unsigned char lds_k[2][kTileKV * kRowBytes];
-    __shared__ __attribute__((aligned(16))) unsigned char lds_vt[2][kD * kRowBytes];
+    // one LDS block: [K tile 0 | V^T tile 0 | K tile 1 | V^T tile 1]; the second half doubles as the staging area of
+    // the Q block before the first tile is stored there, the first half as the staging area of the output block
+    constexpr int kTileBytes = kTileKV * kRowBytes;  // = kD * kRowBytes
+    __shared__ __attribute__((aligned(16))) unsigned char lds_all[4 * kTileBytes];
     __shared__ __attribute__((aligned(16))) float lds_bias[2][kTileKV];
+    unsigned char *const lds_k0 = lds_all, *const lds_vt0 = lds_all + kTileBytes;
+    unsigned char *const lds_k1 = lds_all + 2 * kTileBytes, *const lds_vt1 = lds_all + 3 * kTileBytes;
+    static_assert(BQ * kRowBytes <= 2 * kTileBytes, "Q / O staging must fit half of the tile buffers");
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -117,34 +152,53 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
     // beyond kv_end then carry finite (wrong) data, and their score bias of -inf makes their probability exactly 0,
     // so neither the max, the sum nor P.V sees them; query rows past S are computed but never stored.
     // Q fragments (B operand of S^T = K Q^T): lane (lq, g) holds Q[q0+lq][16*kk + 8*g .. +7]
+    // The block's BQ x 64 Q rows are copied through LDS with whole 128-byte rows per 8 lanes (a lane reading its own
+    // row directly touches 32 rows per instruction with 32 bytes each).
     u32x4 qf[4];
     {
-        int qrow = q0 + lq;
-        qrow     = qrow < S ? qrow : S - 1;
-        const uint16_t *qp = qb + (size_t)qrow * p.q_ss + g * 8;
+        unsigned char *const stage = lds_k1;  // free until the end of the first tile
+        constexpr int Q_VECS = BQ * 8 / NT;
+#pragma unroll
+        for (int i = 0; i < Q_VECS; ++i) {
+            const int v = tid + i * NT, r = v >> 3, c = v & 7;
+            int qrow = (q0 - wave * 32) + r;
+            qrow     = qrow < S ? qrow : S - 1;
+            *reinterpret_cast<u32x4 *>(stage + r * kRowBytes + c * 16) =
+                *reinterpret_cast<const u32x4 *>(qb + (size_t)qrow * p.q_ss + c * 8);
+        }
+        __syncthreads();
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
-            qf[kk] = *reinterpret_cast<const u32x4 *>(qp + kk * 16);
+            qf[kk] = *reinterpret_cast<const u32x4 *>(stage + (wave * 32 + lq) * kRowBytes + kk * 32 + g * 16);
+        __syncthreads();  // the staging area becomes tile buffer 1
     }
 
     const int vrow = tid >> 3, vch = tid & 7;  // this thread's row / 16-byte chunk inside a tile (plus i*ROW_STEP)
+    // one tile of look-ahead in registers (a second register set for two tiles ahead was measured slower: the
+    // extra registers cost a resident wave per SIMD, and the memory latency is already covered)
     u32x4 rk[KV_VECS], rv[KV_VECS];
     float rbias = 0.f;
+    // element offsets from the (batch, head) base fit 32 bits (checked by the launcher)
+    const uint32_t kv_ss32 = (uint32_t)p.kv_ss, vt_sd32 = (uint32_t)p.vt_sd;
+    uint32_t v_off[KV_VECS];  // V^T: row d = vrow + i*ROW_STEP, plus the key offset of the tile
+#pragma unroll
+    for (int i = 0; i < KV_VECS; ++i)
+        v_off[i] = (uint32_t)(vrow + i * ROW_STEP) * vt_sd32;
 
 #define TR_LOAD_TILE(T)                                                                                               \
     {                                                                                                                 \
         const int kv0 = (T) * kTileKV;                                                                                \
+        int k8        = kv0 + vch * 8;                                                                                \
+        k8            = k8 < S ? k8 : S - 8;                                                                          \
         _Pragma("unroll") for (int i = 0; i < KV_VECS; ++i) {                                                         \
             int key = kv0 + vrow + i * ROW_STEP;                                                                      \
             key     = key < S ? key : S - 1;                                                                          \
-            rk[i]   = *reinterpret_cast<const u32x4 *>(kb + (size_t)key * p.kv_ss + vch * 8);                         \
-            if (VT) {                                                                                                 \
-                int k8 = kv0 + vch * 8;                                                                               \
-                k8     = k8 < S ? k8 : S - 8;                                                                         \
-                rv[i]  = *reinterpret_cast<const u32x4 *>(vb + (size_t)(vrow + i * ROW_STEP) * p.vt_sd + k8);         \
-            } else {                                                                                                  \
-                rv[i] = *reinterpret_cast<const u32x4 *>(vb + (size_t)key * p.kv_ss + vch * 8);                       \
-            }                                                                                                         \
+            const uint32_t ko = (uint32_t)key * kv_ss32 + (uint32_t)(vch * 8);                                        \
+            rk[i]   = *reinterpret_cast<const u32x4 *>(kb + ko);                                                      \
+            if (VT)                                                                                                   \
+                rv[i] = *reinterpret_cast<const u32x4 *>(vb + (v_off[i] + (uint32_t)k8));                             \
+            else                                                                                                      \
+                rv[i] = *reinterpret_cast<const u32x4 *>(vb + ko);                                                    \
         }                                                                                                             \
         if (tid < kTileKV) {                                                                                          \
             int key  = kv0 + tid;                                                                                     \
@@ -153,19 +207,28 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
             rbias    = key < kv_end ? mv : -INFINITY;                                                                 \
         }                                                                                                             \
     }
+// V^T rows are stored with the two middle 8-byte chunks of every 16-key group swapped ([k0-3 | k8-11 | k4-7 | k12-15]):
+// the eight keys a lane needs for one MFMA step (16*step + 4*g + 0..3 and 16*step + 8 + 4*g + 0..3) are then one
+// aligned 16-byte read at step*32 + g*16.
 #define TR_STORE_TILE(BUF)                                                                                            \
     {                                                                                                                 \
         _Pragma("unroll") for (int i = 0; i < KV_VECS; ++i) {                                                         \
             const int row = vrow + i * ROW_STEP;                                                                      \
-            *reinterpret_cast<u32x4 *>(&lds_k[BUF][row * kRowBytes + vch * 16]) = rk[i];                              \
+            *reinterpret_cast<u32x4 *>(lds_k##BUF + row * kRowBytes + vch * 16) = rk[i];                              \
             if (VT) {                                                                                                 \
-                *reinterpret_cast<u32x4 *>(&lds_vt[BUF][row * kRowBytes + vch * 16]) = rv[i]; /* row = d, 8 keys */   \
+                /* this thread holds keys 8*vch .. 8*vch+7 of row d: chunk pair (2*(vch&1), 2*(vch&1)+1) of group */  \
+                /* vch/2 goes to chunk positions (vch&1) and (vch&1)+2 */                                             \
+                unsigned char *dst = lds_vt##BUF + row * kRowBytes + (vch >> 1) * 32 + (vch & 1) * 8;                 \
+                *reinterpret_cast<u32x2 *>(dst)      = u32x2{rv[i][0], rv[i][1]};                                     \
+                *reinterpret_cast<u32x2 *>(dst + 16) = u32x2{rv[i][2], rv[i][3]};                                     \
             } else {                                                                                                  \
-                _Pragma("unroll") for (int t = 0; t < 4; ++t) {                                                       \
-                    *reinterpret_cast<uint16_t *>(&lds_vt[BUF][(vch * 8 + 2 * t) * kRowBytes + row * 2]) =            \
-                        (uint16_t)(rv[i][t] & 0xffffu);                                                               \
-                    *reinterpret_cast<uint16_t *>(&lds_vt[BUF][(vch * 8 + 2 * t + 1) * kRowBytes + row * 2]) =        \
-                        (uint16_t)(rv[i][t] >> 16);                                                                   \
+                /* thread holds d = 8*vch .. +7 of key `row`: scatter into the transposed tile at the key's slot */  \
+                const int kslot = (row & ~15) + ((row & 3) | ((row & 4) << 1) | ((row & 8) >> 1));                    \
+                _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                                       \
+                    *reinterpret_cast<uint16_t *>(lds_vt##BUF + (vch * 8 + 2 * e) * kRowBytes + kslot * 2) =          \
+                        (uint16_t)(rv[i][e] & 0xffffu);                                                               \
+                    *reinterpret_cast<uint16_t *>(lds_vt##BUF + (vch * 8 + 2 * e + 1) * kRowBytes + kslot * 2) =      \
+                        (uint16_t)(rv[i][e] >> 16);                                                                   \
                 }                                                                                                     \
             }                                                                                                         \
         }                                                                                                             \
@@ -181,18 +244,10 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
             oacc[dt][r] = 0.f;
     float m_i = -INFINITY, l_i = 0.f;
 
-    if (n_tiles > 0) {
-        TR_LOAD_TILE(0);
-        TR_STORE_TILE(0);
-    }
-    __syncthreads();
-
-    for (int t = 0; t < n_tiles; ++t) {
-        const int buf = t & 1;
-        // look-ahead load of the next tile (clamped to the last one: the redundant copy is never consumed)
-        const int tn = t + 1 < n_tiles ? t + 1 : t;
-        TR_LOAD_TILE(tn);
-
+    // one tile: scores, online softmax, P.V -- reads LDS buffer `buf`, which holds tile t
+    auto tile_body = [&](const int buf, const int t) __attribute__((always_inline)) {
+        const unsigned char *const kbuf  = buf ? lds_k1 : lds_k0;
+        const unsigned char *const vtbuf = buf ? lds_vt1 : lds_vt0;
         // ---- S^T = K Q^T for the 64 keys of the tile: two 32-key blocks
         f32x16 sacc[2];
 #pragma unroll
@@ -202,42 +257,57 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
                 sacc[kt][r] = 0.f;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
-                u32x4 kf = *reinterpret_cast<const u32x4 *>(&lds_k[buf][(kt * 32 + lq) * kRowBytes + kk * 32 + g * 16]);
+                u32x4 kf = *reinterpret_cast<const u32x4 *>(kbuf + (kt * 32 + lq) * kRowBytes + kk * 32 + g * 16);
                 AttnT<DT>::mma(kf, qf[kk], sacc[kt]);
             }
         }
 
-        // ---- online softmax; register r of block kt is key kt*32 + 8*(r/4) + 4*g + (r%4)
+        // ---- online softmax in the exp2 domain; register r of block kt is key kt*32 + 8*(r/4) + 4*g + (r%4).
+        // A tile needs the per-key bias only if it carries an additive mask or reaches past kv_end (the last tile):
+        // all other tiles take the short path, p = exp2(s*c - m) with the row maximum taken on the raw scores.
+        const bool biased = mb != nullptr || (t + 1) * kTileKV > kv_end || !(p.scale_log2e > 0.f);  // workgroup-uniform
         float mx = -INFINITY;
+        if (biased) {
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
+            for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                float4 bias = *reinterpret_cast<const float4 *>(&lds_bias[buf][kt * 32 + r4 * 8 + g * 4]);
-                float bv[4] = {bias.x, bias.y, bias.z, bias.w};
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    float4 bias = *reinterpret_cast<const float4 *>(&lds_bias[buf][kt * 32 + r4 * 8 + g * 4]);
+                    float bv[4] = {bias.x, bias.y, bias.z, bias.w};
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float s2             = fmaf(sacc[kt][r4 * 4 + e], p.scale_log2e, bv[e]);
-                    sacc[kt][r4 * 4 + e] = s2;
-                    mx                   = fmaxf(mx, s2);
+                    for (int e = 0; e < 4; ++e) {
+                        float s2             = fmaf(sacc[kt][r4 * 4 + e], p.scale_log2e, bv[e]);
+                        sacc[kt][r4 * 4 + e] = s2;
+                        mx                   = fmaxf(mx, s2);
+                    }
                 }
             }
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    mx = fmaxf(mx, sacc[kt][r]);
+            mx *= p.scale_log2e;  // scale > 0 on this path: the maximum commutes with it
         }
-        mx          = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx          = half_swap_max(mx);
         float m_new = fmaxf(m_i, mx);
         float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
-        float rs    = 0.f;
+        if (biased) {
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
+            for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float pv    = __builtin_amdgcn_exp2f(sacc[kt][r] - m_use);
-                sacc[kt][r] = pv;
-                rs += pv;
-            }
-        rs += __shfl_xor(rs, 32, 64);
-        l_i = fmaf(l_i, alpha, rs);
+                for (int r = 0; r < 16; ++r)
+                    sacc[kt][r] = __builtin_amdgcn_exp2f(sacc[kt][r] - m_use);
+        } else {
+            const float neg_m = -m_use;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    sacc[kt][r] = __builtin_amdgcn_exp2f(fmaf(sacc[kt][r], p.scale_log2e, neg_m));
+        }
         // the running maximum rarely moves after the first tiles: skip the 32 rescale multiplies when no lane's did
         if (!__all(m_new == m_i)) {
 #pragma unroll
@@ -248,37 +318,55 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
         }
         m_i = m_new;
 
-        // ---- O^T += V^T P^T : four 16-key steps
+        // ---- O^T += V^T P^T : four 16-key steps; the row sum is accumulated while packing
+        float rs = 0.f;
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
             const int kt = st >> 1, j = st & 1;
             u32x4 pf;
-            pf[0] = AttnT<DT>::pack2(sacc[kt][8 * j + 0], sacc[kt][8 * j + 1]);
-            pf[1] = AttnT<DT>::pack2(sacc[kt][8 * j + 2], sacc[kt][8 * j + 3]);
-            pf[2] = AttnT<DT>::pack2(sacc[kt][8 * j + 4], sacc[kt][8 * j + 5]);
-            pf[3] = AttnT<DT>::pack2(sacc[kt][8 * j + 6], sacc[kt][8 * j + 7]);
+            pf[0] = AttnT<DT>::pack_prob(sacc[kt][8 * j + 0], sacc[kt][8 * j + 1], rs);
+            pf[1] = AttnT<DT>::pack_prob(sacc[kt][8 * j + 2], sacc[kt][8 * j + 3], rs);
+            pf[2] = AttnT<DT>::pack_prob(sacc[kt][8 * j + 4], sacc[kt][8 * j + 5], rs);
+            pf[3] = AttnT<DT>::pack_prob(sacc[kt][8 * j + 6], sacc[kt][8 * j + 7], rs);
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt) {
-                const unsigned char *row = &lds_vt[buf][(dt * 32 + lq) * kRowBytes + (st * 16 + g * 4) * 2];
-                u32x2 lo                 = *reinterpret_cast<const u32x2 *>(row);
-                u32x2 hi                 = *reinterpret_cast<const u32x2 *>(row + 16);
-                u32x4 vf                 = {lo[0], lo[1], hi[0], hi[1]};
+                const u32x4 vf = *reinterpret_cast<const u32x4 *>(vtbuf + (dt * 32 + lq) * kRowBytes + st * 32 + g * 16);
                 AttnT<DT>::mma(vf, pf, oacc[dt]);
             }
         }
+        rs  = half_swap_sum(rs);
+        l_i = fmaf(l_i, alpha, rs);
 
-        TR_STORE_TILE(buf ^ 1);
+    };
+
+    if (n_tiles > 0) {
+        TR_LOAD_TILE(0);
+        TR_STORE_TILE(0);
+    }
+    __syncthreads();
+    for (int t = 0; t < n_tiles; t += 2) {
+        // look-ahead load of the next tile (clamped to the last one: the redundant copy is never consumed)
+        TR_LOAD_TILE((t + 1 < n_tiles ? t + 1 : t));
+        tile_body(0, t);
+        TR_STORE_TILE(1);
+        __syncthreads();
+        if (t + 1 >= n_tiles)
+            break;  // uniform over the workgroup
+        TR_LOAD_TILE((t + 2 < n_tiles ? t + 2 : t + 1));
+        tile_body(1, t + 1);
+        TR_STORE_TILE(0);
         __syncthreads();
     }
 #undef TR_LOAD_TILE
 #undef TR_STORE_TILE
 
-    // ---- normalise and store: lane owns query row q0+lq; register r of block dt is
-    //      d = dt*32 + 8*(r/4) + 4*g + (r%4)  -> four consecutive d per register group
-    const int qrow = q0 + lq;
-    if (qrow < S) {
-        float inv = l_i > 0.f ? 1.0f / l_i : 0.f;
-        uint16_t *orow = ob + (size_t)qrow * p.o_ss;
+    // ---- normalise and store.  Lane owns query row q0+lq; register r of block dt is d = dt*32 + 8*(r/4) + 4*g + (r%4).
+    // Written straight from this layout a store instruction would touch 32 rows with 16 bytes each; the wave's 32 x 64
+    // block goes through LDS instead (the tile buffers are free now) and leaves with 8 lanes per 128-byte row.
+    __syncthreads();  // every wave is done with the last tile
+    {
+        unsigned char *const stage = lds_all + wave * 32 * kRowBytes;  // private to this wave
+        const float inv            = l_i > 0.f ? 1.0f / l_i : 0.f;
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -286,8 +374,20 @@ __global__ void __launch_bounds__(NW * 64) attention_kernel(AttnParams p) {
                 u32x2 w;
                 w[0] = AttnT<DT>::pack2(oacc[dt][r4 * 4 + 0] * inv, oacc[dt][r4 * 4 + 1] * inv);
                 w[1] = AttnT<DT>::pack2(oacc[dt][r4 * 4 + 2] * inv, oacc[dt][r4 * 4 + 3] * inv);
-                *reinterpret_cast<u32x2 *>(orow + dt * 32 + r4 * 8 + g * 4) = w;
+                *reinterpret_cast<u32x2 *>(stage + lq * kRowBytes + (dt * 32 + r4 * 8 + g * 4) * 2) = w;
             }
+        // LDS operations of one wave complete in order; the fences keep the compiler from reordering across them
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const int r    = pass * 8 + (lane >> 3);
+            const int qrow = q0 + r;
+            if (qrow < S)
+                *reinterpret_cast<u32x4 *>(ob + (size_t)qrow * p.o_ss + (lane & 7) * 8) =
+                    *reinterpret_cast<const u32x4 *>(stage + r * kRowBytes + (lane & 7) * 16);
+        }
     }
 }
 
@@ -353,6 +453,7 @@ int tnn_rocm_attention(void *stream, int dtype, const void *q, const void *k, co
                    ok(out, o_sb, o_sh, o_ss),
                TNN_ROCM_EALIGN, "attention: pointers must be 16-byte aligned and strides multiples of 8 elements");
     TR_REQUIRE(q_ss >= kD && kv_ss >= kD && o_ss >= kD, TNN_ROCM_ESHAPE, "attention: row stride below head_dim");
+    TR_REQUIRE((long)S * kv_ss < (1l << 31), TNN_ROCM_ESHAPE, "attention: S * row stride exceeds 32-bit tile offsets");
     AttnParams p;
     p.q = (const uint16_t *)q;
     p.k = (const uint16_t *)k;
@@ -391,6 +492,8 @@ int tnn_rocm_attention_vt(void *stream, int dtype, const void *q, const void *k,
                    ok(out, o_sb, o_sh, o_ss),
                TNN_ROCM_EALIGN, "attention_vt: pointers must be 16-byte aligned and strides multiples of 8 elements");
     TR_REQUIRE(q_ss >= kD && k_ss >= kD && o_ss >= kD && vt_sd >= S, TNN_ROCM_ESHAPE, "attention_vt: stride too small");
+    TR_REQUIRE((long)S * k_ss < (1l << 31) && (long)kD * vt_sd + S < (1l << 31), TNN_ROCM_ESHAPE,
+               "attention_vt: per-head extent exceeds 32-bit tile offsets");
     AttnParams p;
     p.q = (const uint16_t *)q;
     p.k = (const uint16_t *)k;
