@@ -142,6 +142,25 @@ TNN_ROCM_API int tnn_rocm_attention_vt(void *stream, int dtype, const void *q, c
                                        long k_sb, long k_sh, long k_ss, long vt_sb, long vt_sh, long vt_sd, long o_sb,
                                        long o_sh, long o_ss, float scale, const float *mask, const int32_t *kv_len);
 
+/* The int8 GEMM above with a float consumer folded in: out_f = (float)q * dequant_scale (+ residual), where q is
+ * the requantised int8 value of tnn_rocm_gemm_i8 (never written).  This is QuantizedInnerProduct -> Reformat
+ * (int8 -> float, x86_compute_int8.cc:1193-1252) -> Add(residual) (compute_elewise.cc:37-65) in one launch; the
+ * product and the sum are rounded separately in fp32 as in that chain.  residual (NULL or dtype out_f_dtype, leading
+ * dimension ldo) has the output's shape. */
+TNN_ROCM_API int tnn_rocm_gemm_i8_dequant_residual(void *stream, const int8_t *A, const int8_t *W, const int32_t *bias,
+                                                   const float *scale, int M, int N, int K, int lda, int ldw,
+                                                   void *out_f, int out_f_dtype, int ldo, float dequant_scale,
+                                                   const void *residual);
+
+/* Quantised Q, K, V projections of one attention layer as a single int8 GEMM over the concatenated weights
+ * wqkv[3H,K] (three QuantizedInnerProduct layers reading the same int8 input): scale[n] = w_scale[n] / o_scale of the
+ * column's projection, dequant[n] = that projection's output blob scale.  Each column is requantised to int8 as in
+ * tnn_rocm_gemm_i8 and written dequantised (the three Reformat layers) in the layout of tnn_rocm_gemm_qkv_split:
+ * Q | K row-major in qk[T,2H], V transposed per head in vt[B][heads][64][S].  out_dtype F16 or BF16. */
+TNN_ROCM_API int tnn_rocm_gemm_i8_qkv_split(void *stream, int out_dtype, const int8_t *x, const int8_t *wqkv,
+                                            const int32_t *bias, const float *scale, const float *dequant, void *qk,
+                                            void *vt, int B, int S, int heads, int K);
+
 /* Fused QKV projection for the attention layer: [T,K] x Wqkv[3H,K]^T + bqkv with the result split on the way out:
  * Q and K go to qk[T, 2H] (row-major, Q | K column blocks), V goes transposed per head to
  * vt[B][heads][64][S] (T = B*S tokens, H = heads*64).  Same arithmetic as three MatMul+Add pairs

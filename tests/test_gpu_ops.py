@@ -403,6 +403,56 @@ def test_gemm_i8_large_accumulators():
     assert np.array_equal(host(q), ref_q)
 
 
+@pytest.mark.parametrize("M,N,K,dtype", [(200, 768, 768, "f32"), (256, 768, 3072, "f32"), (384, 3072, 768, "f16"),
+                                         (3072, 768, 3072, "f16")])
+def test_gemm_i8_dequant_residual_matches_the_three_layer_chain(M, N, K, dtype):
+    """QuantizedInnerProduct -> Reformat(int8->float) -> Add(residual) in one launch: the int8 value is the checker's,
+    the float result is q*s + r with the product and the sum rounded separately in fp32 (then once to fp16)."""
+    say("gemm_i8_dequant_residual M=%d N=%d K=%d %s" % (M, N, K, dtype))
+    rng = np.random.default_rng(M + N + K)
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    bias = rng.integers(-20000, 20000, N).astype(np.int32)
+    w_scale = (rng.uniform(0.5, 1.5, N) * (2e-3 * 768 / K)).astype(np.float32)
+    s_out = np.float32(0.41)
+    scale = orc.fc_int8_scale(w_scale, s_out, N)
+    tdt = torch.float32 if dtype == "f32" else torch.float16
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    if dtype == "f16":
+        res = r16(res)
+    ref_q, _ = orc.fc_int8(a, w, bias, scale)
+    assert np.abs(ref_q).max() > 60  # the int8 range is used
+    deq = orc.dequantize(ref_q, s_out)
+    for r in (None, res):
+        got = host(ops().gemm_i8_dequant_residual(dev(a), dev(w), dev(bias), dev(scale), float(s_out),
+                                                  None if r is None else dev(r, tdt), tdt))
+        want = deq if r is None else (deq + r).astype(np.float32)
+        if dtype == "f16":
+            want = want.astype(np.float16).astype(np.float32)
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("B,S,heads,K", [(2, 64, 2, 128), (3, 40, 12, 768), (8, 384, 12, 768)])
+def test_gemm_i8_qkv_split_bit_exact(B, S, heads, K):
+    """Three quantised projections + their dequantising Reformat layers in one GEMM, written as Q|K rows and V^T."""
+    say("gemm_i8_qkv_split B=%d S=%d heads=%d K=%d" % (B, S, heads, K))
+    rng = np.random.default_rng(B * 7 + S + heads)
+    H, T = heads * 64, B * S
+    x = rng.integers(-128, 128, (T, K), dtype=np.int8)
+    w = rng.integers(-127, 128, (3 * H, K), dtype=np.int8)
+    bias = rng.integers(-20000, 20000, 3 * H).astype(np.int32)
+    w_scale = (rng.uniform(0.5, 1.5, 3 * H) * (2e-3 * 768 / K)).astype(np.float32)
+    s_out = np.array([0.41, 0.37, 0.29], np.float32)  # output blob scales of the q, k, v projections
+    scale = np.concatenate([orc.fc_int8_scale(w_scale[i * H:(i + 1) * H], s_out[i], H) for i in range(3)])
+    dequant = np.repeat(s_out, H).astype(np.float32)
+    qk, vt = ops().gemm_i8_qkv_split(dev(x), dev(w), dev(bias), dev(scale), dev(dequant), B, S, heads)
+    ref_q, _ = orc.fc_int8(x, w, bias, scale)
+    ref = (ref_q.astype(np.float32) * dequant[None, :]).astype(np.float16).astype(np.float32)
+    assert np.array_equal(host(qk), ref[:, :2 * H])
+    v_ref = ref[:, 2 * H:].reshape(B, S, heads, 64).transpose(0, 2, 3, 1)
+    assert np.array_equal(host(vt), v_ref)
+
+
 # ---- fused attention ------------------------------------------------------------------------------
 def _attn_case(B, h, S, lens, seed, dtype=torch.float16, with_mask=False):
     rng = np.random.default_rng(seed)

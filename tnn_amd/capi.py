@@ -41,6 +41,8 @@ SIGNATURES = {
     "tnn_rocm_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
     "tnn_rocm_gemm": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i],
     "tnn_rocm_gemm_i8": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _f],
+    "tnn_rocm_gemm_i8_dequant_residual": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _i, _f, _vp],
+    "tnn_rocm_gemm_i8_qkv_split": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i],
     "tnn_rocm_attention": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _l, _l, _l, _l, _l, _l, _l, _l, _l, _f,
                            _vp, _vp],
     "tnn_rocm_attention_vt": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _l, _l, _l, _l, _l, _l, _l, _l, _l, _l, _l,

@@ -201,6 +201,7 @@ struct Int8Epilogue {
     void *out_f;
     int out_f_dtype;
     float dq;
+    const void *residual;  // optional, type and leading dimension of out_f: out_f = q * dq + residual
     __device__ __forceinline__ void set_batch(int) {}
     struct ColConst {
         int32_t bias;
@@ -225,10 +226,15 @@ struct Int8Epilogue {
                 out[(size_t)m * ldo + n] = q;
             if (out_f) {
                 float d = __fmul_rn((float)q, dq);
-                if (out_f_dtype == TNN_ROCM_F32)
+                if (out_f_dtype == TNN_ROCM_F32) {
+                    if (residual)
+                        d = __fadd_rn(d, ((const float *)residual)[(size_t)m * ldo + n]);
                     ((float *)out_f)[(size_t)m * ldo + n] = d;
-                else
+                } else {
+                    if (residual)
+                        d = __fadd_rn(d, (float)((const half_t *)residual)[(size_t)m * ldo + n]);
                     ((half_t *)out_f)[(size_t)m * ldo + n] = (half_t)d;
+                }
             }
         }
     }
@@ -264,20 +270,99 @@ struct Int8Epilogue {
             if (out)
                 *reinterpret_cast<uint2 *>(out + o) = *reinterpret_cast<const uint2 *>(q);
             if (out_f) {
+                float d[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    d[t] = __fmul_rn((float)q[t], dq);
                 if (out_f_dtype == TNN_ROCM_F32) {
+                    if (residual) {
+                        const float4 *rp = reinterpret_cast<const float4 *>((const float *)residual + o);
+                        float4 r0 = rp[0], r1 = rp[1];
+                        d[0] = __fadd_rn(d[0], r0.x), d[1] = __fadd_rn(d[1], r0.y), d[2] = __fadd_rn(d[2], r0.z),
+                        d[3] = __fadd_rn(d[3], r0.w), d[4] = __fadd_rn(d[4], r1.x), d[5] = __fadd_rn(d[5], r1.y),
+                        d[6] = __fadd_rn(d[6], r1.z), d[7] = __fadd_rn(d[7], r1.w);
+                    }
                     float4 *fp = reinterpret_cast<float4 *>((float *)out_f + o);
-                    fp[0] = make_float4(__fmul_rn((float)q[0], dq), __fmul_rn((float)q[1], dq), __fmul_rn((float)q[2], dq),
-                                        __fmul_rn((float)q[3], dq));
-                    fp[1] = make_float4(__fmul_rn((float)q[4], dq), __fmul_rn((float)q[5], dq), __fmul_rn((float)q[6], dq),
-                                        __fmul_rn((float)q[7], dq));
+                    fp[0] = make_float4(d[0], d[1], d[2], d[3]);
+                    fp[1] = make_float4(d[4], d[5], d[6], d[7]);
                 } else {
                     half_t h[8];
+                    if (residual) {
+                        *reinterpret_cast<u32x4 *>(h) = *reinterpret_cast<const u32x4 *>((const half_t *)residual + o);
+#pragma unroll
+                        for (int t = 0; t < 8; ++t)
+                            d[t] = __fadd_rn(d[t], (float)h[t]);
+                    }
 #pragma unroll
                     for (int t = 0; t < 8; ++t)
-                        h[t] = (half_t)__fmul_rn((float)q[t], dq);
+                        h[t] = (half_t)d[t];
                     *reinterpret_cast<u32x4 *>((half_t *)out_f + o) = *reinterpret_cast<const u32x4 *>(h);
                 }
             }
+        }
+    }
+};
+
+// Quantised QKV projection for the attention layer: the int8 outputs of the three QuantizedInnerProduct layers are
+// formed in registers (requantisation with scale[n] = w_scale[n] / o_scale of the column's section) and written
+// already dequantised (q * dequant[n], the value the following Reformat layer produces) in the layout of
+// QkvSplitEpilogue: columns [0,2H) -> qk[T,2H]; columns [2H,3H) -> V^T[b][head][d][s].
+template <int DT> struct Int8QkvSplitEpilogue {
+    typedef typename Elem<DT>::type T;
+    const int32_t *bias;
+    const float *scale;
+    const float *dequant;
+    T *qk;
+    T *vt;
+    int H, S, heads;
+    __device__ __forceinline__ void set_batch(int) {}
+    struct ColConst {
+        int32_t bias;
+        float scale, dq;
+    };
+    __device__ __forceinline__ ColConst col_const(int n) const {
+        ColConst c;
+        c.bias  = bias ? bias[n] : 0;
+        c.scale = scale[n];
+        c.dq    = dequant[n];
+        return c;
+    }
+    __device__ __forceinline__ void store(int m, int n, int acc, const ColConst &cc) const {
+        int8_t q = float2int8_ref(__fmul_rn((float)(acc + cc.bias), cc.scale));
+        float v  = __fmul_rn((float)q, cc.dq);
+        if (n < 2 * H) {
+            Elem<DT>::st(&qk[(size_t)m * 2 * H + n], v);
+        } else {
+            int c = n - 2 * H, b = m / S, s = m - b * S;
+            Elem<DT>::st(&vt[(((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s], v);
+        }
+    }
+    __device__ __forceinline__ bool direct(int n0) const { return n0 >= 2 * H; }
+    __device__ __forceinline__ void store8(int m, int n, const int (&acc)[8]) const {
+        float v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            int a    = acc[t] + (bias ? bias[n + t] : 0);
+            int8_t q = float2int8_ref(__fmul_rn((float)a, scale[n + t]));
+            v[t]     = __fmul_rn((float)q, dequant[n + t]);
+        }
+        if (n < 2 * H) {
+            constexpr int NV = 8 * sizeof(T) / 16;
+            u32x4 packed[NV];
+            T *pe = reinterpret_cast<T *>(packed);
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                Elem<DT>::st(&pe[t], v[t]);
+            u32x4 *cp = reinterpret_cast<u32x4 *>(qk + (size_t)m * 2 * H + n);
+#pragma unroll
+            for (int q = 0; q < NV; ++q)
+                cp[q] = packed[q];
+        } else {
+            int c = n - 2 * H, b = m / S, s_ = m - b * S;
+            T *dst = vt + (((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s_;
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                Elem<DT>::st(dst + (size_t)t * S, v[t]);
         }
     }
 };
@@ -923,9 +1008,9 @@ int tnn_rocm_gemm(void *stream, int dtype, int b_is_nk, const void *A, const voi
 #undef TR_GEMM_DT
 }
 
-int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W, const int32_t *bias, const float *scale,
-                     int8_t *out_i8, int32_t *acc_i32, int M, int N, int K, int lda, int ldw, int ldo, void *out_f,
-                     int out_f_dtype, float dequant_scale) {
+static int gemm_i8_impl(void *stream, const int8_t *A, const int8_t *W, const int32_t *bias, const float *scale,
+                        int8_t *out_i8, int32_t *acc_i32, int M, int N, int K, int lda, int ldw, int ldo, void *out_f,
+                        int out_f_dtype, float dequant_scale, const void *residual) {
     TR_REQUIRE(M >= 0 && N >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_i8: negative size");
     if (M == 0 || N == 0)
         return 0;
@@ -936,6 +1021,7 @@ int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W, const int32
     TR_REQUIRE(lda >= K && ldw >= K && ldo >= N, TNN_ROCM_ESHAPE, "gemm_i8: leading dimension too small");
     TR_REQUIRE(!out_f || out_f_dtype == TNN_ROCM_F32 || out_f_dtype == TNN_ROCM_F16, TNN_ROCM_EDTYPE,
                "gemm_i8: dequantised output must be F32 or F16");
+    TR_REQUIRE(!residual || out_f, TNN_ROCM_EINVAL, "gemm_i8: a residual needs the dequantised output");
     bool aligned = al16(A) && al16(W) && lda % 16 == 0 && ldw % 16 == 0 && K % 16 == 0;
     Int8Epilogue epi;
     epi.bias        = bias;
@@ -946,12 +1032,65 @@ int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W, const int32
     epi.out_f       = out_f;
     epi.out_f_dtype = out_f_dtype;
     epi.dq          = dequant_scale;
+    epi.residual    = residual;
     bool vec_out = ldo % 8 == 0 && (!bias || al16(bias)) && (!scale || al16(scale)) &&
-                   (!out_i8 || (((uintptr_t)out_i8) & 7u) == 0) && (!acc_i32 || al16(acc_i32)) && (!out_f || al16(out_f));
+                   (!out_i8 || (((uintptr_t)out_i8) & 7u) == 0) && (!acc_i32 || al16(acc_i32)) && (!out_f || al16(out_f)) &&
+                   (!residual || al16(residual));
     if (aligned && vec_out && g_gemm_force_cfg >= 0 && K % 64 == 0)
         return launch_gemm_fast<TNN_ROCM_I8, Int8Epilogue>((hipStream_t)stream, A, W, M, N, K, lda, ldw, epi);
     return launch_gemm<TNN_ROCM_I8, Int8Epilogue>((hipStream_t)stream, true, aligned, A, W, M, N, K, lda, ldw, 1, 1, 1,
                                                   0, 0, epi);
+}
+
+int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W, const int32_t *bias, const float *scale,
+                     int8_t *out_i8, int32_t *acc_i32, int M, int N, int K, int lda, int ldw, int ldo, void *out_f,
+                     int out_f_dtype, float dequant_scale) {
+    return gemm_i8_impl(stream, A, W, bias, scale, out_i8, acc_i32, M, N, K, lda, ldw, ldo, out_f, out_f_dtype,
+                        dequant_scale, nullptr);
+}
+
+int tnn_rocm_gemm_i8_dequant_residual(void *stream, const int8_t *A, const int8_t *W, const int32_t *bias,
+                                      const float *scale, int M, int N, int K, int lda, int ldw, void *out_f,
+                                      int out_f_dtype, int ldo, float dequant_scale, const void *residual) {
+    TR_REQUIRE(out_f, TNN_ROCM_EINVAL, "gemm_i8_dequant_residual: null output");
+    return gemm_i8_impl(stream, A, W, bias, scale, nullptr, nullptr, M, N, K, lda, ldw, ldo, out_f, out_f_dtype,
+                        dequant_scale, residual);
+}
+
+int tnn_rocm_gemm_i8_qkv_split(void *stream, int out_dtype, const int8_t *x, const int8_t *wqkv, const int32_t *bias,
+                               const float *scale, const float *dequant, void *qk, void *vt, int B, int S, int heads,
+                               int K) {
+    TR_REQUIRE(B >= 0 && S >= 0 && heads >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_i8_qkv_split: negative size");
+    if (B == 0 || S == 0 || heads == 0)
+        return 0;
+    TR_REQUIRE(x && wqkv && scale && dequant && qk && vt, TNN_ROCM_EINVAL, "gemm_i8_qkv_split: null pointer");
+    TR_REQUIRE(out_dtype == TNN_ROCM_F16 || out_dtype == TNN_ROCM_BF16, TNN_ROCM_EDTYPE,
+               "gemm_i8_qkv_split: F16 or BF16 outputs only");
+    TR_REQUIRE(K > 0 && K % 64 == 0, TNN_ROCM_ESHAPE, "gemm_i8_qkv_split: K=%d must be a positive multiple of 64", K);
+    TR_REQUIRE((long)B * S < (1l << 24) && (long)B * S * 3 * heads * 64 < (1l << 31), TNN_ROCM_ESHAPE,
+               "gemm_i8_qkv_split: problem too large for 32-bit panel offsets");
+    TR_REQUIRE(al16(x) && al16(wqkv) && al16(qk) && al16(vt) && (!bias || al16(bias)) && al16(scale) && al16(dequant),
+               TNN_ROCM_EALIGN, "gemm_i8_qkv_split: pointers must be 16-byte aligned");
+    const int H = heads * 64, T = B * S;
+#define TR_QKV8(DT)                                                                                                   \
+    {                                                                                                                 \
+        Int8QkvSplitEpilogue<DT> epi;                                                                                 \
+        epi.bias    = bias;                                                                                           \
+        epi.scale   = scale;                                                                                          \
+        epi.dequant = dequant;                                                                                        \
+        epi.qk      = (Elem<DT>::type *)qk;                                                                           \
+        epi.vt      = (Elem<DT>::type *)vt;                                                                           \
+        epi.H       = H;                                                                                              \
+        epi.S       = S;                                                                                              \
+        epi.heads   = heads;                                                                                          \
+        return launch_gemm_fast<TNN_ROCM_I8, Int8QkvSplitEpilogue<DT>>((hipStream_t)stream, x, wqkv, T, 3 * H, K, K, K, \
+                                                                       epi);                                          \
+    }
+    if (out_dtype == TNN_ROCM_F16)
+        TR_QKV8(TNN_ROCM_F16)
+    else
+        TR_QKV8(TNN_ROCM_BF16)
+#undef TR_QKV8
 }
 
 int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *wqkv, const float *bqkv, void *qk,

@@ -59,6 +59,28 @@ def gemm_i8(a, w, bias, scale, want_acc=False, want_q=True, dequant_scale=None, 
     return q, acc, outf
 
 
+def gemm_i8_dequant_residual(a, w, bias, scale, dequant_scale, residual=None, dtype=torch.float32):
+    """float out = requantise(a w^T + bias) * dequant_scale (+ residual); a [M,K] int8, w [N,K] int8"""
+    _chk(a, w, bias, scale, residual)
+    M, K = a.shape
+    N = w.shape[0]
+    out = torch.empty(M, N, dtype=dtype, device=a.device)
+    capi.call("tnn_rocm_gemm_i8_dequant_residual", _stream(), _p(a), _p(w), _p(bias), _p(scale), M, N, K, K, K, _p(out),
+              _DT[dtype], N, float(dequant_scale), _p(residual))
+    return out
+
+
+def gemm_i8_qkv_split(x, wqkv, bias, scale, dequant, B, S, heads, dtype=torch.float16):
+    """x [B*S,K] int8, wqkv [3H,K] int8 -> (qk [B*S,2H], vt [B,heads,64,S]) dequantised"""
+    _chk(x, wqkv, bias, scale, dequant)
+    H = heads * 64
+    qk = torch.empty(B * S, 2 * H, dtype=dtype, device=x.device)
+    vt = torch.empty(B, heads, 64, S, dtype=dtype, device=x.device)
+    capi.call("tnn_rocm_gemm_i8_qkv_split", _stream(), _DT[dtype], _p(x), _p(wqkv), _p(bias), _p(scale), _p(dequant),
+              _p(qk), _p(vt), B, S, heads, x.shape[1])
+    return qk, vt
+
+
 def attention(q, k, v, scale, mask=None, kv_len=None, out=None):
     """q, k, v: [B, h, S, d] contiguous."""
     _chk(q, k, v, mask, kv_len)
