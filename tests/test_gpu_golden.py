@@ -116,3 +116,39 @@ def test_int8_encoder_against_reference_x86(precision):
     # one int8 step of a projection output is ~1/127 of its range, so a float difference upstream that flips a
     # rounding moves the result by more than the float bar; the bound below is two such steps on the final LayerNorm
     assert err <= (2e-2 if precision == "fp16" else 1e-2)
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_int8_encoder_with_folded_reformat_layers(precision, monkeypatch):
+    """The same int8 encoder without extra outputs, so that the ROCm int8 pass may fold every Reformat layer into its
+    neighbour (projection + dequantise + residual, LayerNorm + quantise, int8 GELU, quantised attention block):
+    in fp32 the result is bit-identical to the explicit chain, in fp16 it stays within the bar of the X86 fixture."""
+    from tnn_amd import host, quant
+    cfg, w, B, S, scales, f = golden_util.int8_encoder()
+    say("golden: int8 encoder, Reformat layers folded, " + precision)
+    g = quant.int8_encoder_graph(cfg, w, scales, B, S)
+    outs, types = {}, {}
+    for fuse in ("0", "1"):
+        monkeypatch.setenv("TNN_ROCM_FUSE_INT8", fuse)
+        inst = host.RocmInstance.from_graph(g, precision)
+        types[fuse] = [t for t, _ in inst.layers()]
+        inst.set_input("input_ids", f["ids"])
+        inst.set_input("token_type_ids", f["seg"])
+        inst.set_input("attention_bias", f["mask"].reshape(B, 1, 1, S))
+        inst.forward()
+        outs[fuse] = inst.output("last_hidden")
+        inst.close()
+    say("  explicit: " + " ".join("%s x%d" % (t, types["0"].count(t)) for t in sorted(set(types["0"]))))
+    say("  folded:   " + " ".join("%s x%d" % (t, types["1"].count(t)) for t in sorted(set(types["1"]))))
+    assert types["0"].count("Reformat") == 10 and types["0"].count("QuantizedInnerProduct") == 6
+    assert types["1"].count("RocmGeluInt8") == 1 and types["1"].count("QuantizedInnerProduct") == 1
+    assert types["1"].count("Reformat") == 2  # the encoder input and the attention output are still quantised apart
+    if precision == "fp16":
+        assert types["1"].count("RocmFusedAttention") == 1 and types["1"].count("RocmFusedLinearInt8") == 2
+    else:  # fp32 keeps the decomposed attention core; the q, k, v projections still fold their Reformat layers
+        assert types["1"].count("RocmFusedLinearInt8") == 5
+        assert np.array_equal(outs["0"], outs["1"])
+    ref = f["x86_last_hidden"].reshape(outs["1"].shape)
+    err = rel_err(outs["1"], ref)
+    say("  max rel err vs X86 %.3g (explicit chain %.3g)" % (err, rel_err(outs["0"], ref)))
+    assert err <= (2e-2 if precision == "fp16" else 1e-2)

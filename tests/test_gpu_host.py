@@ -89,7 +89,7 @@ def test_encoder_from_model_files(precision):
     inst.close()
 
 
-def test_int8_ffn_from_model_files_bit_exact():
+def test_int8_ffn_from_model_files_bit_exact(monkeypatch):
     host, tnnmodel, *_ = _mods()
     say("host: QuantizedInnerProduct -> GELU -> QuantizedInnerProduct, fp32 boundaries")
     rng = np.random.default_rng(0)
@@ -103,26 +103,34 @@ def test_int8_ffn_from_model_files_bit_exact():
     ws2 = (rng.uniform(0.5, 1.5, K) * 3e-5).astype(np.float32)
     s_a, s_h, s_g, s_y = (np.float32(v) for v in (0.031, 0.045, 0.027, 0.052))
     g = tnnmodel.int8_ffn_graph(T, K, F, w1, b1, ws1, w2, b2, ws2, s_a, s_h, s_g, s_y)
-    inst = host.RocmInstance.from_graph(g, "fp32")
-    types = [t for t, _ in inst.layers()]
-    assert types.count("Reformat") == 4 and types.count("QuantizedInnerProduct") == 2, types
-    inst.set_input("x", x)
-    inst.forward()
-    got = inst.output("y")
     qa = orc.quantize_x86(x, s_a)
     h, _ = orc.fc_int8(qa, w1, b1, orc.fc_int8_scale(ws1, s_h, F))
     ref_act = orc.gelu(orc.dequantize(h, s_h))
     gq = orc.quantize_x86(ref_act, s_g)
     yq, _ = orc.fc_int8(gq, w2, b2, orc.fc_int8_scale(ws2, s_y, K))
-    ref = orc.dequantize(yq, s_y)
-    # the two int8 GEMMs and both quantisers are bit-exact; the fp32 GELU between them uses the device erff
-    # (last-ulp differences against the CPU's double erf), which can move a value across a rounding boundary of the
-    # second quantiser in rare cases: allow at most 1 LSB on at most 0.1 % of the outputs
-    diff = np.abs(np.rint(got / s_y) - yq.astype(np.float64))
-    say("  mismatching int8 outputs: %d of %d" % (int((diff != 0).sum()), diff.size))
-    assert diff.max() <= 1 and (diff != 0).mean() <= 1e-3
     assert np.abs(h).max() > 20  # the requantisation really exercised the int8 range
-    inst.close()
+    outs = {}
+    # once as the explicit chain (Reformat layers as the engine inserts them), once with the Reformat layers folded
+    # into their neighbours by the ROCm int8 pass
+    for fuse, want in (("0", {"Reformat": 4, "QuantizedInnerProduct": 2}),
+                       ("1", {"Reformat": 1, "QuantizedInnerProduct": 1, "RocmGeluInt8": 1, "RocmFusedLinearInt8": 1})):
+        monkeypatch.setenv("TNN_ROCM_FUSE_INT8", fuse)
+        inst = host.RocmInstance.from_graph(g, "fp32")
+        types = [t for t, _ in inst.layers()]
+        for k, n in want.items():
+            assert types.count(k) == n, types
+        inst.set_input("x", x)
+        inst.forward()
+        got = inst.output("y")
+        inst.close()
+        # the two int8 GEMMs and both quantisers are bit-exact; the fp32 GELU between them uses the device erff
+        # (last-ulp differences against the CPU's double erf), which can move a value across a rounding boundary of
+        # the second quantiser in rare cases: allow at most 1 LSB on at most 0.1 % of the outputs
+        diff = np.abs(np.rint(got / s_y) - yq.astype(np.float64))
+        say("  fuse=%s mismatching int8 outputs: %d of %d" % (fuse, int((diff != 0).sum()), diff.size))
+        assert diff.max() <= 1 and (diff != 0).mean() <= 1e-3
+        outs[fuse] = got
+    assert np.array_equal(outs["0"], outs["1"])  # folding the Reformat layers changes no value in fp32
 
 
 def test_host_error_paths():

@@ -101,6 +101,7 @@ LayerType GlobalConvertLayerType(std::string s) {
         {"LayerNorm", LAYER_LAYER_NORM},      {"GELU", LAYER_GELU},
         {"BlobScale", LAYER_BLOB_SCALE},      {"QuantizedAdd", LAYER_ADD},
         {"RocmFusedLinear", LAYER_ROCM_FUSED_LINEAR}, {"RocmFusedAttention", LAYER_ROCM_FUSED_ATTENTION},
+        {"RocmFusedLinearInt8", LAYER_ROCM_FUSED_LINEAR_INT8}, {"RocmGeluInt8", LAYER_ROCM_GELU_INT8},
     };
     auto it = m.find(s);
     return it == m.end() ? LAYER_NOT_SUPPORT : it->second;
@@ -751,6 +752,19 @@ struct LayerNormLayer : BaseLayer {  // layer/layer_norm_layer.cc:25-35
             return Status(TNNERR_PARAM_ERR, "LayerNormLayer has no input blob of scale or bias");
         return BaseLayer::InferOutputShape();
     }
+    // a second output (added by the ROCm int8 pass) is the quantised copy of the first and stays int8
+    Status InferOutputDataType() override {
+        output_blobs_[0]->GetBlobDesc().data_type = input_blobs_[0]->GetBlobDesc().data_type;
+        return TNN_OK;
+    }
+};
+
+// Layers of the ROCm int8 pass that read an int8 blob and write a float one (or the other way round): the network
+// sets each blob's type before Init (int8 blobs are BlobInt8, float blobs carry the network's float type), so the
+// default rule "outputs take the type of input 0" must not run.
+template <typename Base> struct MixedTypeLayer : Base {
+    using Base::Base;
+    Status InferOutputDataType() override { return TNN_OK; }
 };
 
 struct GatherLayer : BaseLayer {  // layer/gather_layer.cc
@@ -853,9 +867,11 @@ BaseLayer *CreateLayer(LayerType type) {
         case LAYER_CAST: return new CastLayer(type);
         case LAYER_REFORMAT: return new ReformatLayer(type);
         case LAYER_ROCM_FUSED_LINEAR: return new FusedLinearLayer(type);
+        case LAYER_ROCM_FUSED_LINEAR_INT8: return new MixedTypeLayer<InnerProductLayer>(type);
+        case LAYER_ROCM_FUSED_ATTENTION: return new MixedTypeLayer<BaseLayer>(type);
         case LAYER_SOFTMAX:
         case LAYER_GELU:
-        case LAYER_ROCM_FUSED_ATTENTION: return new BaseLayer(type);
+        case LAYER_ROCM_GELU_INT8: return new BaseLayer(type);
         default: return nullptr;
     }
 }
@@ -1065,22 +1081,30 @@ Status DefaultNetwork::InitLayers() {
         layers_.push_back(layer);
         auto param = info->param.get();
         std::vector<Blob *> ins, outs;
-        auto want_int8 = [&](bool is_input) -> bool {  // default_network.cc:362-440
+        auto want_int8 = [&](bool is_input, size_t idx) -> bool {  // default_network.cc:362-440
             if (!quantized_net)
                 return false;
             if (info->type == LAYER_REFORMAT) {
                 auto rp = dynamic_cast<ReformatLayerParam *>(param);
                 return is_input ? rp->src_type == DATA_TYPE_INT8 : rp->dst_type == DATA_TYPE_INT8;
             }
+            // layers written by the ROCm int8 pass with blobs of both kinds
+            if (info->type == LAYER_ROCM_FUSED_LINEAR_INT8)
+                return is_input && idx == 0;
+            if (info->type == LAYER_ROCM_FUSED_ATTENTION)
+                return is_input && idx == 0 && dynamic_cast<RocmFusedAttentionParam *>(param)->quant;
+            if (info->type == LAYER_LAYER_NORM)
+                return !is_input && idx == 1;
             return param->quantized;
         };
-        for (auto &name : info->inputs) {
+        for (size_t i = 0; i < info->inputs.size(); ++i) {
+            const auto &name = info->inputs[i];
             if (!blobs_.count(name))
                 return Status(TNNERR_NET_ERR, "layer " + info->name + " reads blob " + name + " before it is produced");
-            ins.push_back(make_blob(name, want_int8(true)));
+            ins.push_back(make_blob(name, want_int8(true, i)));
         }
-        for (auto &name : info->outputs)
-            outs.push_back(make_blob(name, want_int8(false)));
+        for (size_t i = 0; i < info->outputs.size(); ++i)
+            outs.push_back(make_blob(info->outputs[i], want_int8(false, i)));
         for (auto blobs : {&ins, &outs})
             for (auto b : *blobs)
                 if (auto bi = dynamic_cast<BlobInt8 *>(b)) {
@@ -1094,8 +1118,9 @@ Status DefaultNetwork::InitLayers() {
                                                              b->GetBlobDesc().name + "_scale_data_");
                     bi->SetIntResource(r);
                 }
-        // float outputs of a dequantising Reformat follow the network precision
-        if (info->type == LAYER_REFORMAT)
+        // float outputs of a dequantising Reformat (or of a fused layer that contains one) follow the network precision
+        if (info->type == LAYER_REFORMAT || info->type == LAYER_ROCM_FUSED_LINEAR_INT8 ||
+            info->type == LAYER_ROCM_FUSED_ATTENTION)
             for (auto b : outs)
                 if (!dynamic_cast<BlobInt8 *>(b))
                     b->GetBlobDesc().data_type = half ? DATA_TYPE_HALF : DATA_TYPE_FLOAT;

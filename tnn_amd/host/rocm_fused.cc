@@ -12,7 +12,9 @@
 // so that a BERT layer becomes 7 launches.  A sub-graph is only rewritten when every intermediate blob has a
 // single reader and is not a model output; anything that does not match is left as it is.
 #include <algorithm>
+#include <cfloat>
 #include <cmath>
+#include <cstdlib>
 
 #include "rocm_device.h"
 
@@ -390,8 +392,365 @@ private:
     bool half_               = true;
 };
 
+// ---- quantised nets -----------------------------------------------------------------------------------------------
+// Runs after the engine's own pass has made every float <-> int8 boundary an explicit Reformat layer
+// (net_optimizer_insert_int8_reformat.cc:66-181).  A quantised encoder layer is then
+//   Reformat(x) -> 3 x QuantizedInnerProduct -> 3 x Reformat -> head split, scores, softmax, P.V, head merge ->
+//   Reformat -> QuantizedInnerProduct -> Reformat -> Add(residual) -> LayerNorm -> Reformat -> QuantizedInnerProduct
+//   -> Reformat -> GELU -> Reformat -> QuantizedInnerProduct -> Reformat -> Add(residual) -> LayerNorm
+// and this pass folds the Reformat layers into their neighbours, value for value:
+//   * the three projections + their dequantising Reformats + the attention core  ==> RocmFusedAttention (quant)
+//   * QuantizedInnerProduct -> Reformat(int8->float) [-> Add(residual)]            ==> RocmFusedLinearInt8
+//   * Reformat(int8->float) -> GELU -> Reformat(float->int8)                       ==> RocmGeluInt8
+//   * LayerNorm -> Reformat(float->int8)                                           ==> LayerNorm with a second, int8 output
+// Each fused kernel forms the same int8 values as the chain it replaces (requantisation and quantisation are the
+// reference's float2int8 steps); float intermediates that the chain would have rounded to the blob type (fp16 nets)
+// stay in fp32 inside the fused kernel.
+class RocmInt8FusionPass : public NetOptimizer {
+public:
+    std::string Strategy() override { return "net_optimizer_rocm_fuse_int8"; }
+    bool IsSupported(const NetworkConfig &c) override {
+        half_ = c.precision != PRECISION_HIGH;
+        const char *e = getenv("TNN_ROCM_FUSE_INT8");  // "0" keeps the explicit Reformat chain (used by the tests)
+        return c.device_type == DEVICE_ROCM && !(e && atoi(e) == 0);
+    }
+    Status Optimize(NetStructure *s, NetResource *r) override {
+        structure_ = s;
+        resource_  = r;
+        bool any_q = false;
+        for (auto &l : s->layers)
+            any_q |= l->param->quantized;
+        if (!any_q)
+            return TNN_OK;
+        if (half_)
+            FuseAttention();
+        FoldGelu();
+        FoldDequant();
+        FoldLayerNormQuant();
+        return TNN_OK;
+    }
+
+private:
+    bool IsModelOutput(const std::string &b) const { return structure_->outputs.count(b) > 0; }
+    void Compact() {
+        auto &L = structure_->layers;
+        L.erase(std::remove(L.begin(), L.end(), nullptr), L.end());
+    }
+    template <typename T> T *ParamOf(const std::shared_ptr<LayerInfo> &l) { return dynamic_cast<T *>(l->param.get()); }
+    template <typename T> T *ResOf(const std::string &name) {
+        auto it = resource_->resource_map.find(name);
+        return it == resource_->resource_map.end() ? nullptr : dynamic_cast<T *>(it->second.get());
+    }
+    bool BlobScale(const std::string &blob, float *scale) {
+        auto r = ResOf<IntScaleResource>(blob + "_scale_data_");
+        if (!r || r->scale_handle.GetDataCount() != 1 || r->scale_handle.GetDataType() != DATA_TYPE_FLOAT)
+            return false;
+        *scale = r->scale_handle.force_to<float *>()[0];
+        return true;
+    }
+    // single-input, single-output Reformat in the given direction
+    bool IsReformat(const std::shared_ptr<LayerInfo> &l, bool to_int8) {
+        if (!l || l->type != LAYER_REFORMAT || l->inputs.size() != 1 || l->outputs.size() != 1)
+            return false;
+        auto p = ParamOf<ReformatLayerParam>(l);
+        return p && (to_int8 ? (p->src_type != DATA_TYPE_INT8 && p->dst_type == DATA_TYPE_INT8)
+                             : (p->src_type == DATA_TYPE_INT8 && p->dst_type != DATA_TYPE_INT8));
+    }
+    bool IsQuantFc(const std::shared_ptr<LayerInfo> &l) {
+        if (!l || l->type != LAYER_INNER_PRODUCT || !l->param->quantized || l->inputs.size() != 1)
+            return false;
+        auto ip = ParamOf<InnerProductLayerParam>(l);
+        auto ir = ResOf<InnerProductLayerResource>(l->name);
+        return ip && ir && ip->axis == 1 && ir->weight_handle.GetDataType() == DATA_TYPE_INT8 && ip->num_output > 0 &&
+               ir->weight_handle.GetDataCount() % ip->num_output == 0 &&
+               (ir->scale_handle.GetDataCount() == ip->num_output || ir->scale_handle.GetDataCount() == 1);
+    }
+
+    // `blob` <- Permute(order) <- Reshape(head split) <- Reformat(int8->float) <- QuantizedInnerProduct
+    int QuantHeadSplitSource(const GraphIndex &g, const std::string &blob, const std::vector<int> &order4,
+                             const std::vector<int> &order3, std::vector<int> *chain, DimsVector *split_shape) {
+        auto &L = structure_->layers;
+        int pi  = g.producer_of(blob);
+        if (pi < 0 || !L[pi] || L[pi]->type != LAYER_PERMUTE || g.sole_consumer(blob) < 0 || IsModelOutput(blob))
+            return -1;
+        auto pp = ParamOf<PermuteLayerParam>(L[pi]);
+        if (!pp || (pp->orders != order4 && pp->orders != order3))
+            return -1;
+        const std::string &rb = L[pi]->inputs[0];
+        int ri                = g.producer_of(rb);
+        if (ri < 0 || !L[ri] || L[ri]->type != LAYER_RESHAPE || g.sole_consumer(rb) != pi || IsModelOutput(rb))
+            return -1;
+        auto rp = ParamOf<ReshapeLayerParam>(L[ri]);
+        if (!rp || rp->axis != 0 || rp->shape.size() != pp->orders.size() || L[ri]->inputs.size() != 1)
+            return -1;
+        const std::string &fb = L[ri]->inputs[0];
+        int fi                = g.producer_of(fb);
+        if (fi < 0 || !IsReformat(L[fi], false) || g.sole_consumer(fb) != ri || IsModelOutput(fb))
+            return -1;
+        const std::string &qb = L[fi]->inputs[0];
+        int li                = g.producer_of(qb);
+        if (li < 0 || !IsQuantFc(L[li]) || g.sole_consumer(qb) != fi || IsModelOutput(qb))
+            return -1;
+        chain->push_back(pi);
+        chain->push_back(ri);
+        chain->push_back(fi);
+        chain->push_back(li);
+        *split_shape = rp->shape;
+        return li;
+    }
+
+    void FuseAttention() {
+        auto &L = structure_->layers;
+        bool changed = true;
+        while (changed) {
+            changed = false;
+            GraphIndex g(L);
+            for (int si = 0; si < (int)L.size() && !changed; ++si) {
+                auto sm = L[si];
+                if (!sm || sm->type != LAYER_SOFTMAX)
+                    continue;
+                std::vector<int> chain = {si};
+                std::string cur = sm->inputs[0], mask;
+                float scale = 1.0f;
+                bool have_scale = false;
+                int qk = -1;
+                for (int step = 0; step < 3 && qk < 0; ++step) {
+                    int pi = g.producer_of(cur);
+                    if (pi < 0 || !L[pi] || g.sole_consumer(cur) < 0 || IsModelOutput(cur))
+                        break;
+                    auto pl = L[pi];
+                    if (pl->type == LAYER_ADD && pl->inputs.size() == 2 && mask.empty() && !have_scale) {
+                        int p0 = g.producer_of(pl->inputs[0]);
+                        bool first_is_scores = p0 >= 0 && L[p0] &&
+                                               (L[p0]->type == LAYER_MUL || L[p0]->type == LAYER_DIV || L[p0]->type == LAYER_MATMUL);
+                        mask = first_is_scores ? pl->inputs[1] : pl->inputs[0];
+                        cur  = first_is_scores ? pl->inputs[0] : pl->inputs[1];
+                        chain.push_back(pi);
+                    } else if ((pl->type == LAYER_MUL || pl->type == LAYER_DIV) && pl->inputs.size() == 1 && !have_scale) {
+                        auto er = ResOf<EltwiseLayerResource>(pl->name);
+                        if (!er || er->element_handle.GetDataCount() != 1 || er->element_handle.GetDataType() != DATA_TYPE_FLOAT)
+                            break;
+                        float v    = er->element_handle.force_to<float *>()[0];
+                        scale      = pl->type == LAYER_MUL ? v : 1.0f / v;
+                        have_scale = true;
+                        cur        = pl->inputs[0];
+                        chain.push_back(pi);
+                    } else if (pl->type == LAYER_MATMUL && pl->inputs.size() == 2) {
+                        qk = pi;
+                        chain.push_back(pi);
+                    } else {
+                        break;
+                    }
+                }
+                if (qk < 0)
+                    continue;
+                DimsVector shape_q, shape_k, shape_v;
+                int lq = QuantHeadSplitSource(g, L[qk]->inputs[0], {0, 2, 1, 3}, {1, 0, 2}, &chain, &shape_q);
+                int lk = QuantHeadSplitSource(g, L[qk]->inputs[1], {0, 2, 3, 1}, {1, 2, 0}, &chain, &shape_k);
+                if (lq < 0 || lk < 0)
+                    continue;
+                int pv = g.sole_consumer(sm->outputs[0]);
+                if (pv < 0 || !L[pv] || L[pv]->type != LAYER_MATMUL || L[pv]->inputs.size() != 2 ||
+                    L[pv]->inputs[0] != sm->outputs[0] || IsModelOutput(sm->outputs[0]))
+                    continue;
+                chain.push_back(pv);
+                int lv = QuantHeadSplitSource(g, L[pv]->inputs[1], {0, 2, 1, 3}, {1, 0, 2}, &chain, &shape_v);
+                if (lv < 0 || shape_q != shape_k || shape_q != shape_v)
+                    continue;
+                int pm = g.sole_consumer(L[pv]->outputs[0]);
+                if (pm < 0 || !L[pm] || L[pm]->type != LAYER_PERMUTE || IsModelOutput(L[pv]->outputs[0]))
+                    continue;
+                auto pmp = ParamOf<PermuteLayerParam>(L[pm]);
+                if (!pmp || (pmp->orders != std::vector<int>{0, 2, 1, 3} && pmp->orders != std::vector<int>{1, 0, 2}))
+                    continue;
+                int rs = g.sole_consumer(L[pm]->outputs[0]);
+                if (rs < 0 || !L[rs] || L[rs]->type != LAYER_RESHAPE || IsModelOutput(L[pm]->outputs[0]))
+                    continue;
+                chain.push_back(pm);
+                chain.push_back(rs);
+                // the three projections read the same int8 blob and have the same shape
+                if (L[lq]->inputs[0] != L[lk]->inputs[0] || L[lq]->inputs[0] != L[lv]->inputs[0])
+                    continue;
+                InnerProductLayerResource *src[3] = {ResOf<InnerProductLayerResource>(L[lq]->name),
+                                                     ResOf<InnerProductLayerResource>(L[lk]->name),
+                                                     ResOf<InnerProductLayerResource>(L[lv]->name)};
+                int H = ParamOf<InnerProductLayerParam>(L[lq])->num_output;
+                if (ParamOf<InnerProductLayerParam>(L[lk])->num_output != H || ParamOf<InnerProductLayerParam>(L[lv])->num_output != H)
+                    continue;
+                int K = src[0]->weight_handle.GetDataCount() / H;
+                if (src[1]->weight_handle.GetDataCount() != H * K || src[2]->weight_handle.GetDataCount() != H * K)
+                    continue;
+                int heads = shape_q[shape_q.size() - 2], head_dim = shape_q.back(), seq = shape_q[shape_q.size() - 3];
+                if (heads * head_dim != H || head_dim != 64 || seq <= 0 || seq % 8 != 0 || K % 64 != 0)
+                    continue;
+                float out_scale[3];
+                if (!BlobScale(L[lq]->outputs[0], &out_scale[0]) || !BlobScale(L[lk]->outputs[0], &out_scale[1]) ||
+                    !BlobScale(L[lv]->outputs[0], &out_scale[2]))
+                    continue;
+                int first = *std::min_element(chain.begin(), chain.end());
+                if (!mask.empty()) {
+                    int pmask = g.producer_of(mask);
+                    bool ok   = pmask >= 0 ? pmask < first : structure_->inputs_shape_map.count(mask) > 0 ||
+                                                                 resource_->constant_map.count(mask) > 0;
+                    if (!ok)
+                        continue;
+                }
+                auto fl      = std::make_shared<LayerInfo>();
+                fl->type     = LAYER_ROCM_FUSED_ATTENTION;
+                fl->type_str = "RocmFusedAttention";
+                fl->name     = sm->name + "_fused_attention_int8";
+                fl->inputs   = {L[lq]->inputs[0]};
+                if (!mask.empty())
+                    fl->inputs.push_back(mask);
+                fl->outputs  = {L[rs]->outputs[0]};
+                auto fp      = std::make_shared<RocmFusedAttentionParam>();
+                fp->type     = fl->type_str;
+                fp->name     = fl->name;
+                fp->heads    = heads;
+                fp->head_dim = head_dim;
+                fp->scale    = scale;
+                fp->has_mask = mask.empty() ? 0 : 1;
+                fp->seq_len  = seq;
+                fp->quant    = 1;
+                for (int t = 0; t < 3; ++t)
+                    fp->qkv_out_scale[t] = out_scale[t];
+                fl->param    = fp;
+                auto fr      = std::make_shared<RocmFusedQkvInt8Resource>();
+                fr->name     = fl->name;
+                fr->weight   = RawBuffer(3 * H * K, {3 * H, K});
+                fr->weight.SetDataType(DATA_TYPE_INT8);
+                fr->bias     = RawBuffer(3 * H * 4, {3 * H});
+                fr->bias.SetDataType(DATA_TYPE_INT32);
+                fr->w_scale  = RawBuffer(3 * H * 4, {3 * H});
+                memset(fr->bias.force_to<void *>(), 0, (size_t)3 * H * 4);
+                for (int t = 0; t < 3; ++t) {
+                    memcpy(fr->weight.force_to<int8_t *>() + (size_t)t * H * K, src[t]->weight_handle.force_to<int8_t *>(),
+                           (size_t)H * K);
+                    if (src[t]->bias_handle.GetDataCount() == H)
+                        memcpy(fr->bias.force_to<int32_t *>() + (size_t)t * H, src[t]->bias_handle.force_to<int32_t *>(),
+                               (size_t)H * 4);
+                    const float *ws = src[t]->scale_handle.force_to<float *>();
+                    int n_ws        = src[t]->scale_handle.GetDataCount();
+                    for (int i = 0; i < H; ++i)
+                        fr->w_scale.force_to<float *>()[(size_t)t * H + i] = ws[n_ws == 1 ? 0 : i];
+                }
+                resource_->resource_map[fl->name] = fr;
+                for (int idx : chain)
+                    L[idx] = nullptr;
+                L[first] = fl;
+                changed  = true;
+            }
+            Compact();
+        }
+    }
+
+    // int8 h -> Reformat(int8->float) -> GELU -> Reformat(float->int8) -> int8 g    ==>   RocmGeluInt8(h) -> g
+    void FoldGelu() {
+        auto &L = structure_->layers;
+        GraphIndex g(L);
+        for (int i = 0; i < (int)L.size(); ++i) {
+            if (!IsReformat(L[i], false) || IsModelOutput(L[i]->outputs[0]))
+                continue;
+            int gi = g.sole_consumer(L[i]->outputs[0]);
+            if (gi < 0 || !L[gi] || L[gi]->type != LAYER_GELU || IsModelOutput(L[gi]->outputs[0]))
+                continue;
+            int ri = g.sole_consumer(L[gi]->outputs[0]);
+            if (ri < 0 || !IsReformat(L[ri], true))
+                continue;
+            auto nl      = std::make_shared<LayerInfo>();
+            nl->type     = LAYER_ROCM_GELU_INT8;
+            nl->type_str = "RocmGeluInt8";
+            nl->name     = L[gi]->name + "_int8";
+            nl->inputs   = {L[i]->inputs[0]};
+            nl->outputs  = {L[ri]->outputs[0]};
+            auto p       = std::make_shared<LayerParam>();
+            p->type      = nl->type_str;
+            p->name      = nl->name;
+            p->quantized = true;
+            nl->param    = p;
+            L[i]  = nl;
+            L[gi] = nullptr;
+            L[ri] = nullptr;
+        }
+        Compact();
+    }
+
+    // QuantizedInnerProduct -> int8 y -> Reformat(int8->float) [-> Add(other)]   ==>   RocmFusedLinearInt8
+    void FoldDequant() {
+        auto &L = structure_->layers;
+        GraphIndex g(L);
+        for (int i = 0; i < (int)L.size(); ++i) {
+            if (!IsQuantFc(L[i]) || IsModelOutput(L[i]->outputs[0]))
+                continue;
+            int ri = g.sole_consumer(L[i]->outputs[0]);
+            if (ri < 0 || !IsReformat(L[ri], false))
+                continue;
+            float out_scale;
+            if (!BlobScale(L[i]->outputs[0], &out_scale))
+                continue;
+            auto ip      = ParamOf<InnerProductLayerParam>(L[i]);
+            auto np      = std::make_shared<RocmFusedLinearInt8Param>();
+            static_cast<InnerProductLayerParam &>(*np) = *ip;
+            np->type      = "RocmFusedLinearInt8";
+            np->quantized = true;
+            np->out_scale = out_scale;
+            auto nl       = std::make_shared<LayerInfo>(*L[i]);  // keeps the name: the resource is looked up by it
+            nl->type      = LAYER_ROCM_FUSED_LINEAR_INT8;
+            nl->type_str  = "RocmFusedLinearInt8";
+            nl->param     = np;
+            nl->outputs   = {L[ri]->outputs[0]};
+            // residual: the dequantised value's only reader is a float two-input Add whose other operand exists already
+            const std::string &y = L[ri]->outputs[0];
+            int ai               = g.sole_consumer(y);
+            if (ai > ri && L[ai] && L[ai]->type == LAYER_ADD && L[ai]->inputs.size() == 2 && !L[ai]->param->quantized &&
+                !ResOf<EltwiseLayerResource>(L[ai]->name) && !IsModelOutput(y)) {
+                const std::string &other = L[ai]->inputs[0] == y ? L[ai]->inputs[1] : L[ai]->inputs[0];
+                int po = g.producer_of(other);
+                bool available = other != y && (po >= 0 ? po < i : structure_->inputs_shape_map.count(other) > 0);
+                if (available) {
+                    np->has_residual = 1;
+                    nl->inputs.push_back(other);
+                    nl->outputs = {L[ai]->outputs[0]};
+                    L[ai]       = nullptr;
+                }
+            }
+            L[i]  = nl;
+            L[ri] = nullptr;
+        }
+        Compact();
+    }
+
+    // LayerNorm -> float x -> Reformat(float->int8) -> int8 xq   ==>   LayerNorm with outputs {x, xq}
+    void FoldLayerNormQuant() {
+        auto &L = structure_->layers;
+        GraphIndex g(L);
+        for (int i = 0; i < (int)L.size(); ++i) {
+            if (!L[i] || L[i]->type != LAYER_LAYER_NORM || L[i]->outputs.size() != 1)
+                continue;
+            auto it = g.consumers.find(L[i]->outputs[0]);
+            if (it == g.consumers.end())
+                continue;
+            for (int ri : it->second) {
+                if (ri > i && IsReformat(L[ri], true)) {
+                    L[i]->outputs.push_back(L[ri]->outputs[0]);
+                    L[ri] = nullptr;
+                    break;
+                }
+            }
+        }
+        Compact();
+    }
+
+    NetStructure *structure_ = nullptr;
+    NetResource *resource_   = nullptr;
+    bool half_               = true;
+};
+
 struct RegisterRocmFusion {
-    RegisterRocmFusion() { RegisterNetOptimizer(1, std::make_shared<RocmFusionPass>()); }
+    RegisterRocmFusion() {
+        RegisterNetOptimizer(1, std::make_shared<RocmFusionPass>());
+        RegisterNetOptimizer(3, std::make_shared<RocmInt8FusionPass>());  // after the Reformat insertion (2)
+    }
 } g_register_rocm_fusion;
 
 }  // namespace
@@ -453,18 +812,29 @@ REGISTER_ROCM_ACC(RocmFusedLinearLayerAcc, LAYER_ROCM_FUSED_LINEAR);
 class RocmFusedAttentionLayerAcc : public RocmLayerAcc {
 public:
     Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
-        auto res = dynamic_cast<RocmFusedLinearResource *>(resource_);
-        auto p   = dynamic_cast<RocmFusedAttentionParam *>(param_);
-        CHECK_PARAM_NULL(res);
+        auto res  = dynamic_cast<RocmFusedLinearResource *>(resource_);
+        auto res8 = dynamic_cast<RocmFusedQkvInt8Resource *>(resource_);
+        auto p    = dynamic_cast<RocmFusedAttentionParam *>(param_);
         CHECK_PARAM_NULL(p);
+        if (p->quant ? !res8 : !res)
+            return Status(TNNERR_NULL_PARAM, "fused attention: resource is nil");
         auto in = inputs[0]->GetBlobDesc().dims;
         H_      = p->heads * p->head_dim;
-        if (in.empty() || in.back() != H_ || res->weight_nk.GetBufferDims() != DimsVector({3 * H_, H_}))
-            return Status(TNNERR_PARAM_ERR, "fused attention: hidden size mismatch");
-        DataType dt = inputs[0]->GetBlobDesc().data_type;
+        DataType dt = outputs[0]->GetBlobDesc().data_type;
         if (dt != DATA_TYPE_HALF && dt != DATA_TYPE_BFP16)
             return Status(TNNERR_LAYER_ERR, "fused attention runs in fp16/bf16 only");
-        T_   = DimsVectorUtils::Count(in) / H_;
+        if (p->quant) {
+            auto wd = res8->weight.GetBufferDims();
+            if (in.empty() || wd.size() != 2 || wd[0] != 3 * H_ || in.back() != wd[1] ||
+                inputs[0]->GetBlobDesc().data_type != DATA_TYPE_INT8)
+                return Status(TNNERR_PARAM_ERR, "fused int8 attention: input / weight shape mismatch");
+            K_ = wd[1];
+        } else {
+            if (in.empty() || in.back() != H_ || res->weight_nk.GetBufferDims() != DimsVector({3 * H_, H_}))
+                return Status(TNNERR_PARAM_ERR, "fused attention: hidden size mismatch");
+            K_ = H_;
+        }
+        T_   = DimsVectorUtils::Count(in) / K_;
         seq_ = p->seq_len > 0 ? p->seq_len : (in.size() >= 3 ? in[in.size() - 2] : T_);
         if (seq_ <= 0 || T_ % seq_ != 0)
             return Status(TNNERR_PARAM_ERR, "fused attention: token count is not a multiple of the sequence length");
@@ -472,6 +842,23 @@ public:
         if (p->has_mask) {
             if (inputs.size() < 2 || DimsVectorUtils::Count(In(inputs[1])->GetBlobDesc().dims) != B_ * seq_)
                 return Status(TNNERR_PARAM_ERR, "fused attention: mask must hold B*S additive values");
+        }
+        if (!weight_ && p->quant) {
+            // requantisation factor w_scale / o_scale of each projection as one fp32 division on the host, 0 when
+            // o_scale < FLT_MIN (x86_inner_product_layer_acc.cc:197-222); dequantisation = the projection's blob scale
+            const int N = 3 * H_;
+            std::vector<float> scale(N), dequant(N);
+            const float *ws = res8->w_scale.force_to<float *>();
+            for (int i = 0; i < N; ++i) {
+                float os   = p->qkv_out_scale[i / H_];
+                scale[i]   = os >= FLT_MIN ? ws[i] / os : 0.0f;
+                dequant[i] = os;
+            }
+            RETURN_ON_NEQ(UploadConverted(res8->weight.force_to<void *>(), (size_t)N * K_, DATA_TYPE_INT8, DATA_TYPE_INT8, &weight_),
+                          TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(res8->bias.force_to<void *>(), (size_t)N, DATA_TYPE_INT32, DATA_TYPE_INT32, &bias_), TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(scale.data(), (size_t)N, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &scale_), TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(dequant.data(), (size_t)N, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &dequant_), TNN_OK);
         }
         if (!weight_) {
             RETURN_ON_NEQ(UploadConverted(res->weight_nk.force_to<void *>(), (size_t)3 * H_ * H_, DATA_TYPE_FLOAT, dt, &weight_),
@@ -484,7 +871,7 @@ public:
 
     Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
         auto p      = dynamic_cast<RocmFusedAttentionParam *>(param_);
-        DataType dt = inputs[0]->GetBlobDesc().data_type;
+        DataType dt = outputs[0]->GetBlobDesc().data_type;
         size_t es   = (size_t)DataTypeUtils::GetBytesSize(dt);
         void *qkv   = nullptr;
         RETURN_ON_NEQ(context_->Workspace((size_t)T_ * 3 * H_ * es, &qkv), TNN_OK);
@@ -496,6 +883,19 @@ public:
         }
         const char *base = (const char *)qkv;
         const long d     = p->head_dim;
+        if (p->quant) {
+            // int8 projections, requantised and dequantised in the GEMM epilogue, in the split layout
+            char *vt = (char *)qkv + (size_t)T_ * 2 * H_ * es;
+            ROCM_CALL(tnn_rocm_gemm_i8_qkv_split(Stream(), (int)dt, (const int8_t *)Ptr(inputs[0]), (const int8_t *)weight_,
+                                                 (const int32_t *)bias_, (const float *)scale_, (const float *)dequant_, qkv,
+                                                 vt, B_, seq_, p->heads, K_));
+            const long row = 2L * H_;
+            ROCM_CALL(tnn_rocm_attention_vt(Stream(), (int)dt, base, base + (size_t)H_ * es, vt, Ptr(outputs[0]), B_, p->heads,
+                                            seq_, p->head_dim, (long)seq_ * row, d, row, (long)seq_ * row, d, row,
+                                            (long)p->heads * 64 * seq_, 64L * seq_, (long)seq_, (long)seq_ * H_, d, (long)H_,
+                                            p->scale, mask, kv));
+            return TNN_OK;
+        }
         if (seq_ % 8 == 0 && H_ % 64 == 0) {
             // projection writes Q|K row-major and V already transposed per head: the attention kernel then stages
             // V tiles with 16-byte copies
@@ -519,9 +919,83 @@ public:
     }
 
 private:
-    void *weight_ = nullptr, *bias_ = nullptr;
-    int H_ = 0, T_ = 0, B_ = 0, seq_ = 0;
+    void *weight_ = nullptr, *bias_ = nullptr, *scale_ = nullptr, *dequant_ = nullptr;
+    int H_ = 0, K_ = 0, T_ = 0, B_ = 0, seq_ = 0;
 };
 REGISTER_ROCM_ACC(RocmFusedAttentionLayerAcc, LAYER_ROCM_FUSED_ATTENTION);
+
+// ---- RocmFusedLinearInt8 ---------------------------------------------------------------------------------------
+// QuantizedInnerProduct (x86_inner_product_layer_acc.cc:274-288 -> X86GemvInt8) whose int8 result is read as float:
+// y = float2int8((acc + bias) * w_scale / o_scale) * o_scale (+ residual), the value of
+// QuantizedInnerProduct -> Reformat(int8->float) [-> Add], with the int8 value formed in registers only.
+class RocmFusedLinearInt8LayerAcc : public RocmLayerAcc {
+public:
+    Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        if (weight_)
+            return TNN_OK;
+        auto p   = dynamic_cast<RocmFusedLinearInt8Param *>(param_);
+        auto res = dynamic_cast<InnerProductLayerResource *>(resource_);
+        CHECK_PARAM_NULL(p);
+        if (!res)
+            return Status(TNNERR_MODEL_ERR, "Error: InnerProductLayerResource is nil");
+        const int N = p->num_output;
+        const int K = DimsVectorUtils::Count(inputs[0]->GetBlobDesc().dims, p->axis);
+        if ((long)res->weight_handle.GetDataCount() != (long)N * K || res->weight_handle.GetDataType() != DATA_TYPE_INT8)
+            return Status(TNNERR_MODEL_ERR, "fused int8 linear: int8 weight of num_output x K expected");
+        const DataType odt = outputs[0]->GetBlobDesc().data_type;
+        if (inputs[0]->GetBlobDesc().data_type != DATA_TYPE_INT8 || (odt != DATA_TYPE_FLOAT && odt != DATA_TYPE_HALF))
+            return Status(TNNERR_LAYER_ERR, "fused int8 linear: int8 input and fp32/fp16 output expected");
+        if (p->has_residual && (inputs.size() != 2 || In(inputs[1])->GetBlobDesc().dims != outputs[0]->GetBlobDesc().dims ||
+                                In(inputs[1])->GetBlobDesc().data_type != outputs[0]->GetBlobDesc().data_type))
+            return Status(TNNERR_PARAM_ERR, "fused int8 linear: residual must have the output's shape and type");
+        const float *w_scale = res->scale_handle.force_to<float *>();
+        CHECK_PARAM_NULL(w_scale);
+        const int n_w = res->scale_handle.GetDataCount();
+        std::vector<float> scale(N);
+        for (int i = 0; i < N; ++i)
+            scale[i] = p->out_scale >= FLT_MIN ? w_scale[n_w == 1 ? 0 : i] / p->out_scale : 0.0f;
+        RETURN_ON_NEQ(UploadConverted(res->weight_handle.force_to<void *>(), (size_t)N * K, DATA_TYPE_INT8, DATA_TYPE_INT8,
+                                      &weight_), TNN_OK);
+        RETURN_ON_NEQ(UploadConverted(scale.data(), (size_t)N, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &scale_), TNN_OK);
+        if (p->has_bias && res->bias_handle.GetDataCount() == N)
+            RETURN_ON_NEQ(UploadConverted(res->bias_handle.force_to<void *>(), (size_t)N, DATA_TYPE_INT32, DATA_TYPE_INT32,
+                                          &bias_), TNN_OK);
+        return TNN_OK;
+    }
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto p       = dynamic_cast<RocmFusedLinearInt8Param *>(param_);
+        auto in_dims = inputs[0]->GetBlobDesc().dims;
+        const int N = p->num_output, K = DimsVectorUtils::Count(in_dims, p->axis);
+        const int rows = DimsVectorUtils::Count(in_dims, 0, p->axis);
+        ROCM_CALL(tnn_rocm_gemm_i8_dequant_residual(Stream(), (const int8_t *)Ptr(inputs[0]), (const int8_t *)weight_,
+                                                    (const int32_t *)bias_, (const float *)scale_, rows, N, K, K, K,
+                                                    Ptr(outputs[0]), (int)outputs[0]->GetBlobDesc().data_type, N, p->out_scale,
+                                                    p->has_residual ? Ptr(In(inputs[1])) : nullptr));
+        return TNN_OK;
+    }
+
+private:
+    void *weight_ = nullptr, *bias_ = nullptr, *scale_ = nullptr;
+};
+REGISTER_ROCM_ACC(RocmFusedLinearInt8LayerAcc, LAYER_ROCM_FUSED_LINEAR_INT8);
+
+// ---- RocmGeluInt8 -----------------------------------------------------------------------------------------------
+// Reformat(int8->float) -> GELU -> Reformat(float->int8) on int8 blobs in one pass: q_out =
+// float2int8(gelu(q_in * s_in) * float(1.0 / s_out)) (x86_compute_int8.cc:1193-1318, cpu_gelu_layer_acc.cc:42-45).
+class RocmGeluInt8LayerAcc : public RocmLayerAcc {
+public:
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto in8 = dynamic_cast<BlobInt8 *>(inputs[0]), out8 = dynamic_cast<BlobInt8 *>(outputs[0]);
+        if (!in8 || !out8 || !in8->GetIntResource() || !out8->GetIntResource() ||
+            in8->GetIntResource()->scale_handle.GetDataCount() != 1 || out8->GetIntResource()->scale_handle.GetDataCount() != 1)
+            return Status(TNNERR_LAYER_ERR, "int8 GELU needs per-tensor blob scales on both sides");
+        float s_in  = in8->GetIntResource()->scale_handle.force_to<float *>()[0];
+        float s_out = out8->GetIntResource()->scale_handle.force_to<float *>()[0];
+        ROCM_CALL(tnn_rocm_gelu_i8(Stream(), (const int8_t *)Ptr(inputs[0]), s_in, (float)(1.0 / s_out), (int8_t *)Ptr(outputs[0]),
+                                   (size_t)DimsVectorUtils::Count(inputs[0]->GetBlobDesc().dims)));
+        return TNN_OK;
+    }
+};
+REGISTER_ROCM_ACC(RocmGeluInt8LayerAcc, LAYER_ROCM_GELU_INT8);
 
 }  // namespace TNN_NS

@@ -282,8 +282,20 @@ public:
         int rows = DimsVectorUtils::Count(dims_in, 0, offset), cols = DimsVectorUtils::Count(dims_in, offset);
         if (rows == 0 || cols == 0)
             return Status(TNNERR_COMMON_ERROR, "Error: blob count is zero");
+        // a second output (added by the ROCm int8 pass in place of a following Reformat layer) receives the
+        // quantised copy of the first: float2int8(y * float(1.0 / scale)) on the value as stored in the float blob
+        // (x86_reformat_layer_acc.cc:66-75, x86_compute_int8.cc:1254-1318)
+        int8_t *out_q = nullptr;
+        float q_inv   = 0.f;
+        if (outputs.size() >= 2) {
+            auto b8 = dynamic_cast<BlobInt8 *>(outputs[1]);
+            if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1)
+                return Status(TNNERR_LAYER_ERR, "LayerNorm quantised output needs a per-tensor blob scale");
+            q_inv = (float)(1.0 / b8->GetIntResource()->scale_handle.force_to<float *>()[0]);
+            out_q = (int8_t *)Ptr(outputs[1]);
+        }
         ROCM_CALL(tnn_rocm_layernorm(Stream(), (int)dt, Ptr(inputs[0]), nullptr, (const float *)Ptr(scale),
-                                     (const float *)Ptr(bias), Ptr(outputs[0]), rows, cols, param->eps, nullptr, 0.f));
+                                     (const float *)Ptr(bias), Ptr(outputs[0]), rows, cols, param->eps, out_q, q_inv));
         return TNN_OK;
     }
 

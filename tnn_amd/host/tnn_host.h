@@ -308,8 +308,10 @@ enum LayerType {
     LAYER_GELU          = 327,
     LAYER_BLOB_SCALE    = 600,
     // produced only by the ROCm optimizer pass (no proto spelling in the engine)
-    LAYER_ROCM_FUSED_LINEAR    = 0x7001,
-    LAYER_ROCM_FUSED_ATTENTION = 0x7002,
+    LAYER_ROCM_FUSED_LINEAR      = 0x7001,
+    LAYER_ROCM_FUSED_ATTENTION   = 0x7002,
+    LAYER_ROCM_FUSED_LINEAR_INT8 = 0x7003,
+    LAYER_ROCM_GELU_INT8         = 0x7004,
 };
 LayerType GlobalConvertLayerType(std::string type_str);
 
@@ -381,6 +383,21 @@ struct RocmFusedAttentionParam : public LayerParam {
     float scale  = 1.0f;
     int has_mask = 0;  // second input: additive mask broadcastable to [B,1,1,S]
     int seq_len  = 0;  // S of the matched head split ([B,S,h,d]); 0 = take it from the input blob's shape
+    // quantised form: the first input is the int8 blob the three QuantizedInnerProduct projections read, the
+    // resource is a RocmFusedQkvInt8Resource and qkv_out_scale are the scales of their three int8 output blobs
+    int quant = 0;
+    float qkv_out_scale[3] = {0.f, 0.f, 0.f};
+};
+// QuantizedInnerProduct whose int8 result is consumed as float: y = q * out_scale (+ residual), q never stored.
+// Input 0 is the int8 blob, input 1 (has_residual) a float blob of the output's shape; the output is float.
+struct RocmFusedLinearInt8Param : public InnerProductLayerParam {
+    float out_scale  = 0.f;  // scale of the int8 blob the original layer produced
+    int has_residual = 0;
+};
+struct RocmFusedQkvInt8Resource : public LayerResource {
+    RawBuffer weight;   // int8 [3H, K]
+    RawBuffer bias;     // int32 [3H] (may be empty)
+    RawBuffer w_scale;  // fp32 [3H] per-output-channel weight scales
 };
 
 struct LayerInfo {
