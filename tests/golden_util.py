@@ -60,7 +60,7 @@ def int8_projections(cfg, w, li=0):
             (p + "act", p + "ffn2_o", lw["w2"], lw["b2"])]
 
 
-def check_projections_bit_exact(cfg, w, scales, blobs, T, quantize, layers=None):
+def check_projections_bit_exact(cfg, w, scales, blobs, T, quantize, layers=None, rows=None):
     """Teacher forcing: every projection, fed with the float blob the run itself produced (quantised as its Reformat
     layer does), must reproduce the run's own int8 output exactly.  `blobs` maps blob name -> dequantised array."""
     import orc
@@ -71,9 +71,10 @@ def check_projections_bit_exact(cfg, w, scales, blobs, T, quantize, layers=None)
             if src not in blobs or dst not in blobs:
                 continue
             w_q, b_q, w_s = quant.quantize_fc_params(wt, bias, scales[src])
-            src_q = quantize(np.ascontiguousarray(blobs[src], np.float32).reshape(T, -1), scales[src])
+            sel = slice(None) if rows is None else slice(0, rows)  # a row subset keeps full-size cases fast
+            src_q = quantize(np.ascontiguousarray(blobs[src], np.float32).reshape(T, -1)[sel], scales[src])
             y, acc = orc.fc_int8(src_q, w_q, b_q, orc.fc_int8_scale(w_s, scales[dst], w_q.shape[0]))
-            got = blobs[dst].reshape(T, -1) / scales[dst]
+            got = blobs[dst].reshape(T, -1)[sel] / scales[dst]
             assert np.abs(got - np.rint(got)).max() < 1e-3, dst
             bad = int((np.rint(got).astype(np.int8) != y).sum())
             assert bad == 0, "%s: %d of %d int8 outputs differ" % (dst, bad, y.size)

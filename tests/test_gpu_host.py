@@ -205,3 +205,80 @@ def test_graph_replay_matches_eager_on_every_replay(monkeypatch):
         torch.cuda.synchronize()
     eager.close()
     graph.close()
+
+
+def test_int8_encoder_full_shape_properties(monkeypatch):
+    """Benchmark config 4's per-layer shape (B16 S256, hidden 768, FFN 3072; 3 layers to keep the case short):
+    calibrated on this backend's fp32 forward, then run quantised in fp16 mode.  Size-independent checks: every
+    projection of the first and last layer reproduces its own int8 output bit-exactly from its own input blob (checker
+    on a 192-row slice), the folded graph agrees with the explicit Reformat chain, and the quantised network stays
+    close to the float one."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    import golden_util
+    from tnn_amd import quant
+    say("host: int8 encoder at B16 S256, properties")
+    cfg = EncoderConfig.bert_base(3)
+    w = make_weights(cfg, seed=41)
+    B, S = 16, 256
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 100, 256, seed=42)
+    inputs = {"input_ids": ids, "token_type_ids": seg, "attention_bias": mask.reshape(B, 1, 1, S)}
+    names = quant.calibration_outputs(cfg)
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S, extra_outputs=names), "fp32")
+    for k, v in inputs.items():
+        inst.set_input(k, v)
+    inst.forward()
+    scales = {n: quant.activation_scale(inst.output(n, max_elems=1 << 26)) for n in names}
+    float_out = inst.output("last_hidden")
+    inst.close()
+    check = ["x0"] + ["l%d_%s" % (li, b) for li in (0, 2) for b in quant.CALIBRATION_BLOBS] + ["l1_x2"]
+    runs = {}
+    for fuse, extra in (("0", check), ("1", [])):
+        monkeypatch.setenv("TNN_ROCM_FUSE_INT8", fuse)
+        inst = host.RocmInstance.from_graph(quant.int8_encoder_graph(cfg, w, scales, B, S, extra_outputs=extra), "fp16")
+        for k, v in inputs.items():
+            inst.set_input(k, v)
+        inst.forward()
+        runs[fuse] = inst.output("last_hidden")
+        if fuse == "0":
+            blobs = {n: inst.output(n, max_elems=1 << 26) for n in extra}
+        else:
+            types = [t for t, _ in inst.layers()]
+            assert types.count("RocmFusedAttention") == 3 and types.count("RocmFusedLinearInt8") == 6, types
+        inst.close()
+    n = golden_util.check_projections_bit_exact(cfg, w, scales, blobs, B * S, orc.quantize_x86, layers=(0, 2), rows=192)
+    assert n == 12
+    e_fused, e_float = rel_err(runs["1"], runs["0"]), rel_err(runs["1"], float_out)
+    say("  folded vs explicit chain %.3g ; quantised vs float network %.3g" % (e_fused, e_float))
+    # folding keeps float intermediates in fp32 where the chain rounds them to fp16: a few int8 steps may flip
+    assert e_fused <= 3e-2 and e_float <= 8e-2
+    valid = (np.arange(S)[None, :] < lens[:, None])
+    assert np.isfinite(runs["1"]).all() and np.abs(runs["1"][valid].mean(-1)).max() < 5e-3  # LayerNorm(gamma=1, beta=0)
+
+
+@pytest.mark.parametrize("name,hidden,heads,ffn,B,S,lo,hi", [("config 2 (BERT-base B8 S384)", 768, 12, 3072, 8, 384, 200, 384),
+                                                             ("config 5 (BERT-large B16 S512)", 1024, 16, 4096, 16, 512, 300, 512)])
+def test_encoder_full_batch_shape_against_checker_on_one_sequence(name, hidden, heads, ffn, B, S, lo, hi):
+    """The benchmark configurations at their full batch and sequence length (2 layers): the whole batch runs on the
+    device from model files; sequences are independent, so the checker evaluates ONE of them (the one with the shortest
+    valid length, which has the most padding) and must agree with that slice of the device result."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: %s, fp16, one sequence against the checker" % name)
+    cfg = EncoderConfig(2, hidden, heads, ffn)
+    w = make_weights(cfg, seed=51, bias_std=0.02)
+    ids, seg, lens, mask = make_inputs(cfg, B, S, lo, hi, seed=52)
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), "fp16")
+    inst.set_input("input_ids", ids)
+    inst.set_input("token_type_ids", seg)
+    inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+    for _ in range(4):  # eager, eager, graph capture, graph replay: every mode must give the same result
+        inst.forward()
+    got = inst.output("last_hidden", max_elems=1 << 26).reshape(B, S, hidden)
+    inst.close()
+    b = int(np.argmin(lens))
+    w16 = r16w(w)
+    x0 = encoder_ref.embed(w16, ids[b:b + 1], seg[b:b + 1], cfg.eps)
+    ref = encoder_ref.encoder(w16, cfg, x0, 1, S, mask[b:b + 1])
+    err = rel_err(got[b].reshape(S, hidden), ref)
+    say("  sequence %d (valid length %d of %d): max rel err %.3g" % (b, lens[b], S, err))
+    assert err <= FP16_TOL
+    assert np.isfinite(got).all()

@@ -495,6 +495,29 @@ def test_attention_fp16_varlen():
     assert rel_err(got2, got) <= 1e-3
 
 
+def test_attention_config3_full_shape_slices():
+    """Benchmark config 3 at full size (B32, 12 heads x 64, S512, valid lengths U[16,512], padding masked to -inf,
+    Q/K/V ~ N(0,1)): the device result of a handful of (batch, head) pairs -- the shortest, the longest and a few
+    others -- against the checker in fp32 on the fp16-rounded inputs; (batch, head) pairs are independent."""
+    say("attention fp16 config 3 full shape")
+    rng = np.random.default_rng(20240603)
+    B, h, S = 32, 12, 512
+    lens = rng.integers(16, 513, B).astype(np.int32)
+    q, k, v = (torch.from_numpy(rng.standard_normal((B, h, S, 64)).astype(np.float32)).half() for _ in range(3))
+    got = host(ops().attention(q.cuda(), k.cuda(), v.cuda(), 0.125, kv_len=dev(lens)))
+    assert np.isfinite(got).all()
+    picks = [(int(np.argmin(lens)), 0), (int(np.argmax(lens)), 11), (3, 5), (17, 7), (31, 2)]
+    worst = 0.0
+    for b, hh in picks:
+        mask = np.zeros((1, S), np.float32)
+        mask[0, lens[b]:] = -np.inf
+        sl = lambda t: t[b:b + 1, hh:hh + 1].float().numpy()
+        ref = orc.attention_core(sl(q), sl(k), sl(v), 0.125, mask)
+        worst = max(worst, rel_err(got[b:b + 1, hh:hh + 1], ref))
+    say("  worst of %d slices: max rel err %.3g (lengths %d..%d)" % (len(picks), worst, lens.min(), lens.max()))
+    assert worst <= FP16_TOL
+
+
 def test_attention_fp16_128row_blocks():
     # enough (batch, head, query-block) work that the launcher picks the 4-wave / 128-row variant
     say("attention fp16 4-wave variant")
