@@ -16,7 +16,8 @@ extern "C" {
 
 /* Instance(net_config{DEVICE_ROCM, device_id, precision}, model_config{proto text, model bytes}) + Init()
  * (reference include/tnn/core/instance.h:44-49, include/tnn/core/common.h:142-183).
- * precision: 0 = PRECISION_HIGH (fp32 blobs), 1 = PRECISION_AUTO (fp16 activations).
+ * precision: 0 = PRECISION_HIGH (fp32 blobs), 1 = PRECISION_AUTO (fp16 activations), 2 = PRECISION_LOW (bf16
+ * activations).
  * Returns NULL on failure and writes the status text to err[err_len]. */
 void *tnn_host_create(const char *proto, size_t proto_len, const char *model, size_t model_len, int device_id,
                       int precision, char *err, size_t err_len);

@@ -282,3 +282,28 @@ def test_encoder_full_batch_shape_against_checker_on_one_sequence(name, hidden, 
     say("  sequence %d (valid length %d of %d): max rel err %.3g" % (b, lens[b], S, err))
     assert err <= FP16_TOL
     assert np.isfinite(got).all()
+
+
+def test_encoder_bf16_from_model_files():
+    """PRECISION_LOW: bf16 activations and weights through the same fused layers.  The bar written for this path is
+    4e-2 (bf16 keeps 8 mantissa bits: one rounding is 4e-3 relative, and two encoder layers stack a few dozen)."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: 2-layer encoder, bf16")
+    cfg = EncoderConfig.bert_base(2)
+    w = make_weights(cfg, seed=3, bias_std=0.02)
+    B, S = 2, 96
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 30, 96, seed=4)
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), "bf16")
+    types = [t for t, _ in inst.layers()]
+    assert types.count("RocmFusedAttention") == 2 and types.count("RocmFusedLinear") == 6, types
+    inst.set_input("input_ids", ids)
+    inst.set_input("token_type_ids", seg)
+    inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+    inst.forward()
+    got = inst.output("last_hidden").reshape(B * S, -1)
+    inst.close()
+    x0 = encoder_ref.embed(w, ids, seg, cfg.eps)
+    ref = encoder_ref.encoder(w, cfg, x0, B, S, mask)
+    err = rel_err(got, ref)
+    say("  max rel err %.3g" % err)
+    assert err <= 4e-2

@@ -49,7 +49,8 @@ class HostError(RuntimeError):
 
 
 class RocmInstance:
-    """precision: "fp32" (PRECISION_HIGH) or "fp16" (PRECISION_AUTO: fp16 activations + fused kernels)."""
+    """precision: "fp32" (PRECISION_HIGH), "fp16" (PRECISION_AUTO: fp16 activations + fused kernels) or "bf16"
+    (PRECISION_LOW: bf16 activations + fused kernels)."""
 
     def __init__(self, proto, model, precision="fp16", device_id=0):
         lib = load()
@@ -57,7 +58,7 @@ class RocmInstance:
             proto = proto.encode()
         err = C.create_string_buffer(1024)
         self._h = lib.tnn_host_create(proto, len(proto), model, len(model), device_id,
-                                      0 if precision == "fp32" else 1, err, 1024)
+                                      {"fp32": 0, "fp16": 1, "bf16": 2}[precision], err, 1024)
         if not self._h:
             raise HostError("Instance::Init failed: " + err.value.decode())
         self._keep = []

@@ -26,7 +26,8 @@ int fail(Handle *h, const Status &st) {
 extern "C" {
 #define HOST_API __attribute__((visibility("default")))
 
-// precision: 0 = fp32 blobs (PRECISION_HIGH), 1 = fp16 activations (PRECISION_AUTO).  Returns NULL on failure and
+// precision: 0 = fp32 blobs (PRECISION_HIGH), 1 = fp16 activations (PRECISION_AUTO), 2 = bf16 activations
+// (PRECISION_LOW).  Returns NULL on failure and
 // writes the status text to err.
 HOST_API void *tnn_host_create(const char *proto, size_t proto_len, const char *model, size_t model_len, int device_id,
                                int precision, char *err, size_t err_len) {
@@ -34,7 +35,7 @@ HOST_API void *tnn_host_create(const char *proto, size_t proto_len, const char *
     NetworkConfig nc;
     nc.device_type = DEVICE_ROCM;
     nc.device_id   = device_id;
-    nc.precision   = precision == 0 ? PRECISION_HIGH : PRECISION_AUTO;
+    nc.precision   = precision == 0 ? PRECISION_HIGH : (precision == 2 ? PRECISION_LOW : PRECISION_AUTO);
     ModelConfig mc;
     mc.params.push_back(std::string(proto, proto_len));
     mc.params.push_back(std::string(model, model_len));

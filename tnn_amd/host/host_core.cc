@@ -1026,6 +1026,9 @@ Blob *DefaultNetwork::GetBlob(const std::string &name) {
 Status DefaultNetwork::InitLayers() {
     const bool half = config_.precision != PRECISION_HIGH &&
                       device_->GetImplementedPrecision(LAYER_MATMUL)->fp16_implemented;
+    // PRECISION_LOW selects bfloat16 activations (the engine's meaning of LOW on its bfp16-capable CPU backend,
+    // include/tnn/core/common.h:131-140); every other reduced precision is fp16
+    const DataType half_type = config_.precision == PRECISION_LOW ? DATA_TYPE_BFP16 : DATA_TYPE_HALF;
     bool quantized_net = false;
     for (auto &l : structure_.layers)
         quantized_net |= l->param->quantized;
@@ -1062,7 +1065,7 @@ Status DefaultNetwork::InitLayers() {
         auto dt_it  = structure_.input_data_type_map.find(kv.first);
         DataType dt = dt_it == structure_.input_data_type_map.end() ? DATA_TYPE_FLOAT : dt_it->second;
         if (dt == DATA_TYPE_FLOAT && half)
-            dt = DATA_TYPE_HALF;
+            dt = half_type;
         desc.data_type = dt;
         inputs_[kv.first] = b;
     }
@@ -1123,7 +1126,7 @@ Status DefaultNetwork::InitLayers() {
             info->type == LAYER_ROCM_FUSED_ATTENTION)
             for (auto b : outs)
                 if (!dynamic_cast<BlobInt8 *>(b))
-                    b->GetBlobDesc().data_type = half ? DATA_TYPE_HALF : DATA_TYPE_FLOAT;
+                    b->GetBlobDesc().data_type = half ? half_type : DATA_TYPE_FLOAT;
         LayerResource *res = nullptr;
         auto rit           = resource_.resource_map.find(info->name);
         if (rit != resource_.resource_map.end())
@@ -1135,7 +1138,7 @@ Status DefaultNetwork::InitLayers() {
         if (half)
             for (auto b : outs)
                 if (b->GetBlobDesc().data_type == DATA_TYPE_FLOAT)
-                    b->GetBlobDesc().data_type = DATA_TYPE_HALF;
+                    b->GetBlobDesc().data_type = half_type;
     }
     for (auto &name : structure_.outputs) {
         auto it = blobs_.find(name);
