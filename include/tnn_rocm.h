@@ -208,6 +208,17 @@ TNN_ROCM_API int tnn_rocm_permute(void *stream, int elem_bytes, const void *in, 
 TNN_ROCM_API int tnn_rocm_gather(void *stream, const void *data, const int32_t *indices, void *out, int batch,
                                  int slices, size_t slice_bytes, int n_indices, int32_t *error_flag);
 
+/* Embedding front end of a BERT-style encoder in one launch:
+ *   y[r][:] = LayerNorm((word_table[ids[r]][:] + pos_table[r % period][:]) + type_table[type_ids[r]][:])
+ * i.e. Gather, Gather, Add(position constant), Add, LayerNorm (cpu_gather_layer_acc.cc:27-86,
+ * compute_elewise.cc:37-65, cpu_layer_norm_layer_acc.cc:63-140) with the sums formed in that order.  Tables, y: dtype;
+ * gamma/beta fp32.  Index rules as tnn_rocm_gather (negative wraps; out of range sets *error_flag and reads row 0).
+ * Rows must be 16-byte aligned and at most 64*8 vectors of 16 bytes long. */
+TNN_ROCM_API int tnn_rocm_embed_layernorm(void *stream, int dtype, const int32_t *ids, const int32_t *type_ids,
+                                          const void *word_table, int vocab, const void *type_table, int n_types,
+                                          const void *pos_table, int period, const float *gamma, const float *beta,
+                                          float eps, void *y, int rows, int cols, int32_t *error_flag);
+
 /* dtype conversion between F32, F16 and BF16 (round to nearest even) */
 TNN_ROCM_API int tnn_rocm_cast(void *stream, int src_dtype, const void *src, int dst_dtype, void *dst, size_t count);
 

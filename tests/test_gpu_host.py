@@ -296,6 +296,7 @@ def test_encoder_bf16_from_model_files():
     inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), "bf16")
     types = [t for t, _ in inst.layers()]
     assert types.count("RocmFusedAttention") == 2 and types.count("RocmFusedLinear") == 6, types
+    assert types.count("RocmFusedEmbedding") == 1 and "Gather" not in types, types
     inst.set_input("input_ids", ids)
     inst.set_input("token_type_ids", seg)
     inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))

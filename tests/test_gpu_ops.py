@@ -453,6 +453,36 @@ def test_gemm_i8_qkv_split_bit_exact(B, S, heads, K):
     assert np.array_equal(host(vt), v_ref)
 
 
+def test_embed_layernorm_matches_the_five_layer_chain():
+    """Gather(word) + Add(position constant) + Gather(type) + Add + LayerNorm in one launch.  fp32: the checker's
+    embedding front end (same order of the two additions, double-precision statistics); fp16: within the fp16 bar;
+    an index outside the table raises the error flag like the Gather kernel."""
+    import encoder_ref
+    say("embed_layernorm")
+    rng = np.random.default_rng(11)
+    B, S, H, V = 3, 40, 768, 500
+    w = {"word_emb": rng.standard_normal((V, H)).astype(np.float32) * 0.05,
+         "type_emb": rng.standard_normal((2, H)).astype(np.float32) * 0.05,
+         "pos_emb": rng.standard_normal((64, H)).astype(np.float32) * 0.05,
+         "emb_ln_g": (1 + 0.1 * rng.standard_normal(H)).astype(np.float32),
+         "emb_ln_b": (0.1 * rng.standard_normal(H)).astype(np.float32)}
+    ids = rng.integers(0, V, (B, S)).astype(np.int32)
+    ids[0, 0] = -1  # negative indices wrap (cpu_gather_layer_acc.cc)
+    seg = rng.integers(0, 2, (B, S)).astype(np.int32)
+    ids_ref = np.where(ids < 0, ids + V, ids)
+    ref = encoder_ref.embed({**w, "pos_emb": w["pos_emb"]}, ids_ref, seg, 1e-12)
+    for tdt, tol in ((torch.float32, 2e-6), (torch.float16, FP16_TOL)):
+        y, flag = ops().embed_layernorm(dev(ids), dev(seg), dev(w["word_emb"], tdt), dev(w["type_emb"], tdt),
+                                        dev(w["pos_emb"][:S], tdt), dev(w["emb_ln_g"]), dev(w["emb_ln_b"]), 1e-12)
+        assert int(flag.item()) == 0
+        assert rel_err(host(y), ref) <= tol
+    bad = ids.copy()
+    bad[1, 3] = V
+    _, flag = ops().embed_layernorm(dev(bad), dev(seg), dev(w["word_emb"]), dev(w["type_emb"]), dev(w["pos_emb"][:S]),
+                                    dev(w["emb_ln_g"]), dev(w["emb_ln_b"]), 1e-12)
+    assert int(flag.item()) == 1
+
+
 # ---- fused attention ------------------------------------------------------------------------------
 def _attn_case(B, h, S, lens, seed, dtype=torch.float16, with_mask=False):
     rng = np.random.default_rng(seed)

@@ -24,13 +24,25 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
 // Statistics follow the reference's one-pass form var = E[x^2] - E[x]^2 with its types: the square
 // is an fp32 product, both sums, the mean, the variance and rstd are double.  An all-fp32
 // E[x^2]-E[x]^2 loses the variance to cancellation when |mean| >> std.
+// Optional row sources of the embedding front end: row r of the input is word_table[ids[r]] (x is the table),
+// the residual is pos_table[r % period] (res is the table) and a second addend type_table[type_ids[r]]; the sum is
+// ((word + pos) + type), the order of the Add layers it replaces.
+struct EmbedRows {
+    const int32_t *ids      = nullptr;  // null: plain LayerNorm
+    const int32_t *type_ids = nullptr;
+    const void *type_table  = nullptr;
+    int vocab = 0, n_types = 0, period = 0;
+    int32_t *error_flag = nullptr;
+};
+
 template <int DT, bool VECTOR>
 __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<DT>::type *__restrict__ x,
                                                            const typename Elem<DT>::type *__restrict__ res,
                                                            const float *__restrict__ gamma,
                                                            const float *__restrict__ beta,
                                                            typename Elem<DT>::type *__restrict__ y, int rows, int cols,
-                                                           float eps, int8_t *__restrict__ out_q, float q_inv) {
+                                                           float eps, int8_t *__restrict__ out_q, float q_inv,
+                                                           EmbedRows emb) {
     typedef typename Elem<DT>::type T;
     constexpr int VEC = VECTOR ? (int)(16 / sizeof(T)) : 1;
     const int lane    = threadIdx.x & (kWave - 1);
@@ -39,6 +51,23 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
         return;  // whole wave exits together; no workgroup barrier is used below
     const T *px  = x + (size_t)row * cols;
     const T *pr  = res ? res + (size_t)row * cols : nullptr;
+    const T *pr2 = nullptr;
+    if (VECTOR && emb.ids) {
+        // negative indices wrap, an index outside the table raises the flag and reads row 0
+        // (cpu_gather_layer_acc.cc:27-86)
+        int wi = emb.ids[row], ti = emb.type_ids[row];
+        wi += wi < 0 ? emb.vocab : 0;
+        ti += ti < 0 ? emb.n_types : 0;
+        const bool bad = wi < 0 || wi >= emb.vocab || ti < 0 || ti >= emb.n_types;
+        if (bad) {
+            if (lane == 0 && emb.error_flag)
+                *emb.error_flag = 1;
+            wi = 0, ti = 0;
+        }
+        px  = x + (size_t)wi * cols;
+        pr  = res + (size_t)(row % emb.period) * cols;
+        pr2 = reinterpret_cast<const T *>(emb.type_table) + (size_t)ti * cols;
+    }
     T *py        = y + (size_t)row * cols;
     int8_t *pq   = out_q ? out_q + (size_t)row * cols : nullptr;
     const int nv = cols / VEC;  // VECTOR launches guarantee cols % VEC == 0
@@ -52,15 +81,19 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
             if (VECTOR) {
                 uint4 raw = reinterpret_cast<const uint4 *>(px)[vi];
                 const T *e = reinterpret_cast<const T *>(&raw);
-                uint4 rraw;
-                const T *re = reinterpret_cast<const T *>(&rraw);
+                uint4 rraw, rraw2;
+                const T *re = reinterpret_cast<const T *>(&rraw), *re2 = reinterpret_cast<const T *>(&rraw2);
                 if (pr)
                     rraw = reinterpret_cast<const uint4 *>(pr)[vi];
+                if (pr2)
+                    rraw2 = reinterpret_cast<const uint4 *>(pr2)[vi];
 #pragma unroll
                 for (int t = 0; t < VEC; ++t) {
                     float f = Elem<DT>::ld(&e[t]);
                     if (pr)
                         f = __fadd_rn(f, Elem<DT>::ld(&re[t]));
+                    if (pr2)
+                        f = __fadd_rn(f, Elem<DT>::ld(&re2[t]));
                     v[j][t] = f;
                 }
             } else {
@@ -181,17 +214,22 @@ __global__ void __launch_bounds__(kBlock) layernorm_long_kernel(const typename E
 
 template <int DT>
 int launch_layernorm(hipStream_t s, const void *x, const void *res, const float *gamma, const float *beta, void *y,
-                     int rows, int cols, float eps, int8_t *out_q, float q_inv) {
+                     int rows, int cols, float eps, int8_t *out_q, float q_inv, const EmbedRows &emb = EmbedRows()) {
     typedef typename Elem<DT>::type T;
     constexpr int VEC = 16 / sizeof(T);
     dim3 grid((rows + kRowsPerBlk - 1) / kRowsPerBlk), block(kBlock);
-    bool al = ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)res)) & 15u) == 0 && cols % VEC == 0;
+    bool al = ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)res) | ((uintptr_t)emb.type_table)) & 15u) == 0 && cols % VEC == 0;
+    if (emb.ids && !(al && cols <= kWave * VEC * kMaxVecPerLn)) {
+        set_error("embed_layernorm: hidden size %d needs 16-byte aligned rows of at most %d elements", cols,
+                  kWave * VEC * kMaxVecPerLn);
+        return TNN_ROCM_ESHAPE;
+    }
     if (al && cols <= kWave * VEC * kMaxVecPerLn) {
         hipLaunchKernelGGL((layernorm_kernel<DT, true>), grid, block, 0, s, (const T *)x, (const T *)res, gamma, beta,
-                           (T *)y, rows, cols, eps, out_q, q_inv);
+                           (T *)y, rows, cols, eps, out_q, q_inv, emb);
     } else if (cols <= kWave * kMaxVecPerLn) {
         hipLaunchKernelGGL((layernorm_kernel<DT, false>), grid, block, 0, s, (const T *)x, (const T *)res, gamma, beta,
-                           (T *)y, rows, cols, eps, out_q, q_inv);
+                           (T *)y, rows, cols, eps, out_q, q_inv, emb);
     } else {
         hipLaunchKernelGGL((layernorm_long_kernel<DT>), grid, block, 0, s, (const T *)x, (const T *)res, gamma, beta,
                            (T *)y, rows, cols, eps, out_q, q_inv);
@@ -316,6 +354,36 @@ int tnn_rocm_layernorm(void *stream, int dtype, const void *x, const void *resid
             return launch_layernorm<TNN_ROCM_BF16>(s, x, residual, gamma, beta, y, rows, cols, eps, out_q,
                                                    q_inv_scale);
         default: set_error("layernorm: unsupported dtype %d", dtype); return TNN_ROCM_EDTYPE;
+    }
+}
+
+int tnn_rocm_embed_layernorm(void *stream, int dtype, const int32_t *ids, const int32_t *type_ids, const void *word_table,
+                             int vocab, const void *type_table, int n_types, const void *pos_table, int period,
+                             const float *gamma, const float *beta, float eps, void *y, int rows, int cols,
+                             int32_t *error_flag) {
+    TR_REQUIRE(rows >= 0 && cols > 0 && vocab > 0 && n_types > 0 && period > 0, TNN_ROCM_ESHAPE,
+               "embed_layernorm: sizes must be positive");
+    if (rows == 0)
+        return 0;
+    TR_REQUIRE(ids && type_ids && word_table && type_table && pos_table && gamma && beta && y, TNN_ROCM_EINVAL,
+               "embed_layernorm: null pointer");
+    EmbedRows emb;
+    emb.ids        = ids;
+    emb.type_ids   = type_ids;
+    emb.type_table = type_table;
+    emb.vocab      = vocab;
+    emb.n_types    = n_types;
+    emb.period     = period;
+    emb.error_flag = error_flag;
+    hipStream_t s  = (hipStream_t)stream;
+    switch (dtype) {
+        case TNN_ROCM_F32:
+            return launch_layernorm<TNN_ROCM_F32>(s, word_table, pos_table, gamma, beta, y, rows, cols, eps, nullptr, 0.f, emb);
+        case TNN_ROCM_F16:
+            return launch_layernorm<TNN_ROCM_F16>(s, word_table, pos_table, gamma, beta, y, rows, cols, eps, nullptr, 0.f, emb);
+        case TNN_ROCM_BF16:
+            return launch_layernorm<TNN_ROCM_BF16>(s, word_table, pos_table, gamma, beta, y, rows, cols, eps, nullptr, 0.f, emb);
+        default: set_error("embed_layernorm: unsupported dtype %d", dtype); return TNN_ROCM_EDTYPE;
     }
 }
 

@@ -102,6 +102,7 @@ LayerType GlobalConvertLayerType(std::string s) {
         {"BlobScale", LAYER_BLOB_SCALE},      {"QuantizedAdd", LAYER_ADD},
         {"RocmFusedLinear", LAYER_ROCM_FUSED_LINEAR}, {"RocmFusedAttention", LAYER_ROCM_FUSED_ATTENTION},
         {"RocmFusedLinearInt8", LAYER_ROCM_FUSED_LINEAR_INT8}, {"RocmGeluInt8", LAYER_ROCM_GELU_INT8},
+        {"RocmFusedEmbedding", LAYER_ROCM_FUSED_EMBEDDING},
     };
     auto it = m.find(s);
     return it == m.end() ? LAYER_NOT_SUPPORT : it->second;
@@ -830,6 +831,19 @@ struct ReformatLayer : BaseLayer {  // layer/reformat_layer.cc
     }
 };
 
+struct FusedEmbeddingLayer : BaseLayer {  // ids [..] int32 -> [.., H] in the network's float type (set by the network)
+    using BaseLayer::BaseLayer;
+    Status InferOutputDataType() override { return TNN_OK; }
+    Status InferOutputShape() override {
+        auto r = dynamic_cast<RocmFusedEmbeddingResource *>(resource_);
+        CHECK_PARAM_NULL(r);
+        auto out = input_blobs_[0]->GetBlobDesc().dims;
+        out.push_back(r->word.GetBufferDims().back());
+        output_blobs_[0]->GetBlobDesc().dims = out;
+        return TNN_OK;
+    }
+};
+
 struct FusedLinearLayer : BaseLayer {
     using BaseLayer::BaseLayer;
     Status InferOutputShape() override {
@@ -867,6 +881,7 @@ BaseLayer *CreateLayer(LayerType type) {
         case LAYER_CAST: return new CastLayer(type);
         case LAYER_REFORMAT: return new ReformatLayer(type);
         case LAYER_ROCM_FUSED_LINEAR: return new FusedLinearLayer(type);
+        case LAYER_ROCM_FUSED_EMBEDDING: return new FusedEmbeddingLayer(type);
         case LAYER_ROCM_FUSED_LINEAR_INT8: return new MixedTypeLayer<InnerProductLayer>(type);
         case LAYER_ROCM_FUSED_ATTENTION: return new MixedTypeLayer<BaseLayer>(type);
         case LAYER_SOFTMAX:
@@ -1123,7 +1138,7 @@ Status DefaultNetwork::InitLayers() {
                 }
         // float outputs of a dequantising Reformat (or of a fused layer that contains one) follow the network precision
         if (info->type == LAYER_REFORMAT || info->type == LAYER_ROCM_FUSED_LINEAR_INT8 ||
-            info->type == LAYER_ROCM_FUSED_ATTENTION)
+            info->type == LAYER_ROCM_FUSED_ATTENTION || info->type == LAYER_ROCM_FUSED_EMBEDDING)
             for (auto b : outs)
                 if (!dynamic_cast<BlobInt8 *>(b))
                     b->GetBlobDesc().data_type = half ? half_type : DATA_TYPE_FLOAT;

@@ -56,6 +56,7 @@ public:
     Status Optimize(NetStructure *s, NetResource *r) override {
         structure_ = s;
         resource_  = r;
+        FuseEmbedding();
         FuseLinear();
         FoldGelu();
         FoldResidual();
@@ -108,6 +109,77 @@ private:
         }
         resource_->resource_map[name] = res;
         return l;
+    }
+
+    // Gather(word table, ids) -> Add(position constant [S,H]) -> Add(Gather(type table, type ids)) -> LayerNorm
+    //                                                                                   ==> RocmFusedEmbedding
+    void FuseEmbedding() {
+        auto &L = structure_->layers;
+        GraphIndex g(L);
+        auto table_gather = [&](int i) -> GatherLayerResource * {
+            if (i < 0 || !L[i] || L[i]->type != LAYER_GATHER || L[i]->inputs.size() != 1)
+                return nullptr;
+            auto gp = ParamOf<GatherLayerParam>(L[i]);
+            auto gr = ResOf<GatherLayerResource>(L[i]->name);
+            if (!gp || !gr || gp->axis != 0 || !gp->data_in_resource || gp->indices_in_resource ||
+                gr->data.GetBufferDims().size() != 2 || gr->data.GetDataType() != DATA_TYPE_FLOAT)
+                return nullptr;
+            return gr;
+        };
+        for (int li = 0; li < (int)L.size(); ++li) {
+            auto ln = L[li];
+            if (!ln || ln->type != LAYER_LAYER_NORM || ln->inputs.size() != 3 || ln->outputs.size() != 1)
+                continue;
+            int ai = g.producer_of(ln->inputs[0]);  // Add(word + pos, type)
+            if (ai < 0 || !L[ai] || L[ai]->type != LAYER_ADD || L[ai]->inputs.size() != 2 || g.sole_consumer(ln->inputs[0]) != li ||
+                IsModelOutput(ln->inputs[0]) || ResOf<EltwiseLayerResource>(L[ai]->name))
+                continue;
+            int pi = -1, ti = -1;
+            for (int side = 0; side < 2 && pi < 0; ++side) {
+                int a = g.producer_of(L[ai]->inputs[side]), b = g.producer_of(L[ai]->inputs[1 - side]);
+                if (a >= 0 && L[a] && L[a]->type == LAYER_ADD && L[a]->inputs.size() == 1 && table_gather(b))
+                    pi = a, ti = b;
+            }
+            if (pi < 0)
+                continue;
+            auto pos = ResOf<EltwiseLayerResource>(L[pi]->name);
+            int wi   = g.producer_of(L[pi]->inputs[0]);
+            auto wr = table_gather(wi), tr = table_gather(ti);
+            if (!pos || !wr || !tr || pos->element_handle.GetDataType() != DATA_TYPE_FLOAT)
+                continue;
+            const int H = wr->data.GetBufferDims()[1];
+            auto pd     = pos->element_handle.GetBufferDims();
+            if (tr->data.GetBufferDims()[1] != H || pd.size() < 2 || pd.back() != H ||
+                pos->element_handle.GetDataCount() != pd[pd.size() - 2] * H)
+                continue;  // the constant must be one [S,H] matrix (leading dimensions of extent 1)
+            bool single = true;
+            for (int idx : {pi, ti, wi})
+                single &= g.sole_consumer(L[idx]->outputs[0]) >= 0 && !IsModelOutput(L[idx]->outputs[0]);
+            if (!single)
+                continue;
+            auto lp      = ParamOf<LayerNormLayerParam>(ln);
+            auto fl      = std::make_shared<LayerInfo>();
+            fl->type     = LAYER_ROCM_FUSED_EMBEDDING;
+            fl->type_str = "RocmFusedEmbedding";
+            fl->name     = ln->name + "_fused_embedding";
+            fl->inputs   = {L[wi]->inputs[0], L[ti]->inputs[0], ln->inputs[1], ln->inputs[2]};
+            fl->outputs  = ln->outputs;
+            auto fp      = std::make_shared<RocmFusedEmbeddingParam>();
+            fp->type     = fl->type_str;
+            fp->name     = fl->name;
+            fp->eps      = lp->eps;
+            fl->param    = fp;
+            auto fr      = std::make_shared<RocmFusedEmbeddingResource>();
+            fr->name     = fl->name;
+            fr->word     = wr->data;
+            fr->type     = tr->data;
+            fr->pos      = pos->element_handle;
+            resource_->resource_map[fl->name] = fr;
+            L[wi] = L[ti] = L[pi] = L[ai] = nullptr;
+            // the fused layer goes where the LayerNorm was: every input (ids, constants) exists before that point
+            L[li] = fl;
+        }
+        Compact();
     }
 
     // MatMul(weight_position=1, fp32 [K,N] resource) -> Add(bias resource of N values)   ==> RocmFusedLinear
@@ -923,6 +995,54 @@ private:
     int H_ = 0, K_ = 0, T_ = 0, B_ = 0, seq_ = 0;
 };
 REGISTER_ROCM_ACC(RocmFusedAttentionLayerAcc, LAYER_ROCM_FUSED_ATTENTION);
+
+// ---- RocmFusedEmbedding ----------------------------------------------------------------------------------------
+class RocmFusedEmbeddingLayerAcc : public RocmLayerAcc {
+public:
+    Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto res = dynamic_cast<RocmFusedEmbeddingResource *>(resource_);
+        CHECK_PARAM_NULL(res);
+        if (inputs.size() != 4 || inputs[0]->GetBlobDesc().data_type != DATA_TYPE_INT32 ||
+            inputs[1]->GetBlobDesc().data_type != DATA_TYPE_INT32 ||
+            inputs[0]->GetBlobDesc().dims != inputs[1]->GetBlobDesc().dims)
+            return Status(TNNERR_PARAM_ERR, "fused embedding: two int32 index blobs of equal shape, gamma and beta expected");
+        auto wd = res->word.GetBufferDims(), td = res->type.GetBufferDims(), pd = res->pos.GetBufferDims();
+        auto id = inputs[0]->GetBlobDesc().dims;
+        H_      = wd[1];
+        period_ = pd[pd.size() - 2];
+        if (id.empty() || id.back() != period_)
+            return Status(TNNERR_PARAM_ERR, "fused embedding: the position constant does not match the sequence length");
+        vocab_ = wd[0], types_ = td[0];
+        if (word_)
+            return TNN_OK;
+        DataType dt = outputs[0]->GetBlobDesc().data_type;
+        RETURN_ON_NEQ(UploadConverted(res->word.force_to<void *>(), (size_t)vocab_ * H_, DATA_TYPE_FLOAT, dt, &word_), TNN_OK);
+        RETURN_ON_NEQ(UploadConverted(res->type.force_to<void *>(), (size_t)types_ * H_, DATA_TYPE_FLOAT, dt, &type_), TNN_OK);
+        RETURN_ON_NEQ(UploadConverted(res->pos.force_to<void *>(), (size_t)period_ * H_, DATA_TYPE_FLOAT, dt, &pos_), TNN_OK);
+        return TNN_OK;
+    }
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto p = dynamic_cast<RocmFusedEmbeddingParam *>(param_);
+        Blob *gamma = In(inputs[2]), *beta = In(inputs[3]);
+        if (gamma->GetBlobDesc().data_type != DATA_TYPE_FLOAT || beta->GetBlobDesc().data_type != DATA_TYPE_FLOAT ||
+            DimsVectorUtils::Count(gamma->GetBlobDesc().dims) != H_ || DimsVectorUtils::Count(beta->GetBlobDesc().dims) != H_)
+            return Status(TNNERR_PARAM_ERR, "fused embedding: gamma/beta must be fp32 vectors of the hidden size");
+        const int rows = DimsVectorUtils::Count(inputs[0]->GetBlobDesc().dims);
+        ROCM_CALL(tnn_rocm_embed_layernorm(Stream(), (int)outputs[0]->GetBlobDesc().data_type, (const int32_t *)Ptr(inputs[0]),
+                                           (const int32_t *)Ptr(inputs[1]), word_, vocab_, type_, types_, pos_, period_,
+                                           (const float *)Ptr(gamma), (const float *)Ptr(beta), p->eps, Ptr(outputs[0]), rows,
+                                           H_, context_->ErrorFlag()));
+        return TNN_OK;
+    }
+
+protected:
+    DataType ConstantBlobDataType(const std::vector<Blob *> &, int) override { return DATA_TYPE_FLOAT; }
+
+private:
+    void *word_ = nullptr, *type_ = nullptr, *pos_ = nullptr;
+    int H_ = 0, period_ = 0, vocab_ = 0, types_ = 0;
+};
+REGISTER_ROCM_ACC(RocmFusedEmbeddingLayerAcc, LAYER_ROCM_FUSED_EMBEDDING);
 
 // ---- RocmFusedLinearInt8 ---------------------------------------------------------------------------------------
 // QuantizedInnerProduct (x86_inner_product_layer_acc.cc:274-288 -> X86GemvInt8) whose int8 result is read as float:

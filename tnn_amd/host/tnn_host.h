@@ -312,6 +312,7 @@ enum LayerType {
     LAYER_ROCM_FUSED_ATTENTION   = 0x7002,
     LAYER_ROCM_FUSED_LINEAR_INT8 = 0x7003,
     LAYER_ROCM_GELU_INT8         = 0x7004,
+    LAYER_ROCM_FUSED_EMBEDDING   = 0x7005,
 };
 LayerType GlobalConvertLayerType(std::string type_str);
 
@@ -387,6 +388,16 @@ struct RocmFusedAttentionParam : public LayerParam {
     // resource is a RocmFusedQkvInt8Resource and qkv_out_scale are the scales of their three int8 output blobs
     int quant = 0;
     float qkv_out_scale[3] = {0.f, 0.f, 0.f};
+};
+// Gather(word ids) + Add(position constant) + Gather(type ids) + Add + LayerNorm of a BERT-style front end.
+// Inputs: word ids, type ids (int32), gamma, beta (constant blobs); resource: RocmFusedEmbeddingResource.
+struct RocmFusedEmbeddingParam : public LayerParam {
+    float eps = 1e-5f;
+};
+struct RocmFusedEmbeddingResource : public LayerResource {
+    RawBuffer word;  // [vocab, H]
+    RawBuffer type;  // [types, H]
+    RawBuffer pos;   // [S, H]: the constant added to the word rows, one row per position
 };
 // QuantizedInnerProduct whose int8 result is consumed as float: y = q * out_scale (+ residual), q never stored.
 // Input 0 is the int8 blob, input 1 (has_residual) a float blob of the output's shape; the output is float.

@@ -164,6 +164,18 @@ def layernorm(x, gamma, beta, eps, residual=None, q_inv_scale=None):
     return (y, q) if q is not None else y
 
 
+def embed_layernorm(ids, type_ids, word_table, type_table, pos_table, gamma, beta, eps):
+    """ids/type_ids int32 [B,S] -> LayerNorm(word[ids] + pos[s] + type[type_ids]) as [B*S, H]"""
+    _chk(ids, type_ids, word_table, type_table, pos_table, gamma, beta)
+    rows, H = ids.numel(), word_table.shape[1]
+    y = torch.empty(rows, H, dtype=word_table.dtype, device=word_table.device)
+    flag = torch.zeros(1, dtype=torch.int32, device=word_table.device)
+    capi.call("tnn_rocm_embed_layernorm", _stream(), dt(word_table), _p(ids), _p(type_ids), _p(word_table),
+              word_table.shape[0], _p(type_table), type_table.shape[0], _p(pos_table), pos_table.shape[0], _p(gamma),
+              _p(beta), float(eps), _p(y), rows, H, _p(flag))
+    return y, flag
+
+
 def gelu(x):
     _chk(x)
     y = torch.empty_like(x)
