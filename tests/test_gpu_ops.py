@@ -369,6 +369,42 @@ def test_gemm_half_epilogues(M, N, K, dtype):
     assert rel_err(got, orc.inner_product(af, wf, bias) + rf) <= tol
 
 
+TILE_CODES = [112211, 222221, 224211, 332221, 331182,   # slabs staged through registers
+              2112211, 2222221, 3332221, 3331182]       # slabs loaded global -> LDS directly (2 / 3 stages)
+
+
+@pytest.mark.parametrize("code", TILE_CODES)
+def test_gemm_every_tile_configuration(code):
+    """Each tuning configuration of the tiled kernel, forced for a ragged shape (M and N are no tile multiples, K spans
+    several slabs): fp16 with the fused epilogues against the checker, int8 bit-exact."""
+    from tnn_amd import capi
+    lib = capi.load()
+    say("tile configuration %d" % code)
+    M, N, K = 333, 520, 1536
+    rng = np.random.default_rng(code)
+    a = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).half()
+    w = torch.from_numpy((rng.standard_normal((N, K)) * 0.02).astype(np.float32)).half()
+    res = torch.from_numpy(rng.standard_normal((M, N)).astype(np.float32)).half()
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    af, wf, rf = a.float().numpy(), w.float().numpy(), res.float().numpy()
+    a8 = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w8 = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    b8 = rng.integers(-20000, 20000, N).astype(np.int32)
+    scale = orc.fc_int8_scale((rng.uniform(0.5, 1.5, N) * 1e-3).astype(np.float32), np.float32(0.37), N)
+    ref_q, ref_acc = orc.fc_int8(a8, w8, b8, scale)
+    lib.tnn_rocm_debug_set_gemm_config(code)
+    try:
+        got = host(ops().gemm(a.cuda(), w.cuda(), True, bias=dev(bias), gelu=True))
+        assert rel_err(got, orc.gelu(orc.inner_product(af, wf, bias))) <= FP16_TOL
+        got = host(ops().gemm(a.cuda(), w.cuda(), True, bias=dev(bias), residual=res.cuda()))
+        assert rel_err(got, orc.inner_product(af, wf, bias) + rf) <= FP16_TOL
+        q, acc, _ = ops().gemm_i8(dev(a8), dev(w8), dev(b8), dev(scale), want_acc=True)
+        assert np.array_equal(host(acc), ref_acc)
+        assert np.array_equal(host(q), ref_q)
+    finally:
+        lib.tnn_rocm_debug_set_gemm_config(0)
+
+
 # ---- int8 GEMM: bit-exact accumulators and outputs -----------------------------------------------
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (2, 4, 9), (2, 16, 19), (7, 32, 16), (128, 3072, 768), (128, 768, 3072),
                                    (300, 768, 768), (65, 100, 200)])

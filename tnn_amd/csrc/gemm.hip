@@ -18,6 +18,7 @@
 //
 // Output layout of a 32x32 block: lane l holds column (l % 32); accumulator register r holds row
 // 8*(r/4) + 4*(l/32) + (r%4).
+#include <cstring>
 #include <type_traits>
 
 #include "common.h"
@@ -339,12 +340,20 @@ template <int DT> struct Int8QkvSplitEpilogue {
     }
     __device__ __forceinline__ bool direct(int n0) const { return n0 >= 2 * H; }
     __device__ __forceinline__ void store8(int m, int n, const int (&acc)[8]) const {
+        // per-column constants as 16-byte loads (n % 8 == 0 and the arrays are 16-byte aligned, checked at launch)
+        i32x4 b0 = {0, 0, 0, 0}, b1 = {0, 0, 0, 0};
+        if (bias)
+            b0 = *reinterpret_cast<const i32x4 *>(bias + n), b1 = *reinterpret_cast<const i32x4 *>(bias + n + 4);
+        const float4 s0 = *reinterpret_cast<const float4 *>(scale + n), s1 = *reinterpret_cast<const float4 *>(scale + n + 4);
+        const float4 d0 = *reinterpret_cast<const float4 *>(dequant + n), d1 = *reinterpret_cast<const float4 *>(dequant + n + 4);
+        const int bb[8]   = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+        const float sc[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        const float dq[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
         float v[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            int a    = acc[t] + (bias ? bias[n + t] : 0);
-            int8_t q = float2int8_ref(__fmul_rn((float)a, scale[n + t]));
-            v[t]     = __fmul_rn((float)q, dequant[n + t]);
+            int8_t q = float2int8_ref(__fmul_rn((float)(acc[t] + bb[t]), sc[t]));
+            v[t]     = __fmul_rn((float)q, dq[t]);
         }
         if (n < 2 * H) {
             constexpr int NV = 8 * sizeof(T) / 16;
@@ -585,19 +594,28 @@ __global__ void __launch_bounds__(WM *WN * 64)
 //   * the epilogue turns the accumulators through LDS into a row-contiguous layout, so C, bias and residual
 //     move as whole cache lines.
 // LDS is dynamic: max(2 buffers x (BM + BN) rows x (SLAB + 16) bytes, 4 x 32 x (32*TN + 4) words of staging).
-template <int TM_, int TN_, int WGM_, int WGN_, int WGK_, int SLAB_> struct TileCfg {
-    static constexpr int TM = TM_, TN = TN_, WGM = WGM_, WGN = WGN_, WGK = WGK_, SLAB = SLAB_;
+// NSTAGE = 0: slabs travel global -> registers -> LDS (padded rows, two LDS buffers).
+// NSTAGE = 2 or 3: slabs travel global -> LDS directly (global_load_lds_dwordx4: no staging registers and no LDS
+//     store instructions), into NSTAGE un-padded buffers whose 16-byte chunks are XOR-swizzled per row so that the
+//     fragment reads stay free of bank conflicts; loads run NSTAGE-1 slabs ahead of the MFMAs.
+template <int TM_, int TN_, int WGM_, int WGN_, int WGK_, int SLAB_, int NSTAGE_ = 0> struct TileCfg {
+    static constexpr int TM = TM_, TN = TN_, WGM = WGM_, WGN = WGN_, WGK = WGK_, SLAB = SLAB_, NSTAGE = NSTAGE_;
     static constexpr int BM = 32 * TM * WGM, BN = 32 * TN * WGN;
-    static constexpr int STRIDE = SLAB + 16;
+    static constexpr int STRIDE = NSTAGE_ ? SLAB : SLAB + 16;
     static constexpr int SSTR   = 32 * TN + 4;  // staged row stride in 32-bit words
-    static constexpr size_t slab_bytes  = (size_t)2 * (BM + BN) * STRIDE;
+    static constexpr size_t slab_bytes  = (size_t)(NSTAGE_ ? NSTAGE_ : 2) * (BM + BN) * STRIDE;
     static constexpr size_t stage_bytes = (size_t)WGM_ * WGN_ * WGK_ * 32 * SSTR * 4;
     static constexpr size_t lds_bytes   = slab_bytes > stage_bytes ? slab_bytes : stage_bytes;
     static constexpr int NW = WGM * WGN * WGK, NT = 64 * NW;  // waves and threads per workgroup
     static_assert(NW == 4 || NW == 8, "four or eight waves per workgroup");
     static_assert((SLAB / 32) % WGK == 0, "k-steps of a slab must split evenly over the k-waves");
     static_assert((BM * (SLAB / 16)) % NT == 0 && (BN * (SLAB / 16)) % NT == 0, "slab must divide over the workgroup");
+    static_assert(NSTAGE_ == 0 || NSTAGE_ == 2 || NSTAGE_ == 3, "register-staged, or two / three direct-to-LDS stages");
 };
+
+// s_waitcnt that waits only for the vector-memory counter to drop to n (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4 and lgkmcnt 11:8 left at their maxima)
+#define TR_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n)&0xF) | ((((n) >> 4) & 3) << 14) | (0x7 << 4) | (0xF << 8)))
 
 template <int DT, typename CFG, typename Epi>
 __global__ void __launch_bounds__(CFG::NT)
@@ -642,6 +660,117 @@ __global__ void __launch_bounds__(CFG::NT)
     const int m0       = (first_m + in_grp % rows_g) * BM;
     const int n0       = (in_grp / rows_g) * BN;
 
+    Acc acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0;
+
+    const int frag_row = lane & 31;
+    const int frag_off = (lane >> 5) * 16;
+    const int nk       = K / KB;
+
+    if constexpr (CFG::NSTAGE > 0) {
+        // Direct-to-LDS pipeline.  One load instruction of a wave fills 1024 contiguous LDS bytes (lane L writes
+        // bytes 16L..16L+15), i.e. RPL whole slab rows; the lane picks WHICH 16 global bytes land there, so the
+        // swizzle is applied on the global side: physical chunk p of LDS row r holds logical chunk p ^ f(r),
+        // f(r) = (r / rows per 256 bytes) mod VPR.  Sixteen consecutive rows reading the same logical chunk then
+        // touch sixteen different 16-byte bank groups.
+        constexpr int NS    = CFG::NSTAGE;
+        constexpr int RPL   = 1024 / SLAB;        // slab rows per wave-load
+        constexpr int R256  = 256 / SLAB > 0 ? 256 / SLAB : 1;
+        constexpr int A_LD  = BM / RPL / CFG::NW;  // wave-loads of A per wave and slab
+        constexpr int B_LD  = BN / RPL / CFG::NW;
+        constexpr int STAGE = (BM + BN) * SLAB;
+        static_assert(BM % (RPL * CFG::NW) == 0 && BN % (RPL * CFG::NW) == 0, "slab rows must divide over the waves");
+        static_assert((NS - 1) * (A_LD + B_LD) < 64, "look-ahead must fit the vmcnt counter");
+        uint32_t a_off[A_LD], b_off[B_LD];
+        const int lrow = lane / VPR, lpos = lane % VPR;
+#pragma unroll
+        for (int i = 0; i < A_LD; ++i) {
+            const int r = (wave + i * CFG::NW) * RPL + lrow;
+            int row     = m0 + r;
+            row         = row < M ? row : M - 1;
+            a_off[i]    = (uint32_t)row * (uint32_t)lda + (uint32_t)((lpos ^ ((r / R256) % VPR)) * VEC);
+        }
+#pragma unroll
+        for (int i = 0; i < B_LD; ++i) {
+            const int r = (wave + i * CFG::NW) * RPL + lrow;
+            int row     = n0 + r;
+            row         = row < N ? row : N - 1;
+            b_off[i]    = (uint32_t)row * (uint32_t)ldb + (uint32_t)((lpos ^ ((r / R256) % VPR)) * VEC);
+        }
+        // The load is spelled as inline assembly on purpose: for the compiler's own global_load_lds builtin the
+        // wait-count pass puts vmcnt(0) in front of every later LDS read (it cannot tell the stages apart), which
+        // serialises the pipeline.  Here the waits are placed by hand (TR_WAIT_VMCNT below); the kernel issues no
+        // other vector-memory operation until the loop has drained.  m0 carries the wave-uniform LDS address and
+        // needs one wait state before the load.
+        const uint32_t lds_base = (uint32_t)(uintptr_t)lds_dyn;  // generic -> LDS offset (low 32 bits of the aperture address)
+        const uint32_t wave_dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_base + (uint32_t)wave * 1024u));
+        auto load16 = [](const T *base, uint32_t byte_off, uint32_t lds_addr) {
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :
+                         : "v"(byte_off), "s"(base), "s"(lds_addr)
+                         : "memory");
+        };
+        auto issue = [&](int slab, int stage) {
+            const uint32_t dst = wave_dst + (uint32_t)(stage * STAGE);
+            const T *ga = A + (size_t)slab * KB, *gb = B + (size_t)slab * KB;
+#pragma unroll
+            for (int i = 0; i < A_LD; ++i)
+                load16(ga, a_off[i] * (uint32_t)sizeof(T), dst + i * CFG::NW * 1024);
+#pragma unroll
+            for (int i = 0; i < B_LD; ++i)
+                load16(gb, b_off[i] * (uint32_t)sizeof(T), dst + BM * SLAB + i * CFG::NW * 1024);
+        };
+        // byte offset of this lane's fragment chunk inside a slab row, per k-step of the slab
+        const int fswz = (frag_row / R256) % VPR;
+        const int frow = frag_row * SLAB;
+        auto compute = [&](int stage) {
+            const unsigned char *sa = lds_dyn + stage * STAGE, *sb = sa + BM * SLAB;
+#pragma unroll
+            for (int kk = wk; kk < SLAB / 32; kk += WGK) {
+                const int chunk = ((kk * 2 + (lane >> 5)) ^ fswz) * 16;
+                uint4 fa[TM], fb[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    fa[i] = *reinterpret_cast<const uint4 *>(sa + (wm * TM + i) * 32 * SLAB + frow + chunk);
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    fb[j] = *reinterpret_cast<const uint4 *>(sb + (wn * TN + j) * 32 * SLAB + frow + chunk);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        GemmTraits<DT>::mma(fb[j], fa[i], acc[i][j]);
+            }
+        };
+        constexpr int LPW = A_LD + B_LD;
+#pragma unroll
+        for (int p = 0; p < NS - 1; ++p)
+            if (p < nk)
+                issue(p, p);
+        int stage = 0, fill = NS - 1;  // stage of slab kt; stage that slab kt + NS - 1 goes to
+        for (int kt = 0; kt < nk; ++kt) {
+            // slab kt has landed once at most the loads of the slabs issued after it are outstanding
+            if (NS == 3 && kt + 1 < nk)
+                TR_WAIT_VMCNT(LPW);
+            else
+                TR_WAIT_VMCNT(0);
+            // everyone's part of slab kt is in LDS, and everyone is done reading slab kt - 1 (its fragments were
+            // consumed by MFMAs already issued).  A bare barrier: __syncthreads() adds a fence that waits for
+            // every outstanding load, the look-ahead ones included.
+            __builtin_amdgcn_s_barrier();
+            if (kt + NS - 1 < nk)
+                issue(kt + NS - 1, fill);
+            compute(stage);
+            stage = stage + 1 == NS ? 0 : stage + 1;
+            fill  = fill + 1 == NS ? 0 : fill + 1;
+        }
+    } else {
     u32x4 ra0[A_VECS], rb0[B_VECS], ra1[A_VECS], rb1[B_VECS];
 
     // Loads carry no bounds branches: rows past the matrix edge are clamped to the last row (their products
@@ -696,23 +825,10 @@ __global__ void __launch_bounds__(CFG::NT)
     unsigned char *const lds_a0 = lds_dyn, *const lds_b0 = lds_dyn + BM * STRIDE;
     unsigned char *const lds_a1 = lds_dyn + (BM + BN) * STRIDE, *const lds_b1 = lds_a1 + BM * STRIDE;
 
-    Acc acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                acc[i][j][r] = 0;
-
-    const int frag_row = lane & 31;
-    const int frag_off = (lane >> 5) * 16;
-
     // Slab schedule (two slabs in flight in registers, one in LDS being consumed).  The loop body is branch
     // free: look-ahead loads past the last slab are clamped to it and their LDS copy is never consumed.
     // (Forcing the look-ahead loads to the top of each phase with sched_barrier was measured slower: the
     // compiler's own interleaving of loads, LDS traffic and MFMAs is kept.)
-    const int nk   = K / KB;
     const int last = (nk - 1) * KB;
 #define TR_CLAMPK(SLABIDX) (((SLABIDX)*KB) < last ? ((SLABIDX)*KB) : last)
     TR_LOAD_GLOBAL(ra0, rb0, 0);
@@ -735,6 +851,7 @@ __global__ void __launch_bounds__(CFG::NT)
 #undef TR_STORE_LDS
 #undef TR_COMPUTE
 #undef TR_CLAMPK
+    }
 
     typedef typename std::remove_reference<decltype(acc[0][0][0])>::type AccT;
     // Row-contiguous epilogue.  In the accumulator layout one store instruction touches 32 rows with 16 bytes
@@ -873,16 +990,55 @@ inline int pick_tile_config(long M, long N, size_t kbytes) {
     return 222221;
 }
 
+// Experiment hook: "N:K:code,N:K:code,..." forces a configuration code for given (N, K); set from the environment
+// variable TNN_ROCM_GEMM_TUNE at first use, or through tnn_rocm_debug_set_gemm_tune().
+struct TuneEntry { int n, k, cfg; };
+TuneEntry g_tune_table[16];
+int g_tune_count = -1;
+inline void parse_tune(const char *e) {
+    g_tune_count = 0;
+    while (e && *e && g_tune_count < 16) {
+        TuneEntry t;
+        if (sscanf(e, "%d:%d:%d", &t.n, &t.k, &t.cfg) == 3)
+            g_tune_table[g_tune_count++] = t;
+        e = strchr(e, ',');
+        if (e)
+            ++e;
+    }
+}
+inline int tune_override(int N, int K) {
+    if (g_tune_count < 0)
+        parse_tune(getenv("TNN_ROCM_GEMM_TUNE"));
+    for (int i = 0; i < g_tune_count; ++i)
+        if (g_tune_table[i].n == N && g_tune_table[i].k == K)
+            return g_tune_table[i].cfg;
+    return 0;
+}
+
 template <int DT, typename Epi>
 int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb,
                      const Epi &epi) {
     typedef typename GemmTraits<DT>::elem T;
-    int cfg       = g_gemm_force_cfg > 0 ? g_gemm_force_cfg : 0;
+    int cfg       = g_gemm_force_cfg > 0 ? g_gemm_force_cfg : tune_override(N, K);
     size_t kbytes = (size_t)K * sizeof(T);
-    if (cfg == 0)
-        cfg = pick_tile_config(M, N, kbytes);
-    if (DT == TNN_ROCM_F32 && (cfg == 224211 || cfg == 332221 || cfg == 331182))
+    if (cfg == 0) {
+        // slabs that are whole 128-byte multiples go global -> LDS directly; average kernel durations inside a
+        // 12-layer forward at M=3072 on MI355X (fp16, us, register-staged in parentheses): 192x192 three stages
+        // N=3072 K=768 26.7 (28.7); 96x96 k-split three stages N=768 K=3072 25.9 (28.0); 64x64 two stages
+        // N=768 K=768 11.4 (12.3); 128x128 two stages N=2304 K=768 19.1 (256x128 register-staged 20.5)
+        switch (pick_tile_config(M, N, kbytes)) {
+            case 112211: cfg = 2112211; break;
+            case 222221: cfg = 2222221; break;
+            case 224211: cfg = 2222221; break;  // two 128x128 workgroups per CU beat one 256x128 (19.1 vs 20.3)
+            case 332221: cfg = 3332221; break;
+            case 331182: cfg = 3331182; break;
+            default: cfg = pick_tile_config(M, N, kbytes); break;
+        }
+    }
+    if (DT == TNN_ROCM_F32 && (cfg % 1000000 == 224211 || cfg % 1000000 == 332221 || cfg % 1000000 == 331182))
         cfg = 222221;
+    if (DT == TNN_ROCM_F32)
+        cfg %= 1000000;  // the fp32 instantiations are register-staged only
     if (kbytes % (64u << (cfg % 10)) != 0) {
         set_error("gemm: K=%d is not a whole number of slabs for tuning configuration %d", K, cfg);
         return TNN_ROCM_ESHAPE;
@@ -897,6 +1053,16 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
         default: break;
     }
     if constexpr (DT != TNN_ROCM_F32) {
+#define TR_FAST_DL(TMv, TNv, WGMv, WGNv, WGKv, SLABv, NSv)                                                            \
+    return launch_tiled<DT, TileCfg<TMv, TNv, WGMv, WGNv, WGKv, SLABv, NSv>, Epi>(s, A, B, M, N, K, lda, ldb, epi)
+        switch (cfg) {
+            case 2112211: TR_FAST_DL(1, 1, 2, 2, 1, 128, 2);
+            case 2222221: TR_FAST_DL(2, 2, 2, 2, 2, 128, 2);
+            case 3332221: TR_FAST_DL(3, 3, 2, 2, 2, 128, 3);
+            case 3331182: TR_FAST_DL(3, 3, 1, 1, 8, 256, 3);
+            default: break;
+        }
+#undef TR_FAST_DL
         switch (cfg) {
             case 224211: TR_FAST(2, 2, 4, 2, 1, 128);
             case 332221: TR_FAST(3, 3, 2, 2, 2, 128);
@@ -1128,6 +1294,10 @@ int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *
 // kernel, other values select a configuration code of the tiled kernel.
 __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_config(int cfg) {
     g_gemm_force_cfg = cfg;
+    return 0;
+}
+__attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_tune(const char *spec) {
+    parse_tune(spec);
     return 0;
 }
 __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_group_m(int group_m) {
