@@ -169,6 +169,25 @@ TNN_ROCM_API int tnn_rocm_gemm_i8_qkv_split(void *stream, int out_dtype, const i
 TNN_ROCM_API int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *wqkv, const float *bqkv,
                                          void *qk, void *vt, int B, int S, int heads, int K);
 
+/* LayerNorm folded into the projection that reads it: y = LayerNorm(t) over the last axis of t[M,K]
+ * (cpu_layer_norm_layer_acc.cc:86-135) followed by C = act(y W^T + b) (+ residual) (cpu_mat_mul_layer_acc.cc:64-117,
+ * compute_elewise.cc:37-65, cpu_gelu_layer_acc.cc:42-45) as ONE GEMM on the raw t.  The caller prepares, once,
+ *   w_folded[n,k] = gamma[k] * W[n,k] (in dtype),  colsum[n] = sum_k w_folded[n,k],  bias_folded[n] = b[n] + sum_k beta[k] W[n,k];
+ * the kernel takes each row's mean and variance from the A tiles it streams anyway and forms
+ *   y W^T + b = rstd * (t w_folded^T - mean * colsum) + bias_folded       on its fp32 accumulators.
+ * y (optional, [M,K] in dtype) receives LayerNorm(t) itself for the other readers of that tensor (needs gamma, beta).
+ * flags: TNN_ROCM_EPI_GELU, TNN_ROCM_EPI_RESIDUAL (residual [M,N] in dtype).  dtype F16 or BF16; K a multiple of 128
+ * (the whole normalised row is one GEMM row), N a multiple of 8; all tensors dense row-major. */
+TNN_ROCM_API int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folded, const float *bias_folded,
+                                  const float *colsum, const float *gamma, const float *beta, float eps, void *C, void *y,
+                                  int M, int N, int K, int flags, const void *residual);
+
+/* tnn_rocm_gemm_qkv_split on LayerNorm(t), folded the same way (wqkv_folded, bqkv_folded, colsum over the 3H rows). */
+TNN_ROCM_API int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const void *wqkv_folded,
+                                            const float *bqkv_folded, const float *colsum, const float *gamma,
+                                            const float *beta, float eps, void *qk, void *vt, void *y, int B, int S,
+                                            int heads, int K);
+
 /* kv_len[b] = 1 + the last key index whose additive mask value is > threshold (0 if none). */
 TNN_ROCM_API int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_t *kv_len, int B, int S,
                                          float threshold);

@@ -662,3 +662,50 @@ def test_attention_rejects_bad_args():
     q = torch.zeros(1, 1, 8, 32, dtype=torch.float16, device="cuda")
     with pytest.raises(capi.TnnRocmError):
         ops().attention(q, q, q, 1.0)  # head_dim 32 is not implemented
+
+
+# ---- LayerNorm folded into the projections around it ----------------------------------------------
+def _fold_ln_weights(w, bias, gamma, beta, td):
+    """W' = gamma (.) W rounded to the compute type, its row sums, and bias + W beta"""
+    wf = torch.from_numpy((w * gamma[None, :]).astype(np.float32)).to(td)
+    colsum = wf.double().sum(1).float().numpy()
+    b2 = (bias.astype(np.float64) + w.astype(np.float64) @ beta.astype(np.float64)).astype(np.float32)
+    return wf, colsum, b2
+
+
+@pytest.mark.parametrize("M,dtype", [(300, "f16"), (3072, "f16"), (200, "bf16")])
+def test_gemm_layernorm_folded_into_projection(M, dtype):
+    """FFN1 and the QKV projection on LayerNorm(t), given the raw t and the folded weights, against the checker's
+    LayerNorm -> InnerProduct (-> GELU); the LayerNorm output the kernels also leave for other readers against the
+    checker's LayerNorm; non-trivial mean (the folded form subtracts mean * colsum from the accumulators)."""
+    say("LayerNorm folded into a projection M=%d %s" % (M, dtype))
+    td = torch.float16 if dtype == "f16" else torch.bfloat16
+    tol = FP16_TOL if dtype == "f16" else 4e-2
+    H, F, heads, eps = 768, 3072, 12, 1e-5
+    B, S = (M // 100, 104) if M % 100 == 0 else (M // 384, 384)
+    M = B * S
+    rng = np.random.default_rng(M)
+    r32 = lambda *s: rng.standard_normal(s).astype(np.float32)
+    rnd = lambda a: torch.from_numpy(a).to(td).float().numpy()
+    t = rnd(r32(M, H) * 1.7 + 0.8 + r32(M, 1))          # row means up to a few sigma
+    res = rnd(r32(M, F))
+    w1, wqkv = r32(F, H) * 0.05, r32(3 * H, H) * 0.05
+    b1, bqkv = r32(F) * 0.1, r32(3 * H) * 0.1
+    g, be = 1 + 0.2 * r32(H), 0.3 * r32(H) + 0.5
+    D = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(td).cuda()
+    o = ops()
+    y_ref = orc.layernorm(t, g, be, eps)
+    w1f, cs1, b1f = _fold_ln_weights(w1, b1, g, be, td)
+    h, y = o.gemm_ln(D(t), w1f.cuda(), dev(b1f), dev(cs1), eps, gamma=dev(g), beta=dev(be), gelu=True, want_y=True)
+    assert rel_err(host(y), y_ref) <= tol
+    assert rel_err(host(h), orc.gelu(orc.inner_product(y_ref, rnd(w1), b1))) <= tol
+    h2 = o.gemm_ln(D(t), w1f.cuda(), dev(b1f), dev(cs1), eps, residual=D(res))
+    assert rel_err(host(h2), orc.inner_product(y_ref, rnd(w1), b1) + res) <= tol
+    wqf, csq, bqf = _fold_ln_weights(wqkv, bqkv, g, be, td)
+    qk, vt, y2 = o.qkv_split_ln(D(t), wqf.cuda(), dev(bqf), dev(csq), eps, B, S, heads, gamma=dev(g), beta=dev(be),
+                                want_y=True)
+    ref = orc.inner_product(y_ref, rnd(wqkv), bqkv)
+    assert rel_err(host(y2), y_ref) <= tol
+    assert rel_err(host(qk), ref[:, :2 * H]) <= tol
+    vref = ref[:, 2 * H:].reshape(B, S, heads, 64).transpose(0, 2, 3, 1)
+    assert rel_err(host(vt), vref) <= tol

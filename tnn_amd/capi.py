@@ -48,6 +48,8 @@ SIGNATURES = {
     "tnn_rocm_attention_vt": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _l, _l, _l, _l, _l, _l, _l, _l, _l, _l, _l,
                               _l, _f, _vp, _vp],
     "tnn_rocm_gemm_qkv_split": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i],
+    "tnn_rocm_gemm_ln": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
+    "tnn_rocm_gemm_qkv_split_ln": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i],
     "tnn_rocm_mask_to_kv_len": [_vp, _vp, _vp, _i, _i, _f],
     "tnn_rocm_softmax": [_vp, _i, _vp, _vp, _i, _i, _i],
     "tnn_rocm_layernorm": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp, _f],

@@ -77,6 +77,7 @@ template <> struct GemmTraits<TNN_ROCM_F32> {
 // ---- epilogues ----------------------------------------------------------------------------------
 template <int DT> struct FloatEpilogue {
     typedef typename Elem<DT>::type T;
+    static constexpr bool kRowStats = false;
     int flags;
     const float *bias;
     const T *residual;
@@ -145,6 +146,7 @@ template <int DT> struct FloatEpilogue {
 // QKV projection epilogue: columns [0,2H) -> qk[T,2H]; columns [2H,3H) -> V^T[b][head][d][s]
 template <int DT> struct QkvSplitEpilogue {
     typedef typename Elem<DT>::type T;
+    static constexpr bool kRowStats = false;
     const float *bias;
     T *qk;
     T *vt;
@@ -193,7 +195,139 @@ template <int DT> struct QkvSplitEpilogue {
     }
 };
 
+// ---- LayerNorm folded into the projection that reads it ------------------------------------------------------------
+// y = LayerNorm(t) over the last axis (cpu_layer_norm_layer_acc.cc:86-135: per row mean and variance,
+// (t - mean) * rstd * gamma + beta) followed by y W^T + b, as one GEMM on the raw t:
+//     y W^T + b = rstd * (t W'^T - mean * colsum) + b',   W' = gamma (.) W,  colsum[n] = sum_k W'[n,k],  b' = b + W beta.
+// K is the normalised width, so every workgroup streams whole rows of t through LDS anyway: the row sums and sums of
+// squares are taken from the A fragments the waves already hold for the MFMAs (two dot2 instructions per four
+// values), reduced over the workgroup after the main loop, and applied to the accumulators in the epilogue.
+// Other readers of y (the residual additions) still need the tensor: the workgroup of tile column j writes
+// y for the j-th share of the columns of its rows, so the LayerNorm launch disappears without y disappearing.
+struct LnFold {
+    float inv_cols, eps;
+    const float *colsum;        // [N]
+    const float *gamma, *beta;  // [K], for the y side output
+    void *y;                    // [M, K] in the compute type, or nullptr
+};
+
+// row sum and sum of squares of the eight values of an A fragment register quad
+template <int DT> __device__ __forceinline__ void ln_accumulate(const uint4 &frag, float &s1, float &s2) {
+    const uint32_t w[4] = {frag.x, frag.y, frag.z, frag.w};
+    if constexpr (DT == TNN_ROCM_F16) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 one = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            h2 v = __builtin_bit_cast(h2, w[t]);
+            s1   = __builtin_amdgcn_fdot2(v, one, s1, false);
+            s2   = __builtin_amdgcn_fdot2(v, v, s2, false);
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            float lo = __uint_as_float(w[t] << 16), hi = __uint_as_float(w[t] & 0xffff0000u);
+            s1 += lo + hi;
+            s2 = fmaf(lo, lo, fmaf(hi, hi, s2));
+        }
+    }
+}
+
+template <int DT> struct LnFloatEpilogue {
+    typedef typename Elem<DT>::type T;
+    static constexpr bool kRowStats = true;
+    int flags;
+    const float *bias;  // b' (always present)
+    const T *residual;
+    T *C;
+    long ldc;
+    LnFold ln;
+    __device__ __forceinline__ void set_batch(int) {}
+    __device__ __forceinline__ float col_const(int) const { return 0.f; }
+    __device__ __forceinline__ void store(int, int, float, float) const {}  // N % 8 == 0 is required at launch
+    __device__ __forceinline__ bool direct(int) const { return false; }
+    // st = {rstd, mean} of row m
+    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8], float2 st) const {
+        float4 g0 = *reinterpret_cast<const float4 *>(ln.colsum + n), g1 = *reinterpret_cast<const float4 *>(ln.colsum + n + 4);
+        float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
+        const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+        const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+        float v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            v[t] = st.x * (acc[t] - st.y * g[t]) + b[t];
+        if (flags & TNN_ROCM_EPI_GELU) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                v[t] = gelu_erf_fast(v[t]);
+        }
+        constexpr int NV = 8 * sizeof(T) / 16;
+        u32x4 packed[NV];
+        T *pe = reinterpret_cast<T *>(packed);
+        if (flags & TNN_ROCM_EPI_RESIDUAL) {
+            const u32x4 *rp = reinterpret_cast<const u32x4 *>(residual + (size_t)m * ldc + n);
+#pragma unroll
+            for (int q = 0; q < NV; ++q)
+                packed[q] = rp[q];
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                v[t] += Elem<DT>::ld(&pe[t]);
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            Elem<DT>::st(&pe[t], v[t]);
+        u32x4 *cp = reinterpret_cast<u32x4 *>(C + (size_t)m * ldc + n);
+#pragma unroll
+        for (int q = 0; q < NV; ++q)
+            cp[q] = packed[q];
+    }
+};
+
+// QKV projection of LayerNorm(t): QkvSplitEpilogue's layout with the folded-LayerNorm correction on the accumulators
+template <int DT> struct LnQkvSplitEpilogue {
+    typedef typename Elem<DT>::type T;
+    static constexpr bool kRowStats = true;
+    const float *bias;
+    T *qk;
+    T *vt;
+    int H, S, heads;
+    LnFold ln;
+    __device__ __forceinline__ void set_batch(int) {}
+    __device__ __forceinline__ float col_const(int) const { return 0.f; }
+    __device__ __forceinline__ void store(int, int, float, float) const {}
+    __device__ __forceinline__ bool direct(int n0) const { return n0 >= 2 * H; }
+    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8], float2 st) const {
+        float4 g0 = *reinterpret_cast<const float4 *>(ln.colsum + n), g1 = *reinterpret_cast<const float4 *>(ln.colsum + n + 4);
+        float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
+        const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+        const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+        float v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            v[t] = st.x * (acc[t] - st.y * g[t]) + b[t];
+        if (n < 2 * H) {
+            constexpr int NV = 8 * sizeof(T) / 16;
+            u32x4 packed[NV];
+            T *pe = reinterpret_cast<T *>(packed);
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                Elem<DT>::st(&pe[t], v[t]);
+            u32x4 *cp = reinterpret_cast<u32x4 *>(qk + (size_t)m * 2 * H + n);
+#pragma unroll
+            for (int q = 0; q < NV; ++q)
+                cp[q] = packed[q];
+        } else {
+            int c = n - 2 * H, bb = m / S, s_ = m - bb * S;
+            T *dst = vt + (((size_t)bb * heads + (c >> 6)) * 64 + (c & 63)) * S + s_;
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                Elem<DT>::st(dst + (size_t)t * S, v[t]);
+        }
+    }
+};
+
 struct Int8Epilogue {
+    static constexpr bool kRowStats = false;
     const int32_t *bias;
     const float *scale;
     int8_t *out;
@@ -310,6 +444,7 @@ struct Int8Epilogue {
 // QkvSplitEpilogue: columns [0,2H) -> qk[T,2H]; columns [2H,3H) -> V^T[b][head][d][s].
 template <int DT> struct Int8QkvSplitEpilogue {
     typedef typename Elem<DT>::type T;
+    static constexpr bool kRowStats = false;
     const int32_t *bias;
     const float *scale;
     const float *dequant;
@@ -673,6 +808,12 @@ __global__ void __launch_bounds__(CFG::NT)
     const int frag_off = (lane >> 5) * 16;
     const int nk       = K / KB;
 
+    // LayerNorm-folding epilogues: this lane's share of sum / sum of squares of A row (wm * TM + i) * 32 + frag_row
+    float ln_s1[TM], ln_s2[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+        ln_s1[i] = ln_s2[i] = 0.f;
+
     if constexpr (CFG::NSTAGE > 0) {
         // Direct-to-LDS pipeline.  One load instruction of a wave fills 1024 contiguous LDS bytes (lane L writes
         // bytes 16L..16L+15), i.e. RPL whole slab rows; the lane picks WHICH 16 global bytes land there, so the
@@ -741,6 +882,13 @@ __global__ void __launch_bounds__(CFG::NT)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     fb[j] = *reinterpret_cast<const uint4 *>(sb + (wn * TN + j) * 32 * SLAB + frow + chunk);
+                if constexpr (Epi::kRowStats) {
+                    // the WGN waves that hold the same A rows share the work: wave wn takes the row groups i = wn mod WGN
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+                        if (i % WGN == wn)
+                            ln_accumulate<DT>(fa[i], ln_s1[i], ln_s2[i]);
+                }
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -870,6 +1018,30 @@ __global__ void __launch_bounds__(CFG::NT)
     AccT *const stage_me  = stage_all + wave * (32 * SSTR);  // wave = (wm*WGN + wn)*WGK + wk
     const bool by_rows = epi.direct(n0);
     __syncthreads();  // every wave is done reading the slabs
+    // LayerNorm-folding epilogues: reduce the lanes' partial row sums over the two k-halves of a fragment and the WGK
+    // k-waves (fixed order), giving {rstd, mean} per tile row; both arrays sit behind the staging area
+    float2 *const row_st   = reinterpret_cast<float2 *>(lds_dyn + CFG::stage_bytes);  // [BM]
+    float2 *const row_part = row_st + BM;                                             // [WGK * 2][BM]
+    if constexpr (Epi::kRowStats) {
+        static_assert(CFG::NSTAGE > 0, "LayerNorm-folding epilogues run on the direct-to-LDS pipeline");
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            if (i % WGN == wn)
+                row_part[(wk * 2 + (lane >> 5)) * BM + (wm * TM + i) * 32 + frag_row] = make_float2(ln_s1[i], ln_s2[i]);
+        __syncthreads();
+        if (tid < BM) {
+            double s1 = 0.0, s2 = 0.0;
+            for (int q = 0; q < WGK * 2; ++q) {
+                float2 v = row_part[q * BM + tid];
+                s1 += (double)v.x;
+                s2 += (double)v.y;
+            }
+            const double mean = s1 * (double)epi.ln.inv_cols;
+            const double var  = s2 * (double)epi.ln.inv_cols - mean * mean;
+            row_st[tid]       = make_float2((float)(1.0 / sqrt(var + (double)epi.ln.eps)), (float)mean);
+        }
+        // row_st is read after the first staging barrier below
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -899,7 +1071,12 @@ __global__ void __launch_bounds__(CFG::NT)
             }
             const int m = m0 + ((pos / WGN) * TM + i) * 32 + row;
             const int n = n0 + (pos % WGN) * CW + c8;
-            if (m < M) {
+            if constexpr (Epi::kRowStats) {
+                if (m < M && n + 7 < N) {  // N is a multiple of 8 for these epilogues (checked at launch)
+                    AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    epi.store8(m, n, v, row_st[m - m0]);
+                }
+            } else if (m < M) {
                 AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 if (n + 7 < N) {
                     epi.store8(m, n, v);
@@ -914,6 +1091,33 @@ __global__ void __launch_bounds__(CFG::NT)
         if (i + 1 < TM)
             __syncthreads();
     }
+    if constexpr (Epi::kRowStats) {
+        // y = LayerNorm(t) for this tile's rows and its share of the K columns (eight-column groups dealt out evenly
+        // over the tile columns), in the LayerNorm kernel's half-precision form x * rstd * gamma + (beta - mean * rstd * gamma)
+        if (epi.ln.y) {
+            typedef typename GemmTraits<DT>::elem TY;
+            const int groups = K / 8, tn = n0 / BN;
+            const int g0 = (int)((long)tn * groups / tiles_n), g1 = (int)((long)(tn + 1) * groups / tiles_n);
+            const int gw = g1 - g0;
+            for (int item = tid; item < BM * gw; item += NT) {
+                const int row = item / gw, c = (g0 + item % gw) * 8, m = m0 + row;
+                if (m >= M)
+                    continue;
+                const float2 st = row_st[row];
+                const float mrs = st.y * st.x;
+                float4 k0 = *reinterpret_cast<const float4 *>(epi.ln.gamma + c), k1 = *reinterpret_cast<const float4 *>(epi.ln.gamma + c + 4);
+                float4 e0 = *reinterpret_cast<const float4 *>(epi.ln.beta + c), e1 = *reinterpret_cast<const float4 *>(epi.ln.beta + c + 4);
+                const float kk[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+                const float ee[8] = {e0.x, e0.y, e0.z, e0.w, e1.x, e1.y, e1.z, e1.w};
+                u32x4 raw = *reinterpret_cast<const u32x4 *>(A + (size_t)m * lda + c);
+                TY *pe    = reinterpret_cast<TY *>(&raw);
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    Elem<DT>::st(&pe[t], Elem<DT>::ld(&pe[t]) * st.x * kk[t] + (ee[t] - mrs * kk[t]));
+                *reinterpret_cast<u32x4 *>(reinterpret_cast<TY *>(epi.ln.y) + (size_t)m * K + c) = raw;
+            }
+        }
+    }
 }
 
 // tuning override for experiments: 0 = heuristic, otherwise a configuration code of the tiled kernel
@@ -925,6 +1129,10 @@ int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int 
     typedef typename GemmTraits<DT>::elem T;
     int tiles_m = (M + CFG::BM - 1) / CFG::BM, tiles_n = (N + CFG::BN - 1) / CFG::BN;
     size_t lds  = CFG::lds_bytes;
+    if (Epi::kRowStats) {  // row statistics and the partial-sum buffer sit behind the staging area
+        size_t need = CFG::stage_bytes + (size_t)CFG::BM * 8 * (1 + 2 * CFG::WGK);
+        lds         = lds > need ? lds : need;
+    }
     auto kern   = gemm_nk_tiled_kernel<DT, CFG, Epi>;
     if (lds > 64 * 1024) {
         static bool attr_set = false;  // per instantiation
@@ -1045,6 +1253,21 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
     }
 #define TR_FAST(TMv, TNv, WGMv, WGNv, WGKv, SLABv)                                                                    \
     return launch_tiled<DT, TileCfg<TMv, TNv, WGMv, WGNv, WGKv, SLABv>, Epi>(s, A, B, M, N, K, lda, ldb, epi)
+#define TR_FAST_DL(TMv, TNv, WGMv, WGNv, WGKv, SLABv, NSv)                                                            \
+    return launch_tiled<DT, TileCfg<TMv, TNv, WGMv, WGNv, WGKv, SLABv, NSv>, Epi>(s, A, B, M, N, K, lda, ldb, epi)
+    if constexpr (Epi::kRowStats) {
+        // the LayerNorm-folding epilogues exist for the direct-to-LDS pipeline only (half types, 128-byte slabs)
+        switch (cfg % 1000000) {
+            case 112211: TR_FAST_DL(1, 1, 2, 2, 1, 128, 2);
+            case 222221:
+            case 224211: TR_FAST_DL(2, 2, 2, 2, 2, 128, 2);
+            case 332221: TR_FAST_DL(3, 3, 2, 2, 2, 128, 3);
+            case 331182: TR_FAST_DL(3, 3, 1, 1, 8, 256, 3);
+            default: break;
+        }
+        set_error("gemm: tuning configuration %d has no LayerNorm-folding form", cfg);
+        return TNN_ROCM_EINVAL;
+    } else {
     switch (cfg) {
         case 112210: TR_FAST(1, 1, 2, 2, 1, 64);
         case 112211: TR_FAST(1, 1, 2, 2, 1, 128);
@@ -1053,8 +1276,6 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
         default: break;
     }
     if constexpr (DT != TNN_ROCM_F32) {
-#define TR_FAST_DL(TMv, TNv, WGMv, WGNv, WGKv, SLABv, NSv)                                                            \
-    return launch_tiled<DT, TileCfg<TMv, TNv, WGMv, WGNv, WGKv, SLABv, NSv>, Epi>(s, A, B, M, N, K, lda, ldb, epi)
         switch (cfg) {
             case 2112211: TR_FAST_DL(1, 1, 2, 2, 1, 128, 2);
             case 2222221: TR_FAST_DL(2, 2, 2, 2, 2, 128, 2);
@@ -1062,7 +1283,6 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
             case 3331182: TR_FAST_DL(3, 3, 1, 1, 8, 256, 3);
             default: break;
         }
-#undef TR_FAST_DL
         switch (cfg) {
             case 224211: TR_FAST(2, 2, 4, 2, 1, 128);
             case 332221: TR_FAST(3, 3, 2, 2, 2, 128);
@@ -1070,7 +1290,9 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
             default: break;
         }
     }
+    }
 #undef TR_FAST
+#undef TR_FAST_DL
     set_error("gemm: unknown tuning configuration %d", cfg);
     return TNN_ROCM_EINVAL;
 }
@@ -1288,6 +1510,77 @@ int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *
     else
         TR_QKV(TNN_ROCM_BF16)
 #undef TR_QKV
+}
+
+int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folded, const float *bias_folded,
+                     const float *colsum, const float *gamma, const float *beta, float eps, void *C, void *y, int M, int N,
+                     int K, int flags, const void *residual) {
+    TR_REQUIRE(M >= 0 && N >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_ln: negative size");
+    if (M == 0 || N == 0)
+        return 0;
+    TR_REQUIRE(t && w_folded && bias_folded && colsum && C, TNN_ROCM_EINVAL, "gemm_ln: null pointer");
+    TR_REQUIRE(!y || (gamma && beta), TNN_ROCM_EINVAL, "gemm_ln: the LayerNorm output needs gamma and beta");
+    TR_REQUIRE(dtype == TNN_ROCM_F16 || dtype == TNN_ROCM_BF16, TNN_ROCM_EDTYPE, "gemm_ln: F16 or BF16 only");
+    TR_REQUIRE(K > 0 && K % 128 == 0 && N % 8 == 0, TNN_ROCM_ESHAPE,
+               "gemm_ln: K=%d must be a positive multiple of 128 and N=%d a multiple of 8", K, N);
+    TR_REQUIRE((long)M < (1l << 24) && (long)M * K < (1l << 31) && (long)N * K < (1l << 31) && (long)M * N < (1l << 31),
+               TNN_ROCM_ESHAPE, "gemm_ln: problem too large for 32-bit panel offsets");
+    TR_REQUIRE(!(flags & TNN_ROCM_EPI_RESIDUAL) || residual, TNN_ROCM_EINVAL, "gemm_ln: residual flag without a residual");
+    TR_REQUIRE(al16(t) && al16(w_folded) && al16(C) && al16(bias_folded) && al16(colsum) && (!residual || al16(residual)) &&
+                   (!y || (al16(y) && al16(gamma) && al16(beta))),
+               TNN_ROCM_EALIGN, "gemm_ln: pointers must be 16-byte aligned");
+#define TR_LN(DT)                                                                                                     \
+    {                                                                                                                 \
+        LnFloatEpilogue<DT> epi;                                                                                      \
+        epi.flags    = flags;                                                                                         \
+        epi.bias     = bias_folded;                                                                                   \
+        epi.residual = (const Elem<DT>::type *)residual;                                                              \
+        epi.C        = (Elem<DT>::type *)C;                                                                           \
+        epi.ldc      = N;                                                                                             \
+        epi.ln       = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y};                                          \
+        return launch_gemm_fast<DT, LnFloatEpilogue<DT>>((hipStream_t)stream, t, w_folded, M, N, K, K, K, epi);       \
+    }
+    if (dtype == TNN_ROCM_F16)
+        TR_LN(TNN_ROCM_F16)
+    else
+        TR_LN(TNN_ROCM_BF16)
+#undef TR_LN
+}
+
+int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const void *wqkv_folded, const float *bqkv_folded,
+                               const float *colsum, const float *gamma, const float *beta, float eps, void *qk, void *vt,
+                               void *y, int B, int S, int heads, int K) {
+    TR_REQUIRE(B >= 0 && S >= 0 && heads >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_qkv_split_ln: negative size");
+    if (B == 0 || S == 0 || heads == 0)
+        return 0;
+    TR_REQUIRE(t && wqkv_folded && bqkv_folded && colsum && qk && vt, TNN_ROCM_EINVAL, "gemm_qkv_split_ln: null pointer");
+    TR_REQUIRE(!y || (gamma && beta), TNN_ROCM_EINVAL, "gemm_qkv_split_ln: the LayerNorm output needs gamma and beta");
+    TR_REQUIRE(dtype == TNN_ROCM_F16 || dtype == TNN_ROCM_BF16, TNN_ROCM_EDTYPE, "gemm_qkv_split_ln: F16 or BF16 only");
+    TR_REQUIRE(K > 0 && K % 128 == 0 && S % 8 == 0, TNN_ROCM_ESHAPE,
+               "gemm_qkv_split_ln: K=%d must be a positive multiple of 128 and S=%d a multiple of 8", K, S);
+    TR_REQUIRE((long)B * S < (1l << 24) && (long)B * S * 3 * heads * 64 < (1l << 31), TNN_ROCM_ESHAPE,
+               "gemm_qkv_split_ln: problem too large for 32-bit panel offsets");
+    TR_REQUIRE(al16(t) && al16(wqkv_folded) && al16(qk) && al16(vt) && al16(bqkv_folded) && al16(colsum) &&
+                   (!y || (al16(y) && al16(gamma) && al16(beta))),
+               TNN_ROCM_EALIGN, "gemm_qkv_split_ln: pointers must be 16-byte aligned");
+    const int H = heads * 64, T = B * S;
+#define TR_QKVLN(DT)                                                                                                  \
+    {                                                                                                                 \
+        LnQkvSplitEpilogue<DT> epi;                                                                                   \
+        epi.bias  = bqkv_folded;                                                                                      \
+        epi.qk    = (Elem<DT>::type *)qk;                                                                             \
+        epi.vt    = (Elem<DT>::type *)vt;                                                                             \
+        epi.H     = H;                                                                                                \
+        epi.S     = S;                                                                                                \
+        epi.heads = heads;                                                                                            \
+        epi.ln    = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y};                                             \
+        return launch_gemm_fast<DT, LnQkvSplitEpilogue<DT>>((hipStream_t)stream, t, wqkv_folded, T, 3 * H, K, K, K, epi); \
+    }
+    if (dtype == TNN_ROCM_F16)
+        TR_QKVLN(TNN_ROCM_F16)
+    else
+        TR_QKVLN(TNN_ROCM_BF16)
+#undef TR_QKVLN
 }
 
 // Experiment hook (not part of the documented ABI): 0 restores the shape heuristic, -1 forces the baseline

@@ -861,6 +861,11 @@ struct FusedLinearLayer : BaseLayer {
             out.back() = p->num_output;
         }
         output_blobs_[0]->GetBlobDesc().dims = out;
+        if (p->ln_y) {  // LayerNorm(x) for the other readers of that tensor
+            if (output_blobs_.size() != 2)
+                return Status(TNNERR_PARAM_ERR, "fused linear: the LayerNorm output needs a second output blob");
+            output_blobs_[1]->GetBlobDesc().dims = input_blobs_[0]->GetBlobDesc().dims;
+        }
         return TNN_OK;
     }
 };

@@ -62,6 +62,9 @@ public:
         FoldResidual();
         if (half_)
             FuseAttention();  // the attention kernel computes in fp16; fp32 nets keep the decomposed core
+        const char *fold = getenv("TNN_ROCM_FOLD_LN");
+        if (half_ && !(fold && fold[0] == '0'))
+            FoldLayerNorm();
         return TNN_OK;
     }
 
@@ -459,6 +462,83 @@ private:
         }
     }
 
+    // LayerNorm(t, gamma, beta -> y) whose output is the A operand of exactly one RocmFusedLinear, or the input of
+    // one RocmFusedAttention: that layer reads t instead and applies the normalisation inside its GEMM (see
+    // LnFloatEpilogue in the GEMM source); the LayerNorm launch disappears.  If y has other readers (the residual
+    // additions) the layer also writes y, as a second output; they must come after it in the layer order.
+    // gamma / beta must be constants over the last axis, a multiple of 128 wide.
+    void FoldLayerNorm() {
+        auto &L = structure_->layers;
+        auto constant = [&](const std::string &name, int count) -> RawBuffer * {
+            auto it = resource_->constant_map.find(name);
+            if (it == resource_->constant_map.end() || !it->second || it->second->GetDataType() != DATA_TYPE_FLOAT ||
+                it->second->GetDataCount() != count)
+                return nullptr;
+            return it->second.get();
+        };
+        for (int li = 0; li < (int)L.size(); ++li) {
+            auto ln = L[li];
+            if (!ln || ln->type != LAYER_LAYER_NORM || ln->inputs.size() != 3 || ln->outputs.size() != 1 || ln->param->quantized)
+                continue;
+            GraphIndex g(L);
+            auto lp = ParamOf<LayerNormLayerParam>(ln);
+            const std::string t = ln->inputs[0], y = ln->outputs[0];
+            auto cit = g.consumers.find(y);
+            if (!lp || lp->reduce_dims_size != 1 || IsModelOutput(y) || cit == g.consumers.end())
+                continue;
+            int owner = -1, owners = 0, C = 0;
+            for (int ci : cit->second) {
+                auto c = L[ci];
+                if (!c || c->inputs[0] != y)
+                    continue;
+                if (c->type == LAYER_ROCM_FUSED_LINEAR) {
+                    auto cp = ParamOf<RocmFusedLinearParam>(c);
+                    auto cr = ResOf<RocmFusedLinearResource>(c->name);
+                    if (cr && !cp->ln_fold && cp->num_output % 8 == 0 && std::count(c->inputs.begin(), c->inputs.end(), y) == 1)
+                        owner = ci, C = cr->weight_nk.GetBufferDims()[1];
+                    ++owners;
+                } else if (c->type == LAYER_ROCM_FUSED_ATTENTION) {
+                    auto cp = ParamOf<RocmFusedAttentionParam>(c);
+                    if (!cp->quant && !cp->ln_fold && cp->seq_len > 0 && cp->seq_len % 8 == 0 &&
+                        std::count(c->inputs.begin(), c->inputs.end(), y) == 1)
+                        owner = ci, C = cp->heads * cp->head_dim;
+                    ++owners;
+                }
+            }
+            if (owners != 1 || owner < li || C <= 0 || C % 128 != 0)
+                continue;
+            RawBuffer *gamma = constant(ln->inputs[1], C), *beta = constant(ln->inputs[2], C);
+            bool others = false, ordered = true;
+            for (int ci : cit->second)
+                if (ci != owner) {
+                    others = true;
+                    ordered &= ci > owner;
+                }
+            if (!gamma || !beta || !ordered)
+                continue;
+            auto c = L[owner];
+            auto cr = ResOf<RocmFusedLinearResource>(c->name);
+            c->inputs[0] = t;
+            cr->ln_gamma = *gamma;
+            cr->ln_beta  = *beta;
+            if (c->type == LAYER_ROCM_FUSED_LINEAR) {
+                auto cp     = ParamOf<RocmFusedLinearParam>(c);
+                cp->ln_fold = 1;
+                cp->ln_y    = others ? 1 : 0;
+                cp->ln_eps  = lp->eps;
+            } else {
+                auto cp     = ParamOf<RocmFusedAttentionParam>(c);
+                cp->ln_fold = 1;
+                cp->ln_y    = others ? 1 : 0;
+                cp->ln_eps  = lp->eps;
+            }
+            if (others)
+                c->outputs.push_back(y);
+            L[li] = nullptr;
+        }
+        Compact();
+    }
+
     NetStructure *structure_ = nullptr;
     NetResource *resource_   = nullptr;
     bool half_               = true;
@@ -827,6 +907,53 @@ struct RegisterRocmFusion {
 
 }  // namespace
 
+// ---- LayerNorm folded into a projection: weight preparation ---------------------------------------------------
+// value of f after rounding to the activation type (round to nearest even, as the device conversion does)
+static float RoundToActivationType(float f, DataType dt) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint32_t sign = x & 0x80000000u, a = x & 0x7fffffffu;
+    if (a >= 0x7f800000u)
+        return f;
+    if (dt == DATA_TYPE_BFP16) {
+        a = (a + 0x7fffu + ((a >> 16) & 1u)) & 0xffff0000u;
+    } else if (a < 0x38800000u) {  // below 2^-14: a multiple of the fp16 subnormal step 2^-24
+        float af;
+        memcpy(&af, &a, 4);
+        af = (af + 0.5f) - 0.5f;  // the sum has an ulp of 2^-24: rounds af to that grid, ties to even
+        memcpy(&a, &af, 4);
+    } else {
+        a = (a + 0xfffu + ((a >> 13) & 1u)) & 0xffffe000u;
+        if (a >= 0x47800000u)  // 65520 and above round to infinity
+            a = 0x7f800000u;
+    }
+    x = sign | a;
+    memcpy(&f, &x, 4);
+    return f;
+}
+
+// y W^T + b with y = (t - mean) * rstd * gamma + beta  ==  rstd * (t W'^T - mean * colsum) + b'
+//   W'[n,k] = gamma[k] W[n,k] (as the device will hold it, i.e. rounded to dt),  colsum[n] = sum_k W'[n,k],
+//   b'[n] = b[n] + sum_k beta[k] W[n,k]
+static void FoldLayerNormIntoWeights(const float *w, const float *bias, const float *gamma, const float *beta, int N, int K,
+                                     DataType dt, std::vector<float> *w_folded, std::vector<float> *colsum,
+                                     std::vector<float> *bias_folded) {
+    w_folded->resize((size_t)N * K);
+    colsum->resize(N);
+    bias_folded->resize(N);
+    for (int n = 0; n < N; ++n) {
+        double cs = 0.0, bs = bias ? (double)bias[n] : 0.0;
+        for (int k = 0; k < K; ++k) {
+            float wf = RoundToActivationType(w[(size_t)n * K + k] * gamma[k], dt);
+            (*w_folded)[(size_t)n * K + k] = wf;
+            cs += (double)wf;
+            bs += (double)beta[k] * (double)w[(size_t)n * K + k];
+        }
+        (*colsum)[n]      = (float)cs;
+        (*bias_folded)[n] = (float)bs;
+    }
+}
+
 // ---- RocmFusedLinear ------------------------------------------------------------------------------------------
 // y[rows,N] = act(x[rows,K] W^T + b) (+ residual): the arithmetic of MatMul+Add (cpu_mat_mul_layer_acc.cc:64-117,
 // compute_elewise.cc:37-65) or InnerProduct (naive_compute.cc:271-288), GELU (cpu_gelu_layer_acc.cc:42-45) and the
@@ -851,11 +978,29 @@ public:
                 return Status(TNNERR_PARAM_ERR, "fused linear: residual must have the output's shape and type");
         }
         DataType dt = inputs[0]->GetBlobDesc().data_type;
-        RETURN_ON_NEQ(UploadConverted(res->weight_nk.force_to<void *>(), (size_t)wd[0] * wd[1], DATA_TYPE_FLOAT, dt, &weight_),
-                      TNN_OK);
-        if (p->has_bias)
-            RETURN_ON_NEQ(UploadConverted(res->bias.force_to<void *>(), (size_t)wd[0], DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &bias_),
+        if (p->ln_fold) {
+            if ((dt != DATA_TYPE_HALF && dt != DATA_TYPE_BFP16) || outputs.size() != (p->ln_y ? 2u : 1u) || in.back() != wd[1] ||
+                wd[1] % 128 != 0 || wd[0] % 8 != 0 || res->ln_gamma.GetDataCount() != wd[1] || res->ln_beta.GetDataCount() != wd[1])
+                return Status(TNNERR_PARAM_ERR, "fused linear with a folded LayerNorm: fp16/bf16 blobs, the last axis (a "
+                                                "multiple of 128) contracted, scale / shift of that width are required");
+            std::vector<float> wf, cs, bf;
+            FoldLayerNormIntoWeights(res->weight_nk.force_to<float *>(), p->has_bias ? res->bias.force_to<float *>() : nullptr,
+                                     res->ln_gamma.force_to<float *>(), res->ln_beta.force_to<float *>(), wd[0], wd[1], dt, &wf,
+                                     &cs, &bf);
+            RETURN_ON_NEQ(UploadConverted(wf.data(), wf.size(), DATA_TYPE_FLOAT, dt, &weight_), TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(bf.data(), bf.size(), DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &bias_), TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(cs.data(), cs.size(), DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &colsum_), TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(res->ln_gamma.force_to<void *>(), (size_t)wd[1], DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &gamma_),
                           TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(res->ln_beta.force_to<void *>(), (size_t)wd[1], DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &beta_),
+                          TNN_OK);
+        } else {
+            RETURN_ON_NEQ(UploadConverted(res->weight_nk.force_to<void *>(), (size_t)wd[0] * wd[1], DATA_TYPE_FLOAT, dt, &weight_),
+                          TNN_OK);
+            if (p->has_bias)
+                RETURN_ON_NEQ(UploadConverted(res->bias.force_to<void *>(), (size_t)wd[0], DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &bias_),
+                              TNN_OK);
+        }
         return TNN_OK;
     }
     Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
@@ -865,6 +1010,13 @@ public:
         int N = p->num_output, rows = DimsVectorUtils::Count(in) / (K > 0 ? K : 1);
         int epi = (p->has_bias ? TNN_ROCM_EPI_BIAS : 0) | (p->gelu ? TNN_ROCM_EPI_GELU : 0) |
                   (p->has_residual ? TNN_ROCM_EPI_RESIDUAL : 0);
+        if (p->ln_fold) {
+            ROCM_CALL(tnn_rocm_gemm_ln(Stream(), (int)inputs[0]->GetBlobDesc().data_type, Ptr(inputs[0]), weight_,
+                                       (const float *)bias_, (const float *)colsum_, (const float *)gamma_, (const float *)beta_,
+                                       p->ln_eps, Ptr(outputs[0]), p->ln_y ? Ptr(outputs[1]) : nullptr, rows, N, K,
+                                       epi & ~TNN_ROCM_EPI_BIAS, p->has_residual ? Ptr(In(inputs[1])) : nullptr));
+            return TNN_OK;
+        }
         ROCM_CALL(tnn_rocm_gemm(Stream(), (int)inputs[0]->GetBlobDesc().data_type, 1, Ptr(inputs[0]), weight_, Ptr(outputs[0]),
                                 rows, N, K, K, K, N, 1, 1, 1, epi, (const float *)bias_,
                                 p->has_residual ? Ptr(In(inputs[1])) : nullptr, N));
@@ -872,7 +1024,7 @@ public:
     }
 
 private:
-    void *weight_ = nullptr, *bias_ = nullptr;
+    void *weight_ = nullptr, *bias_ = nullptr, *colsum_ = nullptr, *gamma_ = nullptr, *beta_ = nullptr;
 };
 REGISTER_ROCM_ACC(RocmFusedLinearLayerAcc, LAYER_ROCM_FUSED_LINEAR);
 
@@ -932,6 +1084,21 @@ public:
             RETURN_ON_NEQ(UploadConverted(scale.data(), (size_t)N, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &scale_), TNN_OK);
             RETURN_ON_NEQ(UploadConverted(dequant.data(), (size_t)N, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &dequant_), TNN_OK);
         }
+        if (!weight_ && p->ln_fold) {
+            if (p->quant || seq_ % 8 != 0 || H_ % 128 != 0 || outputs.size() != (p->ln_y ? 2u : 1u) ||
+                res->ln_gamma.GetDataCount() != H_ || res->ln_beta.GetDataCount() != H_)
+                return Status(TNNERR_PARAM_ERR, "fused attention with a folded LayerNorm: S % 8 == 0, hidden size a multiple "
+                                                "of 128 and scale / shift of that width are required");
+            std::vector<float> wf, cs, bf;
+            FoldLayerNormIntoWeights(res->weight_nk.force_to<float *>(), res->bias.force_to<float *>(),
+                                     res->ln_gamma.force_to<float *>(), res->ln_beta.force_to<float *>(), 3 * H_, H_, dt, &wf, &cs,
+                                     &bf);
+            RETURN_ON_NEQ(UploadConverted(wf.data(), wf.size(), DATA_TYPE_FLOAT, dt, &weight_), TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(bf.data(), bf.size(), DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &bias_), TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(cs.data(), cs.size(), DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &colsum_), TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(res->ln_gamma.force_to<void *>(), (size_t)H_, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &gamma_), TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(res->ln_beta.force_to<void *>(), (size_t)H_, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &beta_), TNN_OK);
+        }
         if (!weight_) {
             RETURN_ON_NEQ(UploadConverted(res->weight_nk.force_to<void *>(), (size_t)3 * H_ * H_, DATA_TYPE_FLOAT, dt, &weight_),
                           TNN_OK);
@@ -972,8 +1139,14 @@ public:
             // projection writes Q|K row-major and V already transposed per head: the attention kernel then stages
             // V tiles with 16-byte copies
             char *vt = (char *)qkv + (size_t)T_ * 2 * H_ * es;
-            ROCM_CALL(tnn_rocm_gemm_qkv_split(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_, qkv, vt, B_,
-                                              seq_, p->heads, H_));
+            if (p->ln_fold)
+                ROCM_CALL(tnn_rocm_gemm_qkv_split_ln(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_,
+                                                     (const float *)colsum_, (const float *)gamma_, (const float *)beta_,
+                                                     p->ln_eps, qkv, vt, p->ln_y ? Ptr(outputs[1]) : nullptr, B_, seq_,
+                                                     p->heads, H_));
+            else
+                ROCM_CALL(tnn_rocm_gemm_qkv_split(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_, qkv, vt,
+                                                  B_, seq_, p->heads, H_));
             const long row = 2L * H_;
             ROCM_CALL(tnn_rocm_attention_vt(Stream(), (int)dt, base, base + (size_t)H_ * es, vt, Ptr(outputs[0]), B_, p->heads,
                                             seq_, p->head_dim, (long)seq_ * row, d, row, (long)seq_ * row, d, row,
@@ -991,7 +1164,8 @@ public:
     }
 
 private:
-    void *weight_ = nullptr, *bias_ = nullptr, *scale_ = nullptr, *dequant_ = nullptr;
+    void *weight_ = nullptr, *bias_ = nullptr, *scale_ = nullptr, *dequant_ = nullptr, *colsum_ = nullptr, *gamma_ = nullptr,
+         *beta_ = nullptr;
     int H_ = 0, K_ = 0, T_ = 0, B_ = 0, seq_ = 0;
 };
 REGISTER_ROCM_ACC(RocmFusedAttentionLayerAcc, LAYER_ROCM_FUSED_ATTENTION);

@@ -275,6 +275,8 @@ struct IntScaleResource : public LayerResource {
 struct RocmFusedLinearResource : public LayerResource {
     RawBuffer weight_nk;  // [N, K] fp32
     RawBuffer bias;       // [N] fp32 (may be empty)
+    // scale / shift ([K] fp32) of a LayerNorm folded into this layer (the one whose output was the A operand)
+    RawBuffer ln_gamma, ln_beta;
 };
 
 using ConstantResource = std::map<std::string, std::shared_ptr<RawBuffer>>;
@@ -377,6 +379,11 @@ struct RocmFusedLinearParam : public LayerParam {
     int gelu         = 0;  // erf GELU applied to (x W^T + b)
     int has_residual = 0;  // second input added after the activation
     int axis         = -1; // -1: contract the last dimension; >= 0: InnerProduct form, contract dims[axis:]
+    // LayerNorm folded into this projection (RocmFusionPass::FoldLayerNorm): input 0 is the tensor the LayerNorm
+    // read, the layer computes act(LayerNorm(x) W^T + b); with ln_y a second output blob receives LayerNorm(x)
+    // itself for the other readers of that tensor.
+    int ln_fold = 0, ln_y = 0;
+    float ln_eps = 0.f;
 };
 struct RocmFusedAttentionParam : public LayerParam {
     int heads    = 0;
@@ -388,6 +395,9 @@ struct RocmFusedAttentionParam : public LayerParam {
     // resource is a RocmFusedQkvInt8Resource and qkv_out_scale are the scales of their three int8 output blobs
     int quant = 0;
     float qkv_out_scale[3] = {0.f, 0.f, 0.f};
+    // LayerNorm folded into the QKV projection, as in RocmFusedLinearParam
+    int ln_fold = 0, ln_y = 0;
+    float ln_eps = 0.f;
 };
 // Gather(word ids) + Add(position constant) + Gather(type ids) + Add + LayerNorm of a BERT-style front end.
 // Inputs: word ids, type ids (int32), gamma, beta (constant blobs); resource: RocmFusedEmbeddingResource.

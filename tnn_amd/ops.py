@@ -117,6 +117,31 @@ def qkv_split(x, wqkv, bqkv, B, S, heads):
     return qk, vt
 
 
+def gemm_ln(t, w_folded, bias_folded, colsum, eps, gamma=None, beta=None, gelu=False, residual=None, want_y=False):
+    """C = act(LayerNorm(t) W^T + b) (+ residual) from the raw t and the folded weights; optionally also LayerNorm(t)"""
+    _chk(t, w_folded, bias_folded, colsum, gamma, beta, residual)
+    M, K = t.shape
+    N = w_folded.shape[0]
+    c = torch.empty(M, N, dtype=t.dtype, device=t.device)
+    y = torch.empty_like(t) if want_y else None
+    flags = (2 if gelu else 0) | (4 if residual is not None else 0)
+    capi.call("tnn_rocm_gemm_ln", _stream(), dt(t), _p(t), _p(w_folded), _p(bias_folded), _p(colsum), _p(gamma), _p(beta),
+              float(eps), _p(c), _p(y), M, N, K, flags, _p(residual))
+    return (c, y) if want_y else c
+
+
+def qkv_split_ln(t, wqkv_folded, bqkv_folded, colsum, eps, B, S, heads, gamma=None, beta=None, want_y=False):
+    """qkv_split on LayerNorm(t) given as the raw t and the folded weights; optionally also LayerNorm(t)"""
+    _chk(t, wqkv_folded, bqkv_folded, colsum, gamma, beta)
+    H = heads * 64
+    qk = torch.empty(B * S, 2 * H, dtype=t.dtype, device=t.device)
+    vt = torch.empty(B, heads, 64, S, dtype=t.dtype, device=t.device)
+    y = torch.empty_like(t) if want_y else None
+    capi.call("tnn_rocm_gemm_qkv_split_ln", _stream(), dt(t), _p(t), _p(wqkv_folded), _p(bqkv_folded), _p(colsum), _p(gamma),
+              _p(beta), float(eps), _p(qk), _p(vt), _p(y), B, S, heads, t.shape[1])
+    return (qk, vt, y) if want_y else (qk, vt)
+
+
 def attention_qk_vt(qk, vt, B, S, heads, scale, mask=None, kv_len=None, out=None):
     """qk [B*S, 2H] (Q | K), vt [B, heads, 64, S]; out [B*S, H]"""
     _chk(qk, vt, mask, kv_len, out)
