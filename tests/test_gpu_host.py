@@ -62,8 +62,10 @@ def test_encoder_from_model_files(precision):
     inst = host.RocmInstance.from_graph(g, precision)
     types = [t for t, _ in inst.layers()]
     if precision == "fp16":
-        # per encoder layer: attention, out-proj(+res), LN, ffn1(+gelu), ffn2(+res), LN = 6 host layers (7 launches)
+        # per encoder layer: attention, out-proj(+res), ffn1(+gelu), ffn2(+res); the LayerNorms are folded into the
+        # projection that reads them (ffn1, the next layer's QKV); only the last one, a model output, stays a layer
         assert types.count("RocmFusedAttention") == 2 and types.count("RocmFusedLinear") == 6
+        assert types.count("LayerNorm") == 1, types
         assert not any(t in ("Softmax", "Permute", "Reshape", "MatMul", "GELU") for t in types), types
     else:
         assert types.count("RocmFusedLinear") == 12 and types.count("Softmax") == 2
@@ -308,3 +310,39 @@ def test_encoder_bf16_from_model_files():
     err = rel_err(got, ref)
     say("  max rel err %.3g" % err)
     assert err <= 4e-2
+
+
+def test_layernorm_folding_switch(monkeypatch):
+    """TNN_ROCM_FOLD_LN=0 keeps every LayerNorm a launch of its own; both graphs agree with each other to fp16
+    rounding and with the checker."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: LayerNorm folding on / off, 2-layer encoder fp16")
+    cfg = EncoderConfig.bert_base(2)
+    w = make_weights(cfg, seed=13, bias_std=0.05)
+    rng = np.random.default_rng(14)
+    for lw in w["layers"]:   # non-trivial LayerNorm scale / shift
+        for k in ("ln1_g", "ln2_g"):
+            lw[k] = (1 + 0.2 * rng.standard_normal(cfg.hidden)).astype(np.float32)
+        for k in ("ln1_b", "ln2_b"):
+            lw[k] = (0.3 * rng.standard_normal(cfg.hidden)).astype(np.float32)
+    B, S = 3, 104
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 30, S, seed=15)
+    g = tnnmodel.encoder_graph(cfg, w, B, S)
+    outs = {}
+    for fold, n_ln in (("0", 4), ("1", 1)):
+        monkeypatch.setenv("TNN_ROCM_FOLD_LN", fold)
+        inst = host.RocmInstance.from_graph(g, "fp16")
+        types = [t for t, _ in inst.layers()]
+        assert types.count("LayerNorm") == n_ln, types
+        inst.set_input("input_ids", ids)
+        inst.set_input("token_type_ids", seg)
+        inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+        for _ in range(4):   # the fourth forward replays the captured graph
+            inst.forward()
+        outs[fold] = inst.output("last_hidden").reshape(B * S, -1)
+        inst.close()
+    wr = r16w(w)
+    ref = encoder_ref.encoder(wr, cfg, encoder_ref.embed(wr, ids, seg, cfg.eps), B, S, mask)
+    e0, e1, e01 = rel_err(outs["0"], ref), rel_err(outs["1"], ref), rel_err(outs["1"], outs["0"])
+    say("  un-folded %.3g  folded %.3g  folded vs un-folded %.3g" % (e0, e1, e01))
+    assert e0 <= FP16_TOL and e1 <= FP16_TOL and e01 <= FP16_TOL

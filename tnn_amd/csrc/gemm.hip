@@ -883,10 +883,10 @@ __global__ void __launch_bounds__(CFG::NT)
                 for (int j = 0; j < TN; ++j)
                     fb[j] = *reinterpret_cast<const uint4 *>(sb + (wn * TN + j) * 32 * SLAB + frow + chunk);
                 if constexpr (Epi::kRowStats) {
-                    // the WGN waves that hold the same A rows share the work: wave wn takes the row groups i = wn mod WGN
+                    // the WGN waves that hold the same A rows take turns over the row groups and k-steps
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
-                        if (i % WGN == wn)
+                        if ((i + kk / WGK) % WGN == wn)
                             ln_accumulate<DT>(fa[i], ln_s1[i], ln_s2[i]);
                 }
 #pragma unroll
@@ -1021,17 +1021,16 @@ __global__ void __launch_bounds__(CFG::NT)
     // LayerNorm-folding epilogues: reduce the lanes' partial row sums over the two k-halves of a fragment and the WGK
     // k-waves (fixed order), giving {rstd, mean} per tile row; both arrays sit behind the staging area
     float2 *const row_st   = reinterpret_cast<float2 *>(lds_dyn + CFG::stage_bytes);  // [BM]
-    float2 *const row_part = row_st + BM;                                             // [WGK * 2][BM]
+    float2 *const row_part = row_st + BM;                                             // [WGK * WGN * 2][BM]
     if constexpr (Epi::kRowStats) {
         static_assert(CFG::NSTAGE > 0, "LayerNorm-folding epilogues run on the direct-to-LDS pipeline");
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-            if (i % WGN == wn)
-                row_part[(wk * 2 + (lane >> 5)) * BM + (wm * TM + i) * 32 + frag_row] = make_float2(ln_s1[i], ln_s2[i]);
+            row_part[((wk * WGN + wn) * 2 + (lane >> 5)) * BM + (wm * TM + i) * 32 + frag_row] = make_float2(ln_s1[i], ln_s2[i]);
         __syncthreads();
         if (tid < BM) {
             double s1 = 0.0, s2 = 0.0;
-            for (int q = 0; q < WGK * 2; ++q) {
+            for (int q = 0; q < WGK * WGN * 2; ++q) {
                 float2 v = row_part[q * BM + tid];
                 s1 += (double)v.x;
                 s2 += (double)v.y;
@@ -1092,15 +1091,15 @@ __global__ void __launch_bounds__(CFG::NT)
             __syncthreads();
     }
     if constexpr (Epi::kRowStats) {
-        // y = LayerNorm(t) for this tile's rows and its share of the K columns (eight-column groups dealt out evenly
-        // over the tile columns), in the LayerNorm kernel's half-precision form x * rstd * gamma + (beta - mean * rstd * gamma)
+        // y = LayerNorm(t) for this tile's share of its rows (the BM rows are dealt out evenly over the tile columns, so
+        // every workgroup writes whole rows), in the LayerNorm kernel's half-precision form
+        // x * rstd * gamma + (beta - mean * rstd * gamma)
         if (epi.ln.y) {
             typedef typename GemmTraits<DT>::elem TY;
             const int groups = K / 8, tn = n0 / BN;
-            const int g0 = (int)((long)tn * groups / tiles_n), g1 = (int)((long)(tn + 1) * groups / tiles_n);
-            const int gw = g1 - g0;
-            for (int item = tid; item < BM * gw; item += NT) {
-                const int row = item / gw, c = (g0 + item % gw) * 8, m = m0 + row;
+            const int r0 = (int)((long)tn * BM / tiles_n), r1 = (int)((long)(tn + 1) * BM / tiles_n);
+            for (int item = tid; item < (r1 - r0) * groups; item += NT) {
+                const int row = r0 + item / groups, c = (item % groups) * 8, m = m0 + row;
                 if (m >= M)
                     continue;
                 const float2 st = row_st[row];
@@ -1130,7 +1129,7 @@ int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int 
     int tiles_m = (M + CFG::BM - 1) / CFG::BM, tiles_n = (N + CFG::BN - 1) / CFG::BN;
     size_t lds  = CFG::lds_bytes;
     if (Epi::kRowStats) {  // row statistics and the partial-sum buffer sit behind the staging area
-        size_t need = CFG::stage_bytes + (size_t)CFG::BM * 8 * (1 + 2 * CFG::WGK);
+        size_t need = CFG::stage_bytes + (size_t)CFG::BM * 8 * (1 + 2 * CFG::WGK * CFG::WGN);
         lds         = lds > need ? lds : need;
     }
     auto kern   = gemm_nk_tiled_kernel<DT, CFG, Epi>;
