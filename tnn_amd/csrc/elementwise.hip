@@ -8,6 +8,7 @@
 using namespace tnn_rocm;
 
 namespace {
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBlock     = 256;
 constexpr int kMaxBlocks = 256 * 16;
@@ -300,14 +301,38 @@ __global__ void __launch_bounds__(kBlock) add_i8_kernel(const int8_t *__restrict
     }
 }
 
-__global__ void __launch_bounds__(kBlock) gelu_i8_kernel(const int8_t *__restrict__ qi, float in_scale,
-                                                         float out_inv, int8_t *__restrict__ qo, size_t n) {
-    size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        float x = __fmul_rn((float)qi[i], in_scale);
-        float g = gelu_erf(x);
-        qo[i]   = float2int8_ref(__fmul_rn(g, out_inv));
+// int8 -> GELU -> int8 has only 256 possible inputs: every workgroup first tabulates the exact chain
+// (dequantise, erf GELU, quantise: one entry per thread) in LDS, then maps bytes through the table, sixteen per
+// thread and access.  Value for value the same as evaluating the chain per element.
+__global__ void __launch_bounds__(256) gelu_i8_kernel(const int8_t *__restrict__ qi, float in_scale, float out_inv,
+                                                      int8_t *__restrict__ qo, size_t n, int vector_ok) {
+    __shared__ int8_t table[256];
+    {
+        const int q = (int)threadIdx.x - 128;
+        float x     = __fmul_rn((float)q, in_scale);
+        float g     = gelu_erf(x);
+        table[threadIdx.x] = float2int8_ref(__fmul_rn(g, out_inv));
     }
+    __syncthreads();
+    const size_t stride = (size_t)gridDim.x * blockDim.x, first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t nvec   = vector_ok ? n / 16 : 0;
+    for (size_t i = first; i < nvec; i += stride) {
+        u32x4 v = reinterpret_cast<const u32x4 *>(qi)[i];
+        u32x4 o;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            uint32_t in = v[w], out = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                uint32_t idx = (((in >> (8 * b)) & 0xffu) ^ 0x80u);  // int8 value + 128
+                out |= (uint32_t)(uint8_t)table[idx] << (8 * b);
+            }
+            o[w] = out;
+        }
+        reinterpret_cast<u32x4 *>(qo)[i] = o;
+    }
+    for (size_t i = nvec * 16 + first; i < n; i += stride)
+        qo[i] = table[(int)qi[i] + 128];
 }
 
 }  // namespace
@@ -540,8 +565,11 @@ int tnn_rocm_gelu_i8(void *stream, const int8_t *qi, float in_scale, float out_i
     if (n == 0)
         return 0;
     TR_REQUIRE(qi && qo, TNN_ROCM_EINVAL, "gelu_i8: null pointer");
-    hipLaunchKernelGGL(gelu_i8_kernel, dim3(grid_for(n)), dim3(kBlock), 0, (hipStream_t)stream, qi, in_scale,
-                       out_inv_scale, qo, n);
+    const int vector_ok = ((uintptr_t)qi % 16 == 0 && (uintptr_t)qo % 16 == 0) ? 1 : 0;
+    size_t blocks       = (n / 16 + 255) / 256;
+    blocks              = blocks < 1 ? 1 : (blocks > 2048 ? 2048 : blocks);
+    hipLaunchKernelGGL(gelu_i8_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, qi, in_scale,
+                       out_inv_scale, qo, n, vector_ok);
     TR_CHECK_LAUNCH();
     return 0;
 }
