@@ -142,6 +142,16 @@ TNN_ROCM_API int tnn_rocm_attention_vt(void *stream, int dtype, const void *q, c
                                        long k_sb, long k_sh, long k_ss, long vt_sb, long vt_sh, long vt_sd, long o_sb,
                                        long o_sh, long o_ss, float scale, const float *mask, const int32_t *kv_len);
 
+/* tnn_rocm_attention_vt that also writes the output quantised to int8 (out_q, same element strides as out; NULL = not
+ * wanted): q = float2int8(out * out_q_inv_scale) on the values as stored in out, i.e. the Reformat(float -> int8) layer
+ * that follows the attention block of a quantised net (x86_reformat_layer_acc / naive float2int8: multiply by
+ * 1/scale, round half away from zero, saturate), in the same launch. */
+TNN_ROCM_API int tnn_rocm_attention_vt_q8(void *stream, int dtype, const void *q, const void *k, const void *vt, void *out,
+                                          int8_t *out_q, float out_q_inv_scale, int B, int heads, int S, int head_dim,
+                                          long q_sb, long q_sh, long q_ss, long k_sb, long k_sh, long k_ss, long vt_sb,
+                                          long vt_sh, long vt_sd, long o_sb, long o_sh, long o_ss, float scale,
+                                          const float *mask, const int32_t *kv_len);
+
 /* The int8 GEMM above with a float consumer folded in: out_f = (float)q * dequant_scale (+ residual), where q is
  * the requantised int8 value of tnn_rocm_gemm_i8 (never written).  This is QuantizedInnerProduct -> Reformat
  * (int8 -> float, x86_compute_int8.cc:1193-1252) -> Add(residual) (compute_elewise.cc:37-65) in one launch; the

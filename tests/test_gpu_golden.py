@@ -142,11 +142,13 @@ def test_int8_encoder_with_folded_reformat_layers(precision, monkeypatch):
     say("  folded:   " + " ".join("%s x%d" % (t, types["1"].count(t)) for t in sorted(set(types["1"]))))
     assert types["0"].count("Reformat") == 10 and types["0"].count("QuantizedInnerProduct") == 6
     assert types["1"].count("RocmGeluInt8") == 1 and types["1"].count("QuantizedInnerProduct") == 1
-    assert types["1"].count("Reformat") == 2  # the encoder input and the attention output are still quantised apart
     if precision == "fp16":
+        # only the encoder input is still quantised by a layer of its own: the attention kernel writes its quantised
+        # context itself
+        assert types["1"].count("Reformat") == 1
         assert types["1"].count("RocmFusedAttention") == 1 and types["1"].count("RocmFusedLinearInt8") == 2
     else:  # fp32 keeps the decomposed attention core; the q, k, v projections still fold their Reformat layers
-        assert types["1"].count("RocmFusedLinearInt8") == 5
+        assert types["1"].count("Reformat") == 2 and types["1"].count("RocmFusedLinearInt8") == 5
         assert np.array_equal(outs["0"], outs["1"])
     ref = f["x86_last_hidden"].reshape(outs["1"].shape)
     err = rel_err(outs["1"], ref)

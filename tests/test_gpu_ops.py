@@ -709,3 +709,25 @@ def test_gemm_layernorm_folded_into_projection(M, dtype):
     assert rel_err(host(qk), ref[:, :2 * H]) <= tol
     vref = ref[:, 2 * H:].reshape(B, S, heads, 64).transpose(0, 2, 3, 1)
     assert rel_err(host(vt), vref) <= tol
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_attention_quantised_second_output_bit_exact(dtype):
+    """The int8 tensor the attention kernel can write next to its output equals the checker's x86 quantiser applied to
+    that output (the Reformat layer it replaces), bit for bit; the float output is unchanged by asking for it."""
+    say("attention with a quantised second output, " + dtype)
+    td = torch.float16 if dtype == "f16" else torch.bfloat16
+    B, S, heads, H = 3, 200, 12, 768
+    g = torch.Generator().manual_seed(5)
+    qk = torch.randn(B * S, 2 * H, generator=g).to(td).cuda()
+    vt = torch.randn(B, heads, 64, S, generator=g).to(td).cuda()
+    lens = torch.tensor([200, 77, 130], dtype=torch.int32).cuda()
+    scale = np.float32(0.0173)
+    inv = np.float32(1.0 / scale)
+    plain = ops().attention_qk_vt(qk, vt, B, S, heads, 0.125, kv_len=lens)
+    out, out_q = ops().attention_qk_vt(qk, vt, B, S, heads, 0.125, kv_len=lens, q8_inv_scale=inv)
+    assert torch.equal(plain, out)
+    ref_q = orc.quantize_x86(out.float().cpu().numpy(), scale)
+    assert np.array_equal(host(out_q), ref_q)
+    assert np.array_equal(host(out_q), host(ops().quantize(out, inv)))
+    assert np.abs(host(out_q).astype(int)).max() >= 30  # the scale makes real use of the int8 range

@@ -37,6 +37,7 @@ template <> struct AttnT<TNN_ROCM_F16> {
         c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
                                                    0);
     }
+    static __device__ __forceinline__ float to_float(uint16_t bits) { return (float)__builtin_bit_cast(half_t, bits); }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         half_t l = (half_t)lo, h = (half_t)hi;
         return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
@@ -58,6 +59,7 @@ template <> struct AttnT<TNN_ROCM_BF16> {
         c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
                                                     0, 0);
     }
+    static __device__ __forceinline__ float to_float(uint16_t bits) { return __uint_as_float((uint32_t)bits << 16); }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
     }
@@ -77,6 +79,8 @@ struct AttnParams {
     float scale_log2e;  // scale * log2(e)
     const float *mask;  // [B,S] additive or null
     const int32_t *kv_len;
+    int8_t *oq;   // optional second output: the stored values quantised, same element strides as o
+    float q_inv;  // 1 / scale of that int8 tensor
 };
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -384,9 +388,28 @@ __global__ void __launch_bounds__(NW * 64, 2) attention_kernel(AttnParams p) {
         for (int pass = 0; pass < 4; ++pass) {
             const int r    = pass * 8 + (lane >> 3);
             const int qrow = q0 + r;
-            if (qrow < S)
-                *reinterpret_cast<u32x4 *>(ob + (size_t)qrow * p.o_ss + (lane & 7) * 8) =
-                    *reinterpret_cast<const u32x4 *>(stage + r * kRowBytes + (lane & 7) * 16);
+            if (qrow < S) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + r * kRowBytes + (lane & 7) * 16);
+                *reinterpret_cast<u32x4 *>(ob + (size_t)qrow * p.o_ss + (lane & 7) * 8) = v;
+                if (p.oq) {
+                    // the Reformat layer that follows in a quantised net (x86 form: multiply by 1/scale, round half
+                    // away from zero, saturate), applied to the values as stored
+                    u32x2 q8;
+#pragma unroll
+                    for (int w = 0; w < 2; ++w) {
+                        uint32_t packed = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t word = v[w * 2 + (e >> 1)];
+                            const float f       = AttnT<DT>::to_float((uint16_t)(e & 1 ? word >> 16 : word & 0xffffu));
+                            packed |= (uint32_t)(uint8_t)float2int8_ref(__fmul_rn(f, p.q_inv)) << (8 * e);
+                        }
+                        q8[w] = packed;
+                    }
+                    int8_t *oqb = p.oq + (size_t)b * p.o_sb + (size_t)head * p.o_sh;
+                    *reinterpret_cast<u32x2 *>(oqb + (size_t)qrow * p.o_ss + (lane & 7) * 8) = q8;
+                }
+            }
         }
     }
 }
@@ -469,6 +492,8 @@ int tnn_rocm_attention(void *stream, int dtype, const void *q, const void *k, co
     p.mask        = mask;
     p.kv_len      = kv_len;
     p.vt_sb = p.vt_sh = p.vt_sd = 0;
+    p.oq    = nullptr;
+    p.q_inv = 0.f;
     return launch_attention<false>((hipStream_t)stream, dtype, p, B, heads, S);
 }
 
@@ -476,6 +501,14 @@ int tnn_rocm_attention_vt(void *stream, int dtype, const void *q, const void *k,
                           int heads, int S, int head_dim, long q_sb, long q_sh, long q_ss, long k_sb, long k_sh,
                           long k_ss, long vt_sb, long vt_sh, long vt_sd, long o_sb, long o_sh, long o_ss, float scale,
                           const float *mask, const int32_t *kv_len) {
+    return tnn_rocm_attention_vt_q8(stream, dtype, q, k, vt, out, nullptr, 0.f, B, heads, S, head_dim, q_sb, q_sh, q_ss, k_sb,
+                                    k_sh, k_ss, vt_sb, vt_sh, vt_sd, o_sb, o_sh, o_ss, scale, mask, kv_len);
+}
+
+int tnn_rocm_attention_vt_q8(void *stream, int dtype, const void *q, const void *k, const void *vt, void *out,
+                             int8_t *out_q, float out_q_inv_scale, int B, int heads, int S, int head_dim, long q_sb,
+                             long q_sh, long q_ss, long k_sb, long k_sh, long k_ss, long vt_sb, long vt_sh, long vt_sd,
+                             long o_sb, long o_sh, long o_ss, float scale, const float *mask, const int32_t *kv_len) {
     TR_REQUIRE(B >= 0 && heads >= 0 && S >= 0, TNN_ROCM_ESHAPE, "attention_vt: negative size");
     if (B == 0 || heads == 0 || S == 0)
         return 0;
@@ -509,6 +542,9 @@ int tnn_rocm_attention_vt(void *stream, int dtype, const void *q, const void *k,
     p.scale_log2e = scale * kLog2e;
     p.mask        = mask;
     p.kv_len      = kv_len;
+    TR_REQUIRE(!out_q || (((uintptr_t)out_q) & 7u) == 0, TNN_ROCM_EALIGN, "attention_vt: int8 output must be 8-byte aligned");
+    p.oq    = out_q;
+    p.q_inv = out_q_inv_scale;
     return launch_attention<true>((hipStream_t)stream, dtype, p, B, heads, S);
 }
 

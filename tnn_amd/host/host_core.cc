@@ -1114,8 +1114,10 @@ Status DefaultNetwork::InitLayers() {
             // layers written by the ROCm int8 pass with blobs of both kinds
             if (info->type == LAYER_ROCM_FUSED_LINEAR_INT8)
                 return is_input && idx == 0;
-            if (info->type == LAYER_ROCM_FUSED_ATTENTION)
-                return is_input && idx == 0 && dynamic_cast<RocmFusedAttentionParam *>(param)->quant;
+            if (info->type == LAYER_ROCM_FUSED_ATTENTION) {
+                auto ap = dynamic_cast<RocmFusedAttentionParam *>(param);
+                return is_input ? (idx == 0 && ap->quant) : (ap->out_quant && idx + 1 == info->outputs.size());
+            }
             if (info->type == LAYER_LAYER_NORM)
                 return !is_input && idx == 1;
             return param->quantized;
@@ -1180,6 +1182,9 @@ Status DefaultNetwork::AllocateBlobMemory() {
     for (int i = 0; i < (int)structure_.layers.size(); ++i)
         for (auto &n : structure_.layers[i]->inputs)
             last_use[n] = i;
+    const char *stagger_env = getenv("TNN_ROCM_BLOB_STAGGER");
+    const int64_t stagger   = stagger_env ? atoll(stagger_env) : 0;
+    int64_t total_bytes = 0;
     std::multimap<int64_t, void *> pool;  // free buffers by capacity
     std::map<std::string, std::pair<int64_t, void *>> owned;
     auto alloc_for = [&](Blob *b, bool reusable) -> Status {
@@ -1196,9 +1201,12 @@ Status DefaultNetwork::AllocateBlobMemory() {
         }
         if (!ptr) {
             info.data_type = DATA_TYPE_INT8;
-            info.dims      = {(int)bytes};
+            info.dims      = {(int)(bytes + stagger)};
             RETURN_ON_NEQ(device_->Allocate(&ptr, info), TNN_OK);
             allocations_.push_back(ptr);
+            total_bytes += bytes + stagger;
+            if (stagger > 0)
+                ptr = (char *)ptr + ((int64_t)(allocations_.size() * 4352) % stagger) / 256 * 256;
         }
         BlobHandle h;
         h.base = ptr;
@@ -1227,7 +1235,20 @@ Status DefaultNetwork::AllocateBlobMemory() {
                 owned.erase(it);
             }
         }
+        // an output nobody reads (a float tensor whose only reader was folded away) is free again right after its layer
+        for (auto &n : info->outputs) {
+            if (last_use.count(n) || outputs_.count(n))
+                continue;
+            auto it = owned.find(n);
+            if (it != owned.end()) {
+                pool.insert({it->second.first, it->second.second});
+                owned.erase(it);
+            }
+        }
     }
+    if (getenv("TNN_ROCM_VERBOSE"))
+        fprintf(stderr, "tnn-rocm: %zu blob buffers, %.1f MiB of activation memory for %zu layers\n", allocations_.size(),
+                (double)total_bytes / (1024.0 * 1024.0), structure_.layers.size());
     return TNN_OK;
 }
 

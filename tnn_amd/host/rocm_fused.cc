@@ -579,6 +579,7 @@ public:
         FoldGelu();
         FoldDequant();
         FoldLayerNormQuant();
+        FoldAttentionQuant();
         return TNN_OK;
     }
 
@@ -893,6 +894,35 @@ private:
         Compact();
     }
 
+    // RocmFusedAttention -> Reformat(float -> int8): the attention kernel writes the quantised context as a second
+    // output in the same launch (the float one stays for any other reader)
+    void FoldAttentionQuant() {
+        const char *sw = getenv("TNN_ROCM_FOLD_ATTN_Q8");
+        if (sw && sw[0] == '0')
+            return;
+        auto &L = structure_->layers;
+        GraphIndex g(L);
+        for (int i = 0; i < (int)L.size(); ++i) {
+            if (!L[i] || L[i]->type != LAYER_ROCM_FUSED_ATTENTION || L[i]->outputs.size() != 1)
+                continue;
+            auto ap = ParamOf<RocmFusedAttentionParam>(L[i]);
+            if (!ap || ap->seq_len <= 0 || ap->seq_len % 8 != 0)  // the V^T form of the kernel carries the second output
+                continue;
+            auto it = g.consumers.find(L[i]->outputs[0]);
+            if (it == g.consumers.end())
+                continue;
+            for (int ri : it->second) {
+                if (ri > i && IsReformat(L[ri], true)) {
+                    L[i]->outputs.push_back(L[ri]->outputs[0]);
+                    ap->out_quant = 1;
+                    L[ri]         = nullptr;
+                    break;
+                }
+            }
+        }
+        Compact();
+    }
+
     NetStructure *structure_ = nullptr;
     NetResource *resource_   = nullptr;
     bool half_               = true;
@@ -1085,7 +1115,7 @@ public:
             RETURN_ON_NEQ(UploadConverted(dequant.data(), (size_t)N, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &dequant_), TNN_OK);
         }
         if (!weight_ && p->ln_fold) {
-            if (p->quant || seq_ % 8 != 0 || H_ % 128 != 0 || outputs.size() != (p->ln_y ? 2u : 1u) ||
+            if (p->quant || seq_ % 8 != 0 || H_ % 128 != 0 || outputs.size() != 1u + (p->ln_y ? 1u : 0u) + (p->out_quant ? 1u : 0u) ||
                 res->ln_gamma.GetDataCount() != H_ || res->ln_beta.GetDataCount() != H_)
                 return Status(TNNERR_PARAM_ERR, "fused attention with a folded LayerNorm: S % 8 == 0, hidden size a multiple "
                                                 "of 128 and scale / shift of that width are required");
@@ -1122,6 +1152,16 @@ public:
         }
         const char *base = (const char *)qkv;
         const long d     = p->head_dim;
+        int8_t *out_q    = nullptr;
+        float out_q_inv  = 0.f;
+        if (p->out_quant) {  // the last output: the context quantised as the folded Reformat layer would
+            auto b8 = dynamic_cast<BlobInt8 *>(outputs.back());
+            if (outputs.size() < 2 || !b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1 ||
+                seq_ % 8 != 0)
+                return Status(TNNERR_PARAM_ERR, "fused attention: the quantised output needs an int8 blob with one scale");
+            out_q     = (int8_t *)Ptr(outputs.back());
+            out_q_inv = (float)(1.0 / b8->GetIntResource()->scale_handle.force_to<float *>()[0]);
+        }
         if (p->quant) {
             // int8 projections, requantised and dequantised in the GEMM epilogue, in the split layout
             char *vt = (char *)qkv + (size_t)T_ * 2 * H_ * es;
@@ -1129,10 +1169,10 @@ public:
                                                  (const int32_t *)bias_, (const float *)scale_, (const float *)dequant_, qkv,
                                                  vt, B_, seq_, p->heads, K_));
             const long row = 2L * H_;
-            ROCM_CALL(tnn_rocm_attention_vt(Stream(), (int)dt, base, base + (size_t)H_ * es, vt, Ptr(outputs[0]), B_, p->heads,
-                                            seq_, p->head_dim, (long)seq_ * row, d, row, (long)seq_ * row, d, row,
-                                            (long)p->heads * 64 * seq_, 64L * seq_, (long)seq_, (long)seq_ * H_, d, (long)H_,
-                                            p->scale, mask, kv));
+            ROCM_CALL(tnn_rocm_attention_vt_q8(Stream(), (int)dt, base, base + (size_t)H_ * es, vt, Ptr(outputs[0]), out_q,
+                                               out_q_inv, B_, p->heads, seq_, p->head_dim, (long)seq_ * row, d, row,
+                                               (long)seq_ * row, d, row, (long)p->heads * 64 * seq_, 64L * seq_, (long)seq_,
+                                               (long)seq_ * H_, d, (long)H_, p->scale, mask, kv));
             return TNN_OK;
         }
         if (seq_ % 8 == 0 && H_ % 64 == 0) {
@@ -1148,10 +1188,10 @@ public:
                 ROCM_CALL(tnn_rocm_gemm_qkv_split(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_, qkv, vt,
                                                   B_, seq_, p->heads, H_));
             const long row = 2L * H_;
-            ROCM_CALL(tnn_rocm_attention_vt(Stream(), (int)dt, base, base + (size_t)H_ * es, vt, Ptr(outputs[0]), B_, p->heads,
-                                            seq_, p->head_dim, (long)seq_ * row, d, row, (long)seq_ * row, d, row,
-                                            (long)p->heads * 64 * seq_, 64L * seq_, (long)seq_, (long)seq_ * H_, d, (long)H_,
-                                            p->scale, mask, kv));
+            ROCM_CALL(tnn_rocm_attention_vt_q8(Stream(), (int)dt, base, base + (size_t)H_ * es, vt, Ptr(outputs[0]), out_q,
+                                               out_q_inv, B_, p->heads, seq_, p->head_dim, (long)seq_ * row, d, row,
+                                               (long)seq_ * row, d, row, (long)p->heads * 64 * seq_, 64L * seq_, (long)seq_,
+                                               (long)seq_ * H_, d, (long)H_, p->scale, mask, kv));
             return TNN_OK;
         }
         ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 1, Ptr(inputs[0]), weight_, qkv, T_, 3 * H_, H_, H_, H_, 3 * H_, 1, 1, 1,

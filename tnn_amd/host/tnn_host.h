@@ -398,6 +398,8 @@ struct RocmFusedAttentionParam : public LayerParam {
     // LayerNorm folded into the QKV projection, as in RocmFusedLinearParam
     int ln_fold = 0, ln_y = 0;
     float ln_eps = 0.f;
+    // the last output blob is int8: the context quantised as the Reformat layer that followed would (ROCm int8 pass)
+    int out_quant = 0;
 };
 // Gather(word ids) + Add(position constant) + Gather(type ids) + Add + LayerNorm of a BERT-style front end.
 // Inputs: word ids, type ids (int32), gamma, beta (constant blobs); resource: RocmFusedEmbeddingResource.

@@ -142,14 +142,20 @@ def qkv_split_ln(t, wqkv_folded, bqkv_folded, colsum, eps, B, S, heads, gamma=No
     return (qk, vt, y) if want_y else (qk, vt)
 
 
-def attention_qk_vt(qk, vt, B, S, heads, scale, mask=None, kv_len=None, out=None):
-    """qk [B*S, 2H] (Q | K), vt [B, heads, 64, S]; out [B*S, H]"""
+def attention_qk_vt(qk, vt, B, S, heads, scale, mask=None, kv_len=None, out=None, q8_inv_scale=None):
+    """qk [B*S, 2H] (Q | K), vt [B, heads, 64, S]; out [B*S, H]; with q8_inv_scale also the int8 quantisation of out"""
     _chk(qk, vt, mask, kv_len, out)
     H = heads * 64
     if out is None:
         out = torch.empty(B * S, H, dtype=qk.dtype, device=qk.device)
     es = qk.element_size()
     base = qk.data_ptr()
+    if q8_inv_scale is not None:
+        out_q = torch.empty(B * S, H, dtype=torch.int8, device=qk.device)
+        capi.call("tnn_rocm_attention_vt_q8", _stream(), dt(qk), base, base + H * es, _p(vt), _p(out), _p(out_q),
+                  float(q8_inv_scale), B, heads, S, 64, S * 2 * H, 64, 2 * H, S * 2 * H, 64, 2 * H, heads * 64 * S, 64 * S, S,
+                  S * H, 64, H, float(scale), _p(mask), _p(kv_len))
+        return out, out_q
     capi.call("tnn_rocm_attention_vt", _stream(), dt(qk), base, base + H * es, _p(vt), _p(out), B, heads, S, 64,
               S * 2 * H, 64, 2 * H, S * 2 * H, 64, 2 * H, heads * 64 * S, 64 * S, S, S * H, 64, H, float(scale),
               _p(mask), _p(kv_len))
