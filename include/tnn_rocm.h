@@ -162,6 +162,14 @@ TNN_ROCM_API int tnn_rocm_gemm_i8_dequant_residual(void *stream, const int8_t *A
                                                    void *out_f, int out_f_dtype, int ldo, float dequant_scale,
                                                    const void *residual);
 
+/* tnn_rocm_gemm_i8 whose int8 result is passed through a 256-entry table on the way out: out = lut[q + 128].  Any
+ * int8 -> int8 layer chain that followed the projection can be folded this way, value for value; the host uses it for
+ * QuantizedInnerProduct -> Reformat -> GELU -> Reformat with the table produced by tnn_rocm_gelu_i8 on the 256 inputs
+ * (cpu_gelu_layer_acc.cc:42-45 between the two x86 Reformat forms). */
+TNN_ROCM_API int tnn_rocm_gemm_i8_lut(void *stream, const int8_t *A, const int8_t *W, const int32_t *bias,
+                                      const float *scale, int8_t *out_i8, int M, int N, int K, int lda, int ldw, int ldo,
+                                      const int8_t *lut);
+
 /* Quantised Q, K, V projections of one attention layer as a single int8 GEMM over the concatenated weights
  * wqkv[3H,K] (three QuantizedInnerProduct layers reading the same int8 input): scale[n] = w_scale[n] / o_scale of the
  * column's projection, dequant[n] = that projection's output blob scale.  Each column is requantised to int8 as in

@@ -115,7 +115,7 @@ def test_int8_ffn_from_model_files_bit_exact(monkeypatch):
     # once as the explicit chain (Reformat layers as the engine inserts them), once with the Reformat layers folded
     # into their neighbours by the ROCm int8 pass
     for fuse, want in (("0", {"Reformat": 4, "QuantizedInnerProduct": 2}),
-                       ("1", {"Reformat": 1, "QuantizedInnerProduct": 1, "RocmGeluInt8": 1, "RocmFusedLinearInt8": 1})):
+                       ("1", {"Reformat": 1, "RocmQuantLinearGelu": 1, "RocmFusedLinearInt8": 1})):
         monkeypatch.setenv("TNN_ROCM_FUSE_INT8", fuse)
         inst = host.RocmInstance.from_graph(g, "fp32")
         types = [t for t, _ in inst.layers()]

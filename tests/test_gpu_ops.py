@@ -731,3 +731,29 @@ def test_attention_quantised_second_output_bit_exact(dtype):
     assert np.array_equal(host(out_q), ref_q)
     assert np.array_equal(host(out_q), host(ops().quantize(out, inv)))
     assert np.abs(host(out_q).astype(int)).max() >= 30  # the scale makes real use of the int8 range
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 3072, 768), (65, 100, 200), (4096, 3072, 768)])
+def test_gemm_i8_with_gelu_table_bit_exact(M, N, K):
+    """QuantizedInnerProduct -> int8 GELU as one launch (the 256-entry table applied in the GEMM epilogue) equals the two
+    launches, and the checker's chain, bit for bit."""
+    say("gemm_i8 + GELU table M=%d N=%d K=%d" % (M, N, K))
+    rng = np.random.default_rng(M + N)
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    bias = rng.integers(-20000, 20000, N).astype(np.int32)
+    s_mid, s_out = np.float32(0.031), np.float32(0.027)
+    scale = orc.fc_int8_scale((rng.uniform(0.5, 1.5, N) * 1e-5).astype(np.float32), s_mid, N)
+    inv_out = np.float32(1.0 / s_out)
+    o = ops()
+    iota = torch.arange(-128, 128, dtype=torch.int16).to(torch.int8).cuda()
+    lut = o.gelu_i8(iota, s_mid, inv_out)
+    fused = host(o.gemm_i8_lut(dev(a), dev(w), dev(bias), dev(scale), lut))
+    q, _, _ = o.gemm_i8(dev(a), dev(w), dev(bias), dev(scale))
+    two = host(o.gelu_i8(q, s_mid, inv_out))
+    assert np.array_equal(fused, two)
+    ref_q, _ = orc.fc_int8(a, w, bias, scale)
+    ref = orc.quantize_x86(orc.gelu(orc.dequantize(ref_q, s_mid)), s_out)
+    diff = np.abs(fused.astype(int) - ref.astype(int))
+    assert diff.max() <= 1 and (diff > 0).mean() <= 1e-3   # device erff vs the checker's double erf on a rounding boundary
+    assert len(np.unique(host(q))) > 100                    # the requantised values span the int8 range

@@ -49,6 +49,7 @@ SIGNATURES = {
                               _l, _f, _vp, _vp],
     "tnn_rocm_attention_vt_q8": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _l, _l, _l, _l, _l, _l, _l, _l, _l,
                                  _l, _l, _l, _f, _vp, _vp],
+    "tnn_rocm_gemm_i8_lut": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "tnn_rocm_gemm_qkv_split": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i],
     "tnn_rocm_gemm_ln": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
     "tnn_rocm_gemm_qkv_split_ln": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i],

@@ -328,6 +328,9 @@ template <int DT> struct LnQkvSplitEpilogue {
 
 struct Int8Epilogue {
     static constexpr bool kRowStats = false;
+    // optional 256-entry table applied to the requantised value (index q + 128): an int8 -> int8 function that
+    // followed the layer (dequantise, GELU, quantise) folded into this epilogue.  The tiled kernel keeps a copy in LDS.
+    const int8_t *lut;
     const int32_t *bias;
     const float *scale;
     int8_t *out;
@@ -357,6 +360,8 @@ struct Int8Epilogue {
             // separately rounded steps as on the CPU paths.
             float f  = __fmul_rn((float)a, cc.scale);
             int8_t q = float2int8_ref(f);
+            if (lut)
+                q = lut[(int)q + 128];
             if (out)
                 out[(size_t)m * ldo + n] = q;
             if (out_f) {
@@ -375,7 +380,7 @@ struct Int8Epilogue {
     }
     __device__ __forceinline__ bool direct(int) const { return false; }
     // eight consecutive columns (n % 8 == 0, n + 7 < N, ldo % 8 == 0): same arithmetic as store(), vector accesses
-    __device__ __forceinline__ void store8(int m, int n, const int (&acc)[8]) const {
+    __device__ __forceinline__ void store8(int m, int n, const int (&acc)[8], const int8_t *lut_lds = nullptr) const {
         int a[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t)
@@ -402,6 +407,11 @@ struct Int8Epilogue {
 #pragma unroll
             for (int t = 0; t < 8; ++t)
                 q[t] = float2int8_ref(__fmul_rn((float)a[t], sc[t]));
+            if (lut_lds) {
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    q[t] = lut_lds[(int)q[t] + 128];
+            }
             if (out)
                 *reinterpret_cast<uint2 *>(out + o) = *reinterpret_cast<const uint2 *>(q);
             if (out_f) {
@@ -1022,6 +1032,12 @@ __global__ void __launch_bounds__(CFG::NT)
     // k-waves (fixed order), giving {rstd, mean} per tile row; both arrays sit behind the staging area
     float2 *const row_st   = reinterpret_cast<float2 *>(lds_dyn + CFG::stage_bytes);  // [BM]
     float2 *const row_part = row_st + BM;                                             // [WGK * WGN * 2][BM]
+    int8_t *const lut_lds = reinterpret_cast<int8_t *>(lds_dyn + CFG::stage_bytes);  // Int8Epilogue's table, 256 bytes
+    if constexpr (std::is_same<Epi, Int8Epilogue>::value) {
+        if (epi.lut && tid < 64)
+            reinterpret_cast<uint32_t *>(lut_lds)[tid] = reinterpret_cast<const uint32_t *>(epi.lut)[tid];
+        // read after the first staging barrier below
+    }
     if constexpr (Epi::kRowStats) {
         static_assert(CFG::NSTAGE > 0, "LayerNorm-folding epilogues run on the direct-to-LDS pipeline");
 #pragma unroll
@@ -1078,7 +1094,10 @@ __global__ void __launch_bounds__(CFG::NT)
             } else if (m < M) {
                 AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 if (n + 7 < N) {
-                    epi.store8(m, n, v);
+                    if constexpr (std::is_same<Epi, Int8Epilogue>::value)
+                        epi.store8(m, n, v, epi.lut ? lut_lds : nullptr);
+                    else
+                        epi.store8(m, n, v);
                 } else {
 #pragma unroll
                     for (int t = 0; t < 8; ++t)
@@ -1128,6 +1147,10 @@ int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int 
     typedef typename GemmTraits<DT>::elem T;
     int tiles_m = (M + CFG::BM - 1) / CFG::BM, tiles_n = (N + CFG::BN - 1) / CFG::BN;
     size_t lds  = CFG::lds_bytes;
+    if (std::is_same<Epi, Int8Epilogue>::value) {  // room for the 256-byte table behind the staging area
+        size_t need = CFG::stage_bytes + 256;
+        lds         = lds > need ? lds : need;
+    }
     if (Epi::kRowStats) {  // row statistics and the partial-sum buffer sit behind the staging area
         size_t need = CFG::stage_bytes + (size_t)CFG::BM * 8 * (1 + 2 * CFG::WGK * CFG::WGN);
         lds         = lds > need ? lds : need;
@@ -1397,7 +1420,7 @@ int tnn_rocm_gemm(void *stream, int dtype, int b_is_nk, const void *A, const voi
 
 static int gemm_i8_impl(void *stream, const int8_t *A, const int8_t *W, const int32_t *bias, const float *scale,
                         int8_t *out_i8, int32_t *acc_i32, int M, int N, int K, int lda, int ldw, int ldo, void *out_f,
-                        int out_f_dtype, float dequant_scale, const void *residual) {
+                        int out_f_dtype, float dequant_scale, const void *residual, const int8_t *lut = nullptr) {
     TR_REQUIRE(M >= 0 && N >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_i8: negative size");
     if (M == 0 || N == 0)
         return 0;
@@ -1410,7 +1433,10 @@ static int gemm_i8_impl(void *stream, const int8_t *A, const int8_t *W, const in
                "gemm_i8: dequantised output must be F32 or F16");
     TR_REQUIRE(!residual || out_f, TNN_ROCM_EINVAL, "gemm_i8: a residual needs the dequantised output");
     bool aligned = al16(A) && al16(W) && lda % 16 == 0 && ldw % 16 == 0 && K % 16 == 0;
+    TR_REQUIRE(!lut || (out_i8 && !out_f && (((uintptr_t)lut) & 3u) == 0), TNN_ROCM_EINVAL,
+               "gemm_i8: a lookup table applies to the int8 output only and must be 4-byte aligned");
     Int8Epilogue epi;
+    epi.lut         = lut;
     epi.bias        = bias;
     epi.scale       = scale;
     epi.out         = out_i8;
@@ -1434,6 +1460,12 @@ int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W, const int32
                      int out_f_dtype, float dequant_scale) {
     return gemm_i8_impl(stream, A, W, bias, scale, out_i8, acc_i32, M, N, K, lda, ldw, ldo, out_f, out_f_dtype,
                         dequant_scale, nullptr);
+}
+
+int tnn_rocm_gemm_i8_lut(void *stream, const int8_t *A, const int8_t *W, const int32_t *bias, const float *scale,
+                         int8_t *out_i8, int M, int N, int K, int lda, int ldw, int ldo, const int8_t *lut) {
+    TR_REQUIRE(out_i8 && lut, TNN_ROCM_EINVAL, "gemm_i8_lut: null pointer");
+    return gemm_i8_impl(stream, A, W, bias, scale, out_i8, nullptr, M, N, K, lda, ldw, ldo, nullptr, 0, 0.f, nullptr, lut);
 }
 
 int tnn_rocm_gemm_i8_dequant_residual(void *stream, const int8_t *A, const int8_t *W, const int32_t *bias,

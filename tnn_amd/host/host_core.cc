@@ -102,7 +102,7 @@ LayerType GlobalConvertLayerType(std::string s) {
         {"BlobScale", LAYER_BLOB_SCALE},      {"QuantizedAdd", LAYER_ADD},
         {"RocmFusedLinear", LAYER_ROCM_FUSED_LINEAR}, {"RocmFusedAttention", LAYER_ROCM_FUSED_ATTENTION},
         {"RocmFusedLinearInt8", LAYER_ROCM_FUSED_LINEAR_INT8}, {"RocmGeluInt8", LAYER_ROCM_GELU_INT8},
-        {"RocmFusedEmbedding", LAYER_ROCM_FUSED_EMBEDDING},
+        {"RocmFusedEmbedding", LAYER_ROCM_FUSED_EMBEDDING}, {"RocmQuantLinearGelu", LAYER_ROCM_QUANT_LINEAR_GELU},
     };
     auto it = m.find(s);
     return it == m.end() ? LAYER_NOT_SUPPORT : it->second;
@@ -888,6 +888,7 @@ BaseLayer *CreateLayer(LayerType type) {
         case LAYER_ROCM_FUSED_LINEAR: return new FusedLinearLayer(type);
         case LAYER_ROCM_FUSED_EMBEDDING: return new FusedEmbeddingLayer(type);
         case LAYER_ROCM_FUSED_LINEAR_INT8: return new MixedTypeLayer<InnerProductLayer>(type);
+        case LAYER_ROCM_QUANT_LINEAR_GELU: return new InnerProductLayer(type);
         case LAYER_ROCM_FUSED_ATTENTION: return new MixedTypeLayer<BaseLayer>(type);
         case LAYER_SOFTMAX:
         case LAYER_GELU:

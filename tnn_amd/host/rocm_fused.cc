@@ -577,6 +577,7 @@ public:
         if (half_)
             FuseAttention();
         FoldGelu();
+        FoldGeluIntoProjection();
         FoldDequant();
         FoldLayerNormQuant();
         FoldAttentionQuant();
@@ -824,6 +825,38 @@ private:
             L[i]  = nl;
             L[gi] = nullptr;
             L[ri] = nullptr;
+        }
+        Compact();
+    }
+
+    // QuantizedInnerProduct -> int8 h -> RocmGeluInt8 -> int8 g   ==>   RocmQuantLinearGelu -> g  (the GELU chain has 256
+    // possible inputs: the projection applies it as a table in its epilogue).  TNN_ROCM_FOLD_GELU_LUT=0 keeps two launches.
+    void FoldGeluIntoProjection() {
+        const char *sw = getenv("TNN_ROCM_FOLD_GELU_LUT");
+        if (sw && sw[0] == '0')
+            return;
+        auto &L = structure_->layers;
+        GraphIndex g(L);
+        for (int i = 0; i < (int)L.size(); ++i) {
+            if (!IsQuantFc(L[i]) || IsModelOutput(L[i]->outputs[0]))
+                continue;
+            int gi = g.sole_consumer(L[i]->outputs[0]);
+            float mid_scale;
+            if (gi < 0 || !L[gi] || L[gi]->type != LAYER_ROCM_GELU_INT8 || !BlobScale(L[i]->outputs[0], &mid_scale))
+                continue;
+            auto ip = ParamOf<InnerProductLayerParam>(L[i]);
+            auto np = std::make_shared<RocmQuantLinearGeluParam>();
+            static_cast<InnerProductLayerParam &>(*np) = *ip;
+            np->type      = "RocmQuantLinearGelu";
+            np->quantized = true;
+            np->mid_scale = mid_scale;
+            auto nl       = std::make_shared<LayerInfo>(*L[i]);  // keeps the name: the resource is looked up by it
+            nl->type      = LAYER_ROCM_QUANT_LINEAR_GELU;
+            nl->type_str  = "RocmQuantLinearGelu";
+            nl->param     = np;
+            nl->outputs   = {L[gi]->outputs[0]};
+            L[i]  = nl;
+            L[gi] = nullptr;
         }
         Compact();
     }
@@ -1312,6 +1345,65 @@ private:
     void *weight_ = nullptr, *bias_ = nullptr, *scale_ = nullptr;
 };
 REGISTER_ROCM_ACC(RocmFusedLinearInt8LayerAcc, LAYER_ROCM_FUSED_LINEAR_INT8);
+
+// ---- RocmQuantLinearGelu ------------------------------------------------------------------------------------------
+// QuantizedInnerProduct (x86_inner_product_layer_acc.cc:197-222: requantisation factor w_scale / o_scale as one host
+// fp32 division, 0 below FLT_MIN) with the Reformat -> GELU -> Reformat chain that followed applied to its int8
+// result as a table.  The table is produced once by the int8 GELU kernel itself on the 256 possible inputs.
+class RocmQuantLinearGeluLayerAcc : public RocmLayerAcc {
+public:
+    Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        if (weight_)
+            return TNN_OK;
+        auto p   = dynamic_cast<RocmQuantLinearGeluParam *>(param_);
+        auto res = dynamic_cast<InnerProductLayerResource *>(resource_);
+        auto out8 = dynamic_cast<BlobInt8 *>(outputs[0]);
+        CHECK_PARAM_NULL(p);
+        CHECK_PARAM_NULL(res);
+        if (!out8 || !out8->GetIntResource() || out8->GetIntResource()->scale_handle.GetDataCount() != 1 ||
+            inputs[0]->GetBlobDesc().data_type != DATA_TYPE_INT8 || res->weight_handle.GetDataType() != DATA_TYPE_INT8)
+            return Status(TNNERR_PARAM_ERR, "quantised linear + GELU: int8 input, weights and a per-tensor output scale are required");
+        const int N = p->num_output, K = DimsVectorUtils::Count(inputs[0]->GetBlobDesc().dims, p->axis);
+        if ((long)res->weight_handle.GetDataCount() != (long)N * K)
+            return Status(TNNERR_MODEL_ERR, "InnerProduct weight size does not match num_output x K");
+        const float *w_scale = res->scale_handle.force_to<float *>();
+        CHECK_PARAM_NULL(w_scale);
+        const int n_w = res->scale_handle.GetDataCount();
+        std::vector<float> scale(N);
+        for (int i = 0; i < N; ++i)
+            scale[i] = p->mid_scale >= FLT_MIN ? w_scale[n_w == 1 ? 0 : i] / p->mid_scale : 0.0f;
+        RETURN_ON_NEQ(UploadConverted(res->weight_handle.force_to<void *>(), (size_t)N * K, DATA_TYPE_INT8, DATA_TYPE_INT8, &weight_),
+                      TNN_OK);
+        RETURN_ON_NEQ(UploadConverted(scale.data(), (size_t)N, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &scale_), TNN_OK);
+        if (p->has_bias && res->bias_handle.GetDataCount() == N)
+            RETURN_ON_NEQ(UploadConverted(res->bias_handle.force_to<void *>(), (size_t)N, DATA_TYPE_INT32, DATA_TYPE_INT32, &bias_),
+                          TNN_OK);
+        // the table: GELU chain of every int8 value, computed by the kernel the un-folded graph would run
+        int8_t iota[256];
+        for (int i = 0; i < 256; ++i)
+            iota[i] = (int8_t)(i - 128);
+        void *iota_dev = nullptr;
+        RETURN_ON_NEQ(UploadConverted(iota, 256, DATA_TYPE_INT8, DATA_TYPE_INT8, &iota_dev), TNN_OK);
+        RETURN_ON_NEQ(UploadConverted(iota, 256, DATA_TYPE_INT8, DATA_TYPE_INT8, &lut_), TNN_OK);
+        const float s_out = out8->GetIntResource()->scale_handle.force_to<float *>()[0];
+        ROCM_CALL(tnn_rocm_gelu_i8(Stream(), (const int8_t *)iota_dev, p->mid_scale, (float)(1.0 / s_out), (int8_t *)lut_, 256));
+        ROCM_CALL(tnn_rocm_stream_sync(Stream()));
+        return TNN_OK;
+    }
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        auto p = dynamic_cast<RocmQuantLinearGeluParam *>(param_);
+        auto in_dims = inputs[0]->GetBlobDesc().dims;
+        const int N = p->num_output, K = DimsVectorUtils::Count(in_dims, p->axis);
+        const int rows = DimsVectorUtils::Count(in_dims, 0, p->axis);
+        ROCM_CALL(tnn_rocm_gemm_i8_lut(Stream(), (const int8_t *)Ptr(inputs[0]), (const int8_t *)weight_, (const int32_t *)bias_,
+                                       (const float *)scale_, (int8_t *)Ptr(outputs[0]), rows, N, K, K, K, N, (const int8_t *)lut_));
+        return TNN_OK;
+    }
+
+private:
+    void *weight_ = nullptr, *bias_ = nullptr, *scale_ = nullptr, *lut_ = nullptr;
+};
+REGISTER_ROCM_ACC(RocmQuantLinearGeluLayerAcc, LAYER_ROCM_QUANT_LINEAR_GELU);
 
 // ---- RocmGeluInt8 -----------------------------------------------------------------------------------------------
 // Reformat(int8->float) -> GELU -> Reformat(float->int8) on int8 blobs in one pass: q_out =

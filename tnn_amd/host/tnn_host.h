@@ -314,7 +314,8 @@ enum LayerType {
     LAYER_ROCM_FUSED_ATTENTION   = 0x7002,
     LAYER_ROCM_FUSED_LINEAR_INT8 = 0x7003,
     LAYER_ROCM_GELU_INT8         = 0x7004,
-    LAYER_ROCM_FUSED_EMBEDDING   = 0x7005,
+    LAYER_ROCM_FUSED_EMBEDDING = 0x7005,
+    LAYER_ROCM_QUANT_LINEAR_GELU = 0x7006,
 };
 LayerType GlobalConvertLayerType(std::string type_str);
 
@@ -416,6 +417,12 @@ struct RocmFusedEmbeddingResource : public LayerResource {
 struct RocmFusedLinearInt8Param : public InnerProductLayerParam {
     float out_scale  = 0.f;  // scale of the int8 blob the original layer produced
     int has_residual = 0;
+};
+// QuantizedInnerProduct whose int8 result went through Reformat -> GELU -> Reformat: the projection applies that
+// int8 -> int8 map as a 256-entry table in its epilogue.  mid_scale is the scale of the int8 blob the projection used
+// to write; the output blob is the one the second Reformat wrote.
+struct RocmQuantLinearGeluParam : public InnerProductLayerParam {
+    float mid_scale = 0.f;
 };
 struct RocmFusedQkvInt8Resource : public LayerResource {
     RawBuffer weight;   // int8 [3H, K]
