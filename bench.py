@@ -26,10 +26,10 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 # rocprofv3 --pmc runs of this command (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
 # --counter-reference kernel (64 MiB in, 64 MiB out): FETCH_SIZE reads half the bytes, WRITE_SIZE all of them.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "gemm_qkv": int((2 * 14352.3 + 13978.9) * 1024),   # algorithmic: 4.5 + 3.4 in, 13.5 out MiB
-    "gemm_out": int((2 * 10430.0 + 4608.0) * 1024),    # algorithmic: 4.5 + 1.1 + 4.5 in, 4.5 out MiB
-    "gemm_ffn1": int((2 * 16356.3 + 18432.0) * 1024),  # algorithmic: 4.5 + 4.5 in, 18 out MiB
-    "gemm_ffn2": int((2 * 37071.5 + 4608.2) * 1024),   # algorithmic: 18 + 4.5 + 4.5 in, 4.5 out MiB
+    "gemm_qkv": int((2 * 14518.9 + 18613.1) * 1024),   # algorithmic: 4.5 + 3.4 in, 13.5 + 4.5 (LayerNorm output) out MiB
+    "gemm_out": int((2 * 10431.5 + 4608.0) * 1024),    # algorithmic: 4.5 + 1.1 + 4.5 in, 4.5 out MiB
+    "gemm_ffn1": int((2 * 17782.9 + 23040.0) * 1024),  # algorithmic: 4.5 + 4.5 in, 18 + 4.5 (LayerNorm output) out MiB
+    "gemm_ffn2": int((2 * 37088.5 + 4610.5) * 1024),   # algorithmic: 18 + 4.5 + 4.5 in, 4.5 out MiB
 }
 
 
@@ -144,10 +144,16 @@ def main():
     b_qkv, b_h, b_f = (torch.randn(n, device="cuda") * 0.02 for n in (3 * H, H, F))
     o_h = torch.empty(T, H, device="cuda", dtype=torch.float16)
     o_f = torch.empty(T, F, device="cuda", dtype=torch.float16)
+    # the forms the fused graph launches: QKV and FFN1 read a LayerNorm output, so they run on the raw tensor with the
+    # normalisation folded into the GEMM and also write the LayerNorm output for the residual additions
+    ln_g, ln_b = torch.ones(H, device="cuda"), torch.zeros(H, device="cuda")
+    cs_qkv, cs_f = w_qkv.float().sum(1).contiguous(), w_1.float().sum(1).contiguous()
     gemm_ms = {
-        "gemm_qkv": timed(lambda: ops.qkv_split(x_h, w_qkv, b_qkv, B, S, cfg.heads), n_gemm),
+        "gemm_qkv": timed(lambda: ops.qkv_split_ln(x_h, w_qkv, b_qkv, cs_qkv, cfg.eps, B, S, cfg.heads, gamma=ln_g,
+                                                   beta=ln_b, want_y=True), n_gemm),
         "gemm_out": timed(lambda: ops.gemm(x_h, w_o, True, bias=b_h, residual=res, out=o_h), n_gemm),
-        "gemm_ffn1": timed(lambda: ops.gemm(x_h, w_1, True, bias=b_f, gelu=True, out=o_f), n_gemm),
+        "gemm_ffn1": timed(lambda: ops.gemm_ln(x_h, w_1, b_f, cs_f, cfg.eps, gamma=ln_g, beta=ln_b, gelu=True,
+                                               want_y=True), n_gemm),
         "gemm_ffn2": timed(lambda: ops.gemm(x_f, w_2, True, bias=b_h, residual=res, out=o_h), n_gemm),
     }
     gemm_flops = {"gemm_qkv": 2.0 * T * 3 * H * H, "gemm_out": 2.0 * T * H * H, "gemm_ffn1": 2.0 * T * F * H,
