@@ -346,3 +346,41 @@ def test_layernorm_folding_switch(monkeypatch):
     e0, e1, e01 = rel_err(outs["0"], ref), rel_err(outs["1"], ref), rel_err(outs["1"], outs["0"])
     say("  un-folded %.3g  folded %.3g  folded vs un-folded %.3g" % (e0, e1, e01))
     assert e0 <= FP16_TOL and e1 <= FP16_TOL and e01 <= FP16_TOL
+
+
+@pytest.mark.parametrize("hidden,heads,ffn,B,S,n_ln", [
+    (1024, 16, 4096, 2, 64, 1),    # BERT-large widths: every LayerNorm but the last is folded
+    (768, 12, 3072, 2, 100, 2),    # S is no multiple of 8: packed-QKV attention path, its LayerNorm stays a launch
+    (256, 4, 1024, 3, 40, 1),      # small widths (single-slab K for the 256-byte-slab tiles)
+    (192, 3, 768, 2, 48, 4),       # hidden is no multiple of 128: no LayerNorm is folded
+])
+def test_encoder_other_shapes_fp16(hidden, heads, ffn, B, S, n_ln):
+    """Two encoder layers at other widths / sequence lengths through Instance::Forward (fp16, fused) against the
+    checker; which LayerNorms the fusion pass may fold depends on the shape."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: 2-layer encoder hidden=%d heads=%d ffn=%d B=%d S=%d" % (hidden, heads, ffn, B, S))
+    cfg = EncoderConfig(2, hidden, heads, ffn)
+    w = make_weights(cfg, seed=hidden + S, bias_std=0.05)
+    rng = np.random.default_rng(S)
+    for lw in w["layers"]:
+        for k in ("ln1_g", "ln2_g"):
+            lw[k] = (1 + 0.2 * rng.standard_normal(hidden)).astype(np.float32)
+        for k in ("ln1_b", "ln2_b"):
+            lw[k] = (0.3 * rng.standard_normal(hidden)).astype(np.float32)
+    ids, seg, lens, mask = make_inputs(cfg, B, S, S // 3, S, seed=S + 1)
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), "fp16")
+    types = [t for t, _ in inst.layers()]
+    say("  layers: " + " ".join("%s x%d" % (t, types.count(t)) for t in sorted(set(types))))
+    assert types.count("RocmFusedAttention") == 2 and types.count("LayerNorm") == n_ln, types
+    inst.set_input("input_ids", ids)
+    inst.set_input("token_type_ids", seg)
+    inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+    for _ in range(4):
+        inst.forward()
+    got = inst.output("last_hidden").reshape(B * S, -1)
+    inst.close()
+    wr = r16w(w)
+    ref = encoder_ref.encoder(wr, cfg, encoder_ref.embed(wr, ids, seg, cfg.eps), B, S, mask)
+    err = rel_err(got, ref)
+    say("  max rel err %.3g" % err)
+    assert err <= FP16_TOL
