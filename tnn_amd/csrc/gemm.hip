@@ -1142,6 +1142,8 @@ __global__ void __launch_bounds__(CFG::NT)
 int g_gemm_force_cfg = 0;
 int g_gemm_group_m   = 0;  // 0 = derived from the tile count; otherwise forced
 
+inline int tune_override(int N, int K, int *group_m);
+
 template <int DT, typename CFG, typename Epi>
 int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb, const Epi &epi) {
     typedef typename GemmTraits<DT>::elem T;
@@ -1169,8 +1171,11 @@ int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int 
     per_cu        = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
     long resident = 32 * per_cu, per_xcd = ((long)tiles_m * tiles_n + 7) / 8;
     resident      = resident < per_xcd ? resident : per_xcd;
-    int group_m   = g_gemm_group_m > 0 ? g_gemm_group_m : 1;
-    if (g_gemm_group_m <= 0)
+    int forced_group = g_gemm_group_m;
+    if (forced_group <= 0)
+        tune_override(N, K, &forced_group);
+    int group_m   = forced_group > 0 ? forced_group : 1;
+    if (forced_group <= 0)
         while ((long)(group_m + 1) * (group_m + 1) <= resident)
             ++group_m;
     group_m = group_m > tiles_m ? tiles_m : group_m;
@@ -1222,26 +1227,30 @@ inline int pick_tile_config(long M, long N, size_t kbytes) {
 
 // Experiment hook: "N:K:code,N:K:code,..." forces a configuration code for given (N, K); set from the environment
 // variable TNN_ROCM_GEMM_TUNE at first use, or through tnn_rocm_debug_set_gemm_tune().
-struct TuneEntry { int n, k, cfg; };
+struct TuneEntry { int n, k, cfg, group_m; };
 TuneEntry g_tune_table[16];
 int g_tune_count = -1;
 inline void parse_tune(const char *e) {
     g_tune_count = 0;
     while (e && *e && g_tune_count < 16) {
         TuneEntry t;
-        if (sscanf(e, "%d:%d:%d", &t.n, &t.k, &t.cfg) == 3)
+        t.group_m = 0;
+        if (sscanf(e, "%d:%d:%d:%d", &t.n, &t.k, &t.cfg, &t.group_m) >= 3)
             g_tune_table[g_tune_count++] = t;
         e = strchr(e, ',');
         if (e)
             ++e;
     }
 }
-inline int tune_override(int N, int K) {
+inline int tune_override(int N, int K, int *group_m) {
     if (g_tune_count < 0)
         parse_tune(getenv("TNN_ROCM_GEMM_TUNE"));
     for (int i = 0; i < g_tune_count; ++i)
-        if (g_tune_table[i].n == N && g_tune_table[i].k == K)
+        if (g_tune_table[i].n == N && g_tune_table[i].k == K) {
+            if (group_m)
+                *group_m = g_tune_table[i].group_m;
             return g_tune_table[i].cfg;
+        }
     return 0;
 }
 
@@ -1249,7 +1258,7 @@ template <int DT, typename Epi>
 int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb,
                      const Epi &epi) {
     typedef typename GemmTraits<DT>::elem T;
-    int cfg       = g_gemm_force_cfg > 0 ? g_gemm_force_cfg : tune_override(N, K);
+    int cfg       = g_gemm_force_cfg > 0 ? g_gemm_force_cfg : tune_override(N, K, nullptr);
     size_t kbytes = (size_t)K * sizeof(T);
     if (cfg == 0) {
         // slabs that are whole 128-byte multiples go global -> LDS directly; average kernel durations inside a

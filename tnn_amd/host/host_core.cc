@@ -1183,8 +1183,6 @@ Status DefaultNetwork::AllocateBlobMemory() {
     for (int i = 0; i < (int)structure_.layers.size(); ++i)
         for (auto &n : structure_.layers[i]->inputs)
             last_use[n] = i;
-    const char *stagger_env = getenv("TNN_ROCM_BLOB_STAGGER");
-    const int64_t stagger   = stagger_env ? atoll(stagger_env) : 0;
     int64_t total_bytes = 0;
     std::multimap<int64_t, void *> pool;  // free buffers by capacity
     std::map<std::string, std::pair<int64_t, void *>> owned;
@@ -1202,12 +1200,10 @@ Status DefaultNetwork::AllocateBlobMemory() {
         }
         if (!ptr) {
             info.data_type = DATA_TYPE_INT8;
-            info.dims      = {(int)(bytes + stagger)};
+            info.dims      = {(int)bytes};
             RETURN_ON_NEQ(device_->Allocate(&ptr, info), TNN_OK);
             allocations_.push_back(ptr);
-            total_bytes += bytes + stagger;
-            if (stagger > 0)
-                ptr = (char *)ptr + ((int64_t)(allocations_.size() * 4352) % stagger) / 256 * 256;
+            total_bytes += bytes;
         }
         BlobHandle h;
         h.base = ptr;
