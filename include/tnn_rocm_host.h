@@ -43,6 +43,9 @@ int tnn_host_get_output(void *handle, const char *name, float *out, size_t capac
  * layer.  tnn_host_profile_finish fills up to `capacity` mean milliseconds (layer order) and returns the layer count. */
 int tnn_host_layer_count(void *handle);
 const char *tnn_host_layer_summary(void *handle);
+/* one line per layer of the optimised graph, layer order: name|input blobs|output blobs|input dims|output dims (blob
+ * names comma separated, dims as d0,d1,..;d0,d1,.. per blob): what a per-layer profile table or a per-blob check needs */
+const char *tnn_host_layer_io(void *handle);
 void tnn_host_profile_start(void *handle, const char *only_type);
 int tnn_host_profile_finish(void *handle, double *ms, int capacity);
 

@@ -384,3 +384,33 @@ def test_encoder_other_shapes_fp16(hidden, heads, ffn, B, S, n_ln):
     err = rel_err(got, ref)
     say("  max rel err %.3g" % err)
     assert err <= FP16_TOL
+
+
+def test_model_check_and_profile_report():
+    """The per-blob check tool (fused fp16 graph against the un-fused fp32 graph on the device) on a 2-layer encoder:
+    every surviving blob within the fp16 bar, the checked graph identical to the production graph; and the per-layer
+    profile report lists every layer of the optimised graph with its dims."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    from tnn_amd import model_check
+    say("host: model_check on a 2-layer encoder, fp16")
+    cfg = EncoderConfig.bert_base(2)
+    w = make_weights(cfg, seed=21, bias_std=0.02)
+    B, S = 2, 128
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 40, S, seed=22)
+    graph = tnnmodel.encoder_graph(cfg, w, B, S)
+    inputs = {"input_ids": ids, "token_type_ids": seg, "attention_bias": mask.reshape(B, 1, 1, S)}
+    rows, same = model_check.check(graph, inputs, "fp16")
+    say(model_check.report(rows))
+    assert same and len(rows) >= 10
+    assert all(r["ok"] for r in rows), [r for r in rows if not r["ok"]]
+    assert {"RocmFusedAttention", "RocmFusedLinear", "RocmFusedEmbedding", "LayerNorm"} <= {r["type"] for r in rows}
+    inst = host.RocmInstance.from_graph(graph, "fp16")
+    for k, v in inputs.items():
+        inst.set_input(k, v)
+    for _ in range(3):
+        inst.forward()
+    text = inst.profile_table(3)
+    inst.close()
+    say(text)
+    assert "Profiling Data Sort by Cost time" in text and "kernel runtime total" in text and "[2,128,3072] [2,128,768]" in text
+    assert text.count("RocmFusedLinear") >= 12   # six layers in each of the two per-layer tables

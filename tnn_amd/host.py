@@ -24,6 +24,7 @@ SIGNATURES = {
                                       C.POINTER(C.c_int)]),
     "tnn_host_layer_count": (C.c_int, [C.c_void_p]),
     "tnn_host_layer_summary": (C.c_char_p, [C.c_void_p]),
+    "tnn_host_layer_io": (C.c_char_p, [C.c_void_p]),
     "tnn_host_profile_start": (None, [C.c_void_p, C.c_char_p]),
     "tnn_host_profile_finish": (C.c_int, [C.c_void_p, C.POINTER(C.c_double), C.c_int]),
 }
@@ -104,6 +105,42 @@ class RocmInstance:
     def layers(self):
         text = load().tnn_host_layer_summary(self._h).decode()
         return [tuple(line.split(" ", 1)) for line in text.splitlines() if line]
+
+    def layer_io(self):
+        """[{name, inputs, outputs, input_dims, output_dims}] for the layers of the optimised graph"""
+        out = []
+        for line in load().tnn_host_layer_io(self._h).decode().splitlines():
+            name, ins, outs, din, dout = line.split("|")
+            shape = lambda t: [[int(x) for x in b.split(",") if x] for b in t.split(";")] if t else []
+            out.append({"name": name, "inputs": [x for x in ins.split(",") if x], "outputs": [x for x in outs.split(",") if x],
+                        "input_dims": shape(din), "output_dims": shape(dout)})
+        return out
+
+    def profile_table(self, iters=10):
+        """The engine's TNN_PROFILE report (source/tnn/core/profile.cc:111-201: per-layer table, the same sorted by cost,
+        summary by op type, total) from hipEvent timings of `iters` eager forwards."""
+        prof, io = self.profile(iters), self.layer_io()
+        dims = lambda bl: " ".join("[" + ",".join(str(x) for x in d) + "]" for d in bl)
+        rows = [(nm, t, ms, dims(i["input_dims"]), dims(i["output_dims"])) for (t, nm, ms), i in zip(prof, io)]
+
+        def table(title, header, data):
+            widths = [max(len(str(r[c])) for r in [header] + data) for c in range(len(header))]
+            line = lambda r: "| " + " | ".join(str(v).ljust(w) for v, w in zip(r, widths)) + " |"
+            bar = "-" * len(line(header))
+            return "\n".join([title.center(len(bar), "="), line(header), bar] + [line(r) for r in data] + [bar, ""])
+
+        header = ["name", "Op Type", "Kernel(ms)", "Input Dims", "Output Dims"]
+        fmt = [[nm, t, "%.4f" % ms, di, do] for nm, t, ms, di, do in rows]
+        by_cost = [[nm, t, "%.4f" % ms, di, do] for nm, t, ms, di, do in sorted(rows, key=lambda r: -r[2])]
+        total = sum(r[2] for r in rows)
+        per_type = {}
+        for _, t, ms, _, _ in rows:
+            per_type[t] = per_type.get(t, 0.0) + ms
+        summary = [[t, "%.4f" % ms, "%.2f" % (100.0 * ms / total if total > 0 else 0.0)]
+                   for t, ms in sorted(per_type.items(), key=lambda kv: -kv[1])]
+        return (table("Profiling Data", header, fmt) + table("Profiling Data Sort by Cost time", header, by_cost) +
+                table("Summary", ["Op Type", "Total Kernel Time(ms)", "Percent (%)"], summary) +
+                "kernel runtime total: %.4f ms\n" % total)
 
     def profile_start(self, only_type=""):
         load().tnn_host_profile_start(self._h, only_type.encode())

@@ -121,6 +121,12 @@ HOST_API const char *tnn_host_layer_summary(void *hp) {
     return h->summary.c_str();
 }
 
+HOST_API const char *tnn_host_layer_io(void *hp) {
+    auto h     = static_cast<Handle *>(hp);
+    h->summary = h->inst->GetNetwork()->LayerIo();
+    return h->summary.c_str();
+}
+
 // only_type: NULL or "" times every layer, otherwise only layers of that type string
 HOST_API void tnn_host_profile_start(void *hp, const char *only_type) {
     static_cast<Handle *>(hp)->inst->GetNetwork()->StartProfile(only_type ? only_type : "");

@@ -1332,6 +1332,36 @@ std::string DefaultNetwork::LayerSummary() const {
         os << l->type_str << " " << l->name << "\n";
     return os.str();
 }
+std::string DefaultNetwork::LayerIo() const {
+    std::ostringstream os;
+    auto names = [&](const std::vector<std::string> &v) {
+        for (size_t i = 0; i < v.size(); ++i)
+            os << (i ? "," : "") << v[i];
+    };
+    auto dims = [&](const std::vector<std::string> &v) {
+        for (size_t i = 0; i < v.size(); ++i) {
+            os << (i ? ";" : "");
+            auto it = blobs_.find(v[i]);
+            if (it == blobs_.end())
+                continue;
+            const auto &d = it->second->GetBlobDesc().dims;
+            for (size_t k = 0; k < d.size(); ++k)
+                os << (k ? "," : "") << d[k];
+        }
+    };
+    for (auto &l : structure_.layers) {
+        os << l->name << "|";
+        names(l->inputs);
+        os << "|";
+        names(l->outputs);
+        os << "|";
+        dims(l->inputs);
+        os << "|";
+        dims(l->outputs);
+        os << "\n";
+    }
+    return os.str();
+}
 void DefaultNetwork::StartProfile(const std::string &only_type) {
     prof_.clear();
     prof_on_.clear();

@@ -484,7 +484,7 @@ private:
             auto lp = ParamOf<LayerNormLayerParam>(ln);
             const std::string t = ln->inputs[0], y = ln->outputs[0];
             auto cit = g.consumers.find(y);
-            if (!lp || lp->reduce_dims_size != 1 || IsModelOutput(y) || cit == g.consumers.end())
+            if (!lp || lp->reduce_dims_size != 1 || cit == g.consumers.end())
                 continue;
             int owner = -1, owners = 0, C = 0;
             for (int ci : cit->second) {
@@ -508,7 +508,7 @@ private:
             if (owners != 1 || owner < li || C <= 0 || C % 128 != 0)
                 continue;
             RawBuffer *gamma = constant(ln->inputs[1], C), *beta = constant(ln->inputs[2], C);
-            bool others = false, ordered = true;
+            bool others = IsModelOutput(y), ordered = true;  // a model output is written like any other reader's copy
             for (int ci : cit->second)
                 if (ci != owner) {
                     others = true;

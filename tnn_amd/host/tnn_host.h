@@ -674,6 +674,8 @@ public:
     Blob *GetBlob(const std::string &name);
     int LayerCount() const { return (int)layers_.size(); }
     std::string LayerSummary() const;
+    // one line per layer: name|input blob names (comma separated)|output blob names|input dims (d0,d1,..;d0,..)|output dims
+    std::string LayerIo() const;
     // per-layer hipEvent timing (the engine's TNN_PROFILE hook, source/tnn/core/profile.cc:111-201)
     // only layers whose type string equals `only_type` are timed when it is non-empty
     void StartProfile(const std::string &only_type = "");
