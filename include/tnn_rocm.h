@@ -128,7 +128,8 @@ TNN_ROCM_API int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W
  * K, V (kv strides) and out.  head_dim must be 64.  dtype F16 or BF16.
  *   mask   : optional additive fp32 [B, S] (broadcast over heads and query rows), e.g. 0 / -10000
  *   kv_len : optional int32 [B]; keys j >= kv_len[b] are excluded exactly (−inf) and their tiles
- *            skipped. */
+ *            skipped. 
+ *            (bit 30 of an entry may be set by tnn_rocm_mask_to_kv_len_flagged: mask row b is then not read). */
 TNN_ROCM_API int tnn_rocm_attention(void *stream, int dtype, const void *q, const void *k, const void *v, void *out,
                                     int B, int heads, int S, int head_dim, long q_sb, long q_sh, long q_ss, long kv_sb,
                                     long kv_sh, long kv_ss, long o_sb, long o_sh, long o_ss, float scale,
@@ -207,6 +208,11 @@ TNN_ROCM_API int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void 
                                             int heads, int K);
 
 /* kv_len[b] = 1 + the last key index whose additive mask value is > threshold (0 if none). */
+/* The _flagged form additionally sets bit 30 of kv_len[b] when mask[b][j] is exactly 0 for every j < kv_len[b] (a plain
+ * padding mask): the attention kernels accept such entries and then do not read mask row b at all (the keys at and
+ * beyond kv_len[b] are excluded by the length), which lets full key tiles take the path without a per-key bias. */
+TNN_ROCM_API int tnn_rocm_mask_to_kv_len_flagged(void *stream, const float *mask, int32_t *kv_len, int B, int S,
+                                                 float threshold);
 TNN_ROCM_API int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_t *kv_len, int B, int S,
                                          float threshold);
 

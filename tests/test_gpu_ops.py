@@ -634,10 +634,19 @@ def test_qkv_split_and_attention_vt():
     assert np.array_equal(got_qk, plain[:, :2 * H]) and np.array_equal(got_v, plain[:, 2 * H:])
     lens = np.array([200, 37, 128], np.int32)
     out = host(ops().attention_qk_vt(qk, vt, B, S, h, 0.125, kv_len=dev(lens)))
-    # same inputs through the kernel that transposes V itself: results must agree bit for bit
+    # same inputs through the kernel that transposes V itself: the two feed the keys of a tile into the P.V MFMAs in
+    # a different order, so they agree to fp32 accumulation order (one fp16 ulp after the final rounding)
     qkv = torch.from_numpy(plain.astype(np.float16))
     out2 = host(ops().attention_packed(qkv.cuda(), B, S, h, 0.125, kv_len=dev(lens)))
-    assert np.array_equal(out, out2)
+    assert rel_err(out, out2) <= 1e-3
+    # and the register-staged form of the same V^T kernel
+    from tnn_amd import capi
+    capi.load().tnn_rocm_debug_set_attention_dma(0)
+    try:
+        out3 = host(ops().attention_qk_vt(qk, vt, B, S, h, 0.125, kv_len=dev(lens)))
+    finally:
+        capi.load().tnn_rocm_debug_set_attention_dma(1)
+    assert rel_err(out, out3) <= 1e-3
     xq = plain.reshape(B, S, 3, h, 64)
     q, k, v = (np.ascontiguousarray(xq[:, :, i].transpose(0, 2, 1, 3)) for i in range(3))
     mask = np.zeros((B, S), np.float32)
@@ -655,6 +664,22 @@ def test_mask_to_kv_len():
         m[b, l:] = -10000.0
     got = host(ops().mask_to_kv_len(dev(m)))
     assert got.tolist() == lens
+    # flagged form: bit 30 marks rows whose visible part is exactly zero; a row with any other visible value is not marked
+    m[2, 5] = -0.5
+    got = host(ops().mask_to_kv_len(dev(m), flagged=True))
+    assert [int(v) & ~(1 << 30) for v in got] == lens
+    assert [bool(int(v) >> 30 & 1) for v in got] == [True, True, False, True, True]
+    # attention with flagged lengths + mask equals attention with the mask alone (general additive values kept)
+    B, S, h = 5, 300, 2
+    S8 = 304
+    mm = np.full((B, S8), -10000.0, np.float32)
+    mm[:, :S] = m
+    g = torch.Generator().manual_seed(3)
+    qk = torch.randn(B * S8, 2 * h * 64, generator=g).half().cuda()
+    vt = torch.randn(B, h, 64, S8, generator=g).half().cuda()
+    a1 = ops().attention_qk_vt(qk, vt, B, S8, h, 0.125, mask=dev(mm))
+    a2 = ops().attention_qk_vt(qk, vt, B, S8, h, 0.125, mask=dev(mm), kv_len=ops().mask_to_kv_len(dev(mm), flagged=True))
+    assert rel_err(host(a2), host(a1)) <= 1e-3
 
 
 def test_attention_rejects_bad_args():

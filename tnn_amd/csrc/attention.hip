@@ -16,6 +16,8 @@
 // so V is stored transposed in LDS ([d][key]) and each lane fetches its two 4-key groups with two
 // 8-byte reads.  Padding keys (>= kv_len) are excluded exactly (−inf) in-register and whole tiles
 // past kv_len are never loaded.
+#include <type_traits>
+
 #include "common.h"
 
 using namespace tnn_rocm;
@@ -30,6 +32,7 @@ constexpr int kD        = 64;            // head dim
 constexpr int kTileKV   = 64;            // keys per LDS tile
 constexpr int kRowBytes = kD * 2 + 16;   // padded LDS row (K: one key's 64 halfs; V^T: one d's 64 keys)
 constexpr float kLog2e  = 1.4426950408889634f;
+constexpr int kKvLenMaskZero = 1 << 30;  // flag bit of a kv_len entry, see tnn_rocm_mask_to_kv_len_flagged
 
 template <int DT> struct AttnT;
 template <> struct AttnT<TNN_ROCM_F16> {
@@ -45,6 +48,15 @@ template <> struct AttnT<TNN_ROCM_F16> {
     // Probabilities (0..1) for the second MFMA: one v_cvt_pkrtz per pair.  The row sum is taken over the SAME
     // rounded values (v_dot2 with (1,1), fp32 accumulate), so numerator and denominator of the softmax stay
     // consistent and the truncation does not bias the normalised weights.
+    // the same in two steps, for callers that shuffle the packed pairs before summing them
+    static __device__ __forceinline__ uint32_t pack_only(float lo, float hi) {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+    }
+    static __device__ __forceinline__ void add_packed(uint32_t pk, float &sum) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 one = {(_Float16)1.0f, (_Float16)1.0f};
+        sum    = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, pk), one, sum, false);
+    }
     static __device__ __forceinline__ uint32_t pack_prob(float lo, float hi, float &sum) {
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
         typedef __fp16 fp16x2 __attribute__((ext_vector_type(2)));
@@ -62,6 +74,12 @@ template <> struct AttnT<TNN_ROCM_BF16> {
     static __device__ __forceinline__ float to_float(uint16_t bits) { return __uint_as_float((uint32_t)bits << 16); }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+    }
+    static __device__ __forceinline__ uint32_t pack_only(float lo, float hi) {
+        return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+    }
+    static __device__ __forceinline__ void add_packed(uint32_t pk, float &sum) {
+        sum += __uint_as_float(pk << 16) + __uint_as_float(pk & 0xffff0000u);
     }
     static __device__ __forceinline__ uint32_t pack_prob(float lo, float hi, float &sum) {
         uint32_t l = float_to_bf16(lo), h = float_to_bf16(hi);
@@ -139,9 +157,12 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_kernel(Att
     const int q0   = (vid - bh * n_q) * BQ + wave * 32;
 
     int kv_end = S;
+    bool mask_is_zero = false;  // kv_len[b] may carry kKvLenMaskZero: the mask row is 0 for every key below kv_len[b]
     if (p.kv_len) {
-        int l  = p.kv_len[b];
-        kv_end = l < 0 ? 0 : (l < S ? l : S);
+        int l        = p.kv_len[b];
+        mask_is_zero = l >= 0 && (l & kKvLenMaskZero) != 0;
+        l            = l >= 0 ? (l & ~kKvLenMaskZero) : l;
+        kv_end       = l < 0 ? 0 : (l < S ? l : S);
     }
     const int n_tiles = (kv_end + kTileKV - 1) / kTileKV;
 
@@ -150,7 +171,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_kernel(Att
     const uint16_t *vb = VT ? p.v + (size_t)b * p.vt_sb + (size_t)head * p.vt_sh
                             : p.v + (size_t)b * p.kv_sb + (size_t)head * p.kv_sh;
     uint16_t *ob       = p.o + (size_t)b * p.o_sb + (size_t)head * p.o_sh;
-    const float *mb    = p.mask ? p.mask + (size_t)b * S : nullptr;
+    const float *mb    = p.mask && !mask_is_zero ? p.mask + (size_t)b * S : nullptr;
 
     // No load below is guarded by a branch: row indices past the end are clamped to the last valid row.  Keys at or
     // beyond kv_end then carry finite (wrong) data, and their score bias of -inf makes their probability exactly 0,
@@ -414,8 +435,331 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_kernel(Att
     }
 }
 
+// ---- the same computation with the K and V^T tiles loaded global -> LDS directly -------------------------------------
+// For the V^T layout.  Three 16 KB stages of un-padded 128-byte rows; global_load_lds_dwordx4 writes each lane's 16
+// bytes at consecutive LDS addresses, so the XOR swizzle that keeps the fragment reads conflict-free (chunk p of row r
+// holds logical chunk p ^ ((r >> 1) & 7)) is applied to the global addresses.  No staging registers, no LDS store
+// instructions, no per-tile address arithmetic (the tile advances a scalar base); loads run two tiles ahead and the
+// waits are placed by hand (the kernel issues no other vector-memory load inside the loop; the padding-mask values of
+// a tile travel the same way).  V^T rows are plain here: the eight keys a lane half feeds into one P.V step are made
+// contiguous by exchanging two packed probability registers between the lane halves (v_permlane32_swap) instead of
+// permuting the keys inside the tile.
+#define TR_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n)&0xF) | ((((n) >> 4) & 3) << 14) | (0x7 << 4) | (0xF << 8)))
+
+template <int DT, int NW>
+__global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel(AttnParams p) {
+    constexpr int NT = NW * 64;
+    constexpr int BQ = NW * 32;
+    constexpr int kTile  = kTileKV * 128;  // one K or V^T tile, un-padded rows
+    constexpr int kStage = 2 * kTile;
+    constexpr int LD     = 8 / NW;         // 1 KB wave-loads per wave, tile and operand
+    __shared__ __attribute__((aligned(16))) unsigned char lds_all[3 * kStage];
+    __shared__ __attribute__((aligned(16))) float lds_bias[3][kTileKV];
+    static_assert(BQ * kRowBytes <= 2 * kStage, "Q staging must fit stages 1 and 2");
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int g    = lane >> 5;
+    const int lq   = lane & 31;
+    const int S    = p.S;
+    const int n_q   = (S + BQ - 1) / BQ;
+    const int total = n_q * p.heads * p.B;
+    const int per   = (total + 7) >> 3;
+    const int vid   = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
+    if (vid >= total)
+        return;
+    const int bh   = vid / n_q;
+    const int b    = bh / p.heads;
+    const int head = bh - b * p.heads;
+    const int q0   = (vid - bh * n_q) * BQ + wave * 32;
+
+    int kv_end = S;
+    bool mask_is_zero = false;  // kv_len[b] may carry kKvLenMaskZero: the mask row is 0 for every key below kv_len[b]
+    if (p.kv_len) {
+        int l        = p.kv_len[b];
+        mask_is_zero = l >= 0 && (l & kKvLenMaskZero) != 0;
+        l            = l >= 0 ? (l & ~kKvLenMaskZero) : l;
+        kv_end       = l < 0 ? 0 : (l < S ? l : S);
+    }
+    const int n_tiles = (kv_end + kTileKV - 1) / kTileKV;
+
+    const uint16_t *qb = p.q + (size_t)b * p.q_sb + (size_t)head * p.q_sh;
+    const uint16_t *kb = p.k + (size_t)b * p.kv_sb + (size_t)head * p.kv_sh;
+    const uint16_t *vb = p.v + (size_t)b * p.vt_sb + (size_t)head * p.vt_sh;
+    uint16_t *ob       = p.o + (size_t)b * p.o_sb + (size_t)head * p.o_sh;
+    const float *mb    = p.mask && !mask_is_zero ? p.mask + (size_t)b * S : nullptr;
+
+    // ---- tile loads.  Wave-load j = wave + i*NW covers LDS rows 8j .. 8j+7 of a tile
+    const uint32_t lds_base = (uint32_t)(uintptr_t)lds_all, bias_base = (uint32_t)(uintptr_t)&lds_bias[0][0];
+    const int lrow = lane >> 3, lpos = lane & 7;
+    const uint32_t kv_ss32 = (uint32_t)p.kv_ss, vt_sd32 = (uint32_t)p.vt_sd;
+    uint32_t k_off[LD], v_off[LD];  // byte offsets of this lane's 16 bytes from the tile's first key
+    int l_row[LD], l_chunk[LD];
+#pragma unroll
+    for (int i = 0; i < LD; ++i) {
+        const int r = (wave + i * NW) * 8 + lrow;
+        l_row[i]    = r;
+        l_chunk[i]  = lpos ^ ((r >> 1) & 7);
+        k_off[i]    = ((uint32_t)r * kv_ss32 + (uint32_t)l_chunk[i] * 8u) * 2u;
+        v_off[i]    = ((uint32_t)r * vt_sd32 + (uint32_t)l_chunk[i] * 8u) * 2u;
+    }
+    auto load16 = [](const void *base, uint32_t byte_off, uint32_t lds_addr) {
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
+    };
+    auto load4 = [](const void *base, uint32_t byte_off, uint32_t lds_addr) {
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
+    };
+    const uint32_t wave_dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_base + (uint32_t)wave * 1024u));
+    auto issue = [&](int t, int stage) {
+        const int kv0      = t * kTileKV;
+        const uint32_t dst = wave_dst + (uint32_t)(stage * kStage);
+        if (kv0 + kTileKV <= S) {  // whole tile inside the sequence: the tile only moves the scalar base
+            const uint16_t *kt_base = kb + (size_t)kv0 * p.kv_ss, *vt_base = vb + kv0;
+#pragma unroll
+            for (int i = 0; i < LD; ++i)
+                load16(kt_base, k_off[i], dst + i * NW * 1024);
+#pragma unroll
+            for (int i = 0; i < LD; ++i)
+                load16(vt_base, v_off[i], dst + kTile + i * NW * 1024);
+        } else {  // last, partial tile: rows / key chunks past the end are clamped (their bias is -inf)
+#pragma unroll
+            for (int i = 0; i < LD; ++i) {
+                int key = kv0 + l_row[i];
+                key     = key < S ? key : S - 1;
+                load16(kb, ((uint32_t)key * kv_ss32 + (uint32_t)l_chunk[i] * 8u) * 2u, dst + i * NW * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < LD; ++i) {
+                int k8 = kv0 + l_chunk[i] * 8;
+                k8     = k8 < S ? k8 : S - 8;
+                load16(vb, ((uint32_t)l_row[i] * vt_sd32 + (uint32_t)k8) * 2u, dst + kTile + i * NW * 1024);
+            }
+        }
+        if (mb) {  // the tile's 64 additive mask values; every wave writes the same 256 bytes
+            int key = kv0 + lane;
+            key     = key < S ? key : S - 1;
+            load4(mb, (uint32_t)key * 4u, bias_base + (uint32_t)(stage * kTileKV * 4));
+        }
+    };
+    constexpr int LPW = 2 * LD;
+    if (n_tiles > 0)
+        issue(0, 0);
+
+    // ---- Q fragments through LDS (stages 1 and 2 are free until the second tile is requested)
+    u32x4 qf[4];
+    {
+        unsigned char *const stage = lds_all + kStage;
+        constexpr int Q_VECS = BQ * 8 / NT;
+#pragma unroll
+        for (int i = 0; i < Q_VECS; ++i) {
+            const int v = tid + i * NT, r = v >> 3, c = v & 7;
+            int qrow = (q0 - wave * 32) + r;
+            qrow     = qrow < S ? qrow : S - 1;
+            *reinterpret_cast<u32x4 *>(stage + r * kRowBytes + c * 16) =
+                *reinterpret_cast<const u32x4 *>(qb + (size_t)qrow * p.q_ss + c * 8);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+            qf[kk] = *reinterpret_cast<const u32x4 *>(stage + (wave * 32 + lq) * kRowBytes + kk * 32 + g * 16);
+        __syncthreads();
+    }
+    if (n_tiles > 1)
+        issue(1, 1);
+
+    // fragment chunk x = 2*step + g of row lq (the same expression serves the K and the V^T tile)
+    uint32_t frag_off[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+        frag_off[x] = (uint32_t)(lq * 128 + (((2 * x + g) ^ ((lq >> 1) & 7)) * 16));
+
+    f32x16 oacc[2];
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            oacc[dt][r] = 0.f;
+    float m_i = -INFINITY, l_i = 0.f;
+
+    int stage = 0, fill = 2;
+    for (int t = 0; t < n_tiles; ++t) {
+        // tile t has landed once at most the loads of tile t + 1 are outstanding
+        if (t + 1 < n_tiles) {
+            if (mb)
+                TR_WAIT_VMCNT(LPW + 1);
+            else
+                TR_WAIT_VMCNT(LPW);
+        } else {
+            TR_WAIT_VMCNT(0);
+        }
+        __builtin_amdgcn_s_barrier();  // everyone's part of tile t is in LDS; everyone is done with tile t - 1
+        asm volatile("" ::: "memory");  // no LDS access may be moved across the barrier by the compiler
+        if (t + 2 < n_tiles)
+            issue(t + 2, fill);
+
+        const unsigned char *const kbuf  = lds_all + stage * kStage;
+        const unsigned char *const vtbuf = kbuf + kTile;
+        const int kv0     = t * kTileKV;
+        const bool biased = mb != nullptr || kv0 + kTileKV > kv_end || !(p.scale_log2e > 0.f);  // workgroup-uniform
+        // The whole tile is written twice (with and without the per-key bias) under one branch: with the branch
+        // inside the tile the compiler copies the 32 score registers where the two paths meet.
+        auto tile = [&](auto biased_tag) __attribute__((always_inline)) {
+            constexpr bool BIASED = decltype(biased_tag)::value;
+            f32x16 sacc[2];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    sacc[kt][r] = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) {
+                    u32x4 kf = *reinterpret_cast<const u32x4 *>(kbuf + kt * 32 * 128 + frag_off[kk]);
+                    AttnT<DT>::mma(kf, qf[kk], sacc[kt]);
+                }
+            }
+            float mx = -INFINITY;
+            if (BIASED) {
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; ++r4) {
+                        const int key0 = kt * 32 + r4 * 8 + g * 4;
+                        float bv[4]    = {0.f, 0.f, 0.f, 0.f};
+                        if (mb) {
+                            float4 raw = *reinterpret_cast<const float4 *>(&lds_bias[stage][key0]);
+                            bv[0] = raw.x * kLog2e, bv[1] = raw.y * kLog2e, bv[2] = raw.z * kLog2e, bv[3] = raw.w * kLog2e;
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float be       = kv0 + key0 + e < kv_end ? bv[e] : -INFINITY;
+                            float s2             = fmaf(sacc[kt][r4 * 4 + e], p.scale_log2e, be);
+                            sacc[kt][r4 * 4 + e] = s2;
+                            mx                   = fmaxf(mx, s2);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        mx = fmaxf(mx, sacc[kt][r]);
+                mx *= p.scale_log2e;
+            }
+            mx          = half_swap_max(mx);
+            float m_new = fmaxf(m_i, mx);
+            float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
+            if (BIASED) {
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        sacc[kt][r] = __builtin_amdgcn_exp2f(sacc[kt][r] - m_use);
+            } else {
+                const float neg_m = -m_use;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        sacc[kt][r] = __builtin_amdgcn_exp2f(fmaf(sacc[kt][r], p.scale_log2e, neg_m));
+            }
+            if (!__all(m_new == m_i)) {
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        oacc[dt][r] *= alpha;
+            }
+            m_i = m_new;
+
+            // ---- O^T += V^T P^T.  Register r of block kt is key kt*32 + 8*(r/4) + 4*g + (r%4): a lane half holds four
+            // keys of each 8-key group.  Step st = 2*kt + j uses groups 2j and 2j+1 of the block; after exchanging the
+            // packed pairs (group 2j+1 of the lower half <-> group 2j of the upper half) lane half g holds the eight
+            // consecutive keys of group 2j + g, i.e. 16-byte chunk 2*st + g of the V^T rows.  The row sum is taken on
+            // the exchanged registers (the two halves of a column together still hold every key once), so the
+            // registers before the exchange die there.
+            float rs = 0.f;
+#pragma unroll
+            for (int st = 0; st < 4; ++st) {
+                const int kt = st >> 1, j = st & 1;
+                uint32_t w0 = AttnT<DT>::pack_only(sacc[kt][8 * j + 0], sacc[kt][8 * j + 1]);
+                uint32_t w1 = AttnT<DT>::pack_only(sacc[kt][8 * j + 2], sacc[kt][8 * j + 3]);
+                uint32_t w2 = AttnT<DT>::pack_only(sacc[kt][8 * j + 4], sacc[kt][8 * j + 5]);
+                uint32_t w3 = AttnT<DT>::pack_only(sacc[kt][8 * j + 6], sacc[kt][8 * j + 7]);
+                auto x0 = __builtin_amdgcn_permlane32_swap(w0, w2, false, false);
+                auto x1 = __builtin_amdgcn_permlane32_swap(w1, w3, false, false);
+                u32x4 pf;
+                pf[0] = x0[0], pf[1] = x1[0], pf[2] = x0[1], pf[3] = x1[1];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    AttnT<DT>::add_packed(pf[e], rs);
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt) {
+                    const u32x4 vf = *reinterpret_cast<const u32x4 *>(vtbuf + dt * 32 * 128 + frag_off[st]);
+                    AttnT<DT>::mma(vf, pf, oacc[dt]);
+                }
+            }
+            rs  = half_swap_sum(rs);
+            l_i = fmaf(l_i, alpha, rs);
+        };
+        if (biased)
+            tile(std::true_type());
+        else
+            tile(std::false_type());
+
+        stage = stage == 2 ? 0 : stage + 1;
+        fill  = fill == 2 ? 0 : fill + 1;
+    }
+
+    // ---- normalise and store (see attention_kernel)
+    __syncthreads();
+    {
+        unsigned char *const stg = lds_all + wave * 32 * kRowBytes;
+        const float inv          = l_i > 0.f ? 1.0f / l_i : 0.f;
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                u32x2 w;
+                w[0] = AttnT<DT>::pack2(oacc[dt][r4 * 4 + 0] * inv, oacc[dt][r4 * 4 + 1] * inv);
+                w[1] = AttnT<DT>::pack2(oacc[dt][r4 * 4 + 2] * inv, oacc[dt][r4 * 4 + 3] * inv);
+                *reinterpret_cast<u32x2 *>(stg + lq * kRowBytes + (dt * 32 + r4 * 8 + g * 4) * 2) = w;
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const int r    = pass * 8 + (lane >> 3);
+            const int qrow = q0 + r;
+            if (qrow < S) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(stg + r * kRowBytes + (lane & 7) * 16);
+                *reinterpret_cast<u32x4 *>(ob + (size_t)qrow * p.o_ss + (lane & 7) * 8) = v;
+                if (p.oq) {
+                    u32x2 q8;
+#pragma unroll
+                    for (int w = 0; w < 2; ++w) {
+                        uint32_t packed = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t word = v[w * 2 + (e >> 1)];
+                            const float f       = AttnT<DT>::to_float((uint16_t)(e & 1 ? word >> 16 : word & 0xffffu));
+                            packed |= (uint32_t)(uint8_t)float2int8_ref(__fmul_rn(f, p.q_inv)) << (8 * e);
+                        }
+                        q8[w] = packed;
+                    }
+                    int8_t *oqb = p.oq + (size_t)b * p.o_sb + (size_t)head * p.o_sh;
+                    *reinterpret_cast<u32x2 *>(oqb + (size_t)qrow * p.o_ss + (lane & 7) * 8) = q8;
+                }
+            }
+        }
+    }
+}
+
 __global__ void mask_to_kv_len_kernel(const float *__restrict__ mask, int32_t *__restrict__ kv_len, int S,
-                                      float threshold) {
+                                      float threshold, int flag_zero_rows) {
     // one wave per batch row: the largest index whose mask value is above the threshold
     const int b    = blockIdx.x;
     const int lane = threadIdx.x;
@@ -428,14 +772,42 @@ __global__ void mask_to_kv_len_kernel(const float *__restrict__ mask, int32_t *_
         int other = __shfl_xor(last, o, 64);
         last      = other > last ? other : last;
     }
+    int len = last + 1;
+    if (flag_zero_rows) {
+        // a plain padding mask is exactly 0 on every visible key: the attention kernel then needs the length only
+        int nonzero = 0;
+        for (int j = lane; j < len; j += 64)
+            nonzero |= mask[(size_t)b * S + j] != 0.0f ? 1 : 0;
+        if (!__any(nonzero))
+            len |= kKvLenMaskZero;
+    }
     if (lane == 0)
-        kv_len[b] = last + 1;
+        kv_len[b] = len;
 }
 
 // 128-row query blocks when that already gives >= 2 workgroups per CU, else 64-row blocks
+int g_attention_dma = 1;  // experiment hook: 0 keeps the register-staged kernel for the V^T layout as well
+
 template <bool VT> int launch_attention(hipStream_t s, int dtype, const AttnParams &p, int B, int heads, int S) {
     long blocks128 = (long)((S + 127) / 128) * heads * B;
     auto padded = [&](long n_q) { return dim3((unsigned)(((n_q * heads * B + 7) / 8) * 8)); };
+    if (VT && g_attention_dma) {
+        if (blocks128 >= 512) {
+            dim3 grid = padded((S + 127) / 128);
+            if (dtype == TNN_ROCM_F16)
+                hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_F16, 4>), grid, dim3(256), 0, s, p);
+            else
+                hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_BF16, 4>), grid, dim3(256), 0, s, p);
+        } else {
+            dim3 grid = padded((S + 63) / 64);
+            if (dtype == TNN_ROCM_F16)
+                hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_F16, 2>), grid, dim3(128), 0, s, p);
+            else
+                hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_BF16, 2>), grid, dim3(128), 0, s, p);
+        }
+        TR_CHECK_LAUNCH();
+        return 0;
+    }
     if (blocks128 >= 512) {
         dim3 grid = padded((S + 127) / 128);
         if (dtype == TNN_ROCM_F16)
@@ -548,12 +920,27 @@ int tnn_rocm_attention_vt_q8(void *stream, int dtype, const void *q, const void 
     return launch_attention<true>((hipStream_t)stream, dtype, p, B, heads, S);
 }
 
+__attribute__((visibility("default"))) int tnn_rocm_debug_set_attention_dma(int on) {
+    g_attention_dma = on;
+    return 0;
+}
+
 int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_t *kv_len, int B, int S, float threshold) {
     TR_REQUIRE(B >= 0 && S >= 0, TNN_ROCM_ESHAPE, "mask_to_kv_len: negative size");
     if (B == 0)
         return 0;
     TR_REQUIRE(mask && kv_len, TNN_ROCM_EINVAL, "mask_to_kv_len: null pointer");
-    hipLaunchKernelGGL(mask_to_kv_len_kernel, dim3(B), dim3(64), 0, (hipStream_t)stream, mask, kv_len, S, threshold);
+    hipLaunchKernelGGL(mask_to_kv_len_kernel, dim3(B), dim3(64), 0, (hipStream_t)stream, mask, kv_len, S, threshold, 0);
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+int tnn_rocm_mask_to_kv_len_flagged(void *stream, const float *mask, int32_t *kv_len, int B, int S, float threshold) {
+    TR_REQUIRE(B >= 0 && S >= 0 && S < kKvLenMaskZero, TNN_ROCM_ESHAPE, "mask_to_kv_len: bad size");
+    if (B == 0)
+        return 0;
+    TR_REQUIRE(mask && kv_len, TNN_ROCM_EINVAL, "mask_to_kv_len: null pointer");
+    hipLaunchKernelGGL(mask_to_kv_len_kernel, dim3(B), dim3(64), 0, (hipStream_t)stream, mask, kv_len, S, threshold, 1);
     TR_CHECK_LAUNCH();
     return 0;
 }

@@ -922,6 +922,7 @@ __global__ void __launch_bounds__(CFG::NT)
             // consumed by MFMAs already issued).  A bare barrier: __syncthreads() adds a fence that waits for
             // every outstanding load, the look-ahead ones included.
             __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");  // no LDS access may be moved across the barrier by the compiler
             if (kt + NS - 1 < nk)
                 issue(kt + NS - 1, fill);
             compute(stage);

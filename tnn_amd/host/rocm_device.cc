@@ -70,7 +70,8 @@ Status RocmContext::AttentionMask(const void *mask_blob, int mask_dtype, int B, 
         if (mask_dtype != TNN_ROCM_F32)
             ROCM_CALL(tnn_rocm_cast(stream_, mask_dtype, mask_blob, TNN_ROCM_F32, c.mask_f32, (size_t)B * S));
         // keys whose additive mask is <= -1000 after the last visible key contribute exp(-1000 - max) == 0 in fp32
-        ROCM_CALL(tnn_rocm_mask_to_kv_len(stream_, m, (int32_t *)c.kv_len, B, S, -1000.0f));
+        // (a plain 0 / -10000 padding mask is flagged: the attention kernel then works from the lengths alone)
+        ROCM_CALL(tnn_rocm_mask_to_kv_len_flagged(stream_, m, (int32_t *)c.kv_len, B, S, -1000.0f));
         c.src   = mask_blob;
         c.epoch = forward_epoch_;
     }

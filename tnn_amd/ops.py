@@ -172,11 +172,13 @@ def attention_qk_vt(qk, vt, B, S, heads, scale, mask=None, kv_len=None, out=None
     return out
 
 
-def mask_to_kv_len(mask, threshold=-1000.0):
+def mask_to_kv_len(mask, threshold=-1000.0, flagged=False):
+    """flagged: bit 30 of an entry marks a mask row that is exactly 0 on every visible key"""
     _chk(mask)
     B, S = mask.shape
     out = torch.empty(B, dtype=torch.int32, device=mask.device)
-    capi.call("tnn_rocm_mask_to_kv_len", _stream(), _p(mask), _p(out), B, S, float(threshold))
+    capi.call("tnn_rocm_mask_to_kv_len_flagged" if flagged else "tnn_rocm_mask_to_kv_len", _stream(), _p(mask), _p(out), B,
+              S, float(threshold))
     return out
 
 
