@@ -34,6 +34,8 @@ constexpr int kRowBytes = kD * 2 + 16;   // padded LDS row (K: one key's 64 half
 constexpr float kLog2e  = 1.4426950408889634f;
 constexpr int kKvLenMaskZero = 1 << 30;  // flag bit of a kv_len entry, see tnn_rocm_mask_to_kv_len_flagged
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
 template <int DT> struct AttnT;
 template <> struct AttnT<TNN_ROCM_F16> {
     template <typename V> static __device__ __forceinline__ void mma(const V &a, const V &b, f32x16 &c) {
@@ -45,9 +47,14 @@ template <> struct AttnT<TNN_ROCM_F16> {
         half_t l = (half_t)lo, h = (half_t)hi;
         return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
     }
-    // Probabilities (0..1) for the second MFMA: one v_cvt_pkrtz per pair.  The row sum is taken over the SAME
-    // rounded values (v_dot2 with (1,1), fp32 accumulate), so numerator and denominator of the softmax stay
-    // consistent and the truncation does not bias the normalised weights.
+    // eight packed values times a scalar, rounded to nearest (fp32 product, one rounding)
+    static __device__ __forceinline__ u32x4 scale8(u32x4 v, float c) {
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            o[i] = pack2(to_float((uint16_t)(v[i] & 0xffffu)) * c, to_float((uint16_t)(v[i] >> 16)) * c);
+        return o;
+    }
     // the same in two steps, for callers that shuffle the packed pairs before summing them
     static __device__ __forceinline__ uint32_t pack_only(float lo, float hi) {
         return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
@@ -57,6 +64,9 @@ template <> struct AttnT<TNN_ROCM_F16> {
         h2 one = {(_Float16)1.0f, (_Float16)1.0f};
         sum    = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, pk), one, sum, false);
     }
+    // Probabilities (0..1) for the second MFMA: one v_cvt_pkrtz per pair.  The row sum is taken over the SAME
+    // rounded values (v_dot2 with (1,1), fp32 accumulate), so numerator and denominator of the softmax stay
+    // consistent and the truncation does not bias the normalised weights.
     static __device__ __forceinline__ uint32_t pack_prob(float lo, float hi, float &sum) {
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
         typedef __fp16 fp16x2 __attribute__((ext_vector_type(2)));
@@ -74,6 +84,13 @@ template <> struct AttnT<TNN_ROCM_BF16> {
     static __device__ __forceinline__ float to_float(uint16_t bits) { return __uint_as_float((uint32_t)bits << 16); }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+    }
+    static __device__ __forceinline__ u32x4 scale8(u32x4 v, float c) {
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            o[i] = pack2(to_float((uint16_t)(v[i] & 0xffffu)) * c, to_float((uint16_t)(v[i] >> 16)) * c);
+        return o;
     }
     static __device__ __forceinline__ uint32_t pack_only(float lo, float hi) {
         return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
@@ -101,7 +118,6 @@ struct AttnParams {
     float q_inv;  // 1 / scale of that int8 tensor
 };
 
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 // Combine a value with the one held by lane ^ 32 (the other half of the same query column) with one
@@ -562,7 +578,8 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
         __syncthreads();
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
-            qf[kk] = *reinterpret_cast<const u32x4 *>(stage + (wave * 32 + lq) * kRowBytes + kk * 32 + g * 16);
+            qf[kk] = AttnT<DT>::scale8(*reinterpret_cast<const u32x4 *>(stage + (wave * 32 + lq) * kRowBytes + kk * 32 + g * 16),
+                                       p.scale_log2e);  // scores come out of the MFMA in the exp2 domain
         __syncthreads();
     }
     if (n_tiles > 1)
@@ -601,25 +618,35 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
         const unsigned char *const kbuf  = lds_all + stage * kStage;
         const unsigned char *const vtbuf = kbuf + kTile;
         const int kv0     = t * kTileKV;
-        const bool biased = mb != nullptr || kv0 + kTileKV > kv_end || !(p.scale_log2e > 0.f);  // workgroup-uniform
-        // The whole tile is written twice (with and without the per-key bias) under one branch: with the branch
-        // inside the tile the compiler copies the 32 score registers where the two paths meet.
-        auto tile = [&](auto biased_tag) __attribute__((always_inline)) {
-            constexpr bool BIASED = decltype(biased_tag)::value;
+        const bool biased = mb != nullptr || kv0 + kTileKV > kv_end;  // workgroup-uniform
+        // Q carries scale * log2(e) already, so the MFMA result is the score in the exp2 domain.
+        // The tile body is written three times under one branch (with the branch inside the tile the compiler copies
+        // the 32 score registers where the paths meet):
+        //   BIAS : per-key bias (additive mask, keys past kv_end), exact running maximum
+        //   EXACT: no bias, exact running maximum (the first tile of a row block)
+        //   STALE: no bias; the accumulators start at -m (m = the running maximum so far), so the MFMA result is
+        //          already s - m and goes straight into exp2.  m only follows the true maximum when a score exceeds
+        //          it by more than kStaleMax (2^kStaleMax still fits the packed half-precision probabilities
+        //          comfortably); then the tile's scores, the O accumulators and the row sum are rescaled.  The
+        //          normalised result does not depend on which reference the exponentials use.
+        constexpr float kStaleMax = 10.0f;
+        auto tile = [&](auto mode_tag) __attribute__((always_inline)) {
+            constexpr int MODE = decltype(mode_tag)::value;  // 0 BIAS, 1 EXACT, 2 STALE
             f32x16 sacc[2];
+            const float c_init = MODE == 2 ? -m_i : 0.f;
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
-                    sacc[kt][r] = 0.f;
+                    sacc[kt][r] = c_init;
 #pragma unroll
                 for (int kk = 0; kk < 4; ++kk) {
                     u32x4 kf = *reinterpret_cast<const u32x4 *>(kbuf + kt * 32 * 128 + frag_off[kk]);
                     AttnT<DT>::mma(kf, qf[kk], sacc[kt]);
                 }
             }
-            float mx = -INFINITY;
-            if (BIASED) {
+            float mx = -INFINITY, alpha = 1.0f;
+            if (MODE == 0) {
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
@@ -633,7 +660,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const float be       = kv0 + key0 + e < kv_end ? bv[e] : -INFINITY;
-                            float s2             = fmaf(sacc[kt][r4 * 4 + e], p.scale_log2e, be);
+                            float s2             = sacc[kt][r4 * 4 + e] + be;
                             sacc[kt][r4 * 4 + e] = s2;
                             mx                   = fmaxf(mx, s2);
                         }
@@ -645,34 +672,45 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
                         mx = fmaxf(mx, sacc[kt][r]);
-                mx *= p.scale_log2e;
             }
-            mx          = half_swap_max(mx);
-            float m_new = fmaxf(m_i, mx);
-            float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
-            if (BIASED) {
+            mx = half_swap_max(mx);
+            if (MODE == 2) {
+                if (__any(mx > kStaleMax)) {  // rare: some row's scores outgrew the reference
+                    const float delta = fmaxf(mx, 0.f);
+                    m_i += delta;
+                    alpha = __builtin_amdgcn_exp2f(-delta);
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            sacc[kt][r] -= delta;
+#pragma unroll
+                    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            oacc[dt][r] *= alpha;
+                }
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        sacc[kt][r] = __builtin_amdgcn_exp2f(sacc[kt][r]);
+            } else {
+                float m_new = fmaxf(m_i, mx);
+                float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                alpha       = __builtin_amdgcn_exp2f(m_i - m_use);
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
                         sacc[kt][r] = __builtin_amdgcn_exp2f(sacc[kt][r] - m_use);
-            } else {
-                const float neg_m = -m_use;
-#pragma unroll
-                for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        sacc[kt][r] = __builtin_amdgcn_exp2f(fmaf(sacc[kt][r], p.scale_log2e, neg_m));
-            }
-            if (!__all(m_new == m_i)) {
 #pragma unroll
                 for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
                         oacc[dt][r] *= alpha;
+                m_i = m_new;
             }
-            m_i = m_new;
 
             // ---- O^T += V^T P^T.  Register r of block kt is key kt*32 + 8*(r/4) + 4*g + (r%4): a lane half holds four
             // keys of each 8-key group.  Step st = 2*kt + j uses groups 2j and 2j+1 of the block; after exchanging the
@@ -705,9 +743,11 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
             l_i = fmaf(l_i, alpha, rs);
         };
         if (biased)
-            tile(std::true_type());
+            tile(std::integral_constant<int, 0>());
+        else if (__all(m_i > -INFINITY))  // per wave: the reference must be finite (true from the second tile on)
+            tile(std::integral_constant<int, 2>());
         else
-            tile(std::false_type());
+            tile(std::integral_constant<int, 1>());
 
         stage = stage == 2 ? 0 : stage + 1;
         fill  = fill == 2 ? 0 : fill + 1;
