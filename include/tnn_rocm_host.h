@@ -21,6 +21,17 @@ extern "C" {
  * Returns NULL on failure and writes the status text to err[err_len]. */
 void *tnn_host_create(const char *proto, size_t proto_len, const char *model, size_t model_len, int device_id,
                       int precision, char *err, size_t err_len);
+/* The same with the instance created at other input shapes than the proto's: Instance::Init(interpreter,
+ * min_inputs_shape, max_inputs_shape) (reference source/tnn/core/instance.cc:48-128; include/tnn/core/tnn.h:77-85
+ * CreateInst(config, status, inputs_shape)).  names[i] has ndims[i] dimensions, taken one after another from dims.
+ * Blob memory is planned at these shapes; later tnn_host_reshape calls to anything that fits stay allocation-free. */
+void *tnn_host_create_shaped(const char *proto, size_t proto_len, const char *model, size_t model_len, int device_id,
+                             int precision, int n_inputs, const char *const *names, const int *ndims, const int *dims,
+                             char *err, size_t err_len);
+/* Instance::Reshape (instance.h:62, reference source/tnn/core/instance.cc:143-152 ->
+ * source/tnn/core/default_network.cc:456-500): new dims for the named inputs (same rank), every layer infers its
+ * output shape again and its acc is reshaped; weights stay on the device.  An unknown name is TNNERR_PARAM_ERR. */
+int tnn_host_reshape(void *handle, int n_inputs, const char *const *names, const int *ndims, const int *dims);
 /* ~Instance (instance.h:46) */
 void tnn_host_destroy(void *handle);
 const char *tnn_host_last_error(void *handle);

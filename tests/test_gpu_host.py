@@ -414,3 +414,96 @@ def test_model_check_and_profile_report():
     say(text)
     assert "Profiling Data Sort by Cost time" in text and "kernel runtime total" in text and "[2,128,3072] [2,128,768]" in text
     assert text.count("RocmFusedLinear") >= 12   # six layers in each of the two per-layer tables
+
+
+def test_instance_reshape_matches_fresh_instances():
+    """Instance::Reshape (default_network.cc:456-500): one instance moved through several (B, S) gives, at each shape and
+    on each of four forwards (eager, eager, record + launch, replay), exactly what an instance created at that shape
+    gives; weights are uploaded once; a shape beyond the planned blob memory re-plans it; a shape seen before replays
+    its recording.  One shape is also held against the checker."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: Instance::Reshape through several shapes, 2-layer encoder fp16")
+    cfg = EncoderConfig(2, 256, 4, 512)
+    S_MAX = 96
+    w = make_weights(cfg, seed=21, bias_std=0.05)
+    w["pos_emb"] = w["pos_emb"][:S_MAX]
+
+    def shapes(B, S):
+        return {"input_ids": [B, S], "token_type_ids": [B, S], "attention_bias": [B, 1, 1, S]}
+
+    def feed(inst, B, S, seed):
+        ids, seg, lens, mask = make_inputs(cfg, B, S, max(S // 3, 1), S, seed=seed)
+        inst.set_input("input_ids", ids)
+        inst.set_input("token_type_ids", seg)
+        inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+        return ids, seg, mask
+
+    g = tnnmodel.encoder_graph(cfg, w, 4, S_MAX, dynamic=True)
+    inst = host.RocmInstance.from_graph(g, "fp16", input_shapes=shapes(4, 64))
+    types = [t for t, _ in inst.layers()]
+    assert types.count("RocmFusedAttention") == 2 and types.count("RocmFusedEmbedding") == 1, types
+    assert types.count("LayerNorm") == 1, types     # folding also happens when S is only known at reshape time
+    # (4,64) created; shrink twice; S not a multiple of 8; beyond the planned memory; back to shapes seen before
+    walk = [(4, 64), (2, 40), (3, 24), (2, 36), (5, 96), (2, 40), (4, 64), (1, 8)]
+    for step, (B, S) in enumerate(walk):
+        say("  shape B=%d S=%d" % (B, S))
+        if step:
+            inst.reshape(shapes(B, S))
+        io = {l["name"]: l for l in inst.layer_io()}
+        assert any(d == [B, S, cfg.hidden] for l in io.values() for d in l["output_dims"])
+        ids, seg, mask = feed(inst, B, S, 100 + step)
+        fresh = host.RocmInstance.from_graph(g, "fp16", input_shapes=shapes(B, S))
+        feed(fresh, B, S, 100 + step)
+        fresh.forward()
+        want = fresh.output("last_hidden")
+        fresh.close()
+        assert want.shape == (B, S, cfg.hidden)
+        for it in range(4):
+            inst.forward()
+            got = inst.output("last_hidden")
+            assert got.shape == want.shape
+            assert np.array_equal(got, want), "shape %s forward %d differs from a fresh instance" % ((B, S), it)
+        if (B, S) == (2, 36):
+            wr = r16w(w)
+            ref = encoder_ref.encoder(wr, cfg, encoder_ref.embed(wr, ids, seg, cfg.eps), B, S, mask)
+            err = rel_err(got.reshape(B * S, -1), ref)
+            say("  S=36 against the checker: max rel err %.3g" % err)
+            assert err <= FP16_TOL
+    # error behaviour of default_network.cc:470-475 (unknown blob) plus the rank check
+    with pytest.raises(host.HostError, match="blob name is wrong"):
+        inst.reshape({"no_such_input": [1, 8]})
+    with pytest.raises(host.HostError, match="number of dimensions"):
+        inst.reshape({"input_ids": [8]})
+    # inputs that no longer agree with each other fail in the layer that notices, with its name
+    with pytest.raises(host.HostError):
+        inst.reshape({"input_ids": [2, 16]})
+    inst.close()
+
+
+def test_instance_reshape_fp32_batch_only_with_static_head_split():
+    """A graph whose head split names B and S cannot change them (the element count check of reshape_layer.cc:41-63
+    fails, as in the engine); the error names the layer.  The un-fused fp32 path reshapes through the dynamic graph."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: Instance::Reshape on fp32 graphs")
+    cfg = EncoderConfig(1, 128, 2, 256)
+    w = make_weights(cfg, seed=31, bias_std=0.05)
+    w["pos_emb"] = w["pos_emb"][:32]
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, 2, 32), "fp32")
+    with pytest.raises(host.HostError, match="reshape of layer"):
+        inst.reshape({"input_ids": [2, 16], "token_type_ids": [2, 16], "attention_bias": [2, 1, 1, 16]})
+    inst.close()
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, 2, 32, dynamic=True), "fp32")
+    for B, S in ((2, 32), (3, 16), (1, 24)):
+        if (B, S) != (2, 32):
+            inst.reshape({"input_ids": [B, S], "token_type_ids": [B, S], "attention_bias": [B, 1, 1, S]})
+        ids, seg, lens, mask = make_inputs(cfg, B, S, S // 2, S, seed=40 + S)
+        inst.set_input("input_ids", ids)
+        inst.set_input("token_type_ids", seg)
+        inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+        inst.forward()
+        got = inst.output("last_hidden").reshape(B * S, -1)
+        ref = encoder_ref.encoder(w, cfg, encoder_ref.embed(w, ids, seg, cfg.eps), B, S, mask)
+        err = rel_err(got, ref)
+        say("  fp32 B=%d S=%d max rel err %.3g" % (B, S, err))
+        assert err <= FP32_TOL
+    inst.close()

@@ -13,6 +13,10 @@ LIB_PATH = os.path.join(HERE, "lib", "libtnn_rocm_host.so")
 SIGNATURES = {
     "tnn_host_create": (C.c_void_p, [C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t, C.c_int, C.c_int, C.c_char_p,
                                      C.c_size_t]),
+    "tnn_host_create_shaped": (C.c_void_p, [C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t, C.c_int, C.c_int, C.c_int,
+                                            C.POINTER(C.c_char_p), C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_char_p,
+                                            C.c_size_t]),
+    "tnn_host_reshape": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_char_p), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "tnn_host_destroy": (None, [C.c_void_p]),
     "tnn_host_last_error": (C.c_char_p, [C.c_void_p]),
     "tnn_host_set_input": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]),
@@ -49,24 +53,45 @@ class HostError(RuntimeError):
     pass
 
 
+def _shape_args(input_shapes):
+    items = sorted(input_shapes.items())
+    names = (C.c_char_p * len(items))(*[k.encode() for k, _ in items])
+    ndims = (C.c_int * len(items))(*[len(v) for _, v in items])
+    flat = [int(d) for _, v in items for d in v]
+    dims = (C.c_int * max(len(flat), 1))(*flat)
+    return len(items), names, ndims, dims
+
+
 class RocmInstance:
     """precision: "fp32" (PRECISION_HIGH), "fp16" (PRECISION_AUTO: fp16 activations + fused kernels) or "bf16"
     (PRECISION_LOW: bf16 activations + fused kernels)."""
 
-    def __init__(self, proto, model, precision="fp16", device_id=0):
+    def __init__(self, proto, model, precision="fp16", device_id=0, input_shapes=None):
+        """input_shapes {name: dims}: create the instance at these shapes instead of the proto's (the engine's
+        max_inputs_shape); reshape() later moves within or beyond them."""
         lib = load()
         if isinstance(proto, str):
             proto = proto.encode()
         err = C.create_string_buffer(1024)
-        self._h = lib.tnn_host_create(proto, len(proto), model, len(model), device_id,
-                                      {"fp32": 0, "fp16": 1, "bf16": 2}[precision], err, 1024)
+        prec = {"fp32": 0, "fp16": 1, "bf16": 2}[precision]
+        if input_shapes:
+            n, names, ndims, dims = _shape_args(input_shapes)
+            self._h = lib.tnn_host_create_shaped(proto, len(proto), model, len(model), device_id, prec, n, names, ndims,
+                                                 dims, err, 1024)
+        else:
+            self._h = lib.tnn_host_create(proto, len(proto), model, len(model), device_id, prec, err, 1024)
         if not self._h:
             raise HostError("Instance::Init failed: " + err.value.decode())
         self._keep = []
 
     @classmethod
-    def from_graph(cls, graph, precision="fp16"):
-        return cls(graph.proto(), graph.model(), precision)
+    def from_graph(cls, graph, precision="fp16", input_shapes=None):
+        return cls(graph.proto(), graph.model(), precision, input_shapes=input_shapes)
+
+    def reshape(self, input_shapes):
+        """Instance::Reshape: {input name: new dims}"""
+        n, names, ndims, dims = _shape_args(input_shapes)
+        self._check(load().tnn_host_reshape(self._h, n, names, ndims, dims), "Reshape")
 
     def _check(self, rc, what):
         if rc != 0:

@@ -50,6 +50,43 @@ HOST_API void *tnn_host_create(const char *proto, size_t proto_len, const char *
     return h;
 }
 
+// As tnn_host_create, at other input shapes than the proto's (the max_inputs_shape of instance.cc:48-128): n_inputs
+// names, ndims[i] dimensions each, taken one after another from dims.
+HOST_API void *tnn_host_create_shaped(const char *proto, size_t proto_len, const char *model, size_t model_len, int device_id,
+                                      int precision, int n_inputs, const char *const *names, const int *ndims, const int *dims,
+                                      char *err, size_t err_len) {
+    auto h = new Handle;
+    NetworkConfig nc;
+    nc.device_type = DEVICE_ROCM;
+    nc.device_id   = device_id;
+    nc.precision   = precision == 0 ? PRECISION_HIGH : (precision == 2 ? PRECISION_LOW : PRECISION_AUTO);
+    ModelConfig mc;
+    mc.params.push_back(std::string(proto, proto_len));
+    mc.params.push_back(std::string(model, model_len));
+    InputShapesMap shapes;
+    for (int i = 0, k = 0; i < n_inputs; k += ndims[i], ++i)
+        shapes[names[i]] = DimsVector(dims + k, dims + k + ndims[i]);
+    h->inst   = std::make_shared<Instance>(nc, mc);
+    Status st = h->inst->Init(InputShapesMap(), shapes);
+    if (st != TNN_OK) {
+        if (err && err_len)
+            snprintf(err, err_len, "%s", st.description().c_str());
+        delete h;
+        return nullptr;
+    }
+    return h;
+}
+
+// Instance::Reshape (instance.cc:143-152): new dims for the named inputs; the other inputs keep theirs.
+HOST_API int tnn_host_reshape(void *hp, int n_inputs, const char *const *names, const int *ndims, const int *dims) {
+    auto h = static_cast<Handle *>(hp);
+    InputShapesMap shapes;
+    for (int i = 0, k = 0; i < n_inputs; k += ndims[i], ++i)
+        shapes[names[i]] = DimsVector(dims + k, dims + k + ndims[i]);
+    Status st = h->inst->Reshape(shapes);
+    return st == TNN_OK ? 0 : fail(h, st);
+}
+
 HOST_API void tnn_host_destroy(void *hp) { delete static_cast<Handle *>(hp); }
 HOST_API const char *tnn_host_last_error(void *hp) { return static_cast<Handle *>(hp)->err.c_str(); }
 

@@ -520,7 +520,14 @@ Status BaseLayer::Init(Context *context, LayerParam *param, LayerResource *resou
         RETURN_ON_NEQ(layer_acc_->ResolveBlobDataFormat(b, BLOB_OUTPUT), TNN_OK);
     return layer_acc_->Init(context, param_, resource_, input_blobs_, output_blobs_);
 }
-Status BaseLayer::Reshape() {
+Status BaseLayer::Reshape() {  // base_layer.cc:167-188
+    RETURN_ON_NEQ(InferOutputShape(), TNN_OK);
+    for (auto b : output_blobs_)
+        for (int d : b->GetBlobDesc().dims)
+            if (d < 0)
+                return Status(TNNERR_LAYER_ERR, "layer output dims is invalid");
+    if (layer_acc_ == nullptr)
+        return Status(TNNERR_LAYER_ERR, "layer acc is nil");
     RETURN_ON_NEQ(layer_acc_->ReloadConstantBlobs(input_blobs_, true), TNN_OK);
     return layer_acc_->Reshape(input_blobs_, output_blobs_);
 }
@@ -1004,7 +1011,7 @@ DefaultNetwork::~DefaultNetwork() {
     if (device_)
         for (void *p : allocations_)
             device_->Free(p);
-    tnn_rocm_graph_destroy(graph_exec_);
+    DropGraphs();
     for (auto &e : prof_events_) {
         tnn_rocm_event_destroy(e.first);
         tnn_rocm_event_destroy(e.second);
@@ -1012,7 +1019,7 @@ DefaultNetwork::~DefaultNetwork() {
     delete context_;
 }
 
-Status DefaultNetwork::Init(NetworkConfig &net_config, ModelInterpreter *interpreter) {
+Status DefaultNetwork::Init(NetworkConfig &net_config, ModelInterpreter *interpreter, const InputShapesMap &max_inputs_shape) {
     config_ = net_config;
     if (const char *g = getenv("TNN_ROCM_GRAPH"))
         graph_enabled_ = atoi(g) != 0;
@@ -1030,6 +1037,14 @@ Status DefaultNetwork::Init(NetworkConfig &net_config, ModelInterpreter *interpr
     for (auto &l : interpreter->GetNetStructure()->layers)
         structure_.layers.push_back(std::make_shared<LayerInfo>(*l));
     resource_ = *interpreter->GetNetResource();
+    for (auto &kv : max_inputs_shape) {  // instance.cc:76-83 / default_network.cc:104-108
+        auto it = structure_.inputs_shape_map.find(kv.first);
+        if (it == structure_.inputs_shape_map.end())
+            return Status(TNNERR_PARAM_ERR, "input shape given for " + kv.first + ", which is not an input of the model");
+        if (it->second.size() != kv.second.size())
+            return Status(TNNERR_PARAM_ERR, "input shape given for " + kv.first + " has another number of dimensions than the model's");
+        it->second = kv.second;
+    }
     RETURN_ON_NEQ(RunNetOptimizers(&structure_, &resource_, config_), TNN_OK);
     RETURN_ON_NEQ(InitLayers(), TNN_OK);
     RETURN_ON_NEQ(AllocateBlobMemory(), TNN_OK);
@@ -1037,6 +1052,86 @@ Status DefaultNetwork::Init(NetworkConfig &net_config, ModelInterpreter *interpr
     for (auto l : layers_)
         RETURN_ON_NEQ(l->Reshape(), TNN_OK);
     return context_->OnInstanceReshapeEnd();
+}
+
+std::string DefaultNetwork::ShapeKey() const {
+    std::ostringstream os;
+    for (auto &kv : inputs_) {
+        os << kv.first << ":";
+        for (int d : kv.second->GetBlobDesc().dims)
+            os << d << ",";
+        os << ";";
+    }
+    return os.str();
+}
+void DefaultNetwork::DropGraphs() {
+    for (auto &g : graphs_)
+        tnn_rocm_graph_destroy(g.second);
+    graphs_.clear();
+    graph_exec_ = nullptr;
+}
+Status DefaultNetwork::ReleaseBlobMemory() {
+    RETURN_ON_NEQ(context_->Synchronize(), TNN_OK);
+    for (auto &kv : blob_capacity_)
+        kv.first->SetHandle(BlobHandle());
+    blob_capacity_.clear();
+    for (void *p : allocations_)
+        device_->Free(p);
+    allocations_.clear();
+    return TNN_OK;
+}
+
+// default_network.cc:456-500 (Reshape -> PrepareDoReshape -> DoReshape -> ReshapeLayers)
+Status DefaultNetwork::Reshape(const InputShapesMap &inputs) {
+    bool shape_changed = false;
+    for (auto &kv : inputs) {
+        auto it = inputs_.find(kv.first);
+        if (it == inputs_.end())
+            return Status(TNNERR_PARAM_ERR, "DefaultNetwork reshape blob is empty, maybe the blob name is wrong");
+        auto &dims = it->second->GetBlobDesc().dims;
+        if (dims.size() != kv.second.size())
+            return Status(TNNERR_PARAM_ERR, "DefaultNetwork reshape: input " + kv.first + " keeps its number of dimensions");
+        for (int d : kv.second)
+            if (d <= 0)
+                return Status(TNNERR_PARAM_ERR, "DefaultNetwork reshape: input " + kv.first + " gets a dimension below 1");
+        if (dims != kv.second) {
+            dims          = kv.second;
+            shape_changed = true;
+        }
+    }
+    if (!shape_changed)
+        return TNN_OK;
+    // nothing of the old shape may still be running when blobs change size or move
+    RETURN_ON_NEQ(context_->Synchronize(), TNN_OK);
+    graph_exec_     = nullptr;
+    eager_forwards_ = 0;
+    RETURN_ON_NEQ(context_->OnInstanceReshapeBegin(), TNN_OK);
+    // shapes first (layer order = topological order), then memory, then the accs, which may look at the blobs' memory
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        Status st = layers_[i]->InferOutputShape();
+        if (st != TNN_OK)
+            return Status((int)st, "reshape of layer " + layers_[i]->GetLayerName() + " failed: " + st.description());
+    }
+    bool fits = true;
+    for (auto &kv : blob_capacity_) {
+        BlobMemorySizeInfo info = device_->Calculate(kv.first->GetBlobDesc());
+        fits &= GetBlobMemoryBytesSize(info) <= kv.second;
+    }
+    if (!fits) {
+        DropGraphs();  // they point into the buffers that go away now
+        RETURN_ON_NEQ(ReleaseBlobMemory(), TNN_OK);
+        RETURN_ON_NEQ(AllocateBlobMemory(), TNN_OK);
+    }
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        Status st = layers_[i]->Reshape();
+        if (st != TNN_OK)
+            return Status((int)st, "reshape of layer " + layers_[i]->GetLayerName() + " failed: " + st.description());
+    }
+    RETURN_ON_NEQ(context_->OnInstanceReshapeEnd(), TNN_OK);
+    auto g = graphs_.find(ShapeKey());
+    if (g != graphs_.end() && graphs_epoch_ == context_->MemoryEpoch())
+        graph_exec_ = g->second;
+    return TNN_OK;
 }
 
 Blob *DefaultNetwork::GetBlob(const std::string &name) {
@@ -1208,6 +1303,7 @@ Status DefaultNetwork::AllocateBlobMemory() {
         BlobHandle h;
         h.base = ptr;
         b->SetHandle(h);
+        blob_capacity_[b]            = bytes;
         owned[b->GetBlobDesc().name] = {bytes, ptr};
         return TNN_OK;
     };
@@ -1272,6 +1368,8 @@ Status DefaultNetwork::ForwardAsync() {
     void *stream = nullptr;
     context_->GetCommandQueue(&stream);
     const bool use_graph = graph_enabled_ && !profiling_ && config_.device_type == DEVICE_ROCM && stream != nullptr;
+    if (graph_exec_ && graphs_epoch_ != context_->MemoryEpoch())
+        DropGraphs();  // context scratch moved since the recordings were made
     if (use_graph && graph_exec_) {
         if (tnn_rocm_graph_launch(graph_exec_, stream) != 0)
             return Status(TNNERR_CUDA_KERNEL_LAUNCH_ERROR, std::string("graph launch failed: ") + tnn_rocm_last_error());
@@ -1287,7 +1385,14 @@ Status DefaultNetwork::ForwardAsync() {
                 return st;
             }
             if (rc == 0 && exec) {
-                graph_exec_ = exec;
+                if (graphs_epoch_ != context_->MemoryEpoch())
+                    DropGraphs();
+                graphs_epoch_ = context_->MemoryEpoch();
+                auto key      = ShapeKey();
+                if (graphs_.count(key))
+                    tnn_rocm_graph_destroy(graphs_[key]);
+                graphs_[key] = exec;
+                graph_exec_  = exec;
                 if (tnn_rocm_graph_launch(graph_exec_, stream) != 0)
                     return Status(TNNERR_CUDA_KERNEL_LAUNCH_ERROR,
                                   std::string("graph launch failed: ") + tnn_rocm_last_error());
@@ -1387,7 +1492,8 @@ std::vector<LayerProfile> DefaultNetwork::FinishProfile() {
 }
 
 // ---- instance (source/tnn/core/instance.cc:48-128, 166-169, 203-319) --------------------------------
-Status Instance::Init() {
+Status Instance::Init() { return Init(InputShapesMap(), InputShapesMap()); }
+Status Instance::Init(const InputShapesMap &, const InputShapesMap &max_inputs_shape) {
     interpreter_ = std::make_shared<ModelInterpreter>();
     RETURN_ON_NEQ(interpreter_->Interpret(model_config_.params), TNN_OK);
     auto device = GetDevice(net_config_.device_type);
@@ -1396,7 +1502,13 @@ Status Instance::Init() {
     if (net_config_.network_type == NETWORK_TYPE_AUTO)
         net_config_.network_type = device->ConvertAutoNetworkType();
     network_ = std::make_shared<DefaultNetwork>();
-    return network_->Init(net_config_, interpreter_.get());
+    return network_->Init(net_config_, interpreter_.get(), max_inputs_shape);
+}
+Status Instance::Reshape(const InputShapesMap &inputs) {
+    if (!network_)
+        return Status(TNNERR_INST_ERR, "instance not initialised");
+    output_mats_.clear();
+    return network_->Reshape(inputs);
 }
 Status Instance::Forward() { return network_ ? network_->Forward() : Status(TNNERR_INST_ERR, "instance not initialised"); }
 Status Instance::ForwardAsync() {

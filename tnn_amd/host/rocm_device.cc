@@ -56,15 +56,20 @@ Status RocmContext::OnInstanceForwardBegin() {
 Status RocmContext::AttentionMask(const void *mask_blob, int mask_dtype, int B, int S, const float **mask_f32,
                                   const int32_t **kv_len) {
     auto &c = mask_cache_;
-    if (c.B != B || c.S != S || !c.kv_len) {
+    if ((size_t)B * S > c.cap_mask || (size_t)B > c.cap_len || !c.kv_len) {
         ROCM_CALL(tnn_rocm_stream_sync(stream_));
         tnn_rocm_free(c.mask_f32);
         tnn_rocm_free(c.kv_len);
         c.mask_f32 = c.kv_len = nullptr;
+        c.cap_mask = c.cap_len = 0;
+        ++memory_epoch_;
         ROCM_CALL(tnn_rocm_malloc(&c.mask_f32, (size_t)B * S * sizeof(float)));
         ROCM_CALL(tnn_rocm_malloc(&c.kv_len, (size_t)B * sizeof(int32_t)));
-        c.B = B, c.S = S, c.src = nullptr;
+        c.cap_mask = (size_t)B * S, c.cap_len = (size_t)B;
+        c.src = nullptr;
     }
+    if (c.B != B || c.S != S)
+        c.B = B, c.S = S, c.src = nullptr;
     const float *m = mask_dtype == TNN_ROCM_F32 ? (const float *)mask_blob : (const float *)c.mask_f32;
     if (c.src != mask_blob || c.epoch != forward_epoch_) {
         if (mask_dtype != TNN_ROCM_F32)
@@ -98,6 +103,7 @@ Status RocmContext::Workspace(size_t bytes, void **ptr) {
         tnn_rocm_free(workspace_);
         workspace_    = nullptr;
         workspace_sz_ = 0;
+        ++memory_epoch_;
         size_t want   = bytes + bytes / 4;
         int rc        = tnn_rocm_malloc(&workspace_, want);
         if (rc != 0)

@@ -33,6 +33,7 @@ public:
     Status OnInstanceForwardBegin() override;
     Status OnInstanceForwardEnd() override { return TNN_OK; }
     Status Synchronize() override;
+    uint64_t MemoryEpoch() const override { return memory_epoch_; }
 
     void *Stream() { return stream_; }
     // grow-only scratch owned by the context; valid until the next call with a larger size
@@ -51,10 +52,12 @@ private:
     size_t workspace_sz_ = 0;
     int32_t *error_flag_ = nullptr;
     uint64_t forward_epoch_ = 0;
+    uint64_t memory_epoch_  = 0;
     struct MaskEntry {
         const void *src = nullptr;
         uint64_t epoch  = 0;
         int B = 0, S = 0;
+        size_t cap_mask = 0, cap_len = 0;  // elements allocated (grow-only, so recorded launch sequences stay valid)
         void *mask_f32 = nullptr, *kv_len = nullptr;
     } mask_cache_;
 };

@@ -413,7 +413,9 @@ private:
                 int heads    = shape_q[shape_q.size() - 2];
                 int head_dim = shape_q.back();
                 int seq      = shape_q[shape_q.size() - 3];
-                if (heads * head_dim != H || head_dim != 64 || seq <= 0)
+                // seq 0 / -1: the split copies (or infers) the sequence length, i.e. the model is meant for
+                // Instance::Reshape; the acc then reads S from its input blob [B,S,H] at every reshape
+                if (heads * head_dim != H || head_dim != 64 || seq < -1)
                     continue;
                 int first = *std::min_element(chain.begin(), chain.end());
                 if (!mask.empty()) {
@@ -440,7 +442,7 @@ private:
                 fp->scale    = scale;
                 fp->has_mask = mask.empty() ? 0 : 1;
                 fl->param    = fp;
-                fp->seq_len  = seq;
+                fp->seq_len  = seq > 0 ? seq : 0;
                 auto fr       = std::make_shared<RocmFusedLinearResource>();
                 fr->name      = fl->name;
                 fr->weight_nk = RawBuffer(3 * H * K * 4, {3 * H, K});
@@ -499,7 +501,7 @@ private:
                     ++owners;
                 } else if (c->type == LAYER_ROCM_FUSED_ATTENTION) {
                     auto cp = ParamOf<RocmFusedAttentionParam>(c);
-                    if (!cp->quant && !cp->ln_fold && cp->seq_len > 0 && cp->seq_len % 8 == 0 &&
+                    if (!cp->quant && !cp->ln_fold && cp->seq_len >= 0 && cp->seq_len % 8 == 0 &&
                         std::count(c->inputs.begin(), c->inputs.end(), y) == 1)
                         owner = ci, C = cp->heads * cp->head_dim;
                     ++owners;
@@ -1148,9 +1150,9 @@ public:
             RETURN_ON_NEQ(UploadConverted(dequant.data(), (size_t)N, DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &dequant_), TNN_OK);
         }
         if (!weight_ && p->ln_fold) {
-            if (p->quant || seq_ % 8 != 0 || H_ % 128 != 0 || outputs.size() != 1u + (p->ln_y ? 1u : 0u) + (p->out_quant ? 1u : 0u) ||
+            if (p->quant || H_ % 128 != 0 || outputs.size() != 1u + (p->ln_y ? 1u : 0u) + (p->out_quant ? 1u : 0u) ||
                 res->ln_gamma.GetDataCount() != H_ || res->ln_beta.GetDataCount() != H_)
-                return Status(TNNERR_PARAM_ERR, "fused attention with a folded LayerNorm: S % 8 == 0, hidden size a multiple "
+                return Status(TNNERR_PARAM_ERR, "fused attention with a folded LayerNorm: a hidden size that is a multiple "
                                                 "of 128 and scale / shift of that width are required");
             std::vector<float> wf, cs, bf;
             FoldLayerNormIntoWeights(res->weight_nk.force_to<float *>(), res->bias.force_to<float *>(),
@@ -1227,8 +1229,17 @@ public:
                                                (long)seq_ * H_, d, (long)H_, p->scale, mask, kv));
             return TNN_OK;
         }
-        ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 1, Ptr(inputs[0]), weight_, qkv, T_, 3 * H_, H_, H_, H_, 3 * H_, 1, 1, 1,
-                                TNN_ROCM_EPI_BIAS, (const float *)bias_, nullptr, 0));
+        // sequence lengths that are not a multiple of 8 (only reachable by Instance::Reshape when a fold was decided
+        // at another length): packed Q|K|V rows and the kernel that reads V row-major
+        if (p->out_quant)
+            return Status(TNNERR_PARAM_ERR, "fused attention: the quantised output needs a sequence length that is a multiple of 8");
+        if (p->ln_fold)
+            ROCM_CALL(tnn_rocm_gemm_ln(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_, (const float *)colsum_,
+                                       (const float *)gamma_, (const float *)beta_, p->ln_eps, qkv,
+                                       p->ln_y ? Ptr(outputs[1]) : nullptr, T_, 3 * H_, H_, 0, nullptr));
+        else
+            ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 1, Ptr(inputs[0]), weight_, qkv, T_, 3 * H_, H_, H_, H_, 3 * H_, 1, 1, 1,
+                                    TNN_ROCM_EPI_BIAS, (const float *)bias_, nullptr, 0));
         const long row = 3L * H_;
         ROCM_CALL(tnn_rocm_attention(Stream(), (int)dt, base, base + (size_t)H_ * es, base + (size_t)2 * H_ * es,
                                      Ptr(outputs[0]), B_, p->heads, seq_, p->head_dim, (long)seq_ * row, d, row,
@@ -1255,17 +1266,20 @@ public:
             return Status(TNNERR_PARAM_ERR, "fused embedding: two int32 index blobs of equal shape, gamma and beta expected");
         auto wd = res->word.GetBufferDims(), td = res->type.GetBufferDims(), pd = res->pos.GetBufferDims();
         auto id = inputs[0]->GetBlobDesc().dims;
-        H_      = wd[1];
-        period_ = pd[pd.size() - 2];
-        if (id.empty() || id.back() != period_)
-            return Status(TNNERR_PARAM_ERR, "fused embedding: the position constant does not match the sequence length");
+        H_        = wd[1];
+        pos_rows_ = pd[pd.size() - 2];
+        // row t of the ids gets position t mod S.  The constant was matched at the shape the instance was created
+        // with; after a reshape to a shorter sequence its first S rows are the positions 0..S-1.
+        if (id.empty() || id.back() > pos_rows_ || id.back() <= 0)
+            return Status(TNNERR_PARAM_ERR, "fused embedding: the position constant does not cover the sequence length");
+        period_ = id.back();
         vocab_ = wd[0], types_ = td[0];
         if (word_)
             return TNN_OK;
         DataType dt = outputs[0]->GetBlobDesc().data_type;
         RETURN_ON_NEQ(UploadConverted(res->word.force_to<void *>(), (size_t)vocab_ * H_, DATA_TYPE_FLOAT, dt, &word_), TNN_OK);
         RETURN_ON_NEQ(UploadConverted(res->type.force_to<void *>(), (size_t)types_ * H_, DATA_TYPE_FLOAT, dt, &type_), TNN_OK);
-        RETURN_ON_NEQ(UploadConverted(res->pos.force_to<void *>(), (size_t)period_ * H_, DATA_TYPE_FLOAT, dt, &pos_), TNN_OK);
+        RETURN_ON_NEQ(UploadConverted(res->pos.force_to<void *>(), (size_t)pos_rows_ * H_, DATA_TYPE_FLOAT, dt, &pos_), TNN_OK);
         return TNN_OK;
     }
     Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
@@ -1287,7 +1301,7 @@ protected:
 
 private:
     void *word_ = nullptr, *type_ = nullptr, *pos_ = nullptr;
-    int H_ = 0, period_ = 0, vocab_ = 0, types_ = 0;
+    int H_ = 0, period_ = 0, pos_rows_ = 0, vocab_ = 0, types_ = 0;
 };
 REGISTER_ROCM_ACC(RocmFusedEmbeddingLayerAcc, LAYER_ROCM_FUSED_EMBEDDING);
 

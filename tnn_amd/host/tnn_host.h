@@ -486,6 +486,9 @@ public:
     virtual Status OnInstanceReshapeEnd() { return TNN_OK; }
     virtual Status Synchronize() = 0;
     virtual Status SetNumThreads(int) { return TNN_OK; }
+    // Counts the (re)allocations of device memory the context owns (scratch that grows with the shapes).  A recorded
+    // launch sequence holds raw pointers into that memory, so it is only replayed while this number stands still.
+    virtual uint64_t MemoryEpoch() const { return 0; }
     void SetPrecision(Precision p) { precision_ = p; }
     Precision GetPrecision() { return precision_; }
 
@@ -665,7 +668,13 @@ struct LayerProfile {
 class DefaultNetwork {
 public:
     ~DefaultNetwork();
-    Status Init(NetworkConfig &net_config, ModelInterpreter *interpreter);
+    // max_inputs_shape (may be empty: the model's own input shapes) is what the instance is created and its blob
+    // memory planned at (instance.cc:48-128, default_network.cc:86-137)
+    Status Init(NetworkConfig &net_config, ModelInterpreter *interpreter, const InputShapesMap &max_inputs_shape = InputShapesMap());
+    // default_network.cc:456-500: new dims for the named input blobs, then every layer infers its output shape again
+    // and its acc is reshaped.  Weights stay on the device.  Blob memory is planned again only when a blob outgrows
+    // its buffer; recorded launch sequences are kept per input-shape signature.
+    Status Reshape(const InputShapesMap &inputs);
     Status Forward();
     Status ForwardAsync();
     Status GetCommandQueue(void **command_queue);
@@ -684,6 +693,12 @@ public:
 private:
     Status InitLayers();
     Status AllocateBlobMemory();
+    Status ReleaseBlobMemory();
+    void DropGraphs();
+    std::string ShapeKey() const;
+    std::map<Blob *, int64_t> blob_capacity_;  // bytes behind each planned blob
+    std::map<std::string, void *> graphs_;     // recorded forward per input-shape signature
+    uint64_t graphs_epoch_ = 0;                // Context::MemoryEpoch() the recordings were made under
     NetworkConfig config_;
     AbstractDevice *device_ = nullptr;
     Context *context_       = nullptr;
@@ -708,6 +723,10 @@ class Instance {
 public:
     Instance(NetworkConfig &net_config, ModelConfig &model_config) : net_config_(net_config), model_config_(model_config) {}
     Status Init();
+    // instance.cc:48-128: created at max_inputs_shape (min_inputs_shape only bounds later Reshape calls in the engine;
+    // it is accepted and not used here)
+    Status Init(const InputShapesMap &min_inputs_shape, const InputShapesMap &max_inputs_shape);
+    Status Reshape(const InputShapesMap &inputs);  // instance.cc:143-152
     Status Forward();
     Status ForwardAsync();
     Status GetCommandQueue(void **command_queue);

@@ -150,11 +150,15 @@ def _linear(g, name, x, out, w_nk, bias):
     g.res_eltwise(name + "_add", "Add", bias)
 
 
-def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=()):
+def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=(), dynamic=False):
     """The decomposed encoder graph.  Inputs: input_ids, token_type_ids [B,S] int32 (or `hidden` [B,S,H] fp32
-    without embeddings) and `attention_bias` [B,1,1,S] fp32 additive mask.  Output: `last_hidden` [B,S,H]."""
+    without embeddings) and `attention_bias` [B,1,1,S] fp32 additive mask.  Output: `last_hidden` [B,S,H].
+    dynamic: the head split / merge Reshape layers copy batch and sequence length from their input (shape entries
+    0, as an export with dynamic axes has them) instead of naming B and S, so the graph can be reshaped."""
     g = Graph()
     H, h, d = cfg.hidden, cfg.heads, cfg.head_dim
+    split_shape = [0, 4, 4, 0, 0, h, d, 0] if dynamic else [0, 4, 4, B, S, h, d, 0]
+    merge_shape = [0, 3, 3, 0, 0, H, 0] if dynamic else [0, 3, 3, B, S, H, 0]
     if with_embeddings:
         g.add_input("input_ids", [B, S], DT_INT32)
         g.add_input("token_type_ids", [B, S], DT_INT32)
@@ -179,7 +183,7 @@ def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=()):
         p = "l%d_" % li
         for nm in ("q", "k", "v"):
             _linear(g, p + nm, x, p + nm + "_o", lw["w" + nm], lw["b" + nm])
-            g.add_layer("Reshape", p + nm + "_rs", [p + nm + "_o"], [p + nm + "_4d"], [0, 4, 4, B, S, h, d, 0])
+            g.add_layer("Reshape", p + nm + "_rs", [p + nm + "_o"], [p + nm + "_4d"], split_shape)
         g.add_layer("Permute", p + "q_pm", [p + "q_4d"], [p + "qh"], [4, 0, 2, 1, 3])
         g.add_layer("Permute", p + "k_pm", [p + "k_4d"], [p + "kt"], [4, 0, 2, 3, 1])
         g.add_layer("Permute", p + "v_pm", [p + "v_4d"], [p + "vh"], [4, 0, 2, 1, 3])
@@ -190,7 +194,7 @@ def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=()):
         g.add_layer("Softmax", p + "sm", [p + "masked"], [p + "probs"], [3])
         g.add_layer("MatMul", p + "pv", [p + "probs", p + "vh"], [p + "ctx_h"], [-1])
         g.add_layer("Permute", p + "ctx_pm", [p + "ctx_h"], [p + "ctx_4d"], [4, 0, 2, 1, 3])
-        g.add_layer("Reshape", p + "ctx_rs", [p + "ctx_4d"], [p + "ctx"], [0, 3, 3, B, S, H, 0])
+        g.add_layer("Reshape", p + "ctx_rs", [p + "ctx_4d"], [p + "ctx"], merge_shape)
         _linear(g, p + "o", p + "ctx", p + "attn_o", lw["wo"], lw["bo"])
         g.add_layer("Add", p + "res1", [x, p + "attn_o"], [p + "sum1"], [1])
         g.add_constant(p + "ln1_gamma", lw["ln1_g"])
