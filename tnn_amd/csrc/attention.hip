@@ -47,14 +47,6 @@ template <> struct AttnT<TNN_ROCM_F16> {
         half_t l = (half_t)lo, h = (half_t)hi;
         return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
     }
-    // eight packed values times a scalar, rounded to nearest (fp32 product, one rounding)
-    static __device__ __forceinline__ u32x4 scale8(u32x4 v, float c) {
-        u32x4 o;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            o[i] = pack2(to_float((uint16_t)(v[i] & 0xffffu)) * c, to_float((uint16_t)(v[i] >> 16)) * c);
-        return o;
-    }
     // the same in two steps, for callers that shuffle the packed pairs before summing them
     static __device__ __forceinline__ uint32_t pack_only(float lo, float hi) {
         return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
@@ -84,13 +76,6 @@ template <> struct AttnT<TNN_ROCM_BF16> {
     static __device__ __forceinline__ float to_float(uint16_t bits) { return __uint_as_float((uint32_t)bits << 16); }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
-    }
-    static __device__ __forceinline__ u32x4 scale8(u32x4 v, float c) {
-        u32x4 o;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            o[i] = pack2(to_float((uint16_t)(v[i] & 0xffffu)) * c, to_float((uint16_t)(v[i] >> 16)) * c);
-        return o;
     }
     static __device__ __forceinline__ uint32_t pack_only(float lo, float hi) {
         return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
@@ -578,8 +563,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
         __syncthreads();
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
-            qf[kk] = AttnT<DT>::scale8(*reinterpret_cast<const u32x4 *>(stage + (wave * 32 + lq) * kRowBytes + kk * 32 + g * 16),
-                                       p.scale_log2e);  // scores come out of the MFMA in the exp2 domain
+            qf[kk] = *reinterpret_cast<const u32x4 *>(stage + (wave * 32 + lq) * kRowBytes + kk * 32 + g * 16);
         __syncthreads();
     }
     if (n_tiles > 1)
@@ -619,26 +603,24 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
         const unsigned char *const vtbuf = kbuf + kTile;
         const int kv0     = t * kTileKV;
         const bool biased = mb != nullptr || kv0 + kTileKV > kv_end;  // workgroup-uniform
-        // Q carries scale * log2(e) already, so the MFMA result is the score in the exp2 domain.
         // The tile body is written three times under one branch (with the branch inside the tile the compiler copies
-        // the 32 score registers where the paths meet):
-        //   BIAS : per-key bias (additive mask, keys past kv_end), exact running maximum
-        //   EXACT: no bias, exact running maximum (the first tile of a row block)
-        //   STALE: no bias; the accumulators start at -m (m = the running maximum so far), so the MFMA result is
-        //          already s - m and goes straight into exp2.  m only follows the true maximum when a score exceeds
-        //          it by more than kStaleMax (2^kStaleMax still fits the packed half-precision probabilities
-        //          comfortably); then the tile's scores, the O accumulators and the row sum are rescaled.  The
-        //          normalised result does not depend on which reference the exponentials use.
+        // the 32 score registers where the paths meet).  c = scale * log2(e), s = the raw dot product:
+        //   BIAS : x = s*c + bias (additive mask, -inf for keys past kv_end), exact running maximum m, p = exp2(x - m)
+        //   EXACT: the same without a bias (the first tile of a row block, or c <= 0)
+        //   STALE: no bias, c > 0, m finite.  p = exp2(s*c - m) in one fused multiply-add per score, and m only
+        //          follows the true maximum when a score exceeds it by more than kStaleMax (2^kStaleMax still fits the
+        //          packed half-precision probabilities comfortably); only then are the O accumulators and the row sum
+        //          rescaled.  The normalised result does not depend on which reference the exponentials use.
         constexpr float kStaleMax = 10.0f;
+        const float c = p.scale_log2e;
         auto tile = [&](auto mode_tag) __attribute__((always_inline)) {
             constexpr int MODE = decltype(mode_tag)::value;  // 0 BIAS, 1 EXACT, 2 STALE
             f32x16 sacc[2];
-            const float c_init = MODE == 2 ? -m_i : 0.f;
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
-                    sacc[kt][r] = c_init;
+                    sacc[kt][r] = 0.f;
 #pragma unroll
                 for (int kk = 0; kk < 4; ++kk) {
                     u32x4 kf = *reinterpret_cast<const u32x4 *>(kbuf + kt * 32 * 128 + frag_off[kk]);
@@ -660,30 +642,31 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const float be       = kv0 + key0 + e < kv_end ? bv[e] : -INFINITY;
-                            float s2             = sacc[kt][r4 * 4 + e] + be;
+                            float s2             = fmaf(sacc[kt][r4 * 4 + e], c, be);
                             sacc[kt][r4 * 4 + e] = s2;
                             mx                   = fmaxf(mx, s2);
                         }
                     }
                 }
             } else {
+                // the maximum of the raw products; for MODE 1 the sign of c decides which end of them it is
+                float mn = INFINITY;
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r)
+                    for (int r = 0; r < 16; ++r) {
                         mx = fmaxf(mx, sacc[kt][r]);
+                        if (MODE == 1)
+                            mn = fminf(mn, sacc[kt][r]);
+                    }
+                mx = MODE == 1 ? fmaxf(mx * c, mn * c) : mx * c;
             }
             mx = half_swap_max(mx);
             if (MODE == 2) {
-                if (__any(mx > kStaleMax)) {  // rare: some row's scores outgrew the reference
-                    const float delta = fmaxf(mx, 0.f);
+                if (__any(mx - m_i > kStaleMax)) {  // rare: some row's scores outgrew the reference
+                    const float delta = fmaxf(mx - m_i, 0.f);
                     m_i += delta;
                     alpha = __builtin_amdgcn_exp2f(-delta);
-#pragma unroll
-                    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r)
-                            sacc[kt][r] -= delta;
 #pragma unroll
                     for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -694,7 +677,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
                 for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
-                        sacc[kt][r] = __builtin_amdgcn_exp2f(sacc[kt][r]);
+                        sacc[kt][r] = __builtin_amdgcn_exp2f(fmaf(sacc[kt][r], c, -m_i));
             } else {
                 float m_new = fmaxf(m_i, mx);
                 float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -703,7 +686,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
                 for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
-                        sacc[kt][r] = __builtin_amdgcn_exp2f(sacc[kt][r] - m_use);
+                        sacc[kt][r] = __builtin_amdgcn_exp2f(MODE == 0 ? sacc[kt][r] - m_use : fmaf(sacc[kt][r], c, -m_use));
 #pragma unroll
                 for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -744,7 +727,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
         };
         if (biased)
             tile(std::integral_constant<int, 0>());
-        else if (__all(m_i > -INFINITY))  // per wave: the reference must be finite (true from the second tile on)
+        else if (c > 0.f && __all(m_i > -INFINITY))  // per wave: the reference must be finite (true from the second tile on)
             tile(std::integral_constant<int, 2>());
         else
             tile(std::integral_constant<int, 1>());
