@@ -614,8 +614,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
         constexpr float kStaleMax = 10.0f;
         const float c = p.scale_log2e;
         auto tile = [&](auto mode_tag) __attribute__((always_inline)) {
-            constexpr int MODE = decltype(mode_tag)::value & 3;  // 0 BIAS, 1 EXACT, 2 STALE
-            constexpr bool TAIL = (decltype(mode_tag)::value & 4) == 0;  // BIAS only: keys past kv_end possible
+            constexpr int MODE = decltype(mode_tag)::value;  // 0 BIAS, 1 EXACT, 2 STALE
             f32x16 sacc[2];
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
@@ -642,7 +641,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
                         }
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const float be       = !TAIL || kv0 + key0 + e < kv_end ? bv[e] : -INFINITY;
+                            const float be       = kv0 + key0 + e < kv_end ? bv[e] : -INFINITY;
                             float s2             = fmaf(sacc[kt][r4 * 4 + e], c, be);
                             sacc[kt][r4 * 4 + e] = s2;
                             mx                   = fmaxf(mx, s2);
@@ -726,9 +725,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
             rs  = half_swap_sum(rs);
             l_i = fmaf(l_i, alpha, rs);
         };
-        if (biased && kv0 + kTileKV <= kv_end)
-            tile(std::integral_constant<int, 4>());
-        else if (biased)
+        if (biased)
             tile(std::integral_constant<int, 0>());
         else if (c > 0.f && __all(m_i > -INFINITY))  // per wave: the reference must be finite (true from the second tile on)
             tile(std::integral_constant<int, 2>());
