@@ -21,7 +21,25 @@ HIPCC_FLAGS = [
     # packed fp32 instructions are kept off on this hardware pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-Wno-unknown-attributes",
+    # per-kernel register / scratch figures as remarks; build_kernels() lists the kernels that spill
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+
+
+def spilled_kernels(compiler_output):
+    """[(kernel symbol, spilled VGPRs)] from the kernel-resource-usage remarks of one compilation."""
+    out, name = [], None
+    for line in compiler_output.splitlines():
+        if "remark:" not in line:
+            continue
+        text = line.split("remark:", 1)[1].strip()
+        if text.startswith("Function Name:"):
+            name = text.split(":", 1)[1].split("[")[0].strip()
+        elif text.startswith("VGPRs Spill:") and name:
+            n = int(text.split(":", 1)[1].split("[")[0])
+            if n > 0:
+                out.append((name, n))
+    return out
 
 
 def build_kernels(verbose=True):
@@ -39,7 +57,17 @@ def build_kernels(verbose=True):
     failed = False
     for src, p in procs:
         out, _ = p.communicate()
-        out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)
+        for kernel, n in spilled_kernels(out):
+            print("note: %s: %s spills %d VGPRs" % (src, kernel, n), file=sys.stderr)
+        keep, skip = [], 0
+        for l in out.splitlines():  # drop the remarks (and the two source lines clang prints under each)
+            if "kernel-resource-usage" in l:
+                skip = 2
+            elif skip and (l.lstrip().startswith("|") or "|" in l[:12]):
+                skip -= 1
+            elif "packed-fp32-ops" not in l:
+                keep.append(l)
+        out = "\n".join(keep)
         if out.strip() and verbose:
             print(out)
         if p.returncode != 0:

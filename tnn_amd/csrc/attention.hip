@@ -120,7 +120,7 @@ __device__ __forceinline__ float half_swap_sum(float v) {
 // The second launch bound (at least two waves per SIMD) caps the kernel at 256 registers, which keeps the MFMA accumulators in ordinary VGPRs: the softmax
 // reads and rescales them with VALU instructions, and accumulators parked in AGPRs cost a move per access.
 template <int DT, int NW, bool VT>
-__global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_kernel(AttnParams p) {
+__global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 : 2) attention_kernel(AttnParams p) {
     constexpr int NT = NW * 64;
     constexpr int BQ = NW * 32;
     // per tile: 64 rows (keys, or d for V^T) x 8 sixteen-byte chunks

@@ -147,7 +147,7 @@ int tnn_rocm_graph_end_capture(void *stream, void **graph_exec) {
     TR_CHECK_HIP(hipStreamEndCapture((hipStream_t)stream, &graph));
     hipGraphExec_t exec = nullptr;
     hipError_t e        = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-    hipGraphDestroy(graph);
+    (void)hipGraphDestroy(graph);
     if (e != hipSuccess) {
         set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
         return (int)e;
