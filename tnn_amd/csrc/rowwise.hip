@@ -113,7 +113,16 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
     double d2    = wave_sum_f64(s2);
     double mean  = d1 / cols;
     double var   = d2 / cols - mean * mean;
-    double rstdd = 1.0 / sqrt(var + (double)eps);
+    double rstdd;
+    if (DT == TNN_ROCM_F32) {
+        rstdd = 1.0 / sqrt(var + (double)eps);  // the reference's expression, correctly rounded
+    } else {
+        // only the fp32 roundings of rstd and mean*rstd are used below: the hardware estimate (about 2^-26 relative)
+        // refined by one Newton step is within a few double ulps, far inside what those roundings can see
+        const double a = var + (double)eps;
+        double r       = __builtin_amdgcn_rsq(a);
+        rstdd          = r + r * (0.5 - 0.5 * a * r * r);
+    }
     float rstd   = (float)rstdd;
     float mrs    = (float)(mean * rstdd);
 
@@ -143,10 +152,17 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
                 for (int t = 0; t < VEC; ++t)
                     Elem<DT>::st(&e[t], o[t]);
                 reinterpret_cast<uint4 *>(py)[vi] = raw;
-                if (pq) {
+                if (pq) {  // the VEC (4 or 8) quantised values of this lane leave as one 4- or 8-byte store
+                    uint32_t w[2] = {0u, 0u};
 #pragma unroll
-                    for (int t = 0; t < VEC; ++t)
-                        pq[vi * VEC + t] = float2int8_ref(__fmul_rn(Elem<DT>::ld(&e[t]), q_inv));
+                    for (int t = 0; t < VEC; ++t) {
+                        const int8_t q = float2int8_ref(__fmul_rn(Elem<DT>::ld(&e[t]), q_inv));
+                        w[t >> 2] |= (uint32_t)(uint8_t)q << (8 * (t & 3));
+                    }
+                    if (VEC == 8)
+                        *reinterpret_cast<uint2 *>(pq + (size_t)vi * VEC) = make_uint2(w[0], w[1]);
+                    else
+                        *reinterpret_cast<uint32_t *>(pq + (size_t)vi * VEC) = w[0];
                 }
             } else {
                 T tmp;
@@ -218,7 +234,8 @@ int launch_layernorm(hipStream_t s, const void *x, const void *res, const float 
     typedef typename Elem<DT>::type T;
     constexpr int VEC = 16 / sizeof(T);
     dim3 grid((rows + kRowsPerBlk - 1) / kRowsPerBlk), block(kBlock);
-    bool al = ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)res) | ((uintptr_t)emb.type_table)) & 15u) == 0 && cols % VEC == 0;
+    bool al = ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)res) | ((uintptr_t)emb.type_table) | ((uintptr_t)out_q)) & 15u) == 0 &&
+              cols % VEC == 0;
     if (emb.ids && !(al && cols <= kWave * VEC * kMaxVecPerLn)) {
         set_error("embed_layernorm: hidden size %d needs 16-byte aligned rows of at most %d elements", cols,
                   kWave * VEC * kMaxVecPerLn);
