@@ -262,7 +262,8 @@ TNN_ROCM_API int tnn_rocm_embed_layernorm(void *stream, int dtype, const int32_t
                                           const void *pos_table, int period, const float *gamma, const float *beta,
                                           float eps, void *y, int rows, int cols, int32_t *error_flag);
 
-/* dtype conversion between F32, F16 and BF16 (round to nearest even) */
+/* dtype conversion between F32, F16 and BF16 (round to nearest even), and between I32 and those three
+ * (static_cast both ways: reference source/tnn/device/cpu/acc/cpu_cast_layer_acc.cc:41-53) */
 TNN_ROCM_API int tnn_rocm_cast(void *stream, int src_dtype, const void *src, int dst_dtype, void *dst, size_t count);
 
 /* ---- int8 boundary ops ----------------------------------------------------------------------

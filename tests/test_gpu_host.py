@@ -507,3 +507,39 @@ def test_instance_reshape_fp32_batch_only_with_static_head_split():
         say("  fp32 B=%d S=%d max rel err %.3g" % (B, S, err))
         assert err <= FP32_TOL
     inst.close()
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_encoder_int32_mask_input_builds_the_additive_mask_in_the_graph(precision):
+    """Inputs as the tokenizer hands them over (ids, segment ids and a 0/1 mask, all NC_INT32): the graph builds the
+    additive mask itself (Cast -> Unsqueeze -> Sub -> Mul, the layers an exported BERT carries).  The result is bit for
+    bit that of the same weights fed with the additive mask as a float input."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: int32 mask input, " + precision)
+    cfg = EncoderConfig(2, 256, 4, 512)
+    w = make_weights(cfg, seed=51, bias_std=0.05)
+    B, S = 3, 72
+    w["pos_emb"] = w["pos_emb"][:S]
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 9, S, seed=52)
+    outs = []
+    for int_mask in (False, True):
+        inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S, int_mask=int_mask), precision)
+        types = [t for t, _ in inst.layers()]
+        inst.set_input("input_ids", ids)
+        inst.set_input("token_type_ids", seg)
+        if int_mask:
+            assert all(t in types for t in ("Cast", "Unsqueeze", "Sub", "Mul")), types
+            inst.set_input("input_mask", (mask == 0).astype(np.int32))
+        else:
+            inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+        for _ in range(4):   # the fourth forward replays the recorded graph
+            inst.forward()
+        outs.append(inst.output("last_hidden"))
+        inst.close()
+    assert outs[0].shape == (B, S, cfg.hidden)
+    assert np.array_equal(outs[0], outs[1])
+    wr = r16w(w) if precision == "fp16" else w
+    ref = encoder_ref.encoder(wr, cfg, encoder_ref.embed(wr, ids, seg, cfg.eps), B, S, mask)
+    err = rel_err(outs[1].reshape(B * S, -1), ref)
+    say("  against the checker: max rel err %.3g" % err)
+    assert err <= (FP16_TOL if precision == "fp16" else FP32_TOL)

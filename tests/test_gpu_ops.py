@@ -246,6 +246,22 @@ def test_cast_roundtrip():
     assert torch.equal(bf.cpu(), torch.from_numpy(x).to(torch.bfloat16))
 
 
+def test_cast_int32():
+    # cpu_cast_layer_acc.cc:41-53: static_cast both ways
+    say("cast int32 <-> float types")
+    rng = np.random.default_rng(13)
+    i = rng.integers(-70000, 70000, 10007).astype(np.int32)
+    i[:4] = [0, 1, -1, 30521]
+    assert np.array_equal(host(ops().cast(dev(i), torch.float32)), i.astype(np.float32))
+    assert torch.equal(ops().cast(dev(i), torch.float16).cpu(), torch.from_numpy(i).to(torch.float16))
+    assert torch.equal(ops().cast(dev(i), torch.bfloat16).cpu(), torch.from_numpy(i).to(torch.bfloat16))
+    f = (rng.standard_normal(10007) * 1000).astype(np.float32)
+    f[:6] = [0.0, 0.99, -0.99, 1.5, -1.5, 2.0]
+    assert np.array_equal(ops().cast(dev(f), torch.int32).cpu().numpy(), f.astype(np.int32))   # truncation
+    h = torch.from_numpy(f).to(torch.float16)
+    assert np.array_equal(ops().cast(h.cuda(), torch.int32).cpu().numpy(), h.float().numpy().astype(np.int32))
+
+
 # ---- int8 boundary ops: bit-exact ---------------------------------------------------------------
 def _half_integer_grid(scale):
     """values whose scaled image sits on and next to every .5 boundary of the int8 range"""

@@ -337,6 +337,26 @@ __global__ void __launch_bounds__(256) gelu_i8_kernel(const int8_t *__restrict__
 
 }  // namespace
 
+namespace {
+// int32 <-> float types: static_cast both ways as the CPU path (cpu_cast_layer_acc.cc:41-53); a float outside the int
+// range saturates here (the C++ conversion is undefined there)
+template <int DDT>
+__global__ void __launch_bounds__(kBlock) cast_from_i32_kernel(const int32_t *__restrict__ x,
+                                                               typename Elem<DDT>::type *__restrict__ y, size_t n) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        Elem<DDT>::st(&y[i], (float)x[i]);
+}
+template <int SDT>
+__global__ void __launch_bounds__(kBlock) cast_to_i32_kernel(const typename Elem<SDT>::type *__restrict__ x,
+                                                             int32_t *__restrict__ y, size_t n) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        y[i] = (int32_t)Elem<SDT>::ld(&x[i]);
+}
+
+}  // namespace
+
 extern "C" {
 
 int tnn_rocm_gelu(void *stream, int dtype, const void *x, void *y, size_t count) {
@@ -498,6 +518,27 @@ int tnn_rocm_cast(void *stream, int sdt, const void *src, int ddt, void *dst, si
     TR_CAST(TNN_ROCM_F16, TNN_ROCM_F16)
     TR_CAST(TNN_ROCM_BF16, TNN_ROCM_BF16)
 #undef TR_CAST
+#define TR_CAST_I32(F)                                                                                                \
+    if (sdt == TNN_ROCM_I32 && ddt == F) {                                                                            \
+        hipLaunchKernelGGL((cast_from_i32_kernel<F>), dim3(grid_for(n)), dim3(kBlock), 0, s, (const int32_t *)src,    \
+                           (Elem<F>::type *)dst, n);                                                                  \
+        TR_CHECK_LAUNCH();                                                                                            \
+        return 0;                                                                                                     \
+    }                                                                                                                 \
+    if (sdt == F && ddt == TNN_ROCM_I32) {                                                                            \
+        hipLaunchKernelGGL((cast_to_i32_kernel<F>), dim3(grid_for(n)), dim3(kBlock), 0, s, (const Elem<F>::type *)src, \
+                           (int32_t *)dst, n);                                                                        \
+        TR_CHECK_LAUNCH();                                                                                            \
+        return 0;                                                                                                     \
+    }
+    TR_CAST_I32(TNN_ROCM_F32)
+    TR_CAST_I32(TNN_ROCM_F16)
+    TR_CAST_I32(TNN_ROCM_BF16)
+#undef TR_CAST_I32
+    if (sdt == TNN_ROCM_I32 && ddt == TNN_ROCM_I32) {
+        TR_CHECK_HIP(hipMemcpyAsync(dst, src, n * sizeof(int32_t), hipMemcpyDeviceToDevice, s));
+        return 0;
+    }
     set_error("cast: unsupported dtype pair %d -> %d", sdt, ddt);
     return TNN_ROCM_EDTYPE;
 }

@@ -97,6 +97,7 @@ LayerType GlobalConvertLayerType(std::string s) {
         {"Mul", LAYER_MUL},                   {"Div", LAYER_DIV},
         {"Reshape", LAYER_RESHAPE},           {"Permute", LAYER_PERMUTE},
         {"Cast", LAYER_CAST},                 {"Reformat", LAYER_REFORMAT},
+        {"Squeeze", LAYER_SQUEEZE},           {"Unsqueeze", LAYER_UNSQUEEZE},
         {"Gather", LAYER_GATHER},             {"MatMul", LAYER_MATMUL},
         {"LayerNorm", LAYER_LAYER_NORM},      {"GELU", LAYER_GELU},
         {"BlobScale", LAYER_BLOB_SCALE},      {"QuantizedAdd", LAYER_ADD},
@@ -238,6 +239,15 @@ Status ParseLayerParam(LayerType type, const std::vector<std::string> &cfg, size
             p->data_in_resource    = r.geti(0) != 0;
             p->indices_in_resource = r.geti(1) != 0;
             out                    = p;
+            break;
+        }
+        case LAYER_SQUEEZE:
+        case LAYER_UNSQUEEZE: {  // unsqueeze_layer_interpreter.cc:22-32: count, then the axes
+            auto p = std::make_shared<SqueezeLayerParam>();
+            int n  = r.geti(0);
+            for (int i = 0; i < n; ++i)
+                p->axes.push_back(r.geti(0));
+            out = p;
             break;
         }
         case LAYER_CAST: {
@@ -810,6 +820,41 @@ struct GatherLayer : BaseLayer {  // layer/gather_layer.cc
     }
 };
 
+struct UnsqueezeLayer : BaseLayer {  // layer/unsqueeze_layer.cc:35-59
+    using BaseLayer::BaseLayer;
+    Status InferOutputShape() override {
+        auto p = dynamic_cast<SqueezeLayerParam *>(param_);
+        CHECK_PARAM_NULL(p);
+        DimsVector out = input_blobs_[0]->GetBlobDesc().dims;
+        for (int axis : p->axes) {
+            axis = axis < 0 ? axis + (int)out.size() + 1 : axis;
+            if (axis < 0 || axis > (int)out.size())
+                return Status(TNNERR_PARAM_ERR, "UnsqueezeLayer has invalid input axes");
+            out.insert(out.begin() + axis, 1);
+        }
+        output_blobs_[0]->GetBlobDesc().dims = out;
+        return TNN_OK;
+    }
+};
+struct SqueezeLayer : BaseLayer {  // layer/squeeze_layer.cc:35-60 (axes ascending, removed from the back)
+    using BaseLayer::BaseLayer;
+    Status InferOutputShape() override {
+        auto p = dynamic_cast<SqueezeLayerParam *>(param_);
+        CHECK_PARAM_NULL(p);
+        DimsVector out = input_blobs_[0]->GetBlobDesc().dims;
+        if (out.empty())
+            return Status(TNNERR_PARAM_ERR, "SqueezeLayer has invalid input size");
+        for (auto it = p->axes.rbegin(); it != p->axes.rend(); ++it) {
+            int axis = *it < 0 ? *it + (int)out.size() : *it;
+            if (axis < 0 || axis >= (int)out.size() || out[axis] != 1)
+                return Status(TNNERR_PARAM_ERR, "SqueezeLayer has invalid input axes");
+            out.erase(out.begin() + axis);
+        }
+        output_blobs_[0]->GetBlobDesc().dims = out;
+        return TNN_OK;
+    }
+};
+
 struct CastLayer : BaseLayer {
     using BaseLayer::BaseLayer;
     Status InferOutputDataType() override {
@@ -891,6 +936,8 @@ BaseLayer *CreateLayer(LayerType type) {
         case LAYER_LAYER_NORM: return new LayerNormLayer(type);
         case LAYER_GATHER: return new GatherLayer(type);
         case LAYER_CAST: return new CastLayer(type);
+        case LAYER_SQUEEZE: return new SqueezeLayer(type);
+        case LAYER_UNSQUEEZE: return new UnsqueezeLayer(type);
         case LAYER_REFORMAT: return new ReformatLayer(type);
         case LAYER_ROCM_FUSED_LINEAR: return new FusedLinearLayer(type);
         case LAYER_ROCM_FUSED_EMBEDDING: return new FusedEmbeddingLayer(type);

@@ -348,6 +348,11 @@ public:
     }
 };
 REGISTER_ROCM_ACC(RocmReshapeLayerAcc, LAYER_RESHAPE);
+// Squeeze / Unsqueeze only rename dimensions (cpu_squeeze_layer_acc.cc, cpu_unsqueeze_layer_acc.cc: one copy)
+class RocmSqueezeLayerAcc : public RocmReshapeLayerAcc {};
+class RocmUnsqueezeLayerAcc : public RocmReshapeLayerAcc {};
+REGISTER_ROCM_ACC(RocmSqueezeLayerAcc, LAYER_SQUEEZE);
+REGISTER_ROCM_ACC(RocmUnsqueezeLayerAcc, LAYER_UNSQUEEZE);
 
 // ---- Reformat: float <-> int8 (x86_reformat_layer_acc.cc:50-80, x86_compute_int8.cc:1193-1318) -------------------
 class RocmReformatLayerAcc : public RocmLayerAcc {
@@ -439,6 +444,11 @@ public:
         }
         if (st == dt) {
             ROCM_CALL(tnn_rocm_memcpy_d2d(Ptr(outputs[0]), Ptr(inputs[0]), count * DataTypeUtils::GetBytesSize(st), Stream()));
+            return TNN_OK;
+        }
+        if ((st == DATA_TYPE_INT32 && IsFloatType(dt)) || (IsFloatType(st) && dt == DATA_TYPE_INT32)) {
+            // cpu_cast_layer_acc.cc:41-53; a float output follows the network precision like every float blob
+            ROCM_CALL(tnn_rocm_cast(Stream(), (int)st, Ptr(inputs[0]), (int)dt, Ptr(outputs[0]), count));
             return TNN_OK;
         }
         return Status(TNNERR_LAYER_ERR, "Cast between these data types is not implemented on DEVICE_ROCM");

@@ -304,6 +304,8 @@ enum LayerType {
     LAYER_GATHER        = 104,
     LAYER_MATMUL        = 105,
     LAYER_SUB           = 108,
+    LAYER_SQUEEZE       = 118,
+    LAYER_UNSQUEEZE     = 164,
     LAYER_REFORMAT      = 170,
     LAYER_DIV           = 175,
     LAYER_LAYER_NORM    = 326,
@@ -353,6 +355,9 @@ struct ReshapeLayerParam : public LayerParam {
     int axis         = 0;
     int num_axes     = 0;
     std::vector<int> shape;
+};
+struct SqueezeLayerParam : public LayerParam {  // interpreter/layer_param.h:570-580 (Unsqueeze uses the same fields)
+    std::vector<int> axes;
 };
 struct PermuteLayerParam : public LayerParam {
     std::vector<int> orders;

@@ -150,11 +150,14 @@ def _linear(g, name, x, out, w_nk, bias):
     g.res_eltwise(name + "_add", "Add", bias)
 
 
-def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=(), dynamic=False):
+def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=(), dynamic=False, int_mask=False):
     """The decomposed encoder graph.  Inputs: input_ids, token_type_ids [B,S] int32 (or `hidden` [B,S,H] fp32
     without embeddings) and `attention_bias` [B,1,1,S] fp32 additive mask.  Output: `last_hidden` [B,S,H].
     dynamic: the head split / merge Reshape layers copy batch and sequence length from their input (shape entries
-    0, as an export with dynamic axes has them) instead of naming B and S, so the graph can be reshaped."""
+    0, as an export with dynamic axes has them) instead of naming B and S, so the graph can be reshaped.
+    int_mask: the third input is `input_mask` [B,S] int32 (1 = token, 0 = padding), as the tokenizer hands it over
+    (examples/base/bert_tokenizer.cc:351-355), and the additive mask is built in the graph the way exported BERT
+    models do: Cast(float) -> Unsqueeze(1,2) -> Sub(1 - m) -> Mul(-10000)."""
     g = Graph()
     H, h, d = cfg.hidden, cfg.heads, cfg.head_dim
     split_shape = [0, 4, 4, 0, 0, h, d, 0] if dynamic else [0, 4, 4, B, S, h, d, 0]
@@ -164,7 +167,16 @@ def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=(), dy
         g.add_input("token_type_ids", [B, S], DT_INT32)
     else:
         g.add_input("hidden", [B, S, H], DT_FLOAT)
-    g.add_input("attention_bias", [B, 1, 1, S], DT_FLOAT)
+    if int_mask:
+        g.add_input("input_mask", [B, S], DT_INT32)
+        g.add_layer("Cast", "mask_cast", ["input_mask"], ["mask_f"], [DT_FLOAT])
+        g.add_layer("Unsqueeze", "mask_unsq", ["mask_f"], ["mask_4d"], [2, 1, 2])
+        g.add_layer("Sub", "mask_inv", ["mask_4d"], ["mask_pad"], [0])      # constant first: 1 - m
+        g.res_eltwise("mask_inv", "Sub", np.array([1.0], np.float32))
+        g.add_layer("Mul", "mask_scale", ["mask_pad"], ["attention_bias"], [1])
+        g.res_eltwise("mask_scale", "Mul", np.array([-10000.0], np.float32))
+    else:
+        g.add_input("attention_bias", [B, 1, 1, S], DT_FLOAT)
     if with_embeddings:
         g.add_layer("Gather", "emb_word", ["input_ids"], ["emb_word_o"], [0, 1, 0])
         g.res_gather("emb_word", weights["word_emb"])
