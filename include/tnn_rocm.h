@@ -262,6 +262,15 @@ TNN_ROCM_API int tnn_rocm_embed_layernorm(void *stream, int dtype, const int32_t
                                           const void *pos_table, int period, const float *gamma, const float *beta,
                                           float eps, void *y, int rows, int cols, int32_t *error_flag);
 
+/* The same with the positions looked up as well (a third Gather over a position-id input instead of the constant
+ * position rows): row r adds pos_table[pos_ids[r % n_pos_ids]] (n_pos_ids = rows, or S for ids of shape [1,S] that
+ * broadcast over the batch); pos_table has pos_rows rows, index rules as for the other two tables. */
+TNN_ROCM_API int tnn_rocm_embed_layernorm_pos(void *stream, int dtype, const int32_t *ids, const int32_t *type_ids,
+                                              const int32_t *pos_ids, int n_pos_ids, const void *word_table, int vocab,
+                                              const void *type_table, int n_types, const void *pos_table, int pos_rows,
+                                              const float *gamma, const float *beta, float eps, void *y, int rows,
+                                              int cols, int32_t *error_flag);
+
 /* dtype conversion between F32, F16 and BF16 (round to nearest even), and between I32 and those three
  * (static_cast both ways: reference source/tnn/device/cpu/acc/cpu_cast_layer_acc.cc:41-53) */
 TNN_ROCM_API int tnn_rocm_cast(void *stream, int src_dtype, const void *src, int dst_dtype, void *dst, size_t count);

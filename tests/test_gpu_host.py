@@ -543,3 +543,49 @@ def test_encoder_int32_mask_input_builds_the_additive_mask_in_the_graph(precisio
     err = rel_err(outs[1].reshape(B * S, -1), ref)
     say("  against the checker: max rel err %.3g" % err)
     assert err <= (FP16_TOL if precision == "fp16" else FP32_TOL)
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_encoder_position_ids_input_third_gather(precision):
+    """Exports that keep the position ids a model input look the positions up with a third Gather.  Same result as the
+    graph that adds the first S rows of the table; permuted position ids give the permuted table rows."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: position ids as an input (Gather x3), " + precision)
+    cfg = EncoderConfig(1, 256, 4, 512)
+    w = make_weights(cfg, seed=61, bias_std=0.05)
+    B, S = 2, 40
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 9, S, seed=62)
+    base = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, dict(w, pos_emb=w["pos_emb"][:S]), B, S), precision)
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S, position_ids=True), precision)
+    types = [t for t, _ in inst.layers()]
+    assert types.count("RocmFusedEmbedding") == 1 and "Gather" not in types, types   # the third Gather is folded too
+    pos = np.tile(np.arange(S, dtype=np.int32), (B, 1))
+    for i in (base, inst):
+        i.set_input("input_ids", ids)
+        i.set_input("token_type_ids", seg)
+        i.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+    inst.set_input("position_ids", pos)
+    base.forward()
+    inst.forward()
+    a, b = base.output("last_hidden"), inst.output("last_hidden")
+    assert np.array_equal(a, b)
+    # other positions: row s of sequence 1 takes table row S-1-s
+    pos2 = pos.copy()
+    pos2[1] = pos2[1][::-1]
+    inst.set_input("position_ids", pos2)
+    inst.forward()
+    c = inst.output("last_hidden")
+    wr = r16w(w) if precision == "fp16" else w
+    H = cfg.hidden
+    we = orc.gather(wr["word_emb"], ids.reshape(-1))[0].reshape(B, S, H)
+    pe = orc.gather(wr["pos_emb"], pos2.reshape(-1))[0].reshape(B, S, H)
+    te = orc.gather(wr["type_emb"], seg.reshape(-1))[0].reshape(B, S, H)
+    tok = orc.binary("add", orc.binary("add", we, pe), te)
+    x0 = orc.layernorm(tok.reshape(B * S, H), wr["emb_ln_g"], wr["emb_ln_b"], cfg.eps)
+    ref = encoder_ref.encoder(wr, cfg, x0, B, S, mask)
+    err = rel_err(c.reshape(B * S, -1), ref)
+    say("  permuted positions against the checker: max rel err %.3g" % err)
+    assert err <= (FP16_TOL if precision == "fp16" else FP32_TOL)
+    assert np.array_equal(c[0], a[0]) and not np.array_equal(c[1], a[1])
+    base.close()
+    inst.close()

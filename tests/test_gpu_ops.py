@@ -528,6 +528,29 @@ def test_embed_layernorm_matches_the_five_layer_chain():
                                         dev(w["pos_emb"][:S], tdt), dev(w["emb_ln_g"]), dev(w["emb_ln_b"]), 1e-12)
         assert int(flag.item()) == 0
         assert rel_err(host(y), ref) <= tol
+    # positions looked up through ids of their own (third Gather): the natural order reproduces the result above,
+    # other ids pick other rows; one row of ids [1,S] is shared by the batch; an id outside the table raises the flag
+    pos = np.tile(np.arange(S, dtype=np.int32), (B, 1))
+    y1, flag = ops().embed_layernorm(dev(ids), dev(seg), dev(w["word_emb"]), dev(w["type_emb"]), dev(w["pos_emb"]),
+                                     dev(w["emb_ln_g"]), dev(w["emb_ln_b"]), 1e-12, pos_ids=dev(pos))
+    assert int(flag.item()) == 0 and rel_err(host(y1), ref) <= 2e-6
+    y1b, _ = ops().embed_layernorm(dev(ids), dev(seg), dev(w["word_emb"]), dev(w["type_emb"]), dev(w["pos_emb"]),
+                                   dev(w["emb_ln_g"]), dev(w["emb_ln_b"]), 1e-12, pos_ids=dev(pos[:1]))
+    assert np.array_equal(host(y1b), host(y1))
+    pos2 = rng.integers(0, w["pos_emb"].shape[0], (B, S)).astype(np.int32)
+    pos2[0, 1] = -1
+    y2, flag = ops().embed_layernorm(dev(ids), dev(seg), dev(w["word_emb"]), dev(w["type_emb"]), dev(w["pos_emb"]),
+                                     dev(w["emb_ln_g"]), dev(w["emb_ln_b"]), 1e-12, pos_ids=dev(pos2))
+    H_ = w["word_emb"].shape[1]
+    tok = orc.binary("add", orc.binary("add", orc.gather(w["word_emb"], ids_ref.reshape(-1))[0],
+                                       orc.gather(w["pos_emb"], pos2.reshape(-1))[0]),
+                     orc.gather(w["type_emb"], seg.reshape(-1))[0])
+    ref2 = orc.layernorm(tok.reshape(B * S, H_), w["emb_ln_g"], w["emb_ln_b"], 1e-12)
+    assert int(flag.item()) == 0 and rel_err(host(y2), ref2) <= 2e-6
+    pos2[1, 2] = w["pos_emb"].shape[0]
+    _, flag = ops().embed_layernorm(dev(ids), dev(seg), dev(w["word_emb"]), dev(w["type_emb"]), dev(w["pos_emb"]),
+                                    dev(w["emb_ln_g"]), dev(w["emb_ln_b"]), 1e-12, pos_ids=dev(pos2))
+    assert int(flag.item()) == 1
     bad = ids.copy()
     bad[1, 3] = V
     _, flag = ops().embed_layernorm(dev(bad), dev(seg), dev(w["word_emb"]), dev(w["type_emb"]), dev(w["pos_emb"][:S]),

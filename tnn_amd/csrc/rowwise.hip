@@ -32,6 +32,9 @@ struct EmbedRows {
     const int32_t *type_ids = nullptr;
     const void *type_table  = nullptr;
     int vocab = 0, n_types = 0, period = 0;
+    // optional third lookup: row r takes position row pos_ids[r % n_pos_ids] of a table of pos_rows rows
+    const int32_t *pos_ids = nullptr;
+    int n_pos_ids = 0, pos_rows = 0;
     int32_t *error_flag = nullptr;
 };
 
@@ -56,16 +59,21 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
         // negative indices wrap, an index outside the table raises the flag and reads row 0
         // (cpu_gather_layer_acc.cc:27-86)
         int wi = emb.ids[row], ti = emb.type_ids[row];
+        int pi = emb.pos_ids ? emb.pos_ids[row % emb.n_pos_ids] : row % emb.period;
         wi += wi < 0 ? emb.vocab : 0;
         ti += ti < 0 ? emb.n_types : 0;
-        const bool bad = wi < 0 || wi >= emb.vocab || ti < 0 || ti >= emb.n_types;
+        bool bad = wi < 0 || wi >= emb.vocab || ti < 0 || ti >= emb.n_types;
+        if (emb.pos_ids) {
+            pi += pi < 0 ? emb.pos_rows : 0;
+            bad |= pi < 0 || pi >= emb.pos_rows;
+        }
         if (bad) {
             if (lane == 0 && emb.error_flag)
                 *emb.error_flag = 1;
-            wi = 0, ti = 0;
+            wi = 0, ti = 0, pi = 0;
         }
         px  = x + (size_t)wi * cols;
-        pr  = res + (size_t)(row % emb.period) * cols;
+        pr  = res + (size_t)pi * cols;
         pr2 = reinterpret_cast<const T *>(emb.type_table) + (size_t)ti * cols;
     }
     T *py        = y + (size_t)row * cols;
@@ -374,10 +382,33 @@ int tnn_rocm_layernorm(void *stream, int dtype, const void *x, const void *resid
     }
 }
 
+static int embed_layernorm_impl(void *stream, int dtype, const int32_t *ids, const int32_t *type_ids, const void *word_table,
+                                int vocab, const void *type_table, int n_types, const void *pos_table, int period,
+                                const int32_t *pos_ids, int n_pos_ids, int pos_rows, const float *gamma, const float *beta,
+                                float eps, void *y, int rows, int cols, int32_t *error_flag);
+
 int tnn_rocm_embed_layernorm(void *stream, int dtype, const int32_t *ids, const int32_t *type_ids, const void *word_table,
                              int vocab, const void *type_table, int n_types, const void *pos_table, int period,
                              const float *gamma, const float *beta, float eps, void *y, int rows, int cols,
                              int32_t *error_flag) {
+    return embed_layernorm_impl(stream, dtype, ids, type_ids, word_table, vocab, type_table, n_types, pos_table, period,
+                                nullptr, 0, 0, gamma, beta, eps, y, rows, cols, error_flag);
+}
+
+int tnn_rocm_embed_layernorm_pos(void *stream, int dtype, const int32_t *ids, const int32_t *type_ids,
+                                 const int32_t *pos_ids, int n_pos_ids, const void *word_table, int vocab,
+                                 const void *type_table, int n_types, const void *pos_table, int pos_rows,
+                                 const float *gamma, const float *beta, float eps, void *y, int rows, int cols,
+                                 int32_t *error_flag) {
+    TR_REQUIRE(pos_ids && n_pos_ids > 0 && pos_rows > 0, TNN_ROCM_EINVAL, "embed_layernorm_pos: position ids and table rows required");
+    return embed_layernorm_impl(stream, dtype, ids, type_ids, word_table, vocab, type_table, n_types, pos_table, 1, pos_ids,
+                                n_pos_ids, pos_rows, gamma, beta, eps, y, rows, cols, error_flag);
+}
+
+static int embed_layernorm_impl(void *stream, int dtype, const int32_t *ids, const int32_t *type_ids, const void *word_table,
+                                int vocab, const void *type_table, int n_types, const void *pos_table, int period,
+                                const int32_t *pos_ids, int n_pos_ids, int pos_rows, const float *gamma, const float *beta,
+                                float eps, void *y, int rows, int cols, int32_t *error_flag) {
     TR_REQUIRE(rows >= 0 && cols > 0 && vocab > 0 && n_types > 0 && period > 0, TNN_ROCM_ESHAPE,
                "embed_layernorm: sizes must be positive");
     if (rows == 0)
@@ -385,6 +416,9 @@ int tnn_rocm_embed_layernorm(void *stream, int dtype, const int32_t *ids, const 
     TR_REQUIRE(ids && type_ids && word_table && type_table && pos_table && gamma && beta && y, TNN_ROCM_EINVAL,
                "embed_layernorm: null pointer");
     EmbedRows emb;
+    emb.pos_ids   = pos_ids;
+    emb.n_pos_ids = n_pos_ids;
+    emb.pos_rows  = pos_rows;
     emb.ids        = ids;
     emb.type_ids   = type_ids;
     emb.type_table = type_table;

@@ -137,27 +137,45 @@ private:
             if (ai < 0 || !L[ai] || L[ai]->type != LAYER_ADD || L[ai]->inputs.size() != 2 || g.sole_consumer(ln->inputs[0]) != li ||
                 IsModelOutput(ln->inputs[0]) || ResOf<EltwiseLayerResource>(L[ai]->name))
                 continue;
+            // the inner Add is either Add(word gather, position constant) or Add(word gather, position gather)
             int pi = -1, ti = -1;
             for (int side = 0; side < 2 && pi < 0; ++side) {
                 int a = g.producer_of(L[ai]->inputs[side]), b = g.producer_of(L[ai]->inputs[1 - side]);
-                if (a >= 0 && L[a] && L[a]->type == LAYER_ADD && L[a]->inputs.size() == 1 && table_gather(b))
+                if (a >= 0 && L[a] && L[a]->type == LAYER_ADD && table_gather(b) &&
+                    (L[a]->inputs.size() == 1 ||
+                     (L[a]->inputs.size() == 2 && !ResOf<EltwiseLayerResource>(L[a]->name) &&
+                      table_gather(g.producer_of(L[a]->inputs[0])) && table_gather(g.producer_of(L[a]->inputs[1])))))
                     pi = a, ti = b;
             }
             if (pi < 0)
                 continue;
+            const bool pos_gather = L[pi]->inputs.size() == 2;
             auto pos = ResOf<EltwiseLayerResource>(L[pi]->name);
             int wi   = g.producer_of(L[pi]->inputs[0]);
+            int pgi  = pos_gather ? g.producer_of(L[pi]->inputs[1]) : -1;  // fp32 a+b == b+a: either may be "word"
             auto wr = table_gather(wi), tr = table_gather(ti);
-            if (!pos || !wr || !tr || pos->element_handle.GetDataType() != DATA_TYPE_FLOAT)
+            auto pgr = pos_gather ? table_gather(pgi) : nullptr;
+            if (pgr && wr && pgr->data.GetBufferDims()[0] > wr->data.GetBufferDims()[0]) {
+                std::swap(wi, pgi);  // the vocabulary is the larger table; its ids carry the [B,S] shape
+                std::swap(wr, pgr);
+            }
+            if (!wr || !tr || (pos_gather ? !pgr : (!pos || pos->element_handle.GetDataType() != DATA_TYPE_FLOAT)))
                 continue;
             const int H = wr->data.GetBufferDims()[1];
-            auto pd     = pos->element_handle.GetBufferDims();
-            if (tr->data.GetBufferDims()[1] != H || pd.size() < 2 || pd.back() != H ||
-                pos->element_handle.GetDataCount() != pd[pd.size() - 2] * H)
-                continue;  // the constant must be one [S,H] matrix (leading dimensions of extent 1)
+            if (tr->data.GetBufferDims()[1] != H)
+                continue;
+            if (pos_gather) {
+                if (pgr->data.GetBufferDims()[1] != H)
+                    continue;
+            } else {
+                auto pd = pos->element_handle.GetBufferDims();
+                if (pd.size() < 2 || pd.back() != H || pos->element_handle.GetDataCount() != pd[pd.size() - 2] * H)
+                    continue;  // the constant must be one [S,H] matrix (leading dimensions of extent 1)
+            }
             bool single = true;
-            for (int idx : {pi, ti, wi})
-                single &= g.sole_consumer(L[idx]->outputs[0]) >= 0 && !IsModelOutput(L[idx]->outputs[0]);
+            for (int idx : {pi, ti, wi, pgi})
+                if (idx >= 0)
+                    single &= g.sole_consumer(L[idx]->outputs[0]) >= 0 && !IsModelOutput(L[idx]->outputs[0]);
             if (!single)
                 continue;
             auto lp      = ParamOf<LayerNormLayerParam>(ln);
@@ -166,6 +184,8 @@ private:
             fl->type_str = "RocmFusedEmbedding";
             fl->name     = ln->name + "_fused_embedding";
             fl->inputs   = {L[wi]->inputs[0], L[ti]->inputs[0], ln->inputs[1], ln->inputs[2]};
+            if (pos_gather)
+                fl->inputs.push_back(L[pgi]->inputs[0]);  // fifth input: the position ids
             fl->outputs  = ln->outputs;
             auto fp      = std::make_shared<RocmFusedEmbeddingParam>();
             fp->type     = fl->type_str;
@@ -176,9 +196,11 @@ private:
             fr->name     = fl->name;
             fr->word     = wr->data;
             fr->type     = tr->data;
-            fr->pos      = pos->element_handle;
+            fr->pos      = pos_gather ? pgr->data : pos->element_handle;
             resource_->resource_map[fl->name] = fr;
             L[wi] = L[ti] = L[pi] = L[ai] = nullptr;
+            if (pos_gather)
+                L[pgi] = nullptr;
             // the fused layer goes where the LayerNorm was: every input (ids, constants) exists before that point
             L[li] = fl;
         }
@@ -1260,17 +1282,25 @@ public:
     Status Reshape(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
         auto res = dynamic_cast<RocmFusedEmbeddingResource *>(resource_);
         CHECK_PARAM_NULL(res);
-        if (inputs.size() != 4 || inputs[0]->GetBlobDesc().data_type != DATA_TYPE_INT32 ||
+        if ((inputs.size() != 4 && inputs.size() != 5) || inputs[0]->GetBlobDesc().data_type != DATA_TYPE_INT32 ||
             inputs[1]->GetBlobDesc().data_type != DATA_TYPE_INT32 ||
             inputs[0]->GetBlobDesc().dims != inputs[1]->GetBlobDesc().dims)
             return Status(TNNERR_PARAM_ERR, "fused embedding: two int32 index blobs of equal shape, gamma and beta expected");
+        n_pos_ids_ = 0;
+        if (inputs.size() == 5) {  // position ids: the ids' shape, or one row [1,S] / [S] shared by the batch
+            const int rows = DimsVectorUtils::Count(inputs[0]->GetBlobDesc().dims);
+            n_pos_ids_     = DimsVectorUtils::Count(inputs[4]->GetBlobDesc().dims);
+            if (inputs[4]->GetBlobDesc().data_type != DATA_TYPE_INT32 || n_pos_ids_ <= 0 || rows % n_pos_ids_ != 0 ||
+                (n_pos_ids_ != rows && n_pos_ids_ != inputs[0]->GetBlobDesc().dims.back()))
+                return Status(TNNERR_PARAM_ERR, "fused embedding: position ids must be int32 of the ids' shape or one row of it");
+        }
         auto wd = res->word.GetBufferDims(), td = res->type.GetBufferDims(), pd = res->pos.GetBufferDims();
         auto id = inputs[0]->GetBlobDesc().dims;
         H_        = wd[1];
         pos_rows_ = pd[pd.size() - 2];
         // row t of the ids gets position t mod S.  The constant was matched at the shape the instance was created
         // with; after a reshape to a shorter sequence its first S rows are the positions 0..S-1.
-        if (id.empty() || id.back() > pos_rows_ || id.back() <= 0)
+        if (id.empty() || id.back() <= 0 || (n_pos_ids_ == 0 && id.back() > pos_rows_))
             return Status(TNNERR_PARAM_ERR, "fused embedding: the position constant does not cover the sequence length");
         period_ = id.back();
         vocab_ = wd[0], types_ = td[0];
@@ -1289,6 +1319,14 @@ public:
             DimsVectorUtils::Count(gamma->GetBlobDesc().dims) != H_ || DimsVectorUtils::Count(beta->GetBlobDesc().dims) != H_)
             return Status(TNNERR_PARAM_ERR, "fused embedding: gamma/beta must be fp32 vectors of the hidden size");
         const int rows = DimsVectorUtils::Count(inputs[0]->GetBlobDesc().dims);
+        if (n_pos_ids_ > 0) {
+            ROCM_CALL(tnn_rocm_embed_layernorm_pos(Stream(), (int)outputs[0]->GetBlobDesc().data_type,
+                                                   (const int32_t *)Ptr(inputs[0]), (const int32_t *)Ptr(inputs[1]),
+                                                   (const int32_t *)Ptr(inputs[4]), n_pos_ids_, word_, vocab_, type_, types_,
+                                                   pos_, pos_rows_, (const float *)Ptr(gamma), (const float *)Ptr(beta),
+                                                   p->eps, Ptr(outputs[0]), rows, H_, context_->ErrorFlag()));
+            return TNN_OK;
+        }
         ROCM_CALL(tnn_rocm_embed_layernorm(Stream(), (int)outputs[0]->GetBlobDesc().data_type, (const int32_t *)Ptr(inputs[0]),
                                            (const int32_t *)Ptr(inputs[1]), word_, vocab_, type_, types_, pos_, period_,
                                            (const float *)Ptr(gamma), (const float *)Ptr(beta), p->eps, Ptr(outputs[0]), rows,
@@ -1301,7 +1339,7 @@ protected:
 
 private:
     void *word_ = nullptr, *type_ = nullptr, *pos_ = nullptr;
-    int H_ = 0, period_ = 0, pos_rows_ = 0, vocab_ = 0, types_ = 0;
+    int H_ = 0, period_ = 0, pos_rows_ = 0, vocab_ = 0, types_ = 0, n_pos_ids_ = 0;
 };
 REGISTER_ROCM_ACC(RocmFusedEmbeddingLayerAcc, LAYER_ROCM_FUSED_EMBEDDING);
 

@@ -207,12 +207,18 @@ def layernorm(x, gamma, beta, eps, residual=None, q_inv_scale=None):
     return (y, q) if q is not None else y
 
 
-def embed_layernorm(ids, type_ids, word_table, type_table, pos_table, gamma, beta, eps):
-    """ids/type_ids int32 [B,S] -> LayerNorm(word[ids] + pos[s] + type[type_ids]) as [B*S, H]"""
-    _chk(ids, type_ids, word_table, type_table, pos_table, gamma, beta)
+def embed_layernorm(ids, type_ids, word_table, type_table, pos_table, gamma, beta, eps, pos_ids=None):
+    """ids/type_ids int32 [B,S] -> LayerNorm(word[ids] + pos[s] + type[type_ids]) as [B*S, H]; with pos_ids (int32,
+    [B,S] or [1,S]) the position rows are pos[pos_ids] instead"""
+    _chk(ids, type_ids, word_table, type_table, pos_table, gamma, beta, pos_ids)
     rows, H = ids.numel(), word_table.shape[1]
     y = torch.empty(rows, H, dtype=word_table.dtype, device=word_table.device)
     flag = torch.zeros(1, dtype=torch.int32, device=word_table.device)
+    if pos_ids is not None:
+        capi.call("tnn_rocm_embed_layernorm_pos", _stream(), dt(word_table), _p(ids), _p(type_ids), _p(pos_ids),
+                  pos_ids.numel(), _p(word_table), word_table.shape[0], _p(type_table), type_table.shape[0], _p(pos_table),
+                  pos_table.shape[0], _p(gamma), _p(beta), float(eps), _p(y), rows, H, _p(flag))
+        return y, flag
     capi.call("tnn_rocm_embed_layernorm", _stream(), dt(word_table), _p(ids), _p(type_ids), _p(word_table),
               word_table.shape[0], _p(type_table), type_table.shape[0], _p(pos_table), pos_table.shape[0], _p(gamma),
               _p(beta), float(eps), _p(y), rows, H, _p(flag))

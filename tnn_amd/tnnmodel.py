@@ -150,14 +150,17 @@ def _linear(g, name, x, out, w_nk, bias):
     g.res_eltwise(name + "_add", "Add", bias)
 
 
-def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=(), dynamic=False, int_mask=False):
+def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=(), dynamic=False, int_mask=False,
+                  position_ids=False):
     """The decomposed encoder graph.  Inputs: input_ids, token_type_ids [B,S] int32 (or `hidden` [B,S,H] fp32
     without embeddings) and `attention_bias` [B,1,1,S] fp32 additive mask.  Output: `last_hidden` [B,S,H].
     dynamic: the head split / merge Reshape layers copy batch and sequence length from their input (shape entries
     0, as an export with dynamic axes has them) instead of naming B and S, so the graph can be reshaped.
     int_mask: the third input is `input_mask` [B,S] int32 (1 = token, 0 = padding), as the tokenizer hands it over
     (examples/base/bert_tokenizer.cc:351-355), and the additive mask is built in the graph the way exported BERT
-    models do: Cast(float) -> Unsqueeze(1,2) -> Sub(1 - m) -> Mul(-10000)."""
+    models do: Cast(float) -> Unsqueeze(1,2) -> Sub(1 - m) -> Mul(-10000).
+    position_ids: positions come in as a fourth int32 input `position_ids` [B,S] and are looked up with a third
+    Gather (exports that keep the position ids an input) instead of adding the first S rows of the table."""
     g = Graph()
     H, h, d = cfg.hidden, cfg.heads, cfg.head_dim
     split_shape = [0, 4, 4, 0, 0, h, d, 0] if dynamic else [0, 4, 4, B, S, h, d, 0]
@@ -182,8 +185,14 @@ def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=(), dy
         g.res_gather("emb_word", weights["word_emb"])
         g.add_layer("Gather", "emb_type", ["token_type_ids"], ["emb_type_o"], [0, 1, 0])
         g.res_gather("emb_type", weights["type_emb"])
-        g.add_layer("Add", "emb_pos", ["emb_word_o"], ["emb_pos_o"], [1])
-        g.res_eltwise("emb_pos", "Add", weights["pos_emb"][:S])
+        if position_ids:
+            g.add_input("position_ids", [B, S], DT_INT32)
+            g.add_layer("Gather", "emb_posg", ["position_ids"], ["emb_posg_o"], [0, 1, 0])
+            g.res_gather("emb_posg", weights["pos_emb"])
+            g.add_layer("Add", "emb_pos", ["emb_word_o", "emb_posg_o"], ["emb_pos_o"], [1])
+        else:
+            g.add_layer("Add", "emb_pos", ["emb_word_o"], ["emb_pos_o"], [1])
+            g.res_eltwise("emb_pos", "Add", weights["pos_emb"][:S])
         g.add_layer("Add", "emb_sum", ["emb_pos_o", "emb_type_o"], ["emb_sum_o"], [1])
         g.add_constant("emb_ln_gamma", weights["emb_ln_g"])
         g.add_constant("emb_ln_beta", weights["emb_ln_b"])
