@@ -233,6 +233,8 @@ TNN_ROCM_API int tnn_rocm_layernorm(void *stream, int dtype, const void *x, cons
 /* ---- element-wise ops -----------------------------------------------------------------------
  * erf GELU   cpu_gelu_layer_acc.cc:31-51 */
 TNN_ROCM_API int tnn_rocm_gelu(void *stream, int dtype, const void *x, void *y, size_t count);
+/* tanh (the pooler's activation)   cpu_tanh_layer_acc.cc:23-27 */
+TNN_ROCM_API int tnn_rocm_tanh(void *stream, int dtype, const void *x, void *y, size_t count);
 
 /* out = a op b with numpy-style broadcast (shapes right-aligned, rank <= 6)
  *       CPU_ELEWISE  source/tnn/device/cpu/acc/compute/compute_elewise.cc:37-65

@@ -589,3 +589,35 @@ def test_encoder_position_ids_input_third_gather(precision):
     assert np.array_equal(c[0], a[0]) and not np.array_equal(c[1], a[1])
     base.close()
     inst.close()
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_encoder_pooler_head(precision):
+    """The pooler after the encoder (Gather of the first token with a constant index, Squeeze, dense, Tanh) runs on the
+    device and gives tanh(W h[:, 0] + b) of the hidden states the same instance returns."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: pooler head, " + precision)
+    cfg = EncoderConfig(1, 256, 4, 512)
+    w = make_weights(cfg, seed=71, bias_std=0.05)
+    rng = np.random.default_rng(72)
+    w["pool_w"] = (rng.standard_normal((cfg.hidden, cfg.hidden)) * 0.05).astype(np.float32)
+    w["pool_b"] = (rng.standard_normal(cfg.hidden) * 0.05).astype(np.float32)
+    B, S = 3, 24
+    w["pos_emb"] = w["pos_emb"][:S]
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 5, S, seed=73)
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), precision)
+    types = [t for t, _ in inst.layers()]
+    assert "Tanh" in types and "Squeeze" in types and "Gather" in types, types
+    inst.set_input("input_ids", ids)
+    inst.set_input("token_type_ids", seg)
+    inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+    inst.forward()
+    hidden = inst.output("last_hidden")
+    pooled = inst.output("pooled")
+    inst.close()
+    assert pooled.shape == (B, cfg.hidden)
+    pw = w["pool_w"].astype(np.float16).astype(np.float32) if precision == "fp16" else w["pool_w"]
+    ref = np.tanh(orc.inner_product(np.ascontiguousarray(hidden[:, 0, :]), pw, w["pool_b"]))
+    err = rel_err(pooled, ref)
+    say("  pooled against tanh(W h0 + b): max rel err %.3g" % err)
+    assert err <= (FP16_TOL if precision == "fp16" else 1e-5)

@@ -78,6 +78,17 @@ def test_gelu_fp32(n):
     assert got[0] == 0 and got[1] == 0 and got[2] == np.inf and got[3] == 0 and got[4] == 40.0
 
 
+def test_tanh():
+    say("tanh")
+    x = np.concatenate([np.linspace(-12, 12, 4001), [0.0, 1e-8, -1e-8, 50.0, -50.0]]).astype(np.float32)
+    ref = np.tanh(x.astype(np.float64))
+    got = host(ops().tanh(dev(x)))
+    assert np.max(np.abs(got - ref)) <= 3e-7
+    got16 = host(ops().tanh(dev(x, torch.float16)))
+    ref16 = np.tanh(x.astype(np.float16).astype(np.float64))
+    assert np.max(np.abs(got16 - ref16)) <= 1e-3
+
+
 def test_gelu_fp16():
     say("gelu fp16")
     rng = np.random.default_rng(1)

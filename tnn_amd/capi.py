@@ -61,6 +61,7 @@ SIGNATURES = {
     "tnn_rocm_embed_layernorm_pos": [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _vp, _f, _vp, _i, _i,
                                      _vp],
     "tnn_rocm_gelu": [_vp, _i, _vp, _vp, _sz],
+    "tnn_rocm_tanh": [_vp, _i, _vp, _vp, _sz],
     "tnn_rocm_binary": [_vp, _i, _i, _vp, _ip, _i, _vp, _ip, _i, _vp, _ip, _i],
     "tnn_rocm_permute": [_vp, _i, _vp, _vp, _ip, _ip, _i],
     "tnn_rocm_gather": [_vp, _vp, _vp, _vp, _i, _i, _sz, _i, _vp],

@@ -57,6 +57,9 @@ __global__ void __launch_bounds__(kBlock) unary_scalar_kernel(const typename Ele
 struct GeluOp {
     __device__ __forceinline__ float operator()(float v) const { return gelu_erf(v); }
 };
+struct TanhOp {  // cpu_tanh_layer_acc.cc:23-27
+    __device__ __forceinline__ float operator()(float v) const { return tanhf(v); }
+};
 
 template <int DT, typename F>
 int launch_unary(hipStream_t s, const void *x, void *y, size_t n, F f) {
@@ -369,6 +372,19 @@ int tnn_rocm_gelu(void *stream, int dtype, const void *x, void *y, size_t count)
         case TNN_ROCM_F16: return launch_unary<TNN_ROCM_F16>(s, x, y, count, GeluOp());
         case TNN_ROCM_BF16: return launch_unary<TNN_ROCM_BF16>(s, x, y, count, GeluOp());
         default: set_error("gelu: unsupported dtype %d", dtype); return TNN_ROCM_EDTYPE;
+    }
+}
+
+int tnn_rocm_tanh(void *stream, int dtype, const void *x, void *y, size_t count) {
+    if (count == 0)
+        return 0;
+    TR_REQUIRE(x && y, TNN_ROCM_EINVAL, "tanh: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case TNN_ROCM_F32: return launch_unary<TNN_ROCM_F32>(s, x, y, count, TanhOp());
+        case TNN_ROCM_F16: return launch_unary<TNN_ROCM_F16>(s, x, y, count, TanhOp());
+        case TNN_ROCM_BF16: return launch_unary<TNN_ROCM_BF16>(s, x, y, count, TanhOp());
+        default: set_error("tanh: unsupported dtype %d", dtype); return TNN_ROCM_EDTYPE;
     }
 }
 

@@ -98,6 +98,7 @@ LayerType GlobalConvertLayerType(std::string s) {
         {"Reshape", LAYER_RESHAPE},           {"Permute", LAYER_PERMUTE},
         {"Cast", LAYER_CAST},                 {"Reformat", LAYER_REFORMAT},
         {"Squeeze", LAYER_SQUEEZE},           {"Unsqueeze", LAYER_UNSQUEEZE},
+        {"Tanh", LAYER_TANH},
         {"Gather", LAYER_GATHER},             {"MatMul", LAYER_MATMUL},
         {"LayerNorm", LAYER_LAYER_NORM},      {"GELU", LAYER_GELU},
         {"BlobScale", LAYER_BLOB_SCALE},      {"QuantizedAdd", LAYER_ADD},
@@ -946,6 +947,7 @@ BaseLayer *CreateLayer(LayerType type) {
         case LAYER_ROCM_FUSED_ATTENTION: return new MixedTypeLayer<BaseLayer>(type);
         case LAYER_SOFTMAX:
         case LAYER_GELU:
+        case LAYER_TANH:
         case LAYER_ROCM_GELU_INT8: return new BaseLayer(type);
         default: return nullptr;
     }

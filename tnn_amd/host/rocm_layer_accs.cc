@@ -318,6 +318,19 @@ public:
 };
 REGISTER_ROCM_ACC(RocmGeluLayerAcc, LAYER_GELU);
 
+class RocmTanhLayerAcc : public RocmLayerAcc {  // cpu_tanh_layer_acc.cc:23-31
+public:
+    Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
+        DataType dt = outputs[0]->GetBlobDesc().data_type;
+        if (!IsFloatType(dt))
+            return Status(TNNERR_LAYER_ERR, "RocmTanhLayerAcc dont support data type");
+        ROCM_CALL(tnn_rocm_tanh(Stream(), (int)dt, Ptr(inputs[0]), Ptr(outputs[0]),
+                                (size_t)DimsVectorUtils::Count(outputs[0]->GetBlobDesc().dims)));
+        return TNN_OK;
+    }
+};
+REGISTER_ROCM_ACC(RocmTanhLayerAcc, LAYER_TANH);
+
 // ---- Permute / Reshape (naive_compute.cc:943-956 ; reshape is a copy) ----------------------------------------
 class RocmPermuteLayerAcc : public RocmLayerAcc {
 public:

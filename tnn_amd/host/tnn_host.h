@@ -299,6 +299,7 @@ enum LayerType {
     LAYER_SOFTMAX       = 21,
     LAYER_PERMUTE       = 32,
     LAYER_ADD           = 38,
+    LAYER_TANH          = 39,
     LAYER_MUL           = 42,
     LAYER_CAST          = 103,
     LAYER_GATHER        = 104,

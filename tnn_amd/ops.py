@@ -232,6 +232,13 @@ def gelu(x):
     return y
 
 
+def tanh(x):
+    _chk(x)
+    y = torch.empty_like(x)
+    capi.call("tnn_rocm_tanh", _stream(), dt(x), _p(x), _p(y), x.numel())
+    return y
+
+
 def binary(op, a, b, out_shape=None):
     _chk(a, b)
     if out_shape is None:

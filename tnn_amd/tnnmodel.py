@@ -96,7 +96,7 @@ class Graph:
         self._res(name, type_str, raw_buffer(element))
 
     def res_gather(self, name, data, indices=None):
-        p = _i32(1) + raw_buffer(data)
+        p = (_i32(1) + raw_buffer(data)) if data is not None else _i32(0)
         p += (_i32(1) + raw_buffer(indices)) if indices is not None else _i32(0)
         self._res(name, "Gather", p)
 
@@ -232,6 +232,15 @@ def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=(), dy
         g.add_layer("LayerNorm", p + "ln2", [p + "sum2", p + "ln2_gamma", p + "ln2_beta"], [out], [1, repr(cfg.eps)])
         x = out
     g.add_output("last_hidden")
+    if "pool_w" in weights:
+        # pooler: the first token's hidden state -> dense -> tanh, the way an exported BERT spells it
+        # (Gather with a constant index on the sequence axis, Squeeze, MatMul + Add, Tanh)
+        g.add_layer("Gather", "pool_first", ["last_hidden"], ["pool_tok3"], [1, 0, 1])
+        g.res_gather("pool_first", None, np.array([0], np.int32))
+        g.add_layer("Squeeze", "pool_sq", ["pool_tok3"], ["pool_tok"], [1, 1])
+        _linear(g, "pool_fc", "pool_tok", "pool_fc_o", weights["pool_w"], weights["pool_b"])
+        g.add_layer("Tanh", "pool_act", ["pool_fc_o"], ["pooled"], [])
+        g.add_output("pooled")
     for e in extra_outputs:
         g.add_output(e)
     return g
