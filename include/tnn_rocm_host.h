@@ -32,6 +32,15 @@ void *tnn_host_create_shaped(const char *proto, size_t proto_len, const char *mo
  * source/tnn/core/default_network.cc:456-500): new dims for the named inputs (same rank), every layer infers its
  * output shape again and its acc is reshaped; weights stay on the device.  An unknown name is TNNERR_PARAM_ERR. */
 int tnn_host_reshape(void *handle, int n_inputs, const char *const *names, const int *ndims, const int *dims);
+/* The first half of Instance::Init without a device: interpret the model (reference
+ * source/tnn/interpreter/tnn/model_interpreter.cc:104-476), run the optimizer passes on the instance's copy of the
+ * graph (source/tnn/core/default_network.cc:86-137 -> optimizer/net_optimizer_manager.cc) and infer every blob's type
+ * and shape (default_network.cc:157-331).  out receives one line per layer of the optimised graph:
+ * type|name|input blobs|output blobs|input dims|output dims.  Works on a machine without a GPU.
+ * Returns 0, an engine status code (text in err), or -2 when out is too small. */
+int tnn_host_plan(const char *proto, size_t proto_len, const char *model, size_t model_len, int precision, int n_inputs,
+                  const char *const *names, const int *ndims, const int *dims, char *out, size_t out_len, char *err,
+                  size_t err_len);
 /* ~Instance (instance.h:46) */
 void tnn_host_destroy(void *handle);
 const char *tnn_host_last_error(void *handle);

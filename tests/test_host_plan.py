@@ -1,0 +1,164 @@
+"""Host logic without a GPU: model interpretation, the optimizer passes and shape / type inference of the C++ host
+(tnn_host_plan: everything Instance::Init does short of creating a device context), plus its error behaviour."""
+import collections
+
+import numpy as np
+import pytest
+
+from tnn_amd import host, quant, tnnmodel
+from tnn_amd.encoder import EncoderConfig, make_weights
+
+
+def _graph(layers=2, hidden=256, heads=4, ffn=512, B=2, S=32, seed=1, **kw):
+    cfg = EncoderConfig(layers, hidden, heads, ffn)
+    w = make_weights(cfg, seed=seed)
+    if not kw.get("position_ids"):
+        w["pos_emb"] = w["pos_emb"][:S]
+    return cfg, w, tnnmodel.encoder_graph(cfg, w, B, S, **kw)
+
+
+def _types(plan):
+    return collections.Counter(l["type"] for l in plan)
+
+
+def test_fp16_encoder_is_rewritten_into_fused_layers():
+    cfg, w, g = _graph()
+    plan = host.plan(g, precision="fp16")
+    # per layer: fused attention (QKV + core), out-projection, FFN1 (+GELU), FFN2; every residual Add folded;
+    # every LayerNorm except the one that produces the model output folded into the projection that reads it
+    assert _types(plan) == {"RocmFusedEmbedding": 1, "RocmFusedAttention": 2, "RocmFusedLinear": 6, "LayerNorm": 1}
+    by_out = {o: l for l in plan for o in l["outputs"]}
+    assert by_out["last_hidden"]["output_dims"] == [[2, 32, 256]]
+    att = [l for l in plan if l["type"] == "RocmFusedAttention"]
+    assert all(l["inputs"][1] == "attention_bias" for l in att)
+    assert all(d == [2, 32, 256] for l in att for d in l["output_dims"])
+    ffn1 = [l for l in plan if l["name"].endswith("ffn1_mm") or "ffn1" in l["name"]]
+    assert any(l["output_dims"][0] == [2, 32, 512] for l in ffn1)
+    # layer order stays topological: every input is a model input, a constant or an earlier output
+    seen = {"input_ids", "token_type_ids", "attention_bias"}
+    for l in plan:
+        for i in l["inputs"]:
+            assert i in seen or i.endswith(("gamma", "beta")), (l["name"], i)
+        seen.update(l["outputs"])
+
+
+def test_fp32_keeps_the_decomposed_attention_core():
+    _, _, g = _graph()
+    t = _types(host.plan(g, precision="fp32"))
+    assert "RocmFusedAttention" not in t and t["Softmax"] == 2 and t["MatMul"] == 4 and t["Permute"] == 8
+    assert t["RocmFusedLinear"] == 12 and t["LayerNorm"] == 4 and t["RocmFusedEmbedding"] == 1
+
+
+def test_bf16_plans_like_fp16():
+    _, _, g = _graph()
+    assert _types(host.plan(g, precision="bf16")) == _types(host.plan(g, precision="fp16"))
+
+
+def test_layernorm_fold_switch(monkeypatch):
+    _, _, g = _graph()
+    monkeypatch.setenv("TNN_ROCM_FOLD_LN", "0")
+    assert _types(host.plan(g, precision="fp16"))["LayerNorm"] == 4
+    monkeypatch.setenv("TNN_ROCM_FOLD_LN", "1")
+    assert _types(host.plan(g, precision="fp16"))["LayerNorm"] == 1
+
+
+def test_width_that_cannot_fold_keeps_its_layernorms():
+    # hidden 192 is no multiple of 128: the LayerNorms stay launches of their own, everything else still fuses
+    _, _, g = _graph(hidden=192, heads=3, ffn=384)
+    t = _types(host.plan(g, precision="fp16"))
+    assert t["LayerNorm"] == 4 and t["RocmFusedAttention"] == 2 and t["RocmFusedLinear"] == 6
+
+
+def test_dynamic_head_split_planned_at_other_shapes():
+    _, _, g = _graph(B=4, S=32, dynamic=True)
+    shapes = {"input_ids": [3, 24], "token_type_ids": [3, 24], "attention_bias": [3, 1, 1, 24]}
+    plan = host.plan(g, precision="fp16", input_shapes=shapes)
+    assert _types(plan)["RocmFusedAttention"] == 2 and _types(plan)["LayerNorm"] == 1
+    assert [l for l in plan if "last_hidden" in l["outputs"]][0]["output_dims"] == [[3, 24, 256]]
+    # the static graph names B and S in its Reshape layers: other input shapes fail in the layer that notices (fp32 keeps
+    # those layers)
+    _, _, gs = _graph(B=4, S=32)
+    with pytest.raises(host.HostError, match="reshape"):
+        host.plan(gs, precision="fp32", input_shapes=shapes)
+    with pytest.raises(host.HostError, match="not an input"):
+        host.plan(g, input_shapes={"nope": [1]})
+    with pytest.raises(host.HostError, match="number of dimensions"):
+        host.plan(g, input_shapes={"input_ids": [3]})
+
+
+def test_mask_front_end_position_gather_and_pooler_layers():
+    cfg, w, _ = _graph()
+    rng = np.random.default_rng(3)
+    w["pool_w"] = rng.standard_normal((256, 256)).astype(np.float32)
+    w["pool_b"] = rng.standard_normal(256).astype(np.float32)
+    g = tnnmodel.encoder_graph(cfg, make_weights(cfg, seed=1) | {"pool_w": w["pool_w"], "pool_b": w["pool_b"]}, 2, 32,
+                               int_mask=True, position_ids=True)
+    plan = host.plan(g, precision="fp16")
+    t = _types(plan)
+    assert t["Cast"] == 1 and t["Unsqueeze"] == 1 and t["Sub"] == 1 and t["Mul"] == 1
+    assert t["RocmFusedEmbedding"] == 1 and t["Gather"] == 1 and t["Squeeze"] == 1 and t["Tanh"] == 1
+    emb = [l for l in plan if l["type"] == "RocmFusedEmbedding"][0]
+    assert emb["inputs"][-1] == "position_ids" and len(emb["inputs"]) == 5
+    by_out = {o: l for l in plan for o in l["outputs"]}
+    assert by_out["attention_bias"]["output_dims"] == [[2, 1, 1, 32]]
+    assert by_out["mask_4d"]["output_dims"] == [[2, 1, 1, 32]] and by_out["mask_f"]["output_dims"] == [[2, 32]]
+    assert by_out["pool_tok3"]["output_dims"] == [[2, 1, 256]] and by_out["pool_tok"]["output_dims"] == [[2, 256]]
+    assert by_out["pooled"]["output_dims"] == [[2, 256]]
+
+
+def test_config1_attention_layer_graph():
+    cfg = EncoderConfig(1, 768, 12, 3072)
+    lw = make_weights(cfg, seed=1, with_embeddings=False)["layers"][0]
+    g = tnnmodel.attention_layer_graph(lw, 128, 768, 12)
+    t = _types(host.plan(g, precision="fp32"))
+    assert t["RocmFusedLinear"] == 4 and "RocmFusedAttention" not in t      # InnerProduct x4, decomposed core
+    t16 = _types(host.plan(g, precision="fp16"))
+    assert t16 == {"RocmFusedAttention": 1, "RocmFusedLinear": 1}
+
+
+def test_error_behaviour_of_interpreter_and_layer_creation():
+    _, _, g = _graph(layers=1)
+    proto, model = g.proto(), g.model()
+    text = proto.decode() if isinstance(proto, bytes) else proto
+    # an unknown layer type is TNNERR_PARAM_ERR from layer creation (default_network.cc:246-250)
+    bad = text.replace("\"GELU ", "\"Gelu2 ", 1)
+    assert bad != text
+    with pytest.raises(host.HostError):
+        host.plan(bad, model, "fp32")
+    # a layer that reads a blob nobody produced
+    bad = text.replace("GELU l0_gelu 1 1 l0_ffn1_o", "GELU l0_gelu 1 1 l0_missing", 1)
+    assert bad != text
+    with pytest.raises(host.HostError):
+        host.plan(bad, model, "fp32")
+    # truncated model file
+    with pytest.raises(host.HostError):
+        host.plan(text, model[: len(model) // 2], "fp32")
+    # garbage proto
+    with pytest.raises(host.HostError):
+        host.plan("this is not a proto", model, "fp32")
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_int8_encoder_reformat_layers_are_folded(precision, monkeypatch):
+    """The quantised encoder of the X86 fixture: with the int8 pass off the explicit Reformat / QuantizedInnerProduct
+    chain stays; with it on every Reformat is folded into its neighbour (the counts the device tests also see)."""
+    import golden_util
+    cfg, w, B, S, scales, f = golden_util.int8_encoder()
+    g = quant.int8_encoder_graph(cfg, w, scales, B, S)
+    monkeypatch.setenv("TNN_ROCM_FUSE_INT8", "0")
+    t0 = _types(host.plan(g, precision=precision))
+    assert t0["Reformat"] == 10 and t0["QuantizedInnerProduct"] == 6
+    monkeypatch.setenv("TNN_ROCM_FUSE_INT8", "1")
+    plan = host.plan(g, precision=precision)
+    t1 = _types(plan)
+    assert t1["RocmQuantLinearGelu"] == 1 and t1["QuantizedInnerProduct"] == 0
+    if precision == "fp16":
+        assert t1["Reformat"] == 1 and t1["RocmFusedAttention"] == 1 and t1["RocmFusedLinearInt8"] == 2
+        att = [l for l in plan if l["type"] == "RocmFusedAttention"][0]
+        assert len(att["outputs"]) == 2          # the context and its int8 quantisation
+    else:
+        assert t1["Reformat"] == 2 and t1["RocmFusedLinearInt8"] == 5
+    for fold in ("TNN_ROCM_FOLD_GELU_LUT", "TNN_ROCM_FOLD_ATTN_Q8"):
+        monkeypatch.setenv(fold, "0")
+    t2 = _types(host.plan(g, precision=precision))
+    assert t2["RocmQuantLinearGelu"] == 0 and t2["RocmGeluInt8"] == 1

@@ -17,6 +17,8 @@ SIGNATURES = {
                                             C.POINTER(C.c_char_p), C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_char_p,
                                             C.c_size_t]),
     "tnn_host_reshape": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_char_p), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "tnn_host_plan": (C.c_int, [C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t, C.c_int, C.c_int, C.POINTER(C.c_char_p),
+                                C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t]),
     "tnn_host_destroy": (None, [C.c_void_p]),
     "tnn_host_last_error": (C.c_char_p, [C.c_void_p]),
     "tnn_host_set_input": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]),
@@ -60,6 +62,44 @@ def _shape_args(input_shapes):
     flat = [int(d) for _, v in items for d in v]
     dims = (C.c_int * max(len(flat), 1))(*flat)
     return len(items), names, ndims, dims
+
+
+def _parse_io(lines, with_type):
+    out = []
+    for line in lines:
+        if not line:
+            continue
+        f = line.split("|")
+        t = f.pop(0) if with_type else None
+        name, ins, outs, idims, odims = f
+
+        def dims(sv):
+            return [[int(x) for x in d.split(",") if x] for d in sv.split(";")] if sv else []
+
+        entry = {"name": name, "inputs": [x for x in ins.split(",") if x], "outputs": [x for x in outs.split(",") if x],
+                 "input_dims": dims(idims), "output_dims": dims(odims)}
+        if with_type:
+            entry["type"] = t
+        out.append(entry)
+    return out
+
+
+def plan(graph_or_proto, model=None, precision="fp16", input_shapes=None):
+    """The optimised graph (layer types, blobs, inferred shapes) of a model as an instance on DEVICE_ROCM would run it,
+    computed on the host alone: no GPU is needed.  Raises HostError with the engine's status text."""
+    lib = load()
+    proto = graph_or_proto if model is not None else graph_or_proto.proto()
+    model = model if model is not None else graph_or_proto.model()
+    if isinstance(proto, str):
+        proto = proto.encode()
+    n, names, ndims, dims = _shape_args(input_shapes or {})
+    out = C.create_string_buffer(1 << 22)
+    err = C.create_string_buffer(1024)
+    rc = lib.tnn_host_plan(proto, len(proto), model, len(model), {"fp32": 0, "fp16": 1, "bf16": 2}[precision], n, names,
+                           ndims, dims, out, len(out), err, 1024)
+    if rc != 0:
+        raise HostError("plan failed (0x%x): %s" % (rc & 0xFFFFFFFF, err.value.decode()))
+    return _parse_io(out.value.decode().splitlines(), True)
 
 
 class RocmInstance:

@@ -4,6 +4,7 @@
 // (test/test.cc:101-152: ConvertFromMat -> Forward -> ConvertToMat).
 #include <cstdio>
 #include <cstring>
+#include <sstream>
 #include <string>
 
 #include "tnn_host.h"
@@ -75,6 +76,41 @@ HOST_API void *tnn_host_create_shaped(const char *proto, size_t proto_len, const
         return nullptr;
     }
     return h;
+}
+
+// Interprets the model, runs the optimizer passes and infers every blob's type and shape, without a device context
+// (works on a machine without a GPU).  Writes the optimised graph as tnn_host_layer_io does, each line prefixed with the
+// layer's type and a '|'.  Returns 0, a status code (text in err), or -2 when out is too small.
+HOST_API int tnn_host_plan(const char *proto, size_t proto_len, const char *model, size_t model_len, int precision,
+                           int n_inputs, const char *const *names, const int *ndims, const int *dims, char *out,
+                           size_t out_len, char *err, size_t err_len) {
+    NetworkConfig nc;
+    nc.device_type = DEVICE_ROCM;
+    nc.precision   = precision == 0 ? PRECISION_HIGH : (precision == 2 ? PRECISION_LOW : PRECISION_AUTO);
+    ModelConfig mc;
+    mc.params.push_back(std::string(proto, proto_len));
+    mc.params.push_back(std::string(model, model_len));
+    InputShapesMap shapes;
+    for (int i = 0, k = 0; i < n_inputs; k += ndims[i], ++i)
+        shapes[names[i]] = DimsVector(dims + k, dims + k + ndims[i]);
+    ModelInterpreter interp;
+    Status st = interp.Interpret(mc.params);
+    DefaultNetwork net;
+    if (st == TNN_OK)
+        st = net.Plan(nc, &interp, shapes);
+    if (st != TNN_OK) {
+        if (err && err_len)
+            snprintf(err, err_len, "%s", st.description().c_str());
+        return (int)st == 0 ? -1 : (int)st;
+    }
+    std::istringstream types(net.LayerSummary()), io(net.LayerIo());
+    std::string text, t, l;
+    while (std::getline(types, t) && std::getline(io, l))
+        text += t.substr(0, t.find(' ')) + "|" + l + "\n";
+    if (text.size() + 1 > out_len)
+        return -2;
+    memcpy(out, text.c_str(), text.size() + 1);
+    return 0;
 }
 
 // Instance::Reshape (instance.cc:143-152): new dims for the named inputs; the other inputs keep theirs.

@@ -524,6 +524,11 @@ Status BaseLayer::Init(Context *context, LayerParam *param, LayerResource *resou
     layer_acc_ = device->CreateLayerAcc(type_);
     if (layer_acc_ == nullptr)  // base_layer.cc:83-86
         return Status(TNNERR_LAYER_ERR, "layer acc is nil (type " + param_->type + ")");
+    if (context == nullptr) {  // planning only (no device context): the acc exists, nothing is uploaded
+        delete layer_acc_;
+        layer_acc_ = nullptr;
+        return TNN_OK;
+    }
     layer_acc_->SetConstantResource(consts);
     for (auto b : input_blobs_)
         RETURN_ON_NEQ(layer_acc_->ResolveBlobDataFormat(b, BLOB_INPUT), TNN_OK);
@@ -1066,6 +1071,28 @@ DefaultNetwork::~DefaultNetwork() {
         tnn_rocm_event_destroy(e.second);
     }
     delete context_;
+}
+
+Status DefaultNetwork::Plan(NetworkConfig &net_config, ModelInterpreter *interpreter, const InputShapesMap &inputs_shape) {
+    config_ = net_config;
+    device_ = GetDevice(net_config.device_type);
+    if (!device_)
+        return Status(TNNERR_DEVICE_NOT_SUPPORT, "device not support");
+    structure_ = *interpreter->GetNetStructure();
+    structure_.layers.clear();
+    for (auto &l : interpreter->GetNetStructure()->layers)
+        structure_.layers.push_back(std::make_shared<LayerInfo>(*l));
+    resource_ = *interpreter->GetNetResource();
+    for (auto &kv : inputs_shape) {
+        auto it = structure_.inputs_shape_map.find(kv.first);
+        if (it == structure_.inputs_shape_map.end())
+            return Status(TNNERR_PARAM_ERR, "input shape given for " + kv.first + ", which is not an input of the model");
+        if (it->second.size() != kv.second.size())
+            return Status(TNNERR_PARAM_ERR, "input shape given for " + kv.first + " has another number of dimensions than the model's");
+        it->second = kv.second;
+    }
+    RETURN_ON_NEQ(RunNetOptimizers(&structure_, &resource_, config_), TNN_OK);
+    return InitLayers();  // context_ stays null: shapes and types only
 }
 
 Status DefaultNetwork::Init(NetworkConfig &net_config, ModelInterpreter *interpreter, const InputShapesMap &max_inputs_shape) {

@@ -677,6 +677,10 @@ public:
     // max_inputs_shape (may be empty: the model's own input shapes) is what the instance is created and its blob
     // memory planned at (instance.cc:48-128, default_network.cc:86-137)
     Status Init(NetworkConfig &net_config, ModelInterpreter *interpreter, const InputShapesMap &max_inputs_shape = InputShapesMap());
+    // Everything Init does short of touching a device: the instance's copy of the graph is optimised, layers are
+    // created (an unknown type or a type without an acc fails as in Init), blob types and shapes are inferred.  For
+    // LayerSummary() / LayerIo() on a machine without a GPU.
+    Status Plan(NetworkConfig &net_config, ModelInterpreter *interpreter, const InputShapesMap &inputs_shape = InputShapesMap());
     // default_network.cc:456-500: new dims for the named input blobs, then every layer infers its output shape again
     // and its acc is reshaped.  Weights stay on the device.  Blob memory is planned again only when a blob outgrows
     // its buffer; recorded launch sequences are kept per input-shape signature.
