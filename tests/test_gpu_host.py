@@ -621,3 +621,23 @@ def test_encoder_pooler_head(precision):
     err = rel_err(pooled, ref)
     say("  pooled against tanh(W h0 + b): max rel err %.3g" % err)
     assert err <= (FP16_TOL if precision == "fp16" else 1e-5)
+
+
+def test_plan_without_device_matches_the_instance():
+    """tnn_host_plan (no device context) and a live instance agree on the optimised graph: layer types, blob names and
+    every inferred shape."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: plan vs instance")
+    cfg = EncoderConfig(2, 256, 4, 512)
+    w = make_weights(cfg, seed=81)
+    w["pos_emb"] = w["pos_emb"][:40]
+    g = tnnmodel.encoder_graph(cfg, w, 2, 40, int_mask=True)
+    for precision in ("fp32", "fp16"):
+        plan = host.plan(g, precision=precision)
+        inst = host.RocmInstance.from_graph(g, precision)
+        live = inst.layer_io()
+        types = [t for t, _ in inst.layers()]
+        inst.close()
+        assert [l["type"] for l in plan] == types
+        for a, b in zip(plan, live):
+            assert {k: a[k] for k in b} == b
