@@ -544,6 +544,9 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
         }
     };
     constexpr int LPW = 2 * LD;
+    if (!mb)
+        for (int i = tid; i < 3 * kTileKV; i += NT)
+            (&lds_bias[0][0])[i] = 0.f;  // visible to everyone after the barriers of the Q staging below
     if (n_tiles > 0)
         issue(0, 0);
 
@@ -634,11 +637,10 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
 #pragma unroll
                     for (int r4 = 0; r4 < 4; ++r4) {
                         const int key0 = kt * 32 + r4 * 8 + g * 4;
-                        float bv[4]    = {0.f, 0.f, 0.f, 0.f};
-                        if (mb) {
-                            float4 raw = *reinterpret_cast<const float4 *>(&lds_bias[stage][key0]);
-                            bv[0] = raw.x * kLog2e, bv[1] = raw.y * kLog2e, bv[2] = raw.z * kLog2e, bv[3] = raw.w * kLog2e;
-                        }
+                        // without a mask the three bias rows hold zeros (written once below), so no branch is needed
+                        // and the eight reads of a tile go out together
+                        const float4 raw = *reinterpret_cast<const float4 *>(&lds_bias[stage][key0]);
+                        const float bv[4] = {raw.x * kLog2e, raw.y * kLog2e, raw.z * kLog2e, raw.w * kLog2e};
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const float be       = kv0 + key0 + e < kv_end ? bv[e] : -INFINITY;
