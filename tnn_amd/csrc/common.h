@@ -86,15 +86,15 @@ __device__ __forceinline__ float gelu_erf(float x) {
 // erf GELU for results that are rounded to fp16/bf16.  With q = erfc(|x|/sqrt2)/2 = Phi(-|x|):
 // gelu(x) = x - x*q for x >= 0 and x*q for x < 0 (no cancellation in the negative tail).  q comes from the rational
 // approximation 7.1.26 of Abramowitz & Stegun (|error| <= 1.5e-7 in erf), with the 1/2 folded into the
-// coefficients and 1/sqrt2 into the two constants: one reciprocal, one exp2 and eleven plain operations instead
+// coefficients and 1/sqrt2 into the two constants: one reciprocal, one exp2 and ten plain operations instead
 // of the ~40-instruction erff; the rounded fp16 result differs from the exact one by at most one ulp.
 // fp32 outputs keep gelu_erf.
 __device__ __forceinline__ float gelu_erf_fast(float x) {
     float t  = __builtin_amdgcn_rcpf(fmaf(0.231641888f, fabsf(x), 1.0f));
     float p  = fmaf(fmaf(fmaf(fmaf(0.5307027145f, t, -0.7265760135f), t, 0.7107068705f), t, -0.142248368f), t, 0.127414796f);
     float e  = __builtin_amdgcn_exp2f(x * x * -0.72134752f);
-    float xq = x * (p * t * e);
-    return x < 0.f ? xq : x - xq;
+    // p*t*e = Phi(-|x|), and x*Phi(x) = max(x, 0) - |x| * Phi(-|x|) for either sign
+    return fmaf(-fabsf(x), p * t * e, fmaxf(x, 0.f));
 }
 
 __device__ __forceinline__ float wave_sum(float v) {
