@@ -255,7 +255,7 @@ template <int DT> struct LnFloatEpilogue {
         float v[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t)
-            v[t] = st.x * (acc[t] - st.y * g[t]) + b[t];
+            v[t] = fmaf(st.x, fmaf(-st.y, g[t], acc[t]), b[t]);
         if (flags & TNN_ROCM_EPI_GELU) {
 #pragma unroll
             for (int t = 0; t < 8; ++t)
@@ -304,7 +304,7 @@ template <int DT> struct LnQkvSplitEpilogue {
         float v[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t)
-            v[t] = st.x * (acc[t] - st.y * g[t]) + b[t];
+            v[t] = fmaf(st.x, fmaf(-st.y, g[t], acc[t]), b[t]);
         if (n < 2 * H) {
             constexpr int NV = 8 * sizeof(T) / 16;
             u32x4 packed[NV];
