@@ -209,6 +209,59 @@ def test_graph_replay_matches_eager_on_every_replay(monkeypatch):
     graph.close()
 
 
+def test_two_instances_on_two_threads_match_their_sequential_results():
+    """One Context per Instance, instances used from different threads at the same time (the engine's threading
+    contract, source/tnn/core/instance.cc and default_network.cc:632-633: all work of an instance on its own stream,
+    Forward returns after its own Synchronize).  Each thread drives its own instance through eager forwards, the
+    recording forward and replays; every result must equal the one the same instance gave when it ran alone."""
+    import threading
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: two instances, two threads")
+    cfg = EncoderConfig.bert_base(2)
+    shapes = [(2, 128), (3, 96)]
+    insts, feeds, alone = [], [], []
+    for k, (B, S) in enumerate(shapes):
+        w = make_weights(cfg, seed=70 + k, bias_std=0.02)
+        insts.append(host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), "fp16"))
+        feeds.append([make_inputs(cfg, B, S, 17, S, seed=300 + 10 * k + it) for it in range(6)])
+
+    def run(k, out):
+        B, S = shapes[k]
+        for ids, seg, lens, mask in feeds[k]:
+            insts[k].set_input("input_ids", ids)
+            insts[k].set_input("token_type_ids", seg)
+            insts[k].set_input("attention_bias", mask.reshape(B, 1, 1, S))
+            insts[k].forward()
+            out.append(insts[k].output("last_hidden").copy())
+
+    for k in range(2):
+        ref = []
+        run(k, ref)
+        alone.append(ref)
+    together = [[], []]
+    errors = []
+
+    def guarded(k):
+        try:
+            run(k, together[k])
+        except Exception as e:  # surfaced below: an exception in a thread would otherwise pass silently
+            errors.append((k, repr(e)))
+
+    threads = [threading.Thread(target=guarded, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    assert all(not t.is_alive() for t in threads)
+    for k in range(2):
+        assert len(together[k]) == len(alone[k])
+        for it, (a, b) in enumerate(zip(alone[k], together[k])):
+            assert np.array_equal(a, b), "instance %d forward %d differs when another instance runs beside it" % (k, it)
+    for inst in insts:
+        inst.close()
+
+
 def test_int8_encoder_full_shape_properties(monkeypatch):
     """Benchmark config 4's per-layer shape (B16 S256, hidden 768, FFN 3072; 3 layers to keep the case short):
     calibrated on this backend's fp32 forward, then run quantised in fp16 mode.  Size-independent checks: every

@@ -18,7 +18,9 @@
 //
 // Output layout of a 32x32 block: lane l holds column (l % 32); accumulator register r holds row
 // 8*(r/4) + 4*(l/32) + (r%4).
+#include <atomic>
 #include <cstring>
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -1160,10 +1162,14 @@ int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int 
     }
     auto kern   = gemm_nk_tiled_kernel<DT, CFG, Epi>;
     if (lds > 64 * 1024) {
-        static bool attr_set = false;  // per instantiation
-        if (!attr_set) {
+        // the attribute belongs to the (kernel, device) pair: one bit per device, per instantiation
+        static std::atomic<unsigned long long> attr_set{0};
+        int dev = 0;
+        TR_CHECK_HIP(hipGetDevice(&dev));
+        const unsigned long long bit = 1ull << (dev & 63);
+        if (dev > 63 || !(attr_set.load(std::memory_order_acquire) & bit)) {
             TR_CHECK_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            attr_set = true;
+            attr_set.fetch_or(bit, std::memory_order_release);
         }
     }
     // tiles resident together on one XCD (32 CUs): a square-ish group keeps their panels in that L2
@@ -1244,8 +1250,11 @@ inline void parse_tune(const char *e) {
     }
 }
 inline int tune_override(int N, int K, int *group_m) {
-    if (g_tune_count < 0)
-        parse_tune(getenv("TNN_ROCM_GEMM_TUNE"));
+    static std::once_flag env_read;  // instances on several threads may launch their first GEMM together
+    std::call_once(env_read, [] {
+        if (g_tune_count < 0)
+            parse_tune(getenv("TNN_ROCM_GEMM_TUNE"));
+    });
     for (int i = 0; i < g_tune_count; ++i)
         if (g_tune_table[i].n == N && g_tune_table[i].k == K) {
             if (group_m)
