@@ -57,6 +57,12 @@ __global__ void __launch_bounds__(kBlock) unary_scalar_kernel(const typename Ele
 struct GeluOp {
     __device__ __forceinline__ float operator()(float v) const { return gelu_erf(v); }
 };
+// fp16 / bf16 blobs: the result is rounded to 11 / 8 bits, so the short rational form (at most one ulp of the
+// rounded result away, the same one the GEMM epilogue uses) keeps the launch on the memory side of the roofline:
+// with the ~40 instructions of erff it is bound by the vector ALU at about half the HBM rate.
+struct GeluHalfOp {
+    __device__ __forceinline__ float operator()(float v) const { return gelu_erf_fast(v); }
+};
 struct TanhOp {  // cpu_tanh_layer_acc.cc:23-27
     __device__ __forceinline__ float operator()(float v) const { return tanhf(v); }
 };
@@ -216,8 +222,61 @@ __global__ void __launch_bounds__(kBlock) permute_kernel(const T *__restrict__ i
     }
 }
 
+// Transposing permutes (the output's fastest axis is not the input's): 64 x 64 element tiles over the pair
+// (input-fastest axis F, the input axis A that becomes output-fastest) go through LDS, so both the reads (lanes along
+// F) and the writes (lanes along A) touch whole cache lines.  Every other axis is a batch axis; a workgroup finds its
+// tile and batch offsets from its index.
+struct TransDesc {
+    int n_batch_axes;
+    int batch_dim[4];
+    long batch_in_stride[4], batch_out_stride[4];
+    int len_f, len_a;          // extents of the two tiled axes
+    long in_stride_a;          // input stride of axis A (axis F has input stride 1)
+    long out_stride_f;         // output stride of axis F (axis A has output stride 1)
+    int tiles_f, tiles_a;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) permute_transpose_kernel(const T *__restrict__ in, T *__restrict__ out,
+                                                                   TransDesc d) {
+    constexpr int TILE = 64;
+    __shared__ T tile[TILE][TILE + (sizeof(T) >= 4 ? 1 : (sizeof(T) == 2 ? 2 : 4))];
+    size_t blk  = blockIdx.x;
+    const int tf = (int)(blk % (size_t)d.tiles_f);
+    blk /= (size_t)d.tiles_f;
+    const int ta = (int)(blk % (size_t)d.tiles_a);
+    blk /= (size_t)d.tiles_a;
+    long in_off = 0, out_off = 0;
+#pragma unroll
+    for (int k = 3; k >= 0; --k) {
+        if (k < d.n_batch_axes) {
+            const int idx = (int)(blk % (size_t)d.batch_dim[k]);
+            blk /= (size_t)d.batch_dim[k];
+            in_off += idx * d.batch_in_stride[k];
+            out_off += idx * d.batch_out_stride[k];
+        }
+    }
+    const int f0 = tf * TILE, a0 = ta * TILE;
+    const int col = threadIdx.x & (TILE - 1), row0 = threadIdx.x / TILE;  // 4 rows of 64 lanes per pass
+    const T *src = in + in_off;
+    T *dst       = out + out_off;
+#pragma unroll 4
+    for (int r = row0; r < TILE; r += kBlock / TILE) {
+        const int a = a0 + r, f = f0 + col;
+        if (a < d.len_a && f < d.len_f)
+            tile[r][col] = src[(long)a * d.in_stride_a + f];
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int r = row0; r < TILE; r += kBlock / TILE) {
+        const int f = f0 + r, a = a0 + col;
+        if (a < d.len_a && f < d.len_f)
+            dst[(long)f * d.out_stride_f + a] = tile[col][r];
+    }
+}
+
 // ---- gather --------------------------------------------------------------------------------------
-// one workgroup per output row; rows are copied in 4-byte words when the slice size allows it.
+// one workgroup per output row; rows are copied in 16-byte or 4-byte words when the slice size allows it.
 __global__ void __launch_bounds__(kBlock) gather_kernel(const char *__restrict__ data, const int32_t *__restrict__ idx,
                                                         char *__restrict__ out, int slices, size_t slice_bytes,
                                                         int n_indices, int32_t *error_flag) {
@@ -232,7 +291,11 @@ __global__ void __launch_bounds__(kBlock) gather_kernel(const char *__restrict__
     char *dst       = out + (size_t)row * slice_bytes;
     if (bad && threadIdx.x == 0 && error_flag)
         *error_flag = 1;
-    if ((slice_bytes & 3) == 0 && ((((uintptr_t)src) | ((uintptr_t)dst)) & 3) == 0) {
+    if ((slice_bytes & 15) == 0 && ((((uintptr_t)src) | ((uintptr_t)dst)) & 15) == 0) {
+        size_t vecs = slice_bytes >> 4;
+        for (size_t w = threadIdx.x; w < vecs; w += blockDim.x)
+            reinterpret_cast<uint4 *>(dst)[w] = bad ? make_uint4(0, 0, 0, 0) : reinterpret_cast<const uint4 *>(src)[w];
+    } else if ((slice_bytes & 3) == 0 && ((((uintptr_t)src) | ((uintptr_t)dst)) & 3) == 0) {
         size_t words = slice_bytes >> 2;
         for (size_t w = threadIdx.x; w < words; w += blockDim.x)
             reinterpret_cast<uint32_t *>(dst)[w] = bad ? 0u : reinterpret_cast<const uint32_t *>(src)[w];
@@ -290,6 +353,59 @@ __global__ void __launch_bounds__(kBlock) dequantize_kernel(const int8_t *__rest
     size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
         Elem<DT>::st(&x[i], __fmul_rn((float)q[i], scale));
+}
+
+// sixteen values per lane and access; value for value the scalar kernel's arithmetic
+template <int DT>
+__global__ void __launch_bounds__(kBlock) dequantize_vec_kernel(const int8_t *__restrict__ q, float scale,
+                                                                typename Elem<DT>::type *__restrict__ x, size_t n) {
+    typedef typename Elem<DT>::type T;
+    const size_t stride = (size_t)gridDim.x * blockDim.x, first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t nvec   = n / 16;
+    for (size_t i = first; i < nvec; i += stride) {
+        const u32x4 v = reinterpret_cast<const u32x4 *>(q)[i];
+        __attribute__((aligned(16))) T o[16];
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                Elem<DT>::st(&o[w * 4 + b], __fmul_rn((float)(int8_t)((v[w] >> (8 * b)) & 0xffu), scale));
+        uint4 *dst = reinterpret_cast<uint4 *>(x + i * 16);
+#pragma unroll
+        for (int k = 0; k < (int)sizeof(T); ++k)
+            dst[k] = reinterpret_cast<const uint4 *>(o)[k];
+    }
+    for (size_t t = nvec * 16 + first; t < n; t += stride)
+        Elem<DT>::st(&x[t], __fmul_rn((float)q[t], scale));
+}
+
+__global__ void __launch_bounds__(kBlock) add_i8_vec_kernel(const int8_t *__restrict__ a, float sa,
+                                                            const int8_t *__restrict__ b, float sb, float inv_so,
+                                                            int8_t *__restrict__ y, size_t n) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x, first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t nvec   = n / 16;
+    for (size_t i = first; i < nvec; i += stride) {
+        const u32x4 va = reinterpret_cast<const u32x4 *>(a)[i], vb = reinterpret_cast<const u32x4 *>(b)[i];
+        u32x4 o;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            uint32_t packed = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                float pa = __fmul_rn((float)(int8_t)((va[w] >> (8 * k)) & 0xffu), sa);
+                float pb = __fmul_rn((float)(int8_t)((vb[w] >> (8 * k)) & 0xffu), sb);
+                float sum = __fadd_rn(pa, pb);
+                packed |= ((uint32_t)(uint8_t)float2int8_ref(__fmul_rn(sum, inv_so))) << (8 * k);
+            }
+            o[w] = packed;
+        }
+        reinterpret_cast<u32x4 *>(y)[i] = o;
+    }
+    for (size_t t = nvec * 16 + first; t < n; t += stride) {
+        float pa = __fmul_rn((float)a[t], sa);
+        float pb = __fmul_rn((float)b[t], sb);
+        y[t]     = float2int8_ref(__fmul_rn(__fadd_rn(pa, pb), inv_so));
+    }
 }
 
 __global__ void __launch_bounds__(kBlock) add_i8_kernel(const int8_t *__restrict__ a, float sa,
@@ -369,8 +485,8 @@ int tnn_rocm_gelu(void *stream, int dtype, const void *x, void *y, size_t count)
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case TNN_ROCM_F32: return launch_unary<TNN_ROCM_F32>(s, x, y, count, GeluOp());
-        case TNN_ROCM_F16: return launch_unary<TNN_ROCM_F16>(s, x, y, count, GeluOp());
-        case TNN_ROCM_BF16: return launch_unary<TNN_ROCM_BF16>(s, x, y, count, GeluOp());
+        case TNN_ROCM_F16: return launch_unary<TNN_ROCM_F16>(s, x, y, count, GeluHalfOp());
+        case TNN_ROCM_BF16: return launch_unary<TNN_ROCM_BF16>(s, x, y, count, GeluHalfOp());
         default: set_error("gelu: unsupported dtype %d", dtype); return TNN_ROCM_EDTYPE;
     }
 }
@@ -454,44 +570,175 @@ int tnn_rocm_permute(void *stream, int elem_bytes, const void *in, void *out, co
                      int rank) {
     TR_REQUIRE(in && out && in_dims && order, TNN_ROCM_EINVAL, "permute: null pointer");
     TR_REQUIRE(rank >= 1 && rank <= 6, TNN_ROCM_ESHAPE, "permute: rank %d unsupported (1..6)", rank);
-    long in_stride[6];
     size_t n = 1;
     bool seen[6] = {false, false, false, false, false, false};
     for (int i = rank - 1; i >= 0; --i) {
         TR_REQUIRE(in_dims[i] >= 0, TNN_ROCM_ESHAPE, "permute: negative dim");
-        in_stride[i] = (long)n;
         n *= (size_t)in_dims[i];
-    }
-    PermDesc d;
-    d.rank = rank;
-    for (int j = 0; j < 6; ++j) {
-        d.out_dim[j]               = 1;
-        d.in_stride_of_out_axis[j] = 0;
     }
     for (int j = 0; j < rank; ++j) {
         TR_REQUIRE(order[j] >= 0 && order[j] < rank && !seen[order[j]], TNN_ROCM_EINVAL,
                    "permute: order is not a permutation");
-        seen[order[j]]             = true;
-        d.out_dim[j]               = in_dims[order[j]];
-        d.in_stride_of_out_axis[j] = in_stride[order[j]];
+        seen[order[j]] = true;
     }
     if (n == 0)
         return 0;
     hipStream_t s = (hipStream_t)stream;
-    switch (elem_bytes) {
-        case 1:
-            hipLaunchKernelGGL(permute_kernel<uint8_t>, dim3(grid_for(n)), dim3(kBlock), 0, s, (const uint8_t *)in,
-                               (uint8_t *)out, n, d);
-            break;
-        case 2:
-            hipLaunchKernelGGL(permute_kernel<uint16_t>, dim3(grid_for(n)), dim3(kBlock), 0, s, (const uint16_t *)in,
-                               (uint16_t *)out, n, d);
-            break;
-        case 4:
-            hipLaunchKernelGGL(permute_kernel<uint32_t>, dim3(grid_for(n)), dim3(kBlock), 0, s, (const uint32_t *)in,
-                               (uint32_t *)out, n, d);
-            break;
-        default: set_error("permute: element size %d unsupported", elem_bytes); return TNN_ROCM_EDTYPE;
+    // Normal form: axes of extent 1 dropped, input axes that stay neighbours in the output merged.  nd / nord
+    // describe the same copy with as few axes as possible (output position -> input axis).
+    int nd[6], nord[6], nrank = 0;
+    {
+        int keep_pos[6], kept = 0;  // output positions with extent > 1
+        for (int j = 0; j < rank; ++j)
+            if (in_dims[order[j]] != 1)
+                keep_pos[kept++] = j;
+        // runs of output positions whose input axes are consecutive (ignoring extent-1 axes in between)
+        int run_first_axis[6], run_len_elems[6], runs = 0;
+        for (int k = 0; k < kept; ++k) {
+            const int ax = order[keep_pos[k]];
+            bool joins = false;
+            if (runs > 0) {
+                const int prev = order[keep_pos[k - 1]];
+                joins = ax > prev;
+                for (int t = prev + 1; joins && t < ax; ++t)
+                    joins = in_dims[t] == 1;
+            }
+            if (joins && (long)run_len_elems[runs - 1] * in_dims[ax] < (1l << 31)) {
+                run_len_elems[runs - 1] *= in_dims[ax];
+            } else {
+                run_first_axis[runs] = ax;
+                run_len_elems[runs]  = in_dims[ax];
+                ++runs;
+            }
+        }
+        // input order of the runs = order of their first axes
+        int rank_of_run[6];
+        for (int a = 0; a < runs; ++a) {
+            int pos = 0;
+            for (int b = 0; b < runs; ++b)
+                pos += run_first_axis[b] < run_first_axis[a];
+            rank_of_run[a] = pos;
+        }
+        nrank = runs;
+        for (int a = 0; a < runs; ++a) {
+            nord[a]              = rank_of_run[a];
+            nd[rank_of_run[a]]   = run_len_elems[a];
+        }
+        if (nrank == 0) {  // a single element
+            nrank = 1, nd[0] = 1, nord[0] = 0;
+        }
+    }
+    long nin_stride[6], nout_stride_of_in_axis[6];
+    {
+        long acc = 1;
+        for (int i = nrank - 1; i >= 0; --i) {
+            nin_stride[i] = acc;
+            acc *= nd[i];
+        }
+        acc = 1;
+        for (int j = nrank - 1; j >= 0; --j) {
+            nout_stride_of_in_axis[nord[j]] = acc;
+            acc *= nd[nord[j]];
+        }
+    }
+    auto generic = [&](int unit_bytes, const int *dims_u) -> int {
+        // element-wise gather over units of unit_bytes (the innermost input axis re-expressed in those units)
+        PermDesc d;
+        d.rank = nrank;
+        for (int j = 0; j < 6; ++j) {
+            d.out_dim[j]               = 1;
+            d.in_stride_of_out_axis[j] = 0;
+        }
+        long stride_u[6], acc = 1;
+        size_t total = 1;
+        for (int i = nrank - 1; i >= 0; --i) {
+            stride_u[i] = acc;
+            acc *= dims_u[i];
+            total *= (size_t)dims_u[i];
+        }
+        for (int j = 0; j < nrank; ++j) {
+            d.out_dim[j]               = dims_u[nord[j]];
+            d.in_stride_of_out_axis[j] = stride_u[nord[j]];
+        }
+        switch (unit_bytes) {
+            case 1:
+                hipLaunchKernelGGL(permute_kernel<uint8_t>, dim3(grid_for(total)), dim3(kBlock), 0, s,
+                                   (const uint8_t *)in, (uint8_t *)out, total, d);
+                break;
+            case 2:
+                hipLaunchKernelGGL(permute_kernel<uint16_t>, dim3(grid_for(total)), dim3(kBlock), 0, s,
+                                   (const uint16_t *)in, (uint16_t *)out, total, d);
+                break;
+            case 4:
+                hipLaunchKernelGGL(permute_kernel<uint32_t>, dim3(grid_for(total)), dim3(kBlock), 0, s,
+                                   (const uint32_t *)in, (uint32_t *)out, total, d);
+                break;
+            case 16:
+                hipLaunchKernelGGL(permute_kernel<uint4>, dim3(grid_for(total)), dim3(kBlock), 0, s, (const uint4 *)in,
+                                   (uint4 *)out, total, d);
+                break;
+            default: set_error("permute: element size %d unsupported", unit_bytes); return TNN_ROCM_EDTYPE;
+        }
+        TR_CHECK_LAUNCH();
+        return 0;
+    };
+    TR_REQUIRE(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4, TNN_ROCM_EDTYPE,
+               "permute: element size %d unsupported", elem_bytes);
+    if (nord[nrank - 1] == nrank - 1) {
+        // the innermost run is copied as it is: move it in 16-byte (else 4-byte) units when it divides and is aligned
+        const long inner_bytes = (long)nd[nrank - 1] * elem_bytes;
+        int dims_u[6];
+        for (int i = 0; i < nrank; ++i)
+            dims_u[i] = nd[i];
+        if (inner_bytes % 16 == 0 && aligned16(in) && aligned16(out)) {
+            dims_u[nrank - 1] = (int)(inner_bytes / 16);
+            return generic(16, dims_u);
+        }
+        if (inner_bytes % 4 == 0 && (((uintptr_t)in | (uintptr_t)out) & 3) == 0) {
+            dims_u[nrank - 1] = (int)(inner_bytes / 4);
+            return generic(4, dims_u);
+        }
+        return generic(elem_bytes, nd);
+    }
+    // the output's fastest axis differs from the input's: tiled transpose over that pair of axes
+    {
+        TransDesc t;
+        const int F = nrank - 1, A = nord[nrank - 1];
+        t.n_batch_axes = 0;
+        size_t batch   = 1;
+        for (int i = 0; i < nrank; ++i)
+            if (i != F && i != A) {
+                t.batch_dim[t.n_batch_axes]        = nd[i];
+                t.batch_in_stride[t.n_batch_axes]  = nin_stride[i];
+                t.batch_out_stride[t.n_batch_axes] = nout_stride_of_in_axis[i];
+                ++t.n_batch_axes;
+                batch *= (size_t)nd[i];
+            }
+        for (int k = t.n_batch_axes; k < 4; ++k)
+            t.batch_dim[k] = 1, t.batch_in_stride[k] = 0, t.batch_out_stride[k] = 0;
+        t.len_f        = nd[F];
+        t.len_a        = nd[A];
+        t.in_stride_a  = nin_stride[A];
+        t.out_stride_f = nout_stride_of_in_axis[F];
+        t.tiles_f      = (t.len_f + 63) / 64;
+        t.tiles_a      = (t.len_a + 63) / 64;
+        const size_t blocks = (size_t)t.tiles_f * t.tiles_a * batch;
+        if (blocks >= (1ull << 31))
+            return generic(elem_bytes, nd);
+        switch (elem_bytes) {
+            case 1:
+                hipLaunchKernelGGL(permute_transpose_kernel<uint8_t>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                                   (const uint8_t *)in, (uint8_t *)out, t);
+                break;
+            case 2:
+                hipLaunchKernelGGL(permute_transpose_kernel<uint16_t>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                                   (const uint16_t *)in, (uint16_t *)out, t);
+                break;
+            default:
+                hipLaunchKernelGGL(permute_transpose_kernel<uint32_t>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                                   (const uint32_t *)in, (uint32_t *)out, t);
+                break;
+        }
     }
     TR_CHECK_LAUNCH();
     return 0;
@@ -590,6 +837,26 @@ int tnn_rocm_dequantize(void *stream, const int8_t *q, float scale, int ddt, voi
     TR_REQUIRE(x && q, TNN_ROCM_EINVAL, "dequantize: null pointer");
     hipStream_t s = (hipStream_t)stream;
     int g         = grid_for(n);
+    if (aligned16(q) && aligned16(x) && n >= 16) {
+        g = grid_for(n / 16);
+        switch (ddt) {
+            case TNN_ROCM_F32:
+                hipLaunchKernelGGL(dequantize_vec_kernel<TNN_ROCM_F32>, dim3(g), dim3(kBlock), 0, s, q, scale, (float *)x,
+                                   n);
+                break;
+            case TNN_ROCM_F16:
+                hipLaunchKernelGGL(dequantize_vec_kernel<TNN_ROCM_F16>, dim3(g), dim3(kBlock), 0, s, q, scale, (half_t *)x,
+                                   n);
+                break;
+            case TNN_ROCM_BF16:
+                hipLaunchKernelGGL(dequantize_vec_kernel<TNN_ROCM_BF16>, dim3(g), dim3(kBlock), 0, s, q, scale,
+                                   (bf16_bits *)x, n);
+                break;
+            default: set_error("dequantize: unsupported destination dtype %d", ddt); return TNN_ROCM_EDTYPE;
+        }
+        TR_CHECK_LAUNCH();
+        return 0;
+    }
     switch (ddt) {
         case TNN_ROCM_F32:
             hipLaunchKernelGGL(dequantize_kernel<TNN_ROCM_F32>, dim3(g), dim3(kBlock), 0, s, q, scale, (float *)x, n);
@@ -612,8 +879,12 @@ int tnn_rocm_add_i8(void *stream, const int8_t *a, float sa, const int8_t *b, fl
     if (n == 0)
         return 0;
     TR_REQUIRE(a && b && y, TNN_ROCM_EINVAL, "add_i8: null pointer");
-    hipLaunchKernelGGL(add_i8_kernel, dim3(grid_for(n)), dim3(kBlock), 0, (hipStream_t)stream, a, sa, b, sb, inv_so, y,
-                       n);
+    if (aligned16(a) && aligned16(b) && aligned16(y) && n >= 16)
+        hipLaunchKernelGGL(add_i8_vec_kernel, dim3(grid_for(n / 16)), dim3(kBlock), 0, (hipStream_t)stream, a, sa, b, sb,
+                           inv_so, y, n);
+    else
+        hipLaunchKernelGGL(add_i8_kernel, dim3(grid_for(n)), dim3(kBlock), 0, (hipStream_t)stream, a, sa, b, sb, inv_so,
+                           y, n);
     TR_CHECK_LAUNCH();
     return 0;
 }

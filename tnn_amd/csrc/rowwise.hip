@@ -1,8 +1,8 @@
 // Row-wise HBM-bound kernels: LayerNorm (+residual, +int8 quantised copy) and Softmax.
 //
-// One 64-lane wavefront owns one row: the row is read once with 16-byte accesses, kept in
-// registers, reduced with cross-lane shuffles (no LDS), and written once.  Four waves per
-// workgroup, so a launch over T rows issues T/4 workgroups (>> 256 CUs for encoder shapes).
+// One 64-lane wavefront owns one row (LayerNorm rows of at most 128 vectors: half a wavefront): the row is read
+// once with 16-byte accesses, kept in registers, reduced with cross-lane shuffles (no LDS), and written once.
+// Four waves per workgroup, so a launch over T rows issues T/4 or T/8 workgroups (>> 256 CUs for encoder shapes).
 #include "common.h"
 
 using namespace tnn_rocm;
@@ -16,6 +16,15 @@ constexpr int kMaxVecPerLn = 8;  // row cached in registers when cols <= 64 * VE
 __device__ __forceinline__ double wave_sum_f64(double v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// sum over each aligned group of LPR lanes (32: the two halves of a wave hold different rows)
+template <int LPR>
+__device__ __forceinline__ double lanes_sum_f64(double v) {
+#pragma unroll
+    for (int o = LPR / 2; o > 0; o >>= 1)
         v += __shfl_xor(v, o, 64);
     return v;
 }
@@ -38,7 +47,9 @@ struct EmbedRows {
     int32_t *error_flag = nullptr;
 };
 
-template <int DT, bool VECTOR>
+// LPR lanes own one row (64: a wave per row; 32: a wave holds two rows, which keeps every lane busy and twice the
+// bytes in flight for rows of at most 128 vectors); NV = 16-byte vectors a lane can hold.
+template <int DT, bool VECTOR, int LPR, int NV>
 __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<DT>::type *__restrict__ x,
                                                            const typename Elem<DT>::type *__restrict__ res,
                                                            const float *__restrict__ gamma,
@@ -48,10 +59,10 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
                                                            EmbedRows emb) {
     typedef typename Elem<DT>::type T;
     constexpr int VEC = VECTOR ? (int)(16 / sizeof(T)) : 1;
-    const int lane    = threadIdx.x & (kWave - 1);
-    const int row     = blockIdx.x * kRowsPerBlk + (threadIdx.x >> 6);
+    const int lane    = threadIdx.x & (LPR - 1);
+    const int row     = (blockIdx.x * kRowsPerBlk + (threadIdx.x >> 6)) * (kWave / LPR) + ((threadIdx.x & (kWave - 1)) / LPR);
     if (row >= rows)
-        return;  // whole wave exits together; no workgroup barrier is used below
+        return;  // the lanes of a row exit together; no workgroup barrier is used below and shuffles stay inside a row
     const T *px  = x + (size_t)row * cols;
     const T *pr  = res ? res + (size_t)row * cols : nullptr;
     const T *pr2 = nullptr;
@@ -80,11 +91,11 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
     int8_t *pq   = out_q ? out_q + (size_t)row * cols : nullptr;
     const int nv = cols / VEC;  // VECTOR launches guarantee cols % VEC == 0
 
-    float v[kMaxVecPerLn][VEC];
+    float v[NV][VEC];
     double s1 = 0.0, s2 = 0.0;
 #pragma unroll
-    for (int j = 0; j < kMaxVecPerLn; ++j) {
-        int vi = lane + j * kWave;
+    for (int j = 0; j < NV; ++j) {
+        int vi = lane + j * LPR;
         if (vi < nv) {
             if (VECTOR) {
                 uint4 raw = reinterpret_cast<const uint4 *>(px)[vi];
@@ -117,8 +128,8 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
             }
         }
     }
-    double d1    = wave_sum_f64(s1);
-    double d2    = wave_sum_f64(s2);
+    double d1    = lanes_sum_f64<LPR>(s1);
+    double d2    = lanes_sum_f64<LPR>(s2);
     double mean  = d1 / cols;
     double var   = d2 / cols - mean * mean;
     double rstdd;
@@ -135,8 +146,8 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
     float mrs    = (float)(mean * rstdd);
 
 #pragma unroll
-    for (int j = 0; j < kMaxVecPerLn; ++j) {
-        int vi = lane + j * kWave;
+    for (int j = 0; j < NV; ++j) {
+        int vi = lane + j * LPR;
         if (vi < nv) {
             float o[VEC];
 #pragma unroll
@@ -242,6 +253,7 @@ int launch_layernorm(hipStream_t s, const void *x, const void *res, const float 
     typedef typename Elem<DT>::type T;
     constexpr int VEC = 16 / sizeof(T);
     dim3 grid((rows + kRowsPerBlk - 1) / kRowsPerBlk), block(kBlock);
+    const int nv = cols / VEC;
     bool al = ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)res) | ((uintptr_t)emb.type_table) | ((uintptr_t)out_q)) & 15u) == 0 &&
               cols % VEC == 0;
     if (emb.ids && !(al && cols <= kWave * VEC * kMaxVecPerLn)) {
@@ -250,11 +262,22 @@ int launch_layernorm(hipStream_t s, const void *x, const void *res, const float 
         return TNN_ROCM_ESHAPE;
     }
     if (al && cols <= kWave * VEC * kMaxVecPerLn) {
-        hipLaunchKernelGGL((layernorm_kernel<DT, true>), grid, block, 0, s, (const T *)x, (const T *)res, gamma, beta,
-                           (T *)y, rows, cols, eps, out_q, q_inv, emb);
+#define TR_LN(LPR, NV)                                                                                                \
+    hipLaunchKernelGGL((layernorm_kernel<DT, true, LPR, NV>),                                                         \
+                       dim3((rows + kRowsPerBlk * (kWave / LPR) - 1) / (kRowsPerBlk * (kWave / LPR))), block, 0, s,   \
+                       (const T *)x, (const T *)res, gamma, beta, (T *)y, rows, cols, eps, out_q, q_inv, emb)
+        if (nv <= 64)
+            TR_LN(32, 2);
+        else if (nv <= 128)
+            TR_LN(32, 4);
+        else if (nv <= 256)
+            TR_LN(64, 4);
+        else
+            TR_LN(64, 8);
+#undef TR_LN
     } else if (cols <= kWave * kMaxVecPerLn) {
-        hipLaunchKernelGGL((layernorm_kernel<DT, false>), grid, block, 0, s, (const T *)x, (const T *)res, gamma, beta,
-                           (T *)y, rows, cols, eps, out_q, q_inv, emb);
+        hipLaunchKernelGGL((layernorm_kernel<DT, false, kWave, kMaxVecPerLn>), grid, block, 0, s, (const T *)x,
+                           (const T *)res, gamma, beta, (T *)y, rows, cols, eps, out_q, q_inv, emb);
     } else {
         hipLaunchKernelGGL((layernorm_long_kernel<DT>), grid, block, 0, s, (const T *)x, (const T *)res, gamma, beta,
                            (T *)y, rows, cols, eps, out_q, q_inv);
