@@ -26,10 +26,10 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 # rocprofv3 --pmc runs of this command (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
 # --counter-reference kernel (64 MiB in, 64 MiB out): FETCH_SIZE reads half the bytes, WRITE_SIZE all of them.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "gemm_qkv": int((2 * 14518.9 + 18613.1) * 1024),   # algorithmic: 4.5 + 3.4 in, 13.5 + 4.5 (LayerNorm output) out MiB
-    "gemm_out": int((2 * 10431.5 + 4608.0) * 1024),    # algorithmic: 4.5 + 1.1 + 4.5 in, 4.5 out MiB
-    "gemm_ffn1": int((2 * 17782.9 + 23040.0) * 1024),  # algorithmic: 4.5 + 4.5 in, 18 + 4.5 (LayerNorm output) out MiB
-    "gemm_ffn2": int((2 * 37088.5 + 4610.5) * 1024),   # algorithmic: 18 + 4.5 + 4.5 in, 4.5 out MiB
+    "gemm_qkv": int((2 * 14519.1 + 18596.2) * 1024),   # algorithmic: 4.5 + 3.4 in, 13.5 + 4.5 (LayerNorm output) out MiB
+    "gemm_out": int((2 * 10426.0 + 4608.0) * 1024),    # algorithmic: 4.5 + 1.1 + 4.5 in, 4.5 out MiB
+    "gemm_ffn1": int((2 * 17773.2 + 23040.0) * 1024),  # algorithmic: 4.5 + 4.5 in, 18 + 4.5 (LayerNorm output) out MiB
+    "gemm_ffn2": int((2 * 37095.2 + 4609.8) * 1024),   # algorithmic: 18 + 4.5 + 4.5 in, 4.5 out MiB
 }
 
 
