@@ -1275,13 +1275,23 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
         // 12-layer forward at M=3072 on MI355X (fp16, us, register-staged in parentheses): 192x192 three stages
         // N=3072 K=768 26.7 (28.7); 96x96 k-split three stages N=768 K=3072 25.9 (28.0); 64x64 two stages
         // N=768 K=768 11.4 (12.3); 128x128 two stages N=2304 K=768 19.1 (256x128 register-staged 20.5)
-        switch (pick_tile_config(M, N, kbytes)) {
+        int code = pick_tile_config(M, N, kbytes);
+        if (DT == TNN_ROCM_I8 && kbytes % 128 == 0) {
+            // int8 tiles finish their K loop in half the slabs, so the fixed cost per tile weighs more and small tiles
+            // that fill every CU win earlier than for fp16.  Inside the 12-layer int8 encoder at M=4096 (forward
+            // 1.258 ms): 64x64 for N=768 (192 tiles of 128x128, K=768 and K=3072) and for N=2304 (576 tiles of
+            // 128x128 for 512 slots, a second round for an eighth of the work) -> 1.216 ms.
+            const long t128 = (((long)M + 127) / 128) * (((long)N + 127) / 128), slots = 2 * kNumCU;
+            if (t128 < kNumCU || (code == 222221 && t128 > slots && t128 * 4 <= slots * 5))
+                code = 112211;
+        }
+        switch (code) {
             case 112211: cfg = 2112211; break;
             case 222221: cfg = 2222221; break;
             case 224211: cfg = 2222221; break;  // two 128x128 workgroups per CU beat one 256x128 (19.1 vs 20.3)
             case 332221: cfg = 3332221; break;
             case 331182: cfg = 3331182; break;
-            default: cfg = pick_tile_config(M, N, kbytes); break;
+            default: cfg = code; break;
         }
     }
     if (DT == TNN_ROCM_F32 && (cfg % 1000000 == 224211 || cfg % 1000000 == 332221 || cfg % 1000000 == 331182))
