@@ -83,18 +83,25 @@ __device__ __forceinline__ float gelu_erf(float x) {
     return __fmul_rn(__fmul_rn(0.5f, x), __fadd_rn(e, 1.0f));
 }
 
-// erf GELU for results that are rounded to fp16/bf16.  With q = erfc(|x|/sqrt2)/2 = Phi(-|x|):
-// gelu(x) = x - x*q for x >= 0 and x*q for x < 0 (no cancellation in the negative tail).  q comes from the rational
-// approximation 7.1.26 of Abramowitz & Stegun (|error| <= 1.5e-7 in erf), with the 1/2 folded into the
-// coefficients and 1/sqrt2 into the two constants: one reciprocal, one exp2 and ten plain operations instead
-// of the ~40-instruction erff; the rounded fp16 result differs from the exact one by at most one ulp.
-// fp32 outputs keep gelu_erf.
+// erf GELU for results that are rounded to fp16/bf16.  With a = |x| and Phi(-a) = erfc(a/sqrt2)/2:
+// gelu(x) = x*Phi(x) = max(x, 0) - a*Phi(-a) for either sign (no cancellation in the negative tail).
+// -log2(Phi(-a)) is smooth and nearly quadratic, so Phi(-a) = exp2(-q(a)) with a degree-6 polynomial q, q(0) = 1
+// (minimax fit of the relative error on [0, 9]: 2e-5, i.e. 3e-6 absolute in a*Phi(-a); beyond 9 the term is below
+// 1e-18 and a is clamped so the polynomial stays inside its fitted range).  Six fused multiply-adds, one clamp, one
+// exp2, one max and the final multiply-add: 13 issue slots against 19 for the rational form 7.1.26 of Abramowitz &
+// Stegun used before and ~40 for erff.  Against the correctly rounded fp16 result 0.4 % of the values differ, by one
+// ulp (2.8 % for the rational form).  fp32 outputs keep gelu_erf.
 __device__ __forceinline__ float gelu_erf_fast(float x) {
-    float t  = __builtin_amdgcn_rcpf(fmaf(0.231641888f, fabsf(x), 1.0f));
-    float p  = fmaf(fmaf(fmaf(fmaf(0.5307027145f, t, -0.7265760135f), t, 0.7107068705f), t, -0.142248368f), t, 0.127414796f);
-    float e  = __builtin_amdgcn_exp2f(x * x * -0.72134752f);
-    // p*t*e = Phi(-|x|), and x*Phi(x) = max(x, 0) - |x| * Phi(-|x|) for either sign
-    return fmaf(-fabsf(x), p * t * e, fmaxf(x, 0.f));
+    const float a = fminf(fabsf(x), 9.0f);
+    float q       = -2.8009472064e-05f;
+    q             = fmaf(q, a, 6.8930927528e-04f);
+    q             = fmaf(q, a, -7.6513012845e-03f);
+    q             = fmaf(q, a, 5.2408451099e-02f);
+    q             = fmaf(q, a, 4.5977897954e-01f);
+    q             = fmaf(q, a, 1.1508630942e+00f);
+    q             = fmaf(q, a, 1.0f);
+    const float e = __builtin_amdgcn_exp2f(-q);  // Phi(-a)
+    return fmaf(-fabsf(x), e, fmaxf(x, 0.f));
 }
 
 __device__ __forceinline__ float wave_sum(float v) {
