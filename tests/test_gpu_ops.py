@@ -312,6 +312,49 @@ def test_dequantize_and_add_i8_bit_exact():
     assert np.array_equal(got, orc.add_int8_x86(a, sa, q, sb, so))
 
 
+@pytest.mark.parametrize("n,offset", [(15, 0), (16, 0), (4099, 0), (4099, 1), (100000, 3)])
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_dequantize_and_add_i8_tails_and_unaligned_buffers(n, offset, dtype):
+    """sixteen values per lane when the buffers are 16-byte aligned, one per lane otherwise and for the tail: the
+    same values either way (offset = elements by which the int8 buffers start off a 16-byte boundary)"""
+    say("dequantize / add_i8 n=%d offset=%d %s" % (n, offset, dtype))
+    rng = np.random.default_rng(n + offset)
+    q = rng.integers(-128, 128, n, dtype=np.int8)
+    a = rng.integers(-128, 128, n, dtype=np.int8)
+    qd = dev(np.concatenate([np.zeros(offset, np.int8), q]))[offset:]
+    ad = dev(np.concatenate([np.zeros(offset, np.int8), a]))[offset:]
+    tdt = torch.float32 if dtype == "f32" else torch.float16
+    ref = orc.dequantize(q, np.float32(0.0371))
+    got = ops().dequantize(qd, 0.0371, tdt).cpu().numpy()
+    assert np.array_equal(got, ref if dtype == "f32" else ref.astype(np.float16))
+    sa, sb, so = np.float32(0.021), np.float32(0.047), np.float32(0.052)
+    inv = np.float32(1.0 / np.float64(so))
+    got = host(ops().add_i8(ad, float(sa), qd, float(sb), float(inv)))
+    assert np.array_equal(got, orc.add_int8_x86(a, sa, q, sb, so))
+
+
+@pytest.mark.parametrize("shape,order,offset", [
+    ((2, 130, 3, 70), (0, 2, 3, 1), 0),      # transpose, ragged 64 x 64 tiles, two batch axes
+    ((5, 64, 96), (0, 2, 1), 0),             # plain batched transpose
+    ((3, 4, 5, 6, 7, 8), (5, 0, 4, 1, 3, 2), 0),  # rank 6, three batch axes after merging
+    ((4, 100, 12, 64), (0, 2, 1, 3), 0),     # head split: rows of 64 values copied in 16-byte units
+    ((4, 100, 12, 64), (0, 2, 1, 3), 1),     # the same from a buffer that is not 16-byte aligned
+    ((7, 9, 6), (1, 0, 2), 0),               # innermost run of 6 values: 4-byte units at most
+    ((1, 33, 1, 65), (3, 1, 0, 2), 1),       # extent-1 axes dropped: a 2-D transpose, unaligned
+    ((2, 3, 4, 5), (0, 1, 2, 3), 0),         # identity: one merged axis
+    ((6, 1, 50), (2, 1, 0), 0)])
+def test_permute_normal_form_paths(shape, order, offset):
+    say("permute paths %s %s offset=%d" % (shape, order, offset))
+    rng = np.random.default_rng(sum(shape) + offset)
+    n = int(np.prod(shape))
+    for np_dt in (np.float32, np.float16, np.int8):
+        x = (rng.standard_normal(n) * 50).astype(np_dt)
+        buf = dev(np.concatenate([np.zeros(offset, np_dt), x]))
+        xd = buf[offset:].view(*shape)
+        got = ops().permute(xd, order).cpu().numpy()
+        assert np.array_equal(got, np.transpose(x.reshape(shape), order)), np_dt
+
+
 def test_gelu_i8_matches_three_layer_chain():
     say("gelu_i8")
     q = np.arange(-128, 128, dtype=np.int8)
