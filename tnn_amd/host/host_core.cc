@@ -1348,12 +1348,22 @@ Status DefaultNetwork::InitLayers() {
 
 // Blob memory with liveness-based reuse (the role of source/tnn/core/blob_manager.cc:156-227):
 // a blob's buffer returns to the pool after its last reader; inputs, outputs and constants are
-// never shared.  Reshape/Permute-style accs may alias, so every blob still gets its own pointer.
+// never shared.  The output of a layer that only renames dimensions (Reshape in the ONNX order, Squeeze, Unsqueeze)
+// shares its input's buffer, so the layer has nothing to copy; the buffer returns to the pool after the last reader
+// of any of its names.  TNN_ROCM_ALIAS_VIEWS=0 gives every blob its own buffer again.
 Status DefaultNetwork::AllocateBlobMemory() {
     std::map<std::string, int> last_use;
     for (int i = 0; i < (int)structure_.layers.size(); ++i)
         for (auto &n : structure_.layers[i]->inputs)
             last_use[n] = i;
+    const char *alias_env  = getenv("TNN_ROCM_ALIAS_VIEWS");
+    const bool alias_views = !(alias_env && alias_env[0] == '0');
+    std::map<std::string, std::string> alias_root;  // view output -> the blob that owns the buffer
+    std::map<std::string, int> group_last;          // owner -> last layer that reads the buffer under any name
+    auto root_of = [&](const std::string &n) -> std::string {
+        auto it = alias_root.find(n);
+        return it == alias_root.end() ? n : it->second;
+    };
     int64_t total_bytes = 0;
     std::multimap<int64_t, void *> pool;  // free buffers by capacity
     std::map<std::string, std::pair<int64_t, void *>> owned;
@@ -1387,6 +1397,28 @@ Status DefaultNetwork::AllocateBlobMemory() {
         RETURN_ON_NEQ(alloc_for(kv.second, false), TNN_OK);
     for (int i = 0; i < (int)structure_.layers.size(); ++i) {
         auto &info = structure_.layers[i];
+        bool is_view = alias_views && info->outputs.size() == 1 && !info->inputs.empty() &&
+                       (info->type == LAYER_RESHAPE || info->type == LAYER_SQUEEZE || info->type == LAYER_UNSQUEEZE);
+        if (is_view && info->type == LAYER_RESHAPE) {
+            auto rp = dynamic_cast<ReshapeLayerParam *>(info->param.get());
+            is_view = rp == nullptr || rp->reshape_type == 0;
+        }
+        if (is_view) {
+            const std::string &xn = info->inputs[0], &yn = info->outputs[0];
+            const std::string rn  = root_of(xn);
+            Blob *x = blobs_[xn], *y = blobs_[yn], *r = blobs_[rn];
+            if (!y->GetHandle().base && x->GetHandle().base && owned.count(rn) && !inputs_.count(rn) &&
+                !outputs_.count(yn) && !outputs_.count(rn) && !r->IsConstant() &&
+                x->GetBlobDesc().data_type == y->GetBlobDesc().data_type) {
+                y->SetHandle(x->GetHandle());
+                blob_capacity_[y] = blob_capacity_[r];
+                alias_root[yn]    = rn;
+                int last          = group_last.count(rn) ? group_last[rn] : (last_use.count(rn) ? last_use[rn] : i);
+                if (last_use.count(yn))
+                    last = std::max(last, last_use[yn]);
+                group_last[rn] = std::max(last, i);
+            }
+        }
         for (auto &n : info->outputs) {
             Blob *b = blobs_[n];
             if (b->GetHandle().base)
@@ -1394,11 +1426,13 @@ Status DefaultNetwork::AllocateBlobMemory() {
             bool pinned = outputs_.count(n) > 0;
             RETURN_ON_NEQ(alloc_for(b, !pinned), TNN_OK);
         }
-        // release buffers whose last reader is this layer (never inputs/outputs/constants)
+        // release buffers whose last reader (under any of their names) is this layer (never inputs/outputs/constants)
         for (auto &n : info->inputs) {
-            if (last_use[n] != i || inputs_.count(n) || outputs_.count(n) || blobs_[n]->IsConstant())
+            const std::string rn = root_of(n);
+            const int last       = group_last.count(rn) ? group_last[rn] : last_use[rn];
+            if (last != i || inputs_.count(rn) || outputs_.count(rn) || blobs_[rn]->IsConstant())
                 continue;
-            auto it = owned.find(n);
+            auto it = owned.find(rn);
             if (it != owned.end()) {
                 pool.insert({it->second.first, it->second.second});
                 owned.erase(it);
@@ -1406,7 +1440,7 @@ Status DefaultNetwork::AllocateBlobMemory() {
         }
         // an output nobody reads (a float tensor whose only reader was folded away) is free again right after its layer
         for (auto &n : info->outputs) {
-            if (last_use.count(n) || outputs_.count(n))
+            if (last_use.count(n) || outputs_.count(n) || alias_root.count(n))
                 continue;
             auto it = owned.find(n);
             if (it != owned.end()) {

@@ -356,6 +356,8 @@ public:
             return Status(TNNERR_LAYER_ERR, "Reshape type nhwc is not implemented on DEVICE_ROCM");
         size_t bytes = (size_t)DimsVectorUtils::Count(outputs[0]->GetBlobDesc().dims) *
                        DataTypeUtils::GetBytesSize(outputs[0]->GetBlobDesc().data_type);
+        if (Ptr(outputs[0]) == Ptr(inputs[0]))
+            return TNN_OK;  // the memory planner let the output share the input's buffer: nothing to move
         ROCM_CALL(tnn_rocm_memcpy_d2d(Ptr(outputs[0]), Ptr(inputs[0]), bytes, Stream()));
         return TNN_OK;
     }
