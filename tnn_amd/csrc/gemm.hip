@@ -1197,6 +1197,7 @@ int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int 
 //   112210 / 112211   64 x  64, 4 waves                 222210  128 x 128, 4 waves
 //   222221           128 x 128, 8 waves (two k-waves)   224211  256 x 128, 8 waves
 //   332221           192 x 192, 8 waves (two k-waves)   331182   96 x  96, 8 k-waves, 256-byte slabs
+//   111182            32 x  32, 8 k-waves, 256-byte slabs (fp32 only: small products)
 // Eight-wave workgroups put two waves on every SIMD inside one tile: while one waits for its LDS fragments the
 // other issues MFMAs, and a larger tile per CU moves fewer bytes through LDS and L2 per flop.  Four-wave tiles
 // larger than 128 x 128 (one wave per SIMD) were measured and never won with compiler-scheduled code.
@@ -1298,6 +1299,13 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
         cfg = 222221;
     if (DT == TNN_ROCM_F32)
         cfg %= 1000000;  // the fp32 instantiations are register-staged only
+    if (DT == TNN_ROCM_F32 && g_gemm_force_cfg <= 0 && cfg == 112211 && kbytes % 256 == 0 && kbytes >= 2048 &&
+        (((long)M + 63) / 64) * (((long)N + 63) / 64) * 2 <= kNumCU) {
+        // A small fp32 product (one attention layer at 128 tokens: 24 tiles of 64x64) leaves nine CUs in ten idle,
+        // and the fp32 matrix pipe is 16 times slower than the fp16 one: 32x32 tiles with the K range dealt to
+        // eight waves put four times as many CUs to work on each a quarter of the MFMAs.
+        cfg = 111182;
+    }
     if (kbytes % (64u << (cfg % 10)) != 0) {
         set_error("gemm: K=%d is not a whole number of slabs for tuning configuration %d", K, cfg);
         return TNN_ROCM_ESHAPE;
@@ -1325,6 +1333,10 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
         case 222210: TR_FAST(2, 2, 2, 2, 1, 64);
         case 222221: TR_FAST(2, 2, 2, 2, 2, 128);
         default: break;
+    }
+    if constexpr (DT == TNN_ROCM_F32) {
+        if (cfg == 111182)
+            TR_FAST(1, 1, 1, 1, 8, 256);
     }
     if constexpr (DT != TNN_ROCM_F32) {
         switch (cfg) {
