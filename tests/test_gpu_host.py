@@ -50,6 +50,35 @@ def test_config1_attention_layer_fp32_from_model_files():
     inst.close()
 
 
+def test_view_layers_share_their_input_buffer_and_change_nothing(monkeypatch):
+    """Reshape layers that only rename dimensions copy nothing (their output shares the input's buffer in the memory
+    plan); with TNN_ROCM_ALIAS_VIEWS=0 every blob has its own buffer and the layer copies.  Same graph, same input:
+    bit-identical outputs over several forwards (eager, the recording forward and graph replays)."""
+    host, tnnmodel, EncoderConfig, make_weights, _ = _mods()
+    say("host: view layers alias their input")
+    cfg = EncoderConfig(1, 768, 12, 3072)
+    lw = make_weights(cfg, seed=5, with_embeddings=False)["layers"][0]
+    g = tnnmodel.attention_layer_graph(lw, 128, 768, 12)
+    rng = np.random.default_rng(6)
+    xs = [rng.standard_normal((128, 768)).astype(np.float32) for _ in range(5)]
+    outs = {}
+    for alias in ("1", "0"):
+        monkeypatch.setenv("TNN_ROCM_ALIAS_VIEWS", alias)
+        inst = host.RocmInstance.from_graph(g, "fp32")
+        assert [t for t, _ in inst.layers()].count("Reshape") >= 4
+        res = []
+        for x in xs:
+            inst.set_input("x", x)
+            inst.forward()
+            res.append(inst.output("y").copy())
+        outs[alias] = res
+        inst.close()
+    for a, b in zip(outs["1"], outs["0"]):
+        assert np.array_equal(a, b)
+    ref = encoder_ref.attention_layer(xs[-1], lw, 1, 128, 12, None)
+    assert rel_err(outs["1"][-1], ref) <= 1e-5
+
+
 @pytest.mark.parametrize("precision", ["fp32", "fp16"])
 def test_encoder_from_model_files(precision):
     host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
