@@ -752,7 +752,10 @@ int tnn_rocm_gather(void *stream, const void *data, const int32_t *indices, void
     TR_REQUIRE(data && indices && out, TNN_ROCM_EINVAL, "gather: null pointer");
     TR_REQUIRE(slices > 0, TNN_ROCM_ESHAPE, "gather: empty table");
     TR_REQUIRE((long)batch * n_indices < (1l << 31), TNN_ROCM_ESHAPE, "gather: too many rows");
-    hipLaunchKernelGGL(gather_kernel, dim3(batch * n_indices), dim3(kBlock), 0, (hipStream_t)stream,
+    // a row is copied by as many waves as it has 16-byte vectors to hand out (1536-byte rows: two waves, not four)
+    size_t lanes = (slice_bytes / 16 + 63) / 64 * 64;
+    lanes        = lanes < 64 ? 64 : (lanes > (size_t)kBlock ? (size_t)kBlock : lanes);
+    hipLaunchKernelGGL(gather_kernel, dim3(batch * n_indices), dim3((unsigned)lanes), 0, (hipStream_t)stream,
                        (const char *)data, indices, (char *)out, slices, slice_bytes, n_indices, error_flag);
     TR_CHECK_LAUNCH();
     return 0;
