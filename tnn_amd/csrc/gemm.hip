@@ -206,11 +206,14 @@ template <int DT> struct QkvSplitEpilogue {
 // values), reduced over the workgroup after the main loop, and applied to the accumulators in the epilogue.
 // Other readers of y (the residual additions) still need the tensor: the workgroup of tile column j writes
 // y for the j-th share of the columns of its rows, so the LayerNorm launch disappears without y disappearing.
+int g_ln_y_ahead = 1;  // experiment hook, see tnn_rocm_debug_set_ln_y_ahead
+
 struct LnFold {
     float inv_cols, eps;
     const float *colsum;        // [N]
     const float *gamma, *beta;  // [K], for the y side output
     void *y;                    // [M, K] in the compute type, or nullptr
+    int y_ahead;                // 1: the source vectors of y are requested under the epilogue (0 for experiments)
 };
 
 // row sum and sum of squares of the eight values of an A fragment register quad
@@ -1060,6 +1063,20 @@ __global__ void __launch_bounds__(CFG::NT)
         }
         // row_st is read after the first staging barrier below
     }
+    // The LayerNorm output y is written at the very end from this tile's own share of its rows of A; the vectors it
+    // needs are requested here, once the last accumulators have been staged, so their latency hides under the
+    // remaining epilogue instead of standing alone at the kernel's tail.
+    constexpr int YPRE = 3;  // vectors a thread holds ahead (192 x 192 tiles: 12 rows x K/8 groups over 512 threads)
+    u32x4 y_pre[Epi::kRowStats ? YPRE : 1];
+    int y_r0 = 0, y_items = 0, y_groups = 1;
+    if constexpr (Epi::kRowStats) {
+        if (epi.ln.y) {
+            const int tn = n0 / BN;
+            y_groups     = K / 8;
+            y_r0         = (int)((long)tn * BM / tiles_n);
+            y_items      = ((int)((long)(tn + 1) * BM / tiles_n) - y_r0) * y_groups;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -1068,6 +1085,19 @@ __global__ void __launch_bounds__(CFG::NT)
             for (int r4 = 0; r4 < 4; ++r4)
                 *reinterpret_cast<acc4 *>(stage_me + (lane & 31) * SSTR + j * 32 + 8 * r4 + 4 * (lane >> 5)) =
                     acc4{acc[i][j][r4 * 4 + 0], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2], acc[i][j][r4 * 4 + 3]};
+        if constexpr (Epi::kRowStats) {
+            if (i == TM - 1) {
+#pragma unroll
+                for (int q = 0; q < YPRE; ++q) {
+                    const int item = tid + q * NT;
+                    if (epi.ln.y_ahead && item < y_items) {
+                        const int m = m0 + y_r0 + item / y_groups;
+                        if (m < M)
+                            y_pre[q] = *reinterpret_cast<const u32x4 *>(A + (size_t)m * lda + (item % y_groups) * 8);
+                    }
+                }
+            }
+        }
         __syncthreads();
 #pragma unroll
         for (int it = 0; it < (ITEMS + NT - 1) / NT; ++it) {
@@ -1118,9 +1148,9 @@ __global__ void __launch_bounds__(CFG::NT)
         // x * rstd * gamma + (beta - mean * rstd * gamma)
         if (epi.ln.y) {
             typedef typename GemmTraits<DT>::elem TY;
-            const int groups = K / 8, tn = n0 / BN;
-            const int r0 = (int)((long)tn * BM / tiles_n), r1 = (int)((long)(tn + 1) * BM / tiles_n);
-            for (int item = tid; item < (r1 - r0) * groups; item += NT) {
+            const int groups = y_groups, r0 = y_r0;
+            int q = 0;
+            for (int item = tid; item < y_items; item += NT, ++q) {
                 const int row = r0 + item / groups, c = (item % groups) * 8, m = m0 + row;
                 if (m >= M)
                     continue;
@@ -1130,8 +1160,16 @@ __global__ void __launch_bounds__(CFG::NT)
                 float4 e0 = *reinterpret_cast<const float4 *>(epi.ln.beta + c), e1 = *reinterpret_cast<const float4 *>(epi.ln.beta + c + 4);
                 const float kk[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
                 const float ee[8] = {e0.x, e0.y, e0.z, e0.w, e1.x, e1.y, e1.z, e1.w};
-                u32x4 raw = *reinterpret_cast<const u32x4 *>(A + (size_t)m * lda + c);
-                TY *pe    = reinterpret_cast<TY *>(&raw);
+                u32x4 raw;
+                if (epi.ln.y_ahead && q == 0)
+                    raw = y_pre[0];
+                else if (epi.ln.y_ahead && q == 1 && YPRE > 1)
+                    raw = y_pre[YPRE > 1 ? 1 : 0];
+                else if (epi.ln.y_ahead && q == 2 && YPRE > 2)
+                    raw = y_pre[YPRE > 2 ? 2 : 0];
+                else
+                    raw = *reinterpret_cast<const u32x4 *>(A + (size_t)m * lda + c);
+                TY *pe = reinterpret_cast<TY *>(&raw);
 #pragma unroll
                 for (int t = 0; t < 8; ++t)
                     Elem<DT>::st(&pe[t], Elem<DT>::ld(&pe[t]) * st.x * kk[t] + (ee[t] - mrs * kk[t]));
@@ -1609,7 +1647,7 @@ int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folde
         epi.residual = (const Elem<DT>::type *)residual;                                                              \
         epi.C        = (Elem<DT>::type *)C;                                                                           \
         epi.ldc      = N;                                                                                             \
-        epi.ln       = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y};                                          \
+        epi.ln       = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead};                                          \
         return launch_gemm_fast<DT, LnFloatEpilogue<DT>>((hipStream_t)stream, t, w_folded, M, N, K, K, K, epi);       \
     }
     if (dtype == TNN_ROCM_F16)
@@ -1645,7 +1683,7 @@ int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const voi
         epi.H     = H;                                                                                                \
         epi.S     = S;                                                                                                \
         epi.heads = heads;                                                                                            \
-        epi.ln    = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y};                                             \
+        epi.ln    = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead};                                             \
         return launch_gemm_fast<DT, LnQkvSplitEpilogue<DT>>((hipStream_t)stream, t, wqkv_folded, T, 3 * H, K, K, K, epi); \
     }
     if (dtype == TNN_ROCM_F16)
@@ -1663,6 +1701,10 @@ __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_config(int cf
 }
 __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_tune(const char *spec) {
     parse_tune(spec);
+    return 0;
+}
+__attribute__((visibility("default"))) int tnn_rocm_debug_set_ln_y_ahead(int on) {
+    g_ln_y_ahead = on ? 1 : 0;
     return 0;
 }
 __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_group_m(int group_m) {
