@@ -284,9 +284,13 @@ TNN_ROCM_API int tnn_rocm_quantize(void *stream, int src_dtype, const void *x, f
                                    size_t count);
 /* x = (float)q * scale     X86Int8ToFloat  x86_compute_int8.cc:1193-1252 */
 TNN_ROCM_API int tnn_rocm_dequantize(void *stream, const int8_t *q, float scale, int dst_dtype, void *x, size_t count);
-/* y = float2int8(((float)a*sa + (float)b*sb) * inv_so)   X86MatrixAddInt8 x86_compute_int8.cc:795-831 */
+/* int8 Add, X86MatrixAddInt8 (x86_compute_int8.cc:795-831; scales x86_add_layer_acc.cc:33-66) as the reference's x86
+ * build evaluates it (-mfma -ffast-math contract one product into the sum): y = float2int8(fma(b, sb, a*sa) * inv_so)
+ * in the 8-channel vector body, float2int8(fma(a, sa, b*sb) * inv_so) in the scalar tail, i.e. the last four
+ * channels when round_up(channels, 4) % 8 == 4.  channels = dims[1], inner = count(dims[2:]) of the blobs (plain
+ * row-major); every batch entry is computed (the reference's loop stops after the first). */
 TNN_ROCM_API int tnn_rocm_add_i8(void *stream, const int8_t *a, float sa, const int8_t *b, float sb, float inv_so,
-                                 int8_t *y, size_t count);
+                                 int8_t *y, size_t count, int channels, size_t inner);
 /* q_out = float2int8(gelu((float)q_in * in_scale) * out_inv_scale): Reformat -> GELU -> Reformat
  * collapsed into one pass (same three roundings as the separate layers). */
 TNN_ROCM_API int tnn_rocm_gelu_i8(void *stream, const int8_t *q_in, float in_scale, float out_inv_scale,

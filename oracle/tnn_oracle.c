@@ -314,15 +314,44 @@ ORC_API void orc_dequantize(const int8_t *q, float scale, float *x, size_t n) {
 
 /* int8 residual add, DEVICE_X86 form
  *   device/x86/acc/x86_add_layer_acc.cc:54-58 (dst scale = 1.0 / so), compute/x86_compute_int8.cc:795-831
- * y = float2int8( (a*sa + b*sb) * inv_so ) with separate roundings. */
-ORC_API void orc_add_int8_x86(const int8_t *a, float sa, const int8_t *b, float sb, float so, int8_t *y, size_t n) {
-    float inv = (float)(1.0 / so);
+ * The source reads float2int8( (a*sa + b*sb) * inv_so ).  Its translation unit is built with -mavx2 -mfma
+ * -ffast-math (device/x86/CMakeLists.txt:1-27), and g++ contracts one product into the sum.  Which one was
+ * established against the compiled reference over all 65536 (a, b) pairs on a tie-heavy scale triple
+ * (tests/test_oracle_vs_reference.py): the 8-channel vector body computes fma(b, sb, a*sa), the scalar tail (the last
+ * four channels when round_up(channels, 4) % 8 == 4) computes fma(a, sa, b*sb); the un-contracted form differs from
+ * either in thousands of those pairs.  `channels` = dims[1], `inner` = count(dims[2:]), element i of the plain
+ * row-major array sits in channel (i / inner) % channels.
+ * The x86 acc walks only the first batch entry (dims[0] is never read, :86-87: round_up(dims[1], 4) channels times
+ * count(dims, 2) positions) and leaves the rest of its output unwritten; this restatement computes every entry. */
+ORC_API void orc_add_int8_x86(const int8_t *a, float sa, const int8_t *b, float sb, float so, int8_t *y, size_t n,
+                              int channels, size_t inner) {
+    float inv     = (float)(1.0 / so);
+    int c4        = (channels + 3) / 4 * 4;
+    int vec_end   = c4 - ((c4 % 8 == 4) ? 4 : 0);
 #pragma omp parallel for schedule(static)
     for (size_t i = 0; i < n; ++i) {
-        float pa = (float)a[i] * sa;
-        float pb = (float)b[i] * sb;
-        float s  = pa + pb;
-        y[i]     = orc_float2int8(s * inv);
+        int c = (int)((i / inner) % (size_t)channels);
+        float s;
+        if (c < vec_end) {
+            float pa = (float)a[i] * sa;
+            s        = fmaf((float)b[i], sb, pa);
+        } else {
+            float pb = (float)b[i] * sb;
+            s        = fmaf((float)a[i], sa, pb);
+        }
+        y[i] = orc_float2int8(s * inv);
+    }
+}
+
+/* int8 residual add, DEVICE_NAIVE form
+ *   device/cpu/acc/cpu_add_layer_acc.cc:31-47, compute/compute_int8.cc:54-84 (zero points are 0 on this path)
+ * y = float2int8( (sa*a + sb*b) / so + 0.0f ): a division where the x86 form multiplies by float(1.0/so). */
+ORC_API void orc_add_int8_naive(const int8_t *a, float sa, const int8_t *b, float sb, float so, int8_t *y, size_t n) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) {
+        float acc = sa * ((float)a[i] - 0.0f);
+        acc       = acc + sb * ((float)b[i] - 0.0f);
+        y[i]      = orc_float2int8(acc / so + 0.0f);
     }
 }
 

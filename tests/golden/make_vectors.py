@@ -7,7 +7,7 @@ container by oracle/Makefile.ref) runs small seeded graphs on DEVICE_NAIVE (fp32
 "product" semantics), and inputs + outputs are stored.  The fixtures let the CPU checker and the HIP path be compared
 with the reference's results where the reference tree (and hence oracle/_ref) is absent.
 
-Run from the repository root after `make -C oracle`:   python tests/golden/make_vectors.py
+Run from the repository root after `make -C oracle`:   python tests/golden/make_vectors.py [fixture name ...]
 """
 import os
 import sys
@@ -163,12 +163,27 @@ def int8_encoder():
     np.savez_compressed(os.path.join(HERE, "int8_encoder_x86.npz"), **out)
 
 
+def int8_add():
+    """QuantizedAdd over all 65536 (a, b) int8 pairs for the scale triples of golden_util.INT8_ADD_SCALES, on both
+    devices; the int8 results are stored (the graph's fp32 output divided by the output scale)."""
+    import golden_util
+    out = {}
+    for k in range(len(golden_util.INT8_ADD_SCALES)):
+        qa, qb, x, z, sa, sb, so = golden_util.int8_add_case(k)
+        g = tnnmodel.int8_add_graph(golden_util.INT8_ADD_DIMS, sa, sb, so)
+        for dev in ("NAIVE", "X86"):
+            y = run(g, {"x": x, "z": z}, ["y"], dev)[0] / so
+            assert np.abs(y - np.rint(y)).max() < 1e-3
+            out["y%d_%s" % (k, dev.lower())] = np.rint(y).astype(np.int8)
+    np.savez_compressed(os.path.join(HERE, "int8_add.npz"), **out)
+
+
+ALL = {"single_ops": single_ops, "tiny_encoder": tiny_encoder, "config1_summary": config1_summary,
+       "int8_ffn": int8_ffn, "int8_encoder": int8_encoder, "int8_add": int8_add}
+
 if __name__ == "__main__":
     assert ref_driver.available(), "oracle/_ref is not built: run `make -C oracle` where the reference tree is present"
-    single_ops()
-    tiny_encoder()
-    config1_summary()
-    int8_ffn()
-    int8_encoder()
+    for name in (sys.argv[1:] or list(ALL)):  # no argument: every fixture; else only the named ones
+        ALL[name]()
     for f in sorted(os.listdir(HERE)):
         print("%8d  %s" % (os.path.getsize(os.path.join(HERE, f)), f))

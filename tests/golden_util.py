@@ -51,6 +51,22 @@ def int8_encoder():
     return cfg, w, B, S, scales, f
 
 
+INT8_ADD_DIMS = [1, 256, 256, 1]
+# (scale a, scale b, scale out): a generic triple, and a tie-heavy one (equal input scales, output scale twice that:
+# every odd a+b lands on a half-integer, where the x86 form's multiply by float(1/so) and the naive form's division
+# round differently for thousands of pairs)
+INT8_ADD_SCALES = ((0.031, 0.017, 0.027), (0.031004460528492928, 0.031004460528492928, 0.062008921056985855))
+
+
+def int8_add_case(k):
+    """All 65536 (a, b) int8 pairs as a [1, 256, 256, 1] blob pair: -> (qa, qb, x, z, sa, sb, so); x = qa*sa and
+    z = qb*sb are the float inputs whose quantisation gives qa and qb back exactly."""
+    sa, sb, so = (np.float32(v) for v in INT8_ADD_SCALES[k])
+    qa = np.repeat(np.arange(-128, 128, dtype=np.int8), 256).reshape(INT8_ADD_DIMS)
+    qb = np.tile(np.arange(-128, 128, dtype=np.int8), 256).reshape(INT8_ADD_DIMS)
+    return qa, qb, qa.astype(np.float32) * sa, qb.astype(np.float32) * sb, sa, sb, so
+
+
 def int8_projections(cfg, w, li=0):
     """(input blob, output blob, weight [N,K], bias) of the six projections of layer li in the int8 encoder graph"""
     lw, p = w["layers"][li], "l%d_" % li

@@ -159,10 +159,22 @@ def dequantize(q, scale):
 
 
 def add_int8_x86(a, sa, b, sb, so):
+    """a, b: int8 arrays in the blob's own dims (channel axis 1, as the engine counts it)."""
     a = np.ascontiguousarray(a, np.int8)
     b = np.ascontiguousarray(b, np.int8)
     y = np.empty(a.shape, np.int8)
-    lib().orc_add_int8_x86(_p(a), C.c_float(sa), _p(b), C.c_float(sb), C.c_float(so), _p(y), C.c_size_t(a.size))
+    channels = a.shape[1] if a.ndim >= 2 else 1
+    inner = int(np.prod(a.shape[2:], dtype=np.int64)) if a.ndim > 2 else 1
+    lib().orc_add_int8_x86(_p(a), C.c_float(sa), _p(b), C.c_float(sb), C.c_float(so), _p(y), C.c_size_t(a.size),
+                           channels, C.c_size_t(inner))
+    return y
+
+
+def add_int8_naive(a, sa, b, sb, so):
+    a = np.ascontiguousarray(a, np.int8)
+    b = np.ascontiguousarray(b, np.int8)
+    y = np.empty(a.shape, np.int8)
+    lib().orc_add_int8_naive(_p(a), C.c_float(sa), _p(b), C.c_float(sb), C.c_float(so), _p(y), C.c_size_t(a.size))
     return y
 
 

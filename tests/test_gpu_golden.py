@@ -80,9 +80,26 @@ def test_int8_ffn_bit_exact_against_reference_x86():
     s_y = np.float32(f["scales"][3])
     diff = np.abs(np.rint(got / s_y) - np.rint(f["y_x86"] / s_y))
     say("  mismatching int8 outputs: %d of %d" % (int((diff != 0).sum()), diff.size))
-    # int8 GEMMs and quantisers are bit-exact; the fp32 GELU between them may move a value across a rounding
-    # boundary of the second quantiser (device erff vs the CPU's double erf): at most 1 LSB on at most 0.1 %
-    assert diff.max() <= 1 and (diff != 0).mean() <= 1e-3
+    assert diff.max() == 0  # int8 GEMMs, quantisers and the GELU between them (double erf) are all bit-exact
+
+
+@pytest.mark.parametrize("case", [0, 1])
+def test_int8_add_graph_bit_exact_against_reference_x86(case):
+    """QuantizedAdd through the host (Reformat layers inserted by the optimizer, RocmBinaryLayerAcc<Add> on int8
+    blobs) over all 65536 (a, b) pairs against the reference's DEVICE_X86 run."""
+    from tnn_amd import host, tnnmodel
+    qa, qb, x, z, sa, sb, so = golden_util.int8_add_case(case)
+    say("golden: QuantizedAdd graph on the host vs reference X86 fixture, scales %d" % case)
+    inst = host.RocmInstance.from_graph(tnnmodel.int8_add_graph(golden_util.INT8_ADD_DIMS, sa, sb, so), "fp32")
+    types = [t for t, _ in inst.layers()]
+    assert types.count("Reformat") == 3 and types.count("QuantizedAdd") == 1, types
+    inst.set_input("x", x)
+    inst.set_input("z", z)
+    inst.forward()
+    got = inst.output("y") / so
+    inst.close()
+    assert np.abs(got - np.rint(got)).max() < 1e-3
+    assert np.array_equal(np.rint(got).astype(np.int8), golden_util.load("int8_add.npz")["y%d_x86" % case])
 
 
 @pytest.mark.parametrize("precision", ["fp32", "fp16"])

@@ -154,12 +154,10 @@ def test_int8_ffn_from_model_files_bit_exact(monkeypatch):
         inst.forward()
         got = inst.output("y")
         inst.close()
-        # the two int8 GEMMs and both quantisers are bit-exact; the fp32 GELU between them uses the device erff
-        # (last-ulp differences against the CPU's double erf), which can move a value across a rounding boundary of
-        # the second quantiser in rare cases: allow at most 1 LSB on at most 0.1 % of the outputs
+        # the two int8 GEMMs, both quantisers and the GELU between them (double erf, as the CPU path) are bit-exact
         diff = np.abs(np.rint(got / s_y) - yq.astype(np.float64))
         say("  fuse=%s mismatching int8 outputs: %d of %d" % (fuse, int((diff != 0).sum()), diff.size))
-        assert diff.max() <= 1 and (diff != 0).mean() <= 1e-3
+        assert diff.max() == 0
         outs[fuse] = got
     assert np.array_equal(outs["0"], outs["1"])  # folding the Reformat layers changes no value in fp32
 

@@ -10,6 +10,7 @@ import sys
 import numpy as np
 import pytest
 
+import golden_util
 import orc
 
 torch = pytest.importorskip("torch")
@@ -71,7 +72,9 @@ def test_gelu_fp32(n):
     x[:1] = -2.281006575  # the point where the tanh form is visibly wrong
     got = host(ops().gelu(dev(x)))
     ref = orc.gelu(x)
-    assert rel_err(got, ref) <= 1e-6
+    # the device evaluates the reference's expression (fp32 products, double erf, one rounding to fp32): the only room
+    # left is a last-bit difference between two double erf routines surviving that rounding
+    assert (got != ref).mean() <= 1e-5 and rel_err(got, ref) <= 2e-7
     # special values
     sp = np.array([0.0, -0.0, np.inf, -40.0, 40.0], np.float32)
     got = host(ops().gelu(dev(sp)))
@@ -333,6 +336,24 @@ def test_dequantize_and_add_i8_tails_and_unaligned_buffers(n, offset, dtype):
     assert np.array_equal(got, orc.add_int8_x86(a, sa, q, sb, so))
 
 
+@pytest.mark.parametrize("dims", [(1, 256, 256, 1), (1, 12, 4096, 1), (3, 772, 5), (2, 768), (7, 3)])
+def test_add_i8_tie_heavy_scales_follow_the_compiled_x86_forms(dims):
+    """Equal input scales and an output scale of twice that put every odd a+b on a half-integer, where the two
+    contracted forms of the reference's x86 build (vector body / scalar tail channels) and the un-contracted sum all
+    round differently for thousands of pairs."""
+    say("add_i8 tie-heavy dims=%s" % (dims,))
+    sa, sb, so = (np.float32(v) for v in golden_util.INT8_ADD_SCALES[1])
+    n = int(np.prod(dims))
+    idx = np.arange(n) % 65536
+    a = ((idx // 256) - 128).astype(np.int8).reshape(dims)
+    b = ((idx % 256) - 128).astype(np.int8).reshape(dims)
+    inv = np.float32(1.0 / np.float64(so))
+    got = host(ops().add_i8(dev(a), float(sa), dev(b), float(sb), float(inv)))
+    assert np.array_equal(got, orc.add_int8_x86(a, sa, b, sb, so))
+    if dims == (1, 256, 256, 1):  # the committed result of the reference's own DEVICE_X86 run
+        assert np.array_equal(got, golden_util.load("int8_add.npz")["y1_x86"])
+
+
 @pytest.mark.parametrize("shape,order,offset", [
     ((2, 130, 3, 70), (0, 2, 3, 1), 0),      # transpose, ragged 64 x 64 tiles, two batch axes
     ((5, 64, 96), (0, 2, 1), 0),             # plain batched transpose
@@ -363,10 +384,12 @@ def test_gelu_i8_matches_three_layer_chain():
     inv = np.float32(1.0 / np.float64(s_out))
     got = host(ops().gelu_i8(dev(q), float(s_in), float(inv)))
     ref = orc.quantize_x86(orc.gelu(orc.dequantize(q, s_in)), s_out)
-    # erff on the device and in glibc may differ in the last ulp, which can flip a value that lands on
-    # a rounding boundary: allow +-1 LSB there but require near-total equality
-    diff = np.abs(got.astype(np.int32) - ref.astype(np.int32))
-    assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+    assert np.array_equal(got, ref)  # the table is built with the C library's double erf, as the CPU chain
+    for s_in, s_out in ((0.0005, 0.0003), (0.11, 0.07), (1.7, 0.9), (0.031, 0.25)):
+        s_in, s_out = np.float32(s_in), np.float32(s_out)
+        inv = np.float32(1.0 / np.float64(s_out))
+        got = host(ops().gelu_i8(dev(q), float(s_in), float(inv)))
+        assert np.array_equal(got, orc.quantize_x86(orc.gelu(orc.dequantize(q, s_in)), s_out)), (s_in, s_out)
 
 
 # ---- GEMM ------------------------------------------------------------------------------------------
@@ -916,6 +939,5 @@ def test_gemm_i8_with_gelu_table_bit_exact(M, N, K):
     assert np.array_equal(fused, two)
     ref_q, _ = orc.fc_int8(a, w, bias, scale)
     ref = orc.quantize_x86(orc.gelu(orc.dequantize(ref_q, s_mid)), s_out)
-    diff = np.abs(fused.astype(int) - ref.astype(int))
-    assert diff.max() <= 1 and (diff > 0).mean() <= 1e-3   # device erff vs the checker's double erf on a rounding boundary
+    assert np.array_equal(fused, ref)
     assert len(np.unique(host(q))) > 100                    # the requantised values span the int8 range

@@ -162,3 +162,13 @@ def test_int8_encoder_reformat_layers_are_folded(precision, monkeypatch):
         monkeypatch.setenv(fold, "0")
     t2 = _types(host.plan(g, precision=precision))
     assert t2["RocmQuantLinearGelu"] == 0 and t2["RocmGeluInt8"] == 1
+
+
+def test_quantized_add_graph_gets_reformat_layers_and_int8_blobs():
+    g = tnnmodel.int8_add_graph([1, 256, 256, 1], np.float32(0.031), np.float32(0.017), np.float32(0.027))
+    plan = host.plan(g, precision="fp32")
+    t = _types(plan)
+    assert t["QuantizedAdd"] == 1 and t["Reformat"] == 3 and t["Mul"] == 3, t
+    add = [l for l in plan if l["type"] == "QuantizedAdd"][0]
+    assert add["inputs"] == ["a_int8_reformat", "b_int8_reformat"]
+    assert add["output_dims"] == [[1, 256, 256, 1]]

@@ -159,6 +159,87 @@ def test_int8_ffn_bit_identical(dev):
     assert np.array_equal(got, orc.dequantize(yq, s_y))
 
 
+@pytest.mark.parametrize("dev", ["NAIVE", "X86"])
+@pytest.mark.parametrize("case", [0, 1])
+def test_int8_add_all_pairs_bit_identical(dev, case):
+    """QuantizedAdd over all 65536 (a, b) int8 pairs: each device of the reference equals its own form of the
+    restatement exactly (x86: multiply by float(1/so), x86_add_layer_acc.cc:54-58; naive: divide,
+    compute_int8.cc:54-84), and on the tie-heavy scale triple the two forms differ in thousands of pairs, so a
+    restatement with the wrong form fails here."""
+    import golden_util
+    qa, qb, x, z, sa, sb, so = golden_util.int8_add_case(case)
+    assert np.array_equal(orc.quantize_x86(x, sa), qa) and np.array_equal(orc.quantize_naive(z, sb), qb)
+    g = tnnmodel.int8_add_graph(golden_util.INT8_ADD_DIMS, sa, sb, so)
+    got = _run(g, {"x": x, "z": z}, "y", dev)
+    mine = (orc.add_int8_x86 if dev == "X86" else orc.add_int8_naive)(qa, sa, qb, sb, so)
+    assert np.array_equal(got, orc.dequantize(mine, so))
+    other = (orc.add_int8_naive if dev == "X86" else orc.add_int8_x86)(qa, sa, qb, sb, so)
+    if case == 1:
+        assert (other != mine).sum() > 10000
+    assert np.array_equal(mine, golden_util.load("int8_add.npz")["y%d_%s" % (case, dev.lower())])
+
+
+def _identity_fc_graph(T, N, bias, w_scale, s_in, s_out):
+    """fp32 [T,N] -> quantize(s_in) -> QuantizedInnerProduct with the identity as int8 weight -> dequantize(s_out):
+    the accumulator of column c is the quantised input itself, so the graph exposes the engine's quantiser
+    (bias 0, scales 1: output = q) and its requantiser on chosen (accumulator, scale) pairs (acc = q + bias[c])."""
+    g = tnnmodel.Graph()
+    one = np.array([1.0], np.float32)
+    g.add_input("x", [T, N])
+    g.add_layer("Mul", "in_copy", ["x"], ["a"], [1])
+    g.res_eltwise("in_copy", "Mul", one)
+    g.add_layer("QuantizedInnerProduct", "fc", ["a"], ["h"], [N, 1, 0, 1])
+    g.res_blob_scale("a", s_in)
+    g.res_inner_product("fc", np.eye(N, dtype=np.int8), bias, quant_scale=w_scale)
+    g.res_blob_scale("h", s_out)
+    g.add_layer("Mul", "out_copy", ["h"], ["y"], [1])
+    g.res_eltwise("out_copy", "Mul", one)
+    g.add_output("y")
+    return g
+
+
+@pytest.mark.parametrize("dev", ["NAIVE", "X86"])
+def test_quantiser_band_against_compiled_reference(dev):
+    """Every fp32 within +-12 ulp of (m + 0.5)*s, m = -130..130, for five scales, through the engine's own Reformat
+    layer: the x86 form (multiply by float(1/s)) and the naive form (divide) of the restatement each equal their
+    device exactly - in particular the x86 build does not contract the +-0.5 add into the multiply."""
+    N = 256
+    for s in (0.031, 0.0123, 1.0 / 3, 0.05, 0.7):
+        s = np.float32(s)
+        base = ((np.arange(-130, 131, dtype=np.float64) + 0.5) * np.float64(s)).astype(np.float32)
+        vals, up, dn = [base], base, base
+        for _ in range(12):
+            up = np.nextafter(up, np.float32(np.inf))
+            dn = np.nextafter(dn, np.float32(-np.inf))
+            vals += [up, dn]
+        v = np.concatenate(vals)
+        T = (v.size + N - 1) // N
+        x = np.zeros(T * N, np.float32)
+        x[:v.size] = v
+        x = x.reshape(T, N)
+        g = _identity_fc_graph(T, N, np.zeros(N, np.int32), np.ones(N, np.float32), s, np.float32(1.0))
+        want = (orc.quantize_x86 if dev == "X86" else orc.quantize_naive)(x, s)
+        assert np.array_equal(_run(g, {"x": x}, "y", dev), want.astype(np.float32)), float(s)
+
+
+@pytest.mark.parametrize("dev", ["NAIVE", "X86"])
+def test_requantiser_near_ties_against_compiled_reference(dev):
+    """float2int8((acc + bias) * scale) on the engine's own int8 InnerProduct with per-channel scales a few ulp around
+    k/2^j / {1,3,5,7,100}: products at and next to half-integers."""
+    N, T = 256, 64
+    rng = np.random.default_rng(1)
+    q = rng.integers(-128, 128, (T, N)).astype(np.int8)
+    for _ in range(4):
+        bias = rng.integers(-3000, 3000, N).astype(np.int32)
+        ws = (rng.choice([0.5, 1.5, 0.25, 0.125, 2.5], N) * (1 + rng.integers(-3, 4, N) * 2.0 ** -23)
+              / rng.choice([1, 3, 5, 7, 100], N)).astype(np.float32)
+        g = _identity_fc_graph(T, N, bias, ws, np.float32(1.0), np.float32(1.0))
+        ref, acc = orc.fc_int8(q, np.eye(N, dtype=np.int8), bias, orc.fc_int8_scale(ws, np.float32(1.0), N))
+        assert np.array_equal(acc, q.astype(np.int32) + bias)
+        assert 0.3 < (np.abs(ref.astype(int)) < 127).mean() < 0.7  # half the outputs are not saturated
+        assert np.array_equal(_run(g, {"x": q.astype(np.float32)}, "y", dev), ref.astype(np.float32))
+
+
 def test_float2int8_exhaustive_band_against_definition():
     # every fp32 within +-3 ulp of every half-integer in [-130.5, 130.5]: the add-then-truncate definition
     k = (np.arange(-261, 262, dtype=np.float64) * 0.5).astype(np.float32)

@@ -68,7 +68,7 @@ SIGNATURES = {
     "tnn_rocm_cast": [_vp, _i, _vp, _i, _vp, _sz],
     "tnn_rocm_quantize": [_vp, _i, _vp, _f, _vp, _sz],
     "tnn_rocm_dequantize": [_vp, _vp, _f, _i, _vp, _sz],
-    "tnn_rocm_add_i8": [_vp, _vp, _f, _vp, _f, _f, _vp, _sz],
+    "tnn_rocm_add_i8": [_vp, _vp, _f, _vp, _f, _f, _vp, _sz, _i, _sz],
     "tnn_rocm_gelu_i8": [_vp, _vp, _f, _f, _vp, _sz],
 }
 

@@ -77,10 +77,14 @@ __device__ __forceinline__ int8_t float2int8_ref(float v) {
     return (int8_t)(int)t;
 }
 
-// erf GELU in fp32, the product kept un-contracted in the reference's operand order.
+// erf GELU for fp32 results, evaluated as the reference's CPU path compiles (cpu_gelu_layer_acc.cc:42-45 includes
+// only <cmath>, so its unqualified erf is the double one): x*0.7071f and 0.5f*x are fp32 products, erf, the +1 and the
+// final product are double, and the store rounds once to fp32.  erff would differ in the last ulp, which is enough
+// to move a value across a rounding boundary of a quantiser that follows.
 __device__ __forceinline__ float gelu_erf(float x) {
-    float e = erff(__fmul_rn(x, 0.707106793288165f));
-    return __fmul_rn(__fmul_rn(0.5f, x), __fadd_rn(e, 1.0f));
+    const float hv = __fmul_rn(0.5f, x);
+    const double e = erf((double)__fmul_rn(x, 0.707106793288165f)) + 1.0;
+    return (float)((double)hv * e);
 }
 
 // erf GELU for results that are rounded to fp16/bf16.  With a = |x| and Phi(-a) = erfc(a/sqrt2)/2:

@@ -379,6 +379,16 @@ __global__ void __launch_bounds__(kBlock) dequantize_vec_kernel(const int8_t *__
         Elem<DT>::st(&x[t], __fmul_rn((float)q[t], scale));
 }
 
+// int8 Add in the form the reference's x86 build computes (x86_compute_int8.cc:795-831 compiled with -mfma
+// -ffast-math, device/x86/CMakeLists.txt:1-27: one product is contracted into the sum).  Its 8-channel vector body
+// evaluates fma(b, sb, a*sa); the scalar tail - the last four channels when round_up(channels, 4) % 8 == 4 -
+// evaluates fma(a, sa, b*sb).  `body` selects the form.
+__device__ __forceinline__ int8_t add_i8_value(int8_t a, float sa, int8_t b, float sb, float inv_so, bool body) {
+    const float fa = (float)a, fb = (float)b;
+    const float s  = body ? fmaf(fb, sb, __fmul_rn(fa, sa)) : fmaf(fa, sa, __fmul_rn(fb, sb));
+    return float2int8_ref(__fmul_rn(s, inv_so));
+}
+
 __global__ void __launch_bounds__(kBlock) add_i8_vec_kernel(const int8_t *__restrict__ a, float sa,
                                                             const int8_t *__restrict__ b, float sb, float inv_so,
                                                             int8_t *__restrict__ y, size_t n) {
@@ -392,46 +402,40 @@ __global__ void __launch_bounds__(kBlock) add_i8_vec_kernel(const int8_t *__rest
             uint32_t packed = 0;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                float pa = __fmul_rn((float)(int8_t)((va[w] >> (8 * k)) & 0xffu), sa);
-                float pb = __fmul_rn((float)(int8_t)((vb[w] >> (8 * k)) & 0xffu), sb);
-                float sum = __fadd_rn(pa, pb);
-                packed |= ((uint32_t)(uint8_t)float2int8_ref(__fmul_rn(sum, inv_so))) << (8 * k);
+                const int8_t qa = (int8_t)((va[w] >> (8 * k)) & 0xffu), qb = (int8_t)((vb[w] >> (8 * k)) & 0xffu);
+                packed |= ((uint32_t)(uint8_t)add_i8_value(qa, sa, qb, sb, inv_so, true)) << (8 * k);
             }
             o[w] = packed;
         }
         reinterpret_cast<u32x4 *>(y)[i] = o;
     }
-    for (size_t t = nvec * 16 + first; t < n; t += stride) {
-        float pa = __fmul_rn((float)a[t], sa);
-        float pb = __fmul_rn((float)b[t], sb);
-        y[t]     = float2int8_ref(__fmul_rn(__fadd_rn(pa, pb), inv_so));
-    }
+    for (size_t t = nvec * 16 + first; t < n; t += stride)
+        y[t] = add_i8_value(a[t], sa, b[t], sb, inv_so, true);
 }
 
+// any alignment; channels from `tail_from` on (channel = (i / inner) % channels) take the scalar-tail form
 __global__ void __launch_bounds__(kBlock) add_i8_kernel(const int8_t *__restrict__ a, float sa,
                                                         const int8_t *__restrict__ b, float sb, float inv_so,
-                                                        int8_t *__restrict__ y, size_t n) {
+                                                        int8_t *__restrict__ y, size_t n, unsigned channels,
+                                                        size_t inner, unsigned tail_from) {
     size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        float pa = __fmul_rn((float)a[i], sa);
-        float pb = __fmul_rn((float)b[i], sb);
-        float s  = __fadd_rn(pa, pb);
-        y[i]     = float2int8_ref(__fmul_rn(s, inv_so));
+        const bool body = tail_from >= channels || (unsigned)((i / inner) % channels) < tail_from;
+        y[i]            = add_i8_value(a[i], sa, b[i], sb, inv_so, body);
     }
 }
 
-// int8 -> GELU -> int8 has only 256 possible inputs: every workgroup first tabulates the exact chain
-// (dequantise, erf GELU, quantise: one entry per thread) in LDS, then maps bytes through the table, sixteen per
-// thread and access.  Value for value the same as evaluating the chain per element.
-__global__ void __launch_bounds__(256) gelu_i8_kernel(const int8_t *__restrict__ qi, float in_scale, float out_inv,
+// int8 -> GELU -> int8 has only 256 possible inputs, so the chain (dequantise, erf GELU, quantise) is a 256-entry
+// table.  The launcher evaluates it on the host with the C library's double erf - the very routine the reference's
+// CPU path calls - and hands it over by value as a kernel argument (256 bytes: no device memory, no copy, safe under
+// graph capture); every workgroup copies it to LDS and maps bytes through it, sixteen per thread and access.
+struct GeluTable {
+    int8_t q[256];
+};
+__global__ void __launch_bounds__(256) gelu_i8_kernel(const int8_t *__restrict__ qi, GeluTable tab,
                                                       int8_t *__restrict__ qo, size_t n, int vector_ok) {
     __shared__ int8_t table[256];
-    {
-        const int q = (int)threadIdx.x - 128;
-        float x     = __fmul_rn((float)q, in_scale);
-        float g     = gelu_erf(x);
-        table[threadIdx.x] = float2int8_ref(__fmul_rn(g, out_inv));
-    }
+    table[threadIdx.x] = tab.q[threadIdx.x];
     __syncthreads();
     const size_t stride = (size_t)gridDim.x * blockDim.x, first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t nvec   = vector_ok ? n / 16 : 0;
@@ -878,16 +882,19 @@ int tnn_rocm_dequantize(void *stream, const int8_t *q, float scale, int ddt, voi
 }
 
 int tnn_rocm_add_i8(void *stream, const int8_t *a, float sa, const int8_t *b, float sb, float inv_so, int8_t *y,
-                    size_t n) {
+                    size_t n, int channels, size_t inner) {
     if (n == 0)
         return 0;
     TR_REQUIRE(a && b && y, TNN_ROCM_EINVAL, "add_i8: null pointer");
-    if (aligned16(a) && aligned16(b) && aligned16(y) && n >= 16)
+    TR_REQUIRE(channels >= 1 && inner >= 1, TNN_ROCM_EINVAL, "add_i8: channels %d, inner %zu", channels, inner);
+    const int c4        = (channels + 3) / 4 * 4;
+    const int tail_from = c4 % 8 == 4 ? c4 - 4 : c4;  // first channel of the reference loop's scalar tail
+    if (tail_from >= channels && aligned16(a) && aligned16(b) && aligned16(y) && n >= 16)
         hipLaunchKernelGGL(add_i8_vec_kernel, dim3(grid_for(n / 16)), dim3(kBlock), 0, (hipStream_t)stream, a, sa, b, sb,
                            inv_so, y, n);
     else
         hipLaunchKernelGGL(add_i8_kernel, dim3(grid_for(n)), dim3(kBlock), 0, (hipStream_t)stream, a, sa, b, sb, inv_so,
-                           y, n);
+                           y, n, (unsigned)channels, inner, (unsigned)tail_from);
     TR_CHECK_LAUNCH();
     return 0;
 }
@@ -896,11 +903,25 @@ int tnn_rocm_gelu_i8(void *stream, const int8_t *qi, float in_scale, float out_i
     if (n == 0)
         return 0;
     TR_REQUIRE(qi && qo, TNN_ROCM_EINVAL, "gelu_i8: null pointer");
+    // x86_compute_int8.cc:1193-1252 (q*scale), cpu_gelu_layer_acc.cc:42-45 (fp32 products, double erf, one rounding
+    // to fp32), x86_compute_int8.cc:26-39 + 1254-1318 (x*(1/scale), +-0.5f, clamp, truncate)
+    GeluTable tab;
+    for (int q = -128; q < 128; ++q) {
+        const float x  = (float)q * in_scale;
+        const float hv = 0.5f * x;
+        const double e = erf((double)(x * 0.707106793288165f)) + 1.0;
+        const float g  = (float)((double)hv * e);
+        float t        = g * out_inv_scale;
+        t              = t + (t >= 0.f ? 0.5f : -0.5f);
+        t              = t > 127.0f ? 127.0f : t;
+        t              = t < -128.0f ? -128.0f : t;
+        tab.q[q + 128] = (t != t) ? (int8_t)0 : (int8_t)(int)t;
+    }
     const int vector_ok = ((uintptr_t)qi % 16 == 0 && (uintptr_t)qo % 16 == 0) ? 1 : 0;
     size_t blocks       = (n / 16 + 255) / 256;
     blocks              = blocks < 1 ? 1 : (blocks > 2048 ? 2048 : blocks);
-    hipLaunchKernelGGL(gelu_i8_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, qi, in_scale,
-                       out_inv_scale, qo, n, vector_ok);
+    hipLaunchKernelGGL(gelu_i8_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, qi, tab, qo, n,
+                       vector_ok);
     TR_CHECK_LAUNCH();
     return 0;
 }

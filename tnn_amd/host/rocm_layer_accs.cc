@@ -183,8 +183,11 @@ public:
                 s[i] = b8->GetIntResource()->scale_handle.force_to<float *>()[0];
             }
             float inv_so = (float)(1.0 / s[2]);  // x86_add_layer_acc.cc:54-58
+            const int channels = out_dims.size() > 1 ? out_dims[1] : 1;
+            const size_t inner = out_dims.size() > 2 ? (size_t)DimsVectorUtils::Count(out_dims, 2) : 1;
             ROCM_CALL(tnn_rocm_add_i8(Stream(), (const int8_t *)Ptr(inputs[0]), s[0], (const int8_t *)Ptr(inputs[1]), s[1],
-                                      inv_so, (int8_t *)Ptr(outputs[0]), (size_t)DimsVectorUtils::Count(out_dims)));
+                                      inv_so, (int8_t *)Ptr(outputs[0]), (size_t)DimsVectorUtils::Count(out_dims),
+                                      channels > 0 ? channels : 1, inner > 0 ? inner : 1));
             return TNN_OK;
         }
         if (!IsFloatType(dt))

@@ -296,9 +296,15 @@ def dequantize(q, scale, dtype=torch.float32):
 
 
 def add_i8(a, sa, b, sb, inv_so):
+    """a, b in the blob's own dims: axis 1 is the channel axis the reference's loop walks."""
     _chk(a, b)
     y = torch.empty_like(a)
-    capi.call("tnn_rocm_add_i8", _stream(), _p(a), float(sa), _p(b), float(sb), float(inv_so), _p(y), a.numel())
+    channels = a.shape[1] if a.dim() >= 2 else 1
+    inner = 1
+    for d in a.shape[2:]:
+        inner *= d
+    capi.call("tnn_rocm_add_i8", _stream(), _p(a), float(sa), _p(b), float(sb), float(inv_so), _p(y), a.numel(),
+              int(channels), max(int(inner), 1))
     return y
 
 

@@ -296,3 +296,27 @@ def int8_ffn_graph(T, K, F, w1_q, b1_q, w1_scale, w2_q, b2_q, w2_scale, s_in, s_
     g.res_eltwise("out_copy", "Mul", one)
     g.add_output("y")
     return g
+
+
+def int8_add_graph(dims, s_a, s_b, s_out):
+    """Two fp32 inputs `x`, `z` of shape `dims` -> quantize each -> QuantizedAdd -> dequantize -> fp32 `y`.  As in
+    int8_ffn_graph the Reformat layers are left to the engine's optimizer and the Mul-by-one layers keep the model
+    inputs and the output in fp32; the three int8 blobs carry per-tensor BlobScale resources.  The x86 int8 Add
+    (source/tnn/device/x86/acc/x86_add_layer_acc.cc:77-86) walks dims[1] channels x count(dims[2:]) positions of
+    the first batch entry only, so `dims` should be [1, C, H, W] for the engine's DEVICE_X86 to cover every value."""
+    g = Graph()
+    one = np.array([1.0], np.float32)
+    g.add_input("x", dims)
+    g.add_input("z", dims)
+    g.add_layer("Mul", "in_copy_a", ["x"], ["a"], [1])
+    g.res_eltwise("in_copy_a", "Mul", one)
+    g.add_layer("Mul", "in_copy_b", ["z"], ["b"], [1])
+    g.res_eltwise("in_copy_b", "Mul", one)
+    g.add_layer("QuantizedAdd", "sum", ["a", "b"], ["c"], [1])
+    g.res_blob_scale("a", s_a)
+    g.res_blob_scale("b", s_b)
+    g.res_blob_scale("c", s_out)
+    g.add_layer("Mul", "out_copy", ["c"], ["y"], [1])
+    g.res_eltwise("out_copy", "Mul", one)
+    g.add_output("y")
+    return g
