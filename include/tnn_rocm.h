@@ -296,6 +296,20 @@ TNN_ROCM_API int tnn_rocm_add_i8(void *stream, const int8_t *a, float sa, const 
 TNN_ROCM_API int tnn_rocm_gelu_i8(void *stream, const int8_t *q_in, float in_scale, float out_inv_scale,
                                   int8_t *q_out, size_t count);
 
+/* ---- tuning and test hooks --------------------------------------------------------------------
+ * No counterpart in the reference.  Process-wide switches for experiments and for the tests that force each kernel
+ * variant; plain words read by later launches, so set them while no other thread is launching.  All return 0.
+ *   gemm_config   : 0 = shape heuristic, -1 = the baseline kernel, else a tile-configuration code of the tiled kernel
+ *   gemm_tune     : "MxNxK:code,..." overrides of the heuristic for single shapes (also TNN_ROCM_GEMM_TUNE at first use)
+ *   gemm_group_m  : tiles per group of the XCD-aware tile order (0 = default)
+ *   ln_y_ahead    : 1 (default) = the LayerNorm-folding GEMMs request the source vectors of their y output early
+ *   attention_dma : 1 (default) = V^T attention stages K / V^T tiles global -> LDS directly, 0 = through registers */
+TNN_ROCM_API int tnn_rocm_debug_set_gemm_config(int cfg);
+TNN_ROCM_API int tnn_rocm_debug_set_gemm_tune(const char *spec);
+TNN_ROCM_API int tnn_rocm_debug_set_gemm_group_m(int group_m);
+TNN_ROCM_API int tnn_rocm_debug_set_ln_y_ahead(int on);
+TNN_ROCM_API int tnn_rocm_debug_set_attention_dma(int on);
+
 #ifdef __cplusplus
 }
 #endif

@@ -38,6 +38,17 @@ def test_library_exports_every_declared_symbol(header):
     assert not missing, "declared in include/%s but not exported: %s" % (header, missing)
 
 
+@pytest.mark.parametrize("header", sorted(LIBS))
+def test_library_exports_nothing_undeclared(header):
+    """the reverse direction: every tnn_rocm_* / tnn_host_* function the library exports is declared in its header"""
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", LIBS[header]], capture_output=True, text=True, check=True).stdout
+    exported = {l.split()[-1] for l in out.splitlines() if l.split() and l.split()[-2] in ("T", "t", "W")}
+    prefix = "tnn_rocm_" if header == "tnn_rocm.h" else "tnn_host_"
+    undeclared = sorted(n for n in exported if n.startswith(prefix) and n not in set(declared_functions(header)))
+    assert not undeclared, undeclared
+
+
 def test_ctypes_tables_match_the_headers():
     from tnn_amd import capi
     declared = set(declared_functions("tnn_rocm.h"))

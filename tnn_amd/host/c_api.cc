@@ -144,7 +144,7 @@ HOST_API int tnn_host_forward(void *hp) {
 // enqueue only; pair with tnn_host_sync
 HOST_API int tnn_host_forward_async(void *hp) {
     auto h    = static_cast<Handle *>(hp);
-    Status st = h->inst->ForwardAsync();
+    Status st = h->inst->ForwardAsync(nullptr);
     return st == TNN_OK ? 0 : fail(h, st);
 }
 

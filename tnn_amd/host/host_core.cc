@@ -118,16 +118,19 @@ Mat::Mat(DeviceType device_type, MatType mat_type, DimsVector dims)
     owned_    = std::shared_ptr<char>(new char[n > 0 ? n : 1](), std::default_delete<char[]>());
     data_     = owned_.get();
 }
-std::map<DeviceType, std::shared_ptr<BlobConverterAccCreater>> &GetBlobConverterCreaterMap() {
-    static std::map<DeviceType, std::shared_ptr<BlobConverterAccCreater>> m;
+std::shared_ptr<BlobConverterManager> &BlobConverterManager::Shared() {
+    static std::shared_ptr<BlobConverterManager> m = std::make_shared<BlobConverterManager>();
     return m;
 }
-BlobConverter::BlobConverter(Blob *blob) {
-    auto &m = GetBlobConverterCreaterMap();
-    auto it = m.find(blob->GetBlobDesc().device_type);
-    if (it != m.end())
-        impl_ = it->second->CreateBlobConverterAcc(blob);
+int BlobConverterManager::RegisterBlobConverterAccCreater(DeviceType type, std::shared_ptr<BlobConverterAccCreater> creater) {
+    converter_creater_map_[type] = creater;
+    return 0;
 }
+std::shared_ptr<BlobConverterAcc> BlobConverterManager::CreateBlobConverterAcc(Blob *blob) {
+    auto it = converter_creater_map_.find(blob->GetBlobDesc().device_type);
+    return it == converter_creater_map_.end() ? nullptr : it->second->CreateBlobConverterAcc(blob);
+}
+BlobConverter::BlobConverter(Blob *blob) { impl_ = BlobConverterManager::Shared()->CreateBlobConverterAcc(blob); }
 Status BlobConverter::ConvertToMat(Mat &image, MatConvertParam param, void *q) {
     if (!impl_)
         return Status(TNNERR_INIT_LAYER, "blob converter is nil, check device type");
@@ -960,6 +963,7 @@ BaseLayer *CreateLayer(LayerType type) {
 
 // ---- optimizer manager (source/tnn/optimizer/net_optimizer_manager.cc:33-48) -----------------------
 namespace {
+using optimizer::NetOptimizer;
 std::vector<std::pair<int, std::shared_ptr<NetOptimizer>>> &OptimizerList() {
     static std::vector<std::pair<int, std::shared_ptr<NetOptimizer>>> v;
     return v;
@@ -1033,15 +1037,15 @@ public:
         return TNN_OK;
     }
 };
-struct RegisterBuiltins {
-    RegisterBuiltins() { RegisterNetOptimizer(2, std::make_shared<InsertInt8Reformat>()); }
-} g_register_builtins;
+// net_optimizer_insert_int8_reformat.cc:34
+optimizer::NetOptimizerRegister<InsertInt8Reformat> g_net_optimizer_insert_int8_reformat(optimizer::P2);
 }  // namespace
 
-void RegisterNetOptimizer(int priority, std::shared_ptr<NetOptimizer> opt) {
-    OptimizerList().push_back({priority, opt});
+void optimizer::NetOptimizerManager::RegisterNetOptimizer(NetOptimizer *opt, OptPriority prior) {
+    if (opt && opt->Strategy().length() > 0)
+        OptimizerList().push_back({(int)prior, std::shared_ptr<NetOptimizer>(opt)});
 }
-Status RunNetOptimizers(NetStructure *structure, NetResource *resource, const NetworkConfig &config) {
+Status optimizer::NetOptimizerManager::Optimize(NetStructure *structure, NetResource *resource, const NetworkConfig &config) {
     std::lock_guard<std::mutex> lock(g_optimize_mutex);
     auto list = OptimizerList();
     std::stable_sort(list.begin(), list.end(), [](const std::pair<int, std::shared_ptr<NetOptimizer>> &a,
@@ -1065,7 +1069,6 @@ DefaultNetwork::~DefaultNetwork() {
     if (device_)
         for (void *p : allocations_)
             device_->Free(p);
-    DropGraphs();
     for (auto &e : prof_events_) {
         tnn_rocm_event_destroy(e.first);
         tnn_rocm_event_destroy(e.second);
@@ -1091,14 +1094,12 @@ Status DefaultNetwork::Plan(NetworkConfig &net_config, ModelInterpreter *interpr
             return Status(TNNERR_PARAM_ERR, "input shape given for " + kv.first + " has another number of dimensions than the model's");
         it->second = kv.second;
     }
-    RETURN_ON_NEQ(RunNetOptimizers(&structure_, &resource_, config_), TNN_OK);
+    RETURN_ON_NEQ(optimizer::NetOptimizerManager::Optimize(&structure_, &resource_, config_), TNN_OK);
     return InitLayers();  // context_ stays null: shapes and types only
 }
 
 Status DefaultNetwork::Init(NetworkConfig &net_config, ModelInterpreter *interpreter, const InputShapesMap &max_inputs_shape) {
     config_ = net_config;
-    if (const char *g = getenv("TNN_ROCM_GRAPH"))
-        graph_enabled_ = atoi(g) != 0;
     device_ = GetDevice(net_config.device_type);
     if (!device_)  // instance.cc:60-62
         return Status(TNNERR_DEVICE_NOT_SUPPORT, "device not support");
@@ -1121,7 +1122,7 @@ Status DefaultNetwork::Init(NetworkConfig &net_config, ModelInterpreter *interpr
             return Status(TNNERR_PARAM_ERR, "input shape given for " + kv.first + " has another number of dimensions than the model's");
         it->second = kv.second;
     }
-    RETURN_ON_NEQ(RunNetOptimizers(&structure_, &resource_, config_), TNN_OK);
+    RETURN_ON_NEQ(optimizer::NetOptimizerManager::Optimize(&structure_, &resource_, config_), TNN_OK);
     RETURN_ON_NEQ(InitLayers(), TNN_OK);
     RETURN_ON_NEQ(AllocateBlobMemory(), TNN_OK);
     RETURN_ON_NEQ(context_->OnInstanceReshapeBegin(), TNN_OK);
@@ -1130,22 +1131,6 @@ Status DefaultNetwork::Init(NetworkConfig &net_config, ModelInterpreter *interpr
     return context_->OnInstanceReshapeEnd();
 }
 
-std::string DefaultNetwork::ShapeKey() const {
-    std::ostringstream os;
-    for (auto &kv : inputs_) {
-        os << kv.first << ":";
-        for (int d : kv.second->GetBlobDesc().dims)
-            os << d << ",";
-        os << ";";
-    }
-    return os.str();
-}
-void DefaultNetwork::DropGraphs() {
-    for (auto &g : graphs_)
-        tnn_rocm_graph_destroy(g.second);
-    graphs_.clear();
-    graph_exec_ = nullptr;
-}
 Status DefaultNetwork::ReleaseBlobMemory() {
     RETURN_ON_NEQ(context_->Synchronize(), TNN_OK);
     for (auto &kv : blob_capacity_)
@@ -1179,8 +1164,6 @@ Status DefaultNetwork::Reshape(const InputShapesMap &inputs) {
         return TNN_OK;
     // nothing of the old shape may still be running when blobs change size or move
     RETURN_ON_NEQ(context_->Synchronize(), TNN_OK);
-    graph_exec_     = nullptr;
-    eager_forwards_ = 0;
     RETURN_ON_NEQ(context_->OnInstanceReshapeBegin(), TNN_OK);
     // shapes first (layer order = topological order), then memory, then the accs, which may look at the blobs' memory
     for (size_t i = 0; i < layers_.size(); ++i) {
@@ -1194,7 +1177,6 @@ Status DefaultNetwork::Reshape(const InputShapesMap &inputs) {
         fits &= GetBlobMemoryBytesSize(info) <= kv.second;
     }
     if (!fits) {
-        DropGraphs();  // they point into the buffers that go away now
         RETURN_ON_NEQ(ReleaseBlobMemory(), TNN_OK);
         RETURN_ON_NEQ(AllocateBlobMemory(), TNN_OK);
     }
@@ -1203,11 +1185,7 @@ Status DefaultNetwork::Reshape(const InputShapesMap &inputs) {
         if (st != TNN_OK)
             return Status((int)st, "reshape of layer " + layers_[i]->GetLayerName() + " failed: " + st.description());
     }
-    RETURN_ON_NEQ(context_->OnInstanceReshapeEnd(), TNN_OK);
-    auto g = graphs_.find(ShapeKey());
-    if (g != graphs_.end() && graphs_epoch_ == context_->MemoryEpoch())
-        graph_exec_ = g->second;
-    return TNN_OK;
+    return context_->OnInstanceReshapeEnd();
 }
 
 Blob *DefaultNetwork::GetBlob(const std::string &name) {
@@ -1469,52 +1447,13 @@ Status DefaultNetwork::RunLayers(void *prof_stream) {
     return TNN_OK;
 }
 
-// The layer loop of default_network.cc:571-631.  On DEVICE_ROCM the sequence of launches of a forward pass is
-// fixed once the instance is initialised (static shapes, stable blob/workspace addresses), so after two eager
-// passes (which also perform every lazy allocation) the third is recorded into an executable graph and later calls
-// replay it with a single submission; per-layer profiling and TNN_ROCM_GRAPH=0 keep the eager loop.
-Status DefaultNetwork::ForwardAsync() {
+// The layer loop of default_network.cc:571-631 (ForwardAsync: :672-686), with the per-layer event timing of the
+// profile hook.
+Status DefaultNetwork::ForwardAsync(Callback) {
     RETURN_ON_NEQ(context_->OnInstanceForwardBegin(), TNN_OK);
     void *stream = nullptr;
     context_->GetCommandQueue(&stream);
-    const bool use_graph = graph_enabled_ && !profiling_ && config_.device_type == DEVICE_ROCM && stream != nullptr;
-    if (graph_exec_ && graphs_epoch_ != context_->MemoryEpoch())
-        DropGraphs();  // context scratch moved since the recordings were made
-    if (use_graph && graph_exec_) {
-        if (tnn_rocm_graph_launch(graph_exec_, stream) != 0)
-            return Status(TNNERR_CUDA_KERNEL_LAUNCH_ERROR, std::string("graph launch failed: ") + tnn_rocm_last_error());
-        return context_->OnInstanceForwardEnd();
-    }
-    if (use_graph && eager_forwards_ >= 2) {
-        if (tnn_rocm_graph_begin_capture(stream) == 0) {
-            Status st = RunLayers(nullptr);
-            void *exec = nullptr;
-            int rc     = tnn_rocm_graph_end_capture(stream, &exec);
-            if (st != TNN_OK) {
-                tnn_rocm_graph_destroy(exec);
-                return st;
-            }
-            if (rc == 0 && exec) {
-                if (graphs_epoch_ != context_->MemoryEpoch())
-                    DropGraphs();
-                graphs_epoch_ = context_->MemoryEpoch();
-                auto key      = ShapeKey();
-                if (graphs_.count(key))
-                    tnn_rocm_graph_destroy(graphs_[key]);
-                graphs_[key] = exec;
-                graph_exec_  = exec;
-                if (tnn_rocm_graph_launch(graph_exec_, stream) != 0)
-                    return Status(TNNERR_CUDA_KERNEL_LAUNCH_ERROR,
-                                  std::string("graph launch failed: ") + tnn_rocm_last_error());
-                return context_->OnInstanceForwardEnd();
-            }
-            graph_enabled_ = false;  // capture not possible for this graph of layers: stay eager
-        } else {
-            graph_enabled_ = false;
-        }
-    }
     RETURN_ON_NEQ(RunLayers(stream), TNN_OK);
-    ++eager_forwards_;
     if (profiling_) {
         for (size_t i = 0; i < layers_.size(); ++i) {
             float ms = 0;
@@ -1529,9 +1468,27 @@ Status DefaultNetwork::ForwardAsync() {
     return context_->OnInstanceForwardEnd();
 }
 Status DefaultNetwork::Forward() {
-    RETURN_ON_NEQ(ForwardAsync(), TNN_OK);
+    RETURN_ON_NEQ(DefaultNetwork::ForwardAsync(nullptr), TNN_OK);
     return context_->Synchronize();
 }
+// core/abstract_network.cc:24-45
+namespace {
+std::map<NetworkType, std::shared_ptr<AbstractNetworkImplFactory>> &NetworkImplFactoryMap() {
+    static std::map<NetworkType, std::shared_ptr<AbstractNetworkImplFactory>> m;
+    return m;
+}
+NetworkImplFactoryRegister<NetworkImplFactory<DefaultNetwork>> g_network_impl_default_factory_register(NETWORK_TYPE_DEFAULT);
+}  // namespace
+std::shared_ptr<DefaultNetwork> NetworkImplManager::GetNetworkImpl(NetworkType type) {
+    auto &m = NetworkImplFactoryMap();
+    auto it = m.find(type);
+    return it == m.end() ? nullptr : it->second->CreateNetworkImp();
+}
+void NetworkImplManager::RegisterNetworkImplFactory(NetworkType type, AbstractNetworkImplFactory *factory) {
+    if (factory)
+        NetworkImplFactoryMap()[type] = std::shared_ptr<AbstractNetworkImplFactory>(factory);
+}
+
 Status DefaultNetwork::GetCommandQueue(void **q) { return context_->GetCommandQueue(q); }
 Status DefaultNetwork::GetAllInputBlobs(BlobMap &blobs) {
     blobs = inputs_;
@@ -1611,7 +1568,9 @@ Status Instance::Init(const InputShapesMap &, const InputShapesMap &max_inputs_s
         return Status(TNNERR_DEVICE_NOT_SUPPORT, "device not support");
     if (net_config_.network_type == NETWORK_TYPE_AUTO)
         net_config_.network_type = device->ConvertAutoNetworkType();
-    network_ = std::make_shared<DefaultNetwork>();
+    network_ = NetworkImplManager::GetNetworkImpl(net_config_.network_type);  // instance.cc:75-85
+    if (!network_)
+        return Status(TNNERR_NET_ERR, "network_ is nil, network_type may not support");
     return network_->Init(net_config_, interpreter_.get(), max_inputs_shape);
 }
 Status Instance::Reshape(const InputShapesMap &inputs) {
@@ -1621,8 +1580,8 @@ Status Instance::Reshape(const InputShapesMap &inputs) {
     return network_->Reshape(inputs);
 }
 Status Instance::Forward() { return network_ ? network_->Forward() : Status(TNNERR_INST_ERR, "instance not initialised"); }
-Status Instance::ForwardAsync() {
-    return network_ ? network_->ForwardAsync() : Status(TNNERR_INST_ERR, "instance not initialised");
+Status Instance::ForwardAsync(Callback call_back) {
+    return network_ ? network_->ForwardAsync(call_back) : Status(TNNERR_INST_ERR, "instance not initialised");
 }
 Status Instance::GetCommandQueue(void **q) { return network_->GetCommandQueue(q); }
 Status Instance::GetAllInputBlobs(BlobMap &b) { return network_->GetAllInputBlobs(b); }

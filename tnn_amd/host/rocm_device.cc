@@ -424,13 +424,7 @@ private:
     size_t staging_sz_ = 0;
 };
 
-class RocmBlobConverterAccCreater : public BlobConverterAccCreater {
-    std::shared_ptr<BlobConverterAcc> CreateBlobConverterAcc(Blob *blob) override {
-        return std::make_shared<RocmBlobConverterAcc>(blob);
-    }
-};
-static struct RegisterRocmConverter {
-    RegisterRocmConverter() { GetBlobConverterCreaterMap()[DEVICE_ROCM] = std::make_shared<RocmBlobConverterAccCreater>(); }
-} g_register_rocm_converter;
+DECLARE_BLOB_CONVERTER_CREATER(Rocm);
+REGISTER_BLOB_CONVERTER(Rocm, DEVICE_ROCM);
 
 }  // namespace TNN_NS

@@ -9,7 +9,24 @@
 #ifndef TNN_AMD_HOST_ROCM_DEVICE_H_
 #define TNN_AMD_HOST_ROCM_DEVICE_H_
 
+#ifdef TNN_ROCM_ENGINE_TREE
+// inside the engine tree: the engine's own headers, plus the additions this backend needs from the engine
+// (DEVICE_ROCM, the fused layer types with their params / resources)
+#include "tnn/core/abstract_device.h"
+#include "tnn/core/abstract_layer_acc.h"
+#include "tnn/core/blob_int8.h"
+#include "tnn/core/context.h"
+#include "tnn/interpreter/layer_param.h"
+#include "tnn/interpreter/layer_resource.h"
+#include "tnn/optimizer/net_optimizer.h"
+#include "tnn/optimizer/net_optimizer_manager.h"
+#include "tnn/utils/blob_converter_internal.h"
+#include "tnn/utils/data_type_utils.h"
+#include "tnn/utils/dims_utils.h"
+#include "rocm_engine_additions.h"
+#else
 #include "tnn_host.h"
+#endif
 #include "tnn_rocm.h"
 
 namespace TNN_NS {
@@ -33,7 +50,9 @@ public:
     Status OnInstanceForwardBegin() override;
     Status OnInstanceForwardEnd() override { return TNN_OK; }
     Status Synchronize() override;
-    uint64_t MemoryEpoch() const override { return memory_epoch_; }
+    // Counts the (re)allocations of device memory the context owns (scratch that grows with the shapes).  A recorded
+    // launch sequence holds raw pointers into that memory, so RocmNetwork only replays it while this number stands still.
+    uint64_t MemoryEpoch() const { return memory_epoch_; }
 
     void *Stream() { return stream_; }
     // grow-only scratch owned by the context; valid until the next call with a larger size
@@ -74,7 +93,8 @@ public:
     AbstractLayerAcc *CreateLayerAcc(LayerType type) override;
     Context *CreateContext(int device_id) override;
     std::shared_ptr<const ImplementedPrecision> GetImplementedPrecision(LayerType type) override;
-    NetworkType ConvertAutoNetworkType() override { return NETWORK_TYPE_DEFAULT; }
+    // RocmNetwork (rocm_network.h): DefaultNetwork plus whole-forward graph replay
+    NetworkType ConvertAutoNetworkType() override { return NETWORK_TYPE_ROCM; }
     static Status RegisterLayerAccCreator(LayerType type, LayerAccCreator *creator);
 
 private:

@@ -1,0 +1,91 @@
+// What DEVICE_ROCM adds to the engine's own vocabulary: the device / network type constants, the layer types the
+// ROCm optimizer passes produce, and their params and resources.
+//
+// Included after the engine's headers (include/tnn/core/common.h, source/tnn/core/layer_type.h,
+// source/tnn/interpreter/layer_param.h, layer_resource.h) inside the engine tree, and after this repository's own
+// restatement of them otherwise, so the backend sources read the same in both builds.  The engine's enums are closed
+// (include/tnn/core/common.h:88-116, source/tnn/core/layer_type.h:25-260), so the new values are typed constants
+// outside every range the engine uses; a maintainer who prefers enumerators moves them into the enums and deletes
+// the constants here, nothing else changes.
+#ifndef TNN_AMD_HOST_ROCM_ENGINE_ADDITIONS_H_
+#define TNN_AMD_HOST_ROCM_ENGINE_ADDITIONS_H_
+
+namespace TNN_NS {
+
+// include/tnn/core/common.h:103-115 (DeviceType), :90-100 (NetworkType)
+constexpr DeviceType DEVICE_ROCM        = static_cast<DeviceType>(0x1080);
+constexpr NetworkType NETWORK_TYPE_ROCM = static_cast<NetworkType>(0x9000);
+
+// produced only by the ROCm optimizer passes (no proto spelling, so no layer interpreter)
+constexpr LayerType LAYER_ROCM_FUSED_LINEAR      = static_cast<LayerType>(0x7001);
+constexpr LayerType LAYER_ROCM_FUSED_ATTENTION   = static_cast<LayerType>(0x7002);
+constexpr LayerType LAYER_ROCM_FUSED_LINEAR_INT8 = static_cast<LayerType>(0x7003);
+constexpr LayerType LAYER_ROCM_GELU_INT8         = static_cast<LayerType>(0x7004);
+constexpr LayerType LAYER_ROCM_FUSED_EMBEDDING   = static_cast<LayerType>(0x7005);
+constexpr LayerType LAYER_ROCM_QUANT_LINEAR_GELU = static_cast<LayerType>(0x7006);
+
+struct RocmFusedLinearResource : public LayerResource {
+    RawBuffer weight_nk;  // [N, K] fp32
+    RawBuffer bias;       // [N] fp32 (may be empty)
+    // scale / shift ([K] fp32) of a LayerNorm folded into this layer (the one whose output was the A operand)
+    RawBuffer ln_gamma, ln_beta;
+};
+
+struct RocmFusedLinearParam : public LayerParam {
+    int num_output   = 0;
+    int has_bias     = 0;
+    int gelu         = 0;  // erf GELU applied to (x W^T + b)
+    int has_residual = 0;  // second input added after the activation
+    int axis         = -1; // -1: contract the last dimension; >= 0: InnerProduct form, contract dims[axis:]
+    // LayerNorm folded into this projection (RocmFusionPass::FoldLayerNorm): input 0 is the tensor the LayerNorm
+    // read, the layer computes act(LayerNorm(x) W^T + b); with ln_y a second output blob receives LayerNorm(x)
+    // itself for the other readers of that tensor.
+    int ln_fold = 0, ln_y = 0;
+    float ln_eps = 0.f;
+};
+struct RocmFusedAttentionParam : public LayerParam {
+    int heads    = 0;
+    int head_dim = 0;
+    float scale  = 1.0f;
+    int has_mask = 0;  // second input: additive mask broadcastable to [B,1,1,S]
+    int seq_len  = 0;  // S of the matched head split ([B,S,h,d]); 0 = take it from the input blob's shape
+    // quantised form: the first input is the int8 blob the three QuantizedInnerProduct projections read, the
+    // resource is a RocmFusedQkvInt8Resource and qkv_out_scale are the scales of their three int8 output blobs
+    int quant = 0;
+    float qkv_out_scale[3] = {0.f, 0.f, 0.f};
+    // LayerNorm folded into the QKV projection, as in RocmFusedLinearParam
+    int ln_fold = 0, ln_y = 0;
+    float ln_eps = 0.f;
+    // the last output blob is int8: the context quantised as the Reformat layer that followed would (ROCm int8 pass)
+    int out_quant = 0;
+};
+// Gather(word ids) + Add(position constant) + Gather(type ids) + Add + LayerNorm of a BERT-style front end.
+// Inputs: word ids, type ids (int32), gamma, beta (constant blobs); resource: RocmFusedEmbeddingResource.
+struct RocmFusedEmbeddingParam : public LayerParam {
+    float eps = 1e-5f;
+};
+struct RocmFusedEmbeddingResource : public LayerResource {
+    RawBuffer word;  // [vocab, H]
+    RawBuffer type;  // [types, H]
+    RawBuffer pos;   // [S, H]: the constant added to the word rows, one row per position
+};
+// QuantizedInnerProduct whose int8 result is consumed as float: y = q * out_scale (+ residual), q never stored.
+// Input 0 is the int8 blob, input 1 (has_residual) a float blob of the output's shape; the output is float.
+struct RocmFusedLinearInt8Param : public InnerProductLayerParam {
+    float out_scale  = 0.f;  // scale of the int8 blob the original layer produced
+    int has_residual = 0;
+};
+// QuantizedInnerProduct whose int8 result went through Reformat -> GELU -> Reformat: the projection applies that
+// int8 -> int8 map as a 256-entry table in its epilogue.  mid_scale is the scale of the int8 blob the projection used
+// to write; the output blob is the one the second Reformat wrote.
+struct RocmQuantLinearGeluParam : public InnerProductLayerParam {
+    float mid_scale = 0.f;
+};
+struct RocmFusedQkvInt8Resource : public LayerResource {
+    RawBuffer weight;   // int8 [3H, K]
+    RawBuffer bias;     // int32 [3H] (may be empty)
+    RawBuffer w_scale;  // fp32 [3H] per-output-channel weight scales
+};
+
+}  // namespace TNN_NS
+#endif

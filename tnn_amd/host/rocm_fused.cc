@@ -45,7 +45,7 @@ struct GraphIndex {
     }
 };
 
-class RocmFusionPass : public NetOptimizer {
+class RocmFusionPass : public optimizer::NetOptimizer {
 public:
     std::string Strategy() override { return "net_optimizer_rocm_fuse_encoder"; }
     bool IsSupported(const NetworkConfig &c) override {
@@ -582,7 +582,7 @@ private:
 // Each fused kernel forms the same int8 values as the chain it replaces (requantisation and quantisation are the
 // reference's float2int8 steps); float intermediates that the chain would have rounded to the blob type (fp16 nets)
 // stay in fp32 inside the fused kernel.
-class RocmInt8FusionPass : public NetOptimizer {
+class RocmInt8FusionPass : public optimizer::NetOptimizer {
 public:
     std::string Strategy() override { return "net_optimizer_rocm_fuse_int8"; }
     bool IsSupported(const NetworkConfig &c) override {
@@ -985,12 +985,11 @@ private:
     bool half_               = true;
 };
 
-struct RegisterRocmFusion {
-    RegisterRocmFusion() {
-        RegisterNetOptimizer(1, std::make_shared<RocmFusionPass>());
-        RegisterNetOptimizer(3, std::make_shared<RocmInt8FusionPass>());  // after the Reformat insertion (2)
-    }
-} g_register_rocm_fusion;
+// optimizer/net_optimizer_manager.cc:33-48 runs the passes sorted by (priority, strategy name): the float rewrite runs
+// with the engine's own fusions (P1); the int8 rewrite needs the Reformat layers, so it shares P2 with
+// net_optimizer_insert_int8_reformat and its strategy name sorts behind that one
+optimizer::NetOptimizerRegister<RocmFusionPass> g_net_optimizer_rocm_fuse_encoder(optimizer::P1);
+optimizer::NetOptimizerRegister<RocmInt8FusionPass> g_net_optimizer_rocm_fuse_int8(optimizer::P2);
 
 }  // namespace
 

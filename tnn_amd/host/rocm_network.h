@@ -1,0 +1,42 @@
+// RocmNetwork: the engine's DefaultNetwork plus whole-forward graph replay.
+//
+// On this device the launches of a forward pass are fixed once the instance is initialised (static shapes, stable
+// blob and workspace addresses), so after two eager passes - which also perform every lazy allocation - the third is
+// recorded into an executable graph and later calls submit it at once.  The engine picks the network implementation
+// per NetworkType (source/tnn/core/abstract_network.h:102-136, instance.cc:75-85); RocmDevice::ConvertAutoNetworkType()
+// names this one, and it registers itself like the engine's other networks (default_network.cc:39-40).
+#ifndef TNN_AMD_HOST_ROCM_NETWORK_H_
+#define TNN_AMD_HOST_ROCM_NETWORK_H_
+
+#include "rocm_device.h"
+#ifdef TNN_ROCM_ENGINE_TREE
+#include "tnn/core/default_network.h"
+#endif
+
+namespace TNN_NS {
+
+class RocmNetwork : public DefaultNetwork {
+public:
+    RocmNetwork();
+    ~RocmNetwork() override;
+    Status Forward() override;
+    Status ForwardAsync(Callback call_back) override;
+
+private:
+    // Everything a recording depends on: dims and device address of every blob the layers touch, and the context's
+    // scratch allocation count.  A recording is replayed only under the signature it was made with, so a Reshape, a
+    // re-planned blob pool or a grown workspace lead back to eager passes and a new recording by themselves.
+    void Signature(std::vector<uint64_t> *sig);
+    void DropGraphs();
+    struct Recording {
+        std::vector<uint64_t> signature;
+        void *exec = nullptr;
+    };
+    std::vector<Recording> recordings_;
+    std::vector<uint64_t> eager_signature_;
+    int eager_forwards_ = 0;
+    bool enabled_       = true;  // TNN_ROCM_GRAPH=0 keeps the eager loop
+};
+
+}  // namespace TNN_NS
+#endif

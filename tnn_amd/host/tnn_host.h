@@ -136,9 +136,7 @@ typedef enum {
     DEVICE_X86   = 0x0010,
     DEVICE_ARM   = 0x0020,
     DEVICE_CUDA  = 0x1020,
-    // new enumerator for this backend; the value the integration note proposes for common.h
-    DEVICE_ROCM = 0x1080,
-} DeviceType;
+} DeviceType;  // DEVICE_ROCM is added by rocm_engine_additions.h, as it is inside the engine tree
 
 typedef enum { MODEL_TYPE_TNN = 0x0001 } ModelType;
 
@@ -159,7 +157,7 @@ typedef enum {
 using DimsVector = std::vector<int>;
 
 struct NetworkConfig {
-    DeviceType device_type   = DEVICE_ROCM;
+    DeviceType device_type   = DEVICE_ARM;  // include/tnn/core/common.h:148
     int device_id            = 0;
     DataFormat data_format   = DATA_FORMAT_AUTO;
     NetworkType network_type = NETWORK_TYPE_AUTO;
@@ -271,14 +269,6 @@ struct IntScaleResource : public LayerResource {
     RawBuffer zero_point_handle;
     RawBuffer bias_handle;
 };
-// fused layers produced by the ROCm optimizer pass
-struct RocmFusedLinearResource : public LayerResource {
-    RawBuffer weight_nk;  // [N, K] fp32
-    RawBuffer bias;       // [N] fp32 (may be empty)
-    // scale / shift ([K] fp32) of a LayerNorm folded into this layer (the one whose output was the A operand)
-    RawBuffer ln_gamma, ln_beta;
-};
-
 using ConstantResource = std::map<std::string, std::shared_ptr<RawBuffer>>;
 
 class BlobInt8 : public Blob {
@@ -312,13 +302,6 @@ enum LayerType {
     LAYER_LAYER_NORM    = 326,
     LAYER_GELU          = 327,
     LAYER_BLOB_SCALE    = 600,
-    // produced only by the ROCm optimizer pass (no proto spelling in the engine)
-    LAYER_ROCM_FUSED_LINEAR      = 0x7001,
-    LAYER_ROCM_FUSED_ATTENTION   = 0x7002,
-    LAYER_ROCM_FUSED_LINEAR_INT8 = 0x7003,
-    LAYER_ROCM_GELU_INT8         = 0x7004,
-    LAYER_ROCM_FUSED_EMBEDDING = 0x7005,
-    LAYER_ROCM_QUANT_LINEAR_GELU = 0x7006,
 };
 LayerType GlobalConvertLayerType(std::string type_str);
 
@@ -380,62 +363,6 @@ struct GatherLayerParam : public LayerParam {
     bool data_in_resource    = false;
     bool indices_in_resource = true;
 };
-struct RocmFusedLinearParam : public LayerParam {
-    int num_output   = 0;
-    int has_bias     = 0;
-    int gelu         = 0;  // erf GELU applied to (x W^T + b)
-    int has_residual = 0;  // second input added after the activation
-    int axis         = -1; // -1: contract the last dimension; >= 0: InnerProduct form, contract dims[axis:]
-    // LayerNorm folded into this projection (RocmFusionPass::FoldLayerNorm): input 0 is the tensor the LayerNorm
-    // read, the layer computes act(LayerNorm(x) W^T + b); with ln_y a second output blob receives LayerNorm(x)
-    // itself for the other readers of that tensor.
-    int ln_fold = 0, ln_y = 0;
-    float ln_eps = 0.f;
-};
-struct RocmFusedAttentionParam : public LayerParam {
-    int heads    = 0;
-    int head_dim = 0;
-    float scale  = 1.0f;
-    int has_mask = 0;  // second input: additive mask broadcastable to [B,1,1,S]
-    int seq_len  = 0;  // S of the matched head split ([B,S,h,d]); 0 = take it from the input blob's shape
-    // quantised form: the first input is the int8 blob the three QuantizedInnerProduct projections read, the
-    // resource is a RocmFusedQkvInt8Resource and qkv_out_scale are the scales of their three int8 output blobs
-    int quant = 0;
-    float qkv_out_scale[3] = {0.f, 0.f, 0.f};
-    // LayerNorm folded into the QKV projection, as in RocmFusedLinearParam
-    int ln_fold = 0, ln_y = 0;
-    float ln_eps = 0.f;
-    // the last output blob is int8: the context quantised as the Reformat layer that followed would (ROCm int8 pass)
-    int out_quant = 0;
-};
-// Gather(word ids) + Add(position constant) + Gather(type ids) + Add + LayerNorm of a BERT-style front end.
-// Inputs: word ids, type ids (int32), gamma, beta (constant blobs); resource: RocmFusedEmbeddingResource.
-struct RocmFusedEmbeddingParam : public LayerParam {
-    float eps = 1e-5f;
-};
-struct RocmFusedEmbeddingResource : public LayerResource {
-    RawBuffer word;  // [vocab, H]
-    RawBuffer type;  // [types, H]
-    RawBuffer pos;   // [S, H]: the constant added to the word rows, one row per position
-};
-// QuantizedInnerProduct whose int8 result is consumed as float: y = q * out_scale (+ residual), q never stored.
-// Input 0 is the int8 blob, input 1 (has_residual) a float blob of the output's shape; the output is float.
-struct RocmFusedLinearInt8Param : public InnerProductLayerParam {
-    float out_scale  = 0.f;  // scale of the int8 blob the original layer produced
-    int has_residual = 0;
-};
-// QuantizedInnerProduct whose int8 result went through Reformat -> GELU -> Reformat: the projection applies that
-// int8 -> int8 map as a 256-entry table in its epilogue.  mid_scale is the scale of the int8 blob the projection used
-// to write; the output blob is the one the second Reformat wrote.
-struct RocmQuantLinearGeluParam : public InnerProductLayerParam {
-    float mid_scale = 0.f;
-};
-struct RocmFusedQkvInt8Resource : public LayerResource {
-    RawBuffer weight;   // int8 [3H, K]
-    RawBuffer bias;     // int32 [3H] (may be empty)
-    RawBuffer w_scale;  // fp32 [3H] per-output-channel weight scales
-};
-
 struct LayerInfo {
     LayerType type = LAYER_NOT_SUPPORT;
     std::string type_str;
@@ -492,9 +419,6 @@ public:
     virtual Status OnInstanceReshapeEnd() { return TNN_OK; }
     virtual Status Synchronize() = 0;
     virtual Status SetNumThreads(int) { return TNN_OK; }
-    // Counts the (re)allocations of device memory the context owns (scratch that grows with the shapes).  A recorded
-    // launch sequence holds raw pointers into that memory, so it is only replayed while this number stands still.
-    virtual uint64_t MemoryEpoch() const { return 0; }
     void SetPrecision(Precision p) { precision_ = p; }
     Precision GetPrecision() { return precision_; }
 
@@ -617,7 +541,33 @@ public:
     virtual ~BlobConverterAccCreater() {}
     virtual std::shared_ptr<BlobConverterAcc> CreateBlobConverterAcc(Blob *blob) = 0;
 };
-std::map<DeviceType, std::shared_ptr<BlobConverterAccCreater>> &GetBlobConverterCreaterMap();
+// utils/blob_converter_internal.h:46-81: the per-device creator registry and its registration macros
+class BlobConverterManager {
+public:
+    static std::shared_ptr<BlobConverterManager> &Shared();
+    std::shared_ptr<BlobConverterAcc> CreateBlobConverterAcc(Blob *blob);
+    int RegisterBlobConverterAccCreater(DeviceType type, std::shared_ptr<BlobConverterAccCreater> creater);
+
+private:
+    std::map<DeviceType, std::shared_ptr<BlobConverterAccCreater>> converter_creater_map_;
+};
+template <typename T> class BlobConverterAccRegister {
+public:
+    explicit BlobConverterAccRegister(DeviceType type) {
+        BlobConverterManager::Shared()->RegisterBlobConverterAccCreater(type, std::make_shared<T>());
+    }
+};
+#define DECLARE_BLOB_CONVERTER_CREATER(device)                                                                        \
+    class device##BlobConverterAccCreater : public BlobConverterAccCreater {                                          \
+    public:                                                                                                           \
+        virtual ~device##BlobConverterAccCreater() {}                                                                 \
+        virtual std::shared_ptr<BlobConverterAcc> CreateBlobConverterAcc(Blob *blob) {                                \
+            return std::make_shared<device##BlobConverterAcc>(blob);                                                  \
+        }                                                                                                             \
+    }
+#define REGISTER_BLOB_CONVERTER(device, device_type)                                                                  \
+    BlobConverterAccRegister<device##BlobConverterAccCreater> g_blob_converter_##device(device_type)
+
 class BlobConverter {
 public:
     explicit BlobConverter(Blob *blob);
@@ -653,7 +603,8 @@ protected:
 };
 BaseLayer *CreateLayer(LayerType type);
 
-// ---- optimizer passes -------------------------------------------------------------------------
+// ---- optimizer passes (optimizer/net_optimizer.h:25-37, net_optimizer_manager.h:32-66) -------------
+namespace optimizer {
 class NetOptimizer {
 public:
     virtual ~NetOptimizer() {}
@@ -661,8 +612,18 @@ public:
     virtual bool IsSupported(const NetworkConfig &net_config)                = 0;
     virtual Status Optimize(NetStructure *structure, NetResource *resource)  = 0;
 };
-void RegisterNetOptimizer(int priority, std::shared_ptr<NetOptimizer> opt);
-Status RunNetOptimizers(NetStructure *structure, NetResource *resource, const NetworkConfig &config);
+typedef enum { P0 = 0, P1 = 1, P2 = 2, PLAST = 1000 } OptPriority;
+class NetOptimizerManager {
+public:
+    // passes run in priority order, passes of one priority in the order of their strategy names
+    static Status Optimize(NetStructure *structure, NetResource *resource, const NetworkConfig &net_config);
+    static void RegisterNetOptimizer(NetOptimizer *optimizer, OptPriority prior);
+};
+template <typename T> class NetOptimizerRegister {
+public:
+    explicit NetOptimizerRegister(OptPriority p) { NetOptimizerManager::RegisterNetOptimizer(new T(), p); }
+};
+}  // namespace optimizer
 
 // ---- network + instance -----------------------------------------------------------------------
 struct LayerProfile {
@@ -671,62 +632,83 @@ struct LayerProfile {
     int calls = 0;
 };
 
+typedef std::function<void(void)> Callback;  // include/tnn/core/common.h:207
+
+// core/default_network.h:37-160.  Forward, ForwardAsync, Reshape and the profile switches are virtual and the members
+// a derived network needs are protected, as in the engine, so a device can bring its own network (core/abstract_network.h:
+// 102-136: one factory per NetworkType, chosen by AbstractDevice::ConvertAutoNetworkType()).
 class DefaultNetwork {
 public:
-    ~DefaultNetwork();
+    DefaultNetwork() {}
+    virtual ~DefaultNetwork();
     // max_inputs_shape (may be empty: the model's own input shapes) is what the instance is created and its blob
     // memory planned at (instance.cc:48-128, default_network.cc:86-137)
-    Status Init(NetworkConfig &net_config, ModelInterpreter *interpreter, const InputShapesMap &max_inputs_shape = InputShapesMap());
+    virtual Status Init(NetworkConfig &net_config, ModelInterpreter *interpreter,
+                        const InputShapesMap &max_inputs_shape = InputShapesMap());
     // Everything Init does short of touching a device: the instance's copy of the graph is optimised, layers are
     // created (an unknown type or a type without an acc fails as in Init), blob types and shapes are inferred.  For
     // LayerSummary() / LayerIo() on a machine without a GPU.
     Status Plan(NetworkConfig &net_config, ModelInterpreter *interpreter, const InputShapesMap &inputs_shape = InputShapesMap());
     // default_network.cc:456-500: new dims for the named input blobs, then every layer infers its output shape again
     // and its acc is reshaped.  Weights stay on the device.  Blob memory is planned again only when a blob outgrows
-    // its buffer; recorded launch sequences are kept per input-shape signature.
-    Status Reshape(const InputShapesMap &inputs);
-    Status Forward();
-    Status ForwardAsync();
-    Status GetCommandQueue(void **command_queue);
-    Status GetAllInputBlobs(BlobMap &blobs);
-    Status GetAllOutputBlobs(BlobMap &blobs);
+    // its buffer.
+    virtual Status Reshape(const InputShapesMap &inputs);
+    virtual Status Forward();                           // default_network.cc:558-635: the layer loop, then Synchronize
+    virtual Status ForwardAsync(Callback call_back);    // default_network.cc:672-686: the layer loop alone
+    virtual Status GetCommandQueue(void **command_queue);
+    virtual Status GetAllInputBlobs(BlobMap &blobs);
+    virtual Status GetAllOutputBlobs(BlobMap &blobs);
     Blob *GetBlob(const std::string &name);
     int LayerCount() const { return (int)layers_.size(); }
     std::string LayerSummary() const;
     // one line per layer: name|input blob names (comma separated)|output blob names|input dims (d0,d1,..;d0,..)|output dims
     std::string LayerIo() const;
-    // per-layer hipEvent timing (the engine's TNN_PROFILE hook, source/tnn/core/profile.cc:111-201)
+    // per-layer event timing (the engine's TNN_PROFILE hook, source/tnn/core/profile.cc:111-201)
     // only layers whose type string equals `only_type` are timed when it is non-empty
-    void StartProfile(const std::string &only_type = "");
-    std::vector<LayerProfile> FinishProfile();
+    virtual void StartProfile(const std::string &only_type = "");
+    virtual std::vector<LayerProfile> FinishProfile();
 
-private:
-    Status InitLayers();
-    Status AllocateBlobMemory();
+protected:
+    virtual Status InitLayers();
+    virtual Status AllocateBlobMemory();
     Status ReleaseBlobMemory();
-    void DropGraphs();
-    std::string ShapeKey() const;
-    std::map<Blob *, int64_t> blob_capacity_;  // bytes behind each planned blob
-    std::map<std::string, void *> graphs_;     // recorded forward per input-shape signature
-    uint64_t graphs_epoch_ = 0;                // Context::MemoryEpoch() the recordings were made under
-    NetworkConfig config_;
     AbstractDevice *device_ = nullptr;
     Context *context_       = nullptr;
+    std::vector<BaseLayer *> layers_;
+    NetworkConfig config_;
+    bool profiling_ = false;
+
+private:
+    std::map<Blob *, int64_t> blob_capacity_;  // bytes behind each planned blob
     NetStructure structure_;  // per-instance copy: optimizer rewrites never touch the interpreter
     NetResource resource_;
     std::map<std::string, Blob *> blobs_;
-    std::vector<BaseLayer *> layers_;
     std::vector<void *> allocations_;
     BlobMap inputs_, outputs_;
-    bool profiling_ = false;
     std::vector<char> prof_on_;
-    // whole-forward graph replay (see ForwardAsync)
     Status RunLayers(void *prof_stream);
-    bool graph_enabled_  = true;
-    void *graph_exec_    = nullptr;
-    int eager_forwards_  = 0;
     std::vector<std::pair<void *, void *>> prof_events_;
     std::vector<LayerProfile> prof_;
+};
+
+// core/abstract_network.h:102-136
+class AbstractNetworkImplFactory {
+public:
+    virtual ~AbstractNetworkImplFactory() {}
+    virtual std::shared_ptr<DefaultNetwork> CreateNetworkImp() = 0;
+};
+template <typename T> class NetworkImplFactory : public AbstractNetworkImplFactory {
+public:
+    virtual std::shared_ptr<DefaultNetwork> CreateNetworkImp() { return std::make_shared<T>(); }
+};
+class NetworkImplManager {
+public:
+    static std::shared_ptr<DefaultNetwork> GetNetworkImpl(NetworkType type);
+    static void RegisterNetworkImplFactory(NetworkType type, AbstractNetworkImplFactory *factory);
+};
+template <typename T> class NetworkImplFactoryRegister {
+public:
+    explicit NetworkImplFactoryRegister(NetworkType type) { NetworkImplManager::RegisterNetworkImplFactory(type, new T()); }
 };
 
 class Instance {
@@ -738,7 +720,7 @@ public:
     Status Init(const InputShapesMap &min_inputs_shape, const InputShapesMap &max_inputs_shape);
     Status Reshape(const InputShapesMap &inputs);  // instance.cc:143-152
     Status Forward();
-    Status ForwardAsync();
+    Status ForwardAsync(Callback call_back);
     Status GetCommandQueue(void **command_queue);
     Status GetAllInputBlobs(BlobMap &blobs);
     Status GetAllOutputBlobs(BlobMap &blobs);
@@ -756,4 +738,6 @@ private:
 };
 
 }  // namespace TNN_NS
+
+#include "rocm_engine_additions.h"
 #endif
