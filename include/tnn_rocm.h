@@ -207,7 +207,9 @@ TNN_ROCM_API int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void 
                                             const float *beta, float eps, void *qk, void *vt, void *y, int B, int S,
                                             int heads, int K);
 
-/* kv_len[b] = 1 + the last key index whose additive mask value is > threshold (0 if none). */
+/* kv_len[b] = 1 + the last key index whose additive mask value is > threshold; S if there is none (a padding-only
+ * sequence: the reference's softmax(scores + mask) over all S keys is unchanged by the constant shift, so every key
+ * stays in, with its bias). */
 /* The _flagged form additionally sets bit 30 of kv_len[b] when mask[b][j] is exactly 0 for every j < kv_len[b] (a plain
  * padding mask): the attention kernels accept such entries and then do not read mask row b at all (the keys at and
  * beyond kv_len[b] are excluded by the length), which lets full key tiles take the path without a per-key bias. */

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import golden_util
-from test_gpu_ops import rel_err, say, FP16_TOL, FP32_TOL
+from test_gpu_ops import rel_err, say, FP16_TOL, FP32_TOL, FP32_ASSERT
 
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
@@ -42,7 +42,7 @@ def test_tiny_encoder_from_model_files(precision):
     got = inst.output("last_hidden")
     err = rel_err(got, f["naive_last_hidden"].reshape(got.shape))
     say("  max rel err %.3g" % err)
-    assert err <= (FP32_TOL if precision == "fp32" else FP16_TOL)
+    assert err <= (FP32_ASSERT if precision == "fp32" else FP16_TOL)
     if precision == "fp32":
         assert err <= 1e-4
         assert rel_err(inst.output("x0"), f["naive_x0"].reshape(inst.output("x0").shape)) <= 1e-5

@@ -16,7 +16,8 @@ import orc
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
 
-FP32_TOL = 2e-3
+FP32_TOL = 2e-3      # the bar stated for fp32 against the reference's CPU paths
+FP32_ASSERT = 5e-5   # what the fp32 cases assert: true-fp32 MFMA products, fp32 accumulation (observed <= 1e-5)
 FP16_TOL = 1e-2
 
 
@@ -98,6 +99,9 @@ def test_gelu_fp16():
     x = r16(rng.standard_normal(10001) * 3)
     got = host(ops().gelu(dev(x, torch.float16)))
     assert rel_err(got, orc.gelu(x)) <= 1e-3  # one fp16 rounding of the result
+    sp = np.array([0.0, np.inf, 40.0, -40.0, 65504.0, -65504.0], np.float32)
+    got = host(ops().gelu(dev(sp, torch.float16)))
+    assert got.tolist() == [0.0, np.inf, 40.0, 0.0, 65504.0, 0.0]
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 8), (5, 768), (33, 1024), (7, 100), (3, 5000), (4096, 768)])
@@ -816,6 +820,30 @@ def test_attention_vt_scores_that_outgrow_the_running_reference(dtype, tol):
     assert err2 <= tol
 
 
+def test_attention_padding_only_sequence_matches_the_reference_softmax():
+    """A sequence whose mask is -10000 on every key: the reference computes softmax(scores - 10000) V = softmax(scores) V
+    (in fp32 the shifted scores are quantised to 2^-10, which the fp16 bar absorbs); the kernel must do the same,
+    not write zeros."""
+    say("attention: padding-only sequence")
+    rng = np.random.default_rng(77)
+    B, S, h, d = 3, 136, 2, 64
+    H = h * d
+    q, k, v = (r16(rng.standard_normal((B, h, S, d))) for _ in range(3))
+    mask = np.zeros((B, S), np.float32)
+    mask[0, 100:] = -10000.0
+    mask[1, :] = -10000.0
+    mask[2, 17:] = -10000.0
+    ref = orc.attention_core(q, k, v, 0.125, mask).transpose(0, 2, 1, 3).reshape(B * S, H)
+    qt, kt, vt_ = (torch.from_numpy(t).half() for t in (q, k, v))
+    qk = torch.cat([qt.permute(0, 2, 1, 3).reshape(B * S, H), kt.permute(0, 2, 1, 3).reshape(B * S, H)], 1).contiguous()
+    vt = vt_.permute(0, 1, 3, 2).contiguous()
+    lens = ops().mask_to_kv_len(dev(mask), flagged=True)
+    out = host(ops().attention_qk_vt(qk.cuda(), vt.cuda(), B, S, h, 0.125, mask=dev(mask), kv_len=lens))
+    assert np.abs(out[S:2 * S]).max() > 0.01
+    assert rel_err(out, ref) <= FP16_TOL
+    assert rel_err(out[S:2 * S], ref[S:2 * S]) <= FP16_TOL
+
+
 def test_mask_to_kv_len():
     say("mask_to_kv_len")
     m = np.zeros((5, 300), np.float32)
@@ -824,6 +852,11 @@ def test_mask_to_kv_len():
         m[b, l:] = -10000.0
     got = host(ops().mask_to_kv_len(dev(m)))
     assert got.tolist() == lens
+    # a padding-only row keeps all its keys: the constant -10000 cancels in the reference's softmax
+    m0 = m.copy()
+    m0[1, :] = -10000.0
+    assert host(ops().mask_to_kv_len(dev(m0))).tolist() == [300, 300, 64, 65, 299]
+    assert host(ops().mask_to_kv_len(dev(m0), flagged=True)).tolist()[1] == 300  # not flagged: its bias is not zero
     # flagged form: bit 30 marks rows whose visible part is exactly zero; a row with any other visible value is not marked
     m[2, 5] = -0.5
     got = host(ops().mask_to_kv_len(dev(m), flagged=True))

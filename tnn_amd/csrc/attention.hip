@@ -797,7 +797,9 @@ __global__ void mask_to_kv_len_kernel(const float *__restrict__ mask, int32_t *_
         int other = __shfl_xor(last, o, 64);
         last      = other > last ? other : last;
     }
-    int len = last + 1;
+    // No key above the threshold: a padding-only sequence.  The reference still runs softmax(scores + mask) over all
+    // S keys, and a constant shift cancels there, so every key stays visible (with its bias) instead of none.
+    int len = last < 0 ? S : last + 1;
     if (flag_zero_rows) {
         // a plain padding mask is exactly 0 on every visible key: the attention kernel then needs the length only
         int nonzero = 0;

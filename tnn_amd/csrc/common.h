@@ -105,7 +105,7 @@ __device__ __forceinline__ float gelu_erf_fast(float x) {
     q             = fmaf(q, a, 1.1508630942e+00f);
     q             = fmaf(q, a, 1.0f);
     const float e = __builtin_amdgcn_exp2f(-q);  // Phi(-a)
-    return fmaf(-fabsf(x), e, fmaxf(x, 0.f));
+    return fmaf(-a, e, fmaxf(x, 0.f));  // the clamped a: a*Phi(-a) is below 1e-18 past 9, and +inf stays +inf
 }
 
 __device__ __forceinline__ float wave_sum(float v) {

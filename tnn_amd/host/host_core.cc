@@ -1607,8 +1607,11 @@ Status Instance::SetInputMat(std::shared_ptr<Mat> mat, MatConvertParam param, st
         return Status(TNNERR_INVALID_INPUT, "input mat element count differs from the input blob");
     void *q = nullptr;
     network_->GetCommandQueue(&q);
-    BlobConverter conv(blob);
-    return conv.ConvertFromMat(*mat, param, q);
+    // one converter per input for the life of the instance (instance.cc:228-235), so device staging is allocated once
+    auto &conv = input_converters_[blob->GetBlobDesc().name];
+    if (!conv.second || conv.first != blob)
+        conv = {blob, std::make_shared<BlobConverter>(blob)};
+    return conv.second->ConvertFromMat(*mat, param, q);
 }
 
 Status Instance::GetOutputMat(std::shared_ptr<Mat> &mat, MatConvertParam param, std::string output_name,
@@ -1632,8 +1635,10 @@ Status Instance::GetOutputMat(std::shared_ptr<Mat> &mat, MatConvertParam param, 
         cached = std::make_shared<Mat>(DEVICE_NAIVE, mat_type, blob->GetBlobDesc().dims);
     void *q = nullptr;
     network_->GetCommandQueue(&q);
-    BlobConverter conv(blob);
-    RETURN_ON_NEQ(conv.ConvertToMat(*cached, param, q), TNN_OK);
+    auto &conv = output_converters_[output_name];  // instance.cc:298-305
+    if (!conv.second || conv.first != blob)
+        conv = {blob, std::make_shared<BlobConverter>(blob)};
+    RETURN_ON_NEQ(conv.second->ConvertToMat(*cached, param, q), TNN_OK);
     mat = cached;
     return TNN_OK;
 }

@@ -259,6 +259,8 @@ private:
                     continue;
                 bool hb = ip->has_bias && ir->bias_handle.GetDataCount() == N &&
                           ir->bias_handle.GetDataType() == DATA_TYPE_FLOAT;
+                if (ip->has_bias && !hb && ir->bias_handle.GetDataCount() > 0)
+                    continue;  // a bias of another type or length: leave the layer to its un-fused acc
                 auto fused = MakeLinear(l->name + "_fused", l->inputs[0], l->outputs[0], N, K,
                                         ir->weight_handle.force_to<float *>(), nullptr,
                                         hb ? ir->bias_handle.force_to<float *>() : nullptr, hb);

@@ -735,6 +735,8 @@ private:
     std::shared_ptr<ModelInterpreter> interpreter_;
     std::shared_ptr<DefaultNetwork> network_;
     std::map<std::string, std::shared_ptr<Mat>> output_mats_;
+    // blob name -> (the blob the converter was made for, converter)
+    std::map<std::string, std::pair<Blob *, std::shared_ptr<BlobConverter>>> input_converters_, output_converters_;
 };
 
 }  // namespace TNN_NS
