@@ -57,10 +57,11 @@ def c1(args):
 def c3(args):
     import torch
     from . import ops
-    B, h, S = 32, 12, 512
+    # --batch / --seq move the kernel away from the configuration's own shape (e.g. B4 S4096: its steady state)
+    B, h, S = args.batch or 32, 12, args.seq or 512
     H = h * 64
     rng = np.random.default_rng(20240603)
-    lens = rng.integers(16, 513, B).astype(np.int32)
+    lens = rng.integers(min(16, S), S + 1, B).astype(np.int32)
     qk = torch.randn(B * S, 2 * H, device="cuda").half()
     vt = torch.randn(B, h, 64, S, device="cuda").half()
     out = torch.empty(B * S, H, device="cuda", dtype=torch.half)
@@ -87,7 +88,7 @@ def c3(args):
         torch.cuda.synchronize()
         res[name] = e0.elapsed_time(e1) / (args.steps * n) * 1e3
     eff, pad = 4 * H * S * int(lens.sum()), 4 * B * S * S * H
-    return {"config": "c3", "workload": "attention kernel fp16, B32 h12 d64 S512, lengths U[16,512]",
+    return {"config": "c3", "workload": "attention kernel fp16, B%d h12 d64 S%d, lengths U[%d,%d]" % (B, S, min(16, S), S),
             "us_per_launch": res["varlen"], "tflops_effective": eff / res["varlen"] / 1e6,
             "tflops_padded": pad / res["varlen"] / 1e6, "us_per_launch_full_lengths": res["full"],
             "tflops_full_lengths": pad / res["full"] / 1e6}
@@ -145,6 +146,8 @@ def main():
     ap.add_argument("--config", choices=["c1", "c3", "c4", "c5"], required=True)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration names (c4, c5)")
+    ap.add_argument("--batch", type=int, default=0, help="c3: batch instead of 32")
+    ap.add_argument("--seq", type=int, default=0, help="c3: sequence length instead of 512")
     args = ap.parse_args()
     print(json.dumps({"c1": c1, "c3": c3, "c4": c4, "c5": c5}[args.config](args)))
 

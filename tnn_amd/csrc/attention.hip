@@ -42,6 +42,15 @@ template <> struct AttnT<TNN_ROCM_F16> {
         c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
                                                    0);
     }
+    // First product of an accumulation chain, d = a b + c0, with c0 read from registers of its own and left intact.
+    // Written as an instruction because the compiler only emits the form whose destination is also the C operand and
+    // copies c0 into d first (16 moves per chain).  The early-clobber output keeps d apart from the inputs; the next
+    // MFMA of the chain accumulates into d (same opcode, C = destination of this one: no wait states needed).
+    template <typename V> static __device__ __forceinline__ f32x16 mma_from(const V &a, const V &b, const f32x16 &c0) {
+        f32x16 d;
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c0));
+        return d;
+    }
     static __device__ __forceinline__ float to_float(uint16_t bits) { return (float)__builtin_bit_cast(half_t, bits); }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         half_t l = (half_t)lo, h = (half_t)hi;
@@ -72,6 +81,11 @@ template <> struct AttnT<TNN_ROCM_BF16> {
     template <typename V> static __device__ __forceinline__ void mma(const V &a, const V &b, f32x16 &c) {
         c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
                                                     0, 0);
+    }
+    template <typename V> static __device__ __forceinline__ f32x16 mma_from(const V &a, const V &b, const f32x16 &c0) {
+        f32x16 d;
+        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c0));
+        return d;
     }
     static __device__ __forceinline__ float to_float(uint16_t bits) { return __uint_as_float((uint32_t)bits << 16); }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -448,7 +462,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
 #define TR_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n)&0xF) | ((((n) >> 4) & 3) << 14) | (0x7 << 4) | (0xF << 8)))
 
 template <int DT, int NW>
-__global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel(AttnParams p) {
+__global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 : 2) attention_dma_kernel(AttnParams p) {
     constexpr int NT = NW * 64;
     constexpr int BQ = NW * 32;
     constexpr int kTile  = kTileKV * 128;  // one K or V^T tile, un-padded rows
@@ -571,6 +585,19 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
     }
     if (n_tiles > 1)
         issue(1, 1);
+    // Q is scaled by c = scale * log2(e) once (fp32 product, one rounding back to the input type), so the score
+    // MFMAs deliver s*c and the key loop never multiplies a score again.
+    {
+        const float c = p.scale_log2e;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t word = qf[kk][w];
+                qf[kk][w] = AttnT<DT>::pack2(AttnT<DT>::to_float((uint16_t)(word & 0xffffu)) * c,
+                                             AttnT<DT>::to_float((uint16_t)(word >> 16)) * c);
+            }
+    }
 
     // fragment chunk x = 2*step + g of row lq (the same expression serves the K and the V^T tile)
     uint32_t frag_off[4];
@@ -585,9 +612,28 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
         for (int r = 0; r < 16; ++r)
             oacc[dt][r] = 0.f;
     float m_i = -INFINITY, l_i = 0.f;
+    f32x16 negm;  // -m_i in every register: the start value of the score accumulators in the FAST tile form
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        negm[r] = INFINITY;
+    asm volatile("" : "+v"(negm));
 
+    // The tile body exists in three forms.  x = the scaled score as the MFMA delivers it (Q carries scale*log2 e):
+    //   BIAS : x + bias (additive mask, -inf for keys past kv_end), exact running maximum m, p = exp2(x + bias - m)
+    //   EXACT: the same without a bias (the first tile of a row block)
+    //   FAST : no bias, m finite.  The first MFMA of each score chain starts from a register block holding -m, so the
+    //          accumulators come out as x - m and p = exp2 of them: no per-score arithmetic besides the exponential.
+    //          m is not advanced: the probabilities may use a stale reference as long as they fit the packed
+    //          half-precision operand of the second MFMA.  That is checked on the row sums (a lane's partial sum above
+    //          kStaleLimit, or not finite, means some p may be too large) before anything is added to O; if it fails
+    //          (rare) the wave leaves the FAST loop and takes the same tile again in the EXACT form, which advances m.
+    //          The normalised result does not depend on which reference the exponentials use.
+    // Control flow: an outer loop runs one BIAS / EXACT tile, then an inner loop runs FAST tiles for as long as they
+    // are eligible and pass their check.  The inner loop has one body and one exit, so the O accumulators stay in the
+    // same registers around it.
+    constexpr float kStaleLimit = 1024.0f;  // p up to 2^10: 64 of them still sum far below the half-precision range
     int stage = 0, fill = 2;
-    for (int t = 0; t < n_tiles; ++t) {
+    auto enter_tile = [&](int t) __attribute__((always_inline)) {
         // tile t has landed once at most the loads of tile t + 1 are outstanding
         if (t + 1 < n_tiles) {
             if (mb)
@@ -601,141 +647,163 @@ __global__ void __launch_bounds__(NW * 64, NW == 4 ? 3 : 2) attention_dma_kernel
         asm volatile("" ::: "memory");  // no LDS access may be moved across the barrier by the compiler
         if (t + 2 < n_tiles)
             issue(t + 2, fill);
-
+    };
+    auto leave_tile = [&]() __attribute__((always_inline)) {
+        stage = stage == 2 ? 0 : stage + 1;
+        fill  = fill == 2 ? 0 : fill + 1;
+    };
+    // Probabilities -> packed operands of the second MFMA.  Register r of block kt is key kt*32 + 8*(r/4) + 4*g +
+    // (r%4): a lane half holds four keys of each 8-key group.  Step st = 2*kt + j uses groups 2j and 2j+1 of the
+    // block; after exchanging the packed pairs (group 2j+1 of the lower half <-> group 2j of the upper half) lane half
+    // g holds the eight consecutive keys of group 2j + g, i.e. 16-byte chunk 2*st + g of the V^T rows.  The row sum is
+    // taken on the exchanged registers (the two halves of a column together hold every key once).
+    auto pack_probs = [&](f32x16 (&sacc)[2], u32x4 (&pf)[4], float &rs) __attribute__((always_inline)) {
+        rs = 0.f;
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            const int kt = st >> 1, j = st & 1;
+            uint32_t w0 = AttnT<DT>::pack_only(sacc[kt][8 * j + 0], sacc[kt][8 * j + 1]);
+            uint32_t w1 = AttnT<DT>::pack_only(sacc[kt][8 * j + 2], sacc[kt][8 * j + 3]);
+            uint32_t w2 = AttnT<DT>::pack_only(sacc[kt][8 * j + 4], sacc[kt][8 * j + 5]);
+            uint32_t w3 = AttnT<DT>::pack_only(sacc[kt][8 * j + 6], sacc[kt][8 * j + 7]);
+            auto x0 = __builtin_amdgcn_permlane32_swap(w0, w2, false, false);
+            auto x1 = __builtin_amdgcn_permlane32_swap(w1, w3, false, false);
+            pf[st][0] = x0[0], pf[st][1] = x1[0], pf[st][2] = x0[1], pf[st][3] = x1[1];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                AttnT<DT>::add_packed(pf[st][e], rs);
+        }
+    };
+    // O^T += V^T P^T and the row sum
+    auto accumulate = [&](const unsigned char *vtbuf, u32x4 (&pf)[4], float rs, float alpha) __attribute__((always_inline)) {
+#pragma unroll
+        for (int st = 0; st < 4; ++st)
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt) {
+                const u32x4 vf = *reinterpret_cast<const u32x4 *>(vtbuf + dt * 32 * 128 + frag_off[st]);
+                AttnT<DT>::mma(vf, pf[st], oacc[dt]);
+            }
+        rs  = half_swap_sum(rs);
+        l_i = fmaf(l_i, alpha, rs);
+    };
+    auto general_tile = [&](auto mode_tag, int t) __attribute__((always_inline)) {
+        constexpr int MODE = decltype(mode_tag)::value;  // 0 BIAS, 1 EXACT
         const unsigned char *const kbuf  = lds_all + stage * kStage;
         const unsigned char *const vtbuf = kbuf + kTile;
-        const int kv0     = t * kTileKV;
-        const bool biased = mb != nullptr || kv0 + kTileKV > kv_end;  // workgroup-uniform
-        // The tile body is written three times under one branch (with the branch inside the tile the compiler copies
-        // the 32 score registers where the paths meet).  c = scale * log2(e), s = the raw dot product:
-        //   BIAS : x = s*c + bias (additive mask, -inf for keys past kv_end), exact running maximum m, p = exp2(x - m)
-        //   EXACT: the same without a bias (the first tile of a row block, or c <= 0)
-        //   STALE: no bias, c > 0, m finite.  p = exp2(s*c - m) in one fused multiply-add per score, and m only
-        //          follows the true maximum when a score exceeds it by more than kStaleMax (2^kStaleMax still fits the
-        //          packed half-precision probabilities comfortably); only then are the O accumulators and the row sum
-        //          rescaled.  The normalised result does not depend on which reference the exponentials use.
-        constexpr float kStaleMax = 10.0f;
-        const float c = p.scale_log2e;
-        auto tile = [&](auto mode_tag) __attribute__((always_inline)) {
-            constexpr int MODE = decltype(mode_tag)::value;  // 0 BIAS, 1 EXACT, 2 STALE
-            f32x16 sacc[2];
+        const int kv0 = t * kTileKV;
+        f32x16 sacc[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                sacc[kt][r] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                u32x4 kf = *reinterpret_cast<const u32x4 *>(kbuf + kt * 32 * 128 + frag_off[kk]);
+                AttnT<DT>::mma(kf, qf[kk], sacc[kt]);
+            }
+        }
+        float mx = -INFINITY;
+        if (MODE == 0) {
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    sacc[kt][r] = 0.f;
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    const int key0 = kt * 32 + r4 * 8 + g * 4;
+                    // without a mask the three bias rows hold zeros (written once above), so no branch is needed and
+                    // the eight reads of a tile go out together
+                    const float4 raw = *reinterpret_cast<const float4 *>(&lds_bias[stage][key0]);
+                    const float bv[4] = {raw.x * kLog2e, raw.y * kLog2e, raw.z * kLog2e, raw.w * kLog2e};
 #pragma unroll
-                for (int kk = 0; kk < 4; ++kk) {
-                    u32x4 kf = *reinterpret_cast<const u32x4 *>(kbuf + kt * 32 * 128 + frag_off[kk]);
-                    AttnT<DT>::mma(kf, qf[kk], sacc[kt]);
+                    for (int e = 0; e < 4; ++e) {
+                        const float be       = kv0 + key0 + e < kv_end ? bv[e] : -INFINITY;
+                        float s2             = sacc[kt][r4 * 4 + e] + be;
+                        sacc[kt][r4 * 4 + e] = s2;
+                        mx                   = fmaxf(mx, s2);
+                    }
                 }
             }
-            float mx = -INFINITY, alpha = 1.0f;
-            if (MODE == 0) {
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    mx = fmaxf(mx, sacc[kt][r]);
+        }
+        mx          = half_swap_max(mx);
+        float m_new = fmaxf(m_i, mx);
+        float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                sacc[kt][r] = __builtin_amdgcn_exp2f(sacc[kt][r] - m_use);
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                oacc[dt][r] *= alpha;
+        m_i = m_new;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            negm[r] = -m_new;
+        // the sixteen registers stay a block of their own (the MFMA reads them as its C operand); without this the
+        // compiler keeps one copy and rebuilds the block in front of every tile
+        asm volatile("" : "+v"(negm));
+        u32x4 pf[4];
+        float rs;
+        pack_probs(sacc, pf, rs);
+        accumulate(vtbuf, pf, rs, alpha);
+    };
+
+    int t = 0;
+    bool entered = false;  // the FAST loop gave tile t up after entering it: the barrier of tile t is already behind us
+    while (t < n_tiles) {
+        if (!entered)
+            enter_tile(t);
+        entered = false;
+        if (mb != nullptr || (t + 1) * kTileKV > kv_end)  // workgroup-uniform
+            general_tile(std::integral_constant<int, 0>(), t);
+        else
+            general_tile(std::integral_constant<int, 1>(), t);
+        leave_tile();
+        ++t;
+        if (mb != nullptr || !__all(m_i > -INFINITY))  // per wave: FAST needs a finite reference
+            continue;
+        while (t < n_tiles && (t + 1) * kTileKV <= kv_end) {
+            enter_tile(t);
+            const unsigned char *const kbuf  = lds_all + stage * kStage;
+            const unsigned char *const vtbuf = kbuf + kTile;
+            u32x4 pf[4];
+            float rs;
+            {
+                f32x16 sacc[2];
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt) {
+                    u32x4 kf = *reinterpret_cast<const u32x4 *>(kbuf + kt * 32 * 128 + frag_off[0]);
+                    sacc[kt] = AttnT<DT>::mma_from(kf, qf[0], negm);
 #pragma unroll
-                    for (int r4 = 0; r4 < 4; ++r4) {
-                        const int key0 = kt * 32 + r4 * 8 + g * 4;
-                        // without a mask the three bias rows hold zeros (written once below), so no branch is needed
-                        // and the eight reads of a tile go out together
-                        const float4 raw = *reinterpret_cast<const float4 *>(&lds_bias[stage][key0]);
-                        const float bv[4] = {raw.x * kLog2e, raw.y * kLog2e, raw.z * kLog2e, raw.w * kLog2e};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const float be       = kv0 + key0 + e < kv_end ? bv[e] : -INFINITY;
-                            float s2             = fmaf(sacc[kt][r4 * 4 + e], c, be);
-                            sacc[kt][r4 * 4 + e] = s2;
-                            mx                   = fmaxf(mx, s2);
-                        }
+                    for (int kk = 1; kk < 4; ++kk) {
+                        kf = *reinterpret_cast<const u32x4 *>(kbuf + kt * 32 * 128 + frag_off[kk]);
+                        AttnT<DT>::mma(kf, qf[kk], sacc[kt]);
                     }
                 }
-            } else {
-                // the maximum of the raw products; for MODE 1 the sign of c decides which end of them it is
-                float mn = INFINITY;
-#pragma unroll
-                for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        mx = fmaxf(mx, sacc[kt][r]);
-                        if (MODE == 1)
-                            mn = fminf(mn, sacc[kt][r]);
-                    }
-                mx = MODE == 1 ? fmaxf(mx * c, mn * c) : mx * c;
-            }
-            mx = half_swap_max(mx);
-            if (MODE == 2) {
-                if (__any(mx - m_i > kStaleMax)) {  // rare: some row's scores outgrew the reference
-                    const float delta = fmaxf(mx - m_i, 0.f);
-                    m_i += delta;
-                    alpha = __builtin_amdgcn_exp2f(-delta);
-#pragma unroll
-                    for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r)
-                            oacc[dt][r] *= alpha;
-                }
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
-                        sacc[kt][r] = __builtin_amdgcn_exp2f(fmaf(sacc[kt][r], c, -m_i));
-            } else {
-                float m_new = fmaxf(m_i, mx);
-                float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-                alpha       = __builtin_amdgcn_exp2f(m_i - m_use);
-#pragma unroll
-                for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        sacc[kt][r] = __builtin_amdgcn_exp2f(MODE == 0 ? sacc[kt][r] - m_use : fmaf(sacc[kt][r], c, -m_use));
-#pragma unroll
-                for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        oacc[dt][r] *= alpha;
-                m_i = m_new;
+                        sacc[kt][r] = __builtin_amdgcn_exp2f(sacc[kt][r]);
+                pack_probs(sacc, pf, rs);
             }
-
-            // ---- O^T += V^T P^T.  Register r of block kt is key kt*32 + 8*(r/4) + 4*g + (r%4): a lane half holds four
-            // keys of each 8-key group.  Step st = 2*kt + j uses groups 2j and 2j+1 of the block; after exchanging the
-            // packed pairs (group 2j+1 of the lower half <-> group 2j of the upper half) lane half g holds the eight
-            // consecutive keys of group 2j + g, i.e. 16-byte chunk 2*st + g of the V^T rows.  The row sum is taken on
-            // the exchanged registers (the two halves of a column together still hold every key once), so the
-            // registers before the exchange die there.
-            float rs = 0.f;
-#pragma unroll
-            for (int st = 0; st < 4; ++st) {
-                const int kt = st >> 1, j = st & 1;
-                uint32_t w0 = AttnT<DT>::pack_only(sacc[kt][8 * j + 0], sacc[kt][8 * j + 1]);
-                uint32_t w1 = AttnT<DT>::pack_only(sacc[kt][8 * j + 2], sacc[kt][8 * j + 3]);
-                uint32_t w2 = AttnT<DT>::pack_only(sacc[kt][8 * j + 4], sacc[kt][8 * j + 5]);
-                uint32_t w3 = AttnT<DT>::pack_only(sacc[kt][8 * j + 6], sacc[kt][8 * j + 7]);
-                auto x0 = __builtin_amdgcn_permlane32_swap(w0, w2, false, false);
-                auto x1 = __builtin_amdgcn_permlane32_swap(w1, w3, false, false);
-                u32x4 pf;
-                pf[0] = x0[0], pf[1] = x1[0], pf[2] = x0[1], pf[3] = x1[1];
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    AttnT<DT>::add_packed(pf[e], rs);
-#pragma unroll
-                for (int dt = 0; dt < 2; ++dt) {
-                    const u32x4 vf = *reinterpret_cast<const u32x4 *>(vtbuf + dt * 32 * 128 + frag_off[st]);
-                    AttnT<DT>::mma(vf, pf, oacc[dt]);
-                }
+            if (__builtin_expect(__any(!(rs <= kStaleLimit)), 0)) {
+                entered = true;
+                break;
             }
-            rs  = half_swap_sum(rs);
-            l_i = fmaf(l_i, alpha, rs);
-        };
-        if (biased)
-            tile(std::integral_constant<int, 0>());
-        else if (c > 0.f && __all(m_i > -INFINITY))  // per wave: the reference must be finite (true from the second tile on)
-            tile(std::integral_constant<int, 2>());
-        else
-            tile(std::integral_constant<int, 1>());
-
-        stage = stage == 2 ? 0 : stage + 1;
-        fill  = fill == 2 ? 0 : fill + 1;
+            accumulate(vtbuf, pf, rs, 1.0f);
+            leave_tile();
+            ++t;
+        }
     }
 
     // ---- normalise and store (see attention_kernel)
