@@ -51,7 +51,9 @@ def parse():
 
 def cpu_baseline(cfg, weights, ids, seg, mask, n_seqs):
     """Bounded CPU sample: n_seqs sequences through all layers.  "reference" = the reference engine's DEVICE_X86 path
-    (oracle/_ref, prebuilt); "port" = the plain-C restatement under oracle/ when that library is absent."""
+    (oracle/_ref, prebuilt) timed with the reference benchmark tool's own loop (5 warm-up + 20 timed iterations of
+    SetInputMat + Forward + GetOutputMat) on all host cores, plus a reduced loop on one thread; "port" = the plain-C
+    restatement under oracle/ when that library is absent."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     B, S = ids.shape
     n = min(n_seqs, B)
@@ -109,12 +111,29 @@ def main():
         inst.forward()
 
     # ---- timed region: exactly K Instance::Forward() calls (graph replay + the engine's per-forward synchronise)
+    step_s = []
     inst.sync()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        inst.forward()
+        ts = time.perf_counter()
+        inst.forward()          # returns after the forward's own synchronise
+        step_s.append(time.perf_counter() - ts)
     inst.sync()
     dt = time.perf_counter() - t0
+
+    # ---- untimed for `value`: the loop of the reference's benchmark tool (test/test.cc:101-152), i.e. the host Mats
+    # go in and the output Mat comes out every iteration: SetInputMat x3 (25 KB over PCIe) + Forward + GetOutputMat
+    # (the [8,384,768] result cast to fp32 on the device and copied to the host), 5 warm-up + 20 timed iterations
+    io_s = []
+    for it in range(25):
+        ts = time.perf_counter()
+        inst.set_input("input_ids", ids)
+        inst.set_input("token_type_ids", seg)
+        inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+        inst.forward()
+        inst.output("last_hidden", max_elems=B * S * cfg.hidden)
+        if it >= 5:
+            io_s.append(time.perf_counter() - ts)
 
     ms_per_step = dt / args.steps * 1e3
     seqs_per_s = B * args.steps / dt
@@ -185,6 +204,26 @@ def main():
                 "us_per_launch": round(ms * 1e3, 2),
                 "frac_of_fp16_peak_effective": round(eff / (ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 4)}
 
+    # ---- the int8 path's dominant kernel on its own workload (config 4: B16 S256 -> 4096 tokens): FFN1 as the
+    # quantised graph launches it (int8 x int8 -> int32, requantise, the GELU chain as a table in the epilogue)
+    def int8_roofline():
+        T8 = 16 * 256
+        a8 = torch.randint(-128, 128, (T8, H), device="cuda", dtype=torch.int8)
+        w8 = torch.randint(-127, 128, (F, H), device="cuda", dtype=torch.int8)
+        b8 = torch.randint(-500, 500, (F,), device="cuda", dtype=torch.int32)
+        sc = (torch.rand(F, device="cuda") * 2e-4 + 1e-4).float()
+        iota = torch.arange(-128, 128, dtype=torch.int16).to(torch.int8).cuda()
+        lut = ops.gelu_i8(iota, 0.05, 20.0)
+        o8 = torch.empty(T8, F, device="cuda", dtype=torch.int8)
+        ms = timed(lambda: ops.gemm_i8_lut(a8, w8, b8, sc, lut, out=o8), n_gemm)
+        opsn = 2.0 * T8 * F * H
+        return {"bound": "mfma", "kernel": "gemm_nk_tiled_kernel<int8> (config 4 FFN1: M=%d N=%d K=%d, requantise + GELU "
+                                           "table epilogue)" % (T8, F, H),
+                "achieved": round(opsn / (ms * 1e-3) / 1e12, 2), "peak": 5000.0, "unit": "TOP/s",
+                "frac": round(opsn / (ms * 1e-3) / 1e12 / 5000.0, 4), "traffic": None,
+                "us_per_launch": round(ms * 1e3, 2), "ops_per_launch": opsn}
+
+    roof_i8 = int8_roofline()
     attn_here = attention_tflops(B, S, lens)
     stress_lens = np.random.default_rng(20240603).integers(16, 513, 32)
     attn_stress = attention_tflops(32, 512, stress_lens)
@@ -201,6 +240,12 @@ def main():
         "metric": "BERT-base seq384 fp16 sequences/sec on 1 MI355X; fused-attention TFLOP/s",
         "value": round(seqs_per_s, 2), "unit": "sequences/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "ms_per_step_min_avg_max": [round(min(step_s) * 1e3, 4), round(sum(step_s) / len(step_s) * 1e3, 4),
+                                    round(max(step_s) * 1e3, 4)],
+        "with_mat_io": {"loop": "SetInputMat x3 + Forward + GetOutputMat, 5 warm-up + 20 timed (test/test.cc:101-152)",
+                        "ms_min_avg_max": [round(min(io_s) * 1e3, 4), round(sum(io_s) / len(io_s) * 1e3, 4),
+                                           round(max(io_s) * 1e3, 4)],
+                        "sequences_per_s": round(B * len(io_s) / sum(io_s), 2)},
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": ("12-layer BERT-base encoder fp16, batch 8, seq 384, valid lengths U[200,384] "
                                 "(BASELINE.json configs[1])") if full_cfg else
@@ -223,6 +268,7 @@ def main():
                      "flops_per_launch": gemm_flops[dominant],
                      "all_gemms_us_per_launch": {k: round(v * 1e3, 2) for k, v in sorted(gemm_ms.items())},
                      "all_gemms_tflops": {k: round(gemm_flops[k] / (v * 1e-3) / 1e12, 1) for k, v in sorted(gemm_ms.items())}},
+        "roofline_int8": roof_i8,
         "layer_breakdown_ms_per_step": {k: round(v, 4) for k, v in sorted(breakdown.items())},
     }
     inst.close()

@@ -22,6 +22,7 @@ struct Session {
     TNN net;
     std::shared_ptr<Instance> inst;
     std::string err;
+    std::vector<std::pair<std::string, std::shared_ptr<Mat>>> inputs;  // the host Mats last given per input name
 };
 void put_err(char *buf, size_t n, const std::string &s) {
     if (buf && n) {
@@ -73,6 +74,14 @@ REF_API int tnn_ref_set_input(void *h, const char *name, const void *data, int m
         s->err = st.description();
         return (int)st;
     }
+    bool known = false;
+    for (auto &kv : s->inputs)
+        if (kv.first == name) {
+            kv.second = mat;
+            known     = true;
+        }
+    if (!known)
+        s->inputs.push_back({name, mat});
     return 0;
 }
 
@@ -126,6 +135,43 @@ REF_API double tnn_ref_time_forward(void *h, int warmup, int iters) {
             return -1.0;
     auto t1 = std::chrono::steady_clock::now();
     return std::chrono::duration<double>(t1 - t0).count() / (iters > 0 ? iters : 1);
+}
+
+// The measurement loop of the reference's own benchmark tool (test/test.cc:101-152): `warmup` untimed iterations,
+// then `iters` timed ones, each iteration = SetInputMat of every input (ConvertFromMat) + Forward + GetOutputMat of
+// `out_name` (ConvertToMat).  stats receives {min, avg, max} seconds per iteration.  The caller keeps the input
+// buffers given to tnn_ref_set_input alive.
+REF_API int tnn_ref_time_loop(void *h, int warmup, int iters, const char *out_name, double *stats) {
+    Session *s = static_cast<Session *>(h);
+    double mn = 1e30, mx = 0.0, sum = 0.0;
+    for (int i = 0; i < warmup + iters; ++i) {
+        auto t0 = std::chrono::steady_clock::now();
+        for (auto &kv : s->inputs) {
+            Status st = s->inst->SetInputMat(kv.second, MatConvertParam(), kv.first);
+            if (st != TNN_OK) {
+                s->err = st.description();
+                return (int)st;
+            }
+        }
+        Status st = s->inst->Forward();
+        std::shared_ptr<Mat> mat;
+        if (st == TNN_OK)
+            st = s->inst->GetOutputMat(mat, MatConvertParam(), out_name, DEVICE_NAIVE, NCHW_FLOAT);
+        if (st != TNN_OK) {
+            s->err = st.description();
+            return (int)st;
+        }
+        double dt = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        if (i >= warmup) {
+            mn = dt < mn ? dt : mn;
+            mx = dt > mx ? dt : mx;
+            sum += dt;
+        }
+    }
+    stats[0] = mn;
+    stats[1] = sum / (iters > 0 ? iters : 1);
+    stats[2] = mx;
+    return 0;
 }
 
 }  // extern "C"

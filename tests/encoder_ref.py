@@ -52,6 +52,41 @@ def encoder(w, cfg, x, B, S, mask):
     return x
 
 
+def encoder_blobs(w, cfg, ids, seg, B, S, mask):
+    """Every named blob of tnn_amd.tnnmodel.encoder_graph that is a whole tensor of the decomposed graph and may
+    survive the device's fusion passes, as the CPU evaluates it: {blob name: array}.  Used as the CPU side of the
+    per-blob model check."""
+    out = {}
+    x = embed(w, ids, seg, cfg.eps)
+    out["x0"] = x
+    H, heads, d = cfg.hidden, cfg.heads, cfg.head_dim
+    for li, lw in enumerate(w["layers"]):
+        p = "l%d_" % li
+        q, k, v = (linear(x, lw["w" + n], lw["b" + n]) for n in "qkv")
+        out[p + "q_o"], out[p + "k_o"], out[p + "v_o"] = q, k, v
+        q4, k4, v4 = (orc.permute(t.reshape(B, S, heads, d), (0, 2, 1, 3)) for t in (q, k, v))
+        ctx = orc.attention_core(q4, k4, v4, np.float32(1.0 / np.sqrt(d)), mask)
+        ctx = orc.permute(ctx, (0, 2, 1, 3)).reshape(B * S, H)
+        out[p + "ctx"] = ctx
+        a = linear(ctx, lw["wo"], lw["bo"])
+        out[p + "attn_o"] = a
+        s1 = orc.binary("add", x, a)
+        out[p + "sum1"] = s1
+        x1 = orc.layernorm(s1, lw["ln1_g"], lw["ln1_b"], cfg.eps)
+        out[p + "x1"] = x1
+        f1 = linear(x1, lw["w1"], lw["b1"])
+        out[p + "ffn1_o"] = f1
+        h = orc.gelu(f1)
+        out[p + "act"] = h
+        f2 = linear(h, lw["w2"], lw["b2"])
+        out[p + "ffn2_o"] = f2
+        s2 = orc.binary("add", x1, f2)
+        out[p + "sum2"] = s2
+        x = orc.layernorm(s2, lw["ln2_g"], lw["ln2_b"], cfg.eps)
+        out["last_hidden" if li == cfg.layers - 1 else p + "x2"] = x
+    return out
+
+
 def int8_encoder(w, cfg, scales, x0, B, S, mask, quantize=None):
     """The graph of tnn_amd.quant.int8_encoder_graph evaluated with the checker: every projection is
     quantise(input) -> int8 FC (int32 accumulate, requantise) -> dequantise; everything else in fp32.

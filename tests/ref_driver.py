@@ -30,6 +30,7 @@ def lib():
         _lib.tnn_ref_last_error.argtypes = [C.c_void_p]
         _lib.tnn_ref_time_forward.restype = C.c_double
         _lib.tnn_ref_time_forward.argtypes = [C.c_void_p, C.c_int, C.c_int]
+        _lib.tnn_ref_time_loop.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_char_p, C.POINTER(C.c_double)]
     return _lib
 
 
@@ -73,6 +74,13 @@ class RefSession:
             raise RuntimeError("Forward failed while timing")
         return t
 
+    def time_loop(self, warmup, iters, out_name):
+        """the reference's own benchmark loop (test/test.cc:101-152): SetInputMat + Forward + GetOutputMat per
+        iteration -> (min, avg, max) seconds"""
+        stats = (C.c_double * 3)()
+        self._check(lib().tnn_ref_time_loop(self.h, warmup, iters, out_name.encode(), stats), "timing loop")
+        return stats[0], stats[1], stats[2]
+
     def close(self):
         if self.h:
             lib().tnn_ref_destroy(self.h)
@@ -82,20 +90,33 @@ class RefSession:
         self.close()
 
 
-def time_encoder(cfg, weights, ids, seg, mask):
-    """CPU baseline of the benchmark: the reference's DEVICE_X86 path on the same synthetic encoder, all host
-    cores (OpenMP), `ids.shape[0]` sequences through all layers."""
+def time_encoder(cfg, weights, ids, seg, mask, one_thread_seqs=1):
+    """CPU baseline of the benchmark: the reference's DEVICE_X86 path on the same synthetic encoder, timed with the
+    loop of the reference's own benchmark tool (test/test.cc:101-152: warm-up 5, 20 timed iterations of SetInputMat +
+    Forward + GetOutputMat; min / avg / max) on all host cores, and again on ONE thread with a reduced loop (1 warm-up,
+    2 timed iterations on `one_thread_seqs` sequences), which keeps the whole leg near half a minute."""
     from tnn_amd import tnnmodel
     B, S = ids.shape
-    g = tnnmodel.encoder_graph(cfg, weights, B, S)
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    s = RefSession(g, "X86", threads)
-    s.set_input("input_ids", ids.astype(np.int32))
-    s.set_input("token_type_ids", seg.astype(np.int32))
-    s.set_input("attention_bias", mask.reshape(B, 1, 1, S).astype(np.float32))
-    t = s.time_forward(1, 3)
-    s.close()
-    return {"value": B / t, "unit": "sequences/s", "cores": threads, "kind": "reference",
-            "sample": "%d sequences (S=%d) through all %d layers on the reference engine's DEVICE_X86 path "
-                      "(fp32, AVX2 + OpenMP; its MatMul/Softmax/LayerNorm kernels are single-threaded), "
-                      "mean of 3 Forward() calls after 1 warm-up" % (B, S, cfg.layers)}
+
+    def run(n_seq, n_threads, warmup, iters):
+        g = tnnmodel.encoder_graph(cfg, weights, n_seq, S)
+        s = RefSession(g, "X86", n_threads)
+        s.set_input("input_ids", ids[:n_seq].astype(np.int32))
+        s.set_input("token_type_ids", seg[:n_seq].astype(np.int32))
+        s.set_input("attention_bias", mask[:n_seq].reshape(n_seq, 1, 1, S).astype(np.float32))
+        mn, avg, mx = s.time_loop(warmup, iters, "last_hidden")
+        s.close()
+        return mn, avg, mx
+
+    mn, avg, mx = run(B, threads, 5, 20)
+    n1 = min(one_thread_seqs, B)
+    mn1, avg1, mx1 = run(n1, 1, 1, 2)
+    return {"value": B / avg, "unit": "sequences/s", "cores": threads, "kind": "reference",
+            "ms_per_forward": {"min": mn * 1e3, "avg": avg * 1e3, "max": mx * 1e3},
+            "one_thread": {"value": n1 / avg1, "unit": "sequences/s", "cores": 1,
+                           "ms_per_forward": {"min": mn1 * 1e3, "avg": avg1 * 1e3, "max": mx1 * 1e3},
+                           "sample": "%d sequence(s), 1 warm-up + 2 timed iterations" % n1},
+            "sample": "%d sequences (S=%d) through all %d layers on the reference engine's DEVICE_X86 path (fp32, AVX2 + "
+                      "OpenMP; its MatMul/Softmax/LayerNorm kernels are single-threaded), the reference benchmark "
+                      "tool's loop: 5 warm-up + 20 timed iterations of SetInputMat + Forward + GetOutputMat" % (B, S, cfg.layers)}

@@ -496,6 +496,38 @@ def test_model_check_and_profile_report():
     assert text.count("RocmFusedLinear") >= 12   # six layers in each of the two per-layer tables
 
 
+def test_model_check_device_against_cpu_checker_blob_by_blob():
+    """tools/model_check's comparison proper: every blob of the fused fp16 graph that survives the optimiser passes
+    against the same blob as the CPU evaluates the decomposed graph (tests/encoder_ref.encoder_blobs, the CPU checker
+    layer by layer), plus the engine's own element-wise pass rule."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    from tnn_amd import model_check
+    say("host: model_check, device vs CPU checker, 3-layer encoder fp16")
+    cfg = EncoderConfig.bert_base(3)
+    w = make_weights(cfg, seed=31, bias_std=0.02)
+    B, S = 2, 96
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 30, S, seed=32)
+    graph = tnnmodel.encoder_graph(cfg, w, B, S)
+    inputs = {"input_ids": ids, "token_type_ids": seg, "attention_bias": mask.reshape(B, 1, 1, S)}
+    reference = encoder_ref.encoder_blobs(r16w(w), cfg, ids, seg, B, S, mask)
+    rows, same, skipped = model_check.check_against(graph, inputs, reference, "fp16")
+    say(model_check.report(rows))
+    assert same and not skipped, skipped
+    names = {r["blob"] for r in rows}
+    # what survives per layer: the attention context, the three sums the LayerNorms read (outputs of the projections
+    # with the residual folded in), the LayerNorm outputs still needed as residuals, the FFN activation
+    assert {"x0", "l0_ctx", "l0_sum1", "l0_x1", "l0_act", "l0_sum2", "l2_ctx", "last_hidden"} <= names, sorted(names)
+    assert all(r["ok"] for r in rows), [r for r in rows if not r["ok"]]
+    # the engine's element rule (|d|/(|a|+|b|) > 0.005 and |d| > 1e-3) is written for an fp32 device; in fp16 a value of
+    # size 1 carries an ulp of 1e-3, so a few small elements trip it as the layers stack up: they are reported per blob
+    # and bounded here (observed: none in the first layer, 0.3 % of the last hidden state after three layers)
+    T = B * S
+    for r in rows:
+        n = T * (cfg.ffn if r["blob"].endswith("_act") else cfg.hidden)
+        assert r["engine_rule_failures"] <= 0.01 * n, (r["blob"], r["engine_rule_failures"], n)
+    assert all(r["engine_rule_failures"] == 0 for r in rows if r["blob"] in ("x0", "l0_ctx", "l0_sum1", "l0_act", "l0_x1"))
+
+
 def test_instance_reshape_matches_fresh_instances():
     """Instance::Reshape (default_network.cc:456-500): one instance moved through several (B, S) gives, at each shape and
     on each of four forwards (eager, eager, record + launch, replay), exactly what an instance created at that shape

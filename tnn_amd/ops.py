@@ -59,12 +59,12 @@ def gemm_i8(a, w, bias, scale, want_acc=False, want_q=True, dequant_scale=None, 
     return q, acc, outf
 
 
-def gemm_i8_lut(a, w, bias, scale, lut):
+def gemm_i8_lut(a, w, bias, scale, lut, out=None):
     """int8 out = lut[requantise(a w^T + bias) + 128]; lut: 256 int8 values on the device"""
     _chk(a, w, bias, scale, lut)
     M, K = a.shape
     N = w.shape[0]
-    q = torch.empty(M, N, dtype=torch.int8, device=a.device)
+    q = out if out is not None else torch.empty(M, N, dtype=torch.int8, device=a.device)
     capi.call("tnn_rocm_gemm_i8_lut", _stream(), _p(a), _p(w), _p(bias), _p(scale), _p(q), M, N, K, K, K, N, _p(lut))
     return q
 
