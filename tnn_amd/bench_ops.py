@@ -141,13 +141,61 @@ def run(launches, only=None, sizes=("encoder", "stream"), report=None):
     return results
 
 
+def mall_probe(launches=20):
+    """Does the memory-side cache (256 MB, shared by the eight XCDs) serve the panel re-reads of the projection GEMMs?
+    No counter visible from the GPU separates its hits from HBM accesses, so this times each GEMM of the batch-8 /
+    seq-384 encoder twice with an event pair around the single launch: once with its operands as a previous launch
+    left them (resident in that cache, like the activations a layer has just written), once right after a 1 GiB device
+    copy that evicts them (every first touch then goes to HBM).  A spinning kernel in front of both keeps the queue
+    filled, so the host's launch latency is in neither figure.  The difference is what HBM-side re-reads cost."""
+    capi.load()
+    T, H, F = ROWS_ENC, 768, 3072
+    f16 = torch.float16
+    shapes = {"qkv (M3072 N2304 K768)": (T, 3 * H, H), "out (M3072 N768 K768)": (T, H, H),
+              "ffn1 (M3072 N3072 K768)": (T, F, H), "ffn2 (M3072 N768 K3072)": (T, H, F)}
+    big_a = torch.empty(1 << 28, dtype=torch.float32, device="cuda")
+    big_b = torch.empty(1 << 28, dtype=torch.float32, device="cuda")
+    rows = []
+    for name, (M, N, K) in shapes.items():
+        a, w = _randn((M, K), f16), _randn((N, K), f16) * 0.02
+        bias = torch.zeros(N, device="cuda")
+        res = _randn((M, N), f16)
+        out = torch.empty(M, N, dtype=f16, device="cuda")
+        fn = lambda: ops.gemm(a, w, True, bias=bias, residual=res, out=out)
+        for _ in range(3):
+            fn()
+        t = {}
+        for mode in ("resident", "evicted"):
+            tot = 0.0
+            for _ in range(launches):
+                if mode == "evicted":
+                    big_b.copy_(big_a)
+                torch.cuda._sleep(400000)  # ~0.2 ms without memory traffic: the launches below are queued behind it
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                fn()
+                e1.record()
+                torch.cuda.synchronize()
+                tot += e0.elapsed_time(e1)
+            t[mode] = tot / launches * 1e3
+        rows.append({"gemm": name, "us_resident": round(t["resident"], 2), "us_evicted": round(t["evicted"], 2),
+                     "operand_MiB": round((M * K + N * K + 2 * M * N) * 2 / 2**20, 1)})
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--mall-probe", action="store_true", help="projection GEMMs with resident / evicted operands")
     ap.add_argument("--launches", type=int, default=20)
     ap.add_argument("--only", default="")
     ap.add_argument("--sizes", default="encoder,stream")
     ap.add_argument("--json", action="store_true")
     a = ap.parse_args()
+    if a.mall_probe:
+        for r in mall_probe(a.launches):
+            print(json.dumps(r) if a.json else "%-28s operands %6.1f MiB   resident %7.2f us   evicted %7.2f us" % (
+                r["gemm"], r["operand_MiB"], r["us_resident"], r["us_evicted"]), flush=True)
+        return
     def line(r):
         if a.json:
             print(json.dumps(r), flush=True)

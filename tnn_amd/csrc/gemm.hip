@@ -27,6 +27,19 @@
 
 using namespace tnn_rocm;
 
+// Optional in-kernel timeline (stand-alone probe builds only, see probe_gemm_timeline.hip): thread 0 of every workgroup
+// of the tiled kernel stamps the constant-rate counter (100 MHz) at five points.
+#ifdef TNN_ROCM_TIMELINE
+__device__ unsigned long long g_gemm_timeline[4096 * 8];
+#define TR_TL(i)                                                                                                      \
+    do {                                                                                                              \
+        if (threadIdx.x == 0 && blockIdx.x < 4096)                                                                    \
+            g_gemm_timeline[(size_t)blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime();                         \
+    } while (0)
+#else
+#define TR_TL(i)
+#endif
+
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -797,6 +810,7 @@ __global__ void __launch_bounds__(CFG::NT)
     // the rows first, then the next tile column), so the tiles that are resident together on one XCD form a
     // compact block of the tile grid: their A and W panels fit that L2 and are fetched from HBM once, instead of
     // the whole W panel streaming through every L2 once per tile row.
+    TR_TL(0);  // entry
     const int n_tiles = tiles_m * tiles_n;
     const int per_xcd = (n_tiles + 7) >> 3;
     const int vid     = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
@@ -927,6 +941,8 @@ __global__ void __launch_bounds__(CFG::NT)
             // consumed by MFMAs already issued).  A bare barrier: __syncthreads() adds a fence that waits for
             // every outstanding load, the look-ahead ones included.
             __builtin_amdgcn_s_barrier();
+            if (kt == 0)
+                TR_TL(1);  // first slab landed
             asm volatile("" ::: "memory");  // no LDS access may be moved across the barrier by the compiler
             if (kt + NS - 1 < nk)
                 issue(kt + NS - 1, fill);
@@ -1034,6 +1050,7 @@ __global__ void __launch_bounds__(CFG::NT)
     AccT *const stage_me  = stage_all + wave * (32 * SSTR);  // wave = (wm*WGN + wn)*WGK + wk
     const bool by_rows = epi.direct(n0);
     __syncthreads();  // every wave is done reading the slabs
+    TR_TL(2);         // main loop done
     // LayerNorm-folding epilogues: reduce the lanes' partial row sums over the two k-halves of a fragment and the WGK
     // k-waves (fixed order), giving {rstd, mean} per tile row; both arrays sit behind the staging area
     float2 *const row_st   = reinterpret_cast<float2 *>(lds_dyn + CFG::stage_bytes);  // [BM]
@@ -1142,6 +1159,7 @@ __global__ void __launch_bounds__(CFG::NT)
         if (i + 1 < TM)
             __syncthreads();
     }
+    TR_TL(3);  // C stored
     if constexpr (Epi::kRowStats) {
         // y = LayerNorm(t) for this tile's share of its rows (the BM rows are dealt out evenly over the tile columns, so
         // every workgroup writes whole rows), in the LayerNorm kernel's half-precision form
@@ -1177,6 +1195,10 @@ __global__ void __launch_bounds__(CFG::NT)
             }
         }
     }
+#ifdef TNN_ROCM_TIMELINE
+    __syncthreads();
+    TR_TL(4);  // kernel end
+#endif
 }
 
 // tuning override for experiments: 0 = heuristic, otherwise a configuration code of the tiled kernel
