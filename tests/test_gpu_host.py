@@ -393,8 +393,9 @@ def test_encoder_bf16_from_model_files():
 
 
 def test_layernorm_folding_switch(monkeypatch):
-    """TNN_ROCM_FOLD_LN=0 keeps every LayerNorm a launch of its own; both graphs agree with each other to fp16
-    rounding and with the checker."""
+    """TNN_ROCM_FOLD_LN=0 keeps every LayerNorm a launch of its own, TNN_ROCM_LN_STATS=0 keeps the output tensor of a
+    folded LayerNorm for the residual that reads it; all three graphs agree with each other to fp16 rounding and with
+    the checker."""
     host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
     say("host: LayerNorm folding on / off, 2-layer encoder fp16")
     cfg = EncoderConfig.bert_base(2)
@@ -409,8 +410,9 @@ def test_layernorm_folding_switch(monkeypatch):
     ids, seg, lens, mask = make_inputs(cfg, B, S, 30, S, seed=15)
     g = tnnmodel.encoder_graph(cfg, w, B, S)
     outs = {}
-    for fold, n_ln in (("0", 4), ("1", 1)):
-        monkeypatch.setenv("TNN_ROCM_FOLD_LN", fold)
+    for fold, n_ln in (("0", 4), ("1", 1), ("y", 1)):
+        monkeypatch.setenv("TNN_ROCM_FOLD_LN", "0" if fold == "0" else "1")
+        monkeypatch.setenv("TNN_ROCM_LN_STATS", "0" if fold == "y" else "1")
         inst = host.RocmInstance.from_graph(g, "fp16")
         types = [t for t, _ in inst.layers()]
         assert types.count("LayerNorm") == n_ln, types
@@ -424,8 +426,10 @@ def test_layernorm_folding_switch(monkeypatch):
     wr = r16w(w)
     ref = encoder_ref.encoder(wr, cfg, encoder_ref.embed(wr, ids, seg, cfg.eps), B, S, mask)
     e0, e1, e01 = rel_err(outs["0"], ref), rel_err(outs["1"], ref), rel_err(outs["1"], outs["0"])
-    say("  un-folded %.3g  folded %.3g  folded vs un-folded %.3g" % (e0, e1, e01))
-    assert e0 <= FP16_TOL and e1 <= FP16_TOL and e01 <= FP16_TOL
+    ey, e1y = rel_err(outs["y"], ref), rel_err(outs["1"], outs["y"])
+    say("  un-folded %.3g  folded %.3g  folded, output kept %.3g  folded vs un-folded %.3g  vs output kept %.3g"
+        % (e0, e1, ey, e01, e1y))
+    assert e0 <= FP16_TOL and e1 <= FP16_TOL and ey <= FP16_TOL and e01 <= FP16_TOL and e1y <= FP16_TOL
 
 
 @pytest.mark.parametrize("hidden,heads,ffn,B,S,n_ln", [

@@ -927,6 +927,23 @@ def test_gemm_layernorm_folded_into_projection(M, dtype):
     assert rel_err(host(qk), ref[:, :2 * H]) <= tol
     vref = ref[:, 2 * H:].reshape(B, S, heads, 64).transpose(0, 2, 3, 1)
     assert rel_err(host(vt), vref) <= tol
+    # the rows' {rstd, mean} handed on instead of the LayerNorm output: the statistics themselves, unchanged results,
+    # and a projection that rebuilds LayerNorm(t) from them as its residual (the out-projection / FFN2 form)
+    mean = t.astype(np.float64).mean(1)
+    rstd = 1.0 / np.sqrt(t.astype(np.float64).var(1) + eps)
+    h3, st1 = o.gemm_ln(D(t), w1f.cuda(), dev(b1f), dev(cs1), eps, gelu=True, want_stats=True)
+    qk3, vt3, st2 = o.qkv_split_ln(D(t), wqf.cuda(), dev(bqf), dev(csq), eps, B, S, heads, want_stats=True)
+    assert torch.equal(h3, h) and torch.equal(qk3, qk) and torch.equal(vt3, vt) and torch.equal(st1, st2)
+    assert np.abs(host(st1)[:, 0] / rstd - 1).max() <= 1e-5 and np.abs(host(st1)[:, 1] - mean).max() <= 1e-5
+    x2, w2, b2 = rnd(r32(M, F) * 0.5), r32(H, F) * 0.03, r32(H) * 0.1
+    ref2 = orc.inner_product(x2, rnd(w2), b2) + y_ref
+    got2 = o.gemm_residual_ln(D(x2), D(w2), D(t), st1, dev(g), dev(be), bias=dev(b2))
+    assert rel_err(host(got2), ref2) <= tol
+    via_y = o.gemm(D(x2), D(w2), True, bias=dev(b2), residual=y)   # the same sum with the stored LayerNorm output
+    assert rel_err(host(got2), host(via_y)) <= tol
+    xo, wo = rnd(r32(M, H) * 0.5), r32(H, H) * 0.05               # K = 768: the 64x64-tile shape
+    got3 = o.gemm_residual_ln(D(xo), D(wo), D(t), st1, dev(g), dev(be), bias=dev(b2), gelu=True)
+    assert rel_err(host(got3), orc.gelu(orc.inner_product(xo, rnd(wo), b2)) + y_ref) <= tol
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])

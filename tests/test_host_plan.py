@@ -62,6 +62,26 @@ def test_layernorm_fold_switch(monkeypatch):
     assert _types(host.plan(g, precision="fp16"))["LayerNorm"] == 1
 
 
+def test_row_statistics_hand_over_switch(monkeypatch):
+    """A folded LayerNorm whose output is read once more, as the residual of a projection: by default the output tensor
+    disappears (the folding layer has one output, the residual reader takes the raw tensor); TNN_ROCM_LN_STATS=0 keeps
+    the tensor as a second output."""
+    _, _, g = _graph()
+    for stats, n_out in (("1", 1), ("0", 2)):
+        monkeypatch.setenv("TNN_ROCM_LN_STATS", stats)
+        plan = host.plan(g, precision="fp16")
+        by_out = {o: l for l in plan for o in l["outputs"]}
+        ffn1, ffn2 = by_out["l0_act"], by_out["l0_sum2"]
+        assert ffn1["inputs"][0] == "l0_sum1" and len(ffn1["outputs"]) == n_out
+        assert ffn2["inputs"] == ["l0_act", "l0_sum1" if stats == "1" else "l0_x1"]
+        att, out = by_out["l1_ctx"], by_out["l1_sum1"]
+        assert att["inputs"][0] == "l0_sum2" and len(att["outputs"]) == n_out
+        assert out["inputs"] == ["l1_ctx", "l0_sum2" if stats == "1" else "l0_x2"]
+        assert ("l0_x1" in by_out) == (stats == "0")
+        # layer 0 reads the embedding output, which is a LayerNorm output of the embedding layer itself: nothing to rebuild
+        assert by_out["l0_sum1"]["inputs"] == ["l0_ctx", "x0"]
+
+
 def test_width_that_cannot_fold_keeps_its_layernorms():
     # hidden 192 is no multiple of 128: the LayerNorms stay launches of their own, everything else still fuses
     _, _, g = _graph(hidden=192, heads=3, ffn=384)

@@ -16,6 +16,7 @@
 // so V is stored transposed in LDS ([d][key]) and each lane fetches its two 4-key groups with two
 // 8-byte reads.  Padding keys (>= kv_len) are excluded exactly (−inf) in-register and whole tiles
 // past kv_len are never loaded.
+#include <atomic>
 #include <type_traits>
 
 #include "common.h"
@@ -881,7 +882,7 @@ __global__ void mask_to_kv_len_kernel(const float *__restrict__ mask, int32_t *_
 }
 
 // 128-row query blocks when that already gives >= 2 workgroups per CU, else 64-row blocks
-int g_attention_dma = 1;  // experiment hook: 0 keeps the register-staged kernel for the V^T layout as well
+std::atomic<int> g_attention_dma{1};  // experiment hook: 0 keeps the register-staged kernel for the V^T layout as well
 
 template <bool VT> int launch_attention(hipStream_t s, int dtype, const AttnParams &p, int B, int heads, int S) {
     long blocks128 = (long)((S + 127) / 128) * heads * B;

@@ -158,6 +158,68 @@ template <int DT> struct FloatEpilogue {
     }
 };
 
+// Projection whose residual operand is LayerNorm(t) of a tensor whose row statistics an earlier kernel left behind
+// (LnFold::stats): C = act(x W^T + b) + ((t - mean) * rstd * gamma + beta).  The normalised tensor is rebuilt from t in
+// registers, in the LayerNorm kernel's half-precision form x * rstd * gamma + (beta - mean * rstd * gamma), and never
+// stored.  N is the normalised width.
+template <int DT> struct LnResidualEpilogue {
+    typedef typename Elem<DT>::type T;
+    static constexpr bool kRowStats = false;
+    int flags;  // TNN_ROCM_EPI_BIAS, TNN_ROCM_EPI_GELU
+    const float *bias;
+    const T *t;                 // [M, N]
+    const float2 *st;           // [M] {rstd, mean}
+    const float *gamma, *beta;  // [N]
+    T *C;
+    long ldc;
+    __device__ __forceinline__ void set_batch(int) {}
+    __device__ __forceinline__ float col_const(int n) const { return (flags & TNN_ROCM_EPI_BIAS) ? bias[n] : 0.f; }
+    __device__ __forceinline__ void store(int m, int n, float acc, float bias_n) const {
+        float v = acc;
+        if (flags & TNN_ROCM_EPI_BIAS)
+            v = v + bias_n;
+        if (flags & TNN_ROCM_EPI_GELU)
+            v = gelu_erf(v);
+        const float2 s = st[m];
+        const float mrs = s.y * s.x;
+        v = v + (Elem<DT>::ld(&t[(size_t)m * ldc + n]) * s.x * gamma[n] + (beta[n] - mrs * gamma[n]));
+        Elem<DT>::st(&C[(size_t)m * ldc + n], v);
+    }
+    __device__ __forceinline__ bool direct(int) const { return false; }
+    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8]) const {
+        float v[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            v[q] = acc[q];
+        if (flags & TNN_ROCM_EPI_BIAS) {
+            float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
+            v[0] += b0.x, v[1] += b0.y, v[2] += b0.z, v[3] += b0.w;
+            v[4] += b1.x, v[5] += b1.y, v[6] += b1.z, v[7] += b1.w;
+        }
+        if (flags & TNN_ROCM_EPI_GELU) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+                v[q] = gelu_erf_fast(v[q]);
+        }
+        static_assert(sizeof(T) == 2, "half-precision blobs only");
+        u32x4 packed = *reinterpret_cast<const u32x4 *>(t + (size_t)m * ldc + n);
+        T *pe = reinterpret_cast<T *>(&packed);
+        const float2 s = st[m];
+        const float mrs = s.y * s.x;
+        float4 k0 = *reinterpret_cast<const float4 *>(gamma + n), k1 = *reinterpret_cast<const float4 *>(gamma + n + 4);
+        float4 e0 = *reinterpret_cast<const float4 *>(beta + n), e1 = *reinterpret_cast<const float4 *>(beta + n + 4);
+        const float kk[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+        const float ee[8] = {e0.x, e0.y, e0.z, e0.w, e1.x, e1.y, e1.z, e1.w};
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            v[q] += Elem<DT>::ld(&pe[q]) * s.x * kk[q] + (ee[q] - mrs * kk[q]);
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            Elem<DT>::st(&pe[q], v[q]);
+        *reinterpret_cast<u32x4 *>(C + (size_t)m * ldc + n) = packed;
+    }
+};
+
 // QKV projection epilogue: columns [0,2H) -> qk[T,2H]; columns [2H,3H) -> V^T[b][head][d][s]
 template <int DT> struct QkvSplitEpilogue {
     typedef typename Elem<DT>::type T;
@@ -219,7 +281,7 @@ template <int DT> struct QkvSplitEpilogue {
 // values), reduced over the workgroup after the main loop, and applied to the accumulators in the epilogue.
 // Other readers of y (the residual additions) still need the tensor: the workgroup of tile column j writes
 // y for the j-th share of the columns of its rows, so the LayerNorm launch disappears without y disappearing.
-int g_ln_y_ahead = 1;  // experiment hook, see tnn_rocm_debug_set_ln_y_ahead
+std::atomic<int> g_ln_y_ahead{1};  // experiment hook, see tnn_rocm_debug_set_ln_y_ahead
 
 struct LnFold {
     float inv_cols, eps;
@@ -227,6 +289,7 @@ struct LnFold {
     const float *gamma, *beta;  // [K], for the y side output
     void *y;                    // [M, K] in the compute type, or nullptr
     int y_ahead;                // 1: the source vectors of y are requested under the epilogue (0 for experiments)
+    float2 *stats;              // [M] {rstd, mean} for a later kernel that rebuilds LayerNorm(t) itself, or nullptr
 };
 
 // row sum and sum of squares of the eight values of an A fragment register quad
@@ -1076,7 +1139,10 @@ __global__ void __launch_bounds__(CFG::NT)
             }
             const double mean = s1 * (double)epi.ln.inv_cols;
             const double var  = s2 * (double)epi.ln.inv_cols - mean * mean;
-            row_st[tid]       = make_float2((float)(1.0 / sqrt(var + (double)epi.ln.eps)), (float)mean);
+            const float2 st   = make_float2((float)(1.0 / sqrt(var + (double)epi.ln.eps)), (float)mean);
+            row_st[tid]       = st;
+            if (epi.ln.stats && n0 == 0 && m0 + tid < M)  // every tile column holds them; the first one hands them on
+                epi.ln.stats[m0 + tid] = st;
         }
         // row_st is read after the first staging barrier below
     }
@@ -1202,8 +1268,9 @@ __global__ void __launch_bounds__(CFG::NT)
 }
 
 // tuning override for experiments: 0 = heuristic, otherwise a configuration code of the tiled kernel
-int g_gemm_force_cfg = 0;
-int g_gemm_group_m   = 0;  // 0 = derived from the tile count; otherwise forced
+// the hooks may be set while other threads launch: atomics, and a lock around the tuning table
+std::atomic<int> g_gemm_force_cfg{0};
+std::atomic<int> g_gemm_group_m{0};  // 0 = derived from the tile count; otherwise forced
 
 inline int tune_override(int N, int K, int *group_m);
 
@@ -1298,7 +1365,8 @@ inline int pick_tile_config(long M, long N, size_t kbytes) {
 struct TuneEntry { int n, k, cfg, group_m; };
 TuneEntry g_tune_table[16];
 int g_tune_count = -1;
-inline void parse_tune(const char *e) {
+std::mutex g_tune_lock;
+inline void parse_tune(const char *e) {  // caller holds g_tune_lock
     g_tune_count = 0;
     while (e && *e && g_tune_count < 16) {
         TuneEntry t;
@@ -1313,9 +1381,11 @@ inline void parse_tune(const char *e) {
 inline int tune_override(int N, int K, int *group_m) {
     static std::once_flag env_read;  // instances on several threads may launch their first GEMM together
     std::call_once(env_read, [] {
+        std::lock_guard<std::mutex> hold(g_tune_lock);
         if (g_tune_count < 0)
             parse_tune(getenv("TNN_ROCM_GEMM_TUNE"));
     });
+    std::lock_guard<std::mutex> hold(g_tune_lock);
     for (int i = 0; i < g_tune_count; ++i)
         if (g_tune_table[i].n == N && g_tune_table[i].k == K) {
             if (group_m)
@@ -1329,7 +1399,8 @@ template <int DT, typename Epi>
 int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb,
                      const Epi &epi) {
     typedef typename GemmTraits<DT>::elem T;
-    int cfg       = g_gemm_force_cfg > 0 ? g_gemm_force_cfg : tune_override(N, K, nullptr);
+    const int forced = g_gemm_force_cfg;
+    int cfg       = forced > 0 ? forced : tune_override(N, K, nullptr);
     size_t kbytes = (size_t)K * sizeof(T);
     if (cfg == 0) {
         // slabs that are whole 128-byte multiples go global -> LDS directly; average kernel durations inside a
@@ -1359,7 +1430,7 @@ int launch_gemm_fast(hipStream_t s, const void *A, const void *B, int M, int N, 
         cfg = 222221;
     if (DT == TNN_ROCM_F32)
         cfg %= 1000000;  // the fp32 instantiations are register-staged only
-    if (DT == TNN_ROCM_F32 && g_gemm_force_cfg <= 0 && cfg == 112211 && kbytes % 256 == 0 && kbytes >= 2048 &&
+    if (DT == TNN_ROCM_F32 && forced <= 0 && cfg == 112211 && kbytes % 256 == 0 && kbytes >= 2048 &&
         (((long)M + 63) / 64) * (((long)N + 63) / 64) * 2 <= kNumCU) {
         // A small fp32 product (one attention layer at 128 tokens: 24 tiles of 64x64) leaves nine CUs in ten idle,
         // and the fp32 matrix pipe is 16 times slower than the fp16 one: 32x32 tiles with the K range dealt to
@@ -1645,8 +1716,8 @@ int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *
 }
 
 int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folded, const float *bias_folded,
-                     const float *colsum, const float *gamma, const float *beta, float eps, void *C, void *y, int M, int N,
-                     int K, int flags, const void *residual) {
+                     const float *colsum, const float *gamma, const float *beta, float eps, void *C, void *y,
+                     float *row_stats, int M, int N, int K, int flags, const void *residual) {
     TR_REQUIRE(M >= 0 && N >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_ln: negative size");
     if (M == 0 || N == 0)
         return 0;
@@ -1659,8 +1730,8 @@ int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folde
                TNN_ROCM_ESHAPE, "gemm_ln: problem too large for 32-bit panel offsets");
     TR_REQUIRE(!(flags & TNN_ROCM_EPI_RESIDUAL) || residual, TNN_ROCM_EINVAL, "gemm_ln: residual flag without a residual");
     TR_REQUIRE(al16(t) && al16(w_folded) && al16(C) && al16(bias_folded) && al16(colsum) && (!residual || al16(residual)) &&
-                   (!y || (al16(y) && al16(gamma) && al16(beta))),
-               TNN_ROCM_EALIGN, "gemm_ln: pointers must be 16-byte aligned");
+                   (!y || (al16(y) && al16(gamma) && al16(beta))) && (((uintptr_t)row_stats) & 7u) == 0,
+               TNN_ROCM_EALIGN, "gemm_ln: pointers must be 16-byte aligned (row_stats: 8-byte)");
 #define TR_LN(DT)                                                                                                     \
     {                                                                                                                 \
         LnFloatEpilogue<DT> epi;                                                                                      \
@@ -1669,7 +1740,7 @@ int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folde
         epi.residual = (const Elem<DT>::type *)residual;                                                              \
         epi.C        = (Elem<DT>::type *)C;                                                                           \
         epi.ldc      = N;                                                                                             \
-        epi.ln       = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead};                                          \
+        epi.ln       = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead.load(), (float2 *)row_stats};                                          \
         return launch_gemm_fast<DT, LnFloatEpilogue<DT>>((hipStream_t)stream, t, w_folded, M, N, K, K, K, epi);       \
     }
     if (dtype == TNN_ROCM_F16)
@@ -1681,7 +1752,7 @@ int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folde
 
 int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const void *wqkv_folded, const float *bqkv_folded,
                                const float *colsum, const float *gamma, const float *beta, float eps, void *qk, void *vt,
-                               void *y, int B, int S, int heads, int K) {
+                               void *y, float *row_stats, int B, int S, int heads, int K) {
     TR_REQUIRE(B >= 0 && S >= 0 && heads >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_qkv_split_ln: negative size");
     if (B == 0 || S == 0 || heads == 0)
         return 0;
@@ -1693,8 +1764,8 @@ int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const voi
     TR_REQUIRE((long)B * S < (1l << 24) && (long)B * S * 3 * heads * 64 < (1l << 31), TNN_ROCM_ESHAPE,
                "gemm_qkv_split_ln: problem too large for 32-bit panel offsets");
     TR_REQUIRE(al16(t) && al16(wqkv_folded) && al16(qk) && al16(vt) && al16(bqkv_folded) && al16(colsum) &&
-                   (!y || (al16(y) && al16(gamma) && al16(beta))),
-               TNN_ROCM_EALIGN, "gemm_qkv_split_ln: pointers must be 16-byte aligned");
+                   (!y || (al16(y) && al16(gamma) && al16(beta))) && (((uintptr_t)row_stats) & 7u) == 0,
+               TNN_ROCM_EALIGN, "gemm_qkv_split_ln: pointers must be 16-byte aligned (row_stats: 8-byte)");
     const int H = heads * 64, T = B * S;
 #define TR_QKVLN(DT)                                                                                                  \
     {                                                                                                                 \
@@ -1705,7 +1776,7 @@ int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const voi
         epi.H     = H;                                                                                                \
         epi.S     = S;                                                                                                \
         epi.heads = heads;                                                                                            \
-        epi.ln    = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead};                                             \
+        epi.ln    = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead.load(), (float2 *)row_stats};                                             \
         return launch_gemm_fast<DT, LnQkvSplitEpilogue<DT>>((hipStream_t)stream, t, wqkv_folded, T, 3 * H, K, K, K, epi); \
     }
     if (dtype == TNN_ROCM_F16)
@@ -1715,6 +1786,44 @@ int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const voi
 #undef TR_QKVLN
 }
 
+int tnn_rocm_gemm_residual_ln(void *stream, int dtype, const void *x, const void *w, const float *bias, void *C,
+                              const void *t, const float *row_stats, const float *gamma, const float *beta, int M, int N,
+                              int K, int flags) {
+    TR_REQUIRE(M >= 0 && N >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_residual_ln: negative size");
+    if (M == 0 || N == 0)
+        return 0;
+    TR_REQUIRE(x && w && C && t && row_stats && gamma && beta, TNN_ROCM_EINVAL, "gemm_residual_ln: null pointer");
+    TR_REQUIRE(!(flags & TNN_ROCM_EPI_BIAS) || bias, TNN_ROCM_EINVAL, "gemm_residual_ln: bias flag without a bias");
+    TR_REQUIRE(!(flags & ~(TNN_ROCM_EPI_BIAS | TNN_ROCM_EPI_GELU)), TNN_ROCM_EINVAL,
+               "gemm_residual_ln: flags may name bias and GELU only (the residual is the rebuilt LayerNorm)");
+    TR_REQUIRE(dtype == TNN_ROCM_F16 || dtype == TNN_ROCM_BF16, TNN_ROCM_EDTYPE, "gemm_residual_ln: F16 or BF16 only");
+    TR_REQUIRE(K > 0 && K % 64 == 0 && N % 8 == 0, TNN_ROCM_ESHAPE,
+               "gemm_residual_ln: K=%d must be a positive multiple of 64 and N=%d a multiple of 8", K, N);
+    TR_REQUIRE((long)M < (1l << 24) && (long)M * K < (1l << 31) && (long)N * K < (1l << 31) && (long)M * N < (1l << 31),
+               TNN_ROCM_ESHAPE, "gemm_residual_ln: problem too large for 32-bit panel offsets");
+    TR_REQUIRE(al16(x) && al16(w) && al16(C) && al16(t) && al16(gamma) && al16(beta) && (!bias || al16(bias)) &&
+                   (((uintptr_t)row_stats) & 7u) == 0,
+               TNN_ROCM_EALIGN, "gemm_residual_ln: pointers must be 16-byte aligned (row_stats: 8-byte)");
+#define TR_LNRES(DT)                                                                                                  \
+    {                                                                                                                 \
+        LnResidualEpilogue<DT> epi;                                                                                   \
+        epi.flags = flags;                                                                                            \
+        epi.bias  = bias;                                                                                             \
+        epi.t     = (const Elem<DT>::type *)t;                                                                        \
+        epi.st    = (const float2 *)row_stats;                                                                        \
+        epi.gamma = gamma;                                                                                            \
+        epi.beta  = beta;                                                                                             \
+        epi.C     = (Elem<DT>::type *)C;                                                                              \
+        epi.ldc   = N;                                                                                                \
+        return launch_gemm_fast<DT, LnResidualEpilogue<DT>>((hipStream_t)stream, x, w, M, N, K, K, K, epi);           \
+    }
+    if (dtype == TNN_ROCM_F16)
+        TR_LNRES(TNN_ROCM_F16)
+    else
+        TR_LNRES(TNN_ROCM_BF16)
+#undef TR_LNRES
+}
+
 // Experiment hook (not part of the documented ABI): 0 restores the shape heuristic, -1 forces the baseline
 // kernel, other values select a configuration code of the tiled kernel.
 __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_config(int cfg) {
@@ -1722,6 +1831,7 @@ __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_config(int cf
     return 0;
 }
 __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_tune(const char *spec) {
+    std::lock_guard<std::mutex> hold(g_tune_lock);
     parse_tune(spec);
     return 0;
 }

@@ -5,7 +5,9 @@
 //   cd tnn_amd/csrc && hipcc --offload-arch=gfx950 -O3 -std=c++17 -ffp-contract=off -Xclang -target-feature -Xclang \
 //       -packed-fp32-ops -I ../../include -I . probe_gemm_timeline.hip runtime.hip -o ../lib/probe_gemm_timeline
 //   ../lib/probe_gemm_timeline N K mode        (M = 3072 tokens; mode 0 bias, 1 bias + GELU, 2 LayerNorm folded +
-//                                               GELU + LayerNorm output, 3 bias + residual)
+//                                               GELU + LayerNorm output, 3 bias + residual, 4 as 2 with the row
+//                                               statistics instead of the LayerNorm output, 5 bias + a residual
+//                                               rebuilt from the raw tensor and the row statistics)
 // The kernels are compiled from gemm.hip itself with the timeline stamps switched on.
 #define TNN_ROCM_TIMELINE 1
 #include "gemm.hip"
@@ -22,7 +24,7 @@ int main(int argc, char **argv) {
     }
     const int M = 3072, N = atoi(argv[1]), K = atoi(argv[2]), mode = atoi(argv[3]);
     _Float16 *A, *B, *C, *Y, *R;
-    float *bias, *cs, *g, *be;
+    float *bias, *cs, *g, *be, *stats, *gn, *bn;
     (void)hipMalloc(&A, (size_t)M * K * 2);
     (void)hipMalloc(&B, (size_t)N * K * 2);
     (void)hipMalloc(&C, (size_t)M * N * 2);
@@ -39,11 +41,20 @@ int main(int argc, char **argv) {
     (void)hipMemset(cs, 0, N * 4);
     (void)hipMemset(g, 0, K * 4);
     (void)hipMemset(be, 0, K * 4);
+    (void)hipMalloc(&stats, (size_t)M * 8);
+    (void)hipMalloc(&gn, N * 4);
+    (void)hipMalloc(&bn, N * 4);
+    (void)hipMemset(stats, 0, (size_t)M * 8);
+    (void)hipMemset(gn, 0, N * 4);
+    (void)hipMemset(bn, 0, N * 4);
     hipStream_t s;
     (void)hipStreamCreate(&s);
     auto call = [&]() {
-        if (mode == 2)
-            return tnn_rocm_gemm_ln(s, TNN_ROCM_F16, A, B, bias, cs, g, be, 1e-12f, C, Y, M, N, K, TNN_ROCM_EPI_GELU, nullptr);
+        if (mode == 2 || mode == 4)  // LayerNorm folded in; its output written (2) or the row statistics handed on (4)
+            return tnn_rocm_gemm_ln(s, TNN_ROCM_F16, A, B, bias, cs, g, be, 1e-12f, C, mode == 2 ? Y : nullptr,
+                                    mode == 4 ? stats : nullptr, M, N, K, TNN_ROCM_EPI_GELU, nullptr);
+        if (mode == 5)  // bias + a LayerNorm output rebuilt from the raw tensor as the residual
+            return tnn_rocm_gemm_residual_ln(s, TNN_ROCM_F16, A, B, bias, C, R, stats, gn, bn, M, N, K, TNN_ROCM_EPI_BIAS);
         const int fl = TNN_ROCM_EPI_BIAS | (mode == 1 ? TNN_ROCM_EPI_GELU : 0) | (mode == 3 ? TNN_ROCM_EPI_RESIDUAL : 0);
         return tnn_rocm_gemm(s, TNN_ROCM_F16, 1, A, B, C, M, N, K, K, K, N, 1, 1, 1, fl, bias, mode == 3 ? R : nullptr, N);
     };

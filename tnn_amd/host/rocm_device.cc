@@ -33,6 +33,8 @@ RocmContext::~RocmContext() {
     if (stream_)
         tnn_rocm_stream_sync(stream_);
     tnn_rocm_free(workspace_);
+    for (auto &kv : side_buffers_)
+        tnn_rocm_free(kv.second.ptr);
     tnn_rocm_free(mask_cache_.mask_f32);
     tnn_rocm_free(mask_cache_.kv_len);
     tnn_rocm_free_host(error_flag_);
@@ -111,6 +113,23 @@ Status RocmContext::Workspace(size_t bytes, void **ptr) {
         workspace_sz_ = want;
     }
     *ptr = workspace_;
+    return TNN_OK;
+}
+
+Status RocmContext::SideBuffer(const std::string &name, size_t bytes, void **ptr) {
+    auto &e = side_buffers_[name];
+    if (bytes > e.cap) {
+        ROCM_CALL(tnn_rocm_stream_sync(stream_));
+        tnn_rocm_free(e.ptr);
+        e.ptr = nullptr;
+        e.cap = 0;
+        ++memory_epoch_;
+        int rc = tnn_rocm_malloc(&e.ptr, bytes);
+        if (rc != 0)
+            return RocmStatus(rc, TNNERR_OUTOFMEMORY, "side buffer allocation");
+        e.cap = bytes;
+    }
+    *ptr = e.ptr;
     return TNN_OK;
 }
 
@@ -275,7 +294,10 @@ Status RocmLayerAcc::ReloadConstantBlobs(const std::vector<Blob *> &inputs, bool
 class RocmBlobConverterAcc : public BlobConverterAcc {
 public:
     explicit RocmBlobConverterAcc(Blob *blob) : BlobConverterAcc(blob) {}
-    ~RocmBlobConverterAcc() override { tnn_rocm_free(staging_); }
+    ~RocmBlobConverterAcc() override {
+        tnn_rocm_free(staging_);
+        tnn_rocm_free_host(bounce_);
+    }
 
     Status ConvertFromMat(Mat &mat, MatConvertParam param, void *q) override {
         RETURN_ON_NEQ(ConvertFromMatAsync(mat, param, q), TNN_OK);
@@ -360,7 +382,7 @@ public:
         if (mat.GetMatType() != NCHW_FLOAT)
             return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported mat type");
         if (desc.data_type == DATA_TYPE_FLOAT) {
-            ROCM_CALL(tnn_rocm_memcpy_d2h(mat.GetData(), src, count * 4, q));
+            RETURN_ON_NEQ(ToHost(mat.GetData(), src, count * 4, q), TNN_OK);
         } else {
             RETURN_ON_NEQ(Staging(count * 4), TNN_OK);
             if (desc.data_type == DATA_TYPE_HALF || desc.data_type == DATA_TYPE_BFP16) {
@@ -374,7 +396,7 @@ public:
             } else {
                 return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported blob data type");
             }
-            ROCM_CALL(tnn_rocm_memcpy_d2h(mat.GetData(), staging_, count * 4, q));
+            RETURN_ON_NEQ(ToHost(mat.GetData(), staging_, count * 4, q), TNN_OK);
         }
         if (NeedsScaleBias(param, desc.dims)) {
             std::vector<float> tmp(count);
@@ -420,8 +442,37 @@ private:
         }
         return TNN_OK;
     }
+    // Device to host.  A Mat's memory is pageable, and a copy into pageable memory is staged by the runtime in small
+    // pieces on one thread (about 8 GB/s: 1.1 ms for the 9.4 MB fp32 output of a batch-8 encoder).  Large outputs
+    // therefore go by DMA into a page-locked buffer the converter keeps, and from there into the Mat on a few threads.
+    Status ToHost(void *host_dst, const void *dev_src, size_t bytes, void *q) {
+        if (bytes < kBounceMinBytes) {
+            ROCM_CALL(tnn_rocm_memcpy_d2h(host_dst, dev_src, bytes, q));
+            return TNN_OK;
+        }
+        if (bytes > bounce_sz_) {
+            tnn_rocm_free_host(bounce_);
+            bounce_    = nullptr;
+            bounce_sz_ = 0;
+            int rc     = tnn_rocm_malloc_host(&bounce_, bytes);
+            if (rc != 0)
+                return RocmStatus(rc, TNNERR_OUTOFMEMORY, "converter page-locked buffer");
+            bounce_sz_ = bytes;
+        }
+        ROCM_CALL(tnn_rocm_memcpy_d2h(bounce_, dev_src, bytes, q));
+        const int parts = bytes >= (4u << 20) ? 4 : 2;
+#pragma omp parallel for num_threads(parts) schedule(static)
+        for (int i = 0; i < parts; ++i) {
+            size_t lo = (bytes / parts * i) & ~(size_t)63, hi = i + 1 == parts ? bytes : (bytes / parts * (i + 1)) & ~(size_t)63;
+            memcpy((char *)host_dst + lo, (const char *)bounce_ + lo, hi - lo);
+        }
+        return TNN_OK;
+    }
+    static constexpr size_t kBounceMinBytes = 1u << 20;
     void *staging_     = nullptr;
     size_t staging_sz_ = 0;
+    void *bounce_      = nullptr;
+    size_t bounce_sz_  = 0;
 };
 
 DECLARE_BLOB_CONVERTER_CREATER(Rocm);

@@ -27,6 +27,9 @@
 #else
 #include "tnn_host.h"
 #endif
+#include <map>
+#include <string>
+
 #include "tnn_rocm.h"
 
 namespace TNN_NS {
@@ -57,6 +60,10 @@ public:
     void *Stream() { return stream_; }
     // grow-only scratch owned by the context; valid until the next call with a larger size
     Status Workspace(size_t bytes, void **ptr);
+    // Small named device buffers that one layer of a forward writes and a later one reads without a blob in between
+    // (the rows' LayerNorm statistics: fp32 in a net whose blobs are half precision).  Grow-only per name; a
+    // (re)allocation counts as a memory epoch.
+    Status SideBuffer(const std::string &name, size_t bytes, void **ptr);
     // page-locked word kernels raise on a data error (e.g. Gather index out of range)
     int32_t *ErrorFlag() { return error_flag_; }
     // The padding mask is one blob shared by every attention layer of a forward pass: the first layer that asks
@@ -79,6 +86,11 @@ private:
         size_t cap_mask = 0, cap_len = 0;  // elements allocated (grow-only, so recorded launch sequences stay valid)
         void *mask_f32 = nullptr, *kv_len = nullptr;
     } mask_cache_;
+    struct SideEntry {
+        void *ptr  = nullptr;
+        size_t cap = 0;
+    };
+    std::map<std::string, SideEntry> side_buffers_;
 };
 
 class RocmDevice : public AbstractDevice {

@@ -29,6 +29,8 @@ struct RocmFusedLinearResource : public LayerResource {
     RawBuffer bias;       // [N] fp32 (may be empty)
     // scale / shift ([K] fp32) of a LayerNorm folded into this layer (the one whose output was the A operand)
     RawBuffer ln_gamma, ln_beta;
+    // scale / shift ([N] fp32) of the LayerNorm whose output is this layer's residual operand (residual_ln)
+    RawBuffer residual_gamma, residual_beta;
 };
 
 struct RocmFusedLinearParam : public LayerParam {
@@ -42,6 +44,12 @@ struct RocmFusedLinearParam : public LayerParam {
     // itself for the other readers of that tensor.
     int ln_fold = 0, ln_y = 0;
     float ln_eps = 0.f;
+    // ln_stats: instead of LayerNorm(x) the layer leaves every row's {rstd, mean} in the context's side buffer named
+    // ln_stats_key, for the one other reader of that tensor, which is a RocmFusedLinear with residual_ln: its second
+    // input is then the tensor the LayerNorm read, and it adds LayerNorm(that tensor), rebuilt from the statistics
+    // under residual_ln_key and its resource's residual_gamma / residual_beta (RocmFusionPass::HandOverRowStatistics).
+    int ln_stats = 0, residual_ln = 0;
+    std::string ln_stats_key, residual_ln_key;
 };
 struct RocmFusedAttentionParam : public LayerParam {
     int heads    = 0;
@@ -54,8 +62,9 @@ struct RocmFusedAttentionParam : public LayerParam {
     int quant = 0;
     float qkv_out_scale[3] = {0.f, 0.f, 0.f};
     // LayerNorm folded into the QKV projection, as in RocmFusedLinearParam
-    int ln_fold = 0, ln_y = 0;
+    int ln_fold = 0, ln_y = 0, ln_stats = 0;
     float ln_eps = 0.f;
+    std::string ln_stats_key;
     // the last output blob is int8: the context quantised as the Reformat layer that followed would (ROCm int8 pass)
     int out_quant = 0;
 };

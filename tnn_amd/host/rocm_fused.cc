@@ -65,6 +65,9 @@ public:
         const char *fold = getenv("TNN_ROCM_FOLD_LN");
         if (half_ && !(fold && fold[0] == '0'))
             FoldLayerNorm();
+        const char *hand = getenv("TNN_ROCM_LN_STATS");  // "0" keeps the LayerNorm output of a folding layer a tensor
+        if (half_ && !(fold && fold[0] == '0') && !(hand && hand[0] == '0'))
+            HandOverRowStatistics();
         return TNN_OK;
     }
 
@@ -563,6 +566,50 @@ private:
             L[li] = nullptr;
         }
         Compact();
+    }
+
+    // A folding layer (above) that still writes y = LayerNorm(t) because ONE other layer reads it, and that layer is a
+    // RocmFusedLinear taking y as its residual operand (the block's residual Add): the folding layer hands over the
+    // rows' {rstd, mean} instead (8 bytes per row, context side buffer named after y) and the residual reader takes t
+    // and rebuilds y's values in its epilogue.  y is then neither written nor read: one tensor write and one tensor
+    // read less per LayerNorm, same arithmetic per value.
+    void HandOverRowStatistics() {
+        auto &L = structure_->layers;
+        for (int li = 0; li < (int)L.size(); ++li) {
+            auto p = L[li];
+            if (!p || (p->type != LAYER_ROCM_FUSED_LINEAR && p->type != LAYER_ROCM_FUSED_ATTENTION) || p->outputs.size() != 2)
+                continue;
+            auto pl = ParamOf<RocmFusedLinearParam>(p);
+            auto pa = ParamOf<RocmFusedAttentionParam>(p);
+            if (!(pl ? pl->ln_fold && pl->ln_y : pa && pa->ln_fold && pa->ln_y && !pa->out_quant))
+                continue;
+            auto pr = ResOf<RocmFusedLinearResource>(p->name);
+            const std::string t = p->inputs[0], y = p->outputs[1];
+            GraphIndex g(L);
+            int ri = g.sole_consumer(y);
+            if (!pr || ri <= li || IsModelOutput(y))
+                continue;
+            auto r  = L[ri];
+            auto rp = r && r->type == LAYER_ROCM_FUSED_LINEAR ? ParamOf<RocmFusedLinearParam>(r) : nullptr;
+            auto rr = rp ? ResOf<RocmFusedLinearResource>(r->name) : nullptr;
+            if (!rp || !rr || !rp->has_residual || rp->ln_fold || rp->residual_ln || rp->axis >= 0 || r->inputs.size() != 2 ||
+                r->inputs[1] != y || r->inputs[0] == y)
+                continue;
+            auto wd     = rr->weight_nk.GetBufferDims();
+            const int C = pr->ln_gamma.GetDataCount();
+            if (wd.size() != 2 || wd[0] != C || wd[1] % 64 != 0 || C % 8 != 0 || pr->ln_beta.GetDataCount() != C)
+                continue;
+            if (pl)
+                pl->ln_y = 0, pl->ln_stats = 1, pl->ln_stats_key = y;
+            else
+                pa->ln_y = 0, pa->ln_stats = 1, pa->ln_stats_key = y;
+            p->outputs.pop_back();
+            r->inputs[1]        = t;
+            rp->residual_ln     = 1;
+            rp->residual_ln_key = y;
+            rr->residual_gamma  = pr->ln_gamma;
+            rr->residual_beta   = pr->ln_beta;
+        }
     }
 
     NetStructure *structure_ = nullptr;
@@ -1066,6 +1113,16 @@ public:
                 return Status(TNNERR_PARAM_ERR, "fused linear: residual must have the output's shape and type");
         }
         DataType dt = inputs[0]->GetBlobDesc().data_type;
+        if (p->residual_ln) {
+            if ((dt != DATA_TYPE_HALF && dt != DATA_TYPE_BFP16) || p->ln_fold || !p->has_residual || wd[1] % 64 != 0 || wd[0] % 8 != 0 ||
+                res->residual_gamma.GetDataCount() != wd[0] || res->residual_beta.GetDataCount() != wd[0])
+                return Status(TNNERR_PARAM_ERR, "fused linear with a rebuilt LayerNorm residual: fp16/bf16 blobs, K a multiple "
+                                                "of 64 and scale / shift of the output width are required");
+            RETURN_ON_NEQ(UploadConverted(res->residual_gamma.force_to<void *>(), (size_t)wd[0], DATA_TYPE_FLOAT, DATA_TYPE_FLOAT,
+                                          &res_gamma_), TNN_OK);
+            RETURN_ON_NEQ(UploadConverted(res->residual_beta.force_to<void *>(), (size_t)wd[0], DATA_TYPE_FLOAT, DATA_TYPE_FLOAT,
+                                          &res_beta_), TNN_OK);
+        }
         if (p->ln_fold) {
             if ((dt != DATA_TYPE_HALF && dt != DATA_TYPE_BFP16) || outputs.size() != (p->ln_y ? 2u : 1u) || in.back() != wd[1] ||
                 wd[1] % 128 != 0 || wd[0] % 8 != 0 || res->ln_gamma.GetDataCount() != wd[1] || res->ln_beta.GetDataCount() != wd[1])
@@ -1099,10 +1156,22 @@ public:
         int epi = (p->has_bias ? TNN_ROCM_EPI_BIAS : 0) | (p->gelu ? TNN_ROCM_EPI_GELU : 0) |
                   (p->has_residual ? TNN_ROCM_EPI_RESIDUAL : 0);
         if (p->ln_fold) {
+            void *stats = nullptr;
+            if (p->ln_stats)
+                RETURN_ON_NEQ(context_->SideBuffer(p->ln_stats_key, (size_t)rows * 2 * sizeof(float), &stats), TNN_OK);
             ROCM_CALL(tnn_rocm_gemm_ln(Stream(), (int)inputs[0]->GetBlobDesc().data_type, Ptr(inputs[0]), weight_,
                                        (const float *)bias_, (const float *)colsum_, (const float *)gamma_, (const float *)beta_,
-                                       p->ln_eps, Ptr(outputs[0]), p->ln_y ? Ptr(outputs[1]) : nullptr, rows, N, K,
-                                       epi & ~TNN_ROCM_EPI_BIAS, p->has_residual ? Ptr(In(inputs[1])) : nullptr));
+                                       p->ln_eps, Ptr(outputs[0]), p->ln_y ? Ptr(outputs[1]) : nullptr, (float *)stats, rows, N,
+                                       K, epi & ~TNN_ROCM_EPI_BIAS, p->has_residual ? Ptr(In(inputs[1])) : nullptr));
+            return TNN_OK;
+        }
+        if (p->residual_ln) {
+            void *stats = nullptr;
+            RETURN_ON_NEQ(context_->SideBuffer(p->residual_ln_key, (size_t)rows * 2 * sizeof(float), &stats), TNN_OK);
+            ROCM_CALL(tnn_rocm_gemm_residual_ln(Stream(), (int)inputs[0]->GetBlobDesc().data_type, Ptr(inputs[0]), weight_,
+                                                (const float *)bias_, Ptr(outputs[0]), Ptr(In(inputs[1])), (const float *)stats,
+                                                (const float *)res_gamma_, (const float *)res_beta_, rows, N, K,
+                                                epi & ~TNN_ROCM_EPI_RESIDUAL));
             return TNN_OK;
         }
         ROCM_CALL(tnn_rocm_gemm(Stream(), (int)inputs[0]->GetBlobDesc().data_type, 1, Ptr(inputs[0]), weight_, Ptr(outputs[0]),
@@ -1112,7 +1181,8 @@ public:
     }
 
 private:
-    void *weight_ = nullptr, *bias_ = nullptr, *colsum_ = nullptr, *gamma_ = nullptr, *beta_ = nullptr;
+    void *weight_ = nullptr, *bias_ = nullptr, *colsum_ = nullptr, *gamma_ = nullptr, *beta_ = nullptr, *res_gamma_ = nullptr,
+         *res_beta_ = nullptr;
 };
 REGISTER_ROCM_ACC(RocmFusedLinearLayerAcc, LAYER_ROCM_FUSED_LINEAR);
 
@@ -1202,6 +1272,9 @@ public:
         size_t es   = (size_t)DataTypeUtils::GetBytesSize(dt);
         void *qkv   = nullptr;
         RETURN_ON_NEQ(context_->Workspace((size_t)T_ * 3 * H_ * es, &qkv), TNN_OK);
+        void *stats = nullptr;  // the folded LayerNorm's {rstd, mean} per row, for the layer that rebuilds its output
+        if (p->ln_fold && p->ln_stats)
+            RETURN_ON_NEQ(context_->SideBuffer(p->ln_stats_key, (size_t)T_ * 2 * sizeof(float), &stats), TNN_OK);
         const float *mask = nullptr;
         const int32_t *kv = nullptr;
         if (p->has_mask) {
@@ -1240,8 +1313,8 @@ public:
             if (p->ln_fold)
                 ROCM_CALL(tnn_rocm_gemm_qkv_split_ln(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_,
                                                      (const float *)colsum_, (const float *)gamma_, (const float *)beta_,
-                                                     p->ln_eps, qkv, vt, p->ln_y ? Ptr(outputs[1]) : nullptr, B_, seq_,
-                                                     p->heads, H_));
+                                                     p->ln_eps, qkv, vt, p->ln_y ? Ptr(outputs[1]) : nullptr, (float *)stats,
+                                                     B_, seq_, p->heads, H_));
             else
                 ROCM_CALL(tnn_rocm_gemm_qkv_split(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_, qkv, vt,
                                                   B_, seq_, p->heads, H_));
@@ -1259,7 +1332,7 @@ public:
         if (p->ln_fold)
             ROCM_CALL(tnn_rocm_gemm_ln(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_, (const float *)colsum_,
                                        (const float *)gamma_, (const float *)beta_, p->ln_eps, qkv,
-                                       p->ln_y ? Ptr(outputs[1]) : nullptr, T_, 3 * H_, H_, 0, nullptr));
+                                       p->ln_y ? Ptr(outputs[1]) : nullptr, (float *)stats, T_, 3 * H_, H_, 0, nullptr));
         else
             ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 1, Ptr(inputs[0]), weight_, qkv, T_, 3 * H_, H_, H_, H_, 3 * H_, 1, 1, 1,
                                     TNN_ROCM_EPI_BIAS, (const float *)bias_, nullptr, 0));
