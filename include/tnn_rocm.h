@@ -197,27 +197,39 @@ TNN_ROCM_API int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x,
  * y (optional, [M,K] in dtype) receives LayerNorm(t) itself for the other readers of that tensor (needs gamma, beta).
  * row_stats (optional, [M][2] fp32) receives {rstd, mean} of every row instead, for a reader that rebuilds
  * LayerNorm(t) from t on the fly (tnn_rocm_gemm_residual_ln).
+ * row_sums (optional, [row_sum_blocks][M][2] fp32, as left by tnn_rocm_gemm_residual_ln when it wrote t): every row's
+ * sum and sum of squares per block of columns of t; the kernel then adds those up instead of taking the statistics
+ * from the A tiles.  At most TNN_ROCM_MAX_ROW_SUM_BLOCKS blocks.
  * flags: TNN_ROCM_EPI_GELU, TNN_ROCM_EPI_RESIDUAL (residual [M,N] in dtype).  dtype F16 or BF16; K a multiple of 128
  * (the whole normalised row is one GEMM row), N a multiple of 8; all tensors dense row-major. */
 TNN_ROCM_API int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folded, const float *bias_folded,
                                   const float *colsum, const float *gamma, const float *beta, float eps, void *C, void *y,
-                                  float *row_stats, int M, int N, int K, int flags, const void *residual);
+                                  float *row_stats, const float *row_sums, int row_sum_blocks, int M, int N, int K,
+                                  int flags, const void *residual);
 
 /* tnn_rocm_gemm_qkv_split on LayerNorm(t), folded the same way (wqkv_folded, bqkv_folded, colsum over the 3H rows). */
 TNN_ROCM_API int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const void *wqkv_folded,
                                             const float *bqkv_folded, const float *colsum, const float *gamma,
                                             const float *beta, float eps, void *qk, void *vt, void *y,
-                                            float *row_stats, int B, int S, int heads, int K);
+                                            float *row_stats, const float *row_sums, int row_sum_blocks, int B,
+                                            int S, int heads, int K);
 
 /* C = act(x W^T + b) + LayerNorm(t), the residual Add of a transformer block whose residual operand is the output of
  * a LayerNorm layer (compute_elewise.cc:37-65 after cpu_layer_norm_layer_acc.cc:86-135), without that output ever
  * being stored: t[M,N] is the tensor the LayerNorm read, row_stats[M][2] = {rstd, mean} per row as left by
  * tnn_rocm_gemm_ln / tnn_rocm_gemm_qkv_split_ln on the same t, gamma / beta [N] the LayerNorm's scale and shift; each
  * value is formed as t * rstd * gamma + (beta - mean * rstd * gamma).  x[M,K], W[N,K], C[M,N] dense row-major in dtype
- * (F16 or BF16); K a multiple of 64, N a multiple of 8.  flags: TNN_ROCM_EPI_BIAS, TNN_ROCM_EPI_GELU. */
+ * (F16 or BF16); K a multiple of 64, N a multiple of 8.  flags: TNN_ROCM_EPI_BIAS, TNN_ROCM_EPI_GELU.
+ * row_sums (optional, room for TNN_ROCM_MAX_ROW_SUM_BLOCKS * M pairs of fp32) receives, per block of columns of C (one
+ * block per tile column of the launch) and row, the sum and the sum of squares of the values stored, for a
+ * LayerNorm-folding GEMM that reads C next; *row_sum_blocks receives the number of blocks written, 0 if none were
+ * (N above 64 * TNN_ROCM_MAX_ROW_SUM_BLOCKS, or a tile shape with no room for them): the reader then takes the
+ * statistics itself. */
+#define TNN_ROCM_MAX_ROW_SUM_BLOCKS 24
 TNN_ROCM_API int tnn_rocm_gemm_residual_ln(void *stream, int dtype, const void *x, const void *w, const float *bias,
                                            void *C, const void *t, const float *row_stats, const float *gamma,
-                                           const float *beta, int M, int N, int K, int flags);
+                                           const float *beta, int M, int N, int K, int flags, float *row_sums,
+                                           int *row_sum_blocks);
 
 /* kv_len[b] = 1 + the last key index whose additive mask value is > threshold; S if there is none (a padding-only
  * sequence: the reference's softmax(scores + mask) over all S keys is unchanged by the constant shift, so every key

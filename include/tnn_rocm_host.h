@@ -58,6 +58,11 @@ void *tnn_host_stream(void *handle);
 /* Instance::GetOutputMat (instance.h:128) converted to fp32 NCHW on the host.  dims must hold 8 ints. */
 int tnn_host_get_output(void *handle, const char *name, float *out, size_t capacity, int *dims, int *ndims);
 
+/* The loop of the engine's benchmark tool (test/test.cc:101-152): `warmup` untimed and `iters` timed iterations of
+ * SetInputMat for every input set so far (host copies of those Mats are kept), Forward, GetOutputMat(out_name) as
+ * fp32 NCHW on the host.  stats[3] = {min, avg, max} seconds per iteration. */
+int tnn_host_time_loop(void *handle, int warmup, int iters, const char *out_name, double *stats);
+
 /* The optimised layer list ("Type name\n" per layer) and per-layer timing with events on the instance's stream
  * (the engine's TNN_PROFILE facility, reference source/tnn/core/profile.h:29-100).  only_type NULL or "" times every
  * layer.  tnn_host_profile_finish fills up to `capacity` mean milliseconds (layer order) and returns the layer count. */

@@ -394,8 +394,8 @@ def test_encoder_bf16_from_model_files():
 
 def test_layernorm_folding_switch(monkeypatch):
     """TNN_ROCM_FOLD_LN=0 keeps every LayerNorm a launch of its own, TNN_ROCM_LN_STATS=0 keeps the output tensor of a
-    folded LayerNorm for the residual that reads it; all three graphs agree with each other to fp16 rounding and with
-    the checker."""
+    folded LayerNorm for the residual that reads it, TNN_ROCM_LN_SUMS=0 makes every folding GEMM take the row statistics
+    from its own operand; all four graphs agree with each other to fp16 rounding and with the checker."""
     host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
     say("host: LayerNorm folding on / off, 2-layer encoder fp16")
     cfg = EncoderConfig.bert_base(2)
@@ -410,9 +410,10 @@ def test_layernorm_folding_switch(monkeypatch):
     ids, seg, lens, mask = make_inputs(cfg, B, S, 30, S, seed=15)
     g = tnnmodel.encoder_graph(cfg, w, B, S)
     outs = {}
-    for fold, n_ln in (("0", 4), ("1", 1), ("y", 1)):
+    for fold, n_ln in (("0", 4), ("1", 1), ("y", 1), ("s", 1)):
         monkeypatch.setenv("TNN_ROCM_FOLD_LN", "0" if fold == "0" else "1")
         monkeypatch.setenv("TNN_ROCM_LN_STATS", "0" if fold == "y" else "1")
+        monkeypatch.setenv("TNN_ROCM_LN_SUMS", "0" if fold == "s" else "1")
         inst = host.RocmInstance.from_graph(g, "fp16")
         types = [t for t, _ in inst.layers()]
         assert types.count("LayerNorm") == n_ln, types
@@ -427,9 +428,10 @@ def test_layernorm_folding_switch(monkeypatch):
     ref = encoder_ref.encoder(wr, cfg, encoder_ref.embed(wr, ids, seg, cfg.eps), B, S, mask)
     e0, e1, e01 = rel_err(outs["0"], ref), rel_err(outs["1"], ref), rel_err(outs["1"], outs["0"])
     ey, e1y = rel_err(outs["y"], ref), rel_err(outs["1"], outs["y"])
-    say("  un-folded %.3g  folded %.3g  folded, output kept %.3g  folded vs un-folded %.3g  vs output kept %.3g"
-        % (e0, e1, ey, e01, e1y))
-    assert e0 <= FP16_TOL and e1 <= FP16_TOL and ey <= FP16_TOL and e01 <= FP16_TOL and e1y <= FP16_TOL
+    es, e1s = rel_err(outs["s"], ref), rel_err(outs["1"], outs["s"])
+    say("  un-folded %.3g  folded %.3g  folded, output kept %.3g  folded, own statistics %.3g  folded vs un-folded %.3g  "
+        "vs output kept %.3g  vs own statistics %.3g" % (e0, e1, ey, es, e01, e1y, e1s))
+    assert max(e0, e1, ey, es, e01, e1y, e1s) <= FP16_TOL
 
 
 @pytest.mark.parametrize("hidden,heads,ffn,B,S,n_ln", [
@@ -500,13 +502,17 @@ def test_model_check_and_profile_report():
     assert text.count("RocmFusedLinear") >= 12   # six layers in each of the two per-layer tables
 
 
-def test_model_check_device_against_cpu_checker_blob_by_blob():
+@pytest.mark.parametrize("keep_ln_outputs", [False, True])
+def test_model_check_device_against_cpu_checker_blob_by_blob(keep_ln_outputs, monkeypatch):
     """tools/model_check's comparison proper: every blob of the fused fp16 graph that survives the optimiser passes
     against the same blob as the CPU evaluates the decomposed graph (tests/encoder_ref.encoder_blobs, the CPU checker
-    layer by layer), plus the engine's own element-wise pass rule."""
+    layer by layer), plus the engine's own element-wise pass rule.  By default the LayerNorm outputs inside a layer are
+    rebuilt by their readers and never exist; TNN_ROCM_LN_STATS=0 keeps them as blobs, and they are checked as well."""
     host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
     from tnn_amd import model_check
-    say("host: model_check, device vs CPU checker, 3-layer encoder fp16")
+    say("host: model_check, device vs CPU checker, 3-layer encoder fp16, LayerNorm outputs %s"
+        % ("kept" if keep_ln_outputs else "rebuilt by their readers"))
+    monkeypatch.setenv("TNN_ROCM_LN_STATS", "0" if keep_ln_outputs else "1")
     cfg = EncoderConfig.bert_base(3)
     w = make_weights(cfg, seed=31, bias_std=0.02)
     B, S = 2, 96
@@ -519,8 +525,9 @@ def test_model_check_device_against_cpu_checker_blob_by_blob():
     assert same and not skipped, skipped
     names = {r["blob"] for r in rows}
     # what survives per layer: the attention context, the three sums the LayerNorms read (outputs of the projections
-    # with the residual folded in), the LayerNorm outputs still needed as residuals, the FFN activation
-    assert {"x0", "l0_ctx", "l0_sum1", "l0_x1", "l0_act", "l0_sum2", "l2_ctx", "last_hidden"} <= names, sorted(names)
+    # with the residual folded in), the FFN activation, and (when kept) the LayerNorm outputs needed as residuals
+    assert {"x0", "l0_ctx", "l0_sum1", "l0_act", "l0_sum2", "l2_ctx", "last_hidden"} <= names, sorted(names)
+    assert ({"l0_x1", "l0_x2", "l1_x1"} <= names) == keep_ln_outputs, sorted(names)
     assert all(r["ok"] for r in rows), [r for r in rows if not r["ok"]]
     # the engine's element rule (|d|/(|a|+|b|) > 0.005 and |d| > 1e-3) is written for an fp32 device; in fp16 a value of
     # size 1 carries an ulp of 1e-3, so a few small elements trip it as the layers stack up: they are reported per blob

@@ -944,6 +944,29 @@ def test_gemm_layernorm_folded_into_projection(M, dtype):
     xo, wo = rnd(r32(M, H) * 0.5), r32(H, H) * 0.05               # K = 768: the 64x64-tile shape
     got3 = o.gemm_residual_ln(D(xo), D(wo), D(t), st1, dev(g), dev(be), bias=dev(b2), gelu=True)
     assert rel_err(host(got3), orc.gelu(orc.inner_product(xo, rnd(wo), b2)) + y_ref) <= tol
+    # the same projections also leaving the row sums of what they stored, per tile column; a folding GEMM that is handed
+    # those sums gives the results and statistics of one that takes them from its own operand
+    for xx, ww, plain in ((x2, w2, got2), (xo, wo, None)):
+        c, (sums, blocks) = o.gemm_residual_ln(D(xx), D(ww), D(t), st1, dev(g), dev(be), bias=dev(b2), want_row_sums=True)
+        if plain is not None:
+            assert torch.equal(c, plain)
+        assert 1 <= blocks <= o.MAX_ROW_SUM_BLOCKS and H % blocks == 0
+        cf = c.float().cpu().numpy().astype(np.float64)
+        per = cf.reshape(M, blocks, H // blocks)
+        got_s = host(sums)[:blocks]                               # [blocks, M, 2]
+        assert np.abs(got_s[:, :, 0].T - per.sum(2)).max() <= 1e-3 * max(1.0, np.abs(per.sum(2)).max())
+        assert np.abs(got_s[:, :, 1].T / (per ** 2).sum(2) - 1).max() <= 1e-5
+        assert not host(sums)[blocks:].any()                      # nothing written past the blocks reported
+        own_h, own_st = o.gemm_ln(c, w1f.cuda(), dev(b1f), dev(cs1), eps, gelu=True, want_stats=True)
+        fed_h, fed_st = o.gemm_ln(c, w1f.cuda(), dev(b1f), dev(cs1), eps, gelu=True, want_stats=True, row_sums=(sums, blocks))
+        assert np.abs(host(fed_st)[:, 0] / host(own_st)[:, 0] - 1).max() <= 1e-5
+        assert np.abs(host(fed_st)[:, 1] - host(own_st)[:, 1]).max() <= 1e-5
+        assert rel_err(host(fed_h), host(own_h)) <= 2e-3
+        assert rel_err(host(fed_h), orc.gelu(orc.inner_product(orc.layernorm(cf.astype(np.float32), g, be, eps), rnd(w1), b1))) <= tol
+        own_q = o.qkv_split_ln(c, wqf.cuda(), dev(bqf), dev(csq), eps, B, S, heads, want_stats=True)
+        fed_q = o.qkv_split_ln(c, wqf.cuda(), dev(bqf), dev(csq), eps, B, S, heads, want_stats=True, row_sums=(sums, blocks))
+        assert rel_err(host(fed_q[0]), host(own_q[0])) <= 2e-3 and rel_err(host(fed_q[1]), host(own_q[1])) <= 2e-3
+        assert np.abs(host(fed_q[2])[:, 0] / host(own_q[2])[:, 0] - 1).max() <= 1e-5
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])

@@ -78,6 +78,8 @@ def test_row_statistics_hand_over_switch(monkeypatch):
         assert att["inputs"][0] == "l0_sum2" and len(att["outputs"]) == n_out
         assert out["inputs"] == ["l1_ctx", "l0_sum2" if stats == "1" else "l0_x2"]
         assert ("l0_x1" in by_out) == (stats == "0")
+        # (which layer hands its output's row sums to which folding layer is not part of the blob graph: covered on
+        # the device, where every combination of the switches must give the same encoder output)
         # layer 0 reads the embedding output, which is a LayerNorm output of the embedding layer itself: nothing to rebuild
         assert by_out["l0_sum1"]["inputs"] == ["l0_ctx", "x0"]
 

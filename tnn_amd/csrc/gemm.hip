@@ -90,6 +90,17 @@ template <> struct GemmTraits<TNN_ROCM_F32> {
 
 
 // ---- epilogues ----------------------------------------------------------------------------------
+// Optional abilities of an epilogue type, false where the type does not name them:
+//   kEmitsRowSums  the epilogue's store8 returns the sum and the sum of squares of the eight values it stored, and the
+//                  kernel leaves per tile column and row their totals over the tile's columns (LnResidualEpilogue)
+//   kTakesRowSums  a LayerNorm-folding epilogue that is handed such sums by the kernel that produced its A operand,
+//                  instead of taking them from the A fragments in the main loop
+template <typename E, typename = void> struct EmitsRowSums : std::false_type {};
+template <typename E> struct EmitsRowSums<E, typename std::enable_if<E::kEmitsRowSums>::type> : std::true_type {};
+template <typename E, typename = void> struct TakesRowSums : std::false_type {};
+template <typename E> struct TakesRowSums<E, typename std::enable_if<E::kTakesRowSums>::type> : std::true_type {};
+constexpr int kMaxRowSumBlocks = TNN_ROCM_MAX_ROW_SUM_BLOCKS;  // tile columns of a producer a consumer can add up (768 columns of 32)
+
 template <int DT> struct FloatEpilogue {
     typedef typename Elem<DT>::type T;
     static constexpr bool kRowStats = false;
@@ -155,68 +166,6 @@ template <int DT> struct FloatEpilogue {
 #pragma unroll
         for (int q = 0; q < NV; ++q)
             cp[q] = packed[q];
-    }
-};
-
-// Projection whose residual operand is LayerNorm(t) of a tensor whose row statistics an earlier kernel left behind
-// (LnFold::stats): C = act(x W^T + b) + ((t - mean) * rstd * gamma + beta).  The normalised tensor is rebuilt from t in
-// registers, in the LayerNorm kernel's half-precision form x * rstd * gamma + (beta - mean * rstd * gamma), and never
-// stored.  N is the normalised width.
-template <int DT> struct LnResidualEpilogue {
-    typedef typename Elem<DT>::type T;
-    static constexpr bool kRowStats = false;
-    int flags;  // TNN_ROCM_EPI_BIAS, TNN_ROCM_EPI_GELU
-    const float *bias;
-    const T *t;                 // [M, N]
-    const float2 *st;           // [M] {rstd, mean}
-    const float *gamma, *beta;  // [N]
-    T *C;
-    long ldc;
-    __device__ __forceinline__ void set_batch(int) {}
-    __device__ __forceinline__ float col_const(int n) const { return (flags & TNN_ROCM_EPI_BIAS) ? bias[n] : 0.f; }
-    __device__ __forceinline__ void store(int m, int n, float acc, float bias_n) const {
-        float v = acc;
-        if (flags & TNN_ROCM_EPI_BIAS)
-            v = v + bias_n;
-        if (flags & TNN_ROCM_EPI_GELU)
-            v = gelu_erf(v);
-        const float2 s = st[m];
-        const float mrs = s.y * s.x;
-        v = v + (Elem<DT>::ld(&t[(size_t)m * ldc + n]) * s.x * gamma[n] + (beta[n] - mrs * gamma[n]));
-        Elem<DT>::st(&C[(size_t)m * ldc + n], v);
-    }
-    __device__ __forceinline__ bool direct(int) const { return false; }
-    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8]) const {
-        float v[8];
-#pragma unroll
-        for (int q = 0; q < 8; ++q)
-            v[q] = acc[q];
-        if (flags & TNN_ROCM_EPI_BIAS) {
-            float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
-            v[0] += b0.x, v[1] += b0.y, v[2] += b0.z, v[3] += b0.w;
-            v[4] += b1.x, v[5] += b1.y, v[6] += b1.z, v[7] += b1.w;
-        }
-        if (flags & TNN_ROCM_EPI_GELU) {
-#pragma unroll
-            for (int q = 0; q < 8; ++q)
-                v[q] = gelu_erf_fast(v[q]);
-        }
-        static_assert(sizeof(T) == 2, "half-precision blobs only");
-        u32x4 packed = *reinterpret_cast<const u32x4 *>(t + (size_t)m * ldc + n);
-        T *pe = reinterpret_cast<T *>(&packed);
-        const float2 s = st[m];
-        const float mrs = s.y * s.x;
-        float4 k0 = *reinterpret_cast<const float4 *>(gamma + n), k1 = *reinterpret_cast<const float4 *>(gamma + n + 4);
-        float4 e0 = *reinterpret_cast<const float4 *>(beta + n), e1 = *reinterpret_cast<const float4 *>(beta + n + 4);
-        const float kk[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-        const float ee[8] = {e0.x, e0.y, e0.z, e0.w, e1.x, e1.y, e1.z, e1.w};
-#pragma unroll
-        for (int q = 0; q < 8; ++q)
-            v[q] += Elem<DT>::ld(&pe[q]) * s.x * kk[q] + (ee[q] - mrs * kk[q]);
-#pragma unroll
-        for (int q = 0; q < 8; ++q)
-            Elem<DT>::st(&pe[q], v[q]);
-        *reinterpret_cast<u32x4 *>(C + (size_t)m * ldc + n) = packed;
     }
 };
 
@@ -290,6 +239,8 @@ struct LnFold {
     void *y;                    // [M, K] in the compute type, or nullptr
     int y_ahead;                // 1: the source vectors of y are requested under the epilogue (0 for experiments)
     float2 *stats;              // [M] {rstd, mean} for a later kernel that rebuilds LayerNorm(t) itself, or nullptr
+    const float2 *row_sums;     // kTakesRowSums: [sum_blocks][M] {sum, sum of squares} over a block of columns of t
+    int sum_blocks;
 };
 
 // row sum and sum of squares of the eight values of an A fragment register quad
@@ -314,9 +265,10 @@ template <int DT> __device__ __forceinline__ void ln_accumulate(const uint4 &fra
     }
 }
 
-template <int DT> struct LnFloatEpilogue {
+template <int DT, bool SUMS = false> struct LnFloatEpilogue {
     typedef typename Elem<DT>::type T;
     static constexpr bool kRowStats = true;
+    static constexpr bool kTakesRowSums = SUMS;
     int flags;
     const float *bias;  // b' (always present)
     const T *residual;
@@ -365,9 +317,10 @@ template <int DT> struct LnFloatEpilogue {
 };
 
 // QKV projection of LayerNorm(t): QkvSplitEpilogue's layout with the folded-LayerNorm correction on the accumulators
-template <int DT> struct LnQkvSplitEpilogue {
+template <int DT, bool SUMS = false> struct LnQkvSplitEpilogue {
     typedef typename Elem<DT>::type T;
     static constexpr bool kRowStats = true;
+    static constexpr bool kTakesRowSums = SUMS;
     const float *bias;
     T *qk;
     T *vt;
@@ -404,6 +357,75 @@ template <int DT> struct LnQkvSplitEpilogue {
             for (int t = 0; t < 8; ++t)
                 Elem<DT>::st(dst + (size_t)t * S, v[t]);
         }
+    }
+};
+
+// Projection whose residual operand is LayerNorm(t) of a tensor whose row statistics an earlier kernel left behind
+// (LnFold::stats): C = act(x W^T + b) + ((t - mean) * rstd * gamma + beta).  The normalised tensor is rebuilt from t in
+// registers, in the LayerNorm kernel's half-precision form x * rstd * gamma + (beta - mean * rstd * gamma), and never
+// stored.  N is the normalised width.
+template <int DT, bool SUMS = false> struct LnResidualEpilogue {
+    typedef typename Elem<DT>::type T;
+    static constexpr bool kRowStats = false;
+    static constexpr bool kEmitsRowSums = SUMS;
+    float2 *row_sums;  // kEmitsRowSums: [tile columns][M] {sum, sum of squares} of the stored values of C
+    int flags;  // TNN_ROCM_EPI_BIAS, TNN_ROCM_EPI_GELU
+    const float *bias;
+    const T *t;                 // [M, N]
+    const float2 *st;           // [M] {rstd, mean}
+    const float *gamma, *beta;  // [N]
+    T *C;
+    long ldc;
+    __device__ __forceinline__ void set_batch(int) {}
+    __device__ __forceinline__ float col_const(int n) const { return (flags & TNN_ROCM_EPI_BIAS) ? bias[n] : 0.f; }
+    __device__ __forceinline__ void store(int m, int n, float acc, float bias_n) const {
+        float v = acc;
+        if (flags & TNN_ROCM_EPI_BIAS)
+            v = v + bias_n;
+        if (flags & TNN_ROCM_EPI_GELU)
+            v = gelu_erf(v);
+        const float2 s = st[m];
+        const float mrs = s.y * s.x;
+        v = v + (Elem<DT>::ld(&t[(size_t)m * ldc + n]) * s.x * gamma[n] + (beta[n] - mrs * gamma[n]));
+        Elem<DT>::st(&C[(size_t)m * ldc + n], v);
+    }
+    __device__ __forceinline__ bool direct(int) const { return false; }
+    __device__ __forceinline__ float2 store8(int m, int n, const float (&acc)[8]) const {
+        float v[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            v[q] = acc[q];
+        if (flags & TNN_ROCM_EPI_BIAS) {
+            float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
+            v[0] += b0.x, v[1] += b0.y, v[2] += b0.z, v[3] += b0.w;
+            v[4] += b1.x, v[5] += b1.y, v[6] += b1.z, v[7] += b1.w;
+        }
+        if (flags & TNN_ROCM_EPI_GELU) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+                v[q] = gelu_erf_fast(v[q]);
+        }
+        static_assert(sizeof(T) == 2, "half-precision blobs only");
+        u32x4 packed = *reinterpret_cast<const u32x4 *>(t + (size_t)m * ldc + n);
+        T *pe = reinterpret_cast<T *>(&packed);
+        const float2 s = st[m];
+        const float mrs = s.y * s.x;
+        float4 k0 = *reinterpret_cast<const float4 *>(gamma + n), k1 = *reinterpret_cast<const float4 *>(gamma + n + 4);
+        float4 e0 = *reinterpret_cast<const float4 *>(beta + n), e1 = *reinterpret_cast<const float4 *>(beta + n + 4);
+        const float kk[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+        const float ee[8] = {e0.x, e0.y, e0.z, e0.w, e1.x, e1.y, e1.z, e1.w};
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            v[q] += Elem<DT>::ld(&pe[q]) * s.x * kk[q] + (ee[q] - mrs * kk[q]);
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            Elem<DT>::st(&pe[q], v[q]);
+        *reinterpret_cast<u32x4 *>(C + (size_t)m * ldc + n) = packed;
+        float2 sums = make_float2(0.f, 0.f);
+        if constexpr (SUMS) {  // of the values as stored (rounded to the blob type): what the next GEMM reads
+            ln_accumulate<DT>(__builtin_bit_cast(uint4, packed), sums.x, sums.y);
+        }
+        return sums;
     }
 };
 
@@ -974,7 +996,7 @@ __global__ void __launch_bounds__(CFG::NT)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     fb[j] = *reinterpret_cast<const uint4 *>(sb + (wn * TN + j) * 32 * SLAB + frow + chunk);
-                if constexpr (Epi::kRowStats) {
+                if constexpr (Epi::kRowStats && !TakesRowSums<Epi>::value) {
                     // the WGN waves that hold the same A rows take turns over the row groups and k-steps
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
@@ -989,10 +1011,58 @@ __global__ void __launch_bounds__(CFG::NT)
             }
         };
         constexpr int LPW = A_LD + B_LD;
+        // A folding epilogue that is handed the row sums of A: the first BM threads request their row's sums (one
+        // 8-byte load per tile column of the kernel that wrote A) BEFORE the first slabs, add them up while those are
+        // on their way, and park {rstd, mean} behind everything else in LDS.  The loads are spelled as assembly like
+        // the slab loads, so that the wait can be placed by hand: they are older than every slab load, hence complete
+        // once at most the slab loads are outstanding.
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        f32x2 early[TakesRowSums<Epi>::value ? kMaxRowSumBlocks : 1];
+        if constexpr (TakesRowSums<Epi>::value) {
+            if (tid < BM) {
+                const int m = m0 + tid < M ? m0 + tid : M - 1;
+#pragma unroll
+                for (int q = 0; q < kMaxRowSumBlocks; ++q) {
+                    early[q] = f32x2{0.f, 0.f};
+                    if (q < epi.ln.sum_blocks)
+                        asm volatile("global_load_dwordx2 %0, %1, %2"
+                                     : "=v"(early[q])
+                                     : "v"((uint32_t)(((size_t)q * M + m) * sizeof(float2))), "s"(epi.ln.row_sums)
+                                     : "memory");
+                }
+            }
+        }
+        int issued = 0;
 #pragma unroll
         for (int p = 0; p < NS - 1; ++p)
             if (p < nk)
-                issue(p, p);
+                issue(p, p), ++issued;
+        if constexpr (TakesRowSums<Epi>::value) {
+            if (tid < BM) {
+                if (issued >= 2)
+                    TR_WAIT_VMCNT(2 * LPW);
+                else if (issued == 1)
+                    TR_WAIT_VMCNT(LPW);
+                else
+                    TR_WAIT_VMCNT(0);
+                double s1 = 0.0, s2 = 0.0;
+#pragma unroll
+                for (int q = 0; q < kMaxRowSumBlocks; ++q) {
+                    asm volatile("" : "+v"(early[q]));  // not to be read before the wait above
+                    if (q < epi.ln.sum_blocks) {
+                        s1 += (double)early[q].x;
+                        s2 += (double)early[q].y;
+                    }
+                }
+                // the variance as a difference of doubles; its reciprocal root in single precision with one Newton
+                // step (every other wave of the workgroup waits at the first barrier while these waves do this)
+                const double mean = s1 * (double)epi.ln.inv_cols;
+                const float ve    = (float)(s2 * (double)epi.ln.inv_cols - mean * mean + (double)epi.ln.eps);
+                float r           = __builtin_amdgcn_rsqf(ve);
+                r                 = r * (1.5f - 0.5f * ve * r * r);
+                reinterpret_cast<float2 *>(lds_dyn + CFG::lds_bytes)[tid] = make_float2(r, (float)mean);
+            }
+        }
         int stage = 0, fill = NS - 1;  // stage of slab kt; stage that slab kt + NS - 1 goes to
         for (int kt = 0; kt < nk; ++kt) {
             // slab kt has landed once at most the loads of the slabs issued after it are outstanding
@@ -1116,7 +1186,7 @@ __global__ void __launch_bounds__(CFG::NT)
     TR_TL(2);         // main loop done
     // LayerNorm-folding epilogues: reduce the lanes' partial row sums over the two k-halves of a fragment and the WGK
     // k-waves (fixed order), giving {rstd, mean} per tile row; both arrays sit behind the staging area
-    float2 *const row_st   = reinterpret_cast<float2 *>(lds_dyn + CFG::stage_bytes);  // [BM]
+    float2 *const row_st   = reinterpret_cast<float2 *>(lds_dyn + (TakesRowSums<Epi>::value ? CFG::lds_bytes : CFG::stage_bytes));  // [BM]
     float2 *const row_part = row_st + BM;                                             // [WGK * WGN * 2][BM]
     int8_t *const lut_lds = reinterpret_cast<int8_t *>(lds_dyn + CFG::stage_bytes);  // Int8Epilogue's table, 256 bytes
     if constexpr (std::is_same<Epi, Int8Epilogue>::value) {
@@ -1124,7 +1194,12 @@ __global__ void __launch_bounds__(CFG::NT)
             reinterpret_cast<uint32_t *>(lut_lds)[tid] = reinterpret_cast<const uint32_t *>(epi.lut)[tid];
         // read after the first staging barrier below
     }
-    if constexpr (Epi::kRowStats) {
+    if constexpr (Epi::kRowStats && TakesRowSums<Epi>::value) {
+        // {rstd, mean} were parked in LDS before the main loop (the barrier above orders that write); hand them on
+        if (epi.ln.stats && n0 == 0 && tid < BM && m0 + tid < M)
+            epi.ln.stats[m0 + tid] = row_st[tid];
+    }
+    if constexpr (Epi::kRowStats && !TakesRowSums<Epi>::value) {
         static_assert(CFG::NSTAGE > 0, "LayerNorm-folding epilogues run on the direct-to-LDS pipeline");
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -1207,6 +1282,16 @@ __global__ void __launch_bounds__(CFG::NT)
                     AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                     epi.store8(m, n, v, row_st[m - m0]);
                 }
+            } else if constexpr (EmitsRowSums<Epi>::value) {
+                // N is a multiple of 8 for these epilogues (checked at launch); every item leaves its eight columns'
+                // sums, zero where nothing is stored, so that the totals below see a fully written array
+                float2 sm = make_float2(0.f, 0.f);
+                if (m < M && n + 7 < N) {
+                    AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    sm = epi.store8(m, n, v);
+                }
+                reinterpret_cast<float2 *>(lds_dyn + CFG::lds_bytes)[(((pos / WGN) * TM + i) * 32 + row) * (BN / 8) +
+                                                                     ((pos % WGN) * CW + c8) / 8] = sm;
             } else if (m < M) {
                 AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 if (n + 7 < N) {
@@ -1226,6 +1311,19 @@ __global__ void __launch_bounds__(CFG::NT)
             __syncthreads();
     }
     TR_TL(3);  // C stored
+    if constexpr (EmitsRowSums<Epi>::value) {
+        // this tile's share of every row's sum and sum of squares, added up in a fixed order, for the folding GEMM
+        // that reads C next
+        __syncthreads();
+        if (tid < BM && m0 + tid < M) {
+            const float2 *part = reinterpret_cast<const float2 *>(lds_dyn + CFG::lds_bytes) + tid * (BN / 8);
+            float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int q = 0; q < BN / 8; ++q)
+                s1 += part[q].x, s2 += part[q].y;
+            epi.row_sums[(size_t)(n0 / BN) * M + m0 + tid] = make_float2(s1, s2);
+        }
+    }
     if constexpr (Epi::kRowStats) {
         // y = LayerNorm(t) for this tile's share of its rows (the BM rows are dealt out evenly over the tile columns, so
         // every workgroup writes whole rows), in the LayerNorm kernel's half-precision form
@@ -1273,6 +1371,9 @@ std::atomic<int> g_gemm_force_cfg{0};
 std::atomic<int> g_gemm_group_m{0};  // 0 = derived from the tile count; otherwise forced
 
 inline int tune_override(int N, int K, int *group_m);
+// internal: the chosen tile shape leaves no LDS for the row-sum side output; the caller launches the plain form
+constexpr int kTileTooLargeForSums = -12345;
+thread_local int t_last_tiles_n = 0;  // tile columns of this thread's last tiled launch (the row-sum block count)
 
 template <int DT, typename CFG, typename Epi>
 int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb, const Epi &epi) {
@@ -1287,6 +1388,12 @@ int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int 
         size_t need = CFG::stage_bytes + (size_t)CFG::BM * 8 * (1 + 2 * CFG::WGK * CFG::WGN);
         lds         = lds > need ? lds : need;
     }
+    if (TakesRowSums<Epi>::value)
+        lds = CFG::lds_bytes + (size_t)CFG::BM * 8;  // {rstd, mean} per row, parked behind the slabs before the main loop
+    if (EmitsRowSums<Epi>::value)
+        lds = CFG::lds_bytes + (size_t)CFG::BM * CFG::BN;  // eight bytes per eight columns and row, behind the staging area
+    if (lds > 160 * 1024)
+        return kTileTooLargeForSums;
     auto kern   = gemm_nk_tiled_kernel<DT, CFG, Epi>;
     if (lds > 64 * 1024) {
         // the attribute belongs to the (kernel, device) pair: one bit per device, per instantiation
@@ -1314,6 +1421,7 @@ int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int 
             ++group_m;
     group_m = group_m > tiles_m ? tiles_m : group_m;
     unsigned grid = (unsigned)(((tiles_m * tiles_n + 7) / 8) * 8);
+    t_last_tiles_n = tiles_n;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(CFG::NT), lds, s, (const T *)A, (const T *)B, M, N, K, lda, ldb, tiles_m, tiles_n,
                        group_m, epi);
     TR_CHECK_LAUNCH();
@@ -1717,7 +1825,8 @@ int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *
 
 int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folded, const float *bias_folded,
                      const float *colsum, const float *gamma, const float *beta, float eps, void *C, void *y,
-                     float *row_stats, int M, int N, int K, int flags, const void *residual) {
+                     float *row_stats, const float *row_sums, int row_sum_blocks, int M, int N, int K, int flags,
+                     const void *residual) {
     TR_REQUIRE(M >= 0 && N >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_ln: negative size");
     if (M == 0 || N == 0)
         return 0;
@@ -1729,30 +1838,41 @@ int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folde
     TR_REQUIRE((long)M < (1l << 24) && (long)M * K < (1l << 31) && (long)N * K < (1l << 31) && (long)M * N < (1l << 31),
                TNN_ROCM_ESHAPE, "gemm_ln: problem too large for 32-bit panel offsets");
     TR_REQUIRE(!(flags & TNN_ROCM_EPI_RESIDUAL) || residual, TNN_ROCM_EINVAL, "gemm_ln: residual flag without a residual");
+    TR_REQUIRE(!row_sums || (row_sum_blocks >= 1 && row_sum_blocks <= kMaxRowSumBlocks && (((uintptr_t)row_sums) & 7u) == 0),
+               TNN_ROCM_EINVAL, "gemm_ln: row sums come in 1..%d blocks, 8-byte aligned", kMaxRowSumBlocks);
     TR_REQUIRE(al16(t) && al16(w_folded) && al16(C) && al16(bias_folded) && al16(colsum) && (!residual || al16(residual)) &&
                    (!y || (al16(y) && al16(gamma) && al16(beta))) && (((uintptr_t)row_stats) & 7u) == 0,
                TNN_ROCM_EALIGN, "gemm_ln: pointers must be 16-byte aligned (row_stats: 8-byte)");
-#define TR_LN(DT)                                                                                                     \
+#define TR_LN(DT, SUMS)                                                                                               \
     {                                                                                                                 \
-        LnFloatEpilogue<DT> epi;                                                                                      \
+        LnFloatEpilogue<DT, SUMS> epi;                                                                                      \
         epi.flags    = flags;                                                                                         \
         epi.bias     = bias_folded;                                                                                   \
         epi.residual = (const Elem<DT>::type *)residual;                                                              \
         epi.C        = (Elem<DT>::type *)C;                                                                           \
         epi.ldc      = N;                                                                                             \
-        epi.ln       = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead.load(), (float2 *)row_stats};                                          \
-        return launch_gemm_fast<DT, LnFloatEpilogue<DT>>((hipStream_t)stream, t, w_folded, M, N, K, K, K, epi);       \
+        epi.ln = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead.load(), (float2 *)row_stats,       \
+                        (const float2 *)row_sums, row_sum_blocks};                                                   \
+        return launch_gemm_fast<DT, LnFloatEpilogue<DT, SUMS>>((hipStream_t)stream, t, w_folded, M, N, K, K, K, epi); \
     }
-    if (dtype == TNN_ROCM_F16)
-        TR_LN(TNN_ROCM_F16)
-    else
-        TR_LN(TNN_ROCM_BF16)
+    if (dtype == TNN_ROCM_F16) {
+        if (row_sums)
+            TR_LN(TNN_ROCM_F16, true)
+        else
+            TR_LN(TNN_ROCM_F16, false)
+    } else {
+        if (row_sums)
+            TR_LN(TNN_ROCM_BF16, true)
+        else
+            TR_LN(TNN_ROCM_BF16, false)
+    }
 #undef TR_LN
 }
 
 int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const void *wqkv_folded, const float *bqkv_folded,
                                const float *colsum, const float *gamma, const float *beta, float eps, void *qk, void *vt,
-                               void *y, float *row_stats, int B, int S, int heads, int K) {
+                               void *y, float *row_stats, const float *row_sums, int row_sum_blocks, int B, int S, int heads,
+                               int K) {
     TR_REQUIRE(B >= 0 && S >= 0 && heads >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_qkv_split_ln: negative size");
     if (B == 0 || S == 0 || heads == 0)
         return 0;
@@ -1766,29 +1886,40 @@ int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const voi
     TR_REQUIRE(al16(t) && al16(wqkv_folded) && al16(qk) && al16(vt) && al16(bqkv_folded) && al16(colsum) &&
                    (!y || (al16(y) && al16(gamma) && al16(beta))) && (((uintptr_t)row_stats) & 7u) == 0,
                TNN_ROCM_EALIGN, "gemm_qkv_split_ln: pointers must be 16-byte aligned (row_stats: 8-byte)");
+    TR_REQUIRE(!row_sums || (row_sum_blocks >= 1 && row_sum_blocks <= kMaxRowSumBlocks && (((uintptr_t)row_sums) & 7u) == 0),
+               TNN_ROCM_EINVAL, "gemm_qkv_split_ln: row sums come in 1..%d blocks, 8-byte aligned", kMaxRowSumBlocks);
     const int H = heads * 64, T = B * S;
-#define TR_QKVLN(DT)                                                                                                  \
+#define TR_QKVLN(DT, SUMS)                                                                                            \
     {                                                                                                                 \
-        LnQkvSplitEpilogue<DT> epi;                                                                                   \
+        LnQkvSplitEpilogue<DT, SUMS> epi;                                                                                   \
         epi.bias  = bqkv_folded;                                                                                      \
         epi.qk    = (Elem<DT>::type *)qk;                                                                             \
         epi.vt    = (Elem<DT>::type *)vt;                                                                             \
         epi.H     = H;                                                                                                \
         epi.S     = S;                                                                                                \
         epi.heads = heads;                                                                                            \
-        epi.ln    = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead.load(), (float2 *)row_stats};                                             \
-        return launch_gemm_fast<DT, LnQkvSplitEpilogue<DT>>((hipStream_t)stream, t, wqkv_folded, T, 3 * H, K, K, K, epi); \
+        epi.ln = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead.load(), (float2 *)row_stats,       \
+                        (const float2 *)row_sums, row_sum_blocks};                                                   \
+        return launch_gemm_fast<DT, LnQkvSplitEpilogue<DT, SUMS>>((hipStream_t)stream, t, wqkv_folded, T, 3 * H, K, K, K, \
+                                                                  epi);                                              \
     }
-    if (dtype == TNN_ROCM_F16)
-        TR_QKVLN(TNN_ROCM_F16)
-    else
-        TR_QKVLN(TNN_ROCM_BF16)
+    if (dtype == TNN_ROCM_F16) {
+        if (row_sums)
+            TR_QKVLN(TNN_ROCM_F16, true)
+        else
+            TR_QKVLN(TNN_ROCM_F16, false)
+    } else {
+        if (row_sums)
+            TR_QKVLN(TNN_ROCM_BF16, true)
+        else
+            TR_QKVLN(TNN_ROCM_BF16, false)
+    }
 #undef TR_QKVLN
 }
 
 int tnn_rocm_gemm_residual_ln(void *stream, int dtype, const void *x, const void *w, const float *bias, void *C,
                               const void *t, const float *row_stats, const float *gamma, const float *beta, int M, int N,
-                              int K, int flags) {
+                              int K, int flags, float *row_sums, int *row_sum_blocks) {
     TR_REQUIRE(M >= 0 && N >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_residual_ln: negative size");
     if (M == 0 || N == 0)
         return 0;
@@ -1804,9 +1935,14 @@ int tnn_rocm_gemm_residual_ln(void *stream, int dtype, const void *x, const void
     TR_REQUIRE(al16(x) && al16(w) && al16(C) && al16(t) && al16(gamma) && al16(beta) && (!bias || al16(bias)) &&
                    (((uintptr_t)row_stats) & 7u) == 0,
                TNN_ROCM_EALIGN, "gemm_residual_ln: pointers must be 16-byte aligned (row_stats: 8-byte)");
-#define TR_LNRES(DT)                                                                                                  \
+    TR_REQUIRE(!row_sums || (row_sum_blocks && (((uintptr_t)row_sums) & 7u) == 0), TNN_ROCM_EINVAL,
+               "gemm_residual_ln: the row sums need an 8-byte aligned buffer and a place for their block count");
+    if (row_sum_blocks)
+        *row_sum_blocks = 0;
+#define TR_LNRES(DT, SUMS)                                                                                            \
     {                                                                                                                 \
-        LnResidualEpilogue<DT> epi;                                                                                   \
+        LnResidualEpilogue<DT, SUMS> epi;                                                                             \
+        epi.row_sums = (float2 *)row_sums;                                                                            \
         epi.flags = flags;                                                                                            \
         epi.bias  = bias;                                                                                             \
         epi.t     = (const Elem<DT>::type *)t;                                                                        \
@@ -1815,12 +1951,27 @@ int tnn_rocm_gemm_residual_ln(void *stream, int dtype, const void *x, const void
         epi.beta  = beta;                                                                                             \
         epi.C     = (Elem<DT>::type *)C;                                                                              \
         epi.ldc   = N;                                                                                                \
-        return launch_gemm_fast<DT, LnResidualEpilogue<DT>>((hipStream_t)stream, x, w, M, N, K, K, K, epi);           \
+        rc = launch_gemm_fast<DT, LnResidualEpilogue<DT, SUMS>>((hipStream_t)stream, x, w, M, N, K, K, K, epi);       \
+    }
+    // With the row sums first.  Half-precision tiles are at least 64 columns wide, so N <= 64 * kMaxRowSumBlocks keeps
+    // the tile columns within what a reader adds up (and within the caller's buffer of kMaxRowSumBlocks * M pairs); a
+    // tile shape that leaves no LDS for the sums runs the plain form and reports zero blocks.
+    int rc = kTileTooLargeForSums;
+    if (row_sums && N <= 64 * kMaxRowSumBlocks) {
+        if (dtype == TNN_ROCM_F16)
+            TR_LNRES(TNN_ROCM_F16, true)
+        else
+            TR_LNRES(TNN_ROCM_BF16, true)
+        if (rc == 0)
+            *row_sum_blocks = t_last_tiles_n;
+        if (rc != kTileTooLargeForSums)
+            return rc;
     }
     if (dtype == TNN_ROCM_F16)
-        TR_LNRES(TNN_ROCM_F16)
+        TR_LNRES(TNN_ROCM_F16, false)
     else
-        TR_LNRES(TNN_ROCM_BF16)
+        TR_LNRES(TNN_ROCM_BF16, false)
+    return rc;
 #undef TR_LNRES
 }
 

@@ -7,7 +7,8 @@
 //   ../lib/probe_gemm_timeline N K mode        (M = 3072 tokens; mode 0 bias, 1 bias + GELU, 2 LayerNorm folded +
 //                                               GELU + LayerNorm output, 3 bias + residual, 4 as 2 with the row
 //                                               statistics instead of the LayerNorm output, 5 bias + a residual
-//                                               rebuilt from the raw tensor and the row statistics)
+//                                               rebuilt from the raw tensor and the row statistics, 6 as 4 with the
+//                                               statistics from handed-over row sums, 7 as 5 leaving such sums)
 // The kernels are compiled from gemm.hip itself with the timeline stamps switched on.
 #define TNN_ROCM_TIMELINE 1
 #include "gemm.hip"
@@ -24,7 +25,7 @@ int main(int argc, char **argv) {
     }
     const int M = 3072, N = atoi(argv[1]), K = atoi(argv[2]), mode = atoi(argv[3]);
     _Float16 *A, *B, *C, *Y, *R;
-    float *bias, *cs, *g, *be, *stats, *gn, *bn;
+    float *bias, *cs, *g, *be, *stats, *gn, *bn, *sums;
     (void)hipMalloc(&A, (size_t)M * K * 2);
     (void)hipMalloc(&B, (size_t)N * K * 2);
     (void)hipMalloc(&C, (size_t)M * N * 2);
@@ -45,16 +46,23 @@ int main(int argc, char **argv) {
     (void)hipMalloc(&gn, N * 4);
     (void)hipMalloc(&bn, N * 4);
     (void)hipMemset(stats, 0, (size_t)M * 8);
+    (void)hipMalloc(&sums, (size_t)TNN_ROCM_MAX_ROW_SUM_BLOCKS * M * 8);
+    (void)hipMemset(sums, 0, (size_t)TNN_ROCM_MAX_ROW_SUM_BLOCKS * M * 8);
     (void)hipMemset(gn, 0, N * 4);
     (void)hipMemset(bn, 0, N * 4);
     hipStream_t s;
     (void)hipStreamCreate(&s);
     auto call = [&]() {
-        if (mode == 2 || mode == 4)  // LayerNorm folded in; its output written (2) or the row statistics handed on (4)
+        if (mode == 2 || mode == 4 || mode == 6)  // LayerNorm folded in; 2: its output written, 4: the row statistics
+            // handed on instead, 6: as 4 with the statistics taken from the producer's row sums (twelve blocks)
             return tnn_rocm_gemm_ln(s, TNN_ROCM_F16, A, B, bias, cs, g, be, 1e-12f, C, mode == 2 ? Y : nullptr,
-                                    mode == 4 ? stats : nullptr, M, N, K, TNN_ROCM_EPI_GELU, nullptr);
-        if (mode == 5)  // bias + a LayerNorm output rebuilt from the raw tensor as the residual
-            return tnn_rocm_gemm_residual_ln(s, TNN_ROCM_F16, A, B, bias, C, R, stats, gn, bn, M, N, K, TNN_ROCM_EPI_BIAS);
+                                    mode != 2 ? stats : nullptr, mode == 6 ? sums : nullptr, mode == 6 ? 12 : 0, M, N, K,
+                                    TNN_ROCM_EPI_GELU, nullptr);
+        if (mode == 5 || mode == 7) {  // bias + a LayerNorm output rebuilt from the raw tensor as the residual; 7: also
+            int blocks = 0;            // leaves the row sums of its output
+            return tnn_rocm_gemm_residual_ln(s, TNN_ROCM_F16, A, B, bias, C, R, stats, gn, bn, M, N, K, TNN_ROCM_EPI_BIAS,
+                                             mode == 7 ? sums : nullptr, mode == 7 ? &blocks : nullptr);
+        }
         const int fl = TNN_ROCM_EPI_BIAS | (mode == 1 ? TNN_ROCM_EPI_GELU : 0) | (mode == 3 ? TNN_ROCM_EPI_RESIDUAL : 0);
         return tnn_rocm_gemm(s, TNN_ROCM_F16, 1, A, B, C, M, N, K, K, K, N, 1, 1, 1, fl, bias, mode == 3 ? R : nullptr, N);
     };

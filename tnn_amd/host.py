@@ -28,6 +28,7 @@ SIGNATURES = {
     "tnn_host_stream": (C.c_void_p, [C.c_void_p]),
     "tnn_host_get_output": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
                                       C.POINTER(C.c_int)]),
+    "tnn_host_time_loop": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_char_p, C.POINTER(C.c_double)]),
     "tnn_host_layer_count": (C.c_int, [C.c_void_p]),
     "tnn_host_layer_summary": (C.c_char_p, [C.c_void_p]),
     "tnn_host_layer_io": (C.c_char_p, [C.c_void_p]),
@@ -166,6 +167,13 @@ class RocmInstance:
                                                C.byref(nd)), "GetOutputMat")
         shape = [dims[i] for i in range(nd.value)]
         return buf[:int(np.prod(shape, dtype=np.int64))].reshape(shape).copy()
+
+    def time_loop(self, warmup, iters, out_name):
+        """the engine benchmark tool's loop (SetInputMat for every input set so far + Forward + GetOutputMat per
+        iteration), run natively -> (min, avg, max) seconds"""
+        stats = (C.c_double * 3)()
+        self._check(load().tnn_host_time_loop(self._h, warmup, iters, out_name.encode(), stats), "timing loop")
+        return stats[0], stats[1], stats[2]
 
     def layers(self):
         text = load().tnn_host_layer_summary(self._h).decode()

@@ -2,6 +2,8 @@
 // the Python bench and tests create an instance from proto text + model bytes, feed host arrays,
 // call Forward and read outputs back — the same sequence as the engine's TNNTest
 // (test/test.cc:101-152: ConvertFromMat -> Forward -> ConvertToMat).
+#include <chrono>
+#include <map>
 #include <cstdio>
 #include <cstring>
 #include <sstream>
@@ -17,6 +19,7 @@ struct Handle {
     std::shared_ptr<Instance> inst;
     std::string err;
     std::string summary;
+    std::map<std::string, std::shared_ptr<Mat>> inputs;  // host copies of the last Mats set, for tnn_host_time_loop
 };
 int fail(Handle *h, const Status &st) {
     h->err = st.description();
@@ -132,7 +135,45 @@ HOST_API int tnn_host_set_input(void *hp, const char *name, const void *data, in
     DimsVector d(dims, dims + ndims);
     auto mat  = std::make_shared<Mat>(DEVICE_NAIVE, mat_type == 1 ? NC_INT32 : NCHW_FLOAT, d, const_cast<void *>(data));
     Status st = h->inst->SetInputMat(mat, MatConvertParam(), name ? name : "");
-    return st == TNN_OK ? 0 : fail(h, st);
+    if (st != TNN_OK)
+        return fail(h, st);
+    auto keep = std::make_shared<Mat>(DEVICE_NAIVE, mat->GetMatType(), d);  // owns its memory
+    if (keep->GetData() && data)
+        memcpy(keep->GetData(), data, (size_t)DimsVectorUtils::Count(d) * 4);
+    h->inputs[name ? name : ""] = keep;
+    return 0;
+}
+
+// The loop of the engine's benchmark tool (test/test.cc:101-152): per iteration every input Mat goes in
+// (SetInputMat with the Mats of the last tnn_host_set_input calls), Forward, and the output Mat comes out
+// (GetOutputMat as fp32 NCHW on the host).  stats = {min, avg, max} seconds over the timed iterations.
+HOST_API int tnn_host_time_loop(void *hp, int warmup, int iters, const char *out_name, double *stats) {
+    auto h = static_cast<Handle *>(hp);
+    double mn = 1e30, mx = 0.0, sum = 0.0;
+    for (int i = 0; i < warmup + iters; ++i) {
+        auto t0 = std::chrono::steady_clock::now();
+        for (auto &kv : h->inputs) {
+            Status st = h->inst->SetInputMat(kv.second, MatConvertParam(), kv.first);
+            if (st != TNN_OK)
+                return fail(h, st);
+        }
+        Status st = h->inst->Forward();
+        std::shared_ptr<Mat> mat;
+        if (st == TNN_OK)
+            st = h->inst->GetOutputMat(mat, MatConvertParam(), out_name ? out_name : "", DEVICE_NAIVE, NCHW_FLOAT);
+        if (st != TNN_OK)
+            return fail(h, st);
+        double dt = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        if (i >= warmup) {
+            mn = dt < mn ? dt : mn;
+            mx = dt > mx ? dt : mx;
+            sum += dt;
+        }
+    }
+    stats[0] = mn;
+    stats[1] = sum / (iters > 0 ? iters : 1);
+    stats[2] = mx;
+    return 0;
 }
 
 HOST_API int tnn_host_forward(void *hp) {

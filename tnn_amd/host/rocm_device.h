@@ -64,6 +64,8 @@ public:
     // (the rows' LayerNorm statistics: fp32 in a net whose blobs are half precision).  Grow-only per name; a
     // (re)allocation counts as a memory epoch.
     Status SideBuffer(const std::string &name, size_t bytes, void **ptr);
+    // a number the writer of a side buffer leaves for its reader (how many blocks of row sums the launch produced)
+    int &SideBufferTag(const std::string &name) { return side_buffers_[name].tag; }
     // page-locked word kernels raise on a data error (e.g. Gather index out of range)
     int32_t *ErrorFlag() { return error_flag_; }
     // The padding mask is one blob shared by every attention layer of a forward pass: the first layer that asks
@@ -89,6 +91,7 @@ private:
     struct SideEntry {
         void *ptr  = nullptr;
         size_t cap = 0;
+        int tag    = 0;
     };
     std::map<std::string, SideEntry> side_buffers_;
 };

@@ -50,6 +50,10 @@ struct RocmFusedLinearParam : public LayerParam {
     // under residual_ln_key and its resource's residual_gamma / residual_beta (RocmFusionPass::HandOverRowStatistics).
     int ln_stats = 0, residual_ln = 0;
     std::string ln_stats_key, residual_ln_key;
+    // Row sums: a residual_ln layer whose output feeds a folding layer also leaves every row's sum and sum of squares
+    // per tile column in the side buffer row_sums_key; the folding layer (ln_sums_key, the same name) adds those up
+    // instead of taking the LayerNorm statistics from its A tiles (RocmFusionPass::HandOverRowSums).
+    std::string row_sums_key, ln_sums_key;
 };
 struct RocmFusedAttentionParam : public LayerParam {
     int heads    = 0;
@@ -64,7 +68,7 @@ struct RocmFusedAttentionParam : public LayerParam {
     // LayerNorm folded into the QKV projection, as in RocmFusedLinearParam
     int ln_fold = 0, ln_y = 0, ln_stats = 0;
     float ln_eps = 0.f;
-    std::string ln_stats_key;
+    std::string ln_stats_key, ln_sums_key;
     // the last output blob is int8: the context quantised as the Reformat layer that followed would (ROCm int8 pass)
     int out_quant = 0;
 };

@@ -66,8 +66,12 @@ public:
         if (half_ && !(fold && fold[0] == '0'))
             FoldLayerNorm();
         const char *hand = getenv("TNN_ROCM_LN_STATS");  // "0" keeps the LayerNorm output of a folding layer a tensor
-        if (half_ && !(fold && fold[0] == '0') && !(hand && hand[0] == '0'))
+        if (half_ && !(fold && fold[0] == '0') && !(hand && hand[0] == '0')) {
             HandOverRowStatistics();
+            const char *sums = getenv("TNN_ROCM_LN_SUMS");  // "0": folding layers take the statistics from their A tiles
+            if (!(sums && sums[0] == '0'))
+                HandOverRowSums();
+        }
         return TNN_OK;
     }
 
@@ -612,6 +616,33 @@ private:
         }
     }
 
+    // A folding layer reads t and needs every row's mean and variance.  When t is written by a RocmFusedLinear of the
+    // residual_ln kind (above) whose rows are the normalised rows, that layer's GEMM leaves the rows' sums and sums of
+    // squares per tile column next to t, and the folding GEMM adds them up while its first tiles are on their way,
+    // instead of accumulating them from its A fragments in the main loop.
+    void HandOverRowSums() {
+        auto &L = structure_->layers;
+        GraphIndex g(L);
+        for (auto &f : L) {
+            if (!f || (f->type != LAYER_ROCM_FUSED_LINEAR && f->type != LAYER_ROCM_FUSED_ATTENTION))
+                continue;
+            auto fl = ParamOf<RocmFusedLinearParam>(f);
+            auto fa = ParamOf<RocmFusedAttentionParam>(f);
+            auto fr = ResOf<RocmFusedLinearResource>(f->name);
+            if (!(fl ? fl->ln_fold : fa && fa->ln_fold) || !fr)
+                continue;
+            const std::string t = f->inputs[0];
+            int gi = g.producer_of(t);
+            auto w = gi >= 0 ? L[gi] : nullptr;
+            auto wp = w && w->type == LAYER_ROCM_FUSED_LINEAR ? ParamOf<RocmFusedLinearParam>(w) : nullptr;
+            const int C = fr->ln_gamma.GetDataCount();
+            if (!wp || !wp->residual_ln || wp->num_output != C || C > 64 * TNN_ROCM_MAX_ROW_SUM_BLOCKS || !wp->row_sums_key.empty())
+                continue;
+            wp->row_sums_key = t;
+            (fl ? fl->ln_sums_key : fa->ln_sums_key) = t;
+        }
+    }
+
     NetStructure *structure_ = nullptr;
     NetResource *resource_   = nullptr;
     bool half_               = true;
@@ -1089,6 +1120,21 @@ static void FoldLayerNormIntoWeights(const float *w, const float *bias, const fl
     }
 }
 
+// the side buffer a residual_ln layer leaves its output's row sums in: room for the most tile columns a launch may have
+static size_t RowSumsBytes(int rows) { return (size_t)TNN_ROCM_MAX_ROW_SUM_BLOCKS * (size_t)rows * 2 * sizeof(float); }
+// what a folding layer finds there: the buffer and the block count of the launch that wrote it (0 blocks, or no key:
+// nothing was handed over and the GEMM takes the statistics itself)
+static Status RowSumsOf(RocmContext *ctx, const std::string &key, int rows, void **sums, int *blocks) {
+    *sums   = nullptr;
+    *blocks = 0;
+    if (key.empty())
+        return TNN_OK;
+    *blocks = ctx->SideBufferTag(key);
+    if (*blocks > 0)
+        return ctx->SideBuffer(key, RowSumsBytes(rows), sums);
+    return TNN_OK;
+}
+
 // ---- RocmFusedLinear ------------------------------------------------------------------------------------------
 // y[rows,N] = act(x[rows,K] W^T + b) (+ residual): the arithmetic of MatMul+Add (cpu_mat_mul_layer_acc.cc:64-117,
 // compute_elewise.cc:37-65) or InnerProduct (naive_compute.cc:271-288), GELU (cpu_gelu_layer_acc.cc:42-45) and the
@@ -1156,22 +1202,31 @@ public:
         int epi = (p->has_bias ? TNN_ROCM_EPI_BIAS : 0) | (p->gelu ? TNN_ROCM_EPI_GELU : 0) |
                   (p->has_residual ? TNN_ROCM_EPI_RESIDUAL : 0);
         if (p->ln_fold) {
-            void *stats = nullptr;
+            void *stats = nullptr, *sums = nullptr;
+            int blocks = 0;
             if (p->ln_stats)
                 RETURN_ON_NEQ(context_->SideBuffer(p->ln_stats_key, (size_t)rows * 2 * sizeof(float), &stats), TNN_OK);
+            RETURN_ON_NEQ(RowSumsOf(context_, p->ln_sums_key, rows, &sums, &blocks), TNN_OK);
             ROCM_CALL(tnn_rocm_gemm_ln(Stream(), (int)inputs[0]->GetBlobDesc().data_type, Ptr(inputs[0]), weight_,
                                        (const float *)bias_, (const float *)colsum_, (const float *)gamma_, (const float *)beta_,
-                                       p->ln_eps, Ptr(outputs[0]), p->ln_y ? Ptr(outputs[1]) : nullptr, (float *)stats, rows, N,
-                                       K, epi & ~TNN_ROCM_EPI_BIAS, p->has_residual ? Ptr(In(inputs[1])) : nullptr));
+                                       p->ln_eps, Ptr(outputs[0]), p->ln_y ? Ptr(outputs[1]) : nullptr, (float *)stats,
+                                       (const float *)sums, blocks, rows, N, K, epi & ~TNN_ROCM_EPI_BIAS,
+                                       p->has_residual ? Ptr(In(inputs[1])) : nullptr));
             return TNN_OK;
         }
         if (p->residual_ln) {
             void *stats = nullptr;
             RETURN_ON_NEQ(context_->SideBuffer(p->residual_ln_key, (size_t)rows * 2 * sizeof(float), &stats), TNN_OK);
+            void *sums = nullptr;
+            int blocks = 0;
+            if (!p->row_sums_key.empty())
+                RETURN_ON_NEQ(context_->SideBuffer(p->row_sums_key, RowSumsBytes(rows), &sums), TNN_OK);
             ROCM_CALL(tnn_rocm_gemm_residual_ln(Stream(), (int)inputs[0]->GetBlobDesc().data_type, Ptr(inputs[0]), weight_,
                                                 (const float *)bias_, Ptr(outputs[0]), Ptr(In(inputs[1])), (const float *)stats,
                                                 (const float *)res_gamma_, (const float *)res_beta_, rows, N, K,
-                                                epi & ~TNN_ROCM_EPI_RESIDUAL));
+                                                epi & ~TNN_ROCM_EPI_RESIDUAL, (float *)sums, sums ? &blocks : nullptr));
+            if (sums)
+                context_->SideBufferTag(p->row_sums_key) = blocks;
             return TNN_OK;
         }
         ROCM_CALL(tnn_rocm_gemm(Stream(), (int)inputs[0]->GetBlobDesc().data_type, 1, Ptr(inputs[0]), weight_, Ptr(outputs[0]),
@@ -1275,6 +1330,10 @@ public:
         void *stats = nullptr;  // the folded LayerNorm's {rstd, mean} per row, for the layer that rebuilds its output
         if (p->ln_fold && p->ln_stats)
             RETURN_ON_NEQ(context_->SideBuffer(p->ln_stats_key, (size_t)T_ * 2 * sizeof(float), &stats), TNN_OK);
+        void *sums = nullptr;  // the rows' sums left by the layer that wrote the input, see HandOverRowSums
+        int blocks = 0;
+        if (p->ln_fold)
+            RETURN_ON_NEQ(RowSumsOf(context_, p->ln_sums_key, T_, &sums, &blocks), TNN_OK);
         const float *mask = nullptr;
         const int32_t *kv = nullptr;
         if (p->has_mask) {
@@ -1314,7 +1373,7 @@ public:
                 ROCM_CALL(tnn_rocm_gemm_qkv_split_ln(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_,
                                                      (const float *)colsum_, (const float *)gamma_, (const float *)beta_,
                                                      p->ln_eps, qkv, vt, p->ln_y ? Ptr(outputs[1]) : nullptr, (float *)stats,
-                                                     B_, seq_, p->heads, H_));
+                                                     (const float *)sums, blocks, B_, seq_, p->heads, H_));
             else
                 ROCM_CALL(tnn_rocm_gemm_qkv_split(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_, qkv, vt,
                                                   B_, seq_, p->heads, H_));
@@ -1332,7 +1391,8 @@ public:
         if (p->ln_fold)
             ROCM_CALL(tnn_rocm_gemm_ln(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_, (const float *)colsum_,
                                        (const float *)gamma_, (const float *)beta_, p->ln_eps, qkv,
-                                       p->ln_y ? Ptr(outputs[1]) : nullptr, (float *)stats, T_, 3 * H_, H_, 0, nullptr));
+                                       p->ln_y ? Ptr(outputs[1]) : nullptr, (float *)stats, (const float *)sums, blocks, T_,
+                                       3 * H_, H_, 0, nullptr));
         else
             ROCM_CALL(tnn_rocm_gemm(Stream(), (int)dt, 1, Ptr(inputs[0]), weight_, qkv, T_, 3 * H_, H_, H_, H_, 3 * H_, 1, 1, 1,
                                     TNN_ROCM_EPI_BIAS, (const float *)bias_, nullptr, 0));

@@ -127,10 +127,14 @@ def qkv_split(x, wqkv, bqkv, B, S, heads):
     return qk, vt
 
 
+MAX_ROW_SUM_BLOCKS = 24   # TNN_ROCM_MAX_ROW_SUM_BLOCKS
+
+
 def gemm_ln(t, w_folded, bias_folded, colsum, eps, gamma=None, beta=None, gelu=False, residual=None, want_y=False,
-            want_stats=False):
+            want_stats=False, row_sums=None):
     """C = act(LayerNorm(t) W^T + b) (+ residual) from the raw t and the folded weights; optionally also LayerNorm(t)
-    and / or the rows' {rstd, mean} ([M, 2] fp32); returns C, then y, then the statistics, as asked for"""
+    and / or the rows' {rstd, mean} ([M, 2] fp32); returns C, then y, then the statistics, as asked for.
+    row_sums = (buffer, blocks) as returned by gemm_residual_ln(want_row_sums=True) for the launch that wrote t."""
     _chk(t, w_folded, bias_folded, colsum, gamma, beta, residual)
     M, K = t.shape
     N = w_folded.shape[0]
@@ -138,38 +142,47 @@ def gemm_ln(t, w_folded, bias_folded, colsum, eps, gamma=None, beta=None, gelu=F
     y = torch.empty_like(t) if want_y else None
     st = torch.empty(M, 2, dtype=torch.float32, device=t.device) if want_stats else None
     flags = (2 if gelu else 0) | (4 if residual is not None else 0)
+    sums, blocks = row_sums if row_sums is not None else (None, 0)
     capi.call("tnn_rocm_gemm_ln", _stream(), dt(t), _p(t), _p(w_folded), _p(bias_folded), _p(colsum), _p(gamma), _p(beta),
-              float(eps), _p(c), _p(y), _p(st), M, N, K, flags, _p(residual))
+              float(eps), _p(c), _p(y), _p(st), _p(sums), blocks, M, N, K, flags, _p(residual))
     out = (c,) + ((y,) if want_y else ()) + ((st,) if want_stats else ())
     return out if len(out) > 1 else c
 
 
 def qkv_split_ln(t, wqkv_folded, bqkv_folded, colsum, eps, B, S, heads, gamma=None, beta=None, want_y=False,
-                 want_stats=False):
+                 want_stats=False, row_sums=None):
     """qkv_split on LayerNorm(t) given as the raw t and the folded weights; optionally also LayerNorm(t) and / or the
-    rows' {rstd, mean}"""
+    rows' {rstd, mean}; row_sums as for gemm_ln"""
     _chk(t, wqkv_folded, bqkv_folded, colsum, gamma, beta)
     H = heads * 64
     qk = torch.empty(B * S, 2 * H, dtype=t.dtype, device=t.device)
     vt = torch.empty(B, heads, 64, S, dtype=t.dtype, device=t.device)
     y = torch.empty_like(t) if want_y else None
     st = torch.empty(B * S, 2, dtype=torch.float32, device=t.device) if want_stats else None
+    sums, blocks = row_sums if row_sums is not None else (None, 0)
     capi.call("tnn_rocm_gemm_qkv_split_ln", _stream(), dt(t), _p(t), _p(wqkv_folded), _p(bqkv_folded), _p(colsum), _p(gamma),
-              _p(beta), float(eps), _p(qk), _p(vt), _p(y), _p(st), B, S, heads, t.shape[1])
+              _p(beta), float(eps), _p(qk), _p(vt), _p(y), _p(st), _p(sums), blocks, B, S, heads, t.shape[1])
     return (qk, vt) + ((y,) if want_y else ()) + ((st,) if want_stats else ())
 
 
-def gemm_residual_ln(x, w, t, row_stats, gamma, beta, bias=None, gelu=False, out=None):
-    """C = act(x W^T + b) + LayerNorm(t), the LayerNorm rebuilt from t and its rows' {rstd, mean}"""
+def gemm_residual_ln(x, w, t, row_stats, gamma, beta, bias=None, gelu=False, out=None, want_row_sums=False,
+                     row_sums_out=None):
+    """C = act(x W^T + b) + LayerNorm(t), the LayerNorm rebuilt from t and its rows' {rstd, mean}; with want_row_sums
+    also (buffer, blocks): the sums / sums of squares of C's rows per tile column, for gemm_ln / qkv_split_ln on C"""
+    import ctypes
     _chk(x, w, t, row_stats, gamma, beta, bias, out)
     M, K = x.shape
     N = w.shape[0]
     if out is None:
         out = torch.empty(M, N, dtype=x.dtype, device=x.device)
     flags = (1 if bias is not None else 0) | (2 if gelu else 0)
+    sums, blocks = None, ctypes.c_int(0)
+    if want_row_sums:
+        sums = row_sums_out if row_sums_out is not None else torch.zeros(MAX_ROW_SUM_BLOCKS, M, 2, dtype=torch.float32,
+                                                                       device=x.device)
     capi.call("tnn_rocm_gemm_residual_ln", _stream(), dt(x), _p(x), _p(w), _p(bias), _p(out), _p(t), _p(row_stats), _p(gamma),
-              _p(beta), M, N, K, flags)
-    return out
+              _p(beta), M, N, K, flags, _p(sums), ctypes.addressof(blocks) if want_row_sums else None)
+    return (out, (sums, blocks.value)) if want_row_sums else out
 
 
 def attention_qk_vt(qk, vt, B, S, heads, scale, mask=None, kv_len=None, out=None, q8_inv_scale=None):
