@@ -35,7 +35,7 @@ extern "C" {
 
 #define REF_API __attribute__((visibility("default")))
 
-// device: "NAIVE" or "X86".  Returns nullptr and fills err on failure.
+// device: "NAIVE", "X86", or "ROCM" / "ROCM:fp32" (see below).  Returns nullptr and fills err on failure.
 REF_API void *tnn_ref_create(const char *proto, size_t proto_len, const char *model, size_t model_len,
                              const char *device, int threads, char *err, size_t err_len) {
     std::unique_ptr<Session> s(new Session);
@@ -49,9 +49,18 @@ REF_API void *tnn_ref_create(const char *proto, size_t proto_len, const char *mo
         return nullptr;
     }
     NetworkConfig nc;
-    nc.device_type  = (std::string(device) == "X86") ? DEVICE_X86 : DEVICE_NAIVE;
+    const std::string dev(device);
+    nc.device_type  = dev == "X86" ? DEVICE_X86 : DEVICE_NAIVE;
     nc.network_type = NETWORK_TYPE_DEFAULT;
     nc.precision    = PRECISION_HIGH;
+    if (dev.compare(0, 4, "ROCM") == 0) {
+        // the DEVICE_ROCM backend of this repository built against this engine (oracle/_ref/libtnn_rocm_engine.so, which
+        // the caller has loaded into the process: its static registrations made the device known).  The device and
+        // network type values are the backend's own; "ROCM:fp32" asks for fp32 blobs, "ROCM" for the default (fp16).
+        nc.device_type  = static_cast<DeviceType>(0x1080);
+        nc.network_type = NETWORK_TYPE_AUTO;  // RocmDevice::ConvertAutoNetworkType() names the backend's network
+        nc.precision    = dev == "ROCM:fp32" ? PRECISION_HIGH : PRECISION_AUTO;
+    }
     s->inst         = s->net.CreateInst(nc, st);
     if (st != TNN_OK || !s->inst) {
         put_err(err, err_len, "TNN::CreateInst: " + st.description());

@@ -18,7 +18,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HOST = os.path.join(ROOT, "tnn_amd", "host")
 REF = os.environ.get("TNN_REFERENCE_TREE", "/root/reference")
-BACKEND_SOURCES = ["rocm_device.cc", "rocm_network.cc", "rocm_layer_accs.cc", "rocm_fused.cc"]
+BACKEND_SOURCES = ["rocm_device.cc", "rocm_network.cc", "rocm_layer_accs.cc", "rocm_fused.cc", "rocm_fused_layers.cc"]
 
 pytestmark = pytest.mark.skipif(not os.path.isdir(os.path.join(REF, "source", "tnn", "core")),
                                 reason="reference tree not present")

@@ -1,0 +1,102 @@
+"""The DEVICE_ROCM backend inside the reference engine itself.
+
+oracle/_ref/libtnn_rocm_engine.so is this repository's backend sources compiled against the reference's headers and
+linked against the reference engine built from its own sources (oracle/Makefile.ref).  Loading it registers the device,
+its layer accs, the optimizer passes, the blob converter and the network implementation with that engine, and the
+engine's own TNN / Instance / DefaultNetwork / BlobManager then run a model on DEVICE_ROCM: SetInputMat, Forward,
+GetOutputMat through the reference's code, side by side with its DEVICE_NAIVE path in the same process."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+import ref_driver
+from tnn_amd import tnnmodel
+from tnn_amd.encoder import EncoderConfig, make_inputs, make_weights
+
+pytestmark = pytest.mark.gpu
+
+PLUGIN = os.path.join(ref_driver.ROOT, "oracle", "_ref", "libtnn_rocm_engine.so")
+_plugin = None
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+
+
+def rel_err(a, b):
+    return float(np.abs(a.astype(np.float64) - b.astype(np.float64)).max() / max(np.abs(b).max(), 1e-30))
+
+
+def engine():
+    global _plugin
+    if not (ref_driver.available() and os.path.exists(PLUGIN)):
+        pytest.skip("oracle/_ref (the reference engine and the backend linked against it) was not built")
+    ref_driver.lib()
+    if _plugin is None:
+        _plugin = ctypes.CDLL(PLUGIN)
+    return ref_driver
+
+
+def run(graph, device, inputs, out_name, forwards=1):
+    s = ref_driver.RefSession(graph, device)
+    for name, arr in inputs.items():
+        s.set_input(name, arr)
+    outs = []
+    for _ in range(forwards):
+        s.forward()
+        outs.append(s.output(out_name))
+    s.close()
+    return outs
+
+
+def test_encoder_on_device_rocm_inside_the_reference_engine():
+    """Two BERT-base-width encoder layers with embeddings and a padding mask: the reference engine's DEVICE_NAIVE result
+    against the same engine running DEVICE_ROCM in fp32 blobs (bar 2e-3) and in fp16 blobs with the fused kernels (bar
+    1e-2); five forwards each, so the recorded-graph replay of the backend's network runs under the engine as well; and
+    against this repository's own host running the same backend sources."""
+    engine()
+    from tnn_amd import host
+    say("reference engine: DEVICE_NAIVE vs DEVICE_ROCM (fp32, fp16), 2-layer encoder B3 S64")
+    cfg = EncoderConfig.bert_base(2)
+    w = make_weights(cfg, seed=41, bias_std=0.02)
+    B, S = 3, 64
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 20, S, seed=42)
+    graph = tnnmodel.encoder_graph(cfg, w, B, S)
+    inputs = {"input_ids": ids.astype(np.int32), "token_type_ids": seg.astype(np.int32),
+              "attention_bias": mask.reshape(B, 1, 1, S).astype(np.float32)}
+    naive = run(graph, "NAIVE", inputs, "last_hidden")[0]
+    say("  DEVICE_NAIVE done")
+    for device, bar in (("ROCM:fp32", 2e-3), ("ROCM", 1e-2)):
+        outs = run(graph, device, inputs, "last_hidden", forwards=5)
+        errs = [rel_err(o, naive) for o in outs]
+        say("  %s vs DEVICE_NAIVE over five forwards: %s" % (device, " ".join("%.3g" % e for e in errs)))
+        assert max(errs) <= bar
+        assert all(np.array_equal(o, outs[0]) for o in outs[1:])   # eager, recorded and replayed forwards agree exactly
+        precision = "fp32" if device.endswith("fp32") else "fp16"
+        inst = host.RocmInstance.from_graph(graph, precision)
+        for name, arr in inputs.items():
+            inst.set_input(name, arr)
+        inst.forward()
+        own = inst.output("last_hidden")
+        inst.close()
+        e = rel_err(outs[0], own)
+        say("  %s vs this repository's host (%s): %.3g" % (device, precision, e))
+        assert e <= (1e-6 if precision == "fp32" else 2e-3)
+
+
+def test_single_attention_layer_on_device_rocm_inside_the_reference_engine():
+    """BASELINE configuration 1 (one self-attention layer, fp32, S128 H768 h12, the un-fused op sequence of the
+    reference's own CPU-runnable case) through the reference engine on DEVICE_NAIVE and on DEVICE_ROCM."""
+    engine()
+    say("reference engine: configuration 1 on DEVICE_NAIVE vs DEVICE_ROCM fp32")
+    cfg = EncoderConfig(1, 768, 12, 3072)
+    lw = make_weights(cfg, seed=43, with_embeddings=False)["layers"][0]
+    graph = tnnmodel.attention_layer_graph(lw, 128, 768, 12)
+    x = np.random.default_rng(44).standard_normal((128, 768)).astype(np.float32)
+    naive = run(graph, "NAIVE", {"x": x}, "y")[0]
+    rocm = run(graph, "ROCM:fp32", {"x": x}, "y", forwards=4)
+    errs = [rel_err(o, naive) for o in rocm]
+    say("  rel err over four forwards: %s" % " ".join("%.3g" % e for e in errs))
+    assert max(errs) <= 2e-3

@@ -564,7 +564,7 @@ Status BaseLayer::InferOutputDataType() {
             b->GetBlobDesc().data_type = dt;
     return TNN_OK;
 }
-Status BaseLayer::InferOutputShape() {
+Status BaseLayer::InferOutputShape(bool) {
     if (!input_blobs_.empty())
         for (auto b : output_blobs_)
             b->GetBlobDesc().dims = input_blobs_[0]->GetBlobDesc().dims;
@@ -574,7 +574,7 @@ Status BaseLayer::InferOutputShape() {
 namespace {
 struct InnerProductLayer : BaseLayer {  // layer/inner_product_layer.cc:27-46
     using BaseLayer::BaseLayer;
-    Status InferOutputShape() override {
+    Status InferOutputShape(bool ignore_error = false) override {
         auto p = dynamic_cast<InnerProductLayerParam *>(param_);
         CHECK_PARAM_NULL(p);
         auto in = input_blobs_[0]->GetBlobDesc().dims;
@@ -634,7 +634,7 @@ DimsVector MatMulOutputDims(DimsVector a, DimsVector b, Status *st) {  // layer/
 }
 struct MatMulLayer : BaseLayer {  // layer/mat_mul_layer.cc:116-148
     using BaseLayer::BaseLayer;
-    Status InferOutputShape() override {
+    Status InferOutputShape(bool ignore_error = false) override {
         auto p = dynamic_cast<MatMulLayerParam *>(param_);
         auto r = dynamic_cast<MatMulLayerResource *>(resource_);
         CHECK_PARAM_NULL(p);
@@ -668,7 +668,7 @@ struct MatMulLayer : BaseLayer {  // layer/mat_mul_layer.cc:116-148
 
 struct BinaryLayer : BaseLayer {  // layer/multidir_broadcast_layer.cc:100-190
     using BaseLayer::BaseLayer;
-    Status InferOutputShape() override {
+    Status InferOutputShape(bool ignore_error = false) override {
         std::vector<DimsVector> shapes;
         for (auto b : input_blobs_)
             shapes.push_back(b->GetBlobDesc().dims);
@@ -711,7 +711,7 @@ struct BinaryLayer : BaseLayer {  // layer/multidir_broadcast_layer.cc:100-190
 
 struct ReshapeLayer : BaseLayer {  // layer/reshape_layer.cc:41-63, utils/dims_function_utils.cc:105-157
     using BaseLayer::BaseLayer;
-    Status InferOutputShape() override {
+    Status InferOutputShape(bool ignore_error = false) override {
         auto p = dynamic_cast<ReshapeLayerParam *>(param_);
         CHECK_PARAM_NULL(p);
         auto in = input_blobs_[0]->GetBlobDesc().dims;
@@ -751,7 +751,7 @@ struct ReshapeLayer : BaseLayer {  // layer/reshape_layer.cc:41-63, utils/dims_f
 
 struct PermuteLayer : BaseLayer {  // layer/permute_layer.cc:38-60
     using BaseLayer::BaseLayer;
-    Status InferOutputShape() override {
+    Status InferOutputShape(bool ignore_error = false) override {
         auto p = dynamic_cast<PermuteLayerParam *>(param_);
         CHECK_PARAM_NULL(p);
         auto in = input_blobs_[0]->GetBlobDesc().dims;
@@ -774,24 +774,16 @@ struct PermuteLayer : BaseLayer {  // layer/permute_layer.cc:38-60
 
 struct LayerNormLayer : BaseLayer {  // layer/layer_norm_layer.cc:25-35
     using BaseLayer::BaseLayer;
-    Status InferOutputShape() override {
+    Status InferOutputShape(bool ignore_error = false) override {
         if (input_blobs_.size() < 3)
             return Status(TNNERR_PARAM_ERR, "LayerNormLayer has no input blob of scale or bias");
-        return BaseLayer::InferOutputShape();
+        return BaseLayer::InferOutputShape(ignore_error);
     }
     // a second output (added by the ROCm int8 pass) is the quantised copy of the first and stays int8
     Status InferOutputDataType() override {
         output_blobs_[0]->GetBlobDesc().data_type = input_blobs_[0]->GetBlobDesc().data_type;
         return TNN_OK;
     }
-};
-
-// Layers of the ROCm int8 pass that read an int8 blob and write a float one (or the other way round): the network
-// sets each blob's type before Init (int8 blobs are BlobInt8, float blobs carry the network's float type), so the
-// default rule "outputs take the type of input 0" must not run.
-template <typename Base> struct MixedTypeLayer : Base {
-    using Base::Base;
-    Status InferOutputDataType() override { return TNN_OK; }
 };
 
 struct GatherLayer : BaseLayer {  // layer/gather_layer.cc
@@ -811,7 +803,7 @@ struct GatherLayer : BaseLayer {  // layer/gather_layer.cc
         output_blobs_[0]->GetBlobDesc().data_type = dt;
         return TNN_OK;
     }
-    Status InferOutputShape() override {
+    Status InferOutputShape(bool ignore_error = false) override {
         auto p = dynamic_cast<GatherLayerParam *>(param_);
         auto r = dynamic_cast<GatherLayerResource *>(resource_);
         CHECK_PARAM_NULL(p);
@@ -831,7 +823,7 @@ struct GatherLayer : BaseLayer {  // layer/gather_layer.cc
 
 struct UnsqueezeLayer : BaseLayer {  // layer/unsqueeze_layer.cc:35-59
     using BaseLayer::BaseLayer;
-    Status InferOutputShape() override {
+    Status InferOutputShape(bool ignore_error = false) override {
         auto p = dynamic_cast<SqueezeLayerParam *>(param_);
         CHECK_PARAM_NULL(p);
         DimsVector out = input_blobs_[0]->GetBlobDesc().dims;
@@ -847,7 +839,7 @@ struct UnsqueezeLayer : BaseLayer {  // layer/unsqueeze_layer.cc:35-59
 };
 struct SqueezeLayer : BaseLayer {  // layer/squeeze_layer.cc:35-60 (axes ascending, removed from the back)
     using BaseLayer::BaseLayer;
-    Status InferOutputShape() override {
+    Status InferOutputShape(bool ignore_error = false) override {
         auto p = dynamic_cast<SqueezeLayerParam *>(param_);
         CHECK_PARAM_NULL(p);
         DimsVector out = input_blobs_[0]->GetBlobDesc().dims;
@@ -892,47 +884,19 @@ struct ReformatLayer : BaseLayer {  // layer/reformat_layer.cc
     }
 };
 
-struct FusedEmbeddingLayer : BaseLayer {  // ids [..] int32 -> [.., H] in the network's float type (set by the network)
-    using BaseLayer::BaseLayer;
-    Status InferOutputDataType() override { return TNN_OK; }
-    Status InferOutputShape() override {
-        auto r = dynamic_cast<RocmFusedEmbeddingResource *>(resource_);
-        CHECK_PARAM_NULL(r);
-        auto out = input_blobs_[0]->GetBlobDesc().dims;
-        out.push_back(r->word.GetBufferDims().back());
-        output_blobs_[0]->GetBlobDesc().dims = out;
-        return TNN_OK;
-    }
-};
-
-struct FusedLinearLayer : BaseLayer {
-    using BaseLayer::BaseLayer;
-    Status InferOutputShape() override {
-        auto p = dynamic_cast<RocmFusedLinearParam *>(param_);
-        CHECK_PARAM_NULL(p);
-        auto out = input_blobs_[0]->GetBlobDesc().dims;
-        if (out.empty())
-            return Status(TNNERR_PARAM_ERR, "fused linear on a rank-0 blob");
-        if (p->axis >= 0) {  // InnerProduct form (layer/inner_product_layer.cc:37-44)
-            if (p->axis > (int)out.size())
-                return Status(TNNERR_PARAM_ERR, "fused linear axis out of range");
-            out.resize(p->axis);
-            out.push_back(p->num_output);
-        } else {
-            out.back() = p->num_output;
-        }
-        output_blobs_[0]->GetBlobDesc().dims = out;
-        if (p->ln_y) {  // LayerNorm(x) for the other readers of that tensor
-            if (output_blobs_.size() != 2)
-                return Status(TNNERR_PARAM_ERR, "fused linear: the LayerNorm output needs a second output blob");
-            output_blobs_[1]->GetBlobDesc().dims = input_blobs_[0]->GetBlobDesc().dims;
-        }
-        return TNN_OK;
-    }
-};
 }  // namespace
 
+std::map<LayerType, std::shared_ptr<LayerCreator>> &GetGlobalLayerCreatorMap() {
+    static std::map<LayerType, std::shared_ptr<LayerCreator>> m;
+    return m;
+}
+
 BaseLayer *CreateLayer(LayerType type) {
+    // layer classes that register themselves (base_layer.cc: the global creator map), e.g. the ROCm backend's fused layers
+    auto &reg = GetGlobalLayerCreatorMap();
+    auto it   = reg.find(type);
+    if (it != reg.end())
+        return it->second->CreateLayer();
     switch (type) {
         case LAYER_INNER_PRODUCT: return new InnerProductLayer(type);
         case LAYER_MATMUL: return new MatMulLayer(type);
@@ -948,15 +912,9 @@ BaseLayer *CreateLayer(LayerType type) {
         case LAYER_SQUEEZE: return new SqueezeLayer(type);
         case LAYER_UNSQUEEZE: return new UnsqueezeLayer(type);
         case LAYER_REFORMAT: return new ReformatLayer(type);
-        case LAYER_ROCM_FUSED_LINEAR: return new FusedLinearLayer(type);
-        case LAYER_ROCM_FUSED_EMBEDDING: return new FusedEmbeddingLayer(type);
-        case LAYER_ROCM_FUSED_LINEAR_INT8: return new MixedTypeLayer<InnerProductLayer>(type);
-        case LAYER_ROCM_QUANT_LINEAR_GELU: return new InnerProductLayer(type);
-        case LAYER_ROCM_FUSED_ATTENTION: return new MixedTypeLayer<BaseLayer>(type);
         case LAYER_SOFTMAX:
         case LAYER_GELU:
-        case LAYER_TANH:
-        case LAYER_ROCM_GELU_INT8: return new BaseLayer(type);
+        case LAYER_TANH: return new BaseLayer(type);
         default: return nullptr;
     }
 }
@@ -1255,22 +1213,7 @@ Status DefaultNetwork::InitLayers() {
         auto param = info->param.get();
         std::vector<Blob *> ins, outs;
         auto want_int8 = [&](bool is_input, size_t idx) -> bool {  // default_network.cc:362-440
-            if (!quantized_net)
-                return false;
-            if (info->type == LAYER_REFORMAT) {
-                auto rp = dynamic_cast<ReformatLayerParam *>(param);
-                return is_input ? rp->src_type == DATA_TYPE_INT8 : rp->dst_type == DATA_TYPE_INT8;
-            }
-            // layers written by the ROCm int8 pass with blobs of both kinds
-            if (info->type == LAYER_ROCM_FUSED_LINEAR_INT8)
-                return is_input && idx == 0;
-            if (info->type == LAYER_ROCM_FUSED_ATTENTION) {
-                auto ap = dynamic_cast<RocmFusedAttentionParam *>(param);
-                return is_input ? (idx == 0 && ap->quant) : (ap->out_quant && idx + 1 == info->outputs.size());
-            }
-            if (info->type == LAYER_LAYER_NORM)
-                return !is_input && idx == 1;
-            return param->quantized;
+            return quantized_net && RocmBlobIsInt8(info->type, param, is_input, idx, info->outputs.size());
         };
         for (size_t i = 0; i < info->inputs.size(); ++i) {
             const auto &name = info->inputs[i];

@@ -165,11 +165,15 @@ std::shared_ptr<const ImplementedPrecision> RocmDevice::GetImplementedPrecision(
 BlobMemorySizeInfo RocmDevice::Calculate(BlobDesc &desc) {
     // plain row-major ("NCHW" of any rank) in the blob's own data type; int8 blobs are NOT padded to
     // NHWC4 as on x86 (x86_device.cc:27-38): every channel count on this path is a multiple of 4
+    // One-dimensional, as every linear-memory device reports it (abstract_device.cc Calculate1DMemorySize): the engine's
+    // blob manager keeps one memory pool per number of size dimensions and only the 1-D pool exists off OpenCL
+    // (blob_manager.cc:30-38, 160-175).
     BlobMemorySizeInfo info;
     info.data_type = desc.data_type;
-    info.dims      = desc.dims;
-    if (info.dims.empty())
-        info.dims = {1};
+    int64_t count  = 1;
+    for (int d : desc.dims)
+        count *= d > 0 ? d : 0;
+    info.dims = {(int)(count > 0 ? count : 1)};
     return info;
 }
 Status RocmDevice::Allocate(void **handle, MatType mat_type, DimsVector dims) {

@@ -94,6 +94,25 @@ struct RocmFusedLinearInt8Param : public InnerProductLayerParam {
 struct RocmQuantLinearGeluParam : public InnerProductLayerParam {
     float mid_scale = 0.f;
 };
+// Which blobs of a layer are int8 blobs (BlobInt8 with a scale resource) in a quantised net on this device: the engine's
+// rule (default_network.cc:362-440: all blobs of a layer whose param is quantized; a Reformat's by its src / dst type)
+// plus the layers of the ROCm int8 pass that read one kind of blob and write the other.
+inline bool RocmBlobIsInt8(LayerType type, LayerParam *param, bool is_input, size_t index, size_t n_outputs) {
+    if (type == LAYER_REFORMAT) {
+        auto rp = dynamic_cast<ReformatLayerParam *>(param);
+        return rp && (is_input ? rp->src_type == DATA_TYPE_INT8 : rp->dst_type == DATA_TYPE_INT8);
+    }
+    if (type == LAYER_ROCM_FUSED_LINEAR_INT8)  // int8 in, dequantised (+ residual) out
+        return is_input && index == 0;
+    if (type == LAYER_ROCM_FUSED_ATTENTION) {  // int8 in when the projections are quantised; last output the int8 context
+        auto ap = dynamic_cast<RocmFusedAttentionParam *>(param);
+        return ap && (is_input ? (index == 0 && ap->quant) : (ap->out_quant && index + 1 == n_outputs));
+    }
+    if (type == LAYER_LAYER_NORM)  // a second output is the quantised copy of the first
+        return !is_input && index == 1;
+    return param && param->quantized;
+}
+
 struct RocmFusedQkvInt8Resource : public LayerResource {
     RawBuffer weight;   // int8 [3H, K]
     RawBuffer bias;     // int32 [3H] (may be empty)

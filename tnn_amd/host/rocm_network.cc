@@ -51,6 +51,41 @@ void RocmNetwork::Signature(std::vector<uint64_t> *sig) {
     }
 }
 
+#ifdef TNN_ROCM_ENGINE_TREE
+Status RocmNetwork::InitLayers(NetStructure *net_structure, NetResource *net_resource) {
+    // float blobs follow the network precision (PRECISION_HIGH: fp32; PRECISION_LOW: bfloat16; otherwise fp16), the
+    // blobs a quantised layer reads or writes become BlobInt8 with their scale resource, integer blobs stay
+    const bool half          = config_.precision != PRECISION_HIGH;
+    const DataType half_type = config_.precision == PRECISION_LOW ? DATA_TYPE_BFP16 : DATA_TYPE_HALF;
+    bool quantized_net       = false;
+    for (auto &info : net_structure->layers)
+        quantized_net |= info->param && info->param->quantized;
+    auto &consts = net_resource->constant_map;
+    for (auto &info : net_structure->layers) {
+        for (int side = 0; side < 2; ++side) {
+            auto &names = side == 0 ? info->inputs : info->outputs;
+            for (size_t i = 0; i < names.size(); ++i) {
+                if (consts.find(names[i]) != consts.end())
+                    continue;
+                Blob *blob = blob_manager_->GetBlob(names[i]);
+                if (!blob)
+                    return Status(TNNERR_PARAM_ERR, "layer " + info->name + " names a blob the blob manager does not have");
+                if (quantized_net && RocmBlobIsInt8(info->type, info->param.get(), side == 0, i, info->outputs.size())) {
+                    if (!dynamic_cast<BlobInt8 *>(blob))
+                        RETURN_ON_NEQ(GenerateInt8Blob(names[i], net_resource, &blob), TNN_OK);
+                    blob->GetBlobDesc().data_type = DATA_TYPE_INT8;
+                    continue;
+                }
+                DataType &dt = blob->GetBlobDesc().data_type;
+                if (dt == DATA_TYPE_FLOAT || dt == DATA_TYPE_HALF || dt == DATA_TYPE_BFP16)
+                    dt = half ? half_type : DATA_TYPE_FLOAT;
+            }
+        }
+    }
+    return DefaultNetwork::InitLayers(net_structure, net_resource);
+}
+#endif
+
 Status RocmNetwork::Forward() {
     RETURN_ON_NEQ(RocmNetwork::ForwardAsync(nullptr), TNN_OK);
     return context_->Synchronize();

@@ -22,6 +22,14 @@ public:
     Status Forward() override;
     Status ForwardAsync(Callback call_back) override;
 
+#ifdef TNN_ROCM_ENGINE_TREE
+protected:
+    // The engine settles every blob's data type in UpdateBlobPrecision (default_network.cc:362-440), which returns
+    // at once for a device it does not know; this override does that pass for DEVICE_ROCM and then runs the engine's
+    // own InitLayers.
+    Status InitLayers(NetStructure *net_structure, NetResource *net_resource) override;
+#endif
+
 private:
     // Everything a recording depends on: dims and device address of every blob the layers touch, and the context's
     // scratch allocation count.  A recording is replayed only under the signature it was made with, so a Reshape, a

@@ -579,6 +579,7 @@ private:
 };
 
 // ---- layers (device independent): shape and dtype inference -------------------------------------
+class DefaultNetwork;
 class BaseLayer {
 public:
     explicit BaseLayer(LayerType type) : type_(type) {}
@@ -587,19 +588,40 @@ public:
                 std::vector<Blob *> &outputs, AbstractDevice *device, ConstantResource *consts);
     Status Reshape();
     Status Forward();
-    virtual Status InferOutputShape();
-    virtual Status InferOutputDataType();
     std::string GetLayerName() { return param_ ? param_->name : ""; }
     LayerType GetLayerType() { return type_; }
     std::vector<Blob *> &GetInputBlobs() { return input_blobs_; }
     std::vector<Blob *> &GetOutputBlobs() { return output_blobs_; }
 
 protected:
+    friend class DefaultNetwork;  // this host's Reshape infers every shape before it touches blob memory
+    // base_layer.h:101-105
+    virtual Status InferOutputShape(bool ignore_error = false);
+    virtual Status InferOutputDataType();
     LayerType type_;
     LayerParam *param_       = nullptr;
     LayerResource *resource_ = nullptr;
     std::vector<Blob *> input_blobs_, output_blobs_;
     AbstractLayerAcc *layer_acc_ = nullptr;
+};
+// layer registry (base_layer.h:108-143)
+class LayerCreator {
+public:
+    virtual ~LayerCreator() {}
+    virtual BaseLayer *CreateLayer() = 0;
+};
+template <typename T> class TypeLayerCreator : public LayerCreator {
+public:
+    explicit TypeLayerCreator(LayerType type) : type_(type) {}
+    BaseLayer *CreateLayer() override { return new T(type_); }
+
+protected:
+    LayerType type_;
+};
+std::map<LayerType, std::shared_ptr<LayerCreator>> &GetGlobalLayerCreatorMap();
+template <typename T> class TypeLayerRegister {
+public:
+    explicit TypeLayerRegister(LayerType type) { GetGlobalLayerCreatorMap()[type] = std::shared_ptr<T>(new T(type)); }
 };
 BaseLayer *CreateLayer(LayerType type);
 
