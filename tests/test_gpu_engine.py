@@ -100,3 +100,49 @@ def test_single_attention_layer_on_device_rocm_inside_the_reference_engine():
     errs = [rel_err(o, naive) for o in rocm]
     say("  rel err over four forwards: %s" % " ".join("%.3g" % e for e in errs))
     assert max(errs) <= 2e-3
+
+
+def test_int8_encoder_on_device_rocm_inside_the_reference_engine(monkeypatch):
+    """A two-layer encoder with int8 projections (QuantizedInnerProduct layers and blob scales in the model, no Reformat
+    layers: the backend's own insertion pass writes them, the engine's serves its CPU devices only), calibrated on this
+    repository's fp32 forward.  Inside the reference engine DEVICE_ROCM gives, value for value, what this repository's
+    host gives with the same backend sources - with the explicit Reformat chain and with the fused int8 layers - and
+    stays close to the engine's own DEVICE_NAIVE run of the same quantised model."""
+    engine()
+    from tnn_amd import host, quant
+    say("reference engine: int8 encoder on DEVICE_NAIVE vs DEVICE_ROCM")
+    cfg = EncoderConfig.bert_base(2)
+    w = make_weights(cfg, seed=51)
+    B, S = 2, 64
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 24, S, seed=52)
+    inputs = {"input_ids": ids.astype(np.int32), "token_type_ids": seg.astype(np.int32),
+              "attention_bias": mask.reshape(B, 1, 1, S).astype(np.float32)}
+    names = quant.calibration_outputs(cfg)
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S, extra_outputs=names), "fp32")
+    for k, v in inputs.items():
+        inst.set_input(k, v)
+    inst.forward()
+    scales = {n: quant.activation_scale(inst.output(n, max_elems=1 << 24)) for n in names}
+    inst.close()
+    graph = quant.int8_encoder_graph(cfg, w, scales, B, S)
+    naive = run(graph, "NAIVE", inputs, "last_hidden")[0]
+    x86 = run(graph, "X86", inputs, "last_hidden")[0]    # the quantiser forms this backend follows (reciprocal multiply)
+    say("  DEVICE_NAIVE and DEVICE_X86 done; they differ by %.3g" % rel_err(x86, naive))
+    for fuse in ("0", "1"):
+        monkeypatch.setenv("TNN_ROCM_FUSE_INT8", fuse)
+        for device, precision in (("ROCM:fp32", "fp32"), ("ROCM", "fp16")):
+            outs = run(graph, device, inputs, "last_hidden", forwards=4)
+            assert all(np.array_equal(o, outs[0]) for o in outs[1:])
+            inst = host.RocmInstance.from_graph(graph, precision)
+            for k, v in inputs.items():
+                inst.set_input(k, v)
+            inst.forward()
+            own = inst.output("last_hidden")
+            inst.close()
+            e_own, e_naive, e_x86 = rel_err(outs[0], own), rel_err(outs[0], naive), rel_err(outs[0], x86)
+            say("  fused=%s %s: vs this repository's host %.3g, vs DEVICE_NAIVE %.3g, vs DEVICE_X86 %.3g"
+                % (fuse, device, e_own, e_naive, e_x86))
+            assert e_own == 0.0
+            # a quantised network amplifies last-ulp differences of its float layers into single int8 steps, so the
+            # engines' two CPU devices differ from each other by about as much as the GPU differs from either
+            assert e_naive <= 5e-2 and e_x86 <= 5e-2

@@ -104,6 +104,7 @@ LayerType GlobalConvertLayerType(std::string s) {
         {"BlobScale", LAYER_BLOB_SCALE},      {"QuantizedAdd", LAYER_ADD},
         {"RocmFusedLinear", LAYER_ROCM_FUSED_LINEAR}, {"RocmFusedAttention", LAYER_ROCM_FUSED_ATTENTION},
         {"RocmFusedLinearInt8", LAYER_ROCM_FUSED_LINEAR_INT8}, {"RocmGeluInt8", LAYER_ROCM_GELU_INT8},
+        {"RocmLayerNormQuant", LAYER_ROCM_LAYER_NORM_QUANT},
         {"RocmFusedEmbedding", LAYER_ROCM_FUSED_EMBEDDING}, {"RocmQuantLinearGelu", LAYER_ROCM_QUANT_LINEAR_GELU},
     };
     auto it = m.find(s);
@@ -779,11 +780,6 @@ struct LayerNormLayer : BaseLayer {  // layer/layer_norm_layer.cc:25-35
             return Status(TNNERR_PARAM_ERR, "LayerNormLayer has no input blob of scale or bias");
         return BaseLayer::InferOutputShape(ignore_error);
     }
-    // a second output (added by the ROCm int8 pass) is the quantised copy of the first and stays int8
-    Status InferOutputDataType() override {
-        output_blobs_[0]->GetBlobDesc().data_type = input_blobs_[0]->GetBlobDesc().data_type;
-        return TNN_OK;
-    }
 };
 
 struct GatherLayer : BaseLayer {  // layer/gather_layer.cc
@@ -868,18 +864,11 @@ struct CastLayer : BaseLayer {
 
 struct ReformatLayer : BaseLayer {  // layer/reformat_layer.cc
     using BaseLayer::BaseLayer;
-    Status InferOutputDataType() override {
+    Status InferOutputDataType() override {  // reformat_layer.cc:22-28
         auto p = dynamic_cast<ReformatLayerParam *>(param_);
         CHECK_PARAM_NULL(p);
-        if (p->src_type == DATA_TYPE_INT8 && p->dst_type != DATA_TYPE_INT8)
-            p->type = DEQUANT_ONLY;
-        else if (p->src_type != DATA_TYPE_INT8 && p->dst_type == DATA_TYPE_INT8)
-            p->type = QUANT_ONLY;
-        else
-            p->type = NO_QUANT;
         for (auto b : output_blobs_)
-            if (p->dst_type == DATA_TYPE_INT8)
-                b->GetBlobDesc().data_type = DATA_TYPE_INT8;
+            b->GetBlobDesc().data_type = p->dst_type;
         return TNN_OK;
     }
 };
@@ -928,75 +917,6 @@ std::vector<std::pair<int, std::shared_ptr<NetOptimizer>>> &OptimizerList() {
 }
 std::mutex g_optimize_mutex;
 
-// Quantized nets: insert float<->int8 Reformat layers wherever a quantized layer meets a float one
-// (source/tnn/optimizer/net_optimizer_insert_int8_reformat.cc:66-216, extended to DEVICE_ROCM).
-class InsertInt8Reformat : public NetOptimizer {
-public:
-    std::string Strategy() override { return "net_optimizer_insert_int8_reformat"; }
-    bool IsSupported(const NetworkConfig &c) override { return c.device_type == DEVICE_ROCM; }
-    Status Optimize(NetStructure *s, NetResource *res) override {
-        auto layers = s->layers;
-        bool any_q  = false;
-        for (auto &l : layers)
-            any_q |= l->param->quantized;
-        if (!any_q || layers.size() <= 1)
-            return TNN_OK;
-        std::vector<std::shared_ptr<LayerInfo>> out;
-        const int count = (int)layers.size();
-        for (int i = 0; i < count; ++i) {
-            auto cur = layers[i];
-            out.push_back(cur);
-            if (cur->type == LAYER_REFORMAT)
-                continue;
-            std::vector<std::string> need;
-            for (auto &o : cur->outputs) {
-                bool n = false;
-                for (int j = i + 1; j < count; ++j) {
-                    if (layers[j]->type == LAYER_REFORMAT)
-                        continue;
-                    for (auto &in : layers[j]->inputs)
-                        if (in == o && layers[j]->param->quantized != cur->param->quantized)
-                            n = true;
-                }
-                if (n)
-                    need.push_back(o);
-            }
-            if (need.empty())
-                continue;
-            auto nl      = std::make_shared<LayerInfo>();
-            nl->type     = LAYER_REFORMAT;
-            nl->type_str = "Reformat";
-            nl->name     = cur->name + "_int8_reformat";
-            auto p       = std::make_shared<ReformatLayerParam>();
-            p->LayerParam::type = nl->type_str;  // ReformatLayerParam::type (quant direction) shadows the base field
-            p->name      = nl->name;
-            p->src_type  = cur->param->quantized ? DATA_TYPE_INT8 : DATA_TYPE_FLOAT;
-            p->dst_type  = cur->param->quantized ? DATA_TYPE_FLOAT : DATA_TYPE_INT8;
-            nl->param    = p;
-            nl->inputs   = need;
-            for (auto &o : need) {
-                std::string no = o + "_int8_reformat";
-                nl->outputs.push_back(no);
-                s->blobs.insert(no);
-                for (int j = i + 1; j < count; ++j)
-                    for (auto &in : layers[j]->inputs)
-                        if (in == o && layers[j]->param->quantized != cur->param->quantized)
-                            in = no;
-                if (!cur->param->quantized) {
-                    auto it = res->resource_map.find(o + "_scale_data_");
-                    if (it == res->resource_map.end())
-                        return Status(TNNERR_NULL_PARAM, "can not get blob scale " + o + "_scale_data_");
-                    res->resource_map[no + "_scale_data_"] = it->second;
-                }
-            }
-            out.push_back(nl);
-        }
-        s->layers = out;
-        return TNN_OK;
-    }
-};
-// net_optimizer_insert_int8_reformat.cc:34
-optimizer::NetOptimizerRegister<InsertInt8Reformat> g_net_optimizer_insert_int8_reformat(optimizer::P2);
 }  // namespace
 
 void optimizer::NetOptimizerManager::RegisterNetOptimizer(NetOptimizer *opt, OptPriority prior) {

@@ -23,6 +23,8 @@ constexpr LayerType LAYER_ROCM_FUSED_LINEAR_INT8 = static_cast<LayerType>(0x7003
 constexpr LayerType LAYER_ROCM_GELU_INT8         = static_cast<LayerType>(0x7004);
 constexpr LayerType LAYER_ROCM_FUSED_EMBEDDING   = static_cast<LayerType>(0x7005);
 constexpr LayerType LAYER_ROCM_QUANT_LINEAR_GELU = static_cast<LayerType>(0x7006);
+// LayerNorm (LayerNormLayerParam, inputs x, scale, bias) with a second, int8 output: the quantised copy of the first
+constexpr LayerType LAYER_ROCM_LAYER_NORM_QUANT  = static_cast<LayerType>(0x7007);
 
 struct RocmFusedLinearResource : public LayerResource {
     RawBuffer weight_nk;  // [N, K] fp32
@@ -108,7 +110,7 @@ inline bool RocmBlobIsInt8(LayerType type, LayerParam *param, bool is_input, siz
         auto ap = dynamic_cast<RocmFusedAttentionParam *>(param);
         return ap && (is_input ? (index == 0 && ap->quant) : (ap->out_quant && index + 1 == n_outputs));
     }
-    if (type == LAYER_LAYER_NORM)  // a second output is the quantised copy of the first
+    if (type == LAYER_ROCM_LAYER_NORM_QUANT)  // float in, float out, and the quantised copy of the output
         return !is_input && index == 1;
     return param && param->quantized;
 }

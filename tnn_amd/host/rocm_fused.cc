@@ -649,6 +649,84 @@ private:
 };
 
 // ---- quantised nets -----------------------------------------------------------------------------------------------
+// Quantised nets: insert float<->int8 Reformat layers wherever a quantised layer meets a float one.  The engine's own
+// pass for this (source/tnn/optimizer/net_optimizer_insert_int8_reformat.cc:41-45, 66-216) serves ARM, NAIVE and X86
+// only; this is the same rewrite for DEVICE_ROCM, at the same priority, so that the device needs no change there.
+class RocmInsertInt8Reformat : public optimizer::NetOptimizer {
+public:
+    std::string Strategy() override { return "net_optimizer_rocm_insert_int8_reformat"; }
+    bool IsSupported(const NetworkConfig &c) override {
+        // the float side of every Reformat carries the network's float type, as the blobs around it do
+        float_type_ = c.precision == PRECISION_HIGH ? DATA_TYPE_FLOAT
+                                                    : (c.precision == PRECISION_LOW ? DATA_TYPE_BFP16 : DATA_TYPE_HALF);
+        return c.device_type == DEVICE_ROCM;
+    }
+    Status Optimize(NetStructure *s, NetResource *res) override {
+        std::vector<std::shared_ptr<LayerInfo>> layers = s->layers;
+        bool any_q  = false;
+        for (auto &l : layers)
+            any_q |= l->param->quantized;
+        if (!any_q || layers.size() <= 1)
+            return TNN_OK;
+        std::vector<std::shared_ptr<LayerInfo>> out;
+        const int count = (int)layers.size();
+        for (int i = 0; i < count; ++i) {
+            auto cur = layers[i];
+            out.push_back(cur);
+            if (cur->type == LAYER_REFORMAT)
+                continue;
+            std::vector<std::string> need;
+            for (auto &o : cur->outputs) {
+                bool n = false;
+                for (int j = i + 1; j < count; ++j) {
+                    if (layers[j]->type == LAYER_REFORMAT)
+                        continue;
+                    for (auto &in : layers[j]->inputs)
+                        if (in == o && layers[j]->param->quantized != cur->param->quantized)
+                            n = true;
+                }
+                if (n)
+                    need.push_back(o);
+            }
+            if (need.empty())
+                continue;
+            auto nl      = std::make_shared<LayerInfo>();
+            nl->type     = LAYER_REFORMAT;
+            nl->type_str = "Reformat";
+            nl->name     = cur->name + "_int8_reformat";
+            auto p       = std::make_shared<ReformatLayerParam>();
+            p->LayerParam::type = nl->type_str;  // ReformatLayerParam::type (quant direction) shadows the base field
+            p->name      = nl->name;
+            p->src_type  = cur->param->quantized ? DATA_TYPE_INT8 : float_type_;
+            p->dst_type  = cur->param->quantized ? float_type_ : DATA_TYPE_INT8;
+            nl->param    = p;
+            nl->inputs   = need;
+            for (auto &o : need) {
+                std::string no = o + "_int8_reformat";
+                nl->outputs.push_back(no);
+                s->blobs.insert(no);
+                for (int j = i + 1; j < count; ++j)
+                    for (auto &in : layers[j]->inputs)
+                        if (in == o && layers[j]->param->quantized != cur->param->quantized)
+                            in = no;
+                if (!cur->param->quantized) {
+                    auto it = res->resource_map.find(o + "_scale_data_");
+                    if (it == res->resource_map.end())
+                        return Status(TNNERR_NULL_PARAM, "can not get blob scale " + o + "_scale_data_");
+                    res->resource_map[no + "_scale_data_"] = it->second;
+                }
+            }
+            out.push_back(nl);
+        }
+        s->layers = out;
+        return TNN_OK;
+    }
+
+private:
+    DataType float_type_ = DATA_TYPE_FLOAT;
+};
+
+
 // Runs after the engine's own pass has made every float <-> int8 boundary an explicit Reformat layer
 // (net_optimizer_insert_int8_reformat.cc:66-181).  A quantised encoder layer is then
 //   Reformat(x) -> 3 x QuantizedInnerProduct -> 3 x Reformat -> head split, scores, softmax, P.V, head merge ->
@@ -1022,7 +1100,10 @@ private:
                 continue;
             for (int ri : it->second) {
                 if (ri > i && IsReformat(L[ri], true)) {
+                    // a layer type of its own: the engine's LayerNorm layer class infers shape and type of one output
                     L[i]->outputs.push_back(L[ri]->outputs[0]);
+                    L[i]->type     = LAYER_ROCM_LAYER_NORM_QUANT;
+                    L[i]->type_str = "RocmLayerNormQuant";
                     L[ri] = nullptr;
                     break;
                 }
@@ -1066,10 +1147,12 @@ private:
 };
 
 // optimizer/net_optimizer_manager.cc:33-48 runs the passes sorted by (priority, strategy name): the float rewrite runs
-// with the engine's own fusions (P1); the int8 rewrite needs the Reformat layers, so it shares P2 with
-// net_optimizer_insert_int8_reformat and its strategy name sorts behind that one
+// with the engine's own fusions (P1); the Reformat insertion at the priority of the engine's own (P2); the int8 rewrite
+// needs the Reformat layers and runs last (PLAST; the engine's only other pass there, the layout Reformat insertion,
+// sorts in front of it by name and finds one layout everywhere on this device)
 optimizer::NetOptimizerRegister<RocmFusionPass> g_net_optimizer_rocm_fuse_encoder(optimizer::P1);
-optimizer::NetOptimizerRegister<RocmInt8FusionPass> g_net_optimizer_rocm_fuse_int8(optimizer::P2);
+optimizer::NetOptimizerRegister<RocmInsertInt8Reformat> g_net_optimizer_rocm_insert_int8_reformat(optimizer::P2);
+optimizer::NetOptimizerRegister<RocmInt8FusionPass> g_net_optimizer_rocm_fuse_int8(optimizer::PLAST);
 
 }  // namespace
 

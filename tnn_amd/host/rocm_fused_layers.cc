@@ -128,6 +128,19 @@ protected:
     }
 };
 
+// RocmLayerNormQuant: LayerNorm(x) and its quantised copy, both with the dims of x (float and int8)
+class RocmLayerNormQuantLayer : public RocmFusedLayerBase {
+public:
+    explicit RocmLayerNormQuantLayer(LayerType type) : RocmFusedLayerBase(type) {}
+
+protected:
+    Status InferOutputShape(bool ignore_error = false) override {
+        if (input_blobs_.size() < 3 || output_blobs_.size() != 2)
+            return Status(TNNERR_PARAM_ERR, "RocmLayerNormQuant needs x, scale, bias and two outputs");
+        return RocmFusedLayerBase::InferOutputShape(ignore_error);
+    }
+};
+
 // RocmGeluInt8: element-wise on an int8 blob
 class RocmGeluInt8Layer : public RocmFusedLayerBase {
 public:
@@ -140,6 +153,7 @@ TypeLayerRegister<TypeLayerCreator<RocmFusedEmbeddingLayer>> g_rocm_fused_embedd
 TypeLayerRegister<TypeLayerCreator<RocmInt8LinearLayer>> g_rocm_fused_linear_int8_layer(LAYER_ROCM_FUSED_LINEAR_INT8);
 TypeLayerRegister<TypeLayerCreator<RocmInt8LinearLayer>> g_rocm_quant_linear_gelu_layer(LAYER_ROCM_QUANT_LINEAR_GELU);
 TypeLayerRegister<TypeLayerCreator<RocmGeluInt8Layer>> g_rocm_gelu_int8_layer(LAYER_ROCM_GELU_INT8);
+TypeLayerRegister<TypeLayerCreator<RocmLayerNormQuantLayer>> g_rocm_layer_norm_quant_layer(LAYER_ROCM_LAYER_NORM_QUANT);
 
 }  // namespace
 }  // namespace TNN_NS

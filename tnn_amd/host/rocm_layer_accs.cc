@@ -306,6 +306,9 @@ protected:
     DataType ConstantBlobDataType(const std::vector<Blob *> &, int) override { return DATA_TYPE_FLOAT; }
 };
 REGISTER_ROCM_ACC(RocmLayerNormLayerAcc, LAYER_LAYER_NORM);
+// the same kernel with its second, quantised output (the layer the ROCm int8 pass makes of LayerNorm -> Reformat)
+class RocmLayerNormQuantLayerAcc : public RocmLayerNormLayerAcc {};
+REGISTER_ROCM_ACC(RocmLayerNormQuantLayerAcc, LAYER_ROCM_LAYER_NORM_QUANT);
 
 // ---- GELU (cpu_gelu_layer_acc.cc:31-51) --------------------------------------------------------------------
 class RocmGeluLayerAcc : public RocmLayerAcc {
@@ -375,23 +378,41 @@ REGISTER_ROCM_ACC(RocmUnsqueezeLayerAcc, LAYER_UNSQUEEZE);
 // ---- Reformat: float <-> int8 (x86_reformat_layer_acc.cc:50-80, x86_compute_int8.cc:1193-1318) -------------------
 class RocmReformatLayerAcc : public RocmLayerAcc {
 public:
+    // the direction follows from the two data types, and the acc records it in the param like the engine's own
+    // Reformat accs do (x86_reformat_layer_acc.cc:29-44)
+    Status Init(Context *context, LayerParam *param, LayerResource *resource, const std::vector<Blob *> &inputs,
+                const std::vector<Blob *> &outputs) override {
+        RETURN_ON_NEQ(RocmLayerAcc::Init(context, param, resource, inputs, outputs), TNN_OK);
+        auto p = dynamic_cast<ReformatLayerParam *>(param_);
+        CHECK_PARAM_NULL(p);
+        if (p->src_type == DATA_TYPE_INT8 && IsFloatType(p->dst_type)) {
+            p->type = DEQUANT_ONLY;
+            mode_   = kDequant;
+        } else if (IsFloatType(p->src_type) && p->dst_type == DATA_TYPE_INT8) {
+            p->type = QUANT_ONLY;
+            mode_   = kQuant;
+        } else if (IsFloatType(p->src_type) && IsFloatType(p->dst_type)) {
+            mode_ = kCast;
+        } else {
+            return Status(TNNERR_MODEL_ERR, "unsupport precision mode");
+        }
+        return TNN_OK;
+    }
     Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
-        auto param = dynamic_cast<ReformatLayerParam *>(param_);
-        CHECK_PARAM_NULL(param);
         for (size_t i = 0; i < inputs.size(); ++i) {
             size_t count = (size_t)DimsVectorUtils::Count(outputs[i]->GetBlobDesc().dims);
             DataType st = inputs[i]->GetBlobDesc().data_type, dt = outputs[i]->GetBlobDesc().data_type;
-            if (param->type == QUANT_ONLY) {
+            if (mode_ == kQuant) {
                 auto b8 = dynamic_cast<BlobInt8 *>(outputs[i]);
-                if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1)
-                    return Status(TNNERR_LAYER_ERR, "Reformat(quant) needs a per-tensor blob scale");
+                if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1 || !IsFloatType(st))
+                    return Status(TNNERR_LAYER_ERR, "Reformat(quant) needs a float blob and a per-tensor blob scale");
                 float s   = b8->GetIntResource()->scale_handle.force_to<float *>()[0];
                 float inv = (float)(1.0 / s);  // x86_reformat_layer_acc.cc:70 : double division, stored as float
                 ROCM_CALL(tnn_rocm_quantize(Stream(), (int)st, Ptr(inputs[i]), inv, (int8_t *)Ptr(outputs[i]), count));
-            } else if (param->type == DEQUANT_ONLY) {
+            } else if (mode_ == kDequant) {
                 auto b8 = dynamic_cast<BlobInt8 *>(inputs[i]);
-                if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1)
-                    return Status(TNNERR_LAYER_ERR, "Reformat(dequant) needs a per-tensor blob scale");
+                if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1 || !IsFloatType(dt))
+                    return Status(TNNERR_LAYER_ERR, "Reformat(dequant) needs a per-tensor blob scale and a float blob");
                 float s = b8->GetIntResource()->scale_handle.force_to<float *>()[0];
                 ROCM_CALL(tnn_rocm_dequantize(Stream(), (const int8_t *)Ptr(inputs[i]), s, (int)dt, Ptr(outputs[i]), count));
             } else if (IsFloatType(st) && IsFloatType(dt)) {
@@ -402,6 +423,9 @@ public:
         }
         return TNN_OK;
     }
+
+private:
+    enum { kQuant, kDequant, kCast } mode_ = kCast;
 };
 REGISTER_ROCM_ACC(RocmReformatLayerAcc, LAYER_REFORMAT);
 

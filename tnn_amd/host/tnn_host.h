@@ -350,13 +350,26 @@ struct CastLayerParam : public LayerParam {
     int to   = 0;
     int from = 0;
 };
-typedef enum { DEQUANT_ONLY = 0, QUANT_ONLY = 1, NO_QUANT = 2 } ReformatType;
+typedef enum {  // layer_param.h:446-466; the accs set it from src_type / dst_type (x86_reformat_layer_acc.cc:32-44)
+    QUANT_ONLY   = 0,
+    DEQUANT_ONLY = 1,
+    QUANT_NCHW4_2_NHWC   = 2,
+    DEQUANT_NHWC_2_NCHW4 = 3,
+    NC4HW4FP32_2_NC8HW8FP16 = 4,
+    NC8HW8FP16_2_NC4HW4FP32 = 5,
+    NC4HW4FP32_2_NCHWFP32 = 6,
+    NCHWFP32_2_NC4HW4FP32 = 7,
+    NC8HW8FP16_2_NCHWFP16 = 8,
+    NCHWFP16_2_NC8HW8FP16 = 9,
+    NC4HW4INT32_2_NCHWINT32 = 10,
+    NCHWINT32_2_NC4HW4INT32 = 11,
+} ReformatType;
 struct ReformatLayerParam : public LayerParam {
     DataType src_type     = DATA_TYPE_AUTO;
     DataType dst_type     = DATA_TYPE_AUTO;
     DataFormat src_format = DATA_FORMAT_AUTO;
     DataFormat dst_format = DATA_FORMAT_AUTO;
-    ReformatType type     = NO_QUANT;
+    ReformatType type     = QUANT_ONLY;
 };
 struct GatherLayerParam : public LayerParam {
     int axis                 = 0;
