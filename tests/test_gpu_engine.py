@@ -146,3 +146,40 @@ def test_int8_encoder_on_device_rocm_inside_the_reference_engine(monkeypatch):
             # a quantised network amplifies last-ulp differences of its float layers into single int8 steps, so the
             # engines' two CPU devices differ from each other by about as much as the GPU differs from either
             assert e_naive <= 5e-2 and e_x86 <= 5e-2
+
+
+def test_benchmark_model_inside_the_reference_engine():
+    """The benchmark's own model (12-layer BERT-base, batch 8, seq 384, seeds of bench.py) run by the reference engine on
+    DEVICE_ROCM: the same values as this repository's host gives, and the reference benchmark tool's loop
+    (SetInputMat x3 + Forward + GetOutputMat, 5 warm-up + 20 timed) timed on both, printed side by side."""
+    engine()
+    from tnn_amd import host
+    say("reference engine: the benchmark model on DEVICE_ROCM")
+    cfg = EncoderConfig.bert_base(12)
+    w = make_weights(cfg, seed=20240601)
+    B, S = 8, 384
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 200, S, seed=20240602)
+    graph = tnnmodel.encoder_graph(cfg, w, B, S)
+    inputs = {"input_ids": ids.astype(np.int32), "token_type_ids": seg.astype(np.int32),
+              "attention_bias": mask.reshape(B, 1, 1, S).astype(np.float32)}
+    s = ref_driver.RefSession(graph, "ROCM")
+    for name, arr in inputs.items():
+        s.set_input(name, arr)
+    for _ in range(4):
+        s.forward()
+    in_engine = s.output("last_hidden")
+    mn, avg, mx = s.time_loop(5, 20, "last_hidden")
+    fwd = s.time_forward(5, 50)
+    s.close()
+    inst = host.RocmInstance.from_graph(graph, "fp16")
+    for name, arr in inputs.items():
+        inst.set_input(name, arr)
+    for _ in range(4):
+        inst.forward()
+    own = inst.output("last_hidden")
+    omn, oavg, omx = inst.time_loop(5, 20, "last_hidden")
+    inst.close()
+    say("  in the reference engine: Forward %.3f ms; tool loop min/avg/max %.3f / %.3f / %.3f ms" % (fwd * 1e3, mn * 1e3, avg * 1e3, mx * 1e3))
+    say("  this repository's host:  tool loop min/avg/max %.3f / %.3f / %.3f ms" % (omn * 1e3, oavg * 1e3, omx * 1e3))
+    assert np.isfinite(in_engine).all() and rel_err(in_engine, own) == 0.0
+    assert fwd < 5e-3   # milliseconds, not the seconds of a CPU path: the fused kernels and the graph replay ran
