@@ -53,6 +53,10 @@ int tnn_host_forward(void *handle);
 /* Instance::ForwardAsync (instance.h:92): enqueue only; pair with tnn_host_sync */
 int tnn_host_forward_async(void *handle);
 int tnn_host_sync(void *handle);
+/* Instance::ShareCommandQueue (instance.h:74): `handle` launches on `other`'s stream from now on (other must outlive
+ * it); Instance::SetCpuNumThreads (instance.h:135): accepted, the device does no host-side threading of layers */
+int tnn_host_share_command_queue(void *handle, void *other);
+int tnn_host_set_cpu_num_threads(void *handle, int num_threads);
 /* Instance::GetCommandQueue (instance.h:71): the hipStream_t the instance launches on */
 void *tnn_host_stream(void *handle);
 /* Instance::GetOutputMat (instance.h:128) converted to fp32 NCHW on the host.  dims must hold 8 ints. */

@@ -289,6 +289,44 @@ def test_two_instances_on_two_threads_match_their_sequential_results():
         inst.close()
 
 
+def test_share_command_queue_and_cpu_threads():
+    """Instance::ShareCommandQueue (instance.cc:158-160, default_network.cc:537-556; the CUDA backend's counterpart is
+    cuda_context.cc:91-122): the second instance launches on the first one's stream from then on - its forwards, enqueued
+    without waiting, are ordered behind the first instance's on that one stream, one synchronise covers both, and every
+    result equals the one the instance gave on its own stream (eager, recording and replayed forwards).
+    SetCpuNumThreads is accepted."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: two instances on one shared command queue")
+    cfg = EncoderConfig.bert_base(2)
+    shapes = [(2, 128), (3, 96)]
+    insts, feeds = [], []
+    for k, (B, S) in enumerate(shapes):
+        w = make_weights(cfg, seed=80 + k, bias_std=0.02)
+        insts.append(host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), "fp16"))
+        ids, seg, lens, mask = make_inputs(cfg, B, S, 17, S, seed=400 + k)
+        feeds.append({"input_ids": ids, "token_type_ids": seg, "attention_bias": mask.reshape(B, 1, 1, S)})
+        for name, arr in feeds[k].items():
+            insts[k].set_input(name, arr)
+    alone = []
+    for inst in insts:
+        inst.forward()
+        alone.append(inst.output("last_hidden").copy())
+    assert insts[0].stream != insts[1].stream
+    insts[1].set_cpu_num_threads(4)
+    insts[1].share_command_queue(insts[0])
+    assert insts[0].stream == insts[1].stream
+    for it in range(5):
+        insts[0].forward_async()
+        insts[1].forward_async()
+        insts[0].sync()                      # the one stream: both forwards are done
+        for k in range(2):
+            assert np.array_equal(insts[k].output("last_hidden"), alone[k]), (it, k)
+    insts[1].close()                         # the sharer goes first: the stream belongs to instance 0
+    insts[0].forward()
+    assert np.array_equal(insts[0].output("last_hidden"), alone[0])
+    insts[0].close()
+
+
 def test_int8_encoder_full_shape_properties(monkeypatch):
     """Benchmark config 4's per-layer shape (B16 S256, hidden 768, FFN 3072; 3 layers to keep the case short):
     calibrated on this backend's fp32 forward, then run quantised in fp16 mode.  Size-independent checks: every

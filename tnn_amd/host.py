@@ -26,6 +26,8 @@ SIGNATURES = {
     "tnn_host_forward_async": (C.c_int, [C.c_void_p]),
     "tnn_host_sync": (C.c_int, [C.c_void_p]),
     "tnn_host_stream": (C.c_void_p, [C.c_void_p]),
+    "tnn_host_share_command_queue": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "tnn_host_set_cpu_num_threads": (C.c_int, [C.c_void_p, C.c_int]),
     "tnn_host_get_output": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
                                       C.POINTER(C.c_int)]),
     "tnn_host_time_loop": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_char_p, C.POINTER(C.c_double)]),
@@ -154,6 +156,13 @@ class RocmInstance:
 
     def sync(self):
         self._check(load().tnn_host_sync(self._h), "Synchronize")
+
+    def share_command_queue(self, other):
+        """Instance::ShareCommandQueue: launch on `other`'s stream from now on (other must outlive this instance)"""
+        self._check(load().tnn_host_share_command_queue(self._h, other._h), "ShareCommandQueue")
+
+    def set_cpu_num_threads(self, n):
+        self._check(load().tnn_host_set_cpu_num_threads(self._h, n), "SetCpuNumThreads")
 
     @property
     def stream(self):

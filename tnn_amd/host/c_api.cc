@@ -199,6 +199,18 @@ HOST_API int tnn_host_sync(void *hp) {
     return rc;
 }
 
+HOST_API int tnn_host_share_command_queue(void *hp, void *other) {
+    auto h    = static_cast<Handle *>(hp);
+    Status st = h->inst->ShareCommandQueue(other ? static_cast<Handle *>(other)->inst.get() : nullptr);
+    return st == TNN_OK ? 0 : fail(h, st);
+}
+
+HOST_API int tnn_host_set_cpu_num_threads(void *hp, int num_threads) {
+    auto h    = static_cast<Handle *>(hp);
+    Status st = h->inst->SetCpuNumThreads(num_threads);
+    return st == TNN_OK ? 0 : fail(h, st);
+}
+
 HOST_API void *tnn_host_stream(void *hp) {
     void *q = nullptr;
     static_cast<Handle *>(hp)->inst->GetCommandQueue(&q);

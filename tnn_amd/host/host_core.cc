@@ -1353,6 +1353,12 @@ void NetworkImplManager::RegisterNetworkImplFactory(NetworkType type, AbstractNe
 }
 
 Status DefaultNetwork::GetCommandQueue(void **q) { return context_->GetCommandQueue(q); }
+Status DefaultNetwork::ShareCommandQueue(DefaultNetwork *network) {
+    if (!network || !network->GetContext())
+        return Status(TNNERR_DEVICE_CONTEXT_CREATE, "network is nil");
+    return context_->ShareCommandQueue(network->GetContext());
+}
+Status DefaultNetwork::SetCpuNumThreads(int num_threads) { return context_->SetNumThreads(num_threads); }
 Status DefaultNetwork::GetAllInputBlobs(BlobMap &blobs) {
     blobs = inputs_;
     return TNN_OK;
@@ -1447,6 +1453,12 @@ Status Instance::ForwardAsync(Callback call_back) {
     return network_ ? network_->ForwardAsync(call_back) : Status(TNNERR_INST_ERR, "instance not initialised");
 }
 Status Instance::GetCommandQueue(void **q) { return network_->GetCommandQueue(q); }
+Status Instance::ShareCommandQueue(Instance *instance) {
+    if (!instance)
+        return Status(TNNERR_NULL_PARAM, "instance is nil");
+    return network_->ShareCommandQueue(instance->GetNetwork());
+}
+Status Instance::SetCpuNumThreads(int num_threads) { return network_->SetCpuNumThreads(num_threads); }
 Status Instance::GetAllInputBlobs(BlobMap &b) { return network_->GetAllInputBlobs(b); }
 Status Instance::GetAllOutputBlobs(BlobMap &b) { return network_->GetAllOutputBlobs(b); }
 

@@ -38,7 +38,27 @@ RocmContext::~RocmContext() {
     tnn_rocm_free(mask_cache_.mask_f32);
     tnn_rocm_free(mask_cache_.kv_len);
     tnn_rocm_free_host(error_flag_);
-    tnn_rocm_stream_destroy(stream_);
+    if (own_stream_)
+        tnn_rocm_stream_destroy(stream_);
+}
+
+Status RocmContext::ShareCommandQueue(Context *context) {
+    if (context == nullptr)
+        return Status(TNNERR_NULL_PARAM, "context is nil");
+    auto other = dynamic_cast<RocmContext *>(context);
+    if (other == nullptr || other->device_id_ != device_id_ || other->stream_ == nullptr)
+        return Status(TNNERR_DEVICE_INVALID_COMMAND_QUEUE, "the command queue of another device cannot be shared");
+    if (other == this || other->stream_ == stream_)
+        return TNN_OK;
+    if (stream_) {
+        ROCM_CALL(tnn_rocm_stream_sync(stream_));
+        if (own_stream_)
+            ROCM_CALL(tnn_rocm_stream_destroy(stream_));
+    }
+    own_stream_ = false;
+    stream_     = other->stream_;
+    ++memory_epoch_;
+    return TNN_OK;
 }
 
 Status RocmContext::GetCommandQueue(void **command_queue) {

@@ -50,6 +50,9 @@ public:
     Status Setup();
     Status LoadLibrary(std::vector<std::string> path) override { return TNN_OK; }
     Status GetCommandQueue(void **command_queue) override;
+    // This context launches on the other context's stream from now on (role of cuda_context.cc:91-122); the other
+    // context must outlive this one.  Recordings made on the old stream are dropped (a new memory epoch).
+    Status ShareCommandQueue(Context *context) override;
     Status OnInstanceForwardBegin() override;
     Status OnInstanceForwardEnd() override { return TNN_OK; }
     Status Synchronize() override;
@@ -76,6 +79,7 @@ public:
 private:
     int device_id_       = 0;
     void *stream_        = nullptr;
+    bool own_stream_     = true;
     void *workspace_     = nullptr;
     size_t workspace_sz_ = 0;
     int32_t *error_flag_ = nullptr;

@@ -691,6 +691,11 @@ public:
     virtual Status Forward();                           // default_network.cc:558-635: the layer loop, then Synchronize
     virtual Status ForwardAsync(Callback call_back);    // default_network.cc:672-686: the layer loop alone
     virtual Status GetCommandQueue(void **command_queue);
+    // default_network.cc:537-556: this network's context adopts the other network's command queue; set the threads
+    // the device may use on the host
+    virtual Status ShareCommandQueue(DefaultNetwork *network);
+    virtual Status SetCpuNumThreads(int num_threads);
+    Context *GetContext() { return context_; }
     virtual Status GetAllInputBlobs(BlobMap &blobs);
     virtual Status GetAllOutputBlobs(BlobMap &blobs);
     Blob *GetBlob(const std::string &name);
@@ -757,6 +762,8 @@ public:
     Status Forward();
     Status ForwardAsync(Callback call_back);
     Status GetCommandQueue(void **command_queue);
+    Status ShareCommandQueue(Instance *instance);  // instance.cc:158-160
+    Status SetCpuNumThreads(int num_threads);      // instance.cc:198-200
     Status GetAllInputBlobs(BlobMap &blobs);
     Status GetAllOutputBlobs(BlobMap &blobs);
     Status SetInputMat(std::shared_ptr<Mat> mat, MatConvertParam param, std::string input_name = "");
