@@ -26,10 +26,10 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 # rocprofv3 --pmc runs of this command (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
 # --counter-reference kernel (64 MiB in, 64 MiB out): FETCH_SIZE reads half the bytes, WRITE_SIZE all of them.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "gemm_qkv": int((2 * 14519.1 + 18596.2) * 1024),   # algorithmic: 4.5 + 3.4 in, 13.5 + 4.5 (LayerNorm output) out MiB
-    "gemm_out": int((2 * 10426.0 + 4608.0) * 1024),    # algorithmic: 4.5 + 1.1 + 4.5 in, 4.5 out MiB
-    "gemm_ffn1": int((2 * 17773.2 + 23040.0) * 1024),  # algorithmic: 4.5 + 4.5 in, 18 + 4.5 (LayerNorm output) out MiB
-    "gemm_ffn2": int((2 * 37095.2 + 4609.8) * 1024),   # algorithmic: 18 + 4.5 + 4.5 in, 4.5 out MiB
+    "gemm_qkv": int((2 * 14212.5 + 13868.7) * 1024),   # algorithmic: 4.5 + 3.4 in, 13.5 out MiB (+ row sums / statistics: 0.2)
+    "gemm_out": int((2 * 10458.5 + 4896.0) * 1024),    # algorithmic: 4.5 + 1.1 + 4.5 in, 4.5 (+ 0.3 row sums) out MiB
+    "gemm_ffn1": int((2 * 16752.0 + 18456.0) * 1024),  # algorithmic: 4.5 + 4.5 (+ 0.3 row sums) in, 18 out MiB
+    "gemm_ffn2": int((2 * 37176.5 + 4807.6) * 1024),   # algorithmic: 18 + 4.5 + 4.5 in, 4.5 (+ 0.2 row sums) out MiB
 }
 
 

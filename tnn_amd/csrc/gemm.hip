@@ -1045,19 +1045,20 @@ __global__ void __launch_bounds__(CFG::NT)
                     TR_WAIT_VMCNT(LPW);
                 else
                     TR_WAIT_VMCNT(0);
-                double s1 = 0.0, s2 = 0.0;
+                // Every other wave of the workgroup waits at the first barrier while these waves do this, so it is kept
+                // short: the block sums (fp32 already) are added in fp32 in a fixed order, only the variance is formed
+                // as a difference of doubles, and its reciprocal root is taken in single precision with one Newton step.
+                float f1 = 0.f, f2 = 0.f;
 #pragma unroll
                 for (int q = 0; q < kMaxRowSumBlocks; ++q) {
                     asm volatile("" : "+v"(early[q]));  // not to be read before the wait above
                     if (q < epi.ln.sum_blocks) {
-                        s1 += (double)early[q].x;
-                        s2 += (double)early[q].y;
+                        f1 += early[q].x;
+                        f2 += early[q].y;
                     }
                 }
-                // the variance as a difference of doubles; its reciprocal root in single precision with one Newton
-                // step (every other wave of the workgroup waits at the first barrier while these waves do this)
-                const double mean = s1 * (double)epi.ln.inv_cols;
-                const float ve    = (float)(s2 * (double)epi.ln.inv_cols - mean * mean + (double)epi.ln.eps);
+                const double mean = (double)f1 * (double)epi.ln.inv_cols;
+                const float ve    = (float)((double)f2 * (double)epi.ln.inv_cols - mean * mean + (double)epi.ln.eps);
                 float r           = __builtin_amdgcn_rsqf(ve);
                 r                 = r * (1.5f - 0.5f * ve * r * r);
                 reinterpret_cast<float2 *>(lds_dyn + CFG::lds_bytes)[tid] = make_float2(r, (float)mean);
