@@ -1037,6 +1037,7 @@ __global__ void __launch_bounds__(CFG::NT)
         for (int p = 0; p < NS - 1; ++p)
             if (p < nk)
                 issue(p, p), ++issued;
+        TR_TL(5);  // first slabs requested
         if constexpr (TakesRowSums<Epi>::value) {
             if (tid < BM) {
                 if (issued >= 2)
@@ -1064,6 +1065,7 @@ __global__ void __launch_bounds__(CFG::NT)
                 reinterpret_cast<float2 *>(lds_dyn + CFG::lds_bytes)[tid] = make_float2(r, (float)mean);
             }
         }
+        TR_TL(6);  // handed-over row sums added up (folding epilogues that take them)
         int stage = 0, fill = NS - 1;  // stage of slab kt; stage that slab kt + NS - 1 goes to
         for (int kt = 0; kt < nk; ++kt) {
             // slab kt has landed once at most the loads of the slabs issued after it are outstanding

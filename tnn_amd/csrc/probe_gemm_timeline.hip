@@ -46,7 +46,14 @@ int main(int argc, char **argv) {
     (void)hipMalloc(&gn, N * 4);
     (void)hipMalloc(&bn, N * 4);
     (void)hipMemset(stats, 0, (size_t)M * 8);
-    (void)hipMalloc(&sums, (size_t)TNN_ROCM_MAX_ROW_SUM_BLOCKS * M * 8);
+    // TNN_PROBE_SUMS_BEHIND_A=1: the row sums sit in the allocation of A, right behind it (address translation shared)
+    if (getenv("TNN_PROBE_SUMS_BEHIND_A")) {
+        (void)hipFree(A);
+        (void)hipMalloc(&A, (size_t)M * K * 2 + (size_t)TNN_ROCM_MAX_ROW_SUM_BLOCKS * M * 8);
+        (void)hipMemset(A, 0x11, (size_t)M * K * 2);
+        sums = (float *)((char *)A + (size_t)M * K * 2);
+    } else
+        (void)hipMalloc(&sums, (size_t)TNN_ROCM_MAX_ROW_SUM_BLOCKS * M * 8);
     (void)hipMemset(sums, 0, (size_t)TNN_ROCM_MAX_ROW_SUM_BLOCKS * M * 8);
     (void)hipMemset(gn, 0, N * 4);
     (void)hipMemset(bn, 0, N * 4);
@@ -92,20 +99,23 @@ int main(int argc, char **argv) {
             t0 = std::min(t0, tl[b * 8]);
             nb = b + 1;
         }
-    double sum[5] = {0}, mx[5] = {0}, mn[5] = {1e9, 1e9, 1e9, 1e9, 1e9};
+    const int order[7] = {0, 5, 6, 1, 2, 3, 4};  // stamp slots in the order the kernel passes them
+    const char *nm[7]  = {"entry", "first slabs requested", "row sums added up", "first slab landed", "main loop done",
+                          "C stored", "kernel end"};
+    double sum[7] = {0}, mx[7] = {0}, mn[7] = {1e9, 1e9, 1e9, 1e9, 1e9, 1e9, 1e9};
     int cnt = 0;
     for (int b = 0; b < nb; b++) {
         if (!tl[b * 8 + 4])
             continue;
         cnt++;
-        for (int i = 0; i < 5; i++) {
-            const double v = (tl[b * 8 + i] - t0) * 0.01;  // 100 MHz counter -> microseconds
+        for (int i = 0; i < 7; i++) {
+            const double v = tl[b * 8 + order[i]] ? (tl[b * 8 + order[i]] - t0) * 0.01 : 0.0;  // 100 MHz counter -> us
             sum[i] += v, mx[i] = std::max(mx[i], v), mn[i] = std::min(mn[i], v);
         }
     }
-    const char *nm[5] = {"entry", "first slab landed", "main loop done", "C stored", "kernel end"};
-    for (int i = 0; i < 5; i++)
-        printf("  %-18s mean %6.2f us  min %6.2f  max %6.2f   (%d workgroups, from the first workgroup's entry)\n", nm[i],
-               sum[i] / cnt, mn[i], mx[i], cnt);
+    for (int i = 0; i < 7; i++)
+        if (sum[i] > 0 || i == 0)  // the direct-to-LDS pipeline stamps all seven; the register-staged one five
+            printf("  %-22s mean %6.2f us  min %6.2f  max %6.2f   (%d workgroups, from the first workgroup's entry)\n", nm[i],
+                   sum[i] / cnt, mn[i], mx[i], cnt);
     return 0;
 }
