@@ -854,6 +854,10 @@ template <int TM_, int TN_, int WGM_, int WGN_, int WGK_, int SLAB_, int NSTAGE_
     static constexpr size_t slab_bytes  = (size_t)(NSTAGE_ ? NSTAGE_ : 2) * (BM + BN) * STRIDE;
     static constexpr size_t stage_bytes = (size_t)WGM_ * WGN_ * WGK_ * 32 * SSTR * 4;
     static constexpr size_t lds_bytes   = slab_bytes > stage_bytes ? slab_bytes : stage_bytes;
+    // where an epilogue that leaves row sums keeps its BM x BN / 8 pairs: in the part of the slab area the staging does
+    // not reach when that is large enough (dead by then), else behind everything
+    static constexpr size_t sums_bytes  = (size_t)BM * BN;
+    static constexpr size_t sums_offset = (slab_bytes >= stage_bytes + sums_bytes) ? stage_bytes : lds_bytes;
     static constexpr int NW = WGM * WGN * WGK, NT = 64 * NW;  // waves and threads per workgroup
     static_assert(NW == 4 || NW == 8, "four or eight waves per workgroup");
     static_assert((SLAB / 32) % WGK == 0, "k-steps of a slab must split evenly over the k-waves");
@@ -1293,7 +1297,7 @@ __global__ void __launch_bounds__(CFG::NT)
                     AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                     sm = epi.store8(m, n, v);
                 }
-                reinterpret_cast<float2 *>(lds_dyn + CFG::lds_bytes)[(((pos / WGN) * TM + i) * 32 + row) * (BN / 8) +
+                reinterpret_cast<float2 *>(lds_dyn + CFG::sums_offset)[(((pos / WGN) * TM + i) * 32 + row) * (BN / 8) +
                                                                      ((pos % WGN) * CW + c8) / 8] = sm;
             } else if (m < M) {
                 AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -1319,7 +1323,7 @@ __global__ void __launch_bounds__(CFG::NT)
         // that reads C next
         __syncthreads();
         if (tid < BM && m0 + tid < M) {
-            const float2 *part = reinterpret_cast<const float2 *>(lds_dyn + CFG::lds_bytes) + tid * (BN / 8);
+            const float2 *part = reinterpret_cast<const float2 *>(lds_dyn + CFG::sums_offset) + tid * (BN / 8);
             float s1 = 0.f, s2 = 0.f;
 #pragma unroll
             for (int q = 0; q < BN / 8; ++q)
@@ -1393,10 +1397,14 @@ int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int 
     }
     if (TakesRowSums<Epi>::value)
         lds = CFG::lds_bytes + (size_t)CFG::BM * 8;  // {rstd, mean} per row, parked behind the slabs before the main loop
-    if (EmitsRowSums<Epi>::value)
-        lds = CFG::lds_bytes + (size_t)CFG::BM * CFG::BN;  // eight bytes per eight columns and row, behind the staging area
-    if (lds > 160 * 1024)
-        return kTileTooLargeForSums;
+    if (EmitsRowSums<Epi>::value) {
+        // eight bytes per eight columns and row; not at the price of a workgroup per CU (the plain form runs instead)
+        const size_t with_sums = CFG::sums_offset + CFG::sums_bytes > lds ? CFG::sums_offset + CFG::sums_bytes : lds;
+        const long cu = 160 * 1024;
+        if (with_sums > (size_t)cu || cu / (long)(with_sums + 1024) < (cu / (long)(lds + 1024) > 4 ? 4 : cu / (long)(lds + 1024)))
+            return kTileTooLargeForSums;
+        lds = with_sums;
+    }
     auto kern   = gemm_nk_tiled_kernel<DT, CFG, Epi>;
     if (lds > 64 * 1024) {
         // the attribute belongs to the (kernel, device) pair: one bit per device, per instantiation
