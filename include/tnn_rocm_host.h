@@ -53,6 +53,12 @@ int tnn_host_forward(void *handle);
 /* Instance::ForwardAsync (instance.h:92): enqueue only; pair with tnn_host_sync */
 int tnn_host_forward_async(void *handle);
 int tnn_host_sync(void *handle);
+/* Instance::ForwardWithCallback (instance.h:82, default_network.cc:637-668): the layers one by one, `before` called with a
+ * layer's input blobs, `after` with its output blobs once the layer has finished on the device (either may be NULL). */
+typedef void (*tnn_host_layer_callback)(void *user, const char *layer_name, const char *layer_type, int blobs_are_outputs,
+                                        int n_blobs, const char *const *blob_names, const long long *blob_elements,
+                                        const int *blob_data_types);
+int tnn_host_forward_with_callback(void *handle, tnn_host_layer_callback before, tnn_host_layer_callback after, void *user);
 /* Instance::ShareCommandQueue (instance.h:74): `handle` launches on `other`'s stream from now on (other must outlive
  * it); Instance::SetCpuNumThreads (instance.h:135): accepted, the device does no host-side threading of layers */
 int tnn_host_share_command_queue(void *handle, void *other);

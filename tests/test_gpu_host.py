@@ -289,6 +289,37 @@ def test_two_instances_on_two_threads_match_their_sequential_results():
         inst.close()
 
 
+def test_forward_with_callback_visits_every_layer():
+    """Instance::ForwardWithCallback (default_network.cc:637-668): `before` sees every layer's input blobs, `after` its
+    output blobs once the layer has finished, in layer order; the forward gives the values of a plain Forward."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: ForwardWithCallback")
+    cfg = EncoderConfig.bert_base(2)
+    w = make_weights(cfg, seed=90, bias_std=0.02)
+    B, S = 2, 64
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 17, S, seed=91)
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), "fp16")
+    inst.set_input("input_ids", ids)
+    inst.set_input("token_type_ids", seg)
+    inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+    inst.forward()
+    plain = inst.output("last_hidden").copy()
+    seen = []
+    inst.forward_with_callback(before=lambda name, typ, blobs: seen.append(("in", name, typ, blobs)),
+                               after=lambda name, typ, blobs: seen.append(("out", name, typ, blobs)))
+    assert np.array_equal(inst.output("last_hidden"), plain)
+    layers = inst.layers()
+    io = inst.layer_io()
+    assert len(seen) == 2 * len(layers)
+    for k, ((typ, name), layer) in enumerate(zip(layers, io)):
+        b, a = seen[2 * k], seen[2 * k + 1]
+        assert (b[0], b[1], b[2]) == ("in", name, typ) and (a[0], a[1], a[2]) == ("out", name, typ)
+        assert [x[0] for x in b[3]] == layer["inputs"] and [x[0] for x in a[3]] == layer["outputs"]
+        assert [x[1] for x in a[3]] == [int(np.prod(d)) for d in layer["output_dims"]]
+    assert seen[-1][3][0][0] == "last_hidden" and seen[-1][3][0][1] == B * S * cfg.hidden
+    inst.close()
+
+
 def test_share_command_queue_and_cpu_threads():
     """Instance::ShareCommandQueue (instance.cc:158-160, default_network.cc:537-556; the CUDA backend's counterpart is
     cuda_context.cc:91-122): the second instance launches on the first one's stream from then on - its forwards, enqueued

@@ -26,6 +26,7 @@ SIGNATURES = {
     "tnn_host_forward_async": (C.c_int, [C.c_void_p]),
     "tnn_host_sync": (C.c_int, [C.c_void_p]),
     "tnn_host_stream": (C.c_void_p, [C.c_void_p]),
+    "tnn_host_forward_with_callback": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "tnn_host_share_command_queue": (C.c_int, [C.c_void_p, C.c_void_p]),
     "tnn_host_set_cpu_num_threads": (C.c_int, [C.c_void_p, C.c_int]),
     "tnn_host_get_output": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
@@ -156,6 +157,21 @@ class RocmInstance:
 
     def sync(self):
         self._check(load().tnn_host_sync(self._h), "Synchronize")
+
+    def forward_with_callback(self, before=None, after=None):
+        """Instance::ForwardWithCallback: before(layer_name, layer_type, [(blob, elements, data_type)]) with a layer's
+        inputs, after(...) with its outputs once the layer has finished"""
+        CB = C.CFUNCTYPE(None, C.c_void_p, C.c_char_p, C.c_char_p, C.c_int, C.c_int, C.POINTER(C.c_char_p),
+                         C.POINTER(C.c_longlong), C.POINTER(C.c_int))
+
+        def wrap(fn):
+            if fn is None:
+                return None
+            return CB(lambda user, name, typ, is_out, n, names, counts, types: fn(
+                name.decode(), typ.decode(), [(names[i].decode(), counts[i], types[i]) for i in range(n)]))
+        b, a = wrap(before), wrap(after)
+        self._check(load().tnn_host_forward_with_callback(self._h, C.cast(b, C.c_void_p) if b else None,
+                                                          C.cast(a, C.c_void_p) if a else None, None), "ForwardWithCallback")
 
     def share_command_queue(self, other):
         """Instance::ShareCommandQueue: launch on `other`'s stream from now on (other must outlive this instance)"""

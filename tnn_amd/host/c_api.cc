@@ -11,6 +11,7 @@
 
 #include "tnn_host.h"
 #include "tnn_rocm.h"
+#include "tnn_rocm_host.h"
 
 using namespace TNN_NS;
 
@@ -197,6 +198,30 @@ HOST_API int tnn_host_sync(void *hp) {
     if (rc != 0)
         h->err = tnn_rocm_last_error();
     return rc;
+}
+
+// Instance::ForwardWithCallback for C callers: `before` / `after` receive the layer's name and type, whether the blobs
+// are the layer's outputs, their count and, per blob, name, element count and data type
+HOST_API int tnn_host_forward_with_callback(void *hp, tnn_host_layer_callback before, tnn_host_layer_callback after, void *user) {
+    auto h    = static_cast<Handle *>(hp);
+    auto wrap = [user](tnn_host_layer_callback cb, int is_output) -> BlobStatisticCallback {
+        if (!cb)
+            return nullptr;
+        return [cb, user, is_output](std::vector<Blob *> &blobs, LayerInfo *info) {
+            std::vector<const char *> names;
+            std::vector<long long> counts;
+            std::vector<int> types;
+            for (auto b : blobs) {
+                names.push_back(b->GetBlobDesc().name.c_str());
+                counts.push_back((long long)DimsVectorUtils::Count(b->GetBlobDesc().dims));
+                types.push_back((int)b->GetBlobDesc().data_type);
+            }
+            cb(user, info ? info->name.c_str() : "", info ? info->type_str.c_str() : "", is_output, (int)blobs.size(),
+               names.data(), counts.data(), types.data());
+        };
+    };
+    Status st = h->inst->ForwardWithCallback(wrap(before, 0), wrap(after, 1));
+    return st == TNN_OK ? 0 : fail(h, st);
 }
 
 HOST_API int tnn_host_share_command_queue(void *hp, void *other) {

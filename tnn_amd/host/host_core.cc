@@ -1334,6 +1334,22 @@ Status DefaultNetwork::Forward() {
     RETURN_ON_NEQ(DefaultNetwork::ForwardAsync(nullptr), TNN_OK);
     return context_->Synchronize();
 }
+Status DefaultNetwork::ForwardWithCallback(BlobStatisticCallback before, BlobStatisticCallback after) {
+    RETURN_ON_NEQ(context_->OnInstanceForwardBegin(), TNN_OK);
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        std::vector<Blob *> inputs = layers_[i]->GetInputBlobs(), outputs = layers_[i]->GetOutputBlobs();
+        LayerInfo *info = i < structure_.layers.size() ? structure_.layers[i].get() : nullptr;
+        if (before)
+            before(inputs, info);
+        Status st = layers_[i]->Forward();
+        if (st != TNN_OK)
+            return Status((int)st, "Forward error of layer " + layers_[i]->GetLayerName() + ": " + st.description());
+        RETURN_ON_NEQ(context_->Synchronize(), TNN_OK);  // the callback may read the blobs
+        if (after)
+            after(outputs, info);
+    }
+    return context_->OnInstanceForwardEnd();
+}
 // core/abstract_network.cc:24-45
 namespace {
 std::map<NetworkType, std::shared_ptr<AbstractNetworkImplFactory>> &NetworkImplFactoryMap() {
@@ -1453,6 +1469,9 @@ Status Instance::ForwardAsync(Callback call_back) {
     return network_ ? network_->ForwardAsync(call_back) : Status(TNNERR_INST_ERR, "instance not initialised");
 }
 Status Instance::GetCommandQueue(void **q) { return network_->GetCommandQueue(q); }
+Status Instance::ForwardWithCallback(BlobStatisticCallback before, BlobStatisticCallback after) {
+    return network_->ForwardWithCallback(before, after);
+}
 Status Instance::ShareCommandQueue(Instance *instance) {
     if (!instance)
         return Status(TNNERR_NULL_PARAM, "instance is nil");

@@ -668,6 +668,8 @@ struct LayerProfile {
 };
 
 typedef std::function<void(void)> Callback;  // include/tnn/core/common.h:207
+// include/tnn/core/instance.h:39: called around every layer by ForwardWithCallback
+typedef std::function<void(std::vector<Blob *> &blobs, LayerInfo *info)> BlobStatisticCallback;
 
 // core/default_network.h:37-160.  Forward, ForwardAsync, Reshape and the profile switches are virtual and the members
 // a derived network needs are protected, as in the engine, so a device can bring its own network (core/abstract_network.h:
@@ -690,6 +692,8 @@ public:
     virtual Status Reshape(const InputShapesMap &inputs);
     virtual Status Forward();                           // default_network.cc:558-635: the layer loop, then Synchronize
     virtual Status ForwardAsync(Callback call_back);    // default_network.cc:672-686: the layer loop alone
+    // default_network.cc:637-668: `before` sees a layer's inputs, `after` its outputs once the layer has finished
+    virtual Status ForwardWithCallback(BlobStatisticCallback before, BlobStatisticCallback after);
     virtual Status GetCommandQueue(void **command_queue);
     // default_network.cc:537-556: this network's context adopts the other network's command queue; set the threads
     // the device may use on the host
@@ -761,6 +765,7 @@ public:
     Status Reshape(const InputShapesMap &inputs);  // instance.cc:143-152
     Status Forward();
     Status ForwardAsync(Callback call_back);
+    Status ForwardWithCallback(BlobStatisticCallback before, BlobStatisticCallback after);  // instance.cc:171-174
     Status GetCommandQueue(void **command_queue);
     Status ShareCommandQueue(Instance *instance);  // instance.cc:158-160
     Status SetCpuNumThreads(int num_threads);      // instance.cc:198-200
