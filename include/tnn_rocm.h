@@ -329,12 +329,16 @@ TNN_ROCM_API int tnn_rocm_gelu_i8(void *stream, const int8_t *q_in, float in_sca
  *   gemm_tune     : "MxNxK:code,..." overrides of the heuristic for single shapes (also TNN_ROCM_GEMM_TUNE at first use)
  *   gemm_group_m  : tiles per group of the XCD-aware tile order (0 = default)
  *   ln_y_ahead    : 1 (default) = the LayerNorm-folding GEMMs request the source vectors of their y output early
- *   attention_dma : 1 (default) = V^T attention stages K / V^T tiles global -> LDS directly, 0 = through registers */
+ *   attention_dma : 1 (default) = V^T attention stages K / V^T tiles global -> LDS directly, 0 = through registers
+ *   store_through : 1 (default) = GEMM and attention results are stored through the L2 at device scope, so that no
+ *                   dirty lines wait for the write-back at the end of the kernel; 0 = ordinary write-back stores.
+ *                   Read by the kernels when they run (recorded graphs follow it too); waits for the device first. */
 TNN_ROCM_API int tnn_rocm_debug_set_gemm_config(int cfg);
 TNN_ROCM_API int tnn_rocm_debug_set_gemm_tune(const char *spec);
 TNN_ROCM_API int tnn_rocm_debug_set_gemm_group_m(int group_m);
 TNN_ROCM_API int tnn_rocm_debug_set_ln_y_ahead(int on);
 TNN_ROCM_API int tnn_rocm_debug_set_attention_dma(int on);
+TNN_ROCM_API int tnn_rocm_debug_set_store_through(int on);
 
 #ifdef __cplusplus
 }

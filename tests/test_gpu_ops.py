@@ -776,6 +776,62 @@ def test_qkv_split_and_attention_vt():
     assert rel_err(out, ref_o) <= FP16_TOL
 
 
+def test_store_through_switch_changes_no_result():
+    """GEMM, attention and LayerNorm results leave the kernels through device-scope stores by default and through
+    ordinary write-back stores with the switch off: the same bits either way, in every epilogue form."""
+    say("store-through switch")
+    from tnn_amd import capi
+    lib, o = capi.load(), ops()
+    rng = np.random.default_rng(77)
+    B, S, h = 2, 136, 4
+    H, T = h * 64, 2 * 136
+    x = dev((rng.standard_normal((T, H)) * 0.5).astype(np.float32)).half()
+    w = dev((rng.standard_normal((3 * H, H)) * 0.05).astype(np.float32)).half()
+    b3 = dev((rng.standard_normal(3 * H) * 0.1).astype(np.float32))
+    x32, w32 = x.float(), w.float()
+    a8 = dev(rng.integers(-128, 128, (T, H)).astype(np.int8))
+    w8 = dev(rng.integers(-127, 128, (3 * H, H)).astype(np.int8))
+    bi = dev(rng.integers(-500, 500, 3 * H).astype(np.int32))
+    sc = dev((rng.random(3 * H) * 1e-3 + 1e-4).astype(np.float32))
+    dq = dev((rng.random(3 * H) * 0.05 + 0.01).astype(np.float32))
+    g, be = dev(rng.standard_normal(H).astype(np.float32)), dev(rng.standard_normal(H).astype(np.float32))
+    lens = dev(np.array([136, 51], np.int32))
+    res = x.clone()
+
+    def run():
+        out = []
+        out.append(o.gemm(x, w, True, bias=b3, gelu=True))
+        out.append(o.gemm(x, w[:H], True, bias=b3[:H], residual=res))
+        out.append(o.gemm(x32, w32, True, bias=b3))
+        qk, vt = o.qkv_split(x, w, b3, B, S, h)
+        out += [qk, vt]
+        ctx, ctx_q = o.attention_qk_vt(qk, vt, B, S, h, 0.125, kv_len=lens, q8_inv_scale=20.0)
+        out += [ctx, ctx_q]
+        out.append(o.attention_packed(torch.cat([qk, vt.permute(0, 3, 1, 2).reshape(T, H)], 1).contiguous(), B, S, h,
+                                      0.125, kv_len=lens))
+        q, acc, outf = o.gemm_i8(a8, w8, bi, sc, want_acc=True, dequant_scale=0.03, dequant_dtype=torch.float16)
+        out += [q, acc, outf]
+        out.append(o.gemm_i8_dequant_residual(a8, w8[:H], bi[:H], sc[:H], 0.03, residual=res, dtype=torch.float16))
+        out += list(o.gemm_i8_qkv_split(a8, w8, bi, sc, dq, B, S, h))
+        y, yq = o.layernorm(x, g, be, 1e-5, residual=res, q_inv_scale=8.0)
+        out += [y, yq]
+        torch.cuda.synchronize()
+        return out
+
+    try:
+        assert lib.tnn_rocm_debug_set_store_through(0) == 0
+        back = run()
+    finally:
+        assert lib.tnn_rocm_debug_set_store_through(1) == 0
+    through = run()
+    assert len(back) == len(through)
+    for i, (a, b) in enumerate(zip(back, through)):
+        assert torch.equal(a, b), "result %d differs between the two store forms" % i
+    # and the default form against the checker, on the plain GEMM
+    ref = orc.inner_product(x.float().cpu().numpy(), w.float().cpu().numpy()[:H], host(b3)[:H]) + host(res)
+    assert rel_err(host(through[1]), ref) <= FP16_TOL
+
+
 @pytest.mark.parametrize("dtype,tol", [("f16", FP16_TOL), ("bf16", 3e-2)])
 def test_attention_vt_scores_that_outgrow_the_running_reference(dtype, tol):
     """The V^T kernel keeps a running reference for the exponentials that only moves when a score outgrows it by a

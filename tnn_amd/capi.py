@@ -73,6 +73,7 @@ SIGNATURES = {
     "tnn_rocm_debug_set_gemm_tune": [C.c_char_p],
     "tnn_rocm_debug_set_gemm_group_m": [_i],
     "tnn_rocm_debug_set_ln_y_ahead": [_i],
+    "tnn_rocm_debug_set_store_through": [_i],
     "tnn_rocm_debug_set_attention_dma": [_i],
     "tnn_rocm_add_i8": [_vp, _vp, _f, _vp, _f, _f, _vp, _sz, _i, _sz],
     "tnn_rocm_gelu_i8": [_vp, _vp, _f, _f, _vp, _sz],

@@ -427,7 +427,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
             const int qrow = q0 + r;
             if (qrow < S) {
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + r * kRowBytes + (lane & 7) * 16);
-                *reinterpret_cast<u32x4 *>(ob + (size_t)qrow * p.o_ss + (lane & 7) * 8) = v;
+                store_out16(ob + (size_t)qrow * p.o_ss + (lane & 7) * 8, v);
                 if (p.oq) {
                     // the Reformat layer that follows in a quantised net (x86 form: multiply by 1/scale, round half
                     // away from zero, saturate), applied to the values as stored
@@ -444,7 +444,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
                         q8[w] = packed;
                     }
                     int8_t *oqb = p.oq + (size_t)b * p.o_sb + (size_t)head * p.o_sh;
-                    *reinterpret_cast<u32x2 *>(oqb + (size_t)qrow * p.o_ss + (lane & 7) * 8) = q8;
+                    store_out8(oqb + (size_t)qrow * p.o_ss + (lane & 7) * 8, q8);
                 }
             }
         }
@@ -830,7 +830,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
             const int qrow = q0 + r;
             if (qrow < S) {
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(stg + r * kRowBytes + (lane & 7) * 16);
-                *reinterpret_cast<u32x4 *>(ob + (size_t)qrow * p.o_ss + (lane & 7) * 8) = v;
+                store_out16(ob + (size_t)qrow * p.o_ss + (lane & 7) * 8, v);
                 if (p.oq) {
                     u32x2 q8;
 #pragma unroll
@@ -845,7 +845,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
                         q8[w] = packed;
                     }
                     int8_t *oqb = p.oq + (size_t)b * p.o_sb + (size_t)head * p.o_sh;
-                    *reinterpret_cast<u32x2 *>(oqb + (size_t)qrow * p.o_ss + (lane & 7) * 8) = q8;
+                    store_out8(oqb + (size_t)qrow * p.o_ss + (lane & 7) * 8, q8);
                 }
             }
         }
@@ -1016,6 +1016,7 @@ int tnn_rocm_attention_vt_q8(void *stream, int dtype, const void *q, const void 
     return launch_attention<true>((hipStream_t)stream, dtype, p, B, heads, S);
 }
 
+TR_DEFINE_STORE_THROUGH_SETTER(attention_set_store_through)
 __attribute__((visibility("default"))) int tnn_rocm_debug_set_attention_dma(int on) {
     g_attention_dma = on;
     return 0;

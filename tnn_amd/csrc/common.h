@@ -50,21 +50,69 @@ __device__ __forceinline__ bf16_bits float_to_bf16(float f) {
 }
 
 // Element load/store as float for the three floating dtypes.
+// ---- result stores --------------------------------------------------------------------------------------------------
+// When a kernel ends, the dirty lines of the eight L2s are written back before the next kernel of the stream may start
+// (the L2s are not coherent with each other, so this is what makes one kernel's results visible to the next).  A GEMM
+// that leaves 18 MB of results dirty pays about 1.8 us for that between its last instruction and its successor's first.
+// Stores issued at device scope (sc1) go through the L2 to the memory side as they are made, under the kernel's own
+// remaining work, and leave nothing to write back; they still allocate in the memory-side cache, where the consumer
+// finds them (stores with the non-temporal hint do not, which costs the consumer more than the write-back saved).
+// The compiler has no spelling for a 16-byte store at device scope, hence the assembly; a store of more than 8 bytes
+// needs two wait states before its data registers may be overwritten, which the hazard recognizer cannot see through
+// an asm statement, so they are part of it.  No memory clobber: nothing in these kernels reads what they store.
+// The switch (one copy per translation unit, set together by tnn_rocm_debug_set_store_through) is there for A/B runs.
+typedef unsigned int store_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int store_u32x2 __attribute__((ext_vector_type(2)));
+static __constant__ int g_dev_store_through = 1;
+#define TR_DEFINE_STORE_THROUGH_SETTER(name)                                                          \
+    int name(int on) { return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_dev_store_through), &on, sizeof(int)); }
+
+__device__ __forceinline__ void store_out16(void *p, store_u32x4 v) {
+    if (g_dev_store_through)
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v));
+    else
+        *reinterpret_cast<store_u32x4 *>(p) = v;
+}
+__device__ __forceinline__ void store_out8(void *p, store_u32x2 v) {
+    if (g_dev_store_through)
+        asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(p), "v"(v));
+    else
+        *reinterpret_cast<store_u32x2 *>(p) = v;
+}
+__device__ __forceinline__ void store_out4(void *p, uint32_t v) {
+    if (g_dev_store_through)
+        asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v));
+    else
+        *reinterpret_cast<uint32_t *>(p) = v;
+}
+__device__ __forceinline__ void store_out2(void *p, uint16_t v) {
+    if (g_dev_store_through)
+        asm volatile("global_store_short %0, %1, off sc1" ::"v"(p), "v"((uint32_t)v));
+    else
+        *reinterpret_cast<uint16_t *>(p) = v;
+}
+
 template <int DT> struct Elem;
 template <> struct Elem<TNN_ROCM_F32> {
     typedef float type;
     static __device__ __forceinline__ float ld(const float *p) { return *p; }
     static __device__ __forceinline__ void st(float *p, float v) { *p = v; }
+    static __device__ __forceinline__ void st_out(float *p, float v) { store_out4(p, __float_as_uint(v)); }
 };
 template <> struct Elem<TNN_ROCM_F16> {
     typedef half_t type;
     static __device__ __forceinline__ float ld(const half_t *p) { return (float)*p; }
     static __device__ __forceinline__ void st(half_t *p, float v) { *p = (half_t)v; }
+    static __device__ __forceinline__ void st_out(half_t *p, float v) {
+        const half_t h = (half_t)v;
+        store_out2(p, *reinterpret_cast<const uint16_t *>(&h));
+    }
 };
 template <> struct Elem<TNN_ROCM_BF16> {
     typedef bf16_bits type;
     static __device__ __forceinline__ float ld(const bf16_bits *p) { return bf16_to_float(*p); }
     static __device__ __forceinline__ void st(bf16_bits *p, float v) { *p = float_to_bf16(v); }
+    static __device__ __forceinline__ void st_out(bf16_bits *p, float v) { store_out2(p, float_to_bf16(v)); }
 };
 
 // Round half away from zero exactly as the reference's float2int8: add +-0.5f in fp32 (one

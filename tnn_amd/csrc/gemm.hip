@@ -101,6 +101,7 @@ template <typename E, typename = void> struct TakesRowSums : std::false_type {};
 template <typename E> struct TakesRowSums<E, typename std::enable_if<E::kTakesRowSums>::type> : std::true_type {};
 constexpr int kMaxRowSumBlocks = TNN_ROCM_MAX_ROW_SUM_BLOCKS;  // tile columns of a producer a consumer can add up (768 columns of 32)
 
+
 template <int DT> struct FloatEpilogue {
     typedef typename Elem<DT>::type T;
     static constexpr bool kRowStats = false;
@@ -165,7 +166,7 @@ template <int DT> struct FloatEpilogue {
         u32x4 *cp = reinterpret_cast<u32x4 *>(C + (size_t)m * ldc + n);
 #pragma unroll
         for (int q = 0; q < NV; ++q)
-            cp[q] = packed[q];
+            store_out16(&cp[q], packed[q]);
     }
 };
 
@@ -210,13 +211,13 @@ template <int DT> struct QkvSplitEpilogue {
             u32x4 *cp = reinterpret_cast<u32x4 *>(qk + (size_t)m * 2 * H + n);
 #pragma unroll
             for (int q = 0; q < NV; ++q)
-                cp[q] = packed[q];
+                store_out16(&cp[q], packed[q]);
         } else {
             int c = n - 2 * H, b = m / S, s_ = m - b * S;
             T *dst = vt + (((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s_;
 #pragma unroll
             for (int t = 0; t < 8; ++t)
-                Elem<DT>::st(dst + (size_t)t * S, v[t]);
+                Elem<DT>::st_out(dst + (size_t)t * S, v[t]);
         }
     }
 };
@@ -312,7 +313,7 @@ template <int DT, bool SUMS = false> struct LnFloatEpilogue {
         u32x4 *cp = reinterpret_cast<u32x4 *>(C + (size_t)m * ldc + n);
 #pragma unroll
         for (int q = 0; q < NV; ++q)
-            cp[q] = packed[q];
+            store_out16(&cp[q], packed[q]);
     }
 };
 
@@ -349,13 +350,13 @@ template <int DT, bool SUMS = false> struct LnQkvSplitEpilogue {
             u32x4 *cp = reinterpret_cast<u32x4 *>(qk + (size_t)m * 2 * H + n);
 #pragma unroll
             for (int q = 0; q < NV; ++q)
-                cp[q] = packed[q];
+                store_out16(&cp[q], packed[q]);
         } else {
             int c = n - 2 * H, bb = m / S, s_ = m - bb * S;
             T *dst = vt + (((size_t)bb * heads + (c >> 6)) * 64 + (c & 63)) * S + s_;
 #pragma unroll
             for (int t = 0; t < 8; ++t)
-                Elem<DT>::st(dst + (size_t)t * S, v[t]);
+                Elem<DT>::st_out(dst + (size_t)t * S, v[t]);
         }
     }
 };
@@ -420,7 +421,7 @@ template <int DT, bool SUMS = false> struct LnResidualEpilogue {
 #pragma unroll
         for (int q = 0; q < 8; ++q)
             Elem<DT>::st(&pe[q], v[q]);
-        *reinterpret_cast<u32x4 *>(C + (size_t)m * ldc + n) = packed;
+        store_out16(C + (size_t)m * ldc + n, packed);
         float2 sums = make_float2(0.f, 0.f);
         if constexpr (SUMS) {  // of the values as stored (rounded to the blob type): what the next GEMM reads
             ln_accumulate<DT>(__builtin_bit_cast(uint4, packed), sums.x, sums.y);
@@ -516,7 +517,7 @@ struct Int8Epilogue {
                     q[t] = lut_lds[(int)q[t] + 128];
             }
             if (out)
-                *reinterpret_cast<uint2 *>(out + o) = *reinterpret_cast<const uint2 *>(q);
+                store_out8(out + o, *reinterpret_cast<const store_u32x2 *>(q));
             if (out_f) {
                 float d[8];
 #pragma unroll
@@ -531,8 +532,10 @@ struct Int8Epilogue {
                         d[6] = __fadd_rn(d[6], r1.z), d[7] = __fadd_rn(d[7], r1.w);
                     }
                     float4 *fp = reinterpret_cast<float4 *>((float *)out_f + o);
-                    fp[0] = make_float4(d[0], d[1], d[2], d[3]);
-                    fp[1] = make_float4(d[4], d[5], d[6], d[7]);
+                    store_out16(fp, store_u32x4{__float_as_uint(d[0]), __float_as_uint(d[1]), __float_as_uint(d[2]),
+                                                __float_as_uint(d[3])});
+                    store_out16(fp + 1, store_u32x4{__float_as_uint(d[4]), __float_as_uint(d[5]), __float_as_uint(d[6]),
+                                                    __float_as_uint(d[7])});
                 } else {
                     half_t h[8];
                     if (residual) {
@@ -544,7 +547,7 @@ struct Int8Epilogue {
 #pragma unroll
                     for (int t = 0; t < 8; ++t)
                         h[t] = (half_t)d[t];
-                    *reinterpret_cast<u32x4 *>((half_t *)out_f + o) = *reinterpret_cast<const u32x4 *>(h);
+                    store_out16((half_t *)out_f + o, *reinterpret_cast<const u32x4 *>(h));
                 }
             }
         }
@@ -613,13 +616,13 @@ template <int DT> struct Int8QkvSplitEpilogue {
             u32x4 *cp = reinterpret_cast<u32x4 *>(qk + (size_t)m * 2 * H + n);
 #pragma unroll
             for (int q = 0; q < NV; ++q)
-                cp[q] = packed[q];
+                store_out16(&cp[q], packed[q]);
         } else {
             int c = n - 2 * H, b = m / S, s_ = m - b * S;
             T *dst = vt + (((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s_;
 #pragma unroll
             for (int t = 0; t < 8; ++t)
-                Elem<DT>::st(dst + (size_t)t * S, v[t]);
+                Elem<DT>::st_out(dst + (size_t)t * S, v[t]);
         }
     }
 };
@@ -1997,6 +2000,7 @@ __attribute__((visibility("default"))) int tnn_rocm_debug_set_gemm_tune(const ch
     parse_tune(spec);
     return 0;
 }
+TR_DEFINE_STORE_THROUGH_SETTER(gemm_set_store_through)
 __attribute__((visibility("default"))) int tnn_rocm_debug_set_ln_y_ahead(int on) {
     g_ln_y_ahead = on ? 1 : 0;
     return 0;

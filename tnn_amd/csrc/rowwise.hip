@@ -170,7 +170,7 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
 #pragma unroll
                 for (int t = 0; t < VEC; ++t)
                     Elem<DT>::st(&e[t], o[t]);
-                reinterpret_cast<uint4 *>(py)[vi] = raw;
+                store_out16(reinterpret_cast<uint4 *>(py) + vi, store_u32x4{raw.x, raw.y, raw.z, raw.w});
                 if (pq) {  // the VEC (4 or 8) quantised values of this lane leave as one 4- or 8-byte store
                     uint32_t w[2] = {0u, 0u};
 #pragma unroll
@@ -179,9 +179,9 @@ __global__ void __launch_bounds__(kBlock) layernorm_kernel(const typename Elem<D
                         w[t >> 2] |= (uint32_t)(uint8_t)q << (8 * (t & 3));
                     }
                     if (VEC == 8)
-                        *reinterpret_cast<uint2 *>(pq + (size_t)vi * VEC) = make_uint2(w[0], w[1]);
+                        store_out8(pq + (size_t)vi * VEC, store_u32x2{w[0], w[1]});
                     else
-                        *reinterpret_cast<uint32_t *>(pq + (size_t)vi * VEC) = w[0];
+                        store_out4(pq + (size_t)vi * VEC, w[0]);
                 }
             } else {
                 T tmp;
@@ -385,6 +385,7 @@ int launch_softmax(hipStream_t s, const void *x, void *y, int outer, int channel
 }  // namespace
 
 extern "C" {
+TR_DEFINE_STORE_THROUGH_SETTER(rowwise_set_store_through)
 
 int tnn_rocm_layernorm(void *stream, int dtype, const void *x, const void *residual, const float *gamma,
                        const float *beta, void *y, int rows, int cols, float eps, int8_t *out_q, float q_inv_scale) {

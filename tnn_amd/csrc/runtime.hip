@@ -188,6 +188,23 @@ int tnn_rocm_event_record(void *event, void *stream) {
     return 0;
 }
 
+// every translation unit holds its own copy of the switch (common.h); they are set together (weak: a stand-alone
+// program may link this file with only some of the kernels)
+__attribute__((weak)) int gemm_set_store_through(int on);
+__attribute__((weak)) int attention_set_store_through(int on);
+__attribute__((weak)) int rowwise_set_store_through(int on);
+__attribute__((visibility("default"))) int tnn_rocm_debug_set_store_through(int on) {
+    on = on ? 1 : 0;
+    TR_CHECK_HIP(hipDeviceSynchronize());
+    if (gemm_set_store_through)
+        TR_CHECK_HIP((hipError_t)gemm_set_store_through(on));
+    if (attention_set_store_through)
+        TR_CHECK_HIP((hipError_t)attention_set_store_through(on));
+    if (rowwise_set_store_through)
+        TR_CHECK_HIP((hipError_t)rowwise_set_store_through(on));
+    return 0;
+}
+
 int tnn_rocm_event_elapsed_ms(void *start, void *stop, float *ms) {
     TR_REQUIRE(start && stop && ms, TNN_ROCM_EINVAL, "event_elapsed_ms: null argument");
     TR_CHECK_HIP(hipEventSynchronize((hipEvent_t)stop));
