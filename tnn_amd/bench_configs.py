@@ -7,6 +7,10 @@
 
     python -m tnn_amd.bench_configs --config c5 [--steps 20] [--layers N]
 
+  stores  the headline forward (12-layer BERT-base fp16, B8 S384) with the results of the GEMM / attention / LayerNorm
+          kernels stored through the L2 at device scope (the default) against ordinary write-back stores: one instance,
+          one recorded graph, the switch (tnn_rocm_debug_set_store_through) flipped between timing rounds
+
 Every configuration runs Instance::Forward on DEVICE_ROCM from .tnnproto/.tnnmodel bytes built in memory (synthetic
 weights and inputs, seeded), prints one JSON line and needs the built libraries; nothing falls back to the CPU."""
 import argparse
@@ -141,15 +145,47 @@ def c5(args):
     return out
 
 
+def stores(args):
+    from . import capi
+    lib = capi.load()
+    cfg = EncoderConfig.bert_base(args.layers or 12)
+    B, S = 8, 384
+    w = make_weights(cfg, seed=20240601)
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 200, S, seed=20240602)
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), "fp16")
+    inst.set_input("input_ids", ids)
+    inst.set_input("token_type_ids", seg)
+    inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+    for _ in range(6):
+        inst.forward()
+    ms, outs = {1: [], 0: []}, {}
+    try:
+        for _ in range(10):
+            for through in (1, 0):
+                inst.sync()
+                lib.tnn_rocm_debug_set_store_through(through)
+                ms[through].append(_time_forward(inst, args.steps, warmup=3) * 1e3)
+                outs[through] = inst.output("last_hidden")
+    finally:
+        lib.tnn_rocm_debug_set_store_through(1)
+    inst.close()
+    med = {k: sorted(v)[len(v) // 2] for k, v in ms.items()}
+    return {"config": "stores", "workload": "%d-layer BERT-base fp16, B8 S384, one instance, ten rounds each" % cfg.layers,
+            "ms_per_forward_store_through": round(med[1], 4), "ms_per_forward_write_back": round(med[0], 4),
+            "min_max_store_through": [round(min(ms[1]), 4), round(max(ms[1]), 4)],
+            "min_max_write_back": [round(min(ms[0]), 4), round(max(ms[0]), 4)],
+            "outputs_identical": bool(np.array_equal(outs[0], outs[1]))}
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--config", choices=["c1", "c3", "c4", "c5"], required=True)
+    ap.add_argument("--config", choices=["c1", "c3", "c4", "c5", "stores"], required=True)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration names (c4, c5)")
     ap.add_argument("--batch", type=int, default=0, help="c3: batch instead of 32")
     ap.add_argument("--seq", type=int, default=0, help="c3: sequence length instead of 512")
     args = ap.parse_args()
-    print(json.dumps({"c1": c1, "c3": c3, "c4": c4, "c5": c5}[args.config](args)))
+    print(json.dumps({"c1": c1, "c3": c3, "c4": c4, "c5": c5, "stores": stores}[args.config](args)))
 
 
 if __name__ == "__main__":

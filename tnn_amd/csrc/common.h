@@ -79,6 +79,9 @@ __device__ __forceinline__ void store_out8(void *p, store_u32x2 v) {
     else
         *reinterpret_cast<store_u32x2 *>(p) = v;
 }
+__device__ __forceinline__ void store_out8(float2 *p, float2 v) {
+    store_out8((void *)p, store_u32x2{__float_as_uint(v.x), __float_as_uint(v.y)});
+}
 __device__ __forceinline__ void store_out4(void *p, uint32_t v) {
     if (g_dev_store_through)
         asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v));

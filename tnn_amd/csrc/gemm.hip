@@ -1207,7 +1207,7 @@ __global__ void __launch_bounds__(CFG::NT)
     if constexpr (Epi::kRowStats && TakesRowSums<Epi>::value) {
         // {rstd, mean} were parked in LDS before the main loop (the barrier above orders that write); hand them on
         if (epi.ln.stats && n0 == 0 && tid < BM && m0 + tid < M)
-            epi.ln.stats[m0 + tid] = row_st[tid];
+            store_out8(&epi.ln.stats[m0 + tid], row_st[tid]);
     }
     if constexpr (Epi::kRowStats && !TakesRowSums<Epi>::value) {
         static_assert(CFG::NSTAGE > 0, "LayerNorm-folding epilogues run on the direct-to-LDS pipeline");
@@ -1227,7 +1227,7 @@ __global__ void __launch_bounds__(CFG::NT)
             const float2 st   = make_float2((float)(1.0 / sqrt(var + (double)epi.ln.eps)), (float)mean);
             row_st[tid]       = st;
             if (epi.ln.stats && n0 == 0 && m0 + tid < M)  // every tile column holds them; the first one hands them on
-                epi.ln.stats[m0 + tid] = st;
+                store_out8(&epi.ln.stats[m0 + tid], st);
         }
         // row_st is read after the first staging barrier below
     }
@@ -1331,7 +1331,7 @@ __global__ void __launch_bounds__(CFG::NT)
 #pragma unroll
             for (int q = 0; q < BN / 8; ++q)
                 s1 += part[q].x, s2 += part[q].y;
-            epi.row_sums[(size_t)(n0 / BN) * M + m0 + tid] = make_float2(s1, s2);
+            store_out8(&epi.row_sums[(size_t)(n0 / BN) * M + m0 + tid], make_float2(s1, s2));
         }
     }
     if constexpr (Epi::kRowStats) {

@@ -57,6 +57,9 @@ int main(int argc, char **argv) {
     (void)hipMemset(sums, 0, (size_t)TNN_ROCM_MAX_ROW_SUM_BLOCKS * M * 8);
     (void)hipMemset(gn, 0, N * 4);
     (void)hipMemset(bn, 0, N * 4);
+    // TNN_PROBE_WRITE_BACK=1: ordinary write-back stores for the results instead of the device-scope stores
+    if (getenv("TNN_PROBE_WRITE_BACK"))
+        (void)tnn_rocm_debug_set_store_through(0);
     hipStream_t s;
     (void)hipStreamCreate(&s);
     auto call = [&]() {
@@ -117,5 +120,7 @@ int main(int argc, char **argv) {
         if (sum[i] > 0 || i == 0)  // the direct-to-LDS pipeline stamps all seven; the register-staged one five
             printf("  %-22s mean %6.2f us  min %6.2f  max %6.2f   (%d workgroups, from the first workgroup's entry)\n", nm[i],
                    sum[i] / cnt, mn[i], mx[i], cnt);
+    printf("  %-22s %6.2f us   (launch to launch minus the last workgroup's end)\n", "until the next launch",
+           ms * 1000 / 200 - mx[6]);
     return 0;
 }
