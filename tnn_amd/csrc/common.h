@@ -121,10 +121,11 @@ template <> struct Elem<TNN_ROCM_BF16> {
 // Round half away from zero exactly as the reference's float2int8: add +-0.5f in fp32 (one
 // rounding), clamp in fp32, truncate.  The translation units are compiled with -ffp-contract=off
 // so the add is never fused with the multiply that produced v.
+// (+-0.5 taken from the sign bit and the clamp as one med3 give the same result for every value that is not a NaN --
+// -0.0 lands on 0 either way -- in three instructions instead of seven.)
 __device__ __forceinline__ int8_t float2int8_ref(float v) {
-    float t = __fadd_rn(v, v >= 0.f ? 0.5f : -0.5f);
-    t       = fminf(t, 127.0f);
-    t       = fmaxf(t, -128.0f);
+    float t = __fadd_rn(v, __builtin_copysignf(0.5f, v));
+    t       = __builtin_amdgcn_fmed3f(t, -128.0f, 127.0f);
     return (int8_t)(int)t;
 }
 
@@ -147,7 +148,8 @@ __device__ __forceinline__ float gelu_erf(float x) {
 // Stegun used before and ~40 for erff.  Against the correctly rounded fp16 result 0.4 % of the values differ, by one
 // ulp (2.8 % for the rational form).  fp32 outputs keep gelu_erf.
 __device__ __forceinline__ float gelu_erf_fast(float x) {
-    const float a = fminf(fabsf(x), 9.0f);
+    // med3 instead of fmin / fmax: one instruction each, where the minimum / maximum forms first quiet their operand
+    const float a = __builtin_amdgcn_fmed3f(fabsf(x), 0.f, 9.0f);
     float q       = -2.8009472064e-05f;
     q             = fmaf(q, a, 6.8930927528e-04f);
     q             = fmaf(q, a, -7.6513012845e-03f);
@@ -156,7 +158,8 @@ __device__ __forceinline__ float gelu_erf_fast(float x) {
     q             = fmaf(q, a, 1.1508630942e+00f);
     q             = fmaf(q, a, 1.0f);
     const float e = __builtin_amdgcn_exp2f(-q);  // Phi(-a)
-    return fmaf(-a, e, fmaxf(x, 0.f));  // the clamped a: a*Phi(-a) is below 1e-18 past 9, and +inf stays +inf
+    // the clamped a: a*Phi(-a) is below 1e-18 past 9, and +inf stays +inf
+    return fmaf(-a, e, __builtin_amdgcn_fmed3f(x, 0.f, __builtin_inff()));
 }
 
 __device__ __forceinline__ float wave_sum(float v) {

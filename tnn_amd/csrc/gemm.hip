@@ -99,6 +99,15 @@ template <typename E, typename = void> struct EmitsRowSums : std::false_type {};
 template <typename E> struct EmitsRowSums<E, typename std::enable_if<E::kEmitsRowSums>::type> : std::true_type {};
 template <typename E, typename = void> struct TakesRowSums : std::false_type {};
 template <typename E> struct TakesRowSums<E, typename std::enable_if<E::kTakesRowSums>::type> : std::true_type {};
+//   kColArrays     the epilogue reads that many per-column float arrays (col_src(k, n)) in store8.  The tiled kernel
+//                  copies the tile's columns of each into LDS once, after the main loop, and store8 takes them from
+//                  there (cl[k * cs + j] for column j of the item): an item then waits for two LDS reads instead of
+//                  for global loads that cannot be moved above the previous item's stores
+//   kRowIn         likewise for one float2 per row (row_src(m)), handed to store8 by value
+template <typename E, typename = void> struct ColArrays : std::integral_constant<int, 0> {};
+template <typename E> struct ColArrays<E, typename std::enable_if<(E::kColArrays > 0)>::type> : std::integral_constant<int, E::kColArrays> {};
+template <typename E, typename = void> struct RowIn : std::false_type {};
+template <typename E> struct RowIn<E, typename std::enable_if<E::kRowIn>::type> : std::true_type {};
 constexpr int kMaxRowSumBlocks = TNN_ROCM_MAX_ROW_SUM_BLOCKS;  // tile columns of a producer a consumer can add up (768 columns of 32)
 
 
@@ -133,13 +142,16 @@ template <int DT> struct FloatEpilogue {
     __device__ __forceinline__ bool direct(int) const { return false; }
     // eight consecutive columns n..n+7 of row m (n % 8 == 0, n + 7 < N, rows 16-byte aligned): whole 16-byte
     // (half) / 32-byte (fp32) pieces, so that the lanes of one row together write full cache lines
-    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8]) const {
+    static constexpr int kColArrays = 1;  // bias
+    __device__ __forceinline__ float col_src(int, int n) const { return (flags & TNN_ROCM_EPI_BIAS) ? bias[n] : 0.f; }
+    // cl = the item's eight columns of the bias in LDS
+    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8], const float *cl, int) const {
         float v[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t)
             v[t] = acc[t];
         if (flags & TNN_ROCM_EPI_BIAS) {
-            float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
+            float4 b0 = *reinterpret_cast<const float4 *>(cl), b1 = *reinterpret_cast<const float4 *>(cl + 4);
             v[0] += b0.x, v[1] += b0.y, v[2] += b0.z, v[3] += b0.w;
             v[4] += b1.x, v[5] += b1.y, v[6] += b1.z, v[7] += b1.w;
         }
@@ -191,13 +203,15 @@ template <int DT> struct QkvSplitEpilogue {
     }
     // the V^T columns are written with consecutive lanes along s; Q|K rows with consecutive lanes along the row
     __device__ __forceinline__ bool direct(int n0) const { return n0 >= 2 * H; }
-    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8]) const {
+    static constexpr int kColArrays = 1;  // bias
+    __device__ __forceinline__ float col_src(int, int n) const { return bias ? bias[n] : 0.f; }
+    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8], const float *cl, int) const {
         float v[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t)
             v[t] = acc[t];
         if (bias) {
-            float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
+            float4 b0 = *reinterpret_cast<const float4 *>(cl), b1 = *reinterpret_cast<const float4 *>(cl + 4);
             v[0] += b0.x, v[1] += b0.y, v[2] += b0.z, v[3] += b0.w;
             v[4] += b1.x, v[5] += b1.y, v[6] += b1.z, v[7] += b1.w;
         }
@@ -280,10 +294,12 @@ template <int DT, bool SUMS = false> struct LnFloatEpilogue {
     __device__ __forceinline__ float col_const(int) const { return 0.f; }
     __device__ __forceinline__ void store(int, int, float, float) const {}  // N % 8 == 0 is required at launch
     __device__ __forceinline__ bool direct(int) const { return false; }
-    // st = {rstd, mean} of row m
-    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8], float2 st) const {
-        float4 g0 = *reinterpret_cast<const float4 *>(ln.colsum + n), g1 = *reinterpret_cast<const float4 *>(ln.colsum + n + 4);
-        float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
+    static constexpr int kColArrays = 2;  // colsum, b'
+    __device__ __forceinline__ float col_src(int k, int n) const { return k == 0 ? ln.colsum[n] : bias[n]; }
+    // st = {rstd, mean} of row m; cl = the item's eight columns of the two arrays in LDS, cs apart
+    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8], float2 st, const float *cl, int cs) const {
+        float4 g0 = *reinterpret_cast<const float4 *>(cl), g1 = *reinterpret_cast<const float4 *>(cl + 4);
+        float4 b0 = *reinterpret_cast<const float4 *>(cl + cs), b1 = *reinterpret_cast<const float4 *>(cl + cs + 4);
         const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
         const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
         float v[8];
@@ -331,9 +347,11 @@ template <int DT, bool SUMS = false> struct LnQkvSplitEpilogue {
     __device__ __forceinline__ float col_const(int) const { return 0.f; }
     __device__ __forceinline__ void store(int, int, float, float) const {}
     __device__ __forceinline__ bool direct(int n0) const { return n0 >= 2 * H; }
-    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8], float2 st) const {
-        float4 g0 = *reinterpret_cast<const float4 *>(ln.colsum + n), g1 = *reinterpret_cast<const float4 *>(ln.colsum + n + 4);
-        float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
+    static constexpr int kColArrays = 2;  // colsum, b'
+    __device__ __forceinline__ float col_src(int k, int n) const { return k == 0 ? ln.colsum[n] : bias[n]; }
+    __device__ __forceinline__ void store8(int m, int n, const float (&acc)[8], float2 st, const float *cl, int cs) const {
+        float4 g0 = *reinterpret_cast<const float4 *>(cl), g1 = *reinterpret_cast<const float4 *>(cl + 4);
+        float4 b0 = *reinterpret_cast<const float4 *>(cl + cs), b1 = *reinterpret_cast<const float4 *>(cl + cs + 4);
         const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
         const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
         float v[8];
@@ -391,28 +409,31 @@ template <int DT, bool SUMS = false> struct LnResidualEpilogue {
         Elem<DT>::st(&C[(size_t)m * ldc + n], v);
     }
     __device__ __forceinline__ bool direct(int) const { return false; }
-    __device__ __forceinline__ float2 store8(int m, int n, const float (&acc)[8]) const {
+    static constexpr int kColArrays = 3;  // bias (zeros without one), gamma, beta
+    static constexpr bool kRowIn    = true;  // {rstd, mean} of the rows of t
+    __device__ __forceinline__ float col_src(int k, int n) const {
+        return k == 0 ? ((flags & TNN_ROCM_EPI_BIAS) ? bias[n] : 0.f) : k == 1 ? gamma[n] : beta[n];
+    }
+    __device__ __forceinline__ float2 row_src(int m) const { return st[m]; }
+    // cl = the item's eight columns of the three arrays in LDS, cs apart; s = {rstd, mean} of row m
+    __device__ __forceinline__ float2 store8(int m, int n, const float (&acc)[8], const float *cl, int cs, float2 s) const {
+        static_assert(sizeof(T) == 2, "half-precision blobs only");
+        u32x4 packed = *reinterpret_cast<const u32x4 *>(t + (size_t)m * ldc + n);
         float v[8];
-#pragma unroll
-        for (int q = 0; q < 8; ++q)
-            v[q] = acc[q];
-        if (flags & TNN_ROCM_EPI_BIAS) {
-            float4 b0 = *reinterpret_cast<const float4 *>(bias + n), b1 = *reinterpret_cast<const float4 *>(bias + n + 4);
-            v[0] += b0.x, v[1] += b0.y, v[2] += b0.z, v[3] += b0.w;
-            v[4] += b1.x, v[5] += b1.y, v[6] += b1.z, v[7] += b1.w;
+        {
+            float4 b0 = *reinterpret_cast<const float4 *>(cl), b1 = *reinterpret_cast<const float4 *>(cl + 4);
+            v[0] = acc[0] + b0.x, v[1] = acc[1] + b0.y, v[2] = acc[2] + b0.z, v[3] = acc[3] + b0.w;
+            v[4] = acc[4] + b1.x, v[5] = acc[5] + b1.y, v[6] = acc[6] + b1.z, v[7] = acc[7] + b1.w;
         }
         if (flags & TNN_ROCM_EPI_GELU) {
 #pragma unroll
             for (int q = 0; q < 8; ++q)
                 v[q] = gelu_erf_fast(v[q]);
         }
-        static_assert(sizeof(T) == 2, "half-precision blobs only");
-        u32x4 packed = *reinterpret_cast<const u32x4 *>(t + (size_t)m * ldc + n);
         T *pe = reinterpret_cast<T *>(&packed);
-        const float2 s = st[m];
         const float mrs = s.y * s.x;
-        float4 k0 = *reinterpret_cast<const float4 *>(gamma + n), k1 = *reinterpret_cast<const float4 *>(gamma + n + 4);
-        float4 e0 = *reinterpret_cast<const float4 *>(beta + n), e1 = *reinterpret_cast<const float4 *>(beta + n + 4);
+        float4 k0 = *reinterpret_cast<const float4 *>(cl + cs), k1 = *reinterpret_cast<const float4 *>(cl + cs + 4);
+        float4 e0 = *reinterpret_cast<const float4 *>(cl + 2 * cs), e1 = *reinterpret_cast<const float4 *>(cl + 2 * cs + 4);
         const float kk[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
         const float ee[8] = {e0.x, e0.y, e0.z, e0.w, e1.x, e1.y, e1.z, e1.w};
 #pragma unroll
@@ -484,13 +505,18 @@ struct Int8Epilogue {
     }
     __device__ __forceinline__ bool direct(int) const { return false; }
     // eight consecutive columns (n % 8 == 0, n + 7 < N, ldo % 8 == 0): same arithmetic as store(), vector accesses
-    __device__ __forceinline__ void store8(int m, int n, const int (&acc)[8], const int8_t *lut_lds = nullptr) const {
+    static constexpr int kColArrays = 2;  // bias (its int32 bits), scale
+    __device__ __forceinline__ float col_src(int k, int n) const {
+        return k == 0 ? (bias ? __int_as_float(bias[n]) : 0.f) : (scale ? scale[n] : 0.f);
+    }
+    // cl = the item's eight columns of the two arrays in LDS, cs apart
+    __device__ __forceinline__ void store8(int m, int n, const int (&acc)[8], const int8_t *lut_lds, const float *cl, int cs) const {
         int a[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t)
             a[t] = acc[t];
         if (bias) {
-            i32x4 b0 = *reinterpret_cast<const i32x4 *>(bias + n), b1 = *reinterpret_cast<const i32x4 *>(bias + n + 4);
+            i32x4 b0 = *reinterpret_cast<const i32x4 *>(cl), b1 = *reinterpret_cast<const i32x4 *>(cl + 4);
 #pragma unroll
             for (int t = 0; t < 4; ++t)
                 a[t] += b0[t], a[4 + t] += b1[t];
@@ -504,7 +530,7 @@ struct Int8Epilogue {
         if (out || out_f) {
             float sc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             if (scale) {
-                float4 s0 = *reinterpret_cast<const float4 *>(scale + n), s1 = *reinterpret_cast<const float4 *>(scale + n + 4);
+                float4 s0 = *reinterpret_cast<const float4 *>(cl + cs), s1 = *reinterpret_cast<const float4 *>(cl + cs + 4);
                 sc[0] = s0.x, sc[1] = s0.y, sc[2] = s0.z, sc[3] = s0.w, sc[4] = s1.x, sc[5] = s1.y, sc[6] = s1.z, sc[7] = s1.w;
             }
             int8_t q[8];
@@ -590,13 +616,15 @@ template <int DT> struct Int8QkvSplitEpilogue {
         }
     }
     __device__ __forceinline__ bool direct(int n0) const { return n0 >= 2 * H; }
-    __device__ __forceinline__ void store8(int m, int n, const int (&acc)[8]) const {
-        // per-column constants as 16-byte loads (n % 8 == 0 and the arrays are 16-byte aligned, checked at launch)
-        i32x4 b0 = {0, 0, 0, 0}, b1 = {0, 0, 0, 0};
-        if (bias)
-            b0 = *reinterpret_cast<const i32x4 *>(bias + n), b1 = *reinterpret_cast<const i32x4 *>(bias + n + 4);
-        const float4 s0 = *reinterpret_cast<const float4 *>(scale + n), s1 = *reinterpret_cast<const float4 *>(scale + n + 4);
-        const float4 d0 = *reinterpret_cast<const float4 *>(dequant + n), d1 = *reinterpret_cast<const float4 *>(dequant + n + 4);
+    static constexpr int kColArrays = 3;  // bias (its int32 bits), scale, dequant
+    __device__ __forceinline__ float col_src(int k, int n) const {
+        return k == 0 ? (bias ? __int_as_float(bias[n]) : 0.f) : k == 1 ? scale[n] : dequant[n];
+    }
+    __device__ __forceinline__ void store8(int m, int n, const int (&acc)[8], const float *cl, int cs) const {
+        // the item's eight columns of the three arrays, from LDS
+        const i32x4 b0 = *reinterpret_cast<const i32x4 *>(cl), b1 = *reinterpret_cast<const i32x4 *>(cl + 4);
+        const float4 s0 = *reinterpret_cast<const float4 *>(cl + cs), s1 = *reinterpret_cast<const float4 *>(cl + cs + 4);
+        const float4 d0 = *reinterpret_cast<const float4 *>(cl + 2 * cs), d1 = *reinterpret_cast<const float4 *>(cl + 2 * cs + 4);
         const int bb[8]   = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
         const float sc[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
         const float dq[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
@@ -866,6 +894,27 @@ template <int TM_, int TN_, int WGM_, int WGN_, int WGK_, int SLAB_, int NSTAGE_
     static_assert((SLAB / 32) % WGK == 0, "k-steps of a slab must split evenly over the k-waves");
     static_assert((BM * (SLAB / 16)) % NT == 0 && (BN * (SLAB / 16)) % NT == 0, "slab must divide over the workgroup");
     static_assert(NSTAGE_ == 0 || NSTAGE_ == 2 || NSTAGE_ == 3, "register-staged, or two / three direct-to-LDS stages");
+};
+
+// Dynamic LDS of one (tile shape, epilogue) pair, for the kernel and its launcher alike: the slab / staging area, what
+// the epilogue keeps behind it, and at the very end the tile's columns of the epilogue's per-column arrays followed by
+// its per-row pairs.
+template <typename CFG, typename Epi> struct EpiLds {
+    static constexpr size_t lut_need   = CFG::stage_bytes + 256;  // Int8Epilogue's table behind the staging area
+    static constexpr size_t stats_need = CFG::stage_bytes + (size_t)CFG::BM * 8 * (1 + 2 * CFG::WGK * CFG::WGN);
+    static constexpr size_t base0 = std::is_same<Epi, Int8Epilogue>::value && lut_need > CFG::lds_bytes ? lut_need : CFG::lds_bytes;
+    // row statistics and the partial-sum buffer sit behind the staging area; handed-over sums park {rstd, mean} per row
+    // behind the slabs before the main loop
+    static constexpr size_t base1 = TakesRowSums<Epi>::value ? CFG::lds_bytes + (size_t)CFG::BM * 8
+                                    : (Epi::kRowStats && stats_need > base0) ? stats_need : base0;
+    // without / with the row-sum side output (eight bytes per eight columns and row)
+    static constexpr size_t plain     = base1;
+    static constexpr size_t with_sums = CFG::sums_offset + CFG::sums_bytes > base1 ? CFG::sums_offset + CFG::sums_bytes : base1;
+    static constexpr size_t front      = EmitsRowSums<Epi>::value ? with_sums : plain;
+    static constexpr size_t col_offset = (front + 15) & ~(size_t)15;
+    static constexpr size_t row_offset = col_offset + (size_t)ColArrays<Epi>::value * CFG::BN * 4;
+    static constexpr size_t side_bytes = (size_t)ColArrays<Epi>::value * CFG::BN * 4 + (RowIn<Epi>::value ? (size_t)CFG::BM * 8 : 0);
+    static constexpr size_t total      = col_offset + side_bytes;
 };
 
 // s_waitcnt that waits only for the vector-memory counter to drop to n (gfx9 encoding: vmcnt in bits 3:0 and
@@ -1204,6 +1253,24 @@ __global__ void __launch_bounds__(CFG::NT)
             reinterpret_cast<uint32_t *>(lut_lds)[tid] = reinterpret_cast<const uint32_t *>(epi.lut)[tid];
         // read after the first staging barrier below
     }
+    // the tile's columns of the epilogue's per-column arrays, and its rows' pairs: read after the first staging barrier
+    float *const col_lds        = reinterpret_cast<float *>(lds_dyn + EpiLds<CFG, Epi>::col_offset);
+    const float2 *const row_lds = reinterpret_cast<const float2 *>(lds_dyn + EpiLds<CFG, Epi>::row_offset);
+    if constexpr (ColArrays<Epi>::value > 0) {
+#pragma unroll
+        for (int q = 0; q < (ColArrays<Epi>::value * BN + NT - 1) / NT; ++q) {
+            const int e = q * NT + tid;
+            if (e < ColArrays<Epi>::value * BN) {
+                const int c = e % BN;
+                col_lds[e]  = n0 + c < N ? epi.col_src(e / BN, n0 + c) : 0.f;
+            }
+        }
+    }
+    if constexpr (RowIn<Epi>::value) {
+        if (tid < BM)
+            reinterpret_cast<float2 *>(lds_dyn + EpiLds<CFG, Epi>::row_offset)[tid] =
+                m0 + tid < M ? epi.row_src(m0 + tid) : make_float2(0.f, 0.f);
+    }
     if constexpr (Epi::kRowStats && TakesRowSums<Epi>::value) {
         // {rstd, mean} were parked in LDS before the main loop (the barrier above orders that write); hand them on
         if (epi.ln.stats && n0 == 0 && tid < BM && m0 + tid < M)
@@ -1287,10 +1354,11 @@ __global__ void __launch_bounds__(CFG::NT)
             }
             const int m = m0 + ((pos / WGN) * TM + i) * 32 + row;
             const int n = n0 + (pos % WGN) * CW + c8;
+            const int nl = (pos % WGN) * CW + c8;  // column inside the tile
             if constexpr (Epi::kRowStats) {
                 if (m < M && n + 7 < N) {  // N is a multiple of 8 for these epilogues (checked at launch)
                     AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    epi.store8(m, n, v, row_st[m - m0]);
+                    epi.store8(m, n, v, row_st[m - m0], col_lds + nl, BN);
                 }
             } else if constexpr (EmitsRowSums<Epi>::value) {
                 // N is a multiple of 8 for these epilogues (checked at launch); every item leaves its eight columns'
@@ -1298,7 +1366,7 @@ __global__ void __launch_bounds__(CFG::NT)
                 float2 sm = make_float2(0.f, 0.f);
                 if (m < M && n + 7 < N) {
                     AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    sm = epi.store8(m, n, v);
+                    sm = epi.store8(m, n, v, col_lds + nl, BN, row_lds[m - m0]);
                 }
                 reinterpret_cast<float2 *>(lds_dyn + CFG::sums_offset)[(((pos / WGN) * TM + i) * 32 + row) * (BN / 8) +
                                                                      ((pos % WGN) * CW + c8) / 8] = sm;
@@ -1306,7 +1374,11 @@ __global__ void __launch_bounds__(CFG::NT)
                 AccT v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 if (n + 7 < N) {
                     if constexpr (std::is_same<Epi, Int8Epilogue>::value)
-                        epi.store8(m, n, v, epi.lut ? lut_lds : nullptr);
+                        epi.store8(m, n, v, epi.lut ? lut_lds : nullptr, col_lds + nl, BN);
+                    else if constexpr (RowIn<Epi>::value)
+                        (void)epi.store8(m, n, v, col_lds + nl, BN, row_lds[m - m0]);
+                    else if constexpr (ColArrays<Epi>::value > 0)
+                        epi.store8(m, n, v, col_lds + nl, BN);
                     else
                         epi.store8(m, n, v);
                 } else {
@@ -1389,24 +1461,14 @@ template <int DT, typename CFG, typename Epi>
 int launch_tiled(hipStream_t s, const void *A, const void *B, int M, int N, int K, long lda, long ldb, const Epi &epi) {
     typedef typename GemmTraits<DT>::elem T;
     int tiles_m = (M + CFG::BM - 1) / CFG::BM, tiles_n = (N + CFG::BN - 1) / CFG::BN;
-    size_t lds  = CFG::lds_bytes;
-    if (std::is_same<Epi, Int8Epilogue>::value) {  // room for the 256-byte table behind the staging area
-        size_t need = CFG::stage_bytes + 256;
-        lds         = lds > need ? lds : need;
-    }
-    if (Epi::kRowStats) {  // row statistics and the partial-sum buffer sit behind the staging area
-        size_t need = CFG::stage_bytes + (size_t)CFG::BM * 8 * (1 + 2 * CFG::WGK * CFG::WGN);
-        lds         = lds > need ? lds : need;
-    }
-    if (TakesRowSums<Epi>::value)
-        lds = CFG::lds_bytes + (size_t)CFG::BM * 8;  // {rstd, mean} per row, parked behind the slabs before the main loop
+    typedef EpiLds<CFG, Epi> L;
+    const size_t lds = L::total;
     if (EmitsRowSums<Epi>::value) {
-        // eight bytes per eight columns and row; not at the price of a workgroup per CU (the plain form runs instead)
-        const size_t with_sums = CFG::sums_offset + CFG::sums_bytes > lds ? CFG::sums_offset + CFG::sums_bytes : lds;
+        // the row sums are not taken at the price of a workgroup per CU (the plain form runs instead)
+        const size_t without = L::plain + L::side_bytes + 16;
         const long cu = 160 * 1024;
-        if (with_sums > (size_t)cu || cu / (long)(with_sums + 1024) < (cu / (long)(lds + 1024) > 4 ? 4 : cu / (long)(lds + 1024)))
+        if (lds > (size_t)cu || cu / (long)(lds + 1024) < (cu / (long)(without + 1024) > 4 ? 4 : cu / (long)(without + 1024)))
             return kTileTooLargeForSums;
-        lds = with_sums;
     }
     auto kern   = gemm_nk_tiled_kernel<DT, CFG, Epi>;
     if (lds > 64 * 1024) {
