@@ -1068,62 +1068,81 @@ __global__ void __launch_bounds__(CFG::NT)
         };
         constexpr int LPW = A_LD + B_LD;
         // A folding epilogue that is handed the row sums of A: the first BM threads request their row's sums (one
-        // 8-byte load per tile column of the kernel that wrote A) BEFORE the first slabs, add them up while those are
-        // on their way, and park {rstd, mean} behind everything else in LDS.  The loads are spelled as assembly like
-        // the slab loads, so that the wait can be placed by hand: they are older than every slab load, hence complete
-        // once at most the slab loads are outstanding.
+        // 8-byte load per tile column of the kernel that wrote A), add them up and park {rstd, mean} behind everything
+        // else in LDS, where the epilogue finds them.  The loads are spelled as assembly like the slab loads: the
+        // compiler knows nothing of the slabs in flight, so its own wait-count pass must not be what orders these
+        // loads among them, and the wait is placed by hand.  When:
+        //   late  (tile shapes that have a CU to themselves, hence registers to spare): once the last slab is in LDS.
+        //         Nothing stands between the kernel's entry and its first slabs, the loads' latency passes under the
+        //         last slab's MFMAs, and the sums are added up after the loop while the other waves are on their way
+        //         to the barrier that follows it.  They are the youngest loads of the kernel: wait for all.
+        //   early (shapes that share a CU: the registers the sums would occupy through the last slab would cost a
+        //         resident workgroup): before the first slabs, added up while those are on their way.  Older than
+        //         every slab load, they are complete once at most the slab loads are outstanding.
         typedef float f32x2 __attribute__((ext_vector_type(2)));
+        constexpr bool kLateSums = TakesRowSums<Epi>::value && EpiLds<CFG, Epi>::total > 80 * 1024;
         f32x2 early[TakesRowSums<Epi>::value ? kMaxRowSumBlocks : 1];
-        if constexpr (TakesRowSums<Epi>::value) {
-            if (tid < BM) {
-                const int m = m0 + tid < M ? m0 + tid : M - 1;
+        auto request_sums = [&]() __attribute__((always_inline)) {
+            if constexpr (TakesRowSums<Epi>::value) {
+                if (tid < BM) {
+                    const int m = m0 + tid < M ? m0 + tid : M - 1;
 #pragma unroll
-                for (int q = 0; q < kMaxRowSumBlocks; ++q) {
-                    early[q] = f32x2{0.f, 0.f};
-                    if (q < epi.ln.sum_blocks)
-                        asm volatile("global_load_dwordx2 %0, %1, %2"
-                                     : "=v"(early[q])
-                                     : "v"((uint32_t)(((size_t)q * M + m) * sizeof(float2))), "s"(epi.ln.row_sums)
-                                     : "memory");
+                    for (int q = 0; q < kMaxRowSumBlocks; ++q) {
+                        early[q] = f32x2{0.f, 0.f};
+                        if (q < epi.ln.sum_blocks)
+                            asm volatile("global_load_dwordx2 %0, %1, %2"
+                                         : "=v"(early[q])
+                                         : "v"((uint32_t)(((size_t)q * M + m) * sizeof(float2))), "s"(epi.ln.row_sums)
+                                         : "memory");
+                    }
                 }
             }
-        }
+        };
+        // slab_loads_behind: slab loads requested after the sums that may still be outstanding when the sums are read
+        auto finish_sums = [&](int slab_loads_behind) __attribute__((always_inline)) {
+            if constexpr (TakesRowSums<Epi>::value) {
+                if (tid < BM) {
+                    if (slab_loads_behind >= 2)
+                        TR_WAIT_VMCNT(2 * LPW);
+                    else if (slab_loads_behind == 1)
+                        TR_WAIT_VMCNT(LPW);
+                    else
+                        TR_WAIT_VMCNT(0);
+                    // The other waves wait at a barrier while these do this, so it is kept short: the block sums (fp32
+                    // already) are added in fp32 in a fixed order, only the variance is formed as a difference of
+                    // doubles, and its reciprocal root is taken in single precision with one Newton step.
+                    float f1 = 0.f, f2 = 0.f;
+#pragma unroll
+                    for (int q = 0; q < kMaxRowSumBlocks; ++q) {
+                        asm volatile("" : "+v"(early[q]));  // not to be read before the wait above
+                        if (q < epi.ln.sum_blocks) {
+                            f1 += early[q].x;
+                            f2 += early[q].y;
+                        }
+                    }
+                    const double mean = (double)f1 * (double)epi.ln.inv_cols;
+                    const float ve    = (float)((double)f2 * (double)epi.ln.inv_cols - mean * mean + (double)epi.ln.eps);
+                    float r           = __builtin_amdgcn_rsqf(ve);
+                    r                 = r * (1.5f - 0.5f * ve * r * r);
+                    reinterpret_cast<float2 *>(lds_dyn + CFG::lds_bytes)[tid] = make_float2(r, (float)mean);
+                }
+            }
+        };
+        if constexpr (TakesRowSums<Epi>::value && !kLateSums)
+            request_sums();
         int issued = 0;
 #pragma unroll
         for (int p = 0; p < NS - 1; ++p)
             if (p < nk)
                 issue(p, p), ++issued;
         TR_TL(5);  // first slabs requested
-        if constexpr (TakesRowSums<Epi>::value) {
-            if (tid < BM) {
-                if (issued >= 2)
-                    TR_WAIT_VMCNT(2 * LPW);
-                else if (issued == 1)
-                    TR_WAIT_VMCNT(LPW);
-                else
-                    TR_WAIT_VMCNT(0);
-                // Every other wave of the workgroup waits at the first barrier while these waves do this, so it is kept
-                // short: the block sums (fp32 already) are added in fp32 in a fixed order, only the variance is formed
-                // as a difference of doubles, and its reciprocal root is taken in single precision with one Newton step.
-                float f1 = 0.f, f2 = 0.f;
-#pragma unroll
-                for (int q = 0; q < kMaxRowSumBlocks; ++q) {
-                    asm volatile("" : "+v"(early[q]));  // not to be read before the wait above
-                    if (q < epi.ln.sum_blocks) {
-                        f1 += early[q].x;
-                        f2 += early[q].y;
-                    }
-                }
-                const double mean = (double)f1 * (double)epi.ln.inv_cols;
-                const float ve    = (float)((double)f2 * (double)epi.ln.inv_cols - mean * mean + (double)epi.ln.eps);
-                float r           = __builtin_amdgcn_rsqf(ve);
-                r                 = r * (1.5f - 0.5f * ve * r * r);
-                reinterpret_cast<float2 *>(lds_dyn + CFG::lds_bytes)[tid] = make_float2(r, (float)mean);
-            }
+        if constexpr (TakesRowSums<Epi>::value && !kLateSums) {
+            finish_sums(issued);
+            TR_TL(6);  // handed-over row sums added up
         }
-        TR_TL(6);  // handed-over row sums added up (folding epilogues that take them)
         int stage = 0, fill = NS - 1;  // stage of slab kt; stage that slab kt + NS - 1 goes to
-        for (int kt = 0; kt < nk; ++kt) {
+        // one slab; with_sums (the last slab in the late form) also requests the row sums
+        auto step = [&](int kt, auto with_sums) __attribute__((always_inline)) {
             // slab kt has landed once at most the loads of the slabs issued after it are outstanding
             if (NS == 3 && kt + 1 < nk)
                 TR_WAIT_VMCNT(LPW);
@@ -1138,9 +1157,22 @@ __global__ void __launch_bounds__(CFG::NT)
             asm volatile("" ::: "memory");  // no LDS access may be moved across the barrier by the compiler
             if (kt + NS - 1 < nk)
                 issue(kt + NS - 1, fill);
+            if constexpr (decltype(with_sums)::value)
+                request_sums();
             compute(stage);
             stage = stage + 1 == NS ? 0 : stage + 1;
             fill  = fill + 1 == NS ? 0 : fill + 1;
+        };
+        if constexpr (kLateSums) {
+            // the last slab apart, so that the requested sums cross no loop edge on their way to the wait
+            for (int kt = 0; kt + 1 < nk; ++kt)
+                step(kt, std::false_type());
+            step(nk - 1, std::true_type());
+            finish_sums(0);
+            TR_TL(6);  // handed-over row sums added up
+        } else {
+            for (int kt = 0; kt < nk; ++kt)
+                step(kt, std::false_type());
         }
     } else {
     u32x4 ra0[A_VECS], rb0[B_VECS], ra1[A_VECS], rb1[B_VECS];

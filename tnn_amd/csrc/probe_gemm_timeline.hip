@@ -102,8 +102,10 @@ int main(int argc, char **argv) {
             t0 = std::min(t0, tl[b * 8]);
             nb = b + 1;
         }
-    const int order[7] = {0, 5, 6, 1, 2, 3, 4};  // stamp slots in the order the kernel passes them
-    const char *nm[7]  = {"entry", "first slabs requested", "row sums added up", "first slab landed", "main loop done",
+    // stamp slots roughly in the order the kernel passes them (the row sums are added up before the first slab has
+    // landed in tile shapes that share a CU, after the main loop in those that have one to themselves)
+    const int order[7] = {0, 5, 1, 6, 2, 3, 4};
+    const char *nm[7]  = {"entry", "first slabs requested", "first slab landed", "row sums added up", "main loop done",
                           "C stored", "kernel end"};
     double sum[7] = {0}, mx[7] = {0}, mn[7] = {1e9, 1e9, 1e9, 1e9, 1e9, 1e9, 1e9};
     int cnt = 0;
