@@ -471,7 +471,6 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
     constexpr int LD     = 8 / NW;         // 1 KB wave-loads per wave, tile and operand
     __shared__ __attribute__((aligned(16))) unsigned char lds_all[3 * kStage];
     __shared__ __attribute__((aligned(16))) float lds_bias[3][kTileKV];
-    static_assert(BQ * kRowBytes <= 2 * kStage, "Q staging must fit stages 1 and 2");
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -561,13 +560,25 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
     constexpr int LPW = 2 * LD;
     if (!mb)
         for (int i = tid; i < 3 * kTileKV; i += NT)
-            (&lds_bias[0][0])[i] = 0.f;  // visible to everyone after the barriers of the Q staging below
+            (&lds_bias[0][0])[i] = 0.f;  // visible to everyone after the barrier that opens the first tile
     if (n_tiles > 0)
         issue(0, 0);
 
-    // ---- Q fragments through LDS (stages 1 and 2 are free until the second tile is requested)
+    // ---- Q fragments: lane (lq, g) holds elements 16 kk + 8 g .. + 7 of query row q0 + lq for the four k-steps.
+    // Four waves take them straight from memory (sixteen bytes per row and lane half is a poor shape for one load, but
+    // the four loads of a wave cover whole 128-byte rows between them: B32 S512 lengths U[16,512] 29.7 -> 29.2 us);
+    // two waves go through LDS with whole-row loads (stages 1 and 2 are free until the second tile is requested), where
+    // the direct form measured slower (B8 S384: 11.7 -> 12.3 us).
     u32x4 qf[4];
-    {
+    if constexpr (NW == 4) {
+        int qrow = q0 + lq;
+        qrow     = qrow < S ? qrow : S - 1;
+        const uint16_t *qp = qb + (size_t)qrow * p.q_ss + g * 8;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+            qf[kk] = *reinterpret_cast<const u32x4 *>(qp + kk * 16);
+    } else {
+        static_assert(BQ * kRowBytes <= 2 * kStage, "Q staging must fit stages 1 and 2");
         unsigned char *const stage = lds_all + kStage;
         constexpr int Q_VECS = BQ * 8 / NT;
 #pragma unroll
