@@ -241,6 +241,10 @@ TNN_ROCM_API int tnn_rocm_mask_to_kv_len_flagged(void *stream, const float *mask
                                                  float threshold);
 TNN_ROCM_API int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_t *kv_len, int B, int S,
                                          float threshold);
+/* The flagged form for a mask [B,S] of any float type, in one launch: a half-precision mask is also widened into
+ * mask_f32 [B,S] (the form the attention kernels read; may be NULL for an fp32 mask, which is used where it lies). */
+TNN_ROCM_API int tnn_rocm_mask_prepare(void *stream, int dtype, const void *mask, float *mask_f32, int32_t *kv_len,
+                                       int B, int S, float threshold);
 
 /* ---- row-wise ops ---------------------------------------------------------------------------
  * Softmax over `channel` of x viewed as [outer][channel][inner]

@@ -776,6 +776,38 @@ def test_qkv_split_and_attention_vt():
     assert rel_err(out, ref_o) <= FP16_TOL
 
 
+def test_mask_prepare_any_float_type():
+    """One launch turns an additive mask of any float type into the flagged key counts and, for a half-precision
+    mask, its fp32 copy: the same counts and flags as the fp32 kernel gives on the widened mask, row by row -- plain
+    padding rows (flagged), rows with a non-zero value on a visible key, holes, a row that masks everything (all keys
+    stay visible), a row that masks nothing."""
+    say("mask_prepare")
+    rng = np.random.default_rng(5)
+    B, S = 9, 200
+    m = np.zeros((B, S), np.float32)
+    m[0, 150:] = -10000.0                      # plain padding
+    m[1, 31:] = -10000.0
+    m[2, 100:] = -10000.0
+    m[2, 17] = -0.5                            # a visible key with a bias: not plain
+    m[3, 120:] = -10000.0
+    m[3, 40:60] = -10000.0                     # a hole: not plain
+    m[4, :] = -10000.0                         # everything masked: every key stays
+    m[5, 199:] = -10000.0
+    m[6, 1:] = -10000.0                        # a single key
+    m[7, :] = rng.standard_normal(S) * 0.1     # a bias everywhere, nothing masked
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        md = dev(m).to(dtype)
+        kv, f32 = ops().mask_prepare(md)
+        wide = md.float()
+        want = ops().mask_to_kv_len(wide, flagged=True)
+        assert torch.equal(kv, want), (dtype, host(kv), host(want))
+        assert torch.equal(f32, wide)
+        got = host(kv)
+        plain = (got & (1 << 30)) != 0
+        assert list(plain) == [True, True, False, False, False, True, True, False, True], (dtype, plain)
+        assert list(got & ~(1 << 30)) == [150, 31, 100, 120, 200, 199, 1, 200, 200]
+
+
 def test_store_through_switch_changes_no_result():
     """GEMM, attention and LayerNorm results leave the kernels through device-scope stores by default and through
     ordinary write-back stores with the switch off: the same bits either way, in every epilogue form."""

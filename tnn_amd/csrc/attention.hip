@@ -863,31 +863,36 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
     }
 }
 
-__global__ void mask_to_kv_len_kernel(const float *__restrict__ mask, int32_t *__restrict__ kv_len, int S,
-                                      float threshold, int flag_zero_rows) {
-    // one wave per batch row: the largest index whose mask value is above the threshold
+// One wave per batch row, one pass over it: the largest index whose mask value is above the threshold, and the
+// smallest index whose value is not exactly zero.  A mask in a half-precision type is widened on the way into mask_f32
+// (what the attention kernels read), so the additive mask of a forward pass costs one launch.
+template <int DT>
+__global__ void mask_to_kv_len_kernel(const typename Elem<DT>::type *__restrict__ mask, float *__restrict__ mask_f32,
+                                      int32_t *__restrict__ kv_len, int S, float threshold, int flag_zero_rows) {
     const int b    = blockIdx.x;
     const int lane = threadIdx.x;
-    int last       = -1;
-    for (int j = lane; j < S; j += 64)
-        if (mask[(size_t)b * S + j] > threshold)
+    int last = -1, first_nonzero = S;
+    for (int j = lane; j < S; j += 64) {
+        const float v = Elem<DT>::ld(&mask[(size_t)b * S + j]);
+        if (DT != TNN_ROCM_F32)
+            mask_f32[(size_t)b * S + j] = v;
+        if (v > threshold)
             last = j;
+        if (v != 0.0f && j < first_nonzero)
+            first_nonzero = j;
+    }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
-        int other = __shfl_xor(last, o, 64);
-        last      = other > last ? other : last;
+        const int other = __shfl_xor(last, o, 64), other_nz = __shfl_xor(first_nonzero, o, 64);
+        last            = other > last ? other : last;
+        first_nonzero   = other_nz < first_nonzero ? other_nz : first_nonzero;
     }
     // No key above the threshold: a padding-only sequence.  The reference still runs softmax(scores + mask) over all
     // S keys, and a constant shift cancels there, so every key stays visible (with its bias) instead of none.
     int len = last < 0 ? S : last + 1;
-    if (flag_zero_rows) {
-        // a plain padding mask is exactly 0 on every visible key: the attention kernel then needs the length only
-        int nonzero = 0;
-        for (int j = lane; j < len; j += 64)
-            nonzero |= mask[(size_t)b * S + j] != 0.0f ? 1 : 0;
-        if (!__any(nonzero))
-            len |= kKvLenMaskZero;
-    }
+    // a plain padding mask is exactly 0 on every visible key: the attention kernel then needs the length only
+    if (flag_zero_rows && first_nonzero >= len)
+        len |= kKvLenMaskZero;
     if (lane == 0)
         kv_len[b] = len;
 }
@@ -1038,17 +1043,40 @@ int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_t *kv_len, in
     if (B == 0)
         return 0;
     TR_REQUIRE(mask && kv_len, TNN_ROCM_EINVAL, "mask_to_kv_len: null pointer");
-    hipLaunchKernelGGL(mask_to_kv_len_kernel, dim3(B), dim3(64), 0, (hipStream_t)stream, mask, kv_len, S, threshold, 0);
+    hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_F32>, dim3(B), dim3(64), 0, (hipStream_t)stream, mask, nullptr, kv_len, S,
+                       threshold, 0);
     TR_CHECK_LAUNCH();
     return 0;
 }
 
 int tnn_rocm_mask_to_kv_len_flagged(void *stream, const float *mask, int32_t *kv_len, int B, int S, float threshold) {
-    TR_REQUIRE(B >= 0 && S >= 0 && S < kKvLenMaskZero, TNN_ROCM_ESHAPE, "mask_to_kv_len: bad size");
+    return tnn_rocm_mask_prepare(stream, TNN_ROCM_F32, mask, nullptr, kv_len, B, S, threshold);
+}
+
+int tnn_rocm_mask_prepare(void *stream, int dtype, const void *mask, float *mask_f32, int32_t *kv_len, int B, int S,
+                          float threshold) {
+    TR_REQUIRE(B >= 0 && S >= 0 && S < kKvLenMaskZero, TNN_ROCM_ESHAPE, "mask_prepare: bad size");
     if (B == 0)
         return 0;
-    TR_REQUIRE(mask && kv_len, TNN_ROCM_EINVAL, "mask_to_kv_len: null pointer");
-    hipLaunchKernelGGL(mask_to_kv_len_kernel, dim3(B), dim3(64), 0, (hipStream_t)stream, mask, kv_len, S, threshold, 1);
+    TR_REQUIRE(mask && kv_len, TNN_ROCM_EINVAL, "mask_prepare: null pointer");
+    TR_REQUIRE(dtype == TNN_ROCM_F32 || mask_f32, TNN_ROCM_EINVAL, "mask_prepare: a half-precision mask needs the fp32 buffer");
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case TNN_ROCM_F32:
+            hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_F32>, dim3(B), dim3(64), 0, s, (const float *)mask, nullptr,
+                               kv_len, S, threshold, 1);
+            break;
+        case TNN_ROCM_F16:
+            hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_F16>, dim3(B), dim3(64), 0, s, (const half_t *)mask, mask_f32,
+                               kv_len, S, threshold, 1);
+            break;
+        case TNN_ROCM_BF16:
+            hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_BF16>, dim3(B), dim3(64), 0, s, (const bf16_bits *)mask, mask_f32,
+                               kv_len, S, threshold, 1);
+            break;
+        default:
+            TR_REQUIRE(false, TNN_ROCM_EDTYPE, "mask_prepare: dtype %d unsupported", dtype);
+    }
     TR_CHECK_LAUNCH();
     return 0;
 }

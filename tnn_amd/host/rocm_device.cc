@@ -95,11 +95,10 @@ Status RocmContext::AttentionMask(const void *mask_blob, int mask_dtype, int B, 
         c.B = B, c.S = S, c.src = nullptr;
     const float *m = mask_dtype == TNN_ROCM_F32 ? (const float *)mask_blob : (const float *)c.mask_f32;
     if (c.src != mask_blob || c.epoch != forward_epoch_) {
-        if (mask_dtype != TNN_ROCM_F32)
-            ROCM_CALL(tnn_rocm_cast(stream_, mask_dtype, mask_blob, TNN_ROCM_F32, c.mask_f32, (size_t)B * S));
         // keys whose additive mask is <= -1000 after the last visible key contribute exp(-1000 - max) == 0 in fp32
-        // (a plain 0 / -10000 padding mask is flagged: the attention kernel then works from the lengths alone)
-        ROCM_CALL(tnn_rocm_mask_to_kv_len_flagged(stream_, m, (int32_t *)c.kv_len, B, S, -1000.0f));
+        // (a plain 0 / -10000 padding mask is flagged: the attention kernel then works from the lengths alone); one
+        // launch, which also widens a half-precision mask into the fp32 copy
+        ROCM_CALL(tnn_rocm_mask_prepare(stream_, mask_dtype, mask_blob, (float *)c.mask_f32, (int32_t *)c.kv_len, B, S, -1000.0f));
         c.src   = mask_blob;
         c.epoch = forward_epoch_;
     }

@@ -215,6 +215,17 @@ def mask_to_kv_len(mask, threshold=-1000.0, flagged=False):
     return out
 
 
+def mask_prepare(mask, threshold=-1000.0):
+    """flagged kv_len of a mask [B,S] of any float type and, for a half-precision mask, its fp32 copy: (kv_len, mask_f32)"""
+    _chk(mask)
+    B, S = mask.shape
+    out = torch.empty(B, dtype=torch.int32, device=mask.device)
+    f32 = mask if mask.dtype == torch.float32 else torch.empty(B, S, dtype=torch.float32, device=mask.device)
+    capi.call("tnn_rocm_mask_prepare", _stream(), dt(mask), _p(mask), None if mask.dtype == torch.float32 else _p(f32), _p(out),
+              B, S, float(threshold))
+    return out, f32
+
+
 def softmax(x, axis=-1):
     _chk(x)
     axis = axis % x.dim()
