@@ -108,7 +108,9 @@ template <typename E, typename = void> struct ColArrays : std::integral_constant
 template <typename E> struct ColArrays<E, typename std::enable_if<(E::kColArrays > 0)>::type> : std::integral_constant<int, E::kColArrays> {};
 template <typename E, typename = void> struct RowIn : std::false_type {};
 template <typename E> struct RowIn<E, typename std::enable_if<E::kRowIn>::type> : std::true_type {};
-constexpr int kMaxRowSumBlocks = TNN_ROCM_MAX_ROW_SUM_BLOCKS;  // tile columns of a producer a consumer can add up (768 columns of 32)
+constexpr int kMaxRowSumBlocks = TNN_ROCM_MAX_ROW_SUM_BLOCKS;
+template <typename E, typename = void> struct SumBlocks : std::integral_constant<int, 1> {};
+template <typename E> struct SumBlocks<E, typename std::enable_if<E::kTakesRowSums>::type> : std::integral_constant<int, E::kSumBlocks> {};  // tile columns of a producer a consumer can add up (768 columns of 32)
 
 
 template <int DT> struct FloatEpilogue {
@@ -280,10 +282,13 @@ template <int DT> __device__ __forceinline__ void ln_accumulate(const uint4 &fra
     }
 }
 
-template <int DT, bool SUMS = false> struct LnFloatEpilogue {
+// SUMS: 0 = the statistics come from the A fragments; else the most row-sum blocks the kernel is handed (12 or 24: that
+// many register pairs hold them while they are in flight)
+template <int DT, int SUMS = 0> struct LnFloatEpilogue {
     typedef typename Elem<DT>::type T;
     static constexpr bool kRowStats = true;
-    static constexpr bool kTakesRowSums = SUMS;
+    static constexpr bool kTakesRowSums = SUMS > 0;
+    static constexpr int kSumBlocks     = SUMS;
     int flags;
     const float *bias;  // b' (always present)
     const T *residual;
@@ -334,10 +339,11 @@ template <int DT, bool SUMS = false> struct LnFloatEpilogue {
 };
 
 // QKV projection of LayerNorm(t): QkvSplitEpilogue's layout with the folded-LayerNorm correction on the accumulators
-template <int DT, bool SUMS = false> struct LnQkvSplitEpilogue {
+template <int DT, int SUMS = 0> struct LnQkvSplitEpilogue {
     typedef typename Elem<DT>::type T;
     static constexpr bool kRowStats = true;
-    static constexpr bool kTakesRowSums = SUMS;
+    static constexpr bool kTakesRowSums = SUMS > 0;
+    static constexpr int kSumBlocks     = SUMS;
     const float *bias;
     T *qk;
     T *vt;
@@ -1072,22 +1078,24 @@ __global__ void __launch_bounds__(CFG::NT)
         // else in LDS, where the epilogue finds them.  The loads are spelled as assembly like the slab loads: the
         // compiler knows nothing of the slabs in flight, so its own wait-count pass must not be what orders these
         // loads among them, and the wait is placed by hand.  When:
-        //   late  (tile shapes that have a CU to themselves, hence registers to spare): once the last slab is in LDS.
+        //   late  (tile shapes that have a CU to themselves, hence registers to spare, and any shape when at most twelve
+        //         blocks are handed over: 24 registers): once the last slab is in LDS.
         //         Nothing stands between the kernel's entry and its first slabs, the loads' latency passes under the
         //         last slab's MFMAs, and the sums are added up after the loop while the other waves are on their way
         //         to the barrier that follows it.  They are the youngest loads of the kernel: wait for all.
-        //   early (shapes that share a CU: the registers the sums would occupy through the last slab would cost a
-        //         resident workgroup): before the first slabs, added up while those are on their way.  Older than
+        //   early (shapes that share a CU, with up to 24 blocks: the 48 registers the sums would occupy through the last
+        //         slab would cost a resident workgroup): before the first slabs, added up while those are on their way.  Older than
         //         every slab load, they are complete once at most the slab loads are outstanding.
         typedef float f32x2 __attribute__((ext_vector_type(2)));
-        constexpr bool kLateSums = TakesRowSums<Epi>::value && EpiLds<CFG, Epi>::total > 80 * 1024;
-        f32x2 early[TakesRowSums<Epi>::value ? kMaxRowSumBlocks : 1];
+        constexpr int NSUM      = SumBlocks<Epi>::value;
+        constexpr bool kLateSums = TakesRowSums<Epi>::value && (EpiLds<CFG, Epi>::total > 80 * 1024 || NSUM <= 12);
+        f32x2 early[NSUM];
         auto request_sums = [&]() __attribute__((always_inline)) {
             if constexpr (TakesRowSums<Epi>::value) {
                 if (tid < BM) {
                     const int m = m0 + tid < M ? m0 + tid : M - 1;
 #pragma unroll
-                    for (int q = 0; q < kMaxRowSumBlocks; ++q) {
+                    for (int q = 0; q < NSUM; ++q) {
                         early[q] = f32x2{0.f, 0.f};
                         if (q < epi.ln.sum_blocks)
                             asm volatile("global_load_dwordx2 %0, %1, %2"
@@ -1113,7 +1121,7 @@ __global__ void __launch_bounds__(CFG::NT)
                     // doubles, and its reciprocal root is taken in single precision with one Newton step.
                     float f1 = 0.f, f2 = 0.f;
 #pragma unroll
-                    for (int q = 0; q < kMaxRowSumBlocks; ++q) {
+                    for (int q = 0; q < NSUM; ++q) {
                         asm volatile("" : "+v"(early[q]));  // not to be read before the wait above
                         if (q < epi.ln.sum_blocks) {
                             f1 += early[q].x;
@@ -1964,15 +1972,19 @@ int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folde
         return launch_gemm_fast<DT, LnFloatEpilogue<DT, SUMS>>((hipStream_t)stream, t, w_folded, M, N, K, K, K, epi); \
     }
     if (dtype == TNN_ROCM_F16) {
-        if (row_sums)
-            TR_LN(TNN_ROCM_F16, true)
+        if (row_sums && row_sum_blocks <= 12)
+            TR_LN(TNN_ROCM_F16, 12)
+        else if (row_sums)
+            TR_LN(TNN_ROCM_F16, kMaxRowSumBlocks)
         else
-            TR_LN(TNN_ROCM_F16, false)
+            TR_LN(TNN_ROCM_F16, 0)
     } else {
-        if (row_sums)
-            TR_LN(TNN_ROCM_BF16, true)
+        if (row_sums && row_sum_blocks <= 12)
+            TR_LN(TNN_ROCM_BF16, 12)
+        else if (row_sums)
+            TR_LN(TNN_ROCM_BF16, kMaxRowSumBlocks)
         else
-            TR_LN(TNN_ROCM_BF16, false)
+            TR_LN(TNN_ROCM_BF16, 0)
     }
 #undef TR_LN
 }
@@ -2012,15 +2024,19 @@ int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const voi
                                                                   epi);                                              \
     }
     if (dtype == TNN_ROCM_F16) {
-        if (row_sums)
-            TR_QKVLN(TNN_ROCM_F16, true)
+        if (row_sums && row_sum_blocks <= 12)
+            TR_QKVLN(TNN_ROCM_F16, 12)
+        else if (row_sums)
+            TR_QKVLN(TNN_ROCM_F16, kMaxRowSumBlocks)
         else
-            TR_QKVLN(TNN_ROCM_F16, false)
+            TR_QKVLN(TNN_ROCM_F16, 0)
     } else {
-        if (row_sums)
-            TR_QKVLN(TNN_ROCM_BF16, true)
+        if (row_sums && row_sum_blocks <= 12)
+            TR_QKVLN(TNN_ROCM_BF16, 12)
+        else if (row_sums)
+            TR_QKVLN(TNN_ROCM_BF16, kMaxRowSumBlocks)
         else
-            TR_QKVLN(TNN_ROCM_BF16, false)
+            TR_QKVLN(TNN_ROCM_BF16, 0)
     }
 #undef TR_QKVLN
 }
