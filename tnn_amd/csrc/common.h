@@ -147,6 +147,14 @@ __device__ __forceinline__ float gelu_erf(float x) {
 // exp2, one max and the final multiply-add: 13 issue slots against 19 for the rational form 7.1.26 of Abramowitz &
 // Stegun used before and ~40 for erff.  Against the correctly rounded fp16 result 0.4 % of the values differ, by one
 // ulp (2.8 % for the rational form).  fp32 outputs keep gelu_erf.
+// max(x, 0) as the one instruction it is: written as fmaxf or as a median with +inf the compiler puts a quieting
+// v_max_f32 x, x in front of it
+__device__ __forceinline__ float max_with_zero(float x) {
+    float r;
+    asm("v_max_f32 %0, 0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
+
 __device__ __forceinline__ float gelu_erf_fast(float x) {
     // med3 instead of fmin / fmax: one instruction each, where the minimum / maximum forms first quiet their operand
     const float a = __builtin_amdgcn_fmed3f(fabsf(x), 0.f, 9.0f);
@@ -159,7 +167,7 @@ __device__ __forceinline__ float gelu_erf_fast(float x) {
     q             = fmaf(q, a, 1.0f);
     const float e = __builtin_amdgcn_exp2f(-q);  // Phi(-a)
     // the clamped a: a*Phi(-a) is below 1e-18 past 9, and +inf stays +inf
-    return fmaf(-a, e, __builtin_amdgcn_fmed3f(x, 0.f, __builtin_inff()));
+    return fmaf(-a, e, max_with_zero(x));
 }
 
 __device__ __forceinline__ float wave_sum(float v) {

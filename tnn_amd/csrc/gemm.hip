@@ -316,18 +316,29 @@ template <int DT, int SUMS = 0> struct LnFloatEpilogue {
             for (int t = 0; t < 8; ++t)
                 v[t] = gelu_erf_fast(v[t]);
         }
-        constexpr int NV = 8 * sizeof(T) / 16;
-        u32x4 packed[NV];
-        T *pe = reinterpret_cast<T *>(packed);
+        // the two forms each end in their own conversion and store: joined behind the branch, the form without a
+        // residual pays eight register copies per item for the join
         if (flags & TNN_ROCM_EPI_RESIDUAL) {
+            constexpr int NV = 8 * sizeof(T) / 16;
+            u32x4 packed[NV];
+            const T *pe      = reinterpret_cast<const T *>(packed);
             const u32x4 *rp = reinterpret_cast<const u32x4 *>(residual + (size_t)m * ldc + n);
 #pragma unroll
             for (int q = 0; q < NV; ++q)
                 packed[q] = rp[q];
+            float w[8];
 #pragma unroll
             for (int t = 0; t < 8; ++t)
-                v[t] += Elem<DT>::ld(&pe[t]);
+                w[t] = v[t] + Elem<DT>::ld(&pe[t]);
+            convert_and_store(m, n, w);
+        } else {
+            convert_and_store(m, n, v);
         }
+    }
+    __device__ __forceinline__ void convert_and_store(int m, int n, const float (&v)[8]) const {
+        constexpr int NV = 8 * sizeof(T) / 16;
+        u32x4 packed[NV];
+        T *pe = reinterpret_cast<T *>(packed);
 #pragma unroll
         for (int t = 0; t < 8; ++t)
             Elem<DT>::st(&pe[t], v[t]);
@@ -1281,6 +1292,7 @@ __global__ void __launch_bounds__(CFG::NT)
     AccT *const stage_all = reinterpret_cast<AccT *>(lds_dyn);
     AccT *const stage_me  = stage_all + wave * (32 * SSTR);  // wave = (wm*WGN + wn)*WGK + wk
     const bool by_rows = epi.direct(n0);
+    const int tid_piece = tid % CPR, tid_rowpos = tid / CPR;
     __syncthreads();  // every wave is done reading the slabs
     TR_TL(2);         // main loop done
     // LayerNorm-folding epilogues: reduce the lanes' partial row sums over the two k-halves of a fragment and the WGK
@@ -1381,9 +1393,21 @@ __global__ void __launch_bounds__(CFG::NT)
                 break;
             // consecutive threads walk along a row of C, or down the rows where the epilogue writes a transposed
             // layout (consecutive rows are then consecutive in memory)
-            const int c8  = by_rows ? ((item >> 5) % CPR) * 8 : (item % CPR) * 8;
-            const int row = by_rows ? (item & 31) : (item / CPR) % 32;
-            const int pos = item / (CPR * 32);  // = pm * WGN + pn
+            // item % CPR and item / CPR: where CPR is not a power of two (96-column wave tiles) the thread index is
+            // split once and every item adds its constant share, instead of a multiply-high sequence per item
+            int piece, rowpos;
+            if constexpr ((CPR & (CPR - 1)) != 0) {
+                const int c     = tid_piece + (it * NT) % CPR;
+                const int carry = c >= CPR ? 1 : 0;
+                piece           = c - carry * CPR;
+                rowpos          = tid_rowpos + (it * NT) / CPR + carry;
+            } else {
+                piece  = item % CPR;
+                rowpos = item / CPR;
+            }
+            const int c8  = by_rows ? ((item >> 5) % CPR) * 8 : piece * 8;
+            const int row = by_rows ? (item & 31) : rowpos % 32;
+            const int pos = rowpos / 32;  // = item / (CPR * 32) = pm * WGN + pn
             const AccT *src = stage_all + (pos * WGK) * (32 * SSTR) + row * SSTR + c8;
             acc4 lo = *reinterpret_cast<const acc4 *>(src);
             acc4 hi = *reinterpret_cast<const acc4 *>(src + 4);
