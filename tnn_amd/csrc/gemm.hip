@@ -282,6 +282,13 @@ template <int DT> __device__ __forceinline__ void ln_accumulate(const uint4 &fra
     }
 }
 
+// Element offset of (row m, column n) in a row-major matrix of leading dimension ld, for the epilogues whose entry
+// points have checked rows < 2^24, ld < 2^24 and rows * ld < 2^31: one full-rate 24-bit multiply where the 64-bit
+// product m * ld costs two v_mul_lo_u32 and a v_mad_u64_u32 (quarter rate each) per item.
+__device__ __forceinline__ unsigned elem_offset24(int m, unsigned ld, int n) {
+    return __umul24((unsigned)m, ld) + (unsigned)n;
+}
+
 // SUMS: 0 = the statistics come from the A fragments; else the most row-sum blocks the kernel is handed (12 or 24: that
 // many register pairs hold them while they are in flight)
 template <int DT, int SUMS = 0> struct LnFloatEpilogue {
@@ -322,7 +329,7 @@ template <int DT, int SUMS = 0> struct LnFloatEpilogue {
             constexpr int NV = 8 * sizeof(T) / 16;
             u32x4 packed[NV];
             const T *pe      = reinterpret_cast<const T *>(packed);
-            const u32x4 *rp = reinterpret_cast<const u32x4 *>(residual + (size_t)m * ldc + n);
+            const u32x4 *rp = reinterpret_cast<const u32x4 *>(residual + elem_offset24(m, (unsigned)ldc, n));
 #pragma unroll
             for (int q = 0; q < NV; ++q)
                 packed[q] = rp[q];
@@ -342,7 +349,7 @@ template <int DT, int SUMS = 0> struct LnFloatEpilogue {
 #pragma unroll
         for (int t = 0; t < 8; ++t)
             Elem<DT>::st(&pe[t], v[t]);
-        u32x4 *cp = reinterpret_cast<u32x4 *>(C + (size_t)m * ldc + n);
+        u32x4 *cp = reinterpret_cast<u32x4 *>(C + elem_offset24(m, (unsigned)ldc, n));
 #pragma unroll
         for (int q = 0; q < NV; ++q)
             store_out16(&cp[q], packed[q]);
@@ -382,16 +389,17 @@ template <int DT, int SUMS = 0> struct LnQkvSplitEpilogue {
 #pragma unroll
             for (int t = 0; t < 8; ++t)
                 Elem<DT>::st(&pe[t], v[t]);
-            u32x4 *cp = reinterpret_cast<u32x4 *>(qk + (size_t)m * 2 * H + n);
+            u32x4 *cp = reinterpret_cast<u32x4 *>(qk + elem_offset24(m, 2u * (unsigned)H, n));
 #pragma unroll
             for (int q = 0; q < NV; ++q)
                 store_out16(&cp[q], packed[q]);
         } else {
+            // B * S * 3H < 2^31 is checked at launch: 32-bit offsets throughout
             int c = n - 2 * H, bb = m / S, s_ = m - bb * S;
-            T *dst = vt + (((size_t)bb * heads + (c >> 6)) * 64 + (c & 63)) * S + s_;
+            T *dst = vt + (unsigned)(((bb * heads + (c >> 6)) * 64 + (c & 63)) * S + s_);
 #pragma unroll
             for (int t = 0; t < 8; ++t)
-                Elem<DT>::st_out(dst + (size_t)t * S, v[t]);
+                Elem<DT>::st_out(dst + (unsigned)(t * S), v[t]);
         }
     }
 };
@@ -435,7 +443,8 @@ template <int DT, bool SUMS = false> struct LnResidualEpilogue {
     // cl = the item's eight columns of the three arrays in LDS, cs apart; s = {rstd, mean} of row m
     __device__ __forceinline__ float2 store8(int m, int n, const float (&acc)[8], const float *cl, int cs, float2 s) const {
         static_assert(sizeof(T) == 2, "half-precision blobs only");
-        u32x4 packed = *reinterpret_cast<const u32x4 *>(t + (size_t)m * ldc + n);
+        const unsigned off = elem_offset24(m, (unsigned)ldc, n);
+        u32x4 packed = *reinterpret_cast<const u32x4 *>(t + off);
         float v[8];
         {
             float4 b0 = *reinterpret_cast<const float4 *>(cl), b1 = *reinterpret_cast<const float4 *>(cl + 4);
@@ -459,7 +468,7 @@ template <int DT, bool SUMS = false> struct LnResidualEpilogue {
 #pragma unroll
         for (int q = 0; q < 8; ++q)
             Elem<DT>::st(&pe[q], v[q]);
-        store_out16(C + (size_t)m * ldc + n, packed);
+        store_out16(C + off, packed);
         float2 sums = make_float2(0.f, 0.f);
         if constexpr (SUMS) {  // of the values as stored (rounded to the blob type): what the next GEMM reads
             ln_accumulate<DT>(__builtin_bit_cast(uint4, packed), sums.x, sums.y);
@@ -1975,7 +1984,8 @@ int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folde
     TR_REQUIRE(dtype == TNN_ROCM_F16 || dtype == TNN_ROCM_BF16, TNN_ROCM_EDTYPE, "gemm_ln: F16 or BF16 only");
     TR_REQUIRE(K > 0 && K % 128 == 0 && N % 8 == 0, TNN_ROCM_ESHAPE,
                "gemm_ln: K=%d must be a positive multiple of 128 and N=%d a multiple of 8", K, N);
-    TR_REQUIRE((long)M < (1l << 24) && (long)M * K < (1l << 31) && (long)N * K < (1l << 31) && (long)M * N < (1l << 31),
+    TR_REQUIRE((long)M < (1l << 24) && (long)N < (1l << 24) && (long)M * K < (1l << 31) && (long)N * K < (1l << 31) &&
+                   (long)M * N < (1l << 31),
                TNN_ROCM_ESHAPE, "gemm_ln: problem too large for 32-bit panel offsets");
     TR_REQUIRE(!(flags & TNN_ROCM_EPI_RESIDUAL) || residual, TNN_ROCM_EINVAL, "gemm_ln: residual flag without a residual");
     TR_REQUIRE(!row_sums || (row_sum_blocks >= 1 && row_sum_blocks <= kMaxRowSumBlocks && (((uintptr_t)row_sums) & 7u) == 0),
@@ -2025,8 +2035,8 @@ int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const voi
     TR_REQUIRE(dtype == TNN_ROCM_F16 || dtype == TNN_ROCM_BF16, TNN_ROCM_EDTYPE, "gemm_qkv_split_ln: F16 or BF16 only");
     TR_REQUIRE(K > 0 && K % 128 == 0 && S % 8 == 0, TNN_ROCM_ESHAPE,
                "gemm_qkv_split_ln: K=%d must be a positive multiple of 128 and S=%d a multiple of 8", K, S);
-    TR_REQUIRE((long)B * S < (1l << 24) && (long)B * S * 3 * heads * 64 < (1l << 31), TNN_ROCM_ESHAPE,
-               "gemm_qkv_split_ln: problem too large for 32-bit panel offsets");
+    TR_REQUIRE((long)B * S < (1l << 24) && (long)heads * 192 < (1l << 24) && (long)B * S * 3 * heads * 64 < (1l << 31),
+               TNN_ROCM_ESHAPE, "gemm_qkv_split_ln: problem too large for 32-bit panel offsets");
     TR_REQUIRE(al16(t) && al16(wqkv_folded) && al16(qk) && al16(vt) && al16(bqkv_folded) && al16(colsum) &&
                    (!y || (al16(y) && al16(gamma) && al16(beta))) && (((uintptr_t)row_stats) & 7u) == 0,
                TNN_ROCM_EALIGN, "gemm_qkv_split_ln: pointers must be 16-byte aligned (row_stats: 8-byte)");
@@ -2078,7 +2088,8 @@ int tnn_rocm_gemm_residual_ln(void *stream, int dtype, const void *x, const void
     TR_REQUIRE(dtype == TNN_ROCM_F16 || dtype == TNN_ROCM_BF16, TNN_ROCM_EDTYPE, "gemm_residual_ln: F16 or BF16 only");
     TR_REQUIRE(K > 0 && K % 64 == 0 && N % 8 == 0, TNN_ROCM_ESHAPE,
                "gemm_residual_ln: K=%d must be a positive multiple of 64 and N=%d a multiple of 8", K, N);
-    TR_REQUIRE((long)M < (1l << 24) && (long)M * K < (1l << 31) && (long)N * K < (1l << 31) && (long)M * N < (1l << 31),
+    TR_REQUIRE((long)M < (1l << 24) && (long)N < (1l << 24) && (long)M * K < (1l << 31) && (long)N * K < (1l << 31) &&
+                   (long)M * N < (1l << 31),
                TNN_ROCM_ESHAPE, "gemm_residual_ln: problem too large for 32-bit panel offsets");
     TR_REQUIRE(al16(x) && al16(w) && al16(C) && al16(t) && al16(gamma) && al16(beta) && (!bias || al16(bias)) &&
                    (((uintptr_t)row_stats) & 7u) == 0,
