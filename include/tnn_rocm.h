@@ -201,7 +201,9 @@ TNN_ROCM_API int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x,
  * sum and sum of squares per block of columns of t; the kernel then adds those up instead of taking the statistics
  * from the A tiles.  At most TNN_ROCM_MAX_ROW_SUM_BLOCKS blocks.
  * flags: TNN_ROCM_EPI_GELU, TNN_ROCM_EPI_RESIDUAL (residual [M,N] in dtype).  dtype F16 or BF16; K a multiple of 128
- * (the whole normalised row is one GEMM row), N a multiple of 8; all tensors dense row-major. */
+ * (the whole normalised row is one GEMM row), N a multiple of 8; all tensors dense row-major.
+ * Size limits of the three LayerNorm-folding entry points (TNN_ROCM_ESHAPE beyond them): rows and columns below 2^24,
+ * M*K, N*K and M*N below 2^31 elements (their kernels address with 32-bit offsets). */
 TNN_ROCM_API int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folded, const float *bias_folded,
                                   const float *colsum, const float *gamma, const float *beta, float eps, void *C, void *y,
                                   float *row_stats, const float *row_sums, int row_sum_blocks, int M, int N, int K,
