@@ -233,9 +233,11 @@ TNN_ROCM_API int tnn_rocm_gemm_residual_ln(void *stream, int dtype, const void *
                                            const float *beta, int M, int N, int K, int flags, float *row_sums,
                                            int *row_sum_blocks);
 
-/* kv_len[b] = 1 + the last key index whose additive mask value is > threshold; S if there is none (a padding-only
- * sequence: the reference's softmax(scores + mask) over all S keys is unchanged by the constant shift, so every key
- * stays in, with its bias). */
+/* kv_len[b] = 1 + the last key index whose additive mask value is > (the row's largest value + threshold), threshold
+ * being a large negative number (the host passes -1000): softmax(scores + mask) is unchanged by a constant added to a
+ * whole row, so the cut is taken relative to the row's best key -- a key that far below it contributes
+ * exp(threshold + score difference) = 0 in fp32.  A row that holds no value above the cut (only -inf / NaN) keeps all
+ * S keys, as the reference's softmax over all S keys does; so does a row that masks every key with the same value. */
 /* The _flagged form additionally sets bit 30 of kv_len[b] when mask[b][j] is exactly 0 for every j < kv_len[b] (a plain
  * padding mask): the attention kernels accept such entries and then do not read mask row b at all (the keys at and
  * beyond kv_len[b] are excluded by the length), which lets full key tiles take the path without a per-key bias. */
@@ -247,6 +249,12 @@ TNN_ROCM_API int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_
  * mask_f32 [B,S] (the form the attention kernels read; may be NULL for an fp32 mask, which is used where it lies). */
 TNN_ROCM_API int tnn_rocm_mask_prepare(void *stream, int dtype, const void *mask, float *mask_f32, int32_t *kv_len,
                                        int B, int S, float threshold);
+/* The same for a mask whose row b starts mask_batch_stride elements after row b-1; 0 = one row [S] that serves every
+ * sequence (an additive mask of shape [1,1,1,S], broadcast over the batch as the reference's Add does,
+ * source/tnn/layer/multidir_broadcast_layer.cc:59-111).  mask_f32, when given, receives the dense fp32 [B,S] copy
+ * whatever the source type; it is required unless the source is dense fp32. */
+TNN_ROCM_API int tnn_rocm_mask_prepare_strided(void *stream, int dtype, const void *mask, long mask_batch_stride,
+                                               float *mask_f32, int32_t *kv_len, int B, int S, float threshold);
 
 /* ---- row-wise ops ---------------------------------------------------------------------------
  * Softmax over `channel` of x viewed as [outer][channel][inner]

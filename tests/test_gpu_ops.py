@@ -963,6 +963,38 @@ def test_mask_to_kv_len():
     assert rel_err(host(a2), host(a1)) <= 1e-3
 
 
+def test_mask_cut_is_relative_to_the_row_maximum():
+    """The key count cuts trailing keys whose additive value lies far below the row's best key, not below a fixed
+    number: a row whose visible keys carry -999 and -1001 keeps both groups (their weights differ by exp(-2), not by
+    exp(-1000)), a row shifted by -5000 as a whole is cut where its padding starts, and one mask row can serve every
+    sequence.  The attention result with those counts equals the checker's softmax(scores + mask)."""
+    say("mask cut relative to the row maximum")
+    B, S, h = 4, 128, 2
+    H = h * 64
+    m = np.zeros((B, S), np.float32)
+    m[0, :50], m[0, 50:100], m[0, 100:] = -999.0, -1001.0, -20000.0
+    m[1, :70], m[1, 70:] = -5000.0, -15000.0            # a constant on the whole row: cut at 70, not "nothing visible"
+    m[2, :30], m[2, 30:] = 4000.0, 0.0                  # the zeros are the masked ones here
+    m[3, 90:] = -10000.0
+    kv = host(ops().mask_to_kv_len(dev(m), flagged=True))
+    assert [int(v) & ~(1 << 30) for v in kv] == [100, 70, 30, 90]
+    assert [bool(int(v) >> 30 & 1) for v in kv] == [False, False, False, True]
+    rng = np.random.default_rng(8)
+    q, k, v = (rng.standard_normal((B, h, S, 64)).astype(np.float16).astype(np.float32) for _ in range(3))
+    ref = orc.attention_core(q, k, v, 0.125, m).transpose(0, 2, 1, 3).reshape(B * S, H)
+    qt, kt, vt_ = (torch.from_numpy(t).half() for t in (q, k, v))
+    qk = torch.cat([qt.permute(0, 2, 1, 3).reshape(B * S, H), kt.permute(0, 2, 1, 3).reshape(B * S, H)], 1).contiguous()
+    vt = vt_.permute(0, 1, 3, 2).contiguous()
+    out = host(ops().attention_qk_vt(qk.cuda(), vt.cuda(), B, S, h, 0.125, mask=dev(m), kv_len=dev(kv.astype(np.int32))))
+    assert rel_err(out, ref) <= FP16_TOL
+    # one row for all sequences, any float type: dense fp32 copy + the same count for every sequence
+    for dtype in (torch.float32, torch.float16):
+        row = dev(m[3]).to(dtype)
+        kv1, f32 = ops().mask_prepare_broadcast(row, 5)
+        assert host(kv1).tolist() == [90 | (1 << 30)] * 5
+        assert torch.equal(f32, row.float()[None, :].expand(5, S))
+
+
 def test_attention_rejects_bad_args():
     from tnn_amd import capi
     q = torch.zeros(1, 1, 8, 32, dtype=torch.float16, device="cuda")

@@ -194,3 +194,56 @@ def test_quantized_add_graph_gets_reformat_layers_and_int8_blobs():
     add = [l for l in plan if l["type"] == "QuantizedAdd"][0]
     assert add["inputs"] == ["a_int8_reformat", "b_int8_reformat"]
     assert add["output_dims"] == [[1, 256, 256, 1]]
+
+
+# ---- the attention rewrite: spellings it must accept, graphs it must leave alone ----------------------------------
+def _attention_block(B=2, S=32, H=256, heads=4, **spelling):
+    cfg = EncoderConfig(1, H, heads, 2 * H)
+    lw = make_weights(cfg, seed=3, bias_std=0.02)["layers"][0]
+    return tnnmodel.attention_block_graph(lw, B, S, H, heads, **spelling)
+
+
+ACCEPTED_SPELLINGS = {
+    "mul_scale": dict(),
+    "div_scale": dict(scale="div"),
+    "scale_on_q": dict(scale="q"),
+    "scale_on_q_and_k": dict(scale="qk"),
+    "no_scale": dict(scale="none"),
+    "mask_operand_first": dict(mask_first=True),
+    "mask_first_div": dict(mask_first=True, scale="div"),
+    "no_mask": dict(mask=None),
+    "one_mask_row_for_all": dict(mask="111s"),
+    "inner_product_projections": dict(proj="inner_product"),
+    "rank3_single_sequence": dict(B=1, rank3=True, mask="11s"),
+    "rank3_inner_product_no_mask": dict(B=1, rank3=True, mask=None, proj="inner_product"),
+    "negative_softmax_axis": dict(softmax_axis=-1),
+}
+REFUSED_SPELLINGS = {
+    "softmax_over_queries": dict(softmax_axis=2),
+    "softmax_over_heads": dict(softmax_axis=1),
+    "mask_per_query_and_key": dict(mask="b1ss"),
+    "rank3_mask_per_query": dict(B=1, rank3=True, mask="1ss"),
+    "scores_read_twice": dict(tap_scores=True),
+    "head_dim_32": dict(heads=8),
+}
+
+
+@pytest.mark.parametrize("name", sorted(ACCEPTED_SPELLINGS))
+def test_attention_spelling_is_fused(name):
+    plan = host.plan(_attention_block(**ACCEPTED_SPELLINGS[name]), precision="fp16")
+    t = _types(plan)
+    assert t == {"RocmFusedAttention": 1, "RocmFusedLinear": 1}, (name, t)
+    att = [l for l in plan if l["type"] == "RocmFusedAttention"][0]
+    assert att["inputs"] == (["hidden"] if ACCEPTED_SPELLINGS[name].get("mask", "b11s") is None
+                             else ["hidden", "attention_bias"])
+
+
+@pytest.mark.parametrize("name", sorted(REFUSED_SPELLINGS))
+def test_attention_lookalike_stays_decomposed(name):
+    """Graphs that look like the attention core but are not what the fused kernel computes: a softmax over another
+    axis, a mask with one value per (query, key), scores somebody else reads, a head size the kernel has no form
+    for.  The plan must succeed (Instance::Init would) and keep Softmax and both batched MatMuls as single ops."""
+    plan = host.plan(_attention_block(**REFUSED_SPELLINGS[name]), precision="fp16")
+    t = _types(plan)
+    assert "RocmFusedAttention" not in t and t["Softmax"] == 1 and t["MatMul"] == 2 and t["Permute"] == 4, (name, t)
+    assert t["RocmFusedLinear"] == 4

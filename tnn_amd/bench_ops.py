@@ -15,6 +15,8 @@ stream; the best of five replays counts.  All launches go through the C entry po
 passes raw device pointers); there is no other implementation behind them."""
 import argparse
 import json
+import os
+import sys
 
 import torch
 
@@ -186,11 +188,23 @@ def mall_probe(launches=20):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--mall-probe", action="store_true", help="projection GEMMs with resident / evicted operands")
+    ap.add_argument("--simd-probe", action="store_true",
+                    help="build (if missing) and run the stand-alone SIMD micro-benchmark csrc/probe_simd.hip")
+    ap.add_argument("--build-only", action="store_true", help="with --simd-probe: compile it, do not run it")
     ap.add_argument("--launches", type=int, default=20)
     ap.add_argument("--only", default="")
     ap.add_argument("--sizes", default="encoder,stream")
     ap.add_argument("--json", action="store_true")
     a = ap.parse_args()
+    if a.simd_probe:
+        import subprocess
+        from tnn_amd import build
+        exe = os.path.join(build.LIB_DIR, "probe_simd")
+        if a.build_only or not os.path.exists(exe):
+            build.build_simd_probe()
+        if not a.build_only:
+            sys.exit(subprocess.call([exe]))
+        return
     if a.mall_probe:
         for r in mall_probe(a.launches):
             print(json.dumps(r) if a.json else "%-28s operands %6.1f MiB   resident %7.2f us   evicted %7.2f us" % (

@@ -54,17 +54,6 @@ def build_kernels(verbose=True):
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         objs.append(obj)
-    # the two stand-alone probes (evidence for the figures quoted for attention and the GEMMs; not part of the library)
-    # are compiled alongside: probe_simd (MFMA / vector ALU / LDS sharing one SIMD) and probe_gemm_timeline (the tiled
-    # GEMM with in-kernel time stamps)
-    probe_flags = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-Wno-unused-result", "-Xclang",
-                   "-target-feature", "-Xclang", "-packed-fp32-ops", "-I", os.path.join(ROOT, "include"), "-I", CSRC]
-    probes = []
-    for srcs, exe in ((["probe_simd.hip"], "probe_simd"), (["probe_gemm_timeline.hip", "runtime.hip"], "probe_gemm_timeline")):
-        cmd = ["hipcc"] + probe_flags + [os.path.join(CSRC, f) for f in srcs] + ["-o", os.path.join(LIB_DIR, exe)]
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        probes.append((exe, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
     failed = False
     for src, p in procs:
         out, _ = p.communicate()
@@ -90,12 +79,21 @@ def build_kernels(verbose=True):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
-    for exe, p in probes:
-        out, _ = p.communicate()
-        if p.returncode != 0:
-            print(out, file=sys.stderr)
-            raise RuntimeError("hipcc failed for " + exe)
     return LIB_PATH
+
+
+def build_simd_probe(verbose=True):
+    """Compile csrc/probe_simd.hip (a stand-alone micro-benchmark of one SIMD: matrix pipe, vector ALU and LDS reads
+    sharing its time) into tnn_amd/lib/probe_simd.  On demand only (`python -m tnn_amd.bench_ops --simd-probe`):
+    nothing in the library uses it and build_kernels() does not compile it."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    exe = os.path.join(LIB_DIR, "probe_simd")
+    cmd = ["hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-Wno-unused-result", "-Xclang",
+           "-target-feature", "-Xclang", "-packed-fp32-ops", "-I", CSRC, os.path.join(CSRC, "probe_simd.hip"), "-o", exe]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return exe
 
 
 if __name__ == "__main__":

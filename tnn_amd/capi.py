@@ -57,6 +57,7 @@ SIGNATURES = {
     "tnn_rocm_mask_to_kv_len": [_vp, _vp, _vp, _i, _i, _f],
     "tnn_rocm_mask_to_kv_len_flagged": [_vp, _vp, _vp, _i, _i, _f],
     "tnn_rocm_mask_prepare": [_vp, _i, _vp, _vp, _vp, _i, _i, _f],
+    "tnn_rocm_mask_prepare_strided": [_vp, _i, _vp, _l, _vp, _vp, _i, _i, _f],
     "tnn_rocm_softmax": [_vp, _i, _vp, _vp, _i, _i, _i],
     "tnn_rocm_layernorm": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp, _f],
     "tnn_rocm_embed_layernorm": [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _vp, _f, _vp, _i, _i, _vp],

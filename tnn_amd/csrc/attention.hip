@@ -45,11 +45,14 @@ template <> struct AttnT<TNN_ROCM_F16> {
     }
     // First product of an accumulation chain, d = a b + c0, with c0 read from registers of its own and left intact.
     // Written as an instruction because the compiler only emits the form whose destination is also the C operand and
-    // copies c0 into d first (16 moves per chain).  The early-clobber output keeps d apart from the inputs; the next
-    // MFMA of the chain accumulates into d (same opcode, C = destination of this one: no wait states needed).
+    // copies c0 into d first (16 moves per chain).  The early-clobber output keeps d apart from the inputs.  The compiler
+    // does not look inside the statement, so it inserts none of the wait states an instruction that reads d right
+    // after a matrix instruction needs (none for an accumulating MFMA of the same opcode into d, but up to 19 for a
+    // vector instruction or an MFMA with another destination): the statement carries them itself, so that whatever
+    // the compiler schedules next is safe.  They pass while the matrix pipe works on this product.
     template <typename V> static __device__ __forceinline__ f32x16 mma_from(const V &a, const V &b, const f32x16 &c0) {
         f32x16 d;
-        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c0));
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3\n\ts_nop 15\n\ts_nop 3" : "=&v"(d) : "v"(a), "v"(b), "v"(c0));
         return d;
     }
     static __device__ __forceinline__ float to_float(uint16_t bits) { return (float)__builtin_bit_cast(half_t, bits); }
@@ -85,7 +88,7 @@ template <> struct AttnT<TNN_ROCM_BF16> {
     }
     template <typename V> static __device__ __forceinline__ f32x16 mma_from(const V &a, const V &b, const f32x16 &c0) {
         f32x16 d;
-        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c0));
+        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3\n\ts_nop 15\n\ts_nop 3" : "=&v"(d) : "v"(a), "v"(b), "v"(c0));
         return d;
     }
     static __device__ __forceinline__ float to_float(uint16_t bits) { return __uint_as_float((uint32_t)bits << 16); }
@@ -520,10 +523,10 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
         v_off[i]    = ((uint32_t)r * vt_sd32 + (uint32_t)l_chunk[i] * 8u) * 2u;
     }
     auto load16 = [](const void *base, uint32_t byte_off, uint32_t lds_addr) {
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
     };
     auto load4 = [](const void *base, uint32_t byte_off, uint32_t lds_addr) {
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
     };
     const uint32_t wave_dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_base + (uint32_t)wave * 1024u));
     auto issue = [&](int t, int stage) {
@@ -863,20 +866,36 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
     }
 }
 
-// One wave per batch row, one pass over it: the largest index whose mask value is above the threshold, and the
-// smallest index whose value is not exactly zero.  A mask in a half-precision type is widened on the way into mask_f32
-// (what the attention kernels read), so the additive mask of a forward pass costs one launch.
+// One wave per batch row, two passes over it (the second finds the row in cache): the row's largest value, then the
+// largest index whose mask value is above (largest value + threshold) and the smallest index whose value is not
+// exactly zero.  The cut is relative to the row's maximum because softmax is: a key whose bias lies `threshold` (a
+// large negative number) below the best key's contributes exp(threshold + score difference) = 0 in fp32, whatever
+// constant the whole row carries.  Row b is read at mask + b * src_stride (0: one row serves every sequence); with
+// mask_f32 given, the row is also written there in fp32, densely (what the attention kernels read).
 template <int DT>
-__global__ void mask_to_kv_len_kernel(const typename Elem<DT>::type *__restrict__ mask, float *__restrict__ mask_f32,
-                                      int32_t *__restrict__ kv_len, int S, float threshold, int flag_zero_rows) {
+__global__ void mask_to_kv_len_kernel(const typename Elem<DT>::type *__restrict__ mask, long src_stride,
+                                      float *__restrict__ mask_f32, int32_t *__restrict__ kv_len, int S, float threshold,
+                                      int flag_zero_rows) {
     const int b    = blockIdx.x;
     const int lane = threadIdx.x;
+    const typename Elem<DT>::type *row = mask + (size_t)b * src_stride;
+    float top = -INFINITY;
+    for (int j = lane; j < S; j += 64) {
+        const float v = Elem<DT>::ld(&row[j]);
+        if (mask_f32)
+            mask_f32[(size_t)b * S + j] = v;
+        top = v > top ? v : top;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float other = __shfl_xor(top, o, 64);
+        top               = other > top ? other : top;
+    }
+    const float cut = top + threshold;
     int last = -1, first_nonzero = S;
     for (int j = lane; j < S; j += 64) {
-        const float v = Elem<DT>::ld(&mask[(size_t)b * S + j]);
-        if (DT != TNN_ROCM_F32)
-            mask_f32[(size_t)b * S + j] = v;
-        if (v > threshold)
+        const float v = Elem<DT>::ld(&row[j]);
+        if (v > cut)
             last = j;
         if (v != 0.0f && j < first_nonzero)
             first_nonzero = j;
@@ -887,8 +906,9 @@ __global__ void mask_to_kv_len_kernel(const typename Elem<DT>::type *__restrict_
         last            = other > last ? other : last;
         first_nonzero   = other_nz < first_nonzero ? other_nz : first_nonzero;
     }
-    // No key above the threshold: a padding-only sequence.  The reference still runs softmax(scores + mask) over all
-    // S keys, and a constant shift cancels there, so every key stays visible (with its bias) instead of none.
+    // No key above the cut (a row of -inf or NaN only): the reference still runs softmax(scores + mask) over all S
+    // keys, so every key stays in, with its bias.  A row that masks every key with the same finite value keeps all
+    // its keys by the rule itself: each one is the row's maximum.
     int len = last < 0 ? S : last + 1;
     // a plain padding mask is exactly 0 on every visible key: the attention kernel then needs the length only
     if (flag_zero_rows && first_nonzero >= len)
@@ -1043,8 +1063,8 @@ int tnn_rocm_mask_to_kv_len(void *stream, const float *mask, int32_t *kv_len, in
     if (B == 0)
         return 0;
     TR_REQUIRE(mask && kv_len, TNN_ROCM_EINVAL, "mask_to_kv_len: null pointer");
-    hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_F32>, dim3(B), dim3(64), 0, (hipStream_t)stream, mask, nullptr, kv_len, S,
-                       threshold, 0);
+    hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_F32>, dim3(B), dim3(64), 0, (hipStream_t)stream, mask, (long)S, nullptr,
+                       kv_len, S, threshold, 0);
     TR_CHECK_LAUNCH();
     return 0;
 }
@@ -1053,32 +1073,42 @@ int tnn_rocm_mask_to_kv_len_flagged(void *stream, const float *mask, int32_t *kv
     return tnn_rocm_mask_prepare(stream, TNN_ROCM_F32, mask, nullptr, kv_len, B, S, threshold);
 }
 
-int tnn_rocm_mask_prepare(void *stream, int dtype, const void *mask, float *mask_f32, int32_t *kv_len, int B, int S,
-                          float threshold) {
+int tnn_rocm_mask_prepare_strided(void *stream, int dtype, const void *mask, long mask_batch_stride, float *mask_f32,
+                                  int32_t *kv_len, int B, int S, float threshold) {
     TR_REQUIRE(B >= 0 && S >= 0 && S < kKvLenMaskZero, TNN_ROCM_ESHAPE, "mask_prepare: bad size");
+    TR_REQUIRE(mask_batch_stride == 0 || mask_batch_stride >= S, TNN_ROCM_ESHAPE, "mask_prepare: batch stride %ld below S",
+               mask_batch_stride);
     if (B == 0)
         return 0;
     TR_REQUIRE(mask && kv_len, TNN_ROCM_EINVAL, "mask_prepare: null pointer");
-    TR_REQUIRE(dtype == TNN_ROCM_F32 || mask_f32, TNN_ROCM_EINVAL, "mask_prepare: a half-precision mask needs the fp32 buffer");
+    TR_REQUIRE((dtype == TNN_ROCM_F32 && mask_batch_stride == S) || mask_f32, TNN_ROCM_EINVAL,
+               "mask_prepare: a half-precision or strided mask needs the fp32 buffer");
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
         case TNN_ROCM_F32:
-            hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_F32>, dim3(B), dim3(64), 0, s, (const float *)mask, nullptr,
-                               kv_len, S, threshold, 1);
+            hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_F32>, dim3(B), dim3(64), 0, s, (const float *)mask,
+                               mask_batch_stride, mask_f32, kv_len, S, threshold, 1);
             break;
         case TNN_ROCM_F16:
-            hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_F16>, dim3(B), dim3(64), 0, s, (const half_t *)mask, mask_f32,
-                               kv_len, S, threshold, 1);
+            hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_F16>, dim3(B), dim3(64), 0, s, (const half_t *)mask,
+                               mask_batch_stride, mask_f32, kv_len, S, threshold, 1);
             break;
         case TNN_ROCM_BF16:
-            hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_BF16>, dim3(B), dim3(64), 0, s, (const bf16_bits *)mask, mask_f32,
-                               kv_len, S, threshold, 1);
+            hipLaunchKernelGGL(mask_to_kv_len_kernel<TNN_ROCM_BF16>, dim3(B), dim3(64), 0, s, (const bf16_bits *)mask,
+                               mask_batch_stride, mask_f32, kv_len, S, threshold, 1);
             break;
         default:
             TR_REQUIRE(false, TNN_ROCM_EDTYPE, "mask_prepare: dtype %d unsupported", dtype);
     }
     TR_CHECK_LAUNCH();
     return 0;
+}
+
+int tnn_rocm_mask_prepare(void *stream, int dtype, const void *mask, float *mask_f32, int32_t *kv_len, int B, int S,
+                          float threshold) {
+    // an fp32 mask is used where it lies: no copy
+    return tnn_rocm_mask_prepare_strided(stream, dtype, mask, (long)S, dtype == TNN_ROCM_F32 ? nullptr : mask_f32, kv_len, B, S,
+                                         threshold);
 }
 
 }  // extern "C"

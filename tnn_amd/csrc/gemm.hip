@@ -27,16 +27,10 @@
 
 using namespace tnn_rocm;
 
-// Optional in-kernel timeline (stand-alone probe builds only, see probe_gemm_timeline.hip): thread 0 of every workgroup
-// of the tiled kernel stamps the constant-rate counter (100 MHz) at five points.
-#ifdef TNN_ROCM_TIMELINE
-__device__ unsigned long long g_gemm_timeline[4096 * 8];
-#define TR_TL(i)                                                                                                      \
-    do {                                                                                                              \
-        if (threadIdx.x == 0 && blockIdx.x < 4096)                                                                    \
-            g_gemm_timeline[(size_t)blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime();                         \
-    } while (0)
-#else
+// Hook for scratch builds that include this file to time the tiled kernel from inside: TR_TL(i) marks point i of a
+// workgroup's life (0 entry, 5 first slabs requested, 6 row sums added up, 1 first slab landed, 2 main loop done,
+// 3 C stored, 4 kernel end).  The library itself compiles it to nothing.
+#ifndef TR_TL
 #define TR_TL(i)
 #endif
 
@@ -1051,7 +1045,7 @@ __global__ void __launch_bounds__(CFG::NT)
             asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                          :
                          : "v"(byte_off), "s"(base), "s"(lds_addr)
-                         : "memory");
+                         : "memory", "m0");
         };
         auto issue = [&](int slab, int stage) {
             const uint32_t dst = wave_dst + (uint32_t)(stage * STAGE);
@@ -1095,9 +1089,10 @@ __global__ void __launch_bounds__(CFG::NT)
         constexpr int LPW = A_LD + B_LD;
         // A folding epilogue that is handed the row sums of A: the first BM threads request their row's sums (one
         // 8-byte load per tile column of the kernel that wrote A), add them up and park {rstd, mean} behind everything
-        // else in LDS, where the epilogue finds them.  The loads are spelled as assembly like the slab loads: the
-        // compiler knows nothing of the slabs in flight, so its own wait-count pass must not be what orders these
-        // loads among them, and the wait is placed by hand.  When:
+        // else in LDS, where the epilogue finds them.  In the early form the loads are spelled as assembly like the
+        // slab loads and the wait is placed by hand: the compiler knows nothing of the slabs in flight, and the wait it
+        // would place itself (everything outstanding) would also wait for the slabs requested after the sums.  In the
+        // late form they are ordinary loads.  When:
         //   late  (tile shapes that have a CU to themselves, hence registers to spare, and any shape when at most twelve
         //         blocks are handed over: 24 registers): once the last slab is in LDS.
         //         Nothing stands between the kernel's entry and its first slabs, the loads' latency passes under the
@@ -1117,11 +1112,19 @@ __global__ void __launch_bounds__(CFG::NT)
 #pragma unroll
                     for (int q = 0; q < NSUM; ++q) {
                         early[q] = f32x2{0.f, 0.f};
-                        if (q < epi.ln.sum_blocks)
-                            asm volatile("global_load_dwordx2 %0, %1, %2"
-                                         : "=v"(early[q])
-                                         : "v"((uint32_t)(((size_t)q * M + m) * sizeof(float2))), "s"(epi.ln.row_sums)
-                                         : "memory");
+                        if (q < epi.ln.sum_blocks) {
+                            if constexpr (kLateSums)
+                                // ordinary loads: they are the youngest of the kernel, so the wait the compiler puts in
+                                // front of their first use (everything outstanding) is the wait that is wanted, and
+                                // the compiler knows the registers are not valid before it
+                                early[q] = *reinterpret_cast<const f32x2 *>(
+                                    reinterpret_cast<const char *>(epi.ln.row_sums) + ((size_t)q * M + m) * sizeof(float2));
+                            else
+                                asm volatile("global_load_dwordx2 %0, %1, %2"
+                                             : "=v"(early[q])
+                                             : "v"((uint32_t)(((size_t)q * M + m) * sizeof(float2))), "s"(epi.ln.row_sums)
+                                             : "memory");
+                        }
                     }
                 }
             }
@@ -1130,26 +1133,32 @@ __global__ void __launch_bounds__(CFG::NT)
         auto finish_sums = [&](int slab_loads_behind) __attribute__((always_inline)) {
             if constexpr (TakesRowSums<Epi>::value) {
                 if (tid < BM) {
-                    if (slab_loads_behind >= 2)
-                        TR_WAIT_VMCNT(2 * LPW);
-                    else if (slab_loads_behind == 1)
-                        TR_WAIT_VMCNT(LPW);
-                    else
-                        TR_WAIT_VMCNT(0);
+                    if constexpr (!kLateSums) {
+                        if (slab_loads_behind >= 2)
+                            TR_WAIT_VMCNT(2 * LPW);
+                        else if (slab_loads_behind == 1)
+                            TR_WAIT_VMCNT(LPW);
+                        else
+                            TR_WAIT_VMCNT(0);
+                    }
                     // The other waves wait at a barrier while these do this, so it is kept short: the block sums (fp32
                     // already) are added in fp32 in a fixed order, only the variance is formed as a difference of
                     // doubles, and its reciprocal root is taken in single precision with one Newton step.
                     float f1 = 0.f, f2 = 0.f;
 #pragma unroll
                     for (int q = 0; q < NSUM; ++q) {
-                        asm volatile("" : "+v"(early[q]));  // not to be read before the wait above
+                        if constexpr (!kLateSums)
+                            asm volatile("" : "+v"(early[q]));  // not to be read before the wait above
                         if (q < epi.ln.sum_blocks) {
                             f1 += early[q].x;
                             f2 += early[q].y;
                         }
                     }
                     const double mean = (double)f1 * (double)epi.ln.inv_cols;
-                    const float ve    = (float)((double)f2 * (double)epi.ln.inv_cols - mean * mean + (double)epi.ln.eps);
+                    // fp32 block sums can leave E[x^2] - mean^2 a hair below zero for rows whose spread is tiny next to
+                    // their mean; the variance is clamped there (with eps = 1e-12 the root would otherwise be NaN)
+                    const double var  = (double)f2 * (double)epi.ln.inv_cols - mean * mean;
+                    const float ve    = (float)((var > 0.0 ? var : 0.0) + (double)epi.ln.eps);
                     float r           = __builtin_amdgcn_rsqf(ve);
                     r                 = r * (1.5f - 0.5f * ve * r * r);
                     reinterpret_cast<float2 *>(lds_dyn + CFG::lds_bytes)[tid] = make_float2(r, (float)mean);
@@ -1514,10 +1523,7 @@ __global__ void __launch_bounds__(CFG::NT)
             }
         }
     }
-#ifdef TNN_ROCM_TIMELINE
-    __syncthreads();
     TR_TL(4);  // kernel end
-#endif
 }
 
 // tuning override for experiments: 0 = heuristic, otherwise a configuration code of the tiled kernel

@@ -76,7 +76,7 @@ Status RocmContext::OnInstanceForwardBegin() {
     return TNN_OK;
 }
 
-Status RocmContext::AttentionMask(const void *mask_blob, int mask_dtype, int B, int S, const float **mask_f32,
+Status RocmContext::AttentionMask(const void *mask_blob, int mask_dtype, int B, int S, bool one_row, const float **mask_f32,
                                   const int32_t **kv_len) {
     auto &c = mask_cache_;
     if ((size_t)B * S > c.cap_mask || (size_t)B > c.cap_len || !c.kv_len) {
@@ -91,14 +91,17 @@ Status RocmContext::AttentionMask(const void *mask_blob, int mask_dtype, int B, 
         c.cap_mask = (size_t)B * S, c.cap_len = (size_t)B;
         c.src = nullptr;
     }
-    if (c.B != B || c.S != S)
-        c.B = B, c.S = S, c.src = nullptr;
-    const float *m = mask_dtype == TNN_ROCM_F32 ? (const float *)mask_blob : (const float *)c.mask_f32;
+    if (c.B != B || c.S != S || c.one_row != one_row)
+        c.B = B, c.S = S, c.one_row = one_row, c.src = nullptr;
+    // a dense fp32 mask is read where it lies; any other (half precision, or one row for all sequences) from the copy
+    const bool in_place = mask_dtype == TNN_ROCM_F32 && !one_row;
+    const float *m      = in_place ? (const float *)mask_blob : (const float *)c.mask_f32;
     if (c.src != mask_blob || c.epoch != forward_epoch_) {
-        // keys whose additive mask is <= -1000 after the last visible key contribute exp(-1000 - max) == 0 in fp32
-        // (a plain 0 / -10000 padding mask is flagged: the attention kernel then works from the lengths alone); one
-        // launch, which also widens a half-precision mask into the fp32 copy
-        ROCM_CALL(tnn_rocm_mask_prepare(stream_, mask_dtype, mask_blob, (float *)c.mask_f32, (int32_t *)c.kv_len, B, S, -1000.0f));
+        // Keys after the last one whose additive mask lies within 1000 of the row's largest value contribute
+        // exp(-1000 + score difference) == 0 in fp32 and are cut (a plain 0 / -10000 padding mask is flagged: the
+        // attention kernel then works from the lengths alone); one launch, which also makes the fp32 copy.
+        ROCM_CALL(tnn_rocm_mask_prepare_strided(stream_, mask_dtype, mask_blob, one_row ? 0L : (long)S,
+                                                in_place ? nullptr : (float *)c.mask_f32, (int32_t *)c.kv_len, B, S, -1000.0f));
         c.src   = mask_blob;
         c.epoch = forward_epoch_;
     }

@@ -73,7 +73,8 @@ public:
     int32_t *ErrorFlag() { return error_flag_; }
     // The padding mask is one blob shared by every attention layer of a forward pass: the first layer that asks
     // derives its fp32 copy and the per-sequence key counts, later layers of the same forward reuse them.
-    Status AttentionMask(const void *mask_blob, int mask_dtype, int B, int S, const float **mask_f32,
+    // one_row: the blob holds S values that serve every sequence (an additive mask [1,1,1,S])
+    Status AttentionMask(const void *mask_blob, int mask_dtype, int B, int S, bool one_row, const float **mask_f32,
                          const int32_t **kv_len);
 
 private:
@@ -89,6 +90,7 @@ private:
         const void *src = nullptr;
         uint64_t epoch  = 0;
         int B = 0, S = 0;
+        bool one_row = false;
         size_t cap_mask = 0, cap_len = 0;  // elements allocated (grow-only, so recorded launch sequences stay valid)
         void *mask_f32 = nullptr, *kv_len = nullptr;
     } mask_cache_;

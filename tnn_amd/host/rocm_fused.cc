@@ -15,6 +15,7 @@
 #include <cfloat>
 #include <cmath>
 #include <cstdlib>
+#include <functional>
 
 #include "rocm_device.h"
 
@@ -43,6 +44,260 @@ struct GraphIndex {
         auto it = producer.find(blob);
         return it == producer.end() ? -1 : it->second;
     }
+};
+
+// ---- the attention core, as both rewrites (float and quantised) recognise it --------------------------------------
+// Around a Softmax layer:
+//   scores = MatMul(q_heads, k_heads^T)            q/k/v_heads <- Permute <- Reshape(head split) <- projection of x
+//   [scores * s | scores / s]   (a one-value Mul / Div resource; the same scalar may instead sit on the q or the k^T
+//                                operand of the MatMul)
+//   [+ mask]                    (either operand order)
+//   Softmax over the last axis -> MatMul(probs, v_heads) -> Permute (head merge) -> Reshape
+// A chain is only reported when the fused kernel computes exactly what the chain does: every intermediate blob has
+// one reader and is no model output, the softmax runs over the keys (its axis parameter is read, not assumed), and the
+// additive mask is known -- from the model inputs, the constants and the shape rules of the layers that build it -- to
+// hold one value per key and sequence ([B,1,1,S], or [1,1,1,S] / [1,1,S] for every sequence).  Anything else (a
+// per-query mask [B,1,S,S], a mask of unknown shape, a softmax over another axis, scores with a second reader) stays
+// decomposed and runs through the single-op accs.
+struct AttentionCore {
+    std::vector<int> chain;         // every layer the fused layer replaces
+    std::string mask;               // additive mask blob, empty if there is none
+    float scale = 1.0f;             // product of the scalar factors on the scores
+    int lq = -1, lk = -1, lv = -1;  // the three projections (whatever the caller's head-split walk accepts as one)
+    int rs = -1;                    // the head-merging Reshape: its output is the fused layer's output
+    DimsVector split_shape;         // shape parameter of the head-splitting Reshape layers: [.., S, heads, head_dim]
+};
+
+class AttentionMatcher {
+public:
+    // walks `blob` <- Permute(order4 | order3) <- Reshape(head split) <- ... <- projection; returns the projection's
+    // layer index or -1, appends the walked layers to the chain and reports the Reshape's shape parameter
+    typedef std::function<int(const GraphIndex &, const std::string &, const std::vector<int> &, const std::vector<int> &,
+                              std::vector<int> *, DimsVector *)>
+        HeadSplitFn;
+
+    AttentionMatcher(NetStructure *s, NetResource *r, HeadSplitFn head_split)
+        : structure_(s), resource_(r), head_split_(std::move(head_split)) {}
+
+    bool Match(const GraphIndex &g, int si, AttentionCore *m) {
+        auto &L = structure_->layers;
+        auto sm = L[si];
+        if (!sm || sm->type != LAYER_SOFTMAX || sm->inputs.size() != 1 || sm->outputs.size() != 1)
+            return false;
+        auto sp = dynamic_cast<SoftmaxLayerParam *>(sm->param.get());
+        if (!sp)
+            return false;
+        m->chain = {si};
+        // ---- upstream of the softmax: [Add(mask)] <- [Mul|Div(scalar)] <- MatMul(q, k^T)
+        std::string cur = sm->inputs[0];
+        bool have_scale = false;
+        int qk = -1;
+        for (int step = 0; step < 3 && qk < 0; ++step) {
+            int pi = g.producer_of(cur);
+            if (pi < 0 || !L[pi] || g.sole_consumer(cur) < 0 || IsModelOutput(cur))
+                break;
+            auto pl = L[pi];
+            float v = 0.f;
+            if (pl->type == LAYER_ADD && pl->inputs.size() == 2 && m->mask.empty() && !have_scale && !pl->param->quantized &&
+                !Res<EltwiseLayerResource>(pl->name)) {
+                // scores + mask in either order: the operand that comes out of the score chain is the scores
+                bool first_is_scores = IsScoreChain(g, pl->inputs[0]), second_is_scores = IsScoreChain(g, pl->inputs[1]);
+                if (first_is_scores == second_is_scores)
+                    break;
+                m->mask = first_is_scores ? pl->inputs[1] : pl->inputs[0];
+                cur     = first_is_scores ? pl->inputs[0] : pl->inputs[1];
+                m->chain.push_back(pi);
+            } else if (!have_scale && ScalarFactor(pl, &v)) {
+                m->scale *= v;
+                have_scale = true;
+                cur        = pl->inputs[0];
+                m->chain.push_back(pi);
+            } else if (pl->type == LAYER_MATMUL && pl->inputs.size() == 2 && !Res<MatMulLayerResource>(pl->name)) {
+                qk = pi;
+                m->chain.push_back(pi);
+            } else {
+                break;
+            }
+        }
+        if (qk < 0)
+            return false;
+        // ---- q and k^T operands, each possibly behind a scalar factor of its own (q * s, k^T * sqrt(s) ...)
+        DimsVector shape_k, shape_v;
+        std::string qb = SkipScalar(g, L[qk]->inputs[0], m), kb = SkipScalar(g, L[qk]->inputs[1], m);
+        m->lq = head_split_(g, qb, {0, 2, 1, 3}, {1, 0, 2}, &m->chain, &m->split_shape);
+        m->lk = head_split_(g, kb, {0, 2, 3, 1}, {1, 2, 0}, &m->chain, &shape_k);
+        if (m->lq < 0 || m->lk < 0)
+            return false;
+        // the softmax must run over the keys, i.e. the last axis of the scores, whose rank is the head split's
+        // (axis normalisation of cpu_softmax_layer_acc.cc:43-44)
+        const int rank = (int)m->split_shape.size();
+        if (rank < 3 || ((sp->axis % rank) + rank) % rank != rank - 1)
+            return false;
+        // ---- downstream: MatMul(probs, v) -> Permute -> Reshape
+        int pv = g.sole_consumer(sm->outputs[0]);
+        if (pv < 0 || !L[pv] || L[pv]->type != LAYER_MATMUL || L[pv]->inputs.size() != 2 || L[pv]->inputs[0] != sm->outputs[0] ||
+            L[pv]->inputs[1] == sm->outputs[0] || IsModelOutput(sm->outputs[0]) || Res<MatMulLayerResource>(L[pv]->name))
+            return false;
+        m->chain.push_back(pv);
+        m->lv = head_split_(g, L[pv]->inputs[1], {0, 2, 1, 3}, {1, 0, 2}, &m->chain, &shape_v);
+        if (m->lv < 0 || m->split_shape != shape_k || m->split_shape != shape_v)
+            return false;
+        int pm = g.sole_consumer(L[pv]->outputs[0]);
+        if (pm < 0 || !L[pm] || L[pm]->type != LAYER_PERMUTE || IsModelOutput(L[pv]->outputs[0]))
+            return false;
+        auto pmp = dynamic_cast<PermuteLayerParam *>(L[pm]->param.get());
+        if (!pmp || pmp->orders != (rank == 4 ? std::vector<int>{0, 2, 1, 3} : std::vector<int>{1, 0, 2}))
+            return false;
+        int rs = g.sole_consumer(L[pm]->outputs[0]);
+        if (rs < 0 || !L[rs] || L[rs]->type != LAYER_RESHAPE || L[rs]->inputs.size() != 1 || IsModelOutput(L[pm]->outputs[0]))
+            return false;
+        // the merge must put the heads of one token side by side again: [B, S, hidden] or [tokens, hidden]
+        auto rsp = dynamic_cast<ReshapeLayerParam *>(L[rs]->param.get());
+        const int hidden = m->split_shape[rank - 2] * m->split_shape[rank - 1];
+        if (!rsp || rsp->axis != 0 || rsp->shape.empty() || rsp->shape.back() != hidden)
+            return false;
+        m->chain.push_back(pm);
+        m->chain.push_back(rs);
+        m->rs = rs;
+        if (L[m->lq]->inputs[0] != L[m->lk]->inputs[0] || L[m->lq]->inputs[0] != L[m->lv]->inputs[0])
+            return false;
+        // ---- the mask: computed before the chain starts, and one value per key
+        if (!m->mask.empty()) {
+            int first = *std::min_element(m->chain.begin(), m->chain.end());
+            int pmask = g.producer_of(m->mask);
+            bool early = pmask >= 0 ? pmask < first
+                                    : structure_->inputs_shape_map.count(m->mask) > 0 || resource_->constant_map.count(m->mask) > 0;
+            DimsVector md;
+            if (!early || !StaticDims(g, m->mask, &md, 0) || (int)md.size() != rank)
+                return false;
+            for (int a = 1; a + 1 < rank; ++a)
+                if (md[a] != 1)
+                    return false;  // a per-head or per-query mask
+            if (rank == 3 && md[0] != 1)
+                return false;  // [B*heads, 1, S]: one row per (sequence, head)
+        }
+        return true;
+    }
+
+private:
+    bool IsModelOutput(const std::string &b) const { return structure_->outputs.count(b) > 0; }
+    template <typename T> T *Res(const std::string &name) const {
+        auto it = resource_->resource_map.find(name);
+        return it == resource_->resource_map.end() ? nullptr : dynamic_cast<T *>(it->second.get());
+    }
+    // Mul / Div by one fp32 value held in the layer's resource: *factor is what it multiplies its input by
+    bool ScalarFactor(const std::shared_ptr<LayerInfo> &l, float *factor) const {
+        if (!l || (l->type != LAYER_MUL && l->type != LAYER_DIV) || l->inputs.size() != 1 || l->param->quantized)
+            return false;
+        auto er = Res<EltwiseLayerResource>(l->name);
+        if (!er || er->element_handle.GetDataCount() != 1 || er->element_handle.GetDataType() != DATA_TYPE_FLOAT)
+            return false;
+        auto bp = dynamic_cast<MultidirBroadcastLayerParam *>(l->param.get());
+        float v = er->element_handle.force_to<float *>()[0];
+        if (l->type == LAYER_DIV && bp && bp->weight_input_index == 0)
+            return false;  // s / scores is no scaling
+        *factor = l->type == LAYER_MUL ? v : 1.0f / v;
+        return true;
+    }
+    // does `blob` come out of MatMul(2 inputs), possibly through one scalar factor?
+    bool IsScoreChain(const GraphIndex &g, const std::string &blob) const {
+        auto &L = structure_->layers;
+        int p   = g.producer_of(blob);
+        float v;
+        if (p >= 0 && L[p] && ScalarFactor(L[p], &v))
+            p = g.producer_of(L[p]->inputs[0]);
+        return p >= 0 && L[p] && L[p]->type == LAYER_MATMUL && L[p]->inputs.size() == 2;
+    }
+    // a scalar factor on an operand of the score MatMul is folded into the scale
+    std::string SkipScalar(const GraphIndex &g, const std::string &blob, AttentionCore *m) const {
+        auto &L = structure_->layers;
+        int p   = g.producer_of(blob);
+        float v;
+        if (p < 0 || !L[p] || !ScalarFactor(L[p], &v) || g.sole_consumer(blob) < 0 || IsModelOutput(blob))
+            return blob;
+        m->scale *= v;
+        m->chain.push_back(p);
+        return L[p]->inputs[0];
+    }
+    // The dims of `blob` as far as the graph fixes them before any shape inference has run: model inputs, constants,
+    // and what Cast / Unsqueeze / Squeeze / Reshape(static) / element-wise layers make of them.  false = unknown.
+    bool StaticDims(const GraphIndex &g, const std::string &blob, DimsVector *dims, int depth) const {
+        if (depth > 8)
+            return false;
+        auto in = structure_->inputs_shape_map.find(blob);
+        if (in != structure_->inputs_shape_map.end()) {
+            *dims = in->second;
+            return true;
+        }
+        auto ct = resource_->constant_map.find(blob);
+        if (ct != resource_->constant_map.end() && ct->second) {
+            *dims = ct->second->GetBufferDims();
+            return !dims->empty();
+        }
+        auto &L = structure_->layers;
+        int p   = g.producer_of(blob);
+        if (p < 0 || !L[p] || L[p]->outputs.size() != 1)
+            return false;
+        auto l = L[p];
+        switch (l->type) {
+            case LAYER_CAST:
+                return l->inputs.size() == 1 && StaticDims(g, l->inputs[0], dims, depth + 1);
+            case LAYER_UNSQUEEZE: {  // unsqueeze_layer.cc:44-54
+                auto sp = dynamic_cast<SqueezeLayerParam *>(l->param.get());
+                if (!sp || l->inputs.size() != 1 || !StaticDims(g, l->inputs[0], dims, depth + 1))
+                    return false;
+                for (int axis : sp->axes) {
+                    axis = axis < 0 ? axis + (int)dims->size() + 1 : axis;
+                    if (axis < 0 || axis > (int)dims->size())
+                        return false;
+                    dims->insert(dims->begin() + axis, 1);
+                }
+                return true;
+            }
+            case LAYER_ADD:
+            case LAYER_SUB:
+            case LAYER_MUL:
+            case LAYER_DIV: {
+                // element-wise with broadcasting (multidir_broadcast_layer.cc:59-111): the extent of each axis is the
+                // largest among the operands, shorter shapes are padded in front
+                std::vector<DimsVector> ops;
+                for (auto &i : l->inputs) {
+                    DimsVector d;
+                    if (!StaticDims(g, i, &d, depth + 1))
+                        return false;
+                    ops.push_back(d);
+                }
+                if (auto er = Res<EltwiseLayerResource>(l->name)) {
+                    DimsVector d = er->element_handle.GetBufferDims();
+                    if (er->element_handle.GetDataCount() == 1)
+                        d = {1};
+                    if (d.empty())
+                        return false;
+                    ops.push_back(d);
+                }
+                if (ops.empty())
+                    return false;
+                size_t rank = 0;
+                for (auto &d : ops)
+                    rank = std::max(rank, d.size());
+                dims->assign(rank, 1);
+                for (auto &d : ops)
+                    for (size_t a = 0; a < d.size(); ++a) {
+                        int &o = (*dims)[rank - d.size() + a];
+                        if (d[a] != 1 && o != 1 && d[a] != o)
+                            return false;
+                        o = std::max(o, d[a]);
+                    }
+                return true;
+            }
+            default:
+                return false;
+        }
+    }
+
+    NetStructure *structure_;
+    NetResource *resource_;
+    HeadSplitFn head_split_;
 };
 
 class RocmFusionPass : public optimizer::NetOptimizer {
@@ -366,73 +621,20 @@ private:
                 auto sm = L[si];
                 if (!sm || sm->type != LAYER_SOFTMAX)
                     continue;
-                std::vector<int> chain = {si};
-                // ---- upstream of the softmax: [Add(mask)] <- Mul|Div(scale) <- MatMul(q, k^T)
-                std::string cur = sm->inputs[0];
-                std::string mask;
-                float scale = 1.0f;
-                bool have_scale = false;
-                int qk = -1;
-                for (int step = 0; step < 3 && qk < 0; ++step) {
-                    int pi = g.producer_of(cur);
-                    if (pi < 0 || !L[pi] || g.sole_consumer(cur) < 0 || IsModelOutput(cur))
-                        break;
-                    auto pl = L[pi];
-                    if (pl->type == LAYER_ADD && pl->inputs.size() == 2 && mask.empty() && !have_scale) {
-                        // scores + mask : the operand that is not produced by the score chain is the mask
-                        int p0 = g.producer_of(pl->inputs[0]);
-                        bool first_is_scores = p0 >= 0 && L[p0] &&
-                                               (L[p0]->type == LAYER_MUL || L[p0]->type == LAYER_DIV || L[p0]->type == LAYER_MATMUL);
-                        mask = first_is_scores ? pl->inputs[1] : pl->inputs[0];
-                        cur  = first_is_scores ? pl->inputs[0] : pl->inputs[1];
-                        chain.push_back(pi);
-                    } else if ((pl->type == LAYER_MUL || pl->type == LAYER_DIV) && pl->inputs.size() == 1 && !have_scale) {
-                        auto er = ResOf<EltwiseLayerResource>(pl->name);
-                        if (!er || er->element_handle.GetDataCount() != 1 || er->element_handle.GetDataType() != DATA_TYPE_FLOAT)
-                            break;
-                        float v    = er->element_handle.force_to<float *>()[0];
-                        scale      = pl->type == LAYER_MUL ? v : 1.0f / v;
-                        have_scale = true;
-                        cur        = pl->inputs[0];
-                        chain.push_back(pi);
-                    } else if (pl->type == LAYER_MATMUL && pl->inputs.size() == 2) {
-                        qk = pi;
-                        chain.push_back(pi);
-                    } else {
-                        break;
-                    }
-                }
-                if (qk < 0)
+                AttentionCore m;
+                AttentionMatcher matcher(structure_, resource_,
+                                         [this](const GraphIndex &gi, const std::string &blob, const std::vector<int> &o4,
+                                                const std::vector<int> &o3, std::vector<int> *chain, DimsVector *shape) {
+                                             return HeadSplitSource(gi, blob, o4, o3, chain, shape);
+                                         });
+                if (!matcher.Match(g, si, &m))
                     continue;
-                // ---- q and k^T operands
-                DimsVector shape_q, shape_k, shape_v;
-                int lq = HeadSplitSource(g, L[qk]->inputs[0], {0, 2, 1, 3}, {1, 0, 2}, &chain, &shape_q);
-                int lk = HeadSplitSource(g, L[qk]->inputs[1], {0, 2, 3, 1}, {1, 2, 0}, &chain, &shape_k);
-                if (lq < 0 || lk < 0)
-                    continue;
-                // ---- downstream: MatMul(probs, v) -> Permute -> Reshape
-                int pv = g.sole_consumer(sm->outputs[0]);
-                if (pv < 0 || !L[pv] || L[pv]->type != LAYER_MATMUL || L[pv]->inputs.size() != 2 ||
-                    L[pv]->inputs[0] != sm->outputs[0] || IsModelOutput(sm->outputs[0]))
-                    continue;
-                chain.push_back(pv);
-                int lv = HeadSplitSource(g, L[pv]->inputs[1], {0, 2, 1, 3}, {1, 0, 2}, &chain, &shape_v);
-                if (lv < 0 || shape_q != shape_k || shape_q != shape_v)
-                    continue;
-                int pm = g.sole_consumer(L[pv]->outputs[0]);
-                if (pm < 0 || !L[pm] || L[pm]->type != LAYER_PERMUTE || IsModelOutput(L[pv]->outputs[0]))
-                    continue;
-                auto pmp = ParamOf<PermuteLayerParam>(L[pm]);
-                if (!pmp || (pmp->orders != std::vector<int>{0, 2, 1, 3} && pmp->orders != std::vector<int>{1, 0, 2}))
-                    continue;
-                int rs = g.sole_consumer(L[pm]->outputs[0]);
-                if (rs < 0 || !L[rs] || L[rs]->type != LAYER_RESHAPE || IsModelOutput(L[pm]->outputs[0]))
-                    continue;
-                chain.push_back(pm);
-                chain.push_back(rs);
-                // ---- the three projections read the same x and are plain linears of equal width
-                if (L[lq]->inputs[0] != L[lk]->inputs[0] || L[lq]->inputs[0] != L[lv]->inputs[0])
-                    continue;
+                const std::vector<int> &chain = m.chain;
+                const std::string &mask = m.mask;
+                const float scale = m.scale;
+                const int lq = m.lq, lk = m.lk, lv = m.lv, rs = m.rs;
+                const DimsVector &shape_q = m.split_shape;
+                // ---- the three projections are plain linears of equal width
                 auto rq = ResOf<RocmFusedLinearResource>(L[lq]->name), rk = ResOf<RocmFusedLinearResource>(L[lk]->name),
                      rv = ResOf<RocmFusedLinearResource>(L[lv]->name);
                 if (!rq || !rk || !rv)
@@ -446,16 +648,9 @@ private:
                 int seq      = shape_q[shape_q.size() - 3];
                 // seq 0 / -1: the split copies (or infers) the sequence length, i.e. the model is meant for
                 // Instance::Reshape; the acc then reads S from its input blob [B,S,H] at every reshape
-                if (heads * head_dim != H || head_dim != 64 || seq < -1)
+                if (heads * head_dim != H || K != H || head_dim != 64 || seq < -1)
                     continue;
                 int first = *std::min_element(chain.begin(), chain.end());
-                if (!mask.empty()) {
-                    int pmask = g.producer_of(mask);
-                    bool ok   = pmask >= 0 ? pmask < first : structure_->inputs_shape_map.count(mask) > 0 ||
-                                                                 resource_->constant_map.count(mask) > 0;
-                    if (!ok)
-                        continue;
-                }
                 // ---- build the fused layer
                 auto fl      = std::make_shared<LayerInfo>();
                 fl->type     = LAYER_ROCM_FUSED_ATTENTION;
@@ -845,65 +1040,19 @@ private:
                 auto sm = L[si];
                 if (!sm || sm->type != LAYER_SOFTMAX)
                     continue;
-                std::vector<int> chain = {si};
-                std::string cur = sm->inputs[0], mask;
-                float scale = 1.0f;
-                bool have_scale = false;
-                int qk = -1;
-                for (int step = 0; step < 3 && qk < 0; ++step) {
-                    int pi = g.producer_of(cur);
-                    if (pi < 0 || !L[pi] || g.sole_consumer(cur) < 0 || IsModelOutput(cur))
-                        break;
-                    auto pl = L[pi];
-                    if (pl->type == LAYER_ADD && pl->inputs.size() == 2 && mask.empty() && !have_scale) {
-                        int p0 = g.producer_of(pl->inputs[0]);
-                        bool first_is_scores = p0 >= 0 && L[p0] &&
-                                               (L[p0]->type == LAYER_MUL || L[p0]->type == LAYER_DIV || L[p0]->type == LAYER_MATMUL);
-                        mask = first_is_scores ? pl->inputs[1] : pl->inputs[0];
-                        cur  = first_is_scores ? pl->inputs[0] : pl->inputs[1];
-                        chain.push_back(pi);
-                    } else if ((pl->type == LAYER_MUL || pl->type == LAYER_DIV) && pl->inputs.size() == 1 && !have_scale) {
-                        auto er = ResOf<EltwiseLayerResource>(pl->name);
-                        if (!er || er->element_handle.GetDataCount() != 1 || er->element_handle.GetDataType() != DATA_TYPE_FLOAT)
-                            break;
-                        float v    = er->element_handle.force_to<float *>()[0];
-                        scale      = pl->type == LAYER_MUL ? v : 1.0f / v;
-                        have_scale = true;
-                        cur        = pl->inputs[0];
-                        chain.push_back(pi);
-                    } else if (pl->type == LAYER_MATMUL && pl->inputs.size() == 2) {
-                        qk = pi;
-                        chain.push_back(pi);
-                    } else {
-                        break;
-                    }
-                }
-                if (qk < 0)
+                AttentionCore m;
+                AttentionMatcher matcher(structure_, resource_,
+                                         [this](const GraphIndex &gi, const std::string &blob, const std::vector<int> &o4,
+                                                const std::vector<int> &o3, std::vector<int> *chain, DimsVector *shape) {
+                                             return QuantHeadSplitSource(gi, blob, o4, o3, chain, shape);
+                                         });
+                if (!matcher.Match(g, si, &m))
                     continue;
-                DimsVector shape_q, shape_k, shape_v;
-                int lq = QuantHeadSplitSource(g, L[qk]->inputs[0], {0, 2, 1, 3}, {1, 0, 2}, &chain, &shape_q);
-                int lk = QuantHeadSplitSource(g, L[qk]->inputs[1], {0, 2, 3, 1}, {1, 2, 0}, &chain, &shape_k);
-                if (lq < 0 || lk < 0)
-                    continue;
-                int pv = g.sole_consumer(sm->outputs[0]);
-                if (pv < 0 || !L[pv] || L[pv]->type != LAYER_MATMUL || L[pv]->inputs.size() != 2 ||
-                    L[pv]->inputs[0] != sm->outputs[0] || IsModelOutput(sm->outputs[0]))
-                    continue;
-                chain.push_back(pv);
-                int lv = QuantHeadSplitSource(g, L[pv]->inputs[1], {0, 2, 1, 3}, {1, 0, 2}, &chain, &shape_v);
-                if (lv < 0 || shape_q != shape_k || shape_q != shape_v)
-                    continue;
-                int pm = g.sole_consumer(L[pv]->outputs[0]);
-                if (pm < 0 || !L[pm] || L[pm]->type != LAYER_PERMUTE || IsModelOutput(L[pv]->outputs[0]))
-                    continue;
-                auto pmp = ParamOf<PermuteLayerParam>(L[pm]);
-                if (!pmp || (pmp->orders != std::vector<int>{0, 2, 1, 3} && pmp->orders != std::vector<int>{1, 0, 2}))
-                    continue;
-                int rs = g.sole_consumer(L[pm]->outputs[0]);
-                if (rs < 0 || !L[rs] || L[rs]->type != LAYER_RESHAPE || IsModelOutput(L[pm]->outputs[0]))
-                    continue;
-                chain.push_back(pm);
-                chain.push_back(rs);
+                const std::vector<int> &chain = m.chain;
+                const std::string &mask = m.mask;
+                const float scale = m.scale;
+                const int lq = m.lq, lk = m.lk, lv = m.lv, rs = m.rs;
+                const DimsVector &shape_q = m.split_shape;
                 // the three projections read the same int8 blob and have the same shape
                 if (L[lq]->inputs[0] != L[lk]->inputs[0] || L[lq]->inputs[0] != L[lv]->inputs[0])
                     continue;
@@ -924,13 +1073,6 @@ private:
                     !BlobScale(L[lv]->outputs[0], &out_scale[2]))
                     continue;
                 int first = *std::min_element(chain.begin(), chain.end());
-                if (!mask.empty()) {
-                    int pmask = g.producer_of(mask);
-                    bool ok   = pmask >= 0 ? pmask < first : structure_->inputs_shape_map.count(mask) > 0 ||
-                                                                 resource_->constant_map.count(mask) > 0;
-                    if (!ok)
-                        continue;
-                }
                 auto fl      = std::make_shared<LayerInfo>();
                 fl->type     = LAYER_ROCM_FUSED_ATTENTION;
                 fl->type_str = "RocmFusedAttention";
@@ -1360,8 +1502,11 @@ public:
             return Status(TNNERR_PARAM_ERR, "fused attention: token count is not a multiple of the sequence length");
         B_ = T_ / seq_;
         if (p->has_mask) {
-            if (inputs.size() < 2 || DimsVectorUtils::Count(In(inputs[1])->GetBlobDesc().dims) != B_ * seq_)
-                return Status(TNNERR_PARAM_ERR, "fused attention: mask must hold B*S additive values");
+            // one additive value per key: [B,1,1,S], or one row [1,1,1,S] for every sequence
+            const int count = inputs.size() < 2 ? -1 : DimsVectorUtils::Count(In(inputs[1])->GetBlobDesc().dims);
+            if (count != B_ * seq_ && count != seq_)
+                return Status(TNNERR_PARAM_ERR, "fused attention: mask must hold B*S (or S) additive values");
+            mask_one_row_ = count == seq_ && B_ > 1;
         }
         if (!weight_ && p->quant) {
             // requantisation factor w_scale / o_scale of each projection as one fp32 division on the host, 0 when
@@ -1421,7 +1566,8 @@ public:
         const int32_t *kv = nullptr;
         if (p->has_mask) {
             Blob *mb = In(inputs[1]);
-            RETURN_ON_NEQ(context_->AttentionMask(Ptr(mb), (int)mb->GetBlobDesc().data_type, B_, seq_, &mask, &kv), TNN_OK);
+            RETURN_ON_NEQ(context_->AttentionMask(Ptr(mb), (int)mb->GetBlobDesc().data_type, B_, seq_, mask_one_row_, &mask, &kv),
+                          TNN_OK);
         }
         const char *base = (const char *)qkv;
         const long d     = p->head_dim;
@@ -1490,6 +1636,7 @@ private:
     void *weight_ = nullptr, *bias_ = nullptr, *scale_ = nullptr, *dequant_ = nullptr, *colsum_ = nullptr, *gamma_ = nullptr,
          *beta_ = nullptr;
     int H_ = 0, K_ = 0, T_ = 0, B_ = 0, seq_ = 0;
+    bool mask_one_row_ = false;
 };
 REGISTER_ROCM_ACC(RocmFusedAttentionLayerAcc, LAYER_ROCM_FUSED_ATTENTION);
 

@@ -226,6 +226,16 @@ def mask_prepare(mask, threshold=-1000.0):
     return out, f32
 
 
+def mask_prepare_broadcast(mask_row, B, threshold=-1000.0):
+    """one mask row [S] of any float type serving B sequences: (flagged kv_len [B], dense fp32 mask [B,S])"""
+    _chk(mask_row)
+    S = mask_row.shape[-1]
+    out = torch.empty(B, dtype=torch.int32, device=mask_row.device)
+    f32 = torch.empty(B, S, dtype=torch.float32, device=mask_row.device)
+    capi.call("tnn_rocm_mask_prepare_strided", _stream(), dt(mask_row), _p(mask_row), 0, _p(f32), _p(out), B, S, float(threshold))
+    return out, f32
+
+
 def softmax(x, axis=-1):
     _chk(x)
     axis = axis % x.dim()

@@ -246,6 +246,83 @@ def encoder_graph(cfg, weights, B, S, with_embeddings=True, extra_outputs=(), dy
     return g
 
 
+def attention_block_graph(lw, B, S, H, heads, scale="mul", mask="b11s", mask_first=False, proj="matmul", rank3=False,
+                          softmax_axis=None, tap_scores=False):
+    """One self-attention block (three projections, attention core, output projection) in the spellings exporters
+    produce for the same arithmetic -- what a graph rewrite that recognises the core has to cope with:
+    scale     "mul" scores * (1/sqrt d) | "div" scores / sqrt d | "q" q * (1/sqrt d) ahead of the score product |
+              "qk" q and k^T each scaled by d^-1/4 | "none"
+    mask      None | "b11s" [B,1,1,S] | "111s" one row for every sequence | "b1ss" one value per query and key
+              [B,1,S,S] (rank3: "11s" [1,1,S] | "1ss" [1,S,S]); the model input is `attention_bias`
+    mask_first  Add(mask, scores) instead of Add(scores, mask)
+    proj      "matmul" MatMul + Add on `hidden` [B,S,H] | "inner_product" InnerProduct on `hidden` [B*S,H]
+    rank3     a single sequence (B == 1) split as [S,heads,d] with three-axis Permutes, scores [heads,S,S]
+    softmax_axis  default: the last axis of the scores
+    tap_scores    the scaled scores get a second reader (`scores_tap`, a model output)
+    Output `y` has the shape of `hidden`."""
+    assert H % heads == 0 and (not rank3 or B == 1)
+    d = H // heads
+    g = Graph()
+    flat = proj == "inner_product"
+    g.add_input("hidden", [B * S, H] if flat else [B, S, H])
+    if mask is not None:
+        g.add_input("attention_bias", {"b11s": [B, 1, 1, S], "111s": [1, 1, 1, S], "b1ss": [B, 1, S, S],
+                                       "11s": [1, 1, S], "1ss": [1, S, S]}[mask])
+    for nm in ("q", "k", "v"):
+        if flat:
+            g.add_layer("InnerProduct", "fc_" + nm, ["hidden"], [nm + "_o"], [H, 1, 0, 1])
+            g.res_inner_product("fc_" + nm, lw["w" + nm], lw["b" + nm])
+        else:
+            _linear(g, nm, "hidden", nm + "_o", lw["w" + nm], lw["b" + nm])
+        split = [0, 3, 3, S, heads, d, 0] if rank3 else [0, 4, 4, B, S, heads, d, 0]
+        g.add_layer("Reshape", nm + "_rs", [nm + "_o"], [nm + "_s"], split)
+    po, pt = ([3, 1, 0, 2], [3, 1, 2, 0]) if rank3 else ([4, 0, 2, 1, 3], [4, 0, 2, 3, 1])
+    g.add_layer("Permute", "q_pm", ["q_s"], ["qh"], po)
+    g.add_layer("Permute", "k_pm", ["k_s"], ["kt"], pt)
+    g.add_layer("Permute", "v_pm", ["v_s"], ["vh"], po)
+    qb, kb = "qh", "kt"
+    if scale in ("q", "qk"):
+        f = np.array([d ** -0.5 if scale == "q" else d ** -0.25], np.float32)
+        g.add_layer("Mul", "q_scale", ["qh"], ["qh_scaled"], [1])
+        g.res_eltwise("q_scale", "Mul", f)
+        qb = "qh_scaled"
+        if scale == "qk":
+            g.add_layer("Mul", "k_scale", ["kt"], ["kt_scaled"], [1])
+            g.res_eltwise("k_scale", "Mul", f)
+            kb = "kt_scaled"
+    g.add_layer("MatMul", "qk", [qb, kb], ["scores"], [-1])
+    cur = "scores"
+    if scale == "mul":
+        g.add_layer("Mul", "scale", [cur], ["scaled"], [1])
+        g.res_eltwise("scale", "Mul", np.array([1.0 / np.sqrt(d)], np.float32))
+        cur = "scaled"
+    elif scale == "div":
+        g.add_layer("Div", "scale", [cur], ["scaled"], [1])
+        g.res_eltwise("scale", "Div", np.array([np.sqrt(d)], np.float32))
+        cur = "scaled"
+    if tap_scores:
+        g.add_layer("Mul", "tap", [cur], ["scores_tap"], [1])
+        g.res_eltwise("tap", "Mul", np.array([1.0], np.float32))
+    if mask is not None:
+        g.add_layer("Add", "mask", ["attention_bias", cur] if mask_first else [cur, "attention_bias"], ["masked"], [1])
+        cur = "masked"
+    rank = 3 if rank3 else 4
+    g.add_layer("Softmax", "sm", [cur], ["probs"], [rank - 1 if softmax_axis is None else softmax_axis])
+    g.add_layer("MatMul", "pv", ["probs", "vh"], ["ctx_h"], [-1])
+    g.add_layer("Permute", "ctx_pm", ["ctx_h"], ["ctx_s"], po)
+    merge = [0, 2, 2, B * S, H, 0] if (flat or rank3) else [0, 3, 3, B, S, H, 0]
+    g.add_layer("Reshape", "ctx_rs", ["ctx_s"], ["ctx"], merge)
+    if flat:
+        g.add_layer("InnerProduct", "fc_o", ["ctx"], ["y"], [H, 1, 0, 1])
+        g.res_inner_product("fc_o", lw["wo"], lw["bo"])
+    else:
+        _linear(g, "o", "ctx", "y", lw["wo"], lw["bo"])
+    g.add_output("y")
+    if tap_scores:
+        g.add_output("scores_tap")
+    return g
+
+
 def attention_layer_graph(lw, S, H, heads):
     """Benchmark config 1: one self-attention layer on a [S,H] fp32 input with InnerProduct projections
     (mask all ones, so no Add(mask); scale applied by a Mul)."""
