@@ -47,7 +47,8 @@ def reference(lw, x, mask, B, S, H, heads, scale="mul", mask_first=False, proj="
     p = orc.softmax(s, (rank - 1) if softmax_axis is None else softmax_axis)
     c = orc.matmul(p, vh)
     c = orc.permute(c, (1, 0, 2) if rank3 else (0, 2, 1, 3)).reshape(B * S, H)
-    return lin(c, "wo", "bo").reshape(x.shape)
+    y = lin(c, "wo", "bo")
+    return y if (rank3 or proj == "inner_product") else y.reshape(B, S, H)   # the head-merging Reshape's dims
 
 
 def _run(name, spelling, fused):

@@ -219,8 +219,10 @@ ACCEPTED_SPELLINGS = {
     "negative_softmax_axis": dict(softmax_axis=-1),
 }
 REFUSED_SPELLINGS = {
-    "softmax_over_queries": dict(softmax_axis=2),
-    "softmax_over_heads": dict(softmax_axis=1),
+    # (no mask in these two: in fp16 blobs -10000 + score keeps nothing of the score, and a softmax across the queries
+    #  or heads of a masked key would then compare the fp16 rounding of the device with the fp32 of the checker)
+    "softmax_over_queries": dict(softmax_axis=2, mask=None),
+    "softmax_over_heads": dict(softmax_axis=1, mask=None),
     "mask_per_query_and_key": dict(mask="b1ss"),
     "rank3_mask_per_query": dict(B=1, rank3=True, mask="1ss"),
     "scores_read_twice": dict(tap_scores=True),
@@ -236,6 +238,11 @@ def test_attention_spelling_is_fused(name):
     att = [l for l in plan if l["type"] == "RocmFusedAttention"][0]
     assert att["inputs"] == (["hidden"] if ACCEPTED_SPELLINGS[name].get("mask", "b11s") is None
                              else ["hidden", "attention_bias"])
+    # the fused layer's output is the head-merging Reshape's output, with that layer's dims
+    sp = ACCEPTED_SPELLINGS[name]
+    B = sp.get("B", 2)
+    flat = sp.get("rank3") or sp.get("proj") == "inner_product"
+    assert att["output_dims"] == [[B * 32, 256] if flat else [B, 32, 256]], att["output_dims"]
 
 
 @pytest.mark.parametrize("name", sorted(REFUSED_SPELLINGS))

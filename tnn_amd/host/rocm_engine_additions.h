@@ -63,6 +63,12 @@ struct RocmFusedAttentionParam : public LayerParam {
     float scale  = 1.0f;
     int has_mask = 0;  // second input: additive mask broadcastable to [B,1,1,S]
     int seq_len  = 0;  // S of the matched head split ([B,S,h,d]); 0 = take it from the input blob's shape
+    // The fused layer's output is the output of the head-merging Reshape it replaced and must have that layer's dims:
+    // split_rank is the rank of the head split (4: [B,S,h,d], 3: [S,h,d]), merge_shape the Reshape's shape parameter
+    // (0 copies the dim of the split tensor, -1 is inferred; source/tnn/layer/reshape_layer.cc:41-63).  Empty = the
+    // dims of input 0.
+    int split_rank = 0;
+    std::vector<int> merge_shape;
     // quantised form: the first input is the int8 blob the three QuantizedInnerProduct projections read, the
     // resource is a RocmFusedQkvInt8Resource and qkv_out_scale are the scales of their three int8 output blobs
     int quant = 0;

@@ -667,6 +667,8 @@ private:
                 fp->head_dim = head_dim;
                 fp->scale    = scale;
                 fp->has_mask = mask.empty() ? 0 : 1;
+                fp->split_rank  = (int)shape_q.size();
+                fp->merge_shape = ParamOf<ReshapeLayerParam>(L[rs])->shape;
                 fl->param    = fp;
                 fp->seq_len  = seq > 0 ? seq : 0;
                 auto fr       = std::make_shared<RocmFusedLinearResource>();
@@ -1088,6 +1090,8 @@ private:
                 fp->head_dim = head_dim;
                 fp->scale    = scale;
                 fp->has_mask = mask.empty() ? 0 : 1;
+                fp->split_rank  = (int)shape_q.size();
+                fp->merge_shape = ParamOf<ReshapeLayerParam>(L[rs])->shape;
                 fp->seq_len  = seq;
                 fp->quant    = 1;
                 for (int t = 0; t < 3; ++t)

@@ -87,6 +87,58 @@ protected:
 class RocmFusedAttentionLayer : public RocmFusedLayerBase {
 public:
     explicit RocmFusedAttentionLayer(LayerType type) : RocmFusedLayerBase(type) {}
+
+protected:
+    // The context (output 0, and its quantised copy when there is one) gets the dims the head-merging Reshape of the
+    // replaced chain would have given it; a LayerNorm output keeps the dims of input 0.
+    Status InferOutputShape(bool ignore_error = false) override {
+        Status st = RocmFusedLayerBase::InferOutputShape(ignore_error);
+        if (st != TNN_OK)
+            return st;
+        auto p = dynamic_cast<RocmFusedAttentionParam *>(param_);
+        if (!p)
+            return Status(TNNERR_NULL_PARAM, "fused attention: param is nil");
+        if (p->merge_shape.empty() || p->heads <= 0 || p->head_dim <= 0)
+            return TNN_OK;
+        const DimsVector in = input_blobs_[0]->GetBlobDesc().dims;
+        const int hidden    = p->heads * p->head_dim;
+        if (in.empty() || in.back() <= 0)
+            return TNN_OK;
+        const int tokens = DimsVectorUtils::Count(in) / in.back();
+        const int seq    = p->seq_len > 0 ? p->seq_len : (in.size() >= 3 ? in[in.size() - 2] : tokens);
+        if (seq <= 0 || tokens % seq != 0)
+            return Status(TNNERR_PARAM_ERR, "fused attention: token count is not a multiple of the sequence length");
+        DimsVector split = p->split_rank == 3 ? DimsVector({seq, p->heads, p->head_dim})
+                                              : DimsVector({tokens / seq, seq, p->heads, p->head_dim});
+        if (p->split_rank == 3 && tokens != seq)
+            return Status(TNNERR_PARAM_ERR, "fused attention: a three-axis head split holds one sequence");
+        DimsVector out;
+        int infer = -1, known = 1;
+        for (size_t i = 0; i < p->merge_shape.size(); ++i) {
+            int v = p->merge_shape[i];
+            if (v == 0) {
+                if (i >= split.size())
+                    return Status(TNNERR_PARAM_ERR, "fused attention: head-merge shape copies a dim that does not exist");
+                v = split[i];
+            }
+            if (v == -1) {
+                if (infer >= 0)
+                    return Status(TNNERR_PARAM_ERR, "fused attention: head-merge shape infers two dims");
+                infer = (int)i;
+                v     = 1;
+            }
+            known *= v;
+            out.push_back(v);
+        }
+        if (infer >= 0 && known > 0)
+            out[infer] = tokens * hidden / known;
+        if (DimsVectorUtils::Count(out) != tokens * hidden)
+            return Status(TNNERR_PARAM_ERR, "fused attention: head-merge shape does not hold the context");
+        output_blobs_[0]->GetBlobDesc().dims = out;
+        if (p->out_quant && output_blobs_.size() >= 2)
+            output_blobs_.back()->GetBlobDesc().dims = out;
+        return TNN_OK;
+    }
 };
 
 // RocmFusedEmbedding: ids [..] int32 -> [.., H] in the network's float type
