@@ -331,6 +331,11 @@ TNN_ROCM_API int tnn_rocm_dequantize(void *stream, const int8_t *q, float scale,
  * row-major); every batch entry is computed (the reference's loop stops after the first). */
 TNN_ROCM_API int tnn_rocm_add_i8(void *stream, const int8_t *a, float sa, const int8_t *b, float sb, float inv_so,
                                  int8_t *y, size_t count, int channels, size_t inner);
+/* The same with one scale per channel for each blob, as the reference's acc prepares them (x86_add_layer_acc.cc:33-66:
+ * a_scale[c], b_scale[c] and 1.0 / o_scale[c]); sa, sb, inv_so are device arrays of `channels` values. */
+TNN_ROCM_API int tnn_rocm_add_i8_per_channel(void *stream, const int8_t *a, const float *sa, const int8_t *b,
+                                             const float *sb, const float *inv_so, int8_t *y, size_t count,
+                                             int channels, size_t inner);
 /* q_out = float2int8(gelu((float)q_in * in_scale) * out_inv_scale): Reformat -> GELU -> Reformat
  * collapsed into one pass (same three roundings as the separate layers). */
 TNN_ROCM_API int tnn_rocm_gelu_i8(void *stream, const int8_t *q_in, float in_scale, float out_inv_scale,

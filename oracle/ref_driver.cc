@@ -56,10 +56,11 @@ REF_API void *tnn_ref_create(const char *proto, size_t proto_len, const char *mo
     if (dev.compare(0, 4, "ROCM") == 0) {
         // the DEVICE_ROCM backend of this repository built against this engine (oracle/_ref/libtnn_rocm_engine.so, which
         // the caller has loaded into the process: its static registrations made the device known).  The device and
-        // network type values are the backend's own; "ROCM:fp32" asks for fp32 blobs, "ROCM" for the default (fp16).
+        // network type values are the backend's own; "ROCM:fp32" asks for fp32 blobs (PRECISION_HIGH), "ROCM:bf16" for
+        // bf16 (PRECISION_LOW), "ROCM" for the default (PRECISION_AUTO: fp16).
         nc.device_type  = static_cast<DeviceType>(0x1080);
         nc.network_type = NETWORK_TYPE_AUTO;  // RocmDevice::ConvertAutoNetworkType() names the backend's network
-        nc.precision    = dev == "ROCM:fp32" ? PRECISION_HIGH : PRECISION_AUTO;
+        nc.precision    = dev == "ROCM:fp32" ? PRECISION_HIGH : (dev == "ROCM:bf16" ? PRECISION_LOW : PRECISION_AUTO);
     }
     s->inst         = s->net.CreateInst(nc, st);
     if (st != TNN_OK || !s->inst) {
@@ -73,11 +74,14 @@ REF_API void *tnn_ref_create(const char *proto, size_t proto_len, const char *mo
 
 REF_API void tnn_ref_destroy(void *h) { delete static_cast<Session *>(h); }
 
-// mat_type: 0 = NCHW_FLOAT (fp32 data), 1 = NC_INT32 (int32 data)
+// mat_type: 0 = NCHW_FLOAT (fp32 data), 1 = NC_INT32 (int32 data), 2 = RESERVED_INT8_TEST (int8 data copied as it is
+// into an int8 blob: what the reference's layer unit tests feed quantised layers with, layer_test.cc:258-261)
+static MatType mat_type_of(int code) { return code == 1 ? NC_INT32 : (code == 2 ? RESERVED_INT8_TEST : NCHW_FLOAT); }
+
 REF_API int tnn_ref_set_input(void *h, const char *name, const void *data, int mat_type, const int *dims, int ndims) {
     Session *s = static_cast<Session *>(h);
     DimsVector d(dims, dims + ndims);
-    auto mat = std::make_shared<Mat>(DEVICE_NAIVE, mat_type == 1 ? NC_INT32 : NCHW_FLOAT, d, const_cast<void *>(data));
+    auto mat = std::make_shared<Mat>(DEVICE_NAIVE, mat_type_of(mat_type), d, const_cast<void *>(data));
     Status st = s->inst->SetInputMat(mat, MatConvertParam(), name);
     if (st != TNN_OK) {
         s->err = st.description();
@@ -127,6 +131,44 @@ REF_API int tnn_ref_get_output(void *h, const char *name, float *out, size_t cap
         return -2;
     }
     memcpy(out, mat->GetData(), count * sizeof(float));
+    return 0;
+}
+
+// The data type of output blob `name` as the network settled it (DATA_TYPE_FLOAT 0, HALF 1, INT8 2, INT32 3, BFP16 4),
+// -1 if there is no such output: the reference's layer tests choose their comparison rule by it (layer_test.cc:386-404).
+REF_API int tnn_ref_output_data_type(void *h, const char *name) {
+    Session *s = static_cast<Session *>(h);
+    BlobMap blobs;
+    if (s->inst->GetAllOutputBlobs(blobs) != TNN_OK || !blobs.count(name))
+        return -1;
+    return (int)blobs[name]->GetBlobDesc().data_type;
+}
+
+// As tnn_ref_get_output with the Mat type chosen by the caller (codes of tnn_ref_set_input); capacity in bytes.
+REF_API int tnn_ref_get_output_as(void *h, const char *name, int mat_type, void *out, size_t capacity_bytes, int *dims,
+                                  int *ndims) {
+    Session *s = static_cast<Session *>(h);
+    std::shared_ptr<Mat> mat;
+    Status st = s->inst->GetOutputMat(mat, MatConvertParam(), name, DEVICE_NAIVE, mat_type_of(mat_type));
+    if (st != TNN_OK || !mat) {
+        s->err = st.description();
+        return st != TNN_OK ? (int)st : -1;
+    }
+    DimsVector d = mat->GetDims();
+    size_t count = 1;
+    for (int v : d)
+        count *= (size_t)v;
+    if (ndims)
+        *ndims = (int)d.size();
+    if (dims)
+        for (size_t i = 0; i < d.size() && i < 8; ++i)
+            dims[i] = d[i];
+    const size_t bytes = count * (mat_type == 2 ? 1 : 4);
+    if (bytes > capacity_bytes) {
+        s->err = "output buffer too small";
+        return -2;
+    }
+    memcpy(out, mat->GetData(), bytes);
     return 0;
 }
 

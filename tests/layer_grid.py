@@ -1,0 +1,319 @@
+"""The parameter grids of the reference's own layer unit tests for the ops of the encoder path, restated as one-layer
+model files, so that its edge cases (broadcast classes, every permutation, softmax over any axis of 2..5-D blobs,
+LayerNorm over 2..5 trailing dims, MatMul with a constant on either side, InnerProduct over a flattened [C,H,W],
+per-channel blob scales of the int8 layers) can be run against DEVICE_ROCM inside the reference engine, next to its
+DEVICE_NAIVE, the way test/unit_test/layer_test/layer_test.cc:53-215 runs them.
+
+The reference's `unit_test` binary itself cannot be built in this image: test/flags.h needs <gflags/gflags.h>, and the
+vendored third_party/gflags only ships the templates (gflags.h.in, gflags_declare.h.in) from which its CMake build
+generates those headers.  So each grid below is the INSTANTIATE_TEST_SUITE_P of the cited file with that test's own
+skip rules, the inputs take the values the harness draws (a 16-step grid in [-range, range), range = 1 + input index:
+source/tnn/utils/random_data_utils.cc:22-28, layer_test.cc:266-292), weights follow the resource generator
+(source/tnn/interpreter/layer_resource_generator.cc), and results are compared with the harness's rules
+(test/test_utils.cc:104-172, layer_test.cc:386-404).  What the image's ROCm device is not asked for is listed where a
+grid is cut: the skip rules that name other devices are left out, the ones that hold for every device are kept."""
+import itertools
+
+import numpy as np
+
+from tnn_amd import tnnmodel
+
+BASIC_BATCH_CHANNEL_SIZE = ([1, 2], [1, 2, 3, 4, 10, 32], [9, 10, 16, 19])   # test/unit_test/unit_test_macro.h:31-32
+UNARY_BATCH_CHANNEL_SIZE = ([1, 2], [1, 3, 4], [3])                           # unit_test_macro.h:34-35
+
+DT_FLOAT, DT_HALF, DT_INT8, DT_INT32, DT_BFP16 = 0, 1, 2, 3, 4
+MAX_ELEMS = 1 << 22   # cases with a larger blob are listed but not run (inputs None): they only cost time
+
+
+class Case:
+    """one TEST_P instance: a one-layer graph, its float / int8 inputs and a readable id"""
+
+    def __init__(self, op, ident, graph, inputs, int8=False, precisions=("fp16", "fp32")):
+        self.op, self.ident, self.graph, self.inputs, self.int8, self.precisions = op, ident, graph, inputs, int8, precisions
+
+
+def grid_values(rng, shape, rng_range=1.0):
+    """InitRandom(T *, n, range): (rand() % 16 - 8) / 8 * range (random_data_utils.cc:22-28)"""
+    return ((rng.integers(0, 16, size=shape) - 8) / 8.0 * rng_range).astype(np.float32)
+
+
+def int8_values(rng, shape, rng_range=8):
+    return ((rng.integers(0, 16, size=shape) - 8) / 8.0 * rng_range).astype(np.int8)
+
+
+def _dims(lead, tail_value, count):
+    d = list(lead)
+    while len(d) < count:
+        d.append(tail_value)
+    return d
+
+
+def _single(op_type, name, in_dims, params, in_types=None):
+    g = tnnmodel.Graph()
+    ins = []
+    for i, d in enumerate(in_dims):
+        g.add_input("input%d" % i, d, DT_FLOAT if in_types is None else in_types[i])
+        ins.append("input%d" % i)
+    g.add_layer(op_type, name, ins, ["output0"], params)
+    g.add_output("output0")
+    return g
+
+
+def _blob_scale(g, blob, channels, rng):
+    """BlobScaleLayerResourceGenerator (layer_resource_generator.cc:348-371): one scale per channel (dims[1]) drawn
+    uniformly from (0, 1), zero points 0"""
+    s = rng.uniform(0.0, 1.0, size=channels).astype(np.float32)
+    s[np.abs(s) < np.finfo(np.float32).eps] = 1.0
+    g.res_blob_scale(blob, s)
+    return s
+
+
+# ---- MatMul: test_matmul_layer.cc:59-124 ----------------------------------------------------------------------------
+def _cross_broadcast(d0, d1):  # test_matmul_layer.cc:25-51
+    a, b = list(d0), list(d1)
+    while len(a) < len(b):
+        a.insert(0, 1)
+    while len(b) < len(a):
+        b.insert(0, 1)
+    b0 = any(x < y for x, y in zip(a[:-2], b[:-2]))
+    b1 = any(x > y for x, y in zip(a[:-2], b[:-2]))
+    return b0 and b1
+
+
+def matmul_cases(rng):
+    a_dims = ([3, 4, 8, 16], [3, 1, 8, 16], [1, 4, 8, 16], [4, 8, 16], [1, 8, 16], [8, 16])
+    b_dims = ([16, 9], [1, 16, 9], [4, 16, 9], [3, 4, 16, 9], [1, 4, 16, 9], [3, 1, 16, 9])
+    for d0, d1, pos in itertools.product(a_dims, b_dims, (-1, 0, 1)):
+        batch0, batch1 = int(np.prod(d0[:-2])), int(np.prod(d1[:-2]))
+        if _cross_broadcast(d0, d1) or (batch0 > 1 and batch1 > 1 and batch0 != batch1):
+            continue
+        ident = "a%s_b%s_w%d" % ("x".join(map(str, d0)), "x".join(map(str, d1)), pos)
+        if pos == -1:
+            g = _single("MatMul", "layer_name", [d0, d1], [-1])
+            inputs = {"input0": grid_values(rng, d0, 1.0), "input1": grid_values(rng, d1, 2.0)}
+        else:
+            wd, xd = (d0, d1) if pos == 0 else (d1, d0)
+            g = _single("MatMul", "layer_name", [xd], [pos])
+            g.res_matmul("layer_name", grid_values(rng, wd, 1.0))
+            inputs = {"input0": grid_values(rng, xd, 1.0)}
+        yield Case("MatMul", ident, g, inputs)
+
+
+# ---- InnerProduct: test_innerproduct_layer.cc:27-74 (axis 1 over [C,H,W]) -------------------------------------------
+def inner_product_cases(rng):
+    for batch, ch, size, out_ch, has_bias in itertools.product((1, 2, 8, 11), (1, 3, 10, 32), (9, 10, 16, 19),
+                                                               (4, 8, 21, 50), (0, 1)):
+        dims = [batch, ch, size, size]
+        k = ch * size * size
+        g = _single("InnerProduct", "layer_name", [dims], [out_ch, has_bias, 0, 1])
+        g.res_inner_product("layer_name", grid_values(rng, (out_ch, k), 1.0),
+                            grid_values(rng, (out_ch,), 1.0) if has_bias else None)
+        yield Case("InnerProduct", "n%d_c%d_s%d_o%d_b%d" % (batch, ch, size, out_ch, has_bias), g,
+                   {"input0": grid_values(rng, dims, 1.0)}, precisions=("fp16", "fp32", "bf16"))
+
+
+# ---- quantised InnerProduct: test_innerproduct_int8_layer.cc:27-59 -------------------------------------------------
+def inner_product_int8_cases(rng):
+    for batch, ch, size, out_ch in itertools.product((1, 2), (1, 8, 9, 16), (1, 9, 16, 19), (1, 4, 8, 16, 32)):
+        dims = [batch, ch, size, size]
+        k = ch * size * size
+        g = _single("QuantizedInnerProduct", "layer_name", [dims], [out_ch, 0, 0, 1])
+        # InnerProductLayerResourceGenerator, quantised branch (layer_resource_generator.cc:199-212): int8 weights in
+        # [-4, 4), int32 bias in [-8, 8), one scale per output channel from (0, 1)
+        w = int8_values(rng, (out_ch, k), 4)
+        b = ((rng.integers(0, 16, size=out_ch) - 8)).astype(np.int32)
+        g.res_inner_product("layer_name", w, b, quant_scale=rng.uniform(0.0, 1.0, size=out_ch).astype(np.float32))
+        _blob_scale(g, "input0", ch, rng)
+        _blob_scale(g, "output0", out_ch, rng)
+        yield Case("QuantizedInnerProduct", "n%d_c%d_s%d_o%d" % (batch, ch, size, out_ch), g,
+                   {"input0": int8_values(rng, dims, 8)}, int8=True, precisions=("fp16",))
+
+
+# ---- Softmax: test_softmax_layer.cc:27-94 ----------------------------------------------------------------------------
+def softmax_cases(rng):
+    for batch, ch, h, w, axis, nd in itertools.product((1, 2), (10, 12, 512), (10, 512), (1, 4, 8, 10, 512),
+                                                        (-1, 0, 1, 2, 3, 4), (2, 3, 4, 5)):
+        if axis >= nd:
+            continue
+        if (ch == 512 and h == 512) or (w == 512 and h == 512) or (ch == 512 and w == 512):
+            continue
+        dims, sizes, i = [batch, ch], [h, w], 0
+        while len(dims) < nd:
+            dims.append(sizes[i])
+            i = (i + 1) % 2
+        yield Case("Softmax", "%s_axis%d" % ("x".join(map(str, dims)), axis), _single("Softmax", "layer_name", [dims], [axis]),
+                   {"input0": grid_values(rng, dims, 1.0)} if np.prod(dims) <= MAX_ELEMS else None,
+                   precisions=("fp16", "fp32", "bf16"))
+
+
+# ---- LayerNorm: test_layer_norm_layer.cc:26-89 (scale and bias are model inputs) ----------------------------------
+def layer_norm_cases(rng):
+    for batch, ch, size, reduce, nd in itertools.product((1, 2), (1, 4, 6), (10, 20, 65, 128), (2, 3, 4, 5), (2, 3, 4, 5)):
+        if nd - reduce < 0:
+            continue
+        dims = _dims([batch, ch], size, nd)
+        sb = dims[nd - reduce:]
+        g = _single("LayerNorm", "layer_name", [dims, sb, sb], [reduce, repr(1e-5)])
+        yield Case("LayerNorm", "%s_r%d" % ("x".join(map(str, dims)), reduce), g,
+                   {"input0": grid_values(rng, dims, 1.0), "input1": grid_values(rng, sb, 2.0),
+                    "input2": grid_values(rng, sb, 3.0)} if np.prod(dims) <= MAX_ELEMS else None)
+
+
+# ---- GELU: test_gelu_layer.cc:26-70 ; Tanh: test_tanh_layer.cc + test_unary_layer.cc:24-70 ---------------------------
+def gelu_cases(rng):
+    for batch, ch, size, nd in itertools.product((1, 2), (1, 4, 15), (1, 6, 8, 13), (2, 3, 4, 5)):
+        dims = _dims([batch, ch], size, nd)
+        yield Case("GELU", "x".join(map(str, dims)), _single("GELU", "layer_name", [dims], []),
+                   {"input0": grid_values(rng, dims, 1.0)})
+
+
+def tanh_cases(rng):
+    for batch, ch, size, nd in itertools.product(*UNARY_BATCH_CHANNEL_SIZE, (2, 3, 4, 5)):
+        dims = _dims([batch, ch], size, nd)
+        yield Case("Tanh", "x".join(map(str, dims)), _single("Tanh", "layer_name", [dims], []),
+                   {"input0": grid_values(rng, dims, 1.0)})
+
+
+# ---- Permute: test_permute_layer.cc:24-70 (every permutation of 2..5 axes) -------------------------------------------
+def permute_cases(rng):
+    for batch, ch, size, nd in itertools.product(*BASIC_BATCH_CHANNEL_SIZE, (2, 3, 4, 5)):
+        dims = _dims([batch, ch], size, nd)
+        x = grid_values(rng, dims, 1.0)
+        for order in itertools.permutations(range(nd)):
+            yield Case("Permute", "%s_o%s" % ("x".join(map(str, dims)), "".join(map(str, order))),
+                       _single("Permute", "layer_name", [dims], [nd] + list(order)), {"input0": x})
+
+
+# ---- Add / Sub / Mul / Div: test_binary_layer.cc:24-150, test_{add,sub,mul,div}_layer.cc ---------------------------
+def binary_cases(rng, op):
+    for batch, ch, size, n_in, ptype, widx, nd in itertools.product(*BASIC_BATCH_CHANNEL_SIZE, (1, 2), (0, 1, 2, 3),
+                                                                    (-1, 0, 1), (2, 3, 4)):
+        if n_in == 1 and widx == -1:
+            continue  # "this case doesn't exist" (test_binary_layer.cc:119-121)
+        in_dims = [batch, ch, size, size][:nd]
+        p_dims = {0: [1, 1, 1, 1], 1: [1, ch, 1, 1], 2: [1, ch, size, size], 3: [1, 1, size, size]}[ptype][:nd]
+        ident = "%s_in%d_p%d_w%d" % ("x".join(map(str, in_dims)), n_in, ptype, widx)
+        positive = op == "Div"   # a constant divisor is kept away from zero (test_div_layer.cc:39: resource_positive)
+        draw = (lambda shape, r: rng.uniform(0.001, 1.0, size=shape).astype(np.float32)) if positive else \
+            (lambda shape, r: grid_values(rng, shape, r))
+        if n_in == 1:
+            g = _single(op, "layer_name", [in_dims], [widx])
+            g.res_eltwise("layer_name", op, draw(p_dims, 1.0))
+            inputs = {"input0": grid_values(rng, in_dims, 1.0)}
+        else:
+            d0, d1 = (in_dims, in_dims) if widx == -1 else ((p_dims, in_dims) if widx == 0 else (in_dims, p_dims))
+            g = _single(op, "layer_name", [d0, d1], [widx])
+            inputs = {"input0": grid_values(rng, d0, 1.0), "input1": grid_values(rng, d1, 2.0)}
+        yield Case(op, ident, g, inputs)
+
+
+def add_int8_cases(rng):
+    """the int8 leg of test_add_layer.cc:31-44: single batch, two inputs of the full shape"""
+    for ch, size, widx, nd in itertools.product(BASIC_BATCH_CHANNEL_SIZE[1], BASIC_BATCH_CHANNEL_SIZE[2], (-1, 0, 1), (2, 3, 4)):
+        dims = [1, ch, size, size][:nd]
+        g = _single("QuantizedAdd", "layer_name", [dims, dims], [widx])
+        for blob in ("input0", "input1", "output0"):
+            _blob_scale(g, blob, ch, rng)
+        yield Case("QuantizedAdd", "%s_w%d" % ("x".join(map(str, dims)), widx), g,
+                   {"input0": int8_values(rng, dims, 8), "input1": int8_values(rng, dims, 8)}, int8=True,
+                   precisions=("fp16",))
+
+
+# ---- Reshape / Squeeze / Unsqueeze: test_reshape_layer.cc:27-87, test_squeeze_layer.cc:32-98, test_unsqueeze_layer.cc
+def reshape_cases(rng):
+    for batch, ch, size, nd, rtype in itertools.product(*BASIC_BATCH_CHANNEL_SIZE, (2, 3, 4, 5, 6), (0, 1)):
+        if rtype == 1 and nd > 4:
+            continue
+        dims = _dims([batch, ch], size, nd)
+        if np.prod(dims) > MAX_ELEMS:
+            continue
+        shape = _dims([0, -1], 1, nd)
+        g = _single("Reshape", "layer_name", [dims], [0, nd, nd] + shape + [rtype])
+        yield Case("Reshape", "%s_t%d" % ("x".join(map(str, dims)), rtype), g, {"input0": grid_values(rng, dims, 1.0)},
+                   precisions=("fp16", "fp32", "bf16"))
+
+
+SQUEEZE_AXES = ([0], [1], [2], [3], [0, 1], [0, 2], [1, -2], [0, -1], [0, 3], [1, 3], [1, 2, -1])
+UNSQUEEZE_AXES = ([0], [1], [2], [3], [0, 1], [0, 2], [1, -2], [0, -1], [0, 3], [1, 2], [0, 1, -2])
+
+
+def squeeze_cases(rng):
+    for d0, d1, d2, nd, axes in itertools.product(*BASIC_BATCH_CHANNEL_SIZE, (2, 3, 4, 5, 6), SQUEEZE_AXES):
+        dims = _dims([d0, d1], d2, nd)
+        if len(dims) - len(axes) < 2:
+            continue
+        erased, ok = 0, True
+        for a in reversed(axes):
+            a = a if a >= 0 else a + len(dims) - erased
+            if a >= len(dims) or a < 0:
+                ok = False
+                break
+            dims[a] = 1
+            erased += 1
+        if not ok or np.prod(dims) > MAX_ELEMS:
+            continue
+        g = _single("Squeeze", "layer_name", [dims], [len(axes)] + list(axes))
+        yield Case("Squeeze", "%s_a%s" % ("x".join(map(str, dims)), "_".join(map(str, axes))), g,
+                   {"input0": grid_values(rng, dims, 1.0)})
+
+
+def unsqueeze_cases(rng):
+    for d0, d1, d2, nd, axes in itertools.product(*BASIC_BATCH_CHANNEL_SIZE, (2, 3, 4, 5, 6), UNSQUEEZE_AXES):
+        dims = _dims([d0, d1], d2, nd)
+        if any(not (0 <= (a if a >= 0 else a + len(dims) + i) <= len(dims)) for i, a in enumerate(axes)):
+            continue
+        if len(axes) + len(dims) > 6 or np.prod(dims) > MAX_ELEMS:
+            continue
+        g = _single("Unsqueeze", "layer_name", [dims], [len(axes)] + list(axes))
+        yield Case("Unsqueeze", "%s_a%s" % ("x".join(map(str, dims)), "_".join(map(str, axes))), g,
+                   {"input0": grid_values(rng, dims, 1.0)})
+
+
+GRIDS = {
+    "MatMul": matmul_cases,
+    "InnerProduct": inner_product_cases,
+    "QuantizedInnerProduct": inner_product_int8_cases,
+    "Softmax": softmax_cases,
+    "LayerNorm": layer_norm_cases,
+    "GELU": gelu_cases,
+    "Tanh": tanh_cases,
+    "Permute": permute_cases,
+    "Add": lambda rng: binary_cases(rng, "Add"),
+    "Sub": lambda rng: binary_cases(rng, "Sub"),
+    "Mul": lambda rng: binary_cases(rng, "Mul"),
+    "Div": lambda rng: binary_cases(rng, "Div"),
+    "QuantizedAdd": add_int8_cases,
+    "Reshape": reshape_cases,
+    "Squeeze": squeeze_cases,
+    "Unsqueeze": unsqueeze_cases,
+}
+
+
+# ---- the harness's comparison rules (test/test_utils.cc:104-172, chosen by the device blob's type: layer_test.cc:386-404)
+def compare(ref, got, data_type):
+    """None if the harness would pass the pair, else a short description of the first offence"""
+    if ref.shape != got.shape:
+        return "dims %s vs %s" % (list(ref.shape), list(got.shape))
+    if data_type in (DT_INT8,):
+        d = np.abs(ref.astype(np.int32) - got.astype(np.int32))
+        return None if d.size == 0 or d.max() <= 1 else "int8 differs by %d at %d" % (d.max(), int(d.argmax()))
+    if data_type == DT_INT32:
+        return None if np.array_equal(ref, got) else "int32 values differ"
+    ref64, got64 = ref.astype(np.float64).ravel(), got.astype(np.float64).ravel()
+    with np.errstate(divide="ignore", invalid="ignore"):   # x / 0 cases: inf and NaN on both sides compare as the harness's
+        diff, tot = np.abs(got64 - ref64), np.abs(got64) + np.abs(ref64)
+        rel = np.where(tot > 0, diff / tot, 0.0)
+    if not np.all(np.isfinite(got64) | ~np.isfinite(ref64)):
+        return "non-finite result"
+    if data_type == DT_BFP16:
+        bad = (rel > 0.05) & (diff > 5e-2)
+        return None if not bad.any() else "bf16 at %d: %.6f vs %.6f" % (int(bad.argmax()), got64[bad.argmax()], ref64[bad.argmax()])
+    dp = 1e-4 if data_type == DT_FLOAT else 1e-3
+    bad = (rel > 0.01) & (diff > dp)
+    if not bad.any():
+        return None
+    cos = float(np.dot(got64, ref64) / ((np.sqrt(np.dot(got64, got64)) + 1e-9) * (np.sqrt(np.dot(ref64, ref64)) + 1e-9)))
+    if np.isnan(cos) or cos < 0.9998:
+        i = int(bad.argmax())
+        return "at %d: %.6f vs %.6f (cosine %.6f)" % (i, got64[i], ref64[i], cos)
+    return None

@@ -26,6 +26,9 @@ def lib():
         _lib.tnn_ref_forward.argtypes = [C.c_void_p]
         _lib.tnn_ref_get_output.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
                                             C.POINTER(C.c_int)]
+        _lib.tnn_ref_get_output_as.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
+                                               C.POINTER(C.c_int)]
+        _lib.tnn_ref_output_data_type.argtypes = [C.c_void_p, C.c_char_p]
         _lib.tnn_ref_last_error.restype = C.c_char_p
         _lib.tnn_ref_last_error.argtypes = [C.c_void_p]
         _lib.tnn_ref_time_forward.restype = C.c_double
@@ -50,11 +53,12 @@ class RefSession:
 
     def set_input(self, name, arr):
         a = np.ascontiguousarray(arr)
-        assert a.dtype in (np.float32, np.int32)
+        assert a.dtype in (np.float32, np.int32, np.int8)   # int8: RESERVED_INT8_TEST, copied as it is into an int8 blob
         self._keep.append(a)
         dims = (C.c_int * a.ndim)(*a.shape)
         self._check(lib().tnn_ref_set_input(self.h, name.encode(), a.ctypes.data_as(C.c_void_p),
-                                            1 if a.dtype == np.int32 else 0, dims, a.ndim), "SetInputMat")
+                                            {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.int8): 2}[a.dtype],
+                                            dims, a.ndim), "SetInputMat")
 
     def forward(self):
         self._check(lib().tnn_ref_forward(self.h), "Forward")
@@ -65,6 +69,22 @@ class RefSession:
         nd = C.c_int(0)
         self._check(lib().tnn_ref_get_output(self.h, name.encode(), buf.ctypes.data_as(C.c_void_p), max_elems, dims,
                                              C.byref(nd)), "GetOutputMat")
+        shape = [dims[i] for i in range(nd.value)]
+        return buf[:int(np.prod(shape))].reshape(shape).copy()
+
+    def output_data_type(self, name):
+        """0 float, 1 half, 2 int8, 3 int32, 4 bf16: the output blob's type inside the network"""
+        return lib().tnn_ref_output_data_type(self.h, name.encode())
+
+    def output_as(self, name, dtype, max_elems=1 << 26):
+        """the output through a Mat of the given numpy type (float32, int32, or int8 = RESERVED_INT8_TEST)"""
+        dtype = np.dtype(dtype)
+        buf = np.empty(max_elems, dtype)
+        dims = (C.c_int * 8)()
+        nd = C.c_int(0)
+        code = {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.int8): 2}[dtype]
+        self._check(lib().tnn_ref_get_output_as(self.h, name.encode(), code, buf.ctypes.data_as(C.c_void_p), buf.nbytes,
+                                                dims, C.byref(nd)), "GetOutputMat")
         shape = [dims[i] for i in range(nd.value)]
         return buf[:int(np.prod(shape))].reshape(shape).copy()
 

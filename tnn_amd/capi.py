@@ -78,6 +78,7 @@ SIGNATURES = {
     "tnn_rocm_debug_set_store_through": [_i],
     "tnn_rocm_debug_set_attention_dma": [_i],
     "tnn_rocm_add_i8": [_vp, _vp, _f, _vp, _f, _f, _vp, _sz, _i, _sz],
+    "tnn_rocm_add_i8_per_channel": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _sz],
     "tnn_rocm_gelu_i8": [_vp, _vp, _f, _f, _vp, _sz],
 }
 

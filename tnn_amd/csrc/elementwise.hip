@@ -425,6 +425,19 @@ __global__ void __launch_bounds__(kBlock) add_i8_kernel(const int8_t *__restrict
     }
 }
 
+// the same with one scale per channel for each of the three blobs (device arrays of `channels` values)
+__global__ void __launch_bounds__(kBlock) add_i8_per_channel_kernel(const int8_t *__restrict__ a, const float *__restrict__ sa,
+                                                                    const int8_t *__restrict__ b, const float *__restrict__ sb,
+                                                                    const float *__restrict__ inv_so, int8_t *__restrict__ y,
+                                                                    size_t n, unsigned channels, size_t inner,
+                                                                    unsigned tail_from) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const unsigned c = (unsigned)((i / inner) % channels);
+        y[i]             = add_i8_value(a[i], sa[c], b[i], sb[c], inv_so[c], tail_from >= channels || c < tail_from);
+    }
+}
+
 // int8 -> GELU -> int8 has only 256 possible inputs, so the chain (dequantise, erf GELU, quantise) is a 256-entry
 // table.  The launcher evaluates it on the host with the C library's double erf - the very routine the reference's
 // CPU path calls - and hands it over by value as a kernel argument (256 bytes: no device memory, no copy, safe under
@@ -895,6 +908,20 @@ int tnn_rocm_add_i8(void *stream, const int8_t *a, float sa, const int8_t *b, fl
     else
         hipLaunchKernelGGL(add_i8_kernel, dim3(grid_for(n)), dim3(kBlock), 0, (hipStream_t)stream, a, sa, b, sb, inv_so,
                            y, n, (unsigned)channels, inner, (unsigned)tail_from);
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+int tnn_rocm_add_i8_per_channel(void *stream, const int8_t *a, const float *sa, const int8_t *b, const float *sb,
+                                const float *inv_so, int8_t *y, size_t n, int channels, size_t inner) {
+    if (n == 0)
+        return 0;
+    TR_REQUIRE(a && b && y && sa && sb && inv_so, TNN_ROCM_EINVAL, "add_i8_per_channel: null pointer");
+    TR_REQUIRE(channels >= 1 && inner >= 1, TNN_ROCM_EINVAL, "add_i8_per_channel: channels %d, inner %zu", channels, inner);
+    const int c4        = (channels + 3) / 4 * 4;
+    const int tail_from = c4 % 8 == 4 ? c4 - 4 : c4;
+    hipLaunchKernelGGL(add_i8_per_channel_kernel, dim3(grid_for(n)), dim3(kBlock), 0, (hipStream_t)stream, a, sa, b, sb,
+                       inv_so, y, n, (unsigned)channels, inner, (unsigned)tail_from);
     TR_CHECK_LAUNCH();
     return 0;
 }

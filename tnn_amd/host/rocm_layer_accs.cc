@@ -176,15 +176,43 @@ public:
                 return Status(TNNERR_LAYER_ERR, "int8 element-wise op other than a 2-input Add");
             float s[3];
             Blob *bl[3] = {inputs[0], inputs[1], outputs[0]};
-            for (int i = 0; i < 3; ++i) {
-                auto b8 = dynamic_cast<BlobInt8 *>(bl[i]);
-                if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1)
-                    return Status(TNNERR_LAYER_ERR, "int8 Add needs per-tensor blob scales");
-                s[i] = b8->GetIntResource()->scale_handle.force_to<float *>()[0];
-            }
-            float inv_so = (float)(1.0 / s[2]);  // x86_add_layer_acc.cc:54-58
             const int channels = out_dims.size() > 1 ? out_dims[1] : 1;
             const size_t inner = out_dims.size() > 2 ? (size_t)DimsVectorUtils::Count(out_dims, 2) : 1;
+            bool per_channel = false;
+            const float *hs[3];
+            int ns[3];
+            for (int i = 0; i < 3; ++i) {
+                auto b8 = dynamic_cast<BlobInt8 *>(bl[i]);
+                if (!b8 || !b8->GetIntResource())
+                    return Status(TNNERR_LAYER_ERR, "int8 Add needs blob scales");
+                ns[i] = b8->GetIntResource()->scale_handle.GetDataCount();
+                hs[i] = b8->GetIntResource()->scale_handle.force_to<float *>();
+                if (ns[i] != 1 && ns[i] < channels)
+                    return Status(TNNERR_LAYER_ERR, "int8 Add: a blob has fewer scales than channels");
+                per_channel |= ns[i] != 1;
+                s[i] = hs[i][0];
+            }
+            if (per_channel) {
+                // one scale per channel (dims[1]): the three arrays x86_add_layer_acc.cc:33-66 prepares, kept on the device
+                if (!chan_scale_ || chan_count_ != channels) {
+                    std::vector<float> host(3 * (size_t)channels);
+                    for (int c = 0; c < channels; ++c) {
+                        host[c]                = hs[0][ns[0] == 1 ? 0 : c];
+                        host[channels + c]     = hs[1][ns[1] == 1 ? 0 : c];
+                        host[2 * channels + c] = (float)(1.0 / hs[2][ns[2] == 1 ? 0 : c]);
+                    }
+                    chan_scale_ = nullptr;
+                    RETURN_ON_NEQ(UploadConverted(host.data(), host.size(), DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &chan_scale_), TNN_OK);
+                    chan_count_ = channels;
+                }
+                const float *d = (const float *)chan_scale_;
+                ROCM_CALL(tnn_rocm_add_i8_per_channel(Stream(), (const int8_t *)Ptr(inputs[0]), d, (const int8_t *)Ptr(inputs[1]),
+                                                      d + channels, d + 2 * channels, (int8_t *)Ptr(outputs[0]),
+                                                      (size_t)DimsVectorUtils::Count(out_dims), channels > 0 ? channels : 1,
+                                                      inner > 0 ? inner : 1));
+                return TNN_OK;
+            }
+            float inv_so = (float)(1.0 / s[2]);  // x86_add_layer_acc.cc:54-58
             ROCM_CALL(tnn_rocm_add_i8(Stream(), (const int8_t *)Ptr(inputs[0]), s[0], (const int8_t *)Ptr(inputs[1]), s[1],
                                       inv_so, (int8_t *)Ptr(outputs[0]), (size_t)DimsVectorUtils::Count(out_dims),
                                       channels > 0 ? channels : 1, inner > 0 ? inner : 1));
@@ -229,6 +257,8 @@ public:
 
 private:
     void *weight_ = nullptr;
+    void *chan_scale_ = nullptr;  // int8 Add with per-channel blob scales: a, b scales and reciprocal output scales
+    int chan_count_   = 0;
 };
 typedef RocmBinaryLayerAcc<0> RocmAddLayerAcc;
 typedef RocmBinaryLayerAcc<1> RocmSubLayerAcc;
@@ -277,14 +307,29 @@ public:
             if (offset < 0 || dims_in[i + offset] != dims_s[i])
                 return Status(TNNERR_PARAM_ERR, "LayerNormLayer has invalid dims for input blob");
         param->reduce_dims_size = (int)dims_s.size();  // InferRuntimeOutputShape, cpu_layer_norm_layer_acc.cc:30-61
-        if (scale->GetBlobDesc().data_type != DATA_TYPE_FLOAT || bias->GetBlobDesc().data_type != DATA_TYPE_FLOAT)
-            return Status(TNNERR_LAYER_ERR, "LayerNorm scale/bias must be fp32 on DEVICE_ROCM");
         DataType dt = outputs[0]->GetBlobDesc().data_type;
         if (!IsFloatType(dt))
             return Unsupported("RocmLayerNormLayerAcc", dt);
         int rows = DimsVectorUtils::Count(dims_in, 0, offset), cols = DimsVectorUtils::Count(dims_in, offset);
         if (rows == 0 || cols == 0)
             return Status(TNNERR_COMMON_ERROR, "Error: blob count is zero");
+        // Scale and bias are constants of the model as a rule (kept in fp32, ConstantBlobDataType below).  When they are
+        // ordinary input blobs (the reference's layer test feeds them so, test_layer_norm_layer.cc:70) they carry the
+        // network's float type and are widened into a side buffer of the context first.
+        const float *gamma = (const float *)Ptr(scale), *beta = (const float *)Ptr(bias);
+        const DataType st = scale->GetBlobDesc().data_type, bt = bias->GetBlobDesc().data_type;
+        if (!IsFloatType(st) || !IsFloatType(bt))
+            return Unsupported("RocmLayerNormLayerAcc scale/bias", IsFloatType(st) ? bt : st);
+        if (st != DATA_TYPE_FLOAT || bt != DATA_TYPE_FLOAT) {
+            void *wide = nullptr;
+            RETURN_ON_NEQ(context_->SideBuffer(param_->name + "/layernorm_scale_bias_f32", (size_t)cols * 2 * sizeof(float), &wide),
+                          TNN_OK);
+            float *w = (float *)wide;
+            ROCM_CALL(tnn_rocm_cast(Stream(), (int)st, Ptr(scale), (int)DATA_TYPE_FLOAT, w, (size_t)cols));
+            ROCM_CALL(tnn_rocm_cast(Stream(), (int)bt, Ptr(bias), (int)DATA_TYPE_FLOAT, w + cols, (size_t)cols));
+            gamma = w;
+            beta  = w + cols;
+        }
         // a second output (added by the ROCm int8 pass in place of a following Reformat layer) receives the
         // quantised copy of the first: float2int8(y * float(1.0 / scale)) on the value as stored in the float blob
         // (x86_reformat_layer_acc.cc:66-75, x86_compute_int8.cc:1254-1318)
@@ -297,8 +342,8 @@ public:
             q_inv = (float)(1.0 / b8->GetIntResource()->scale_handle.force_to<float *>()[0]);
             out_q = (int8_t *)Ptr(outputs[1]);
         }
-        ROCM_CALL(tnn_rocm_layernorm(Stream(), (int)dt, Ptr(inputs[0]), nullptr, (const float *)Ptr(scale),
-                                     (const float *)Ptr(bias), Ptr(outputs[0]), rows, cols, param->eps, out_q, q_inv));
+        ROCM_CALL(tnn_rocm_layernorm(Stream(), (int)dt, Ptr(inputs[0]), nullptr, gamma, beta, Ptr(outputs[0]), rows, cols,
+                                     param->eps, out_q, q_inv));
         return TNN_OK;
     }
 
@@ -358,10 +403,34 @@ class RocmReshapeLayerAcc : public RocmLayerAcc {
 public:
     Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
         auto param = dynamic_cast<ReshapeLayerParam *>(param_);
-        if (param && param->reshape_type != 0)
-            return Status(TNNERR_LAYER_ERR, "Reshape type nhwc is not implemented on DEVICE_ROCM");
         size_t bytes = (size_t)DimsVectorUtils::Count(outputs[0]->GetBlobDesc().dims) *
                        DataTypeUtils::GetBytesSize(outputs[0]->GetBlobDesc().data_type);
+        if (param && param->reshape_type == 1) {
+            // The "TensorFlow" reshape (cpu_reshape_layer_acc.cc:101-131): the input, taken as [N,C,H,W], is laid out
+            // channels-last, and that sequence of values, taken as channels-last data of the OUTPUT's [N,C,H,W], is
+            // brought back to channels-first.  Two permutes through the context workspace.
+            auto nchw = [](const DimsVector &d) {
+                return std::vector<int>{d.size() > 0 ? d[0] : 1, d.size() > 1 ? d[1] : 1, d.size() > 2 ? d[2] : 1,
+                                        d.size() > 3 ? d[3] : 1};
+            };
+            const DimsVector od = outputs[0]->GetBlobDesc().dims, id = inputs[0]->GetBlobDesc().dims;
+            if (od.size() > 4 || id.size() > 4)
+                return Status(TNNERR_MODEL_ERR, "Error: RocmReshapeLayerAcc: reshape type 1 does not support dims > 4");
+            if (bytes == 0)
+                return TNN_OK;
+            const int es = DataTypeUtils::GetBytesSize(outputs[0]->GetBlobDesc().data_type);
+            void *tmp    = nullptr;
+            RETURN_ON_NEQ(context_->Workspace(bytes, &tmp), TNN_OK);
+            std::vector<int> in4 = nchw(id), out4 = nchw(od);
+            const int to_last[4]  = {0, 2, 3, 1};
+            ROCM_CALL(tnn_rocm_permute(Stream(), es, Ptr(inputs[0]), tmp, in4.data(), to_last, 4));
+            const int nhwc[4]     = {out4[0], out4[2], out4[3], out4[1]};
+            const int to_first[4] = {0, 3, 1, 2};
+            ROCM_CALL(tnn_rocm_permute(Stream(), es, tmp, Ptr(outputs[0]), nhwc, to_first, 4));
+            return TNN_OK;
+        }
+        if (param && param->reshape_type != 0)
+            return Status(TNNERR_MODEL_ERR, "Error: RocmReshapeLayerAcc: unsupported reshape type");
         if (Ptr(outputs[0]) == Ptr(inputs[0]))
             return TNN_OK;  // the memory planner let the output share the input's buffer: nothing to move
         ROCM_CALL(tnn_rocm_memcpy_d2d(Ptr(outputs[0]), Ptr(inputs[0]), bytes, Stream()));
