@@ -45,7 +45,8 @@ int tnn_host_plan(const char *proto, size_t proto_len, const char *model, size_t
 void tnn_host_destroy(void *handle);
 const char *tnn_host_last_error(void *handle);
 
-/* Instance::SetInputMat (instance.h:123) from a host array.  mat_type: 0 = NCHW_FLOAT (fp32), 1 = NC_INT32.
+/* Instance::SetInputMat (instance.h:123) from a host array.  mat_type: 0 = NCHW_FLOAT (fp32), 1 = NC_INT32,
+ * 2 = RESERVED_INT8_TEST (int8 values copied as they are into an int8 blob, blob_converter_default.cc:190-193).
  * name NULL or "" selects the only input. */
 int tnn_host_set_input(void *handle, const char *name, const void *data, int mat_type, const int *dims, int ndims);
 /* Instance::Forward (instance.h:78): runs every layer and waits for the stream */
@@ -67,6 +68,10 @@ int tnn_host_set_cpu_num_threads(void *handle, int num_threads);
 void *tnn_host_stream(void *handle);
 /* Instance::GetOutputMat (instance.h:128) converted to fp32 NCHW on the host.  dims must hold 8 ints. */
 int tnn_host_get_output(void *handle, const char *name, float *out, size_t capacity, int *dims, int *ndims);
+/* The same through a Mat of the caller's choice (mat_type as for tnn_host_set_input; RESERVED_INT8_TEST hands out an int8
+ * blob's values as they are, blob_converter_default.cc:347-350); capacity in bytes. */
+int tnn_host_get_output_as(void *handle, const char *name, int mat_type, void *out, size_t capacity_bytes, int *dims,
+                           int *ndims);
 
 /* The loop of the engine's benchmark tool (test/test.cc:101-152): `warmup` untimed and `iters` timed iterations of
  * SetInputMat for every input set so far (host copies of those Mats are kept), Forward, GetOutputMat(out_name) as

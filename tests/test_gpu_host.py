@@ -833,3 +833,47 @@ def test_plan_without_device_matches_the_instance():
         assert [l["type"] for l in plan] == types
         for a, b in zip(plan, live):
             assert {k: a[k] for k in b} == b
+
+
+def test_int8_mats_in_and_out_with_per_channel_blob_scales():
+    """The int8 I/O contract of the blob converter (blob_converter_default.cc:190-193, 347-350, 396-403): an int8 Mat
+    (RESERVED_INT8_TEST) is copied as it is into an int8 input blob and out of an int8 output blob; a float Mat goes
+    through the blob's scales, one per channel when the blob has that many.  One quantised InnerProduct over
+    [2, 8, 5, 5] -> [2, 16] with per-channel input and output blob scales, as the reference's int8 layer test builds
+    it; int8 results against the checker bit for bit."""
+    host, tnnmodel, *_ = _mods()
+    say("host: int8 Mats in and out, per-channel blob scales")
+    rng = np.random.default_rng(31)
+    dims, N = [2, 8, 5, 5], 16
+    K = 8 * 5 * 5
+    g = tnnmodel.Graph()
+    g.add_input("input0", dims)
+    g.add_layer("QuantizedInnerProduct", "fc", ["input0"], ["output0"], [N, 1, 0, 1])
+    w = rng.integers(-127, 128, size=(N, K)).astype(np.int8)
+    b = rng.integers(-2000, 2000, size=N).astype(np.int32)
+    w_scale = rng.uniform(0.001, 0.01, size=N).astype(np.float32)
+    s_in = rng.uniform(0.02, 0.05, size=8).astype(np.float32)
+    s_out = rng.uniform(0.5, 1.5, size=N).astype(np.float32)
+    g.res_inner_product("fc", w, b, quant_scale=w_scale)
+    g.res_blob_scale("input0", s_in)
+    g.res_blob_scale("output0", s_out)
+    g.add_output("output0")
+    xq = rng.integers(-128, 128, size=dims).astype(np.int8)
+    want, _ = orc.fc_int8(xq.reshape(2, K), w, b, orc.fc_int8_scale(w_scale, s_out, N))
+    inst = host.RocmInstance.from_graph(g, "fp16")
+    # int8 Mat in, int8 Mat out
+    inst.set_input("input0", xq)
+    inst.forward()
+    got = inst.output_as("output0", np.int8)
+    assert got.shape == (2, N) and np.array_equal(got, want)
+    # the same int8 output through a float Mat: value * its channel's scale
+    assert np.array_equal(inst.output("output0"), want.astype(np.float32) * s_out[None, :])
+    # float Mat in: quantised with the input blob's per-channel scales
+    xf = (xq.astype(np.float32) * s_in[None, :, None, None]).astype(np.float32)
+    inst.set_input("input0", xf)
+    inst.forward()
+    inv = (1.0 / s_in.astype(np.float64)).astype(np.float32)
+    xq2 = orc.float2int8(xf * inv[None, :, None, None])
+    want2, _ = orc.fc_int8(xq2.reshape(2, K), w, b, orc.fc_int8_scale(w_scale, s_out, N))
+    assert np.array_equal(inst.output_as("output0", np.int8), want2)
+    inst.close()

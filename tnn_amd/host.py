@@ -31,6 +31,8 @@ SIGNATURES = {
     "tnn_host_set_cpu_num_threads": (C.c_int, [C.c_void_p, C.c_int]),
     "tnn_host_get_output": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
                                       C.POINTER(C.c_int)]),
+    "tnn_host_get_output_as": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
+                                         C.POINTER(C.c_int)]),
     "tnn_host_time_loop": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_char_p, C.POINTER(C.c_double)]),
     "tnn_host_layer_count": (C.c_int, [C.c_void_p]),
     "tnn_host_layer_summary": (C.c_char_p, [C.c_void_p]),
@@ -53,6 +55,9 @@ def load():
             fn.restype, fn.argtypes = res, args
         _lib = lib
     return _lib
+
+
+_MAT_CODE = {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.int8): 2}
 
 
 class HostError(RuntimeError):
@@ -143,11 +148,11 @@ class RocmInstance:
 
     def set_input(self, name, arr):
         a = np.ascontiguousarray(arr)
-        if a.dtype not in (np.float32, np.int32):
-            raise TypeError("inputs are fp32 (NCHW_FLOAT) or int32 (NC_INT32) host arrays")
+        if a.dtype not in (np.float32, np.int32, np.int8):
+            raise TypeError("inputs are fp32 (NCHW_FLOAT), int32 (NC_INT32) or int8 (RESERVED_INT8_TEST) host arrays")
         dims = (C.c_int * max(a.ndim, 1))(*a.shape)
         self._check(load().tnn_host_set_input(self._h, name.encode(), a.ctypes.data_as(C.c_void_p),
-                                              1 if a.dtype == np.int32 else 0, dims, a.ndim), "SetInputMat")
+                                              _MAT_CODE[a.dtype], dims, a.ndim), "SetInputMat")
 
     def forward(self):
         self._check(load().tnn_host_forward(self._h), "Forward")
@@ -190,6 +195,17 @@ class RocmInstance:
         nd = C.c_int(0)
         self._check(load().tnn_host_get_output(self._h, name.encode(), buf.ctypes.data_as(C.c_void_p), max_elems, dims,
                                                C.byref(nd)), "GetOutputMat")
+        shape = [dims[i] for i in range(nd.value)]
+        return buf[:int(np.prod(shape, dtype=np.int64))].reshape(shape).copy()
+
+    def output_as(self, name, dtype, max_elems=1 << 25):
+        """the output through a Mat of the given numpy type: float32, int32, or int8 (an int8 blob's values as they are)"""
+        dtype = np.dtype(dtype)
+        buf = np.empty(max_elems, dtype)
+        dims = (C.c_int * 8)()
+        nd = C.c_int(0)
+        self._check(load().tnn_host_get_output_as(self._h, name.encode(), _MAT_CODE[dtype], buf.ctypes.data_as(C.c_void_p),
+                                                  buf.nbytes, dims, C.byref(nd)), "GetOutputMat")
         shape = [dims[i] for i in range(nd.value)]
         return buf[:int(np.prod(shape, dtype=np.int64))].reshape(shape).copy()
 

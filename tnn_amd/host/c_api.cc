@@ -130,17 +130,21 @@ HOST_API int tnn_host_reshape(void *hp, int n_inputs, const char *const *names, 
 HOST_API void tnn_host_destroy(void *hp) { delete static_cast<Handle *>(hp); }
 HOST_API const char *tnn_host_last_error(void *hp) { return static_cast<Handle *>(hp)->err.c_str(); }
 
-// mat_type: 0 NCHW_FLOAT (fp32 host data), 1 NC_INT32
+// mat_type: 0 NCHW_FLOAT (fp32 host data), 1 NC_INT32, 2 RESERVED_INT8_TEST (int8 host data, copied as it is into an
+// int8 blob: blob_converter_default.cc:190-193, 347-350)
+static MatType MatTypeOf(int code) { return code == 1 ? NC_INT32 : (code == 2 ? RESERVED_INT8_TEST : NCHW_FLOAT); }
+static size_t MatElemBytes(int code) { return code == 2 ? 1 : 4; }
+
 HOST_API int tnn_host_set_input(void *hp, const char *name, const void *data, int mat_type, const int *dims, int ndims) {
     auto h = static_cast<Handle *>(hp);
     DimsVector d(dims, dims + ndims);
-    auto mat  = std::make_shared<Mat>(DEVICE_NAIVE, mat_type == 1 ? NC_INT32 : NCHW_FLOAT, d, const_cast<void *>(data));
+    auto mat  = std::make_shared<Mat>(DEVICE_NAIVE, MatTypeOf(mat_type), d, const_cast<void *>(data));
     Status st = h->inst->SetInputMat(mat, MatConvertParam(), name ? name : "");
     if (st != TNN_OK)
         return fail(h, st);
     auto keep = std::make_shared<Mat>(DEVICE_NAIVE, mat->GetMatType(), d);  // owns its memory
     if (keep->GetData() && data)
-        memcpy(keep->GetData(), data, (size_t)DimsVectorUtils::Count(d) * 4);
+        memcpy(keep->GetData(), data, (size_t)DimsVectorUtils::Count(d) * MatElemBytes(mat_type));
     h->inputs[name ? name : ""] = keep;
     return 0;
 }
@@ -260,6 +264,29 @@ HOST_API int tnn_host_get_output(void *hp, const char *name, float *out, size_t 
         return -2;
     }
     memcpy(out, mat->GetData(), count * sizeof(float));
+    return 0;
+}
+
+// GetOutputMat through a Mat of the caller's choice (codes of tnn_host_set_input); capacity in bytes
+HOST_API int tnn_host_get_output_as(void *hp, const char *name, int mat_type, void *out, size_t capacity_bytes, int *dims,
+                                    int *ndims) {
+    auto h = static_cast<Handle *>(hp);
+    std::shared_ptr<Mat> mat;
+    Status st = h->inst->GetOutputMat(mat, MatConvertParam(), name ? name : "", DEVICE_NAIVE, MatTypeOf(mat_type));
+    if (st != TNN_OK)
+        return fail(h, st);
+    DimsVector d = mat->GetDims();
+    size_t bytes = (size_t)DimsVectorUtils::Count(d) * MatElemBytes(mat_type);
+    if (ndims)
+        *ndims = (int)d.size();
+    if (dims)
+        for (size_t i = 0; i < d.size() && i < 8; ++i)
+            dims[i] = d[i];
+    if (bytes > capacity_bytes) {
+        h->err = "output buffer too small";
+        return -2;
+    }
+    memcpy(out, mat->GetData(), bytes);
     return 0;
 }
 

@@ -381,7 +381,29 @@ public:
             auto bi = dynamic_cast<BlobInt8 *>(blob_);
             if (!bi || !bi->GetIntResource() || bi->GetIntResource()->scale_handle.GetDataCount() < 1)
                 return Status(TNNERR_NULL_PARAM, "int8 blob without scale resource");
-            float s   = bi->GetIntResource()->scale_handle.force_to<float *>()[0];
+            const int n_scale = bi->GetIntResource()->scale_handle.GetDataCount();
+            const float *sc   = bi->GetIntResource()->scale_handle.force_to<float *>();
+            if (n_scale > 1) {
+                // one scale per channel (dims[1]), NaiveQuantBias's indexing (naive_compute.cc:1671-1690): a rare path
+                // (model inputs are per-tensor as a rule), quantised on the host with the device quantiser's arithmetic
+                // (multiply by float(1.0 / scale), add +-0.5, truncate, clamp) and copied as int8
+                const int ch    = desc.dims.size() > 1 ? desc.dims[1] : 1;
+                const size_t hw = (size_t)std::max(1, DimsVectorUtils::Count(desc.dims, 2));
+                if (n_scale < ch)
+                    return Status(TNNERR_PARAM_ERR, "int8 blob with fewer scales than channels");
+                std::vector<int8_t> qv(count);
+                for (size_t i = 0; i < count; ++i) {
+                    const float s = sc[(i / hw) % (size_t)ch];
+                    float v       = s != 0.f ? src[i] * (float)(1.0 / s) : 0.f;
+                    v             = v < 0.f ? v - 0.5f : v + 0.5f;
+                    v             = v > 127.f ? 127.f : (v < -128.f ? -128.f : v);
+                    qv[i]         = (int8_t)(int)v;
+                }
+                ROCM_CALL(tnn_rocm_memcpy_h2d(dst, qv.data(), count, q));
+                ROCM_CALL(tnn_rocm_stream_sync(q));  // the host vector goes away with this call
+                return TNN_OK;
+            }
+            float s   = sc[0];
             float inv = (float)(1.0 / s);
             ROCM_CALL(tnn_rocm_quantize(q, TNN_ROCM_F32, staging_, inv, (int8_t *)dst, count));
         } else {
@@ -422,7 +444,26 @@ public:
                 auto bi = dynamic_cast<BlobInt8 *>(blob_);
                 if (!bi || !bi->GetIntResource() || bi->GetIntResource()->scale_handle.GetDataCount() < 1)
                     return Status(TNNERR_NULL_PARAM, "int8 blob without scale resource");
-                float s = bi->GetIntResource()->scale_handle.force_to<float *>()[0];
+                const int n_scale = bi->GetIntResource()->scale_handle.GetDataCount();
+                const float *sc   = bi->GetIntResource()->scale_handle.force_to<float *>();
+                if (n_scale > 1) {  // per-channel scales: NaiveDequant's indexing (naive_compute.cc:1617-1633), on the host
+                    const int ch    = desc.dims.size() > 1 ? desc.dims[1] : 1;
+                    const size_t hw = (size_t)std::max(1, DimsVectorUtils::Count(desc.dims, 2));
+                    if (n_scale < ch)
+                        return Status(TNNERR_PARAM_ERR, "int8 blob with fewer scales than channels");
+                    std::vector<int8_t> qv(count);
+                    RETURN_ON_NEQ(ToHost(qv.data(), src, count, q), TNN_OK);
+                    float *out = (float *)mat.GetData();
+                    for (size_t i = 0; i < count; ++i)
+                        out[i] = sc[(i / hw) % (size_t)ch] * (float)qv[i];
+                    if (NeedsScaleBias(param, desc.dims)) {
+                        std::vector<float> tmp(count);
+                        ApplyScaleBias(out, tmp.data(), desc.dims, param);
+                        memcpy(out, tmp.data(), count * 4);
+                    }
+                    return TNN_OK;
+                }
+                float s = sc[0];
                 ROCM_CALL(tnn_rocm_dequantize(q, (const int8_t *)src, s, TNN_ROCM_F32, staging_, count));
             } else {
                 return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported blob data type");
