@@ -172,6 +172,26 @@ REF_API int tnn_ref_get_output_as(void *h, const char *name, int mat_type, void 
     return 0;
 }
 
+#if TNN_PROFILE
+// A profiler build of the engine only: Instance::StartProfile, `forwards` Forward calls, Instance::FinishProfile
+// (instance.cc:321-340); the report (the per-layer table and the per-type summary of core/profile.cc:111-201) is
+// copied into buf.  Returns 0, or the failing Forward's status.
+REF_API int tnn_ref_profile(void *h, int forwards, char *buf, size_t buf_len) {
+    Session *s = static_cast<Session *>(h);
+    s->inst->StartProfile();
+    for (int i = 0; i < forwards; ++i) {
+        Status st = s->inst->Forward();
+        if (st != TNN_OK) {
+            s->err = st.description();
+            s->inst->FinishProfile(false);
+            return (int)st;
+        }
+    }
+    put_err(buf, buf_len, s->inst->FinishProfile(false));
+    return 0;
+}
+#endif
+
 REF_API const char *tnn_ref_last_error(void *h) { return static_cast<Session *>(h)->err.c_str(); }
 
 // Mean wall time (seconds) of `iters` Forward() calls after `warmup` untimed ones.

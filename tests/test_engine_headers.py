@@ -35,6 +35,18 @@ def test_backend_source_compiles_against_engine_headers(src, std):
     assert r.returncode == 0 and not errors, "\n".join(errors[:20]) or r.stderr[-2000:]
 
 
+@pytest.mark.parametrize("src", BACKEND_SOURCES)
+def test_backend_source_compiles_in_a_profiler_build_of_the_engine(src):
+    """-DTNN_PROFILE (the engine's TNN_PROFILER_ENABLE option, CMakeLists.txt:74-76) adds StartProfile / FinishProfile /
+    AddProfilingData to Context and the networks; the backend's per-layer timing (RocmNetwork::ProfiledForward) only
+    exists in that form"""
+    cmd = ["g++", "-std=c++11", "-fsyntax-only", "-DTNN_ROCM_ENGINE_TREE", "-DTNN_PROFILE", "-I" + os.path.join(REF, "include"),
+           "-I" + os.path.join(REF, "source"), "-I" + os.path.join(ROOT, "include"), "-I" + HOST, os.path.join(HOST, src)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    errors = [l for l in r.stderr.splitlines() if " error" in l]
+    assert r.returncode == 0 and not errors, "\n".join(errors[:20]) or r.stderr[-2000:]
+
+
 def test_backend_sources_do_not_include_the_restated_contract_in_engine_form():
     """in the engine form nothing of tnn_host.h may be reachable: the only headers of this repository the backend
     pulls in are its own rocm_*.h and the C ABI"""

@@ -19,6 +19,13 @@ RocmNetwork::~RocmNetwork() {
     if (context_)
         context_->Synchronize();
     DropGraphs();
+    DropProfileEvents();
+}
+
+void RocmNetwork::DropProfileEvents() {
+    for (void *e : profile_events_)
+        tnn_rocm_event_destroy(e);
+    profile_events_.clear();
 }
 
 void RocmNetwork::DropGraphs() {
@@ -86,6 +93,52 @@ Status RocmNetwork::InitLayers(NetStructure *net_structure, NetResource *net_res
 }
 #endif
 
+#if defined(TNN_ROCM_ENGINE_TREE) && TNN_PROFILE
+// The engine's forward loop (default_network.cc:558-635) with a hipEvent pair around each layer; after the one
+// synchronisation at the end every layer's ProfilingData (name, op type, dims, kernel time in ms: the fields
+// AbstractLayerAcc::UpdateProfilingData fills, abstract_layer_acc.cc:102-125) goes to Context::AddProfilingData, from
+// where Instance::FinishProfile prints the tables of core/profile.cc:111-201.
+Status RocmNetwork::ProfiledForward() {
+    RETURN_ON_NEQ(blob_manager_->CheckBlobMemoryState(), TNN_OK);
+    if (runtime_blob_pool_)
+        runtime_blob_pool_->ClearBlobMemoryPool();
+    void *stream = nullptr;
+    context_->GetCommandQueue(&stream);
+    while (profile_events_.size() < 2 * layers_.size()) {
+        void *e = nullptr;
+        if (tnn_rocm_event_create(&e) != 0)
+            return Status(TNNERR_CUDA_TENSORRT_ERROR, std::string("event create failed: ") + tnn_rocm_last_error());
+        profile_events_.push_back(e);
+    }
+    RETURN_ON_NEQ(context_->OnInstanceForwardBegin(), TNN_OK);
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        tnn_rocm_event_record(profile_events_[2 * i], stream);
+        Status st = layers_[i]->Forward();
+        tnn_rocm_event_record(profile_events_[2 * i + 1], stream);
+        if (st != TNN_OK)
+            return st;
+    }
+    context_->OnInstanceForwardEnd();
+    RETURN_ON_NEQ(context_->Synchronize(), TNN_OK);
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        auto pdata = std::make_shared<ProfilingData>();
+        pdata->layer_name = layers_[i]->GetLayerName();
+        if (i < net_structure_->layers.size() && net_structure_->layers[i])
+            pdata->op_name = net_structure_->layers[i]->type_str;
+        const auto ins = layers_[i]->GetInputBlobs(), outs = layers_[i]->GetOutputBlobs();
+        if (!ins.empty())
+            pdata->input_dims = ins[0]->GetBlobDesc().dims;
+        if (!outs.empty())
+            pdata->output_dims = outs[0]->GetBlobDesc().dims;
+        float ms = 0.f;
+        tnn_rocm_event_elapsed_ms(profile_events_[2 * i], profile_events_[2 * i + 1], &ms);
+        pdata->kernel_time = ms;
+        context_->AddProfilingData(pdata);
+    }
+    return TNN_OK;
+}
+#endif
+
 Status RocmNetwork::Forward() {
     RETURN_ON_NEQ(RocmNetwork::ForwardAsync(nullptr), TNN_OK);
     return context_->Synchronize();
@@ -95,7 +148,14 @@ Status RocmNetwork::ForwardAsync(Callback call_back) {
     void *stream = nullptr;
     context_->GetCommandQueue(&stream);
 #ifdef TNN_ROCM_ENGINE_TREE
-    const bool profiling = false;  // a TNN_PROFILE build times layers through the context; build it with TNN_ROCM_GRAPH=0
+#if TNN_PROFILE
+    // a profiler build of the engine (TNN_PROFILER_ENABLE): between Instance::StartProfile and FinishProfile every layer
+    // is timed with an event pair and reported to the context, as the engine's own accs do around their DoForward
+    // (x86_layer_acc.cc:55-72); no graph replay then - a replayed graph has no layer boundaries on the host
+    if (context_->profile_layer)
+        return ProfiledForward();
+#endif
+    const bool profiling = false;
 #else
     const bool profiling = profiling_;
 #endif

@@ -28,6 +28,9 @@ protected:
     // at once for a device it does not know; this override does that pass for DEVICE_ROCM and then runs the engine's
     // own InitLayers.
     Status InitLayers(NetStructure *net_structure, NetResource *net_resource) override;
+#if TNN_PROFILE
+    Status ProfiledForward();  // the forward loop with every layer timed (a profiler build of the engine)
+#endif
 #endif
 
 private:
@@ -36,6 +39,8 @@ private:
     // re-planned blob pool or a grown workspace lead back to eager passes and a new recording by themselves.
     void Signature(std::vector<uint64_t> *sig);
     void DropGraphs();
+    void DropProfileEvents();
+    std::vector<void *> profile_events_;  // two per layer, created at the first profiled forward
     struct Recording {
         std::vector<uint64_t> signature;
         void *exec = nullptr;
