@@ -225,6 +225,13 @@ def main():
                 "frac": round(opsn / (ms * 1e-3) / 1e12 / 5000.0, 4), "traffic": None,
                 "us_per_launch": round(ms * 1e3, 2), "ops_per_launch": opsn}
 
+    # the dominant GEMM inside the forward: the event pair the eager layer loop puts around its layer (profile pass above),
+    # averaged over the layers.  It spans from the previous layer's last kernel to this layer's last kernel on the
+    # stream, i.e. the kernel plus the gap in front of it with the weights as the previous layers left them in the
+    # caches; the eager loop's host-side launch cost can widen that gap, which a graph replay does not pay.  The QKV
+    # projection shares its layer with the attention kernel and has no figure of its own.
+    dom_in_forward_ms = breakdown[dominant] / cfg.layers if dominant in breakdown else None
+
     roof_i8 = int8_roofline()
     attn_here = attention_tflops(B, S, lens)
     stress_lens = np.random.default_rng(20240603).integers(16, 513, 32)
@@ -263,7 +270,15 @@ def main():
                      "achieved": round(achieved, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
                      "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get(dominant) if full_cfg else None,
+                     "traffic_source": ("profiles/bench_c2_bert_base_b8_s384_hbm_traffic_counters.txt: rocprofv3 --pmc "
+                                        "FETCH_SIZE and WRITE_SIZE runs of this command, typed into bench.py, not "
+                                        "measured by this run") if full_cfg else None,
                      "us_per_launch": round(dom_ms * 1e3, 2),
+                     "us_in_forward": None if dom_in_forward_ms is None else round(dom_in_forward_ms * 1e3, 2),
+                     "frac_in_forward": None if dom_in_forward_ms is None else round(
+                         gemm_flops[dominant] / (dom_in_forward_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 4),
+                     "in_forward_is": "this GEMM's layer between the event pair of the eager layer loop, mean over the "
+                                      "layers: kernel + the gap in front of it (frac stays on the back-to-back figure)",
                      "timed_over": "%d back-to-back launches between two events on the launch stream, right after "
                                    "the timed region (which replays a captured graph)" % n_gemm,
                      "flops_per_launch": gemm_flops[dominant],

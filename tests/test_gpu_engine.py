@@ -247,3 +247,20 @@ def test_profiler_build_of_the_engine_reports_every_layer():
         assert layer["name"] in table, layer["name"]
     for type_str in ("RocmFusedAttention", "RocmFusedLinear", "RocmFusedEmbedding", "LayerNorm"):
         assert type_str in table, type_str
+
+
+def test_model_input_shared_by_quantised_and_float_layers():
+    """A model input that a quantised layer and a float layer both read (the head-of-graph Reformat case of
+    net_optimizer_insert_int8_reformat.cc:84-131): DEVICE_ROCM in the reference engine against its DEVICE_X86, whose
+    quantiser forms the backend follows, value for value in fp32 blobs."""
+    engine()
+    from test_host_plan import _input_read_by_both_kinds
+    say("reference engine: model input read by quantised and float layers")
+    g = _input_read_by_both_kinds()
+    x = (np.random.default_rng(3).standard_normal((64, 128)) * 0.8).astype(np.float32)
+    x86 = run(g, "X86", {"x": x}, "z")[0]
+    rocm = run(g, "ROCM:fp32", {"x": x}, "z", forwards=4)
+    assert all(np.array_equal(o, rocm[0]) for o in rocm[1:])
+    d = np.abs(rocm[0] - x86)
+    say("  max |d| vs DEVICE_X86 %.3g (one int8 step of the output scale is 0.05)" % d.max())
+    assert d.max() <= 1e-6

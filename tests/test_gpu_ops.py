@@ -102,6 +102,15 @@ def test_gelu_fp16():
     sp = np.array([0.0, np.inf, 40.0, -40.0, 65504.0, -65504.0], np.float32)
     got = host(ops().gelu(dev(sp, torch.float16)))
     assert got.tolist() == [0.0, np.inf, 40.0, 0.0, 65504.0, 0.0]
+    # a NaN stays a NaN (an overflow upstream must not turn into zeros), in every float type and in the GEMM epilogue
+    for td in (torch.float32, torch.float16, torch.bfloat16):
+        got = host(ops().gelu(dev(np.array([np.nan, 1.0, -np.inf], np.float32), td)))
+        assert np.isnan(got[0]) and abs(got[1] - 0.8413) < 5e-3 and np.isnan(got[2]), (td, got)
+    a = torch.zeros(64, 64, dtype=torch.float16, device="cuda")
+    a[3, 5] = float("nan")
+    w = torch.eye(64, dtype=torch.float16, device="cuda")
+    y = host(ops().gemm(a, w, True, bias=torch.zeros(64, device="cuda"), gelu=True))
+    assert np.isnan(y[3]).any() and not np.isnan(np.delete(y, 3, axis=0)).any()
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 8), (5, 768), (33, 1024), (7, 100), (3, 5000), (4096, 768)])
@@ -305,6 +314,10 @@ def test_quantize_bit_exact(scale):
                         np.array([0.0, -0.0, 1e30, -1e30], np.float32)])
     got = host(ops().quantize(dev(x), float(inv)))
     assert np.array_equal(got, orc.quantize_x86(x, scale))
+    # values no sane activation holds, pinned so that a change shows: infinities saturate, a NaN becomes -128 (what the
+    # reference's x86 quantiser makes of it: INT_MIN out of the truncating conversion, then the saturating pack)
+    got = host(ops().quantize(dev(np.array([np.inf, -np.inf, np.nan], np.float32)), float(inv)))
+    assert got.tolist() == [127, -128, -128]
 
 
 def test_dequantize_and_add_i8_bit_exact():
@@ -1087,6 +1100,56 @@ def test_gemm_layernorm_folded_into_projection(M, dtype):
         fed_q = o.qkv_split_ln(c, wqf.cuda(), dev(bqf), dev(csq), eps, B, S, heads, want_stats=True, row_sums=(sums, blocks))
         assert rel_err(host(fed_q[0]), host(own_q[0])) <= 2e-3 and rel_err(host(fed_q[1]), host(own_q[1])) <= 2e-3
         assert np.abs(host(fed_q[2])[:, 0] / host(own_q[2])[:, 0] - 1).max() <= 1e-5
+
+
+@pytest.mark.parametrize("blocks", [4, 12, 16, 24])
+@pytest.mark.parametrize("offset_rows", [False, True])
+def test_folding_gemm_fed_row_sums_against_own_statistics(blocks, offset_rows):
+    """A LayerNorm-folding GEMM that is handed its rows' sums per block of columns (made here on the host, so the block
+    count is free: up to twelve blocks the kernels request them late, above that the shapes that share a CU request them
+    ahead of their first slabs) against the same GEMM taking the statistics from its own operand: FFN1-shaped
+    (192x192 tiles) and QKV-shaped (128x128 tiles) at M = 3072.  offset_rows: every row sits at 20 +- 0.1, where
+    E[x^2] - mean^2 loses most of its digits in fp32 block sums and must still not go negative."""
+    say("folding GEMM, fed row sums, %d blocks%s" % (blocks, ", offset rows" if offset_rows else ""))
+    o = ops()
+    rng = np.random.default_rng(100 + blocks)
+    M, H, F, B, S, heads = 3072, 768, 3072, 8, 384, 12
+    eps = 1e-12
+    t = rng.standard_normal((M, H)).astype(np.float32)
+    if offset_rows:
+        t = (20.0 + 0.1 * t).astype(np.float32)
+    t16 = torch.from_numpy(t).half()
+    tf = t16.float().numpy().astype(np.float64)
+    per = tf.reshape(M, blocks, H // blocks)
+    sums = np.zeros((o.MAX_ROW_SUM_BLOCKS, M, 2), np.float32)
+    sums[:blocks, :, 0] = per.sum(2).T
+    sums[:blocks, :, 1] = (per ** 2).sum(2).T
+    g, be = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32), (0.1 * rng.standard_normal(H)).astype(np.float32)
+    w1, b1 = (rng.standard_normal((F, H)) * 0.03).astype(np.float32), (rng.standard_normal(F) * 0.1).astype(np.float32)
+    wq, bq = (rng.standard_normal((3 * H, H)) * 0.03).astype(np.float32), (rng.standard_normal(3 * H) * 0.1).astype(np.float32)
+    w1f, cs1, b1f = _fold_ln_weights(w1, b1, g, be, torch.float16)
+    wqf, csq, bqf = _fold_ln_weights(wq, bq, g, be, torch.float16)
+    c, dsums = t16.cuda(), dev(sums)
+    own_h, own_st = o.gemm_ln(c, w1f.cuda(), dev(b1f), dev(cs1), eps, gelu=True, want_stats=True)
+    fed_h, fed_st = o.gemm_ln(c, w1f.cuda(), dev(b1f), dev(cs1), eps, gelu=True, want_stats=True, row_sums=(dsums, blocks))
+    own_q = o.qkv_split_ln(c, wqf.cuda(), dev(bqf), dev(csq), eps, B, S, heads, want_stats=True)
+    fed_q = o.qkv_split_ln(c, wqf.cuda(), dev(bqf), dev(csq), eps, B, S, heads, want_stats=True, row_sums=(dsums, blocks))
+    mean = tf.mean(1)
+    rstd = 1.0 / np.sqrt(tf.var(1) + eps)
+    # with rows at 20 +- 0.1 the variance is 1e-2 out of E[x^2] = 400: fp32 sums of squares leave it ~3 digits
+    rtol = 3e-3 if offset_rows else 1e-5
+    for st in (fed_st, fed_q[2]):
+        st = host(st)
+        assert np.isfinite(st).all()
+        assert np.abs(st[:, 0] / rstd - 1).max() <= rtol and np.abs(st[:, 1] - mean).max() <= 1e-5 * max(1.0, np.abs(mean).max())
+    if not offset_rows:
+        assert np.abs(host(fed_st)[:, 0] / host(own_st)[:, 0] - 1).max() <= 1e-5
+        assert rel_err(host(fed_h), host(own_h)) <= 2e-3
+        assert rel_err(host(fed_q[0]), host(own_q[0])) <= 2e-3 and rel_err(host(fed_q[1]), host(own_q[1])) <= 2e-3
+    else:
+        assert np.isfinite(host(fed_h)).all() and np.isfinite(host(fed_q[0])).all()
+        ref = orc.gelu(orc.inner_product(orc.layernorm(tf.astype(np.float32), g, be, eps), w1f.float().numpy() / g[None, :], b1))
+        assert rel_err(host(fed_h), ref) <= 3e-2     # three digits of rstd, then a 768-term product
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])

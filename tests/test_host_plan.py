@@ -254,3 +254,33 @@ def test_attention_lookalike_stays_decomposed(name):
     t = _types(plan)
     assert "RocmFusedAttention" not in t and t["Softmax"] == 1 and t["MatMul"] == 2 and t["Permute"] == 4, (name, t)
     assert t["RocmFusedLinear"] == 4
+
+
+def _input_read_by_both_kinds(T=64, K=128, N=128, seed=5):
+    """x feeds a quantised InnerProduct and, as a residual, a float Add: the model-input case of the engine's Reformat
+    insertion (net_optimizer_insert_int8_reformat.cc:84-131)"""
+    rng = np.random.default_rng(seed)
+    g = tnnmodel.Graph()
+    one = np.array([1.0], np.float32)
+    g.add_input("x", [T, K])
+    g.add_layer("QuantizedInnerProduct", "fc", ["x"], ["yq"], [N, 1, 0, 1])
+    w = rng.integers(-127, 128, size=(N, K)).astype(np.int8)
+    g.res_inner_product("fc", w, rng.integers(-500, 500, size=N).astype(np.int32),
+                        quant_scale=rng.uniform(1e-3, 2e-3, size=N).astype(np.float32))
+    g.res_blob_scale("x", np.float32(0.03))
+    g.res_blob_scale("yq", np.float32(0.05))
+    g.add_layer("Mul", "out_copy", ["yq"], ["y"], [1])
+    g.res_eltwise("out_copy", "Mul", one)
+    g.add_layer("Add", "res", ["y", "x"], ["z"], [1])
+    g.add_output("z")
+    return g
+
+
+def test_model_input_read_by_quantised_and_float_layers_gets_a_reformat_at_the_head():
+    plan = host.plan(_input_read_by_both_kinds(), precision="fp32")
+    assert plan[0]["type"] == "Reformat" and plan[0]["inputs"] == ["x"]
+    assert plan[0]["name"] == "x_int8_reformat__from_model_input__"
+    by_name = {l["name"]: l for l in plan}
+    fc = [l for l in plan if "fc" in l["name"]][0]
+    assert fc["inputs"][0] == "x_int8_reformat"            # the quantised reader takes the int8 copy ...
+    assert "x" in by_name["res"]["inputs"]                 # ... the float reader the model input itself

@@ -47,12 +47,13 @@ template <> struct AttnT<TNN_ROCM_F16> {
     // Written as an instruction because the compiler only emits the form whose destination is also the C operand and
     // copies c0 into d first (16 moves per chain).  The early-clobber output keeps d apart from the inputs.  The compiler
     // does not look inside the statement, so it inserts none of the wait states an instruction that reads d right
-    // after a matrix instruction needs (none for an accumulating MFMA of the same opcode into d, but up to 19 for a
-    // vector instruction or an MFMA with another destination): the statement carries them itself, so that whatever
-    // the compiler schedules next is safe.  They pass while the matrix pipe works on this product.
+    // after a matrix instruction needs (none for an accumulating MFMA of the same opcode into d; passes + 3 = 11 for a
+    // vector instruction and passes + 2 for an MFMA with another destination, this product taking 8 passes of 4
+    // clocks): the statement carries them itself, so that whatever the compiler schedules next is safe.  They pass
+    // while the matrix pipe works on this product.
     template <typename V> static __device__ __forceinline__ f32x16 mma_from(const V &a, const V &b, const f32x16 &c0) {
         f32x16 d;
-        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3\n\ts_nop 15\n\ts_nop 3" : "=&v"(d) : "v"(a), "v"(b), "v"(c0));
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3\n\ts_nop 10" : "=&v"(d) : "v"(a), "v"(b), "v"(c0));
         return d;
     }
     static __device__ __forceinline__ float to_float(uint16_t bits) { return (float)__builtin_bit_cast(half_t, bits); }
@@ -88,7 +89,7 @@ template <> struct AttnT<TNN_ROCM_BF16> {
     }
     template <typename V> static __device__ __forceinline__ f32x16 mma_from(const V &a, const V &b, const f32x16 &c0) {
         f32x16 d;
-        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3\n\ts_nop 15\n\ts_nop 3" : "=&v"(d) : "v"(a), "v"(b), "v"(c0));
+        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3\n\ts_nop 10" : "=&v"(d) : "v"(a), "v"(b), "v"(c0));
         return d;
     }
     static __device__ __forceinline__ float to_float(uint16_t bits) { return __uint_as_float((uint32_t)bits << 16); }

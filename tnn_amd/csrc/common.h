@@ -122,7 +122,9 @@ template <> struct Elem<TNN_ROCM_BF16> {
 // rounding), clamp in fp32, truncate.  The translation units are compiled with -ffp-contract=off
 // so the add is never fused with the multiply that produced v.
 // (+-0.5 taken from the sign bit and the clamp as one med3 give the same result for every value that is not a NaN --
-// -0.0 lands on 0 either way -- in three instructions instead of seven.)
+// -0.0 lands on 0 either way -- in three instructions instead of seven.  A NaN comes out as -128: the median of three
+// with a NaN operand is the minimum of the other two, and -128 is also what the reference's x86 path makes of a NaN,
+// whose truncating conversion yields INT_MIN before the saturating pack, x86_compute_int8.cc:31-39.)
 __device__ __forceinline__ int8_t float2int8_ref(float v) {
     float t = __fadd_rn(v, __builtin_copysignf(0.5f, v));
     t       = __builtin_amdgcn_fmed3f(t, -128.0f, 127.0f);
@@ -147,12 +149,13 @@ __device__ __forceinline__ float gelu_erf(float x) {
 // exp2, one max and the final multiply-add: 13 issue slots against 19 for the rational form 7.1.26 of Abramowitz &
 // Stegun used before and ~40 for erff.  Against the correctly rounded fp16 result 0.4 % of the values differ, by one
 // ulp (2.8 % for the rational form).  fp32 outputs keep gelu_erf.
-// max(x, 0) as the one instruction it is: written as fmaxf or as a median with +inf the compiler puts a quieting
-// v_max_f32 x, x in front of it
+// max(x, 0) is formed as x/2 + |x/2|: exact for every finite x (halving and the sum of equal or opposite halves do not
+// round), and unlike the maximum instruction, which returns its other operand for a NaN, it hands a NaN through, as the
+// reference's GELU does (and gives NaN for -inf, where the reference's 0.5 x (erf + 1) is -inf times 0).  An overflow
+// upstream therefore stays visible in the output instead of turning into zeros.
 __device__ __forceinline__ float max_with_zero(float x) {
-    float r;
-    asm("v_max_f32 %0, 0, %1" : "=v"(r) : "v"(x));
-    return r;
+    const float h = __fmul_rn(0.5f, x);
+    return __fadd_rn(h, fabsf(h));
 }
 
 __device__ __forceinline__ float gelu_erf_fast(float x) {

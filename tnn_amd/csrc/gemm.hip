@@ -1141,23 +1141,24 @@ __global__ void __launch_bounds__(CFG::NT)
                         else
                             TR_WAIT_VMCNT(0);
                     }
-                    // The other waves wait at a barrier while these do this, so it is kept short: the block sums (fp32
-                    // already) are added in fp32 in a fixed order, only the variance is formed as a difference of
-                    // doubles, and its reciprocal root is taken in single precision with one Newton step.
-                    float f1 = 0.f, f2 = 0.f;
+                    // The other waves wait at a barrier while these do this, so it is kept short: the block sums (fp32)
+                    // are added up in double in a fixed order (the sum of squares of a row that sits far from zero
+                    // would lose the variance's digits in fp32), the variance is formed as a difference of doubles,
+                    // and its reciprocal root is taken in single precision with one Newton step.
+                    double f1 = 0.0, f2 = 0.0;
 #pragma unroll
                     for (int q = 0; q < NSUM; ++q) {
                         if constexpr (!kLateSums)
                             asm volatile("" : "+v"(early[q]));  // not to be read before the wait above
                         if (q < epi.ln.sum_blocks) {
-                            f1 += early[q].x;
-                            f2 += early[q].y;
+                            f1 += (double)early[q].x;
+                            f2 += (double)early[q].y;
                         }
                     }
-                    const double mean = (double)f1 * (double)epi.ln.inv_cols;
+                    const double mean = f1 * (double)epi.ln.inv_cols;
                     // fp32 block sums can leave E[x^2] - mean^2 a hair below zero for rows whose spread is tiny next to
                     // their mean; the variance is clamped there (with eps = 1e-12 the root would otherwise be NaN)
-                    const double var  = (double)f2 * (double)epi.ln.inv_cols - mean * mean;
+                    const double var  = f2 * (double)epi.ln.inv_cols - mean * mean;
                     const float ve    = (float)((var > 0.0 ? var : 0.0) + (double)epi.ln.eps);
                     float r           = __builtin_amdgcn_rsqf(ve);
                     r                 = r * (1.5f - 0.5f * ve * r * r);

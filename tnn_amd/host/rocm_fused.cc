@@ -867,6 +867,64 @@ public:
             return TNN_OK;
         std::vector<std::shared_ptr<LayerInfo>> out;
         const int count = (int)layers.size();
+        // the Reformat layer behind `producer` (a layer, or a stand-in for a model input) for the blobs in `need`: readers
+        // after position `index` whose kind differs from the producer's are redirected to its outputs
+        // (net_optimizer_insert_int8_reformat.cc:183-216, AdjustLayer)
+        auto insert_reformat = [&](const std::string &name, bool producer_quantized, const std::vector<std::string> &need,
+                                   int index, std::shared_ptr<LayerInfo> *made) -> Status {
+            auto nl      = std::make_shared<LayerInfo>();
+            nl->type     = LAYER_REFORMAT;
+            nl->type_str = "Reformat";
+            nl->name     = name;
+            auto p       = std::make_shared<ReformatLayerParam>();
+            p->LayerParam::type = nl->type_str;  // ReformatLayerParam::type (quant direction) shadows the base field
+            p->name      = nl->name;
+            p->src_type  = producer_quantized ? DATA_TYPE_INT8 : float_type_;
+            p->dst_type  = producer_quantized ? float_type_ : DATA_TYPE_INT8;
+            nl->param    = p;
+            nl->inputs   = need;
+            for (auto &o : need) {
+                std::string no = o + "_int8_reformat";
+                nl->outputs.push_back(no);
+                s->blobs.insert(no);
+                for (int j = index + 1; j < count; ++j)
+                    for (auto &in : layers[j]->inputs)
+                        if (in == o && layers[j]->param->quantized != producer_quantized)
+                            in = no;
+                if (!producer_quantized) {
+                    auto it = res->resource_map.find(o + "_scale_data_");
+                    if (it == res->resource_map.end())
+                        return Status(TNNERR_NULL_PARAM, "can not get blob scale " + o + "_scale_data_");
+                    res->resource_map[no + "_scale_data_"] = it->second;
+                }
+            }
+            *made = nl;
+            return TNN_OK;
+        };
+        // A model input read by quantised and by float layers alike gets its Reformat at the head of the graph
+        // (net_optimizer_insert_int8_reformat.cc:84-131); the input blob keeps the type the model declares for it.
+        for (const auto &kv : s->inputs_shape_map) {
+            const std::string &model_input = kv.first;
+            int need_int8 = 0, need_float = 0;
+            for (auto &l : layers)
+                for (auto &in : l->inputs)
+                    if (in == model_input) {
+                        (l->param->quantized ? need_int8 : need_float)++;
+                        break;
+                    }
+            if (need_int8 == 0 || need_float == 0)
+                continue;
+            auto ti = s->input_data_type_map.find(model_input);
+            const DataType in_type = ti == s->input_data_type_map.end() ? DATA_TYPE_FLOAT : ti->second;
+            if (in_type != DATA_TYPE_FLOAT && in_type != DATA_TYPE_INT8)
+                return Status(TNNERR_UNSUPPORT_NET, "RocmInsertInt8Reformat: model input " + model_input +
+                                                        " feeds quantised and float layers but is neither float nor int8");
+            std::shared_ptr<LayerInfo> nl;
+            RETURN_ON_NEQ(insert_reformat(model_input + "_int8_reformat__from_model_input__", in_type == DATA_TYPE_INT8,
+                                          {model_input}, -1, &nl),
+                          TNN_OK);
+            out.push_back(nl);
+        }
         for (int i = 0; i < count; ++i) {
             auto cur = layers[i];
             out.push_back(cur);
@@ -887,32 +945,8 @@ public:
             }
             if (need.empty())
                 continue;
-            auto nl      = std::make_shared<LayerInfo>();
-            nl->type     = LAYER_REFORMAT;
-            nl->type_str = "Reformat";
-            nl->name     = cur->name + "_int8_reformat";
-            auto p       = std::make_shared<ReformatLayerParam>();
-            p->LayerParam::type = nl->type_str;  // ReformatLayerParam::type (quant direction) shadows the base field
-            p->name      = nl->name;
-            p->src_type  = cur->param->quantized ? DATA_TYPE_INT8 : float_type_;
-            p->dst_type  = cur->param->quantized ? float_type_ : DATA_TYPE_INT8;
-            nl->param    = p;
-            nl->inputs   = need;
-            for (auto &o : need) {
-                std::string no = o + "_int8_reformat";
-                nl->outputs.push_back(no);
-                s->blobs.insert(no);
-                for (int j = i + 1; j < count; ++j)
-                    for (auto &in : layers[j]->inputs)
-                        if (in == o && layers[j]->param->quantized != cur->param->quantized)
-                            in = no;
-                if (!cur->param->quantized) {
-                    auto it = res->resource_map.find(o + "_scale_data_");
-                    if (it == res->resource_map.end())
-                        return Status(TNNERR_NULL_PARAM, "can not get blob scale " + o + "_scale_data_");
-                    res->resource_map[no + "_scale_data_"] = it->second;
-                }
-            }
+            std::shared_ptr<LayerInfo> nl;
+            RETURN_ON_NEQ(insert_reformat(cur->name + "_int8_reformat", cur->param->quantized, need, i, &nl), TNN_OK);
             out.push_back(nl);
         }
         s->layers = out;

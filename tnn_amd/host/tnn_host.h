@@ -43,6 +43,7 @@ enum StatusCode {
     TNNERR_INVALID_NETCFG                     = 0x1002,
     TNNERR_NULL_PARAM                         = 0x1004,
     TNNERR_NET_ERR                            = 0x2000,
+    TNNERR_UNSUPPORT_NET                      = 0x2001,
     TNNERR_LAYER_ERR                          = 0x3000,
     TNNERR_UNKNOWN_LAYER                      = 0x3001,
     TNNERR_CREATE_LAYER                       = 0x3002,
