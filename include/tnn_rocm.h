@@ -151,7 +151,7 @@ TNN_ROCM_API int tnn_rocm_attention_vt_q8(void *stream, int dtype, const void *q
                                           int8_t *out_q, float out_q_inv_scale, int B, int heads, int S, int head_dim,
                                           long q_sb, long q_sh, long q_ss, long k_sb, long k_sh, long k_ss, long vt_sb,
                                           long vt_sh, long vt_sd, long o_sb, long o_sh, long o_ss, float scale,
-                                          const float *mask, const int32_t *kv_len);
+                                          const float *mask, const int32_t *kv_len, int vt_key_order);
 
 /* The int8 GEMM above with a float consumer folded in: out_f = (float)q * dequant_scale (+ residual), where q is
  * the requantised int8 value of tnn_rocm_gemm_i8 (never written).  This is QuantizedInnerProduct -> Reformat
@@ -178,15 +178,20 @@ TNN_ROCM_API int tnn_rocm_gemm_i8_lut(void *stream, const int8_t *A, const int8_
  * Q | K row-major in qk[T,2H], V transposed per head in vt[B][heads][64][S].  out_dtype F16 or BF16. */
 TNN_ROCM_API int tnn_rocm_gemm_i8_qkv_split(void *stream, int out_dtype, const int8_t *x, const int8_t *wqkv,
                                             const int32_t *bias, const float *scale, const float *dequant, void *qk,
-                                            void *vt, int B, int S, int heads, int K);
+                                            void *vt, int B, int S, int heads, int K, int vt_key_order);
 
 /* Fused QKV projection for the attention layer: [T,K] x Wqkv[3H,K]^T + bqkv with the result split on the way out:
  * Q and K go to qk[T, 2H] (row-major, Q | K column blocks), V goes transposed per head to
  * vt[B][heads][64][S] (T = B*S tokens, H = heads*64).  Same arithmetic as three MatMul+Add pairs
  * (cpu_mat_mul_layer_acc.cc:64-117, compute_elewise.cc:37-65) followed by the head-split Permutes
  * (naive_compute.cc:943-956).  dtype F16 or BF16; K and H multiples of 64. */
+/* V^T key order (vt_key_order of the three QKV-split projections and of tnn_rocm_attention_vt_q8; no counterpart in the
+ * reference, whose Permute layers this layout replaces).  0: row d of a head holds its S keys in natural order.  1: inside
+ * every group of 16 keys the blocks k4-7 and k8-11 have changed places ([k0-3 | k8-11 | k4-7 | k12-15]), the order in
+ * which the attention kernel's lanes hold a score tile's probabilities, so that it needs no register exchange in front of
+ * its second MFMA.  Needs S % 16 == 0; producer and consumer must agree.  tnn_rocm_attention_vt reads order 0. */
 TNN_ROCM_API int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *wqkv, const float *bqkv,
-                                         void *qk, void *vt, int B, int S, int heads, int K);
+                                         void *qk, void *vt, int B, int S, int heads, int K, int vt_key_order);
 
 /* LayerNorm folded into the projection that reads it: y = LayerNorm(t) over the last axis of t[M,K]
  * (cpu_layer_norm_layer_acc.cc:86-135) followed by C = act(y W^T + b) (+ residual) (cpu_mat_mul_layer_acc.cc:64-117,
@@ -214,7 +219,7 @@ TNN_ROCM_API int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void 
                                             const float *bqkv_folded, const float *colsum, const float *gamma,
                                             const float *beta, float eps, void *qk, void *vt, void *y,
                                             float *row_stats, const float *row_sums, int row_sum_blocks, int B,
-                                            int S, int heads, int K);
+                                            int S, int heads, int K, int vt_key_order);
 
 /* C = act(x W^T + b) + LayerNorm(t), the residual Add of a transformer block whose residual operand is the output of
  * a LayerNorm layer (compute_elewise.cc:37-65 after cpu_layer_norm_layer_acc.cc:86-135), without that output ever

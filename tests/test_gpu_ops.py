@@ -19,6 +19,7 @@ pytestmark = pytest.mark.gpu
 FP32_TOL = 2e-3      # the bar stated for fp32 against the reference's CPU paths
 FP32_ASSERT = 5e-5   # what the fp32 cases assert: true-fp32 MFMA products, fp32 accumulation (observed <= 1e-5)
 FP16_TOL = 1e-2
+BF16_TOL = 4e-2
 
 
 def say(msg):
@@ -787,6 +788,67 @@ def test_qkv_split_and_attention_vt():
         mask[b_, l:] = -np.inf
     ref_o = orc.attention_core(q, k, v, 0.125, mask).transpose(0, 2, 1, 3).reshape(B * S, H)
     assert rel_err(out, ref_o) <= FP16_TOL
+
+
+@pytest.mark.parametrize("B,S,h,dtype", [(3, 208, 12, "f16"), (2, 80, 4, "f16"), (8, 384, 12, "f16"), (32, 512, 12, "f16"),
+                                         (3, 208, 12, "bf16"), (32, 512, 12, "bf16")])
+def test_vt_in_accumulator_key_order(B, S, h, dtype):
+    """V^T key order 1 (inside every 16 keys the blocks k4-7 and k8-11 exchanged): the three QKV-split projections write
+    exactly the natural-order tensor with its keys permuted, and the attention kernels -- the two- and the four-wave form,
+    the direct-to-LDS and the register-staged one, plain lengths and an additive mask -- give on the permuted tensor
+    what they give on the natural one (the keys of a 16-group meet the P.V MFMA in another order: fp32 accumulation
+    order, one fp16 ulp) and what the checker gives."""
+    say("V^T in accumulator key order B%d S%d h%d %s" % (B, S, h, dtype))
+    from tnn_amd import capi
+    o = ops()
+    td = torch.float16 if dtype == "f16" else torch.bfloat16
+    tol = FP16_TOL if dtype == "f16" else BF16_TOL
+    H = h * 64
+    rng = np.random.default_rng(B * S)
+    x = torch.from_numpy(rng.standard_normal((B * S, H)).astype(np.float32)).to(td).cuda()
+    w = torch.from_numpy((rng.standard_normal((3 * H, H)) * 0.05).astype(np.float32)).to(td).cuda()
+    bias = dev((rng.standard_normal(3 * H) * 0.1).astype(np.float32))
+    qk0, vt0 = o.qkv_split(x, w, bias, B, S, h)
+    qk1, vt1 = o.qkv_split(x, w, bias, B, S, h, vt_key_order=1)
+    assert torch.equal(qk0, qk1) and torch.equal(vt1, o.permute_keys(vt0)) and not torch.equal(vt1, vt0)
+    if H % 128 == 0:   # the LayerNorm-folding form (its weights need no meaning here: same launch, two key orders)
+        cs, eps = w.float().sum(1).contiguous(), 1e-12
+        a0 = o.qkv_split_ln(x, w, bias, cs, eps, B, S, h)
+        a1 = o.qkv_split_ln(x, w, bias, cs, eps, B, S, h, vt_key_order=1)
+        assert torch.equal(a0[0], a1[0]) and torch.equal(a1[1], o.permute_keys(a0[1]))
+    x8 = torch.randint(-128, 128, (B * S, H), dtype=torch.int8, device="cuda")
+    w8 = torch.randint(-127, 128, (3 * H, H), dtype=torch.int8, device="cuda")
+    sc = (torch.rand(3 * H, device="cuda") * 2e-4 + 1e-4).float()
+    dq = torch.full((3 * H,), 0.05, device="cuda")
+    i0 = o.gemm_i8_qkv_split(x8, w8, None, sc, dq, B, S, h, dtype=td)
+    i1 = o.gemm_i8_qkv_split(x8, w8, None, sc, dq, B, S, h, dtype=td, vt_key_order=1)
+    assert torch.equal(i0[0], i1[0]) and torch.equal(i1[1], o.permute_keys(i0[1]))
+    lens = rng.integers(1, S + 1, B).astype(np.int32)
+    lens[0] = S
+    mask = np.zeros((B, S), np.float32)
+    for b_, l in enumerate(lens):
+        mask[b_, l:] = -10000.0
+    mask[0, 3] = -0.75                                   # a visible key with a bias: that row takes the biased tile form
+    plain = host(o.gemm(x, w, True, bias=bias)).reshape(B, S, 3, h, 64)
+    q, k, v = (np.ascontiguousarray(plain[:, :, i].transpose(0, 2, 1, 3)) for i in range(3))
+    for use_mask in (False, True):
+        kw = dict(mask=dev(mask), kv_len=o.mask_to_kv_len(dev(mask), flagged=True)) if use_mask else dict(kv_len=dev(lens))
+        ref_mask = mask if use_mask else np.where(np.arange(S)[None, :] < lens[:, None], 0.0, -np.inf).astype(np.float32)
+        ref = orc.attention_core(q, k, v, 0.125, ref_mask).transpose(0, 2, 1, 3).reshape(B * S, H)
+        for dma in (1, 0):
+            capi.load().tnn_rocm_debug_set_attention_dma(dma)
+            try:
+                nat = host(o.attention_qk_vt(qk0, vt0, B, S, h, 0.125, **kw))
+                per = host(o.attention_qk_vt(qk1, vt1, B, S, h, 0.125, vt_key_order=1, **kw))
+            finally:
+                capi.load().tnn_rocm_debug_set_attention_dma(1)
+            assert rel_err(per, nat) <= (1e-3 if dtype == "f16" else 8e-3), (use_mask, dma)
+            assert rel_err(per, ref) <= tol, (use_mask, dma)
+    # the quantised second output rides along unchanged
+    out, out_q = o.attention_qk_vt(qk1, vt1, B, S, h, 0.125, kv_len=dev(lens), q8_inv_scale=np.float32(40.0), vt_key_order=1)
+    assert np.array_equal(host(out_q), host(o.quantize(out, np.float32(40.0))))
+    with pytest.raises(capi.TnnRocmError):
+        o.attention_qk_vt(qk1[: B * 8], vt1[:, :, :, :8].contiguous(), B, 8, h, 0.125, vt_key_order=1)   # S % 16 != 0
 
 
 def test_mask_prepare_any_float_type():

@@ -74,7 +74,7 @@ def c3(args):
     for name, kvl in (("varlen", kv), ("full", None)):
         # launches recorded into one graph, so the host's launch rate is not what is measured
         def call():
-            ops.attention_qk_vt(qk, vt, B, S, h, 0.125, kv_len=kvl, out=out)
+            ops.attention_qk_vt(qk, vt, B, S, h, 0.125, kv_len=kvl, out=out, vt_key_order=1 if S % 16 == 0 else 0)
         for _ in range(3):
             call()
         torch.cuda.synchronize()

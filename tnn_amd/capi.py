@@ -42,17 +42,17 @@ SIGNATURES = {
     "tnn_rocm_gemm": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i],
     "tnn_rocm_gemm_i8": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _f],
     "tnn_rocm_gemm_i8_dequant_residual": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _i, _f, _vp],
-    "tnn_rocm_gemm_i8_qkv_split": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i],
+    "tnn_rocm_gemm_i8_qkv_split": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i],
     "tnn_rocm_attention": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _l, _l, _l, _l, _l, _l, _l, _l, _l, _f,
                            _vp, _vp],
     "tnn_rocm_attention_vt": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _l, _l, _l, _l, _l, _l, _l, _l, _l, _l, _l,
                               _l, _f, _vp, _vp],
     "tnn_rocm_attention_vt_q8": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _l, _l, _l, _l, _l, _l, _l, _l, _l,
-                                 _l, _l, _l, _f, _vp, _vp],
+                                 _l, _l, _l, _f, _vp, _vp, _i],
     "tnn_rocm_gemm_i8_lut": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
-    "tnn_rocm_gemm_qkv_split": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i],
+    "tnn_rocm_gemm_qkv_split": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i],
     "tnn_rocm_gemm_ln": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
-    "tnn_rocm_gemm_qkv_split_ln": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i],
+    "tnn_rocm_gemm_qkv_split_ln": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i],
     "tnn_rocm_gemm_residual_ln": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp],
     "tnn_rocm_mask_to_kv_len": [_vp, _vp, _vp, _i, _i, _f],
     "tnn_rocm_mask_to_kv_len_flagged": [_vp, _vp, _vp, _i, _i, _f],

@@ -120,6 +120,11 @@ struct AttnParams {
     const int32_t *kv_len;
     int8_t *oq;   // optional second output: the stored values quantised, same element strides as o
     float q_inv;  // 1 / scale of that int8 tensor
+    // V^T key order (VT kernels).  0: natural.  1: inside every group of 16 keys the two middle blocks of four have
+    // changed places ([k0-3 | k8-11 | k4-7 | k12-15]), which is the order in which a lane half holds the probabilities
+    // of a score tile (rows 8*(r/4) + 4*half + r%4 of the accumulator block): the packed probabilities then feed the
+    // second MFMA as they are, with no exchange between the lane halves.  Needs S % 16 == 0.
+    int vt_perm;
 };
 
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
@@ -260,7 +265,10 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
         _Pragma("unroll") for (int i = 0; i < KV_VECS; ++i) {                                                         \
             const int row = vrow + i * ROW_STEP;                                                                      \
             *reinterpret_cast<u32x4 *>(lds_k##BUF + row * kRowBytes + vch * 16) = rk[i];                              \
-            if (VT) {                                                                                                 \
+            if (VT && p.vt_perm) {                                                                                    \
+                /* the rows already come in the order the fragments want */                                          \
+                *reinterpret_cast<u32x4 *>(lds_vt##BUF + row * kRowBytes + vch * 16) = rv[i];                         \
+            } else if (VT) {                                                                                          \
                 /* this thread holds keys 8*vch .. 8*vch+7 of row d: chunk pair (2*(vch&1), 2*(vch&1)+1) of group */  \
                 /* vch/2 goes to chunk positions (vch&1) and (vch&1)+2 */                                             \
                 unsigned char *dst = lds_vt##BUF + row * kRowBytes + (vch >> 1) * 32 + (vch & 1) * 8;                 \
@@ -466,7 +474,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
 // permuting the keys inside the tile.
 #define TR_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n)&0xF) | ((((n) >> 4) & 3) << 14) | (0x7 << 4) | (0xF << 8)))
 
-template <int DT, int NW>
+template <int DT, int NW, bool PERM>
 __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 : 2) attention_dma_kernel(AttnParams p) {
     constexpr int NT = NW * 64;
     constexpr int BQ = NW * 32;
@@ -682,9 +690,15 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
             uint32_t w1 = AttnT<DT>::pack_only(sacc[kt][8 * j + 2], sacc[kt][8 * j + 3]);
             uint32_t w2 = AttnT<DT>::pack_only(sacc[kt][8 * j + 4], sacc[kt][8 * j + 5]);
             uint32_t w3 = AttnT<DT>::pack_only(sacc[kt][8 * j + 6], sacc[kt][8 * j + 7]);
-            auto x0 = __builtin_amdgcn_permlane32_swap(w0, w2, false, false);
-            auto x1 = __builtin_amdgcn_permlane32_swap(w1, w3, false, false);
-            pf[st][0] = x0[0], pf[st][1] = x1[0], pf[st][2] = x0[1], pf[st][3] = x1[1];
+            if constexpr (PERM) {
+                // V^T comes with its keys in the accumulators' order (AttnParams::vt_perm): chunk 2*st + g of its rows
+                // holds exactly the eight keys this lane half has just packed
+                pf[st][0] = w0, pf[st][1] = w1, pf[st][2] = w2, pf[st][3] = w3;
+            } else {
+                auto x0 = __builtin_amdgcn_permlane32_swap(w0, w2, false, false);
+                auto x1 = __builtin_amdgcn_permlane32_swap(w1, w3, false, false);
+                pf[st][0] = x0[0], pf[st][1] = x1[0], pf[st][2] = x0[1], pf[st][3] = x1[1];
+            }
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 AttnT<DT>::add_packed(pf[st][e], rs);
@@ -925,19 +939,25 @@ template <bool VT> int launch_attention(hipStream_t s, int dtype, const AttnPara
     long blocks128 = (long)((S + 127) / 128) * heads * B;
     auto padded = [&](long n_q) { return dim3((unsigned)(((n_q * heads * B + 7) / 8) * 8)); };
     if (VT && g_attention_dma) {
+#define TR_LAUNCH_DMA(NWv, THREADS)                                                                                   \
+    do {                                                                                                              \
+        if (dtype == TNN_ROCM_F16 && p.vt_perm)                                                                       \
+            hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_F16, NWv, true>), grid, dim3(THREADS), 0, s, p);        \
+        else if (dtype == TNN_ROCM_F16)                                                                               \
+            hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_F16, NWv, false>), grid, dim3(THREADS), 0, s, p);       \
+        else if (p.vt_perm)                                                                                           \
+            hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_BF16, NWv, true>), grid, dim3(THREADS), 0, s, p);       \
+        else                                                                                                          \
+            hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_BF16, NWv, false>), grid, dim3(THREADS), 0, s, p);      \
+    } while (0)
         if (blocks128 >= 512) {
             dim3 grid = padded((S + 127) / 128);
-            if (dtype == TNN_ROCM_F16)
-                hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_F16, 4>), grid, dim3(256), 0, s, p);
-            else
-                hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_BF16, 4>), grid, dim3(256), 0, s, p);
+            TR_LAUNCH_DMA(4, 256);
         } else {
             dim3 grid = padded((S + 63) / 64);
-            if (dtype == TNN_ROCM_F16)
-                hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_F16, 2>), grid, dim3(128), 0, s, p);
-            else
-                hipLaunchKernelGGL((attention_dma_kernel<TNN_ROCM_BF16, 2>), grid, dim3(128), 0, s, p);
+            TR_LAUNCH_DMA(2, 128);
         }
+#undef TR_LAUNCH_DMA
         TR_CHECK_LAUNCH();
         return 0;
     }
@@ -997,8 +1017,9 @@ int tnn_rocm_attention(void *stream, int dtype, const void *q, const void *k, co
     p.mask        = mask;
     p.kv_len      = kv_len;
     p.vt_sb = p.vt_sh = p.vt_sd = 0;
-    p.oq    = nullptr;
-    p.q_inv = 0.f;
+    p.oq      = nullptr;
+    p.q_inv   = 0.f;
+    p.vt_perm = 0;
     return launch_attention<false>((hipStream_t)stream, dtype, p, B, heads, S);
 }
 
@@ -1007,14 +1028,17 @@ int tnn_rocm_attention_vt(void *stream, int dtype, const void *q, const void *k,
                           long k_ss, long vt_sb, long vt_sh, long vt_sd, long o_sb, long o_sh, long o_ss, float scale,
                           const float *mask, const int32_t *kv_len) {
     return tnn_rocm_attention_vt_q8(stream, dtype, q, k, vt, out, nullptr, 0.f, B, heads, S, head_dim, q_sb, q_sh, q_ss, k_sb,
-                                    k_sh, k_ss, vt_sb, vt_sh, vt_sd, o_sb, o_sh, o_ss, scale, mask, kv_len);
+                                    k_sh, k_ss, vt_sb, vt_sh, vt_sd, o_sb, o_sh, o_ss, scale, mask, kv_len, 0);
 }
 
 int tnn_rocm_attention_vt_q8(void *stream, int dtype, const void *q, const void *k, const void *vt, void *out,
                              int8_t *out_q, float out_q_inv_scale, int B, int heads, int S, int head_dim, long q_sb,
                              long q_sh, long q_ss, long k_sb, long k_sh, long k_ss, long vt_sb, long vt_sh, long vt_sd,
-                             long o_sb, long o_sh, long o_ss, float scale, const float *mask, const int32_t *kv_len) {
+                             long o_sb, long o_sh, long o_ss, float scale, const float *mask, const int32_t *kv_len,
+                             int vt_key_order) {
     TR_REQUIRE(B >= 0 && heads >= 0 && S >= 0, TNN_ROCM_ESHAPE, "attention_vt: negative size");
+    TR_REQUIRE(vt_key_order == 0 || (vt_key_order == 1 && S % 16 == 0), TNN_ROCM_EINVAL,
+               "attention_vt: V^T key order %d (0 natural, 1 accumulator order, which needs S %% 16 == 0; S=%d)", vt_key_order, S);
     if (B == 0 || heads == 0 || S == 0)
         return 0;
     TR_REQUIRE(q && k && vt && out, TNN_ROCM_EINVAL, "attention_vt: null pointer");
@@ -1048,8 +1072,9 @@ int tnn_rocm_attention_vt_q8(void *stream, int dtype, const void *q, const void 
     p.mask        = mask;
     p.kv_len      = kv_len;
     TR_REQUIRE(!out_q || (((uintptr_t)out_q) & 7u) == 0, TNN_ROCM_EALIGN, "attention_vt: int8 output must be 8-byte aligned");
-    p.oq    = out_q;
-    p.q_inv = out_q_inv_scale;
+    p.oq      = out_q;
+    p.q_inv   = out_q_inv_scale;
+    p.vt_perm = vt_key_order;
     return launch_attention<true>((hipStream_t)stream, dtype, p, B, heads, S);
 }
 

@@ -178,6 +178,11 @@ template <int DT> struct FloatEpilogue {
     }
 };
 
+// Where key s goes inside its V^T row.  sh = 0: at s.  sh = 1: inside every group of 16 keys the blocks of four
+// k4-7 and k8-11 change places ([k0-3 | k8-11 | k4-7 | k12-15]), the order in which the lane halves of the attention
+// kernel hold a tile's probabilities, so that kernel feeds them to its second MFMA without exchanging registers.
+__device__ __forceinline__ int key_slot(int s, int sh) { return (s & ~12) | ((s & 4) << sh) | ((s & 8) >> sh); }
+
 // QKV projection epilogue: columns [0,2H) -> qk[T,2H]; columns [2H,3H) -> V^T[b][head][d][s]
 template <int DT> struct QkvSplitEpilogue {
     typedef typename Elem<DT>::type T;
@@ -186,6 +191,7 @@ template <int DT> struct QkvSplitEpilogue {
     T *qk;
     T *vt;
     int H, S, heads;
+    int vt_sh;  // 0: V^T keys in natural order; 1: bits 2 and 3 of the key index change places (see key_slot)
     __device__ __forceinline__ void set_batch(int) {}
     __device__ __forceinline__ float col_const(int n) const { return bias ? bias[n] : 0.f; }
     __device__ __forceinline__ void store(int m, int n, float acc, float bias_n) const {
@@ -193,7 +199,7 @@ template <int DT> struct QkvSplitEpilogue {
         if (n < 2 * H) {
             Elem<DT>::st(&qk[(size_t)m * 2 * H + n], v);
         } else {
-            int c = n - 2 * H, b = m / S, s = m - b * S;
+            int c = n - 2 * H, b = m / S, s = key_slot(m - b * S, vt_sh);
             Elem<DT>::st(&vt[(((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s], v);
         }
     }
@@ -223,7 +229,7 @@ template <int DT> struct QkvSplitEpilogue {
             for (int q = 0; q < NV; ++q)
                 store_out16(&cp[q], packed[q]);
         } else {
-            int c = n - 2 * H, b = m / S, s_ = m - b * S;
+            int c = n - 2 * H, b = m / S, s_ = key_slot(m - b * S, vt_sh);
             T *dst = vt + (((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s_;
 #pragma unroll
             for (int t = 0; t < 8; ++t)
@@ -360,6 +366,7 @@ template <int DT, int SUMS = 0> struct LnQkvSplitEpilogue {
     T *qk;
     T *vt;
     int H, S, heads;
+    int vt_sh;  // 0: V^T keys in natural order; 1: bits 2 and 3 of the key index change places (see key_slot)
     LnFold ln;
     __device__ __forceinline__ void set_batch(int) {}
     __device__ __forceinline__ float col_const(int) const { return 0.f; }
@@ -389,7 +396,7 @@ template <int DT, int SUMS = 0> struct LnQkvSplitEpilogue {
                 store_out16(&cp[q], packed[q]);
         } else {
             // B * S * 3H < 2^31 is checked at launch: 32-bit offsets throughout
-            int c = n - 2 * H, bb = m / S, s_ = m - bb * S;
+            int c = n - 2 * H, bb = m / S, s_ = key_slot(m - bb * S, vt_sh);
             T *dst = vt + (unsigned)(((bb * heads + (c >> 6)) * 64 + (c & 63)) * S + s_);
 #pragma unroll
             for (int t = 0; t < 8; ++t)
@@ -613,6 +620,7 @@ template <int DT> struct Int8QkvSplitEpilogue {
     T *qk;
     T *vt;
     int H, S, heads;
+    int vt_sh;  // 0: V^T keys in natural order; 1: bits 2 and 3 of the key index change places (see key_slot)
     __device__ __forceinline__ void set_batch(int) {}
     struct ColConst {
         int32_t bias;
@@ -631,7 +639,7 @@ template <int DT> struct Int8QkvSplitEpilogue {
         if (n < 2 * H) {
             Elem<DT>::st(&qk[(size_t)m * 2 * H + n], v);
         } else {
-            int c = n - 2 * H, b = m / S, s = m - b * S;
+            int c = n - 2 * H, b = m / S, s = key_slot(m - b * S, vt_sh);
             Elem<DT>::st(&vt[(((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s], v);
         }
     }
@@ -666,7 +674,7 @@ template <int DT> struct Int8QkvSplitEpilogue {
             for (int q = 0; q < NV; ++q)
                 store_out16(&cp[q], packed[q]);
         } else {
-            int c = n - 2 * H, b = m / S, s_ = m - b * S;
+            int c = n - 2 * H, b = m / S, s_ = key_slot(m - b * S, vt_sh);
             T *dst = vt + (((size_t)b * heads + (c >> 6)) * 64 + (c & 63)) * S + s_;
 #pragma unroll
             for (int t = 0; t < 8; ++t)
@@ -1914,7 +1922,9 @@ int tnn_rocm_gemm_i8_dequant_residual(void *stream, const int8_t *A, const int8_
 
 int tnn_rocm_gemm_i8_qkv_split(void *stream, int out_dtype, const int8_t *x, const int8_t *wqkv, const int32_t *bias,
                                const float *scale, const float *dequant, void *qk, void *vt, int B, int S, int heads,
-                               int K) {
+                               int K, int vt_key_order) {
+    TR_REQUIRE(vt_key_order == 0 || (vt_key_order == 1 && S % 16 == 0), TNN_ROCM_EINVAL,
+               "gemm_i8_qkv_split: V^T key order %d (0 or 1; 1 needs S %% 16 == 0, S=%d)", vt_key_order, S);
     TR_REQUIRE(B >= 0 && S >= 0 && heads >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_i8_qkv_split: negative size");
     if (B == 0 || S == 0 || heads == 0)
         return 0;
@@ -1938,6 +1948,7 @@ int tnn_rocm_gemm_i8_qkv_split(void *stream, int out_dtype, const int8_t *x, con
         epi.H       = H;                                                                                              \
         epi.S       = S;                                                                                              \
         epi.heads   = heads;                                                                                          \
+        epi.vt_sh   = vt_key_order;                                                                                   \
         return launch_gemm_fast<TNN_ROCM_I8, Int8QkvSplitEpilogue<DT>>((hipStream_t)stream, x, wqkv, T, 3 * H, K, K, K, \
                                                                        epi);                                          \
     }
@@ -1949,7 +1960,9 @@ int tnn_rocm_gemm_i8_qkv_split(void *stream, int out_dtype, const int8_t *x, con
 }
 
 int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *wqkv, const float *bqkv, void *qk,
-                            void *vt, int B, int S, int heads, int K) {
+                            void *vt, int B, int S, int heads, int K, int vt_key_order) {
+    TR_REQUIRE(vt_key_order == 0 || (vt_key_order == 1 && S % 16 == 0), TNN_ROCM_EINVAL,
+               "gemm_qkv_split: V^T key order %d (0 or 1; 1 needs S %% 16 == 0, S=%d)", vt_key_order, S);
     TR_REQUIRE(B >= 0 && S >= 0 && heads >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_qkv_split: negative size");
     if (B == 0 || S == 0 || heads == 0)
         return 0;
@@ -1970,6 +1983,7 @@ int tnn_rocm_gemm_qkv_split(void *stream, int dtype, const void *x, const void *
         epi.H     = H;                                                                                                \
         epi.S     = S;                                                                                                \
         epi.heads = heads;                                                                                            \
+        epi.vt_sh = vt_key_order;                                                                                     \
         return launch_gemm_fast<DT, QkvSplitEpilogue<DT>>((hipStream_t)stream, x, wqkv, T, 3 * H, K, K, K, epi);      \
     }
     if (dtype == TNN_ROCM_F16)
@@ -2033,7 +2047,9 @@ int tnn_rocm_gemm_ln(void *stream, int dtype, const void *t, const void *w_folde
 int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const void *wqkv_folded, const float *bqkv_folded,
                                const float *colsum, const float *gamma, const float *beta, float eps, void *qk, void *vt,
                                void *y, float *row_stats, const float *row_sums, int row_sum_blocks, int B, int S, int heads,
-                               int K) {
+                               int K, int vt_key_order) {
+    TR_REQUIRE(vt_key_order == 0 || (vt_key_order == 1 && S % 16 == 0), TNN_ROCM_EINVAL,
+               "gemm_qkv_split_ln: V^T key order %d (0 or 1; 1 needs S %% 16 == 0, S=%d)", vt_key_order, S);
     TR_REQUIRE(B >= 0 && S >= 0 && heads >= 0 && K >= 0, TNN_ROCM_ESHAPE, "gemm_qkv_split_ln: negative size");
     if (B == 0 || S == 0 || heads == 0)
         return 0;
@@ -2059,6 +2075,7 @@ int tnn_rocm_gemm_qkv_split_ln(void *stream, int dtype, const void *t, const voi
         epi.H     = H;                                                                                                \
         epi.S     = S;                                                                                                \
         epi.heads = heads;                                                                                            \
+        epi.vt_sh = vt_key_order;                                                                                     \
         epi.ln = LnFold{1.0f / (float)K, eps, colsum, gamma, beta, y, g_ln_y_ahead.load(), (float2 *)row_stats,       \
                         (const float2 *)row_sums, row_sum_blocks};                                                   \
         return launch_gemm_fast<DT, LnQkvSplitEpilogue<DT, SUMS>>((hipStream_t)stream, t, wqkv_folded, T, 3 * H, K, K, K, \

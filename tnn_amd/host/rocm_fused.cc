@@ -1609,6 +1609,9 @@ public:
         }
         const char *base = (const char *)qkv;
         const long d     = p->head_dim;
+        // V^T leaves the projection with its keys in the order the attention kernel's accumulators hold them (no
+        // register exchange in front of the second MFMA) whenever whole groups of 16 keys exist
+        const int vt_order = seq_ % 16 == 0 ? 1 : 0;
         int8_t *out_q    = nullptr;
         float out_q_inv  = 0.f;
         if (p->out_quant) {  // the last output: the context quantised as the folded Reformat layer would
@@ -1624,12 +1627,12 @@ public:
             char *vt = (char *)qkv + (size_t)T_ * 2 * H_ * es;
             ROCM_CALL(tnn_rocm_gemm_i8_qkv_split(Stream(), (int)dt, (const int8_t *)Ptr(inputs[0]), (const int8_t *)weight_,
                                                  (const int32_t *)bias_, (const float *)scale_, (const float *)dequant_, qkv,
-                                                 vt, B_, seq_, p->heads, K_));
+                                                 vt, B_, seq_, p->heads, K_, vt_order));
             const long row = 2L * H_;
             ROCM_CALL(tnn_rocm_attention_vt_q8(Stream(), (int)dt, base, base + (size_t)H_ * es, vt, Ptr(outputs[0]), out_q,
                                                out_q_inv, B_, p->heads, seq_, p->head_dim, (long)seq_ * row, d, row,
                                                (long)seq_ * row, d, row, (long)p->heads * 64 * seq_, 64L * seq_, (long)seq_,
-                                               (long)seq_ * H_, d, (long)H_, p->scale, mask, kv));
+                                               (long)seq_ * H_, d, (long)H_, p->scale, mask, kv, vt_order));
             return TNN_OK;
         }
         if (seq_ % 8 == 0 && H_ % 64 == 0) {
@@ -1640,15 +1643,15 @@ public:
                 ROCM_CALL(tnn_rocm_gemm_qkv_split_ln(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_,
                                                      (const float *)colsum_, (const float *)gamma_, (const float *)beta_,
                                                      p->ln_eps, qkv, vt, p->ln_y ? Ptr(outputs[1]) : nullptr, (float *)stats,
-                                                     (const float *)sums, blocks, B_, seq_, p->heads, H_));
+                                                     (const float *)sums, blocks, B_, seq_, p->heads, H_, vt_order));
             else
                 ROCM_CALL(tnn_rocm_gemm_qkv_split(Stream(), (int)dt, Ptr(inputs[0]), weight_, (const float *)bias_, qkv, vt,
-                                                  B_, seq_, p->heads, H_));
+                                                  B_, seq_, p->heads, H_, vt_order));
             const long row = 2L * H_;
             ROCM_CALL(tnn_rocm_attention_vt_q8(Stream(), (int)dt, base, base + (size_t)H_ * es, vt, Ptr(outputs[0]), out_q,
                                                out_q_inv, B_, p->heads, seq_, p->head_dim, (long)seq_ * row, d, row,
                                                (long)seq_ * row, d, row, (long)p->heads * 64 * seq_, 64L * seq_, (long)seq_,
-                                               (long)seq_ * H_, d, (long)H_, p->scale, mask, kv));
+                                               (long)seq_ * H_, d, (long)H_, p->scale, mask, kv, vt_order));
             return TNN_OK;
         }
         // sequence lengths that are not a multiple of 8 (only reachable by Instance::Reshape when a fold was decided

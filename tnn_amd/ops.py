@@ -80,14 +80,14 @@ def gemm_i8_dequant_residual(a, w, bias, scale, dequant_scale, residual=None, dt
     return out
 
 
-def gemm_i8_qkv_split(x, wqkv, bias, scale, dequant, B, S, heads, dtype=torch.float16):
+def gemm_i8_qkv_split(x, wqkv, bias, scale, dequant, B, S, heads, dtype=torch.float16, vt_key_order=0):
     """x [B*S,K] int8, wqkv [3H,K] int8 -> (qk [B*S,2H], vt [B,heads,64,S]) dequantised"""
     _chk(x, wqkv, bias, scale, dequant)
     H = heads * 64
     qk = torch.empty(B * S, 2 * H, dtype=dtype, device=x.device)
     vt = torch.empty(B, heads, 64, S, dtype=dtype, device=x.device)
     capi.call("tnn_rocm_gemm_i8_qkv_split", _stream(), _DT[dtype], _p(x), _p(wqkv), _p(bias), _p(scale), _p(dequant),
-              _p(qk), _p(vt), B, S, heads, x.shape[1])
+              _p(qk), _p(vt), B, S, heads, x.shape[1], int(vt_key_order))
     return qk, vt
 
 
@@ -116,14 +116,15 @@ def attention_packed(qkv, B, S, heads, scale, mask=None, kv_len=None, out=None):
     return out
 
 
-def qkv_split(x, wqkv, bqkv, B, S, heads):
-    """x [B*S, K], wqkv [3H, K] -> (qk [B*S, 2H], vt [B, heads, 64, S])"""
+def qkv_split(x, wqkv, bqkv, B, S, heads, vt_key_order=0):
+    """x [B*S, K], wqkv [3H, K] -> (qk [B*S, 2H], vt [B, heads, 64, S]); vt_key_order 1: the keys of vt in the order
+    the attention kernel's accumulators hold them (see permute_keys)"""
     _chk(x, wqkv, bqkv)
     H = heads * 64
     qk = torch.empty(B * S, 2 * H, dtype=x.dtype, device=x.device)
     vt = torch.empty(B, heads, 64, S, dtype=x.dtype, device=x.device)
     capi.call("tnn_rocm_gemm_qkv_split", _stream(), dt(x), _p(x), _p(wqkv), _p(bqkv), _p(qk), _p(vt), B, S, heads,
-              x.shape[1])
+              x.shape[1], int(vt_key_order))
     return qk, vt
 
 
@@ -150,7 +151,7 @@ def gemm_ln(t, w_folded, bias_folded, colsum, eps, gamma=None, beta=None, gelu=F
 
 
 def qkv_split_ln(t, wqkv_folded, bqkv_folded, colsum, eps, B, S, heads, gamma=None, beta=None, want_y=False,
-                 want_stats=False, row_sums=None):
+                 want_stats=False, row_sums=None, vt_key_order=0):
     """qkv_split on LayerNorm(t) given as the raw t and the folded weights; optionally also LayerNorm(t) and / or the
     rows' {rstd, mean}; row_sums as for gemm_ln"""
     _chk(t, wqkv_folded, bqkv_folded, colsum, gamma, beta)
@@ -161,7 +162,7 @@ def qkv_split_ln(t, wqkv_folded, bqkv_folded, colsum, eps, B, S, heads, gamma=No
     st = torch.empty(B * S, 2, dtype=torch.float32, device=t.device) if want_stats else None
     sums, blocks = row_sums if row_sums is not None else (None, 0)
     capi.call("tnn_rocm_gemm_qkv_split_ln", _stream(), dt(t), _p(t), _p(wqkv_folded), _p(bqkv_folded), _p(colsum), _p(gamma),
-              _p(beta), float(eps), _p(qk), _p(vt), _p(y), _p(st), _p(sums), blocks, B, S, heads, t.shape[1])
+              _p(beta), float(eps), _p(qk), _p(vt), _p(y), _p(st), _p(sums), blocks, B, S, heads, t.shape[1], int(vt_key_order))
     return (qk, vt) + ((y,) if want_y else ()) + ((st,) if want_stats else ())
 
 
@@ -185,7 +186,16 @@ def gemm_residual_ln(x, w, t, row_stats, gamma, beta, bias=None, gelu=False, out
     return (out, (sums, blocks.value)) if want_row_sums else out
 
 
-def attention_qk_vt(qk, vt, B, S, heads, scale, mask=None, kv_len=None, out=None, q8_inv_scale=None):
+def permute_keys(vt):
+    """vt [..., S] with S % 16 == 0 -> the same tensor with, inside every group of 16 keys, the blocks k4-7 and k8-11
+    exchanged: V^T key order 1 of the C ABI"""
+    S = vt.shape[-1]
+    idx = torch.arange(S, device=vt.device)
+    src = (idx & ~12) | ((idx & 4) << 1) | ((idx & 8) >> 1)
+    return vt.index_select(-1, src).contiguous()
+
+
+def attention_qk_vt(qk, vt, B, S, heads, scale, mask=None, kv_len=None, out=None, q8_inv_scale=None, vt_key_order=0):
     """qk [B*S, 2H] (Q | K), vt [B, heads, 64, S]; out [B*S, H]; with q8_inv_scale also the int8 quantisation of out"""
     _chk(qk, vt, mask, kv_len, out)
     H = heads * 64
@@ -193,12 +203,12 @@ def attention_qk_vt(qk, vt, B, S, heads, scale, mask=None, kv_len=None, out=None
         out = torch.empty(B * S, H, dtype=qk.dtype, device=qk.device)
     es = qk.element_size()
     base = qk.data_ptr()
-    if q8_inv_scale is not None:
-        out_q = torch.empty(B * S, H, dtype=torch.int8, device=qk.device)
+    if q8_inv_scale is not None or vt_key_order:
+        out_q = torch.empty(B * S, H, dtype=torch.int8, device=qk.device) if q8_inv_scale is not None else None
         capi.call("tnn_rocm_attention_vt_q8", _stream(), dt(qk), base, base + H * es, _p(vt), _p(out), _p(out_q),
-                  float(q8_inv_scale), B, heads, S, 64, S * 2 * H, 64, 2 * H, S * 2 * H, 64, 2 * H, heads * 64 * S, 64 * S, S,
-                  S * H, 64, H, float(scale), _p(mask), _p(kv_len))
-        return out, out_q
+                  float(q8_inv_scale or 0.0), B, heads, S, 64, S * 2 * H, 64, 2 * H, S * 2 * H, 64, 2 * H, heads * 64 * S,
+                  64 * S, S, S * H, 64, H, float(scale), _p(mask), _p(kv_len), int(vt_key_order))
+        return (out, out_q) if q8_inv_scale is not None else out
     capi.call("tnn_rocm_attention_vt", _stream(), dt(qk), base, base + H * es, _p(vt), _p(out), B, heads, S, 64,
               S * 2 * H, 64, 2 * H, S * 2 * H, 64, 2 * H, heads * 64 * S, 64 * S, S, S * H, 64, H, float(scale),
               _p(mask), _p(kv_len))
