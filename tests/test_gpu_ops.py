@@ -939,15 +939,16 @@ def test_store_through_switch_changes_no_result():
     assert rel_err(host(through[1]), ref) <= FP16_TOL
 
 
+@pytest.mark.parametrize("S,order", [(328, 0), (336, 1)])
 @pytest.mark.parametrize("dtype,tol", [("f16", FP16_TOL), ("bf16", 3e-2)])
-def test_attention_vt_scores_that_outgrow_the_running_reference(dtype, tol):
+def test_attention_vt_scores_that_outgrow_the_running_reference(dtype, tol, S, order):
     """The V^T kernel keeps a running reference for the exponentials that only moves when a score outgrows it by a
     margin.  Keys whose scores jump by far more than that margin from one 64-key tile to the next (both upwards and
     downwards), a ragged last tile, a length-1 and a length-0 sequence, without and with an additive mask given as
     data, against the checker."""
-    say("attention V^T kernel, score jumps across key tiles, " + dtype)
+    say("attention V^T kernel, score jumps across key tiles, %s, S %d, key order %d" % (dtype, S, order))
     tdt = torch.float16 if dtype == "f16" else torch.bfloat16
-    B, h, S = 5, 2, 328
+    B, h = 5, 2
     H = h * 64
     rng = np.random.default_rng(77)
     q = rng.standard_normal((B, h, S, 64)).astype(np.float32) * 2
@@ -956,19 +957,23 @@ def test_attention_vt_scores_that_outgrow_the_running_reference(dtype, tol):
     gain = np.ones((B, S), np.float32) * 0.2
     gain[0, 128:] = 4.0                      # up by ~30 in the exp2 domain after two tiles
     gain[1, :128] = 4.0                      # down after two tiles
-    gain[2] = 0.2 + 6.0 * (np.arange(S) % 64 == 63) * (np.arange(S) // 64) / 5   # one outlier key per tile, growing
+    # one outlier key per tile, growing: in the second 32 keys of tiles 1 and 2 (the kernel then gives the tile up
+    # between its halves), in the first 32 keys of the later ones
+    gain[2] = 0.2 + 6.0 * (np.arange(S) % 64 == np.where(np.arange(S) // 64 < 3, 63, 5)) * (np.arange(S) // 64) / 5
     gain[3] = np.linspace(0.1, 5.0, S)
     k *= gain[:, None, :, None]
     q, k, v = (torch.from_numpy(t).to(tdt) for t in (q, k, v))
-    lens = np.array([328, 328, 300, 1, 0], np.int32)
+    lens = np.array([S, S, 300, 1, 0], np.int32)
     qk = torch.cat([q.permute(0, 2, 1, 3).reshape(B * S, H), k.permute(0, 2, 1, 3).reshape(B * S, H)], 1).contiguous()
     vt = v.permute(0, 1, 3, 2).contiguous()
+    if order:
+        vt = ops().permute_keys(vt)
     mask = np.zeros((B, S), np.float32)
     for b_, l in enumerate(lens):
         mask[b_, l:] = -np.inf
     qf, kf, vf = (t.float().numpy() for t in (q, k, v))
     ref = orc.attention_core(qf[:4], kf[:4], vf[:4], 0.125, mask[:4]).transpose(0, 2, 1, 3).reshape(4 * S, H)
-    out = host(ops().attention_qk_vt(qk.cuda(), vt.cuda(), B, S, h, 0.125, kv_len=dev(lens)))
+    out = host(ops().attention_qk_vt(qk.cuda(), vt.cuda(), B, S, h, 0.125, kv_len=dev(lens), vt_key_order=order))
     assert np.isfinite(out).all()
     err = rel_err(out[:4 * S], ref)
     say("  lengths only: max rel err %.3g" % err)
@@ -977,7 +982,7 @@ def test_attention_vt_scores_that_outgrow_the_running_reference(dtype, tol):
     # additive mask as data (a bias on some visible keys too), keys past the length still cut by kv_len
     add = (rng.standard_normal((B, S)) * 3).astype(np.float32)
     ref2 = orc.attention_core(qf[:4], kf[:4], vf[:4], 0.125, (mask + add)[:4]).transpose(0, 2, 1, 3).reshape(4 * S, H)
-    out2 = host(ops().attention_qk_vt(qk.cuda(), vt.cuda(), B, S, h, 0.125, mask=dev(add), kv_len=dev(lens)))
+    out2 = host(ops().attention_qk_vt(qk.cuda(), vt.cuda(), B, S, h, 0.125, mask=dev(add), kv_len=dev(lens), vt_key_order=order))
     err2 = rel_err(out2[:4 * S], ref2)
     say("  with additive mask: max rel err %.3g" % err2)
     assert err2 <= tol

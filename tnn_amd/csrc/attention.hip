@@ -532,10 +532,10 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
         v_off[i]    = ((uint32_t)r * vt_sd32 + (uint32_t)l_chunk[i] * 8u) * 2u;
     }
     auto load16 = [](const void *base, uint32_t byte_off, uint32_t lds_addr) {
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
     };
     auto load4 = [](const void *base, uint32_t byte_off, uint32_t lds_addr) {
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
     };
     const uint32_t wave_dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_base + (uint32_t)wave * 1024u));
     auto issue = [&](int t, int stage) {
@@ -716,7 +716,9 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
         rs  = half_swap_sum(rs);
         l_i = fmaf(l_i, alpha, rs);
     };
-    auto general_tile = [&](auto mode_tag, int t) __attribute__((always_inline)) {
+    // skip_half0 (wave-uniform): the first 32 keys of the tile are already in O and l (the FAST loop gave the tile up
+    // between its halves); their scores are replaced by -inf, so they take no part in the maximum and add nothing
+    auto general_tile = [&](auto mode_tag, int t, bool skip_half0) __attribute__((always_inline)) {
         constexpr int MODE = decltype(mode_tag)::value;  // 0 BIAS, 1 EXACT
         const unsigned char *const kbuf  = lds_all + stage * kStage;
         const unsigned char *const vtbuf = kbuf + kTile;
@@ -732,6 +734,11 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
                 u32x4 kf = *reinterpret_cast<const u32x4 *>(kbuf + kt * 32 * 128 + frag_off[kk]);
                 AttnT<DT>::mma(kf, qf[kk], sacc[kt]);
             }
+        }
+        if (skip_half0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                sacc[0][r] = -INFINITY;
         }
         float mx = -INFINITY;
         if (MODE == 0) {
@@ -787,28 +794,118 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
         accumulate(vtbuf, pf, rs, alpha);
     };
 
+    // A quarter of that (four accumulator registers: four exponentials, two packs, two additions to the row sum), for
+    // the key order in which the packed pairs need no exchange between the lane halves.  Register 4k + i of block kt is
+    // element 2*(k&1) + i/2 of the operand of P.V step 2*kt + k/2.
+    auto fast_quarter = [&](auto kt_tag, auto k_tag, f32x16 &sk, u32x4 (&pf)[4], float &rs) __attribute__((always_inline)) {
+        constexpr int kt = decltype(kt_tag)::value, k = decltype(k_tag)::value;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            sk[4 * k + i] = __builtin_amdgcn_exp2f(sk[4 * k + i]);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t w = AttnT<DT>::pack_only(sk[4 * k + 2 * h], sk[4 * k + 2 * h + 1]);
+            pf[2 * kt + (k >> 1)][2 * (k & 1) + h] = w;
+            AttnT<DT>::add_packed(w, rs);
+        }
+    };
+    // One half (32 keys, accumulator block kt) of a FAST tile: exponentials, packed operands of the two P.V steps the
+    // half feeds, and this lane's part of the row sum.
+    auto fast_half = [&](auto kt_tag, f32x16 &sk, u32x4 (&pf)[4], float &rs) __attribute__((always_inline)) {
+        constexpr int kt = decltype(kt_tag)::value;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            sk[r] = __builtin_amdgcn_exp2f(sk[r]);
+        rs = 0.f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int st = 2 * kt + j;
+            uint32_t w0 = AttnT<DT>::pack_only(sk[8 * j + 0], sk[8 * j + 1]);
+            uint32_t w1 = AttnT<DT>::pack_only(sk[8 * j + 2], sk[8 * j + 3]);
+            uint32_t w2 = AttnT<DT>::pack_only(sk[8 * j + 4], sk[8 * j + 5]);
+            uint32_t w3 = AttnT<DT>::pack_only(sk[8 * j + 6], sk[8 * j + 7]);
+            if constexpr (PERM) {
+                pf[st][0] = w0, pf[st][1] = w1, pf[st][2] = w2, pf[st][3] = w3;
+            } else {
+                auto x0 = __builtin_amdgcn_permlane32_swap(w0, w2, false, false);
+                auto x1 = __builtin_amdgcn_permlane32_swap(w1, w3, false, false);
+                pf[st][0] = x0[0], pf[st][1] = x1[0], pf[st][2] = x0[1], pf[st][3] = x1[1];
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                AttnT<DT>::add_packed(pf[st][e], rs);
+        }
+    };
+    // the two P.V steps of half kt
+    auto pv_half = [&](auto kt_tag, const unsigned char *vtbuf, u32x4 (&pf)[4]) __attribute__((always_inline)) {
+        constexpr int kt = decltype(kt_tag)::value;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt) {
+                const u32x4 vf = *reinterpret_cast<const u32x4 *>(vtbuf + dt * 32 * 128 + frag_off[2 * kt + j]);
+                AttnT<DT>::mma(vf, pf[2 * kt + j], oacc[dt]);
+            }
+    };
+
     int t = 0;
     bool entered = false;  // the FAST loop gave tile t up after entering it: the barrier of tile t is already behind us
+    bool half0_done = false;  // ... and after its first 32 keys had gone into O and l
     while (t < n_tiles) {
         if (!entered)
             enter_tile(t);
         entered = false;
         if (mb != nullptr || (t + 1) * kTileKV > kv_end)  // workgroup-uniform
-            general_tile(std::integral_constant<int, 0>(), t);
+            general_tile(std::integral_constant<int, 0>(), t, false);
         else
-            general_tile(std::integral_constant<int, 1>(), t);
+            general_tile(std::integral_constant<int, 1>(), t, half0_done);
+        half0_done = false;
         leave_tile();
         ++t;
         if (mb != nullptr || !__all(m_i > -INFINITY))  // per wave: FAST needs a finite reference
             continue;
+        // FAST tiles.  On one SIMD the matrix pipe and the vector ALU overlap only for independent instruction streams
+        // of one wave, and a tile as a whole is a dependent chain (scores -> exponentials -> P.V).  Its two 32-key
+        // halves are independent of each other, though, so they are skewed by one step:
+        //     scores 0 | scores 1 under the exponentials of half 0 | P.V 0 under the exponentials of half 1 | P.V 1
+        // with eight vector instructions behind each MFMA.  The reference is checked per half, before the half's P.V
+        // step is issued.
         while (t < n_tiles && (t + 1) * kTileKV <= kv_end) {
             enter_tile(t);
             const unsigned char *const kbuf  = lds_all + stage * kStage;
             const unsigned char *const vtbuf = kbuf + kTile;
             u32x4 pf[4];
-            float rs;
-            {
-                f32x16 sacc[2];
+            float rs0 = 0.f, rs1 = 0.f;
+            f32x16 sacc[2];
+            if constexpr (PERM) {
+                // The issue order is written out: a fence (nothing may be moved across it by the compiler) after every
+                // MFMA-plus-eight-vector-instructions step.
+                u32x4 kf[2][4];
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int kk = 0; kk < 4; ++kk)
+                        kf[kt][kk] = *reinterpret_cast<const u32x4 *>(kbuf + kt * 32 * 128 + frag_off[kk]);
+                sacc[0] = AttnT<DT>::mma_from(kf[0][0], qf[0], negm);
+#pragma unroll
+                for (int kk = 1; kk < 4; ++kk)
+                    AttnT<DT>::mma(kf[0][kk], qf[kk], sacc[0]);
+                __builtin_amdgcn_sched_barrier(0);
+                sacc[1] = AttnT<DT>::mma_from(kf[1][0], qf[0], negm);
+                fast_quarter(std::integral_constant<int, 0>(), std::integral_constant<int, 0>(), sacc[0], pf, rs0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int kk = 1; kk < 4; ++kk) {
+                    AttnT<DT>::mma(kf[1][kk], qf[kk], sacc[1]);
+                    if (kk == 1)
+                        fast_quarter(std::integral_constant<int, 0>(), std::integral_constant<int, 1>(), sacc[0], pf, rs0);
+                    else if (kk == 2)
+                        fast_quarter(std::integral_constant<int, 0>(), std::integral_constant<int, 2>(), sacc[0], pf, rs0);
+                    else
+                        fast_quarter(std::integral_constant<int, 0>(), std::integral_constant<int, 3>(), sacc[0], pf, rs0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt) {
                     u32x4 kf = *reinterpret_cast<const u32x4 *>(kbuf + kt * 32 * 128 + frag_off[0]);
@@ -819,18 +916,44 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && DT == TNN_ROCM_F16) ? 3 :
                         AttnT<DT>::mma(kf, qf[kk], sacc[kt]);
                     }
                 }
-#pragma unroll
-                for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        sacc[kt][r] = __builtin_amdgcn_exp2f(sacc[kt][r]);
-                pack_probs(sacc, pf, rs);
+                fast_half(std::integral_constant<int, 0>(), sacc[0], pf, rs0);
             }
-            if (__builtin_expect(__any(!(rs <= kStaleLimit)), 0)) {
+            if (__builtin_expect(__any(!(rs0 <= kStaleLimit)), 0)) {
                 entered = true;
                 break;
             }
-            accumulate(vtbuf, pf, rs, 1.0f);
+            if constexpr (PERM) {
+                u32x4 vf[2][2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int dt = 0; dt < 2; ++dt)
+                        vf[j][dt] = *reinterpret_cast<const u32x4 *>(vtbuf + dt * 32 * 128 + frag_off[j]);
+                __builtin_amdgcn_sched_barrier(0);
+                AttnT<DT>::mma(vf[0][0], pf[0], oacc[0]);
+                fast_quarter(std::integral_constant<int, 1>(), std::integral_constant<int, 0>(), sacc[1], pf, rs1);
+                __builtin_amdgcn_sched_barrier(0);
+                AttnT<DT>::mma(vf[0][1], pf[0], oacc[1]);
+                fast_quarter(std::integral_constant<int, 1>(), std::integral_constant<int, 1>(), sacc[1], pf, rs1);
+                __builtin_amdgcn_sched_barrier(0);
+                AttnT<DT>::mma(vf[1][0], pf[1], oacc[0]);
+                fast_quarter(std::integral_constant<int, 1>(), std::integral_constant<int, 2>(), sacc[1], pf, rs1);
+                __builtin_amdgcn_sched_barrier(0);
+                AttnT<DT>::mma(vf[1][1], pf[1], oacc[1]);
+                fast_quarter(std::integral_constant<int, 1>(), std::integral_constant<int, 3>(), sacc[1], pf, rs1);
+                __builtin_amdgcn_sched_barrier(0);
+            } else {
+                pv_half(std::integral_constant<int, 0>(), vtbuf, pf);
+                fast_half(std::integral_constant<int, 1>(), sacc[1], pf, rs1);
+            }
+            if (__builtin_expect(__any(!(rs1 <= kStaleLimit)), 0)) {
+                l_i += half_swap_sum(rs0);
+                entered    = true;
+                half0_done = true;
+                break;
+            }
+            pv_half(std::integral_constant<int, 1>(), vtbuf, pf);
+            l_i += half_swap_sum(rs0 + rs1);
             leave_tile();
             ++t;
         }

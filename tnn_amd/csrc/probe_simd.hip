@@ -15,6 +15,15 @@
 //   lds       the sixteen fragment reads alone
 //   tile      chain + fragment reads feeding the MFMAs (the whole tile)
 //   ahead     tile with every fragment requested before the first MFMA that needs one (latency taken out)
+//   pipe      the same instruction counts as chain, software-pipelined inside ONE wave: while the vector work of tile i
+//             runs, the matrix pipe is given the score MFMAs of tile i + 1 and the P.V MFMAs of tile i - 1, all on
+//             registers the vector work does not touch (one MFMA, then four vector instructions, sixteen times per
+//             tile; two register sets, the loop unrolled twice so that no set is copied).  Operands from registers.
+//   pipe+lds  pipe with the sixteen fragment reads of the MFMAs it issues, requested one group ahead
+//   skew      the overlap available INSIDE one tile, no state carried between tiles: the two 32-key halves are skewed
+//             by one step -- scores of half 0 | scores of half 1 under the vector work of half 0 | P.V of half 0 under
+//             the vector work of half 1 | P.V of half 1.  Same instruction counts as chain, operands from registers.
+//   skew+lds  skew with the fragment reads from LDS
 // Each is run with 1, 2 and 3 waves per SIMD (256 x k workgroups of four waves, one wave per SIMD each) and reported
 // as nanoseconds per tile and SIMD, i.e. the time divided by the waves per SIMD.
 #include <hip/hip_runtime.h>
@@ -26,7 +35,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-enum { MFMA_ONLY, VALU_ONLY, CHAIN, LDS_ONLY, TILE, TILE_AHEAD };
+enum { MFMA_ONLY, VALU_ONLY, CHAIN, LDS_ONLY, TILE, TILE_AHEAD, PIPE, PIPE_LDS, SKEW, SKEW_LDS };
 
 template <int MODE> __global__ void __launch_bounds__(256) probe(float *out, int iters, float seed) {
     __shared__ __attribute__((aligned(16))) unsigned char lds[32768];
@@ -162,6 +171,170 @@ template <int MODE> __global__ void __launch_bounds__(256) probe(float *out, int
         out[0] = t;
 }
 
+// The pipelined variants.  Per tile and wave: 16 MFMAs (8 for the scores of the NEXT tile into s_next, 8 for P.V of the
+// PREVIOUS tile from pf_prev into o0 / o1) and the 64 vector instructions of the CURRENT tile (32 exp2 on s_cur, 16
+// packs into pf_cur, 16 dot2 for the row sum); nothing issued in one half depends on the other half within the tile.
+// sched_group_barrier pins the order: one MFMA, four vector instructions, and so on.
+template <bool WITH_LDS> __global__ void __launch_bounds__(256) probe_pipe(float *out, int iters, float seed) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[32768];
+    for (int i = threadIdx.x; i < 8192; i += 256)
+        ((float *)lds)[i] = seed * 1e-3f * (i & 15);
+    __syncthreads();
+    const unsigned lq = threadIdx.x & 31, g = (threadIdx.x >> 5) & 1;
+    unsigned fo[4];
+    for (int x = 0; x < 4; ++x)
+        fo[x] = lq * 128 + (((2 * x + g) ^ ((lq >> 1) & 7)) * 16);
+    f32x16 o0, o1, z, sa0, sa1, sb0, sb1;
+    for (int r = 0; r < 16; ++r)
+        o0[r] = 0.f, o1[r] = 0.f, z[r] = -seed, sa0[r] = seed * r, sa1[r] = -seed * r, sb0[r] = seed, sb1[r] = seed;
+    f16x8 kreg, q;
+    for (int r = 0; r < 8; ++r)
+        kreg[r] = (_Float16)(seed * 0.01f + r * 0.001f), q[r] = (_Float16)(seed * 0.02f - r * 0.001f);
+    u32x4 pa[4], pb[4];
+    for (int st = 0; st < 4; ++st)
+        pa[st] = __builtin_bit_cast(u32x4, kreg), pb[st] = __builtin_bit_cast(u32x4, kreg);
+    float rs         = 0.f;
+    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    // one tile: vector work on (s0, s1) -> pf_cur; MFMAs: scores of the next tile -> (n0, n1), P.V of pf_prev -> o
+    auto tile = [&](int i, f32x16 &s0, f32x16 &s1, f32x16 &n0, f32x16 &n1, u32x4 (&pf_prev)[4], u32x4 (&pf_cur)[4])
+                    __attribute__((always_inline)) {
+        const unsigned char *kb = lds + (i & 1) * 16384, *vb = kb + 8192;
+        f16x8 kf[8], vf[8];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            if (WITH_LDS) {
+                kf[x] = *reinterpret_cast<const f16x8 *>(kb + (x & 1) * 4096 + fo[x >> 1]);
+                vf[x] = *reinterpret_cast<const f16x8 *>(vb + (x & 1) * 4096 + fo[x >> 1]);
+            } else {
+                kf[x] = kreg, vf[x] = kreg;
+                kf[x][x] = (_Float16)(float)(i + x);
+                vf[x][7 - x] = (_Float16)(float)(i - x);
+            }
+        }
+        n0 = z, n1 = z;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            n0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[2 * x], q, n0, 0, 0, 0);
+            n1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[2 * x + 1], q, n1, 0, 0, 0);
+        }
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            const f16x8 p = __builtin_bit_cast(f16x8, pf_prev[st]);
+            o0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[2 * st], p, o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[2 * st + 1], p, o1, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            s0[r] = __builtin_amdgcn_exp2f(s0[r]), s1[r] = __builtin_amdgcn_exp2f(s1[r]);
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            f32x16 &s = st < 2 ? s0 : s1;
+            const int j = st & 1;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                pf_cur[st][e] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(s[8 * j + 2 * e], s[8 * j + 2 * e + 1]));
+                rs = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pf_cur[st][e]), ones, rs, false);
+            }
+        }
+        // the issue order: (LDS reads first,) then one MFMA followed by four vector instructions, sixteen times
+        if (WITH_LDS)
+            __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);  // DS reads
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // VALU
+        }
+    };
+    for (int i = 0; i < iters; i += 2) {
+        tile(i, sa0, sa1, sb0, sb1, pb, pa);      // vector work on set a; scores into set b; P.V from the pairs of b
+        tile(i + 1, sb0, sb1, sa0, sa1, pa, pb);  // and the other way round
+    }
+    float t = rs;
+    for (int r = 0; r < 16; ++r)
+        t += o0[r] + o1[r] + sa0[r] + sb0[r] + sa1[r] + sb1[r];
+    if (t == 12345.678f)
+        out[0] = t;
+}
+
+// Half-tile skew: see the variant list at the top.
+template <bool WITH_LDS> __global__ void __launch_bounds__(256) probe_skew(float *out, int iters, float seed) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[32768];
+    for (int i = threadIdx.x; i < 8192; i += 256)
+        ((float *)lds)[i] = seed * 1e-3f * (i & 15);
+    __syncthreads();
+    const unsigned lq = threadIdx.x & 31, g = (threadIdx.x >> 5) & 1;
+    unsigned fo[4];
+    for (int x = 0; x < 4; ++x)
+        fo[x] = lq * 128 + (((2 * x + g) ^ ((lq >> 1) & 7)) * 16);
+    f32x16 o0, o1, z, s0, s1;
+    for (int r = 0; r < 16; ++r)
+        o0[r] = 0.f, o1[r] = 0.f, z[r] = -seed;
+    f16x8 kreg, q;
+    for (int r = 0; r < 8; ++r)
+        kreg[r] = (_Float16)(seed * 0.01f + r * 0.001f), q[r] = (_Float16)(seed * 0.02f - r * 0.001f);
+    float rs         = 0.f;
+    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    for (int i = 0; i < iters; ++i) {
+        const unsigned char *kb = lds + (i & 1) * 16384, *vb = kb + 8192;
+        f16x8 kf[8], vf[8];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            if (WITH_LDS) {
+                kf[x] = *reinterpret_cast<const f16x8 *>(kb + (x >> 2) * 4096 + fo[x & 3]);   // half x/4, k-step x%4
+                vf[x] = *reinterpret_cast<const f16x8 *>(vb + (x & 1) * 4096 + fo[x >> 1]);   // step x/2, d block x%2
+            } else {
+                kf[x] = kreg, vf[x] = kreg;
+                kf[x][x] = (_Float16)(float)(i + x);
+                vf[x][7 - x] = (_Float16)(float)(i - x);
+            }
+        }
+        u32x4 pf[4];
+        s0 = z, s1 = z;
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+            s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[x], q, s0, 0, 0, 0);
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+            s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[4 + x], q, s1, 0, 0, 0);
+        auto softmax_half = [&](f32x16 &s, int half) __attribute__((always_inline)) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                s[r] = __builtin_amdgcn_exp2f(s[r]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    pf[2 * half + j][e] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(s[8 * j + 2 * e], s[8 * j + 2 * e + 1]));
+                    rs = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pf[2 * half + j][e]), ones, rs, false);
+                }
+        };
+        softmax_half(s0, 0);
+        softmax_half(s1, 1);
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            const f16x8 p = __builtin_bit_cast(f16x8, pf[st]);
+            o0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[2 * st], p, o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[2 * st + 1], p, o1, 0, 0, 0);
+        }
+        // issue order: (reads,) 4 MFMA [scores 0]; 4 x {MFMA [scores 1], 8 VALU [half 0]}; 4 x {MFMA [P.V 0], 8 VALU
+        // [half 1]}; 4 MFMA [P.V 1]
+        if (WITH_LDS)
+            __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    }
+    float t = rs;
+    for (int r = 0; r < 16; ++r)
+        t += o0[r] + o1[r] + s0[r] + s1[r];
+    if (t == 12345.678f)
+        out[0] = t;
+}
+
 template <int MODE> double ns_per_tile_and_simd(int waves_per_simd, int iters) {
     float *d = nullptr;
     if (hipMalloc(&d, 4) != hipSuccess)
@@ -170,10 +343,22 @@ template <int MODE> double ns_per_tile_and_simd(int waves_per_simd, int iters) {
     (void)hipEventCreate(&e0);
     (void)hipEventCreate(&e1);
     dim3 grid(256 * waves_per_simd), block(256);
-    hipLaunchKernelGGL((probe<MODE>), grid, block, 0, 0, d, 10, 0.5f);
+    auto launch = [&](int n) {
+        if (MODE == PIPE)
+            hipLaunchKernelGGL((probe_pipe<false>), grid, block, 0, 0, d, n, 0.5f);
+        else if (MODE == PIPE_LDS)
+            hipLaunchKernelGGL((probe_pipe<true>), grid, block, 0, 0, d, n, 0.5f);
+        else if (MODE == SKEW)
+            hipLaunchKernelGGL((probe_skew<false>), grid, block, 0, 0, d, n, 0.5f);
+        else if (MODE == SKEW_LDS)
+            hipLaunchKernelGGL((probe_skew<true>), grid, block, 0, 0, d, n, 0.5f);
+        else
+            hipLaunchKernelGGL((probe<(MODE >= PIPE ? (int)CHAIN : MODE)>), grid, block, 0, 0, d, n, 0.5f);
+    };
+    launch(10);
     (void)hipDeviceSynchronize();
     (void)hipEventRecord(e0);
-    hipLaunchKernelGGL((probe<MODE>), grid, block, 0, 0, d, iters, 0.5f);
+    launch(iters);
     (void)hipEventRecord(e1);
     (void)hipEventSynchronize(e1);
     float ms = 0.f;
@@ -187,11 +372,14 @@ template <int MODE> double ns_per_tile_and_simd(int waves_per_simd, int iters) {
 int main() {
     const int iters = 20000;
     printf("ns per tile and SIMD (time of one wave's tile divided by the waves sharing the SIMD)\n");
-    printf("%-11s %9s %9s %9s %9s %9s %9s\n", "waves/SIMD", "mfma", "valu", "chain", "lds", "tile", "ahead");
+    printf("%-11s %9s %9s %9s %9s %9s %9s %9s %9s %9s %9s\n", "waves/SIMD", "mfma", "valu", "chain", "lds", "tile", "ahead",
+           "pipe", "pipe+lds", "skew", "skew+lds");
     for (int w = 1; w <= 3; ++w)
-        printf("%-11d %9.1f %9.1f %9.1f %9.1f %9.1f %9.1f\n", w, ns_per_tile_and_simd<MFMA_ONLY>(w, iters),
+        printf("%-11d %9.1f %9.1f %9.1f %9.1f %9.1f %9.1f %9.1f %9.1f %9.1f %9.1f\n", w, ns_per_tile_and_simd<MFMA_ONLY>(w, iters),
                ns_per_tile_and_simd<VALU_ONLY>(w, iters), ns_per_tile_and_simd<CHAIN>(w, iters),
                ns_per_tile_and_simd<LDS_ONLY>(w, iters), ns_per_tile_and_simd<TILE>(w, iters),
-               ns_per_tile_and_simd<TILE_AHEAD>(w, iters));
+               ns_per_tile_and_simd<TILE_AHEAD>(w, iters), ns_per_tile_and_simd<PIPE>(w, iters),
+               ns_per_tile_and_simd<PIPE_LDS>(w, iters), ns_per_tile_and_simd<SKEW>(w, iters),
+               ns_per_tile_and_simd<SKEW_LDS>(w, iters));
     return 0;
 }
