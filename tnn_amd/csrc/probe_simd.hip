@@ -26,9 +26,15 @@
 //   skew+lds  skew with the fragment reads from LDS
 // Each is run with 1, 2 and 3 waves per SIMD (256 x k workgroups of four waves, one wave per SIMD each) and reported
 // as nanoseconds per tile and SIMD, i.e. the time divided by the waves per SIMD.
+// A second table gives the matrix rate the whole chip sustains: one wave per SIMD that issues nothing but independent
+// MFMAs (sixteen accumulators, eight operand fragments loaded once), about a millisecond per launch, with operands that
+// are all zero, all one, or normally distributed.  The power the matrix pipe draws depends on the operand bits, and the
+// clock follows the power: that rate, not the data-sheet figure, is what a GEMM main loop can be held against.
 #include <hip/hip_runtime.h>
 
+#include <cmath>
 #include <cstdio>
+#include <cstdlib>
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -335,6 +341,76 @@ template <bool WITH_LDS> __global__ void __launch_bounds__(256) probe_skew(float
         out[0] = t;
 }
 
+__global__ void __launch_bounds__(256) matrix_rate(const u32x4 *__restrict__ operands, float *out, int iters) {
+    f16x8 a[4], b[4];
+    for (int i = 0; i < 4; ++i) {
+        a[i] = __builtin_bit_cast(f16x8, operands[(i * 2 + 0) * 64 + (threadIdx.x & 63)]);
+        b[i] = __builtin_bit_cast(f16x8, operands[(i * 2 + 1) * 64 + (threadIdx.x & 63)]);
+    }
+    f32x16 acc[4][4];
+    for (int i = 0; i < 4; ++i)
+        for (int j = 0; j < 4; ++j)
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[j], a[i], acc[i][j], 0, 0, 0);
+    }
+    float t = 0.f;
+    for (int i = 0; i < 4; ++i)
+        for (int j = 0; j < 4; ++j)
+            for (int r = 0; r < 16; ++r)
+                t += acc[i][j][r];
+    if (t == 12345.678f)
+        out[0] = t;
+}
+
+// PFLOP/s of the chip with every SIMD issuing MFMAs only; data: 0 zeros, 1 ones, 2 normal (sigma 0.5 x sigma 0.02, the
+// scale of activations times weights)
+double matrix_rate_pflops(int data) {
+    const int n = 8 * 64 * 8;  // eight fragments of 64 lanes x 8 halves
+    _Float16 *h = (_Float16 *)malloc(n * sizeof(_Float16));
+    unsigned long long st = 88172645463325252ull;
+    auto uni = [&]() {
+        st = st * 6364136223846793005ull + 1442695040888963407ull;
+        return (double)((st >> 11) + 1) / 9007199254740994.0;
+    };
+    for (int i = 0; i < n; ++i) {
+        const double g = sqrt(-2.0 * log(uni())) * cos(6.283185307179586 * uni());
+        const bool is_b = (i / 512) & 1;
+        h[i] = data == 0 ? (_Float16)0.f : data == 1 ? (_Float16)1.f : (_Float16)(g * (is_b ? 0.02 : 0.5));
+    }
+    u32x4 *d = nullptr;
+    float *o = nullptr;
+    if (hipMalloc(&d, n * sizeof(_Float16)) != hipSuccess || hipMalloc(&o, 4) != hipSuccess)
+        return -1.0;
+    (void)hipMemcpy(d, h, n * sizeof(_Float16), hipMemcpyHostToDevice);
+    free(h);
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    const int iters = 4000, reps = 6;  // 64 000 MFMAs per wave and launch: about 0.8 ms
+    dim3 grid(256), block(256);
+    hipLaunchKernelGGL(matrix_rate, grid, block, 0, 0, d, o, iters);
+    (void)hipDeviceSynchronize();
+    (void)hipEventRecord(e0);
+    for (int r = 0; r < reps; ++r)
+        hipLaunchKernelGGL(matrix_rate, grid, block, 0, 0, d, o, iters);
+    (void)hipEventRecord(e1);
+    (void)hipEventSynchronize(e1);
+    float ms = 0.f;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    (void)hipFree(d);
+    (void)hipFree(o);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    const double flop = 1024.0 * 16.0 * iters * reps * 32768.0;  // 1024 waves x 16 MFMAs x 32*32*16*2
+    return flop / (ms * 1e-3) / 1e15;
+}
+
 template <int MODE> double ns_per_tile_and_simd(int waves_per_simd, int iters) {
     float *d = nullptr;
     if (hipMalloc(&d, 4) != hipSuccess)
@@ -381,5 +457,12 @@ int main() {
                ns_per_tile_and_simd<TILE_AHEAD>(w, iters), ns_per_tile_and_simd<PIPE>(w, iters),
                ns_per_tile_and_simd<PIPE_LDS>(w, iters), ns_per_tile_and_simd<SKEW>(w, iters),
                ns_per_tile_and_simd<SKEW_LDS>(w, iters));
+    printf("\nmatrix rate of the chip, one wave per SIMD issuing independent MFMAs 32x32x16 f16 only (PFLOP/s; the clock it implies\n"
+           "at 1024 FLOP per clock and SIMD over 1024 SIMDs)\n");
+    const char *names[3] = {"operands all zero", "operands all one", "operands normally distributed"};
+    for (int data = 0; data < 3; ++data) {
+        const double pf = matrix_rate_pflops(data);
+        printf("%-32s %6.3f PFLOP/s   %5.2f GHz\n", names[data], pf, pf * 1e15 / (1024.0 * 1024.0) / 1e9);
+    }
     return 0;
 }
