@@ -738,6 +738,45 @@ def test_encoder_int32_mask_input_builds_the_additive_mask_in_the_graph(precisio
 
 
 @pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_reading_comprehension_demo_shape(precision):
+    """The shape the reference's BERT demo feeds (examples/linux/src/BertReadingComprehension/BertReadingComprehension.cc:
+    43, 73 and examples/base/bert_tokenizer.cc:351-355): one sequence of 256 tokens, ids / 0-1 mask / segment ids as
+    NC_INT32 Mats of dims [1, 256], BERT-base width.  A padded question + paragraph: 141 valid tokens, segment 1 after
+    the first 17."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: demo shape [1, 256], " + precision)
+    cfg = EncoderConfig(2, 768, 12, 3072)
+    w = make_weights(cfg, seed=91, bias_std=0.05)
+    B, S, valid = 1, 256, 141
+    w["pos_emb"] = w["pos_emb"][:S]
+    rng = np.random.default_rng(92)
+    ids = np.zeros((B, S), np.int32)
+    ids[0, :valid] = rng.integers(1, cfg.vocab, size=valid)
+    seg = np.zeros((B, S), np.int32)
+    seg[0, 17:valid] = 1
+    m01 = np.zeros((B, S), np.int32)
+    m01[0, :valid] = 1
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S, int_mask=True), precision)
+    types = [t for t, _ in inst.layers()]
+    if precision == "fp16":
+        assert types.count("RocmFusedAttention") == cfg.layers, types
+    inst.set_input("input_ids", ids)
+    inst.set_input("token_type_ids", seg)
+    inst.set_input("input_mask", m01)
+    for _ in range(4):   # the fourth forward replays the recorded graph
+        inst.forward()
+    out = inst.output("last_hidden")
+    inst.close()
+    assert out.shape == (B, S, cfg.hidden)
+    mask = ((1 - m01) * -10000.0).astype(np.float32)
+    wr = r16w(w) if precision == "fp16" else w
+    ref = encoder_ref.encoder(wr, cfg, encoder_ref.embed(wr, ids, seg, cfg.eps), B, S, mask)
+    err = rel_err(out.reshape(B * S, -1)[:valid], ref[:valid])
+    say("  valid rows against the checker: max rel err %.3g" % err)
+    assert err <= (FP16_TOL if precision == "fp16" else FP32_ASSERT)
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
 def test_encoder_position_ids_input_third_gather(precision):
     """Exports that keep the position ids a model input look the positions up with a third Gather.  Same result as the
     graph that adds the first S rows of the table; permuted position ids give the permuted table rows."""
