@@ -21,6 +21,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+SUSTAINED_FP16_TFLOPS = 1692.0  # measured: MFMA-only loop on every SIMD, normally distributed operands (the SIMD probe)
 
 # HBM bytes per launch (fetched + written) of the projection GEMMs at the batch-8 / seq-384 workload, from two
 # rocprofv3 --pmc runs of this command (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
@@ -284,6 +285,13 @@ def main():
                      "timed_over": "%d back-to-back launches between two events on the launch stream, right after "
                                    "the timed region (which replays a captured graph)" % n_gemm,
                      "flops_per_launch": gemm_flops[dominant],
+                     "sustained_matrix_rate": {
+                         "tflops": SUSTAINED_FP16_TFLOPS, "frac": round(achieved / SUSTAINED_FP16_TFLOPS, 4),
+                         "what": "what the chip holds with every SIMD issuing nothing but independent fp16 MFMAs on normally "
+                                 "distributed operands (2474 on all-zero ones): power management, not the kernel, sets it; "
+                                 "context only, frac above stays on the data-sheet peak",
+                         "source": "profiles/simd_probe_mfma_valu_lds.txt (python -m tnn_amd.bench_ops --simd-probe), typed into "
+                                   "bench.py, not measured by this run"},
                      "all_gemms_us_per_launch": {k: round(v * 1e3, 2) for k, v in sorted(gemm_ms.items())},
                      "all_gemms_tflops": {k: round(gemm_flops[k] / (v * 1e-3) / 1e12, 1) for k, v in sorted(gemm_ms.items())}},
         "roofline_int8": roof_i8,
