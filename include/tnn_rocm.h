@@ -329,6 +329,14 @@ TNN_ROCM_API int tnn_rocm_quantize(void *stream, int src_dtype, const void *x, f
                                    size_t count);
 /* x = (float)q * scale     X86Int8ToFloat  x86_compute_int8.cc:1193-1252 */
 TNN_ROCM_API int tnn_rocm_dequantize(void *stream, const int8_t *q, float scale, int dst_dtype, void *x, size_t count);
+/* The same two with one scale per channel: element i of a [batch, channels, inner] blob takes entry (i / inner) % channels
+ * of a device array of `channels` fp32 values (inverse scales for the quantiser, prepared by the host as above).
+ *       X86FloatToInt8 / X86Int8ToFloat take the scale array and the channel count  x86_compute_int8.cc:1193-1318 ;
+ *       per-channel blob scales as the int8 unit tests generate them  layer_resource_generator.cc:348-371 */
+TNN_ROCM_API int tnn_rocm_quantize_per_channel(void *stream, int src_dtype, const void *x, const float *inv_scale, int8_t *q,
+                                               size_t count, int channels, size_t inner);
+TNN_ROCM_API int tnn_rocm_dequantize_per_channel(void *stream, const int8_t *q, const float *scale, int dst_dtype, void *x,
+                                                 size_t count, int channels, size_t inner);
 /* int8 Add, X86MatrixAddInt8 (x86_compute_int8.cc:795-831; scales x86_add_layer_acc.cc:33-66) as the reference's x86
  * build evaluates it (-mfma -ffast-math contract one product into the sum): y = float2int8(fma(b, sb, a*sa) * inv_so)
  * in the 8-channel vector body, float2int8(fma(a, sa, b*sb) * inv_so) in the scalar tail, i.e. the last four

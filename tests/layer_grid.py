@@ -219,6 +219,18 @@ def add_int8_cases(rng):
                    precisions=("fp16",))
 
 
+# ---- Reformat: test_reformat_layer.cc:22-55 (the harness skips it off DEVICE_ARM; the grid is run here all the same:
+# the layer is what stands on either side of every quantised layer of the path)
+def reformat_cases(rng):
+    for batch, ch, size, src in itertools.product(*BASIC_BATCH_CHANNEL_SIZE, (DT_INT8, DT_FLOAT)):
+        dims = [batch, ch, size, size]
+        dst = DT_FLOAT if src == DT_INT8 else DT_INT8
+        g = _single("Reformat", "Reformat", [dims], [src, dst])
+        _blob_scale(g, "input0" if src == DT_INT8 else "output0", ch, rng)
+        values = int8_values(rng, dims, 8) if src == DT_INT8 else grid_values(rng, dims, 1.0)
+        yield Case("Reformat", "%s_src%d" % ("x".join(map(str, dims)), src), g, {"input0": values}, int8=True)
+
+
 # ---- Reshape / Squeeze / Unsqueeze: test_reshape_layer.cc:27-87, test_squeeze_layer.cc:32-98, test_unsqueeze_layer.cc
 def reshape_cases(rng):
     for batch, ch, size, nd, rtype in itertools.product(*BASIC_BATCH_CHANNEL_SIZE, (2, 3, 4, 5, 6), (0, 1)):
@@ -283,6 +295,7 @@ GRIDS = {
     "Mul": lambda rng: binary_cases(rng, "Mul"),
     "Div": lambda rng: binary_cases(rng, "Div"),
     "QuantizedAdd": add_int8_cases,
+    "Reformat": reformat_cases,
     "Reshape": reshape_cases,
     "Squeeze": squeeze_cases,
     "Unsqueeze": unsqueeze_cases,

@@ -333,6 +333,28 @@ def test_dequantize_and_add_i8_bit_exact():
     assert np.array_equal(got, orc.add_int8_x86(a, sa, q, sb, so))
 
 
+@pytest.mark.parametrize("dims", [(2, 10, 9, 9), (1, 32, 19, 19), (3, 4, 16), (5, 7)])
+def test_quantize_and_dequantize_with_one_scale_per_channel(dims):
+    """Blob scales with one entry per channel (axis 1), as the reference's int8 unit tests generate them and its Reformat
+    kernels take them (x86_compute_int8.cc:1193-1318): every channel's slice equals the per-tensor routine of the
+    checker with that channel's scale, bit for bit."""
+    say("per-channel quantize / dequantize %s" % (dims,))
+    rng = np.random.default_rng(sum(dims))
+    C = dims[1]
+    scales = rng.uniform(0.01, 1.0, size=C).astype(np.float32)
+    inv = (1.0 / scales.astype(np.float64)).astype(np.float32)
+    x = (rng.standard_normal(dims) * 20).astype(np.float32) * scales.reshape((1, C) + (1,) * (len(dims) - 2))
+    x.reshape(-1)[:: 7] = (np.round(x.reshape(-1)[:: 7] / 0.5) * 0.5).astype(np.float32)
+    q = host(ops().quantize_per_channel(dev(x), dev(inv)))
+    back = host(ops().dequantize_per_channel(dev(q), dev(scales)))
+    for c in range(C):
+        sl = (slice(None), c)
+        assert np.array_equal(q[sl], orc.quantize_x86(np.ascontiguousarray(x[sl]).reshape(-1), scales[c]).reshape(q[sl].shape)), c
+        assert np.array_equal(back[sl], orc.dequantize(np.ascontiguousarray(q[sl]).reshape(-1), scales[c]).reshape(q[sl].shape)), c
+    h = ops().dequantize_per_channel(dev(q), dev(scales), torch.float16).cpu().numpy()
+    assert np.array_equal(h, back.astype(np.float16))
+
+
 @pytest.mark.parametrize("n,offset", [(15, 0), (16, 0), (4099, 0), (4099, 1), (100000, 3)])
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
 def test_dequantize_and_add_i8_tails_and_unaligned_buffers(n, offset, dtype):

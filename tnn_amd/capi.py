@@ -71,6 +71,8 @@ SIGNATURES = {
     "tnn_rocm_cast": [_vp, _i, _vp, _i, _vp, _sz],
     "tnn_rocm_quantize": [_vp, _i, _vp, _f, _vp, _sz],
     "tnn_rocm_dequantize": [_vp, _vp, _f, _i, _vp, _sz],
+    "tnn_rocm_quantize_per_channel": [_vp, _i, _vp, _vp, _vp, _sz, _i, _sz],
+    "tnn_rocm_dequantize_per_channel": [_vp, _vp, _vp, _i, _vp, _sz, _i, _sz],
     "tnn_rocm_debug_set_gemm_config": [_i],
     "tnn_rocm_debug_set_gemm_tune": [C.c_char_p],
     "tnn_rocm_debug_set_gemm_group_m": [_i],

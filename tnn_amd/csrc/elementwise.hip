@@ -355,6 +355,27 @@ __global__ void __launch_bounds__(kBlock) dequantize_kernel(const int8_t *__rest
         Elem<DT>::st(&x[i], __fmul_rn((float)q[i], scale));
 }
 
+// one scale per channel (a device array of `channels` values; element i belongs to channel (i / inner) % channels): the
+// blob scales the reference's int8 unit tests generate, and what its Reformat kernels take (x86_compute_int8.cc:1193-1318)
+template <int DT>
+__global__ void __launch_bounds__(kBlock) quantize_per_channel_kernel(const typename Elem<DT>::type *__restrict__ x,
+                                                                      const float *__restrict__ inv, int8_t *__restrict__ q,
+                                                                      size_t n, unsigned channels, size_t inner) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        q[i] = float2int8_ref(__fmul_rn(Elem<DT>::ld(&x[i]), inv[(i / inner) % channels]));
+}
+
+template <int DT>
+__global__ void __launch_bounds__(kBlock) dequantize_per_channel_kernel(const int8_t *__restrict__ q,
+                                                                        const float *__restrict__ scale,
+                                                                        typename Elem<DT>::type *__restrict__ x, size_t n,
+                                                                        unsigned channels, size_t inner) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        Elem<DT>::st(&x[i], __fmul_rn((float)q[i], scale[(i / inner) % channels]));
+}
+
 // sixteen values per lane and access; value for value the scalar kernel's arithmetic
 template <int DT>
 __global__ void __launch_bounds__(kBlock) dequantize_vec_kernel(const int8_t *__restrict__ q, float scale,
@@ -889,6 +910,60 @@ int tnn_rocm_dequantize(void *stream, const int8_t *q, float scale, int ddt, voi
                                n);
             break;
         default: set_error("dequantize: unsupported destination dtype %d", ddt); return TNN_ROCM_EDTYPE;
+    }
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+int tnn_rocm_quantize_per_channel(void *stream, int sdt, const void *x, const float *inv_scale, int8_t *q, size_t n,
+                                  int channels, size_t inner) {
+    if (n == 0)
+        return 0;
+    TR_REQUIRE(x && q && inv_scale, TNN_ROCM_EINVAL, "quantize_per_channel: null pointer");
+    TR_REQUIRE(channels >= 1 && inner >= 1, TNN_ROCM_EINVAL, "quantize_per_channel: channels %d, inner %zu", channels, inner);
+    hipStream_t s = (hipStream_t)stream;
+    const int g   = grid_for(n);
+    switch (sdt) {
+        case TNN_ROCM_F32:
+            hipLaunchKernelGGL(quantize_per_channel_kernel<TNN_ROCM_F32>, dim3(g), dim3(kBlock), 0, s, (const float *)x,
+                               inv_scale, q, n, (unsigned)channels, inner);
+            break;
+        case TNN_ROCM_F16:
+            hipLaunchKernelGGL(quantize_per_channel_kernel<TNN_ROCM_F16>, dim3(g), dim3(kBlock), 0, s, (const half_t *)x,
+                               inv_scale, q, n, (unsigned)channels, inner);
+            break;
+        case TNN_ROCM_BF16:
+            hipLaunchKernelGGL(quantize_per_channel_kernel<TNN_ROCM_BF16>, dim3(g), dim3(kBlock), 0, s,
+                               (const bf16_bits *)x, inv_scale, q, n, (unsigned)channels, inner);
+            break;
+        default: set_error("quantize_per_channel: unsupported source dtype %d", sdt); return TNN_ROCM_EDTYPE;
+    }
+    TR_CHECK_LAUNCH();
+    return 0;
+}
+
+int tnn_rocm_dequantize_per_channel(void *stream, const int8_t *q, const float *scale, int ddt, void *x, size_t n,
+                                    int channels, size_t inner) {
+    if (n == 0)
+        return 0;
+    TR_REQUIRE(x && q && scale, TNN_ROCM_EINVAL, "dequantize_per_channel: null pointer");
+    TR_REQUIRE(channels >= 1 && inner >= 1, TNN_ROCM_EINVAL, "dequantize_per_channel: channels %d, inner %zu", channels, inner);
+    hipStream_t s = (hipStream_t)stream;
+    const int g   = grid_for(n);
+    switch (ddt) {
+        case TNN_ROCM_F32:
+            hipLaunchKernelGGL(dequantize_per_channel_kernel<TNN_ROCM_F32>, dim3(g), dim3(kBlock), 0, s, q, scale, (float *)x,
+                               n, (unsigned)channels, inner);
+            break;
+        case TNN_ROCM_F16:
+            hipLaunchKernelGGL(dequantize_per_channel_kernel<TNN_ROCM_F16>, dim3(g), dim3(kBlock), 0, s, q, scale,
+                               (half_t *)x, n, (unsigned)channels, inner);
+            break;
+        case TNN_ROCM_BF16:
+            hipLaunchKernelGGL(dequantize_per_channel_kernel<TNN_ROCM_BF16>, dim3(g), dim3(kBlock), 0, s, q, scale,
+                               (bf16_bits *)x, n, (unsigned)channels, inner);
+            break;
+        default: set_error("dequantize_per_channel: unsupported destination dtype %d", ddt); return TNN_ROCM_EDTYPE;
     }
     TR_CHECK_LAUNCH();
     return 0;

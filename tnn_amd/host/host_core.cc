@@ -1133,7 +1133,8 @@ Status DefaultNetwork::InitLayers() {
         auto param = info->param.get();
         std::vector<Blob *> ins, outs;
         auto want_int8 = [&](bool is_input, size_t idx) -> bool {  // default_network.cc:362-440
-            return quantized_net && RocmBlobIsInt8(info->type, param, is_input, idx, info->outputs.size());
+            return (quantized_net || info->type == LAYER_REFORMAT) &&
+                   RocmBlobIsInt8(info->type, param, is_input, idx, info->outputs.size());
         };
         for (size_t i = 0; i < info->inputs.size(); ++i) {
             const auto &name = info->inputs[i];

@@ -471,19 +471,42 @@ public:
         for (size_t i = 0; i < inputs.size(); ++i) {
             size_t count = (size_t)DimsVectorUtils::Count(outputs[i]->GetBlobDesc().dims);
             DataType st = inputs[i]->GetBlobDesc().data_type, dt = outputs[i]->GetBlobDesc().data_type;
-            if (mode_ == kQuant) {
-                auto b8 = dynamic_cast<BlobInt8 *>(outputs[i]);
-                if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1 || !IsFloatType(st))
-                    return Status(TNNERR_LAYER_ERR, "Reformat(quant) needs a float blob and a per-tensor blob scale");
-                float s   = b8->GetIntResource()->scale_handle.force_to<float *>()[0];
-                float inv = (float)(1.0 / s);  // x86_reformat_layer_acc.cc:70 : double division, stored as float
-                ROCM_CALL(tnn_rocm_quantize(Stream(), (int)st, Ptr(inputs[i]), inv, (int8_t *)Ptr(outputs[i]), count));
-            } else if (mode_ == kDequant) {
-                auto b8 = dynamic_cast<BlobInt8 *>(inputs[i]);
-                if (!b8 || !b8->GetIntResource() || b8->GetIntResource()->scale_handle.GetDataCount() != 1 || !IsFloatType(dt))
-                    return Status(TNNERR_LAYER_ERR, "Reformat(dequant) needs a per-tensor blob scale and a float blob");
-                float s = b8->GetIntResource()->scale_handle.force_to<float *>()[0];
-                ROCM_CALL(tnn_rocm_dequantize(Stream(), (const int8_t *)Ptr(inputs[i]), s, (int)dt, Ptr(outputs[i]), count));
+            if (mode_ == kQuant || mode_ == kDequant) {
+                // the int8 side's blob scale: one value, or one per channel (dims[1]) as x86_reformat_layer_acc.cc:50-80
+                // prepares them (reciprocals for the quantiser: a double division stored as float)
+                auto b8 = dynamic_cast<BlobInt8 *>(mode_ == kQuant ? outputs[i] : inputs[i]);
+                if (!b8 || !b8->GetIntResource() || !IsFloatType(mode_ == kQuant ? st : dt))
+                    return Status(TNNERR_LAYER_ERR, "Reformat needs a float blob on one side and an int8 blob with a scale on the other");
+                const auto &dims   = outputs[i]->GetBlobDesc().dims;
+                const int channels = dims.size() > 1 ? dims[1] : 1;
+                const size_t inner = dims.size() > 2 ? (size_t)DimsVectorUtils::Count(dims, 2) : 1;
+                const int ns       = b8->GetIntResource()->scale_handle.GetDataCount();
+                const float *hs    = b8->GetIntResource()->scale_handle.force_to<float *>();
+                if (ns != 1 && ns < channels)
+                    return Status(TNNERR_LAYER_ERR, "Reformat: the int8 blob has fewer scales than channels");
+                if (ns != 1) {
+                    if (i >= chan_scale_.size())
+                        chan_scale_.resize(i + 1, nullptr), chan_count_.resize(i + 1, 0);
+                    if (!chan_scale_[i] || chan_count_[i] != channels) {
+                        std::vector<float> host((size_t)channels);
+                        for (int c = 0; c < channels; ++c)
+                            host[c] = mode_ == kQuant ? (float)(1.0 / hs[c]) : hs[c];
+                        chan_scale_[i] = nullptr;
+                        RETURN_ON_NEQ(UploadConverted(host.data(), host.size(), DATA_TYPE_FLOAT, DATA_TYPE_FLOAT, &chan_scale_[i]), TNN_OK);
+                        chan_count_[i] = channels;
+                    }
+                    if (mode_ == kQuant)
+                        ROCM_CALL(tnn_rocm_quantize_per_channel(Stream(), (int)st, Ptr(inputs[i]), (const float *)chan_scale_[i],
+                                                                (int8_t *)Ptr(outputs[i]), count, channels, inner > 0 ? inner : 1));
+                    else
+                        ROCM_CALL(tnn_rocm_dequantize_per_channel(Stream(), (const int8_t *)Ptr(inputs[i]), (const float *)chan_scale_[i],
+                                                                  (int)dt, Ptr(outputs[i]), count, channels, inner > 0 ? inner : 1));
+                } else if (mode_ == kQuant) {
+                    float inv = (float)(1.0 / hs[0]);  // x86_reformat_layer_acc.cc:70 : double division, stored as float
+                    ROCM_CALL(tnn_rocm_quantize(Stream(), (int)st, Ptr(inputs[i]), inv, (int8_t *)Ptr(outputs[i]), count));
+                } else {
+                    ROCM_CALL(tnn_rocm_dequantize(Stream(), (const int8_t *)Ptr(inputs[i]), hs[0], (int)dt, Ptr(outputs[i]), count));
+                }
             } else if (IsFloatType(st) && IsFloatType(dt)) {
                 ROCM_CALL(tnn_rocm_cast(Stream(), (int)st, Ptr(inputs[i]), (int)dt, Ptr(outputs[i]), count));
             } else {
@@ -495,6 +518,8 @@ public:
 
 private:
     enum { kQuant, kDequant, kCast } mode_ = kCast;
+    std::vector<void *> chan_scale_;  // per blob pair: the per-channel scales (reciprocals for the quantiser) on the device
+    std::vector<int> chan_count_;
 };
 REGISTER_ROCM_ACC(RocmReformatLayerAcc, LAYER_REFORMAT);
 

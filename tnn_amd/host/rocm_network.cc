@@ -77,7 +77,10 @@ Status RocmNetwork::InitLayers(NetStructure *net_structure, NetResource *net_res
                 Blob *blob = blob_manager_->GetBlob(names[i]);
                 if (!blob)
                     return Status(TNNERR_PARAM_ERR, "layer " + info->name + " names a blob the blob manager does not have");
-                if (quantized_net && RocmBlobIsInt8(info->type, info->param.get(), side == 0, i, info->outputs.size())) {
+                // a Reformat's blobs follow its src / dst type in any net (default_network.cc:404-421), the others' only in a
+                // quantised one
+                if ((quantized_net || info->type == LAYER_REFORMAT) &&
+                    RocmBlobIsInt8(info->type, info->param.get(), side == 0, i, info->outputs.size())) {
                     if (!dynamic_cast<BlobInt8 *>(blob))
                         RETURN_ON_NEQ(GenerateInt8Blob(names[i], net_resource, &blob), TNN_OK);
                     blob->GetBlobDesc().data_type = DATA_TYPE_INT8;

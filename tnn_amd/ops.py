@@ -359,6 +359,31 @@ def dequantize(q, scale, dtype=torch.float32):
     return x
 
 
+def _channel_layout(t):
+    channels = t.shape[1] if t.dim() >= 2 else 1
+    inner = 1
+    for d in t.shape[2:]:
+        inner *= d
+    return channels, inner
+
+
+def quantize_per_channel(x, inv_scales):
+    """x in the blob's own dims (axis 1 = channels); inv_scales: fp32 device tensor of x.shape[1] reciprocal scales"""
+    _chk(x, inv_scales)
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    channels, inner = _channel_layout(x)
+    capi.call("tnn_rocm_quantize_per_channel", _stream(), dt(x), _p(x), _p(inv_scales), _p(q), x.numel(), channels, inner)
+    return q
+
+
+def dequantize_per_channel(q, scales, dtype=torch.float32):
+    _chk(q, scales)
+    x = torch.empty(q.shape, dtype=dtype, device=q.device)
+    channels, inner = _channel_layout(q)
+    capi.call("tnn_rocm_dequantize_per_channel", _stream(), _p(q), _p(scales), _DT[dtype], _p(x), q.numel(), channels, inner)
+    return x
+
+
 def add_i8(a, sa, b, sb, inv_so):
     """a, b in the blob's own dims: axis 1 is the channel axis the reference's loop walks."""
     _chk(a, b)
