@@ -281,6 +281,49 @@ def unsqueeze_cases(rng):
                    {"input0": grid_values(rng, dims, 1.0)})
 
 
+# ---- Gather and Cast: the reference has no unit test for either; these two grids are this repository's own, over the
+# parameters the layers take (cpu_gather_layer_acc.cc:27-86: axis, data and / or indices as a resource, negative
+# indices; cpu_cast_layer_acc.cc:41-53: float <-> int32), judged against DEVICE_NAIVE like the others
+def gather_cases(rng):
+    for dims in ([12, 7], [5, 6, 9], [2, 3, 4, 5]):
+        for axis in range(len(dims)):
+            for idx_dims in ([4], [2, 3], [1]):
+                n = dims[axis]
+                idx = rng.integers(-n, n, size=idx_dims).astype(np.int32)
+                for data_res, idx_res, as_int in itertools.product((0, 1), (0, 1), (0, 1)):
+                    if as_int and not data_res and axis:   # one int32 data blob per shape is enough
+                        continue
+                    data = (rng.integers(-1000, 1000, size=dims).astype(np.int32) if as_int else grid_values(rng, dims, 1.0))
+                    in_dims, in_types, inputs = [], [], {}
+                    if not data_res:
+                        inputs["input%d" % len(in_dims)] = data
+                        in_dims.append(dims)
+                        in_types.append(DT_INT32 if as_int else DT_FLOAT)
+                    if not idx_res:
+                        inputs["input%d" % len(in_dims)] = idx
+                        in_dims.append(idx_dims)
+                        in_types.append(DT_INT32)
+                    if not in_dims:   # a layer needs an input blob: both as resources is not a graph the engine runs
+                        continue
+                    g = _single("Gather", "layer_name", in_dims, [axis, data_res, idx_res], in_types)
+                    g.res_gather("layer_name", data if data_res else None, idx if idx_res else None)
+                    ident = "d%s_a%d_i%s_r%d%d%s" % ("x".join(map(str, dims)), axis, "x".join(map(str, idx_dims)), data_res, idx_res,
+                                                    "_int32" if as_int else "")
+                    case = Case("Gather", ident, g, inputs)
+                    case.expect = (data, idx, axis)   # numpy.take(data, idx, axis) is the result
+                    yield case
+
+
+def cast_cases(rng):
+    for dims in ([7], [3, 5], [2, 3, 16], [1, 4, 9, 9]):
+        x = grid_values(rng, dims, 40.0)
+        g = _single("Cast", "layer_name", [dims], [DT_INT32])
+        yield Case("Cast", "%s_to_int32" % "x".join(map(str, dims)), g, {"input0": x})
+        xi = rng.integers(-2000, 2000, size=dims).astype(np.int32)
+        g = _single("Cast", "layer_name", [dims], [DT_FLOAT], [DT_INT32])
+        yield Case("Cast", "%s_to_float" % "x".join(map(str, dims)), g, {"input0": xi})
+
+
 GRIDS = {
     "MatMul": matmul_cases,
     "InnerProduct": inner_product_cases,
@@ -296,6 +339,8 @@ GRIDS = {
     "Div": lambda rng: binary_cases(rng, "Div"),
     "QuantizedAdd": add_int8_cases,
     "Reformat": reformat_cases,
+    "Gather": gather_cases,
+    "Cast": cast_cases,
     "Reshape": reshape_cases,
     "Squeeze": squeeze_cases,
     "Unsqueeze": unsqueeze_cases,

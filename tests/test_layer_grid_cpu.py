@@ -37,12 +37,12 @@ def test_comparison_rules():
 
 @pytest.mark.skipif(not ref_driver.available(), reason="oracle/_ref (the reference engine) was not built")
 @pytest.mark.parametrize("op", ["MatMul", "InnerProduct", "QuantizedInnerProduct", "Softmax", "LayerNorm", "GELU", "Permute",
-                                "Add", "Div", "QuantizedAdd", "Reformat", "Reshape", "Squeeze", "Unsqueeze"])
+                                "Add", "Cast", "Div", "QuantizedAdd", "Reformat", "Reshape", "Squeeze", "Unsqueeze"])
 def test_sampled_cases_run_on_the_reference_engine(op):
     rng = np.random.default_rng(7)
     ran = 0
     for i, case in enumerate(layer_grid.GRIDS[op](rng)):
-        if i % (97 if op != "Reformat" else 19) or case.inputs is None:
+        if i % ({"Reformat": 19, "Cast": 1}.get(op, 97)) or case.inputs is None:
             continue
         outs = []
         for device in ("NAIVE", "X86"):
@@ -51,9 +51,33 @@ def test_sampled_cases_run_on_the_reference_engine(op):
                 s.set_input(name, arr)
             s.forward()
             dt = s.output_data_type("output0")
-            outs.append(s.output_as("output0", np.int8 if dt == layer_grid.DT_INT8 else np.float32))
+            outs.append(s.output_as("output0", np.int8 if dt == layer_grid.DT_INT8 else
+                                    (np.int32 if dt == layer_grid.DT_INT32 else np.float32)))
             s.close()
         why = layer_grid.compare(outs[0], outs[1], dt)
         assert why is None, (case.ident, why)
         ran += 1
     assert ran > 0
+
+
+@pytest.mark.skipif(not ref_driver.available(), reason="oracle/_ref (the reference engine) was not built")
+def test_gather_grid_on_the_reference_engine_is_numpy_take():
+    """The Gather grid is this repository's own (the reference has no unit test for the layer): on DEVICE_NAIVE every
+    case equals numpy's take with the negative indices wrapped (cpu_gather_layer_acc.cc:74-77; the reference's x86 acc
+    refuses negative indices, x86_gather_layer_acc.cc:66-70, so it is not the second device here)."""
+    rng = np.random.default_rng(7)
+    ran = 0
+    for i, case in enumerate(layer_grid.GRIDS["Gather"](rng)):
+        if i % 3:
+            continue
+        s = ref_driver.RefSession(case.graph, "NAIVE")
+        for name, arr in case.inputs.items():
+            s.set_input(name, arr)
+        s.forward()
+        dt = s.output_data_type("output0")
+        out = s.output_as("output0", np.int32 if dt == layer_grid.DT_INT32 else np.float32)
+        s.close()
+        data, idx, axis = case.expect
+        assert np.array_equal(out, np.take(data, idx, axis=axis)), case.ident
+        ran += 1
+    assert ran > 20
