@@ -49,7 +49,14 @@ REF_API void *tnn_ref_create(const char *proto, size_t proto_len, const char *mo
         return nullptr;
     }
     NetworkConfig nc;
-    const std::string dev(device);
+    std::string dev(device);
+    // "+extmem" behind the device: the caller brings the blob memory (SHARE_MEMORY_MODE_SET_FROM_EXTERNAL,
+    // Instance::GetForwardMemorySize / SetForwardMemory)
+    const size_t ext = dev.find("+extmem");
+    if (ext != std::string::npos) {
+        dev.erase(ext);
+        nc.share_memory_mode = SHARE_MEMORY_MODE_SET_FROM_EXTERNAL;
+    }
     nc.device_type  = dev == "X86" ? DEVICE_X86 : DEVICE_NAIVE;
     nc.network_type = NETWORK_TYPE_DEFAULT;
     nc.precision    = PRECISION_HIGH;
@@ -95,6 +102,27 @@ REF_API int tnn_ref_set_input(void *h, const char *name, const void *data, int m
         }
     if (!known)
         s->inputs.push_back({name, mat});
+    return 0;
+}
+
+// blob memory brought by the caller (a pointer the session's device can use): instance.cc GetForwardMemorySize / SetForwardMemory
+REF_API int tnn_ref_forward_memory_size(void *h, int *bytes) {
+    Session *s = static_cast<Session *>(h);
+    Status st  = s->inst->GetForwardMemorySize(*bytes);
+    if (st != TNN_OK) {
+        s->err = st.description();
+        return (int)st;
+    }
+    return 0;
+}
+
+REF_API int tnn_ref_set_forward_memory(void *h, void *memory) {
+    Session *s = static_cast<Session *>(h);
+    Status st  = s->inst->SetForwardMemory(memory);
+    if (st != TNN_OK) {
+        s->err = st.description();
+        return (int)st;
+    }
     return 0;
 }
 

@@ -24,6 +24,8 @@ def lib():
         _lib.tnn_ref_destroy.argtypes = [C.c_void_p]
         _lib.tnn_ref_set_input.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]
         _lib.tnn_ref_forward.argtypes = [C.c_void_p]
+        _lib.tnn_ref_forward_memory_size.argtypes = [C.c_void_p, C.POINTER(C.c_int)]
+        _lib.tnn_ref_set_forward_memory.argtypes = [C.c_void_p, C.c_void_p]
         _lib.tnn_ref_get_output.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
                                             C.POINTER(C.c_int)]
         _lib.tnn_ref_get_output_as.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
@@ -62,6 +64,14 @@ class RefSession:
 
     def forward(self):
         self._check(lib().tnn_ref_forward(self.h), "Forward")
+
+    def forward_memory_size(self):
+        n = C.c_int(0)
+        self._check(lib().tnn_ref_forward_memory_size(self.h, C.byref(n)), "GetForwardMemorySize")
+        return n.value
+
+    def set_forward_memory(self, pointer):
+        self._check(lib().tnn_ref_set_forward_memory(self.h, C.c_void_p(pointer)), "SetForwardMemory")
 
     def output(self, name, max_elems=1 << 26):
         buf = np.empty(max_elems, np.float32)

@@ -264,3 +264,40 @@ def test_model_input_shared_by_quantised_and_float_layers():
     d = np.abs(rocm[0] - x86)
     say("  max |d| vs DEVICE_X86 %.3g (one int8 step of the output scale is 0.05)" % d.max())
     assert d.max() <= 1e-6
+
+
+def test_blob_memory_brought_by_the_caller():
+    """SHARE_MEMORY_MODE_SET_FROM_EXTERNAL (include/tnn/core/common.h, instance.cc GetForwardMemorySize /
+    SetForwardMemory, blob_manager.cc): the engine allocates no blob memory, reports the size, and the caller hands over
+    device memory; blobs are then base + bytes_offset into it.  Same result as the engine-allocated run, also after the
+    memory is exchanged for another buffer between forwards (the recorded graph names the old addresses and must not be
+    replayed)."""
+    engine()
+    import torch
+    say("reference engine: DEVICE_ROCM with blob memory brought by the caller")
+    cfg = EncoderConfig.bert_base(2)
+    w = make_weights(cfg, seed=43, bias_std=0.02)
+    B, S = 2, 64
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 20, S, seed=44)
+    graph = tnnmodel.encoder_graph(cfg, w, B, S)
+    inputs = {"input_ids": ids.astype(np.int32), "token_type_ids": seg.astype(np.int32),
+              "attention_bias": mask.reshape(B, 1, 1, S).astype(np.float32)}
+    for device in ("ROCM:fp32", "ROCM"):
+        plain = run(graph, device, inputs, "last_hidden")[0]
+        s = ref_driver.RefSession(graph, device + "+extmem")
+        size = s.forward_memory_size()
+        say("  %s: forward memory %d bytes" % (device, size))
+        assert size > 0
+        first = torch.full((size + 256,), 0x5a, dtype=torch.uint8, device="cuda")
+        second = torch.full((size + 256,), 0xa5, dtype=torch.uint8, device="cuda")
+        outs = []
+        for buf, forwards in ((first, 4), (second, 4), (first, 1)):
+            base = (buf.data_ptr() + 255) // 256 * 256
+            s.set_forward_memory(base)
+            for name, arr in inputs.items():
+                s.set_input(name, arr)
+            for _ in range(forwards):
+                s.forward()
+                outs.append(s.output("last_hidden"))
+        s.close()
+        assert all(np.array_equal(o, plain) for o in outs), device
