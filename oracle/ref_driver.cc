@@ -35,9 +35,39 @@ extern "C" {
 
 #define REF_API __attribute__((visibility("default")))
 
+// "name:d0,d1,...;name:..." -> InputShapesMap
+static InputShapesMap parse_shapes(const char *spec) {
+    InputShapesMap m;
+    std::string s(spec ? spec : "");
+    size_t pos = 0;
+    while (pos < s.size()) {
+        size_t end = s.find(';', pos);
+        if (end == std::string::npos)
+            end = s.size();
+        const std::string item = s.substr(pos, end - pos);
+        const size_t colon     = item.find(':');
+        if (colon != std::string::npos) {
+            DimsVector d;
+            size_t p = colon + 1;
+            while (p < item.size()) {
+                size_t q = item.find(',', p);
+                if (q == std::string::npos)
+                    q = item.size();
+                d.push_back(atoi(item.substr(p, q - p).c_str()));
+                p = q + 1;
+            }
+            m[item.substr(0, colon)] = d;
+        }
+        pos = end + 1;
+    }
+    return m;
+}
+
 // device: "NAIVE", "X86", or "ROCM" / "ROCM:fp32" (see below).  Returns nullptr and fills err on failure.
-REF_API void *tnn_ref_create(const char *proto, size_t proto_len, const char *model, size_t model_len,
-                             const char *device, int threads, char *err, size_t err_len) {
+// min_shapes / max_shapes ("name:d0,d1;..."; both empty: the model's own shapes): the ranges Instance::Reshape may move in
+REF_API void *tnn_ref_create_shaped(const char *proto, size_t proto_len, const char *model, size_t model_len,
+                                    const char *device, int threads, const char *min_shapes, const char *max_shapes,
+                                    char *err, size_t err_len) {
     std::unique_ptr<Session> s(new Session);
     ModelConfig mc;
     mc.model_type = MODEL_TYPE_TNN;
@@ -69,7 +99,8 @@ REF_API void *tnn_ref_create(const char *proto, size_t proto_len, const char *mo
         nc.network_type = NETWORK_TYPE_AUTO;  // RocmDevice::ConvertAutoNetworkType() names the backend's network
         nc.precision    = dev == "ROCM:fp32" ? PRECISION_HIGH : (dev == "ROCM:bf16" ? PRECISION_LOW : PRECISION_AUTO);
     }
-    s->inst         = s->net.CreateInst(nc, st);
+    const InputShapesMap lo = parse_shapes(min_shapes), hi = parse_shapes(max_shapes);
+    s->inst = hi.empty() ? s->net.CreateInst(nc, st) : s->net.CreateInst(nc, st, lo.empty() ? hi : lo, hi);
     if (st != TNN_OK || !s->inst) {
         put_err(err, err_len, "TNN::CreateInst: " + st.description());
         return nullptr;
@@ -79,7 +110,24 @@ REF_API void *tnn_ref_create(const char *proto, size_t proto_len, const char *mo
     return s.release();
 }
 
+REF_API void *tnn_ref_create(const char *proto, size_t proto_len, const char *model, size_t model_len,
+                             const char *device, int threads, char *err, size_t err_len) {
+    return tnn_ref_create_shaped(proto, proto_len, model, model_len, device, threads, "", "", err, err_len);
+}
+
 REF_API void tnn_ref_destroy(void *h) { delete static_cast<Session *>(h); }
+
+// Instance::Reshape to the input shapes named ("name:d0,d1;...")
+REF_API int tnn_ref_reshape(void *h, const char *shapes) {
+    Session *s = static_cast<Session *>(h);
+    Status st  = s->inst->Reshape(parse_shapes(shapes));
+    if (st != TNN_OK) {
+        s->err = st.description();
+        return (int)st;
+    }
+    s->inputs.clear();
+    return 0;
+}
 
 // mat_type: 0 = NCHW_FLOAT (fp32 data), 1 = NC_INT32 (int32 data), 2 = RESERVED_INT8_TEST (int8 data copied as it is
 // into an int8 blob: what the reference's layer unit tests feed quantised layers with, layer_test.cc:258-261)

@@ -21,6 +21,10 @@ def lib():
         _lib.tnn_ref_create.restype = C.c_void_p
         _lib.tnn_ref_create.argtypes = [C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t, C.c_char_p, C.c_int,
                                         C.c_char_p, C.c_size_t]
+        _lib.tnn_ref_create_shaped.restype = C.c_void_p
+        _lib.tnn_ref_create_shaped.argtypes = [C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t, C.c_char_p, C.c_int,
+                                               C.c_char_p, C.c_char_p, C.c_char_p, C.c_size_t]
+        _lib.tnn_ref_reshape.argtypes = [C.c_void_p, C.c_char_p]
         _lib.tnn_ref_destroy.argtypes = [C.c_void_p]
         _lib.tnn_ref_set_input.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]
         _lib.tnn_ref_forward.argtypes = [C.c_void_p]
@@ -39,12 +43,17 @@ def lib():
     return _lib
 
 
+def _shape_spec(shapes):
+    return ";".join("%s:%s" % (k, ",".join(str(int(d)) for d in v)) for k, v in (shapes or {}).items()).encode()
+
+
 class RefSession:
-    def __init__(self, graph, device="NAIVE", threads=0):
+    def __init__(self, graph, device="NAIVE", threads=0, min_shapes=None, max_shapes=None):
         proto = graph.proto().encode()
         model = graph.model()
         err = C.create_string_buffer(512)
-        self.h = lib().tnn_ref_create(proto, len(proto), model, len(model), device.encode(), threads, err, 512)
+        self.h = lib().tnn_ref_create_shaped(proto, len(proto), model, len(model), device.encode(), threads,
+                                             _shape_spec(min_shapes), _shape_spec(max_shapes), err, 512)
         if not self.h:
             raise RuntimeError("reference engine refused the model: " + err.value.decode())
         self._keep = []
@@ -61,6 +70,10 @@ class RefSession:
         self._check(lib().tnn_ref_set_input(self.h, name.encode(), a.ctypes.data_as(C.c_void_p),
                                             {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.int8): 2}[a.dtype],
                                             dims, a.ndim), "SetInputMat")
+
+    def reshape(self, shapes):
+        self._check(lib().tnn_ref_reshape(self.h, _shape_spec(shapes)), "Reshape")
+        self._keep = []
 
     def forward(self):
         self._check(lib().tnn_ref_forward(self.h), "Forward")

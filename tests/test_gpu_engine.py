@@ -301,3 +301,46 @@ def test_blob_memory_brought_by_the_caller():
                 outs.append(s.output("last_hidden"))
         s.close()
         assert all(np.array_equal(o, plain) for o in outs), device
+
+
+def test_instance_reshape_inside_the_reference_engine():
+    """Instance::Reshape of the reference engine itself (instance.cc:48-128, default_network.cc:456-500) on DEVICE_ROCM: an
+    instance created for shapes up to B4 S96 walks through several (B, S), among them a sequence length that is no
+    multiple of 8 and shapes seen before; at each shape, on each of three forwards, the result is that of the engine's
+    DEVICE_NAIVE reshaped the same way (fp32 blobs 2e-3, fp16 blobs 1e-2)."""
+    engine()
+    say("reference engine: Instance::Reshape on DEVICE_ROCM next to DEVICE_NAIVE")
+    cfg = EncoderConfig(2, 256, 4, 512)
+    S_MAX = 96
+    w = make_weights(cfg, seed=61, bias_std=0.05)
+    w["pos_emb"] = w["pos_emb"][:S_MAX]
+    # positions looked up by a third Gather: the constant-rows form names S_MAX rows, which the engine's own Add cannot
+    # broadcast against a shorter sequence
+    graph = tnnmodel.encoder_graph(cfg, w, 4, S_MAX, dynamic=True, position_ids=True)
+
+    def shapes(B, S):
+        return {"input_ids": [B, S], "token_type_ids": [B, S], "position_ids": [B, S], "attention_bias": [B, 1, 1, S]}
+
+    sessions = {d: ref_driver.RefSession(graph, d, min_shapes=shapes(1, 8), max_shapes=shapes(4, S_MAX))
+                for d in ("NAIVE", "ROCM:fp32", "ROCM")}
+    for step, (B, S) in enumerate([(4, 96), (2, 40), (3, 24), (2, 36), (4, 96), (1, 8), (2, 40)]):
+        ids, seg, lens, mask = make_inputs(cfg, B, S, max(S // 3, 1), S, seed=200 + step)
+        outs = {}
+        for d, s in sessions.items():
+            s.reshape(shapes(B, S))
+            s.set_input("input_ids", ids.astype(np.int32))
+            s.set_input("token_type_ids", seg.astype(np.int32))
+            s.set_input("position_ids", np.tile(np.arange(S, dtype=np.int32), (B, 1)))
+            s.set_input("attention_bias", mask.reshape(B, 1, 1, S).astype(np.float32))
+            res = []
+            for _ in range(1 if d == "NAIVE" else 3):
+                s.forward()
+                res.append(s.output("last_hidden"))
+            assert res[0].shape == (B, S, cfg.hidden), (d, res[0].shape)
+            assert all(np.array_equal(r, res[0]) for r in res[1:]), d
+            outs[d] = res[0]
+        e32, e16 = rel_err(outs["ROCM:fp32"], outs["NAIVE"]), rel_err(outs["ROCM"], outs["NAIVE"])
+        say("  B=%d S=%d: fp32 blobs %.3g, fp16 blobs %.3g" % (B, S, e32, e16))
+        assert e32 <= 2e-3 and e16 <= 1e-2
+    for s in sessions.values():
+        s.close()
