@@ -284,3 +284,38 @@ def test_model_input_read_by_quantised_and_float_layers_gets_a_reformat_at_the_h
     fc = [l for l in plan if "fc" in l["name"]][0]
     assert fc["inputs"][0] == "x_int8_reformat"            # the quantised reader takes the int8 copy ...
     assert "x" in by_name["res"]["inputs"]                 # ... the float reader the model input itself
+
+
+@pytest.mark.parametrize("blob", ["q_o", "qh", "kt", "scores", "scaled", "masked", "probs", "ctx_h", "ctx_s", "ctx"])
+def test_intermediate_blob_named_as_model_output_survives_the_rewrites(blob):
+    """TNN::AddOutput / an output line in the model file can name any blob of the attention block.  Whatever the
+    rewrites fold, a blob the caller asked for must still be written by some layer of the plan, with the dims the
+    un-rewritten graph gives it."""
+    g = _attention_block()
+    names = {b for l in host.plan(g, precision="fp32") for b in l["outputs"]}
+    if blob not in names:
+        pytest.skip("the block's writer does not name a blob %r" % blob)
+    want = {b: d for l in host.plan(g, precision="fp32") for b, d in zip(l["outputs"], l["output_dims"])}[blob]
+    g.add_output(blob)
+    plan = host.plan(g, precision="fp16")
+    got = {b: d for l in plan for b, d in zip(l["outputs"], l["output_dims"])}
+    assert blob in got, (blob, _types(plan))
+    assert got[blob] == want
+
+
+def test_every_encoder_blob_named_as_model_output_survives_the_rewrites():
+    """The same for the whole encoder graph, one blob at a time: embeddings, every LayerNorm output that the rewrites
+    would otherwise leave un-materialised, the FFN's GELU input and output, the residual sums."""
+    base = _graph(layers=2)[2]
+    first = host.plan(base, precision="fp32")
+    dims = {b: d for l in first for b, d in zip(l["outputs"], l["output_dims"])}
+    kept_anyway = {b for l in host.plan(base, precision="fp16") for b in l["outputs"]}
+    asked = 0
+    for blob in sorted(dims):
+        if blob in kept_anyway:
+            continue
+        g = _graph(layers=2, extra_outputs=(blob,))[2]
+        got = {b: d for l in host.plan(g, precision="fp16") for b, d in zip(l["outputs"], l["output_dims"])}
+        assert blob in got and got[blob] == dims[blob], blob
+        asked += 1
+    assert asked > 20
