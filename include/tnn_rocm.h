@@ -128,7 +128,8 @@ TNN_ROCM_API int tnn_rocm_gemm_i8(void *stream, const int8_t *A, const int8_t *W
  * K, V (kv strides) and out.  head_dim must be 64.  dtype F16 or BF16.
  *   mask   : optional additive fp32 [B, S] (broadcast over heads and query rows), e.g. 0 / -10000
  *   kv_len : optional int32 [B]; keys j >= kv_len[b] are excluded exactly (−inf) and their tiles
- *            skipped. 
+ *            skipped.  kv_len[b] = 0 (the mask routines below never produce it: a row that masks every key keeps all
+ *            of them, as the reference's softmax does) writes the sequence's output rows as zeros.
  *            (bit 30 of an entry may be set by tnn_rocm_mask_to_kv_len_flagged: mask row b is then not read). */
 TNN_ROCM_API int tnn_rocm_attention(void *stream, int dtype, const void *q, const void *k, const void *v, void *out,
                                     int B, int heads, int S, int head_dim, long q_sb, long q_sh, long q_ss, long kv_sb,
@@ -137,7 +138,11 @@ TNN_ROCM_API int tnn_rocm_attention(void *stream, int dtype, const void *q, cons
 
 /* Same computation with V supplied transposed per head, V^T[b][head][d][s] (element at
  * vt[b*vt_sb + head*vt_sh + d*vt_sd + s], s contiguous, S a multiple of 8): the layout tnn_rocm_gemm_qkv_split
- * writes, which lets the kernel stage V tiles with 16-byte copies instead of transposing them. */
+ * writes, which lets the kernel stage V tiles with 16-byte copies instead of transposing them.
+ * Precision: this form multiplies Q by scale * log2(e) in the half type before the score product (so that the scores
+ * leave the matrix pipe ready for exp2).  That second rounding of Q moves a score s by about |s| * 2^-11 / sqrt(head_dim) in
+ * the exponent: nothing next to the blob type's own rounding while |s * scale| stays below ~20, as encoder
+ * activations do, and up to 1e-2 of the output range once |s * scale| reaches ~70 (a softmax that is one-hot anyway). */
 TNN_ROCM_API int tnn_rocm_attention_vt(void *stream, int dtype, const void *q, const void *k, const void *vt, void *out,
                                        int B, int heads, int S, int head_dim, long q_sb, long q_sh, long q_ss,
                                        long k_sb, long k_sh, long k_ss, long vt_sb, long vt_sh, long vt_sd, long o_sb,

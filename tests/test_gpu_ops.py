@@ -1010,6 +1010,37 @@ def test_attention_vt_scores_that_outgrow_the_running_reference(dtype, tol, S, o
     assert err2 <= tol
 
 
+def test_attention_vt_precision_on_very_peaked_softmax():
+    """What the pre-scaled Q of the V^T kernel costs, pinned so that a change shows.  Projection weights six times the
+    usual width give scores whose scaled magnitude reaches ~70 (every softmax row is one-hot but for near ties): the
+    direct-to-LDS form, which multiplies Q by scale * log2(e) in fp16 ahead of the score product, stays within 3e-2 of
+    the checker there, the register-staged form, which scales the fp32 scores, within 2e-3; at the usual width both are
+    inside 2e-3."""
+    say("attention V^T kernel, very peaked softmax")
+    from tnn_amd import capi
+    o = ops()
+    B, S, h = 1, 192, 12
+    H = h * 64
+    for wstd, bar_dma, bar_staged in ((0.3, 3e-2, 2e-3), (0.05, 2e-3, 2e-3)):
+        rng = np.random.default_rng(53)
+        x = torch.from_numpy(rng.standard_normal((B * S, H)).astype(np.float32)).half().cuda()
+        w = torch.from_numpy((rng.standard_normal((3 * H, H)) * wstd).astype(np.float32)).half().cuda()
+        bias = dev((rng.standard_normal(3 * H) * 0.1).astype(np.float32))
+        plain = host(o.gemm(x, w, True, bias=bias)).reshape(B, S, 3, h, 64)
+        q, k, v = (np.ascontiguousarray(plain[:, :, i].transpose(0, 2, 1, 3)) for i in range(3))
+        ref = orc.attention_core(q, k, v, 0.125, np.zeros((B, S), np.float32)).transpose(0, 2, 1, 3).reshape(B * S, H)
+        qk, vt = o.qkv_split(x, w, bias, B, S, h, vt_key_order=1)
+        errs = {}
+        for dma in (1, 0):
+            capi.load().tnn_rocm_debug_set_attention_dma(dma)
+            try:
+                errs[dma] = rel_err(host(o.attention_qk_vt(qk, vt, B, S, h, 0.125, vt_key_order=1)), ref)
+            finally:
+                capi.load().tnn_rocm_debug_set_attention_dma(1)
+        say("  weight width %.2f: direct-to-LDS form %.3g, register-staged form %.3g" % (wstd, errs[1], errs[0]))
+        assert errs[1] <= bar_dma and errs[0] <= bar_staged
+
+
 def test_attention_padding_only_sequence_matches_the_reference_softmax():
     """A sequence whose mask is -10000 on every key: the reference computes softmax(scores - 10000) V = softmax(scores) V
     (in fp32 the shifted scores are quantised to 2^-10, which the fp16 bar absorbs); the kernel must do the same,
