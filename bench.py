@@ -107,11 +107,11 @@ def main():
     inst.set_input("token_type_ids", seg)
     inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
 
-    # warm-up: the first two forwards run eagerly (lazy allocations), the third records the whole-forward graph
+    # warm-up: the first forwards perform every lazy allocation (and, with TNN_ROCM_GRAPH=1, the third records the graph)
     for _ in range(max(args.warmup, 3)):
         inst.forward()
 
-    # ---- timed region: exactly K Instance::Forward() calls (graph replay + the engine's per-forward synchronise)
+    # ---- timed region: exactly K Instance::Forward() calls (the layer loop + the engine's per-forward synchronise)
     step_s = []
     inst.sync()
     t0 = time.perf_counter()
@@ -231,7 +231,7 @@ def main():
     # the dominant GEMM inside the forward: the event pair the eager layer loop puts around its layer (profile pass above),
     # averaged over the layers.  It spans from the previous layer's last kernel to this layer's last kernel on the
     # stream, i.e. the kernel plus the gap in front of it with the weights as the previous layers left them in the
-    # caches; the eager loop's host-side launch cost can widen that gap, which a graph replay does not pay.  The QKV
+    # caches; the profile pass synchronises per layer, so the host-side launch cost can widen that gap.  The QKV
     # projection shares its layer with the attention kernel and has no figure of its own.
     dom_in_forward_ms = breakdown[dominant] / cfg.layers if dominant in breakdown else None
 
@@ -261,8 +261,9 @@ def main():
         "config": {"workload": ("12-layer BERT-base encoder fp16, batch 8, seq 384, valid lengths U[200,384] "
                                 "(BASELINE.json configs[1])") if full_cfg else
                    "%d-layer BERT-base encoder fp16, batch %d, seq %d" % (args.layers, B, S),
-                   "path": "Instance::Forward on DEVICE_ROCM from .tnnproto/.tnnmodel, ROCm fusion pass on, "
-                           "whole-forward graph replay",
+                   "path": "Instance::Forward on DEVICE_ROCM from .tnnproto/.tnnmodel, ROCm fusion pass on, " +
+                           ("whole-forward graph replay" if os.environ.get("TNN_ROCM_GRAPH", "0") not in ("", "0") else
+                            "eager layer loop on one stream (graph replay behind TNN_ROCM_GRAPH=1 measured 0.5-1.8 % slower)"),
                    "layers": args.layers, "batch": B, "seq_len": S, "hidden": H, "heads": cfg.heads, "ffn": F,
                    "sum_valid_len": int(lens.sum()), "host_layers": len(layer_types)},
         "model_tflops": round(cfg.flops_per_sequence(S) * seqs_per_s / 1e12, 2),
@@ -283,7 +284,7 @@ def main():
                      "in_forward_is": "this GEMM's layer between the event pair of the eager layer loop, mean over the "
                                       "layers: kernel + the gap in front of it (frac stays on the back-to-back figure)",
                      "timed_over": "%d back-to-back launches between two events on the launch stream, right after "
-                                   "the timed region (which replays a captured graph)" % n_gemm,
+                                   "the timed region" % n_gemm,
                      "flops_per_launch": gemm_flops[dominant],
                      "sustained_matrix_rate": {
                          "tflops": SUSTAINED_FP16_TFLOPS, "frac": round(achieved / SUSTAINED_FP16_TFLOPS, 4),

@@ -9,6 +9,12 @@ if ROOT not in sys.path:
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 
+# The suite runs the host with whole-forward graph replay switched on (the library's default is the eager layer loop):
+# the replay is the path with more machinery - recording, signatures, invalidation - and the tests that compare it with
+# the eager loop set the switch themselves either way.
+os.environ.setdefault("TNN_ROCM_GRAPH", "1")
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 

@@ -217,23 +217,26 @@ def test_graph_replay_matches_eager_on_every_replay(monkeypatch):
     eager = host.RocmInstance.from_graph(g, "fp16")
     monkeypatch.setenv("TNN_ROCM_GRAPH", "1")
     graph = host.RocmInstance.from_graph(g, "fp16")
+    monkeypatch.delenv("TNN_ROCM_GRAPH")          # the library's own default (the eager loop)
+    default = host.RocmInstance.from_graph(g, "fp16")
     scratch = torch.zeros(1 << 20, device="cuda")
     for it in range(7):
         ids, seg, lens, mask = make_inputs(cfg, B, S, 20, 128, seed=100 + it)
         outs = []
-        for inst in (eager, graph):
+        for inst in (eager, graph, default):
             inst.set_input("input_ids", ids)
             inst.set_input("token_type_ids", seg)
             inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
             inst.forward()
             outs.append(inst.output("last_hidden"))
-        assert np.array_equal(outs[0], outs[1]), "replay %d differs from eager" % it
+        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2]), "replay %d differs from eager" % it
         # unrelated eager work + a device synchronisation between replays
         scratch.add_(1.0)
         assert float(scratch.sum().item()) == (it + 1) * (1 << 20)
         torch.cuda.synchronize()
     eager.close()
     graph.close()
+    default.close()
 
 
 def test_two_instances_on_two_threads_match_their_sequential_results():

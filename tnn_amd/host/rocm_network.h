@@ -1,8 +1,12 @@
-// RocmNetwork: the engine's DefaultNetwork plus whole-forward graph replay.
+// RocmNetwork: the engine's DefaultNetwork plus, behind a switch, whole-forward graph replay.
 //
 // On this device the launches of a forward pass are fixed once the instance is initialised (static shapes, stable
-// blob and workspace addresses), so after two eager passes - which also perform every lazy allocation - the third is
-// recorded into an executable graph and later calls submit it at once.  The engine picks the network implementation
+// blob and workspace addresses), so after two eager passes - which also perform every lazy allocation - the third can
+// be recorded into an executable graph that later calls submit at once (TNN_ROCM_GRAPH=1).  The default is the
+// engine's eager layer loop: with the sixty-odd launches a fused encoder is left with, the host stays ahead of the
+// device, the gaps between kernels on the device are the same either way, and submitting the recorded graph costs
+// more up front than the first eager launch (12-layer encoder, three machines: the replay is 0.5 - 1.8 % slower).
+// The replay is for callers whose host thread is slow or busy.  The engine picks the network implementation
 // per NetworkType (source/tnn/core/abstract_network.h:102-136, instance.cc:75-85); RocmDevice::ConvertAutoNetworkType()
 // names this one, and it registers itself like the engine's other networks (default_network.cc:39-40).
 #ifndef TNN_AMD_HOST_ROCM_NETWORK_H_
@@ -48,7 +52,7 @@ private:
     std::vector<Recording> recordings_;
     std::vector<uint64_t> eager_signature_;
     int eager_forwards_ = 0;
-    bool enabled_       = true;  // TNN_ROCM_GRAPH=0 keeps the eager loop
+    bool enabled_       = false;  // TNN_ROCM_GRAPH=1 turns the replay on; the default is the engine's eager loop
 };
 
 }  // namespace TNN_NS
