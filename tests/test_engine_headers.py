@@ -35,6 +35,21 @@ def test_backend_source_compiles_against_engine_headers(src, std):
     assert r.returncode == 0 and not errors, "\n".join(errors[:20]) or r.stderr[-2000:]
 
 
+CLANG = "/opt/rocm/llvm/bin/clang++"
+
+
+@pytest.mark.skipif(not os.path.exists(CLANG), reason="no clang in this image")
+@pytest.mark.parametrize("src", BACKEND_SOURCES)
+def test_backend_source_compiles_with_clang_against_engine_headers(src):
+    """a second compiler: clang rejects what g++ lets through, e.g. a constant of an engine enum whose value lies outside
+    the enum's range of values (LayerType ends at 1001, so a constant of 0x7001 is not a constant expression)"""
+    cmd = [CLANG, "-std=c++11", "-fsyntax-only", "-DTNN_ROCM_ENGINE_TREE", "-I" + os.path.join(REF, "include"),
+           "-I" + os.path.join(REF, "source"), "-I" + os.path.join(ROOT, "include"), "-I" + HOST, os.path.join(HOST, src)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    errors = [l for l in r.stderr.splitlines() if " error" in l]
+    assert r.returncode == 0 and not errors, "\n".join(errors[:20]) or r.stderr[-2000:]
+
+
 @pytest.mark.parametrize("src", BACKEND_SOURCES)
 def test_backend_source_compiles_in_a_profiler_build_of_the_engine(src):
     """-DTNN_PROFILE (the engine's TNN_PROFILER_ENABLE option, CMakeLists.txt:74-76) adds StartProfile / FinishProfile /

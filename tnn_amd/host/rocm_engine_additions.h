@@ -4,9 +4,11 @@
 // Included after the engine's headers (include/tnn/core/common.h, source/tnn/core/layer_type.h,
 // source/tnn/interpreter/layer_param.h, layer_resource.h) inside the engine tree, and after this repository's own
 // restatement of them otherwise, so the backend sources read the same in both builds.  The engine's enums are closed
-// (include/tnn/core/common.h:88-116, source/tnn/core/layer_type.h:25-260), so the new values are typed constants
-// outside every range the engine uses; a maintainer who prefers enumerators moves them into the enums and deletes
-// the constants here, nothing else changes.
+// (include/tnn/core/common.h:88-116, source/tnn/core/layer_type.h:25-260), so the new values are typed constants that
+// no enumerator of the engine uses and that lie inside each enum's range of values (a cast to a value outside it is
+// undefined, and clang rejects it in a constant expression): LayerType ends at 1001, so its range is [0, 1023];
+// NetworkType spans -1 ... 0x8000 (range up to 0xFFFF), DeviceType 0 ... 0x1070 (range up to 0x1FFF).  A maintainer who prefers enumerators moves them into the
+// enums and deletes the constants here, nothing else changes.
 #ifndef TNN_AMD_HOST_ROCM_ENGINE_ADDITIONS_H_
 #define TNN_AMD_HOST_ROCM_ENGINE_ADDITIONS_H_
 
@@ -17,14 +19,14 @@ constexpr DeviceType DEVICE_ROCM        = static_cast<DeviceType>(0x1080);
 constexpr NetworkType NETWORK_TYPE_ROCM = static_cast<NetworkType>(0x9000);
 
 // produced only by the ROCm optimizer passes (no proto spelling, so no layer interpreter)
-constexpr LayerType LAYER_ROCM_FUSED_LINEAR      = static_cast<LayerType>(0x7001);
-constexpr LayerType LAYER_ROCM_FUSED_ATTENTION   = static_cast<LayerType>(0x7002);
-constexpr LayerType LAYER_ROCM_FUSED_LINEAR_INT8 = static_cast<LayerType>(0x7003);
-constexpr LayerType LAYER_ROCM_GELU_INT8         = static_cast<LayerType>(0x7004);
-constexpr LayerType LAYER_ROCM_FUSED_EMBEDDING   = static_cast<LayerType>(0x7005);
-constexpr LayerType LAYER_ROCM_QUANT_LINEAR_GELU = static_cast<LayerType>(0x7006);
+constexpr LayerType LAYER_ROCM_FUSED_LINEAR      = static_cast<LayerType>(901);
+constexpr LayerType LAYER_ROCM_FUSED_ATTENTION   = static_cast<LayerType>(902);
+constexpr LayerType LAYER_ROCM_FUSED_LINEAR_INT8 = static_cast<LayerType>(903);
+constexpr LayerType LAYER_ROCM_GELU_INT8         = static_cast<LayerType>(904);
+constexpr LayerType LAYER_ROCM_FUSED_EMBEDDING   = static_cast<LayerType>(905);
+constexpr LayerType LAYER_ROCM_QUANT_LINEAR_GELU = static_cast<LayerType>(906);
 // LayerNorm (LayerNormLayerParam, inputs x, scale, bias) with a second, int8 output: the quantised copy of the first
-constexpr LayerType LAYER_ROCM_LAYER_NORM_QUANT  = static_cast<LayerType>(0x7007);
+constexpr LayerType LAYER_ROCM_LAYER_NORM_QUANT  = static_cast<LayerType>(907);
 
 struct RocmFusedLinearResource : public LayerResource {
     RawBuffer weight_nk;  // [N, K] fp32

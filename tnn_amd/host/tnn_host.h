@@ -130,7 +130,7 @@ typedef enum {
     PRECISION_LOW    = 2,
 } Precision;
 
-typedef enum { NETWORK_TYPE_AUTO = -1, NETWORK_TYPE_DEFAULT = 0 } NetworkType;
+typedef enum { NETWORK_TYPE_AUTO = -1, NETWORK_TYPE_DEFAULT = 0, NETWORK_TYPE_TENSORRT = 0x8000 } NetworkType;  // the engine's smallest and largest values: the enum's range is the engine's
 
 typedef enum {
     DEVICE_NAIVE = 0x0000,
@@ -303,6 +303,7 @@ enum LayerType {
     LAYER_LAYER_NORM    = 326,
     LAYER_GELU          = 327,
     LAYER_BLOB_SCALE    = 600,
+    LAYER_ANY_TYPE      = 1001,  // the engine's largest value (layer_type.h:243): the enum's range is the engine's
 };
 LayerType GlobalConvertLayerType(std::string type_str);
 
