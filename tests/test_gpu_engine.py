@@ -344,3 +344,47 @@ def test_instance_reshape_inside_the_reference_engine():
         assert e32 <= 2e-3 and e16 <= 1e-2
     for s in sessions.values():
         s.close()
+
+
+def test_sessions_inside_the_reference_engine_leave_no_memory_behind():
+    """TNN::Init + CreateInst + Forward x4 + the instance's and the interpreter's destruction, in the reference engine on
+    DEVICE_ROCM, twenty times over: the device memory in use (read from the driver) and the resident host memory stay
+    where they were after the first four rounds"""
+    engine()
+    torch = pytest.importorskip("torch")
+    say("reference engine: create / forward / destroy cycles on DEVICE_ROCM, memory in use")
+    cfg = EncoderConfig(2, 256, 4, 512)
+    w = make_weights(cfg, seed=11, bias_std=0.02)
+    B, S = 2, 64
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 20, S, seed=12)
+    graph = tnnmodel.encoder_graph(cfg, w, B, S)
+
+    def resident():
+        with open("/proc/self/statm") as f:
+            return int(f.read().split()[1]) * 4096
+
+    def in_use():
+        free, total = torch.cuda.mem_get_info()
+        return total - free
+
+    def cycle(device):
+        s = ref_driver.RefSession(graph, device)
+        s.set_input("input_ids", ids.astype(np.int32))
+        s.set_input("token_type_ids", seg.astype(np.int32))
+        s.set_input("attention_bias", mask.reshape(B, 1, 1, S).astype(np.float32))
+        for _ in range(4):
+            s.forward()
+        s.output("last_hidden")
+        s.close()
+
+    for device in ("ROCM", "ROCM:fp32"):
+        for _ in range(4):
+            cycle(device)
+        dev0, host0 = in_use(), resident()
+        for _ in range(16):
+            cycle(device)
+        dev1, host1 = in_use(), resident()
+        say("  %s: device in use %.1f -> %.1f MiB, host resident %.1f -> %.1f MiB over 16 cycles"
+            % (device, dev0 / 2**20, dev1 / 2**20, host0 / 2**20, host1 / 2**20))
+        assert dev1 - dev0 <= 2 << 20, (device, dev0, dev1)
+        assert host1 - host0 <= 4 << 20, (device, host0, host1)

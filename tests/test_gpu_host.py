@@ -919,3 +919,58 @@ def test_int8_mats_in_and_out_with_per_channel_blob_scales():
     want2, _ = orc.fc_int8(xq2.reshape(2, K), w, b, orc.fc_int8_scale(w_scale, s_out, N))
     assert np.array_equal(inst.output_as("output0", np.int8), want2)
     inst.close()
+
+
+@pytest.mark.parametrize("precision", ["fp16", "fp32"])
+def test_instances_come_and_go_without_leaving_memory_behind(precision):
+    """A serving process creates, reshapes and destroys instances for as long as it lives: after a few cycles of
+    Init + Forward (eager, eager, record, replay) + Reshape + Forward + destroy, neither the device memory in use (blob
+    pool, weights, workspace, converter buffers, recorded graphs) nor the process's resident host memory may keep
+    growing.  Device memory is read from the driver (hipMemGetInfo through torch), so allocations of this library count
+    whoever made them."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: create / reshape / forward / destroy cycles, %s: memory in use" % precision)
+    cfg = EncoderConfig(2, 256, 4, 512)
+    w = make_weights(cfg, seed=11, bias_std=0.02)
+    g = tnnmodel.encoder_graph(cfg, w, 2, 64, dynamic=True)
+    proto, model = g.proto(), g.model()
+
+    def resident():
+        with open("/proc/self/statm") as f:
+            return int(f.read().split()[1]) * 4096
+
+    def cycle():
+        inst = host.RocmInstance(proto, model, precision)
+        for rep, (b, s) in enumerate([(2, 64), (1, 32), (2, 64)]):
+            if rep:
+                inst.reshape({"input_ids": [b, s], "token_type_ids": [b, s], "attention_bias": [b, 1, 1, s]})
+            ids, seg, lens, mask = make_inputs(cfg, b, s, 10, s, seed=rep)
+            inst.set_input("input_ids", ids)
+            inst.set_input("token_type_ids", seg)
+            inst.set_input("attention_bias", mask.reshape(b, 1, 1, s))
+            for _ in range(4):
+                inst.forward()
+            inst.output("last_hidden")
+        inst.close()
+        torch.cuda.synchronize()
+
+    def device_in_use():
+        free, total = torch.cuda.mem_get_info()
+        return total - free
+
+    before = device_in_use()
+    held = [host.RocmInstance(proto, model, precision) for _ in range(8)]   # the probe sees what instances hold
+    dev_held = device_in_use()
+    for inst in held:
+        inst.close()
+    assert dev_held - before >= 8 << 20, (before, dev_held)
+    for _ in range(4):   # the runtime's own pools (streams, kernel arguments, signals) have grown to their size after these
+        cycle()
+    dev0, host0 = device_in_use(), resident()
+    for _ in range(16):
+        cycle()
+    dev1, host1 = device_in_use(), resident()
+    say("  device in use %.1f -> %.1f MiB, host resident %.1f -> %.1f MiB over 16 cycles"
+        % (dev0 / 2**20, dev1 / 2**20, host0 / 2**20, host1 / 2**20))
+    assert dev1 - dev0 <= 2 << 20, (dev0, dev1)       # the driver hands memory out in 2 MiB pieces
+    assert host1 - host0 <= 4 << 20, (host0, host1)   # one instance of this model holds far more than that
