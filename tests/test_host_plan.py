@@ -160,6 +160,67 @@ def test_error_behaviour_of_interpreter_and_layer_creation():
         host.plan("this is not a proto", model, "fp32")
 
 
+def _raw_buffer_records(model):
+    """offsets of the weight records of a model file: magic 0x0FABC0004, element type, byte length, rank, dims (objseri.h:57-77)"""
+    import struct
+    magic, out, at = struct.pack("<I", 0x0FABC0004), [], 0
+    while True:
+        at = model.find(magic, at)
+        if at < 0 or at + 16 > len(model):
+            return out
+        dt, length, rank = struct.unpack("<3i", model[at + 4:at + 16])
+        if 0 <= dt <= 6 and 0 < length <= len(model) and 0 <= rank <= 8:
+            dims = struct.unpack("<%di" % rank, model[at + 16:at + 16 + 4 * rank])
+            out.append((at, dt, length, dims))
+        at += 4
+
+
+def test_malformed_model_files_are_refused_with_a_status():
+    """Files that promise more than they hold end in a Status, never in a read beyond a buffer: a count in a layer line
+    larger than the line, a layer of the path without blobs, a weight record whose dims or element type do not fit its
+    bytes, an input line with an absurd rank.  (The parser and the passes were also run over some thousand randomly
+    damaged files under the address sanitizer; these are the kinds of damage that found something.)"""
+    import re
+    import struct
+    _, _, g = _graph(layers=1)
+    proto, model = g.proto(), g.model()
+    text = proto.decode() if isinstance(proto, bytes) else proto
+    host.plan(text, model, "fp16")  # the undamaged pair plans
+
+    def refused(t, m, why):
+        with pytest.raises(host.HostError):
+            host.plan(t, m, "fp16")
+        with pytest.raises(host.HostError):
+            host.plan(t, m, "fp32")
+
+    # counts in front of a list larger than the list: Reshape dims, Permute orders, the rank of an input
+    refused(text.replace("l0_q_4d 0 4 4 2 32 4 64 0", "l0_q_4d 0 4 2147483647 2 32 4 64 0", 1), model, "reshape count")
+    refused(text.replace("l0_qh 4 0 2 1 3", "l0_qh 2147483647 0 2 1 3", 1), model, "permute count")
+    refused(text.replace("input_ids 2 2 32 3", "input_ids 2147483647 2 32 3", 1), model, "input rank")
+    refused(text.replace("input_ids 2 2 32 3", "input_ids 2 2 32 77", 1), model, "input data type")
+    # layers of the path without an input or an output blob
+    refused(text.replace("Reshape l0_q_rs 1 1 l0_q_o l0_q_4d", "Reshape l0_q_rs 0 1 l0_q_4d", 1), model, "no input")
+    refused(text.replace("Permute l0_q_pm 1 1 l0_q_4d l0_qh", "Permute l0_q_pm 1 0 l0_q_4d", 1), model, "no output")
+    refused(text.replace("MatMul l0_q_mm 1 1 x0 l0_q_mm_o", "MatMul l0_q_mm 0 1 l0_q_mm_o", 1), model, "no input")
+    # weight records: dims that promise more (or fewer) elements than the record holds, an element type outside the format
+    records = [r for r in _raw_buffer_records(model) if len(r[3]) == 2 and r[1] == 0]
+    assert len(records) >= 6, len(records)
+    for at, dt, length, dims in records[:8]:
+        bigger = bytearray(model)
+        bigger[at + 16:at + 20] = struct.pack("<i", dims[0] * 2)
+        refused(text, bytes(bigger), "dims larger than the data")
+        smaller = bytearray(model)
+        smaller[at + 20:at + 24] = struct.pack("<i", max(dims[1] // 2, 1))
+        refused(text, bytes(smaller), "dims smaller than the data")
+    at = records[0][0]
+    alien = bytearray(model)
+    alien[at + 4:at + 8] = struct.pack("<i", 77)
+    refused(text, bytes(alien), "element type")
+    negative = bytearray(model)
+    negative[at + 16:at + 20] = struct.pack("<i", -records[0][3][0])
+    refused(text, bytes(negative), "negative dim")
+
+
 @pytest.mark.parametrize("precision", ["fp32", "fp16"])
 def test_int8_encoder_reformat_layers_are_folded(precision, monkeypatch):
     """The quantised encoder of the X86 fixture: with the int8 pass off the explicit Reformat / QuantizedInnerProduct

@@ -107,8 +107,8 @@ def plan(graph_or_proto, model=None, precision="fp16", input_shapes=None):
     rc = lib.tnn_host_plan(proto, len(proto), model, len(model), {"fp32": 0, "fp16": 1, "bf16": 2}[precision], n, names,
                            ndims, dims, out, len(out), err, 1024)
     if rc != 0:
-        raise HostError("plan failed (0x%x): %s" % (rc & 0xFFFFFFFF, err.value.decode()))
-    return _parse_io(out.value.decode().splitlines(), True)
+        raise HostError("plan failed (0x%x): %s" % (rc & 0xFFFFFFFF, err.value.decode(errors="replace")))
+    return _parse_io(out.value.decode(errors="replace").splitlines(), True)
 
 
 class RocmInstance:
@@ -130,7 +130,7 @@ class RocmInstance:
         else:
             self._h = lib.tnn_host_create(proto, len(proto), model, len(model), device_id, prec, err, 1024)
         if not self._h:
-            raise HostError("Instance::Init failed: " + err.value.decode())
+            raise HostError("Instance::Init failed: " + err.value.decode(errors="replace"))
         self._keep = []
 
     @classmethod
@@ -144,7 +144,7 @@ class RocmInstance:
 
     def _check(self, rc, what):
         if rc != 0:
-            raise HostError("%s failed (0x%x): %s" % (what, rc & 0xFFFFFFFF, load().tnn_host_last_error(self._h).decode()))
+            raise HostError("%s failed (0x%x): %s" % (what, rc & 0xFFFFFFFF, load().tnn_host_last_error(self._h).decode(errors="replace")))
 
     def set_input(self, name, arr):
         a = np.ascontiguousarray(arr)
@@ -173,7 +173,7 @@ class RocmInstance:
             if fn is None:
                 return None
             return CB(lambda user, name, typ, is_out, n, names, counts, types: fn(
-                name.decode(), typ.decode(), [(names[i].decode(), counts[i], types[i]) for i in range(n)]))
+                name.decode(errors="replace"), typ.decode(errors="replace"), [(names[i].decode(errors="replace"), counts[i], types[i]) for i in range(n)]))
         b, a = wrap(before), wrap(after)
         self._check(load().tnn_host_forward_with_callback(self._h, C.cast(b, C.c_void_p) if b else None,
                                                           C.cast(a, C.c_void_p) if a else None, None), "ForwardWithCallback")
@@ -217,13 +217,13 @@ class RocmInstance:
         return stats[0], stats[1], stats[2]
 
     def layers(self):
-        text = load().tnn_host_layer_summary(self._h).decode()
+        text = load().tnn_host_layer_summary(self._h).decode(errors="replace")
         return [tuple(line.split(" ", 1)) for line in text.splitlines() if line]
 
     def layer_io(self):
         """[{name, inputs, outputs, input_dims, output_dims}] for the layers of the optimised graph"""
         out = []
-        for line in load().tnn_host_layer_io(self._h).decode().splitlines():
+        for line in load().tnn_host_layer_io(self._h).decode(errors="replace").splitlines():
             name, ins, outs, din, dout = line.split("|")
             shape = lambda t: [[int(x) for x in b.split(",") if x] for b in t.split(";")] if t else []
             out.append({"name": name, "inputs": [x for x in ins.split(",") if x], "outputs": [x for x in outs.split(",") if x],

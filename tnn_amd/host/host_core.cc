@@ -172,6 +172,7 @@ struct ArgReader {
     const std::vector<std::string> &a;
     size_t i;
     bool has() const { return i < a.size(); }
+    size_t left() const { return i < a.size() ? a.size() - i : 0; }
     int geti(int def) { return has() ? atoi(a[i++].c_str()) : def; }
     float getf(float def) { return has() ? (float)atof(a[i++].c_str()) : def; }
 };
@@ -222,7 +223,7 @@ Status ParseLayerParam(LayerType type, const std::vector<std::string> &cfg, size
             p->axis     = r.geti(0);
             p->num_axes = r.geti(0);
             int n       = r.geti(-1);
-            if (n < 0)
+            if (n < 0 || (size_t)n > r.left())
                 return Status(TNNERR_PARAM_ERR, "ReshapeLayerInterpreter: invalid layer param");
             for (int i = 0; i < n; ++i)
                 p->shape.push_back(r.geti(0));
@@ -233,6 +234,8 @@ Status ParseLayerParam(LayerType type, const std::vector<std::string> &cfg, size
         case LAYER_PERMUTE: {
             auto p = std::make_shared<PermuteLayerParam>();
             int n  = r.geti(0);
+            if (n < 0 || (size_t)n > r.left())
+                return Status(TNNERR_PARAM_ERR, "PermuteLayerInterpreter: fewer orders than the count in front of them");
             for (int i = 0; i < n; ++i)
                 p->orders.push_back(r.geti(0));
             out = p;
@@ -250,6 +253,8 @@ Status ParseLayerParam(LayerType type, const std::vector<std::string> &cfg, size
         case LAYER_UNSQUEEZE: {  // unsqueeze_layer_interpreter.cc:22-32: count, then the axes
             auto p = std::make_shared<SqueezeLayerParam>();
             int n  = r.geti(0);
+            if (n < 0 || (size_t)n > r.left())
+                return Status(TNNERR_PARAM_ERR, "SqueezeLayerInterpreter: fewer axes than the count in front of them");
             for (int i = 0; i < n; ++i)
                 p->axes.push_back(r.geti(0));
             out = p;
@@ -294,10 +299,13 @@ public:
     }
     void GetRaw(RawBuffer &value) {
         uint32_t magic = (uint32_t)GetInt();
-        DataType dt    = (DataType)GetInt();
+        int dt_v       = GetInt();
         int length     = GetInt();
+        if (dt_v < (int)DATA_TYPE_FLOAT || dt_v > (int)DATA_TYPE_UINT32)
+            bad_ = true;  // no element type of the format (include/tnn/core/common.h:55-64)
         if (length <= 0 || bad_)
             return;
+        DataType dt = (DataType)dt_v;
         DimsVector dims;
         if (magic == kMagicV2) {
             int n = GetInt();
@@ -377,11 +385,14 @@ Status ModelInterpreter::InterpretProto(const std::string &content) {
                 shape.push_back(atoi(f[i].c_str()));
         } else if (version_magic_number_ == kMagicV2) {
             int n = atoi(f[1].c_str());
-            if ((int)f.size() < n + 2)
+            if (n < 0 || n > 16 || (int)f.size() < n + 2)
                 return Status(TNNERR_INVALID_NETCFG, "get input dims error");
             for (int i = 2; i < n + 2; ++i)
                 shape.push_back(atoi(f[i].c_str()));
-            structure_.input_data_type_map[f[0]] = (DataType)atoi(f.back().c_str());
+            const int dt = atoi(f.back().c_str());
+            if (dt < (int)DATA_TYPE_FLOAT || dt > (int)DATA_TYPE_UINT32)
+                return Status(TNNERR_INVALID_NETCFG, "input " + f[0] + " has no data type of the format");
+            structure_.input_data_type_map[f[0]] = (DataType)dt;
         } else {
             return Status(TNNERR_INVALID_MODEL, "Do not support tnn proto type");
         }
@@ -520,6 +531,10 @@ Status BaseLayer::Init(Context *context, LayerParam *param, LayerResource *resou
     output_blobs_ = outputs;
     param_        = param;
     resource_     = resource;
+    if (output_blobs_.empty())
+        return Status(TNNERR_INVALID_MODEL, "layer " + param_->name + " has no output blob");
+    if (input_blobs_.empty() && type_ != LAYER_GATHER)  // a Gather may hold both operands as resources
+        return Status(TNNERR_INVALID_MODEL, "layer " + param_->name + " has no input blob");
     RETURN_ON_NEQ(InferOutputDataType(), TNN_OK);
     RETURN_ON_NEQ(InferOutputShape(), TNN_OK);
     for (auto b : output_blobs_)
@@ -794,6 +809,8 @@ struct GatherLayer : BaseLayer {  // layer/gather_layer.cc
                 return Status(TNNERR_MODEL_ERR, "Gather resource is invalid");
             dt = r->data.GetDataType();
         } else {
+            if (input_blobs_.empty())
+                return Status(TNNERR_INVALID_MODEL, "Gather without a data blob");
             dt = input_blobs_[0]->GetBlobDesc().data_type;
         }
         output_blobs_[0]->GetBlobDesc().data_type = dt;
@@ -805,6 +822,8 @@ struct GatherLayer : BaseLayer {  // layer/gather_layer.cc
         CHECK_PARAM_NULL(p);
         if ((p->data_in_resource || p->indices_in_resource) && !r)
             return Status(TNNERR_MODEL_ERR, "Gather resource is invalid");
+        if (input_blobs_.size() < (size_t)(!p->data_in_resource) + (size_t)(!p->indices_in_resource))
+            return Status(TNNERR_INVALID_MODEL, "Gather with fewer input blobs than operands outside its resource");
         DimsVector data = p->data_in_resource ? r->data.GetBufferDims() : input_blobs_.front()->GetBlobDesc().dims;
         DimsVector idx  = p->indices_in_resource ? r->indices.GetBufferDims() : input_blobs_.back()->GetBlobDesc().dims;
         if (p->axis < 0 || p->axis >= (int)data.size())

@@ -300,6 +300,65 @@ private:
     HeadSplitFn head_split_;
 };
 
+// What the passes below take for granted when they index a layer's blob lists and read weights by the dims written
+// next to them, checked once per pass: a model file that breaks one of these (a layer of the path without input or
+// output, a weight record whose dims promise more elements than it holds) is reported as an invalid model here instead
+// of being read out of bounds further down.
+static Status RocmCheckModel(NetStructure *s, NetResource *r) {
+    for (auto &l : s->layers) {
+        if (!l || !l->param)
+            return Status(TNNERR_INVALID_MODEL, "a layer record is empty");
+        if (l->outputs.empty())
+            return Status(TNNERR_INVALID_MODEL, "layer " + l->name + " has no output blob");
+        switch (l->type) {
+            case LAYER_MATMUL: case LAYER_INNER_PRODUCT: case LAYER_ADD: case LAYER_SUB: case LAYER_MUL: case LAYER_DIV:
+            case LAYER_SOFTMAX: case LAYER_PERMUTE: case LAYER_RESHAPE: case LAYER_LAYER_NORM: case LAYER_GELU:
+            case LAYER_REFORMAT: case LAYER_CAST: case LAYER_UNSQUEEZE: case LAYER_SQUEEZE: case LAYER_TANH:
+                if (l->inputs.empty())
+                    return Status(TNNERR_INVALID_MODEL, "layer " + l->name + " has no input blob");
+                break;
+            default: break;
+        }
+    }
+    auto holds = [](const RawBuffer &b) {
+        const DimsVector d = b.GetBufferDims();
+        if (d.empty())
+            return true;  // records of the first file version carry no dims
+        long n = 1;
+        for (int v : d) {
+            if (v < 0 || (n *= v) > (1L << 31))
+                return false;
+        }
+        return n == (long)b.GetDataCount();
+    };
+    auto bad = [](const std::string &owner, const char *what) {
+        return Status(TNNERR_INVALID_MODEL, "resource of " + owner + ": the dims of " + what + " do not match its data");
+    };
+    for (auto &kv : r->resource_map) {
+        LayerResource *res = kv.second.get();
+        if (auto m = dynamic_cast<MatMulLayerResource *>(res)) {
+            if (!holds(m->weight))
+                return bad(kv.first, "the weight");
+        } else if (auto ip = dynamic_cast<InnerProductLayerResource *>(res)) {
+            if (!holds(ip->weight_handle) || !holds(ip->bias_handle) || !holds(ip->scale_handle))
+                return bad(kv.first, "weight, bias or scale");
+        } else if (auto e = dynamic_cast<EltwiseLayerResource *>(res)) {
+            if (!holds(e->element_handle))
+                return bad(kv.first, "the operand");
+        } else if (auto g = dynamic_cast<GatherLayerResource *>(res)) {
+            if (!holds(g->data) || !holds(g->indices))
+                return bad(kv.first, "data or indices");
+        } else if (auto q = dynamic_cast<IntScaleResource *>(res)) {
+            if (!holds(q->scale_handle) || !holds(q->bias_handle))
+                return bad(kv.first, "scale or bias");
+        }
+    }
+    for (auto &kv : r->constant_map)
+        if (kv.second && !holds(*kv.second))
+            return bad(kv.first, "the constant");
+    return TNN_OK;
+}
+
 class RocmFusionPass : public optimizer::NetOptimizer {
 public:
     std::string Strategy() override { return "net_optimizer_rocm_fuse_encoder"; }
@@ -309,6 +368,7 @@ public:
     }
 
     Status Optimize(NetStructure *s, NetResource *r) override {
+        RETURN_ON_NEQ(RocmCheckModel(s, r), TNN_OK);
         structure_ = s;
         resource_  = r;
         FuseEmbedding();
@@ -487,6 +547,8 @@ private:
                 if (wd.size() != 2)
                     continue;
                 int K = wd[0], N = wd[1];
+                if (K <= 0 || N <= 0 || (long)K * N != (long)mr->weight.GetDataCount())
+                    continue;
                 const std::string &mid = l->outputs[0];
                 int j = g.sole_consumer(mid);
                 const float *bias = nullptr;
@@ -859,6 +921,7 @@ public:
         return c.device_type == DEVICE_ROCM;
     }
     Status Optimize(NetStructure *s, NetResource *res) override {
+        RETURN_ON_NEQ(RocmCheckModel(s, res), TNN_OK);
         std::vector<std::shared_ptr<LayerInfo>> layers = s->layers;
         bool any_q  = false;
         for (auto &l : layers)
@@ -980,6 +1043,7 @@ public:
         return c.device_type == DEVICE_ROCM && !(e && atoi(e) == 0);
     }
     Status Optimize(NetStructure *s, NetResource *r) override {
+        RETURN_ON_NEQ(RocmCheckModel(s, r), TNN_OK);
         structure_ = s;
         resource_  = r;
         bool any_q = false;
