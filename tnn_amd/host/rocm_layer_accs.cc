@@ -229,6 +229,9 @@ public:
         for (auto b : inputs)
             ops.push_back({Ptr(In(b)), In(b)->GetBlobDesc().dims});
         if (weight_ && res) {
+            // the shape the layer derived for the resource operand must be the shape of what was uploaded
+            if ((long)DimsVectorUtils::Count(res->element_shape) != (long)res->element_handle.GetDataCount())
+                return Status(TNNERR_MODEL_ERR, "binary op: the resource operand's shape does not match its data");
             Operand w{weight_, res->element_shape};
             if (param && param->weight_input_index == 0)
                 ops.insert(ops.begin(), w);
@@ -548,8 +551,18 @@ public:
     Status Forward(const std::vector<Blob *> &inputs, const std::vector<Blob *> &outputs) override {
         auto param = dynamic_cast<GatherLayerParam *>(param_);
         auto res   = dynamic_cast<GatherLayerResource *>(resource_);
+        CHECK_PARAM_NULL(param);
+        if ((param->data_in_resource || param->indices_in_resource) && !res)
+            return Status(TNNERR_MODEL_ERR, "Gather resource is invalid");
+        if (inputs.size() < (size_t)(!param->data_in_resource) + (size_t)(!param->indices_in_resource))
+            return Status(TNNERR_MODEL_ERR, "Gather with fewer input blobs than operands outside its resource");
         DimsVector data_dims = param->data_in_resource ? res->data.GetBufferDims() : inputs.front()->GetBlobDesc().dims;
         DimsVector idx_dims  = param->indices_in_resource ? res->indices.GetBufferDims() : inputs.back()->GetBlobDesc().dims;
+        if (param->axis < 0 || param->axis >= (int)data_dims.size())
+            return Status(TNNERR_PARAM_ERR, "Gather axis out of range");
+        if ((param->data_in_resource && (long)DimsVectorUtils::Count(data_dims) != (long)res->data.GetDataCount()) ||
+            (param->indices_in_resource && (long)DimsVectorUtils::Count(idx_dims) != (long)res->indices.GetDataCount()))
+            return Status(TNNERR_MODEL_ERR, "Gather: the dims of a resource operand do not match its data");
         const void *data = param->data_in_resource ? data_ : Ptr(In(inputs.front()));
         const void *idx  = param->indices_in_resource ? indices_ : Ptr(In(inputs.back()));
         if (!param->indices_in_resource && inputs.back()->GetBlobDesc().data_type != DATA_TYPE_INT32)
