@@ -974,3 +974,64 @@ def test_instances_come_and_go_without_leaving_memory_behind(precision):
         % (dev0 / 2**20, dev1 / 2**20, host0 / 2**20, host1 / 2**20))
     assert dev1 - dev0 <= 2 << 20, (dev0, dev1)       # the driver hands memory out in 2 MiB pieces
     assert host1 - host0 <= 4 << 20, (host0, host1)   # one instance of this model holds far more than that
+
+
+def _bf16_bits(x32):
+    """float32 -> bfloat16 bit patterns, round to nearest even (finite values)"""
+    u = np.ascontiguousarray(x32, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def _bf16_to_f32(bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16", "bf16"])
+def test_half_and_bfloat16_mats_in_and_out(precision):
+    """RESERVED_FP16_TEST / RESERVED_BFP16_TEST Mats, the host types the engine's layer test feeds half-precision blobs
+    with (layer_test.cc:266-275, blob_converter_default.cc:205-208, 323-330).  In: values that the half type holds exactly
+    give, fed as a half Mat, the bits they give fed as an fp32 Mat, whatever the blob's type.  Out: the half Mat of an
+    output is the fp32 Mat of that output rounded to the half type (to nearest even), exactly."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: half / bfloat16 Mats in and out, blobs %s" % precision)
+    cfg = EncoderConfig(1, 256, 4, 512)
+    lw = make_weights(cfg, seed=5, bias_std=0.05)["layers"][0]
+    B, S, H = 2, 40, 256
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((B, S, H)).astype(np.float32)
+    mask = np.zeros((B, 1, 1, S), np.float32)
+    mask[1, 0, 0, 29:] = -10000.0
+    g = tnnmodel.attention_block_graph(lw, B, S, H, 4)
+    inst = host.RocmInstance.from_graph(g, precision)
+
+    def run(hidden, bias):
+        inst.set_input("hidden", hidden)
+        inst.set_input("attention_bias", bias)
+        inst.forward()
+        return inst.output("y")
+
+    x16 = x.astype(np.float16)
+    xb = _bf16_bits(x)
+    as_f32_of_half = run(x16.astype(np.float32), mask)
+    as_half = run(x16, mask.astype(np.float16))            # -10000 is a half value
+    assert np.array_equal(as_half, as_f32_of_half)
+    as_f32_of_bf16 = run(_bf16_to_f32(xb), mask)
+    as_bf16 = run(xb, mask)
+    assert np.array_equal(as_bf16, as_f32_of_bf16)
+    assert not np.array_equal(as_bf16, as_half)            # the two roundings of x are different inputs
+
+    y32 = inst.output("y")
+    y16 = inst.output_as("y", np.float16)
+    yb = inst.output_as("y", np.uint16)
+    assert y16.shape == y32.shape and yb.shape == y32.shape
+    assert np.array_equal(y16, y32.astype(np.float16))
+    assert np.array_equal(yb, _bf16_bits(y32))
+    # int32 blobs take no half Mat
+    inst.close()
+    cfg2 = EncoderConfig(1, 128, 2, 256)
+    w2 = make_weights(cfg2, seed=6)
+    w2["pos_emb"] = w2["pos_emb"][:16]
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg2, w2, 1, 16), precision)
+    with pytest.raises(host.HostError):
+        inst.set_input("input_ids", np.zeros((1, 16), np.float16))
+    inst.close()

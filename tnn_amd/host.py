@@ -57,7 +57,9 @@ def load():
     return _lib
 
 
-_MAT_CODE = {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.int8): 2}
+# numpy type of the host array -> Mat type of the C API; bfloat16 has no numpy type: uint16 arrays carry its bit patterns
+_MAT_CODE = {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.int8): 2, np.dtype(np.uint16): 3,
+             np.dtype(np.float16): 4}
 
 
 class HostError(RuntimeError):
@@ -148,8 +150,9 @@ class RocmInstance:
 
     def set_input(self, name, arr):
         a = np.ascontiguousarray(arr)
-        if a.dtype not in (np.float32, np.int32, np.int8):
-            raise TypeError("inputs are fp32 (NCHW_FLOAT), int32 (NC_INT32) or int8 (RESERVED_INT8_TEST) host arrays")
+        if a.dtype not in _MAT_CODE:
+            raise TypeError("inputs are fp32 (NCHW_FLOAT), int32 (NC_INT32), int8 (RESERVED_INT8_TEST), float16 "
+                            "(RESERVED_FP16_TEST) or uint16 holding bfloat16 bits (RESERVED_BFP16_TEST) host arrays")
         dims = (C.c_int * max(a.ndim, 1))(*a.shape)
         self._check(load().tnn_host_set_input(self._h, name.encode(), a.ctypes.data_as(C.c_void_p),
                                               _MAT_CODE[a.dtype], dims, a.ndim), "SetInputMat")
@@ -199,7 +202,8 @@ class RocmInstance:
         return buf[:int(np.prod(shape, dtype=np.int64))].reshape(shape).copy()
 
     def output_as(self, name, dtype, max_elems=1 << 25):
-        """the output through a Mat of the given numpy type: float32, int32, or int8 (an int8 blob's values as they are)"""
+        """the output through a Mat of the given numpy type: float32, int32, int8 (an int8 blob's values as they are),
+        float16, or uint16 (bfloat16 bit patterns)"""
         dtype = np.dtype(dtype)
         buf = np.empty(max_elems, dtype)
         dims = (C.c_int * 8)()

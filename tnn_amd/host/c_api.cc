@@ -132,8 +132,18 @@ HOST_API const char *tnn_host_last_error(void *hp) { return static_cast<Handle *
 
 // mat_type: 0 NCHW_FLOAT (fp32 host data), 1 NC_INT32, 2 RESERVED_INT8_TEST (int8 host data, copied as it is into an
 // int8 blob: blob_converter_default.cc:190-193, 347-350)
-static MatType MatTypeOf(int code) { return code == 1 ? NC_INT32 : (code == 2 ? RESERVED_INT8_TEST : NCHW_FLOAT); }
-static size_t MatElemBytes(int code) { return code == 2 ? 1 : 4; }
+// 3 RESERVED_BFP16_TEST (bfloat16 bit patterns), 4 RESERVED_FP16_TEST (IEEE half): the Mats the engine's layer test
+// feeds half-precision blobs with (layer_test.cc:266-275)
+static MatType MatTypeOf(int code) {
+    switch (code) {
+        case 1: return NC_INT32;
+        case 2: return RESERVED_INT8_TEST;
+        case 3: return RESERVED_BFP16_TEST;
+        case 4: return RESERVED_FP16_TEST;
+        default: return NCHW_FLOAT;
+    }
+}
+static size_t MatElemBytes(int code) { return code == 2 ? 1 : ((code == 3 || code == 4) ? 2 : 4); }
 
 HOST_API int tnn_host_set_input(void *hp, const char *name, const void *data, int mat_type, const int *dims, int ndims) {
     auto h = static_cast<Handle *>(hp);

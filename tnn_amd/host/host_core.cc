@@ -114,7 +114,7 @@ LayerType GlobalConvertLayerType(std::string s) {
 // ---- Mat / BlobConverter (source/tnn/core/mat.cc:70-87, utils/blob_converter_internal.cc:39-135) --
 Mat::Mat(DeviceType device_type, MatType mat_type, DimsVector dims)
     : device_type_(device_type), mat_type_(mat_type), dims_(std::move(dims)) {
-    size_t es = (mat_type == NCHW_FLOAT || mat_type == NC_INT32) ? 4 : (mat_type == RESERVED_FP16_TEST ? 2 : 1);
+    size_t es = (mat_type == NCHW_FLOAT || mat_type == NC_INT32) ? 4 : ((mat_type == RESERVED_FP16_TEST || mat_type == RESERVED_BFP16_TEST) ? 2 : 1);
     size_t n  = (size_t)DimsVectorUtils::Count(dims_) * es;
     owned_    = std::shared_ptr<char>(new char[n > 0 ? n : 1](), std::default_delete<char[]>());
     data_     = owned_.get();

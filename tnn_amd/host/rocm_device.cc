@@ -201,7 +201,11 @@ BlobMemorySizeInfo RocmDevice::Calculate(BlobDesc &desc) {
 }
 Status RocmDevice::Allocate(void **handle, MatType mat_type, DimsVector dims) {
     BlobMemorySizeInfo info;
-    info.data_type = (mat_type == NCHW_FLOAT) ? DATA_TYPE_FLOAT : (mat_type == NC_INT32 ? DATA_TYPE_INT32 : DATA_TYPE_INT8);
+    info.data_type = mat_type == NCHW_FLOAT            ? DATA_TYPE_FLOAT
+                     : mat_type == NC_INT32            ? DATA_TYPE_INT32
+                     : mat_type == RESERVED_FP16_TEST  ? DATA_TYPE_HALF
+                     : mat_type == RESERVED_BFP16_TEST ? DATA_TYPE_BFP16
+                                                       : DATA_TYPE_INT8;
     info.dims      = dims;
     return Allocate(handle, info);
 }
@@ -358,6 +362,22 @@ public:
             ROCM_CALL(tnn_rocm_memcpy_h2d(dst, mat.GetData(), count, q));
             return TNN_OK;
         }
+        if (mat.GetMatType() == RESERVED_BFP16_TEST || mat.GetMatType() == RESERVED_FP16_TEST) {
+            // host values that are bfloat16 / half already (how the engine's layer test feeds a half-precision blob:
+            // layer_test.cc:266-275; blob_converter_default.cc:323-330): copied as they are into a blob of that type,
+            // converted on the device into a float blob of another
+            const DataType mt = mat.GetMatType() == RESERVED_BFP16_TEST ? DATA_TYPE_BFP16 : DATA_TYPE_HALF;
+            if (desc.data_type != DATA_TYPE_FLOAT && desc.data_type != DATA_TYPE_HALF && desc.data_type != DATA_TYPE_BFP16)
+                return Status(TNNERR_PARAM_ERR, "a half or bfloat16 mat needs a float blob");
+            if (desc.data_type == mt) {
+                ROCM_CALL(tnn_rocm_memcpy_h2d(dst, mat.GetData(), count * 2, q));
+                return TNN_OK;
+            }
+            RETURN_ON_NEQ(Staging(count * 2), TNN_OK);
+            ROCM_CALL(tnn_rocm_memcpy_h2d(staging_, mat.GetData(), count * 2, q));
+            ROCM_CALL(tnn_rocm_cast(q, (int)mt, staging_, (int)desc.data_type, dst, count));
+            return TNN_OK;
+        }
         if (mat.GetMatType() != NCHW_FLOAT)
             return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported mat type");
         const float *src = (const float *)mat.GetData();
@@ -427,6 +447,18 @@ public:
         if (mat.GetMatType() == RESERVED_INT8_TEST && desc.data_type == DATA_TYPE_INT8) {
             ROCM_CALL(tnn_rocm_memcpy_d2h(mat.GetData(), src, count, q));
             return TNN_OK;
+        }
+        if (mat.GetMatType() == RESERVED_BFP16_TEST || mat.GetMatType() == RESERVED_FP16_TEST) {
+            // the blob's values as bfloat16 / half on the host (blob_converter_default.cc:205-208, 245-249): copied from a
+            // blob of that type, rounded to it on the device from a float blob of another
+            const DataType mt = mat.GetMatType() == RESERVED_BFP16_TEST ? DATA_TYPE_BFP16 : DATA_TYPE_HALF;
+            if (desc.data_type != DATA_TYPE_FLOAT && desc.data_type != DATA_TYPE_HALF && desc.data_type != DATA_TYPE_BFP16)
+                return Status(TNNERR_PARAM_ERR, "a half or bfloat16 mat needs a float blob");
+            if (desc.data_type == mt)
+                return ToHost(mat.GetData(), src, count * 2, q);
+            RETURN_ON_NEQ(Staging(count * 2), TNN_OK);
+            ROCM_CALL(tnn_rocm_cast(q, (int)desc.data_type, src, (int)mt, staging_, count));
+            return ToHost(mat.GetData(), staging_, count * 2, q);
         }
         if (mat.GetMatType() != NCHW_FLOAT)
             return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported mat type");
