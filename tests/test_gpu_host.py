@@ -1035,3 +1035,23 @@ def test_half_and_bfloat16_mats_in_and_out(precision):
     with pytest.raises(host.HostError):
         inst.set_input("input_ids", np.zeros((1, 16), np.float16))
     inst.close()
+
+
+def test_int32_output_blob_read_as_a_float_mat():
+    """An int32 blob fetched as an NCHW_FLOAT Mat comes out converted to float (blob_converter_default.cc:213-221), and
+    as an NC_INT32 Mat as it is: a Cast to int32 as the model's last layer."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: int32 output blob as float and as int32 Mat")
+    g = tnnmodel.Graph()
+    g.add_input("x", [2, 3, 5])
+    g.add_layer("Cast", "to_int", ["x"], ["xi"], [tnnmodel.DT_INT32])
+    g.add_output("xi")
+    inst = host.RocmInstance.from_graph(g, "fp32")
+    x = (np.random.default_rng(3).standard_normal((2, 3, 5)) * 50).astype(np.float32)
+    inst.set_input("x", x)
+    inst.forward()
+    as_int = inst.output_as("xi", np.int32)
+    as_float = inst.output("xi")
+    inst.close()
+    assert np.array_equal(as_int, x.astype(np.int32))          # Cast truncates toward zero (cpu_cast_layer_acc.cc)
+    assert as_float.dtype == np.float32 and np.array_equal(as_float, as_int.astype(np.float32))

@@ -462,7 +462,15 @@ public:
         }
         if (mat.GetMatType() != NCHW_FLOAT)
             return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported mat type");
-        if (desc.data_type == DATA_TYPE_FLOAT) {
+        if (desc.data_type == DATA_TYPE_INT32) {
+            // an int32 blob read as a float Mat: the values converted, then scale and bias as for a float blob
+            // (blob_converter_default.cc:213-221)
+            std::vector<int32_t> iv(count);
+            RETURN_ON_NEQ(ToHost(iv.data(), src, count * 4, q), TNN_OK);
+            float *out = (float *)mat.GetData();
+            for (size_t i = 0; i < count; ++i)
+                out[i] = (float)iv[i];
+        } else if (desc.data_type == DATA_TYPE_FLOAT) {
             RETURN_ON_NEQ(ToHost(mat.GetData(), src, count * 4, q), TNN_OK);
         } else if (desc.data_type == DATA_TYPE_HALF && count * 2 >= kBounceMinBytes && CpuWidensHalf()) {
             // a large half-precision blob crosses the bus as it is (half the bytes of its fp32 form) and is widened on
