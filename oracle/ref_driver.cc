@@ -14,6 +14,7 @@
 #include "tnn/core/instance.h"
 #include "tnn/core/mat.h"
 #include "tnn/core/tnn.h"
+#include "tnn/utils/blob_converter.h"
 
 using namespace TNN_NS;
 
@@ -126,6 +127,40 @@ REF_API int tnn_ref_reshape(void *h, const char *shapes) {
         return (int)st;
     }
     s->inputs.clear();
+    return 0;
+}
+
+// The flow of the reference's blob-converter unit test (test/unit_test/blob_converter_test.cc:287-349) on an input blob of
+// this session: a BlobConverter of the blob's own device takes an fp32 NCHW Mat in with per-channel scale and bias
+// (ConvertFromMat) and gives the blob back as an fp32 NCHW Mat with the same scale and bias applied again
+// (ConvertToMat).  in / out hold the blob's element count; scale / bias hold n_param values.
+REF_API int tnn_ref_input_blob_round_trip(void *h, const char *name, const float *in, const float *scale, const float *bias,
+                                          int n_param, float *out) {
+    Session *s = static_cast<Session *>(h);
+    BlobMap blobs;
+    Status st = s->inst->GetAllInputBlobs(blobs);
+    if (st != TNN_OK || blobs.find(name) == blobs.end()) {
+        s->err = st != TNN_OK ? st.description() : std::string("no input blob named ") + name;
+        return st != TNN_OK ? (int)st : -1;
+    }
+    Blob *blob = blobs[name];
+    void *queue = nullptr;
+    s->inst->GetCommandQueue(&queue);
+    MatConvertParam param;
+    param.scale.assign(scale, scale + n_param);
+    param.bias.assign(bias, bias + n_param);
+    DimsVector dims = blob->GetBlobDesc().dims;
+    BlobConverter converter(blob);
+    Mat mat_in(DEVICE_NAIVE, NCHW_FLOAT, dims, const_cast<float *>(in));
+    st = converter.ConvertFromMat(mat_in, param, queue);
+    if (st == TNN_OK) {
+        Mat mat_out(DEVICE_NAIVE, NCHW_FLOAT, dims, out);
+        st = converter.ConvertToMat(mat_out, param, queue);
+    }
+    if (st != TNN_OK) {
+        s->err = st.description();
+        return (int)st;
+    }
     return 0;
 }
 

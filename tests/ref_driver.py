@@ -28,6 +28,8 @@ def lib():
         _lib.tnn_ref_destroy.argtypes = [C.c_void_p]
         _lib.tnn_ref_set_input.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]
         _lib.tnn_ref_forward.argtypes = [C.c_void_p]
+        _lib.tnn_ref_input_blob_round_trip.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                                       C.c_void_p]
         _lib.tnn_ref_forward_memory_size.argtypes = [C.c_void_p, C.POINTER(C.c_int)]
         _lib.tnn_ref_set_forward_memory.argtypes = [C.c_void_p, C.c_void_p]
         _lib.tnn_ref_get_output.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
@@ -70,6 +72,18 @@ class RefSession:
         self._check(lib().tnn_ref_set_input(self.h, name.encode(), a.ctypes.data_as(C.c_void_p),
                                             {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.int8): 2}[a.dtype],
                                             dims, a.ndim), "SetInputMat")
+
+    def input_blob_round_trip(self, name, arr, scale, bias):
+        """fp32 NCHW Mat -> the input blob (ConvertFromMat with per-channel scale, bias) -> fp32 NCHW Mat (ConvertToMat with
+        the same scale, bias), through a BlobConverter of the blob's device"""
+        a = np.ascontiguousarray(arr, np.float32)
+        sc, bi = np.ascontiguousarray(scale, np.float32), np.ascontiguousarray(bias, np.float32)
+        assert sc.size == bi.size
+        out = np.empty_like(a)
+        self._check(lib().tnn_ref_input_blob_round_trip(self.h, name.encode(), a.ctypes.data_as(C.c_void_p),
+                                                        sc.ctypes.data_as(C.c_void_p), bi.ctypes.data_as(C.c_void_p),
+                                                        int(sc.size), out.ctypes.data_as(C.c_void_p)), "blob converter")
+        return out
 
     def reshape(self, shapes):
         self._check(lib().tnn_ref_reshape(self.h, _shape_spec(shapes)), "Reshape")

@@ -388,3 +388,34 @@ def test_sessions_inside_the_reference_engine_leave_no_memory_behind():
             % (device, dev0 / 2**20, dev1 / 2**20, host0 / 2**20, host1 / 2**20))
         assert dev1 - dev0 <= 2 << 20, (device, dev0, dev1)
         assert host1 - host0 <= 4 << 20, (device, host0, host1)
+
+
+def test_blob_converter_grid_inside_the_reference_engine():
+    """The reference's BlobConverterTest (test/unit_test/blob_converter_test.cc) for the Mat type of this path: the same
+    fp32 NCHW Mat through ConvertFromMat and ConvertToMat with per-channel scale and bias, by a BlobConverter on a
+    DEVICE_NAIVE blob and by one on a DEVICE_ROCM blob of the same dims, over the test's grid of batch, channel, size,
+    scale and bias (96 cases); the test's bar is 0.01, fp32 blobs meet it with no difference at all."""
+    engine()
+    from test_gpu_host import converter_grid
+    say("reference engine: blob converter grid, DEVICE_ROCM next to DEVICE_NAIVE")
+    rng = np.random.default_rng(10)
+    worst16 = 0.0
+    for batch, channel, size, scale, bias in converter_grid():
+        g = tnnmodel.Graph()
+        g.add_input("x", [batch, channel, size, size])
+        g.add_layer("GELU", "act", ["x"], ["y"])
+        g.add_output("y")
+        x = rng.random((batch, channel, size, size), dtype=np.float32)
+        sc = [scale * (c + 1) for c in range(channel)]
+        bi = [bias * (c + 1) for c in range(channel)]
+        outs = {}
+        for device in ("NAIVE", "ROCM:fp32", "ROCM"):
+            s = ref_driver.RefSession(g, device)
+            outs[device] = s.input_blob_round_trip("x", x, sc, bi)
+            s.close()
+        case = (batch, channel, size, scale, bias)
+        assert np.array_equal(outs["ROCM:fp32"], outs["NAIVE"]), case
+        d16 = np.abs(outs["ROCM"] - outs["NAIVE"])
+        assert np.all(d16 <= 1e-3 + 1e-3 * np.abs(outs["NAIVE"])), case     # one half rounding of the blob, then * scale
+        worst16 = max(worst16, float(d16.max()))
+    say("  fp32 blobs identical to DEVICE_NAIVE; half blobs differ by at most %.3g" % worst16)

@@ -1055,3 +1055,49 @@ def test_int32_output_blob_read_as_a_float_mat():
     inst.close()
     assert np.array_equal(as_int, x.astype(np.int32))          # Cast truncates toward zero (cpu_cast_layer_acc.cc)
     assert as_float.dtype == np.float32 and np.array_equal(as_float, as_int.astype(np.float32))
+
+
+def converter_grid():
+    """the parameter grid of the engine's BlobConverterTest for NCHW_FLOAT Mats (test/unit_test/blob_converter_test.cc:
+    154-172): batch, channel, input size, scale, bias; per-channel values scale * (c + 1), bias * (c + 1) (:287-293)"""
+    import itertools
+    return list(itertools.product((1, 2), (1, 3, 4, 16), (1, 15, 16), (0.5, 1.0), (0.0, 1.0)))
+
+
+def converter_round_trip_expected(x, scale, bias, half_blob):
+    n, c = x.shape[:2]
+    s = np.asarray(scale, np.float32).reshape(1, c, 1, 1)
+    b = np.asarray(bias, np.float32).reshape(1, c, 1, 1)
+    blob = (x * s + b).astype(np.float32)
+    if half_blob:
+        blob = blob.astype(np.float16).astype(np.float32)
+    return (blob * s + b).astype(np.float32)
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_blob_converter_scale_and_bias_grid(precision):
+    """The engine's blob-converter unit test restated for this device's Mat type: an fp32 NCHW Mat goes into the blob with
+    per-channel scale and bias and comes back out with them applied again, over the test's whole grid (96 cases).  fp32
+    blobs give exactly what fp32 arithmetic gives; half blobs that with one rounding of the blob."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: blob converter with scale and bias, 96 cases, blobs " + precision)
+    rng = np.random.default_rng(9)
+    worst = 0.0
+    for batch, channel, size, scale, bias in converter_grid():
+        g = tnnmodel.Graph()
+        g.add_input("x", [batch, channel, size, size])
+        g.add_layer("GELU", "act", ["x"], ["y"])
+        g.add_output("y")
+        inst = host.RocmInstance.from_graph(g, precision)
+        x = rng.random((batch, channel, size, size), dtype=np.float32)      # InitRandom(0, 1): blob_converter_test.cc:213
+        sc = [scale * (c + 1) for c in range(channel)]
+        bi = [bias * (c + 1) for c in range(channel)]
+        got = inst.input_blob_round_trip("x", x, sc, bi)
+        inst.close()
+        want = converter_round_trip_expected(x, sc, bi, precision == "fp16")
+        if precision == "fp32":
+            assert np.array_equal(got, want), (batch, channel, size, scale, bias)
+        else:
+            assert np.all(np.abs(got - want) <= 1e-6 + 1e-6 * np.abs(want)), (batch, channel, size, scale, bias)
+        worst = max(worst, float(np.abs(got - want).max()))
+    say("  largest difference to the expected Mat %.3g" % worst)

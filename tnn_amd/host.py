@@ -22,6 +22,8 @@ SIGNATURES = {
     "tnn_host_destroy": (None, [C.c_void_p]),
     "tnn_host_last_error": (C.c_char_p, [C.c_void_p]),
     "tnn_host_set_input": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]),
+    "tnn_host_input_blob_round_trip": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                                 C.c_void_p]),
     "tnn_host_forward": (C.c_int, [C.c_void_p]),
     "tnn_host_forward_async": (C.c_int, [C.c_void_p]),
     "tnn_host_sync": (C.c_int, [C.c_void_p]),
@@ -156,6 +158,18 @@ class RocmInstance:
         dims = (C.c_int * max(a.ndim, 1))(*a.shape)
         self._check(load().tnn_host_set_input(self._h, name.encode(), a.ctypes.data_as(C.c_void_p),
                                               _MAT_CODE[a.dtype], dims, a.ndim), "SetInputMat")
+
+    def input_blob_round_trip(self, name, arr, scale, bias):
+        """fp32 NCHW Mat -> the input blob (ConvertFromMat with per-channel scale, bias) -> fp32 NCHW Mat (ConvertToMat with
+        the same scale, bias): the flow of the engine's blob-converter unit test"""
+        a = np.ascontiguousarray(arr, np.float32)
+        sc, bi = np.ascontiguousarray(scale, np.float32), np.ascontiguousarray(bias, np.float32)
+        assert sc.size == bi.size
+        out = np.empty_like(a)
+        self._check(load().tnn_host_input_blob_round_trip(self._h, name.encode(), a.ctypes.data_as(C.c_void_p),
+                                                          sc.ctypes.data_as(C.c_void_p), bi.ctypes.data_as(C.c_void_p),
+                                                          int(sc.size), out.ctypes.data_as(C.c_void_p)), "blob converter")
+        return out
 
     def forward(self):
         self._check(load().tnn_host_forward(self._h), "Forward")

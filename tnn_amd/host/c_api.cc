@@ -159,6 +159,35 @@ HOST_API int tnn_host_set_input(void *hp, const char *name, const void *data, in
     return 0;
 }
 
+// The flow of the engine's blob-converter unit test (test/unit_test/blob_converter_test.cc:287-349) on an input blob of
+// this instance: fp32 NCHW Mat in with per-channel scale and bias, the blob back out as an fp32 NCHW Mat with the same
+// scale and bias applied again.
+HOST_API int tnn_host_input_blob_round_trip(void *hp, const char *name, const float *in, const float *scale,
+                                            const float *bias, int n_param, float *out) {
+    auto h = static_cast<Handle *>(hp);
+    BlobMap blobs;
+    Status st = h->inst->GetAllInputBlobs(blobs);
+    if (st != TNN_OK)
+        return fail(h, st);
+    auto it = blobs.find(name ? name : "");
+    if (it == blobs.end())
+        return fail(h, Status(TNNERR_PARAM_ERR, std::string("no input blob named ") + (name ? name : "")));
+    void *queue = nullptr;
+    h->inst->GetCommandQueue(&queue);
+    MatConvertParam param;
+    param.scale.assign(scale, scale + n_param);
+    param.bias.assign(bias, bias + n_param);
+    DimsVector dims = it->second->GetBlobDesc().dims;
+    BlobConverter converter(it->second);
+    Mat mat_in(DEVICE_NAIVE, NCHW_FLOAT, dims, const_cast<float *>(in));
+    st = converter.ConvertFromMat(mat_in, param, queue);
+    if (st != TNN_OK)
+        return fail(h, st);
+    Mat mat_out(DEVICE_NAIVE, NCHW_FLOAT, dims, out);
+    st = converter.ConvertToMat(mat_out, param, queue);
+    return st == TNN_OK ? 0 : fail(h, st);
+}
+
 // The loop of the engine's benchmark tool (test/test.cc:101-152): per iteration every input Mat goes in
 // (SetInputMat with the Mats of the last tnn_host_set_input calls), Forward, and the output Mat comes out
 // (GetOutputMat as fp32 NCHW on the host).  stats = {min, avg, max} seconds over the timed iterations.
