@@ -46,7 +46,9 @@ void tnn_host_destroy(void *handle);
 const char *tnn_host_last_error(void *handle);
 
 /* Instance::SetInputMat (instance.h:123) from a host array.  mat_type: 0 = NCHW_FLOAT (fp32), 1 = NC_INT32,
- * 2 = RESERVED_INT8_TEST (int8 values copied as they are into an int8 blob, blob_converter_default.cc:190-193).
+ * 2 = RESERVED_INT8_TEST (int8 values copied as they are into an int8 blob, blob_converter_default.cc:190-193),
+ * 3 = RESERVED_BFP16_TEST (bfloat16 bit patterns), 4 = RESERVED_FP16_TEST (IEEE half): the Mats the engine's layer test
+ * feeds half-precision blobs with (layer_test.cc:266-275); they go into a float blob of any type.
  * name NULL or "" selects the only input. */
 int tnn_host_set_input(void *handle, const char *name, const void *data, int mat_type, const int *dims, int ndims);
 /* Instance::Forward (instance.h:78): runs every layer and waits for the stream */
@@ -72,6 +74,12 @@ int tnn_host_get_output(void *handle, const char *name, float *out, size_t capac
  * blob's values as they are, blob_converter_default.cc:347-350); capacity in bytes. */
 int tnn_host_get_output_as(void *handle, const char *name, int mat_type, void *out, size_t capacity_bytes, int *dims,
                            int *ndims);
+/* BlobConverter::ConvertFromMat followed by ConvertToMat on the input blob `name` (include/tnn/utils/blob_converter.h:
+ * 60-78), the flow of the engine's blob-converter unit test (test/unit_test/blob_converter_test.cc:287-349): the fp32 NCHW
+ * Mat `in` enters the blob with per-channel scale and bias (n_param values each, channel = dims[1]) and the blob comes
+ * back in `out` with the same scale and bias applied again.  in / out hold the blob's element count. */
+int tnn_host_input_blob_round_trip(void *handle, const char *name, const float *in, const float *scale, const float *bias,
+                                   int n_param, float *out);
 
 /* The loop of the engine's benchmark tool (test/test.cc:101-152): `warmup` untimed and `iters` timed iterations of
  * SetInputMat for every input set so far (host copies of those Mats are kept), Forward, GetOutputMat(out_name) as
