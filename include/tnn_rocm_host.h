@@ -74,17 +74,28 @@ int tnn_host_get_output(void *handle, const char *name, float *out, size_t capac
  * blob's values as they are, blob_converter_default.cc:347-350); capacity in bytes. */
 int tnn_host_get_output_as(void *handle, const char *name, int mat_type, void *out, size_t capacity_bytes, int *dims,
                            int *ndims);
+/* The same two calls with Mats whose memory is on the device (Mat(DEVICE_ROCM, ...), the counterpart of the DEVICE_CUDA
+ * branches of source/tnn/device/cuda/cuda_blob_converter.cc:62-81, 141-161): nothing crosses the bus.  The input memory
+ * is the caller's and must stay unchanged until the instance's stream has passed the conversion; the output Mat belongs
+ * to the instance and lives until the next call for that output. */
+int tnn_host_set_input_device(void *handle, const char *name, const void *device_data, int mat_type, const int *dims,
+                              int ndims);
+int tnn_host_get_output_device(void *handle, const char *name, int mat_type, void **device_data, int *dims, int *ndims);
 /* BlobConverter::ConvertFromMat followed by ConvertToMat on the input blob `name` (include/tnn/utils/blob_converter.h:
  * 60-78), the flow of the engine's blob-converter unit test (test/unit_test/blob_converter_test.cc:287-349): the fp32 NCHW
  * Mat `in` enters the blob with per-channel scale and bias (n_param values each, channel = dims[1]) and the blob comes
- * back in `out` with the same scale and bias applied again.  in / out hold the blob's element count. */
+ * back in `out` with the same scale and bias applied again.  in / out hold the blob's element count; with on_device
+ * they are device addresses and the Mats are DEVICE_ROCM Mats. */
 int tnn_host_input_blob_round_trip(void *handle, const char *name, const float *in, const float *scale, const float *bias,
-                                   int n_param, float *out);
+                                   int n_param, float *out, int on_device);
 
 /* The loop of the engine's benchmark tool (test/test.cc:101-152): `warmup` untimed and `iters` timed iterations of
  * SetInputMat for every input set so far (host copies of those Mats are kept), Forward, GetOutputMat(out_name) as
  * fp32 NCHW on the host.  stats[3] = {min, avg, max} seconds per iteration. */
 int tnn_host_time_loop(void *handle, int warmup, int iters, const char *out_name, double *stats);
+/* The same loop with Mats in device memory: SetInputMat with the device Mats last given to tnn_host_set_input_device,
+ * Forward, GetOutputMat(out_name) as a device Mat of out_mat_type. */
+int tnn_host_time_loop_device(void *handle, int warmup, int iters, const char *out_name, int out_mat_type, double *stats);
 
 /* The optimised layer list ("Type name\n" per layer) and per-layer timing with events on the instance's stream
  * (the engine's TNN_PROFILE facility, reference source/tnn/core/profile.h:29-100).  only_type NULL or "" times every

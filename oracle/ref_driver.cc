@@ -24,6 +24,7 @@ struct Session {
     std::shared_ptr<Instance> inst;
     std::string err;
     std::vector<std::pair<std::string, std::shared_ptr<Mat>>> inputs;  // the host Mats last given per input name
+    std::shared_ptr<Mat> device_output;                                // the device Mat last handed out
 };
 void put_err(char *buf, size_t n, const std::string &s) {
     if (buf && n) {
@@ -135,7 +136,7 @@ REF_API int tnn_ref_reshape(void *h, const char *shapes) {
 // (ConvertFromMat) and gives the blob back as an fp32 NCHW Mat with the same scale and bias applied again
 // (ConvertToMat).  in / out hold the blob's element count; scale / bias hold n_param values.
 REF_API int tnn_ref_input_blob_round_trip(void *h, const char *name, const float *in, const float *scale, const float *bias,
-                                          int n_param, float *out) {
+                                          int n_param, float *out, int on_device) {
     Session *s = static_cast<Session *>(h);
     BlobMap blobs;
     Status st = s->inst->GetAllInputBlobs(blobs);
@@ -151,16 +152,64 @@ REF_API int tnn_ref_input_blob_round_trip(void *h, const char *name, const float
     param.bias.assign(bias, bias + n_param);
     DimsVector dims = blob->GetBlobDesc().dims;
     BlobConverter converter(blob);
-    Mat mat_in(DEVICE_NAIVE, NCHW_FLOAT, dims, const_cast<float *>(in));
+    // on_device: in / out are addresses in the memory of the blob's own device, the Mats are Mats of that device
+    const DeviceType where = on_device ? blob->GetBlobDesc().device_type : DEVICE_NAIVE;
+    Mat mat_in(where, NCHW_FLOAT, dims, const_cast<float *>(in));
     st = converter.ConvertFromMat(mat_in, param, queue);
     if (st == TNN_OK) {
-        Mat mat_out(DEVICE_NAIVE, NCHW_FLOAT, dims, out);
+        Mat mat_out(where, NCHW_FLOAT, dims, out);
         st = converter.ConvertToMat(mat_out, param, queue);
     }
     if (st != TNN_OK) {
         s->err = st.description();
         return (int)st;
     }
+    return 0;
+}
+
+// SetInputMat / GetOutputMat with Mats in the memory of the session's own device (instance.cc:214-320 with a device other
+// than DEVICE_NAIVE): the input Mat wraps the caller's device address, the output Mat is allocated by the engine through
+// AbstractDevice::Allocate(mat type, dims) and stays with the session until the next call for that output.
+REF_API int tnn_ref_set_input_device(void *h, const char *name, const void *device_data, int is_int32, const int *dims,
+                                     int ndims) {
+    Session *s = static_cast<Session *>(h);
+    BlobMap blobs;
+    s->inst->GetAllInputBlobs(blobs);
+    if (blobs.find(name) == blobs.end()) {
+        s->err = std::string("no input blob named ") + name;
+        return -1;
+    }
+    DimsVector d(dims, dims + ndims);
+    auto mat  = std::make_shared<Mat>(blobs[name]->GetBlobDesc().device_type, is_int32 ? NC_INT32 : NCHW_FLOAT, d,
+                                     const_cast<void *>(device_data));
+    Status st = s->inst->SetInputMat(mat, MatConvertParam(), name);
+    if (st != TNN_OK) {
+        s->err = st.description();
+        return (int)st;
+    }
+    return 0;
+}
+
+REF_API int tnn_ref_get_output_device(void *h, const char *name, void **device_data, int *dims, int *ndims) {
+    Session *s = static_cast<Session *>(h);
+    BlobMap blobs;
+    s->inst->GetAllOutputBlobs(blobs);
+    if (blobs.find(name) == blobs.end()) {
+        s->err = std::string("no output blob named ") + name;
+        return -1;
+    }
+    std::shared_ptr<Mat> mat;
+    Status st = s->inst->GetOutputMat(mat, MatConvertParam(), name, blobs[name]->GetBlobDesc().device_type, NCHW_FLOAT);
+    if (st != TNN_OK) {
+        s->err = st.description();
+        return (int)st;
+    }
+    s->device_output = mat;
+    DimsVector d     = mat->GetDims();
+    *ndims           = (int)d.size();
+    for (size_t i = 0; i < d.size() && i < 8; ++i)
+        dims[i] = d[i];
+    *device_data = mat->GetData();
     return 0;
 }
 

@@ -29,7 +29,10 @@ def lib():
         _lib.tnn_ref_set_input.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]
         _lib.tnn_ref_forward.argtypes = [C.c_void_p]
         _lib.tnn_ref_input_blob_round_trip.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
-                                                       C.c_void_p]
+                                                       C.c_void_p, C.c_int]
+        _lib.tnn_ref_set_input_device.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]
+        _lib.tnn_ref_get_output_device.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_int),
+                                                   C.POINTER(C.c_int)]
         _lib.tnn_ref_forward_memory_size.argtypes = [C.c_void_p, C.POINTER(C.c_int)]
         _lib.tnn_ref_set_forward_memory.argtypes = [C.c_void_p, C.c_void_p]
         _lib.tnn_ref_get_output.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_int),
@@ -73,17 +76,39 @@ class RefSession:
                                             {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.int8): 2}[a.dtype],
                                             dims, a.ndim), "SetInputMat")
 
-    def input_blob_round_trip(self, name, arr, scale, bias):
+    def input_blob_round_trip(self, name, arr, scale, bias, device_ptrs=None):
         """fp32 NCHW Mat -> the input blob (ConvertFromMat with per-channel scale, bias) -> fp32 NCHW Mat (ConvertToMat with
-        the same scale, bias), through a BlobConverter of the blob's device"""
-        a = np.ascontiguousarray(arr, np.float32)
+        the same scale, bias), through a BlobConverter of the blob's device.  device_ptrs = (in, out): Mats in the memory
+        of the blob's device at these addresses instead of host Mats (arr is ignored, nothing is returned)."""
         sc, bi = np.ascontiguousarray(scale, np.float32), np.ascontiguousarray(bias, np.float32)
         assert sc.size == bi.size
+        if device_ptrs is not None:
+            self._check(lib().tnn_ref_input_blob_round_trip(self.h, name.encode(), C.c_void_p(device_ptrs[0]),
+                                                            sc.ctypes.data_as(C.c_void_p), bi.ctypes.data_as(C.c_void_p),
+                                                            int(sc.size), C.c_void_p(device_ptrs[1]), 1), "blob converter")
+            return None
+        a = np.ascontiguousarray(arr, np.float32)
         out = np.empty_like(a)
         self._check(lib().tnn_ref_input_blob_round_trip(self.h, name.encode(), a.ctypes.data_as(C.c_void_p),
                                                         sc.ctypes.data_as(C.c_void_p), bi.ctypes.data_as(C.c_void_p),
-                                                        int(sc.size), out.ctypes.data_as(C.c_void_p)), "blob converter")
+                                                        int(sc.size), out.ctypes.data_as(C.c_void_p), 0), "blob converter")
         return out
+
+    def set_input_device(self, name, data_ptr, is_int32, shape):
+        """SetInputMat with a Mat in the memory of the session's device at data_ptr (fp32, or int32 values)"""
+        dims = (C.c_int * len(shape))(*shape)
+        self._check(lib().tnn_ref_set_input_device(self.h, name.encode(), C.c_void_p(data_ptr), 1 if is_int32 else 0, dims,
+                                                   len(shape)), "SetInputMat (device mat)")
+
+    def output_device(self, name):
+        """GetOutputMat as an fp32 Mat in the memory of the session's device -> (address, shape); the Mat stays with the
+        session until the next call"""
+        ptr = C.c_void_p()
+        dims = (C.c_int * 8)()
+        nd = C.c_int(0)
+        self._check(lib().tnn_ref_get_output_device(self.h, name.encode(), C.byref(ptr), dims, C.byref(nd)),
+                    "GetOutputMat (device mat)")
+        return ptr.value, [dims[i] for i in range(nd.value)]
 
     def reshape(self, shapes):
         self._check(lib().tnn_ref_reshape(self.h, _shape_spec(shapes)), "Reshape")

@@ -419,3 +419,60 @@ def test_blob_converter_grid_inside_the_reference_engine():
         assert np.all(d16 <= 1e-3 + 1e-3 * np.abs(outs["NAIVE"])), case     # one half rounding of the blob, then * scale
         worst16 = max(worst16, float(d16.max()))
     say("  fp32 blobs identical to DEVICE_NAIVE; half blobs differ by at most %.3g" % worst16)
+
+
+def test_device_mats_inside_the_reference_engine():
+    """Instance::SetInputMat / GetOutputMat of the reference engine with Mats in DEVICE_ROCM memory (the engine allocates the
+    output Mat through RocmDevice::Allocate(mat type, dims)): same bits as with host Mats; and the converter grid with
+    device Mats against DEVICE_NAIVE."""
+    engine()
+    torch = pytest.importorskip("torch")
+    from test_gpu_host import converter_grid, _device_to_numpy
+    say("reference engine: Mats in device memory")
+    cfg = EncoderConfig(2, 256, 4, 512)
+    w = make_weights(cfg, seed=83, bias_std=0.05)
+    B, S = 2, 40
+    w["pos_emb"] = w["pos_emb"][:S]
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 9, S, seed=84)
+    graph = tnnmodel.encoder_graph(cfg, w, B, S)
+    for device in ("ROCM:fp32", "ROCM"):
+        s = ref_driver.RefSession(graph, device)
+        s.set_input("input_ids", ids.astype(np.int32))
+        s.set_input("token_type_ids", seg.astype(np.int32))
+        s.set_input("attention_bias", mask.reshape(B, 1, 1, S).astype(np.float32))
+        s.forward()
+        want = s.output("last_hidden")
+        s.set_input("input_ids", np.zeros((B, S), np.int32))
+        s.forward()
+        d_ids = torch.from_numpy(ids.astype(np.int32)).cuda()
+        d_seg = torch.from_numpy(seg.astype(np.int32)).cuda()
+        d_mask = torch.from_numpy(mask.reshape(B, 1, 1, S).astype(np.float32)).cuda()
+        torch.cuda.synchronize()
+        s.set_input_device("input_ids", d_ids.data_ptr(), True, [B, S])
+        s.set_input_device("token_type_ids", d_seg.data_ptr(), True, [B, S])
+        s.set_input_device("attention_bias", d_mask.data_ptr(), False, [B, 1, 1, S])
+        s.forward()
+        ptr, shape = s.output_device("last_hidden")
+        got = _device_to_numpy(ptr, shape, np.float32)
+        assert shape == list(want.shape) and np.array_equal(got, want), device
+        s.close()
+    rng = np.random.default_rng(11)
+    for batch, channel, size, scale, bias in converter_grid():
+        g = tnnmodel.Graph()
+        g.add_input("x", [batch, channel, size, size])
+        g.add_layer("GELU", "act", ["x"], ["y"])
+        g.add_output("y")
+        x = rng.random((batch, channel, size, size), dtype=np.float32)
+        sc = [scale * (c + 1) for c in range(channel)]
+        bi = [bias * (c + 1) for c in range(channel)]
+        s = ref_driver.RefSession(g, "NAIVE")
+        want = s.input_blob_round_trip("x", x, sc, bi)
+        s.close()
+        s = ref_driver.RefSession(g, "ROCM:fp32")
+        d_in = torch.from_numpy(x).cuda()
+        d_out = torch.full_like(d_in, -7.0)
+        torch.cuda.synchronize()
+        s.input_blob_round_trip("x", None, sc, bi, device_ptrs=(d_in.data_ptr(), d_out.data_ptr()))
+        torch.cuda.synchronize()
+        s.close()
+        assert np.array_equal(d_out.cpu().numpy(), want), (batch, channel, size, scale, bias)

@@ -1101,3 +1101,91 @@ def test_blob_converter_scale_and_bias_grid(precision):
             assert np.all(np.abs(got - want) <= 1e-6 + 1e-6 * np.abs(want)), (batch, channel, size, scale, bias)
         worst = max(worst, float(np.abs(got - want).max()))
     say("  largest difference to the expected Mat %.3g" % worst)
+
+
+def _device_to_numpy(ptr, shape, np_dtype):
+    """the bytes at a device address as a numpy array (one device-to-device copy into a tensor, then torch's own download)"""
+    from tnn_amd import capi
+    tdt = {np.dtype(np.float32): torch.float32, np.dtype(np.float16): torch.float16, np.dtype(np.int32): torch.int32,
+           np.dtype(np.int8): torch.int8, np.dtype(np.uint16): torch.int16}[np.dtype(np_dtype)]
+    t = torch.empty(shape, dtype=tdt, device="cuda")
+    torch.cuda.synchronize()
+    capi.call("tnn_rocm_memcpy_d2d", t.data_ptr(), ptr, t.numel() * t.element_size(), None)
+    torch.cuda.synchronize()
+    return t.cpu().numpy().view(np_dtype)
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_mats_in_device_memory(precision):
+    """Mats whose memory is on the device (Mat(DEVICE_ROCM, ...), what cuda_blob_converter.cc:62-81, 141-161 does for
+    DEVICE_CUDA Mats): token ids, segment ids and mask given as device arrays, the output taken as fp32, half and
+    bfloat16 device Mats.  Every result is bit for bit that of the same call with host Mats."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: Mats in device memory, " + precision)
+    cfg = EncoderConfig(2, 256, 4, 512)
+    w = make_weights(cfg, seed=81, bias_std=0.05)
+    B, S = 3, 48
+    w["pos_emb"] = w["pos_emb"][:S]
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 11, S, seed=82)
+    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), precision)
+    inst.set_input("input_ids", ids)
+    inst.set_input("token_type_ids", seg)
+    inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+    inst.forward()
+    want32 = inst.output("last_hidden")
+    want16 = inst.output_as("last_hidden", np.float16)
+    wantb = inst.output_as("last_hidden", np.uint16)
+
+    # other values first, so that the blobs cannot still hold the right ones
+    inst.set_input("input_ids", np.zeros_like(ids))
+    inst.forward()
+    d_ids = torch.from_numpy(ids.astype(np.int32)).cuda()
+    d_seg = torch.from_numpy(seg.astype(np.int32)).cuda()
+    d_mask = torch.from_numpy(mask.reshape(B, 1, 1, S).astype(np.float32)).cuda()
+    torch.cuda.synchronize()
+    inst.set_input_device("input_ids", d_ids.data_ptr(), np.int32, [B, S])
+    inst.set_input_device("token_type_ids", d_seg.data_ptr(), np.int32, [B, S])
+    inst.set_input_device("attention_bias", d_mask.data_ptr(), np.float32, [B, 1, 1, S])
+    inst.forward()
+    for np_dtype, want in ((np.float32, want32), (np.float16, want16), (np.uint16, wantb)):
+        ptr, shape = inst.output_device("last_hidden", np_dtype)
+        assert shape == list(want.shape)
+        got = _device_to_numpy(ptr, shape, np_dtype)
+        assert np.array_equal(got, want), np_dtype
+    assert np.array_equal(inst.output("last_hidden"), want32)          # and host Mats after device Mats
+    # a half Mat on the device into the float mask input
+    d_mask16 = d_mask.half()
+    torch.cuda.synchronize()
+    inst.set_input_device("attention_bias", d_mask16.data_ptr(), np.float16, [B, 1, 1, S])
+    inst.forward()
+    assert np.array_equal(inst.output("last_hidden"), want32)          # 0 and -10000 are half values
+    with pytest.raises(host.HostError):                                # an int32 Mat needs an int32 blob, on the device too
+        inst.set_input_device("attention_bias", d_ids.data_ptr(), np.int32, [B, 1, 1, S])
+    inst.close()
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_blob_converter_scale_and_bias_grid_with_device_mats(precision):
+    """the converter grid again with the Mats in device memory: scale and bias are applied by two broadcast kernels, and
+    the result is bit for bit what the host-Mat form gives"""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: blob converter with scale and bias on device Mats, 96 cases, blobs " + precision)
+    rng = np.random.default_rng(19)
+    for batch, channel, size, scale, bias in converter_grid():
+        g = tnnmodel.Graph()
+        g.add_input("x", [batch, channel, size, size])
+        g.add_layer("GELU", "act", ["x"], ["y"])
+        g.add_output("y")
+        inst = host.RocmInstance.from_graph(g, precision)
+        x = rng.random((batch, channel, size, size), dtype=np.float32)
+        sc = [scale * (c + 1) for c in range(channel)]
+        bi = [bias * (c + 1) for c in range(channel)]
+        want = inst.input_blob_round_trip("x", x, sc, bi)
+        d_in = torch.from_numpy(x).cuda()
+        d_out = torch.full_like(d_in, -7.0)
+        torch.cuda.synchronize()
+        inst.input_blob_round_trip("x", None, sc, bi, device_ptrs=(d_in.data_ptr(), d_out.data_ptr()))
+        torch.cuda.synchronize()
+        inst.close()
+        assert np.array_equal(d_out.cpu().numpy(), want), (batch, channel, size, scale, bias)
+        assert np.array_equal(d_in.cpu().numpy(), x)                   # the caller's Mat is left as it was

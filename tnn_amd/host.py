@@ -22,8 +22,12 @@ SIGNATURES = {
     "tnn_host_destroy": (None, [C.c_void_p]),
     "tnn_host_last_error": (C.c_char_p, [C.c_void_p]),
     "tnn_host_set_input": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]),
+    "tnn_host_time_loop_device": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_char_p, C.c_int, C.POINTER(C.c_double)]),
+    "tnn_host_set_input_device": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]),
+    "tnn_host_get_output_device": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_int),
+                                             C.POINTER(C.c_int)]),
     "tnn_host_input_blob_round_trip": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
-                                                 C.c_void_p]),
+                                                 C.c_void_p, C.c_int]),
     "tnn_host_forward": (C.c_int, [C.c_void_p]),
     "tnn_host_forward_async": (C.c_int, [C.c_void_p]),
     "tnn_host_sync": (C.c_int, [C.c_void_p]),
@@ -159,16 +163,38 @@ class RocmInstance:
         self._check(load().tnn_host_set_input(self._h, name.encode(), a.ctypes.data_as(C.c_void_p),
                                               _MAT_CODE[a.dtype], dims, a.ndim), "SetInputMat")
 
-    def input_blob_round_trip(self, name, arr, scale, bias):
+    def set_input_device(self, name, data_ptr, np_dtype, shape):
+        """SetInputMat with a Mat in device memory (data_ptr: a device address holding `shape` elements of np_dtype, e.g. a
+        torch tensor's data_ptr()); the memory must stay unchanged until the instance's stream has passed the copy"""
+        dims = (C.c_int * max(len(shape), 1))(*shape)
+        self._check(load().tnn_host_set_input_device(self._h, name.encode(), C.c_void_p(data_ptr), _MAT_CODE[np.dtype(np_dtype)],
+                                                     dims, len(shape)), "SetInputMat (device mat)")
+
+    def output_device(self, name, np_dtype):
+        """GetOutputMat as a Mat in device memory the instance owns -> (device address, shape)"""
+        ptr = C.c_void_p()
+        dims = (C.c_int * 8)()
+        nd = C.c_int(0)
+        self._check(load().tnn_host_get_output_device(self._h, name.encode(), _MAT_CODE[np.dtype(np_dtype)], C.byref(ptr), dims,
+                                                      C.byref(nd)), "GetOutputMat (device mat)")
+        return ptr.value, [dims[i] for i in range(nd.value)]
+
+    def input_blob_round_trip(self, name, arr, scale, bias, device_ptrs=None):
         """fp32 NCHW Mat -> the input blob (ConvertFromMat with per-channel scale, bias) -> fp32 NCHW Mat (ConvertToMat with
-        the same scale, bias): the flow of the engine's blob-converter unit test"""
-        a = np.ascontiguousarray(arr, np.float32)
+        the same scale, bias): the flow of the engine's blob-converter unit test.  device_ptrs = (in, out) device
+        addresses: the same with DEVICE_ROCM Mats (arr is ignored, nothing is returned)."""
         sc, bi = np.ascontiguousarray(scale, np.float32), np.ascontiguousarray(bias, np.float32)
         assert sc.size == bi.size
+        if device_ptrs is not None:
+            self._check(load().tnn_host_input_blob_round_trip(self._h, name.encode(), C.c_void_p(device_ptrs[0]),
+                                                              sc.ctypes.data_as(C.c_void_p), bi.ctypes.data_as(C.c_void_p),
+                                                              int(sc.size), C.c_void_p(device_ptrs[1]), 1), "blob converter")
+            return None
+        a = np.ascontiguousarray(arr, np.float32)
         out = np.empty_like(a)
         self._check(load().tnn_host_input_blob_round_trip(self._h, name.encode(), a.ctypes.data_as(C.c_void_p),
                                                           sc.ctypes.data_as(C.c_void_p), bi.ctypes.data_as(C.c_void_p),
-                                                          int(sc.size), out.ctypes.data_as(C.c_void_p)), "blob converter")
+                                                          int(sc.size), out.ctypes.data_as(C.c_void_p), 0), "blob converter")
         return out
 
     def forward(self):
@@ -232,6 +258,14 @@ class RocmInstance:
         iteration), run natively -> (min, avg, max) seconds"""
         stats = (C.c_double * 3)()
         self._check(load().tnn_host_time_loop(self._h, warmup, iters, out_name.encode(), stats), "timing loop")
+        return stats[0], stats[1], stats[2]
+
+    def time_loop_device(self, warmup, iters, out_name, out_dtype=np.float32):
+        """time_loop with the Mats in device memory (inputs: the device Mats last given to set_input_device; output: a
+        device Mat of out_dtype) -> (min, avg, max) seconds"""
+        stats = (C.c_double * 3)()
+        self._check(load().tnn_host_time_loop_device(self._h, warmup, iters, out_name.encode(), _MAT_CODE[np.dtype(out_dtype)],
+                                                     stats), "timing loop (device mats)")
         return stats[0], stats[1], stats[2]
 
     def layers(self):

@@ -21,6 +21,7 @@ struct Handle {
     std::string err;
     std::string summary;
     std::map<std::string, std::shared_ptr<Mat>> inputs;  // host copies of the last Mats set, for tnn_host_time_loop
+    std::map<std::string, std::shared_ptr<Mat>> device_inputs;  // the device Mats last set (the caller's memory)
 };
 int fail(Handle *h, const Status &st) {
     h->err = st.description();
@@ -159,11 +160,45 @@ HOST_API int tnn_host_set_input(void *hp, const char *name, const void *data, in
     return 0;
 }
 
+// SetInputMat with a Mat whose memory is on the device already (Mat(DEVICE_ROCM, type, dims, pointer)): nothing crosses
+// the bus, the converter copies or converts on the instance's stream.  The caller keeps the memory alive and unchanged
+// until that stream has passed the conversion (tnn_host_sync, or any Forward).
+HOST_API int tnn_host_set_input_device(void *hp, const char *name, const void *device_data, int mat_type, const int *dims,
+                                       int ndims) {
+    auto h = static_cast<Handle *>(hp);
+    DimsVector d(dims, dims + ndims);
+    auto mat  = std::make_shared<Mat>(DEVICE_ROCM, MatTypeOf(mat_type), d, const_cast<void *>(device_data));
+    Status st = h->inst->SetInputMat(mat, MatConvertParam(), name ? name : "");
+    if (st != TNN_OK)
+        return fail(h, st);
+    h->device_inputs[name ? name : ""] = mat;
+    return 0;
+}
+
+// GetOutputMat on the device: the output as a Mat of the given type in device memory the instance owns (valid until the
+// next call for this output or the instance's end).  *device_data receives its address.
+HOST_API int tnn_host_get_output_device(void *hp, const char *name, int mat_type, void **device_data, int *dims, int *ndims) {
+    auto h = static_cast<Handle *>(hp);
+    std::shared_ptr<Mat> mat;
+    Status st = h->inst->GetOutputMat(mat, MatConvertParam(), name ? name : "", DEVICE_ROCM, MatTypeOf(mat_type));
+    if (st != TNN_OK)
+        return fail(h, st);
+    DimsVector d = mat->GetDims();
+    if (ndims)
+        *ndims = (int)d.size();
+    if (dims)
+        for (size_t i = 0; i < d.size() && i < 8; ++i)
+            dims[i] = d[i];
+    if (device_data)
+        *device_data = mat->GetData();
+    return 0;
+}
+
 // The flow of the engine's blob-converter unit test (test/unit_test/blob_converter_test.cc:287-349) on an input blob of
 // this instance: fp32 NCHW Mat in with per-channel scale and bias, the blob back out as an fp32 NCHW Mat with the same
 // scale and bias applied again.
 HOST_API int tnn_host_input_blob_round_trip(void *hp, const char *name, const float *in, const float *scale,
-                                            const float *bias, int n_param, float *out) {
+                                            const float *bias, int n_param, float *out, int on_device) {
     auto h = static_cast<Handle *>(hp);
     BlobMap blobs;
     Status st = h->inst->GetAllInputBlobs(blobs);
@@ -179,11 +214,12 @@ HOST_API int tnn_host_input_blob_round_trip(void *hp, const char *name, const fl
     param.bias.assign(bias, bias + n_param);
     DimsVector dims = it->second->GetBlobDesc().dims;
     BlobConverter converter(it->second);
-    Mat mat_in(DEVICE_NAIVE, NCHW_FLOAT, dims, const_cast<float *>(in));
+    const DeviceType where = on_device ? DEVICE_ROCM : DEVICE_NAIVE;  // in / out are device addresses then
+    Mat mat_in(where, NCHW_FLOAT, dims, const_cast<float *>(in));
     st = converter.ConvertFromMat(mat_in, param, queue);
     if (st != TNN_OK)
         return fail(h, st);
-    Mat mat_out(DEVICE_NAIVE, NCHW_FLOAT, dims, out);
+    Mat mat_out(where, NCHW_FLOAT, dims, out);
     st = converter.ConvertToMat(mat_out, param, queue);
     return st == TNN_OK ? 0 : fail(h, st);
 }
@@ -205,6 +241,39 @@ HOST_API int tnn_host_time_loop(void *hp, int warmup, int iters, const char *out
         std::shared_ptr<Mat> mat;
         if (st == TNN_OK)
             st = h->inst->GetOutputMat(mat, MatConvertParam(), out_name ? out_name : "", DEVICE_NAIVE, NCHW_FLOAT);
+        if (st != TNN_OK)
+            return fail(h, st);
+        double dt = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        if (i >= warmup) {
+            mn = dt < mn ? dt : mn;
+            mx = dt > mx ? dt : mx;
+            sum += dt;
+        }
+    }
+    stats[0] = mn;
+    stats[1] = sum / (iters > 0 ? iters : 1);
+    stats[2] = mx;
+    return 0;
+}
+
+// The same loop for a caller whose data lives on the device: SetInputMat with the device Mats last given
+// (tnn_host_set_input_device), Forward, GetOutputMat as a device Mat of `out_mat_type`; nothing crosses the bus.
+HOST_API int tnn_host_time_loop_device(void *hp, int warmup, int iters, const char *out_name, int out_mat_type, double *stats) {
+    auto h = static_cast<Handle *>(hp);
+    if (h->device_inputs.empty())
+        return fail(h, Status(TNNERR_PARAM_ERR, "no device Mat has been set as an input"));
+    double mn = 1e30, mx = 0.0, sum = 0.0;
+    for (int i = 0; i < warmup + iters; ++i) {
+        auto t0 = std::chrono::steady_clock::now();
+        for (auto &kv : h->device_inputs) {
+            Status st = h->inst->SetInputMat(kv.second, MatConvertParam(), kv.first);
+            if (st != TNN_OK)
+                return fail(h, st);
+        }
+        Status st = h->inst->Forward();
+        std::shared_ptr<Mat> mat;
+        if (st == TNN_OK)
+            st = h->inst->GetOutputMat(mat, MatConvertParam(), out_name ? out_name : "", DEVICE_ROCM, MatTypeOf(out_mat_type));
         if (st != TNN_OK)
             return fail(h, st);
         double dt = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();

@@ -116,6 +116,15 @@ Mat::Mat(DeviceType device_type, MatType mat_type, DimsVector dims)
     : device_type_(device_type), mat_type_(mat_type), dims_(std::move(dims)) {
     size_t es = (mat_type == NCHW_FLOAT || mat_type == NC_INT32) ? 4 : ((mat_type == RESERVED_FP16_TEST || mat_type == RESERVED_BFP16_TEST) ? 2 : 1);
     size_t n  = (size_t)DimsVectorUtils::Count(dims_) * es;
+    if (device_type != DEVICE_NAIVE) {  // memory of the Mat's own device, returned to it with the last owner (mat.cc:70-87)
+        AbstractDevice *device = GetDevice(device_type);
+        void *p                = nullptr;
+        if (device && device->Allocate(&p, mat_type, dims_) == TNN_OK && p) {
+            owned_ = std::shared_ptr<char>((char *)p, [device](char *q) { device->Free(q); });
+            data_  = p;
+        }
+        return;
+    }
     owned_    = std::shared_ptr<char>(new char[n > 0 ? n : 1](), std::default_delete<char[]>());
     data_     = owned_.get();
 }
@@ -141,6 +150,16 @@ Status BlobConverter::ConvertFromMat(Mat &image, MatConvertParam param, void *q)
     if (!impl_)
         return Status(TNNERR_INIT_LAYER, "blob converter is nil, check device type");
     return impl_->ConvertFromMat(image, param, q);
+}
+Status BlobConverter::ConvertToMatAsync(Mat &image, MatConvertParam param, void *q) {
+    if (!impl_)
+        return Status(TNNERR_INIT_LAYER, "blob converter is nil, check device type");
+    return impl_->ConvertToMatAsync(image, param, q);
+}
+Status BlobConverter::ConvertFromMatAsync(Mat &image, MatConvertParam param, void *q) {
+    if (!impl_)
+        return Status(TNNERR_INIT_LAYER, "blob converter is nil, check device type");
+    return impl_->ConvertFromMatAsync(image, param, q);
 }
 
 // ---- model interpreter (source/tnn/interpreter/tnn/model_interpreter.cc:174-476) ----------------
@@ -1525,7 +1544,7 @@ Status Instance::SetInputMat(std::shared_ptr<Mat> mat, MatConvertParam param, st
     auto &conv = input_converters_[blob->GetBlobDesc().name];
     if (!conv.second || conv.first != blob)
         conv = {blob, std::make_shared<BlobConverter>(blob)};
-    return conv.second->ConvertFromMat(*mat, param, q);
+    return conv.second->ConvertFromMatAsync(*mat, param, q);  // instance.cc:241: the forward that follows is on the same queue
 }
 
 Status Instance::GetOutputMat(std::shared_ptr<Mat> &mat, MatConvertParam param, std::string output_name,
@@ -1545,8 +1564,14 @@ Status Instance::GetOutputMat(std::shared_ptr<Mat> &mat, MatConvertParam param, 
         blob = it->second;
     }
     auto &cached = output_mats_[output_name];
-    if (!cached || cached->GetMatType() != mat_type || cached->GetDims() != blob->GetBlobDesc().dims)
-        cached = std::make_shared<Mat>(DEVICE_NAIVE, mat_type, blob->GetBlobDesc().dims);
+    if (!cached || cached->GetMatType() != mat_type || cached->GetDeviceType() != device ||
+        cached->GetDims() != blob->GetBlobDesc().dims) {
+        cached = std::make_shared<Mat>(device, mat_type, blob->GetBlobDesc().dims);
+        if (!cached->GetData()) {
+            cached.reset();
+            return Status(TNNERR_OUTOFMEMORY, "no memory for the output mat on the device asked for");
+        }
+    }
     void *q = nullptr;
     network_->GetCommandQueue(&q);
     auto &conv = output_converters_[output_name];  // instance.cc:298-305

@@ -327,6 +327,7 @@ public:
     explicit RocmBlobConverterAcc(Blob *blob) : BlobConverterAcc(blob) {}
     ~RocmBlobConverterAcc() override {
         tnn_rocm_free(staging_);
+        tnn_rocm_free(params_);
         tnn_rocm_free_host(bounce_);
     }
 
@@ -343,13 +344,15 @@ public:
     Status ConvertFromMatAsync(Mat &mat, MatConvertParam param, void *q) override {
         auto &desc   = blob_->GetBlobDesc();
         size_t count = (size_t)DimsVectorUtils::Count(desc.dims);
-        if (mat.GetDeviceType() != DEVICE_NAIVE)
-            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: only host mats are supported");
+        if (mat.GetDeviceType() != DEVICE_NAIVE && mat.GetDeviceType() != DEVICE_ROCM)
+            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: the mat lives on another device");
         if ((size_t)DimsVectorUtils::Count(mat.GetDims()) != count)
             return Status(TNNERR_INVALID_INPUT, "mat and blob element counts differ");
         void *dst = (char *)blob_->GetHandle().base + blob_->GetHandle().bytes_offset;
         if (count == 0)
             return TNN_OK;
+        if (mat.GetDeviceType() == DEVICE_ROCM)
+            return FromDeviceMat(mat, param, dst, count, q);
         if (mat.GetMatType() == NC_INT32) {
             if (desc.data_type != DATA_TYPE_INT32)
                 return Status(TNNERR_PARAM_ERR, "NC_INT32 mat needs an int32 blob");
@@ -440,6 +443,10 @@ public:
         void *src = (char *)blob_->GetHandle().base + blob_->GetHandle().bytes_offset;
         if (count == 0)
             return TNN_OK;
+        if (mat.GetDeviceType() == DEVICE_ROCM)
+            return ToDeviceMat(mat, param, src, count, q);
+        if (mat.GetDeviceType() != DEVICE_NAIVE)
+            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: the mat lives on another device");
         if (mat.GetMatType() == NC_INT32 && desc.data_type == DATA_TYPE_INT32) {
             ROCM_CALL(tnn_rocm_memcpy_d2h(mat.GetData(), src, count * 4, q));
             return TNN_OK;
@@ -519,6 +526,134 @@ public:
     }
 
 private:
+    // ---- Mats whose memory is on this device (role of the DEVICE_CUDA branches of cuda_blob_converter.cc:62-81, 141-161):
+    // nothing crosses the bus and nothing waits for the stream except the few bytes of scale and bias ----
+    static bool IsFloatBlob(DataType t) { return t == DATA_TYPE_FLOAT || t == DATA_TYPE_HALF || t == DATA_TYPE_BFP16; }
+    // per-channel x * scale + bias over dims[1], in place on fp32 device data: a multiply and an add with the operand
+    // broadcast along every other axis (two roundings, as the host form has)
+    Status ScaleBiasOnDevice(float *data, const DimsVector &dims, const MatConvertParam &p, void *q) {
+        const int rank = (int)dims.size();
+        if (rank < 1 || rank > 6)
+            return Status(TNNERR_PARAM_ERR, "scale and bias on a device mat need a rank between 1 and 6");
+        const int c = rank > 1 ? dims[1] : 1;
+        std::vector<float> host(2 * (size_t)c);
+        for (int j = 0; j < c; ++j) {
+            host[j]     = j < (int)p.scale.size() ? p.scale[j] : 1.0f;
+            host[c + j] = j < (int)p.bias.size() ? p.bias[j] : 0.0f;
+        }
+        if (host.size() * 4 > params_sz_) {
+            tnn_rocm_free(params_);
+            params_    = nullptr;
+            params_sz_ = 0;
+            int rc     = tnn_rocm_malloc(&params_, host.size() * 4);
+            if (rc != 0)
+                return RocmStatus(rc, TNNERR_OUTOFMEMORY, "converter scale and bias");
+            params_sz_ = host.size() * 4;
+        }
+        ROCM_CALL(tnn_rocm_memcpy_h2d(params_, host.data(), host.size() * 4, q));  // returns when the bytes have left the vector
+        DimsVector pd((size_t)rank, 1);
+        if (rank > 1)
+            pd[1] = c;
+        const float *sc = (const float *)params_;
+        ROCM_CALL(tnn_rocm_binary(q, TNN_ROCM_F32, 2, data, dims.data(), rank, sc, pd.data(), rank, data, dims.data(), rank));
+        ROCM_CALL(tnn_rocm_binary(q, TNN_ROCM_F32, 0, data, dims.data(), rank, sc + c, pd.data(), rank, data, dims.data(), rank));
+        return TNN_OK;
+    }
+    Status FromDeviceMat(Mat &mat, const MatConvertParam &param, void *dst, size_t count, void *q) {
+        auto &desc      = blob_->GetBlobDesc();
+        const void *src = mat.GetData();
+        if (!src)
+            return Status(TNNERR_NULL_PARAM, "device mat without memory");
+        const MatType mt = mat.GetMatType();
+        if (mt == NC_INT32 || mt == RESERVED_INT8_TEST) {
+            const DataType want = mt == NC_INT32 ? DATA_TYPE_INT32 : DATA_TYPE_INT8;
+            if (desc.data_type != want)
+                return Status(TNNERR_PARAM_ERR, mt == NC_INT32 ? "NC_INT32 mat needs an int32 blob" : "int8 mat needs an int8 blob");
+            ROCM_CALL(tnn_rocm_memcpy_d2d(dst, src, count * (mt == NC_INT32 ? 4 : 1), q));
+            return TNN_OK;
+        }
+        if (mt == RESERVED_BFP16_TEST || mt == RESERVED_FP16_TEST) {
+            const DataType half_type = mt == RESERVED_BFP16_TEST ? DATA_TYPE_BFP16 : DATA_TYPE_HALF;
+            if (!IsFloatBlob(desc.data_type))
+                return Status(TNNERR_PARAM_ERR, "a half or bfloat16 mat needs a float blob");
+            if (desc.data_type == half_type)
+                ROCM_CALL(tnn_rocm_memcpy_d2d(dst, src, count * 2, q));
+            else
+                ROCM_CALL(tnn_rocm_cast(q, (int)half_type, src, (int)desc.data_type, dst, count));
+            return TNN_OK;
+        }
+        if (mt != NCHW_FLOAT)
+            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported mat type");
+        const float *f = (const float *)src;
+        if (NeedsScaleBias(param, desc.dims)) {  // the caller's Mat stays as it is: the scaled values go through the staging buffer
+            RETURN_ON_NEQ(Staging(count * 4), TNN_OK);
+            ROCM_CALL(tnn_rocm_memcpy_d2d(staging_, src, count * 4, q));
+            RETURN_ON_NEQ(ScaleBiasOnDevice((float *)staging_, desc.dims, param, q), TNN_OK);
+            f = (const float *)staging_;
+        }
+        if (desc.data_type == DATA_TYPE_FLOAT) {
+            ROCM_CALL(tnn_rocm_memcpy_d2d(dst, f, count * 4, q));
+        } else if (desc.data_type == DATA_TYPE_HALF || desc.data_type == DATA_TYPE_BFP16) {
+            ROCM_CALL(tnn_rocm_cast(q, TNN_ROCM_F32, f, (int)desc.data_type, dst, count));
+        } else if (desc.data_type == DATA_TYPE_INT8) {
+            auto bi = dynamic_cast<BlobInt8 *>(blob_);
+            if (!bi || !bi->GetIntResource() || bi->GetIntResource()->scale_handle.GetDataCount() < 1)
+                return Status(TNNERR_NULL_PARAM, "int8 blob without scale resource");
+            if (bi->GetIntResource()->scale_handle.GetDataCount() != 1)
+                return Status(TNNERR_PARAM_ERR, "a device mat into an int8 blob needs a per-tensor blob scale");
+            const float s = bi->GetIntResource()->scale_handle.force_to<float *>()[0];
+            ROCM_CALL(tnn_rocm_quantize(q, TNN_ROCM_F32, f, (float)(1.0 / s), (int8_t *)dst, count));
+        } else {
+            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported blob data type");
+        }
+        return TNN_OK;
+    }
+    Status ToDeviceMat(Mat &mat, const MatConvertParam &param, const void *src, size_t count, void *q) {
+        auto &desc = blob_->GetBlobDesc();
+        void *out  = mat.GetData();
+        if (!out)
+            return Status(TNNERR_NULL_PARAM, "device mat without memory");
+        const MatType mt = mat.GetMatType();
+        if (mt == NC_INT32 && desc.data_type == DATA_TYPE_INT32) {
+            ROCM_CALL(tnn_rocm_memcpy_d2d(out, src, count * 4, q));
+            return TNN_OK;
+        }
+        if (mt == RESERVED_INT8_TEST && desc.data_type == DATA_TYPE_INT8) {
+            ROCM_CALL(tnn_rocm_memcpy_d2d(out, src, count, q));
+            return TNN_OK;
+        }
+        if (mt == RESERVED_BFP16_TEST || mt == RESERVED_FP16_TEST) {
+            const DataType half_type = mt == RESERVED_BFP16_TEST ? DATA_TYPE_BFP16 : DATA_TYPE_HALF;
+            if (!IsFloatBlob(desc.data_type))
+                return Status(TNNERR_PARAM_ERR, "a half or bfloat16 mat needs a float blob");
+            if (desc.data_type == half_type)
+                ROCM_CALL(tnn_rocm_memcpy_d2d(out, src, count * 2, q));
+            else
+                ROCM_CALL(tnn_rocm_cast(q, (int)desc.data_type, src, (int)half_type, out, count));
+            return TNN_OK;
+        }
+        if (mt != NCHW_FLOAT)
+            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported mat type");
+        if (desc.data_type == DATA_TYPE_FLOAT) {
+            ROCM_CALL(tnn_rocm_memcpy_d2d(out, src, count * 4, q));
+        } else if (desc.data_type == DATA_TYPE_HALF || desc.data_type == DATA_TYPE_BFP16 || desc.data_type == DATA_TYPE_INT32) {
+            ROCM_CALL(tnn_rocm_cast(q, (int)desc.data_type, src, TNN_ROCM_F32, out, count));
+        } else if (desc.data_type == DATA_TYPE_INT8) {
+            auto bi = dynamic_cast<BlobInt8 *>(blob_);
+            if (!bi || !bi->GetIntResource() || bi->GetIntResource()->scale_handle.GetDataCount() < 1)
+                return Status(TNNERR_NULL_PARAM, "int8 blob without scale resource");
+            if (bi->GetIntResource()->scale_handle.GetDataCount() != 1)
+                return Status(TNNERR_PARAM_ERR, "an int8 blob into a device mat needs a per-tensor blob scale");
+            const float s = bi->GetIntResource()->scale_handle.force_to<float *>()[0];
+            ROCM_CALL(tnn_rocm_dequantize(q, (const int8_t *)src, s, TNN_ROCM_F32, out, count));
+        } else {
+            return Status(TNNERR_PARAM_ERR, "RocmBlobConverter: unsupported blob data type");
+        }
+        if (NeedsScaleBias(param, desc.dims))
+            RETURN_ON_NEQ(ScaleBiasOnDevice((float *)out, desc.dims, param, q), TNN_OK);
+        return TNN_OK;
+    }
+
     static bool NeedsScaleBias(const MatConvertParam &p, const DimsVector &dims) {
         for (float s : p.scale)
             if (s != 1.0f)
@@ -613,6 +748,8 @@ private:
     size_t staging_sz_ = 0;
     void *bounce_      = nullptr;
     size_t bounce_sz_  = 0;
+    void *params_      = nullptr;  // scale and bias of a device mat's conversion, on the device
+    size_t params_sz_  = 0;
 };
 
 DECLARE_BLOB_CONVERTER_CREATER(Rocm);

@@ -519,7 +519,7 @@ class Mat {
 public:
     Mat(DeviceType device_type, MatType mat_type, DimsVector dims, void *data)
         : device_type_(device_type), mat_type_(mat_type), data_(data), dims_(std::move(dims)) {}
-    Mat(DeviceType device_type, MatType mat_type, DimsVector dims);  // allocates host memory (DEVICE_NAIVE only)
+    Mat(DeviceType device_type, MatType mat_type, DimsVector dims);  // allocates: host memory, or the device's through AbstractDevice::Allocate
     DeviceType GetDeviceType() { return device_type_; }
     MatType GetMatType() { return mat_type_; }
     void *GetData() { return data_; }
@@ -588,6 +588,8 @@ public:
     explicit BlobConverter(Blob *blob);
     Status ConvertToMat(Mat &image, MatConvertParam param, void *command_queue);
     Status ConvertFromMat(Mat &image, MatConvertParam param, void *command_queue);
+    Status ConvertToMatAsync(Mat &image, MatConvertParam param, void *command_queue);
+    Status ConvertFromMatAsync(Mat &image, MatConvertParam param, void *command_queue);
 
 private:
     std::shared_ptr<BlobConverterAcc> impl_;
