@@ -81,6 +81,10 @@ int tnn_host_get_output_as(void *handle, const char *name, int mat_type, void *o
 int tnn_host_set_input_device(void *handle, const char *name, const void *device_data, int mat_type, const int *dims,
                               int ndims);
 int tnn_host_get_output_device(void *handle, const char *name, int mat_type, void **device_data, int *dims, int *ndims);
+/* MatUtils::Copy (include/tnn/utils/mat_utils.h:77-79) host Mat -> DEVICE_ROCM Mat -> a second DEVICE_ROCM Mat (allocated by
+ * the copy) -> host Mat `out`; mat_type as for tnn_host_set_input.  No instance is involved. */
+int tnn_host_mat_copy_round_trip(const void *in, void *out, int mat_type, const int *dims, int ndims, char *err,
+                                 size_t err_len);
 /* BlobConverter::ConvertFromMat followed by ConvertToMat on the input blob `name` (include/tnn/utils/blob_converter.h:
  * 60-78), the flow of the engine's blob-converter unit test (test/unit_test/blob_converter_test.cc:287-349): the fp32 NCHW
  * Mat `in` enters the blob with per-channel scale and bias (n_param values each, channel = dims[1]) and the blob comes

@@ -15,6 +15,7 @@
 #include "tnn/core/mat.h"
 #include "tnn/core/tnn.h"
 #include "tnn/utils/blob_converter.h"
+#include "tnn/utils/mat_utils.h"
 
 using namespace TNN_NS;
 
@@ -162,6 +163,30 @@ REF_API int tnn_ref_input_blob_round_trip(void *h, const char *name, const float
     }
     if (st != TNN_OK) {
         s->err = st.description();
+        return (int)st;
+    }
+    return 0;
+}
+
+// MatUtils::Copy of the reference (include/tnn/utils/mat_utils.h:77-79) three times: host Mat `in` -> a Mat of `device` the
+// engine allocates -> a second Mat of that device, allocated by the copy -> host Mat `out`.  fp32 values.
+REF_API int tnn_ref_mat_copy_round_trip(const char *device, const float *in, float *out, const int *dims, int ndims, char *err,
+                                        size_t err_len) {
+    DeviceType dt = DEVICE_NAIVE;
+    std::string name(device ? device : "");
+    if (name.compare(0, 4, "ROCM") == 0)
+        dt = (DeviceType)0x1080;
+    DimsVector d(dims, dims + ndims);
+    Mat src(DEVICE_NAIVE, NCHW_FLOAT, d, const_cast<float *>(in));
+    Mat first(dt, NCHW_FLOAT, d), second(dt, NCHW_FLOAT, d, nullptr);
+    Mat back(DEVICE_NAIVE, NCHW_FLOAT, d, out);
+    Status st = MatUtils::Copy(src, first, nullptr);
+    if (st == TNN_OK)
+        st = MatUtils::Copy(first, second, nullptr);
+    if (st == TNN_OK)
+        st = MatUtils::Copy(second, back, nullptr);
+    if (st != TNN_OK) {
+        put_err(err, err_len, st.description());
         return (int)st;
     }
     return 0;

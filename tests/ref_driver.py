@@ -30,6 +30,8 @@ def lib():
         _lib.tnn_ref_forward.argtypes = [C.c_void_p]
         _lib.tnn_ref_input_blob_round_trip.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
                                                        C.c_void_p, C.c_int]
+        _lib.tnn_ref_mat_copy_round_trip.argtypes = [C.c_char_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_char_p,
+                                                     C.c_size_t]
         _lib.tnn_ref_set_input_device.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]
         _lib.tnn_ref_get_output_device.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_int),
                                                    C.POINTER(C.c_int)]
@@ -50,6 +52,19 @@ def lib():
 
 def _shape_spec(shapes):
     return ";".join("%s:%s" % (k, ",".join(str(int(d)) for d in v)) for k, v in (shapes or {}).items()).encode()
+
+
+def mat_copy_round_trip(device, arr):
+    """the reference's MatUtils::Copy host -> `device` -> `device` -> host of an fp32 array"""
+    a = np.ascontiguousarray(arr, np.float32)
+    out = np.empty_like(a)
+    dims = (C.c_int * a.ndim)(*a.shape)
+    err = C.create_string_buffer(512)
+    rc = lib().tnn_ref_mat_copy_round_trip(device.encode(), a.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p), dims,
+                                           a.ndim, err, 512)
+    if rc != 0:
+        raise RuntimeError("MatUtils::Copy failed (0x%x): %s" % (rc & 0xFFFFFFFF, err.value.decode(errors="replace")))
+    return out
 
 
 class RefSession:

@@ -476,3 +476,14 @@ def test_device_mats_inside_the_reference_engine():
         torch.cuda.synchronize()
         s.close()
         assert np.array_equal(d_out.cpu().numpy(), want), (batch, channel, size, scale, bias)
+
+
+def test_mat_utils_copy_inside_the_reference_engine():
+    """the reference's own MatUtils::Copy finds DEVICE_ROCM's Mat converter (REGISTER_MAT_CONVERTER) and the device's
+    Allocate(mat type, dims): host -> DEVICE_ROCM -> DEVICE_ROCM -> host returns the values"""
+    engine()
+    say("reference engine: MatUtils::Copy through DEVICE_ROCM")
+    rng = np.random.default_rng(5)
+    for shape in ((1, 1, 1, 1), (2, 3, 7, 5), (4, 1, 96, 256)):   # the engine's check wants the four image dims
+        a = rng.standard_normal(shape).astype(np.float32)
+        assert np.array_equal(ref_driver.mat_copy_round_trip("ROCM", a), a), shape

@@ -1189,3 +1189,18 @@ def test_blob_converter_scale_and_bias_grid_with_device_mats(precision):
         inst.close()
         assert np.array_equal(d_out.cpu().numpy(), want), (batch, channel, size, scale, bias)
         assert np.array_equal(d_in.cpu().numpy(), x)                   # the caller's Mat is left as it was
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.int8, np.float16, np.uint16])
+def test_mat_utils_copy_to_the_device_and_back(np_dtype):
+    """MatUtils::Copy (mat_utils.cc:73-100) with the device's Mat converter: host Mat -> DEVICE_ROCM Mat -> a second
+    DEVICE_ROCM Mat that the copy allocates -> host Mat gives the bytes it was given, for every Mat type of the path"""
+    host, *_ = _mods()
+    say("host: MatUtils::Copy host -> device -> device -> host, %s" % np.dtype(np_dtype).name)
+    rng = np.random.default_rng(4)
+    for shape in ((1,), (3, 5), (2, 3, 7, 5), (8, 384, 768)):
+        if np.dtype(np_dtype).kind == "f":
+            a = (rng.standard_normal(shape) * 100).astype(np_dtype)
+        else:
+            a = rng.integers(-120, 120, shape).astype(np_dtype)
+        assert np.array_equal(host.mat_copy_round_trip(a).view(np.uint8), a.view(np.uint8)), shape

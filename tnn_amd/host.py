@@ -23,6 +23,8 @@ SIGNATURES = {
     "tnn_host_last_error": (C.c_char_p, [C.c_void_p]),
     "tnn_host_set_input": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]),
     "tnn_host_time_loop_device": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_char_p, C.c_int, C.POINTER(C.c_double)]),
+    "tnn_host_mat_copy_round_trip": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int, C.c_char_p,
+                                               C.c_size_t]),
     "tnn_host_set_input_device": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int]),
     "tnn_host_get_output_device": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_int),
                                              C.POINTER(C.c_int)]),
@@ -117,6 +119,19 @@ def plan(graph_or_proto, model=None, precision="fp16", input_shapes=None):
     if rc != 0:
         raise HostError("plan failed (0x%x): %s" % (rc & 0xFFFFFFFF, err.value.decode(errors="replace")))
     return _parse_io(out.value.decode(errors="replace").splitlines(), True)
+
+
+def mat_copy_round_trip(arr):
+    """MatUtils::Copy host -> DEVICE_ROCM -> DEVICE_ROCM -> host of an array whose type names a Mat type"""
+    a = np.ascontiguousarray(arr)
+    out = np.empty_like(a)
+    dims = (C.c_int * max(a.ndim, 1))(*a.shape)
+    err = C.create_string_buffer(512)
+    rc = load().tnn_host_mat_copy_round_trip(a.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p), _MAT_CODE[a.dtype],
+                                             dims, a.ndim, err, 512)
+    if rc != 0:
+        raise HostError("MatUtils::Copy failed (0x%x): %s" % (rc & 0xFFFFFFFF, err.value.decode(errors="replace")))
+    return out
 
 
 class RocmInstance:

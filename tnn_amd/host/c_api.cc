@@ -194,6 +194,27 @@ HOST_API int tnn_host_get_output_device(void *hp, const char *name, int mat_type
     return 0;
 }
 
+// MatUtils::Copy (include/tnn/utils/mat_utils.h:77-79) three times: the host Mat `in` into a DEVICE_ROCM Mat the engine
+// allocates, that one into a second DEVICE_ROCM Mat, and that one back into the host Mat `out`.
+HOST_API int tnn_host_mat_copy_round_trip(const void *in, void *out, int mat_type, const int *dims, int ndims, char *err,
+                                          size_t err_len) {
+    DimsVector d(dims, dims + ndims);
+    Mat src(DEVICE_NAIVE, MatTypeOf(mat_type), d, const_cast<void *>(in));
+    Mat first(DEVICE_ROCM, MatTypeOf(mat_type), d), second(DEVICE_ROCM, MatTypeOf(mat_type), d, nullptr);
+    Mat back(DEVICE_NAIVE, MatTypeOf(mat_type), d, out);
+    Status st = MatUtils::Copy(src, first, nullptr);
+    if (st == TNN_OK)
+        st = MatUtils::Copy(first, second, nullptr);  // `second` has no memory yet: Copy allocates it on its device
+    if (st == TNN_OK)
+        st = MatUtils::Copy(second, back, nullptr);
+    if (st != TNN_OK) {
+        if (err && err_len)
+            snprintf(err, err_len, "%s", st.description().c_str());
+        return (int)st == 0 ? -1 : (int)st;
+    }
+    return 0;
+}
+
 // The flow of the engine's blob-converter unit test (test/unit_test/blob_converter_test.cc:287-349) on an input blob of
 // this instance: fp32 NCHW Mat in with per-channel scale and bias, the blob back out as an fp32 NCHW Mat with the same
 // scale and bias applied again.

@@ -46,11 +46,14 @@ int DataTypeUtils::GetBytesSize(DataType dt) {
     }
 }
 
+// the engine's rule (memory_manager/blob_memory_size_info.cc:21-36): linear memory is one dimension, two dimensions
+// are a four-channel image, anything else has no size
 int64_t GetBlobMemoryBytesSize(BlobMemorySizeInfo &info) {
-    int64_t n = 1;
-    for (int d : info.dims)
-        n *= d;
-    return n * DataTypeUtils::GetBytesSize(info.data_type);
+    if (info.dims.size() == 1)
+        return (int64_t)info.dims[0] * DataTypeUtils::GetBytesSize(info.data_type);
+    if (info.dims.size() == 2)
+        return (int64_t)info.dims[0] * info.dims[1] * 4 * DataTypeUtils::GetBytesSize(info.data_type);
+    return 0;
 }
 
 // ---- registries (source/tnn/core/abstract_device.cc:51-64, layer_type.cc:24-270) ----------------
@@ -160,6 +163,41 @@ Status BlobConverter::ConvertFromMatAsync(Mat &image, MatConvertParam param, voi
     if (!impl_)
         return Status(TNNERR_INIT_LAYER, "blob converter is nil, check device type");
     return impl_->ConvertFromMatAsync(image, param, q);
+}
+
+std::shared_ptr<MatConverterManager> &MatConverterManager::Shared() {
+    static std::shared_ptr<MatConverterManager> m = std::make_shared<MatConverterManager>();
+    return m;
+}
+int MatConverterManager::RegisterMatConverterAccCreater(DeviceType type, std::shared_ptr<MatConverterAccCreater> creater) {
+    converter_creater_map_[type] = creater;
+    return 0;
+}
+std::shared_ptr<MatConverterAcc> MatConverterManager::CreateMatConverterAcc(DeviceType device_type) {
+    auto it = converter_creater_map_.find(device_type);
+    return it == converter_creater_map_.end() ? nullptr : it->second->CreateMatConverterAcc();
+}
+Status MatUtils::Copy(Mat &src, Mat &dst, void *command_queue) {  // mat_utils.cc:73-100
+    if (src.GetMatType() != dst.GetMatType())
+        return Status(TNNERR_PARAM_ERR, "src and dst have different mat types");
+    if (!DimsVectorUtils::Equal(src.GetDims(), dst.GetDims()))
+        return Status(TNNERR_PARAM_ERR, "src and dst dims not equal");
+    const DeviceType s = src.GetDeviceType(), d = dst.GetDeviceType();
+    DeviceType where;
+    if (s == d)
+        where = s;
+    else if (s == DEVICE_NAIVE || s == DEVICE_ARM)
+        where = d;
+    else if (d == DEVICE_NAIVE || d == DEVICE_ARM)
+        where = s;
+    else
+        return Status(TNNERR_PARAM_ERR, "src and dst DeviceType need be equal or one is device cpu");
+    if (dst.GetData() == nullptr)
+        dst = Mat(dst.GetDeviceType(), dst.GetMatType(), dst.GetDims());
+    auto converter = MatConverterManager::Shared()->CreateMatConverterAcc(where);
+    if (!converter)
+        return Status(TNNERR_INIT_LAYER, "image converter is nil, check device type");
+    return converter->Copy(src, dst, command_queue);
 }
 
 // ---- model interpreter (source/tnn/interpreter/tnn/model_interpreter.cc:174-476) ----------------

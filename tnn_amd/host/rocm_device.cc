@@ -2,6 +2,7 @@
 #include "rocm_device.h"
 #include <immintrin.h>
 
+#include <cstdint>
 #include <cstdio>
 
 namespace TNN_NS {
@@ -206,7 +207,14 @@ Status RocmDevice::Allocate(void **handle, MatType mat_type, DimsVector dims) {
                      : mat_type == RESERVED_FP16_TEST  ? DATA_TYPE_HALF
                      : mat_type == RESERVED_BFP16_TEST ? DATA_TYPE_BFP16
                                                        : DATA_TYPE_INT8;
-    info.dims      = dims;
+    // one dimension: the engine's byte count knows linear memory only in that form (blob_memory_size_info.cc:21-36 gives 0
+    // for any other rank); the image Mat types hold one byte per element of dims
+    int64_t count = 1;
+    for (int d : dims)
+        count *= d > 0 ? d : 0;
+    if (count > INT32_MAX)
+        return Status(TNNERR_PARAM_ERR, "mat with more than 2^31 elements");
+    info.dims = {(int)(count > 0 ? count : 1)};
     return Allocate(handle, info);
 }
 Status RocmDevice::Allocate(void **handle, BlobMemorySizeInfo &size_info) {
@@ -751,6 +759,58 @@ private:
     void *params_      = nullptr;  // scale and bias of a device mat's conversion, on the device
     size_t params_sz_  = 0;
 };
+
+// ---- Mat converter (role of source/tnn/device/cuda/cuda_mat_converter.cc): MatUtils::Copy between a host Mat and a
+// DEVICE_ROCM Mat, or between two DEVICE_ROCM Mats.  The image operations (resize, crop, warp, colour conversion, border)
+// prepare camera frames for vision models and are not part of this backend. ----
+class RocmMatConverterAcc : public MatConverterAcc {
+public:
+    Status Copy(Mat &src, Mat &dst, void *command_queue = nullptr) override {
+        if (!src.GetData() || !dst.GetData())
+            return Status(TNNERR_NULL_PARAM, "mat without memory");
+        if (src.GetMatType() != dst.GetMatType())
+            return Status(TNNERR_PARAM_ERR, "src and dst have different mat types");
+        size_t elem = 0;
+        switch (src.GetMatType()) {
+            case NCHW_FLOAT:
+            case NC_INT32: elem = 4; break;
+            case RESERVED_BFP16_TEST:
+            case RESERVED_FP16_TEST: elem = 2; break;
+            case RESERVED_INT8_TEST:
+            case N8UC3:
+            case N8UC4:
+            case NGRAY: elem = 1; break;
+            default: return Status(TNNERR_PARAM_ERR, "RocmMatConverter: mat type without a plain element layout");
+        }
+        const size_t bytes = (size_t)DimsVectorUtils::Count(src.GetDims()) * elem;
+        if ((size_t)DimsVectorUtils::Count(dst.GetDims()) * elem != bytes)
+            return Status(TNNERR_PARAM_ERR, "src and dst dims not equal");
+        const bool src_dev = src.GetDeviceType() == DEVICE_ROCM, dst_dev = dst.GetDeviceType() == DEVICE_ROCM;
+        if (src_dev && dst_dev) {
+            ROCM_CALL(tnn_rocm_memcpy_d2d(dst.GetData(), src.GetData(), bytes, command_queue));
+            ROCM_CALL(tnn_rocm_stream_sync(command_queue));
+        } else if (dst_dev) {
+            ROCM_CALL(tnn_rocm_memcpy_h2d(dst.GetData(), src.GetData(), bytes, command_queue));  // waits for the stream
+        } else if (src_dev) {
+            ROCM_CALL(tnn_rocm_memcpy_d2h(dst.GetData(), src.GetData(), bytes, command_queue));
+        } else {
+            return Status(TNNERR_PARAM_ERR, "RocmMatConverter: neither mat is on DEVICE_ROCM");
+        }
+        return TNN_OK;
+    }
+    Status Resize(Mat &, Mat &, ResizeParam, void * = nullptr) override { return NotBuilt("Resize"); }
+    Status Crop(Mat &, Mat &, CropParam, void * = nullptr) override { return NotBuilt("Crop"); }
+    Status WarpAffine(Mat &, Mat &, WarpAffineParam, void * = nullptr) override { return NotBuilt("WarpAffine"); }
+    Status CvtColor(Mat &, Mat &, ColorConversionType, void * = nullptr) override { return NotBuilt("CvtColor"); }
+    Status CopyMakeBorder(Mat &, Mat &, CopyMakeBorderParam, void * = nullptr) override { return NotBuilt("CopyMakeBorder"); }
+
+private:
+    static Status NotBuilt(const char *what) {
+        return Status(TNNERR_PARAM_ERR, std::string("RocmMatConverter: ") + what + " (image preparation) is not part of DEVICE_ROCM");
+    }
+};
+DECLARE_MAT_CONVERTER_CREATER(Rocm);
+REGISTER_MAT_CONVERTER(Rocm, DEVICE_ROCM);
 
 DECLARE_BLOB_CONVERTER_CREATER(Rocm);
 REGISTER_BLOB_CONVERTER(Rocm, DEVICE_ROCM);

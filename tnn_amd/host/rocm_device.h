@@ -22,6 +22,7 @@
 #include "tnn/optimizer/net_optimizer_manager.h"
 #include "tnn/utils/blob_converter_internal.h"
 #include "tnn/utils/data_type_utils.h"
+#include "tnn/utils/mat_converter_acc.h"
 #include "tnn/utils/dims_utils.h"
 #include "rocm_engine_additions.h"
 #else

@@ -595,6 +595,60 @@ private:
     std::shared_ptr<BlobConverterAcc> impl_;
 };
 
+// ---- Mat utilities (include/tnn/utils/mat_utils.h:90-114, source/tnn/utils/mat_converter_acc.h:28-86): of the
+// engine's operations on Mats only Copy concerns this path (the rest prepares camera images); the parameter structs of
+// the others are declared so that a device's converter has the engine's interface ----
+struct ResizeParam {};
+struct CropParam {};
+struct WarpAffineParam {};
+struct CopyMakeBorderParam {};
+typedef enum { COLOR_CONVERT_NV12TOBGR = 0 } ColorConversionType;
+class MatConverterAcc {
+public:
+    virtual ~MatConverterAcc() {}
+    virtual Status Copy(Mat &src, Mat &dst, void *command_queue = nullptr)                                      = 0;
+    virtual Status Resize(Mat &src, Mat &dst, ResizeParam param, void *command_queue = nullptr)                 = 0;
+    virtual Status Crop(Mat &src, Mat &dst, CropParam param, void *command_queue = nullptr)                     = 0;
+    virtual Status WarpAffine(Mat &src, Mat &dst, WarpAffineParam param, void *command_queue = nullptr)         = 0;
+    virtual Status CvtColor(Mat &src, Mat &dst, ColorConversionType type, void *command_queue = nullptr)        = 0;
+    virtual Status CopyMakeBorder(Mat &src, Mat &dst, CopyMakeBorderParam param, void *command_queue = nullptr) = 0;
+};
+class MatConverterAccCreater {
+public:
+    virtual ~MatConverterAccCreater() {}
+    virtual std::shared_ptr<MatConverterAcc> CreateMatConverterAcc() = 0;
+};
+class MatConverterManager {
+public:
+    static std::shared_ptr<MatConverterManager> &Shared();
+    std::shared_ptr<MatConverterAcc> CreateMatConverterAcc(DeviceType device_type);
+    int RegisterMatConverterAccCreater(DeviceType type, std::shared_ptr<MatConverterAccCreater> creater);
+
+private:
+    std::map<DeviceType, std::shared_ptr<MatConverterAccCreater>> converter_creater_map_;
+};
+template <typename T> class MatConverterAccRegister {
+public:
+    explicit MatConverterAccRegister(DeviceType type) {
+        MatConverterManager::Shared()->RegisterMatConverterAccCreater(type, std::make_shared<T>());
+    }
+};
+#define DECLARE_MAT_CONVERTER_CREATER(device)                                                                          \
+    class device##MatConverterAccCreater : public MatConverterAccCreater {                                             \
+    public:                                                                                                            \
+        virtual ~device##MatConverterAccCreater() {}                                                                   \
+        virtual std::shared_ptr<MatConverterAcc> CreateMatConverterAcc() {                                             \
+            return std::make_shared<device##MatConverterAcc>();                                                        \
+        }                                                                                                              \
+    }
+#define REGISTER_MAT_CONVERTER(device, device_type)                                                                    \
+    MatConverterAccRegister<device##MatConverterAccCreater> g_mat_converter_##device(device_type)
+class MatUtils {
+public:
+    // copy between a host Mat and a device Mat, or two Mats of one device, of equal dims (mat_utils.cc:73-100)
+    static Status Copy(Mat &src, Mat &dst, void *command_queue);
+};
+
 // ---- layers (device independent): shape and dtype inference -------------------------------------
 class DefaultNetwork;
 class BaseLayer {
