@@ -487,3 +487,30 @@ def test_mat_utils_copy_inside_the_reference_engine():
     for shape in ((1, 1, 1, 1), (2, 3, 7, 5), (4, 1, 96, 256)):   # the engine's check wants the four image dims
         a = rng.standard_normal(shape).astype(np.float32)
         assert np.array_equal(ref_driver.mat_copy_round_trip("ROCM", a), a), shape
+
+
+def test_weight_only_int8_model_inside_the_reference_engine():
+    """A dynamic-range quantised model (int8 MatMul weights and embedding tables + fp32 scales) in the reference engine:
+    its own dequantisation pass runs ahead of the ROCm passes (both at priority P1, ordered by name), so DEVICE_ROCM
+    still runs the fused layers and agrees with DEVICE_NAIVE on the same file."""
+    engine()
+    say("reference engine: weight-only int8 model, DEVICE_ROCM next to DEVICE_NAIVE")
+    cfg = EncoderConfig(2, 256, 4, 512)
+    w = make_weights(cfg, seed=93, bias_std=0.05)
+    B, S = 2, 40
+    w["pos_emb"] = w["pos_emb"][:S]
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 9, S, seed=94)
+    graph = tnnmodel.encoder_graph(cfg, w, B, S)
+    graph.weight_only_int8()
+    inputs = {"input_ids": ids.astype(np.int32), "token_type_ids": seg.astype(np.int32),
+              "attention_bias": mask.reshape(B, 1, 1, S).astype(np.float32)}
+    want = run(graph, "NAIVE", inputs, "last_hidden")[0]
+    got32 = run(graph, "ROCM:fp32", inputs, "last_hidden", forwards=2)
+    got16 = run(graph, "ROCM", inputs, "last_hidden", forwards=4)
+    assert all(np.array_equal(g, got32[0]) for g in got32) and all(np.array_equal(g, got16[0]) for g in got16)
+    e32, e16 = rel_err(got32[0], want), rel_err(got16[0], want)
+    say("  fp32 blobs %.3g, fp16 blobs (fused) %.3g" % (e32, e16))
+    assert e32 <= 2e-3 and e16 <= 1e-2
+    # and against the float model: the quantisation itself costs something, the device adds nothing to it
+    plain = run(tnnmodel.encoder_graph(cfg, w, B, S), "NAIVE", inputs, "last_hidden")[0]
+    assert 1e-4 < rel_err(want, plain) < 0.2

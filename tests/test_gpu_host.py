@@ -1204,3 +1204,86 @@ def test_mat_utils_copy_to_the_device_and_back(np_dtype):
         else:
             a = rng.integers(-120, 120, shape).astype(np_dtype)
         assert np.array_equal(host.mat_copy_round_trip(a).view(np.uint8), a.view(np.uint8)), shape
+
+
+def _grid_weights(cfg, S, seed):
+    """encoder weights that are int8 multiples of 2^-9 with the largest magnitude (127 * 2^-9) present in every matrix
+    and in every table row: quantising them by max|w| / 127 gives them back exactly"""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    w = make_weights(cfg, seed=seed, bias_std=0.05)
+    w["pos_emb"] = w["pos_emb"][:S]
+    step = np.float32(2.0 ** -9)
+
+    def snap(a, per_row):
+        q = np.clip(np.rint(a / step), -127, 127).astype(np.float32)
+        if per_row:
+            q[:, 0] = 127.0
+        else:
+            q.flat[0] = 127.0
+        return (q * step).astype(np.float32)
+
+    for key in ("word_emb", "type_emb"):
+        w[key] = snap(w[key], True)
+    for lw in w["layers"]:
+        for key, a in lw.items():
+            if a.ndim == 2:
+                lw[key] = snap(a, False)
+    return w
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_weight_only_int8_model_runs_as_its_dequantised_float_form(precision):
+    """Dynamic range quantisation (int8 MatMul weights and embedding tables with fp32 scales in the model file, float
+    arithmetic at run time: net_optimizer_dynamic_range_dequant.cc): the model gives bit for bit what the float model
+    with the weights scale * int8 gives, through the fused layers."""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: weight-only int8 model against its dequantised float form, " + precision)
+    cfg = EncoderConfig(2, 256, 4, 512)
+    B, S = 2, 48
+    w = _grid_weights(cfg, S, seed=91)
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 13, S, seed=92)
+    outs = []
+    for quantised in (False, True):
+        g = tnnmodel.encoder_graph(cfg, w, B, S)
+        if quantised:
+            deq = g.weight_only_int8()
+            assert np.array_equal(deq["emb_word"], w["word_emb"]) and np.array_equal(deq["l0_q_mm"], w["layers"][0]["wq"].T)
+        inst = host.RocmInstance.from_graph(g, precision)
+        if precision == "fp16":
+            assert any(t == "RocmFusedAttention" for t, _ in inst.layers())
+        inst.set_input("input_ids", ids)
+        inst.set_input("token_type_ids", seg)
+        inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+        inst.forward()
+        outs.append(inst.output("last_hidden"))
+        inst.close()
+    assert np.isfinite(outs[0]).all() and np.abs(outs[0]).max() > 0.1
+    assert np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_weight_only_int8_inner_product_form(precision):
+    """the InnerProduct spelling of the projections with weight-only int8 weights (DynamicRangeQuantizedInnerProduct: int8
+    weight, float bias, one scale): bit for bit the float model with the weights scale * int8"""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: weight-only int8 InnerProduct projections, " + precision)
+    cfg = EncoderConfig(1, 256, 4, 512)
+    B, S, H = 2, 40, 256
+    lw = _grid_weights(cfg, S, seed=95)["layers"][0]
+    rng = np.random.default_rng(96)
+    x = rng.standard_normal((B * S, H)).astype(np.float32)
+    mask = np.zeros((B, 1, 1, S), np.float32)
+    mask[0, 0, 0, 31:] = -10000.0
+    outs = []
+    for quantised in (False, True):
+        g = tnnmodel.attention_block_graph(lw, B, S, H, 4, proj="inner_product")
+        if quantised:
+            deq = g.weight_only_int8()
+            assert len(deq) == 4 and "DynamicRangeQuantizedInnerProduct" in g.proto()
+        inst = host.RocmInstance.from_graph(g, precision)
+        inst.set_input("hidden", x)
+        inst.set_input("attention_bias", mask)
+        inst.forward()
+        outs.append(inst.output("y"))
+        inst.close()
+    assert np.abs(outs[0]).max() > 0.1 and np.array_equal(outs[0], outs[1])

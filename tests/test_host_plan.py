@@ -380,3 +380,28 @@ def test_every_encoder_blob_named_as_model_output_survives_the_rewrites():
         assert blob in got and got[blob] == dims[blob], blob
         asked += 1
     assert asked > 20
+
+
+def test_weight_only_int8_model_plans_like_its_float_form():
+    """A model whose MatMul weights and embedding tables were stored as int8 + scale (the engine's dynamic range
+    quantisation: DynamicRangeQuantizedMatMul / Gather layers, net_optimizer_dynamic_range_dequant.cc) is dequantised
+    before the device's passes see it, so it is rewritten into the same fused layers as the float model; a weight record
+    whose scale is missing is refused."""
+    cfg, w, g = _graph()
+    plain = _types(host.plan(g, precision="fp16"))
+    _, _, g8 = _graph()
+    deq = g8.weight_only_int8()
+    assert len(deq) == 2 + 6 * cfg.layers            # two tables, six projections per layer
+    text = g8.proto()
+    assert text.count("DynamicRangeQuantizedMatMul") == 6 * cfg.layers and text.count("DynamicRangeQuantizedGather") == 2
+    assert len(g8.model()) < len(g.model()) // 3
+    assert _types(host.plan(g8, precision="fp16")) == plain
+    assert _types(host.plan(g8, precision="fp32")) == _types(host.plan(g, precision="fp32"))
+    # the scale record of the first MatMul taken out of the file: the int8 weight is left without a float scale
+    model = g8.model()
+    first = [r for r in _raw_buffer_records(model) if r[1] == 2 and len(r[3]) == 2 and r[3][0] == cfg.hidden][0]
+    at = first[0] + 16 + 4 * len(first[3]) + first[2]     # the record behind the int8 weight: its scale
+    damaged = bytearray(model)
+    damaged[at + 4:at + 8] = (2).to_bytes(4, "little")     # typed int8 instead of float
+    with pytest.raises(host.HostError):
+        host.plan(text, bytes(damaged), "fp16")

@@ -105,6 +105,9 @@ LayerType GlobalConvertLayerType(std::string s) {
         {"Gather", LAYER_GATHER},             {"MatMul", LAYER_MATMUL},
         {"LayerNorm", LAYER_LAYER_NORM},      {"GELU", LAYER_GELU},
         {"BlobScale", LAYER_BLOB_SCALE},      {"QuantizedAdd", LAYER_ADD},
+        // weight-only int8 ("dynamic range quantisation", layer_type.cc:261-265): the layer computes in float
+        {"DynamicRangeQuantizedMatMul", LAYER_MATMUL}, {"DynamicRangeQuantizedInnerProduct", LAYER_INNER_PRODUCT},
+        {"DynamicRangeQuantizedGather", LAYER_GATHER},
         {"RocmFusedLinear", LAYER_ROCM_FUSED_LINEAR}, {"RocmFusedAttention", LAYER_ROCM_FUSED_ATTENTION},
         {"RocmFusedLinearInt8", LAYER_ROCM_FUSED_LINEAR_INT8}, {"RocmGeluInt8", LAYER_ROCM_GELU_INT8},
         {"RocmLayerNormQuant", LAYER_ROCM_LAYER_NORM_QUANT},
@@ -485,6 +488,8 @@ Status ModelInterpreter::InterpretProto(const std::string &content) {
         RETURN_ON_NEQ(ParseLayerParam(layer->type, f, idx, layer->param), TNN_OK);
         if (layer->type_str.compare(0, 9, "Quantized") == 0)
             layer->param->quantized = true;  // model_interpreter.cc:371-373
+        if (layer->type_str.compare(0, 21, "DynamicRangeQuantized") == 0)
+            layer->param->dynamic_range_quantized = true;  // model_interpreter.cc:375-378
         layer->param->type = layer->type_str;
         layer->param->name = layer->name;
         structure_.layers.push_back(layer);
@@ -999,6 +1004,110 @@ void optimizer::NetOptimizerManager::RegisterNetOptimizer(NetOptimizer *opt, Opt
     if (opt && opt->Strategy().length() > 0)
         OptimizerList().push_back({(int)prior, std::shared_ptr<NetOptimizer>(opt)});
 }
+// The engine's own pass for weight-only int8 models (optimizer/net_optimizer_dynamic_range_dequant.cc:44-330, priority
+// P1, ahead of every device's passes by its name): the int8 weights of MatMul (resource or constant-map form),
+// InnerProduct and Gather tables become fp32 = scale * value before any layer is created, and the layers run as float
+// layers from then on.
+namespace {
+class DynamicRangeDequantPass : public optimizer::NetOptimizer {
+public:
+    std::string Strategy() override { return "net_optimizer_dynamic_range_dequant"; }
+    bool IsSupported(const NetworkConfig &) override { return true; }
+    Status Optimize(NetStructure *structure, NetResource *resource) override {
+        if (!structure)
+            return Status(TNNERR_NET_ERR, "Error: empty NetStructure");
+        if (structure->layers.size() <= 1)
+            return TNN_OK;
+        for (auto &layer : structure->layers) {
+            if (!layer || !layer->param || !layer->param->dynamic_range_quantized)
+                continue;
+            auto it            = resource->resource_map.find(layer->name);
+            LayerResource *res = it == resource->resource_map.end() ? nullptr : it->second.get();
+            switch (layer->type) {
+                case LAYER_MATMUL: {
+                    auto p = dynamic_cast<MatMulLayerParam *>(layer->param.get());
+                    auto r = dynamic_cast<MatMulLayerResource *>(res);
+                    if (p && p->weight_position == 1) {
+                        if (!r)
+                            return Status(TNNERR_INVALID_MODEL, "dynamic range quantised MatMul without resource: " + layer->name);
+                        RETURN_ON_NEQ(PerTensor(r->weight, r->scale_handle, layer->name), TNN_OK);
+                    } else if (p && p->weight_position == -1 && layer->inputs.size() == 2) {
+                        // the int8 operand is a constant, its scale sits next to it under a suffixed name (:203-238)
+                        for (const std::string &name : layer->inputs) {
+                            auto c = resource->constant_map.find(name);
+                            if (c == resource->constant_map.end() || !c->second || c->second->GetDataType() != DATA_TYPE_INT8)
+                                continue;
+                            const std::string scale_name = name + "_dynamic_range_quant_scale";
+                            auto sc                      = resource->constant_map.find(scale_name);
+                            if (sc == resource->constant_map.end() || !sc->second)
+                                return Status(TNNERR_PARAM_ERR, "scale is not found in constant map");
+                            RETURN_ON_NEQ(PerTensor(*c->second, *sc->second, layer->name), TNN_OK);
+                            resource->constant_map.erase(scale_name);
+                            break;
+                        }
+                    }
+                    break;
+                }
+                case LAYER_INNER_PRODUCT: {
+                    auto r = dynamic_cast<InnerProductLayerResource *>(res);
+                    if (!r)
+                        return Status(TNNERR_INVALID_MODEL, "dynamic range quantised InnerProduct without resource: " + layer->name);
+                    RETURN_ON_NEQ(PerTensor(r->weight_handle, r->scale_handle, layer->name), TNN_OK);
+                    break;
+                }
+                case LAYER_GATHER: {  // one scale per row of the table (:277-322)
+                    auto p = dynamic_cast<GatherLayerParam *>(layer->param.get());
+                    auto r = dynamic_cast<GatherLayerResource *>(res);
+                    if (!p || !p->data_in_resource || !r)
+                        break;
+                    const DimsVector dims = r->data.GetBufferDims();
+                    if (r->data.GetDataType() != DATA_TYPE_INT8 || dims.size() < 2 || r->scale_data.GetDataCount() != dims[0] ||
+                        r->scale_data.GetDataType() != DATA_TYPE_FLOAT)
+                        break;  // "might have been dequantized before"
+                    const int count = r->data.GetDataCount(), rows = dims[0];
+                    if (rows <= 0 || count % rows != 0)
+                        return Status(TNNERR_INVALID_MODEL, "dynamic range quantised Gather table with ragged rows: " + layer->name);
+                    const int stride = count / rows;
+                    RawBuffer wide(count * 4, dims);
+                    wide.SetDataType(DATA_TYPE_FLOAT);
+                    const int8_t *q  = r->data.force_to<int8_t *>();
+                    const float *sc  = r->scale_data.force_to<float *>();
+                    float *w         = wide.force_to<float *>();
+                    for (int i = 0; i < rows; ++i)
+                        for (int j = 0; j < stride; ++j)
+                            w[(size_t)i * stride + j] = sc[i] * (float)q[(size_t)i * stride + j];
+                    r->data = wide;
+                    break;
+                }
+                default: break;
+            }
+            layer->param->dynamic_range_quantized = false;
+        }
+        return TNN_OK;
+    }
+
+private:
+    // fp32 = scale[0] * int8 in place of the int8 record, dims kept (:176-192, 249-268)
+    static Status PerTensor(RawBuffer &weight, const RawBuffer &scale, const std::string &layer) {
+        if (weight.GetDataType() != DATA_TYPE_INT8)
+            return TNN_OK;  // "might have been dequantized before"
+        if (scale.GetDataCount() < 1 || scale.GetDataType() != DATA_TYPE_FLOAT)
+            return Status(TNNERR_INVALID_MODEL, "dynamic range quantised weight without a float scale: " + layer);
+        const int count = weight.GetDataCount();
+        RawBuffer wide(count * 4, weight.GetBufferDims());
+        wide.SetDataType(DATA_TYPE_FLOAT);
+        const int8_t *q = weight.force_to<int8_t *>();
+        const float s   = scale.force_to<float *>()[0];
+        float *w        = wide.force_to<float *>();
+        for (int i = 0; i < count; ++i)
+            w[i] = s * (float)q[i];
+        weight = wide;
+        return TNN_OK;
+    }
+};
+optimizer::NetOptimizerRegister<DynamicRangeDequantPass> g_dynamic_range_dequant(optimizer::P1);
+}  // namespace
+
 Status optimizer::NetOptimizerManager::Optimize(NetStructure *structure, NetResource *resource, const NetworkConfig &config) {
     std::lock_guard<std::mutex> lock(g_optimize_mutex);
     auto list = OptimizerList();

@@ -27,7 +27,8 @@ _NP2DT = {np.dtype(np.float32): DT_FLOAT, np.dtype(np.float16): DT_HALF, np.dtyp
 # LayerType numbers (source/tnn/core/layer_type.h) for the resource headers; the reader re-derives the type
 # from the type string, the number only has to be in range.
 _LAYER_TYPE_NUM = {"InnerProduct": 19, "QuantizedInnerProduct": 19, "Add": 38, "Mul": 42, "Sub": 39, "Div": 43,
-                   "Gather": 104, "MatMul": 105, "BlobScale": 600}
+                   "Gather": 104, "MatMul": 105, "BlobScale": 600, "DynamicRangeQuantizedMatMul": 105,
+                   "DynamicRangeQuantizedGather": 104, "DynamicRangeQuantizedInnerProduct": 19}
 BLOB_SCALE_SUFFIX = "_scale_data_"
 
 
@@ -64,6 +65,7 @@ class Graph:
         self.resources = []   # (name, type_str, payload bytes) in layer order
         self.constants = {}   # blob name -> ndarray
         self.blobs = []
+        self._float_weights = {}  # layer name -> ("MatMul" | "Gather", fp32 array): what weight_only_int8() rewrites
 
     def _blob(self, name):
         if name not in self.blobs:
@@ -91,6 +93,7 @@ class Graph:
 
     def res_matmul(self, name, weight_kn):
         self._res(name, "MatMul", raw_buffer(weight_kn))
+        self._float_weights[name] = ("MatMul", np.ascontiguousarray(weight_kn, np.float32))
 
     def res_eltwise(self, name, type_str, element):
         self._res(name, type_str, raw_buffer(element))
@@ -99,6 +102,8 @@ class Graph:
         p = (_i32(1) + raw_buffer(data)) if data is not None else _i32(0)
         p += (_i32(1) + raw_buffer(indices)) if indices is not None else _i32(0)
         self._res(name, "Gather", p)
+        if data is not None and indices is None and np.asarray(data).dtype == np.float32 and np.asarray(data).ndim == 2:
+            self._float_weights[name] = ("Gather", np.ascontiguousarray(data, np.float32))
 
     def res_inner_product(self, name, weight_nk, bias=None, quant_scale=None):
         """fp32: weight [N,K] + bias [N].  int8: int8 weight, int32 bias, zero points (int8 zeros), fp32 scale."""
@@ -108,6 +113,8 @@ class Graph:
             type_str = "QuantizedInnerProduct"
             zp = np.zeros(quant_scale.shape, np.int8)
             p += raw_buffer(zp) + raw_buffer(np.asarray(quant_scale, np.float32))
+        elif np.asarray(weight_nk).dtype == np.float32:
+            self._float_weights[name] = ("InnerProduct", np.ascontiguousarray(weight_nk, np.float32), bias)
         self._res(name, type_str, p)
 
     def res_blob_scale(self, blob_name, scale):
@@ -115,6 +122,36 @@ class Graph:
         zp = np.zeros(scale.shape, np.int8)
         bias = np.zeros(scale.shape, np.int32)
         self._res(blob_name + BLOB_SCALE_SUFFIX, "BlobScale", raw_buffer(zp) + raw_buffer(scale) + raw_buffer(bias))
+
+    def weight_only_int8(self):
+        """The model as the engine's weight-only quantiser leaves it (tools/dynamic_range_quantization; the file format of
+        model_packer.cc:148-153 and mat_mul / gather_layer_interpreter.cc): every MatMul weight resource becomes int8 with
+        one fp32 scale (max|w| / 127, symmetric), every fp32 Gather table int8 with one scale per row, and the layers are
+        typed DynamicRangeQuantized*.  Returns {layer name: the fp32 weights scale * int8 the engine will compute with}."""
+        dequantised = {}
+        for name, entry in self._float_weights.items():
+            kind, w = entry[0], entry[1]
+            if kind == "InnerProduct":   # weight, bias, then the scale alone (inner_product_layer_interpreter.cc:111-114)
+                scale = np.float32(np.abs(w).max() / 127.0) if w.size and np.abs(w).max() > 0 else np.float32(1.0)
+                q = np.clip(np.rint(w / scale), -127, 127).astype(np.int8)
+                payload = _str(name) + raw_buffer(q) + raw_buffer(entry[2]) + raw_buffer(np.array([scale], np.float32))
+                dequantised[name] = (scale * q.astype(np.float32)).astype(np.float32)
+            elif kind == "MatMul":
+                scale = np.float32(np.abs(w).max() / 127.0) if w.size and np.abs(w).max() > 0 else np.float32(1.0)
+                q = np.clip(np.rint(w / scale), -127, 127).astype(np.int8)
+                payload = raw_buffer(q) + raw_buffer(np.array([scale], np.float32))
+                dequantised[name] = (scale * q.astype(np.float32)).astype(np.float32)
+            else:
+                amax = np.abs(w).max(axis=1)
+                scale = np.where(amax > 0, amax / 127.0, 1.0).astype(np.float32)
+                q = np.clip(np.rint(w / scale[:, None]), -127, 127).astype(np.int8)
+                payload = _i32(1) + raw_buffer(q) + _i32(0) + raw_buffer(scale)
+                dequantised[name] = (scale[:, None] * q.astype(np.float32)).astype(np.float32)
+            new_type = "DynamicRangeQuantized" + kind
+            self.resources = [(n, new_type, payload) if n == name else (n, t, pl) for n, t, pl in self.resources]
+            self.layers = [(new_type, n, i, o, pr) if n == name else (t, n, i, o, pr) for t, n, i, o, pr in self.layers]
+        self._float_weights = {}
+        return dequantised
 
     # ---- serialisation ------------------------------------------------------------------------------
     def proto(self):
