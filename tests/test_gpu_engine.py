@@ -514,3 +514,33 @@ def test_weight_only_int8_model_inside_the_reference_engine():
     # and against the float model: the quantisation itself costs something, the device adds nothing to it
     plain = run(tnnmodel.encoder_graph(cfg, w, B, S), "NAIVE", inputs, "last_hidden")[0]
     assert 1e-4 < rel_err(want, plain) < 0.2
+
+
+def test_half_precision_weight_file_inside_the_reference_engine():
+    """a model file with half-precision weight records in the reference engine: DEVICE_NAIVE widens them layer by layer,
+    DEVICE_ROCM ahead of its rewrites; the two agree as they do on the fp32 file, and DEVICE_ROCM gives on the half file
+    exactly what it gives on the fp32 file of the same values"""
+    engine()
+    say("reference engine: half-precision weight file, DEVICE_ROCM next to DEVICE_NAIVE")
+    cfg = EncoderConfig(2, 256, 4, 512)
+    w = make_weights(cfg, seed=99, bias_std=0.05)
+    B, S = 2, 40
+    w["pos_emb"] = w["pos_emb"][:S]
+
+    def r16(a):
+        return a.astype(np.float16).astype(np.float32)
+    w = {k: ([{n: r16(a) for n, a in lw.items()} for lw in v] if k == "layers" else r16(v)) for k, v in w.items()}
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 9, S, seed=100)
+    inputs = {"input_ids": ids.astype(np.int32), "token_type_ids": seg.astype(np.int32),
+              "attention_bias": mask.reshape(B, 1, 1, S).astype(np.float32)}
+    plain = tnnmodel.encoder_graph(cfg, w, B, S)
+    half = tnnmodel.encoder_graph(cfg, w, B, S)
+    half.half_weights(tables=False, constants=False)   # what the engine's CPU devices widen: layer resources
+    want = run(half, "NAIVE", inputs, "last_hidden")[0]
+    assert np.array_equal(want, run(plain, "NAIVE", inputs, "last_hidden")[0])
+    for device, bar in (("ROCM:fp32", 2e-3), ("ROCM", 1e-2)):
+        got = run(half, device, inputs, "last_hidden", forwards=2)[0]
+        assert np.array_equal(got, run(plain, device, inputs, "last_hidden")[0]), device
+        e = rel_err(got, want)
+        say("  %s: %.3g" % (device, e))
+        assert e <= bar

@@ -1287,3 +1287,36 @@ def test_weight_only_int8_inner_product_form(precision):
         outs.append(inst.output("y"))
         inst.close()
     assert np.abs(outs[0]).max() > 0.1 and np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_half_precision_weight_file_runs_as_its_float_form(precision):
+    """a model file whose weights, biases, tables and constants are stored as IEEE half gives bit for bit what the fp32 file
+    holding the same (half-representable) values gives: the records are widened exactly, ahead of the rewrites"""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: half-precision weight file against the fp32 file of the same values, " + precision)
+    cfg = EncoderConfig(2, 256, 4, 512)
+    B, S = 2, 48
+    w = make_weights(cfg, seed=97, bias_std=0.05)
+    w["pos_emb"] = w["pos_emb"][:S]
+
+    def r16(a):
+        return a.astype(np.float16).astype(np.float32)
+    w = {k: ([{n: r16(a) for n, a in lw.items()} for lw in v] if k == "layers" else r16(v)) for k, v in w.items()}
+    ids, seg, lens, mask = make_inputs(cfg, B, S, 13, S, seed=98)
+    outs = []
+    for half_file in (False, True):
+        g = tnnmodel.encoder_graph(cfg, w, B, S)
+        if half_file:
+            g.half_weights()
+        inst = host.RocmInstance.from_graph(g, precision)
+        if precision == "fp16":
+            types = [t for t, _ in inst.layers()]
+            assert "RocmFusedAttention" in types and "RocmFusedEmbedding" in types, types
+        inst.set_input("input_ids", ids)
+        inst.set_input("token_type_ids", seg)
+        inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+        inst.forward()
+        outs.append(inst.output("last_hidden"))
+        inst.close()
+    assert np.abs(outs[0]).max() > 0.1 and np.array_equal(outs[0], outs[1])

@@ -405,3 +405,15 @@ def test_weight_only_int8_model_plans_like_its_float_form():
     damaged[at + 4:at + 8] = (2).to_bytes(4, "little")     # typed int8 instead of float
     with pytest.raises(host.HostError):
         host.plan(text, bytes(damaged), "fp16")
+
+
+def test_half_precision_weight_file_plans_like_its_float_form():
+    """a model file with its weights stored as IEEE half (the converter's option for files of half the size) is widened
+    ahead of the rewrites and ends as the same fused layers"""
+    cfg, w, g = _graph()
+    plain16, plain32 = _types(host.plan(g, precision="fp16")), _types(host.plan(g, precision="fp32"))
+    _, _, gh = _graph()
+    gh.half_weights()
+    assert len(gh.model()) < len(g.model()) * 0.55
+    assert _types(host.plan(gh, precision="fp16")) == plain16
+    assert _types(host.plan(gh, precision="fp32")) == plain32

@@ -359,6 +359,64 @@ static Status RocmCheckModel(NetStructure *s, NetResource *r) {
     return TNN_OK;
 }
 
+// Weights a model file stores in half precision (the converter's option for files of half the size) are widened to fp32
+// records before the rewrites look at them: the rewrites fold, transpose and concatenate weights in fp32, and the CPU
+// devices widen them as well, layer by layer (ConvertHalfResource, cpu_layer_acc.h:70-82, x86_mat_mul_layer_acc.cc:36-40).
+// Exact: every half value is an fp32 value.
+static float RocmHalfBitsToFloat(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu, man = h & 0x3FFu, bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else {  // subnormal: normalise
+            int shift = 0;
+            while (!(man & 0x400u)) {
+                man <<= 1;
+                ++shift;
+            }
+            bits = sign | ((uint32_t)(113 - shift) << 23) | ((man & 0x3FFu) << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7F800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 112) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+static void RocmWidenHalfRecord(RawBuffer &b) {
+    if (b.GetDataType() != DATA_TYPE_HALF || b.GetBytesSize() <= 0)
+        return;
+    const int count = b.GetDataCount();
+    RawBuffer wide(count * 4, b.GetBufferDims());
+    wide.SetDataType(DATA_TYPE_FLOAT);
+    const uint16_t *src = b.force_to<uint16_t *>();
+    float *dst          = wide.force_to<float *>();
+    for (int i = 0; i < count; ++i)
+        dst[i] = RocmHalfBitsToFloat(src[i]);
+    b = wide;
+}
+static void RocmWidenHalfWeights(NetResource *r) {
+    for (auto &kv : r->resource_map) {
+        LayerResource *res = kv.second.get();
+        if (auto m = dynamic_cast<MatMulLayerResource *>(res)) {
+            RocmWidenHalfRecord(m->weight);
+        } else if (auto ip = dynamic_cast<InnerProductLayerResource *>(res)) {
+            RocmWidenHalfRecord(ip->weight_handle);
+            RocmWidenHalfRecord(ip->bias_handle);
+        } else if (auto e = dynamic_cast<EltwiseLayerResource *>(res)) {
+            RocmWidenHalfRecord(e->element_handle);
+        } else if (auto g = dynamic_cast<GatherLayerResource *>(res)) {
+            RocmWidenHalfRecord(g->data);
+        }
+    }
+    for (auto &kv : r->constant_map)
+        if (kv.second)
+            RocmWidenHalfRecord(*kv.second);
+}
+
 class RocmFusionPass : public optimizer::NetOptimizer {
 public:
     std::string Strategy() override { return "net_optimizer_rocm_fuse_encoder"; }
@@ -369,6 +427,7 @@ public:
 
     Status Optimize(NetStructure *s, NetResource *r) override {
         RETURN_ON_NEQ(RocmCheckModel(s, r), TNN_OK);
+        RocmWidenHalfWeights(r);
         structure_ = s;
         resource_  = r;
         FuseEmbedding();

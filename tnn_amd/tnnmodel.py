@@ -65,7 +65,9 @@ class Graph:
         self.resources = []   # (name, type_str, payload bytes) in layer order
         self.constants = {}   # blob name -> ndarray
         self.blobs = []
-        self._float_weights = {}  # layer name -> ("MatMul" | "Gather", fp32 array): what weight_only_int8() rewrites
+        self._float_weights = {}  # layer name -> ("MatMul" | "Gather" | "InnerProduct", fp32 array[, bias]): what
+        #                           weight_only_int8() and half_weights() rewrite
+        self._float_operands = {}  # layer name -> (type string, fp32 operand of an Add / Sub / Mul / Div resource)
 
     def _blob(self, name):
         if name not in self.blobs:
@@ -97,6 +99,8 @@ class Graph:
 
     def res_eltwise(self, name, type_str, element):
         self._res(name, type_str, raw_buffer(element))
+        if element is not None and np.asarray(element).dtype == np.float32:
+            self._float_operands[name] = (type_str, np.ascontiguousarray(element, np.float32))
 
     def res_gather(self, name, data, indices=None):
         p = (_i32(1) + raw_buffer(data)) if data is not None else _i32(0)
@@ -152,6 +156,30 @@ class Graph:
             self.layers = [(new_type, n, i, o, pr) if n == name else (t, n, i, o, pr) for t, n, i, o, pr in self.layers]
         self._float_weights = {}
         return dequantised
+
+    def half_weights(self, tables=True, constants=True):
+        """The model as the converter's half-precision option stores it: every fp32 weight record (MatMul and InnerProduct
+        weights and biases, embedding tables, the operands of Add / Sub / Mul / Div resources, the constants) as IEEE half.
+        Layer types are unchanged; the devices widen the records when they load them (ConvertHalfResource,
+        source/tnn/interpreter/layer_resource_generator.cc:52-58).  tables / constants False leave the embedding tables
+        and the constant map in fp32 (the engine's CPU devices take half records for layer resources only)."""
+        def h(a):
+            return None if a is None else np.ascontiguousarray(a, np.float32).astype(np.float16)
+        new = {}
+        for name, entry in self._float_weights.items():
+            kind, w = entry[0], entry[1]
+            if kind == "MatMul":
+                new[name] = raw_buffer(h(w))
+            elif kind == "InnerProduct":
+                new[name] = _str(name) + raw_buffer(h(w)) + raw_buffer(h(entry[2]))
+            elif tables:
+                new[name] = _i32(1) + raw_buffer(h(w)) + _i32(0)
+        for name, (type_str, element) in self._float_operands.items():
+            new[name] = raw_buffer(h(element))
+        self.resources = [(n, t, new.get(n, pl)) for n, t, pl in self.resources]
+        if constants:
+            self.constants = {k: (h(v) if v.dtype == np.float32 else v) for k, v in self.constants.items()}
+        self._float_weights, self._float_operands = {}, {}
 
     # ---- serialisation ------------------------------------------------------------------------------
     def proto(self):
