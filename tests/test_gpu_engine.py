@@ -544,3 +544,27 @@ def test_half_precision_weight_file_inside_the_reference_engine():
         e = rel_err(got, want)
         say("  %s: %.3g" % (device, e))
         assert e <= bar
+
+
+def test_first_version_of_the_file_format_inside_the_reference_engine():
+    """the same attention block written in the first version of the file format (no rank or type on the input lines, no
+    dims in the weight records), read by the reference's own parser: DEVICE_ROCM agrees with DEVICE_NAIVE and gives the
+    bits it gives on the current format"""
+    engine()
+    say("reference engine: first version of the file format")
+    cfg = EncoderConfig(1, 256, 4, 512)
+    lw = make_weights(cfg, seed=5, bias_std=0.05)["layers"][0]
+    B, S, H = 2, 40, 256
+    x = np.random.default_rng(6).standard_normal((B * S, H)).astype(np.float32)
+    mask = np.zeros((B, 1, 1, S), np.float32)
+    mask[1, 0, 0, 25:] = -10000.0
+    inputs = {"hidden": x, "attention_bias": mask}
+    current = tnnmodel.attention_block_graph(lw, B, S, H, 4, proj="inner_product")
+    with tnnmodel.legacy_format():
+        old = tnnmodel.attention_block_graph(lw, B, S, H, 4, proj="inner_product")
+        got = {d: run(old, d, inputs, "y")[0] for d in ("NAIVE", "ROCM:fp32", "ROCM")}
+    for d in ("ROCM:fp32", "ROCM"):
+        assert np.array_equal(got[d], run(current, d, inputs, "y")[0]), d
+    e32, e16 = rel_err(got["ROCM:fp32"], got["NAIVE"]), rel_err(got["ROCM"], got["NAIVE"])
+    say("  fp32 blobs %.3g, fp16 blobs %.3g" % (e32, e16))
+    assert e32 <= 2e-3 and e16 <= 1e-2

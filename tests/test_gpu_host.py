@@ -1320,3 +1320,32 @@ def test_half_precision_weight_file_runs_as_its_float_form(precision):
         outs.append(inst.output("last_hidden"))
         inst.close()
     assert np.abs(outs[0]).max() > 0.1 and np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("precision", ["fp32", "fp16"])
+def test_first_version_of_the_file_format_runs_like_the_current_one(precision):
+    """an attention block stored in the first version of the file format gives the bits the current format gives"""
+    host, tnnmodel, EncoderConfig, make_weights, make_inputs = _mods()
+    say("host: first version of the file format, " + precision)
+    cfg = EncoderConfig(1, 256, 4, 512)
+    lw = make_weights(cfg, seed=5, bias_std=0.05)["layers"][0]
+    B, S, H = 2, 40, 256
+    x = np.random.default_rng(6).standard_normal((B * S, H)).astype(np.float32)
+    mask = np.zeros((B, 1, 1, S), np.float32)
+    mask[1, 0, 0, 25:] = -10000.0
+    outs = []
+    for legacy in (False, True):
+        if legacy:
+            with tnnmodel.legacy_format():
+                g = tnnmodel.attention_block_graph(lw, B, S, H, 4, proj="inner_product")
+                proto, model = g.proto(), g.model()
+        else:
+            g = tnnmodel.attention_block_graph(lw, B, S, H, 4, proj="inner_product")
+            proto, model = g.proto(), g.model()
+        inst = host.RocmInstance(proto, model, precision)
+        inst.set_input("hidden", x)
+        inst.set_input("attention_bias", mask)
+        inst.forward()
+        outs.append(inst.output("y"))
+        inst.close()
+    assert np.abs(outs[0]).max() > 0.1 and np.array_equal(outs[0], outs[1])

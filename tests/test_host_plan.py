@@ -417,3 +417,19 @@ def test_half_precision_weight_file_plans_like_its_float_form():
     assert len(gh.model()) < len(g.model()) * 0.55
     assert _types(host.plan(gh, precision="fp16")) == plain16
     assert _types(host.plan(gh, precision="fp32")) == plain32
+
+
+def test_first_version_of_the_file_format_plans_like_the_current_one():
+    """files of the first format version (proto magic 0x0FABC0002: input lines without rank and type, weight records
+    without dims; model_interpreter.cc:262-272, objseri.h:57-77) are read as the current ones are"""
+    cfg = EncoderConfig(1, 256, 4, 512)
+    lw = make_weights(cfg, seed=5)["layers"][0]
+    current = tnnmodel.attention_block_graph(lw, 2, 40, 256, 4, proj="inner_product")
+    with tnnmodel.legacy_format():
+        old = tnnmodel.attention_block_graph(lw, 2, 40, 256, 4, proj="inner_product")
+        proto, model = old.proto(), old.model()
+    assert "4206624770" in proto.split("\n")[0] and "hidden 80 256 :" in proto
+    assert len(model) < len(current.model())                      # no dims in the records
+    for precision in ("fp16", "fp32"):
+        a, b = host.plan(proto, model, precision), host.plan(current, precision=precision)
+        assert [(l["type"], l["output_dims"]) for l in a] == [(l["type"], l["output_dims"]) for l in b]

@@ -20,6 +20,8 @@ import struct
 import numpy as np
 
 MAGIC_V2 = 0x0FABC0004
+MAGIC_V1 = 0x0FABC0002
+_version = 2  # file version written: 2, or 1 inside `with legacy_format():`
 DT_FLOAT, DT_HALF, DT_INT8, DT_INT32 = 0, 1, 2, 3
 _NP2DT = {np.dtype(np.float32): DT_FLOAT, np.dtype(np.float16): DT_HALF, np.dtype(np.int8): DT_INT8,
           np.dtype(np.int32): DT_INT32}
@@ -45,15 +47,30 @@ def _str(s):
     return _i32(len(b)) + b
 
 
+class legacy_format:
+    """`with legacy_format():` -- graphs built AND serialised inside write the first version of the file format (proto
+    magic 0x0FABC0002: input lines are a name and its dims, every input is float; weight records carry no dims:
+    model_interpreter.cc:262-272, objseri.h:57-77), which old model files still have."""
+    def __enter__(self):
+        global _version
+        self._saved, _version = _version, 1
+
+    def __exit__(self, *exc):
+        global _version
+        _version = self._saved
+
+
 def raw_buffer(arr, dims=None):
     """Serialise one RawBuffer record.  `arr` None or empty gives the zero-length form."""
+    magic = MAGIC_V2 if _version == 2 else MAGIC_V1
     if arr is None or arr.size == 0:
-        return _u32(MAGIC_V2) + _i32(DT_FLOAT) + _i32(0)
+        return _u32(magic) + _i32(DT_FLOAT) + _i32(0)
     a = np.ascontiguousarray(arr)
     dt = _NP2DT[a.dtype]
-    dims = list(a.shape if dims is None else dims)
-    out = _u32(MAGIC_V2) + _i32(dt) + _i32(a.nbytes) + _i32(len(dims))
-    out += b"".join(_i32(d) for d in dims)
+    out = _u32(magic) + _i32(dt) + _i32(a.nbytes)
+    if _version == 2:
+        dims = list(a.shape if dims is None else dims)
+        out += _i32(len(dims)) + b"".join(_i32(d) for d in dims)
     return out + a.tobytes()
 
 
@@ -183,9 +200,13 @@ class Graph:
 
     # ---- serialisation ------------------------------------------------------------------------------
     def proto(self):
-        lines = ['"1 %d 1 %d ,"' % (len(self.blobs), MAGIC_V2)]
+        lines = ['"1 %d 1 %d ,"' % (len(self.blobs), MAGIC_V2 if _version == 2 else MAGIC_V1)]
         ins = []
         for name, dims, dt in self.inputs:
+            if _version == 1:
+                assert dt == DT_FLOAT, "the first file version has float inputs only"
+                ins.append("%s %s" % (name, " ".join(str(d) for d in dims)))
+                continue
             ins.append("%s %d %s %d" % (name, len(dims), " ".join(str(d) for d in dims), dt))
         lines.append('"%s ,"' % " : ".join(ins))
         lines.append('" %s ,"' % " ".join(self.blobs))
@@ -196,11 +217,12 @@ class Graph:
         return "\n".join(lines) + "\n"
 
     def model(self):
-        out = _u32(MAGIC_V2) + _i32(len(self.resources))
+        magic = MAGIC_V2 if _version == 2 else MAGIC_V1
+        out = _u32(magic) + _i32(len(self.resources))
         for name, type_str, payload in self.resources:
             out += _i32(_LAYER_TYPE_NUM.get(type_str, 0)) + _str(type_str) + _str(name) + payload
         if self.constants:
-            out += _u32(MAGIC_V2) + _i32(len(self.constants))
+            out += _u32(magic) + _i32(len(self.constants))
             for key in sorted(self.constants):
                 out += _str(key) + raw_buffer(self.constants[key])
         return out
