@@ -43,6 +43,9 @@ def parse():
     ap.add_argument("--seq", type=int, default=384)
     ap.add_argument("--layers", type=int, default=12)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-second-instance", action="store_true",
+                    help="leave out the untimed two-instances-at-once leg (kernel traces: its overlapping launches would "
+                         "mix into the per-kernel averages)")
     ap.add_argument("--cpu-seqs", type=int, default=2, help="sequences in the bounded CPU-baseline sample")
     ap.add_argument("--counter-reference", action="store_true",
                     help="also launch one element-wise kernel of known size (64 MiB read, 64 MiB written) so that a "
@@ -138,6 +141,37 @@ def main():
     inst.set_input_device("token_type_ids", d_in[1].data_ptr(), np.int32, [B, S])
     inst.set_input_device("attention_bias", d_in[2].data_ptr(), np.float32, [B, 1, 1, S])
     dev_min, dev_avg, dev_max = inst.time_loop_device(5, 20, "last_hidden", np.float16)
+
+    # ---- untimed for `value`: two instances of the same model driven from two host threads at once, each on its own
+    # stream with its own batch of 8 resident in HBM.  One forward is a chain of dependent launches, each with a ramp, a
+    # tail and a gap in front of it; a second chain fills them.  Sequences/s over both instances; the latency of one
+    # forward roughly doubles.
+    pair_dt = None
+    if not args.no_second_instance:
+        import threading
+        inst_b = host.RocmInstance.from_graph(graph, "fp16")
+        inst_b.set_input("input_ids", ids)
+        inst_b.set_input("token_type_ids", seg)
+        inst_b.set_input("attention_bias", mask.reshape(B, 1, 1, S))
+        for _ in range(max(args.warmup, 3)):
+            inst_b.forward()
+        pair = [inst, inst_b]
+
+        def drive(i):
+            for _ in range(args.steps):
+                pair[i].forward()
+        inst.sync()
+        inst_b.sync()
+        tp0 = time.perf_counter()
+        threads = [threading.Thread(target=drive, args=(i,)) for i in range(2)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        inst.sync()
+        inst_b.sync()
+        pair_dt = time.perf_counter() - tp0
+        inst_b.close()
 
     ms_per_step = dt / args.steps * 1e3
     seqs_per_s = B * args.steps / dt
@@ -271,6 +305,12 @@ def main():
                                         "ms_min_avg_max": [round(dev_min * 1e3, 4), round(dev_avg * 1e3, 4),
                                                            round(dev_max * 1e3, 4)],
                                         "sequences_per_s": round(B / dev_avg, 2)}},
+        "two_instances_at_once": None if pair_dt is None else {
+            "what": "two Instances of this model, each with its own batch of %d, driven from two host threads on two "
+                    "streams: %d forwards each; not `value` (two batches in flight, a forward's latency about doubles)"
+                    % (B, args.steps),
+            "sequences_per_s": round(2 * B * args.steps / pair_dt, 2),
+            "ms_per_forward_per_instance": round(pair_dt / args.steps * 1e3, 4)},
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": ("12-layer BERT-base encoder fp16, batch 8, seq 384, valid lengths U[200,384] "
                                 "(BASELINE.json configs[1])") if full_cfg else
