@@ -26,10 +26,24 @@ def mixed_violations(got, ref, atol=ATOL, rtol=RTOL):
     return int((d > atol + rtol * np.abs(ref)).sum()), float(d.max()), float(np.sqrt((d ** 2).mean()))
 
 
-def _run_full_depth(cfg, w, B, S, lo, hi, seed, precision="fp16"):
+def _progress(capsys, text):
+    """a line past pytest's capture: these tests spend minutes in the CPU checker and in building gigabyte model files,
+    and a run that prints nothing for that long looks hung from outside"""
+    if capsys is None:
+        print(text, flush=True)
+        return
+    with capsys.disabled():
+        print(text, flush=True)
+
+
+def _run_full_depth(cfg, w, B, S, lo, hi, seed, precision="fp16", capsys=None):
     host, tnnmodel, _, _, make_inputs = _mods()
     ids, seg, lens, mask = make_inputs(cfg, B, S, lo, hi, seed=seed)
-    inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S), precision)
+    _progress(capsys, "[depth] writing the model files (%d layers, hidden %d)" % (cfg.layers, cfg.hidden))
+    graph = tnnmodel.encoder_graph(cfg, w, B, S)
+    _progress(capsys, "[depth] creating the instance")
+    inst = host.RocmInstance.from_graph(graph, precision)
+    _progress(capsys, "[depth] forward x4")
     inst.set_input("input_ids", ids)
     inst.set_input("token_type_ids", seg)
     inst.set_input("attention_bias", mask.reshape(B, 1, 1, S))
@@ -49,9 +63,7 @@ def _check_one_sequence(cfg, w, ids, seg, lens, mask, got, S, what, capsys):
     ref = encoder_ref.embed(w16, ids[b:b + 1], seg[b:b + 1], cfg.eps)
     for li, lw in enumerate(w16["layers"]):  # the checker takes seconds per layer: show progress past pytest's capture
         ref = encoder_ref.encoder_layer(ref, lw, 1, S, cfg.heads, mask[b:b + 1], cfg.eps)
-        if li % 4 == 3:
-            with capsys.disabled():
-                print("[checker] %s: layer %d of %d" % (what, li + 1, cfg.layers), flush=True)
+        _progress(capsys, "[checker] %s: layer %d of %d" % (what, li + 1, cfg.layers))
     g = got[b].reshape(S, cfg.hidden)
     err = rel_err(g, ref)
     bad, dmax, rms = mixed_violations(g, ref)
@@ -74,7 +86,7 @@ def test_bench_model_12_layers_against_checker(capsys):
     say("depth: bench.py's model, 12 layers B8 S384 fp16")
     cfg = EncoderConfig.bert_base(12)
     w = make_weights(cfg, seed=20240601)
-    ids, seg, lens, mask, got = _run_full_depth(cfg, w, 8, 384, 200, 384, 20240602)
+    ids, seg, lens, mask, got = _run_full_depth(cfg, w, 8, 384, 200, 384, 20240602, capsys=capsys)
     _check_one_sequence(cfg, w, ids, seg, lens, mask, got, 384, "config 2", capsys)
 
 
@@ -84,13 +96,14 @@ def test_bert_large_24_layers_against_checker(capsys):
     _, _, EncoderConfig, make_weights, _ = _mods()
     say("depth: config 5, 24 layers B16 S512 fp16")
     cfg = EncoderConfig.bert_large(24)
+    _progress(capsys, "[depth] drawing the weights of 24 BERT-large layers")
     w = make_weights(cfg, seed=20240605)
-    ids, seg, lens, mask, got = _run_full_depth(cfg, w, 16, 512, 384, 512, 20240606)
+    ids, seg, lens, mask, got = _run_full_depth(cfg, w, 16, 512, 384, 512, 20240606, capsys=capsys)
     _check_one_sequence(cfg, w, ids, seg, lens, mask, got, 512, "config 5", capsys)
 
 
 @pytest.mark.timeout(600)
-def test_int8_model_12_layers_properties(monkeypatch):
+def test_int8_model_12_layers_properties(monkeypatch, capsys):
     """Config 4 at full depth (12 layers, B16 S256, hidden 768, FFN 3072): calibrated on this backend's fp32 forward,
     run quantised.  Every projection of the first and of the last layer reproduces its own int8 output bit-exactly from
     its own input blob (checker on a 192-row slice; the int32 accumulators behind them are pinned by an integer matmul
@@ -106,6 +119,7 @@ def test_int8_model_12_layers_properties(monkeypatch):
     ids, seg, lens, mask = make_inputs(cfg, B, S, 100, 256, seed=42)
     inputs = {"input_ids": ids, "token_type_ids": seg, "attention_bias": mask.reshape(B, 1, 1, S)}
     names = quant.calibration_outputs(cfg)
+    _progress(capsys, "[depth] calibration forward in fp32")
     inst = host.RocmInstance.from_graph(tnnmodel.encoder_graph(cfg, w, B, S, extra_outputs=names), "fp32")
     for k, v in inputs.items():
         inst.set_input(k, v)
@@ -118,6 +132,7 @@ def test_int8_model_12_layers_properties(monkeypatch):
     runs = {}
     for fuse, extra in (("0", check), ("1", [])):
         monkeypatch.setenv("TNN_ROCM_FUSE_INT8", fuse)
+        _progress(capsys, "[depth] quantised model, TNN_ROCM_FUSE_INT8=" + fuse)
         inst = host.RocmInstance.from_graph(quant.int8_encoder_graph(cfg, w, scales, B, S, extra_outputs=extra), "fp16")
         for k, v in inputs.items():
             inst.set_input(k, v)
@@ -126,6 +141,7 @@ def test_int8_model_12_layers_properties(monkeypatch):
         if fuse == "0":
             blobs = {n: inst.output(n, max_elems=1 << 26) for n in extra}
         inst.close()
+    _progress(capsys, "[depth] checker: twelve projections on 192 rows")
     n = golden_util.check_projections_bit_exact(cfg, w, scales, blobs, B * S, orc.quantize_x86, layers=(0, last), rows=192)
     assert n == 12
     e_fused, e_float = rel_err(runs["1"], runs["0"]), rel_err(runs["1"], float_out)
