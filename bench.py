@@ -22,6 +22,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 SUSTAINED_FP16_TFLOPS = 1692.0  # measured: MFMA-only loop on every SIMD, normally distributed operands (the SIMD probe)
+SUSTAINED_INT8_TOPS = 3439.0    # the same loop with v_mfma_i32_32x32x32_i8 on operands uniform in [-127, 127]
 
 # HBM bytes per launch (fetched + written) of the projection GEMMs at the batch-8 / seq-384 workload, from two
 # rocprofv3 --pmc runs of this command (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
@@ -269,7 +270,14 @@ def main():
                                            "table epilogue)" % (T8, F, H),
                 "achieved": round(opsn / (ms * 1e-3) / 1e12, 2), "peak": 5000.0, "unit": "TOP/s",
                 "frac": round(opsn / (ms * 1e-3) / 1e12 / 5000.0, 4), "traffic": None,
-                "us_per_launch": round(ms * 1e3, 2), "ops_per_launch": opsn}
+                "us_per_launch": round(ms * 1e3, 2), "ops_per_launch": opsn,
+                "sustained_matrix_rate": {"tops": SUSTAINED_INT8_TOPS,
+                                          "frac": round(opsn / (ms * 1e-3) / 1e12 / SUSTAINED_INT8_TOPS, 4),
+                                          "what": "what the chip holds with every SIMD issuing nothing but independent int8 "
+                                                  "MFMAs on operands that use the whole int8 range (4897 on all-zero ones); "
+                                                  "context only, frac above stays on the data-sheet peak",
+                                          "source": "profiles/simd_probe_mfma_valu_lds.txt (python -m tnn_amd.bench_ops "
+                                                    "--simd-probe), typed into bench.py, not measured by this run"}}
 
     # the dominant GEMM inside the forward: the event pair the eager layer loop puts around its layer (profile pass above),
     # averaged over the layers.  It spans from the previous layer's last kernel to this layer's last kernel on the

@@ -40,6 +40,8 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
 
 enum { MFMA_ONLY, VALU_ONLY, CHAIN, LDS_ONLY, TILE, TILE_AHEAD, PIPE, PIPE_LDS, SKEW, SKEW_LDS };
 
@@ -368,6 +370,72 @@ __global__ void __launch_bounds__(256) matrix_rate(const u32x4 *__restrict__ ope
         out[0] = t;
 }
 
+// the int8 counterpart: sixteen independent v_mfma_i32_32x32x32_i8 per iteration
+__global__ void __launch_bounds__(256) matrix_rate_i8(const u32x4 *__restrict__ operands, int *out, int iters) {
+    i32x4 a[4], b[4];
+    for (int i = 0; i < 4; ++i) {
+        a[i] = __builtin_bit_cast(i32x4, operands[(i * 2 + 0) * 64 + (threadIdx.x & 63)]);
+        b[i] = __builtin_bit_cast(i32x4, operands[(i * 2 + 1) * 64 + (threadIdx.x & 63)]);
+    }
+    i32x16 acc[4][4];
+    for (int i = 0; i < 4; ++i)
+        for (int j = 0; j < 4; ++j)
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[j], a[i], acc[i][j], 0, 0, 0);
+    }
+    int t = 0;
+    for (int i = 0; i < 4; ++i)
+        for (int j = 0; j < 4; ++j)
+            for (int r = 0; r < 16; ++r)
+                t += acc[i][j][r];
+    if (t == 123456789)
+        out[0] = t;
+}
+
+// POP/s of the chip with every SIMD issuing int8 MFMAs only; data: 0 zeros, 1 ones, 2 uniform in [-127, 127] (quantised
+// activations and weights use the whole range)
+double matrix_rate_i8_pops(int data) {
+    const int n = 8 * 64 * 16;  // eight fragments of 64 lanes x 16 bytes
+    signed char *h = (signed char *)malloc(n);
+    unsigned long long st = 1442695040888963407ull;
+    for (int i = 0; i < n; ++i) {
+        st = st * 6364136223846793005ull + 1442695040888963407ull;
+        h[i] = data == 0 ? 0 : data == 1 ? 1 : (signed char)((int)((st >> 33) % 255) - 127);
+    }
+    u32x4 *d = nullptr;
+    int *o   = nullptr;
+    if (hipMalloc(&d, n) != hipSuccess || hipMalloc(&o, 4) != hipSuccess)
+        return -1.0;
+    (void)hipMemcpy(d, h, n, hipMemcpyHostToDevice);
+    free(h);
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    const int iters = 4000, reps = 6;
+    dim3 grid(256), block(256);
+    hipLaunchKernelGGL(matrix_rate_i8, grid, block, 0, 0, d, o, iters);
+    (void)hipDeviceSynchronize();
+    (void)hipEventRecord(e0);
+    for (int r = 0; r < reps; ++r)
+        hipLaunchKernelGGL(matrix_rate_i8, grid, block, 0, 0, d, o, iters);
+    (void)hipEventRecord(e1);
+    (void)hipEventSynchronize(e1);
+    float ms = 0.f;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    (void)hipFree(d);
+    (void)hipFree(o);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    const double ops = 1024.0 * 16.0 * iters * reps * 65536.0;  // 1024 waves x 16 MFMAs x 32*32*32*2
+    return ops / (ms * 1e-3) / 1e15;
+}
+
 // PFLOP/s of the chip with every SIMD issuing MFMAs only; data: 0 zeros, 1 ones, 2 normal (sigma 0.5 x sigma 0.02, the
 // scale of activations times weights)
 double matrix_rate_pflops(int data) {
@@ -463,6 +531,12 @@ int main() {
     for (int data = 0; data < 3; ++data) {
         const double pf = matrix_rate_pflops(data);
         printf("%-32s %6.3f PFLOP/s   %5.2f GHz\n", names[data], pf, pf * 1e15 / (1024.0 * 1024.0) / 1e9);
+    }
+    printf("\nint8: sixteen independent v_mfma_i32_32x32x32_i8 per iteration (5.0 POP/s dense peak = 2048 OP per clock and SIMD)\n");
+    const char *names8[3] = {"operands all zero", "operands all one", "operands uniform in [-127,127]"};
+    for (int data = 0; data < 3; ++data) {
+        const double po = matrix_rate_i8_pops(data);
+        printf("%-32s %6.3f POP/s    %5.2f GHz\n", names8[data], po, po * 1e15 / (2048.0 * 1024.0) / 1e9);
     }
     return 0;
 }
