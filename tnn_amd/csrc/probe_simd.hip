@@ -343,6 +343,10 @@ template <bool WITH_LDS> __global__ void __launch_bounds__(256) probe_skew(float
         out[0] = t;
 }
 
+// ORDER: the sequence in which the sixteen accumulators take their MFMA within one iteration.  0 row-major (the A
+// fragment stays on its port for four MFMAs in a row), 1 diagonals (both operand ports change with every MFMA), 2
+// boustrophedon (exactly one port changes with every MFMA)
+template <int ORDER>
 __global__ void __launch_bounds__(256) matrix_rate(const u32x4 *__restrict__ operands, float *out, int iters) {
     f16x8 a[4], b[4];
     for (int i = 0; i < 4; ++i) {
@@ -356,10 +360,11 @@ __global__ void __launch_bounds__(256) matrix_rate(const u32x4 *__restrict__ ope
                 acc[i][j][r] = 0.f;
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[j], a[i], acc[i][j], 0, 0, 0);
+        for (int s = 0; s < 16; ++s) {
+            const int i = ORDER == 1 ? (s & 3) : (s >> 2);
+            const int j = ORDER == 1 ? ((s & 3) + (s >> 2)) & 3 : (ORDER == 2 && ((s >> 2) & 1) ? 3 - (s & 3) : (s & 3));
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[j], a[i], acc[i][j], 0, 0, 0);
+        }
     }
     float t = 0.f;
     for (int i = 0; i < 4; ++i)
@@ -438,7 +443,7 @@ double matrix_rate_i8_pops(int data) {
 
 // PFLOP/s of the chip with every SIMD issuing MFMAs only; data: 0 zeros, 1 ones, 2 normal (sigma 0.5 x sigma 0.02, the
 // scale of activations times weights)
-double matrix_rate_pflops(int data) {
+double matrix_rate_pflops(int data, int order = 0) {
     const int n = 8 * 64 * 8;  // eight fragments of 64 lanes x 8 halves
     _Float16 *h = (_Float16 *)malloc(n * sizeof(_Float16));
     unsigned long long st = 88172645463325252ull;
@@ -462,11 +467,19 @@ double matrix_rate_pflops(int data) {
     (void)hipEventCreate(&e1);
     const int iters = 4000, reps = 6;  // 64 000 MFMAs per wave and launch: about 0.8 ms
     dim3 grid(256), block(256);
-    hipLaunchKernelGGL(matrix_rate, grid, block, 0, 0, d, o, iters);
+    auto launch = [&]() {
+        if (order == 1)
+            hipLaunchKernelGGL(matrix_rate<1>, grid, block, 0, 0, d, o, iters);
+        else if (order == 2)
+            hipLaunchKernelGGL(matrix_rate<2>, grid, block, 0, 0, d, o, iters);
+        else
+            hipLaunchKernelGGL(matrix_rate<0>, grid, block, 0, 0, d, o, iters);
+    };
+    launch();
     (void)hipDeviceSynchronize();
     (void)hipEventRecord(e0);
     for (int r = 0; r < reps; ++r)
-        hipLaunchKernelGGL(matrix_rate, grid, block, 0, 0, d, o, iters);
+        launch();
     (void)hipEventRecord(e1);
     (void)hipEventSynchronize(e1);
     float ms = 0.f;
@@ -532,6 +545,13 @@ int main() {
         const double pf = matrix_rate_pflops(data);
         printf("%-32s %6.3f PFLOP/s   %5.2f GHz\n", names[data], pf, pf * 1e15 / (1024.0 * 1024.0) / 1e9);
     }
+    printf("\nthe same on normally distributed operands, by the order of the sixteen MFMAs of an iteration\n");
+    const char *orders[3] = {"row-major (A kept for four)", "diagonals (both ports change)", "boustrophedon (one port changes)"};
+    for (int rep = 0; rep < 2; ++rep)
+        for (int order = 0; order < 3; ++order) {
+            const double pf = matrix_rate_pflops(2, order);
+            printf("%-36s %6.3f PFLOP/s   %5.2f GHz\n", orders[order], pf, pf * 1e15 / (1024.0 * 1024.0) / 1e9);
+        }
     printf("\nint8: sixteen independent v_mfma_i32_32x32x32_i8 per iteration (5.0 POP/s dense peak = 2048 OP per clock and SIMD)\n");
     const char *names8[3] = {"operands all zero", "operands all one", "operands uniform in [-127,127]"};
     for (int data = 0; data < 3; ++data) {
